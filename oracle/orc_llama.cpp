@@ -1,0 +1,132 @@
+// CPU oracle (test infrastructure only): the dense-transformer forward pass of
+// cera's LlamaModel on the CPU int8 path -- cera/src/model/llama.rs:468-597
+// (run_layers, project_logits), :1585-1605 (forward) and
+// cera/src/model/transformer.rs:1313-1652 (attention / FFN blocks).
+#include "orc_llama.h"
+
+#include <cmath>
+#include <cstring>
+#include <vector>
+
+struct OrcLlama {
+    OrcLlamaConfig cfg;
+    OrcTensor embd, output;
+    bool has_output = false;
+    const float* output_norm = nullptr;
+    std::vector<OrcLlamaLayer> layers;
+    // state (kv_cache.rs:201-221): per layer time-major f32 K and V, [pos][kv_dim]
+    std::vector<std::vector<float>> kc, vc;
+    uint32_t seq_len = 0;
+    int variant = 0;
+    void* pool = nullptr;  // optional worker pool for the GEMVs (timing only)
+};
+
+static void gemv(OrcLlama* m, const OrcTensor& t, const float* x, float* y) {
+    if (m->pool) orc_gemv_mt(m->pool, t.dtype, t.data, x, y, t.m, t.k);
+    else orc_gemv(t.dtype, t.data, x, y, t.m, t.k, m->variant);
+}
+
+OrcLlama* orc_llama_create(const OrcLlamaConfig* cfg, const OrcTensor* embd, const OrcTensor* output,
+                           const float* output_norm, const OrcLlamaLayer* layers, int variant) {
+    OrcLlama* m = new OrcLlama();
+    m->cfg = *cfg;
+    m->embd = *embd;
+    if (output) { m->output = *output; m->has_output = true; }
+    m->output_norm = output_norm;
+    m->layers.assign(layers, layers + cfg->n_layers);
+    m->kc.resize(cfg->n_layers);
+    m->vc.resize(cfg->n_layers);
+    m->variant = variant;
+    return m;
+}
+void orc_llama_destroy(OrcLlama* m) { delete m; }
+void orc_llama_set_pool(OrcLlama* m, void* pool) { m->pool = pool; }
+uint32_t orc_llama_seq_len(const OrcLlama* m) { return m->seq_len; }
+void orc_llama_truncate(OrcLlama* m, uint32_t len) {
+    if (len >= m->seq_len) return;
+    uint64_t kv_dim = uint64_t(m->cfg.n_kv_heads) * m->cfg.head_dim;
+    for (auto& v : m->kc) v.resize(len * kv_dim);
+    for (auto& v : m->vc) v.resize(len * kv_dim);
+    m->seq_len = len;
+}
+
+// llama.rs:1585-1605 + :468-597.  Writes vocab logits; optionally the final
+// normed hidden state (for intermediate-value checks).
+int orc_llama_forward(OrcLlama* m, uint32_t token, uint32_t pos, float* logits, float* hidden_out) {
+    const OrcLlamaConfig& c = m->cfg;
+    if (token >= c.vocab || pos != m->seq_len) return -1;
+    const uint32_t hs = c.hidden, hd = c.head_dim;
+    const uint32_t q_dim = c.n_heads * hd, kv_dim = c.n_kv_heads * hd;
+    std::vector<float> hidden(hs), normed(hs), ffn_in(hs), q(q_dim), k(kv_dim), v(kv_dim),
+        attn_out(q_dim), out(hs), gate(c.ffn), up(c.ffn);
+
+    const uint8_t* erow = static_cast<const uint8_t*>(m->embd.data) +
+                          uint64_t(token) * orc_row_bytes(m->embd.dtype, m->embd.k);
+    if (orc_dequantize_row(m->embd.dtype, erow, m->embd.k, hidden.data())) return -2;
+    if (c.embed_scale != 1.0f) for (auto& x : hidden) x *= c.embed_scale;
+
+    const float scale = c.attn_scale != 0.0f ? c.attn_scale : 1.0f / std::sqrt(float(hd));
+    for (uint32_t l = 0; l < c.n_layers; ++l) {
+        const OrcLlamaLayer& L = m->layers[l];
+        normed = hidden;
+        orc_rmsnorm(normed.data(), L.attn_norm, hs, c.rms_eps);
+        gemv(m, L.attn_q, normed.data(), q.data());
+        gemv(m, L.attn_k, normed.data(), k.data());
+        gemv(m, L.attn_v, normed.data(), v.data());
+        if (L.q_bias && L.k_bias && L.v_bias) {
+            orc_add(q.data(), L.q_bias, q_dim);
+            orc_add(k.data(), L.k_bias, kv_dim);
+            orc_add(v.data(), L.v_bias, kv_dim);
+        }
+        if (L.q_norm && L.k_norm) {
+            for (uint32_t h = 0; h < c.n_heads; ++h) orc_rmsnorm(q.data() + h * hd, L.q_norm, hd, c.rms_eps);
+            for (uint32_t h = 0; h < c.n_kv_heads; ++h) orc_rmsnorm(k.data() + h * hd, L.k_norm, hd, c.rms_eps);
+        }
+        if (c.rope_type == 0) orc_rope_neox(q.data(), k.data(), pos, c.n_heads, c.n_kv_heads, hd, c.rope_theta);
+        else orc_rope_norm(q.data(), k.data(), pos, c.n_heads, c.n_kv_heads, hd, c.rope_theta, c.rope_freqs);
+        m->kc[l].insert(m->kc[l].end(), k.begin(), k.end());
+        m->vc[l].insert(m->vc[l].end(), v.begin(), v.end());
+        uint64_t L_ctx = m->kc[l].size() / kv_dim;
+        orc_decode_attention(q.data(), m->kc[l].data(), m->vc[l].data(), c.n_heads, c.n_kv_heads, hd,
+                             scale, L_ctx, attn_out.data(), m->variant);
+        gemv(m, L.attn_output, attn_out.data(), out.data());
+        if (c.residual_scale != 1.0f) for (auto& x : out) x *= c.residual_scale;
+        orc_add(hidden.data(), out.data(), hs);
+
+        ffn_in = hidden;
+        orc_rmsnorm(ffn_in.data(), L.ffn_norm, hs, c.rms_eps);
+        gemv(m, L.ffn_gate, ffn_in.data(), gate.data());
+        gemv(m, L.ffn_up, ffn_in.data(), up.data());
+        orc_silu_mul(gate.data(), up.data(), c.ffn);
+        gemv(m, L.ffn_down, gate.data(), out.data());
+        if (c.residual_scale != 1.0f) for (auto& x : out) x *= c.residual_scale;
+        orc_add(hidden.data(), out.data(), hs);
+    }
+    orc_rmsnorm(hidden.data(), m->output_norm, hs, c.rms_eps);
+    m->seq_len += 1;
+    if (hidden_out) std::memcpy(hidden_out, hidden.data(), hs * sizeof(float));
+    if (logits) {
+        const OrcTensor& o = m->has_output ? m->output : m->embd;
+        gemv(m, o, hidden.data(), logits);
+        if (c.logit_scale != 1.0f) {
+            float inv = 1.0f / c.logit_scale;
+            for (uint32_t i = 0; i < c.vocab; ++i) logits[i] *= inv;
+        }
+    }
+    return 0;
+}
+
+// llama.rs:1607-1649 per-token route (tokens.len() == 1 or oracle-dump mode);
+// the batched route is orc_llama_forward_prefill_batched.
+int orc_llama_forward_prefill_per_token(OrcLlama* m, const uint32_t* tokens, uint32_t n,
+                                        uint32_t start_pos, float* last_logits) {
+    if (n == 0 || start_pos != m->seq_len) return -1;
+    for (uint32_t i = 0; i < n; ++i) {
+        int rc = orc_llama_forward(m, tokens[i], start_pos + i, i + 1 == n ? last_logits : nullptr, nullptr);
+        if (rc) return rc;
+    }
+    return 0;
+}
+
+const float* orc_llama_kcache(const OrcLlama* m, uint32_t layer) { return m->kc[layer].data(); }
+const float* orc_llama_vcache(const OrcLlama* m, uint32_t layer) { return m->vc[layer].data(); }

@@ -1,0 +1,230 @@
+// CPU oracle (test infrastructure only): glue ops and decode attention,
+// restating cera/src/backend/cpu.rs and cera/src/model/transformer.rs.
+#include "orc_common.h"
+
+#include <cmath>
+#include <cstring>
+#include <vector>
+
+#if defined(__x86_64__)
+#include <immintrin.h>
+#define ORC_X86 1
+#define ORC_AVX2 __attribute__((target("avx2,fma")))
+#else
+#define ORC_X86 0
+#endif
+
+static inline float bits_f32(uint32_t b) { float f; std::memcpy(&f, &b, 4); return f; }
+static inline uint32_t f32_bits(float f) { uint32_t b; std::memcpy(&b, &f, 4); return b; }
+
+// cpu.rs:2479-2496 -- f64 sum of squares, inv_rms narrowed to f32.
+void orc_rmsnorm(float* x, const float* weight, uint64_t n, float eps) {
+    double sum_sq = 0.0;
+    for (uint64_t i = 0; i < n; ++i) sum_sq += double(x[i]) * double(x[i]);
+    double mean = sum_sq / double(n);
+    double rms = std::sqrt(mean + double(eps));
+    float inv_rms = float(1.0 / rms);
+    for (uint64_t i = 0; i < n; ++i) x[i] = x[i] * inv_rms * weight[i];
+}
+
+// cpu.rs:2504-2544 -- ggml's polynomial expf, no FMA contraction.
+float orc_expf(float x) {
+    const float R = bits_f32(0x4B400000u);
+    const float LOG2E = bits_f32(0x3FB8AA3Bu);
+    const float LN2_HI = bits_f32(0x3F317200u);
+    const float LN2_LO = bits_f32(0x35BFBE8Eu);
+    const float C1 = bits_f32(0x3F7FFFF6u);
+    const float C2 = bits_f32(0x3EFFFEDBu);
+    const float C3 = bits_f32(0x3E2AAF33u);
+    const float C4 = bits_f32(0x3D2B9F17u);
+    const float C5 = bits_f32(0x3C072010u);
+
+    float z = R + x * LOG2E;
+    float n = z - R;
+    float b = x - n * LN2_HI - n * LN2_LO;
+    uint32_t e = f32_bits(z) << 23;
+    float k = bits_f32(e + f32_bits(1.0f));
+    float u = b * b;
+    float j = C1 * b + (C2 + C3 * b + (C4 + C5 * b) * u) * u;
+    float abs_n = bits_f32(f32_bits(n) & 0x7FFFFFFFu);
+    if (abs_n <= 126.0f) {
+        return k + j * k;
+    } else if (abs_n > 192.0f) {
+        return n > 0.0f ? INFINITY : 0.0f;
+    } else {
+        uint32_t d = n <= 0.0f ? 0x82000000u : 0u;
+        float s1 = bits_f32(d + 0x7f000000u);
+        float s2 = bits_f32(e - d);
+        return (s2 + s2 * j) * s1;
+    }
+}
+
+// cpu.rs:2570-2575
+void orc_silu_mul(float* gate, const float* up, uint64_t n) {
+    for (uint64_t i = 0; i < n; ++i) gate[i] = gate[i] / (1.0f + orc_expf(-gate[i])) * up[i];
+}
+
+// cpu.rs:2617-2633 -- max via f32::max, f64 sum, f32 inverse.
+void orc_softmax(float* x, uint64_t n) {
+    float mx = -INFINITY;
+    for (uint64_t i = 0; i < n; ++i) mx = fmaxf(mx, x[i]);
+    double sum = 0.0;
+    for (uint64_t i = 0; i < n; ++i) {
+        x[i] = orc_expf(x[i] - mx);
+        sum += double(x[i]);
+    }
+    float inv_sum = float(1.0 / sum);
+    for (uint64_t i = 0; i < n; ++i) x[i] *= inv_sum;
+}
+
+// cpu.rs:5223-5228
+void orc_add(float* a, const float* b, uint64_t n) {
+    for (uint64_t i = 0; i < n; ++i) a[i] += b[i];
+}
+
+// cpu.rs:5161-5180 (rope_norm_pairs): interleaved pairs, theta iterated in f32,
+// libm sincos.
+static void rope_norm_head(float* head, float theta_start, uint32_t head_dim, float freq_base,
+                           const float* ff) {
+    float theta_scale = powf(freq_base, -2.0f / float(head_dim));
+    float theta_base = theta_start;
+    for (uint32_t i = 0; i < head_dim / 2; ++i) {
+        float f = ff ? ff[i] : 1.0f;
+        float theta = theta_base / f;
+        float s = sinf(theta), c = cosf(theta);
+        float x0 = head[2 * i], x1 = head[2 * i + 1];
+        head[2 * i] = x0 * c - x1 * s;
+        head[2 * i + 1] = x0 * s + x1 * c;
+        theta_base *= theta_scale;
+    }
+}
+// cpu.rs:5091-5125
+void orc_rope_norm(float* q, float* k, uint64_t pos, uint32_t n_heads, uint32_t n_kv_heads,
+                   uint32_t head_dim, float freq_base, const float* freq_factors) {
+    for (uint32_t h = 0; h < n_heads; ++h) rope_norm_head(q + h * head_dim, float(pos), head_dim, freq_base, freq_factors);
+    for (uint32_t h = 0; h < n_kv_heads; ++h) rope_norm_head(k + h * head_dim, float(pos), head_dim, freq_base, freq_factors);
+}
+// cpu.rs:5031-5045 (apply_rope_to_head): split-half (NEOX) pairing.
+static void rope_neox_head(float* head, float theta_start, uint32_t head_dim, float freq_base) {
+    uint32_t half = head_dim / 2;
+    float theta_scale = powf(freq_base, -2.0f / float(head_dim));
+    float theta = theta_start;
+    for (uint32_t i = 0; i < half; ++i) {
+        float s = sinf(theta), c = cosf(theta);
+        float x0 = head[i], x1 = head[i + half];
+        head[i] = x0 * c - x1 * s;
+        head[i + half] = x0 * s + x1 * c;
+        theta *= theta_scale;
+    }
+}
+void orc_rope_neox(float* q, float* k, uint64_t pos, uint32_t n_heads, uint32_t n_kv_heads,
+                   uint32_t head_dim, float freq_base) {
+    for (uint32_t h = 0; h < n_heads; ++h) rope_neox_head(q + h * head_dim, float(pos), head_dim, freq_base);
+    for (uint32_t h = 0; h < n_kv_heads; ++h) rope_neox_head(k + h * head_dim, float(pos), head_dim, freq_base);
+}
+
+// sampler.rs:20-30 -- strict >, lowest index on ties, NaN never wins.
+uint32_t orc_argmax(const float* logits, uint64_t n) {
+    uint32_t best_i = 0;
+    float best_v = -INFINITY;
+    for (uint64_t i = 0; i < n; ++i)
+        if (logits[i] > best_v) { best_v = logits[i]; best_i = uint32_t(i); }
+    return best_i;
+}
+
+// ---------------------------------------------------------------------------
+// Decode attention.  variant 0: the scalar loops (cpu.rs:3275-3282, 3352-3362);
+// variant 1: the AVX2 twins (cpu.rs:3503-3553, 3555-3589).  They differ in
+// float summation order, as in the reference.
+#if ORC_X86
+ORC_AVX2 static inline float v_hsum256(__m256 v) {  // cpu.rs:3489
+    __m128 hi = _mm256_extractf128_ps(v, 1);
+    __m128 lo = _mm256_castps256_ps128(v);
+    __m128 s128 = _mm_add_ps(lo, hi);
+    __m128 s64 = _mm_add_ps(s128, _mm_movehl_ps(s128, s128));
+    __m128 s32 = _mm_add_ss(s64, _mm_shuffle_ps(s64, s64, 1));
+    return _mm_cvtss_f32(s32);
+}
+ORC_AVX2 static void v_attn_scores(const float* q, const float* kc, float* scores, uint64_t kv_dim,
+                                   uint64_t off, uint32_t hd, float scale, uint64_t L) {
+    __m256 qv[32];
+    uint32_t nq = hd / 8;
+    for (uint32_t i = 0; i < nq; ++i) qv[i] = _mm256_loadu_ps(q + 8 * i);
+    for (uint64_t t = 0; t < L; ++t) {
+        const float* kp = kc + t * kv_dim + off;
+        __m256 s0 = _mm256_setzero_ps(), s1 = _mm256_setzero_ps();
+        uint32_t i = 0;
+        while (i + 2 <= nq) {
+            s0 = _mm256_fmadd_ps(qv[i], _mm256_loadu_ps(kp + 8 * i), s0);
+            s1 = _mm256_fmadd_ps(qv[i + 1], _mm256_loadu_ps(kp + 8 * (i + 1)), s1);
+            i += 2;
+        }
+        if (i < nq) s0 = _mm256_fmadd_ps(qv[i], _mm256_loadu_ps(kp + 8 * i), s0);
+        scores[t] = v_hsum256(_mm256_add_ps(s0, s1)) * scale;
+    }
+}
+ORC_AVX2 static void v_attn_values(const float* scores, const float* vc, float* out, uint64_t kv_dim,
+                                   uint64_t off, uint32_t hd, uint64_t L) {
+    __m256 acc[32];
+    uint32_t nv = hd / 8;
+    for (uint32_t i = 0; i < nv; ++i) acc[i] = _mm256_setzero_ps();
+    for (uint64_t t = 0; t < L; ++t) {
+        __m256 s = _mm256_set1_ps(scores[t]);
+        const float* vp = vc + t * kv_dim + off;
+        for (uint32_t i = 0; i < nv; ++i) acc[i] = _mm256_fmadd_ps(s, _mm256_loadu_ps(vp + 8 * i), acc[i]);
+    }
+    for (uint32_t i = 0; i < nv; ++i) _mm256_storeu_ps(out + 8 * i, acc[i]);
+}
+static bool avx2_ok() { return __builtin_cpu_supports("avx2") && __builtin_cpu_supports("fma"); }
+#else
+static bool avx2_ok() { return false; }
+#endif
+
+void orc_attn_scores(const float* q, const float* kc, float* scores, uint64_t kv_dim, uint64_t off,
+                     uint32_t hd, float scale, uint64_t L, int variant) {
+#if ORC_X86
+    if (variant == 1 && hd % 8 == 0 && hd <= 256 && avx2_ok()) {
+        v_attn_scores(q, kc, scores, kv_dim, off, hd, scale, L);
+        return;
+    }
+#endif
+    (void)variant;
+    for (uint64_t t = 0; t < L; ++t) {
+        float dot = 0.0f;
+        const float* kp = kc + t * kv_dim + off;
+        for (uint32_t d = 0; d < hd; ++d) dot += q[d] * kp[d];
+        scores[t] = dot * scale;
+    }
+}
+void orc_attn_values(const float* scores, const float* vc, float* out, uint64_t kv_dim, uint64_t off,
+                     uint32_t hd, uint64_t L, int variant) {
+#if ORC_X86
+    if (variant == 1 && hd % 8 == 0 && hd <= 256 && avx2_ok()) {
+        v_attn_values(scores, vc, out, kv_dim, off, hd, L);
+        return;
+    }
+#endif
+    (void)variant;
+    for (uint32_t d = 0; d < hd; ++d) out[d] = 0.0f;
+    for (uint64_t t = 0; t < L; ++t) {
+        float s = scores[t];
+        const float* vp = vc + t * kv_dim + off;
+        for (uint32_t d = 0; d < hd; ++d) out[d] += s * vp[d];
+    }
+}
+
+// transformer.rs:1164-1220 (decode_attn_head) over all heads (:1249-1305);
+// query head h reads kv head h / (n_heads / n_kv_heads).
+void orc_decode_attention(const float* q, const float* kc, const float* vc, uint32_t n_heads,
+                          uint32_t n_kv_heads, uint32_t hd, float scale, uint64_t L, float* out,
+                          int variant) {
+    std::vector<float> scores(L);
+    uint64_t kv_dim = uint64_t(n_kv_heads) * hd;
+    uint32_t group = n_heads / n_kv_heads;
+    for (uint32_t h = 0; h < n_heads; ++h) {
+        uint64_t off = uint64_t(h / group) * hd;
+        orc_attn_scores(q + h * hd, kc, scores.data(), kv_dim, off, hd, scale, L, variant);
+        orc_softmax(scores.data(), L);
+        orc_attn_values(scores.data(), vc, out + h * hd, kv_dim, off, hd, L, variant);
+    }
+}
