@@ -39,17 +39,39 @@ def hipcc_path() -> str:
     raise RuntimeError("hipcc not found")
 
 
-def build_hip(verbose: bool = False) -> Path:
+def build_hip(verbose: bool = False, jobs: int = 8) -> Path:
+    """Compile every csrc/*.hip to an object (in parallel) and link the C-ABI library."""
+    from concurrent.futures import ThreadPoolExecutor
+
     LIB_DIR.mkdir(exist_ok=True)
+    obj_dir = LIB_DIR / "obj"
+    obj_dir.mkdir(exist_ok=True)
     srcs = sorted((PKG / "csrc").glob("*.hip"))
-    cmd = [hipcc_path(), *HIPCC_FLAGS, f"-I{ROOT / 'include'}", f"-I{PKG / 'csrc'}",
-           *map(str, srcs), "-o", str(HIP_LIB)]
+    hipcc = hipcc_path()
+    flags = [f for f in HIPCC_FLAGS if f != "-shared"]
+
+    def compile_one(src: Path):
+        obj = obj_dir / (src.stem + ".o")
+        cmd = [hipcc, *flags, f"-I{ROOT / 'include'}", f"-I{PKG / 'csrc'}", "-c", str(src), "-o", str(obj)]
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        return src, obj, cmd, r
+
+    objs = []
+    with ThreadPoolExecutor(max_workers=jobs) as ex:
+        for src, obj, cmd, r in ex.map(compile_one, srcs):
+            if verbose or r.returncode:
+                print(" ".join(cmd))
+                print(r.stdout + r.stderr)
+            if r.returncode:
+                raise RuntimeError(f"hipcc failed on {src.name}")
+            objs.append(str(obj))
+    cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", str(HIP_LIB)]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if verbose or r.returncode:
         print(" ".join(cmd))
         print(r.stdout + r.stderr)
     if r.returncode:
-        raise RuntimeError("hipcc failed")
+        raise RuntimeError("hipcc link failed")
     return HIP_LIB
 
 

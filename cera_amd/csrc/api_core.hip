@@ -1,0 +1,575 @@
+// C ABI: context, device memory, events, weight upload and the kernel-level
+// entry points (see include/cera_hip.h for the contract of each).
+#include <cstring>
+#include <new>
+
+#include "attention.cuh"
+#include "gemv_launch.cuh"
+#include "glue.cuh"
+#include "host_common.h"
+#include "quantize.cuh"
+
+bool cera_gemv_launch_q4k(const GemvArgs&, int, int, int, bool, dim3, hipStream_t);
+bool cera_gemv_launch_q6k(const GemvArgs&, int, int, int, bool, dim3, hipStream_t);
+bool cera_gemv_launch_q4_0(const GemvArgs&, int, int, int, bool, dim3, hipStream_t);
+bool cera_gemv_launch_q4_1(const GemvArgs&, int, int, int, bool, dim3, hipStream_t);
+bool cera_gemv_launch_q8_0(const GemvArgs&, int, int, int, bool, dim3, hipStream_t);
+
+// ---------------------------------------------------------------------------
+static std::mutex g_err_mu;
+static std::string g_err;
+
+void cera_set_global_error(const std::string& s) {
+    std::lock_guard<std::mutex> lk(g_err_mu);
+    g_err = s;
+}
+cera_hip_status cera_fail(cera_hip_ctx* ctx, cera_hip_status st, const std::string& msg) {
+    if (ctx) ctx->err = msg;
+    cera_set_global_error(msg);
+    return st;
+}
+
+bool cera_type_geometry(uint32_t t, uint32_t* e, uint32_t* b) {
+    switch (t) {
+        case CERA_HIP_F32: *e = 1; *b = 4; return true;
+        case CERA_HIP_F16: case CERA_HIP_BF16: *e = 1; *b = 2; return true;
+        case CERA_HIP_Q4_0: *e = 32; *b = 18; return true;
+        case CERA_HIP_Q4_1: *e = 32; *b = 20; return true;
+        case CERA_HIP_Q8_0: *e = 32; *b = 34; return true;
+        case CERA_HIP_Q4_K: *e = 256; *b = 144; return true;
+        case CERA_HIP_Q5_K: *e = 256; *b = 176; return true;
+        case CERA_HIP_Q6_K: *e = 256; *b = 210; return true;
+        default: return false;
+    }
+}
+
+cera_hip_status cera_scratch(cera_hip_ctx* ctx, int slot, uint64_t nbytes, void** out) {
+    if (nbytes == 0) nbytes = 256;
+    if (ctx->scratch_bytes[slot] < nbytes) {
+        if (ctx->scratch[slot]) {
+            HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+            HIP_TRY(ctx, hipFree(ctx->scratch[slot]));
+            ctx->scratch[slot] = nullptr;
+            ctx->scratch_bytes[slot] = 0;
+        }
+        uint64_t want = (nbytes + 4095) & ~uint64_t(4095);
+        HIP_TRY(ctx, hipMalloc(&ctx->scratch[slot], want));
+        ctx->scratch_bytes[slot] = want;
+    }
+    *out = ctx->scratch[slot];
+    return CERA_HIP_OK;
+}
+
+extern "C" {
+
+cera_hip_status cera_hip_ctx_create(int device, cera_hip_ctx** out) {
+    if (!out) return cera_fail(nullptr, CERA_HIP_ERR_ARGUMENT, "cera_hip_ctx_create: out is null");
+    *out = nullptr;
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess || n == 0)
+        return cera_fail(nullptr, CERA_HIP_ERR_DEVICE,
+                         std::string("no HIP device available: ") + (e != hipSuccess ? hipGetErrorString(e) : "count is 0"));
+    if (device < 0 || device >= n) return cera_fail(nullptr, CERA_HIP_ERR_ARGUMENT, "device index out of range");
+    cera_hip_ctx* ctx = new (std::nothrow) cera_hip_ctx();
+    if (!ctx) return cera_fail(nullptr, CERA_HIP_ERR_OOM, "host allocation failed");
+    ctx->device = device;
+    hipDeviceProp_t prop;
+    if ((e = hipSetDevice(device)) != hipSuccess || (e = hipGetDeviceProperties(&prop, device)) != hipSuccess ||
+        (e = hipStreamCreate(&ctx->stream)) != hipSuccess) {
+        delete ctx;
+        return cera_fail(nullptr, CERA_HIP_ERR_DEVICE, std::string("device init: ") + hipGetErrorString(e));
+    }
+    if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0) {
+        std::string arch = prop.gcnArchName;
+        hipStreamDestroy(ctx->stream);
+        delete ctx;
+        return cera_fail(nullptr, CERA_HIP_ERR_DEVICE, "kernels are built for gfx950 only; device is " + arch);
+    }
+    ctx->n_cu = static_cast<uint32_t>(prop.multiProcessorCount);
+    *out = ctx;
+    return CERA_HIP_OK;
+}
+
+void cera_hip_ctx_destroy(cera_hip_ctx* ctx) {
+    if (!ctx) return;
+    (void)hipSetDevice(ctx->device);
+    (void)hipStreamSynchronize(ctx->stream);
+    for (auto& p : ctx->scratch)
+        if (p) (void)hipFree(p);
+    if (ctx->attn_acc) (void)hipFree(ctx->attn_acc);
+    if (ctx->attn_ml) (void)hipFree(ctx->attn_ml);
+    (void)hipStreamDestroy(ctx->stream);
+    delete ctx;
+}
+
+const char* cera_hip_last_error(const cera_hip_ctx* ctx) {
+    if (ctx) return ctx->err.c_str();
+    static thread_local std::string copy;
+    std::lock_guard<std::mutex> lk(g_err_mu);
+    copy = g_err;
+    return copy.c_str();
+}
+
+cera_hip_status cera_hip_sync(cera_hip_ctx* ctx) {
+    if (!ctx) return CERA_HIP_ERR_ARGUMENT;
+    HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    return CERA_HIP_OK;
+}
+
+cera_hip_status cera_hip_device_info(cera_hip_ctx* ctx, char* name256, uint32_t* n_cu, uint64_t* hbm) {
+    if (!ctx) return CERA_HIP_ERR_ARGUMENT;
+    hipDeviceProp_t prop;
+    HIP_TRY(ctx, hipGetDeviceProperties(&prop, ctx->device));
+    if (name256) {
+        std::snprintf(name256, 256, "%s (%s)", prop.name, prop.gcnArchName);
+    }
+    if (n_cu) *n_cu = static_cast<uint32_t>(prop.multiProcessorCount);
+    if (hbm) *hbm = prop.totalGlobalMem;
+    return CERA_HIP_OK;
+}
+
+// ---- memory / events --------------------------------------------------------
+cera_hip_status cera_hip_malloc(cera_hip_ctx* ctx, uint64_t nbytes, void** out) {
+    if (!ctx || !out) return CERA_HIP_ERR_ARGUMENT;
+    *out = nullptr;
+    HIP_TRY(ctx, hipMalloc(out, nbytes ? nbytes : 256));
+    return CERA_HIP_OK;
+}
+cera_hip_status cera_hip_free(cera_hip_ctx* ctx, void* dev) {
+    if (!ctx) return CERA_HIP_ERR_ARGUMENT;
+    if (!dev) return CERA_HIP_OK;
+    HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    HIP_TRY(ctx, hipFree(dev));
+    return CERA_HIP_OK;
+}
+cera_hip_status cera_hip_upload(cera_hip_ctx* ctx, void* dst, const void* src, uint64_t n) {
+    if (!ctx || (!dst && n) || (!src && n)) return CERA_HIP_ERR_ARGUMENT;
+    if (n == 0) return CERA_HIP_OK;
+    HIP_TRY(ctx, hipMemcpyAsync(dst, src, n, hipMemcpyHostToDevice, ctx->stream));
+    HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    return CERA_HIP_OK;
+}
+cera_hip_status cera_hip_download(cera_hip_ctx* ctx, void* dst, const void* src, uint64_t n) {
+    if (!ctx || (!dst && n) || (!src && n)) return CERA_HIP_ERR_ARGUMENT;
+    if (n == 0) return CERA_HIP_OK;
+    HIP_TRY(ctx, hipMemcpyAsync(dst, src, n, hipMemcpyDeviceToHost, ctx->stream));
+    HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    return CERA_HIP_OK;
+}
+cera_hip_status cera_hip_copy_dev(cera_hip_ctx* ctx, void* dst, const void* src, uint64_t n) {
+    if (!ctx || (!dst && n) || (!src && n)) return CERA_HIP_ERR_ARGUMENT;
+    if (n == 0) return CERA_HIP_OK;
+    HIP_TRY(ctx, hipMemcpyAsync(dst, src, n, hipMemcpyDeviceToDevice, ctx->stream));
+    return CERA_HIP_OK;
+}
+cera_hip_status cera_hip_event_create(cera_hip_ctx* ctx, cera_hip_event** out) {
+    if (!ctx || !out) return CERA_HIP_ERR_ARGUMENT;
+    cera_hip_event* e = new (std::nothrow) cera_hip_event();
+    if (!e) return cera_fail(ctx, CERA_HIP_ERR_OOM, "host allocation failed");
+    hipError_t r = hipEventCreate(&e->ev);
+    if (r != hipSuccess) {
+        delete e;
+        return cera_fail(ctx, CERA_HIP_ERR_DEVICE, std::string("hipEventCreate: ") + hipGetErrorString(r));
+    }
+    *out = e;
+    return CERA_HIP_OK;
+}
+void cera_hip_event_destroy(cera_hip_event* e) {
+    if (!e) return;
+    (void)hipEventDestroy(e->ev);
+    delete e;
+}
+cera_hip_status cera_hip_event_record(cera_hip_ctx* ctx, cera_hip_event* e) {
+    if (!ctx || !e) return CERA_HIP_ERR_ARGUMENT;
+    HIP_TRY(ctx, hipEventRecord(e->ev, ctx->stream));
+    return CERA_HIP_OK;
+}
+cera_hip_status cera_hip_event_elapsed_ms(cera_hip_ctx* ctx, cera_hip_event* a, cera_hip_event* b, float* ms) {
+    if (!ctx || !a || !b || !ms) return CERA_HIP_ERR_ARGUMENT;
+    HIP_TRY(ctx, hipEventSynchronize(b->ev));
+    HIP_TRY(ctx, hipEventElapsedTime(ms, a->ev, b->ev));
+    return CERA_HIP_OK;
+}
+
+// ---- weights ------------------------------------------------------------------
+static cera_hip_status check_tensor(cera_hip_ctx* ctx, const cera_hip_tensor* t, uint64_t* row_bytes) {
+    if (!t || !t->data) return cera_fail(ctx, CERA_HIP_ERR_ARGUMENT, "tensor or tensor data is null");
+    uint32_t e, b;
+    if (!cera_type_geometry(t->ggml_type, &e, &b))
+        return cera_fail(ctx, CERA_HIP_ERR_UNSUPPORTED_DTYPE,
+                         "no hip kernel for ggml type " + std::to_string(t->ggml_type));
+    if (t->m == 0 || t->k == 0 || t->k % e)
+        return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "k=" + std::to_string(t->k) + " is not a whole number of " +
+                                                      std::to_string(e) + "-element blocks (or m/k is zero)");
+    *row_bytes = t->k / e * b;
+    if (t->nbytes != t->m * *row_bytes)
+        return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "tensor nbytes " + std::to_string(t->nbytes) + " != m*row_bytes " +
+                                                      std::to_string(t->m * *row_bytes));
+    if (t->m > 0xFFFFFFFFull || t->k > 0xFFFFFFFFull) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "dimension exceeds 2^32");
+    return CERA_HIP_OK;
+}
+
+static cera_hip_status alloc_dtensor(cera_hip_ctx* ctx, uint32_t dtype, uint64_t m, uint64_t k, uint64_t row_bytes,
+                                     cera_hip_dtensor** out) {
+    cera_hip_dtensor* d = new (std::nothrow) cera_hip_dtensor();
+    if (!d) return cera_fail(ctx, CERA_HIP_ERR_OOM, "host allocation failed");
+    d->dtype = dtype; d->m = m; d->k = k; d->row_bytes = row_bytes; d->nbytes = m * row_bytes;
+    // 64 bytes of slack: a dead lane may read up to one unit past its own data
+    hipError_t e = hipMalloc(reinterpret_cast<void**>(&d->dev), d->nbytes + 64);
+    if (e != hipSuccess) {
+        delete d;
+        return cera_fail(ctx, e == hipErrorOutOfMemory ? CERA_HIP_ERR_OOM : CERA_HIP_ERR_DEVICE,
+                         std::string("hipMalloc(weights): ") + hipGetErrorString(e));
+    }
+    *out = d;
+    return CERA_HIP_OK;
+}
+
+cera_hip_status cera_hip_tensor_upload(cera_hip_ctx* ctx, const cera_hip_tensor* t, cera_hip_dtensor** out) {
+    if (!ctx || !out) return CERA_HIP_ERR_ARGUMENT;
+    *out = nullptr;
+    uint64_t rb;
+    CERA_TRY(check_tensor(ctx, t, &rb));
+    cera_hip_dtensor* d;
+    CERA_TRY(alloc_dtensor(ctx, t->ggml_type, t->m, t->k, rb, &d));
+    hipError_t e = hipMemcpyAsync(d->dev, t->data, d->nbytes, hipMemcpyHostToDevice, ctx->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+    if (e != hipSuccess) {
+        (void)hipFree(d->dev);
+        delete d;
+        return cera_fail(ctx, CERA_HIP_ERR_DEVICE, std::string("weight upload: ") + hipGetErrorString(e));
+    }
+    *out = d;
+    return CERA_HIP_OK;
+}
+
+cera_hip_status cera_hip_tensor_clone(cera_hip_ctx* ctx, const cera_hip_dtensor* src, cera_hip_dtensor** out) {
+    if (!ctx || !src || !out) return CERA_HIP_ERR_ARGUMENT;
+    *out = nullptr;
+    cera_hip_dtensor* d;
+    CERA_TRY(alloc_dtensor(ctx, src->dtype, src->m, src->k, src->row_bytes, &d));
+    hipError_t e = hipMemcpyAsync(d->dev, src->dev, d->nbytes, hipMemcpyDeviceToDevice, ctx->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+    if (e != hipSuccess) {
+        (void)hipFree(d->dev);
+        delete d;
+        return cera_fail(ctx, CERA_HIP_ERR_DEVICE, std::string("weight clone: ") + hipGetErrorString(e));
+    }
+    *out = d;
+    return CERA_HIP_OK;
+}
+
+void cera_hip_tensor_free(cera_hip_ctx* ctx, cera_hip_dtensor* d) {
+    if (!d) return;
+    if (ctx) (void)hipStreamSynchronize(ctx->stream);
+    if (d->dev) (void)hipFree(d->dev);
+    delete d;
+}
+uint64_t cera_hip_tensor_nbytes(const cera_hip_dtensor* d) { return d ? d->nbytes : 0; }
+
+}  // extern "C"
+
+// ---------------------------------------------------------------------------
+// launchers
+cera_hip_status cera_launch_quantize(cera_hip_ctx* ctx, const float* x, uint64_t k, float* scales, int8_t* quants) {
+    if (k == 0 || k % 32) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "quantize_q8_0: k must be a positive multiple of 32");
+    uint64_t threads = k / 4;
+    dim3 grid(static_cast<uint32_t>((threads + 255) / 256));
+    hipLaunchKernelGGL(quantize_q8_0_kernel, grid, dim3(256), 0, ctx->stream, x, k, scales, quants);
+    HIP_TRY(ctx, hipGetLastError());
+    return CERA_HIP_OK;
+}
+
+static bool is_int8_type(uint32_t t) {
+    return t == CERA_HIP_Q4_0 || t == CERA_HIP_Q4_1 || t == CERA_HIP_Q8_0 || t == CERA_HIP_Q4_K || t == CERA_HIP_Q6_K;
+}
+
+cera_hip_status cera_launch_gemv(cera_hip_ctx* ctx, const cera_hip_dtensor* w, const cera_hip_dtensor* w2,
+                                 const float* xs, const int8_t* xq, float* y, const float* resid, int epi,
+                                 int32_t* dbg_dots, int32_t* dbg_asums) {
+    if (!is_int8_type(w->dtype))
+        return cera_fail(ctx, CERA_HIP_ERR_UNSUPPORTED_DTYPE, "no int8 gemv kernel for ggml type " + std::to_string(w->dtype));
+    if (epi == CERA_EPI_SILU_MUL) {
+        if (!w2 || w2->dtype != w->dtype || w2->m != w->m || w2->k != w->k)
+            return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "fused gate/up gemv needs two matrices of identical type and shape");
+    }
+    if (epi == CERA_EPI_ADD && !resid) return cera_fail(ctx, CERA_HIP_ERR_ARGUMENT, "residual pointer is null");
+    uint32_t n_units = static_cast<uint32_t>(w->k / 32);  // every format uses one unit per 32 weights
+    GemvArgs a;
+    a.w = w->dev;
+    a.w2 = w2 ? w2->dev : nullptr;
+    a.xq = xq;
+    a.xs = xs;
+    a.y = y;
+    a.resid = resid;
+    a.m = static_cast<uint32_t>(w->m);
+    a.n_units = n_units;
+    a.row_bytes = static_cast<uint32_t>(w->row_bytes);
+    a.dbg_dots = dbg_dots;
+    a.dbg_asums = dbg_asums;
+    a.dbg_stride = static_cast<uint32_t>(w->dtype == CERA_HIP_Q6_K ? w->k / 16 : w->k / 32);
+    GemvPlan p = gemv_plan(a.m, n_units, ctx->n_cu, dbg_dots != nullptr);
+    if (p.U == 0)
+        return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "gemv: k=" + std::to_string(w->k) + " exceeds the 16384 supported by the register-resident kernel");
+    a.rows_per_wave = p.rows_per_wave;
+    dim3 grid(p.n_blocks);
+    bool ok = false;
+    switch (w->dtype) {
+        case CERA_HIP_Q4_K: ok = cera_gemv_launch_q4k(a, p.U, p.RB, epi, dbg_dots != nullptr, grid, ctx->stream); break;
+        case CERA_HIP_Q6_K: ok = cera_gemv_launch_q6k(a, p.U, p.RB, epi, dbg_dots != nullptr, grid, ctx->stream); break;
+        case CERA_HIP_Q4_0: ok = cera_gemv_launch_q4_0(a, p.U, p.RB, epi, dbg_dots != nullptr, grid, ctx->stream); break;
+        case CERA_HIP_Q4_1: ok = cera_gemv_launch_q4_1(a, p.U, p.RB, epi, dbg_dots != nullptr, grid, ctx->stream); break;
+        case CERA_HIP_Q8_0: ok = cera_gemv_launch_q8_0(a, p.U, p.RB, epi, dbg_dots != nullptr, grid, ctx->stream); break;
+    }
+    if (!ok) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "gemv: no kernel instance for this shape");
+    HIP_TRY(ctx, hipGetLastError());
+    return CERA_HIP_OK;
+}
+
+cera_hip_status cera_launch_gemv_q5k_f32(cera_hip_ctx* ctx, const cera_hip_dtensor* w, const float* x, float* y) {
+    dim3 grid(static_cast<uint32_t>((w->m + 3) / 4));
+    hipLaunchKernelGGL(gemv_q5k_f32_kernel, grid, dim3(256), 0, ctx->stream, w->dev, x, y,
+                       static_cast<uint32_t>(w->m), static_cast<uint32_t>(w->k));
+    HIP_TRY(ctx, hipGetLastError());
+    return CERA_HIP_OK;
+}
+
+cera_hip_status cera_launch_attn_decode(cera_hip_ctx* ctx, const float* q, const float* kc, const float* vc,
+                                        uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, uint64_t seq_len,
+                                        uint64_t max_seq, float scale, uint32_t n_splits, float* out,
+                                        float* out_scales, int8_t* out_quants) {
+    if (head_dim != ATTN_HD) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "attn_decode: head_dim must be 128");
+    if (n_kv_heads == 0 || n_heads % n_kv_heads) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "attn_decode: n_heads must be a multiple of n_kv_heads");
+    uint32_t G = n_heads / n_kv_heads;
+    if (G != 1 && G != 2 && G != 4 && G != 8) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "attn_decode: group size must be 1, 2, 4 or 8");
+    if (seq_len == 0 || seq_len > max_seq || max_seq > 0x7FFFFFFFull) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "attn_decode: need 0 < seq_len <= max_seq < 2^31");
+    if (n_heads % 2) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "attn_decode: n_heads must be even");
+    uint32_t n_chunks = static_cast<uint32_t>((seq_len + ATTN_CHUNK - 1) / ATTN_CHUNK);
+    // parts (wavefronts) per kv head: enough to fill the chip ~8 waves per CU
+    // deep, but at least one chunk each
+    uint32_t want_parts = n_splits ? n_splits : std::max(1u, ctx->n_cu * 8 / n_kv_heads);
+    uint32_t chunks_per_part = std::max(1u, (n_chunks + want_parts - 1) / want_parts);
+    uint32_t n_parts = (n_chunks + chunks_per_part - 1) / chunks_per_part;
+    uint64_t acc_bytes = static_cast<uint64_t>(n_kv_heads) * n_parts * G * ATTN_HD * sizeof(float);
+    uint64_t ml_bytes = static_cast<uint64_t>(n_kv_heads) * n_parts * G * 2 * sizeof(float);
+    if (ctx->attn_acc_bytes < acc_bytes) {
+        HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+        if (ctx->attn_acc) HIP_TRY(ctx, hipFree(ctx->attn_acc));
+        ctx->attn_acc = nullptr; ctx->attn_acc_bytes = 0;
+        HIP_TRY(ctx, hipMalloc(reinterpret_cast<void**>(&ctx->attn_acc), acc_bytes));
+        ctx->attn_acc_bytes = acc_bytes;
+    }
+    if (ctx->attn_ml_bytes < ml_bytes) {
+        HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+        if (ctx->attn_ml) HIP_TRY(ctx, hipFree(ctx->attn_ml));
+        ctx->attn_ml = nullptr; ctx->attn_ml_bytes = 0;
+        HIP_TRY(ctx, hipMalloc(reinterpret_cast<void**>(&ctx->attn_ml), ml_bytes));
+        ctx->attn_ml_bytes = ml_bytes;
+    }
+    dim3 grid((n_parts + 3) / 4, n_kv_heads);
+    uint32_t sl = static_cast<uint32_t>(seq_len), ms = static_cast<uint32_t>(max_seq);
+#define ATTN_LAUNCH(GG)                                                                                    \
+    hipLaunchKernelGGL((attn_decode_partial_kernel<GG>), grid, dim3(256), 0, ctx->stream, q, kc, vc, sl, ms, \
+                       scale, chunks_per_part, n_parts, ctx->attn_acc, ctx->attn_ml)
+    switch (G) {
+        case 1: ATTN_LAUNCH(1); break;
+        case 2: ATTN_LAUNCH(2); break;
+        case 4: ATTN_LAUNCH(4); break;
+        default: ATTN_LAUNCH(8); break;
+    }
+#undef ATTN_LAUNCH
+    HIP_TRY(ctx, hipGetLastError());
+    if (out_quants)
+        hipLaunchKernelGGL((attn_decode_merge_kernel<true>), dim3(n_heads / 2), dim3(64), 0, ctx->stream,
+                           ctx->attn_acc, ctx->attn_ml, n_parts, G, out, out_scales, out_quants);
+    else
+        hipLaunchKernelGGL((attn_decode_merge_kernel<false>), dim3(n_heads / 2), dim3(64), 0, ctx->stream,
+                           ctx->attn_acc, ctx->attn_ml, n_parts, G, out, nullptr, nullptr);
+    HIP_TRY(ctx, hipGetLastError());
+    return CERA_HIP_OK;
+}
+
+// ---------------------------------------------------------------------------
+// kernel-level entry points
+extern "C" {
+
+cera_hip_status cera_hip_quantize_q8_0_dev(cera_hip_ctx* ctx, const float* x, uint64_t k, float* scales, int8_t* quants) {
+    if (!ctx || !x || !scales || !quants) return CERA_HIP_ERR_ARGUMENT;
+    return cera_launch_quantize(ctx, x, k, scales, quants);
+}
+
+cera_hip_status cera_hip_quantize_q8_0(cera_hip_ctx* ctx, const float* x, uint64_t k, float* scales, int8_t* quants) {
+    if (!ctx || !x || !scales || !quants) return CERA_HIP_ERR_ARGUMENT;
+    if (k == 0 || k % 32) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "quantize_q8_0: k must be a positive multiple of 32");
+    void *dx, *ds, *dq;
+    CERA_TRY(cera_scratch(ctx, 0, k * 4, &dx));
+    CERA_TRY(cera_scratch(ctx, 1, k / 32 * 4, &ds));
+    CERA_TRY(cera_scratch(ctx, 2, k, &dq));
+    CERA_TRY(cera_hip_upload(ctx, dx, x, k * 4));
+    CERA_TRY(cera_launch_quantize(ctx, static_cast<float*>(dx), k, static_cast<float*>(ds), static_cast<int8_t*>(dq)));
+    CERA_TRY(cera_hip_download(ctx, scales, ds, k / 32 * 4));
+    CERA_TRY(cera_hip_download(ctx, quants, dq, k));
+    return CERA_HIP_OK;
+}
+
+cera_hip_status cera_hip_gemv_q8_dev(cera_hip_ctx* ctx, const cera_hip_dtensor* w, const float* xs, const int8_t* xq, float* y) {
+    if (!ctx || !w || !xs || !xq || !y) return CERA_HIP_ERR_ARGUMENT;
+    return cera_launch_gemv(ctx, w, nullptr, xs, xq, y, nullptr, CERA_EPI_STORE);
+}
+
+cera_hip_status cera_hip_gemv_seq_dev(cera_hip_ctx* ctx, const cera_hip_gemv_op* ops, uint32_t n) {
+    if (!ctx || (!ops && n)) return CERA_HIP_ERR_ARGUMENT;
+    for (uint32_t i = 0; i < n; ++i) {
+        if (!ops[i].w || !ops[i].xs || !ops[i].xq || !ops[i].y) return cera_fail(ctx, CERA_HIP_ERR_ARGUMENT, "gemv_seq: null field in op " + std::to_string(i));
+        CERA_TRY(cera_launch_gemv(ctx, ops[i].w, nullptr, ops[i].xs, ops[i].xq, ops[i].y, nullptr, CERA_EPI_STORE));
+    }
+    return CERA_HIP_OK;
+}
+
+cera_hip_status cera_hip_gemv(cera_hip_ctx* ctx, const cera_hip_tensor* t, const float* x, float* y,
+                              int32_t* dbg_dots, int32_t* dbg_asums) {
+    if (!ctx || !x || !y) return CERA_HIP_ERR_ARGUMENT;
+    cera_hip_dtensor* w = nullptr;
+    CERA_TRY(cera_hip_tensor_upload(ctx, t, &w));
+    cera_hip_status st = CERA_HIP_OK;
+    const uint64_t k = w->k, m = w->m;
+    void *dx = nullptr, *ds = nullptr, *dq = nullptr, *dy = nullptr, *dd = nullptr;
+    auto run = [&]() -> cera_hip_status {
+        CERA_TRY(cera_scratch(ctx, 0, k * 4, &dx));
+        CERA_TRY(cera_scratch(ctx, 3, m * 4, &dy));
+        CERA_TRY(cera_hip_upload(ctx, dx, x, k * 4));
+        if (w->dtype == CERA_HIP_Q5_K) {
+            if (dbg_dots || dbg_asums) return cera_fail(ctx, CERA_HIP_ERR_ARGUMENT, "Q5_K has no integer block dots (f32 activation path)");
+            CERA_TRY(cera_launch_gemv_q5k_f32(ctx, w, static_cast<float*>(dx), static_cast<float*>(dy)));
+        } else {
+            if (!is_int8_type(w->dtype))
+                return cera_fail(ctx, CERA_HIP_ERR_UNSUPPORTED_DTYPE, "no gemv kernel for ggml type " + std::to_string(w->dtype));
+            CERA_TRY(cera_scratch(ctx, 1, k / 32 * 4, &ds));
+            CERA_TRY(cera_scratch(ctx, 2, k, &dq));
+            CERA_TRY(cera_launch_quantize(ctx, static_cast<float*>(dx), k, static_cast<float*>(ds), static_cast<int8_t*>(dq)));
+            uint64_t nd = (w->dtype == CERA_HIP_Q6_K ? k / 16 : k / 32);
+            const bool dbg = dbg_dots || dbg_asums;
+            void* da = nullptr;
+            if (dbg) {
+                // the debug instance accumulates partial integer dots with atomics: start from zero
+                CERA_TRY(cera_scratch(ctx, 4, m * nd * 4, &dd));
+                CERA_TRY(cera_scratch(ctx, 7, nd * 4, &da));
+                HIP_TRY(ctx, hipMemsetAsync(dd, 0, m * nd * 4, ctx->stream));
+                HIP_TRY(ctx, hipMemsetAsync(da, 0, nd * 4, ctx->stream));
+            }
+            CERA_TRY(cera_launch_gemv(ctx, w, nullptr, static_cast<float*>(ds), static_cast<int8_t*>(dq),
+                                      static_cast<float*>(dy), nullptr, CERA_EPI_STORE, static_cast<int32_t*>(dd),
+                                      static_cast<int32_t*>(da)));
+            if (dbg_dots) CERA_TRY(cera_hip_download(ctx, dbg_dots, dd, m * nd * 4));
+            if (dbg_asums) CERA_TRY(cera_hip_download(ctx, dbg_asums, da, nd * 4));
+        }
+        CERA_TRY(cera_hip_download(ctx, y, dy, m * 4));
+        return CERA_HIP_OK;
+    };
+    st = run();
+    cera_hip_tensor_free(ctx, w);
+    return st;
+}
+
+cera_hip_status cera_hip_attn_decode_dev(cera_hip_ctx* ctx, const float* q, const float* k, const float* v,
+                                         uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, uint64_t seq_len,
+                                         uint64_t max_seq, float scale, uint32_t n_splits, float* out) {
+    if (!ctx || !q || !k || !v || !out) return CERA_HIP_ERR_ARGUMENT;
+    return cera_launch_attn_decode(ctx, q, k, v, n_heads, n_kv_heads, head_dim, seq_len, max_seq, scale, n_splits, out, nullptr, nullptr);
+}
+
+cera_hip_status cera_hip_attn_decode(cera_hip_ctx* ctx, const float* q, const float* k, const float* v,
+                                     uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, uint64_t seq_len,
+                                     float scale, uint32_t n_splits, float* out) {
+    if (!ctx || !q || !k || !v || !out) return CERA_HIP_ERR_ARGUMENT;
+    if (seq_len == 0 || n_kv_heads == 0 || head_dim == 0) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "attn_decode: empty input");
+    const uint64_t kv_dim = static_cast<uint64_t>(n_kv_heads) * head_dim;
+    const uint64_t kv_bytes = seq_len * kv_dim * 4;
+    // time-major [pos][kv_dim] (reference layout) -> head-major [kv_head][pos][head_dim]
+    std::vector<float> hk(seq_len * kv_dim), hv(seq_len * kv_dim);
+    for (uint64_t t = 0; t < seq_len; ++t)
+        for (uint32_t h = 0; h < n_kv_heads; ++h) {
+            std::memcpy(&hk[(h * seq_len + t) * head_dim], k + t * kv_dim + h * head_dim, head_dim * 4);
+            std::memcpy(&hv[(h * seq_len + t) * head_dim], v + t * kv_dim + h * head_dim, head_dim * 4);
+        }
+    void *dq, *dk, *dv, *dout;
+    CERA_TRY(cera_scratch(ctx, 0, static_cast<uint64_t>(n_heads) * head_dim * 4, &dq));
+    CERA_TRY(cera_scratch(ctx, 5, kv_bytes, &dk));
+    CERA_TRY(cera_scratch(ctx, 6, kv_bytes, &dv));
+    CERA_TRY(cera_scratch(ctx, 3, static_cast<uint64_t>(n_heads) * head_dim * 4, &dout));
+    CERA_TRY(cera_hip_upload(ctx, dq, q, static_cast<uint64_t>(n_heads) * head_dim * 4));
+    CERA_TRY(cera_hip_upload(ctx, dk, hk.data(), kv_bytes));
+    CERA_TRY(cera_hip_upload(ctx, dv, hv.data(), kv_bytes));
+    CERA_TRY(cera_launch_attn_decode(ctx, static_cast<float*>(dq), static_cast<float*>(dk), static_cast<float*>(dv),
+                                     n_heads, n_kv_heads, head_dim, seq_len, seq_len, scale, n_splits,
+                                     static_cast<float*>(dout), nullptr, nullptr));
+    CERA_TRY(cera_hip_download(ctx, out, dout, static_cast<uint64_t>(n_heads) * head_dim * 4));
+    return CERA_HIP_OK;
+}
+
+cera_hip_status cera_hip_rmsnorm(cera_hip_ctx* ctx, const float* x, const float* weight, uint64_t n, float eps, float* y) {
+    if (!ctx || !x || !weight || !y) return CERA_HIP_ERR_ARGUMENT;
+    if (n == 0 || n % 4 || n > 0xFFFFFFFFull) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "rmsnorm: n must be a positive multiple of 4");
+    void *dx, *dw, *dy;
+    CERA_TRY(cera_scratch(ctx, 0, n * 4, &dx));
+    CERA_TRY(cera_scratch(ctx, 1, n * 4, &dw));
+    CERA_TRY(cera_scratch(ctx, 3, n * 4, &dy));
+    CERA_TRY(cera_hip_upload(ctx, dx, x, n * 4));
+    CERA_TRY(cera_hip_upload(ctx, dw, weight, n * 4));
+    hipLaunchKernelGGL((rmsnorm_kernel<false>), dim3(1), dim3(256), 0, ctx->stream, static_cast<float*>(dx),
+                       static_cast<float*>(dw), static_cast<uint32_t>(n), eps, static_cast<float*>(dy), nullptr, nullptr);
+    HIP_TRY(ctx, hipGetLastError());
+    return cera_hip_download(ctx, y, dy, n * 4);
+}
+
+cera_hip_status cera_hip_silu_mul(cera_hip_ctx* ctx, const float* gate, const float* up, uint64_t n, float* out) {
+    if (!ctx || !gate || !up || !out) return CERA_HIP_ERR_ARGUMENT;
+    if (n == 0 || n % 4) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "silu_mul: n must be a positive multiple of 4");
+    void *dg, *du, *dy;
+    CERA_TRY(cera_scratch(ctx, 0, n * 4, &dg));
+    CERA_TRY(cera_scratch(ctx, 1, n * 4, &du));
+    CERA_TRY(cera_scratch(ctx, 3, n * 4, &dy));
+    CERA_TRY(cera_hip_upload(ctx, dg, gate, n * 4));
+    CERA_TRY(cera_hip_upload(ctx, du, up, n * 4));
+    hipLaunchKernelGGL((silu_mul_kernel<false>), dim3(static_cast<uint32_t>((n / 4 + 255) / 256)), dim3(256), 0,
+                       ctx->stream, static_cast<float*>(dg), static_cast<float*>(du), n, static_cast<float*>(dy),
+                       nullptr, nullptr);
+    HIP_TRY(ctx, hipGetLastError());
+    return cera_hip_download(ctx, out, dy, n * 4);
+}
+
+cera_hip_status cera_hip_argmax(cera_hip_ctx* ctx, const float* logits, uint64_t n, uint32_t* index) {
+    if (!ctx || !index || (!logits && n)) return CERA_HIP_ERR_ARGUMENT;
+    if (n > 0xFFFFFFFFull) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "argmax: n exceeds 2^32");
+    if (n == 0) { *index = 0; return CERA_HIP_OK; }
+    void *dx, *di;
+    CERA_TRY(cera_scratch(ctx, 0, n * 4, &dx));
+    CERA_TRY(cera_scratch(ctx, 1, 4, &di));
+    CERA_TRY(cera_hip_upload(ctx, dx, logits, n * 4));
+    hipLaunchKernelGGL(argmax_kernel, dim3(1), dim3(1024), 0, ctx->stream, static_cast<float*>(dx),
+                       static_cast<uint32_t>(n), static_cast<uint32_t*>(di));
+    HIP_TRY(ctx, hipGetLastError());
+    return cera_hip_download(ctx, index, di, 4);
+}
+
+cera_hip_status cera_hip_dequantize_row(cera_hip_ctx* ctx, const cera_hip_tensor* t, uint64_t row, float* out) {
+    if (!ctx || !out) return CERA_HIP_ERR_ARGUMENT;
+    uint64_t rb;
+    CERA_TRY(check_tensor(ctx, t, &rb));
+    if (row >= t->m) return cera_fail(ctx, CERA_HIP_ERR_ARGUMENT, "dequantize_row: row index out of range");
+    void *dw, *dy, *dt;
+    CERA_TRY(cera_scratch(ctx, 0, rb, &dw));
+    CERA_TRY(cera_scratch(ctx, 3, t->k * 4, &dy));
+    CERA_TRY(cera_scratch(ctx, 1, 4, &dt));
+    CERA_TRY(cera_hip_upload(ctx, dw, static_cast<const uint8_t*>(t->data) + row * rb, rb));
+    uint32_t zero = 0;
+    CERA_TRY(cera_hip_upload(ctx, dt, &zero, 4));
+    hipLaunchKernelGGL(embed_row_kernel, dim3(static_cast<uint32_t>((t->k + 255) / 256)), dim3(256), 0, ctx->stream,
+                       t->ggml_type, static_cast<uint8_t*>(dw), rb, static_cast<uint32_t*>(dt),
+                       static_cast<uint32_t>(t->k), 1.0f, static_cast<float*>(dy));
+    HIP_TRY(ctx, hipGetLastError());
+    return cera_hip_download(ctx, out, dy, t->k * 4);
+}
+
+}  // extern "C"

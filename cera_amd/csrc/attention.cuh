@@ -1,0 +1,207 @@
+// GQA flash-decode attention for one new query token, split-K over context.
+//
+// Semantics (cera/src/model/transformer.rs:1164-1305, cera/src/backend/cpu.rs:
+// 3222-3363, 2617-2633): per query head h, s[t] = (q_h . K[t]) * scale over all
+// cached positions of kv head h / group, p = softmax(s), out_h = sum_t p[t] V[t].
+// The CPU computes a global max and a single softmax; this kernel computes the
+// same quantity with the online-softmax recurrence over chunks of 64 positions
+// and merges partial (max, sum, acc) triples, which agrees to f32 rounding.
+//
+// KV cache layout in HBM: [kv_head][max_seq][head_dim] f32 (head-major), so a
+// wavefront streams one contiguous region.  head_dim is 128 and the group
+// size G = n_heads / n_kv_heads is a template parameter: all G query heads of
+// a kv head are served by one pass over its K/V (4x fewer bytes than per-head
+// passes for Llama-3's 32/8 heads).
+//
+// Work split: part = one wavefront = `chunks_per_part` chunks of 64 positions.
+// Eight lanes share a position (16 floats each, as four float4 spaced 128 B
+// apart so every load instruction covers whole 128-byte lines); a wavefront
+// covers 8 positions per step and 64 per chunk.  The P.V accumulation keeps
+// positions lane-local (lane group g accumulates positions == g mod 8), so the
+// only cross-lane traffic is the 3-step reduction of the q.k partials and one
+// reduction at the end of the part.
+#pragma once
+#include "common.cuh"
+#include "quantize.cuh"
+
+#define ATTN_HD 128
+#define ATTN_CHUNK 64
+
+struct AttnPart {  // per (part, query head): running max, sum and unnormalised output
+    float m, l;
+};
+
+template <int G>
+__global__ __launch_bounds__(256) void attn_decode_partial_kernel(
+    const float* __restrict__ q,       // [n_heads][128]
+    const float* __restrict__ kc,      // [n_kv][max_seq][128]
+    const float* __restrict__ vc,
+    uint32_t seq_len, uint32_t max_seq, float scale, uint32_t chunks_per_part, uint32_t n_parts,
+    float* __restrict__ part_acc,      // [n_kv][n_parts][G][128]
+    float* __restrict__ part_ml) {     // [n_kv][n_parts][G][2]
+    const uint32_t lane = threadIdx.x & 63;
+    const uint32_t part = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    const uint32_t kvh = blockIdx.y;
+    if (part >= n_parts) return;
+    const uint32_t j = lane & 7, pg = lane >> 3;  // float4 column group, position group
+
+    // this lane's 16 q values for each of the G heads
+    float4 qv[G][4];
+#pragma unroll
+    for (int h = 0; h < G; ++h)
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+            qv[h][c] = reinterpret_cast<const float4*>(q + (kvh * G + h) * ATTN_HD)[j + 8 * c];
+
+    float4 acc[G][4];
+    float m[G], l[G];
+#pragma unroll
+    for (int h = 0; h < G; ++h) {
+        m[h] = -__builtin_inff();
+        l[h] = 0.0f;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) acc[h][c] = make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+
+    const float* kbase = kc + static_cast<uint64_t>(kvh) * max_seq * ATTN_HD;
+    const float* vbase = vc + static_cast<uint64_t>(kvh) * max_seq * ATTN_HD;
+    const uint32_t t_begin = part * chunks_per_part * ATTN_CHUNK;
+    const uint32_t t_end = min(seq_len, t_begin + chunks_per_part * ATTN_CHUNK);
+
+    for (uint32_t t0 = t_begin; t0 < t_end; t0 += ATTN_CHUNK) {
+        // ---- scores for 64 positions: step s covers positions t0 + 8s + pg
+        float sc[G][8];
+#pragma unroll
+        for (int s = 0; s < 8; ++s) {
+            uint32_t t = t0 + 8 * s + pg;
+            bool live = t < t_end;
+            const float4* kp = reinterpret_cast<const float4*>(kbase + static_cast<uint64_t>(live ? t : t_begin) * ATTN_HD);
+            float4 kv[4];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) kv[c] = kp[j + 8 * c];
+#pragma unroll
+            for (int h = 0; h < G; ++h) {
+                float d = 0.0f;
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    d = fmaf(qv[h][c].x, kv[c].x, d);
+                    d = fmaf(qv[h][c].y, kv[c].y, d);
+                    d = fmaf(qv[h][c].z, kv[c].z, d);
+                    d = fmaf(qv[h][c].w, kv[c].w, d);
+                }
+                d += dpp_f<0xB1>(d);
+                d += dpp_f<0x4E>(d);
+                d += dpp_f<0x141>(d);
+                sc[h][s] = live ? d * scale : -__builtin_inff();
+            }
+        }
+        // ---- online softmax update per head
+        float corr[G];
+#pragma unroll
+        for (int h = 0; h < G; ++h) {
+            float mx = sc[h][0];
+#pragma unroll
+            for (int s = 1; s < 8; ++s) mx = fmaxf(mx, sc[h][s]);
+            mx = wave_max(mx);
+            float m_new = fmaxf(m[h], mx);
+            corr[h] = cera_expf(m[h] - m_new);  // 0 on the first chunk (m = -inf)
+            m[h] = m_new;
+            l[h] *= corr[h];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                acc[h][c].x *= corr[h]; acc[h][c].y *= corr[h];
+                acc[h][c].z *= corr[h]; acc[h][c].w *= corr[h];
+            }
+        }
+        // ---- P.V: this lane's positions, its 16 columns
+#pragma unroll
+        for (int s = 0; s < 8; ++s) {
+            uint32_t t = t0 + 8 * s + pg;
+            bool live = t < t_end;
+            const float4* vp = reinterpret_cast<const float4*>(vbase + static_cast<uint64_t>(live ? t : t_begin) * ATTN_HD);
+            float4 vv[4];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) vv[c] = vp[j + 8 * c];
+#pragma unroll
+            for (int h = 0; h < G; ++h) {
+                float p = cera_expf(sc[h][s] - m[h]);  // -inf score -> 0
+                // all 8 lanes of a position add the same p; count it once (lane j == 0)
+                l[h] += (j == 0) ? p : 0.0f;
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    acc[h][c].x = fmaf(p, vv[c].x, acc[h][c].x);
+                    acc[h][c].y = fmaf(p, vv[c].y, acc[h][c].y);
+                    acc[h][c].z = fmaf(p, vv[c].z, acc[h][c].z);
+                    acc[h][c].w = fmaf(p, vv[c].w, acc[h][c].w);
+                }
+            }
+        }
+    }
+
+    // ---- fold the 8 position groups (lanes differing in bits 3..5) together
+#pragma unroll
+    for (int h = 0; h < G; ++h) {
+        l[h] = wave_sum(l[h]);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            float* f = reinterpret_cast<float*>(&acc[h][c]);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                float v = f[e];
+                v += __shfl_xor(v, 8, 64);
+                v += __shfl_xor(v, 16, 64);
+                v += __shfl_xor(v, 32, 64);
+                f[e] = v;
+            }
+        }
+    }
+    if (pg == 0) {
+        uint64_t base = (static_cast<uint64_t>(kvh) * n_parts + part) * G;
+#pragma unroll
+        for (int h = 0; h < G; ++h) {
+            float4* dst = reinterpret_cast<float4*>(part_acc + (base + h) * ATTN_HD);
+#pragma unroll
+            for (int c = 0; c < 4; ++c) dst[j + 8 * c] = acc[h][c];
+            if (j == 0) {
+                part_ml[(base + h) * 2] = m[h];
+                part_ml[(base + h) * 2 + 1] = l[h];
+            }
+        }
+    }
+}
+
+// Merge the parts of one query head: out = sum_p e^{m_p - M} acc_p / sum_p e^{m_p - M} l_p.
+// 32 threads per head (a float4 of the 128 columns each).  Optionally writes
+// the Q8_0 quantisation of the result for the output projection.
+template <bool QUANT>
+__global__ __launch_bounds__(64) void attn_decode_merge_kernel(const float* __restrict__ part_acc,
+                                                               const float* __restrict__ part_ml,
+                                                               uint32_t n_parts, uint32_t G,
+                                                               float* __restrict__ out,
+                                                               float* __restrict__ scales,
+                                                               int8_t* __restrict__ quants) {
+    const uint32_t head = blockIdx.x * 2 + (threadIdx.x >> 5), c = threadIdx.x & 31;
+    const uint32_t kvh = head / G, hg = head % G;
+    float M = -__builtin_inff();
+    for (uint32_t p = 0; p < n_parts; ++p)
+        M = fmaxf(M, part_ml[((static_cast<uint64_t>(kvh) * n_parts + p) * G + hg) * 2]);
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    float L = 0.0f;
+    for (uint32_t p = 0; p < n_parts; ++p) {
+        uint64_t idx = (static_cast<uint64_t>(kvh) * n_parts + p) * G + hg;
+        float w = cera_expf(part_ml[idx * 2] - M);
+        L = fmaf(w, part_ml[idx * 2 + 1], L);
+        float4 a = reinterpret_cast<const float4*>(part_acc + idx * ATTN_HD)[c];
+        acc.x = fmaf(w, a.x, acc.x); acc.y = fmaf(w, a.y, acc.y);
+        acc.z = fmaf(w, a.z, acc.z); acc.w = fmaf(w, a.w, acc.w);
+    }
+    float inv = 1.0f / L;
+    float4 o = make_float4(acc.x * inv, acc.y * inv, acc.z * inv, acc.w * inv);
+    reinterpret_cast<float4*>(out + head * ATTN_HD)[c] = o;
+    if (QUANT) {
+        float sc;
+        uint32_t packed = q8_quantize_quad(o, sc);
+        reinterpret_cast<uint32_t*>(quants)[head * 32 + c] = packed;
+        if ((c & 7) == 0) scales[head * 4 + (c >> 3)] = sc;
+    }
+}

@@ -1,0 +1,100 @@
+// Device-side helpers shared by the gfx950 kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#define WAVE 64
+
+// ---- unaligned global loads ------------------------------------------------
+// GGUF blocks of 18/34/210 bytes are only 2-byte aligned inside a row, and
+// 20-byte blocks 4-byte aligned.  gfx950 global loads accept any alignment;
+// these typedefs tell the compiler the true (small) alignment so it still
+// emits one wide load instead of byte loads.
+typedef uint32_t u32_a2 __attribute__((aligned(2)));
+typedef uint2 uint2_a2 __attribute__((aligned(2)));
+typedef uint4 uint4_a2 __attribute__((aligned(2)));
+typedef uint4 uint4_a4 __attribute__((aligned(4)));
+typedef uint2 uint2_a4 __attribute__((aligned(4)));
+
+__device__ __forceinline__ uint32_t ld_u32_a2(const uint8_t* p) { return *reinterpret_cast<const u32_a2*>(p); }
+__device__ __forceinline__ uint2 ld_u64_a2(const uint8_t* p) { return *reinterpret_cast<const uint2_a2*>(p); }
+__device__ __forceinline__ uint4 ld_u128_a2(const uint8_t* p) { return *reinterpret_cast<const uint4_a2*>(p); }
+__device__ __forceinline__ uint4 ld_u128_a4(const uint8_t* p) { return *reinterpret_cast<const uint4_a4*>(p); }
+__device__ __forceinline__ uint4 ld_u128(const uint8_t* p) { return *reinterpret_cast<const uint4*>(p); }
+__device__ __forceinline__ uint32_t ld_u16(const uint8_t* p) { return *reinterpret_cast<const uint16_t*>(p); }
+
+// IEEE half bits -> float (v_cvt_f32_f16).
+__device__ __forceinline__ float h2f(uint32_t bits16) {
+    return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(bits16)));
+}
+// float -> IEEE half bits, round to nearest even (v_cvt_f16_f32).
+__device__ __forceinline__ uint32_t f2h(float v) {
+    return __builtin_bit_cast(uint16_t, static_cast<_Float16>(v));
+}
+
+// 4 x int8 dot with int32 accumulate (v_dot4_i32_i8).
+__device__ __forceinline__ int dot4(uint32_t a, uint32_t b, int c) {
+    return __builtin_amdgcn_sdot4(static_cast<int>(a), static_cast<int>(b), c, false);
+}
+// sum of the four signed bytes of a
+__device__ __forceinline__ int sum4(uint32_t a, int c) { return dot4(a, 0x01010101u, c); }
+
+// ---- wavefront reductions (DPP; gfx9 row/bank semantics) --------------------
+template <int CTRL, int ROW_MASK = 0xF>
+__device__ __forceinline__ float dpp_f(float v) {
+    return __builtin_bit_cast(
+        float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xF, true));
+}
+// Sum over the 64 lanes; the total is returned in every lane.
+__device__ __forceinline__ float wave_sum(float v) {
+    v += dpp_f<0xB1>(v);   // quad_perm [1,0,3,2]
+    v += dpp_f<0x4E>(v);   // quad_perm [2,3,0,1]
+    v += dpp_f<0x141>(v);  // row_half_mirror
+    v += dpp_f<0x140>(v);  // row_mirror: every lane of a 16-lane row holds the row sum
+    float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 0));
+    float r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 16));
+    float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 32));
+    float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 48));
+    return (r0 + r1) + (r2 + r3);
+}
+__device__ __forceinline__ float wave_max(float v) {
+    v = fmaxf(v, dpp_f<0xB1>(v));
+    v = fmaxf(v, dpp_f<0x4E>(v));
+    v = fmaxf(v, dpp_f<0x141>(v));
+    v = fmaxf(v, dpp_f<0x140>(v));
+    float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 0));
+    float r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 16));
+    float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 32));
+    float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 48));
+    return fmaxf(fmaxf(r0, r1), fmaxf(r2, r3));
+}
+
+// ggml's polynomial expf as cera uses it (cera/src/backend/cpu.rs:2504-2544),
+// evaluated without FMA contraction so it rounds exactly like the CPU path.
+__device__ __forceinline__ float cera_expf(float x) {
+    const float R = __builtin_bit_cast(float, 0x4B400000u);
+    const float LOG2E = __builtin_bit_cast(float, 0x3FB8AA3Bu);
+    const float LN2_HI = __builtin_bit_cast(float, 0x3F317200u);
+    const float LN2_LO = __builtin_bit_cast(float, 0x35BFBE8Eu);
+    const float C1 = __builtin_bit_cast(float, 0x3F7FFFF6u);
+    const float C2 = __builtin_bit_cast(float, 0x3EFFFEDBu);
+    const float C3 = __builtin_bit_cast(float, 0x3E2AAF33u);
+    const float C4 = __builtin_bit_cast(float, 0x3D2B9F17u);
+    const float C5 = __builtin_bit_cast(float, 0x3C072010u);
+    float z = __fadd_rn(R, __fmul_rn(x, LOG2E));
+    float n = __fsub_rn(z, R);
+    float b = __fsub_rn(__fsub_rn(x, __fmul_rn(n, LN2_HI)), __fmul_rn(n, LN2_LO));
+    uint32_t e = __builtin_bit_cast(uint32_t, z) << 23;
+    float k = __builtin_bit_cast(float, e + 0x3F800000u);
+    float u = __fmul_rn(b, b);
+    float t45 = __fadd_rn(C4, __fmul_rn(C5, b));
+    float t23 = __fadd_rn(C2, __fmul_rn(C3, b));
+    float j = __fadd_rn(__fmul_rn(C1, b), __fmul_rn(__fadd_rn(t23, __fmul_rn(t45, u)), u));
+    float abs_n = fabsf(n);
+    if (abs_n <= 126.0f) return __fadd_rn(k, __fmul_rn(j, k));
+    if (abs_n > 192.0f) return n > 0.0f ? __builtin_inff() : 0.0f;
+    uint32_t d = n <= 0.0f ? 0x82000000u : 0u;
+    float s1 = __builtin_bit_cast(float, d + 0x7f000000u);
+    float s2 = __builtin_bit_cast(float, e - d);
+    return __fmul_rn(__fadd_rn(s2, __fmul_rn(s2, j)), s1);
+}

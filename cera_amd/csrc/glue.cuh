@@ -1,0 +1,244 @@
+// Small per-token kernels between the GEMVs: embedding row lookup, RMSNorm
+// (+ Q8_0 quantize), RoPE + KV-cache append, SiLU*mul (+ quantize), argmax.
+// All of them mirror cera's scalar CPU code operation by operation
+// (cera/src/backend/cpu.rs) so that their f32 outputs match it bit for bit
+// wherever the CPU order is a plain elementwise expression.
+#pragma once
+#include "common.cuh"
+#include "quantize.cuh"
+
+// ---------------------------------------------------------------------------
+// Row dequantisation (cera/src/quant.rs:364-886 via
+// cera/src/model/transformer.rs:949-1017): out[k] = dequant(row).  One thread
+// per element; runs once per token for the embedding lookup.
+__device__ __forceinline__ float dequant_elem(uint32_t dtype, const uint8_t* row, uint32_t e) {
+    switch (dtype) {
+        case 0: return reinterpret_cast<const float*>(row)[e];
+        case 1: return h2f(reinterpret_cast<const uint16_t*>(row)[e]);
+        case 30: {
+            uint32_t b = reinterpret_cast<const uint16_t*>(row)[e];
+            uint32_t quiet = ((b & 0x7FFF) > 0x7F80) ? 0x00400000u : 0u;
+            return __builtin_bit_cast(float, (b << 16) | quiet);
+        }
+        case 2: {  // Q4_0
+            const uint8_t* blk = row + (e >> 5) * 18;
+            uint32_t i = e & 31, byte = blk[2 + (i & 15)];
+            int q = static_cast<int>(i < 16 ? (byte & 0xF) : (byte >> 4)) - 8;
+            return static_cast<float>(q) * h2f(ld_u16(blk));
+        }
+        case 3: {  // Q4_1
+            const uint8_t* blk = row + (e >> 5) * 20;
+            uint32_t i = e & 31, byte = blk[4 + (i & 15)];
+            uint32_t q = i < 16 ? (byte & 0xF) : (byte >> 4);
+            return __fadd_rn(__fmul_rn(static_cast<float>(q), h2f(ld_u16(blk))), h2f(ld_u16(blk + 2)));
+        }
+        case 8: {  // Q8_0
+            const uint8_t* blk = row + (e >> 5) * 34;
+            return static_cast<float>(static_cast<int8_t>(blk[2 + (e & 31)])) * h2f(ld_u16(blk));
+        }
+        case 12:
+        case 13: {  // Q4_K / Q5_K
+            const bool q5 = dtype == 13;
+            const uint8_t* blk = row + (e >> 8) * (q5 ? 176 : 144);
+            uint32_t i = e & 255, s = i >> 5, l = i & 31, j = s >> 1;
+            const uint8_t* sc12 = blk + 4;
+            uint32_t sc, mn;
+            if (s < 4) {
+                sc = sc12[s] & 63;
+                mn = sc12[s + 4] & 63;
+            } else {
+                sc = (sc12[s + 4] & 0xF) | ((sc12[s - 4] >> 6) << 4);
+                mn = (sc12[s + 4] >> 4) | ((sc12[s] >> 6) << 4);
+            }
+            uint32_t byte = blk[(q5 ? 48 : 16) + 32 * j + l];
+            float q = static_cast<float>((s & 1) ? (byte >> 4) : (byte & 0xF));
+            if (q5 && ((blk[16 + l] >> s) & 1)) q = __fadd_rn(q, 16.0f);
+            float d = h2f(ld_u16(blk)), dmin = h2f(ld_u16(blk + 2));
+            return __fsub_rn(__fmul_rn(__fmul_rn(d, static_cast<float>(sc)), q),
+                             __fmul_rn(dmin, static_cast<float>(mn)));
+        }
+        case 14: {  // Q6_K
+            const uint8_t* blk = row + (e >> 8) * 210;
+            uint32_t i = e & 255, n = i >> 7, r = i & 127, t = r >> 5, l = r & 31;
+            uint32_t ql = blk[64 * n + (t & 1) * 32 + l];
+            uint32_t nib = t < 2 ? (ql & 0xF) : (ql >> 4);
+            uint32_t h2 = (blk[128 + 32 * n + l] >> (2 * t)) & 3;
+            int q = static_cast<int>(nib | (h2 << 4)) - 32;
+            float sc = static_cast<float>(static_cast<int8_t>(blk[192 + 8 * n + (l >> 4) + 2 * t]));
+            return __fmul_rn(__fmul_rn(h2f(ld_u16(blk + 208)), sc), static_cast<float>(q));
+        }
+        default: return 0.0f;
+    }
+}
+
+// token comes from device memory so a graph-captured decode step can chain on
+// the previous step's argmax without a host round trip.
+static __global__ void embed_row_kernel(uint32_t dtype, const uint8_t* __restrict__ w, uint64_t row_bytes,
+                                 const uint32_t* __restrict__ token, uint32_t k, float scale,
+                                 float* __restrict__ out) {
+    uint32_t e = blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= k) return;
+    float v = dequant_elem(dtype, w + static_cast<uint64_t>(*token) * row_bytes, e);
+    out[e] = scale != 1.0f ? __fmul_rn(v, scale) : v;
+}
+
+// ---------------------------------------------------------------------------
+// RMSNorm (cera/src/backend/cpu.rs:2479-2496): f64 sum of squares,
+// inv = (1/sqrt(mean + eps)) as f32, y = (x*inv)*w.  One 256-thread block per
+// row of n elements; optionally also emits the Q8_0 quantisation of y.
+// The f64 sum is a tree instead of the CPU's serial chain: f64 rounding
+// differences (~1e-16 relative) vanish when inv is narrowed to f32 except in
+// astronomically rare double-rounding cases.
+template <bool QUANT>
+static __global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                                                      uint32_t n, float eps, float* __restrict__ y,
+                                                      float* __restrict__ scales, int8_t* __restrict__ quants) {
+    __shared__ double part[4];
+    const float* xr = x + static_cast<uint64_t>(blockIdx.x) * n;
+    float* yr = y + static_cast<uint64_t>(blockIdx.x) * n;
+    double s = 0.0;
+    for (uint32_t i = threadIdx.x * 4; i < n; i += 1024) {
+        float4 v = *reinterpret_cast<const float4*>(xr + i);
+        s += static_cast<double>(v.x) * v.x;
+        s += static_cast<double>(v.y) * v.y;
+        s += static_cast<double>(v.z) * v.z;
+        s += static_cast<double>(v.w) * v.w;
+    }
+    for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = s;
+    __syncthreads();
+    double tot = (part[0] + part[1]) + (part[2] + part[3]);
+    double mean = tot / static_cast<double>(n);
+    float inv = static_cast<float>(1.0 / sqrt(mean + static_cast<double>(eps)));
+    for (uint32_t i = threadIdx.x * 4; i < n; i += 1024) {
+        float4 v = *reinterpret_cast<const float4*>(xr + i);
+        float4 g = *reinterpret_cast<const float4*>(w + i);
+        float4 o;
+        o.x = __fmul_rn(__fmul_rn(v.x, inv), g.x);
+        o.y = __fmul_rn(__fmul_rn(v.y, inv), g.y);
+        o.z = __fmul_rn(__fmul_rn(v.z, inv), g.z);
+        o.w = __fmul_rn(__fmul_rn(v.w, inv), g.w);
+        *reinterpret_cast<float4*>(yr + i) = o;
+        if (QUANT) {
+            // n % 32 == 0 and i advances in float4 steps: the 8 lanes of a block stay together
+            float sc;
+            uint32_t packed = q8_quantize_quad(o, sc);
+            uint64_t e = static_cast<uint64_t>(blockIdx.x) * n + i;
+            reinterpret_cast<uint32_t*>(quants)[e >> 2] = packed;
+            if ((threadIdx.x & 7) == 0) scales[e >> 5] = sc;
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// RoPE on q and k in place + append k, v to the head-major KV cache.
+// cos/sin come from a host-built table [max_seq][head_dim/2] computed with the
+// same libm calls and the same iterated f32 theta as the CPU path
+// (cera/src/backend/cpu.rs:5031-5045 NEOX, :5161-5180 NORM), so rotated values
+// are bit-identical to it.  grid = n_heads + 2*n_kv_heads blocks of head_dim/2
+// threads: blocks [0, n_heads) rotate q; the next n_kv_heads rotate k and
+// store it; the last n_kv_heads copy v.
+// KV cache layout: [kv_head][max_seq][head_dim] f32.
+static __global__ void rope_kv_kernel(float* __restrict__ q, float* __restrict__ k, const float* __restrict__ v,
+                               const float* __restrict__ cs_table, const uint32_t* __restrict__ pos_ptr,
+                               uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, uint32_t rope_type,
+                               float* __restrict__ k_cache, float* __restrict__ v_cache, uint32_t max_seq) {
+    const uint32_t pos = *pos_ptr;
+    const uint32_t half = head_dim / 2, i = threadIdx.x, b = blockIdx.x;
+    if (b < n_heads + n_kv_heads) {
+        float* head = b < n_heads ? q + b * head_dim : k + (b - n_heads) * head_dim;
+        float2 cs = reinterpret_cast<const float2*>(cs_table)[static_cast<uint64_t>(pos) * half + i];
+        uint32_t i0 = rope_type == 1 ? 2 * i : i, i1 = rope_type == 1 ? 2 * i + 1 : i + half;
+        float x0 = head[i0], x1 = head[i1];
+        float r0 = __fsub_rn(__fmul_rn(x0, cs.x), __fmul_rn(x1, cs.y));
+        float r1 = __fadd_rn(__fmul_rn(x0, cs.y), __fmul_rn(x1, cs.x));
+        head[i0] = r0;
+        head[i1] = r1;
+        if (b >= n_heads && k_cache) {
+            float* dst = k_cache + (static_cast<uint64_t>(b - n_heads) * max_seq + pos) * head_dim;
+            dst[i0] = r0;
+            dst[i1] = r1;
+        }
+    } else if (v_cache) {
+        uint32_t h = b - n_heads - n_kv_heads;
+        float* dst = v_cache + (static_cast<uint64_t>(h) * max_seq + pos) * head_dim;
+        dst[2 * i] = v[h * head_dim + 2 * i];
+        dst[2 * i + 1] = v[h * head_dim + 2 * i + 1];
+    }
+}
+
+// out = a + b (cera/src/backend/cpu.rs:5223-5228), optional scale on b first.
+static __global__ void add_kernel(const float* __restrict__ a, const float* __restrict__ b, float bscale, uint32_t n,
+                           float* __restrict__ out) {
+    uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    float t = bscale != 1.0f ? __fmul_rn(b[i], bscale) : b[i];
+    out[i] = __fadd_rn(a[i], t);
+}
+
+// bias add in place: x[i] += b[i]
+static __global__ void bias_kernel(float* __restrict__ x, const float* __restrict__ b, uint32_t n) {
+    uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) x[i] = __fadd_rn(x[i], b[i]);
+}
+static __global__ void scale_kernel(float* __restrict__ x, float s, uint32_t n) {
+    uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) x[i] = __fmul_rn(x[i], s);
+}
+
+// SiLU(gate)*up (cera/src/backend/cpu.rs:2570-2575) with optional Q8_0
+// quantisation of the result (the activation of the down projection).
+template <bool QUANT>
+static __global__ __launch_bounds__(256) void silu_mul_kernel(const float* __restrict__ gate, const float* __restrict__ up,
+                                                       uint64_t n, float* __restrict__ out,
+                                                       float* __restrict__ scales, int8_t* __restrict__ quants) {
+    uint64_t t = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    bool live = 4 * t < n;
+    float4 g = live ? reinterpret_cast<const float4*>(gate)[t] : make_float4(0, 0, 0, 0);
+    float4 u = live ? reinterpret_cast<const float4*>(up)[t] : make_float4(0, 0, 0, 0);
+    float4 o;
+    o.x = __fmul_rn(__fdiv_rn(g.x, __fadd_rn(1.0f, cera_expf(-g.x))), u.x);
+    o.y = __fmul_rn(__fdiv_rn(g.y, __fadd_rn(1.0f, cera_expf(-g.y))), u.y);
+    o.z = __fmul_rn(__fdiv_rn(g.z, __fadd_rn(1.0f, cera_expf(-g.z))), u.z);
+    o.w = __fmul_rn(__fdiv_rn(g.w, __fadd_rn(1.0f, cera_expf(-g.w))), u.w);
+    if (QUANT) {
+        float sc;
+        uint32_t packed = q8_quantize_quad(o, sc);
+        if (live) {
+            reinterpret_cast<uint32_t*>(quants)[t] = packed;
+            if ((t & 7) == 0) scales[t >> 3] = sc;
+        }
+    }
+    if (live && out) reinterpret_cast<float4*>(out)[t] = o;
+}
+
+// ---------------------------------------------------------------------------
+// argmax (cera/src/sampler.rs:20-30): strict >, lowest index on ties, NaN never
+// wins, index 0 when nothing beats -inf.  Single block of 1024 threads: each
+// scans a strided slice keeping (best value, lowest index), then a tree merge
+// with the same tie rule.
+__device__ __forceinline__ void argmax_merge(float& bv, uint32_t& bi, float ov, uint32_t oi) {
+    if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+}
+static __global__ __launch_bounds__(1024) void argmax_kernel(const float* __restrict__ x, uint32_t n,
+                                                      uint32_t* __restrict__ out) {
+    __shared__ float sv[16];
+    __shared__ uint32_t si[16];
+    float bv = -__builtin_inff();
+    uint32_t bi = 0xFFFFFFFFu;  // "no candidate yet": loses every tie
+    for (uint32_t i = threadIdx.x; i < n; i += 1024) {
+        float v = x[i];
+        if (v > bv) { bv = v; bi = i; }
+    }
+    for (int off = 32; off > 0; off >>= 1) {
+        float ov = __shfl_xor(bv, off, 64);
+        uint32_t oi = __shfl_xor(bi, off, 64);
+        argmax_merge(bv, bi, ov, oi);
+    }
+    if ((threadIdx.x & 63) == 0) { sv[threadIdx.x >> 6] = bv; si[threadIdx.x >> 6] = bi; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < 16; ++w) argmax_merge(bv, bi, sv[w], si[w]);
+        *out = bi == 0xFFFFFFFFu ? 0u : bi;
+    }
+}

@@ -1,0 +1,69 @@
+// Host-side types shared by the C-ABI translation units.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "cera_hip.h"
+
+struct cera_hip_event {
+    hipEvent_t ev = nullptr;
+};
+
+struct cera_hip_dtensor {
+    uint32_t dtype = 0;
+    uint64_t m = 0, k = 0;
+    uint64_t row_bytes = 0, nbytes = 0;
+    uint8_t* dev = nullptr;
+};
+
+struct cera_hip_ctx {
+    int device = 0;
+    hipStream_t stream = nullptr;
+    std::string err;
+    uint32_t n_cu = 0;
+    // grow-only device scratch for the host-pointer entry points
+    void* scratch[8] = {nullptr};
+    uint64_t scratch_bytes[8] = {0};
+    // attention split-K workspace
+    float* attn_acc = nullptr;
+    float* attn_ml = nullptr;
+    uint64_t attn_acc_bytes = 0, attn_ml_bytes = 0;
+};
+
+void cera_set_global_error(const std::string& s);
+cera_hip_status cera_fail(cera_hip_ctx* ctx, cera_hip_status st, const std::string& msg);
+
+#define HIP_TRY(ctx, call)                                                                     \
+    do {                                                                                       \
+        hipError_t e_ = (call);                                                                \
+        if (e_ != hipSuccess)                                                                  \
+            return cera_fail((ctx), e_ == hipErrorOutOfMemory ? CERA_HIP_ERR_OOM : CERA_HIP_ERR_DEVICE, \
+                             std::string(#call) + ": " + hipGetErrorString(e_));               \
+    } while (0)
+
+#define CERA_TRY(expr)                          \
+    do {                                        \
+        cera_hip_status s_ = (expr);            \
+        if (s_ != CERA_HIP_OK) return s_;       \
+    } while (0)
+
+// element / byte geometry of a GGML type; false when there is no kernel for it
+bool cera_type_geometry(uint32_t t, uint32_t* block_elems, uint32_t* block_bytes);
+cera_hip_status cera_scratch(cera_hip_ctx* ctx, int slot, uint64_t nbytes, void** out);
+
+// ---- launchers (defined next to their kernels) --------------------------------
+enum CeraEpilogue { CERA_EPI_STORE = 0, CERA_EPI_ADD = 1, CERA_EPI_SILU_MUL = 2 };
+
+cera_hip_status cera_launch_quantize(cera_hip_ctx* ctx, const float* x, uint64_t k, float* scales, int8_t* quants);
+// y = W.(xs,xq) [+ resid]; w2 != null with EPI_SILU_MUL computes silu(W.x)*(W2.x)
+cera_hip_status cera_launch_gemv(cera_hip_ctx* ctx, const cera_hip_dtensor* w, const cera_hip_dtensor* w2,
+                                 const float* xs, const int8_t* xq, float* y, const float* resid, int epi,
+                                 int32_t* dbg_dots = nullptr, int32_t* dbg_asums = nullptr);
+cera_hip_status cera_launch_gemv_q5k_f32(cera_hip_ctx* ctx, const cera_hip_dtensor* w, const float* x, float* y);
+cera_hip_status cera_launch_attn_decode(cera_hip_ctx* ctx, const float* q, const float* kc, const float* vc,
+                                        uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, uint64_t seq_len,
+                                        uint64_t max_seq, float scale, uint32_t n_splits, float* out,
+                                        float* out_scales, int8_t* out_quants);

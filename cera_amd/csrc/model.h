@@ -1,0 +1,42 @@
+// Device-resident model state shared by model.hip and prefill.hip.
+#pragma once
+#include <mutex>
+#include <vector>
+
+#include "host_common.h"
+
+struct LayerDev {
+    cera_hip_dtensor *q = nullptr, *k = nullptr, *v = nullptr, *o = nullptr, *gate = nullptr, *up = nullptr,
+                     *down = nullptr;
+    float *attn_norm = nullptr, *ffn_norm = nullptr;
+    float *q_bias = nullptr, *k_bias = nullptr, *v_bias = nullptr, *q_norm = nullptr, *k_norm = nullptr;
+    float *kc = nullptr, *vc = nullptr;  // [n_kv_heads][max_seq_len][head_dim] f32
+};
+
+struct cera_hip_model {
+    cera_hip_ctx* ctx = nullptr;
+    cera_hip_config cfg{};
+    cera_hip_dtensor *embd = nullptr, *output = nullptr;
+    float* output_norm = nullptr;
+    std::vector<LayerDev> layers;
+    float* rope_table = nullptr;  // [max_seq_len][head_dim/2] (cos, sin)
+    // single-token activations
+    float *hidden = nullptr, *normed = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *attn_out = nullptr,
+          *proj = nullptr, *act = nullptr, *up = nullptr, *xs = nullptr, *logits = nullptr;
+    int8_t* xq = nullptr;
+    uint32_t* scalars = nullptr;  // device: [token, pos, argmax result, spare]
+    std::vector<void*> owned;     // plain device allocations freed with the model
+    uint32_t seq_len = 0;
+    uint64_t bytes = 0;
+    // every trait call is serialised, like the reference GPU backends' infer_lock
+    // (cera/src/model/mod.rs:184-199)
+    std::mutex infer_lock;
+};
+
+void cera_build_rope_table(uint32_t max_seq, uint32_t head_dim, float base, const float* ff, std::vector<float>& out);
+cera_hip_status cera_model_prefill_per_token(cera_hip_model* m, const uint32_t* tokens, uint32_t n, uint32_t start_pos,
+                                             float* last_logits);
+// batched route (prefill.hip); falls back to the per-token route when a weight
+// type has no int8 GEMM
+cera_hip_status cera_model_prefill(cera_hip_model* m, const uint32_t* tokens, uint32_t n, uint32_t start_pos,
+                                   float* last_logits);

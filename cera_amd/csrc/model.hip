@@ -1,0 +1,429 @@
+// C ABI, model level: a device-resident dense transformer (llama architecture)
+// driven through the `Model`-trait surface -- forward / forward_greedy /
+// forward_prefill / truncate_kv (cera/src/model/mod.rs:200-606) -- with the
+// layer graph of LlamaModel (cera/src/model/llama.rs:468-597, 1585-1649;
+// cera/src/model/transformer.rs:1313-1652).
+#include <cmath>
+#include <cstring>
+#include <new>
+
+#include "glue.cuh"
+#include "host_common.h"
+#include "model.h"
+
+// ---------------------------------------------------------------------------
+static cera_hip_status dev_alloc(cera_hip_ctx* ctx, uint64_t bytes, void** out, uint64_t* total) {
+    *out = nullptr;
+    HIP_TRY(ctx, hipMalloc(out, bytes ? bytes : 256));
+    if (total) *total += bytes;
+    return CERA_HIP_OK;
+}
+template <class T>
+static cera_hip_status dev_alloc_t(cera_hip_ctx* ctx, uint64_t n, T** out, uint64_t* total) {
+    return dev_alloc(ctx, n * sizeof(T), reinterpret_cast<void**>(out), total);
+}
+static cera_hip_status upload_f32(cera_hip_ctx* ctx, const float* host, uint64_t n, float** out, uint64_t* total) {
+    if (!host) { *out = nullptr; return CERA_HIP_OK; }
+    CERA_TRY(dev_alloc_t(ctx, n, out, total));
+    return cera_hip_upload(ctx, *out, host, n * 4);
+}
+
+// cos/sin table [max_seq][head_dim/2] built with the CPU path's own recurrence:
+// theta_scale = base^(-2/hd); theta_0 = pos as f32; theta_{i+1} = theta_i *
+// theta_scale (f32); angle = theta_i / freq_factor_i; libm sinf/cosf
+// (cera/src/backend/cpu.rs:5031-5045, 5161-5180).
+void cera_build_rope_table(uint32_t max_seq, uint32_t head_dim, float base, const float* ff, std::vector<float>& out) {
+    const uint32_t half = head_dim / 2;
+    out.resize(static_cast<size_t>(max_seq) * half * 2);
+    const float theta_scale = powf(base, -2.0f / static_cast<float>(head_dim));
+    for (uint32_t p = 0; p < max_seq; ++p) {
+        float theta = static_cast<float>(p);
+        float* row = out.data() + static_cast<size_t>(p) * half * 2;
+        for (uint32_t i = 0; i < half; ++i) {
+            float ang = ff ? theta / ff[i] : theta;
+            row[2 * i] = cosf(ang);
+            row[2 * i + 1] = sinf(ang);
+            theta *= theta_scale;
+        }
+    }
+}
+
+static void free_model(cera_hip_model* m) {
+    if (!m) return;
+    cera_hip_ctx* ctx = m->ctx;
+    (void)hipStreamSynchronize(ctx->stream);
+    auto ft = [&](cera_hip_dtensor* t) { if (t) cera_hip_tensor_free(ctx, t); };
+    for (auto& L : m->layers) {
+        ft(L.q); ft(L.k); ft(L.v); ft(L.o); ft(L.gate); ft(L.up); ft(L.down);
+        for (float* p : {L.attn_norm, L.ffn_norm, L.q_bias, L.k_bias, L.v_bias, L.q_norm, L.k_norm, L.kc, L.vc})
+            if (p) (void)hipFree(p);
+    }
+    ft(m->embd);
+    ft(m->output);
+    for (void* p : m->owned)
+        if (p) (void)hipFree(p);
+    delete m;
+}
+
+static bool gemv_type_ok(uint32_t t) {
+    return t == CERA_HIP_Q4_0 || t == CERA_HIP_Q4_1 || t == CERA_HIP_Q8_0 || t == CERA_HIP_Q4_K ||
+           t == CERA_HIP_Q5_K || t == CERA_HIP_Q6_K;
+}
+
+extern "C" cera_hip_status cera_hip_model_create(cera_hip_ctx* ctx, const cera_hip_config* cfg,
+                                                 const cera_hip_tensor* token_embd, const cera_hip_tensor* output,
+                                                 const float* output_norm, const cera_hip_layer* layers,
+                                                 cera_hip_model** out) {
+    if (!ctx || !cfg || !token_embd || !output_norm || !layers || !out) return CERA_HIP_ERR_ARGUMENT;
+    *out = nullptr;
+    const cera_hip_config& c = *cfg;
+    if (c.n_layers == 0 || c.hidden == 0 || c.ffn == 0 || c.n_heads == 0 || c.n_kv_heads == 0 || c.vocab == 0 ||
+        c.max_seq_len == 0)
+        return cera_fail(ctx, CERA_HIP_ERR_ARGUMENT, "model_create: zero dimension in config");
+    if (c.head_dim != 128) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "model_create: head_dim must be 128");
+    if (c.n_heads % c.n_kv_heads) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "model_create: n_heads % n_kv_heads != 0");
+    if (c.hidden % 32 || c.ffn % 32) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "model_create: hidden and ffn must be multiples of 32");
+    if (c.rope_type > 1) return cera_fail(ctx, CERA_HIP_ERR_ARGUMENT, "model_create: rope_type must be 0 (neox) or 1 (norm)");
+    const uint32_t q_dim = c.n_heads * c.head_dim, kv_dim = c.n_kv_heads * c.head_dim;
+
+    // shape checks before anything is uploaded: refuse, never silently skip a matmul
+    auto expect = [&](const cera_hip_tensor& t, uint64_t m, uint64_t k, const char* name, bool matmul) -> cera_hip_status {
+        if (t.m != m || t.k != k)
+            return cera_fail(ctx, CERA_HIP_ERR_SHAPE, std::string(name) + ": expected [" + std::to_string(m) + " x " +
+                                                          std::to_string(k) + "], got [" + std::to_string(t.m) + " x " +
+                                                          std::to_string(t.k) + "]");
+        if (matmul && !gemv_type_ok(t.ggml_type))
+            return cera_fail(ctx, CERA_HIP_ERR_UNSUPPORTED_DTYPE,
+                             std::string(name) + ": no hip GEMV kernel for ggml type " + std::to_string(t.ggml_type));
+        return CERA_HIP_OK;
+    };
+    CERA_TRY(expect(*token_embd, c.vocab, c.hidden, "token_embd", output == nullptr));
+    if (output) CERA_TRY(expect(*output, c.vocab, c.hidden, "output", true));
+    for (uint32_t i = 0; i < c.n_layers; ++i) {
+        const cera_hip_layer& L = layers[i];
+        if (!L.attn_norm || !L.ffn_norm) return cera_fail(ctx, CERA_HIP_ERR_ARGUMENT, "layer norm weights missing");
+        CERA_TRY(expect(L.attn_q, q_dim, c.hidden, "attn_q", true));
+        CERA_TRY(expect(L.attn_k, kv_dim, c.hidden, "attn_k", true));
+        CERA_TRY(expect(L.attn_v, kv_dim, c.hidden, "attn_v", true));
+        CERA_TRY(expect(L.attn_output, c.hidden, q_dim, "attn_output", true));
+        CERA_TRY(expect(L.ffn_gate, c.ffn, c.hidden, "ffn_gate", true));
+        CERA_TRY(expect(L.ffn_up, c.ffn, c.hidden, "ffn_up", true));
+        CERA_TRY(expect(L.ffn_down, c.hidden, c.ffn, "ffn_down", true));
+    }
+
+    cera_hip_model* m = new (std::nothrow) cera_hip_model();
+    if (!m) return cera_fail(ctx, CERA_HIP_ERR_OOM, "host allocation failed");
+    m->ctx = ctx;
+    m->cfg = c;
+    m->cfg.rope_freqs = nullptr;
+    m->layers.resize(c.n_layers);
+    uint64_t* tot = &m->bytes;
+    auto build = [&]() -> cera_hip_status {
+        CERA_TRY(cera_hip_tensor_upload(ctx, token_embd, &m->embd));
+        *tot += m->embd->nbytes;
+        if (output) {
+            CERA_TRY(cera_hip_tensor_upload(ctx, output, &m->output));
+            *tot += m->output->nbytes;
+        }
+        float* tmp;
+        CERA_TRY(upload_f32(ctx, output_norm, c.hidden, &tmp, tot));
+        m->output_norm = tmp; m->owned.push_back(tmp);
+        const uint64_t kv_elems = static_cast<uint64_t>(c.n_kv_heads) * c.max_seq_len * c.head_dim;
+        for (uint32_t i = 0; i < c.n_layers; ++i) {
+            const cera_hip_layer& L = layers[i];
+            LayerDev& D = m->layers[i];
+            const cera_hip_tensor* src[7] = {&L.attn_q, &L.attn_k, &L.attn_v, &L.attn_output, &L.ffn_gate, &L.ffn_up, &L.ffn_down};
+            cera_hip_dtensor** dst[7] = {&D.q, &D.k, &D.v, &D.o, &D.gate, &D.up, &D.down};
+            for (int t = 0; t < 7; ++t) {
+                CERA_TRY(cera_hip_tensor_upload(ctx, src[t], dst[t]));
+                *tot += (*dst[t])->nbytes;
+            }
+            CERA_TRY(upload_f32(ctx, L.attn_norm, c.hidden, &D.attn_norm, tot));
+            CERA_TRY(upload_f32(ctx, L.ffn_norm, c.hidden, &D.ffn_norm, tot));
+            if (L.q_bias && L.k_bias && L.v_bias) {
+                CERA_TRY(upload_f32(ctx, L.q_bias, q_dim, &D.q_bias, tot));
+                CERA_TRY(upload_f32(ctx, L.k_bias, kv_dim, &D.k_bias, tot));
+                CERA_TRY(upload_f32(ctx, L.v_bias, kv_dim, &D.v_bias, tot));
+            }
+            if (L.q_norm && L.k_norm) {
+                CERA_TRY(upload_f32(ctx, L.q_norm, c.head_dim, &D.q_norm, tot));
+                CERA_TRY(upload_f32(ctx, L.k_norm, c.head_dim, &D.k_norm, tot));
+            }
+            CERA_TRY(dev_alloc_t(ctx, kv_elems, &D.kc, tot));
+            CERA_TRY(dev_alloc_t(ctx, kv_elems, &D.vc, tot));
+        }
+        std::vector<float> table;
+        cera_build_rope_table(c.max_seq_len, c.head_dim, c.rope_theta, cfg->rope_freqs, table);
+        CERA_TRY(upload_f32(ctx, table.data(), table.size(), &tmp, tot));
+        m->rope_table = tmp; m->owned.push_back(tmp);
+
+        const uint64_t maxk = std::max<uint64_t>(std::max(c.hidden, c.ffn), q_dim);
+        auto af = [&](uint64_t n, float** p) -> cera_hip_status {
+            CERA_TRY(dev_alloc_t(ctx, n, p, tot));
+            m->owned.push_back(*p);
+            return CERA_HIP_OK;
+        };
+        CERA_TRY(af(c.hidden, &m->hidden));
+        CERA_TRY(af(c.hidden, &m->normed));
+        CERA_TRY(af(q_dim, &m->q));
+        CERA_TRY(af(kv_dim, &m->k));
+        CERA_TRY(af(kv_dim, &m->v));
+        CERA_TRY(af(q_dim, &m->attn_out));
+        CERA_TRY(af(c.hidden, &m->proj));
+        CERA_TRY(af(c.ffn, &m->act));
+        CERA_TRY(af(c.ffn, &m->up));
+        CERA_TRY(af(maxk / 32, &m->xs));
+        CERA_TRY(af(c.vocab, &m->logits));
+        CERA_TRY(dev_alloc_t(ctx, maxk, &m->xq, tot));
+        m->owned.push_back(m->xq);
+        CERA_TRY(dev_alloc_t(ctx, 4, &m->scalars, tot));  // [token, pos, argmax, spare]
+        m->owned.push_back(m->scalars);
+        return CERA_HIP_OK;
+    };
+    cera_hip_status st = build();
+    if (st != CERA_HIP_OK) {
+        std::string keep = ctx->err;
+        free_model(m);
+        ctx->err = keep;
+        return st;
+    }
+    *out = m;
+    return CERA_HIP_OK;
+}
+
+extern "C" void cera_hip_model_destroy(cera_hip_model* m) { free_model(m); }
+extern "C" uint32_t cera_hip_seq_len(const cera_hip_model* m) { return m ? m->seq_len : 0; }
+extern "C" uint64_t cera_hip_memory_bytes(const cera_hip_model* m) { return m ? m->bytes : 0; }
+
+extern "C" cera_hip_status cera_hip_truncate_kv(cera_hip_model* m, uint32_t len) {
+    if (!m) return CERA_HIP_ERR_ARGUMENT;
+    std::lock_guard<std::mutex> lk(m->infer_lock);
+    if (len < m->seq_len) m->seq_len = len;  // rows past len are simply overwritten later
+    return CERA_HIP_OK;
+}
+
+// ---------------------------------------------------------------------------
+// One projection: int8 kernels read the quantized activations, Q5_K the f32 ones.
+static cera_hip_status project(cera_hip_model* m, const cera_hip_dtensor* w, const float* x_f32, float* y,
+                               const float* resid) {
+    cera_hip_ctx* ctx = m->ctx;
+    const float rs = m->cfg.residual_scale;
+    if (w->dtype == CERA_HIP_Q5_K) {
+        float* dst = resid ? m->proj : y;
+        CERA_TRY(cera_launch_gemv_q5k_f32(ctx, w, x_f32, dst));
+        if (resid) {
+            hipLaunchKernelGGL(add_kernel, dim3((w->m + 255) / 256), dim3(256), 0, ctx->stream, resid, dst, rs,
+                               static_cast<uint32_t>(w->m), y);
+            HIP_TRY(ctx, hipGetLastError());
+        }
+        return CERA_HIP_OK;
+    }
+    if (resid && rs != 1.0f) {
+        CERA_TRY(cera_launch_gemv(ctx, w, nullptr, m->xs, m->xq, m->proj, nullptr, CERA_EPI_STORE));
+        hipLaunchKernelGGL(add_kernel, dim3((w->m + 255) / 256), dim3(256), 0, ctx->stream, resid, m->proj, rs,
+                           static_cast<uint32_t>(w->m), y);
+        HIP_TRY(ctx, hipGetLastError());
+        return CERA_HIP_OK;
+    }
+    return cera_launch_gemv(ctx, w, nullptr, m->xs, m->xq, y, resid, resid ? CERA_EPI_ADD : CERA_EPI_STORE);
+}
+
+static cera_hip_status norm_quant(cera_hip_model* m, const float* x, const float* w, uint32_t n, uint32_t rows, float* y) {
+    hipLaunchKernelGGL((rmsnorm_kernel<true>), dim3(rows), dim3(256), 0, m->ctx->stream, x, w, n, m->cfg.rms_eps, y,
+                       m->xs, m->xq);
+    HIP_TRY(m->ctx, hipGetLastError());
+    return CERA_HIP_OK;
+}
+
+// The per-token layer stack: LlamaModel::run_layers + project_logits.  The
+// token id and position are read by the kernels from m->scalars[0..1].
+static cera_hip_status decode_step(cera_hip_model* m, uint32_t pos, bool want_logits) {
+    cera_hip_ctx* ctx = m->ctx;
+    const cera_hip_config& c = m->cfg;
+    hipStream_t s = ctx->stream;
+    const uint32_t q_dim = c.n_heads * c.head_dim, kv_dim = c.n_kv_heads * c.head_dim;
+    const float scale = c.attn_scale != 0.0f ? c.attn_scale : 1.0f / std::sqrt(static_cast<float>(c.head_dim));
+
+    hipLaunchKernelGGL(embed_row_kernel, dim3((c.hidden + 255) / 256), dim3(256), 0, s, m->embd->dtype, m->embd->dev,
+                       m->embd->row_bytes, m->scalars, c.hidden, c.embed_scale, m->hidden);
+    HIP_TRY(ctx, hipGetLastError());
+
+    for (uint32_t i = 0; i < c.n_layers; ++i) {
+        LayerDev& L = m->layers[i];
+        CERA_TRY(norm_quant(m, m->hidden, L.attn_norm, c.hidden, 1, m->normed));
+        CERA_TRY(project(m, L.q, m->normed, m->q, nullptr));
+        CERA_TRY(project(m, L.k, m->normed, m->k, nullptr));
+        CERA_TRY(project(m, L.v, m->normed, m->v, nullptr));
+        if (L.q_bias) {
+            hipLaunchKernelGGL(bias_kernel, dim3((q_dim + 255) / 256), dim3(256), 0, s, m->q, L.q_bias, q_dim);
+            hipLaunchKernelGGL(bias_kernel, dim3((kv_dim + 255) / 256), dim3(256), 0, s, m->k, L.k_bias, kv_dim);
+            hipLaunchKernelGGL(bias_kernel, dim3((kv_dim + 255) / 256), dim3(256), 0, s, m->v, L.v_bias, kv_dim);
+        }
+        if (L.q_norm) {
+            hipLaunchKernelGGL((rmsnorm_kernel<false>), dim3(c.n_heads), dim3(256), 0, s, m->q, L.q_norm, c.head_dim,
+                               c.rms_eps, m->q, nullptr, nullptr);
+            hipLaunchKernelGGL((rmsnorm_kernel<false>), dim3(c.n_kv_heads), dim3(256), 0, s, m->k, L.k_norm, c.head_dim,
+                               c.rms_eps, m->k, nullptr, nullptr);
+        }
+        hipLaunchKernelGGL(rope_kv_kernel, dim3(c.n_heads + 2 * c.n_kv_heads), dim3(c.head_dim / 2), 0, s, m->q, m->k,
+                           m->v, m->rope_table, m->scalars + 1, c.n_heads, c.n_kv_heads, c.head_dim, c.rope_type,
+                           L.kc, L.vc, c.max_seq_len);
+        HIP_TRY(ctx, hipGetLastError());
+        // attention over positions [0, pos]; the merge also quantizes for the O projection
+        CERA_TRY(cera_launch_attn_decode(ctx, m->q, L.kc, L.vc, c.n_heads, c.n_kv_heads, c.head_dim, pos + 1,
+                                         c.max_seq_len, scale, 0, m->attn_out, m->xs, m->xq));
+        CERA_TRY(project(m, L.o, m->attn_out, m->hidden, m->hidden));
+
+        CERA_TRY(norm_quant(m, m->hidden, L.ffn_norm, c.hidden, 1, m->normed));
+        const bool fuse = L.gate->dtype == L.up->dtype && L.gate->dtype != CERA_HIP_Q5_K;
+        if (fuse) {
+            CERA_TRY(cera_launch_gemv(ctx, L.gate, L.up, m->xs, m->xq, m->act, nullptr, CERA_EPI_SILU_MUL));
+            CERA_TRY(cera_launch_quantize(ctx, m->act, c.ffn, m->xs, m->xq));
+        } else {
+            CERA_TRY(project(m, L.gate, m->normed, m->act, nullptr));
+            CERA_TRY(project(m, L.up, m->normed, m->up, nullptr));
+            hipLaunchKernelGGL((silu_mul_kernel<true>), dim3((c.ffn / 4 + 255) / 256), dim3(256), 0, s, m->act, m->up,
+                               static_cast<uint64_t>(c.ffn), m->act, m->xs, m->xq);
+            HIP_TRY(ctx, hipGetLastError());
+        }
+        CERA_TRY(project(m, L.down, m->act, m->hidden, m->hidden));
+    }
+    // final norm in place (run_layers ends with rmsnorm(hidden, output_norm))
+    CERA_TRY(norm_quant(m, m->hidden, m->output_norm, c.hidden, 1, m->hidden));
+    if (want_logits) {
+        const cera_hip_dtensor* o = m->output ? m->output : m->embd;
+        CERA_TRY(project(m, o, m->hidden, m->logits, nullptr));
+        if (c.logit_scale != 1.0f) {
+            hipLaunchKernelGGL(scale_kernel, dim3((c.vocab + 255) / 256), dim3(256), 0, s, m->logits,
+                               1.0f / c.logit_scale, c.vocab);
+            HIP_TRY(ctx, hipGetLastError());
+        }
+    }
+    return CERA_HIP_OK;
+}
+
+static cera_hip_status check_step(cera_hip_model* m, uint32_t token, uint32_t pos) {
+    if (token >= m->cfg.vocab)
+        return cera_fail(m->ctx, CERA_HIP_ERR_ARGUMENT, "token id " + std::to_string(token) + " out of range (vocab " + std::to_string(m->cfg.vocab) + ")");
+    if (pos != m->seq_len)
+        return cera_fail(m->ctx, CERA_HIP_ERR_POSITION, "pos " + std::to_string(pos) + " != seq_len " + std::to_string(m->seq_len));
+    if (pos >= m->cfg.max_seq_len)
+        return cera_fail(m->ctx, CERA_HIP_ERR_POSITION, "context full: pos " + std::to_string(pos) + " >= max_seq_len " + std::to_string(m->cfg.max_seq_len));
+    return CERA_HIP_OK;
+}
+
+// Kernel arguments are captured at launch, so (unlike an async copy from a
+// stack variable) the values cannot change under a launch that is still queued.
+static __global__ void set_token_pos_kernel(uint32_t* scalars, uint32_t token, uint32_t pos) {
+    scalars[0] = token;
+    scalars[1] = pos;
+}
+static cera_hip_status set_token_pos(cera_hip_model* m, uint32_t token, uint32_t pos) {
+    hipLaunchKernelGGL(set_token_pos_kernel, dim3(1), dim3(1), 0, m->ctx->stream, m->scalars, token, pos);
+    HIP_TRY(m->ctx, hipGetLastError());
+    return CERA_HIP_OK;
+}
+
+extern "C" cera_hip_status cera_hip_forward(cera_hip_model* m, uint32_t token, uint32_t pos, float* logits) {
+    if (!m || !logits) return CERA_HIP_ERR_ARGUMENT;
+    std::lock_guard<std::mutex> lk(m->infer_lock);
+    CERA_TRY(check_step(m, token, pos));
+    CERA_TRY(set_token_pos(m, token, pos));
+    CERA_TRY(decode_step(m, pos, true));
+    CERA_TRY(cera_hip_download(m->ctx, logits, m->logits, static_cast<uint64_t>(m->cfg.vocab) * 4));
+    m->seq_len = pos + 1;
+    return CERA_HIP_OK;
+}
+
+extern "C" cera_hip_status cera_hip_forward_greedy(cera_hip_model* m, uint32_t token, uint32_t pos, uint32_t* next) {
+    if (!m || !next) return CERA_HIP_ERR_ARGUMENT;
+    std::lock_guard<std::mutex> lk(m->infer_lock);
+    CERA_TRY(check_step(m, token, pos));
+    CERA_TRY(set_token_pos(m, token, pos));
+    CERA_TRY(decode_step(m, pos, true));
+    hipLaunchKernelGGL(argmax_kernel, dim3(1), dim3(1024), 0, m->ctx->stream, m->logits, m->cfg.vocab, m->scalars + 2);
+    HIP_TRY(m->ctx, hipGetLastError());
+    CERA_TRY(cera_hip_download(m->ctx, next, m->scalars + 2, 4));
+    m->seq_len = pos + 1;
+    return CERA_HIP_OK;
+}
+
+extern "C" cera_hip_status cera_hip_forward_prefill(cera_hip_model* m, const uint32_t* tokens, uint32_t n,
+                                                    uint32_t start_pos, float* last_logits) {
+    if (!m || !tokens || !last_logits) return CERA_HIP_ERR_ARGUMENT;
+    if (n == 0) return cera_fail(m->ctx, CERA_HIP_ERR_ARGUMENT, "forward_prefill requires at least one token");
+    std::lock_guard<std::mutex> lk(m->infer_lock);
+    if (start_pos != m->seq_len)
+        return cera_fail(m->ctx, CERA_HIP_ERR_POSITION, "forward_prefill: start_pos " + std::to_string(start_pos) +
+                                                            " must equal seq_len " + std::to_string(m->seq_len));
+    if (static_cast<uint64_t>(start_pos) + n > m->cfg.max_seq_len)
+        return cera_fail(m->ctx, CERA_HIP_ERR_POSITION, "forward_prefill: prompt does not fit max_seq_len");
+    for (uint32_t i = 0; i < n; ++i)
+        if (tokens[i] >= m->cfg.vocab) return cera_fail(m->ctx, CERA_HIP_ERR_ARGUMENT, "token id out of range");
+    return cera_model_prefill(m, tokens, n, start_pos, last_logits);
+}
+
+// Token-at-a-time prefill (LlamaModel::forward_prefill's per-token route,
+// cera/src/model/llama.rs:1643-1648); the batched route replaces it when the
+// weight types support the int8 GEMM.
+cera_hip_status cera_model_prefill_per_token(cera_hip_model* m, const uint32_t* tokens, uint32_t n,
+                                             uint32_t start_pos, float* last_logits) {
+    for (uint32_t i = 0; i < n; ++i) {
+        CERA_TRY(set_token_pos(m, tokens[i], start_pos + i));
+        CERA_TRY(decode_step(m, start_pos + i, i + 1 == n));
+        m->seq_len = start_pos + i + 1;
+    }
+    return cera_hip_download(m->ctx, last_logits, m->logits, static_cast<uint64_t>(m->cfg.vocab) * 4);
+}
+
+extern "C" cera_hip_status cera_hip_read_kv(cera_hip_model* m, uint32_t layer, float* k_out, float* v_out) {
+    if (!m || !k_out || !v_out || layer >= m->cfg.n_layers) return CERA_HIP_ERR_ARGUMENT;
+    std::lock_guard<std::mutex> lk(m->infer_lock);
+    const cera_hip_config& c = m->cfg;
+    const uint64_t per_head = static_cast<uint64_t>(c.max_seq_len) * c.head_dim;
+    std::vector<float> hk(static_cast<uint64_t>(m->seq_len) * c.head_dim), hv(hk.size());
+    const uint64_t kv_dim = static_cast<uint64_t>(c.n_kv_heads) * c.head_dim;
+    for (uint32_t h = 0; h < c.n_kv_heads; ++h) {
+        CERA_TRY(cera_hip_download(m->ctx, hk.data(), m->layers[layer].kc + h * per_head, hk.size() * 4));
+        CERA_TRY(cera_hip_download(m->ctx, hv.data(), m->layers[layer].vc + h * per_head, hv.size() * 4));
+        for (uint32_t t = 0; t < m->seq_len; ++t) {
+            std::memcpy(k_out + t * kv_dim + h * c.head_dim, hk.data() + static_cast<uint64_t>(t) * c.head_dim, c.head_dim * 4);
+            std::memcpy(v_out + t * kv_dim + h * c.head_dim, hv.data() + static_cast<uint64_t>(t) * c.head_dim, c.head_dim * 4);
+        }
+    }
+    return CERA_HIP_OK;
+}
+
+extern "C" cera_hip_status cera_hip_read_hidden(cera_hip_model* m, float* hidden_out) {
+    if (!m || !hidden_out) return CERA_HIP_ERR_ARGUMENT;
+    std::lock_guard<std::mutex> lk(m->infer_lock);
+    return cera_hip_download(m->ctx, hidden_out, m->hidden, static_cast<uint64_t>(m->cfg.hidden) * 4);
+}
+
+// cpu::rope / cpu::rope_norm on host buffers (test entry point).
+extern "C" cera_hip_status cera_hip_rope(cera_hip_ctx* ctx, float* q, float* k, uint32_t pos, uint32_t n_heads,
+                                         uint32_t n_kv_heads, uint32_t head_dim, float freq_base, uint32_t rope_type,
+                                         const float* freq_factors) {
+    if (!ctx || !q || !k) return CERA_HIP_ERR_ARGUMENT;
+    if (head_dim == 0 || head_dim % 2 || head_dim > 2048 || rope_type > 1) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "rope: bad head_dim or rope_type");
+    std::vector<float> table;
+    cera_build_rope_table(pos + 1, head_dim, freq_base, freq_factors, table);
+    const uint64_t half = head_dim / 2;
+    void *dq, *dk, *dt, *dp;
+    CERA_TRY(cera_scratch(ctx, 0, static_cast<uint64_t>(n_heads) * head_dim * 4, &dq));
+    CERA_TRY(cera_scratch(ctx, 1, static_cast<uint64_t>(n_kv_heads) * head_dim * 4, &dk));
+    CERA_TRY(cera_scratch(ctx, 2, half * 8, &dt));
+    CERA_TRY(cera_scratch(ctx, 3, 4, &dp));
+    uint32_t zero = 0;
+    CERA_TRY(cera_hip_upload(ctx, dq, q, static_cast<uint64_t>(n_heads) * head_dim * 4));
+    CERA_TRY(cera_hip_upload(ctx, dk, k, static_cast<uint64_t>(n_kv_heads) * head_dim * 4));
+    CERA_TRY(cera_hip_upload(ctx, dt, table.data() + static_cast<uint64_t>(pos) * half * 2, half * 8));
+    CERA_TRY(cera_hip_upload(ctx, dp, &zero, 4));
+    hipLaunchKernelGGL(rope_kv_kernel, dim3(n_heads + n_kv_heads), dim3(head_dim / 2), 0, ctx->stream,
+                       static_cast<float*>(dq), static_cast<float*>(dk), static_cast<const float*>(nullptr),
+                       static_cast<float*>(dt), static_cast<uint32_t*>(dp), n_heads, n_kv_heads, head_dim, rope_type,
+                       static_cast<float*>(nullptr), static_cast<float*>(nullptr), 1u);
+    HIP_TRY(ctx, hipGetLastError());
+    CERA_TRY(cera_hip_download(ctx, q, dq, static_cast<uint64_t>(n_heads) * head_dim * 4));
+    return cera_hip_download(ctx, k, dk, static_cast<uint64_t>(n_kv_heads) * head_dim * 4);
+}

@@ -1,0 +1,389 @@
+"""ctypes binding of the C-ABI HIP library (``include/cera_hip.h``).
+
+This is plumbing for the tests and the benchmark: every call goes straight to
+``libcera_hip.so``.  There is no CPU fallback -- if the library or a GPU is
+missing, loading fails with an error.
+"""
+from __future__ import annotations
+
+import ctypes as C
+
+import numpy as np
+
+from . import _build
+
+F32, F16, Q4_0, Q4_1, Q8_0, Q4_K, Q5_K, Q6_K, BF16 = 0, 1, 2, 3, 8, 12, 13, 14, 30
+STATUS = {0: "OK", 1: "ERR_DEVICE", 2: "ERR_OOM", 3: "ERR_UNSUPPORTED_DTYPE", 4: "ERR_SHAPE", 5: "ERR_POSITION",
+          6: "ERR_ARGUMENT"}
+
+# every symbol include/cera_hip.h declares
+SYMBOLS = [
+    "cera_hip_ctx_create", "cera_hip_ctx_destroy", "cera_hip_last_error", "cera_hip_sync", "cera_hip_device_info",
+    "cera_hip_malloc", "cera_hip_free", "cera_hip_upload", "cera_hip_download", "cera_hip_copy_dev",
+    "cera_hip_event_create", "cera_hip_event_destroy", "cera_hip_event_record", "cera_hip_event_elapsed_ms",
+    "cera_hip_tensor_upload", "cera_hip_tensor_clone", "cera_hip_tensor_free", "cera_hip_tensor_nbytes",
+    "cera_hip_quantize_q8_0", "cera_hip_gemv", "cera_hip_gemm", "cera_hip_attn_decode", "cera_hip_rmsnorm",
+    "cera_hip_silu_mul", "cera_hip_rope", "cera_hip_argmax", "cera_hip_dequantize_row",
+    "cera_hip_quantize_q8_0_dev", "cera_hip_gemv_q8_dev", "cera_hip_gemv_seq_dev", "cera_hip_attn_decode_dev",
+    "cera_hip_gemm_dev",
+    "cera_hip_model_create", "cera_hip_model_destroy", "cera_hip_forward", "cera_hip_forward_greedy",
+    "cera_hip_forward_prefill", "cera_hip_truncate_kv", "cera_hip_seq_len", "cera_hip_memory_bytes",
+    "cera_hip_read_kv", "cera_hip_read_hidden",
+]
+
+
+class HipError(RuntimeError):
+    def __init__(self, status: int, message: str):
+        super().__init__(f"cera_hip {STATUS.get(status, status)}: {message}")
+        self.status = status
+        self.message = message
+
+
+class Tensor(C.Structure):
+    _fields_ = [("ggml_type", C.c_uint32), ("_reserved", C.c_uint32), ("m", C.c_uint64), ("k", C.c_uint64),
+                ("data", C.c_void_p), ("nbytes", C.c_uint64)]
+
+
+class Layer(C.Structure):
+    _fields_ = [("attn_norm", C.c_void_p), ("ffn_norm", C.c_void_p),
+                ("attn_q", Tensor), ("attn_k", Tensor), ("attn_v", Tensor), ("attn_output", Tensor),
+                ("ffn_gate", Tensor), ("ffn_up", Tensor), ("ffn_down", Tensor),
+                ("q_bias", C.c_void_p), ("k_bias", C.c_void_p), ("v_bias", C.c_void_p),
+                ("q_norm", C.c_void_p), ("k_norm", C.c_void_p)]
+
+
+class Config(C.Structure):
+    _fields_ = [("n_layers", C.c_uint32), ("hidden", C.c_uint32), ("ffn", C.c_uint32), ("n_heads", C.c_uint32),
+                ("n_kv_heads", C.c_uint32), ("head_dim", C.c_uint32), ("vocab", C.c_uint32),
+                ("max_seq_len", C.c_uint32), ("rope_type", C.c_uint32),
+                ("rope_theta", C.c_float), ("rms_eps", C.c_float), ("embed_scale", C.c_float),
+                ("residual_scale", C.c_float), ("attn_scale", C.c_float), ("logit_scale", C.c_float),
+                ("rope_freqs", C.c_void_p)]
+
+
+class GemvOp(C.Structure):
+    _fields_ = [("w", C.c_void_p), ("xs", C.c_void_p), ("xq", C.c_void_p), ("y", C.c_void_p)]
+
+
+_lib = None
+
+
+def load_library() -> C.CDLL:
+    """Load libcera_hip.so (never builds it: build with ``__graft_entry__.build()``)."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not _build.HIP_LIB.exists():
+        raise RuntimeError(f"{_build.HIP_LIB} is missing: run `python -c 'import __graft_entry__ as g; g.build()'`")
+    L = C.CDLL(str(_build.HIP_LIB))
+    vp, u32, u64, f32, i32 = C.c_void_p, C.c_uint32, C.c_uint64, C.c_float, C.c_int
+    pp = C.POINTER(C.c_void_p)
+    sig = {
+        "cera_hip_ctx_create": (i32, [i32, pp]), "cera_hip_ctx_destroy": (None, [vp]),
+        "cera_hip_last_error": (C.c_char_p, [vp]), "cera_hip_sync": (i32, [vp]),
+        "cera_hip_device_info": (i32, [vp, C.c_char_p, C.POINTER(u32), C.POINTER(u64)]),
+        "cera_hip_malloc": (i32, [vp, u64, pp]), "cera_hip_free": (i32, [vp, vp]),
+        "cera_hip_upload": (i32, [vp, vp, vp, u64]), "cera_hip_download": (i32, [vp, vp, vp, u64]),
+        "cera_hip_copy_dev": (i32, [vp, vp, vp, u64]),
+        "cera_hip_event_create": (i32, [vp, pp]), "cera_hip_event_destroy": (None, [vp]),
+        "cera_hip_event_record": (i32, [vp, vp]),
+        "cera_hip_event_elapsed_ms": (i32, [vp, vp, vp, C.POINTER(f32)]),
+        "cera_hip_tensor_upload": (i32, [vp, C.POINTER(Tensor), pp]),
+        "cera_hip_tensor_clone": (i32, [vp, vp, pp]),
+        "cera_hip_tensor_free": (None, [vp, vp]), "cera_hip_tensor_nbytes": (u64, [vp]),
+        "cera_hip_quantize_q8_0": (i32, [vp, vp, u64, vp, vp]),
+        "cera_hip_gemv": (i32, [vp, C.POINTER(Tensor), vp, vp, vp, vp]),
+        "cera_hip_gemm": (i32, [vp, C.POINTER(Tensor), vp, u64, vp]),
+        "cera_hip_attn_decode": (i32, [vp, vp, vp, vp, u32, u32, u32, u64, f32, u32, vp]),
+        "cera_hip_rmsnorm": (i32, [vp, vp, vp, u64, f32, vp]),
+        "cera_hip_silu_mul": (i32, [vp, vp, vp, u64, vp]),
+        "cera_hip_rope": (i32, [vp, vp, vp, u32, u32, u32, u32, f32, u32, vp]),
+        "cera_hip_argmax": (i32, [vp, vp, u64, C.POINTER(u32)]),
+        "cera_hip_dequantize_row": (i32, [vp, C.POINTER(Tensor), u64, vp]),
+        "cera_hip_quantize_q8_0_dev": (i32, [vp, vp, u64, vp, vp]),
+        "cera_hip_gemv_q8_dev": (i32, [vp, vp, vp, vp, vp]),
+        "cera_hip_gemv_seq_dev": (i32, [vp, C.POINTER(GemvOp), u32]),
+        "cera_hip_attn_decode_dev": (i32, [vp, vp, vp, vp, u32, u32, u32, u64, u64, f32, u32, vp]),
+        "cera_hip_gemm_dev": (i32, [vp, vp, vp, u64, vp]),
+        "cera_hip_model_create": (i32, [vp, C.POINTER(Config), C.POINTER(Tensor), C.POINTER(Tensor), vp,
+                                        C.POINTER(Layer), pp]),
+        "cera_hip_model_destroy": (None, [vp]),
+        "cera_hip_forward": (i32, [vp, u32, u32, vp]),
+        "cera_hip_forward_greedy": (i32, [vp, u32, u32, C.POINTER(u32)]),
+        "cera_hip_forward_prefill": (i32, [vp, vp, u32, u32, vp]),
+        "cera_hip_truncate_kv": (i32, [vp, u32]),
+        "cera_hip_seq_len": (u32, [vp]), "cera_hip_memory_bytes": (u64, [vp]),
+        "cera_hip_read_kv": (i32, [vp, u32, vp, vp]), "cera_hip_read_hidden": (i32, [vp, vp]),
+    }
+    for name, (res, args) in sig.items():
+        fn = getattr(L, name)
+        fn.restype, fn.argtypes = res, args
+    _lib = L
+    return L
+
+
+def _p(a: np.ndarray) -> int:
+    assert a.flags["C_CONTIGUOUS"]
+    return a.ctypes.data
+
+
+def make_tensor(ggml_type: int, m: int, k: int, blocks: np.ndarray) -> Tensor:
+    blocks = np.ascontiguousarray(blocks).reshape(-1).view(np.uint8)
+    t = Tensor(ggml_type, 0, m, k, blocks.ctypes.data, blocks.size)
+    t._keep = blocks  # keep the host bytes alive as long as the descriptor
+    return t
+
+
+class Context:
+    """One HIP device + stream (cera_hip_ctx)."""
+
+    def __init__(self, device: int = 0):
+        self.lib = load_library()
+        h = C.c_void_p()
+        st = self.lib.cera_hip_ctx_create(device, C.byref(h))
+        if st != 0:
+            raise HipError(st, (self.lib.cera_hip_last_error(None) or b"").decode())
+        self.h = h
+
+    # -- helpers
+    def check(self, st: int):
+        if st != 0:
+            raise HipError(st, (self.lib.cera_hip_last_error(self.h) or b"").decode())
+
+    def close(self):
+        if getattr(self, "h", None):
+            self.lib.cera_hip_ctx_destroy(self.h)
+            self.h = None
+
+    def sync(self):
+        self.check(self.lib.cera_hip_sync(self.h))
+
+    def device_info(self):
+        name = C.create_string_buffer(256)
+        cu, hbm = C.c_uint32(), C.c_uint64()
+        self.check(self.lib.cera_hip_device_info(self.h, name, C.byref(cu), C.byref(hbm)))
+        return name.value.decode(), cu.value, hbm.value
+
+    # -- device memory
+    def malloc(self, nbytes: int) -> int:
+        p = C.c_void_p()
+        self.check(self.lib.cera_hip_malloc(self.h, nbytes, C.byref(p)))
+        return p.value
+
+    def free(self, dev: int):
+        self.check(self.lib.cera_hip_free(self.h, dev))
+
+    def upload(self, dev: int, arr: np.ndarray):
+        arr = np.ascontiguousarray(arr)
+        self.check(self.lib.cera_hip_upload(self.h, dev, _p(arr), arr.nbytes))
+
+    def to_device(self, arr: np.ndarray) -> int:
+        arr = np.ascontiguousarray(arr)
+        d = self.malloc(arr.nbytes)
+        self.upload(d, arr)
+        return d
+
+    def download(self, dev: int, shape, dtype) -> np.ndarray:
+        out = np.empty(shape, dtype)
+        self.check(self.lib.cera_hip_download(self.h, _p(out), dev, out.nbytes))
+        return out
+
+    # -- events
+    def event(self) -> int:
+        e = C.c_void_p()
+        self.check(self.lib.cera_hip_event_create(self.h, C.byref(e)))
+        return e.value
+
+    def record(self, ev: int):
+        self.check(self.lib.cera_hip_event_record(self.h, ev))
+
+    def elapsed_ms(self, a: int, b: int) -> float:
+        ms = C.c_float()
+        self.check(self.lib.cera_hip_event_elapsed_ms(self.h, a, b, C.byref(ms)))
+        return ms.value
+
+    def event_destroy(self, ev: int):
+        self.lib.cera_hip_event_destroy(ev)
+
+    # -- weights
+    def tensor_upload(self, ggml_type: int, m: int, k: int, blocks: np.ndarray) -> int:
+        t = make_tensor(ggml_type, m, k, blocks)
+        h = C.c_void_p()
+        self.check(self.lib.cera_hip_tensor_upload(self.h, C.byref(t), C.byref(h)))
+        return h.value
+
+    def tensor_clone(self, dt: int) -> int:
+        h = C.c_void_p()
+        self.check(self.lib.cera_hip_tensor_clone(self.h, dt, C.byref(h)))
+        return h.value
+
+    def tensor_free(self, dt: int):
+        self.lib.cera_hip_tensor_free(self.h, dt)
+
+    # -- kernel level, host buffers
+    def quantize_q8_0(self, x: np.ndarray):
+        x = np.ascontiguousarray(x, np.float32).reshape(-1)
+        k = x.size
+        scales = np.empty(max(k // 32, 0), np.float32)
+        quants = np.empty(k, np.int8)
+        self.check(self.lib.cera_hip_quantize_q8_0(self.h, _p(x), k, _p(scales), _p(quants)))
+        return scales, quants
+
+    def gemv(self, ggml_type: int, blocks: np.ndarray, x: np.ndarray, m: int, k: int, debug: bool = False):
+        t = make_tensor(ggml_type, m, k, blocks)
+        x = np.ascontiguousarray(x, np.float32)
+        y = np.empty(m, np.float32)
+        if not debug:
+            self.check(self.lib.cera_hip_gemv(self.h, C.byref(t), _p(x), _p(y), None, None))
+            return y
+        nd = k // 16 if ggml_type == Q6_K else k // 32
+        dots = np.zeros((m, nd), np.int32)
+        asums = np.zeros(nd, np.int32)
+        self.check(self.lib.cera_hip_gemv(self.h, C.byref(t), _p(x), _p(y), _p(dots), _p(asums)))
+        return y, dots, asums
+
+    def gemm(self, ggml_type: int, blocks: np.ndarray, x: np.ndarray, m: int, n: int, k: int) -> np.ndarray:
+        t = make_tensor(ggml_type, m, k, blocks)
+        x = np.ascontiguousarray(x, np.float32).reshape(n, k)
+        out = np.empty((m, n), np.float32)
+        self.check(self.lib.cera_hip_gemm(self.h, C.byref(t), _p(x), n, _p(out)))
+        return out
+
+    def attn_decode(self, q, k, v, n_heads, n_kv_heads, head_dim, seq_len, scale, n_splits=0) -> np.ndarray:
+        q = np.ascontiguousarray(q, np.float32)
+        k = np.ascontiguousarray(k, np.float32)
+        v = np.ascontiguousarray(v, np.float32)
+        out = np.empty(n_heads * head_dim, np.float32)
+        self.check(self.lib.cera_hip_attn_decode(self.h, _p(q), _p(k), _p(v), n_heads, n_kv_heads, head_dim, seq_len,
+                                                 scale, n_splits, _p(out)))
+        return out
+
+    def rmsnorm(self, x, w, eps) -> np.ndarray:
+        x = np.ascontiguousarray(x, np.float32)
+        w = np.ascontiguousarray(w, np.float32)
+        y = np.empty_like(x)
+        self.check(self.lib.cera_hip_rmsnorm(self.h, _p(x), _p(w), x.size, eps, _p(y)))
+        return y
+
+    def silu_mul(self, gate, up) -> np.ndarray:
+        g = np.ascontiguousarray(gate, np.float32)
+        u = np.ascontiguousarray(up, np.float32)
+        y = np.empty_like(g)
+        self.check(self.lib.cera_hip_silu_mul(self.h, _p(g), _p(u), g.size, _p(y)))
+        return y
+
+    def rope(self, q, k, pos, n_heads, n_kv_heads, head_dim, base, norm=True, freq_factors=None):
+        q2 = np.array(q, np.float32, copy=True).reshape(-1)
+        k2 = np.array(k, np.float32, copy=True).reshape(-1)
+        ff = None if freq_factors is None else np.ascontiguousarray(freq_factors, np.float32)
+        self.check(self.lib.cera_hip_rope(self.h, _p(q2), _p(k2), pos, n_heads, n_kv_heads, head_dim, base,
+                                          1 if norm else 0, None if ff is None else _p(ff)))
+        return q2, k2
+
+    def argmax(self, logits) -> int:
+        l = np.ascontiguousarray(logits, np.float32)
+        idx = C.c_uint32()
+        self.check(self.lib.cera_hip_argmax(self.h, _p(l) if l.size else None, l.size, C.byref(idx)))
+        return idx.value
+
+    def dequantize_row(self, ggml_type, blocks, m, k, row) -> np.ndarray:
+        t = make_tensor(ggml_type, m, k, blocks)
+        out = np.empty(k, np.float32)
+        self.check(self.lib.cera_hip_dequantize_row(self.h, C.byref(t), row, _p(out)))
+        return out
+
+
+class Model:
+    """cera_hip_model: the `Model`-trait surface over a device-resident llama.
+
+    ``weights``: name -> (ggml_type, m, k, uint8 blocks) for matrices and
+    name -> float32 array for norm vectors, GGUF tensor names.
+    """
+
+    def __init__(self, ctx: Context, cfg: dict, weights: dict):
+        self.ctx = ctx
+        c = Config()
+        for f in ("n_layers", "hidden", "ffn", "n_heads", "n_kv_heads", "head_dim", "vocab", "max_seq_len"):
+            setattr(c, f, int(cfg[f]))
+        c.rope_type = int(cfg.get("rope_type", 1))
+        c.rope_theta = float(cfg.get("rope_theta", 10000.0))
+        c.rms_eps = float(cfg.get("rms_eps", 1e-5))
+        c.embed_scale = float(cfg.get("embed_scale", 1.0))
+        c.residual_scale = float(cfg.get("residual_scale", 1.0))
+        c.attn_scale = float(cfg.get("attn_scale", 0.0))
+        c.logit_scale = float(cfg.get("logit_scale", 1.0))
+        c.rope_freqs = None
+        self.cfg = dict(cfg)
+        keep = []
+        layers = (Layer * c.n_layers)()
+        for i in range(c.n_layers):
+            L = layers[i]
+            for nm in ("attn_norm", "ffn_norm"):
+                a = np.ascontiguousarray(weights[f"blk.{i}.{nm}.weight"], np.float32)
+                keep.append(a)
+                setattr(L, nm, a.ctypes.data)
+            for nm in ("attn_q", "attn_k", "attn_v", "attn_output", "ffn_gate", "ffn_up", "ffn_down"):
+                dt, m, k, arr = weights[f"blk.{i}.{nm}.weight"]
+                t = make_tensor(dt, m, k, arr)
+                keep.append(t)
+                setattr(L, nm, t)
+            for nm in ("q_bias", "k_bias", "v_bias", "q_norm", "k_norm"):
+                setattr(L, nm, None)
+        dt, m, k, arr = weights["token_embd.weight"]
+        embd = make_tensor(dt, m, k, arr)
+        outp = None
+        if "output.weight" in weights:
+            dt, m, k, arr = weights["output.weight"]
+            outp = make_tensor(dt, m, k, arr)
+        onorm = np.ascontiguousarray(weights["output_norm.weight"], np.float32)
+        h = C.c_void_p()
+        st = ctx.lib.cera_hip_model_create(ctx.h, C.byref(c), C.byref(embd), C.byref(outp) if outp is not None else None,
+                                           onorm.ctypes.data, layers, C.byref(h))
+        ctx.check(st)
+        self.h = h
+        self.vocab = c.vocab
+        self.hidden = c.hidden
+
+    @property
+    def seq_len(self) -> int:
+        return int(self.ctx.lib.cera_hip_seq_len(self.h))
+
+    @property
+    def memory_bytes(self) -> int:
+        return int(self.ctx.lib.cera_hip_memory_bytes(self.h))
+
+    def forward(self, token: int, pos: int) -> np.ndarray:
+        logits = np.empty(self.vocab, np.float32)
+        self.ctx.check(self.ctx.lib.cera_hip_forward(self.h, token, pos, _p(logits)))
+        return logits
+
+    def forward_greedy(self, token: int, pos: int) -> int:
+        nxt = C.c_uint32()
+        self.ctx.check(self.ctx.lib.cera_hip_forward_greedy(self.h, token, pos, C.byref(nxt)))
+        return nxt.value
+
+    def forward_prefill(self, tokens, start_pos: int) -> np.ndarray:
+        t = np.ascontiguousarray(tokens, np.uint32)
+        logits = np.empty(self.vocab, np.float32)
+        self.ctx.check(self.ctx.lib.cera_hip_forward_prefill(self.h, _p(t), t.size, start_pos, _p(logits)))
+        return logits
+
+    def truncate_kv(self, n: int):
+        self.ctx.check(self.ctx.lib.cera_hip_truncate_kv(self.h, n))
+
+    def read_kv(self, layer: int):
+        n = self.seq_len * self.cfg["n_kv_heads"] * self.cfg["head_dim"]
+        k = np.empty(n, np.float32)
+        v = np.empty(n, np.float32)
+        self.ctx.check(self.ctx.lib.cera_hip_read_kv(self.h, layer, _p(k), _p(v)))
+        return k, v
+
+    def read_hidden(self) -> np.ndarray:
+        h = np.empty(self.hidden, np.float32)
+        self.ctx.check(self.ctx.lib.cera_hip_read_hidden(self.h, _p(h)))
+        return h
+
+    def close(self):
+        if getattr(self, "h", None):
+            self.ctx.lib.cera_hip_model_destroy(self.h)
+            self.h = None

@@ -1,0 +1,237 @@
+/* cera_hip.h -- C ABI of the MI355X `hip` compute backend for cera's dense
+ * transformer decode/prefill hot path.
+ *
+ * This is the boundary a `cera-hip-sys` Rust crate binds (plain pointers and
+ * sizes, no C++ types).  Each entry point names the cera interface it stands
+ * in for (paths relative to the cera source tree).
+ *
+ * Conventions
+ *  - every function that can fail returns a cera_hip_status; the message for
+ *    the last failure on a context is returned by cera_hip_last_error();
+ *  - nothing aborts or throws across this boundary;
+ *  - "host" pointers are ordinary CPU memory owned by the caller and only
+ *    borrowed for the duration of the call; "dev" pointers come from
+ *    cera_hip_malloc() on the same context;
+ *  - all work of a context runs on that context's single HIP stream;
+ *  - weights stay in their native GGUF block layout in device memory.
+ */
+#ifndef CERA_HIP_H
+#define CERA_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#if defined(__GNUC__)
+#define CERA_HIP_API __attribute__((visibility("default")))
+#else
+#define CERA_HIP_API
+#endif
+
+typedef struct cera_hip_ctx cera_hip_ctx;         /* device, stream, scratch            */
+typedef struct cera_hip_model cera_hip_model;     /* device weights, KV cache, seq_len   */
+typedef struct cera_hip_dtensor cera_hip_dtensor; /* one weight matrix resident in HBM   */
+typedef struct cera_hip_event cera_hip_event;     /* HIP event on the context's stream   */
+
+typedef enum {
+    CERA_HIP_OK = 0,
+    CERA_HIP_ERR_DEVICE = 1,            /* HIP runtime error (message has the HIP string)  */
+    CERA_HIP_ERR_OOM = 2,               /* device or host allocation failed                */
+    CERA_HIP_ERR_UNSUPPORTED_DTYPE = 3, /* no kernel for this GGML type: refuse, never skip */
+    CERA_HIP_ERR_SHAPE = 4,             /* size/shape/alignment does not fit the kernel    */
+    CERA_HIP_ERR_POSITION = 5,          /* pos/start_pos != current sequence length        */
+    CERA_HIP_ERR_ARGUMENT = 6           /* null pointer or out-of-range scalar             */
+} cera_hip_status;
+
+/* GGML type ids as cera maps them: cera/src/gguf.rs:259-278. */
+enum {
+    CERA_HIP_F32 = 0, CERA_HIP_F16 = 1, CERA_HIP_Q4_0 = 2, CERA_HIP_Q4_1 = 3, CERA_HIP_Q8_0 = 8,
+    CERA_HIP_Q4_K = 12, CERA_HIP_Q5_K = 13, CERA_HIP_Q6_K = 14, CERA_HIP_BF16 = 30
+};
+
+/* A weight matrix as cera resolves it from a GGUF: `WeightRef` {dtype, m, k}
+ * plus the mmap slice (cera/src/model/transformer.rs:127-139, 187-231).
+ * m = output rows, k = inner dimension; data is m rows of k/block_elems blocks. */
+typedef struct {
+    uint32_t ggml_type;
+    uint32_t _reserved;
+    uint64_t m, k;
+    const void* data; /* host */
+    uint64_t nbytes;
+} cera_hip_tensor;
+
+/* Per-layer weights: the fields of `LayerRefs` + norm/bias vectors that
+ * LlamaModel::from_gguf_with_id resolves (cera/src/model/llama.rs:158-450). */
+typedef struct {
+    const float *attn_norm, *ffn_norm; /* f32[hidden] */
+    cera_hip_tensor attn_q, attn_k, attn_v, attn_output, ffn_gate, ffn_up, ffn_down;
+    const float *q_bias, *k_bias, *v_bias; /* nullable (Qwen2) */
+    const float *q_norm, *k_norm;          /* nullable, f32[head_dim] (Qwen3) */
+} cera_hip_layer;
+
+/* `ModelConfig` + `AttnDims` (cera/src/model/mod.rs:117-145, llama.rs:450-466). */
+typedef struct {
+    uint32_t n_layers, hidden, ffn, n_heads, n_kv_heads, head_dim, vocab, max_seq_len;
+    uint32_t rope_type; /* 0 = NEOX (split halves), 1 = NORM (interleaved pairs) */
+    float rope_theta, rms_eps, embed_scale, residual_scale;
+    float attn_scale;  /* 0 => 1/sqrt(head_dim) */
+    float logit_scale; /* logits are divided by this; 1 = off */
+    const float* rope_freqs; /* nullable, f32[head_dim/2] */
+} cera_hip_config;
+
+/* ---- context ------------------------------------------------------------ */
+
+/* Create a context on HIP device `device` (kernels are embedded in this
+ * library as a gfx950 code object).  Stands where a GPU backend's context
+ * constructor does (cera/src/model/mod.rs:672-703 builds one per load). */
+CERA_HIP_API cera_hip_status cera_hip_ctx_create(int device, cera_hip_ctx** out);
+CERA_HIP_API void cera_hip_ctx_destroy(cera_hip_ctx*);
+/* Message of the most recent failure on `ctx` (ctx may be NULL for a failed
+ * cera_hip_ctx_create: then the process-wide last message).  Valid until the
+ * next call on the same context. */
+CERA_HIP_API const char* cera_hip_last_error(const cera_hip_ctx*);
+CERA_HIP_API cera_hip_status cera_hip_sync(cera_hip_ctx*);
+/* Device properties for reporting: name (<= 255 chars), CU count, bytes of HBM. */
+CERA_HIP_API cera_hip_status cera_hip_device_info(cera_hip_ctx*, char* name256, uint32_t* n_cu,
+                                                  uint64_t* hbm_bytes);
+
+/* ---- device memory and events (benchmark / timing plumbing) ------------- */
+CERA_HIP_API cera_hip_status cera_hip_malloc(cera_hip_ctx*, uint64_t nbytes, void** dev_out);
+CERA_HIP_API cera_hip_status cera_hip_free(cera_hip_ctx*, void* dev);
+CERA_HIP_API cera_hip_status cera_hip_upload(cera_hip_ctx*, void* dev_dst, const void* host_src, uint64_t nbytes);
+CERA_HIP_API cera_hip_status cera_hip_download(cera_hip_ctx*, void* host_dst, const void* dev_src, uint64_t nbytes);
+CERA_HIP_API cera_hip_status cera_hip_copy_dev(cera_hip_ctx*, void* dev_dst, const void* dev_src, uint64_t nbytes);
+CERA_HIP_API cera_hip_status cera_hip_event_create(cera_hip_ctx*, cera_hip_event** out);
+CERA_HIP_API void cera_hip_event_destroy(cera_hip_event*);
+CERA_HIP_API cera_hip_status cera_hip_event_record(cera_hip_ctx*, cera_hip_event*);
+/* Waits for `stop`, then returns milliseconds between the two events. */
+CERA_HIP_API cera_hip_status cera_hip_event_elapsed_ms(cera_hip_ctx*, cera_hip_event* start,
+                                                       cera_hip_event* stop, float* ms);
+
+/* ---- weights in HBM, native GGUF block layout --------------------------- */
+/* Copies `t->data` to device memory unchanged (the GPU loaders' upload step,
+ * cera/src/model/gpu_weight_source.rs:40-118 consumers).  Refuses types
+ * without a kernel and k that is not a whole number of blocks. */
+CERA_HIP_API cera_hip_status cera_hip_tensor_upload(cera_hip_ctx*, const cera_hip_tensor* t, cera_hip_dtensor** out);
+/* A second handle of the same shape whose bytes are a device-side copy of
+ * `src` (distinct addresses: lets a benchmark rotate its working set past the
+ * last-level cache without re-uploading). */
+CERA_HIP_API cera_hip_status cera_hip_tensor_clone(cera_hip_ctx*, const cera_hip_dtensor* src, cera_hip_dtensor** out);
+CERA_HIP_API void cera_hip_tensor_free(cera_hip_ctx*, cera_hip_dtensor*);
+CERA_HIP_API uint64_t cera_hip_tensor_nbytes(const cera_hip_dtensor*);
+
+/* ---- kernel-level entry points, host buffers (parity tests) ------------- */
+
+/* cpu::quantize_f32_to_q8_0_into (cera/src/backend/cpu.rs:969-1041; arithmetic
+ * at :942-958).  x f32[k], k % 32 == 0 -> scales f32[k/32], quants i8[k]. */
+CERA_HIP_API cera_hip_status cera_hip_quantize_q8_0(cera_hip_ctx*, const float* x, uint64_t k, float* scales,
+                                                    int8_t* quants);
+
+/* cpu::gemv_dispatch (cera/src/backend/cpu.rs:2360-2474): y[m] = W[m,k] . x[k].
+ * Q4_0/Q4_1/Q8_0/Q4_K/Q6_K quantize x to Q8_0 and run the int8 kernel; Q5_K
+ * dots against the unquantized f32 x, as the CPU path does.
+ * dbg_block_dots / dbg_block_asums (nullable) receive the integer block dots
+ * the kernel formed: Q4_0 [m][k/32] sum (q-8)a; Q8_0 [m][k/32] sum w a;
+ * Q4_1, Q4_K [m][k/32] sum q a with asums [k/32] = sum a; Q6_K [m][k/16]
+ * sum q a (q unsigned 0..63) with asums [k/16]. */
+CERA_HIP_API cera_hip_status cera_hip_gemv(cera_hip_ctx*, const cera_hip_tensor* w, const float* x, float* y,
+                                           int32_t* dbg_block_dots, int32_t* dbg_block_asums);
+
+/* transformer::gemm_preq over quantize_columns (cera/src/model/transformer.rs:
+ * 710-788, 865-946; kernels cera/src/backend/cpu.rs:1437-1557).
+ * x is [n][k] row-major f32 (one activation row per token), each row is
+ * quantized to Q8_0; out is [m][n] row-major -- the reference's
+ * out[m_out_features][n_tokens] layout (cera/src/backend/simd.rs:5130-5148). */
+CERA_HIP_API cera_hip_status cera_hip_gemm(cera_hip_ctx*, const cera_hip_tensor* w, const float* x, uint64_t n,
+                                           float* out);
+
+/* transformer::decode_attention (cera/src/model/transformer.rs:1249-1305) with
+ * cpu::attn_scores / softmax_inplace / attn_values (cera/src/backend/cpu.rs:
+ * 3222-3363, 2617-2633).  q f32[n_heads*head_dim]; k, v f32 time-major
+ * [seq_len][n_kv_heads*head_dim] (cera/src/kv_cache.rs:201-212);
+ * out f32[n_heads*head_dim]; all seq_len positions visible.
+ * n_splits = 0 lets the library choose the split-K factor. */
+CERA_HIP_API cera_hip_status cera_hip_attn_decode(cera_hip_ctx*, const float* q, const float* k, const float* v,
+                                                  uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim,
+                                                  uint64_t seq_len, float scale, uint32_t n_splits, float* out);
+
+/* cpu::rmsnorm (cera/src/backend/cpu.rs:2479-2496), out of place: y = x*inv_rms*w. */
+CERA_HIP_API cera_hip_status cera_hip_rmsnorm(cera_hip_ctx*, const float* x, const float* weight, uint64_t n,
+                                              float eps, float* y);
+/* cpu::silu_mul_inplace (cera/src/backend/cpu.rs:2570-2575): out = silu(gate)*up. */
+CERA_HIP_API cera_hip_status cera_hip_silu_mul(cera_hip_ctx*, const float* gate, const float* up, uint64_t n,
+                                               float* out);
+/* cpu::rope / cpu::rope_norm (cera/src/backend/cpu.rs:5008-5180), in place on
+ * host copies of q [n_heads*head_dim] and k [n_kv_heads*head_dim]. */
+CERA_HIP_API cera_hip_status cera_hip_rope(cera_hip_ctx*, float* q, float* k, uint32_t pos, uint32_t n_heads,
+                                           uint32_t n_kv_heads, uint32_t head_dim, float freq_base,
+                                           uint32_t rope_type, const float* freq_factors);
+/* sampler::argmax (cera/src/sampler.rs:20-30). */
+CERA_HIP_API cera_hip_status cera_hip_argmax(cera_hip_ctx*, const float* logits, uint64_t n, uint32_t* index);
+/* transformer::dequantize_row_into (cera/src/model/transformer.rs:949-1017). */
+CERA_HIP_API cera_hip_status cera_hip_dequantize_row(cera_hip_ctx*, const cera_hip_tensor* w, uint64_t row,
+                                                     float* out);
+
+/* ---- kernel-level entry points, device buffers (timing) ----------------- */
+CERA_HIP_API cera_hip_status cera_hip_quantize_q8_0_dev(cera_hip_ctx*, const float* x, uint64_t k, float* scales,
+                                                        int8_t* quants);
+/* int8 GEMV on already-quantized activations (transformer::gemv_preq shape,
+ * cera/src/model/transformer.rs:455-533): y[m] = W . (xs, xq). */
+CERA_HIP_API cera_hip_status cera_hip_gemv_q8_dev(cera_hip_ctx*, const cera_hip_dtensor* w, const float* xs,
+                                                  const int8_t* xq, float* y);
+typedef struct {
+    const cera_hip_dtensor* w;
+    const float* xs;  /* dev f32[k/32] */
+    const int8_t* xq; /* dev i8[k]     */
+    float* y;         /* dev f32[m]    */
+} cera_hip_gemv_op;
+/* Launches ops[0..n) back to back on the context's stream (one decode token's
+ * worth of GEMVs without per-call host overhead). */
+CERA_HIP_API cera_hip_status cera_hip_gemv_seq_dev(cera_hip_ctx*, const cera_hip_gemv_op* ops, uint32_t n);
+CERA_HIP_API cera_hip_status cera_hip_attn_decode_dev(cera_hip_ctx*, const float* q, const float* k_headmajor,
+                                                      const float* v_headmajor, uint32_t n_heads,
+                                                      uint32_t n_kv_heads, uint32_t head_dim, uint64_t seq_len,
+                                                      uint64_t max_seq, float scale, uint32_t n_splits, float* out);
+/* out[m][n] = W . quantize(x[n][k]) with x, out on the device. */
+CERA_HIP_API cera_hip_status cera_hip_gemm_dev(cera_hip_ctx*, const cera_hip_dtensor* w, const float* x, uint64_t n,
+                                               float* out);
+
+/* ---- model level: the `Model` trait surface ------------------------------ */
+
+/* load_model_gpu-style construction from resolved weights
+ * (cera/src/model/mod.rs:672-703; cera/src/model/llama.rs:158-450).  Host
+ * pointers are borrowed for the call only; everything is copied to HBM. */
+CERA_HIP_API cera_hip_status cera_hip_model_create(cera_hip_ctx*, const cera_hip_config*,
+                                                   const cera_hip_tensor* token_embd,
+                                                   const cera_hip_tensor* output /* nullable => tied */,
+                                                   const float* output_norm, const cera_hip_layer* layers,
+                                                   cera_hip_model** out);
+CERA_HIP_API void cera_hip_model_destroy(cera_hip_model*);
+/* Model::forward (cera/src/model/mod.rs:200-606; LlamaModel::forward,
+ * cera/src/model/llama.rs:1585-1605): one token at `pos` -> vocab logits. */
+CERA_HIP_API cera_hip_status cera_hip_forward(cera_hip_model*, uint32_t token, uint32_t pos, float* logits);
+/* Model::forward_greedy (cera/src/model/mod.rs:494-497): forward + argmax on
+ * the device, 4-byte readback. */
+CERA_HIP_API cera_hip_status cera_hip_forward_greedy(cera_hip_model*, uint32_t token, uint32_t pos, uint32_t* next);
+/* Model::forward_prefill (cera/src/model/llama.rs:1607-1649): n tokens from
+ * start_pos, logits of the last one. */
+CERA_HIP_API cera_hip_status cera_hip_forward_prefill(cera_hip_model*, const uint32_t* tokens, uint32_t n,
+                                                      uint32_t start_pos, float* last_logits);
+/* Model::truncate_kv (cera/src/model/mod.rs:251-283). */
+CERA_HIP_API cera_hip_status cera_hip_truncate_kv(cera_hip_model*, uint32_t len);
+CERA_HIP_API uint32_t cera_hip_seq_len(const cera_hip_model*);
+/* Model::gpu_memory_bytes. */
+CERA_HIP_API uint64_t cera_hip_memory_bytes(const cera_hip_model*);
+/* Test hook: copies layer `layer`'s K and V cache rows [0, seq_len) to host in
+ * the reference's time-major [pos][kv_dim] order. */
+CERA_HIP_API cera_hip_status cera_hip_read_kv(cera_hip_model*, uint32_t layer, float* k_out, float* v_out);
+/* Test hook: final normed hidden state of the last forward (f32[hidden]). */
+CERA_HIP_API cera_hip_status cera_hip_read_hidden(cera_hip_model*, float* hidden_out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CERA_HIP_H */

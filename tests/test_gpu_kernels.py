@@ -1,0 +1,287 @@
+"""GPU parity: every kernel-level entry point of the C ABI against the CPU
+oracle on the same seeded inputs.
+
+Bars (from the north star): Q8_0 activation quants + scales and per-block int32
+dots bit-exact; GEMV float outputs max|err| <= 1e-3 * rms(ref); attention
+<= 2e-3 * rms(ref).
+"""
+import math
+
+import numpy as np
+import pytest
+
+import util
+from util import Q4_0, Q4_1, Q8_0, Q4_K, Q5_K, Q6_K
+
+pytestmark = pytest.mark.gpu
+
+GEMV_TOL = 1e-3   # x rms(ref)
+ATTN_TOL = 2e-3   # x rms(ref)
+
+
+def _say(msg):
+    print(msg, flush=True)
+
+
+# ---- Q8_0 activation quantizer ------------------------------------------------
+@pytest.mark.parametrize("k,scale,seed", [(4096, 1.0, 1), (14336, 1.0, 2), (32, 1.0, 3), (256, 1e-4, 4),
+                                          (512, 3e4, 5), (4096 * 8, 0.3, 6)])
+def test_quantize_q8_0_bit_exact(hip, orc, k, scale, seed):
+    _say(f"quantize k={k} scale={scale} seed={seed}")
+    x = util.make_x(k, seed) * np.float32(scale)
+    s, q = hip.quantize_q8_0(x)
+    s0, q0 = orc.quantize_q8_0(x)
+    assert np.array_equal(s.view(np.uint32), s0.view(np.uint32))
+    assert np.array_equal(q, q0)
+
+
+def test_quantize_q8_0_edge_cases_bit_exact(hip, orc):
+    _say("quantize edge cases")
+    x = util.make_x(32 * 12, 7)
+    x[0:32] = 0.0                                   # zero block
+    x[32:64] = np.float32(1e-44)                    # subnormal amax -> id = 0
+    x[64 + 5] = np.nan                              # NaN lane
+    x[96:128] = 0; x[96] = 127.0                    # id == 1 exactly, ties below
+    x[97:105] = [0.5, 1.5, 2.5, -0.5, -1.5, -2.5, 3.5, -3.5]
+    x[128 + 3] = np.inf                             # inf -> d = inf, id = 0
+    x[160:192] = np.float32(1e-38)                  # subnormal-ish d, finite 1/d
+    x[192:224] = -np.abs(x[192:224])                # all negative
+    x[224:256] = np.float32(3.0e38)                 # huge, d finite, f16 scale = inf
+    x[256:288] = np.float32(6e-8) * util.make_x(32, 8)   # scale lands in f16 subnormals
+    x[288:320] = np.nan                             # all NaN
+    x[320 + 1] = -np.inf
+    x[352:384] = np.float32(65504.0 * 127.0)        # f16 scale exactly max finite
+    s, q = hip.quantize_q8_0(x)
+    s0, q0 = orc.quantize_q8_0(x)
+    assert np.array_equal(s.view(np.uint32), s0.view(np.uint32)), (s, s0)
+    assert np.array_equal(q, q0)
+
+
+def test_quantize_rejects_bad_length(hip):
+    from cera_amd.hip_api import HipError
+    with pytest.raises(HipError):
+        hip.quantize_q8_0(np.zeros(33, np.float32))
+    with pytest.raises(HipError):
+        hip.quantize_q8_0(np.zeros(0, np.float32))
+
+
+# ---- GEMV ------------------------------------------------------------------------
+def _check_gemv(hip, orc, dtype, m, k, seed, debug=True):
+    _say(f"gemv {util.NAMES[dtype]} m={m} k={k} seed={seed}")
+    w, _ = util.make_weights(dtype, m, k, seed)
+    x = util.make_x(k, seed + 1000)
+    ref = orc.gemv(dtype, w, x, m, k)
+    if debug:
+        y, dots, asums = hip.gemv(dtype, w, x, m, k, debug=True)
+        _, xq = orc.quantize_q8_0(x)
+        dots0, asums0 = orc.block_dots(dtype, w, m, k, xq)
+        assert np.array_equal(dots, dots0), "per-block int32 dots differ"
+        if dtype in (Q4_1, Q4_K, Q6_K):
+            assert np.array_equal(asums, asums0), "activation sums differ"
+    y2 = hip.gemv(dtype, w, x, m, k)
+    err = np.abs(y2.astype(np.float64) - ref).max()
+    assert err <= GEMV_TOL * util.rms(ref), (err, util.rms(ref))
+    if debug:
+        assert np.array_equal(y.view(np.uint32), y2.view(np.uint32)), "debug and production kernels disagree"
+    return err / util.rms(ref)
+
+
+@pytest.mark.parametrize("dtype", util.INT8_TYPES)
+@pytest.mark.parametrize("m,k", [(7, 256), (64, 512), (33, 1024), (130, 4096), (9, 14336), (1, 2048), (5, 11008 // 256 * 256)])
+def test_gemv_small_shapes(hip, orc, dtype, m, k):
+    _check_gemv(hip, orc, dtype, m, k, seed=dtype * 100 + m)
+
+
+def test_gemv_config1_q4_0_4096(hip, orc):
+    # BASELINE config 1: single Q4_0 GEMV, 4096 x 4096
+    rel = _check_gemv(hip, orc, Q4_0, 4096, 4096, seed=11)
+    _say(f"  config1 max|err|/rms = {rel:.2e}")
+
+
+@pytest.mark.parametrize("dtype,m,k", [(Q4_K, 6144, 4096), (Q4_K, 4096, 4096), (Q4_K, 14336, 4096),
+                                       (Q6_K, 4096, 14336)])
+def test_gemv_config2_llama3_shapes(hip, orc, dtype, m, k):
+    rel = _check_gemv(hip, orc, dtype, m, k, seed=21 + m % 97, debug=False)
+    _say(f"  {util.NAMES[dtype]} {m}x{k} max|err|/rms = {rel:.2e}")
+
+
+def test_gemv_config2_head_rows_sampled(hip, orc):
+    """Output head 128256 x 4096 Q6_K: full GPU result, oracle on a row sample."""
+    m, k = 128256, 4096
+    _say("gemv Q6_K head 128256x4096")
+    r = util.rng(5)
+    base = (r.standard_normal((2048, k)) * 0.02).astype(np.float32)
+    wb = util.H.quantize(Q6_K, base, 8).reshape(2048, -1)
+    reps = (m + 2047) // 2048
+    w = np.ascontiguousarray(np.tile(wb, (reps, 1))[:m])
+    # make rows distinct: permute blocks of rows with a roll per repetition
+    for i in range(1, reps):
+        seg = w[i * 2048:min(m, (i + 1) * 2048)]
+        seg[:] = np.roll(wb, i * 7, axis=0)[:seg.shape[0]]
+    x = util.make_x(k, 6)
+    y = hip.gemv(Q6_K, w.reshape(-1), x, m, k)
+    rows = np.unique(np.concatenate([np.arange(0, 64), r.integers(0, m, 512), np.arange(m - 64, m)]))
+    ref = orc.gemv(Q6_K, np.ascontiguousarray(w[rows]).reshape(-1), x, rows.size, k)
+    err = np.abs(y[rows].astype(np.float64) - ref).max()
+    assert err <= GEMV_TOL * util.rms(ref)
+
+
+def test_gemv_q5k_f32_activation_path(hip, orc):
+    # Q5_K dots against unquantized f32 x on both sides (cpu.rs:1830-1854)
+    for m, k in [(9, 512), (64, 4096)]:
+        _say(f"gemv Q5_K m={m} k={k}")
+        w, _ = util.make_weights(Q5_K, m, k, seed=31)
+        x = util.make_x(k, 32)
+        y = hip.gemv(Q5_K, w, x, m, k)
+        ref = orc.gemv(Q5_K, w, x, m, k)
+        assert np.abs(y.astype(np.float64) - ref).max() <= GEMV_TOL * util.rms(ref)
+
+
+def test_gemv_weight_extremes(hip, orc):
+    """Q8_0 weights at -128 / 127 against activations at +-127 (simd.rs:6436-6475)."""
+    m, k = 8, 256
+    _say("gemv Q8_0 extremes")
+    blocks = np.zeros((m * k // 32, 34), np.uint8)
+    blocks[:, 0:2] = np.array([0.01], np.float16).view(np.uint8)
+    q = util.rng(9).integers(-128, 128, size=(m * k // 32, 32)).astype(np.int8)
+    q[:, 0:2] = -128
+    q[:, 2:4] = 127
+    blocks[:, 2:] = q.view(np.uint8)
+    x = util.make_x(k, 10)
+    x[0::32] = 10.0   # forces +-127 quants at the head of each block
+    x[1::32] = 10.0
+    x[2::32] = -10.0
+    y, dots, _ = hip.gemv(Q8_0, blocks.reshape(-1), x, m, k, debug=True)
+    _, xq = orc.quantize_q8_0(x)
+    dots0, _ = orc.block_dots(Q8_0, blocks.reshape(-1), m, k, xq)
+    assert np.array_equal(dots, dots0)
+    ref = orc.gemv(Q8_0, blocks.reshape(-1), x, m, k)
+    assert np.abs(y - ref).max() <= GEMV_TOL * util.rms(ref)
+
+
+def test_gemv_refuses_unsupported(hip):
+    from cera_amd.hip_api import HipError
+    with pytest.raises(HipError) as e:
+        hip.gemv(7, np.zeros(64, np.uint8), np.zeros(32, np.float32), 2, 32)   # unknown ggml type
+    assert e.value.status == 3
+    with pytest.raises(HipError) as e:
+        hip.gemv(Q4_K, np.zeros(144, np.uint8), np.zeros(100, np.float32), 1, 100)  # k not a block multiple
+    assert e.value.status == 4
+    with pytest.raises(HipError) as e:   # wrong byte count
+        hip.gemv(Q4_0, np.zeros(18, np.uint8), np.zeros(64, np.float32), 1, 64)
+    assert e.value.status == 4
+
+
+# ---- glue ops -------------------------------------------------------------------
+def test_rmsnorm_bit_exact(hip, orc):
+    for n, seed in [(4096, 1), (128, 2), (14336, 3), (256, 4)]:
+        _say(f"rmsnorm n={n}")
+        x = util.make_x(n, seed) * 3
+        w = util.make_x(n, seed + 10)
+        y = hip.rmsnorm(x, w, 1e-5)
+        ref = orc.rmsnorm(x, w, 1e-5)
+        assert np.array_equal(y.view(np.uint32), ref.view(np.uint32))
+
+
+def test_silu_mul_bit_exact(hip, orc):
+    _say("silu_mul")
+    g = util.make_x(14336, 5) * 6
+    u = util.make_x(14336, 6)
+    g[:8] = [0.0, -0.0, 100.0, -100.0, 88.5, -88.5, -104.0, 20.0]
+    y = hip.silu_mul(g, u)
+    ref = orc.silu_mul(g, u)
+    assert np.array_equal(y.view(np.uint32), ref.view(np.uint32))
+
+
+@pytest.mark.parametrize("norm", [True, False])
+def test_rope_bit_exact(hip, orc, norm):
+    nh, nkv, hd = 32, 8, 128
+    for pos in (0, 1, 17, 511, 4095):
+        _say(f"rope norm={norm} pos={pos}")
+        q = util.make_x(nh * hd, 40 + pos)
+        k = util.make_x(nkv * hd, 41 + pos)
+        qa, ka = hip.rope(q, k, pos, nh, nkv, hd, 500000.0, norm)
+        qb, kb = orc.rope(q, k, pos, nh, nkv, hd, 500000.0, norm)
+        assert np.array_equal(qa.view(np.uint32), qb.view(np.uint32))
+        assert np.array_equal(ka.view(np.uint32), kb.view(np.uint32))
+
+
+def test_argmax_rules(hip, orc):
+    _say("argmax")
+    r = util.rng(3)
+    for n in (1, 7, 1024, 128256):
+        x = r.standard_normal(n).astype(np.float32)
+        assert hip.argmax(x) == orc.argmax(x)
+    x = np.zeros(5000, np.float32); x[[100, 4000, 77]] = 5.0
+    assert hip.argmax(x) == 77                         # lowest index on ties
+    x = np.full(3000, np.nan, np.float32); x[2500] = -3.0; x[2900] = -3.0
+    assert hip.argmax(x) == 2500                       # NaN never wins
+    assert hip.argmax(np.full(100, np.nan, np.float32)) == 0
+    assert hip.argmax(np.full(100, -np.inf, np.float32)) == 0
+    assert hip.argmax(np.zeros(0, np.float32)) == 0
+
+
+@pytest.mark.parametrize("dtype", util.ALL_TYPES)
+def test_dequantize_row_bit_exact(hip, orc, dtype):
+    _say(f"dequantize_row {util.NAMES[dtype]}")
+    m, k = 6, 1024
+    w, _ = util.make_weights(dtype, m, k, seed=50 + dtype, sigma=0.3)
+    ref = orc.dequantize(dtype, w, m, k)
+    for row in (0, 3, 5):
+        out = hip.dequantize_row(dtype, w, m, k, row)
+        assert np.array_equal(out.view(np.uint32), ref[row].view(np.uint32))
+
+
+# ---- decode attention ----------------------------------------------------------------
+@pytest.mark.parametrize("L", [1, 2, 63, 64, 65, 512, 1000, 4096])
+def test_attn_decode_vs_oracle(hip, orc, L):
+    nh, nkv, hd = 32, 8, 128
+    _say(f"attn_decode L={L}")
+    q = util.make_x(nh * hd, 60)
+    k = util.make_x(L * nkv * hd, 61 + L)
+    v = util.make_x(L * nkv * hd, 62 + L)
+    scale = 1.0 / math.sqrt(hd)
+    out = hip.attn_decode(q, k, v, nh, nkv, hd, L, scale)
+    ref = orc.decode_attention(q, k, v, nh, nkv, hd, scale, L)
+    err = np.abs(out.astype(np.float64) - ref).max()
+    assert err <= ATTN_TOL * util.rms(ref), (err, util.rms(ref))
+
+
+@pytest.mark.parametrize("splits", [1, 3, 16, 1000])
+def test_attn_decode_split_invariance(hip, orc, splits):
+    nh, nkv, hd, L = 32, 8, 128, 777
+    _say(f"attn_decode splits={splits}")
+    q = util.make_x(nh * hd, 70)
+    k = util.make_x(L * nkv * hd, 71)
+    v = util.make_x(L * nkv * hd, 72)
+    out = hip.attn_decode(q, k, v, nh, nkv, hd, L, 0.088, n_splits=splits)
+    ref = orc.decode_attention(q, k, v, nh, nkv, hd, 0.088, L)
+    assert np.abs(out - ref).max() <= ATTN_TOL * util.rms(ref)
+
+
+def test_attn_decode_peaked_softmax(hip, orc):
+    """One dominant key (large logit) and large-magnitude scores: online softmax must not overflow."""
+    nh, nkv, hd, L = 8, 2, 128, 300
+    _say("attn_decode peaked")
+    q = util.make_x(nh * hd, 80) * 4
+    k = util.make_x(L * nkv * hd, 81)
+    v = util.make_x(L * nkv * hd, 82)
+    k.reshape(L, nkv, hd)[200] = q.reshape(nh, hd)[::4] * 2   # aligned with q heads 0 and 4
+    out = hip.attn_decode(q, k, v, nh, nkv, hd, L, 1.0)
+    ref = orc.decode_attention(q, k, v, nh, nkv, hd, 1.0, L)
+    assert np.all(np.isfinite(out))
+    assert np.abs(out - ref).max() <= ATTN_TOL * util.rms(ref)
+
+
+def test_attn_decode_gqa_groupings(hip, orc):
+    hd, L = 128, 130
+    for nh, nkv in [(8, 8), (8, 4), (16, 2), (4, 1)]:
+        _say(f"attn_decode nh={nh} nkv={nkv}")
+        if nh // nkv not in (1, 2, 4, 8):
+            continue
+        q = util.make_x(nh * hd, 90)
+        k = util.make_x(L * nkv * hd, 91)
+        v = util.make_x(L * nkv * hd, 92)
+        out = hip.attn_decode(q, k, v, nh, nkv, hd, L, 0.1)
+        ref = orc.decode_attention(q, k, v, nh, nkv, hd, 0.1, L)
+        assert np.abs(out - ref).max() <= ATTN_TOL * util.rms(ref)

@@ -1,0 +1,149 @@
+"""GPU parity at the model level: device-resident llama forward vs the oracle's
+LlamaModel twin on the same seeded random-init weights."""
+import numpy as np
+import pytest
+
+import util
+from cera_amd import hip_api, synth
+
+pytestmark = pytest.mark.gpu
+
+
+def _say(msg):
+    print(msg, flush=True)
+
+
+def orc_argmax(l):
+    from oracle import binding
+    return binding.argmax(l)
+
+
+def _cos(a, b):
+    a = a.astype(np.float64); b = b.astype(np.float64)
+    return float(a @ b / np.sqrt((a @ a) * (b @ b)))
+
+
+@pytest.fixture(scope="module")
+def tiny(hip, orc):
+    cfg = dict(synth.TINY)
+    weights = synth.make_llama(cfg, seed=1234, sigma=0.05, norm_jitter=0.1)
+    gm = hip_api.Model(hip, cfg, weights)
+    om = orc.Llama(cfg, weights)
+    yield cfg, weights, gm, om
+    gm.close()
+    om.close()
+
+
+def test_single_token_logits_and_kv(tiny):
+    cfg, weights, gm, om = tiny
+    gm.truncate_kv(0); om.truncate(0)
+    _say("model: forward token 17 @0")
+    lg = gm.forward(17, 0)
+    lo = om.forward(17, 0)
+    err = np.abs(lg - lo).max()
+    _say(f"  logits max|err|={err:.3e} rms={util.rms(lo):.3e} cos={_cos(lg, lo):.8f}")
+    assert err <= 1e-3 * util.rms(lo) * 10 or _cos(lg, lo) > 0.99999
+    for layer in range(cfg["n_layers"]):
+        kg, vg = gm.read_kv(layer)
+        ko, vo = om.kv(layer)
+        assert np.abs(kg - ko).max() <= 2e-3 * util.rms(ko) + 1e-6
+        assert np.abs(vg - vo).max() <= 2e-3 * util.rms(vo) + 1e-6
+
+
+def test_greedy_decode_matches_oracle_tokens(tiny):
+    """Greedy decode, teacher-forced on the oracle's tokens.
+
+    The int8 path re-quantizes activations to Q8_0 before every projection.  A
+    last-bit difference in an f32 activation (the GPU sums partial products in a
+    different order than the CPU's eight-lane FMA chains) can land on the other
+    side of a rounding tie and move one int8 code by one step; that changes the
+    logits by ~LSB/sqrt(hidden) and is inherent to any second implementation,
+    including the reference's own GPU backends, whose parity test is near-tie
+    tolerant for this reason (cera/tests/gpu_transformer_parity.rs:5-13).  So:
+    logits must stay close at every step, and the token must be identical
+    whenever the oracle's top-1/top-2 margin exceeds the observed logit error.
+    """
+    cfg, weights, gm, om = tiny
+    gm.truncate_kv(0); om.truncate(0)
+    prompt = [3, 99, 250, 7, 42]
+    _say("model: prefill + greedy 32 (teacher forced)")
+    lg = gm.forward_prefill(prompt, 0)
+    lo = om.forward_prefill_per_token(prompt, 0)
+    assert gm.seq_len == om.seq_len == len(prompt)
+    same = ties = 0
+    tok = orc_argmax(lo)
+    for i in range(32):
+        err = float(np.abs(lg - lo).max())
+        s = np.sort(lo)
+        margin = float(s[-1] - s[-2])
+        assert _cos(lg, lo) > 0.999, (i, _cos(lg, lo))
+        assert err <= 0.1 * util.rms(lo), (i, err)
+        tg, to = int(orc_argmax(lg)), int(orc_argmax(lo))
+        if tg == to:
+            same += 1
+        else:
+            ties += 1
+            assert margin <= 2 * err, f"step {i}: tokens differ ({tg} vs {to}) with margin {margin} > 2*err {err}"
+        tok = to
+        pos = len(prompt) + i
+        lg = gm.forward(tok, pos)
+        lo = om.forward(tok, pos)
+    _say(f"  identical tokens {same}/32, near-tie disagreements {ties}")
+    assert same >= 28
+
+
+def test_greedy_free_running_prefix(tiny):
+    """Free-running greedy decode on both sides: identical until the first
+    near-tie (where the oracle's own margin is below the logit error)."""
+    cfg, weights, gm, om = tiny
+    gm.truncate_kv(0); om.truncate(0)
+    tg = to = 11
+    n_same = 0
+    for pos in range(24):
+        lo = om.forward(to, pos)
+        to = int(orc_argmax(lo))
+        tg = gm.forward_greedy(tg, pos)
+        if tg != to:
+            s = np.sort(lo)
+            _say(f"  diverged at step {pos}: margin {float(s[-1] - s[-2]):.3e}")
+            assert float(s[-1] - s[-2]) < 0.05 * util.rms(lo)
+            break
+        n_same += 1
+    _say(f"  free-running identical prefix: {n_same} tokens")
+    assert n_same >= 2
+
+
+def test_position_contract(tiny):
+    cfg, weights, gm, om = tiny
+    gm.truncate_kv(0)
+    gm.forward(1, 0)
+    with pytest.raises(hip_api.HipError) as e:
+        gm.forward(1, 5)          # pos must equal seq_len
+    assert e.value.status == 5
+    with pytest.raises(hip_api.HipError) as e:
+        gm.forward_prefill([1, 2], 0)
+    assert e.value.status == 5
+    with pytest.raises(hip_api.HipError) as e:
+        gm.forward(cfg["vocab"], 1)   # token out of range
+    assert e.value.status == 6
+    assert gm.seq_len == 1
+    gm.truncate_kv(0)
+    assert gm.seq_len == 0
+    assert gm.memory_bytes > 0
+
+
+def test_model_create_refuses_bad_shapes(hip):
+    cfg = dict(synth.TINY)
+    weights = synth.make_llama(cfg, seed=1)
+    bad = dict(weights)
+    t, m, k, arr = bad["blk.0.attn_q.weight"]
+    bad["blk.0.attn_q.weight"] = (t, m // 2, k, arr[: arr.size // 2])
+    with pytest.raises(hip_api.HipError) as e:
+        hip_api.Model(hip, cfg, bad)
+    assert e.value.status == 4 and "attn_q" in e.value.message
+    bad = dict(weights)
+    t, m, k, arr = bad["blk.1.ffn_up.weight"]
+    bad["blk.1.ffn_up.weight"] = (0, m, k, np.zeros(m * k * 4, np.uint8))   # F32 matrix: no GEMV kernel
+    with pytest.raises(hip_api.HipError) as e:
+        hip_api.Model(hip, cfg, bad)
+    assert e.value.status == 3
