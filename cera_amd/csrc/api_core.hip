@@ -9,11 +9,11 @@
 #include "host_common.h"
 #include "quantize.cuh"
 
-bool cera_gemv_launch_q4k(const GemvArgs&, int, int, int, bool, dim3, hipStream_t);
-bool cera_gemv_launch_q6k(const GemvArgs&, int, int, int, bool, dim3, hipStream_t);
-bool cera_gemv_launch_q4_0(const GemvArgs&, int, int, int, bool, dim3, hipStream_t);
-bool cera_gemv_launch_q4_1(const GemvArgs&, int, int, int, bool, dim3, hipStream_t);
-bool cera_gemv_launch_q8_0(const GemvArgs&, int, int, int, bool, dim3, hipStream_t);
+bool cera_gemv_launch_q4k(const GemvArgs&, const GemvPlan&, int, bool, hipStream_t);
+bool cera_gemv_launch_q6k(const GemvArgs&, const GemvPlan&, int, bool, hipStream_t);
+bool cera_gemv_launch_q4_0(const GemvArgs&, const GemvPlan&, int, bool, hipStream_t);
+bool cera_gemv_launch_q4_1(const GemvArgs&, const GemvPlan&, int, bool, hipStream_t);
+bool cera_gemv_launch_q8_0(const GemvArgs&, const GemvPlan&, int, bool, hipStream_t);
 
 // ---------------------------------------------------------------------------
 static std::mutex g_err_mu;
@@ -295,7 +295,8 @@ cera_hip_status cera_launch_gemv(cera_hip_ctx* ctx, const cera_hip_dtensor* w, c
             return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "fused gate/up gemv needs two matrices of identical type and shape");
     }
     if (epi == CERA_EPI_ADD && !resid) return cera_fail(ctx, CERA_HIP_ERR_ARGUMENT, "residual pointer is null");
-    uint32_t n_units = static_cast<uint32_t>(w->k / 32);  // every format uses one unit per 32 weights
+    // unit = 32 weights, except Q6_K whose lanes take 64
+    uint32_t n_units = static_cast<uint32_t>(w->k / (w->dtype == CERA_HIP_Q6_K ? Q6K::ELEMS_PER_UNIT : 32));
     GemvArgs a;
     a.w = w->dev;
     a.w2 = w2 ? w2->dev : nullptr;
@@ -309,18 +310,18 @@ cera_hip_status cera_launch_gemv(cera_hip_ctx* ctx, const cera_hip_dtensor* w, c
     a.dbg_dots = dbg_dots;
     a.dbg_asums = dbg_asums;
     a.dbg_stride = static_cast<uint32_t>(w->dtype == CERA_HIP_Q6_K ? w->k / 16 : w->k / 32);
-    GemvPlan p = gemv_plan(a.m, n_units, ctx->n_cu, dbg_dots != nullptr);
-    if (p.U == 0)
-        return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "gemv: k=" + std::to_string(w->k) + " exceeds the 16384 supported by the register-resident kernel");
-    a.rows_per_wave = p.rows_per_wave;
-    dim3 grid(p.n_blocks);
+    const bool dbg = dbg_dots != nullptr;
+    GemvPlan p;
+    if (!gemv_plan(a.m, n_units, ctx->n_cu, dbg, w->dtype == CERA_HIP_Q6_K ? 2 : 4, &p))
+        return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "gemv: k=" + std::to_string(w->k) + " exceeds the 32768 supported by the register-resident kernel");
+    a.rows_per_wave = p.rows_per_block;
     bool ok = false;
     switch (w->dtype) {
-        case CERA_HIP_Q4_K: ok = cera_gemv_launch_q4k(a, p.U, p.RB, epi, dbg_dots != nullptr, grid, ctx->stream); break;
-        case CERA_HIP_Q6_K: ok = cera_gemv_launch_q6k(a, p.U, p.RB, epi, dbg_dots != nullptr, grid, ctx->stream); break;
-        case CERA_HIP_Q4_0: ok = cera_gemv_launch_q4_0(a, p.U, p.RB, epi, dbg_dots != nullptr, grid, ctx->stream); break;
-        case CERA_HIP_Q4_1: ok = cera_gemv_launch_q4_1(a, p.U, p.RB, epi, dbg_dots != nullptr, grid, ctx->stream); break;
-        case CERA_HIP_Q8_0: ok = cera_gemv_launch_q8_0(a, p.U, p.RB, epi, dbg_dots != nullptr, grid, ctx->stream); break;
+        case CERA_HIP_Q4_K: ok = cera_gemv_launch_q4k(a, p, epi, dbg, ctx->stream); break;
+        case CERA_HIP_Q6_K: ok = cera_gemv_launch_q6k(a, p, epi, dbg, ctx->stream); break;
+        case CERA_HIP_Q4_0: ok = cera_gemv_launch_q4_0(a, p, epi, dbg, ctx->stream); break;
+        case CERA_HIP_Q4_1: ok = cera_gemv_launch_q4_1(a, p, epi, dbg, ctx->stream); break;
+        case CERA_HIP_Q8_0: ok = cera_gemv_launch_q8_0(a, p, epi, dbg, ctx->stream); break;
     }
     if (!ok) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "gemv: no kernel instance for this shape");
     HIP_TRY(ctx, hipGetLastError());
@@ -422,7 +423,8 @@ cera_hip_status cera_hip_gemv_seq_dev(cera_hip_ctx* ctx, const cera_hip_gemv_op*
     if (!ctx || (!ops && n)) return CERA_HIP_ERR_ARGUMENT;
     for (uint32_t i = 0; i < n; ++i) {
         if (!ops[i].w || !ops[i].xs || !ops[i].xq || !ops[i].y) return cera_fail(ctx, CERA_HIP_ERR_ARGUMENT, "gemv_seq: null field in op " + std::to_string(i));
-        CERA_TRY(cera_launch_gemv(ctx, ops[i].w, nullptr, ops[i].xs, ops[i].xq, ops[i].y, nullptr, CERA_EPI_STORE));
+        CERA_TRY(cera_launch_gemv(ctx, ops[i].w, ops[i].w2, ops[i].xs, ops[i].xq, ops[i].y, nullptr,
+                                  ops[i].w2 ? CERA_EPI_SILU_MUL : CERA_EPI_STORE));
     }
     return CERA_HIP_OK;
 }

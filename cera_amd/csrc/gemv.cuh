@@ -11,13 +11,15 @@
 //
 // Design: "activation-stationary lanes".  The K dimension is cut into
 // fixed-size *units* (16 B of Q4_K nibbles, 24 B of Q6_K codes, one Q4_0 /
-// Q4_1 / Q8_0 block).  Unit u of every row belongs to lane u % 64, so a lane
-// keeps the int8 activations, activation scales and activation sums of its
-// units in registers for the whole kernel and only streams weights.  A
-// wavefront walks a contiguous range of rows, RB rows at a time; for each row
-// its 64 lanes read one contiguous span of the row (coalesced 16/8-byte
-// loads), so HBM sees pure sequential streams.  Per row the 64 partial sums
-// are combined with a DPP reduction.  No LDS, no atomics.
+// Q4_1 / Q8_0 block).  A workgroup is KS wavefronts that split K between them:
+// wavefront kw owns units kw*64 .. kw*64+63 (+ 64*KS*i for i < U), one per
+// lane, so a lane keeps the int8 activations, activation scales and activation
+// sums of its units in registers for the whole kernel and only streams weights.
+// The workgroup walks a contiguous range of rows, RB rows at a time; for each
+// row its lanes read one contiguous span of the row (coalesced 16/8-byte
+// loads), so HBM sees pure sequential streams.  Per row each wavefront reduces
+// its 64 partial sums with DPP; the KS per-wavefront sums meet in LDS and are
+// added in wavefront order (deterministic, no atomics).
 #pragma once
 #include "common.cuh"
 
@@ -31,7 +33,7 @@ struct GemvArgs {
     uint32_t m;
     uint32_t n_units;        // units per row
     uint32_t row_bytes;
-    uint32_t rows_per_wave;
+    uint32_t rows_per_wave;  // rows per workgroup
     int32_t* dbg_dots;   // nullable: integer block dots, layout per type
     uint32_t dbg_stride; // ints per row in dbg_dots
     int32_t* dbg_asums;  // nullable: integer activation sums per 32 (Q6_K: per 16)
@@ -43,26 +45,31 @@ enum { EPI_STORE = 0, EPI_ADD = 1, EPI_SILU_MUL = 2 };
 // Q4_K: unit = 16 bytes of qs (32 nibbles): 16 codes of sub-block 2g (low
 // nibbles) and 16 of sub-block 2g+1 (high nibbles); 8 units per 144-byte block.
 struct Q4K {
-    static constexpr int UNITS_PER_BLOCK = 8;
+    static constexpr int ELEMS_PER_UNIT = 32;
     struct Act { uint32_t lo[4], hi[4]; float xs0, xs1, c0, c1; int s0, s1; };
     struct Wt { uint4 q; uint4 h; };
     __device__ static void dbg_asum(const Act& a, uint32_t u, int32_t* out) {
         atomicAdd(out + (u >> 3) * 8 + ((u >> 1) & 3) * 2, a.s0);
         atomicAdd(out + (u >> 3) * 8 + ((u >> 1) & 3) * 2 + 1, a.s1);
     }
+    // `u` is always a valid unit (dead lanes pass unit 0); `live` zeroes the result,
+    // so the loads themselves are unconditional 16-byte loads.
     __device__ static void load_act(Act& a, const int8_t* xq, const float* xs, uint32_t u, bool live) {
         uint32_t b = u >> 3, w8 = u & 7, g = w8 >> 1, h = w8 & 1;
-        const uint32_t* p = reinterpret_cast<const uint32_t*>(xq + b * 256 + g * 64 + h * 16);
+        const uint4 lo = *reinterpret_cast<const uint4*>(xq + b * 256 + g * 64 + h * 16);
+        const uint4 hi = *reinterpret_cast<const uint4*>(xq + b * 256 + g * 64 + h * 16 + 32);
+        const float2 sc = *reinterpret_cast<const float2*>(xs + b * 8 + 2 * g);
+        const uint32_t keep = live ? 0xFFFFFFFFu : 0u;
+        a.lo[0] = lo.x & keep; a.lo[1] = lo.y & keep; a.lo[2] = lo.z & keep; a.lo[3] = lo.w & keep;
+        a.hi[0] = hi.x & keep; a.hi[1] = hi.y & keep; a.hi[2] = hi.z & keep; a.hi[3] = hi.w & keep;
         int s0 = 0, s1 = 0;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            a.lo[i] = live ? p[i] : 0u;
-            a.hi[i] = live ? p[8 + i] : 0u;
             s0 = sum4(a.lo[i], s0);
             s1 = sum4(a.hi[i], s1);
         }
-        a.xs0 = live ? xs[b * 8 + 2 * g] : 0.0f;
-        a.xs1 = live ? xs[b * 8 + 2 * g + 1] : 0.0f;
+        a.xs0 = live ? sc.x : 0.0f;
+        a.xs1 = live ? sc.y : 0.0f;
         // xs has an 11-bit significand and |s| <= 16*127: the products are exact.
         a.c0 = a.xs0 * static_cast<float>(s0);
         a.c1 = a.xs1 * static_cast<float>(s1);
@@ -79,8 +86,11 @@ struct Q4K {
         // 6-bit scales/mins of sub-blocks 2g, 2g+1 (get_scale_min_k4)
         uint32_t sh = 16 * (g & 1);
         uint32_t y2 = (w.h.y >> sh) & 0xFFFF, z2 = (w.h.z >> sh) & 0xFFFF, w2 = (w.h.w >> sh) & 0xFFFF;
-        uint32_t sc2 = g < 2 ? (y2 & 0x3F3F) : ((w2 & 0x0F0F) | ((y2 >> 2) & 0x3030));
-        uint32_t mn2 = g < 2 ? (z2 & 0x3F3F) : (((w2 >> 4) & 0x0F0F) | ((z2 >> 2) & 0x3030));
+        // branch-free select between the two packings (low sub-blocks keep 6 bits in
+        // place; high ones splice a nibble of bytes 8..11 with the top two bits)
+        const uint32_t low = g < 2 ? 0xFFFFFFFFu : 0u;
+        uint32_t sc2 = ((y2 & 0x3F3F) & low) | (((w2 & 0x0F0F) | ((y2 >> 2) & 0x3030)) & ~low);
+        uint32_t mn2 = ((z2 & 0x3F3F) & low) | ((((w2 >> 4) & 0x0F0F) | ((z2 >> 2) & 0x3030)) & ~low);
         float d = h2f(w.h.x & 0xFFFF), dmin = h2f(w.h.x >> 16);
         int dl = 0, dh = 0;
         const uint32_t q[4] = {w.q.x, w.q.y, w.q.z, w.q.w};
@@ -102,46 +112,50 @@ struct Q4K {
 };
 
 // ---------------------------------------------------------------------------
-// Q6_K: unit = 8 consecutive positions l0..l0+7 of one 128-element half:
-// 8 B of ql (low half), 8 B of ql (+32), 8 B of qh -> 32 six-bit codes in four
-// runs of 8 (elements +0, +32, +64, +96); 8 units per 210-byte block.
+// Q6_K: unit = 16 consecutive positions l0..l0+15 of one 128-element half:
+// 16 B of ql (low half), 16 B of ql (+32), 16 B of qh -> 64 six-bit codes in
+// four runs of 16 (elements +0, +32, +64, +96), each run with its own int8
+// scale; 4 units per 210-byte block.  Blocks are only 2-byte aligned.
 struct Q6K {
-    static constexpr int UNITS_PER_BLOCK = 8;
-    struct Act { uint32_t a[4][2]; float xs[4]; int init[4]; };
-    struct Wt { uint2 qa, qb, qh, sc; uint32_t d; };
+    static constexpr int ELEMS_PER_UNIT = 64;
+    struct Act { uint32_t a[4][4]; float xs[4]; int init[4]; };
+    struct Wt { uint4 qa, qb, qh; uint2 sc; uint32_t d; };
     __device__ static void dbg_asum(const Act& a, uint32_t u, int32_t* out) {
-        uint32_t base = (u >> 3) * 16 + ((u >> 2) & 1) * 8 + ((u >> 1) & 1);
+        uint32_t base = (u >> 2) * 16 + ((u >> 1) & 1) * 8 + (u & 1);
 #pragma unroll
-        for (int t = 0; t < 4; ++t) atomicAdd(out + base + 2 * t, a.init[t] / -32);
+        for (int t = 0; t < 4; ++t) out[base + 2 * t] = a.init[t] / -32;
     }
     __device__ static void load_act(Act& a, const int8_t* xq, const float* xs, uint32_t u, bool live) {
-        uint32_t b = u >> 3, nh = (u >> 2) & 1, j = u & 3;
-        const int8_t* base = xq + b * 256 + nh * 128 + j * 8;
+        uint32_t b = u >> 2, nh = (u >> 1) & 1, j = u & 1;
+        const int8_t* base = xq + b * 256 + nh * 128 + j * 16;
+        const float4 sc = *reinterpret_cast<const float4*>(xs + b * 8 + nh * 4);
+        const float scv[4] = {sc.x, sc.y, sc.z, sc.w};
+        const uint32_t keep = live ? 0xFFFFFFFFu : 0u;
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
-            const uint32_t* p = reinterpret_cast<const uint32_t*>(base + 32 * t);
-            a.a[t][0] = live ? p[0] : 0u;
-            a.a[t][1] = live ? p[1] : 0u;
-            a.xs[t] = live ? xs[b * 8 + nh * 4 + t] : 0.0f;
+            const uint4 v = *reinterpret_cast<const uint4*>(base + 32 * t);
+            a.a[t][0] = v.x & keep; a.a[t][1] = v.y & keep; a.a[t][2] = v.z & keep; a.a[t][3] = v.w & keep;
+            a.xs[t] = live ? scv[t] : 0.0f;
             // codes are stored +32: start each dot at -32 * sum(a)
-            a.init[t] = -32 * sum4(a.a[t][1], sum4(a.a[t][0], 0));
+            a.init[t] = -32 * sum4(a.a[t][3], sum4(a.a[t][2], sum4(a.a[t][1], sum4(a.a[t][0], 0))));
         }
     }
     __device__ static void load_w(Wt& w, const uint8_t* row, uint32_t u) {
-        const uint8_t* blk = row + (u >> 3) * 210;
-        uint32_t nh = (u >> 2) & 1, j = u & 3;
-        w.qa = ld_u64_a2(blk + nh * 64 + j * 8);
-        w.qb = ld_u64_a2(blk + nh * 64 + 32 + j * 8);
-        w.qh = ld_u64_a2(blk + 128 + nh * 32 + j * 8);
+        const uint8_t* blk = row + (u >> 2) * 210;
+        uint32_t nh = (u >> 1) & 1, j = u & 1;
+        w.qa = ld_u128_a2(blk + nh * 64 + j * 16);
+        w.qb = ld_u128_a2(blk + nh * 64 + 32 + j * 16);
+        w.qh = ld_u128_a2(blk + 128 + nh * 32 + j * 16);
         w.sc = ld_u64_a2(blk + 192 + nh * 8);
         w.d = ld_u16(blk + 208);
     }
     __device__ static float dot(const Wt& w, const Act& a, uint32_t u, int32_t* dbg) {
-        uint32_t is = (u >> 1) & 1;  // (l0 / 16) with l0 = 8 * (u & 3)
+        uint32_t is = u & 1;  // l0 / 16
         int acc[4] = {a.init[0], a.init[1], a.init[2], a.init[3]};
-        const uint32_t qa[2] = {w.qa.x, w.qa.y}, qb[2] = {w.qb.x, w.qb.y}, qh[2] = {w.qh.x, w.qh.y};
+        const uint32_t qa[4] = {w.qa.x, w.qa.y, w.qa.z, w.qa.w}, qb[4] = {w.qb.x, w.qb.y, w.qb.z, w.qb.w},
+                       qh[4] = {w.qh.x, w.qh.y, w.qh.z, w.qh.w};
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
+        for (int i = 0; i < 4; ++i) {
             uint32_t q0 = (qa[i] & 0x0F0F0F0Fu) | ((qh[i] << 4) & 0x30303030u);
             uint32_t q1 = (qb[i] & 0x0F0F0F0Fu) | ((qh[i] << 2) & 0x30303030u);
             uint32_t q2 = ((qa[i] >> 4) & 0x0F0F0F0Fu) | (qh[i] & 0x30303030u);
@@ -153,9 +167,9 @@ struct Q6K {
         }
         if (dbg) {
             // report the unsigned dot (sum q*a, q in 0..63) per 16-element run
-            uint32_t base = (u >> 3) * 16 + ((u >> 2) & 1) * 8 + is;
+            uint32_t base = (u >> 2) * 16 + ((u >> 1) & 1) * 8 + is;
 #pragma unroll
-            for (int t = 0; t < 4; ++t) atomicAdd(dbg + base + 2 * t, acc[t] - a.init[t]);
+            for (int t = 0; t < 4; ++t) dbg[base + 2 * t] = acc[t] - a.init[t];
         }
         // scales nh*8 + is + {0, 2, 4, 6}: bytes is, is+2 of each dword
         uint32_t slo = w.sc.x >> (8 * is), shi = w.sc.y >> (8 * is);
@@ -176,19 +190,23 @@ struct Q6K {
 struct ActB32 { uint32_t a[8]; float xs; int asum; };
 __device__ __forceinline__ void dbg_asum_b32(const ActB32& a, uint32_t u, int32_t* out) { out[u] = a.asum; }
 __device__ __forceinline__ void load_act_b32(ActB32& a, const int8_t* xq, const float* xs, uint32_t u, bool live) {
-    const uint32_t* p = reinterpret_cast<const uint32_t*>(xq + u * 32);
+    const uint4 v0 = *reinterpret_cast<const uint4*>(xq + u * 32);
+    const uint4 v1 = *reinterpret_cast<const uint4*>(xq + u * 32 + 16);
+    const uint32_t keep = live ? 0xFFFFFFFFu : 0u;
+    const uint32_t v[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
     int s = 0;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-        a.a[i] = live ? p[i] : 0u;
+        a.a[i] = v[i] & keep;
         s = sum4(a.a[i], s);
     }
-    a.xs = live ? xs[u] : 0.0f;
+    const float t = xs[u];
+    a.xs = live ? t : 0.0f;
     a.asum = s;
 }
 
 struct Q4_0 {  // 18 B: d, qs[16]; byte i = element i (low nibble), element i+16 (high); code - 8
-    static constexpr int UNITS_PER_BLOCK = 1;
+    static constexpr int ELEMS_PER_UNIT = 32;
     using Act = ActB32;
     __device__ static void dbg_asum(const Act& a, uint32_t u, int32_t* out) { dbg_asum_b32(a, u, out); }
     struct Wt { uint4 q; uint32_t d; };
@@ -214,7 +232,7 @@ struct Q4_0 {  // 18 B: d, qs[16]; byte i = element i (low nibble), element i+16
 };
 
 struct Q4_1 {  // 20 B: d, m, qs[16]; value = q*d + m
-    static constexpr int UNITS_PER_BLOCK = 1;
+    static constexpr int ELEMS_PER_UNIT = 32;
     using Act = ActB32;
     __device__ static void dbg_asum(const Act& a, uint32_t u, int32_t* out) { dbg_asum_b32(a, u, out); }
     struct Wt { uint4 q; uint32_t dm; };
@@ -241,7 +259,7 @@ struct Q4_1 {  // 20 B: d, m, qs[16]; value = q*d + m
 };
 
 struct Q8_0 {  // 34 B: d, int8[32]
-    static constexpr int UNITS_PER_BLOCK = 1;
+    static constexpr int ELEMS_PER_UNIT = 32;
     using Act = ActB32;
     __device__ static void dbg_asum(const Act& a, uint32_t u, int32_t* out) { dbg_asum_b32(a, u, out); }
     struct Wt { uint4 q0, q1; uint32_t d; };
@@ -265,68 +283,123 @@ struct Q8_0 {  // 34 B: d, int8[32]
 };
 
 // ---------------------------------------------------------------------------
-// The kernel.  U = units per lane held in registers (ceil(n_units / 64)),
-// RB = rows in flight per wavefront, EPI = epilogue.
-template <class T, int U, int RB, int EPI, bool DBG>
-static __global__ __launch_bounds__(256) void gemv_kernel(GemvArgs p) {
-    const uint32_t lane = threadIdx.x & 63;
-    const uint32_t wave = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
-    uint32_t r0 = wave * p.rows_per_wave;
-    if (r0 >= p.m) return;
-    uint32_t r1 = min(p.m, r0 + p.rows_per_wave);
-
-    typename T::Act act[U];
-    uint32_t unit[U];
-#pragma unroll
-    for (int i = 0; i < U; ++i) {
-        uint32_t u = lane + 64 * i;
-        bool live = u < p.n_units;
-        unit[i] = live ? u : 0;  // dead lanes re-read unit 0 with zeroed activations
-        T::load_act(act[i], p.xq, p.xs, unit[i], live);
-        if (DBG && wave == 0 && live && p.dbg_asums) T::dbg_asum(act[i], u, p.dbg_asums);
-    }
-
-    constexpr int NM = EPI == EPI_SILU_MUL ? 2 : 1;
-    for (uint32_t r = r0; r < r1; r += RB) {
-        typename T::Wt wt[NM][RB][U];
+// The kernel.  U = units per lane, KS = wavefronts per workgroup (K split),
+// RB = rows in flight per workgroup, EPI = epilogue.
+//
+// Latency structure: a wavefront first issues the weight loads of its first row
+// group, then loads its activations (so the two memory round trips overlap),
+// and from then on keeps the next row group's loads in flight while it computes
+// the current one (two register buffers, loop unrolled by two so no copies).
+template <class T, int U, int RB, int NM>
+struct GemvTile {
+    typename T::Wt w[NM][RB][U];
+    __device__ __forceinline__ void load(const GemvArgs& p, const uint32_t (&unit)[U], uint32_t r, uint32_t r1) {
 #pragma unroll
         for (int mi = 0; mi < NM; ++mi) {
             const uint8_t* base = mi == 0 ? p.w : p.w2;
 #pragma unroll
             for (int rb = 0; rb < RB; ++rb) {
-                uint32_t row = min(r + rb, r1 - 1);
+                uint32_t row = min(r + rb, r1 - 1);  // rows past the range re-read the last row; results unused
                 const uint8_t* rp = base + static_cast<uint64_t>(row) * p.row_bytes;
 #pragma unroll
-                for (int i = 0; i < U; ++i) T::load_w(wt[mi][rb][i], rp, unit[i]);
+                for (int i = 0; i < U; ++i) T::load_w(w[mi][rb][i], rp, unit[i]);
             }
         }
+    }
+};
+
+template <int EPI>
+__device__ __forceinline__ void gemv_store(const GemvArgs& p, uint32_t row, float v0, float v1) {
+    float v = v0;
+    if (EPI == EPI_ADD) v = p.resid[row] + v;
+    if (EPI == EPI_SILU_MUL) {
+        // cera/src/backend/cpu.rs:2570-2575: g / (1 + expf(-g)) * u
+        v = __fmul_rn(__fdiv_rn(v0, __fadd_rn(1.0f, cera_expf(-v0))), v1);
+    }
+    p.y[row] = v;
+}
+
+template <class T, int U, int KS, int RB, int EPI, bool DBG>
+__device__ __forceinline__ void gemv_compute(const GemvArgs& p, const GemvTile<T, U, RB, (EPI == EPI_SILU_MUL ? 2 : 1)>& t,
+                                             const typename T::Act (&act)[U], const uint32_t (&unit)[U],
+                                             const bool (&live)[U], uint32_t lane, uint32_t kw, uint32_t r,
+                                             uint32_t r1, float (*part)[RB][KS]) {
+    constexpr int NM = EPI == EPI_SILU_MUL ? 2 : 1;
 #pragma unroll
-        for (int rb = 0; rb < RB; ++rb) {
-            uint32_t row = r + rb;
-            float tot[NM];
+    for (int rb = 0; rb < RB; ++rb) {
+        uint32_t row = r + rb;
+        float tot[NM];
+#pragma unroll
+        for (int mi = 0; mi < NM; ++mi) {
+            float acc = 0.0f;
+#pragma unroll
+            for (int i = 0; i < U; ++i) {
+                int32_t* dbg = nullptr;
+                if (DBG) dbg = (live[i] && row < r1) ? p.dbg_dots + static_cast<uint64_t>(row) * p.dbg_stride : nullptr;
+                acc += T::dot(t.w[mi][rb][i], act[i], unit[i], dbg);
+            }
+            tot[mi] = wave_sum(acc);
+        }
+        if (KS == 1) {
+            if (lane == 0 && row < r1) gemv_store<EPI>(p, row, tot[0], tot[NM - 1]);
+        } else if (lane == 0) {
+#pragma unroll
+            for (int mi = 0; mi < NM; ++mi) part[mi][rb][kw] = tot[mi];
+        }
+    }
+    if (KS > 1) {
+        __syncthreads();
+        if (threadIdx.x < RB && r + threadIdx.x < r1) {
+            float v[NM];
 #pragma unroll
             for (int mi = 0; mi < NM; ++mi) {
-                float acc = 0.0f;
+                float s = part[mi][threadIdx.x][0];
 #pragma unroll
-                for (int i = 0; i < U; ++i) {
-                    int32_t* dbg = nullptr;
-                    if (DBG) dbg = (lane + 64 * i < p.n_units && row < r1)
-                                       ? p.dbg_dots + static_cast<uint64_t>(row) * p.dbg_stride : nullptr;
-                    acc += T::dot(wt[mi][rb][i], act[i], unit[i], dbg);
-                }
-                tot[mi] = wave_sum(acc);
+                for (int w = 1; w < KS; ++w) s += part[mi][threadIdx.x][w];
+                v[mi] = s;
             }
-            if (lane == 0 && row < r1) {
-                float v = tot[0];
-                if (EPI == EPI_ADD) v = p.resid[row] + v;
-                if (EPI == EPI_SILU_MUL) {
-                    // cera/src/backend/cpu.rs:2570-2575: g / (1 + expf(-g)) * u
-                    float g = tot[0], up = tot[NM - 1];
-                    v = __fmul_rn(__fdiv_rn(g, __fadd_rn(1.0f, cera_expf(-g))), up);
-                }
-                p.y[row] = v;
-            }
+            gemv_store<EPI>(p, r + threadIdx.x, v[0], v[NM - 1]);
         }
+    }
+}
+
+template <class T, int U, int KS, int RB, int EPI, bool DBG>
+static __global__ __launch_bounds__(64 * KS) void gemv_kernel(GemvArgs p) {
+    constexpr int NM = EPI == EPI_SILU_MUL ? 2 : 1;
+    // two LDS buffers: a buffer is rewritten two row groups later, after another barrier
+    __shared__ float part[2][NM][RB][KS];
+    const uint32_t lane = threadIdx.x & 63, kw = threadIdx.x >> 6;
+    uint32_t r = blockIdx.x * p.rows_per_wave;  // rows per workgroup
+    if (r >= p.m) return;
+    const uint32_t r1 = min(p.m, r + p.rows_per_wave);
+
+    uint32_t unit[U];
+    bool live[U];
+#pragma unroll
+    for (int i = 0; i < U; ++i) {
+        uint32_t u = kw * 64 + lane + 64 * KS * i;
+        live[i] = u < p.n_units;
+        unit[i] = live[i] ? u : 0;  // dead lanes re-read unit 0 with zeroed activations
+    }
+    GemvTile<T, U, RB, NM> ta, tb;
+    ta.load(p, unit, r, r1);
+
+    typename T::Act act[U];
+#pragma unroll
+    for (int i = 0; i < U; ++i) {
+        T::load_act(act[i], p.xq, p.xs, unit[i], live[i]);
+        if (DBG && blockIdx.x == 0 && live[i] && p.dbg_asums) T::dbg_asum(act[i], unit[i], p.dbg_asums);
+    }
+
+    for (;;) {
+        if (r + RB < r1) tb.load(p, unit, r + RB, r1);
+        gemv_compute<T, U, KS, RB, EPI, DBG>(p, ta, act, unit, live, lane, kw, r, r1, part[0]);
+        r += RB;
+        if (r >= r1) break;
+        if (r + RB < r1) ta.load(p, unit, r + RB, r1);
+        gemv_compute<T, U, KS, RB, EPI, DBG>(p, tb, act, unit, live, lane, kw, r, r1, part[1]);
+        r += RB;
+        if (r >= r1) break;
     }
 }
 

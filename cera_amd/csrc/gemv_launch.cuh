@@ -1,61 +1,69 @@
-// Host-side dispatch of gemv_kernel<T, U, RB, EPI, DBG> over the run-time
-// values of U (units per lane), RB (rows in flight) and the epilogue.
+// Host-side dispatch of gemv_kernel<T, U, KS, RB, EPI, DBG> over the run-time
+// values of the K split (KS wavefronts per workgroup, U units per lane), RB
+// (rows in flight) and the epilogue.
 #pragma once
 #include "gemv.cuh"
 #include "host_common.h"
 
-// U is rounded up to the next instantiated width; the surplus lanes carry
-// zeroed activations.
-static inline int gemv_pick_u(uint32_t n_units) {
-    uint32_t u = (n_units + 63) / 64;
+struct GemvPlan {
+    int U, KS, RB;
+    uint32_t rows_per_block, n_blocks;
+};
+
+// n_units = K / 32.  One unit per lane while K <= 16384 (KS up to 8 wavefronts),
+// two per lane up to 32768.  KS is rounded up to an instantiated width; surplus
+// lanes carry zeroed activations.
+static inline bool gemv_pick_split(uint32_t n_units, int* U, int* KS) {
     const int widths[] = {1, 2, 4, 7, 8};
-    for (int w : widths)
-        if (u <= static_cast<uint32_t>(w)) return w;
-    return 0;  // K too large for the register-resident kernel
+    for (int u = 1; u <= 2; ++u)
+        for (int w : widths)
+            if (n_units <= static_cast<uint32_t>(64 * w * u)) { *U = u; *KS = w; return true; }
+    return false;
 }
 
-template <class T, int U, int RB>
+// Measured on MI355X: ~32 wavefronts per CU in flight, four rows per workgroup
+// step for the 16-byte-unit formats and two for Q6_K (15 registers per row).
+static inline bool gemv_plan(uint32_t m, uint32_t n_units, uint32_t n_cu, bool dbg, int max_rb, GemvPlan* p) {
+    if (!gemv_pick_split(n_units, &p->U, &p->KS)) return false;
+    const uint32_t target_blocks = std::max(1u, n_cu * 32 / static_cast<uint32_t>(p->KS));
+    uint32_t rpb = (m + target_blocks - 1) / target_blocks;
+    p->RB = rpb >= 4 ? 4 : (rpb >= 2 ? 2 : 1);
+    if (p->RB > max_rb) p->RB = max_rb;
+    if (dbg) p->RB = 1;
+    rpb = (rpb + p->RB - 1) / p->RB * p->RB;
+    p->rows_per_block = rpb;
+    p->n_blocks = (m + rpb - 1) / rpb;
+    return true;
+}
+
+template <class T, int U, int KS, int RB>
 static void gemv_launch_epi(const GemvArgs& a, int epi, bool dbg, dim3 grid, hipStream_t s) {
+    const dim3 block(64 * KS);
     if (dbg) {
-        hipLaunchKernelGGL((gemv_kernel<T, U, RB, EPI_STORE, true>), grid, dim3(256), 0, s, a);
+        if (RB == 1) hipLaunchKernelGGL((gemv_kernel<T, U, KS, 1, EPI_STORE, true>), grid, block, 0, s, a);
         return;
     }
     switch (epi) {
-        case EPI_ADD: hipLaunchKernelGGL((gemv_kernel<T, U, RB, EPI_ADD, false>), grid, dim3(256), 0, s, a); break;
-        case EPI_SILU_MUL: hipLaunchKernelGGL((gemv_kernel<T, U, RB, EPI_SILU_MUL, false>), grid, dim3(256), 0, s, a); break;
-        default: hipLaunchKernelGGL((gemv_kernel<T, U, RB, EPI_STORE, false>), grid, dim3(256), 0, s, a); break;
+        case EPI_ADD: hipLaunchKernelGGL((gemv_kernel<T, U, KS, RB, EPI_ADD, false>), grid, block, 0, s, a); break;
+        case EPI_SILU_MUL: hipLaunchKernelGGL((gemv_kernel<T, U, KS, RB, EPI_SILU_MUL, false>), grid, block, 0, s, a); break;
+        default: hipLaunchKernelGGL((gemv_kernel<T, U, KS, RB, EPI_STORE, false>), grid, block, 0, s, a); break;
     }
 }
 
-// Wide rows keep two rows in flight, narrow rows four (when a wavefront has
-// that many rows at all): enough bytes outstanding per CU without spilling.
+template <class T, int U, int KS>
+static void gemv_launch_rb(const GemvArgs& a, int RB, int epi, bool dbg, dim3 grid, hipStream_t s) {
+    switch (RB) {
+        case 1: gemv_launch_epi<T, U, KS, 1>(a, epi, dbg, grid, s); break;
+        case 2: gemv_launch_epi<T, U, KS, 2>(a, epi, dbg, grid, s); break;
+        default: gemv_launch_epi<T, U, KS, 4>(a, epi, dbg, grid, s); break;
+    }
+}
+
 template <class T>
-static bool gemv_launch_t(const GemvArgs& a, int U, int RB, int epi, bool dbg, dim3 grid, hipStream_t s) {
-    switch (U) {
-        case 1: if (RB == 4) gemv_launch_epi<T, 1, 4>(a, epi, dbg, grid, s); else gemv_launch_epi<T, 1, 2>(a, epi, dbg, grid, s); return true;
-        case 2: if (RB == 4) gemv_launch_epi<T, 2, 4>(a, epi, dbg, grid, s); else gemv_launch_epi<T, 2, 2>(a, epi, dbg, grid, s); return true;
-        case 4: gemv_launch_epi<T, 4, 2>(a, epi, dbg, grid, s); return true;
-        case 7: gemv_launch_epi<T, 7, 2>(a, epi, dbg, grid, s); return true;
-        case 8: gemv_launch_epi<T, 8, 2>(a, epi, dbg, grid, s); return true;
-        default: return false;
-    }
-}
-
-struct GemvPlan {
-    int U, RB;
-    uint32_t rows_per_wave, n_blocks;
-};
-
-static inline GemvPlan gemv_plan(uint32_t m, uint32_t n_units, uint32_t n_cu, bool dbg) {
-    GemvPlan p;
-    p.U = gemv_pick_u(n_units);
-    const uint32_t target_waves = n_cu * 8;
-    uint32_t rpw = (m + target_waves - 1) / target_waves;
-    p.RB = (p.U <= 2 && rpw >= 4) ? 4 : 2;
-    if (dbg) p.RB = 2;
-    rpw = (rpw + p.RB - 1) / p.RB * p.RB;
-    p.rows_per_wave = rpw;
-    uint32_t waves = (m + rpw - 1) / rpw;
-    p.n_blocks = (waves + 3) / 4;
-    return p;
+static bool gemv_launch_t(const GemvArgs& a, const GemvPlan& p, int epi, bool dbg, hipStream_t s) {
+    dim3 grid(p.n_blocks);
+#define CASE(UU, KK) if (p.U == UU && p.KS == KK) { gemv_launch_rb<T, UU, KK>(a, p.RB, epi, dbg, grid, s); return true; }
+    CASE(1, 1) CASE(1, 2) CASE(1, 4) CASE(1, 7) CASE(1, 8) CASE(2, 7) CASE(2, 8)
+#undef CASE
+    return false;
 }

@@ -2,6 +2,6 @@
 // the device compile parallel).
 #include "gemv_launch.cuh"
 
-bool cera_gemv_launch_q8_0(const GemvArgs& a, int U, int RB, int epi, bool dbg, dim3 grid, hipStream_t s) {
-    return gemv_launch_t<Q8_0>(a, U, RB, epi, dbg, grid, s);
+bool cera_gemv_launch_q8_0(const GemvArgs& a, const GemvPlan& p, int epi, bool dbg, hipStream_t s) {
+    return gemv_launch_t<Q8_0>(a, p, epi, dbg, s);
 }

@@ -62,7 +62,7 @@ class Config(C.Structure):
 
 
 class GemvOp(C.Structure):
-    _fields_ = [("w", C.c_void_p), ("xs", C.c_void_p), ("xq", C.c_void_p), ("y", C.c_void_p)]
+    _fields_ = [("w", C.c_void_p), ("w2", C.c_void_p), ("xs", C.c_void_p), ("xq", C.c_void_p), ("y", C.c_void_p)]
 
 
 _lib = None

@@ -184,6 +184,9 @@ CERA_HIP_API cera_hip_status cera_hip_gemv_q8_dev(cera_hip_ctx*, const cera_hip_
                                                   const int8_t* xq, float* y);
 typedef struct {
     const cera_hip_dtensor* w;
+    const cera_hip_dtensor* w2; /* nullable; when set (same type and shape as w) the launch is
+                                   the fused FFN pair: y = silu(w.x) * (w2.x), the gate/up step of
+                                   transformer::forward_ffn_block (cera/src/model/transformer.rs:1541) */
     const float* xs;  /* dev f32[k/32] */
     const int8_t* xq; /* dev i8[k]     */
     float* y;         /* dev f32[m]    */
