@@ -272,11 +272,12 @@ uint64_t cera_hip_tensor_nbytes(const cera_hip_dtensor* d) { return d ? d->nbyte
 
 // ---------------------------------------------------------------------------
 // launchers
-cera_hip_status cera_launch_quantize(cera_hip_ctx* ctx, const float* x, uint64_t k, float* scales, int8_t* quants) {
+cera_hip_status cera_launch_quantize(cera_hip_ctx* ctx, const float* x, uint64_t k, float* scales, int8_t* quants,
+                                     float* bsum) {
     if (k == 0 || k % 32) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "quantize_q8_0: k must be a positive multiple of 32");
     uint64_t threads = k / 4;
     dim3 grid(static_cast<uint32_t>((threads + 255) / 256));
-    hipLaunchKernelGGL(quantize_q8_0_kernel, grid, dim3(256), 0, ctx->stream, x, k, scales, quants);
+    hipLaunchKernelGGL(quantize_q8_0_kernel, grid, dim3(256), 0, ctx->stream, x, k, scales, quants, bsum);
     HIP_TRY(ctx, hipGetLastError());
     return CERA_HIP_OK;
 }
@@ -336,24 +337,27 @@ cera_hip_status cera_launch_gemv_q5k_f32(cera_hip_ctx* ctx, const cera_hip_dtens
     return CERA_HIP_OK;
 }
 
-cera_hip_status cera_launch_attn_decode(cera_hip_ctx* ctx, const float* q, const float* kc, const float* vc,
-                                        uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, uint64_t seq_len,
-                                        uint64_t max_seq, float scale, uint32_t n_splits, float* out,
-                                        float* out_scales, int8_t* out_quants) {
-    if (head_dim != ATTN_HD) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "attn_decode: head_dim must be 128");
-    if (n_kv_heads == 0 || n_heads % n_kv_heads) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "attn_decode: n_heads must be a multiple of n_kv_heads");
+cera_hip_status cera_launch_attn(cera_hip_ctx* ctx, const float* q, const float* kc, const float* vc,
+                                 uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, uint64_t seq_len,
+                                 uint64_t max_seq, float scale, uint32_t n_splits, uint32_t n_queries, float* out,
+                                 float* out_scales, int8_t* out_quants, float* out_bsum) {
+    if (head_dim != ATTN_HD) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "attention: head_dim must be 128");
+    if (n_kv_heads == 0 || n_heads % n_kv_heads) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "attention: n_heads must be a multiple of n_kv_heads");
     uint32_t G = n_heads / n_kv_heads;
-    if (G != 1 && G != 2 && G != 4 && G != 8) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "attn_decode: group size must be 1, 2, 4 or 8");
-    if (seq_len == 0 || seq_len > max_seq || max_seq > 0x7FFFFFFFull) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "attn_decode: need 0 < seq_len <= max_seq < 2^31");
-    if (n_heads % 2) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "attn_decode: n_heads must be even");
-    uint32_t n_chunks = static_cast<uint32_t>((seq_len + ATTN_CHUNK - 1) / ATTN_CHUNK);
-    // parts (wavefronts) per kv head: enough to fill the chip ~8 waves per CU
+    if (G != 1 && G != 2 && G != 4 && G != 8) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "attention: group size must be 1, 2, 4 or 8");
+    if (n_queries == 0 || n_queries > 65535) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "attention: 1..65535 queries per call");
+    // seq_len = keys visible to the first query; the last query sees seq_len + n_queries - 1
+    const uint64_t last_len = seq_len + n_queries - 1;
+    if (seq_len == 0 || last_len > max_seq || max_seq > 0x7FFFFFFFull) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "attention: need 0 < seq_len <= max_seq < 2^31");
+    if (n_heads % 2) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "attention: n_heads must be even");
+    uint32_t n_chunks = static_cast<uint32_t>((last_len + ATTN_CHUNK - 1) / ATTN_CHUNK);
+    // parts (wavefronts) per (query, kv head): enough to fill the chip ~8 waves per CU
     // deep, but at least one chunk each
-    uint32_t want_parts = n_splits ? n_splits : std::max(1u, ctx->n_cu * 8 / n_kv_heads);
+    uint32_t want_parts = n_splits ? n_splits : std::max(1u, ctx->n_cu * 8 / (n_kv_heads * n_queries));
     uint32_t chunks_per_part = std::max(1u, (n_chunks + want_parts - 1) / want_parts);
     uint32_t n_parts = (n_chunks + chunks_per_part - 1) / chunks_per_part;
-    uint64_t acc_bytes = static_cast<uint64_t>(n_kv_heads) * n_parts * G * ATTN_HD * sizeof(float);
-    uint64_t ml_bytes = static_cast<uint64_t>(n_kv_heads) * n_parts * G * 2 * sizeof(float);
+    uint64_t acc_bytes = static_cast<uint64_t>(n_queries) * n_kv_heads * n_parts * G * ATTN_HD * sizeof(float);
+    uint64_t ml_bytes = static_cast<uint64_t>(n_queries) * n_kv_heads * n_parts * G * 2 * sizeof(float);
     if (ctx->attn_acc_bytes < acc_bytes) {
         HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
         if (ctx->attn_acc) HIP_TRY(ctx, hipFree(ctx->attn_acc));
@@ -368,11 +372,12 @@ cera_hip_status cera_launch_attn_decode(cera_hip_ctx* ctx, const float* q, const
         HIP_TRY(ctx, hipMalloc(reinterpret_cast<void**>(&ctx->attn_ml), ml_bytes));
         ctx->attn_ml_bytes = ml_bytes;
     }
-    dim3 grid((n_parts + 3) / 4, n_kv_heads);
+    dim3 grid((n_parts + 3) / 4, n_kv_heads, n_queries);
     uint32_t sl = static_cast<uint32_t>(seq_len), ms = static_cast<uint32_t>(max_seq);
+    uint32_t q_stride = n_heads * head_dim;
 #define ATTN_LAUNCH(GG)                                                                                    \
     hipLaunchKernelGGL((attn_decode_partial_kernel<GG>), grid, dim3(256), 0, ctx->stream, q, kc, vc, sl, ms, \
-                       scale, chunks_per_part, n_parts, ctx->attn_acc, ctx->attn_ml)
+                       scale, chunks_per_part, n_parts, q_stride, ctx->attn_acc, ctx->attn_ml)
     switch (G) {
         case 1: ATTN_LAUNCH(1); break;
         case 2: ATTN_LAUNCH(2); break;
@@ -381,14 +386,24 @@ cera_hip_status cera_launch_attn_decode(cera_hip_ctx* ctx, const float* q, const
     }
 #undef ATTN_LAUNCH
     HIP_TRY(ctx, hipGetLastError());
+    dim3 mgrid(n_heads / 2, n_queries);
     if (out_quants)
-        hipLaunchKernelGGL((attn_decode_merge_kernel<true>), dim3(n_heads / 2), dim3(64), 0, ctx->stream,
-                           ctx->attn_acc, ctx->attn_ml, n_parts, G, out, out_scales, out_quants);
+        hipLaunchKernelGGL((attn_decode_merge_kernel<true>), mgrid, dim3(64), 0, ctx->stream, ctx->attn_acc,
+                           ctx->attn_ml, n_parts, G, n_heads, out, out_scales, out_quants, out_bsum);
     else
-        hipLaunchKernelGGL((attn_decode_merge_kernel<false>), dim3(n_heads / 2), dim3(64), 0, ctx->stream,
-                           ctx->attn_acc, ctx->attn_ml, n_parts, G, out, nullptr, nullptr);
+        hipLaunchKernelGGL((attn_decode_merge_kernel<false>), mgrid, dim3(64), 0, ctx->stream, ctx->attn_acc,
+                           ctx->attn_ml, n_parts, G, n_heads, out, static_cast<float*>(nullptr),
+                           static_cast<int8_t*>(nullptr), static_cast<float*>(nullptr));
     HIP_TRY(ctx, hipGetLastError());
     return CERA_HIP_OK;
+}
+
+cera_hip_status cera_launch_attn_decode(cera_hip_ctx* ctx, const float* q, const float* kc, const float* vc,
+                                        uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, uint64_t seq_len,
+                                        uint64_t max_seq, float scale, uint32_t n_splits, float* out,
+                                        float* out_scales, int8_t* out_quants) {
+    return cera_launch_attn(ctx, q, kc, vc, n_heads, n_kv_heads, head_dim, seq_len, max_seq, scale, n_splits, 1, out,
+                            out_scales, out_quants, nullptr);
 }
 
 // ---------------------------------------------------------------------------
@@ -520,7 +535,7 @@ cera_hip_status cera_hip_rmsnorm(cera_hip_ctx* ctx, const float* x, const float*
     CERA_TRY(cera_hip_upload(ctx, dx, x, n * 4));
     CERA_TRY(cera_hip_upload(ctx, dw, weight, n * 4));
     hipLaunchKernelGGL((rmsnorm_kernel<false>), dim3(1), dim3(256), 0, ctx->stream, static_cast<float*>(dx),
-                       static_cast<float*>(dw), static_cast<uint32_t>(n), eps, static_cast<float*>(dy), nullptr, nullptr);
+                       static_cast<float*>(dw), static_cast<uint32_t>(n), eps, static_cast<float*>(dy), nullptr, nullptr, nullptr);
     HIP_TRY(ctx, hipGetLastError());
     return cera_hip_download(ctx, y, dy, n * 4);
 }
@@ -536,7 +551,7 @@ cera_hip_status cera_hip_silu_mul(cera_hip_ctx* ctx, const float* gate, const fl
     CERA_TRY(cera_hip_upload(ctx, du, up, n * 4));
     hipLaunchKernelGGL((silu_mul_kernel<false>), dim3(static_cast<uint32_t>((n / 4 + 255) / 256)), dim3(256), 0,
                        ctx->stream, static_cast<float*>(dg), static_cast<float*>(du), n, static_cast<float*>(dy),
-                       nullptr, nullptr);
+                       nullptr, nullptr, nullptr);
     HIP_TRY(ctx, hipGetLastError());
     return cera_hip_download(ctx, out, dy, n * 4);
 }

@@ -37,12 +37,16 @@ __global__ __launch_bounds__(256) void attn_decode_partial_kernel(
     const float* __restrict__ kc,      // [n_kv][max_seq][128]
     const float* __restrict__ vc,
     uint32_t seq_len, uint32_t max_seq, float scale, uint32_t chunks_per_part, uint32_t n_parts,
-    float* __restrict__ part_acc,      // [n_kv][n_parts][G][128]
-    float* __restrict__ part_ml) {     // [n_kv][n_parts][G][2]
+    uint32_t q_stride,                 // floats between consecutive queries (prefill batches queries on grid.z)
+    float* __restrict__ part_acc,      // [n_queries][n_kv][n_parts][G][128]
+    float* __restrict__ part_ml) {     // [n_queries][n_kv][n_parts][G][2]
     const uint32_t lane = threadIdx.x & 63;
     const uint32_t part = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
-    const uint32_t kvh = blockIdx.y;
+    const uint32_t kvh = blockIdx.y, qi = blockIdx.z;
     if (part >= n_parts) return;
+    // causal prefill: query qi sits at position seq_len - 1 + qi and sees seq_len + qi keys
+    seq_len += qi;
+    q += static_cast<uint64_t>(qi) * q_stride;
     const uint32_t j = lane & 7, pg = lane >> 3;  // float4 column group, position group
 
     // this lane's 16 q values for each of the G heads
@@ -156,7 +160,7 @@ __global__ __launch_bounds__(256) void attn_decode_partial_kernel(
         }
     }
     if (pg == 0) {
-        uint64_t base = (static_cast<uint64_t>(kvh) * n_parts + part) * G;
+        uint64_t base = ((static_cast<uint64_t>(qi) * gridDim.y + kvh) * n_parts + part) * G;
 #pragma unroll
         for (int h = 0; h < G; ++h) {
             float4* dst = reinterpret_cast<float4*>(part_acc + (base + h) * ATTN_HD);
@@ -176,19 +180,20 @@ __global__ __launch_bounds__(256) void attn_decode_partial_kernel(
 template <bool QUANT>
 __global__ __launch_bounds__(64) void attn_decode_merge_kernel(const float* __restrict__ part_acc,
                                                                const float* __restrict__ part_ml,
-                                                               uint32_t n_parts, uint32_t G,
+                                                               uint32_t n_parts, uint32_t G, uint32_t n_heads,
                                                                float* __restrict__ out,
                                                                float* __restrict__ scales,
-                                                               int8_t* __restrict__ quants) {
+                                                               int8_t* __restrict__ quants,
+                                                               float* __restrict__ bsum) {
     const uint32_t head = blockIdx.x * 2 + (threadIdx.x >> 5), c = threadIdx.x & 31;
-    const uint32_t kvh = head / G, hg = head % G;
+    const uint32_t kvh = head / G, hg = head % G, qi = blockIdx.y, n_kv = n_heads / G;
+    const uint64_t pbase = (static_cast<uint64_t>(qi) * n_kv + kvh) * n_parts;
     float M = -__builtin_inff();
-    for (uint32_t p = 0; p < n_parts; ++p)
-        M = fmaxf(M, part_ml[((static_cast<uint64_t>(kvh) * n_parts + p) * G + hg) * 2]);
+    for (uint32_t p = 0; p < n_parts; ++p) M = fmaxf(M, part_ml[((pbase + p) * G + hg) * 2]);
     float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
     float L = 0.0f;
     for (uint32_t p = 0; p < n_parts; ++p) {
-        uint64_t idx = (static_cast<uint64_t>(kvh) * n_parts + p) * G + hg;
+        uint64_t idx = (pbase + p) * G + hg;
         float w = cera_expf(part_ml[idx * 2] - M);
         L = fmaf(w, part_ml[idx * 2 + 1], L);
         float4 a = reinterpret_cast<const float4*>(part_acc + idx * ATTN_HD)[c];
@@ -197,11 +202,16 @@ __global__ __launch_bounds__(64) void attn_decode_merge_kernel(const float* __re
     }
     float inv = 1.0f / L;
     float4 o = make_float4(acc.x * inv, acc.y * inv, acc.z * inv, acc.w * inv);
-    reinterpret_cast<float4*>(out + head * ATTN_HD)[c] = o;
+    const uint64_t row = static_cast<uint64_t>(qi) * n_heads + head;  // outputs are [n_queries][n_heads][128]
+    reinterpret_cast<float4*>(out + row * ATTN_HD)[c] = o;
     if (QUANT) {
         float sc;
         uint32_t packed = q8_quantize_quad(o, sc);
-        reinterpret_cast<uint32_t*>(quants)[head * 32 + c] = packed;
-        if ((c & 7) == 0) scales[head * 4 + (c >> 3)] = sc;
+        float ssum = bsum ? q8_block_scaled_sum(packed, sc) : 0.0f;
+        reinterpret_cast<uint32_t*>(quants)[row * 32 + c] = packed;
+        if ((c & 7) == 0) {
+            scales[row * 4 + (c >> 3)] = sc;
+            if (bsum) bsum[row * 4 + (c >> 3)] = ssum;
+        }
     }
 }

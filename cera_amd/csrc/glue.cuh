@@ -73,13 +73,14 @@ __device__ __forceinline__ float dequant_elem(uint32_t dtype, const uint8_t* row
 
 // token comes from device memory so a graph-captured decode step can chain on
 // the previous step's argmax without a host round trip.
+// grid.y = number of tokens (prefill looks up a batch of rows: out is [n][k]).
 static __global__ void embed_row_kernel(uint32_t dtype, const uint8_t* __restrict__ w, uint64_t row_bytes,
                                  const uint32_t* __restrict__ token, uint32_t k, float scale,
                                  float* __restrict__ out) {
     uint32_t e = blockIdx.x * blockDim.x + threadIdx.x;
     if (e >= k) return;
-    float v = dequant_elem(dtype, w + static_cast<uint64_t>(*token) * row_bytes, e);
-    out[e] = scale != 1.0f ? __fmul_rn(v, scale) : v;
+    float v = dequant_elem(dtype, w + static_cast<uint64_t>(token[blockIdx.y]) * row_bytes, e);
+    out[static_cast<uint64_t>(blockIdx.y) * k + e] = scale != 1.0f ? __fmul_rn(v, scale) : v;
 }
 
 // ---------------------------------------------------------------------------
@@ -92,7 +93,8 @@ static __global__ void embed_row_kernel(uint32_t dtype, const uint8_t* __restric
 template <bool QUANT>
 static __global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ x, const float* __restrict__ w,
                                                       uint32_t n, float eps, float* __restrict__ y,
-                                                      float* __restrict__ scales, int8_t* __restrict__ quants) {
+                                                      float* __restrict__ scales, int8_t* __restrict__ quants,
+                                                      float* __restrict__ bsum) {
     __shared__ double part[4];
     const float* xr = x + static_cast<uint64_t>(blockIdx.x) * n;
     float* yr = y + static_cast<uint64_t>(blockIdx.x) * n;
@@ -124,8 +126,12 @@ static __global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __rest
             float sc;
             uint32_t packed = q8_quantize_quad(o, sc);
             uint64_t e = static_cast<uint64_t>(blockIdx.x) * n + i;
+            float ssum = bsum ? q8_block_scaled_sum(packed, sc) : 0.0f;
             reinterpret_cast<uint32_t*>(quants)[e >> 2] = packed;
-            if ((threadIdx.x & 7) == 0) scales[e >> 5] = sc;
+            if ((threadIdx.x & 7) == 0) {
+                scales[e >> 5] = sc;
+                if (bsum) bsum[e >> 5] = ssum;
+            }
         }
     }
 }
@@ -139,11 +145,16 @@ static __global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __rest
 // threads: blocks [0, n_heads) rotate q; the next n_kv_heads rotate k and
 // store it; the last n_kv_heads copy v.
 // KV cache layout: [kv_head][max_seq][head_dim] f32.
-static __global__ void rope_kv_kernel(float* __restrict__ q, float* __restrict__ k, const float* __restrict__ v,
+static __global__ void rope_kv_kernel(float* __restrict__ q, float* __restrict__ k, const float* v,
                                const float* __restrict__ cs_table, const uint32_t* __restrict__ pos_ptr,
                                uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, uint32_t rope_type,
                                float* __restrict__ k_cache, float* __restrict__ v_cache, uint32_t max_seq) {
-    const uint32_t pos = *pos_ptr;
+    // grid.y = tokens of a prefill batch: token t sits at position *pos_ptr + t and its
+    // q/k/v rows follow each other ([n][n_heads*head_dim], [n][n_kv_heads*head_dim])
+    const uint32_t pos = *pos_ptr + blockIdx.y;
+    q += static_cast<uint64_t>(blockIdx.y) * n_heads * head_dim;
+    k += static_cast<uint64_t>(blockIdx.y) * n_kv_heads * head_dim;
+    if (v) v += static_cast<uint64_t>(blockIdx.y) * n_kv_heads * head_dim;
     const uint32_t half = head_dim / 2, i = threadIdx.x, b = blockIdx.x;
     if (b < n_heads + n_kv_heads) {
         float* head = b < n_heads ? q + b * head_dim : k + (b - n_heads) * head_dim;
@@ -191,7 +202,8 @@ static __global__ void scale_kernel(float* __restrict__ x, float s, uint32_t n) 
 template <bool QUANT>
 static __global__ __launch_bounds__(256) void silu_mul_kernel(const float* __restrict__ gate, const float* __restrict__ up,
                                                        uint64_t n, float* __restrict__ out,
-                                                       float* __restrict__ scales, int8_t* __restrict__ quants) {
+                                                       float* __restrict__ scales, int8_t* __restrict__ quants,
+                                                       float* __restrict__ bsum) {
     uint64_t t = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     bool live = 4 * t < n;
     float4 g = live ? reinterpret_cast<const float4*>(gate)[t] : make_float4(0, 0, 0, 0);
@@ -204,9 +216,13 @@ static __global__ __launch_bounds__(256) void silu_mul_kernel(const float* __res
     if (QUANT) {
         float sc;
         uint32_t packed = q8_quantize_quad(o, sc);
+        float ssum = bsum ? q8_block_scaled_sum(packed, sc) : 0.0f;
         if (live) {
             reinterpret_cast<uint32_t*>(quants)[t] = packed;
-            if ((t & 7) == 0) scales[t >> 3] = sc;
+            if ((t & 7) == 0) {
+                scales[t >> 3] = sc;
+                if (bsum) bsum[t >> 3] = ssum;
+            }
         }
     }
     if (live && out) reinterpret_cast<float4*>(out)[t] = o;

@@ -57,7 +57,8 @@ cera_hip_status cera_scratch(cera_hip_ctx* ctx, int slot, uint64_t nbytes, void*
 // ---- launchers (defined next to their kernels) --------------------------------
 enum CeraEpilogue { CERA_EPI_STORE = 0, CERA_EPI_ADD = 1, CERA_EPI_SILU_MUL = 2 };
 
-cera_hip_status cera_launch_quantize(cera_hip_ctx* ctx, const float* x, uint64_t k, float* scales, int8_t* quants);
+cera_hip_status cera_launch_quantize(cera_hip_ctx* ctx, const float* x, uint64_t k, float* scales, int8_t* quants,
+                                     float* bsum = nullptr);
 // y = W.(xs,xq) [+ resid]; w2 != null with EPI_SILU_MUL computes silu(W.x)*(W2.x)
 cera_hip_status cera_launch_gemv(cera_hip_ctx* ctx, const cera_hip_dtensor* w, const cera_hip_dtensor* w2,
                                  const float* xs, const int8_t* xq, float* y, const float* resid, int epi,
@@ -67,3 +68,9 @@ cera_hip_status cera_launch_attn_decode(cera_hip_ctx* ctx, const float* q, const
                                         uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, uint64_t seq_len,
                                         uint64_t max_seq, float scale, uint32_t n_splits, float* out,
                                         float* out_scales, int8_t* out_quants);
+// n_queries consecutive queries (causal): query i sees seq_len + i keys; q and the outputs are
+// [n_queries][n_heads*head_dim]
+cera_hip_status cera_launch_attn(cera_hip_ctx* ctx, const float* q, const float* kc, const float* vc,
+                                 uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, uint64_t seq_len,
+                                 uint64_t max_seq, float scale, uint32_t n_splits, uint32_t n_queries, float* out,
+                                 float* out_scales, int8_t* out_quants, float* out_bsum);

@@ -26,6 +26,13 @@ struct cera_hip_model {
     int8_t* xq = nullptr;
     uint32_t* scalars = nullptr;  // device: [token, pos, argmax result, spare]
     std::vector<void*> owned;     // plain device allocations freed with the model
+    // batched-prefill activations, token-major [n][dim], allocated on first use
+    uint32_t pf_cap = 0;
+    float *pf_hidden = nullptr, *pf_normed = nullptr, *pf_q = nullptr, *pf_k = nullptr, *pf_v = nullptr,
+          *pf_attn = nullptr, *pf_gate = nullptr, *pf_up = nullptr, *pf_xs = nullptr, *pf_bsum = nullptr;
+    int8_t* pf_xq = nullptr;
+    uint32_t* pf_tokens = nullptr;
+    std::vector<void*> pf_owned;
     uint32_t seq_len = 0;
     uint64_t bytes = 0;
     // every trait call is serialised, like the reference GPU backends' infer_lock

@@ -62,6 +62,8 @@ static void free_model(cera_hip_model* m) {
     ft(m->output);
     for (void* p : m->owned)
         if (p) (void)hipFree(p);
+    for (void* p : m->pf_owned)
+        if (p) (void)hipFree(p);
     delete m;
 }
 
@@ -230,7 +232,7 @@ static cera_hip_status project(cera_hip_model* m, const cera_hip_dtensor* w, con
 
 static cera_hip_status norm_quant(cera_hip_model* m, const float* x, const float* w, uint32_t n, uint32_t rows, float* y) {
     hipLaunchKernelGGL((rmsnorm_kernel<true>), dim3(rows), dim3(256), 0, m->ctx->stream, x, w, n, m->cfg.rms_eps, y,
-                       m->xs, m->xq);
+                       m->xs, m->xq, static_cast<float*>(nullptr));
     HIP_TRY(m->ctx, hipGetLastError());
     return CERA_HIP_OK;
 }
@@ -261,9 +263,9 @@ static cera_hip_status decode_step(cera_hip_model* m, uint32_t pos, bool want_lo
         }
         if (L.q_norm) {
             hipLaunchKernelGGL((rmsnorm_kernel<false>), dim3(c.n_heads), dim3(256), 0, s, m->q, L.q_norm, c.head_dim,
-                               c.rms_eps, m->q, nullptr, nullptr);
+                               c.rms_eps, m->q, nullptr, nullptr, nullptr);
             hipLaunchKernelGGL((rmsnorm_kernel<false>), dim3(c.n_kv_heads), dim3(256), 0, s, m->k, L.k_norm, c.head_dim,
-                               c.rms_eps, m->k, nullptr, nullptr);
+                               c.rms_eps, m->k, nullptr, nullptr, nullptr);
         }
         hipLaunchKernelGGL(rope_kv_kernel, dim3(c.n_heads + 2 * c.n_kv_heads), dim3(c.head_dim / 2), 0, s, m->q, m->k,
                            m->v, m->rope_table, m->scalars + 1, c.n_heads, c.n_kv_heads, c.head_dim, c.rope_type,
@@ -283,7 +285,7 @@ static cera_hip_status decode_step(cera_hip_model* m, uint32_t pos, bool want_lo
             CERA_TRY(project(m, L.gate, m->normed, m->act, nullptr));
             CERA_TRY(project(m, L.up, m->normed, m->up, nullptr));
             hipLaunchKernelGGL((silu_mul_kernel<true>), dim3((c.ffn / 4 + 255) / 256), dim3(256), 0, s, m->act, m->up,
-                               static_cast<uint64_t>(c.ffn), m->act, m->xs, m->xq);
+                               static_cast<uint64_t>(c.ffn), m->act, m->xs, m->xq, static_cast<float*>(nullptr));
             HIP_TRY(ctx, hipGetLastError());
         }
         CERA_TRY(project(m, L.down, m->act, m->hidden, m->hidden));

@@ -1,19 +1,222 @@
-// Prefill: batched int8 GEMM over Q8_0-quantized activation rows and the
-// batched forward pass built on it.
+// Prefill: batched int8-MFMA GEMM over Q8_0-quantized activation rows
+// (transformer::gemm_preq over quantize_columns, cera/src/model/transformer.rs:
+// 710-788, 865-946) and the batched forward pass built on it
+// (LlamaModel::forward_prefill_batched, cera/src/model/llama.rs:738-1523).
+#include <cmath>
+#include <cstring>
+
+#include "gemm.cuh"
+#include "glue.cuh"
 #include "model.h"
 
-cera_hip_status cera_model_prefill(cera_hip_model* m, const uint32_t* tokens, uint32_t n, uint32_t start_pos,
-                                   float* last_logits) {
-    return cera_model_prefill_per_token(m, tokens, n, start_pos, last_logits);
+static bool gemm_type_ok(uint32_t t) {
+    return t == CERA_HIP_Q4_0 || t == CERA_HIP_Q4_1 || t == CERA_HIP_Q8_0 || t == CERA_HIP_Q4_K || t == CERA_HIP_Q6_K;
+}
+
+// batched_gemm_supports (cera/src/model/transformer.rs:536-565): the int8 GEMM
+// takes K in whole 256-element steps.
+bool cera_gemm_supports(uint32_t dtype, uint64_t k) { return gemm_type_ok(dtype) && k % GEMM_KT == 0 && k > 0; }
+
+// out[i*ld_m + j*ld_n] = (W . B)[i][j] (+ resid)
+cera_hip_status cera_launch_gemm(cera_hip_ctx* ctx, const cera_hip_dtensor* w, const float* bs, const int8_t* bq,
+                                 const float* bsum, uint32_t n, float* out, uint64_t ld_m, uint64_t ld_n,
+                                 const float* resid, float resid_scale) {
+    if (!cera_gemm_supports(w->dtype, w->k))
+        return cera_fail(ctx, CERA_HIP_ERR_UNSUPPORTED_DTYPE,
+                         "gemm: no int8 GEMM for ggml type " + std::to_string(w->dtype) + " with k=" + std::to_string(w->k));
+    if (n == 0) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "gemm: n must be positive");
+    GemmArgs a;
+    a.w = w->dev; a.bq = bq; a.bs = bs; a.bsum = bsum; a.out = out;
+    a.m = static_cast<uint32_t>(w->m); a.n = n; a.k = static_cast<uint32_t>(w->k);
+    a.row_bytes = static_cast<uint32_t>(w->row_bytes);
+    a.ld_m = ld_m; a.ld_n = ld_n; a.resid = resid; a.resid_scale = resid_scale;
+    dim3 grid((n + GEMM_BN - 1) / GEMM_BN, (a.m + GEMM_BM - 1) / GEMM_BM);
+    switch (w->dtype) {
+        case CERA_HIP_Q4_K: hipLaunchKernelGGL((gemm_kernel<GemmQ4K>), grid, dim3(256), 0, ctx->stream, a); break;
+        case CERA_HIP_Q6_K: hipLaunchKernelGGL((gemm_kernel<GemmQ6K>), grid, dim3(256), 0, ctx->stream, a); break;
+        case CERA_HIP_Q4_0: hipLaunchKernelGGL((gemm_kernel<GemmQ4_0>), grid, dim3(256), 0, ctx->stream, a); break;
+        case CERA_HIP_Q4_1: hipLaunchKernelGGL((gemm_kernel<GemmQ4_1>), grid, dim3(256), 0, ctx->stream, a); break;
+        default: hipLaunchKernelGGL((gemm_kernel<GemmQ8_0>), grid, dim3(256), 0, ctx->stream, a); break;
+    }
+    HIP_TRY(ctx, hipGetLastError());
+    return CERA_HIP_OK;
+}
+
+// quantize n rows of k floats: quants [n][k], scales and bsum [n][k/32]
+static cera_hip_status quantize_rows(cera_hip_ctx* ctx, const float* x, uint64_t n, uint64_t k, float* scales,
+                                     int8_t* quants, float* bsum) {
+    return cera_launch_quantize(ctx, x, n * k, scales, quants, bsum);
 }
 
 extern "C" cera_hip_status cera_hip_gemm_dev(cera_hip_ctx* ctx, const cera_hip_dtensor* w, const float* x, uint64_t n,
                                              float* out) {
-    (void)w; (void)x; (void)n; (void)out;
-    return cera_fail(ctx, CERA_HIP_ERR_UNSUPPORTED_DTYPE, "gemm: not built yet");
+    if (!ctx || !w || !x || !out) return CERA_HIP_ERR_ARGUMENT;
+    if (n == 0 || n > 0x7FFFFFFFull) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "gemm: bad n");
+    if (!cera_gemm_supports(w->dtype, w->k))
+        return cera_fail(ctx, CERA_HIP_ERR_UNSUPPORTED_DTYPE,
+                         "gemm: no int8 GEMM for ggml type " + std::to_string(w->dtype) + " with k=" + std::to_string(w->k));
+    void *ds, *dq, *db;
+    CERA_TRY(cera_scratch(ctx, 1, n * (w->k / 32) * 4, &ds));
+    CERA_TRY(cera_scratch(ctx, 2, n * w->k, &dq));
+    CERA_TRY(cera_scratch(ctx, 7, n * (w->k / 32) * 4, &db));
+    CERA_TRY(quantize_rows(ctx, x, n, w->k, static_cast<float*>(ds), static_cast<int8_t*>(dq), static_cast<float*>(db)));
+    // reference layout: out[m][n]
+    return cera_launch_gemm(ctx, w, static_cast<float*>(ds), static_cast<int8_t*>(dq), static_cast<float*>(db),
+                            static_cast<uint32_t>(n), out, n, 1, nullptr, 1.0f);
 }
-extern "C" cera_hip_status cera_hip_gemm(cera_hip_ctx* ctx, const cera_hip_tensor* w, const float* x, uint64_t n,
+
+extern "C" cera_hip_status cera_hip_gemm(cera_hip_ctx* ctx, const cera_hip_tensor* t, const float* x, uint64_t n,
                                          float* out) {
-    (void)w; (void)x; (void)n; (void)out;
-    return cera_fail(ctx, CERA_HIP_ERR_UNSUPPORTED_DTYPE, "gemm: not built yet");
+    if (!ctx || !x || !out) return CERA_HIP_ERR_ARGUMENT;
+    if (n == 0 || n > 0x7FFFFFFFull) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "gemm: bad n");
+    cera_hip_dtensor* w = nullptr;
+    CERA_TRY(cera_hip_tensor_upload(ctx, t, &w));
+    auto run = [&]() -> cera_hip_status {
+        void *dx, *dy;
+        CERA_TRY(cera_scratch(ctx, 0, n * w->k * 4, &dx));
+        CERA_TRY(cera_scratch(ctx, 3, n * w->m * 4, &dy));
+        CERA_TRY(cera_hip_upload(ctx, dx, x, n * w->k * 4));
+        CERA_TRY(cera_hip_gemm_dev(ctx, w, static_cast<float*>(dx), n, static_cast<float*>(dy)));
+        return cera_hip_download(ctx, out, dy, n * w->m * 4);
+    };
+    cera_hip_status st = run();
+    cera_hip_tensor_free(ctx, w);
+    return st;
+}
+
+// ---------------------------------------------------------------------------
+// Batched prefill of one chunk of n <= CHUNK tokens.
+static constexpr uint32_t PREFILL_CHUNK = 512;  // Session's default ubatch (cera/src/model/mod.rs:303-332)
+
+static cera_hip_status ensure_prefill_buffers(cera_hip_model* m, uint32_t n) {
+    if (m->pf_cap >= n) return CERA_HIP_OK;
+    cera_hip_ctx* ctx = m->ctx;
+    const cera_hip_config& c = m->cfg;
+    const uint64_t q_dim = static_cast<uint64_t>(c.n_heads) * c.head_dim, kv_dim = static_cast<uint64_t>(c.n_kv_heads) * c.head_dim;
+    const uint64_t maxk = std::max<uint64_t>(std::max<uint64_t>(c.hidden, c.ffn), q_dim);
+    HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    for (void* p : m->pf_owned) (void)hipFree(p);
+    m->pf_owned.clear();
+    m->pf_cap = 0;
+    const uint32_t cap = std::min<uint32_t>(PREFILL_CHUNK, std::max<uint32_t>(n, 64));
+    auto alloc = [&](uint64_t bytes, void** p) -> cera_hip_status {
+        HIP_TRY(ctx, hipMalloc(p, bytes));
+        m->pf_owned.push_back(*p);
+        m->bytes += bytes;
+        return CERA_HIP_OK;
+    };
+    CERA_TRY(alloc(cap * c.hidden * 4ull, reinterpret_cast<void**>(&m->pf_hidden)));
+    CERA_TRY(alloc(cap * c.hidden * 4ull, reinterpret_cast<void**>(&m->pf_normed)));
+    CERA_TRY(alloc(cap * q_dim * 4, reinterpret_cast<void**>(&m->pf_q)));
+    CERA_TRY(alloc(cap * kv_dim * 4, reinterpret_cast<void**>(&m->pf_k)));
+    CERA_TRY(alloc(cap * kv_dim * 4, reinterpret_cast<void**>(&m->pf_v)));
+    CERA_TRY(alloc(cap * q_dim * 4, reinterpret_cast<void**>(&m->pf_attn)));
+    CERA_TRY(alloc(cap * c.ffn * 4ull, reinterpret_cast<void**>(&m->pf_gate)));
+    CERA_TRY(alloc(cap * c.ffn * 4ull, reinterpret_cast<void**>(&m->pf_up)));
+    CERA_TRY(alloc(cap * maxk, reinterpret_cast<void**>(&m->pf_xq)));
+    CERA_TRY(alloc(cap * (maxk / 32) * 4, reinterpret_cast<void**>(&m->pf_xs)));
+    CERA_TRY(alloc(cap * (maxk / 32) * 4, reinterpret_cast<void**>(&m->pf_bsum)));
+    CERA_TRY(alloc(cap * 4ull, reinterpret_cast<void**>(&m->pf_tokens)));
+    m->pf_cap = cap;
+    return CERA_HIP_OK;
+}
+
+static __global__ void set_pos_kernel(uint32_t* scalars, uint32_t pos) { scalars[1] = pos; }
+
+static cera_hip_status prefill_chunk(cera_hip_model* m, const uint32_t* tokens, uint32_t n, uint32_t start_pos,
+                                     bool want_logits) {
+    cera_hip_ctx* ctx = m->ctx;
+    const cera_hip_config& c = m->cfg;
+    hipStream_t s = ctx->stream;
+    const uint32_t hs = c.hidden, q_dim = c.n_heads * c.head_dim, kv_dim = c.n_kv_heads * c.head_dim;
+    const float scale = c.attn_scale != 0.0f ? c.attn_scale : 1.0f / std::sqrt(static_cast<float>(c.head_dim));
+    CERA_TRY(ensure_prefill_buffers(m, n));
+    CERA_TRY(cera_hip_upload(ctx, m->pf_tokens, tokens, n * 4ull));
+    hipLaunchKernelGGL(set_pos_kernel, dim3(1), dim3(1), 0, s, m->scalars, start_pos);
+    hipLaunchKernelGGL(embed_row_kernel, dim3((hs + 255) / 256, n), dim3(256), 0, s, m->embd->dtype, m->embd->dev,
+                       m->embd->row_bytes, m->pf_tokens, hs, c.embed_scale, m->pf_hidden);
+    HIP_TRY(ctx, hipGetLastError());
+
+    auto norm_rows = [&](const float* x, const float* w, float* y) -> cera_hip_status {
+        hipLaunchKernelGGL((rmsnorm_kernel<true>), dim3(n), dim3(256), 0, s, x, w, hs, c.rms_eps, y, m->pf_xs, m->pf_xq,
+                           m->pf_bsum);
+        HIP_TRY(ctx, hipGetLastError());
+        return CERA_HIP_OK;
+    };
+    // out[n][w->m] (token-major rows) = B . W^T, optionally added onto resid
+    auto gemm = [&](const cera_hip_dtensor* w, float* out, const float* resid) -> cera_hip_status {
+        return cera_launch_gemm(ctx, w, m->pf_xs, m->pf_xq, m->pf_bsum, n, out, 1, w->m, resid, c.residual_scale);
+    };
+
+    for (uint32_t i = 0; i < c.n_layers; ++i) {
+        LayerDev& L = m->layers[i];
+        CERA_TRY(norm_rows(m->pf_hidden, L.attn_norm, m->pf_normed));
+        CERA_TRY(gemm(L.q, m->pf_q, nullptr));
+        CERA_TRY(gemm(L.k, m->pf_k, nullptr));
+        CERA_TRY(gemm(L.v, m->pf_v, nullptr));
+        if (L.q_bias) {
+            // bias rows: one launch per token keeps the kernel trivial; models with biases are rare here
+            for (uint32_t t = 0; t < n; ++t) {
+                hipLaunchKernelGGL(bias_kernel, dim3((q_dim + 255) / 256), dim3(256), 0, s, m->pf_q + static_cast<uint64_t>(t) * q_dim, L.q_bias, q_dim);
+                hipLaunchKernelGGL(bias_kernel, dim3((kv_dim + 255) / 256), dim3(256), 0, s, m->pf_k + static_cast<uint64_t>(t) * kv_dim, L.k_bias, kv_dim);
+                hipLaunchKernelGGL(bias_kernel, dim3((kv_dim + 255) / 256), dim3(256), 0, s, m->pf_v + static_cast<uint64_t>(t) * kv_dim, L.v_bias, kv_dim);
+            }
+        }
+        if (L.q_norm) {
+            hipLaunchKernelGGL((rmsnorm_kernel<false>), dim3(n * c.n_heads), dim3(256), 0, s, m->pf_q, L.q_norm, c.head_dim,
+                               c.rms_eps, m->pf_q, nullptr, nullptr, nullptr);
+            hipLaunchKernelGGL((rmsnorm_kernel<false>), dim3(n * c.n_kv_heads), dim3(256), 0, s, m->pf_k, L.k_norm, c.head_dim,
+                               c.rms_eps, m->pf_k, nullptr, nullptr, nullptr);
+        }
+        hipLaunchKernelGGL(rope_kv_kernel, dim3(c.n_heads + 2 * c.n_kv_heads, n), dim3(c.head_dim / 2), 0, s, m->pf_q, m->pf_k,
+                           m->pf_v, m->rope_table, m->scalars + 1, c.n_heads, c.n_kv_heads, c.head_dim, c.rope_type, L.kc, L.vc,
+                           c.max_seq_len);
+        HIP_TRY(ctx, hipGetLastError());
+        // causal attention: query t sees positions 0 .. start_pos + t
+        CERA_TRY(cera_launch_attn(ctx, m->pf_q, L.kc, L.vc, c.n_heads, c.n_kv_heads, c.head_dim, start_pos + 1ull,
+                                  c.max_seq_len, scale, 0, n, m->pf_attn, m->pf_xs, m->pf_xq, m->pf_bsum));
+        CERA_TRY(gemm(L.o, m->pf_hidden, m->pf_hidden));
+
+        CERA_TRY(norm_rows(m->pf_hidden, L.ffn_norm, m->pf_normed));
+        CERA_TRY(gemm(L.gate, m->pf_gate, nullptr));
+        CERA_TRY(gemm(L.up, m->pf_up, nullptr));
+        const uint64_t tot = static_cast<uint64_t>(n) * c.ffn;
+        hipLaunchKernelGGL((silu_mul_kernel<true>), dim3(static_cast<uint32_t>((tot / 4 + 255) / 256)), dim3(256), 0, s,
+                           m->pf_gate, m->pf_up, tot, m->pf_gate, m->pf_xs, m->pf_xq, m->pf_bsum);
+        HIP_TRY(ctx, hipGetLastError());
+        CERA_TRY(gemm(L.down, m->pf_hidden, m->pf_hidden));
+    }
+    m->seq_len = start_pos + n;
+    if (want_logits) {
+        // last token: final norm then the decode-style GEMV (project_logits)
+        const float* last = m->pf_hidden + static_cast<uint64_t>(n - 1) * hs;
+        hipLaunchKernelGGL((rmsnorm_kernel<true>), dim3(1), dim3(256), 0, s, last, m->output_norm, hs, c.rms_eps, m->hidden,
+                           m->xs, m->xq, static_cast<float*>(nullptr));
+        HIP_TRY(ctx, hipGetLastError());
+        const cera_hip_dtensor* o = m->output ? m->output : m->embd;
+        if (o->dtype == CERA_HIP_Q5_K) CERA_TRY(cera_launch_gemv_q5k_f32(ctx, o, m->hidden, m->logits));
+        else CERA_TRY(cera_launch_gemv(ctx, o, nullptr, m->xs, m->xq, m->logits, nullptr, CERA_EPI_STORE));
+        if (c.logit_scale != 1.0f) {
+            hipLaunchKernelGGL(scale_kernel, dim3((c.vocab + 255) / 256), dim3(256), 0, s, m->logits, 1.0f / c.logit_scale, c.vocab);
+            HIP_TRY(ctx, hipGetLastError());
+        }
+    }
+    return CERA_HIP_OK;
+}
+
+cera_hip_status cera_model_prefill(cera_hip_model* m, const uint32_t* tokens, uint32_t n, uint32_t start_pos,
+                                   float* last_logits) {
+    // A single token, or a weight type without an int8 GEMM, takes the per-token
+    // route -- the same decision LlamaModel::forward_prefill makes (llama.rs:1643,
+    // 762-795); it is still the HIP path, only slower.
+    bool batched = n > 1;
+    for (const LayerDev& L : m->layers)
+        for (const cera_hip_dtensor* w : {L.q, L.k, L.v, L.o, L.gate, L.up, L.down})
+            if (!cera_gemm_supports(w->dtype, w->k)) batched = false;
+    if (!batched) return cera_model_prefill_per_token(m, tokens, n, start_pos, last_logits);
+    for (uint32_t off = 0; off < n; off += PREFILL_CHUNK) {
+        uint32_t len = std::min(PREFILL_CHUNK, n - off);
+        CERA_TRY(prefill_chunk(m, tokens + off, len, start_pos + off, off + len == n));
+    }
+    return cera_hip_download(m->ctx, last_logits, m->logits, static_cast<uint64_t>(m->cfg.vocab) * 4);
 }

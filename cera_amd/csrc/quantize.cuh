@@ -39,18 +39,35 @@ __device__ __forceinline__ uint32_t q8_quantize_quad(float4 v, float& scale_out)
     return q0 | (q1 << 8) | (q2 << 16) | (q3 << 24);
 }
 
+// scale * (sum of the 32 quants of the block this lane belongs to): the
+// activation-side factor of the Q4_K / Q4_1 min terms.  |sum| <= 32*128 and the
+// scale has an 11-bit significand, so the product is exact in f32.
+__device__ __forceinline__ float q8_block_scaled_sum(uint32_t packed, float scale) {
+    int s = sum4(packed, 0);
+    s += __builtin_amdgcn_update_dpp(0, s, 0xB1, 0xF, 0xF, true);
+    s += __builtin_amdgcn_update_dpp(0, s, 0x4E, 0xF, 0xF, true);
+    s += __builtin_amdgcn_update_dpp(0, s, 0x141, 0xF, 0xF, true);
+    return scale * static_cast<float>(s);
+}
+
 // grid: ceil(k/4 / 256) blocks of 256 threads; thread t owns x[4t .. 4t+3].
+// bsum (nullable): per-block scale * sum(quants), consumed by the prefill GEMM.
 static __global__ __launch_bounds__(256) void quantize_q8_0_kernel(const float* __restrict__ x, uint64_t k,
                                                             float* __restrict__ scales,
-                                                            int8_t* __restrict__ quants) {
+                                                            int8_t* __restrict__ quants,
+                                                            float* __restrict__ bsum) {
     uint64_t t = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     bool live = 4 * t < k;
     // k % 32 == 0, so a whole 8-lane group is live or dead together.
     float4 v = live ? reinterpret_cast<const float4*>(x)[t] : make_float4(0.f, 0.f, 0.f, 0.f);
     float scale;
     uint32_t packed = q8_quantize_quad(v, scale);
+    float ssum = bsum ? q8_block_scaled_sum(packed, scale) : 0.0f;
     if (live) {
         reinterpret_cast<uint32_t*>(quants)[t] = packed;
-        if ((t & 7) == 0) scales[t >> 3] = scale;
+        if ((t & 7) == 0) {
+            scales[t >> 3] = scale;
+            if (bsum) bsum[t >> 3] = ssum;
+        }
     }
 }

@@ -94,6 +94,8 @@ def lib() -> C.CDLL:
         "orc_llama_seq_len": (u32, [vp]), "orc_llama_truncate": (None, [vp, u32]),
         "orc_llama_forward": (i32, [vp, u32, u32, vp, vp]),
         "orc_llama_forward_prefill_per_token": (i32, [vp, vp, u32, u32, vp]),
+        "orc_llama_forward_prefill_batched": (i32, [vp, vp, u32, u32, vp, vp]),
+        "orc_flash_attention_head": (None, [vp, vp, vp, vp, u64, u64, u64, u32, f32, u64]),
         "orc_llama_kcache": (vp, [vp, u32]), "orc_llama_vcache": (vp, [vp, u32]),
     }
     for name, (res, args) in sig.items():
@@ -251,6 +253,17 @@ def decode_attention(q, k_cache, v_cache, n_heads, n_kv_heads, head_dim, scale, 
     return out
 
 
+def flash_attention_head(q, k_cache, v_cache, n_queries, kv_dim, kv_h_offset, head_dim, scale, start_pos):
+    """q [n_queries][head_dim] of one head; caches time-major [pos][kv_dim]."""
+    q = np.ascontiguousarray(q, np.float32)
+    kc = np.ascontiguousarray(k_cache, np.float32)
+    vc = np.ascontiguousarray(v_cache, np.float32)
+    out = np.empty((n_queries, head_dim), np.float32)
+    lib().orc_flash_attention_head(_p(q), _p(kc), _p(vc), _p(out), n_queries, kv_dim, kv_h_offset, head_dim, scale,
+                                   start_pos)
+    return out
+
+
 class Pool:
     def __init__(self, n_threads: int):
         self.h = lib().orc_pool_create(n_threads)
@@ -343,6 +356,15 @@ class Llama:
         rc = lib().orc_llama_forward_prefill_per_token(self.h, _p(t), t.size, start_pos, _p(logits))
         assert rc == 0, rc
         return logits
+
+    def forward_prefill_batched(self, tokens, start_pos: int, want_hidden: bool = False):
+        t = np.ascontiguousarray(tokens, np.uint32)
+        logits = np.empty(self.vocab, np.float32)
+        hid = np.empty((t.size, self.hidden), np.float32) if want_hidden else None
+        rc = lib().orc_llama_forward_prefill_batched(self.h, _p(t), t.size, start_pos, _p(logits),
+                                                     _p(hid) if want_hidden else None)
+        assert rc == 0, rc
+        return (logits, hid) if want_hidden else logits
 
     def kv(self, layer: int):
         n = self.seq_len * self.cfg["n_kv_heads"] * self.cfg["head_dim"]

@@ -120,3 +120,8 @@ ORC_API void orc_attn_values(const float* scores, const float* v_cache, float* o
 ORC_API void orc_decode_attention(const float* q, const float* k_cache, const float* v_cache,
                                   uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim,
                                   float scale, uint64_t seq_len, float* out, int variant);
+
+// One head of flash_attention_gqa_cpu (scalar route): q, out are [n_queries][head_dim].
+ORC_API void orc_flash_attention_head(const float* q, const float* k_cache, const float* v_cache, float* out,
+                                      uint64_t n_queries, uint64_t kv_dim, uint64_t kv_h_offset,
+                                      uint32_t head_dim, float scale, uint64_t start_pos);

@@ -130,3 +130,124 @@ int orc_llama_forward_prefill_per_token(OrcLlama* m, const uint32_t* tokens, uin
 
 const float* orc_llama_kcache(const OrcLlama* m, uint32_t layer) { return m->kc[layer].data(); }
 const float* orc_llama_vcache(const OrcLlama* m, uint32_t layer) { return m->vc[layer].data(); }
+
+// ---------------------------------------------------------------------------
+// forward_prefill_batched (llama.rs:738-1523), no-`blas` int8 route.  The
+// reference keeps activations column-major [dim][n]; here they are row-major
+// [n][dim] -- the same numbers, and every per-element operation is in the
+// reference's order.  GEMMs are gemm_preq over quantize_columns
+// (transformer.rs:710-788, 865-946) with the tiled (n > 1) accumulator order.
+static void quantize_rows(const std::vector<float>& x, uint32_t n, uint32_t dim, std::vector<float>& bs,
+                          std::vector<int8_t>& bq) {
+    bs.resize(size_t(n) * (dim / 32));
+    bq.resize(size_t(n) * dim);
+    for (uint32_t j = 0; j < n; ++j)
+        orc_quantize_q8_0(x.data() + size_t(j) * dim, dim, bs.data() + size_t(j) * (dim / 32), bq.data() + size_t(j) * dim);
+}
+// out_rows[n][m] = (W . B)^T, B given as quantized rows
+static int gemm_rows(OrcLlama* m, const OrcTensor& t, const std::vector<float>& bs, const std::vector<int8_t>& bq,
+                     uint32_t n, std::vector<float>& out_rows, std::vector<float>& tmp) {
+    tmp.resize(size_t(t.m) * n);
+    int rc = orc_gemm_preq(t.dtype, t.data, bs.data(), bq.data(), tmp.data(), t.m, n, t.k, m->variant);
+    if (rc) return rc;
+    out_rows.resize(size_t(n) * t.m);
+    for (uint64_t i = 0; i < t.m; ++i)
+        for (uint32_t j = 0; j < n; ++j) out_rows[size_t(j) * t.m + i] = tmp[i * n + j];
+    return 0;
+}
+
+int orc_llama_forward_prefill_batched(OrcLlama* m, const uint32_t* tokens, uint32_t n, uint32_t start_pos,
+                                      float* last_logits, float* all_hidden) {
+    const OrcLlamaConfig& c = m->cfg;
+    if (n == 0 || start_pos != m->seq_len) return -1;
+    const uint32_t hs = c.hidden, hd = c.head_dim, is = c.ffn;
+    const uint32_t q_dim = c.n_heads * hd, kv_dim = c.n_kv_heads * hd, group = c.n_heads / c.n_kv_heads;
+    const float scale = c.attn_scale != 0.0f ? c.attn_scale : 1.0f / std::sqrt(float(hd));
+    std::vector<float> hidden(size_t(n) * hs), normed(size_t(n) * hs), qm, km, vm, attn(size_t(n) * q_dim), blk, gate, up, tmp;
+    std::vector<float> bs;
+    std::vector<int8_t> bq;
+    for (uint32_t j = 0; j < n; ++j) {
+        if (tokens[j] >= c.vocab) return -1;
+        const uint8_t* erow = static_cast<const uint8_t*>(m->embd.data) + uint64_t(tokens[j]) * orc_row_bytes(m->embd.dtype, m->embd.k);
+        if (orc_dequantize_row(m->embd.dtype, erow, m->embd.k, hidden.data() + size_t(j) * hs)) return -2;
+        if (c.embed_scale != 1.0f) for (uint32_t i = 0; i < hs; ++i) hidden[size_t(j) * hs + i] *= c.embed_scale;
+    }
+    const bool use_flash = n >= 256;  // FLASH_ATTN_THRESHOLD, llama.rs:845
+    std::vector<float> qh(size_t(n) * hd), oh(size_t(n) * hd), scores;
+    for (uint32_t l = 0; l < c.n_layers; ++l) {
+        const OrcLlamaLayer& L = m->layers[l];
+        normed = hidden;
+        for (uint32_t j = 0; j < n; ++j) orc_rmsnorm(normed.data() + size_t(j) * hs, L.attn_norm, hs, c.rms_eps);
+        quantize_rows(normed, n, hs, bs, bq);
+        if (gemm_rows(m, L.attn_q, bs, bq, n, qm, tmp) || gemm_rows(m, L.attn_k, bs, bq, n, km, tmp) ||
+            gemm_rows(m, L.attn_v, bs, bq, n, vm, tmp))
+            return -3;
+        for (uint32_t j = 0; j < n; ++j) {
+            float* q = qm.data() + size_t(j) * q_dim;
+            float* k = km.data() + size_t(j) * kv_dim;
+            float* v = vm.data() + size_t(j) * kv_dim;
+            if (L.q_bias && L.k_bias && L.v_bias) {
+                orc_add(q, L.q_bias, q_dim);
+                orc_add(k, L.k_bias, kv_dim);
+                orc_add(v, L.v_bias, kv_dim);
+            }
+            if (L.q_norm && L.k_norm) {
+                for (uint32_t h = 0; h < c.n_heads; ++h) orc_rmsnorm(q + h * hd, L.q_norm, hd, c.rms_eps);
+                for (uint32_t h = 0; h < c.n_kv_heads; ++h) orc_rmsnorm(k + h * hd, L.k_norm, hd, c.rms_eps);
+            }
+            if (c.rope_type == 0) orc_rope_neox(q, k, start_pos + j, c.n_heads, c.n_kv_heads, hd, c.rope_theta);
+            else orc_rope_norm(q, k, start_pos + j, c.n_heads, c.n_kv_heads, hd, c.rope_theta, c.rope_freqs);
+            m->kc[l].insert(m->kc[l].end(), k, k + kv_dim);
+            m->vc[l].insert(m->vc[l].end(), v, v + kv_dim);
+        }
+        const float* kcache = m->kc[l].data();
+        const float* vcache = m->vc[l].data();
+        if (use_flash) {
+            for (uint32_t h = 0; h < c.n_heads; ++h) {
+                for (uint32_t j = 0; j < n; ++j)
+                    std::memcpy(qh.data() + size_t(j) * hd, qm.data() + size_t(j) * q_dim + h * hd, hd * sizeof(float));
+                orc_flash_attention_head(qh.data(), kcache, vcache, oh.data(), n, kv_dim, uint64_t(h / group) * hd, hd, scale, start_pos);
+                for (uint32_t j = 0; j < n; ++j)
+                    std::memcpy(attn.data() + size_t(j) * q_dim + h * hd, oh.data() + size_t(j) * hd, hd * sizeof(float));
+            }
+        } else {
+            for (uint32_t j = 0; j < n; ++j) {
+                uint64_t L_ctx = uint64_t(start_pos) + j + 1;
+                orc_decode_attention(qm.data() + size_t(j) * q_dim, kcache, vcache, c.n_heads, c.n_kv_heads, hd, scale, L_ctx,
+                                     attn.data() + size_t(j) * q_dim, m->variant);
+            }
+        }
+        quantize_rows(attn, n, q_dim, bs, bq);
+        if (gemm_rows(m, L.attn_output, bs, bq, n, blk, tmp)) return -3;
+        if (c.residual_scale != 1.0f) for (auto& x : blk) x *= c.residual_scale;
+        orc_add(hidden.data(), blk.data(), size_t(n) * hs);
+
+        normed = hidden;
+        for (uint32_t j = 0; j < n; ++j) orc_rmsnorm(normed.data() + size_t(j) * hs, L.ffn_norm, hs, c.rms_eps);
+        quantize_rows(normed, n, hs, bs, bq);
+        if (gemm_rows(m, L.ffn_gate, bs, bq, n, gate, tmp) || gemm_rows(m, L.ffn_up, bs, bq, n, up, tmp)) return -3;
+        orc_silu_mul(gate.data(), up.data(), size_t(n) * is);
+        quantize_rows(gate, n, is, bs, bq);
+        if (gemm_rows(m, L.ffn_down, bs, bq, n, blk, tmp)) return -3;
+        if (c.residual_scale != 1.0f) for (auto& x : blk) x *= c.residual_scale;
+        orc_add(hidden.data(), blk.data(), size_t(n) * hs);
+    }
+    m->seq_len = start_pos + n;
+    if (all_hidden) {
+        for (uint32_t j = 0; j < n; ++j) {
+            std::memcpy(all_hidden + size_t(j) * hs, hidden.data() + size_t(j) * hs, hs * sizeof(float));
+            orc_rmsnorm(all_hidden + size_t(j) * hs, m->output_norm, hs, c.rms_eps);
+        }
+    }
+    if (last_logits) {
+        std::vector<float> last(hidden.begin() + size_t(n - 1) * hs, hidden.end());
+        orc_rmsnorm(last.data(), m->output_norm, hs, c.rms_eps);
+        const OrcTensor& o = m->has_output ? m->output : m->embd;
+        gemv(m, o, last.data(), last_logits);  // project_logits: the n == 1 GEMV branch
+        if (c.logit_scale != 1.0f) {
+            float inv = 1.0f / c.logit_scale;
+            for (uint32_t i = 0; i < c.vocab; ++i) last_logits[i] *= inv;
+        }
+    }
+    return 0;
+}

@@ -37,5 +37,10 @@ ORC_API int      orc_llama_forward(OrcLlama*, uint32_t token, uint32_t pos, floa
                                    float* hidden_out /*nullable*/);
 ORC_API int      orc_llama_forward_prefill_per_token(OrcLlama*, const uint32_t* tokens, uint32_t n,
                                                      uint32_t start_pos, float* last_logits);
+// LlamaModel::forward_prefill_batched (llama.rs:738-1523): all n tokens through
+// each layer together; logits of the last token.  all_hidden (nullable)
+// receives the per-token final-normed hidden states [n][hidden].
+ORC_API int      orc_llama_forward_prefill_batched(OrcLlama*, const uint32_t* tokens, uint32_t n,
+                                                   uint32_t start_pos, float* last_logits, float* all_hidden);
 ORC_API const float* orc_llama_kcache(const OrcLlama*, uint32_t layer);
 ORC_API const float* orc_llama_vcache(const OrcLlama*, uint32_t layer);

@@ -228,3 +228,54 @@ void orc_decode_attention(const float* q, const float* kc, const float* vc, uint
         orc_attn_values(scores.data(), vc, out + h * hd, kv_dim, off, hd, L, variant);
     }
 }
+
+// ---------------------------------------------------------------------------
+// Causal prefill attention, tiled online softmax -- the scalar route of
+// flash_attention_gqa_cpu (cpu.rs:4028-4241, FLASH_TILE_KV = 32): per query j
+// (absolute position start_pos + j) scores over positions 0..=start_pos+j in
+// tiles of 32, running max, f64 running sum, ggml expf.  The reference's AVX2
+// twin (cpu.rs:4261-4412) differs only in f32 summation order.
+// q is [n_queries][head_dim] for ONE head (row-major); out likewise.
+void orc_flash_attention_head(const float* q, const float* k_cache, const float* v_cache, float* out,
+                              uint64_t n_queries, uint64_t kv_dim, uint64_t kv_h_offset,
+                              uint32_t head_dim, float scale, uint64_t start_pos) {
+    const int TILE = 32;
+    std::vector<float> acc(head_dim);
+    float tile_scores[TILE];
+    for (uint64_t j = 0; j < n_queries; ++j) {
+        uint64_t max_kv = start_pos + j + 1;
+        const float* ql = q + j * head_dim;
+        float running_max = -INFINITY;
+        double running_sum = 0.0;
+        for (auto& a : acc) a = 0.0f;
+        for (uint64_t kv_start = 0; kv_start < max_kv; kv_start += TILE) {
+            uint64_t kv_end = kv_start + TILE < max_kv ? kv_start + TILE : max_kv;
+            int tile_len = int(kv_end - kv_start);
+            for (int ti = 0; ti < tile_len; ++ti) {
+                const float* kp = k_cache + (kv_start + ti) * kv_dim + kv_h_offset;
+                float dot = 0.0f;
+                for (uint32_t d = 0; d < head_dim; ++d) dot += ql[d] * kp[d];
+                tile_scores[ti] = dot * scale;
+            }
+            float tile_max = -INFINITY;
+            for (int ti = 0; ti < tile_len; ++ti) tile_max = fmaxf(tile_max, tile_scores[ti]);
+            float new_max = fmaxf(running_max, tile_max);
+            float rescale = running_max > -INFINITY ? orc_expf(running_max - new_max) : 0.0f;
+            double tile_sum = 0.0;
+            for (int ti = 0; ti < tile_len; ++ti) {
+                tile_scores[ti] = orc_expf(tile_scores[ti] - new_max);
+                tile_sum += double(tile_scores[ti]);
+            }
+            for (uint32_t d = 0; d < head_dim; ++d) acc[d] *= rescale;
+            for (int ti = 0; ti < tile_len; ++ti) {
+                float s = tile_scores[ti];
+                const float* vp = v_cache + (kv_start + ti) * kv_dim + kv_h_offset;
+                for (uint32_t d = 0; d < head_dim; ++d) acc[d] += s * vp[d];
+            }
+            running_sum = running_sum * double(rescale) + tile_sum;
+            running_max = new_max;
+        }
+        float inv_sum = float(1.0 / running_sum);
+        for (uint32_t d = 0; d < head_dim; ++d) out[j * head_dim + d] = acc[d] * inv_sum;
+    }
+}
