@@ -263,12 +263,46 @@ cera_hip_status cera_hip_tensor_clone(cera_hip_ctx* ctx, const cera_hip_dtensor*
 void cera_hip_tensor_free(cera_hip_ctx* ctx, cera_hip_dtensor* d) {
     if (!d) return;
     if (ctx) (void)hipStreamSynchronize(ctx->stream);
-    if (d->dev) (void)hipFree(d->dev);
+    if (d->dev && d->owns) (void)hipFree(d->dev);
     delete d;
 }
 uint64_t cera_hip_tensor_nbytes(const cera_hip_dtensor* d) { return d ? d->nbytes : 0; }
 
 }  // extern "C"
+
+cera_hip_status cera_tensor_upload_concat(cera_hip_ctx* ctx, const cera_hip_tensor* const* parts, int n_parts,
+                                          cera_hip_dtensor** fused, cera_hip_dtensor** views) {
+    *fused = nullptr;
+    uint64_t rb = 0, rows = 0;
+    for (int i = 0; i < n_parts; ++i) {
+        uint64_t r;
+        CERA_TRY(check_tensor(ctx, parts[i], &r));
+        if (parts[i]->ggml_type != parts[0]->ggml_type || parts[i]->k != parts[0]->k)
+            return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "concat: parts differ in type or k");
+        rb = r;
+        rows += parts[i]->m;
+    }
+    cera_hip_dtensor* f;
+    CERA_TRY(alloc_dtensor(ctx, parts[0]->ggml_type, rows, parts[0]->k, rb, &f));
+    uint64_t off = 0;
+    for (int i = 0; i < n_parts; ++i) {
+        hipError_t e = hipMemcpyAsync(f->dev + off, parts[i]->data, parts[i]->nbytes, hipMemcpyHostToDevice, ctx->stream);
+        if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+        cera_hip_dtensor* v = e == hipSuccess ? new (std::nothrow) cera_hip_dtensor() : nullptr;
+        if (!v) {
+            for (int j = 0; j < i; ++j) { delete views[j]; views[j] = nullptr; }
+            cera_hip_tensor_free(ctx, f);
+            return cera_fail(ctx, e != hipSuccess ? CERA_HIP_ERR_DEVICE : CERA_HIP_ERR_OOM,
+                             e != hipSuccess ? std::string("weight upload: ") + hipGetErrorString(e) : "host allocation failed");
+        }
+        v->dtype = f->dtype; v->m = parts[i]->m; v->k = f->k; v->row_bytes = rb; v->nbytes = parts[i]->nbytes;
+        v->dev = f->dev + off; v->owns = false;
+        views[i] = v;
+        off += parts[i]->nbytes;
+    }
+    *fused = f;
+    return CERA_HIP_OK;
+}
 
 // ---------------------------------------------------------------------------
 // launchers
@@ -349,11 +383,14 @@ cera_hip_status cera_launch_attn(cera_hip_ctx* ctx, const float* q, const float*
     // seq_len = keys visible to the first query; the last query sees seq_len + n_queries - 1
     const uint64_t last_len = seq_len + n_queries - 1;
     if (seq_len == 0 || last_len > max_seq || max_seq > 0x7FFFFFFFull) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "attention: need 0 < seq_len <= max_seq < 2^31");
-    if (n_heads % 2) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "attention: n_heads must be even");
-    uint32_t n_chunks = static_cast<uint32_t>((last_len + ATTN_CHUNK - 1) / ATTN_CHUNK);
+    // positions per chunk: small chunks while the context is short (one memory round
+    // trip per wavefront, many wavefronts), 64 once there is plenty of work
+    const uint32_t S = last_len >= 16384 ? 8 : (last_len >= 4096 ? 4 : (last_len >= 1024 ? 2 : 1));
+    uint32_t n_chunks = static_cast<uint32_t>((last_len + 8 * S - 1) / (8 * S));
     // parts (wavefronts) per (query, kv head): enough to fill the chip ~8 waves per CU
-    // deep, but at least one chunk each
+    // deep, but at least one chunk each and at most ATTN_MAX_PARTS
     uint32_t want_parts = n_splits ? n_splits : std::max(1u, ctx->n_cu * 8 / (n_kv_heads * n_queries));
+    want_parts = std::min<uint32_t>(want_parts, ATTN_MAX_PARTS);
     uint32_t chunks_per_part = std::max(1u, (n_chunks + want_parts - 1) / want_parts);
     uint32_t n_parts = (n_chunks + chunks_per_part - 1) / chunks_per_part;
     uint64_t acc_bytes = static_cast<uint64_t>(n_queries) * n_kv_heads * n_parts * G * ATTN_HD * sizeof(float);
@@ -375,23 +412,31 @@ cera_hip_status cera_launch_attn(cera_hip_ctx* ctx, const float* q, const float*
     dim3 grid((n_parts + 3) / 4, n_kv_heads, n_queries);
     uint32_t sl = static_cast<uint32_t>(seq_len), ms = static_cast<uint32_t>(max_seq);
     uint32_t q_stride = n_heads * head_dim;
-#define ATTN_LAUNCH(GG)                                                                                    \
-    hipLaunchKernelGGL((attn_decode_partial_kernel<GG>), grid, dim3(256), 0, ctx->stream, q, kc, vc, sl, ms, \
+#define ATTN_LAUNCH_S(GG, SS)                                                                                  \
+    hipLaunchKernelGGL((attn_decode_partial_kernel<GG, SS>), grid, dim3(256), 0, ctx->stream, q, kc, vc, sl, ms, \
                        scale, chunks_per_part, n_parts, q_stride, ctx->attn_acc, ctx->attn_ml)
+#define ATTN_LAUNCH(GG)                              \
+    switch (S) {                                     \
+        case 1: ATTN_LAUNCH_S(GG, 1); break;         \
+        case 2: ATTN_LAUNCH_S(GG, 2); break;         \
+        case 4: ATTN_LAUNCH_S(GG, 4); break;         \
+        default: ATTN_LAUNCH_S(GG, 8); break;        \
+    }
     switch (G) {
         case 1: ATTN_LAUNCH(1); break;
         case 2: ATTN_LAUNCH(2); break;
         case 4: ATTN_LAUNCH(4); break;
         default: ATTN_LAUNCH(8); break;
     }
+#undef ATTN_LAUNCH_S
 #undef ATTN_LAUNCH
     HIP_TRY(ctx, hipGetLastError());
-    dim3 mgrid(n_heads / 2, n_queries);
+    dim3 mgrid(n_heads, n_queries);
     if (out_quants)
-        hipLaunchKernelGGL((attn_decode_merge_kernel<true>), mgrid, dim3(64), 0, ctx->stream, ctx->attn_acc,
+        hipLaunchKernelGGL((attn_decode_merge_kernel<true>), mgrid, dim3(256), 0, ctx->stream, ctx->attn_acc,
                            ctx->attn_ml, n_parts, G, n_heads, out, out_scales, out_quants, out_bsum);
     else
-        hipLaunchKernelGGL((attn_decode_merge_kernel<false>), mgrid, dim3(64), 0, ctx->stream, ctx->attn_acc,
+        hipLaunchKernelGGL((attn_decode_merge_kernel<false>), mgrid, dim3(256), 0, ctx->stream, ctx->attn_acc,
                            ctx->attn_ml, n_parts, G, n_heads, out, static_cast<float*>(nullptr),
                            static_cast<int8_t*>(nullptr), static_cast<float*>(nullptr));
     HIP_TRY(ctx, hipGetLastError());

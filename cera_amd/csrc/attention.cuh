@@ -25,13 +25,17 @@
 #include "quantize.cuh"
 
 #define ATTN_HD 128
-#define ATTN_CHUNK 64
+#define ATTN_MAX_PARTS 1024  // the merge kernel keeps one weight per part in LDS
 
 struct AttnPart {  // per (part, query head): running max, sum and unnormalised output
     float m, l;
 };
 
-template <int G>
+// S = steps of 8 positions per chunk.  Short contexts use small chunks so that
+// every wavefront has a single memory round trip (all its K and V loads in
+// flight at once) and there are enough wavefronts to cover the chip; long
+// contexts use 64-position chunks to amortise the softmax bookkeeping.
+template <int G, int S>
 __global__ __launch_bounds__(256) void attn_decode_partial_kernel(
     const float* __restrict__ q,       // [n_heads][128]
     const float* __restrict__ kc,      // [n_kv][max_seq][128]
@@ -69,14 +73,26 @@ __global__ __launch_bounds__(256) void attn_decode_partial_kernel(
 
     const float* kbase = kc + static_cast<uint64_t>(kvh) * max_seq * ATTN_HD;
     const float* vbase = vc + static_cast<uint64_t>(kvh) * max_seq * ATTN_HD;
-    const uint32_t t_begin = part * chunks_per_part * ATTN_CHUNK;
-    const uint32_t t_end = min(seq_len, t_begin + chunks_per_part * ATTN_CHUNK);
+    constexpr uint32_t CHUNK = 8 * S;
+    constexpr bool PREFETCH_V = S <= 2;  // small chunks: V loads issued together with K
+    const uint32_t t_begin = part * chunks_per_part * CHUNK;
+    const uint32_t t_end = min(seq_len, t_begin + chunks_per_part * CHUNK);
 
-    for (uint32_t t0 = t_begin; t0 < t_end; t0 += ATTN_CHUNK) {
-        // ---- scores for 64 positions: step s covers positions t0 + 8s + pg
-        float sc[G][8];
+    for (uint32_t t0 = t_begin; t0 < t_end; t0 += CHUNK) {
+        float4 vpre[PREFETCH_V ? S : 1][4];
+        if (PREFETCH_V) {
 #pragma unroll
-        for (int s = 0; s < 8; ++s) {
+            for (int s = 0; s < S; ++s) {
+                uint32_t t = t0 + 8 * s + pg;
+                const float4* vp = reinterpret_cast<const float4*>(vbase + static_cast<uint64_t>(t < t_end ? t : t_begin) * ATTN_HD);
+#pragma unroll
+                for (int c = 0; c < 4; ++c) vpre[s][c] = vp[j + 8 * c];
+            }
+        }
+        // ---- scores: step s covers positions t0 + 8s + pg
+        float sc[G][S];
+#pragma unroll
+        for (int s = 0; s < S; ++s) {
             uint32_t t = t0 + 8 * s + pg;
             bool live = t < t_end;
             const float4* kp = reinterpret_cast<const float4*>(kbase + static_cast<uint64_t>(live ? t : t_begin) * ATTN_HD);
@@ -105,7 +121,7 @@ __global__ __launch_bounds__(256) void attn_decode_partial_kernel(
         for (int h = 0; h < G; ++h) {
             float mx = sc[h][0];
 #pragma unroll
-            for (int s = 1; s < 8; ++s) mx = fmaxf(mx, sc[h][s]);
+            for (int s = 1; s < S; ++s) mx = fmaxf(mx, sc[h][s]);
             mx = wave_max(mx);
             float m_new = fmaxf(m[h], mx);
             corr[h] = cera_expf(m[h] - m_new);  // 0 on the first chunk (m = -inf)
@@ -119,13 +135,17 @@ __global__ __launch_bounds__(256) void attn_decode_partial_kernel(
         }
         // ---- P.V: this lane's positions, its 16 columns
 #pragma unroll
-        for (int s = 0; s < 8; ++s) {
-            uint32_t t = t0 + 8 * s + pg;
-            bool live = t < t_end;
-            const float4* vp = reinterpret_cast<const float4*>(vbase + static_cast<uint64_t>(live ? t : t_begin) * ATTN_HD);
+        for (int s = 0; s < S; ++s) {
             float4 vv[4];
+            if (PREFETCH_V) {
 #pragma unroll
-            for (int c = 0; c < 4; ++c) vv[c] = vp[j + 8 * c];
+                for (int c = 0; c < 4; ++c) vv[c] = vpre[s][c];
+            } else {
+                uint32_t t = t0 + 8 * s + pg;
+                const float4* vp = reinterpret_cast<const float4*>(vbase + static_cast<uint64_t>(t < t_end ? t : t_begin) * ATTN_HD);
+#pragma unroll
+                for (int c = 0; c < 4; ++c) vv[c] = vp[j + 8 * c];
+            }
 #pragma unroll
             for (int h = 0; h < G; ++h) {
                 float p = cera_expf(sc[h][s] - m[h]);  // -inf score -> 0
@@ -175,43 +195,72 @@ __global__ __launch_bounds__(256) void attn_decode_partial_kernel(
 }
 
 // Merge the parts of one query head: out = sum_p e^{m_p - M} acc_p / sum_p e^{m_p - M} l_p.
-// 32 threads per head (a float4 of the 128 columns each).  Optionally writes
-// the Q8_0 quantisation of the result for the output projection.
+// One workgroup of 256 threads per (head, query): the maxima and weights are
+// computed with the parts spread over all threads, the weighted accumulation
+// with the parts spread over 8 groups of 32 lanes (a float4 of the 128 columns
+// per lane), so the dependent-load chain is n_parts / 8 long.  Group 0 folds
+// the groups together and optionally writes the Q8_0 quantisation of the
+// result for the output projection.
 template <bool QUANT>
-__global__ __launch_bounds__(64) void attn_decode_merge_kernel(const float* __restrict__ part_acc,
-                                                               const float* __restrict__ part_ml,
-                                                               uint32_t n_parts, uint32_t G, uint32_t n_heads,
-                                                               float* __restrict__ out,
-                                                               float* __restrict__ scales,
-                                                               int8_t* __restrict__ quants,
-                                                               float* __restrict__ bsum) {
-    const uint32_t head = blockIdx.x * 2 + (threadIdx.x >> 5), c = threadIdx.x & 31;
+__global__ __launch_bounds__(256) void attn_decode_merge_kernel(const float* __restrict__ part_acc,
+                                                                const float* __restrict__ part_ml,
+                                                                uint32_t n_parts, uint32_t G, uint32_t n_heads,
+                                                                float* __restrict__ out,
+                                                                float* __restrict__ scales,
+                                                                int8_t* __restrict__ quants,
+                                                                float* __restrict__ bsum) {
+    __shared__ float wbuf[ATTN_MAX_PARTS];
+    __shared__ float red[8];
+    __shared__ float4 sacc[8][32];
+    const uint32_t head = blockIdx.x, tid = threadIdx.x, c = tid & 31, grp = tid >> 5, wave = tid >> 6;
     const uint32_t kvh = head / G, hg = head % G, qi = blockIdx.y, n_kv = n_heads / G;
     const uint64_t pbase = (static_cast<uint64_t>(qi) * n_kv + kvh) * n_parts;
     float M = -__builtin_inff();
-    for (uint32_t p = 0; p < n_parts; ++p) M = fmaxf(M, part_ml[((pbase + p) * G + hg) * 2]);
-    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (uint32_t p = tid; p < n_parts; p += 256) M = fmaxf(M, part_ml[((pbase + p) * G + hg) * 2]);
+    M = wave_max(M);
+    if ((tid & 63) == 0) red[wave] = M;
+    __syncthreads();
+    M = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
     float L = 0.0f;
-    for (uint32_t p = 0; p < n_parts; ++p) {
-        uint64_t idx = (pbase + p) * G + hg;
-        float w = cera_expf(part_ml[idx * 2] - M);
-        L = fmaf(w, part_ml[idx * 2 + 1], L);
-        float4 a = reinterpret_cast<const float4*>(part_acc + idx * ATTN_HD)[c];
+    for (uint32_t p = tid; p < n_parts; p += 256) {
+        const float2 ml = *reinterpret_cast<const float2*>(part_ml + ((pbase + p) * G + hg) * 2);
+        float w = cera_expf(ml.x - M);
+        wbuf[p] = w;
+        L = fmaf(w, ml.y, L);
+    }
+    L = wave_sum(L);
+    if ((tid & 63) == 0) red[4 + wave] = L;
+    __syncthreads();
+    L = (red[4] + red[5]) + (red[6] + red[7]);
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll 2
+    for (uint32_t p = grp; p < n_parts; p += 8) {
+        const float w = wbuf[p];
+        const float4 a = reinterpret_cast<const float4*>(part_acc + ((pbase + p) * G + hg) * ATTN_HD)[c];
         acc.x = fmaf(w, a.x, acc.x); acc.y = fmaf(w, a.y, acc.y);
         acc.z = fmaf(w, a.z, acc.z); acc.w = fmaf(w, a.w, acc.w);
     }
-    float inv = 1.0f / L;
-    float4 o = make_float4(acc.x * inv, acc.y * inv, acc.z * inv, acc.w * inv);
-    const uint64_t row = static_cast<uint64_t>(qi) * n_heads + head;  // outputs are [n_queries][n_heads][128]
-    reinterpret_cast<float4*>(out + row * ATTN_HD)[c] = o;
-    if (QUANT) {
-        float sc;
-        uint32_t packed = q8_quantize_quad(o, sc);
-        float ssum = bsum ? q8_block_scaled_sum(packed, sc) : 0.0f;
-        reinterpret_cast<uint32_t*>(quants)[row * 32 + c] = packed;
-        if ((c & 7) == 0) {
-            scales[row * 4 + (c >> 3)] = sc;
-            if (bsum) bsum[row * 4 + (c >> 3)] = ssum;
+    sacc[grp][c] = acc;
+    __syncthreads();
+    if (grp == 0) {
+#pragma unroll
+        for (int g = 1; g < 8; ++g) {
+            const float4 a = sacc[g][c];
+            acc.x += a.x; acc.y += a.y; acc.z += a.z; acc.w += a.w;
+        }
+        float inv = 1.0f / L;
+        float4 o = make_float4(acc.x * inv, acc.y * inv, acc.z * inv, acc.w * inv);
+        const uint64_t row = static_cast<uint64_t>(qi) * n_heads + head;  // outputs are [n_queries][n_heads][128]
+        reinterpret_cast<float4*>(out + row * ATTN_HD)[c] = o;
+        if (QUANT) {
+            float sc;
+            uint32_t packed = q8_quantize_quad(o, sc);
+            float ssum = bsum ? q8_block_scaled_sum(packed, sc) : 0.0f;
+            reinterpret_cast<uint32_t*>(quants)[row * 32 + c] = packed;
+            if ((c & 7) == 0) {
+                scales[row * 4 + (c >> 3)] = sc;
+                if (bsum) bsum[row * 4 + (c >> 3)] = ssum;
+            }
         }
     }
 }

@@ -136,6 +136,55 @@ static __global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __rest
     }
 }
 
+// Single-pass variant for the decode step (one row, n <= 16384): 1024 threads
+// keep the row in registers, so the row is read once and the whole kernel is
+// one memory round trip plus the reduction.  Same arithmetic as rmsnorm_kernel.
+template <bool QUANT>
+static __global__ __launch_bounds__(1024) void rmsnorm_row_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                                                                  uint32_t n, float eps, float* __restrict__ y,
+                                                                  float* __restrict__ scales, int8_t* __restrict__ quants) {
+    __shared__ double part[16];
+    float4 v[4], g[4];
+    double s = 0.0;
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+        uint32_t i = threadIdx.x * 4 + 4096 * it;
+        if (i < n) {
+            v[it] = *reinterpret_cast<const float4*>(x + i);
+            g[it] = *reinterpret_cast<const float4*>(w + i);
+            s += static_cast<double>(v[it].x) * v[it].x;
+            s += static_cast<double>(v[it].y) * v[it].y;
+            s += static_cast<double>(v[it].z) * v[it].z;
+            s += static_cast<double>(v[it].w) * v[it].w;
+        }
+    }
+    for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = s;
+    __syncthreads();
+    double tot = 0.0;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) tot += part[i];
+    float inv = static_cast<float>(1.0 / sqrt(tot / static_cast<double>(n) + static_cast<double>(eps)));
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+        uint32_t i = threadIdx.x * 4 + 4096 * it;
+        if (i < n) {
+            float4 o;
+            o.x = __fmul_rn(__fmul_rn(v[it].x, inv), g[it].x);
+            o.y = __fmul_rn(__fmul_rn(v[it].y, inv), g[it].y);
+            o.z = __fmul_rn(__fmul_rn(v[it].z, inv), g[it].z);
+            o.w = __fmul_rn(__fmul_rn(v[it].w, inv), g[it].w);
+            *reinterpret_cast<float4*>(y + i) = o;
+            if (QUANT) {
+                float sc;
+                uint32_t packed = q8_quantize_quad(o, sc);
+                reinterpret_cast<uint32_t*>(quants)[i >> 2] = packed;
+                if ((threadIdx.x & 7) == 0) scales[i >> 5] = sc;
+            }
+        }
+    }
+}
+
 // ---------------------------------------------------------------------------
 // RoPE on q and k in place + append k, v to the head-major KV cache.
 // cos/sin come from a host-built table [max_seq][head_dim/2] computed with the

@@ -17,6 +17,7 @@ struct cera_hip_dtensor {
     uint64_t m = 0, k = 0;
     uint64_t row_bytes = 0, nbytes = 0;
     uint8_t* dev = nullptr;
+    bool owns = true;  // false: a row-range view into another tensor's allocation
 };
 
 struct cera_hip_ctx {
@@ -74,3 +75,7 @@ cera_hip_status cera_launch_attn(cera_hip_ctx* ctx, const float* q, const float*
                                  uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, uint64_t seq_len,
                                  uint64_t max_seq, float scale, uint32_t n_splits, uint32_t n_queries, float* out,
                                  float* out_scales, int8_t* out_quants, float* out_bsum);
+// One allocation holding the rows of several same-type, same-k matrices back to back
+// (`fused`), plus a non-owning view per part.  Lets the decode step run Q|K(|V) as one GEMV.
+cera_hip_status cera_tensor_upload_concat(cera_hip_ctx* ctx, const cera_hip_tensor* const* parts, int n_parts,
+                                          cera_hip_dtensor** fused, cera_hip_dtensor** views);

@@ -8,6 +8,10 @@
 struct LayerDev {
     cera_hip_dtensor *q = nullptr, *k = nullptr, *v = nullptr, *o = nullptr, *gate = nullptr, *up = nullptr,
                      *down = nullptr;
+    // q|k (and |v when all three share a type) stored back to back so decode runs them as one
+    // GEMV; then q, k (, v) above are row-range views into it
+    cera_hip_dtensor* qkv = nullptr;
+    uint32_t qkv_rows = 0;  // rows covered by the fused launch (0: not fused)
     float *attn_norm = nullptr, *ffn_norm = nullptr;
     float *q_bias = nullptr, *k_bias = nullptr, *v_bias = nullptr, *q_norm = nullptr, *k_norm = nullptr;
     float *kc = nullptr, *vc = nullptr;  // [n_kv_heads][max_seq_len][head_dim] f32

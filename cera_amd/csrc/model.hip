@@ -54,7 +54,7 @@ static void free_model(cera_hip_model* m) {
     (void)hipStreamSynchronize(ctx->stream);
     auto ft = [&](cera_hip_dtensor* t) { if (t) cera_hip_tensor_free(ctx, t); };
     for (auto& L : m->layers) {
-        ft(L.q); ft(L.k); ft(L.v); ft(L.o); ft(L.gate); ft(L.up); ft(L.down);
+        ft(L.q); ft(L.k); ft(L.v); ft(L.o); ft(L.gate); ft(L.up); ft(L.down); ft(L.qkv);
         for (float* p : {L.attn_norm, L.ffn_norm, L.q_bias, L.k_bias, L.v_bias, L.q_norm, L.k_norm, L.kc, L.vc})
             if (p) (void)hipFree(p);
     }
@@ -136,7 +136,19 @@ extern "C" cera_hip_status cera_hip_model_create(cera_hip_ctx* ctx, const cera_h
             LayerDev& D = m->layers[i];
             const cera_hip_tensor* src[7] = {&L.attn_q, &L.attn_k, &L.attn_v, &L.attn_output, &L.ffn_gate, &L.ffn_up, &L.ffn_down};
             cera_hip_dtensor** dst[7] = {&D.q, &D.k, &D.v, &D.o, &D.gate, &D.up, &D.down};
-            for (int t = 0; t < 7; ++t) {
+            // Q and K (and V) of one type and width share an allocation: one decode GEMV
+            int fuse = 0;
+            if (L.attn_q.ggml_type == L.attn_k.ggml_type && L.attn_q.ggml_type != CERA_HIP_Q5_K)
+                fuse = (L.attn_v.ggml_type == L.attn_q.ggml_type) ? 3 : 2;
+            if (fuse) {
+                cera_hip_dtensor* views[3] = {nullptr, nullptr, nullptr};
+                CERA_TRY(cera_tensor_upload_concat(ctx, src, fuse, &D.qkv, views));
+                D.q = views[0]; D.k = views[1];
+                if (fuse == 3) D.v = views[2];
+                D.qkv_rows = static_cast<uint32_t>(D.qkv->m);
+                *tot += D.qkv->nbytes;
+            }
+            for (int t = fuse; t < 7; ++t) {
                 CERA_TRY(cera_hip_tensor_upload(ctx, src[t], dst[t]));
                 *tot += (*dst[t])->nbytes;
             }
@@ -167,9 +179,9 @@ extern "C" cera_hip_status cera_hip_model_create(cera_hip_ctx* ctx, const cera_h
         };
         CERA_TRY(af(c.hidden, &m->hidden));
         CERA_TRY(af(c.hidden, &m->normed));
-        CERA_TRY(af(q_dim, &m->q));
-        CERA_TRY(af(kv_dim, &m->k));
-        CERA_TRY(af(kv_dim, &m->v));
+        CERA_TRY(af(q_dim + 2 * kv_dim, &m->q));  // q | k | v contiguous: the fused GEMV writes them in one go
+        m->k = m->q + q_dim;
+        m->v = m->k + kv_dim;
         CERA_TRY(af(q_dim, &m->attn_out));
         CERA_TRY(af(c.hidden, &m->proj));
         CERA_TRY(af(c.ffn, &m->act));
@@ -231,8 +243,12 @@ static cera_hip_status project(cera_hip_model* m, const cera_hip_dtensor* w, con
 }
 
 static cera_hip_status norm_quant(cera_hip_model* m, const float* x, const float* w, uint32_t n, uint32_t rows, float* y) {
-    hipLaunchKernelGGL((rmsnorm_kernel<true>), dim3(rows), dim3(256), 0, m->ctx->stream, x, w, n, m->cfg.rms_eps, y,
-                       m->xs, m->xq, static_cast<float*>(nullptr));
+    if (rows == 1 && n <= 16384)
+        hipLaunchKernelGGL((rmsnorm_row_kernel<true>), dim3(1), dim3(1024), 0, m->ctx->stream, x, w, n, m->cfg.rms_eps, y,
+                           m->xs, m->xq);
+    else
+        hipLaunchKernelGGL((rmsnorm_kernel<true>), dim3(rows), dim3(256), 0, m->ctx->stream, x, w, n, m->cfg.rms_eps, y,
+                           m->xs, m->xq, static_cast<float*>(nullptr));
     HIP_TRY(m->ctx, hipGetLastError());
     return CERA_HIP_OK;
 }
@@ -253,9 +269,14 @@ static cera_hip_status decode_step(cera_hip_model* m, uint32_t pos, bool want_lo
     for (uint32_t i = 0; i < c.n_layers; ++i) {
         LayerDev& L = m->layers[i];
         CERA_TRY(norm_quant(m, m->hidden, L.attn_norm, c.hidden, 1, m->normed));
-        CERA_TRY(project(m, L.q, m->normed, m->q, nullptr));
-        CERA_TRY(project(m, L.k, m->normed, m->k, nullptr));
-        CERA_TRY(project(m, L.v, m->normed, m->v, nullptr));
+        if (L.qkv) {
+            CERA_TRY(project(m, L.qkv, m->normed, m->q, nullptr));
+            if (L.qkv_rows == q_dim + kv_dim) CERA_TRY(project(m, L.v, m->normed, m->v, nullptr));
+        } else {
+            CERA_TRY(project(m, L.q, m->normed, m->q, nullptr));
+            CERA_TRY(project(m, L.k, m->normed, m->k, nullptr));
+            CERA_TRY(project(m, L.v, m->normed, m->v, nullptr));
+        }
         if (L.q_bias) {
             hipLaunchKernelGGL(bias_kernel, dim3((q_dim + 255) / 256), dim3(256), 0, s, m->q, L.q_bias, q_dim);
             hipLaunchKernelGGL(bias_kernel, dim3((kv_dim + 255) / 256), dim3(256), 0, s, m->k, L.k_bias, kv_dim);
