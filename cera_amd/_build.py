@@ -1,7 +1,9 @@
 """Build the two native libraries of the package in-tree.
 
 * ``cera_amd/lib/libcera_hip.so``  -- HIP kernels + C-ABI (hipcc, gfx950)
-* ``cera_amd/lib/libcera_host.so`` -- CPU host layer (g++)
+* ``cera_amd/lib/libcera_host.so`` -- CPU host layer: quantizers, GGUF, synthetic models (g++)
+* ``cera_amd/lib/libcera_hip_llama.so`` + ``cera_amd/lib/cera-hip`` -- the Model-trait layer
+  above the C-ABI and its command-line driver (g++)
 """
 from __future__ import annotations
 
@@ -15,6 +17,8 @@ ROOT = PKG.parent
 LIB_DIR = PKG / "lib"
 HIP_LIB = LIB_DIR / "libcera_hip.so"
 HOST_LIB = LIB_DIR / "libcera_host.so"
+LLAMA_LIB = LIB_DIR / "libcera_hip_llama.so"
+CLI_BIN = LIB_DIR / "cera-hip"
 
 HIP_SRCS = sorted((PKG / "csrc").glob("*.hip"))
 HOST_SRCS = sorted((PKG / "host").glob("*.cpp"))
@@ -89,9 +93,35 @@ def build_host(verbose: bool = False) -> Path:
     return HOST_LIB
 
 
+def build_backend(verbose: bool = False) -> Path:
+    """HipLlamaModel + its C face (libcera_hip_llama.so) and the cera-hip driver binary.
+
+    Both link against the two libraries above, found at run time next to themselves.
+    """
+    common = ["g++", "-O2", "-std=c++17", "-fPIC", "-pthread", "-Wall", "-Wextra", "-fvisibility=hidden",
+              f"-I{ROOT / 'include'}", f"-I{PKG / 'host'}", f"-I{PKG / 'backend'}"]
+    link = [f"-L{LIB_DIR}", "-lcera_hip", "-lcera_host", "-Wl,-rpath,$ORIGIN"]
+    b = PKG / "backend"
+    gguf = str(PKG / "host" / "gguf.cpp")  # C++ classes are not exported by the host library: compile them in
+    cmds = [
+        [*common, "-shared", str(b / "hip_llama.cpp"), str(b / "hip_llama_capi.cpp"), gguf, "-o", str(LLAMA_LIB),
+         *link],
+        [*common, str(b / "cli.cpp"), str(b / "hip_llama.cpp"), gguf, "-o", str(CLI_BIN), *link],
+    ]
+    for cmd in cmds:
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if verbose or r.returncode:
+            print(" ".join(cmd))
+            print(r.stdout + r.stderr)
+        if r.returncode:
+            raise RuntimeError("g++ failed building the backend layer")
+    return LLAMA_LIB
+
+
 def build_all(verbose: bool = False) -> None:
     build_host(verbose)
     build_hip(verbose)
+    build_backend(verbose)
 
 
 if __name__ == "__main__":

@@ -1,0 +1,134 @@
+#include "hip_llama_capi.h"
+
+#include <chrono>
+#include <cmath>
+#include <cstring>
+
+#include "hip_llama.h"
+
+struct cera_llama {
+    std::unique_ptr<cera::GgufFile> gguf;
+    std::unique_ptr<cera::HipLlamaModel> model;
+    cera::InferenceState state;
+    std::atomic<bool> cancel{false};
+    std::string err;
+};
+
+namespace {
+void set_err(char* err, uint64_t n, const std::string& m) {
+    if (!err || !n) return;
+    std::strncpy(err, m.c_str(), n - 1);
+    err[n - 1] = 0;
+}
+template <class F>
+int guarded(cera_llama* h, F&& f) {
+    try {
+        f();
+        return 0;
+    } catch (const std::exception& e) {
+        h->err = e.what();
+    } catch (...) {
+        h->err = "unknown error";
+    }
+    return -1;
+}
+double now_s() {
+    return std::chrono::duration<double>(std::chrono::steady_clock::now().time_since_epoch()).count();
+}
+}  // namespace
+
+extern "C" {
+
+cera_llama* cera_llama_open(const char* path, uint64_t context_size, int device, char* err, uint64_t err_len) {
+    if (!path) {
+        set_err(err, err_len, "null path");
+        return nullptr;
+    }
+    std::unique_ptr<cera_llama> h(new cera_llama());
+    std::string e;
+    h->gguf = cera::GgufFile::open(path, &e);
+    if (!h->gguf) {
+        set_err(err, err_len, e);
+        return nullptr;
+    }
+    try {
+        h->model = cera::HipLlamaModel::from_gguf(*h->gguf, context_size, device);
+    } catch (const std::exception& ex) {
+        set_err(err, err_len, ex.what());
+        return nullptr;
+    }
+    // the weights are in HBM now; the mapping is only needed for metadata afterwards
+    return h.release();
+}
+void cera_llama_close(cera_llama* h) { delete h; }
+const char* cera_llama_last_error(const cera_llama* h) { return h ? h->err.c_str() : ""; }
+
+int cera_llama_get_config(const cera_llama* h, cera_llama_config* out) {
+    if (!h || !out) return -1;
+    const cera::ModelConfig& c = h->model->config();
+    out->n_layers = c.n_layers;
+    out->hidden_size = c.hidden_size;
+    out->intermediate_size = c.intermediate_size;
+    out->n_heads = c.n_heads;
+    out->n_kv_heads = c.n_kv_heads;
+    out->head_dim = c.head_dim;
+    out->vocab_size = c.vocab_size;
+    out->max_seq_len = c.max_seq_len;
+    out->rope_theta = c.rope_theta;
+    out->rms_norm_eps = c.rms_norm_eps;
+    out->rope_type = h->model->rope_type() == cera::RopeType::Norm ? 1u : 0u;
+    return 0;
+}
+uint64_t cera_llama_seq_len(const cera_llama* h) { return h->state.seq_len; }
+uint64_t cera_llama_gpu_memory_bytes(const cera_llama* h) { return h->model->gpu_memory_bytes(); }
+
+int cera_llama_forward(cera_llama* h, uint32_t token, uint64_t pos, float* logits) {
+    return guarded(h, [&] {
+        std::vector<float> l = h->model->forward(&token, 1, pos, h->state);
+        std::memcpy(logits, l.data(), l.size() * sizeof(float));
+    });
+}
+int cera_llama_forward_greedy(cera_llama* h, uint32_t token, uint64_t pos, uint32_t* next) {
+    return guarded(h, [&] { *next = h->model->forward_greedy(&token, 1, pos, h->state); });
+}
+int cera_llama_forward_prefill(cera_llama* h, const uint32_t* tokens, uint64_t n, uint64_t start_pos, float* logits) {
+    return guarded(h, [&] {
+        std::vector<float> l = h->model->forward_prefill(tokens, n, start_pos, h->state);
+        std::memcpy(logits, l.data(), l.size() * sizeof(float));
+    });
+}
+int cera_llama_forward_prefill_chunked(cera_llama* h, const uint32_t* tokens, uint64_t n, uint64_t start_pos,
+                                       uint64_t ubatch, uint64_t* consumed, float* logits) {
+    return guarded(h, [&] {
+        auto r = h->model->forward_prefill_chunked(tokens, n, start_pos, h->state, ubatch, h->cancel);
+        if (consumed) *consumed = r.first;
+        if (r.second && logits) std::memcpy(logits, r.second->data(), r.second->size() * sizeof(float));
+    });
+}
+void cera_llama_set_cancel(cera_llama* h, int c) { h->cancel.store(c != 0); }
+int cera_llama_truncate_kv(cera_llama* h, uint64_t len) {
+    return guarded(h, [&] { h->model->truncate_kv(h->state, len); });
+}
+
+int cera_llama_generate_greedy(cera_llama* h, const uint32_t* prompt, uint64_t n_prompt, uint64_t n_new,
+                               uint64_t ubatch, uint32_t* out, double* prefill_s, double* decode_s) {
+    return guarded(h, [&] {
+        if (!n_prompt || !n_new) throw cera::BackendError("generate_greedy needs a prompt and n_new > 0");
+        std::atomic<bool> never{false};
+        double t0 = now_s();
+        auto r = h->model->forward_prefill_chunked(prompt, n_prompt, h->state.seq_len, h->state, ubatch, never);
+        const std::vector<float>& l = *r.second;
+        size_t best = 0;
+        float bv = -INFINITY;
+        for (size_t i = 0; i < l.size(); ++i)
+            if (l[i] > bv) { bv = l[i]; best = i; }
+        out[0] = static_cast<uint32_t>(best);
+        double t1 = now_s();
+        for (uint64_t i = 1; i < n_new; ++i) out[i] = h->model->forward_greedy(&out[i - 1], 1, h->state.seq_len, h->state);
+        double t2 = now_s();
+        if (prefill_s) *prefill_s = t1 - t0;
+        if (decode_s) *decode_s = t2 - t1;
+    });
+}
+
+}  // extern "C"

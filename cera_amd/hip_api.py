@@ -315,6 +315,11 @@ class Model:
         c.rope_freqs = None
         self.cfg = dict(cfg)
         keep = []
+        rf = weights.get("rope_freqs.weight")
+        if rf is not None:
+            rf = np.ascontiguousarray(rf, np.float32)
+            keep.append(rf)
+            c.rope_freqs = rf.ctypes.data
         layers = (Layer * c.n_layers)()
         for i in range(c.n_layers):
             L = layers[i]
@@ -327,8 +332,13 @@ class Model:
                 t = make_tensor(dt, m, k, arr)
                 keep.append(t)
                 setattr(L, nm, t)
-            for nm in ("q_bias", "k_bias", "v_bias", "q_norm", "k_norm"):
-                setattr(L, nm, None)
+            for nm, key in (("q_bias", "attn_q.bias"), ("k_bias", "attn_k.bias"), ("v_bias", "attn_v.bias"),
+                            ("q_norm", "attn_q_norm.weight"), ("k_norm", "attn_k_norm.weight")):
+                a = weights.get(f"blk.{i}.{key}")
+                if a is not None:
+                    a = np.ascontiguousarray(a, np.float32)
+                    keep.append(a)
+                setattr(L, nm, a.ctypes.data if a is not None else None)
         dt, m, k, arr = weights["token_embd.weight"]
         embd = make_tensor(dt, m, k, arr)
         outp = None

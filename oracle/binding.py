@@ -311,6 +311,12 @@ class Llama:
         c.logit_scale = float(cfg.get("logit_scale", 1.0))
         c.rope_freqs = None
         self.cfg = cfg
+        self._opt = []
+        rf = weights.get("rope_freqs.weight")
+        if rf is not None:
+            rf = np.ascontiguousarray(rf, np.float32)
+            self._opt.append(rf)
+            c.rope_freqs = rf.ctypes.data
         layers = (OrcLlamaLayer * c.n_layers)()
         for i in range(c.n_layers):
             L = layers[i]
@@ -319,8 +325,13 @@ class Llama:
             for nm in ("attn_q", "attn_k", "attn_v", "attn_output", "ffn_gate", "ffn_up", "ffn_down"):
                 dt, m, k, arr = weights[f"blk.{i}.{nm}.weight"]
                 setattr(L, nm, _tensor(dt, m, k, arr))
-            for nm in ("q_bias", "k_bias", "v_bias", "q_norm", "k_norm"):
-                setattr(L, nm, None)
+            for nm, key in (("q_bias", "attn_q.bias"), ("k_bias", "attn_k.bias"), ("v_bias", "attn_v.bias"),
+                            ("q_norm", "attn_q_norm.weight"), ("k_norm", "attn_k_norm.weight")):
+                a = weights.get(f"blk.{i}.{key}")
+                if a is not None:
+                    a = np.ascontiguousarray(a, np.float32)
+                    self._opt.append(a)
+                setattr(L, nm, a.ctypes.data if a is not None else None)
         dt, m, k, arr = weights["token_embd.weight"]
         embd = _tensor(dt, m, k, arr)
         outp = None

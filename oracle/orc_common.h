@@ -91,6 +91,8 @@ ORC_API int orc_have_avx2(void);
 ORC_API void* orc_pool_create(int n_threads);
 ORC_API void  orc_pool_destroy(void* pool);
 ORC_API int   orc_pool_threads(void* pool);
+// fn(tid, n_threads, arg) on every worker of the pool (tid 0 = the caller); returns when all are done
+ORC_API void  orc_pool_run(void* pool, void (*fn)(int, int, void*), void* arg);
 // Row-parallel gemv on the pool (AVX2 variant when available): the timed
 // "restated cera AVX2 path" baseline.  Quantizes x on the calling thread first.
 ORC_API int orc_gemv_mt(void* pool, uint32_t dtype, const void* w, const float* x, float* y,

@@ -4,6 +4,8 @@
 // cera/src/model/transformer.rs:1313-1652 (attention / FFN blocks).
 #include "orc_llama.h"
 
+#include <atomic>
+
 #include <cmath>
 #include <cstring>
 #include <vector>
@@ -144,11 +146,31 @@ static void quantize_rows(const std::vector<float>& x, uint32_t n, uint32_t dim,
     for (uint32_t j = 0; j < n; ++j)
         orc_quantize_q8_0(x.data() + size_t(j) * dim, dim, bs.data() + size_t(j) * (dim / 32), bq.data() + size_t(j) * dim);
 }
-// out_rows[n][m] = (W . B)^T, B given as quantized rows
+// out_rows[n][m] = (W . B)^T, B given as quantized rows.  With a pool the weight rows are
+// split into contiguous ranges, one per worker; every output row is computed by the same
+// code either way (the strip kernels are row-independent), so the result does not change.
 static int gemm_rows(OrcLlama* m, const OrcTensor& t, const std::vector<float>& bs, const std::vector<int8_t>& bq,
                      uint32_t n, std::vector<float>& out_rows, std::vector<float>& tmp) {
     tmp.resize(size_t(t.m) * n);
-    int rc = orc_gemm_preq(t.dtype, t.data, bs.data(), bq.data(), tmp.data(), t.m, n, t.k, m->variant);
+    int rc = 0;
+    if (m->pool) {
+        struct Job { OrcLlama* m; const OrcTensor* t; const float* bs; const int8_t* bq; uint32_t n; float* tmp; uint64_t rb; std::atomic<int> rc; };
+        Job job{m, &t, bs.data(), bq.data(), n, tmp.data(), orc_row_bytes(t.dtype, t.k), {0}};
+        orc_pool_run(m->pool, [](int tid, int nt, void* a) {
+            Job& j = *static_cast<Job*>(a);
+            // ranges on multiples of 8 rows so a range never splits a row tile
+            uint64_t tiles = (j.t->m + 7) / 8;
+            uint64_t r0 = std::min<uint64_t>(j.t->m, tiles * uint64_t(tid) / uint64_t(nt) * 8);
+            uint64_t r1 = std::min<uint64_t>(j.t->m, tiles * uint64_t(tid + 1) / uint64_t(nt) * 8);
+            if (r1 <= r0) return;
+            int e = orc_gemm_preq(j.t->dtype, static_cast<const uint8_t*>(j.t->data) + r0 * j.rb, j.bs, j.bq,
+                                  j.tmp + r0 * j.n, r1 - r0, j.n, j.t->k, j.m->variant);
+            if (e) j.rc = e;
+        }, &job);
+        rc = job.rc;
+    } else {
+        rc = orc_gemm_preq(t.dtype, t.data, bs.data(), bq.data(), tmp.data(), t.m, n, t.k, m->variant);
+    }
     if (rc) return rc;
     out_rows.resize(size_t(n) * t.m);
     for (uint64_t i = 0; i < t.m; ++i)
@@ -173,7 +195,6 @@ int orc_llama_forward_prefill_batched(OrcLlama* m, const uint32_t* tokens, uint3
         if (c.embed_scale != 1.0f) for (uint32_t i = 0; i < hs; ++i) hidden[size_t(j) * hs + i] *= c.embed_scale;
     }
     const bool use_flash = n >= 256;  // FLASH_ATTN_THRESHOLD, llama.rs:845
-    std::vector<float> qh(size_t(n) * hd), oh(size_t(n) * hd), scores;
     for (uint32_t l = 0; l < c.n_layers; ++l) {
         const OrcLlamaLayer& L = m->layers[l];
         normed = hidden;
@@ -203,13 +224,22 @@ int orc_llama_forward_prefill_batched(OrcLlama* m, const uint32_t* tokens, uint3
         const float* kcache = m->kc[l].data();
         const float* vcache = m->vc[l].data();
         if (use_flash) {
-            for (uint32_t h = 0; h < c.n_heads; ++h) {
-                for (uint32_t j = 0; j < n; ++j)
-                    std::memcpy(qh.data() + size_t(j) * hd, qm.data() + size_t(j) * q_dim + h * hd, hd * sizeof(float));
-                orc_flash_attention_head(qh.data(), kcache, vcache, oh.data(), n, kv_dim, uint64_t(h / group) * hd, hd, scale, start_pos);
-                for (uint32_t j = 0; j < n; ++j)
-                    std::memcpy(attn.data() + size_t(j) * q_dim + h * hd, oh.data() + size_t(j) * hd, hd * sizeof(float));
-            }
+            struct Job { const OrcLlamaConfig* c; const float *qm, *kc, *vc; float* attn; uint32_t n, start_pos, q_dim, kv_dim, group; float scale; };
+            Job job{&c, qm.data(), kcache, vcache, attn.data(), n, start_pos, q_dim, kv_dim, group, scale};
+            auto heads = [](int tid, int nt, void* a) {   // heads are independent: one range per worker
+                Job& j = *static_cast<Job*>(a);
+                const uint32_t hd = j.c->head_dim;
+                std::vector<float> qh(size_t(j.n) * hd), oh(size_t(j.n) * hd);
+                for (uint32_t h = j.c->n_heads * uint32_t(tid) / uint32_t(nt); h < j.c->n_heads * uint32_t(tid + 1) / uint32_t(nt); ++h) {
+                    for (uint32_t t = 0; t < j.n; ++t)
+                        std::memcpy(qh.data() + size_t(t) * hd, j.qm + size_t(t) * j.q_dim + h * hd, hd * sizeof(float));
+                    orc_flash_attention_head(qh.data(), j.kc, j.vc, oh.data(), j.n, j.kv_dim, uint64_t(h / j.group) * hd, hd, j.scale, j.start_pos);
+                    for (uint32_t t = 0; t < j.n; ++t)
+                        std::memcpy(j.attn + size_t(t) * j.q_dim + h * hd, oh.data() + size_t(t) * hd, hd * sizeof(float));
+                }
+            };
+            if (m->pool) orc_pool_run(m->pool, heads, &job);
+            else heads(0, 1, &job);
         } else {
             for (uint32_t j = 0; j < n; ++j) {
                 uint64_t L_ctx = uint64_t(start_pos) + j + 1;

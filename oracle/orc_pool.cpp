@@ -72,6 +72,11 @@ struct Pool {
 void* orc_pool_create(int n_threads) { return new Pool(n_threads); }
 void orc_pool_destroy(void* p) { delete static_cast<Pool*>(p); }
 int orc_pool_threads(void* p) { return static_cast<Pool*>(p)->n; }
+void orc_pool_run(void* p, void (*fn)(int, int, void*), void* arg) {
+    Pool* pool = static_cast<Pool*>(p);
+    int n = pool->n;
+    pool->run([=](int tid) { fn(tid, n, arg); });
+}
 
 int orc_gemv_mt(void* pool, uint32_t dtype, const void* wv, const float* x, float* y, uint64_t m,
                 uint64_t k) {

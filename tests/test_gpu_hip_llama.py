@@ -1,0 +1,189 @@
+"""GPU parity of the Model-trait layer: a GGUF file on disk -> HipLlamaModel
+(C++ host layer over the C-ABI) against the oracle's LlamaModel twin built from
+the very same file.  Mirrors the harness shape of the reference's test for a
+new GPU backend (cera/tests/gpu_transformer_parity.rs:75-103: prefill, then
+greedy continuation, logits compared per step with near-tie tolerance)."""
+import json
+import subprocess
+
+import numpy as np
+import pytest
+
+import util
+from cera_amd import _build, host_api as H, llama_api, synth
+
+pytestmark = pytest.mark.gpu
+
+
+def _say(msg):
+    print(msg, flush=True)
+
+
+def _cos(a, b):
+    a = a.astype(np.float64); b = b.astype(np.float64)
+    return float(a @ b / np.sqrt((a @ a) * (b @ b)))
+
+
+def _close(lg, lo, what):
+    err = float(np.abs(lg - lo).max())
+    _say(f"  {what}: max|err|={err:.3e} rms={util.rms(lo):.3e} cos={_cos(lg, lo):.8f}")
+    assert _cos(lg, lo) > 0.999 and err <= 0.1 * util.rms(lo), what
+    return err
+
+
+def _teacher_forced(gm, om, orc, prompt, n_new, min_same):
+    lg = gm.forward_prefill(prompt, 0)
+    lo = om.forward_prefill_per_token(prompt, 0)
+    same = 0
+    for i in range(n_new):
+        err = _close(lg, lo, f"step {i}")
+        tg, to = int(orc.argmax(lg)), int(orc.argmax(lo))
+        if tg == to:
+            same += 1
+        else:
+            srt = np.sort(lo)
+            assert float(srt[-1] - srt[-2]) <= 2 * err, f"step {i}: {tg} vs {to} beyond a near-tie"
+        pos = len(prompt) + i
+        lg, lo = gm.forward(to, pos), om.forward(to, pos)
+    assert same >= min_same, same
+
+
+@pytest.fixture(scope="module")
+def tiny_llama(tmp_path_factory, orc, hip):
+    path = str(tmp_path_factory.mktemp("gguf") / "tiny.gguf")
+    H.synth_llama_gguf(path, dict(synth.TINY), seed=77, sigma=0.05, norm_jitter=0.1)
+    cfg, weights = H.Gguf(path).llama_weights()
+    gm = llama_api.HipLlama(path, context_size=64)
+    om = orc.Llama(cfg, weights)
+    yield path, cfg, gm, om
+    gm.close()
+    om.close()
+
+
+def test_config_comes_from_the_file(tiny_llama):
+    path, cfg, gm, om = tiny_llama
+    c = gm.config
+    assert (c["n_layers"], c["hidden_size"], c["intermediate_size"], c["n_heads"], c["n_kv_heads"], c["head_dim"],
+            c["vocab_size"]) == (cfg["n_layers"], cfg["hidden"], cfg["ffn"], cfg["n_heads"], cfg["n_kv_heads"],
+                                 cfg["head_dim"], cfg["vocab"])
+    assert c["max_seq_len"] == 64 and c["rope_type"] == 1
+    assert gm.gpu_memory_bytes > sum(w[3].size for w in H.Gguf(path).llama_weights()[1].values() if isinstance(w, tuple))
+
+
+def test_forward_and_prefill_match_the_oracle(tiny_llama, orc):
+    path, cfg, gm, om = tiny_llama
+    gm.truncate_kv(0); om.truncate(0)
+    _say("hip_llama: teacher-forced greedy from a GGUF")
+    _teacher_forced(gm, om, orc, [5, 400, 31, 2, 77, 123, 9], 20, 17)
+    assert gm.seq_len == om.seq_len == 27
+
+
+def test_generate_greedy_equals_stepwise_calls(tiny_llama):
+    path, cfg, gm, om = tiny_llama
+    prompt = [9, 8, 7, 300, 12]
+    gm.truncate_kv(0)
+    toks, tp, td = gm.generate_greedy(prompt, 12, ubatch=512)
+    assert gm.seq_len == len(prompt) + 11 and tp > 0 and td > 0
+    gm.truncate_kv(0)
+    logits = gm.forward_prefill(prompt, 0)
+    step = [int(np.argmax(logits))]
+    while len(step) < 12:
+        step.append(gm.forward_greedy(step[-1], gm.seq_len))
+    assert list(toks) == step
+
+
+def test_chunked_prefill_and_cancel(tiny_llama):
+    path, cfg, gm, om = tiny_llama
+    tokens = [3, 1, 4, 1, 5, 9, 2, 6, 5, 35]
+    gm.truncate_kv(0)
+    whole = gm.forward_prefill(tokens, 0)
+    gm.truncate_kv(0)
+    consumed, chunked = gm.forward_prefill_chunked(tokens, 0, ubatch=4)
+    assert consumed == 10 and gm.seq_len == 10
+    _close(chunked, whole, "chunked vs whole")
+    gm.truncate_kv(0)
+    consumed, same = gm.forward_prefill_chunked(tokens, 0, ubatch=0)       # 0 = one chunk
+    assert consumed == 10 and np.array_equal(same, whole)
+    # a cancel raised before the call still advances by exactly one chunk (mod.rs:323-329)
+    gm.truncate_kv(0)
+    gm.set_cancel(True)
+    consumed, part = gm.forward_prefill_chunked(tokens, 0, ubatch=4)
+    gm.set_cancel(False)
+    assert consumed == 4 and gm.seq_len == 4 and part is not None
+    consumed, none = gm.forward_prefill_chunked([], 4, ubatch=4)
+    assert consumed == 0 and none is None
+
+
+def test_truncate_then_replay_is_bit_identical(tiny_llama):
+    path, cfg, gm, om = tiny_llama
+    gm.truncate_kv(0)
+    gm.forward_prefill([1, 2, 3, 4, 5, 6], 0)
+    a = gm.forward(50, 6)
+    gm.truncate_kv(6)
+    assert gm.seq_len == 6
+    b = gm.forward(50, 6)
+    assert np.array_equal(a, b)
+    gm.truncate_kv(7)          # len == seq_len: the common, free case
+    assert gm.seq_len == 7
+
+
+def test_contract_violations_fail_loudly(tiny_llama):
+    path, cfg, gm, om = tiny_llama
+    gm.truncate_kv(0)
+    gm.forward(1, 0)
+    for call, needle in ((lambda: gm.forward(1, 5), "pos"), (lambda: gm.forward_prefill([1, 2], 0), "start_pos"),
+                         (lambda: gm.forward(cfg["vocab"], 1), "out of range"),
+                         (lambda: gm.truncate_kv(3), "exceeds"),
+                         (lambda: gm.forward_prefill(list(range(70)), 1), "")):
+        with pytest.raises(llama_api.BackendError) as e:
+            call()
+        assert needle in str(e.value), str(e.value)
+    assert gm.seq_len == 1
+    lg = gm.forward(2, 1)       # still usable after refused calls
+    assert np.isfinite(lg).all()
+
+
+def test_qwen3_style_file(tmp_path, orc, hip):
+    """NEOX RoPE, Q/K/V biases, per-head QK-norm, tied output head, other weight types."""
+    path = str(tmp_path / "q3.gguf")
+    H.synth_llama_gguf(path, dict(synth.TINY), seed=5, sigma=0.05, norm_jitter=0.1, arch="qwen3", tied_output=True,
+                       qkv_bias=True, qk_norm=True,
+                       types=dict(token_embd=H.Q8_0, attn_q=H.Q4_0, attn_k=H.Q4_0, attn_v=H.Q4_0, attn_output=H.Q8_0,
+                                  ffn_down=H.Q4_K))
+    cfg, weights = H.Gguf(path).llama_weights()
+    gm = llama_api.HipLlama(path, context_size=64)
+    om = orc.Llama(cfg, weights)
+    try:
+        assert gm.config["rope_type"] == 0
+        _say("hip_llama: qwen3-style file")
+        _teacher_forced(gm, om, orc, [11, 22, 33, 44, 55], 12, 10)
+    finally:
+        gm.close(); om.close()
+
+
+def test_context_size_caps_max_seq_len(tiny_llama):
+    path = tiny_llama[0]
+    gm = llama_api.HipLlama(path, context_size=8)
+    try:
+        assert gm.config["max_seq_len"] == 8
+        gm.forward_prefill(list(range(8)), 0)
+        with pytest.raises(llama_api.BackendError):
+            gm.forward(1, 8)
+    finally:
+        gm.close()
+
+
+def test_cli_run_agrees_with_the_library(tiny_llama):
+    path, cfg, gm, om = tiny_llama
+    _say("hip_llama: cera-hip run")
+    r = subprocess.run([str(_build.CLI_BIN), "run", "--model", path, "--prompt-len", "12", "--n-predict", "6",
+                        "--seed", "3", "--ctx", "64", "--tokens-out", path + ".tok"],
+                       capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stderr
+    rep = json.loads(r.stdout.strip().splitlines()[-1])
+    assert rep["prompt_len"] == 12 and rep["n_predict"] == 6 and rep["decode_tok_s"] > 0 and rep["prefill_tok_s"] > 0
+    prompt, out = (list(map(int, line.split())) for line in open(path + ".tok").read().strip().splitlines())
+    assert len(prompt) == 12 and len(out) == 6 and max(prompt) < cfg["vocab"]
+    gm.truncate_kv(0)
+    toks, _, _ = gm.generate_greedy(prompt, 6)
+    assert list(toks) == out
