@@ -27,6 +27,12 @@ ROOT = Path(__file__).resolve().parent
 sys.path.insert(0, str(ROOT))
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+# HBM bytes per launch of the fused Q4_K gate+up GEMV from hardware counters (FETCH_SIZE + WRITE_SIZE,
+# each scaled by what the same counter reads for this library's 1 GiB copy kernel; the two passes run
+# `bench.py --pmc-probe` under rocprofv3 --pmc, summary in profiles/gemv_q4k_gate_up_hbm_traffic_pmc.txt).
+# It is a recorded measurement of this kernel configuration, not taken live: counters need the profiler.
+GATE_UP_TRAFFIC_BYTES = 66_328_548
+GATE_UP_TRAFFIC_KERNEL = "gemv_kernel<Q4K,1,2,4,2,false>"
 
 # (name, ggml type name, m, k, copies per step)
 LAYER_SET = [
@@ -46,6 +52,111 @@ def algorithmic_bytes(H, tname, m, k):
     return m * H.row_bytes(H.TYPE_IDS[tname], k) + k + k // 32 * 4 + m * 4
 
 
+def measure_attention(ctx, hip_api, rng):
+    """BASELINE.json configs[3]: GQA flash-decode, 32 q heads / 8 kv heads / head_dim 128, f32 KV
+    resident in HBM in the kernel's head-major layout; bytes = K + V read once."""
+    n_heads, n_kv, hd = 32, 8, 128
+    out = []
+    max_l = 131072
+    chunk = rng.standard_normal(1 << 22, dtype=np.float32)            # 16 MiB of N(0,1), tiled over the cache
+    kv_bytes = n_kv * max_l * hd * 4
+    dk, dv = ctx.malloc(kv_bytes), ctx.malloc(kv_bytes)
+    dchunk = ctx.to_device(chunk)
+    for off in range(0, kv_bytes, chunk.nbytes):
+        ctx.check(ctx.lib.cera_hip_copy_dev(ctx.h, dk + off, dchunk, chunk.nbytes))
+        ctx.check(ctx.lib.cera_hip_copy_dev(ctx.h, dv + off, dchunk, chunk.nbytes))
+    dq = ctx.to_device(rng.standard_normal(n_heads * hd, dtype=np.float32))
+    dout = ctx.malloc(n_heads * hd * 4)
+    scale = 1.0 / np.sqrt(hd)
+    for L in (512, 4096, 32768, 131072):
+        # each context length gets its own cache stride = L, as a model with max_seq_len = L would
+        call = lambda: ctx.check(ctx.lib.cera_hip_attn_decode_dev(ctx.h, dq, dk, dv, n_heads, n_kv, hd, L, L,
+                                                                  C.c_float(scale), 0, dout))
+        iters = 200 if L <= 4096 else 50
+        for _ in range(5):
+            call()
+        e0, e1 = ctx.event(), ctx.event()
+        ctx.record(e0)
+        for _ in range(iters):
+            call()
+        ctx.record(e1)
+        ctx.sync()
+        us = ctx.elapsed_ms(e0, e1) * 1e3 / iters
+        nbytes = 2 * n_kv * L * hd * 4 + 2 * n_heads * hd * 4
+        # below ~32k the K/V working set fits the 256 MB last-level cache when launched back to back
+        out.append({"context": L, "us_per_call": round(us, 2), "GB/s": round(nbytes / us / 1e3, 1),
+                    "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
+                    "cache_resident": 2 * n_kv * L * hd * 4 <= 256 << 20})
+    for d in (dk, dv, dchunk, dq, dout):
+        ctx.free(d)
+    return out
+
+
+def measure_gemm(ctx, H, dts, shape, rng):
+    """BASELINE.json configs[2]: prefill GEMM out[N][M] = W_q . Q8_0(X[M][K]) on int8 MFMA, activation
+    quantization included in the timed call."""
+    INT8_PEAK_TOPS = 5000.0  # MI355X published dense int8 MFMA rate
+    res = []
+    for name in ("ffn_gate", "ffn_down"):
+        tname, n_out, k = shape[name]
+        for m_tok in (128, 512, 2048):
+            dx = ctx.to_device(rng.standard_normal((m_tok, k), dtype=np.float32))
+            dout = ctx.malloc(n_out * m_tok * 4)
+            call = lambda: ctx.check(ctx.lib.cera_hip_gemm_dev(ctx.h, dts[name][0], dx, m_tok, dout))
+            for _ in range(3):
+                call()
+            e0, e1 = ctx.event(), ctx.event()
+            iters = 20
+            ctx.record(e0)
+            for _ in range(iters):
+                call()
+            ctx.record(e1)
+            ctx.sync()
+            us = ctx.elapsed_ms(e0, e1) * 1e3 / iters
+            tops = 2.0 * m_tok * n_out * k / us / 1e6
+            res.append({"weight": f"{name} {tname} {n_out}x{k}", "tokens": m_tok, "us_per_call": round(us, 1),
+                        "TOP/s": round(tops, 1), "frac_of_int8_mfma_peak": round(tops / INT8_PEAK_TOPS, 4)})
+            ctx.free(dx)
+            ctx.free(dout)
+    return res
+
+
+def measure_e2e(seed: int, n_thr: int):
+    """BASELINE.json configs[4]: random-init Llama-3-8B-architecture GGUF written to a temp file, loaded
+    through the GGUF reader + HipLlamaModel, 512-token prefill + 256 greedy tokens."""
+    import tempfile
+    from cera_amd import host_api as H, llama_api, synth
+    cfg = dict(synth.LLAMA3_8B, max_seq_len=1024)
+    with tempfile.TemporaryDirectory() as td:
+        path = os.path.join(td, "llama3_8b_synth.gguf")
+        t0 = time.time()
+        H.synth_llama_gguf(path, cfg, seed=seed, n_threads=n_thr, explicit_head_dim=False)
+        gen_s = time.time() - t0
+        size = os.path.getsize(path)
+        t0 = time.time()
+        m = llama_api.HipLlama(path, context_size=1024)
+        load_s = time.time() - t0
+    prompt = np.random.default_rng(seed).integers(0, cfg["vocab"], 512).astype(np.uint32)
+    m.generate_greedy(prompt, 8)                      # warm-up (first-use allocations)
+    runs = []
+    for _ in range(3):
+        m.truncate_kv(0)
+        toks, tp, td_ = m.generate_greedy(prompt, 256, ubatch=512)
+        runs.append((512 / tp, 255 / td_))
+    mem = m.gpu_memory_bytes
+    m.close()
+    runs.sort(key=lambda r: r[1])
+    pf, dec = runs[len(runs) // 2]
+    weight_bytes_per_token = 4_875_853_824   # every projection + head read once per token
+    return {"workload": "random-init Llama-3-8B arch GGUF (Q4_K_M-style mix), prefill 512 + greedy 256, batch 1, "
+                        "host API calls included",
+            "decode_tok_s": round(dec, 1), "prefill_tok_s": round(pf, 1),
+            "decode_weight_GB/s": round(dec * weight_bytes_per_token / 1e9, 1),
+            "decode_frac_of_hbm_peak": round(dec * weight_bytes_per_token / 1e9 / HBM_PEAK_GBS, 4),
+            "gguf_bytes": size, "gpu_memory_bytes": mem, "gguf_write_s": round(gen_s, 1), "load_s": round(load_s, 1),
+            "runs": 3, "statistic": "median by decode rate"}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -54,6 +165,11 @@ def main() -> int:
     ap.add_argument("--seed", type=int, default=20250)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    ap.add_argument("--no-e2e", action="store_true", help="skip the end-to-end model run (prefill 512 + greedy 256)")
+    ap.add_argument("--no-extras", action="store_true", help="skip the flash-decode and prefill-GEMM side measurements")
+    ap.add_argument("--pmc-probe", action="store_true",
+                    help="run only a 1 GiB copy kernel and one step of the fused gate+up GEMVs, for a "
+                         "hardware-counter pass under rocprofv3 --pmc; prints no JSON")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the hot path has no multi-GPU part); "
@@ -119,6 +235,20 @@ def main() -> int:
     step_bytes = sum(grp_bytes.values())
     weight_bytes = sum(N_LAYERS * len(host[n]) for n, *_ in LAYER_SET) + len(host["output"])
 
+    if args.pmc_probe:
+        n = 1 << 30
+        src, dst = ctx.malloc(n), ctx.malloc(n)
+        ctx.check(ctx.lib.cera_hip_copy_kernel(ctx.h, dst, src, n))   # first touch
+        for _ in range(3):
+            ctx.check(ctx.lib.cera_hip_copy_kernel(ctx.h, dst, src, n))
+        for _ in range(2):
+            ctx.check(ctx.lib.cera_hip_gemv_seq_dev(ctx.h, grp_a, len(grp_a)))
+            ctx.check(ctx.lib.cera_hip_gemv_seq_dev(ctx.h, grp_c, len(grp_c)))
+        ctx.sync()
+        print(f"pmc probe done: copy kernel {n} B read + {n} B written per launch; fused gate+up "
+              f"{grp_bytes['q4k_gate_up'] // N_LAYERS} algorithmic B per launch", file=sys.stderr)
+        return 0
+
     def run_step(events=None):
         for gi, (_, ops) in enumerate(groups):
             ctx.check(ctx.lib.cera_hip_gemv_seq_dev(ctx.h, ops, len(ops)))
@@ -152,7 +282,9 @@ def main() -> int:
     ach = pair_bytes / (avg_launch_ms * 1e-3) / 1e9
     roofline = {"bound": "hbm", "kernel": "gemv_kernel<Q4K,1,2,4,2,false> (Q4_K gate+up, 2 x 14336x4096)",
                 "achieved": round(ach, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": None,
+                "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": GATE_UP_TRAFFIC_BYTES,
+                "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE passes over bench.py --pmc-probe, "
+                                  "calibrated on a 1 GiB copy kernel (recorded, see profiles/)",
                 "bytes_per_launch": pair_bytes, "avg_launch_us": round(avg_launch_ms * 1e3, 2)}
     per_group = {g: {"GB/s": round(grp_bytes[g] / (grp_ms[g] / args.steps * 1e-3) / 1e9, 1),
                      "ms_per_step": round(grp_ms[g] / args.steps, 4)} for g, _ in groups}
@@ -193,6 +325,12 @@ def main() -> int:
                                   f"incl. per-call Q8_0 quantize, {n_copies} rotating weight copies",
                         "avx2": bool(orc.lib().orc_have_avx2())}
 
+    extras = {}
+    if not args.no_extras:
+        extras["flash_decode"] = measure_attention(ctx, hip_api, rng)
+        extras["prefill_gemm"] = measure_gemm(ctx, H, dts, shape, rng)
+    e2e = None if args.no_e2e else measure_e2e(args.seed, n_thr)
+
     out = {
         "metric": "Q4_K GEMV HBM GB/s (% of peak); Llama-3-8B-arch Q4_K decode tok/s, 1 GPU",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -208,6 +346,8 @@ def main() -> int:
         "per_group": per_group,
         "roofline": roofline,
         "cpu_baseline": cpu_baseline,
+        "e2e": e2e,
+        **extras,
         "device": dev_name, "n_cu": n_cu, "setup_s": round(gen_s, 1),
     }
     print(json.dumps(out))

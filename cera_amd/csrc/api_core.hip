@@ -163,6 +163,23 @@ cera_hip_status cera_hip_copy_dev(cera_hip_ctx* ctx, void* dst, const void* src,
     HIP_TRY(ctx, hipMemcpyAsync(dst, src, n, hipMemcpyDeviceToDevice, ctx->stream));
     return CERA_HIP_OK;
 }
+// Plain streaming copy, 16 bytes per lane per step: a kernel of exactly known HBM traffic
+// (n read + n written) against which hardware byte counters can be calibrated.
+static __global__ void __launch_bounds__(256) copy_kernel(uint4* __restrict__ dst, const uint4* __restrict__ src, uint64_t n16) {
+    for (uint64_t i = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x; i < n16; i += uint64_t(gridDim.x) * blockDim.x)
+        dst[i] = src[i];
+}
+cera_hip_status cera_hip_copy_kernel(cera_hip_ctx* ctx, void* dst, const void* src, uint64_t n) {
+    if (!ctx || !dst || !src) return CERA_HIP_ERR_ARGUMENT;
+    if (n == 0 || n % 16 || (reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src)) % 16)
+        return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "copy_kernel: size and pointers must be multiples of 16 bytes");
+    uint64_t n16 = n / 16;
+    uint32_t blocks = static_cast<uint32_t>(std::min<uint64_t>((n16 + 255) / 256, uint64_t(ctx->n_cu) * 16));
+    hipLaunchKernelGGL(copy_kernel, dim3(blocks), dim3(256), 0, ctx->stream, static_cast<uint4*>(dst),
+                       static_cast<const uint4*>(src), n16);
+    HIP_TRY(ctx, hipGetLastError());
+    return CERA_HIP_OK;
+}
 cera_hip_status cera_hip_event_create(cera_hip_ctx* ctx, cera_hip_event** out) {
     if (!ctx || !out) return CERA_HIP_ERR_ARGUMENT;
     cera_hip_event* e = new (std::nothrow) cera_hip_event();

@@ -19,7 +19,7 @@ STATUS = {0: "OK", 1: "ERR_DEVICE", 2: "ERR_OOM", 3: "ERR_UNSUPPORTED_DTYPE", 4:
 # every symbol include/cera_hip.h declares
 SYMBOLS = [
     "cera_hip_ctx_create", "cera_hip_ctx_destroy", "cera_hip_last_error", "cera_hip_sync", "cera_hip_device_info",
-    "cera_hip_malloc", "cera_hip_free", "cera_hip_upload", "cera_hip_download", "cera_hip_copy_dev",
+    "cera_hip_malloc", "cera_hip_free", "cera_hip_upload", "cera_hip_download", "cera_hip_copy_dev", "cera_hip_copy_kernel",
     "cera_hip_event_create", "cera_hip_event_destroy", "cera_hip_event_record", "cera_hip_event_elapsed_ms",
     "cera_hip_tensor_upload", "cera_hip_tensor_clone", "cera_hip_tensor_free", "cera_hip_tensor_nbytes",
     "cera_hip_quantize_q8_0", "cera_hip_gemv", "cera_hip_gemm", "cera_hip_attn_decode", "cera_hip_rmsnorm",
@@ -85,6 +85,7 @@ def load_library() -> C.CDLL:
         "cera_hip_malloc": (i32, [vp, u64, pp]), "cera_hip_free": (i32, [vp, vp]),
         "cera_hip_upload": (i32, [vp, vp, vp, u64]), "cera_hip_download": (i32, [vp, vp, vp, u64]),
         "cera_hip_copy_dev": (i32, [vp, vp, vp, u64]),
+        "cera_hip_copy_kernel": (i32, [vp, vp, vp, u64]),
         "cera_hip_event_create": (i32, [vp, pp]), "cera_hip_event_destroy": (None, [vp]),
         "cera_hip_event_record": (i32, [vp, vp]),
         "cera_hip_event_elapsed_ms": (i32, [vp, vp, vp, C.POINTER(f32)]),

@@ -104,6 +104,11 @@ CERA_HIP_API cera_hip_status cera_hip_free(cera_hip_ctx*, void* dev);
 CERA_HIP_API cera_hip_status cera_hip_upload(cera_hip_ctx*, void* dev_dst, const void* host_src, uint64_t nbytes);
 CERA_HIP_API cera_hip_status cera_hip_download(cera_hip_ctx*, void* host_dst, const void* dev_src, uint64_t nbytes);
 CERA_HIP_API cera_hip_status cera_hip_copy_dev(cera_hip_ctx*, void* dev_dst, const void* dev_src, uint64_t nbytes);
+/* Device-to-device copy done by a plain streaming kernel of this library (not the runtime's
+ * copy engine): exactly nbytes read + nbytes written, the known-traffic kernel used to
+ * calibrate hardware byte counters.  nbytes and both pointers must be multiples of 16.
+ * Measurement aid; no counterpart in the reference. */
+CERA_HIP_API cera_hip_status cera_hip_copy_kernel(cera_hip_ctx*, void* dev_dst, const void* dev_src, uint64_t nbytes);
 CERA_HIP_API cera_hip_status cera_hip_event_create(cera_hip_ctx*, cera_hip_event** out);
 CERA_HIP_API void cera_hip_event_destroy(cera_hip_event*);
 CERA_HIP_API cera_hip_status cera_hip_event_record(cera_hip_ctx*, cera_hip_event*);
