@@ -380,6 +380,18 @@ cera_hip_status cera_launch_gemv(cera_hip_ctx* ctx, const cera_hip_dtensor* w, c
     return CERA_HIP_OK;
 }
 
+cera_hip_status cera_launch_argmax(cera_hip_ctx* ctx, const float* x, uint32_t n, uint32_t* out_dev) {
+    void* part;
+    CERA_TRY(cera_scratch(ctx, 8, ARGMAX_PARTS * 8, &part));
+    float* pv = static_cast<float*>(part);
+    uint32_t* pi = reinterpret_cast<uint32_t*>(pv + ARGMAX_PARTS);
+    const uint32_t np = std::max(1u, std::min<uint32_t>(ARGMAX_PARTS, (n + 1023) / 1024));
+    hipLaunchKernelGGL(argmax_partial_kernel, dim3(np), dim3(256), 0, ctx->stream, x, n, pv, pi);
+    hipLaunchKernelGGL(argmax_final_kernel, dim3(1), dim3(256), 0, ctx->stream, pv, pi, np, out_dev);
+    HIP_TRY(ctx, hipGetLastError());
+    return CERA_HIP_OK;
+}
+
 cera_hip_status cera_launch_gemv_q5k_f32(cera_hip_ctx* ctx, const cera_hip_dtensor* w, const float* x, float* y) {
     dim3 grid(static_cast<uint32_t>((w->m + 3) / 4));
     hipLaunchKernelGGL(gemv_q5k_f32_kernel, grid, dim3(256), 0, ctx->stream, w->dev, x, y,
@@ -626,9 +638,7 @@ cera_hip_status cera_hip_argmax(cera_hip_ctx* ctx, const float* logits, uint64_t
     CERA_TRY(cera_scratch(ctx, 0, n * 4, &dx));
     CERA_TRY(cera_scratch(ctx, 1, 4, &di));
     CERA_TRY(cera_hip_upload(ctx, dx, logits, n * 4));
-    hipLaunchKernelGGL(argmax_kernel, dim3(1), dim3(1024), 0, ctx->stream, static_cast<float*>(dx),
-                       static_cast<uint32_t>(n), static_cast<uint32_t*>(di));
-    HIP_TRY(ctx, hipGetLastError());
+    CERA_TRY(cera_launch_argmax(ctx, static_cast<float*>(dx), static_cast<uint32_t>(n), static_cast<uint32_t*>(di)));
     return cera_hip_download(ctx, index, di, 4);
 }
 

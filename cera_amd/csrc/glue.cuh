@@ -279,22 +279,15 @@ static __global__ __launch_bounds__(256) void silu_mul_kernel(const float* __res
 
 // ---------------------------------------------------------------------------
 // argmax (cera/src/sampler.rs:20-30): strict >, lowest index on ties, NaN never
-// wins, index 0 when nothing beats -inf.  Single block of 1024 threads: each
-// scans a strided slice keeping (best value, lowest index), then a tree merge
-// with the same tie rule.
+// wins, index 0 when nothing beats -inf.  Two stages: ARGMAX_PARTS workgroups each
+// scan a contiguous slice keeping (best value, lowest index) and leave one
+// candidate; a single workgroup merges the candidates with the same tie rule.
+#define ARGMAX_PARTS 256
 __device__ __forceinline__ void argmax_merge(float& bv, uint32_t& bi, float ov, uint32_t oi) {
     if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
 }
-static __global__ __launch_bounds__(1024) void argmax_kernel(const float* __restrict__ x, uint32_t n,
-                                                      uint32_t* __restrict__ out) {
-    __shared__ float sv[16];
-    __shared__ uint32_t si[16];
-    float bv = -__builtin_inff();
-    uint32_t bi = 0xFFFFFFFFu;  // "no candidate yet": loses every tie
-    for (uint32_t i = threadIdx.x; i < n; i += 1024) {
-        float v = x[i];
-        if (v > bv) { bv = v; bi = i; }
-    }
+// reduces the workgroup's (bv, bi) candidates into thread 0
+__device__ __forceinline__ void argmax_block_reduce(float& bv, uint32_t& bi, float* sv, uint32_t* si) {
     for (int off = 32; off > 0; off >>= 1) {
         float ov = __shfl_xor(bv, off, 64);
         uint32_t oi = __shfl_xor(bi, off, 64);
@@ -302,8 +295,31 @@ static __global__ __launch_bounds__(1024) void argmax_kernel(const float* __rest
     }
     if ((threadIdx.x & 63) == 0) { sv[threadIdx.x >> 6] = bv; si[threadIdx.x >> 6] = bi; }
     __syncthreads();
-    if (threadIdx.x == 0) {
-        for (int w = 1; w < 16; ++w) argmax_merge(bv, bi, sv[w], si[w]);
-        *out = bi == 0xFFFFFFFFu ? 0u : bi;
+    if (threadIdx.x == 0)
+        for (uint32_t w = 1; w < blockDim.x / 64; ++w) argmax_merge(bv, bi, sv[w], si[w]);
+}
+static __global__ __launch_bounds__(256) void argmax_partial_kernel(const float* __restrict__ x, uint32_t n,
+                                                             float* __restrict__ pv, uint32_t* __restrict__ pi) {
+    __shared__ float sv[4];
+    __shared__ uint32_t si[4];
+    const uint32_t chunk = (n + gridDim.x - 1) / gridDim.x;
+    const uint32_t lo = blockIdx.x * chunk, hi = min(n, lo + chunk);
+    float bv = -__builtin_inff();
+    uint32_t bi = 0xFFFFFFFFu;  // "no candidate yet": loses every tie
+    for (uint32_t i = lo + threadIdx.x; i < hi; i += 256) {
+        float v = x[i];
+        if (v > bv) { bv = v; bi = i; }
     }
+    argmax_block_reduce(bv, bi, sv, si);
+    if (threadIdx.x == 0) { pv[blockIdx.x] = bv; pi[blockIdx.x] = bi; }
+}
+static __global__ __launch_bounds__(256) void argmax_final_kernel(const float* __restrict__ pv, const uint32_t* __restrict__ pi,
+                                                           uint32_t np, uint32_t* __restrict__ out) {
+    __shared__ float sv[4];
+    __shared__ uint32_t si[4];
+    float bv = -__builtin_inff();
+    uint32_t bi = 0xFFFFFFFFu;
+    for (uint32_t i = threadIdx.x; i < np; i += 256) argmax_merge(bv, bi, pv[i], pi[i]);
+    argmax_block_reduce(bv, bi, sv, si);
+    if (threadIdx.x == 0) *out = bi == 0xFFFFFFFFu ? 0u : bi;
 }

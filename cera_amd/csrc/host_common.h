@@ -26,8 +26,8 @@ struct cera_hip_ctx {
     std::string err;
     uint32_t n_cu = 0;
     // grow-only device scratch for the host-pointer entry points
-    void* scratch[8] = {nullptr};
-    uint64_t scratch_bytes[8] = {0};
+    void* scratch[9] = {nullptr};
+    uint64_t scratch_bytes[9] = {0};
     // attention split-K workspace
     float* attn_acc = nullptr;
     float* attn_ml = nullptr;
@@ -64,6 +64,8 @@ cera_hip_status cera_launch_quantize(cera_hip_ctx* ctx, const float* x, uint64_t
 cera_hip_status cera_launch_gemv(cera_hip_ctx* ctx, const cera_hip_dtensor* w, const cera_hip_dtensor* w2,
                                  const float* xs, const int8_t* xq, float* y, const float* resid, int epi,
                                  int32_t* dbg_dots = nullptr, int32_t* dbg_asums = nullptr);
+// index of the maximum of x[0, n) into *out_dev (device); uses scratch slot 8 of the context
+cera_hip_status cera_launch_argmax(cera_hip_ctx* ctx, const float* x, uint32_t n, uint32_t* out_dev);
 cera_hip_status cera_launch_gemv_q5k_f32(cera_hip_ctx* ctx, const cera_hip_dtensor* w, const float* x, float* y);
 cera_hip_status cera_launch_attn_decode(cera_hip_ctx* ctx, const float* q, const float* kc, const float* vc,
                                         uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, uint64_t seq_len,

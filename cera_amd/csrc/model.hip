@@ -364,8 +364,7 @@ extern "C" cera_hip_status cera_hip_forward_greedy(cera_hip_model* m, uint32_t t
     CERA_TRY(check_step(m, token, pos));
     CERA_TRY(set_token_pos(m, token, pos));
     CERA_TRY(decode_step(m, pos, true));
-    hipLaunchKernelGGL(argmax_kernel, dim3(1), dim3(1024), 0, m->ctx->stream, m->logits, m->cfg.vocab, m->scalars + 2);
-    HIP_TRY(m->ctx, hipGetLastError());
+    CERA_TRY(cera_launch_argmax(m->ctx, m->logits, m->cfg.vocab, m->scalars + 2));
     CERA_TRY(cera_hip_download(m->ctx, next, m->scalars + 2, 4));
     m->seq_len = pos + 1;
     return CERA_HIP_OK;

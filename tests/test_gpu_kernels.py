@@ -285,3 +285,30 @@ def test_attn_decode_gqa_groupings(hip, orc):
         out = hip.attn_decode(q, k, v, nh, nkv, hd, L, 0.1)
         ref = orc.decode_attention(q, k, v, nh, nkv, hd, 0.1, L)
         assert np.abs(out - ref).max() <= ATTN_TOL * util.rms(ref)
+
+
+@pytest.mark.parametrize("L", [32768, 131072])
+def test_attn_decode_config4_long_contexts(hip, orc, L):
+    """The long contexts of the flash-decode configuration, against the oracle, plus two
+    properties that hold at any size: softmax weights sum to one (a V cache whose rows are all
+    the same vector must return that vector) and the result does not depend on how the context
+    is split over workgroups."""
+    nh, nkv, hd = 32, 8, 128
+    _say(f"attn_decode L={L}")
+    r = util.rng(1000 + L)
+    q = r.standard_normal(nh * hd, dtype=np.float32)
+    k = r.standard_normal(L * nkv * hd, dtype=np.float32)
+    v = r.standard_normal(L * nkv * hd, dtype=np.float32)
+    scale = 1.0 / math.sqrt(hd)
+    out = hip.attn_decode(q, k, v, nh, nkv, hd, L, scale)
+    ref = orc.decode_attention(q, k, v, nh, nkv, hd, scale, L)
+    err = np.abs(out.astype(np.float64) - ref).max()
+    _say(f"  max|err|={err:.3e} rms={util.rms(ref):.3e}")
+    assert err <= ATTN_TOL * util.rms(ref), (err, util.rms(ref))
+    other = hip.attn_decode(q, k, v, nh, nkv, hd, L, scale, n_splits=7)
+    assert np.abs(other - out).max() <= 1e-5 * max(1.0, float(np.abs(out).max()))
+    row = r.standard_normal(nkv * hd, dtype=np.float32)
+    vconst = np.tile(row, L)
+    same = hip.attn_decode(q, k, vconst, nh, nkv, hd, L, scale).reshape(nh, hd)
+    want = row.reshape(nkv, hd).repeat(nh // nkv, axis=0)
+    assert np.abs(same - want).max() <= 2e-6 * float(np.abs(want).max())
