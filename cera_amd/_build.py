@@ -30,6 +30,9 @@ HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
     "-ffp-contract=off", "-fno-fast-math",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # MFMA results straight into VGPRs: the GEMM epilogue consumes every accumulator element
+    # on the VALU, and the AGPR form would cost one v_accvgpr_read per element on top
+    "-mllvm", "-amdgpu-mfma-vgpr-form=1",
     "-Wall", "-Wno-unused-function",
 ]
 HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-shared", "-ffp-contract=off", "-fno-fast-math",

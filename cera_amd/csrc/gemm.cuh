@@ -9,31 +9,43 @@
 //
 // Mapping to gfx950: one v_mfma_i32_32x32x32_i8 computes the 32x32 int32 dots
 // of one 32-element block for 32 weight rows x 32 tokens (Q6_K uses the
-// 32x32x16 form, one per 16-element scale run).  Because every block carries
-// its own pair of f32 scales (weight side x activation side), the int32 tile
-// is converted and folded into f32 accumulators after each MFMA; that VALU
-// epilogue (cvt, mul, fma per output) is the throughput limit of this kernel,
-// not the matrix core.
+// 32x32x16 form, one per 16-element scale run).  Every block carries its own
+// pair of scales (weight side x activation side), so the int32 tile is folded
+// into f32 accumulators after each block; that VALU work (convert, scale,
+// accumulate: three to four instructions per output per block against 32 matrix-core
+// cycles per 1024 outputs) is the throughput limit of this kernel, not the matrix
+// core.  Two things keep it down:
+//   * the min terms  dmin*mn[row][b] * (xs*sum a)[tok][b]  (Q4_K, Q4_1) are a small
+//     f32 contraction over blocks of their own; they run on the matrix core too
+//     (v_mfma_f32_32x32x2_f32, two blocks per instruction) instead of one FMA per
+//     output per block;
+//   * Q6_K's int8 group scales are applied in integer (dot16_a*sc_a + dot16_b*sc_b,
+//     24-bit multiplies) so a 32-block costs one convert and one FMA with the
+//     activation scale; the f16 super-block scale d is applied once per 256.
 //
 // Workgroup: 256 threads = 4 wavefronts as 2 (M) x 2 (N); block tile 128 rows x
 // 64 tokens; each wavefront owns 64 x 32 (two MFMA row tiles).  K advances in
-// steps of 256 elements.  Per step the workgroup stages into LDS
-//   A: 128 rows x 256 weight codes unpacked to int8 (Q6_K/Q4_0 re-centred to
-//      signed so no activation-sum correction is needed), row stride 272 B so
-//      16-byte fragment reads do not collide on banks;
-//   rs/rm: per-row scale (d*sc) and min (dmin*mn) per sub-block, stored
-//      [sub][row] so a lane fetches its four consecutive rows with one b128;
-//   B: 64 tokens x 256 int8 activations, cs/cm: activation scale and
+// steps of 128 elements (half a K-quant super-block): the LDS footprint stays
+// near 32 KB, so several workgroups share a CU and one's global loads and
+// unpacking overlap another's MFMA/VALU phase.  Per step the workgroup stages
+//   A: 128 rows x 128 weight codes unpacked to int8 (Q6_K/Q4_0 re-centred to
+//      signed so no activation-sum correction is needed), row stride 144 B so
+//      16-byte fragment reads of 16 consecutive rows fall in distinct banks;
+//   rs/rm: per-row scale (d*sc, or the int8 scale for Q6_K) and min (dmin*mn) per
+//      sub-block, stored [sub][row] so a lane fetches four consecutive rows with one b128;
+//   B: 64 tokens x 128 int8 activations, cs/cm: activation scale and
 //      scale*sum(a) per 32-block.
 #pragma once
 #include "common.cuh"
 
 #define GEMM_BM 128
 #define GEMM_BN 64
-#define GEMM_KT 256
-#define GEMM_LDA 272  // bytes per staged row (256 + 16 pad)
+#define GEMM_KT 128      // K elements per staged tile
+#define GEMM_KSUPER 256  // K must be a whole number of these (the K-quant super-block)
+#define GEMM_LDA 144     // bytes per staged row (128 + 16 pad)
 
 typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v16f __attribute__((ext_vector_type(16)));
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v2i __attribute__((ext_vector_type(2)));
 
@@ -48,19 +60,27 @@ struct GemmArgs {
     uint64_t ld_m, ld_n;  // out[i*ld_m + j*ld_n]
     const float* resid;   // nullable: out = resid + W.B (same strides)
     float resid_scale;
+    // split-K: workgroup z covers k in [z*k_chunk, (z+1)*k_chunk) and writes its partial
+    // sums to out + z*part_stride (k_chunk == k, part_stride == 0 when not split)
+    uint32_t k_chunk;
+    uint64_t part_stride;
 };
 
-// ---- per-type staging of one 256-element K step of one row ------------------
-// Each type writes 256 int8 codes to `dst` (LDS row) and its per-sub-block row
-// scales.  NSUB = MFMA steps per K tile, KSTEP = elements per MFMA.
+// ---- per-type staging of one 128-element K tile of one row -------------------
+// `blk` points at the row's 256-element super-block (or run of eight 32-blocks)
+// containing the tile, `hs` says which half.  unpack() handles one 16-byte word
+// `w` of the tile's packed codes and writes int8 codes to `dst` (the LDS row);
+// scales() writes the row's per-sub-block scales.  NSUB = MFMA steps per tile,
+// KSTEP = elements per MFMA.
 struct GemmQ4K {
-    static constexpr int NSUB = 8, KSTEP = 32;
-    static constexpr bool HAS_MIN = true;
+    static constexpr int NSUB = 4, KSTEP = 32;
+    static constexpr bool HAS_MIN = true, INT_SCALE = false;
     static constexpr int BLOCK_BYTES = 144;
-    // thread handles one 16-byte packed word `wi` (0..7) of the row's block
-    __device__ static void unpack(const uint8_t* blk, uint32_t wi, int8_t* dst) {
+    static constexpr int WORDS = 4;
+    __device__ static void unpack(const uint8_t* blk, uint32_t hs, uint32_t w, int8_t* dst) {
+        const uint32_t wi = 4 * hs + w;
         uint4 q = ld_u128(blk + 16 + wi * 16);
-        uint32_t g = wi >> 1, h = wi & 1;
+        uint32_t g = w >> 1, h = w & 1;   // sub-block pair within the tile, half of it
         uint4 lo, hi;
         lo.x = q.x & 0x0F0F0F0Fu; lo.y = q.y & 0x0F0F0F0Fu; lo.z = q.z & 0x0F0F0F0Fu; lo.w = q.w & 0x0F0F0F0Fu;
         hi.x = (q.x >> 4) & 0x0F0F0F0Fu; hi.y = (q.y >> 4) & 0x0F0F0F0Fu;
@@ -68,35 +88,34 @@ struct GemmQ4K {
         *reinterpret_cast<uint4*>(dst + 64 * g + 16 * h) = lo;
         *reinterpret_cast<uint4*>(dst + 64 * g + 32 + 16 * h) = hi;
     }
-    static constexpr int WORDS = 8;
-    __device__ static void scales(const uint8_t* blk, float* rs, float* rm, uint32_t ld) {
+    __device__ static void scales(const uint8_t* blk, uint32_t hs, float* rs, float* rm, float* rd, uint32_t ld) {
         uint4 h = ld_u128(blk);
         float d = h2f(h.x & 0xFFFF), dmin = h2f(h.x >> 16);
         const uint32_t s[3] = {h.y, h.z, h.w};
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
+        for (int jj = 0; jj < 4; ++jj) {
             uint32_t sc, mn;
-            if (j < 4) {
-                sc = (s[0] >> (8 * j)) & 63;
-                mn = (s[1] >> (8 * j)) & 63;
+            if (hs == 0) {
+                sc = (s[0] >> (8 * jj)) & 63;
+                mn = (s[1] >> (8 * jj)) & 63;
             } else {
-                uint32_t b8 = (s[2] >> (8 * (j - 4))) & 0xFF;
-                sc = (b8 & 0xF) | ((((s[0] >> (8 * (j - 4))) & 0xFF) >> 6) << 4);
-                mn = (b8 >> 4) | ((((s[1] >> (8 * (j - 4))) & 0xFF) >> 6) << 4);
+                uint32_t b8 = (s[2] >> (8 * jj)) & 0xFF;
+                sc = (b8 & 0xF) | ((((s[0] >> (8 * jj)) & 0xFF) >> 6) << 4);
+                mn = (b8 >> 4) | ((((s[1] >> (8 * jj)) & 0xFF) >> 6) << 4);
             }
-            rs[j * ld] = d * static_cast<float>(sc);
-            rm[j * ld] = dmin * static_cast<float>(mn);
+            rs[jj * ld] = d * static_cast<float>(sc);
+            rm[jj * ld] = dmin * static_cast<float>(mn);
         }
+        (void)rd;
     }
 };
 
 struct GemmQ6K {
-    static constexpr int NSUB = 16, KSTEP = 16;
-    static constexpr bool HAS_MIN = false;
+    static constexpr int NSUB = 8, KSTEP = 16;
+    static constexpr bool HAS_MIN = false, INT_SCALE = true;
     static constexpr int BLOCK_BYTES = 210;
-    static constexpr int WORDS = 4;  // (nh, j): 16 positions l0..l0+15 -> 64 codes
-    __device__ static void unpack(const uint8_t* blk, uint32_t wi, int8_t* dst) {
-        uint32_t nh = wi >> 1, j = wi & 1;
+    static constexpr int WORDS = 2;  // j: 16 positions l0..l0+15 of the half -> 64 codes
+    __device__ static void unpack(const uint8_t* blk, uint32_t nh, uint32_t j, int8_t* dst) {
         uint4 qa = ld_u128_a2(blk + nh * 64 + j * 16);
         uint4 qb = ld_u128_a2(blk + nh * 64 + 32 + j * 16);
         uint4 qh = ld_u128_a2(blk + 128 + nh * 32 + j * 16);
@@ -118,27 +137,28 @@ struct GemmQ6K {
         }
 #pragma unroll
         for (int t = 0; t < 4; ++t)
-            *reinterpret_cast<uint4*>(dst + nh * 128 + 32 * t + 16 * j) = make_uint4(o[t][0], o[t][1], o[t][2], o[t][3]);
+            *reinterpret_cast<uint4*>(dst + 32 * t + 16 * j) = make_uint4(o[t][0], o[t][1], o[t][2], o[t][3]);
     }
-    __device__ static void scales(const uint8_t* blk, float* rs, float* rm, uint32_t ld) {
-        float d = h2f(ld_u16(blk + 208));
-        uint4 sc = ld_u128_a2(blk + 192);
-        const uint32_t s[4] = {sc.x, sc.y, sc.z, sc.w};
+    // rs holds the int8 group scales as int32 (bit pattern), rd the super-block scale
+    __device__ static void scales(const uint8_t* blk, uint32_t nh, float* rs, float* rm, float* rd, uint32_t ld) {
+        uint2 sc = ld_u64_a2(blk + 192 + nh * 8);
+        const uint32_t s[2] = {sc.x, sc.y};
 #pragma unroll
-        for (int h = 0; h < 16; ++h)
-            rs[h * ld] = d * static_cast<float>(static_cast<int8_t>((s[h >> 2] >> (8 * (h & 3))) & 0xFF));
+        for (int h = 0; h < 8; ++h)
+            rs[h * ld] = __builtin_bit_cast(float, static_cast<int>(static_cast<int8_t>((s[h >> 2] >> (8 * (h & 3))) & 0xFF)));
+        *rd = h2f(ld_u16(blk + 208));
         (void)rm;
     }
 };
 
-// 32-element block formats: a K tile is 8 blocks; word wi = block index.
+// 32-element block formats: a tile is 4 blocks; word w = block index within the tile.
 struct GemmQ4_0 {
-    static constexpr int NSUB = 8, KSTEP = 32;
-    static constexpr bool HAS_MIN = false;
+    static constexpr int NSUB = 4, KSTEP = 32;
+    static constexpr bool HAS_MIN = false, INT_SCALE = false;
     static constexpr int BLOCK_BYTES = 18 * 8;  // bytes per 256 elements
-    static constexpr int WORDS = 8;
-    __device__ static void unpack(const uint8_t* blk, uint32_t wi, int8_t* dst) {
-        uint4 q = ld_u128_a2(blk + wi * 18 + 2);
+    static constexpr int WORDS = 4;
+    __device__ static void unpack(const uint8_t* blk, uint32_t hs, uint32_t w, int8_t* dst) {
+        uint4 q = ld_u128_a2(blk + (4 * hs + w) * 18 + 2);
         uint4 lo, hi;  // code - 8, per byte: codes 0..15 -> flip bit 3, sign-extend the nibble
         const uint32_t v[4] = {q.x, q.y, q.z, q.w};
         uint32_t l[4], h[4];
@@ -150,64 +170,66 @@ struct GemmQ4_0 {
         }
         lo = make_uint4(l[0], l[1], l[2], l[3]);
         hi = make_uint4(h[0], h[1], h[2], h[3]);
-        *reinterpret_cast<uint4*>(dst + 32 * wi) = lo;
-        *reinterpret_cast<uint4*>(dst + 32 * wi + 16) = hi;
+        *reinterpret_cast<uint4*>(dst + 32 * w) = lo;
+        *reinterpret_cast<uint4*>(dst + 32 * w + 16) = hi;
     }
-    __device__ static void scales(const uint8_t* blk, float* rs, float* rm, uint32_t ld) {
+    __device__ static void scales(const uint8_t* blk, uint32_t hs, float* rs, float* rm, float* rd, uint32_t ld) {
 #pragma unroll
-        for (int b = 0; b < 8; ++b) rs[b * ld] = h2f(ld_u16(blk + 18 * b));
-        (void)rm;
+        for (int b = 0; b < 4; ++b) rs[b * ld] = h2f(ld_u16(blk + 18 * (4 * hs + b)));
+        (void)rm; (void)rd;
     }
 };
 struct GemmQ4_1 {
-    static constexpr int NSUB = 8, KSTEP = 32;
-    static constexpr bool HAS_MIN = true;   // rm holds -m so that out = rs*dot - rm*sum(a) covers q*d + m
+    static constexpr int NSUB = 4, KSTEP = 32;
+    static constexpr bool HAS_MIN = true, INT_SCALE = false;   // rm holds -m so that out = rs*dot - rm*sum(a) covers q*d + m
     static constexpr int BLOCK_BYTES = 20 * 8;
-    static constexpr int WORDS = 8;
-    __device__ static void unpack(const uint8_t* blk, uint32_t wi, int8_t* dst) {
-        uint4 q = ld_u128_a4(blk + wi * 20 + 4);
+    static constexpr int WORDS = 4;
+    __device__ static void unpack(const uint8_t* blk, uint32_t hs, uint32_t w, int8_t* dst) {
+        uint4 q = ld_u128_a4(blk + (4 * hs + w) * 20 + 4);
         uint4 lo, hi;
         lo.x = q.x & 0x0F0F0F0Fu; lo.y = q.y & 0x0F0F0F0Fu; lo.z = q.z & 0x0F0F0F0Fu; lo.w = q.w & 0x0F0F0F0Fu;
         hi.x = (q.x >> 4) & 0x0F0F0F0Fu; hi.y = (q.y >> 4) & 0x0F0F0F0Fu;
         hi.z = (q.z >> 4) & 0x0F0F0F0Fu; hi.w = (q.w >> 4) & 0x0F0F0F0Fu;
-        *reinterpret_cast<uint4*>(dst + 32 * wi) = lo;
-        *reinterpret_cast<uint4*>(dst + 32 * wi + 16) = hi;
+        *reinterpret_cast<uint4*>(dst + 32 * w) = lo;
+        *reinterpret_cast<uint4*>(dst + 32 * w + 16) = hi;
     }
-    __device__ static void scales(const uint8_t* blk, float* rs, float* rm, uint32_t ld) {
+    __device__ static void scales(const uint8_t* blk, uint32_t hs, float* rs, float* rm, float* rd, uint32_t ld) {
 #pragma unroll
-        for (int b = 0; b < 8; ++b) {
-            uint32_t dm = *reinterpret_cast<const uint32_t*>(blk + 20 * b);
+        for (int b = 0; b < 4; ++b) {
+            uint32_t dm = *reinterpret_cast<const uint32_t*>(blk + 20 * (4 * hs + b));
             rs[b * ld] = h2f(dm & 0xFFFF);
             rm[b * ld] = -h2f(dm >> 16);
         }
+        (void)rd;
     }
 };
 struct GemmQ8_0 {
-    static constexpr int NSUB = 8, KSTEP = 32;
-    static constexpr bool HAS_MIN = false;
+    static constexpr int NSUB = 4, KSTEP = 32;
+    static constexpr bool HAS_MIN = false, INT_SCALE = false;
     static constexpr int BLOCK_BYTES = 34 * 8;
-    static constexpr int WORDS = 8;
-    __device__ static void unpack(const uint8_t* blk, uint32_t wi, int8_t* dst) {
-        *reinterpret_cast<uint4*>(dst + 32 * wi) = ld_u128_a2(blk + wi * 34 + 2);
-        *reinterpret_cast<uint4*>(dst + 32 * wi + 16) = ld_u128_a2(blk + wi * 34 + 18);
+    static constexpr int WORDS = 4;
+    __device__ static void unpack(const uint8_t* blk, uint32_t hs, uint32_t w, int8_t* dst) {
+        const uint8_t* b = blk + (4 * hs + w) * 34;
+        *reinterpret_cast<uint4*>(dst + 32 * w) = ld_u128_a2(b + 2);
+        *reinterpret_cast<uint4*>(dst + 32 * w + 16) = ld_u128_a2(b + 18);
     }
-    __device__ static void scales(const uint8_t* blk, float* rs, float* rm, uint32_t ld) {
+    __device__ static void scales(const uint8_t* blk, uint32_t hs, float* rs, float* rm, float* rd, uint32_t ld) {
 #pragma unroll
-        for (int b = 0; b < 8; ++b) rs[b * ld] = h2f(ld_u16(blk + 34 * b));
-        (void)rm;
+        for (int b = 0; b < 4; ++b) rs[b * ld] = h2f(ld_u16(blk + 34 * (4 * hs + b)));
+        (void)rm; (void)rd;
     }
 };
 
 template <class T>
 static __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
+    constexpr int NB = GEMM_KT / 32;  // 32-blocks per tile
     __shared__ __attribute__((aligned(16))) int8_t sA[GEMM_BM * GEMM_LDA];
     __shared__ __attribute__((aligned(16))) int8_t sB[GEMM_BN * GEMM_LDA];
     __shared__ __attribute__((aligned(16))) float sRS[T::NSUB * GEMM_BM];
-    // the min arrays exist only for formats with a per-block minimum (keeps the
-    // workgroup under 64 KB of LDS)
-    __shared__ __attribute__((aligned(16))) float sRM[T::HAS_MIN ? 8 * GEMM_BM : 4];
-    __shared__ __attribute__((aligned(16))) float sCS[8 * GEMM_BN];
-    __shared__ __attribute__((aligned(16))) float sCM[T::HAS_MIN ? 8 * GEMM_BN : 4];
+    __shared__ __attribute__((aligned(16))) float sRD[T::INT_SCALE ? GEMM_BM : 4];
+    __shared__ __attribute__((aligned(16))) float sRM[T::HAS_MIN ? NB * GEMM_BM : 4];
+    __shared__ __attribute__((aligned(16))) float sCS[NB * GEMM_BN];
+    __shared__ __attribute__((aligned(16))) float sCM[T::HAS_MIN ? NB * GEMM_BN : 4];
 
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const uint32_t wm = wave >> 1, wn = wave & 1;           // wavefront position in the 2 x 2 grid
@@ -215,86 +237,141 @@ static __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
     const uint32_t col = lane & 31, half = lane >> 5;
     const uint32_t nb32 = p.k / 32;
 
-    float acc[2][16], macc[2][16];
+    float acc[2][16], accsb[2][16];
+    v16f macc[2];
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) { acc[t][r] = 0.0f; macc[t][r] = 0.0f; }
+        for (int r = 0; r < 16; ++r) { acc[t][r] = 0.0f; accsb[t][r] = 0.0f; macc[t][r] = 0.0f; }
 
-    for (uint32_t k0 = 0; k0 < p.k; k0 += GEMM_KT) {
-        // ---- stage A: 128 rows x WORDS words; B: 64 tokens x 16 words of 16 B
-        for (uint32_t it = tid; it < GEMM_BM * T::WORDS; it += 256) {
-            uint32_t r = it / T::WORDS, wi = it % T::WORDS;
-            uint32_t row = min(m0 + r, p.m - 1);
-            const uint8_t* blk = p.w + static_cast<uint64_t>(row) * p.row_bytes + static_cast<uint64_t>(k0 / 256) * T::BLOCK_BYTES;
-            T::unpack(blk, wi, sA + r * GEMM_LDA);
+    // per-thread staging assignments, fixed for the whole K loop: AI weight words, one row's
+    // scales (threads 0..127), two activation words, one activation scale
+    constexpr int AI = GEMM_BM * T::WORDS / 256;
+    const uint8_t* a_src[AI];
+    int8_t* a_dst[AI];
+    uint32_t a_w[AI];
+#pragma unroll
+    for (int i = 0; i < AI; ++i) {
+        const uint32_t it = tid + 256 * i, r = it / T::WORDS;
+        a_w[i] = it % T::WORDS;
+        a_src[i] = p.w + static_cast<uint64_t>(min(m0 + r, p.m - 1)) * p.row_bytes;
+        a_dst[i] = sA + r * GEMM_LDA;
+    }
+    const uint8_t* s_src = p.w + static_cast<uint64_t>(min(m0 + (tid & (GEMM_BM - 1)), p.m - 1)) * p.row_bytes;
+    const int8_t* b_src[2];
+    int8_t* b_dst[2];
+    bool b_live[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const uint32_t it = tid + 256 * i, c = it >> 3, wi = it & 7;
+        b_live[i] = n0 + c < p.n;
+        b_src[i] = p.bq + static_cast<uint64_t>(min(n0 + c, p.n - 1)) * p.k + wi * 16;
+        b_dst[i] = sB + c * GEMM_LDA + wi * 16;
+    }
+    const uint32_t c_tok = tid >> 2, c_b = tid & 3;   // 64 tokens x 4 blocks = 256 threads
+    const bool c_live = n0 + c_tok < p.n;
+    const uint64_t c_off = static_cast<uint64_t>(min(n0 + c_tok, p.n - 1)) * nb32 + c_b;
+
+    const uint32_t k_begin = blockIdx.z * p.k_chunk, k_end = k_begin + p.k_chunk;
+    for (uint32_t k0 = k_begin; k0 < k_end; k0 += GEMM_KT) {
+        const uint32_t hs = (k0 / GEMM_KT) & 1;
+        const uint32_t sb_off = (k0 / 256) * T::BLOCK_BYTES;
+        // ---- stage A: 128 rows x WORDS words; B: 64 tokens x 8 words of 16 B
+#pragma unroll
+        for (int i = 0; i < AI; ++i) T::unpack(a_src[i] + sb_off, hs, a_w[i], a_dst[i]);
+        if (tid < GEMM_BM) T::scales(s_src + sb_off, hs, sRS + tid, sRM + tid, sRD + tid, GEMM_BM);
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            uint4 v = *reinterpret_cast<const uint4*>(b_src[i] + k0);
+            if (!b_live[i]) v = make_uint4(0, 0, 0, 0);
+            *reinterpret_cast<uint4*>(b_dst[i]) = v;
         }
-        if (tid < GEMM_BM) {
-            uint32_t row = min(m0 + tid, p.m - 1);
-            const uint8_t* blk = p.w + static_cast<uint64_t>(row) * p.row_bytes + static_cast<uint64_t>(k0 / 256) * T::BLOCK_BYTES;
-            T::scales(blk, sRS + tid, sRM + tid, GEMM_BM);
-        }
-        for (uint32_t it = tid; it < GEMM_BN * 16; it += 256) {
-            uint32_t c = it >> 4, wi = it & 15;
-            uint32_t tok = n0 + c;
-            uint4 v = make_uint4(0, 0, 0, 0);
-            if (tok < p.n) v = *reinterpret_cast<const uint4*>(p.bq + static_cast<uint64_t>(tok) * p.k + k0 + wi * 16);
-            *reinterpret_cast<uint4*>(sB + c * GEMM_LDA + wi * 16) = v;
-        }
-        for (uint32_t it = tid; it < GEMM_BN * 8; it += 256) {
-            uint32_t c = it >> 3, b = it & 7;
-            uint32_t tok = n0 + c;
-            float s = 0.0f, sm = 0.0f;
-            if (tok < p.n) {
-                s = p.bs[static_cast<uint64_t>(tok) * nb32 + k0 / 32 + b];
-                if (T::HAS_MIN) sm = p.bsum[static_cast<uint64_t>(tok) * nb32 + k0 / 32 + b];
-            }
-            sCS[b * GEMM_BN + c] = s;
-            if (T::HAS_MIN) sCM[b * GEMM_BN + c] = sm;
+        {
+            float s = p.bs[c_off + k0 / 32], sm = 0.0f;
+            if (T::HAS_MIN) sm = p.bsum[c_off + k0 / 32];
+            if (!c_live) { s = 0.0f; sm = 0.0f; }
+            sCS[c_b * GEMM_BN + c_tok] = s;
+            if (T::HAS_MIN) sCM[c_b * GEMM_BN + c_tok] = sm;
         }
         __syncthreads();
 
         // ---- MFMA over the K tile
         const int8_t* bRow = sB + (wn * 32 + col) * GEMM_LDA;
 #pragma unroll
-        for (int sub = 0; sub < T::NSUB; ++sub) {
-            const int b32 = sub * T::KSTEP / 32;  // 32-block index of this step
-            const float xs = sCS[b32 * GEMM_BN + wn * 32 + col];
-            const float xm = T::HAS_MIN ? sCM[b32 * GEMM_BN + wn * 32 + col] : 0.0f;
+        for (int b = 0; b < NB; ++b) {
+            const float xs = sCS[b * GEMM_BN + wn * 32 + col];
+            if (!T::INT_SCALE) {
+                const v4i bf = *reinterpret_cast<const v4i*>(bRow + b * 32 + half * 16);
 #pragma unroll
-            for (int t = 0; t < 2; ++t) {
-                const int8_t* aRow = sA + (wm * 64 + t * 32 + col) * GEMM_LDA;
-                v16i c = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-                if (T::KSTEP == 32) {
-                    v4i a = *reinterpret_cast<const v4i*>(aRow + sub * 32 + half * 16);
-                    v4i b = *reinterpret_cast<const v4i*>(bRow + sub * 32 + half * 16);
-                    c = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c, 0, 0, 0);
-                } else {
-                    long a = *reinterpret_cast<const long*>(aRow + sub * 16 + half * 8);
-                    long b = *reinterpret_cast<const long*>(bRow + sub * 16 + half * 8);
-                    c = __builtin_amdgcn_mfma_i32_32x32x16_i8(a, b, c, 0, 0, 0);
+                for (int t = 0; t < 2; ++t) {
+                    const int8_t* aRow = sA + (wm * 64 + t * 32 + col) * GEMM_LDA;
+                    const v4i af = *reinterpret_cast<const v4i*>(aRow + b * 32 + half * 16);
+                    v16i c = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+                    c = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, bf, c, 0, 0, 0);
+                    // rows held by this lane: 8*blk + 4*half + r, blk = 0..3, r = 0..3
+#pragma unroll
+                    for (int blk = 0; blk < 4; ++blk) {
+                        const uint32_t rbase = wm * 64 + t * 32 + blk * 8 + half * 4;
+                        const float4 rs = *reinterpret_cast<const float4*>(sRS + b * GEMM_BM + rbase);
+                        const float rsv[4] = {rs.x, rs.y, rs.z, rs.w};
+#pragma unroll
+                        for (int r = 0; r < 4; ++r)
+                            acc[t][blk * 4 + r] = fmaf(static_cast<float>(c[blk * 4 + r]), rsv[r] * xs, acc[t][blk * 4 + r]);
+                    }
                 }
-                // rows held by this lane: 8*blk + 4*half + r, blk = 0..3, r = 0..3
+            } else {
+                // two 16-element scale groups share this block's activation scale
+                const long bf0 = *reinterpret_cast<const long*>(bRow + b * 32 + half * 8);
+                const long bf1 = *reinterpret_cast<const long*>(bRow + b * 32 + 16 + half * 8);
 #pragma unroll
-                for (int blk = 0; blk < 4; ++blk) {
-                    const uint32_t rbase = wm * 64 + t * 32 + blk * 8 + half * 4;
-                    const float4 rs = *reinterpret_cast<const float4*>(sRS + sub * GEMM_BM + rbase);
-                    const float rsv[4] = {rs.x, rs.y, rs.z, rs.w};
+                for (int t = 0; t < 2; ++t) {
+                    const int8_t* aRow = sA + (wm * 64 + t * 32 + col) * GEMM_LDA;
+                    const long af0 = *reinterpret_cast<const long*>(aRow + b * 32 + half * 8);
+                    const long af1 = *reinterpret_cast<const long*>(aRow + b * 32 + 16 + half * 8);
+                    v16i z = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+                    v16i c0 = __builtin_amdgcn_mfma_i32_32x32x16_i8(af0, bf0, z, 0, 0, 0);
+                    v16i c1 = __builtin_amdgcn_mfma_i32_32x32x16_i8(af1, bf1, z, 0, 0, 0);
 #pragma unroll
-                    for (int r = 0; r < 4; ++r)
-                        acc[t][blk * 4 + r] = fmaf(static_cast<float>(c[blk * 4 + r]), rsv[r] * xs, acc[t][blk * 4 + r]);
-                    if (T::HAS_MIN) {
-                        const float4 rm = *reinterpret_cast<const float4*>(sRM + b32 * GEMM_BM + rbase);
-                        const float rmv[4] = {rm.x, rm.y, rm.z, rm.w};
+                    for (int blk = 0; blk < 4; ++blk) {
+                        const uint32_t rbase = wm * 64 + t * 32 + blk * 8 + half * 4;
+                        const v4i s0 = *reinterpret_cast<const v4i*>(sRS + (2 * b) * GEMM_BM + rbase);
+                        const v4i s1 = *reinterpret_cast<const v4i*>(sRS + (2 * b + 1) * GEMM_BM + rbase);
 #pragma unroll
-                        for (int r = 0; r < 4; ++r) macc[t][blk * 4 + r] = fmaf(rmv[r], xm, macc[t][blk * 4 + r]);
+                        for (int r = 0; r < 4; ++r) {
+                            // |dot16| <= 16*32*127 and |scale| <= 128: 24-bit operands, 32-bit result
+                            const int iv = __mul24(c0[blk * 4 + r], s0[r]) + __mul24(c1[blk * 4 + r], s1[r]);
+                            accsb[t][blk * 4 + r] = fmaf(static_cast<float>(iv), xs, accsb[t][blk * 4 + r]);
+                        }
                     }
                 }
             }
+            if (T::HAS_MIN && (b & 1)) {
+                // min terms of blocks b-1, b: a rank-2 f32 update on the matrix core
+                const float xm = sCM[(b - 1 + half) * GEMM_BN + wn * 32 + col];
+#pragma unroll
+                for (int t = 0; t < 2; ++t) {
+                    const float rm = sRM[(b - 1 + half) * GEMM_BM + wm * 64 + t * 32 + col];
+                    macc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(rm, xm, macc[t], 0, 0, 0);
+                }
+            }
+        }
+        if (T::INT_SCALE && hs == 1) {
+            // the super-block's f16 scale, once per 256 elements
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int blk = 0; blk < 4; ++blk) {
+                    const float4 d = *reinterpret_cast<const float4*>(sRD + wm * 64 + t * 32 + blk * 8 + half * 4);
+                    const float dv[4] = {d.x, d.y, d.z, d.w};
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        acc[t][blk * 4 + r] = fmaf(dv[r], accsb[t][blk * 4 + r], acc[t][blk * 4 + r]);
+                        accsb[t][blk * 4 + r] = 0.0f;
+                    }
+                }
         }
         __syncthreads();
     }
-
     // ---- store: lane holds token n0 + wn*32 + col, 32 rows
     const uint32_t tok = n0 + wn * 32 + col;
     if (tok < p.n) {
@@ -306,12 +383,31 @@ static __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
                 for (int r = 0; r < 4; ++r) {
                     uint32_t row = m0 + wm * 64 + t * 32 + blk * 8 + half * 4 + r;
                     if (row < p.m) {
-                        float v = acc[t][blk * 4 + r] - macc[t][blk * 4 + r];
+                        float v = acc[t][blk * 4 + r] - (T::HAS_MIN ? macc[t][blk * 4 + r] : 0.0f);
                         uint64_t idx = row * p.ld_m + tok * p.ld_n;
                         if (p.resid) v = p.resid[idx] + (p.resid_scale != 1.0f ? v * p.resid_scale : v);
-                        p.out[idx] = v;
+                        p.out[idx + blockIdx.z * p.part_stride] = v;
                     }
                 }
     }
 }
 
+
+// Sums the split-K partials in a fixed order: out[e] = (resid[e] +) sum_z part[z][e].
+static __global__ __launch_bounds__(256) void gemm_reduce_kernel(const float* __restrict__ part, uint32_t n_split,
+                                                          uint64_t stride, uint64_t n4, float* __restrict__ out,
+                                                          const float* resid, float resid_scale) {
+    const uint64_t e = static_cast<uint64_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (e >= n4) return;
+    float4 s = reinterpret_cast<const float4*>(part)[e];
+    for (uint32_t z = 1; z < n_split; ++z) {
+        const float4 v = reinterpret_cast<const float4*>(part + z * stride)[e];
+        s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+    }
+    if (resid) {
+        const float4 r = reinterpret_cast<const float4*>(resid)[e];
+        if (resid_scale != 1.0f) { s.x *= resid_scale; s.y *= resid_scale; s.z *= resid_scale; s.w *= resid_scale; }
+        s.x = r.x + s.x; s.y = r.y + s.y; s.z = r.z + s.z; s.w = r.w + s.w;
+    }
+    reinterpret_cast<float4*>(out)[e] = s;
+}

@@ -15,7 +15,7 @@ static bool gemm_type_ok(uint32_t t) {
 
 // batched_gemm_supports (cera/src/model/transformer.rs:536-565): the int8 GEMM
 // takes K in whole 256-element steps.
-bool cera_gemm_supports(uint32_t dtype, uint64_t k) { return gemm_type_ok(dtype) && k % GEMM_KT == 0 && k > 0; }
+bool cera_gemm_supports(uint32_t dtype, uint64_t k) { return gemm_type_ok(dtype) && k % GEMM_KSUPER == 0 && k > 0; }
 
 // out[i*ld_m + j*ld_n] = (W . B)[i][j] (+ resid)
 cera_hip_status cera_launch_gemm(cera_hip_ctx* ctx, const cera_hip_dtensor* w, const float* bs, const int8_t* bq,
@@ -31,6 +31,29 @@ cera_hip_status cera_launch_gemm(cera_hip_ctx* ctx, const cera_hip_dtensor* w, c
     a.row_bytes = static_cast<uint32_t>(w->row_bytes);
     a.ld_m = ld_m; a.ld_n = ld_n; a.resid = resid; a.resid_scale = resid_scale;
     dim3 grid((n + GEMM_BN - 1) / GEMM_BN, (a.m + GEMM_BM - 1) / GEMM_BM);
+    // Few output tiles and a long K (the down projection at a few hundred tokens): split K over
+    // grid.z so the chip is filled, partial sums to scratch, then one fixed-order reduction.
+    // The outputs must be dense in m*n floats for the elementwise reduction.
+    uint32_t split = 1;
+    const uint32_t wgs = grid.x * grid.y, nsb = a.k / GEMM_KSUPER;
+    const bool dense = (ld_m == 1 && ld_n == a.m) || (ld_n == 1 && ld_m == n);
+    if (wgs < 2 * ctx->n_cu && nsb >= 8 && dense && (static_cast<uint64_t>(a.m) * n) % 4 == 0) {
+        // smallest divisor of the super-block count that gives at least two workgroups per CU
+        const uint32_t want = std::min<uint32_t>(8, (2 * ctx->n_cu + wgs - 1) / wgs);
+        for (uint32_t d = 2; d <= 8 && split < want; ++d)
+            if (nsb % d == 0 && nsb / d >= 4) split = d;
+    }
+    a.k_chunk = a.k / split;
+    a.part_stride = 0;
+    const uint64_t mn = static_cast<uint64_t>(a.m) * n;
+    if (split > 1) {
+        void* part;
+        CERA_TRY(cera_scratch(ctx, 9, split * mn * sizeof(float), &part));
+        a.out = static_cast<float*>(part);
+        a.part_stride = mn;
+        a.resid = nullptr;
+        grid.z = split;
+    }
     switch (w->dtype) {
         case CERA_HIP_Q4_K: hipLaunchKernelGGL((gemm_kernel<GemmQ4K>), grid, dim3(256), 0, ctx->stream, a); break;
         case CERA_HIP_Q6_K: hipLaunchKernelGGL((gemm_kernel<GemmQ6K>), grid, dim3(256), 0, ctx->stream, a); break;
@@ -38,6 +61,9 @@ cera_hip_status cera_launch_gemm(cera_hip_ctx* ctx, const cera_hip_dtensor* w, c
         case CERA_HIP_Q4_1: hipLaunchKernelGGL((gemm_kernel<GemmQ4_1>), grid, dim3(256), 0, ctx->stream, a); break;
         default: hipLaunchKernelGGL((gemm_kernel<GemmQ8_0>), grid, dim3(256), 0, ctx->stream, a); break;
     }
+    if (split > 1)
+        hipLaunchKernelGGL(gemm_reduce_kernel, dim3(static_cast<uint32_t>((mn / 4 + 255) / 256)), dim3(256), 0, ctx->stream,
+                           a.out, split, mn, mn / 4, out, resid, resid_scale);
     HIP_TRY(ctx, hipGetLastError());
     return CERA_HIP_OK;
 }
