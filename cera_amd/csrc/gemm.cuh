@@ -77,9 +77,12 @@ struct GemmQ4K {
     static constexpr bool HAS_MIN = true, INT_SCALE = false;
     static constexpr int BLOCK_BYTES = 144;
     static constexpr int WORDS = 4;
-    __device__ static void unpack(const uint8_t* blk, uint32_t hs, uint32_t w, int8_t* dst) {
-        const uint32_t wi = 4 * hs + w;
-        uint4 q = ld_u128(blk + 16 + wi * 16);
+    struct Raw { uint4 q; };
+    struct RawS { uint4 h; };
+    __device__ static void load(Raw& r, const uint8_t* blk, uint32_t hs, uint32_t w) { r.q = ld_u128(blk + 16 + (4 * hs + w) * 16); }
+    __device__ static void load_scales(RawS& r, const uint8_t* blk, uint32_t) { r.h = ld_u128(blk); }
+    __device__ static void unpack(const Raw& raw, uint32_t w, int8_t* dst) {
+        const uint4 q = raw.q;
         uint32_t g = w >> 1, h = w & 1;   // sub-block pair within the tile, half of it
         uint4 lo, hi;
         lo.x = q.x & 0x0F0F0F0Fu; lo.y = q.y & 0x0F0F0F0Fu; lo.z = q.z & 0x0F0F0F0Fu; lo.w = q.w & 0x0F0F0F0Fu;
@@ -88,8 +91,8 @@ struct GemmQ4K {
         *reinterpret_cast<uint4*>(dst + 64 * g + 16 * h) = lo;
         *reinterpret_cast<uint4*>(dst + 64 * g + 32 + 16 * h) = hi;
     }
-    __device__ static void scales(const uint8_t* blk, uint32_t hs, float* rs, float* rm, float* rd, uint32_t ld) {
-        uint4 h = ld_u128(blk);
+    __device__ static void scales(const RawS& raw, uint32_t hs, float* rs, float* rm, float* rd, uint32_t ld) {
+        const uint4 h = raw.h;
         float d = h2f(h.x & 0xFFFF), dmin = h2f(h.x >> 16);
         const uint32_t s[3] = {h.y, h.z, h.w};
 #pragma unroll
@@ -115,10 +118,19 @@ struct GemmQ6K {
     static constexpr bool HAS_MIN = false, INT_SCALE = true;
     static constexpr int BLOCK_BYTES = 210;
     static constexpr int WORDS = 2;  // j: 16 positions l0..l0+15 of the half -> 64 codes
-    __device__ static void unpack(const uint8_t* blk, uint32_t nh, uint32_t j, int8_t* dst) {
-        uint4 qa = ld_u128_a2(blk + nh * 64 + j * 16);
-        uint4 qb = ld_u128_a2(blk + nh * 64 + 32 + j * 16);
-        uint4 qh = ld_u128_a2(blk + 128 + nh * 32 + j * 16);
+    struct Raw { uint4 qa, qb, qh; };
+    struct RawS { uint2 sc; uint32_t d; };
+    __device__ static void load(Raw& r, const uint8_t* blk, uint32_t nh, uint32_t j) {
+        r.qa = ld_u128_a2(blk + nh * 64 + j * 16);
+        r.qb = ld_u128_a2(blk + nh * 64 + 32 + j * 16);
+        r.qh = ld_u128_a2(blk + 128 + nh * 32 + j * 16);
+    }
+    __device__ static void load_scales(RawS& r, const uint8_t* blk, uint32_t nh) {
+        r.sc = ld_u64_a2(blk + 192 + nh * 8);
+        r.d = ld_u16(blk + 208);
+    }
+    __device__ static void unpack(const Raw& raw, uint32_t j, int8_t* dst) {
+        const uint4 qa = raw.qa, qb = raw.qb, qh = raw.qh;
         const uint32_t a[4] = {qa.x, qa.y, qa.z, qa.w}, b[4] = {qb.x, qb.y, qb.z, qb.w}, h[4] = {qh.x, qh.y, qh.z, qh.w};
         uint32_t o[4][4];
 #pragma unroll
@@ -140,13 +152,12 @@ struct GemmQ6K {
             *reinterpret_cast<uint4*>(dst + 32 * t + 16 * j) = make_uint4(o[t][0], o[t][1], o[t][2], o[t][3]);
     }
     // rs holds the int8 group scales as int32 (bit pattern), rd the super-block scale
-    __device__ static void scales(const uint8_t* blk, uint32_t nh, float* rs, float* rm, float* rd, uint32_t ld) {
-        uint2 sc = ld_u64_a2(blk + 192 + nh * 8);
-        const uint32_t s[2] = {sc.x, sc.y};
+    __device__ static void scales(const RawS& raw, uint32_t, float* rs, float* rm, float* rd, uint32_t ld) {
+        const uint32_t s[2] = {raw.sc.x, raw.sc.y};
 #pragma unroll
         for (int h = 0; h < 8; ++h)
             rs[h * ld] = __builtin_bit_cast(float, static_cast<int>(static_cast<int8_t>((s[h >> 2] >> (8 * (h & 3))) & 0xFF)));
-        *rd = h2f(ld_u16(blk + 208));
+        *rd = h2f(raw.d);
         (void)rm;
     }
 };
@@ -157,8 +168,15 @@ struct GemmQ4_0 {
     static constexpr bool HAS_MIN = false, INT_SCALE = false;
     static constexpr int BLOCK_BYTES = 18 * 8;  // bytes per 256 elements
     static constexpr int WORDS = 4;
-    __device__ static void unpack(const uint8_t* blk, uint32_t hs, uint32_t w, int8_t* dst) {
-        uint4 q = ld_u128_a2(blk + (4 * hs + w) * 18 + 2);
+    struct Raw { uint4 q; };
+    struct RawS { uint32_t d[4]; };
+    __device__ static void load(Raw& r, const uint8_t* blk, uint32_t hs, uint32_t w) { r.q = ld_u128_a2(blk + (4 * hs + w) * 18 + 2); }
+    __device__ static void load_scales(RawS& r, const uint8_t* blk, uint32_t hs) {
+#pragma unroll
+        for (int b = 0; b < 4; ++b) r.d[b] = ld_u16(blk + 18 * (4 * hs + b));
+    }
+    __device__ static void unpack(const Raw& raw, uint32_t w, int8_t* dst) {
+        const uint4 q = raw.q;
         uint4 lo, hi;  // code - 8, per byte: codes 0..15 -> flip bit 3, sign-extend the nibble
         const uint32_t v[4] = {q.x, q.y, q.z, q.w};
         uint32_t l[4], h[4];
@@ -173,9 +191,9 @@ struct GemmQ4_0 {
         *reinterpret_cast<uint4*>(dst + 32 * w) = lo;
         *reinterpret_cast<uint4*>(dst + 32 * w + 16) = hi;
     }
-    __device__ static void scales(const uint8_t* blk, uint32_t hs, float* rs, float* rm, float* rd, uint32_t ld) {
+    __device__ static void scales(const RawS& raw, uint32_t, float* rs, float* rm, float* rd, uint32_t ld) {
 #pragma unroll
-        for (int b = 0; b < 4; ++b) rs[b * ld] = h2f(ld_u16(blk + 18 * (4 * hs + b)));
+        for (int b = 0; b < 4; ++b) rs[b * ld] = h2f(raw.d[b]);
         (void)rm; (void)rd;
     }
 };
@@ -184,8 +202,15 @@ struct GemmQ4_1 {
     static constexpr bool HAS_MIN = true, INT_SCALE = false;   // rm holds -m so that out = rs*dot - rm*sum(a) covers q*d + m
     static constexpr int BLOCK_BYTES = 20 * 8;
     static constexpr int WORDS = 4;
-    __device__ static void unpack(const uint8_t* blk, uint32_t hs, uint32_t w, int8_t* dst) {
-        uint4 q = ld_u128_a4(blk + (4 * hs + w) * 20 + 4);
+    struct Raw { uint4 q; };
+    struct RawS { uint32_t dm[4]; };
+    __device__ static void load(Raw& r, const uint8_t* blk, uint32_t hs, uint32_t w) { r.q = ld_u128_a4(blk + (4 * hs + w) * 20 + 4); }
+    __device__ static void load_scales(RawS& r, const uint8_t* blk, uint32_t hs) {
+#pragma unroll
+        for (int b = 0; b < 4; ++b) r.dm[b] = *reinterpret_cast<const uint32_t*>(blk + 20 * (4 * hs + b));
+    }
+    __device__ static void unpack(const Raw& raw, uint32_t w, int8_t* dst) {
+        const uint4 q = raw.q;
         uint4 lo, hi;
         lo.x = q.x & 0x0F0F0F0Fu; lo.y = q.y & 0x0F0F0F0Fu; lo.z = q.z & 0x0F0F0F0Fu; lo.w = q.w & 0x0F0F0F0Fu;
         hi.x = (q.x >> 4) & 0x0F0F0F0Fu; hi.y = (q.y >> 4) & 0x0F0F0F0Fu;
@@ -193,10 +218,10 @@ struct GemmQ4_1 {
         *reinterpret_cast<uint4*>(dst + 32 * w) = lo;
         *reinterpret_cast<uint4*>(dst + 32 * w + 16) = hi;
     }
-    __device__ static void scales(const uint8_t* blk, uint32_t hs, float* rs, float* rm, float* rd, uint32_t ld) {
+    __device__ static void scales(const RawS& raw, uint32_t, float* rs, float* rm, float* rd, uint32_t ld) {
 #pragma unroll
         for (int b = 0; b < 4; ++b) {
-            uint32_t dm = *reinterpret_cast<const uint32_t*>(blk + 20 * (4 * hs + b));
+            uint32_t dm = raw.dm[b];
             rs[b * ld] = h2f(dm & 0xFFFF);
             rm[b * ld] = -h2f(dm >> 16);
         }
@@ -208,14 +233,24 @@ struct GemmQ8_0 {
     static constexpr bool HAS_MIN = false, INT_SCALE = false;
     static constexpr int BLOCK_BYTES = 34 * 8;
     static constexpr int WORDS = 4;
-    __device__ static void unpack(const uint8_t* blk, uint32_t hs, uint32_t w, int8_t* dst) {
+    struct Raw { uint4 q0, q1; };
+    struct RawS { uint32_t d[4]; };
+    __device__ static void load(Raw& r, const uint8_t* blk, uint32_t hs, uint32_t w) {
         const uint8_t* b = blk + (4 * hs + w) * 34;
-        *reinterpret_cast<uint4*>(dst + 32 * w) = ld_u128_a2(b + 2);
-        *reinterpret_cast<uint4*>(dst + 32 * w + 16) = ld_u128_a2(b + 18);
+        r.q0 = ld_u128_a2(b + 2);
+        r.q1 = ld_u128_a2(b + 18);
     }
-    __device__ static void scales(const uint8_t* blk, uint32_t hs, float* rs, float* rm, float* rd, uint32_t ld) {
+    __device__ static void load_scales(RawS& r, const uint8_t* blk, uint32_t hs) {
 #pragma unroll
-        for (int b = 0; b < 4; ++b) rs[b * ld] = h2f(ld_u16(blk + 34 * (4 * hs + b)));
+        for (int b = 0; b < 4; ++b) r.d[b] = ld_u16(blk + 34 * (4 * hs + b));
+    }
+    __device__ static void unpack(const Raw& raw, uint32_t w, int8_t* dst) {
+        *reinterpret_cast<uint4*>(dst + 32 * w) = raw.q0;
+        *reinterpret_cast<uint4*>(dst + 32 * w + 16) = raw.q1;
+    }
+    __device__ static void scales(const RawS& raw, uint32_t, float* rs, float* rm, float* rd, uint32_t ld) {
+#pragma unroll
+        for (int b = 0; b < 4; ++b) rs[b * ld] = h2f(raw.d[b]);
         (void)rm; (void)rd;
     }
 };
@@ -272,28 +307,37 @@ static __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
     const bool c_live = n0 + c_tok < p.n;
     const uint64_t c_off = static_cast<uint64_t>(min(n0 + c_tok, p.n - 1)) * nb32 + c_b;
 
-    const uint32_t k_begin = blockIdx.z * p.k_chunk, k_end = k_begin + p.k_chunk;
-    for (uint32_t k0 = k_begin; k0 < k_end; k0 += GEMM_KT) {
+    // Register prefetch: the global loads of tile k+1 are issued right after tile k has been
+    // written to LDS and stay in flight while tile k is multiplied.
+    typename T::Raw ra[AI];
+    typename T::RawS rsc;
+    uint4 rb[2];
+    float rcs, rcm;
+    auto fetch = [&](uint32_t k0) {
         const uint32_t hs = (k0 / GEMM_KT) & 1;
         const uint32_t sb_off = (k0 / 256) * T::BLOCK_BYTES;
-        // ---- stage A: 128 rows x WORDS words; B: 64 tokens x 8 words of 16 B
 #pragma unroll
-        for (int i = 0; i < AI; ++i) T::unpack(a_src[i] + sb_off, hs, a_w[i], a_dst[i]);
-        if (tid < GEMM_BM) T::scales(s_src + sb_off, hs, sRS + tid, sRM + tid, sRD + tid, GEMM_BM);
+        for (int i = 0; i < AI; ++i) T::load(ra[i], a_src[i] + sb_off, hs, a_w[i]);
+        if (tid < GEMM_BM) T::load_scales(rsc, s_src + sb_off, hs);
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            uint4 v = *reinterpret_cast<const uint4*>(b_src[i] + k0);
-            if (!b_live[i]) v = make_uint4(0, 0, 0, 0);
-            *reinterpret_cast<uint4*>(b_dst[i]) = v;
-        }
-        {
-            float s = p.bs[c_off + k0 / 32], sm = 0.0f;
-            if (T::HAS_MIN) sm = p.bsum[c_off + k0 / 32];
-            if (!c_live) { s = 0.0f; sm = 0.0f; }
-            sCS[c_b * GEMM_BN + c_tok] = s;
-            if (T::HAS_MIN) sCM[c_b * GEMM_BN + c_tok] = sm;
-        }
+        for (int i = 0; i < 2; ++i) rb[i] = *reinterpret_cast<const uint4*>(b_src[i] + k0);
+        rcs = p.bs[c_off + k0 / 32];
+        rcm = T::HAS_MIN ? p.bsum[c_off + k0 / 32] : 0.0f;
+    };
+    const uint32_t k_begin = blockIdx.z * p.k_chunk, k_end = k_begin + p.k_chunk;
+    fetch(k_begin);
+    for (uint32_t k0 = k_begin; k0 < k_end; k0 += GEMM_KT) {
+        const uint32_t hs = (k0 / GEMM_KT) & 1;
+        // ---- registers -> LDS: A 128 rows x WORDS words (unpacked), B 64 tokens x 8 words
+#pragma unroll
+        for (int i = 0; i < AI; ++i) T::unpack(ra[i], a_w[i], a_dst[i]);
+        if (tid < GEMM_BM) T::scales(rsc, hs, sRS + tid, sRM + tid, sRD + tid, GEMM_BM);
+#pragma unroll
+        for (int i = 0; i < 2; ++i) *reinterpret_cast<uint4*>(b_dst[i]) = b_live[i] ? rb[i] : make_uint4(0, 0, 0, 0);
+        sCS[c_b * GEMM_BN + c_tok] = c_live ? rcs : 0.0f;
+        if (T::HAS_MIN) sCM[c_b * GEMM_BN + c_tok] = c_live ? rcm : 0.0f;
         __syncthreads();
+        if (k0 + GEMM_KT < k_end) fetch(k0 + GEMM_KT);
 
         // ---- MFMA over the K tile
         const int8_t* bRow = sB + (wn * 32 + col) * GEMM_LDA;
