@@ -165,6 +165,9 @@ def main() -> int:
     ap.add_argument("--seed", type=int, default=20250)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    ap.add_argument("--weight-copies", type=int, default=N_LAYERS,
+                    help="distinct HBM copies of the layer weights the step rotates over (default: one per layer; "
+                         "fewer lets the last-level cache hold them, which is NOT the reported configuration)")
     ap.add_argument("--no-e2e", action="store_true", help="skip the end-to-end model run (prefill 512 + greedy 256)")
     ap.add_argument("--no-extras", action="store_true", help="skip the flash-decode and prefill-GEMM side measurements")
     ap.add_argument("--pmc-probe", action="store_true",
@@ -194,7 +197,8 @@ def main() -> int:
     dts = {}   # name -> list of device tensor handles (one per layer)
     for name, tname, m, k in LAYER_SET:
         first = ctx.tensor_upload(H.TYPE_IDS[tname], m, k, host[name])
-        dts[name] = [first] + [ctx.tensor_clone(first) for _ in range(N_LAYERS - 1)]
+        copies = [first] + [ctx.tensor_clone(first) for _ in range(max(1, min(N_LAYERS, args.weight_copies)) - 1)]
+        dts[name] = [copies[l % len(copies)] for l in range(N_LAYERS)]
     name, tname, m, k = HEAD
     dts[name] = [ctx.tensor_upload(H.TYPE_IDS[tname], m, k, host[name])]
     gen_s = time.time() - t0
@@ -340,7 +344,7 @@ def main() -> int:
                                "gate+up 14336x4096 Q4_K; down 4096x14336 Q6_K) + head 128256x4096 Q6_K",
                    "launches_per_step": sum(len(o) for _, o in groups), "weight_bytes_per_step": weight_bytes,
                    "algorithmic_bytes_per_step": step_bytes, "w_sigma": 0.02, "seed": args.seed,
-                   "distinct_weight_copies": N_LAYERS},
+                   "distinct_weight_copies": max(1, min(N_LAYERS, args.weight_copies))},
         "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2),
         "gemv_only_tok_s_equiv": round(1e3 / ms_per_step, 1),
         "per_group": per_group,

@@ -412,16 +412,27 @@ cera_hip_status cera_launch_attn(cera_hip_ctx* ctx, const float* q, const float*
     // seq_len = keys visible to the first query; the last query sees seq_len + n_queries - 1
     const uint64_t last_len = seq_len + n_queries - 1;
     if (seq_len == 0 || last_len > max_seq || max_seq > 0x7FFFFFFFull) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "attention: need 0 < seq_len <= max_seq < 2^31");
-    // positions per chunk: small chunks while the context is short (one memory round
-    // trip per wavefront, many wavefronts), 64 once there is plenty of work
-    const uint32_t S = last_len >= 16384 ? 8 : (last_len >= 4096 ? 4 : (last_len >= 1024 ? 2 : 1));
-    uint32_t n_chunks = static_cast<uint32_t>((last_len + 8 * S - 1) / (8 * S));
-    // parts (wavefronts) per (query, kv head): enough to fill the chip ~8 waves per CU
-    // deep, but at least one chunk each and at most ATTN_MAX_PARTS
-    uint32_t want_parts = n_splits ? n_splits : std::max(1u, ctx->n_cu * 8 / (n_kv_heads * n_queries));
-    want_parts = std::min<uint32_t>(want_parts, ATTN_MAX_PARTS);
-    uint32_t chunks_per_part = std::max(1u, (n_chunks + want_parts - 1) / want_parts);
-    uint32_t n_parts = (n_chunks + chunks_per_part - 1) / chunks_per_part;
+    // A batch of queries (prefill) runs the tiled MFMA kernel: a K/V tile is read once per 32
+    // queries instead of once per query.  Parts of 128 keys while the context is short, about
+    // eight parts per query block beyond that.
+    const bool batch = n_queries >= 16;
+    uint32_t n_parts, part_keys = 0, chunks_per_part = 0;
+    uint32_t S = 1;
+    if (batch) {
+        part_keys = last_len <= 1024 ? 128u : static_cast<uint32_t>(((last_len + 7) / 8 + 31) / 32 * 32);
+        n_parts = static_cast<uint32_t>((last_len + part_keys - 1) / part_keys);
+    } else {
+        // positions per chunk: small chunks while the context is short (one memory round
+        // trip per wavefront, many wavefronts), 64 once there is plenty of work
+        S = last_len >= 16384 ? 8 : (last_len >= 4096 ? 4 : (last_len >= 1024 ? 2 : 1));
+        uint32_t n_chunks = static_cast<uint32_t>((last_len + 8 * S - 1) / (8 * S));
+        // parts (wavefronts) per (query, kv head): enough to fill the chip ~8 waves per CU
+        // deep, but at least one chunk each and at most ATTN_MAX_PARTS
+        uint32_t want_parts = n_splits ? n_splits : std::max(1u, ctx->n_cu * 8 / (n_kv_heads * n_queries));
+        want_parts = std::min<uint32_t>(want_parts, ATTN_MAX_PARTS);
+        chunks_per_part = std::max(1u, (n_chunks + want_parts - 1) / want_parts);
+        n_parts = (n_chunks + chunks_per_part - 1) / chunks_per_part;
+    }
     uint64_t acc_bytes = static_cast<uint64_t>(n_queries) * n_kv_heads * n_parts * G * ATTN_HD * sizeof(float);
     uint64_t ml_bytes = static_cast<uint64_t>(n_queries) * n_kv_heads * n_parts * G * 2 * sizeof(float);
     if (ctx->attn_acc_bytes < acc_bytes) {
@@ -438,9 +449,15 @@ cera_hip_status cera_launch_attn(cera_hip_ctx* ctx, const float* q, const float*
         HIP_TRY(ctx, hipMalloc(reinterpret_cast<void**>(&ctx->attn_ml), ml_bytes));
         ctx->attn_ml_bytes = ml_bytes;
     }
-    dim3 grid((n_parts + 3) / 4, n_kv_heads, n_queries);
     uint32_t sl = static_cast<uint32_t>(seq_len), ms = static_cast<uint32_t>(max_seq);
     uint32_t q_stride = n_heads * head_dim;
+    if (batch) {
+        // heaviest query blocks (most visible keys) first
+        dim3 pgrid((n_queries + 31) / 32, n_heads, n_parts);
+        hipLaunchKernelGGL(attn_prefill_partial_kernel, pgrid, dim3(64), 0, ctx->stream, q, kc, vc, sl, n_queries, ms, scale,
+                           part_keys, n_parts, q_stride, G, ctx->attn_acc, ctx->attn_ml);
+    } else {
+    dim3 grid((n_parts + 3) / 4, n_kv_heads, n_queries);
 #define ATTN_LAUNCH_S(GG, SS)                                                                                  \
     hipLaunchKernelGGL((attn_decode_partial_kernel<GG, SS>), grid, dim3(256), 0, ctx->stream, q, kc, vc, sl, ms, \
                        scale, chunks_per_part, n_parts, q_stride, ctx->attn_acc, ctx->attn_ml)
@@ -459,6 +476,7 @@ cera_hip_status cera_launch_attn(cera_hip_ctx* ctx, const float* q, const float*
     }
 #undef ATTN_LAUNCH_S
 #undef ATTN_LAUNCH
+    }
     HIP_TRY(ctx, hipGetLastError());
     dim3 mgrid(n_heads, n_queries);
     if (out_quants)
@@ -597,6 +615,35 @@ cera_hip_status cera_hip_attn_decode(cera_hip_ctx* ctx, const float* q, const fl
                                      static_cast<float*>(dout), nullptr, nullptr));
     CERA_TRY(cera_hip_download(ctx, out, dout, static_cast<uint64_t>(n_heads) * head_dim * 4));
     return CERA_HIP_OK;
+}
+
+cera_hip_status cera_hip_attn_prefill(cera_hip_ctx* ctx, const float* q, const float* k, const float* v,
+                                      uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, uint64_t start_pos,
+                                      uint32_t n_queries, float scale, float* out) {
+    if (!ctx || !q || !k || !v || !out) return CERA_HIP_ERR_ARGUMENT;
+    if (n_queries == 0 || n_kv_heads == 0 || head_dim == 0) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "attn_prefill: empty input");
+    const uint64_t seq_len = start_pos + n_queries;
+    const uint64_t kv_dim = static_cast<uint64_t>(n_kv_heads) * head_dim, q_dim = static_cast<uint64_t>(n_heads) * head_dim;
+    const uint64_t kv_bytes = seq_len * kv_dim * 4, q_bytes = n_queries * q_dim * 4;
+    // time-major [pos][kv_dim] (reference layout) -> head-major [kv_head][pos][head_dim]
+    std::vector<float> hk(seq_len * kv_dim), hv(seq_len * kv_dim);
+    for (uint64_t t = 0; t < seq_len; ++t)
+        for (uint32_t h = 0; h < n_kv_heads; ++h) {
+            std::memcpy(&hk[(h * seq_len + t) * head_dim], k + t * kv_dim + h * head_dim, head_dim * 4);
+            std::memcpy(&hv[(h * seq_len + t) * head_dim], v + t * kv_dim + h * head_dim, head_dim * 4);
+        }
+    void *dq, *dk, *dv, *dout;
+    CERA_TRY(cera_scratch(ctx, 0, q_bytes, &dq));
+    CERA_TRY(cera_scratch(ctx, 5, kv_bytes, &dk));
+    CERA_TRY(cera_scratch(ctx, 6, kv_bytes, &dv));
+    CERA_TRY(cera_scratch(ctx, 3, q_bytes, &dout));
+    CERA_TRY(cera_hip_upload(ctx, dq, q, q_bytes));
+    CERA_TRY(cera_hip_upload(ctx, dk, hk.data(), kv_bytes));
+    CERA_TRY(cera_hip_upload(ctx, dv, hv.data(), kv_bytes));
+    CERA_TRY(cera_launch_attn(ctx, static_cast<float*>(dq), static_cast<float*>(dk), static_cast<float*>(dv), n_heads,
+                              n_kv_heads, head_dim, start_pos + 1, seq_len, scale, 0, n_queries, static_cast<float*>(dout),
+                              nullptr, nullptr, nullptr));
+    return cera_hip_download(ctx, out, dout, q_bytes);
 }
 
 cera_hip_status cera_hip_rmsnorm(cera_hip_ctx* ctx, const float* x, const float* weight, uint64_t n, float eps, float* y) {

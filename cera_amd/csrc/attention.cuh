@@ -194,6 +194,157 @@ __global__ __launch_bounds__(256) void attn_decode_partial_kernel(
     }
 }
 
+// ---------------------------------------------------------------------------
+// Causal attention for a batch of queries (prefill) on the f32 matrix cores.
+//
+// The decode kernel above reads the whole visible K/V range once per query; for a
+// prompt of n tokens that is n passes over the cache.  Here one wavefront owns a
+// block of 32 consecutive queries of one head and walks the keys in tiles of 32, so
+// a K/V tile is read once per 32 queries, and both contractions run as
+// v_mfma_f32_32x32x2_f32 (f32 products, f32 accumulation: the same arithmetic class
+// as the reference's f32 dot products, cera/src/backend/cpu.rs:4028-4241).
+//
+//   S^T = K . Q^T   A = K tile (row = key, from LDS, transposed there so the lanes
+//                   of one step read consecutive words), B = the lane's query
+//                   (registers).  A lane ends up with 16 keys of ONE query, so the
+//                   softmax reduction over keys is over registers plus one exchange
+//                   between the wavefront halves.
+//   O  += P . V     A = P straight from those registers (the MFMA step (blk, r) pairs
+//                   key 8blk+r of the lower half with key 8blk+4+r of the upper half,
+//                   exactly the rows the two halves hold), B = V rows from HBM/L2.
+//
+// Online softmax per key tile with the reference's polynomial expf and an f64
+// running sum.  The key range is cut into parts of `part_keys`; a workgroup
+// produces the (m, l, acc) partial of one (query block, head, part) in the layout
+// the merge kernel below consumes, so long prompts spread over the chip and the
+// merge (and its fused Q8_0 quantisation) is shared with the decode path.
+// grid = (query blocks, heads, parts), 64 threads.
+#define ATTN_PF_LD 33  // words per LDS row of the transposed K tile (32 + 1 pad)
+typedef float attn_v16f __attribute__((ext_vector_type(16)));
+
+__global__ __launch_bounds__(64) void attn_prefill_partial_kernel(
+    const float* __restrict__ q,       // [n_queries][q_stride]
+    const float* __restrict__ kc,      // [n_kv][max_seq][128], already holding the batch's keys
+    const float* __restrict__ vc,
+    uint32_t first_len,                // keys visible to query 0; query i sees first_len + i
+    uint32_t n_queries, uint32_t max_seq, float scale, uint32_t part_keys, uint32_t n_parts, uint32_t q_stride,
+    uint32_t G,
+    float* __restrict__ part_acc,      // [n_queries][n_kv][n_parts][G][128]
+    float* __restrict__ part_ml) {     // [n_queries][n_kv][n_parts][G][2]
+    __shared__ float sKt[ATTN_HD * ATTN_PF_LD];
+    __shared__ __attribute__((aligned(16))) float sX[32];
+    const uint32_t lane = threadIdx.x, col = lane & 31, half = lane >> 5;
+    const uint32_t head = blockIdx.y, kvh = head / G, hg = head % G, n_kv = gridDim.y / G;
+    const uint32_t part = blockIdx.z;
+    const uint32_t q0 = blockIdx.x * 32, qidx = q0 + col;
+    const bool q_live = qidx < n_queries;
+    const uint32_t my_len = first_len + qidx;                             // keys this lane's query sees
+    const uint32_t block_len = first_len + min(n_queries, q0 + 32) - 1;   // ... and the block's last query
+    const uint32_t key_lo = part * part_keys;
+    const uint32_t key_hi = min(key_lo + part_keys, block_len);
+
+    const float* kbase = kc + static_cast<uint64_t>(kvh) * max_seq * ATTN_HD;
+    const float* vbase = vc + static_cast<uint64_t>(kvh) * max_seq * ATTN_HD;
+
+    // this lane's query, the dims of its half: d = 2s + half
+    float qreg[64];
+    {
+        const float* qp = q + static_cast<uint64_t>(min(qidx, n_queries - 1)) * q_stride + head * ATTN_HD + half;
+#pragma unroll
+        for (int s = 0; s < 64; ++s) qreg[s] = qp[2 * s];
+    }
+    attn_v16f acc[4];
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[dt][e] = 0.0f;
+    float m = -__builtin_inff();
+    double l = 0.0;
+
+    for (uint32_t k0 = key_lo; k0 < key_hi; k0 += 32) {
+        // ---- K tile -> LDS, transposed: 32 keys x 32 float4, 16 per lane
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const uint32_t f = lane + 64 * i, key = f >> 5, c4 = f & 31;
+            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (k0 + key < key_hi) v = reinterpret_cast<const float4*>(kbase + static_cast<uint64_t>(k0 + key) * ATTN_HD)[c4];
+            sKt[(4 * c4 + 0) * ATTN_PF_LD + key] = v.x;
+            sKt[(4 * c4 + 1) * ATTN_PF_LD + key] = v.y;
+            sKt[(4 * c4 + 2) * ATTN_PF_LD + key] = v.z;
+            sKt[(4 * c4 + 3) * ATTN_PF_LD + key] = v.w;
+        }
+        __syncthreads();
+        // ---- scores, transposed: c[4blk + r] = <K[k0 + 8blk + 4half + r], Q[qidx]>
+        attn_v16f c;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) c[e] = 0.0f;
+#pragma unroll
+        for (int s = 0; s < 64; ++s)
+            c = __builtin_amdgcn_mfma_f32_32x32x2f32(sKt[(2 * s + half) * ATTN_PF_LD + col], qreg[s], c, 0, 0, 0);
+        float mx = -__builtin_inff();
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            const uint32_t kg = k0 + 8 * (e >> 2) + 4 * half + (e & 3);
+            const bool ok = q_live && kg < my_len && kg < key_hi;
+            c[e] = ok ? c[e] * scale : -__builtin_inff();
+            mx = fmaxf(mx, c[e]);
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float m_new = fmaxf(m, mx);
+        // a query with nothing visible yet keeps m = -inf: weights and correction are then 0 / 1
+        const float corr = m_new == -__builtin_inff() ? 1.0f : cera_expf(m - m_new);
+        float ps = 0.0f;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            c[e] = c[e] == -__builtin_inff() ? 0.0f : cera_expf(c[e] - m_new);
+            ps += c[e];
+        }
+        ps += __shfl_xor(ps, 32, 64);
+        l = l * static_cast<double>(corr) + static_cast<double>(ps);
+        m = m_new;
+        // ---- the correction factors, re-laid out by output row (query 8blk + 4half + r)
+        if (half == 0) sX[col] = corr;
+        __syncthreads();
+#pragma unroll
+        for (int blk = 0; blk < 4; ++blk) {
+            const float4 cr = *reinterpret_cast<const float4*>(sX + 8 * blk + 4 * half);
+            const float crv[4] = {cr.x, cr.y, cr.z, cr.w};
+#pragma unroll
+            for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) acc[dt][4 * blk + r] *= crv[r];
+        }
+        // ---- O += P . V
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            const uint32_t kg = min(k0 + 8 * (e >> 2) + 4 * half + (e & 3), key_hi - 1);   // masked keys have p = 0
+            const float* vrow = vbase + static_cast<uint64_t>(kg) * ATTN_HD + col;
+#pragma unroll
+            for (int dt = 0; dt < 4; ++dt)
+                acc[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(c[e], vrow[32 * dt], acc[dt], 0, 0, 0);
+        }
+        __syncthreads();   // sKt and sX are rewritten by the next tile
+    }
+
+    // ---- partial out: rows of acc are queries 8blk + 4half + r, columns 32dt + col
+#pragma unroll
+    for (int blk = 0; blk < 4; ++blk)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const uint32_t qi = q0 + 8 * blk + 4 * half + r;
+            if (qi < n_queries) {
+                float* dst = part_acc + (((static_cast<uint64_t>(qi) * n_kv + kvh) * n_parts + part) * G + hg) * ATTN_HD + col;
+#pragma unroll
+                for (int dt = 0; dt < 4; ++dt) dst[32 * dt] = acc[dt][4 * blk + r];
+            }
+        }
+    if (half == 0 && q_live) {
+        float* ml = part_ml + (((static_cast<uint64_t>(qidx) * n_kv + kvh) * n_parts + part) * G + hg) * 2;
+        ml[0] = m;
+        ml[1] = static_cast<float>(l);
+    }
+}
+
 // Merge the parts of one query head: out = sum_p e^{m_p - M} acc_p / sum_p e^{m_p - M} l_p.
 // One workgroup of 256 threads per (head, query): the maxima and weights are
 // computed with the parts spread over all threads, the weighted accumulation

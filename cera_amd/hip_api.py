@@ -22,7 +22,7 @@ SYMBOLS = [
     "cera_hip_malloc", "cera_hip_free", "cera_hip_upload", "cera_hip_download", "cera_hip_copy_dev", "cera_hip_copy_kernel",
     "cera_hip_event_create", "cera_hip_event_destroy", "cera_hip_event_record", "cera_hip_event_elapsed_ms",
     "cera_hip_tensor_upload", "cera_hip_tensor_clone", "cera_hip_tensor_free", "cera_hip_tensor_nbytes",
-    "cera_hip_quantize_q8_0", "cera_hip_gemv", "cera_hip_gemm", "cera_hip_attn_decode", "cera_hip_rmsnorm",
+    "cera_hip_quantize_q8_0", "cera_hip_gemv", "cera_hip_gemm", "cera_hip_attn_decode", "cera_hip_attn_prefill", "cera_hip_rmsnorm",
     "cera_hip_silu_mul", "cera_hip_rope", "cera_hip_argmax", "cera_hip_dequantize_row",
     "cera_hip_quantize_q8_0_dev", "cera_hip_gemv_q8_dev", "cera_hip_gemv_seq_dev", "cera_hip_attn_decode_dev",
     "cera_hip_gemm_dev",
@@ -96,6 +96,7 @@ def load_library() -> C.CDLL:
         "cera_hip_gemv": (i32, [vp, C.POINTER(Tensor), vp, vp, vp, vp]),
         "cera_hip_gemm": (i32, [vp, C.POINTER(Tensor), vp, u64, vp]),
         "cera_hip_attn_decode": (i32, [vp, vp, vp, vp, u32, u32, u32, u64, f32, u32, vp]),
+        "cera_hip_attn_prefill": (i32, [vp, vp, vp, vp, u32, u32, u32, u64, u32, f32, vp]),
         "cera_hip_rmsnorm": (i32, [vp, vp, vp, u64, f32, vp]),
         "cera_hip_silu_mul": (i32, [vp, vp, vp, u64, vp]),
         "cera_hip_rope": (i32, [vp, vp, vp, u32, u32, u32, u32, f32, u32, vp]),
@@ -258,6 +259,15 @@ class Context:
         self.check(self.lib.cera_hip_attn_decode(self.h, _p(q), _p(k), _p(v), n_heads, n_kv_heads, head_dim, seq_len,
                                                  scale, n_splits, _p(out)))
         return out
+
+    def attn_prefill(self, q, k, v, n_heads, n_kv_heads, head_dim, start_pos, n_queries, scale) -> np.ndarray:
+        q = np.ascontiguousarray(q, np.float32)
+        k = np.ascontiguousarray(k, np.float32)
+        v = np.ascontiguousarray(v, np.float32)
+        out = np.empty(n_queries * n_heads * head_dim, np.float32)
+        self.check(self.lib.cera_hip_attn_prefill(self.h, _p(q), _p(k), _p(v), n_heads, n_kv_heads, head_dim, start_pos,
+                                                  n_queries, scale, _p(out)))
+        return out.reshape(n_queries, n_heads * head_dim)
 
     def rmsnorm(self, x, w, eps) -> np.ndarray:
         x = np.ascontiguousarray(x, np.float32)

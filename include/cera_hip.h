@@ -163,6 +163,16 @@ CERA_HIP_API cera_hip_status cera_hip_attn_decode(cera_hip_ctx*, const float* q,
                                                   uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim,
                                                   uint64_t seq_len, float scale, uint32_t n_splits, float* out);
 
+/* Causal attention of a batch of n_queries new tokens, the attention step of
+ * LlamaModel::forward_prefill_batched (cera/src/model/llama.rs:845-1010; flash route
+ * cera/src/backend/cpu.rs:4028-4241, per-query route transformer.rs:1249-1305).
+ * q f32 [n_queries][n_heads*head_dim]; k, v f32 time-major [start_pos + n_queries][n_kv_heads*head_dim]
+ * already containing the batch's own keys/values; query i sees positions 0 .. start_pos + i.
+ * out f32 [n_queries][n_heads*head_dim]. */
+CERA_HIP_API cera_hip_status cera_hip_attn_prefill(cera_hip_ctx*, const float* q, const float* k, const float* v,
+                                                   uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim,
+                                                   uint64_t start_pos, uint32_t n_queries, float scale, float* out);
+
 /* cpu::rmsnorm (cera/src/backend/cpu.rs:2479-2496), out of place: y = x*inv_rms*w. */
 CERA_HIP_API cera_hip_status cera_hip_rmsnorm(cera_hip_ctx*, const float* x, const float* weight, uint64_t n,
                                               float eps, float* y);

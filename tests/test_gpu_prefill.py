@@ -37,7 +37,7 @@ def test_gemm_small_shapes(hip, orc, dtype, m, n, k):
 
 
 @pytest.mark.parametrize("dtype,m,k", [(Q4_K, 4096, 4096), (Q6_K, 4096, 14336)])
-@pytest.mark.parametrize("n", [128, 512])
+@pytest.mark.parametrize("n", [128, 512, 2048])
 def test_gemm_config3_shapes_row_sample(hip, orc, dtype, m, k, n):
     """BASELINE config 3 shapes; the oracle checks a sample of output rows."""
     _say(f"gemm {util.NAMES[dtype]} m={m} n={n} k={k}")
@@ -125,3 +125,26 @@ def test_prefill_equals_decode_on_gpu(hip):
     kb, vb = b.read_kv(0)
     assert np.abs(ka - kb).max() <= 2e-3 * util.rms(kb)
     a.close(); b.close()
+
+
+@pytest.mark.parametrize("nh,nkv,start,n", [(32, 8, 0, 512), (8, 2, 0, 40), (8, 8, 300, 100), (16, 2, 1000, 33),
+                                             (4, 1, 0, 16), (32, 8, 4000, 96)])
+def test_attn_prefill_batch_vs_oracle(hip, orc, nh, nkv, start, n):
+    """Causal attention of a batch of queries (the tiled MFMA kernel) against the oracle's
+    decode_attention evaluated query by query: query i sees positions 0 .. start + i."""
+    hd = 128
+    _say(f"attn_prefill nh={nh} nkv={nkv} start={start} n={n}")
+    r = util.rng(7 * n + start)
+    L = start + n
+    q = r.standard_normal((n, nh * hd), dtype=np.float32)
+    k = r.standard_normal(L * nkv * hd, dtype=np.float32)
+    v = r.standard_normal(L * nkv * hd, dtype=np.float32)
+    scale = 1.0 / np.sqrt(hd)
+    out = hip.attn_prefill(q, k, v, nh, nkv, hd, start, n, scale)
+    picks = sorted(set([0, 1, 15, 16, 31, 32, n // 2, n - 2, n - 1]) & set(range(n)))
+    for i in picks:
+        Li = start + i + 1
+        ref = orc.decode_attention(q[i], k[:Li * nkv * hd], v[:Li * nkv * hd], nh, nkv, hd, scale, Li)
+        err = np.abs(out[i].astype(np.float64) - ref).max()
+        assert err <= 2e-3 * util.rms(ref), (i, err, util.rms(ref))
+    assert np.isfinite(out).all()
