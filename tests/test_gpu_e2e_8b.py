@@ -73,6 +73,7 @@ def test_llama3_8b_prefill_512_greedy_256(tmp_path, orc, hip):
         return abs(p - q) / max(abs(p), abs(q), 1.0)
 
     same_g = same_b = 0
+    worst_g = worst_b = 0.0   # largest margin of a disagreement, in units of the per-logit noise rms
     rel_g, rel_b, cos_g, cos_b = [], [], [], []
     t0 = time.time()
     for i in range(n_new):
@@ -81,23 +82,30 @@ def test_llama3_8b_prefill_512_greedy_256(tmp_path, orc, hip):
         cos_g.append(cos(lg, la)); cos_b.append(cos(lb, la))
         tg, ta, tb = int(toks[i]), int(orc.argmax(la)), int(orc.argmax(lb))
         same_b += ta == tb
+        if ta != tb:
+            worst_b = max(worst_b, max(float(la[ta] - la[tb]), float(lb[tb] - lb[ta])) / util.rms(lb - la))
         if ta == tg:
             same_g += 1
         else:
-            # a disagreement must be explained by the measured logit noise on both sides
-            # (the difference of two logits carries sqrt(2) x the per-logit noise)
+            # a disagreement must be explained by the measured logit noise on both sides: the
+            # difference of two logits carries sqrt(2) x the per-logit noise, and with ~1e5
+            # candidates x 256 steps a 4-sigma swing of some pair is expected, so the bound is
+            # 5 sigma of the pair difference (7 x the per-logit rms)
             noise = util.rms(lg - la)
             m_a, m_g = float(la[ta] - la[tg]), float(lg[tg] - lg[ta])
             _say(f"  step {i}: GPU {tg} vs oracle {ta}: margins {m_a:.3f} / {m_g:.3f}, logit noise rms {noise:.3f}, "
                  f"relative gaps {gap_rel(la, ta, tg):.4f} / {gap_rel(lg, ta, tg):.4f}")
-            assert m_a <= 4 * noise and m_g <= 4 * noise, f"step {i}: different token beyond the noise"
+            worst_g = max(worst_g, max(m_a, m_g) / noise)
+            assert m_a <= 7 * noise and m_g <= 7 * noise, f"step {i}: different token beyond the noise"
         if i + 1 < n_new:       # teacher-forced on the GPU's sequence
             la, lb = oa.forward(tg, n_prompt + i), ob.forward(tg, n_prompt + i)
     _say(f"e2e: oracle decode {time.time() - t0:.0f} s")
     _say(f"e2e: GPU vs oracle(batched):            identical greedy tokens {same_g}/{n_new}, "
-         f"cosine min {min(cos_g):.5f} mean {np.mean(cos_g):.5f}, rms(diff)/rms mean {np.mean(rel_g):.4f}")
+         f"cosine min {min(cos_g):.5f} mean {np.mean(cos_g):.5f}, rms(diff)/rms mean {np.mean(rel_g):.4f}, "
+         f"largest disagreement margin {worst_g:.1f} x noise")
     _say(f"e2e: oracle(per-token) vs oracle(batched): identical greedy tokens {same_b}/{n_new}, "
-         f"cosine min {min(cos_b):.5f} mean {np.mean(cos_b):.5f}, rms(diff)/rms mean {np.mean(rel_b):.4f}")
+         f"cosine min {min(cos_b):.5f} mean {np.mean(cos_b):.5f}, rms(diff)/rms mean {np.mean(rel_b):.4f}, "
+         f"largest disagreement margin {worst_b:.1f} x noise")
     oa.set_pool(None); ob.set_pool(None)
     pool.close()
     oa.close(); ob.close()
