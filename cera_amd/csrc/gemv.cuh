@@ -323,7 +323,7 @@ template <class T, int U, int KS, int RB, int EPI, bool DBG>
 __device__ __forceinline__ void gemv_compute(const GemvArgs& p, const GemvTile<T, U, RB, (EPI == EPI_SILU_MUL ? 2 : 1)>& t,
                                              const typename T::Act (&act)[U], const uint32_t (&unit)[U],
                                              const bool (&live)[U], uint32_t lane, uint32_t kw, uint32_t r,
-                                             uint32_t r1, float (*part)[RB][KS]) {
+                                             uint32_t r1, float (*part)[RB][KS * 4]) {
     constexpr int NM = EPI == EPI_SILU_MUL ? 2 : 1;
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) {
@@ -338,13 +338,15 @@ __device__ __forceinline__ void gemv_compute(const GemvArgs& p, const GemvTile<T
                 if (DBG) dbg = (live[i] && row < r1) ? p.dbg_dots + static_cast<uint64_t>(row) * p.dbg_stride : nullptr;
                 acc += T::dot(t.w[mi][rb][i], act[i], unit[i], dbg);
             }
-            tot[mi] = wave_sum(acc);
+            // K-split workgroups leave the four 16-lane row sums of each wavefront to the LDS
+            // combine below instead of folding them with cross-lane reads here
+            tot[mi] = KS == 1 ? wave_sum(acc) : wave_row_sum(acc);
         }
         if (KS == 1) {
             if (lane == 0 && row < r1) gemv_store<EPI>(p, row, tot[0], tot[NM - 1]);
-        } else if (lane == 0) {
+        } else if ((lane & 15) == 0) {
 #pragma unroll
-            for (int mi = 0; mi < NM; ++mi) part[mi][rb][kw] = tot[mi];
+            for (int mi = 0; mi < NM; ++mi) part[mi][rb][kw * 4 + (lane >> 4)] = tot[mi];
         }
     }
     if (KS > 1) {
@@ -353,9 +355,12 @@ __device__ __forceinline__ void gemv_compute(const GemvArgs& p, const GemvTile<T
             float v[NM];
 #pragma unroll
             for (int mi = 0; mi < NM; ++mi) {
-                float s = part[mi][threadIdx.x][0];
+                float s = 0.0f;
 #pragma unroll
-                for (int w = 1; w < KS; ++w) s += part[mi][threadIdx.x][w];
+                for (int w = 0; w < KS; ++w) {   // wavefront order, rows paired as wave_sum pairs them
+                    const float* q4 = &part[mi][threadIdx.x][4 * w];
+                    s += (q4[0] + q4[1]) + (q4[2] + q4[3]);
+                }
                 v[mi] = s;
             }
             gemv_store<EPI>(p, r + threadIdx.x, v[0], v[NM - 1]);
@@ -367,7 +372,7 @@ template <class T, int U, int KS, int RB, int EPI, bool DBG>
 static __global__ __launch_bounds__(64 * KS) void gemv_kernel(GemvArgs p) {
     constexpr int NM = EPI == EPI_SILU_MUL ? 2 : 1;
     // two LDS buffers: a buffer is rewritten two row groups later, after another barrier
-    __shared__ float part[2][NM][RB][KS];
+    __shared__ float part[2][NM][RB][KS * 4];
     const uint32_t lane = threadIdx.x & 63, kw = threadIdx.x >> 6;
     uint32_t r = blockIdx.x * p.rows_per_wave;  // rows per workgroup
     if (r >= p.m) return;
@@ -391,15 +396,24 @@ static __global__ __launch_bounds__(64 * KS) void gemv_kernel(GemvArgs p) {
         if (DBG && blockIdx.x == 0 && live[i] && p.dbg_asums) T::dbg_asum(act[i], unit[i], p.dbg_asums);
     }
 
+    // Each prefetch sits in the same straight-line block as the compute it overlaps, so the
+    // compiler can wait for exactly the older tile's loads (a prefetch under its own
+    // condition would force a wait for everything at the join).
     for (;;) {
-        if (r + RB < r1) tb.load(p, unit, r + RB, r1);
+        if (r + RB >= r1) {
+            gemv_compute<T, U, KS, RB, EPI, DBG>(p, ta, act, unit, live, lane, kw, r, r1, part[0]);
+            break;
+        }
+        tb.load(p, unit, r + RB, r1);
         gemv_compute<T, U, KS, RB, EPI, DBG>(p, ta, act, unit, live, lane, kw, r, r1, part[0]);
         r += RB;
-        if (r >= r1) break;
-        if (r + RB < r1) ta.load(p, unit, r + RB, r1);
+        if (r + RB >= r1) {
+            gemv_compute<T, U, KS, RB, EPI, DBG>(p, tb, act, unit, live, lane, kw, r, r1, part[1]);
+            break;
+        }
+        ta.load(p, unit, r + RB, r1);
         gemv_compute<T, U, KS, RB, EPI, DBG>(p, tb, act, unit, live, lane, kw, r, r1, part[1]);
         r += RB;
-        if (r >= r1) break;
     }
 }
 

@@ -25,7 +25,10 @@ static inline bool gemv_pick_split(uint32_t n_units, int* U, int* KS) {
 // step for the 16-byte-unit formats and two for Q6_K (15 registers per row).
 static inline bool gemv_plan(uint32_t m, uint32_t n_units, uint32_t n_cu, bool dbg, int max_rb, GemvPlan* p) {
     if (!gemv_pick_split(n_units, &p->U, &p->KS)) return false;
-    const uint32_t target_blocks = std::max(1u, n_cu * 32 / static_cast<uint32_t>(p->KS));
+    // very tall matrices (the vocabulary head) do better with few long-lived workgroups that
+    // stream row groups through the two register buffers; everything else with many short ones
+    const uint32_t per_cu = m >= 65536 ? 4 : 32;
+    const uint32_t target_blocks = std::max(1u, n_cu * per_cu / static_cast<uint32_t>(p->KS));
     uint32_t rpb = (m + target_blocks - 1) / target_blocks;
     p->RB = rpb >= 4 ? 4 : (rpb >= 2 ? 2 : 1);
     if (p->RB > max_rb) p->RB = max_rb;
