@@ -403,7 +403,7 @@ cera_hip_status cera_launch_gemv_q5k_f32(cera_hip_ctx* ctx, const cera_hip_dtens
 cera_hip_status cera_launch_attn(cera_hip_ctx* ctx, const float* q, const float* kc, const float* vc,
                                  uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, uint64_t seq_len,
                                  uint64_t max_seq, float scale, uint32_t n_splits, uint32_t n_queries, float* out,
-                                 float* out_scales, int8_t* out_quants, float* out_bsum) {
+                                 float* out_scales, int8_t* out_quants, float* out_bsum, const AttnNewKV* new_kv) {
     if (head_dim != ATTN_HD) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "attention: head_dim must be 128");
     if (n_kv_heads == 0 || n_heads % n_kv_heads) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "attention: n_heads must be a multiple of n_kv_heads");
     uint32_t G = n_heads / n_kv_heads;
@@ -415,7 +415,9 @@ cera_hip_status cera_launch_attn(cera_hip_ctx* ctx, const float* q, const float*
     // A batch of queries (prefill) runs the tiled MFMA kernel: a K/V tile is read once per 32
     // queries instead of once per query.  Parts of 128 keys while the context is short, about
     // eight parts per query block beyond that.
+    if (new_kv && n_queries != 1) return cera_fail(ctx, CERA_HIP_ERR_ARGUMENT, "attention: fused RoPE/append is for single-token decode");
     const bool batch = n_queries >= 16;
+    const AttnNewKV nk = new_kv ? *new_kv : AttnNewKV{};
     uint32_t n_parts, part_keys = 0, chunks_per_part = 0;
     uint32_t S = 1;
     if (batch) {
@@ -458,9 +460,15 @@ cera_hip_status cera_launch_attn(cera_hip_ctx* ctx, const float* q, const float*
                            part_keys, n_parts, q_stride, G, ctx->attn_acc, ctx->attn_ml);
     } else {
     dim3 grid((n_parts + 3) / 4, n_kv_heads, n_queries);
-#define ATTN_LAUNCH_S(GG, SS)                                                                                  \
-    hipLaunchKernelGGL((attn_decode_partial_kernel<GG, SS>), grid, dim3(256), 0, ctx->stream, q, kc, vc, sl, ms, \
-                       scale, chunks_per_part, n_parts, q_stride, ctx->attn_acc, ctx->attn_ml)
+#define ATTN_LAUNCH_S(GG, SS)                                                                                         \
+    do {                                                                                                              \
+        if (new_kv)                                                                                                   \
+            hipLaunchKernelGGL((attn_decode_partial_kernel<GG, SS, true>), grid, dim3(256), 0, ctx->stream, q, kc, vc, \
+                               sl, ms, scale, chunks_per_part, n_parts, q_stride, ctx->attn_acc, ctx->attn_ml, nk);   \
+        else                                                                                                          \
+            hipLaunchKernelGGL((attn_decode_partial_kernel<GG, SS, false>), grid, dim3(256), 0, ctx->stream, q, kc, vc, \
+                               sl, ms, scale, chunks_per_part, n_parts, q_stride, ctx->attn_acc, ctx->attn_ml, nk);   \
+    } while (0)
 #define ATTN_LAUNCH(GG)                              \
     switch (S) {                                     \
         case 1: ATTN_LAUNCH_S(GG, 1); break;         \
@@ -493,9 +501,9 @@ cera_hip_status cera_launch_attn(cera_hip_ctx* ctx, const float* q, const float*
 cera_hip_status cera_launch_attn_decode(cera_hip_ctx* ctx, const float* q, const float* kc, const float* vc,
                                         uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, uint64_t seq_len,
                                         uint64_t max_seq, float scale, uint32_t n_splits, float* out,
-                                        float* out_scales, int8_t* out_quants) {
+                                        float* out_scales, int8_t* out_quants, const AttnNewKV* new_kv) {
     return cera_launch_attn(ctx, q, kc, vc, n_heads, n_kv_heads, head_dim, seq_len, max_seq, scale, n_splits, 1, out,
-                            out_scales, out_quants, nullptr);
+                            out_scales, out_quants, nullptr, new_kv);
 }
 
 // ---------------------------------------------------------------------------

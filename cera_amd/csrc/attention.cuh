@@ -22,6 +22,7 @@
 // reduction at the end of the part.
 #pragma once
 #include "common.cuh"
+#include "attn_types.h"
 #include "quantize.cuh"
 
 #define ATTN_HD 128
@@ -35,7 +36,38 @@ struct AttnPart {  // per (part, query head): running max, sum and unnormalised 
 // every wavefront has a single memory round trip (all its K and V loads in
 // flight at once) and there are enough wavefronts to cover the chip; long
 // contexts use 64-position chunks to amortise the softmax bookkeeping.
-template <int G, int S>
+// In-place RoPE of the 16 values a lane holds of one 128-wide head (float4 c sits at float4
+// index j + 8c), same arithmetic as rope_kv_kernel.  rope_row = the position's 64 (cos, sin).
+__device__ __forceinline__ void attn_rope16(float4 (&x)[4], const float* __restrict__ rope_row, uint32_t j, uint32_t rope_type) {
+    if (rope_type == 1) {   // NORM: pairs (2i, 2i+1) = (x, y) and (z, w) of each float4
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const float4 cs = reinterpret_cast<const float4*>(rope_row)[j + 8 * c];
+            const float4 v = x[c];
+            x[c].x = __fsub_rn(__fmul_rn(v.x, cs.x), __fmul_rn(v.y, cs.y));
+            x[c].y = __fadd_rn(__fmul_rn(v.x, cs.y), __fmul_rn(v.y, cs.x));
+            x[c].z = __fsub_rn(__fmul_rn(v.z, cs.z), __fmul_rn(v.w, cs.w));
+            x[c].w = __fadd_rn(__fmul_rn(v.z, cs.w), __fmul_rn(v.w, cs.z));
+        }
+    } else {                // NEOX: pairs (i, i + 64): float4 c with float4 c + 2
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+            const float4 c01 = reinterpret_cast<const float4*>(rope_row)[2 * (j + 8 * c)];
+            const float4 c23 = reinterpret_cast<const float4*>(rope_row)[2 * (j + 8 * c) + 1];
+            const float4 a = x[c], b = x[c + 2];
+            x[c].x = __fsub_rn(__fmul_rn(a.x, c01.x), __fmul_rn(b.x, c01.y));
+            x[c + 2].x = __fadd_rn(__fmul_rn(a.x, c01.y), __fmul_rn(b.x, c01.x));
+            x[c].y = __fsub_rn(__fmul_rn(a.y, c01.z), __fmul_rn(b.y, c01.w));
+            x[c + 2].y = __fadd_rn(__fmul_rn(a.y, c01.w), __fmul_rn(b.y, c01.z));
+            x[c].z = __fsub_rn(__fmul_rn(a.z, c23.x), __fmul_rn(b.z, c23.y));
+            x[c + 2].z = __fadd_rn(__fmul_rn(a.z, c23.y), __fmul_rn(b.z, c23.x));
+            x[c].w = __fsub_rn(__fmul_rn(a.w, c23.z), __fmul_rn(b.w, c23.w));
+            x[c + 2].w = __fadd_rn(__fmul_rn(a.w, c23.w), __fmul_rn(b.w, c23.z));
+        }
+    }
+}
+
+template <int G, int S, bool NEWKV>
 __global__ __launch_bounds__(256) void attn_decode_partial_kernel(
     const float* __restrict__ q,       // [n_heads][128]
     const float* __restrict__ kc,      // [n_kv][max_seq][128]
@@ -43,7 +75,8 @@ __global__ __launch_bounds__(256) void attn_decode_partial_kernel(
     uint32_t seq_len, uint32_t max_seq, float scale, uint32_t chunks_per_part, uint32_t n_parts,
     uint32_t q_stride,                 // floats between consecutive queries (prefill batches queries on grid.z)
     float* __restrict__ part_acc,      // [n_queries][n_kv][n_parts][G][128]
-    float* __restrict__ part_ml) {     // [n_queries][n_kv][n_parts][G][2]
+    float* __restrict__ part_ml,       // [n_queries][n_kv][n_parts][G][2]
+    AttnNewKV nk) {
     const uint32_t lane = threadIdx.x & 63;
     const uint32_t part = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
     const uint32_t kvh = blockIdx.y, qi = blockIdx.z;
@@ -60,6 +93,11 @@ __global__ __launch_bounds__(256) void attn_decode_partial_kernel(
 #pragma unroll
         for (int c = 0; c < 4; ++c)
             qv[h][c] = reinterpret_cast<const float4*>(q + (kvh * G + h) * ATTN_HD)[j + 8 * c];
+    if (NEWKV) {
+#pragma unroll
+        for (int h = 0; h < G; ++h) attn_rope16(qv[h], nk.rope_row, j, nk.rope_type);
+    }
+    const uint32_t new_pos = seq_len - 1;   // NEWKV: the position whose K/V are not in the cache yet
 
     float4 acc[G][4];
     float m[G], l[G];
@@ -85,8 +123,14 @@ __global__ __launch_bounds__(256) void attn_decode_partial_kernel(
             for (int s = 0; s < S; ++s) {
                 uint32_t t = t0 + 8 * s + pg;
                 const float4* vp = reinterpret_cast<const float4*>(vbase + static_cast<uint64_t>(t < t_end ? t : t_begin) * ATTN_HD);
+                if (NEWKV && t == new_pos) vp = reinterpret_cast<const float4*>(nk.v_new + kvh * ATTN_HD);
 #pragma unroll
                 for (int c = 0; c < 4; ++c) vpre[s][c] = vp[j + 8 * c];
+                if (NEWKV && t == new_pos) {
+                    float4* dst = reinterpret_cast<float4*>(nk.vc_w + (static_cast<uint64_t>(kvh) * max_seq + t) * ATTN_HD);
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) dst[j + 8 * c] = vpre[s][c];
+                }
             }
         }
         // ---- scores: step s covers positions t0 + 8s + pg
@@ -96,9 +140,16 @@ __global__ __launch_bounds__(256) void attn_decode_partial_kernel(
             uint32_t t = t0 + 8 * s + pg;
             bool live = t < t_end;
             const float4* kp = reinterpret_cast<const float4*>(kbase + static_cast<uint64_t>(live ? t : t_begin) * ATTN_HD);
+            if (NEWKV && t == new_pos) kp = reinterpret_cast<const float4*>(nk.k_new + kvh * ATTN_HD);
             float4 kv[4];
 #pragma unroll
             for (int c = 0; c < 4; ++c) kv[c] = kp[j + 8 * c];
+            if (NEWKV && t == new_pos) {
+                attn_rope16(kv, nk.rope_row, j, nk.rope_type);
+                float4* dst = reinterpret_cast<float4*>(nk.kc_w + (static_cast<uint64_t>(kvh) * max_seq + t) * ATTN_HD);
+#pragma unroll
+                for (int c = 0; c < 4; ++c) dst[j + 8 * c] = kv[c];
+            }
 #pragma unroll
             for (int h = 0; h < G; ++h) {
                 float d = 0.0f;
@@ -143,8 +194,14 @@ __global__ __launch_bounds__(256) void attn_decode_partial_kernel(
             } else {
                 uint32_t t = t0 + 8 * s + pg;
                 const float4* vp = reinterpret_cast<const float4*>(vbase + static_cast<uint64_t>(t < t_end ? t : t_begin) * ATTN_HD);
+                if (NEWKV && t == new_pos) vp = reinterpret_cast<const float4*>(nk.v_new + kvh * ATTN_HD);
 #pragma unroll
                 for (int c = 0; c < 4; ++c) vv[c] = vp[j + 8 * c];
+                if (NEWKV && t == new_pos) {
+                    float4* dst = reinterpret_cast<float4*>(nk.vc_w + (static_cast<uint64_t>(kvh) * max_seq + t) * ATTN_HD);
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) dst[j + 8 * c] = vv[c];
+                }
             }
 #pragma unroll
             for (int h = 0; h < G; ++h) {
