@@ -251,6 +251,20 @@ std::vector<float> HipLlamaModel::forward_prefill(const uint32_t* tokens, size_t
     return logits;
 }
 
+std::vector<float> HipLlamaModel::forward_prefill_logits_all(const uint32_t* tokens, size_t n, size_t start_pos,
+                                                             InferenceState& state) {
+    if (n == 0) bail("forward_prefill_logits_all requires at least one token");
+    if (start_pos != state.seq_len)
+        bail("forward_prefill_logits_all: start_pos (" + std::to_string(start_pos) + ") must equal state.seq_len (" +
+             std::to_string(state.seq_len) + ")");
+    std::vector<float> logits(n * config_.vocab_size);
+    if (cera_hip_forward_prefill_logits_all(model_, tokens, static_cast<uint32_t>(n), static_cast<uint32_t>(start_pos),
+                                            logits.data()) != CERA_HIP_OK)
+        device_panic("forward_prefill_logits_all");
+    state.seq_len = cera_hip_seq_len(model_);
+    return logits;
+}
+
 uint32_t HipLlamaModel::forward_greedy(const uint32_t* tokens, size_t n, size_t pos, InferenceState& state) {
     if (n != 1) bail("HipLlamaModel forward_greedy expects single token");
     uint32_t next = 0;

@@ -65,6 +65,8 @@ public:
     virtual std::vector<float> forward_prefill(const uint32_t* tokens, size_t n_tokens, size_t start_pos,
                                                InferenceState& state);
     virtual uint32_t forward_greedy(const uint32_t* tokens, size_t n_tokens, size_t pos, InferenceState& state);
+    // logits of every position, row-major [n_tokens * vocab]; empty unless supports_all_logits()
+    virtual std::vector<float> forward_prefill_logits_all(const uint32_t*, size_t, size_t, InferenceState&) { return {}; }
     virtual void truncate_kv(InferenceState& state, size_t len) = 0;
     // (tokens consumed, logits of the last processed chunk); chunks of `ubatch` (0 = one chunk),
     // `cancel` polled after each chunk.
@@ -94,6 +96,9 @@ public:
     std::vector<float> forward_prefill(const uint32_t* tokens, size_t n_tokens, size_t start_pos,
                                        InferenceState& state) override;
     uint32_t forward_greedy(const uint32_t* tokens, size_t n_tokens, size_t pos, InferenceState& state) override;
+    std::vector<float> forward_prefill_logits_all(const uint32_t* tokens, size_t n_tokens, size_t start_pos,
+                                                  InferenceState& state) override;
+    bool supports_all_logits() const override { return true; }
     void truncate_kv(InferenceState& state, size_t len) override;
     const ModelConfig& config() const override { return config_; }
     uint64_t gpu_memory_bytes() const override;

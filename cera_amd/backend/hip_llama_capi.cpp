@@ -97,6 +97,13 @@ int cera_llama_forward_prefill(cera_llama* h, const uint32_t* tokens, uint64_t n
         std::memcpy(logits, l.data(), l.size() * sizeof(float));
     });
 }
+int cera_llama_forward_prefill_logits_all(cera_llama* h, const uint32_t* tokens, uint64_t n, uint64_t start_pos,
+                                          float* logits) {
+    return guarded(h, [&] {
+        std::vector<float> l = h->model->forward_prefill_logits_all(tokens, n, start_pos, h->state);
+        std::memcpy(logits, l.data(), l.size() * sizeof(float));
+    });
+}
 int cera_llama_forward_prefill_chunked(cera_llama* h, const uint32_t* tokens, uint64_t n, uint64_t start_pos,
                                        uint64_t ubatch, uint64_t* consumed, float* logits) {
     return guarded(h, [&] {

@@ -31,6 +31,9 @@ CERA_LLAMA_API int cera_llama_forward(cera_llama*, uint32_t token, uint64_t pos,
 CERA_LLAMA_API int cera_llama_forward_greedy(cera_llama*, uint32_t token, uint64_t pos, uint32_t* next);
 CERA_LLAMA_API int cera_llama_forward_prefill(cera_llama*, const uint32_t* tokens, uint64_t n, uint64_t start_pos,
                                               float* last_logits);
+/* Model::forward_prefill_logits_all: logits_all[n][vocab] */
+CERA_LLAMA_API int cera_llama_forward_prefill_logits_all(cera_llama*, const uint32_t* tokens, uint64_t n,
+                                                         uint64_t start_pos, float* logits_all);
 /* Model::forward_prefill_chunked: *consumed tokens went into the KV cache; last_logits is
  * written when at least one chunk ran.  The cancel flag is the one set by cera_llama_set_cancel. */
 CERA_LLAMA_API int cera_llama_forward_prefill_chunked(cera_llama*, const uint32_t* tokens, uint64_t n,

@@ -36,6 +36,8 @@ struct cera_hip_model {
           *pf_attn = nullptr, *pf_gate = nullptr, *pf_up = nullptr, *pf_xs = nullptr, *pf_bsum = nullptr;
     int8_t* pf_xq = nullptr;
     uint32_t* pf_tokens = nullptr;
+    float* pf_logits = nullptr;   // [pf_cap][head rows], allocated on the first all-logits call
+    uint32_t pf_logits_cap = 0;
     std::vector<void*> pf_owned;
     uint32_t seq_len = 0;
     uint64_t bytes = 0;
@@ -51,3 +53,7 @@ cera_hip_status cera_model_prefill_per_token(cera_hip_model* m, const uint32_t* 
 // type has no int8 GEMM
 cera_hip_status cera_model_prefill(cera_hip_model* m, const uint32_t* tokens, uint32_t n, uint32_t start_pos,
                                    float* last_logits);
+// same, logits of every position into logits_all[n][vocab] (host)
+cera_hip_status cera_model_prefill_logits_all(cera_hip_model* m, const uint32_t* tokens, uint32_t n, uint32_t start_pos,
+                                              float* logits_all);
+cera_hip_status cera_model_decode_logits(cera_hip_model* m, uint32_t token, uint32_t pos, float* logits);

@@ -64,6 +64,7 @@ static void free_model(cera_hip_model* m) {
         if (p) (void)hipFree(p);
     for (void* p : m->pf_owned)
         if (p) (void)hipFree(p);
+    if (m->pf_logits) (void)hipFree(m->pf_logits);
     delete m;
 }
 
@@ -388,6 +389,29 @@ extern "C" cera_hip_status cera_hip_forward_prefill(cera_hip_model* m, const uin
     for (uint32_t i = 0; i < n; ++i)
         if (tokens[i] >= m->cfg.vocab) return cera_fail(m->ctx, CERA_HIP_ERR_ARGUMENT, "token id out of range");
     return cera_model_prefill(m, tokens, n, start_pos, last_logits);
+}
+
+extern "C" cera_hip_status cera_hip_forward_prefill_logits_all(cera_hip_model* m, const uint32_t* tokens, uint32_t n,
+                                                               uint32_t start_pos, float* logits_all) {
+    if (!m || !tokens || !logits_all) return CERA_HIP_ERR_ARGUMENT;
+    if (n == 0) return cera_fail(m->ctx, CERA_HIP_ERR_ARGUMENT, "forward_prefill_logits_all requires at least one token");
+    std::lock_guard<std::mutex> lk(m->infer_lock);
+    if (start_pos != m->seq_len)
+        return cera_fail(m->ctx, CERA_HIP_ERR_POSITION, "forward_prefill_logits_all: start_pos " + std::to_string(start_pos) +
+                                                            " must equal seq_len " + std::to_string(m->seq_len));
+    if (static_cast<uint64_t>(start_pos) + n > m->cfg.max_seq_len)
+        return cera_fail(m->ctx, CERA_HIP_ERR_POSITION, "forward_prefill_logits_all: tokens do not fit max_seq_len");
+    for (uint32_t i = 0; i < n; ++i)
+        if (tokens[i] >= m->cfg.vocab) return cera_fail(m->ctx, CERA_HIP_ERR_ARGUMENT, "token id out of range");
+    return cera_model_prefill_logits_all(m, tokens, n, start_pos, logits_all);
+}
+
+// one decode step with the logits copied out (the per-token route of the all-logits call)
+cera_hip_status cera_model_decode_logits(cera_hip_model* m, uint32_t token, uint32_t pos, float* logits) {
+    CERA_TRY(set_token_pos(m, token, pos));
+    CERA_TRY(decode_step(m, pos, true));
+    m->seq_len = pos + 1;
+    return cera_hip_download(m->ctx, logits, m->logits, static_cast<uint64_t>(m->cfg.vocab) * 4);
 }
 
 // Token-at-a-time prefill (LlamaModel::forward_prefill's per-token route,

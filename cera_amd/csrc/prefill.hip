@@ -149,8 +149,10 @@ static cera_hip_status ensure_prefill_buffers(cera_hip_model* m, uint32_t n) {
 
 static __global__ void set_pos_kernel(uint32_t* scalars, uint32_t pos) { scalars[1] = pos; }
 
+// all_logits (host, [n][vocab]): when set, every position is projected through the LM head in one
+// GEMM (project_logits_batched, cera/src/model/llama.rs:645-722) instead of the last one only.
 static cera_hip_status prefill_chunk(cera_hip_model* m, const uint32_t* tokens, uint32_t n, uint32_t start_pos,
-                                     bool want_logits) {
+                                     bool want_logits, float* all_logits = nullptr) {
     cera_hip_ctx* ctx = m->ctx;
     const cera_hip_config& c = m->cfg;
     hipStream_t s = ctx->stream;
@@ -213,6 +215,35 @@ static cera_hip_status prefill_chunk(cera_hip_model* m, const uint32_t* tokens, 
         CERA_TRY(gemm(L.down, m->pf_hidden, m->pf_hidden));
     }
     m->seq_len = start_pos + n;
+    if (all_logits) {
+        const cera_hip_dtensor* o = m->output ? m->output : m->embd;
+        const uint64_t rows = o->m;   // >= vocab; pad rows of a tied table are computed and dropped
+        if (m->pf_logits_cap < n) {
+            HIP_TRY(ctx, hipStreamSynchronize(s));
+            if (m->pf_logits) {
+                (void)hipFree(m->pf_logits);
+                m->bytes -= static_cast<uint64_t>(m->pf_logits_cap) * rows * 4;
+                m->pf_logits = nullptr;
+                m->pf_logits_cap = 0;
+            }
+            HIP_TRY(ctx, hipMalloc(reinterpret_cast<void**>(&m->pf_logits), static_cast<uint64_t>(m->pf_cap) * rows * 4));
+            m->pf_logits_cap = m->pf_cap;
+            m->bytes += static_cast<uint64_t>(m->pf_cap) * rows * 4;
+        }
+        // final norm of every row (+ Q8_0), then logits[n][rows] = normed . head^T
+        CERA_TRY(norm_rows(m->pf_hidden, m->output_norm, m->pf_normed));
+        CERA_TRY(cera_launch_gemm(ctx, o, m->pf_xs, m->pf_xq, m->pf_bsum, n, m->pf_logits, 1, rows, nullptr, 1.0f));
+        if (c.logit_scale != 1.0f) {
+            const uint64_t tot = static_cast<uint64_t>(n) * rows;
+            hipLaunchKernelGGL(scale_kernel, dim3(static_cast<uint32_t>((tot + 255) / 256)), dim3(256), 0, s, m->pf_logits,
+                               1.0f / c.logit_scale, static_cast<uint32_t>(tot));
+            HIP_TRY(ctx, hipGetLastError());
+        }
+        HIP_TRY(ctx, hipMemcpy2DAsync(all_logits, static_cast<size_t>(c.vocab) * 4, m->pf_logits, rows * 4,
+                                      static_cast<size_t>(c.vocab) * 4, n, hipMemcpyDeviceToHost, s));
+        HIP_TRY(ctx, hipStreamSynchronize(s));
+        return CERA_HIP_OK;
+    }
     if (want_logits) {
         // last token: final norm then the decode-style GEMV (project_logits)
         const float* last = m->pf_hidden + static_cast<uint64_t>(n - 1) * hs;
@@ -226,6 +257,31 @@ static cera_hip_status prefill_chunk(cera_hip_model* m, const uint32_t* tokens, 
             hipLaunchKernelGGL(scale_kernel, dim3((c.vocab + 255) / 256), dim3(256), 0, s, m->logits, 1.0f / c.logit_scale, c.vocab);
             HIP_TRY(ctx, hipGetLastError());
         }
+    }
+    return CERA_HIP_OK;
+}
+
+static bool prefill_batchable(const cera_hip_model* m) {
+    for (const LayerDev& L : m->layers)
+        for (const cera_hip_dtensor* w : {L.q, L.k, L.v, L.o, L.gate, L.up, L.down})
+            if (!cera_gemm_supports(w->dtype, w->k)) return false;
+    return true;
+}
+
+cera_hip_status cera_model_prefill_logits_all(cera_hip_model* m, const uint32_t* tokens, uint32_t n, uint32_t start_pos,
+                                              float* logits_all) {
+    const cera_hip_dtensor* head = m->output ? m->output : m->embd;
+    const uint64_t vocab = m->cfg.vocab;
+    // single token, or a weight / head type without an int8 GEMM: each forward returns that
+    // position's logits (the reference's fallback, cera/src/model/llama.rs:1712-1720)
+    if (n == 1 || !prefill_batchable(m) || !cera_gemm_supports(head->dtype, head->k)) {
+        for (uint32_t i = 0; i < n; ++i)
+            CERA_TRY(cera_model_decode_logits(m, tokens[i], start_pos + i, logits_all + i * vocab));
+        return CERA_HIP_OK;
+    }
+    for (uint32_t off = 0; off < n; off += PREFILL_CHUNK) {
+        uint32_t len = std::min(PREFILL_CHUNK, n - off);
+        CERA_TRY(prefill_chunk(m, tokens + off, len, start_pos + off, false, logits_all + off * vocab));
     }
     return CERA_HIP_OK;
 }

@@ -27,7 +27,7 @@ SYMBOLS = [
     "cera_hip_quantize_q8_0_dev", "cera_hip_gemv_q8_dev", "cera_hip_gemv_seq_dev", "cera_hip_attn_decode_dev",
     "cera_hip_gemm_dev",
     "cera_hip_model_create", "cera_hip_model_destroy", "cera_hip_forward", "cera_hip_forward_greedy",
-    "cera_hip_forward_prefill", "cera_hip_truncate_kv", "cera_hip_seq_len", "cera_hip_memory_bytes",
+    "cera_hip_forward_prefill", "cera_hip_forward_prefill_logits_all", "cera_hip_truncate_kv", "cera_hip_seq_len", "cera_hip_memory_bytes",
     "cera_hip_read_kv", "cera_hip_read_hidden",
 ]
 
@@ -113,6 +113,7 @@ def load_library() -> C.CDLL:
         "cera_hip_forward": (i32, [vp, u32, u32, vp]),
         "cera_hip_forward_greedy": (i32, [vp, u32, u32, C.POINTER(u32)]),
         "cera_hip_forward_prefill": (i32, [vp, vp, u32, u32, vp]),
+        "cera_hip_forward_prefill_logits_all": (i32, [vp, vp, u32, u32, vp]),
         "cera_hip_truncate_kv": (i32, [vp, u32]),
         "cera_hip_seq_len": (u32, [vp]), "cera_hip_memory_bytes": (u64, [vp]),
         "cera_hip_read_kv": (i32, [vp, u32, vp, vp]), "cera_hip_read_hidden": (i32, [vp, vp]),
@@ -388,6 +389,13 @@ class Model:
         logits = np.empty(self.vocab, np.float32)
         self.ctx.check(self.ctx.lib.cera_hip_forward_prefill(self.h, _p(t), t.size, start_pos, _p(logits)))
         return logits
+
+    def forward_prefill_logits_all(self, tokens, start_pos: int) -> np.ndarray:
+        t = np.ascontiguousarray(tokens, np.uint32)
+        out = np.empty((t.size, self.vocab), np.float32)
+        self.ctx.check(self.ctx.lib.cera_hip_forward_prefill_logits_all(self.h, _p(t) if t.size else None, t.size, start_pos,
+                                                                        _p(out)))
+        return out
 
     def truncate_kv(self, n: int):
         self.ctx.check(self.ctx.lib.cera_hip_truncate_kv(self.h, n))

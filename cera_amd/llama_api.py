@@ -13,7 +13,7 @@ from . import _build
 
 LLAMA_SYMBOLS = ["cera_llama_open", "cera_llama_close", "cera_llama_last_error", "cera_llama_get_config",
                  "cera_llama_seq_len", "cera_llama_gpu_memory_bytes", "cera_llama_forward",
-                 "cera_llama_forward_greedy", "cera_llama_forward_prefill", "cera_llama_forward_prefill_chunked",
+                 "cera_llama_forward_greedy", "cera_llama_forward_prefill", "cera_llama_forward_prefill_logits_all", "cera_llama_forward_prefill_chunked",
                  "cera_llama_set_cancel", "cera_llama_truncate_kv", "cera_llama_generate_greedy"]
 
 
@@ -43,6 +43,7 @@ def lib() -> C.CDLL:
             "cera_llama_forward": (C.c_int, [vp, u32, u64, vp]),
             "cera_llama_forward_greedy": (C.c_int, [vp, u32, u64, C.POINTER(u32)]),
             "cera_llama_forward_prefill": (C.c_int, [vp, vp, u64, u64, vp]),
+            "cera_llama_forward_prefill_logits_all": (C.c_int, [vp, vp, u64, u64, vp]),
             "cera_llama_forward_prefill_chunked": (C.c_int, [vp, vp, u64, u64, u64, C.POINTER(u64), vp]),
             "cera_llama_set_cancel": (None, [vp, C.c_int]),
             "cera_llama_truncate_kv": (C.c_int, [vp, u64]),
@@ -107,6 +108,13 @@ class HipLlama:
         out = np.empty(self.vocab, np.float32)
         self._check(lib().cera_llama_forward_prefill(self.h, t.ctypes.data if t.size else None, t.size, start_pos,
                                                      out.ctypes.data))
+        return out
+
+    def forward_prefill_logits_all(self, tokens, start_pos: int) -> np.ndarray:
+        t = np.ascontiguousarray(tokens, np.uint32)
+        out = np.empty((t.size, self.vocab), np.float32)
+        self._check(lib().cera_llama_forward_prefill_logits_all(self.h, t.ctypes.data if t.size else None, t.size,
+                                                                start_pos, out.ctypes.data))
         return out
 
     def forward_prefill_chunked(self, tokens, start_pos: int, ubatch: int):

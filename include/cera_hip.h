@@ -238,6 +238,12 @@ CERA_HIP_API cera_hip_status cera_hip_forward_greedy(cera_hip_model*, uint32_t t
  * start_pos, logits of the last one. */
 CERA_HIP_API cera_hip_status cera_hip_forward_prefill(cera_hip_model*, const uint32_t* tokens, uint32_t n,
                                                       uint32_t start_pos, float* last_logits);
+/* Model::forward_prefill_logits_all (cera/src/model/llama.rs:1655-1722; the projection is
+ * project_logits_batched, :645-722): like forward_prefill, but returns the logits of EVERY
+ * position, row-major [n][vocab] -- the verification primitive of speculative decoding
+ * (cera/src/model/mod.rs:221-249).  The LM head is read once for all n positions. */
+CERA_HIP_API cera_hip_status cera_hip_forward_prefill_logits_all(cera_hip_model*, const uint32_t* tokens, uint32_t n,
+                                                                 uint32_t start_pos, float* logits_all);
 /* Model::truncate_kv (cera/src/model/mod.rs:251-283). */
 CERA_HIP_API cera_hip_status cera_hip_truncate_kv(cera_hip_model*, uint32_t len);
 CERA_HIP_API uint32_t cera_hip_seq_len(const cera_hip_model*);

@@ -187,3 +187,59 @@ def test_cli_run_agrees_with_the_library(tiny_llama):
     gm.truncate_kv(0)
     toks, _, _ = gm.generate_greedy(prompt, 6)
     assert list(toks) == out
+
+
+def test_all_position_logits_match_per_token_forward(tiny_llama, orc, hip):
+    """cera/tests/spec_decode_logits.rs:72-115: [n * vocab] rows, KV appended for all n tokens,
+    every row against the per-token forward of the same position (cosine floor 0.99 there;
+    the tighter 0.999 and a near-tie argmax here)."""
+    path, cfg, gm, om = tiny_llama
+    toks = [int(t) for t in util.rng(21).integers(0, cfg["vocab"], 24)]
+    gm.truncate_kv(0); om.truncate(0)
+    _say("hip_llama: all-position logits, 24 tokens")
+    rows = gm.forward_prefill_logits_all(toks, 0)
+    assert rows.shape == (24, cfg["vocab"]) and gm.seq_len == 24
+    for i, t in enumerate(toks):
+        lo = om.forward(t, i)
+        err = _close(rows[i], lo, f"pos {i}")
+        if int(orc.argmax(rows[i])) != int(orc.argmax(lo)):
+            srt = np.sort(lo)
+            assert float(srt[-1] - srt[-2]) <= 2 * err, i
+    # the last row is what forward_prefill returns for the same prompt (GEMM vs GEMV head: float order only)
+    gm.truncate_kv(0)
+    last = gm.forward_prefill(toks, 0)
+    assert np.abs(rows[-1] - last).max() <= 1e-3 * util.rms(last)
+    # the cache it leaves continues like forward_prefill's
+    om_next, gm_next = om.forward(7, 24), gm.forward(7, 24)
+    _close(gm_next, om_next, "decode after prefill")
+    # a second call on top of the cache (start_pos > 0), and the single-token form
+    gm.truncate_kv(24); om.truncate(24)
+    more = [3, 99, 250, 17, 8]
+    rows2 = gm.forward_prefill_logits_all(more, 24)
+    for i, t in enumerate(more):
+        _close(rows2[i], om.forward(t, 24 + i), f"pos {24 + i}")
+    one = gm.forward_prefill_logits_all([11], 29)
+    _close(one[0], om.forward(11, 29), "single token")
+    assert gm.seq_len == om.seq_len == 30
+    with pytest.raises(llama_api.BackendError):
+        gm.forward_prefill_logits_all([1, 2], 5)  # start_pos must equal the cache length
+    with pytest.raises(llama_api.BackendError):
+        gm.forward_prefill_logits_all([], 30)
+
+
+def test_truncate_restores_the_cache(tiny_llama):
+    """cera/tests/spec_decode_logits.rs:130-178: prefill 0..8, truncate to 4, prefill 4..8 gives
+    the logits of prefill 0..4 then 4..8 (max |diff| < 1e-3 and the same argmax)."""
+    path, cfg, gm, om = tiny_llama
+    toks = [1, 150, 318, 297, 422, 298, 306, 62]
+    gm.truncate_kv(0)
+    gm.forward_prefill(toks[:4], 0)
+    ref = gm.forward_prefill(toks[4:], 4)
+    gm.truncate_kv(0)
+    gm.forward_prefill(toks, 0)
+    assert gm.seq_len == 8
+    gm.truncate_kv(4)
+    assert gm.seq_len == 4
+    got = gm.forward_prefill(toks[4:], 4)
+    assert gm.seq_len == 8
+    assert int(np.argmax(ref)) == int(np.argmax(got)) and float(np.abs(ref - got).max()) < 1e-3
