@@ -427,6 +427,7 @@ cera_hip_status cera_launch_attn(cera_hip_ctx* ctx, const float* q, const float*
         // positions per chunk: small chunks while the context is short (one memory round
         // trip per wavefront, many wavefronts), 64 once there is plenty of work
         S = last_len >= 16384 ? 8 : (last_len >= 4096 ? 4 : (last_len >= 1024 ? 2 : 1));
+        if (G == 8 && S == 8) S = 4;   // eight heads x 64 positions per chunk does not fit the register file
         uint32_t n_chunks = static_cast<uint32_t>((last_len + 8 * S - 1) / (8 * S));
         // parts (wavefronts) per (query, kv head): enough to fill the chip ~8 waves per CU
         // deep, but at least one chunk each and at most ATTN_MAX_PARTS

@@ -27,6 +27,7 @@
 
 #define ATTN_HD 128
 #define ATTN_MAX_PARTS 1024  // the merge kernel keeps one weight per part in LDS
+#define ATTN_MERGE_PF 4       // parts per lane group the merge kernel requests up front (x8 groups)
 
 struct AttnPart {  // per (part, query head): running max, sum and unnormalised output
     float m, l;
@@ -67,23 +68,17 @@ __device__ __forceinline__ void attn_rope16(float4 (&x)[4], const float* __restr
     }
 }
 
+// One wavefront's share of the keys: chunks of 8*S positions at t_begin, t_begin + t_step, ...
+// below t_end, for the G query heads of one kv head.  Returns the online-softmax state with
+// the eight position groups already folded: every lane holds its 16 columns of acc and the
+// wavefront-wide m and l.  `q` points at the first of the G heads; `write_new` says whether
+// this caller stores the new position's K/V row into the cache (NEWKV only).
 template <int G, int S, bool NEWKV>
-__global__ __launch_bounds__(256) void attn_decode_partial_kernel(
-    const float* __restrict__ q,       // [n_heads][128]
-    const float* __restrict__ kc,      // [n_kv][max_seq][128]
-    const float* __restrict__ vc,
-    uint32_t seq_len, uint32_t max_seq, float scale, uint32_t chunks_per_part, uint32_t n_parts,
-    uint32_t q_stride,                 // floats between consecutive queries (prefill batches queries on grid.z)
-    float* __restrict__ part_acc,      // [n_queries][n_kv][n_parts][G][128]
-    float* __restrict__ part_ml,       // [n_queries][n_kv][n_parts][G][2]
-    AttnNewKV nk) {
-    const uint32_t lane = threadIdx.x & 63;
-    const uint32_t part = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
-    const uint32_t kvh = blockIdx.y, qi = blockIdx.z;
-    if (part >= n_parts) return;
-    // causal prefill: query qi sits at position seq_len - 1 + qi and sees seq_len + qi keys
-    seq_len += qi;
-    q += static_cast<uint64_t>(qi) * q_stride;
+__device__ __forceinline__ void attn_decode_range(const float* __restrict__ q, const float* __restrict__ kbase,
+                                                  const float* __restrict__ vbase, uint32_t kvh, uint32_t max_seq,
+                                                  uint32_t seq_len, uint32_t t_begin, uint32_t t_end, uint32_t t_step,
+                                                  float scale, const AttnNewKV& nk, bool write_new, uint32_t lane,
+                                                  float4 (&acc)[G][4], float (&m)[G], float (&l)[G]) {
     const uint32_t j = lane & 7, pg = lane >> 3;  // float4 column group, position group
 
     // this lane's 16 q values for each of the G heads
@@ -92,15 +87,13 @@ __global__ __launch_bounds__(256) void attn_decode_partial_kernel(
     for (int h = 0; h < G; ++h)
 #pragma unroll
         for (int c = 0; c < 4; ++c)
-            qv[h][c] = reinterpret_cast<const float4*>(q + (kvh * G + h) * ATTN_HD)[j + 8 * c];
+            qv[h][c] = reinterpret_cast<const float4*>(q + h * ATTN_HD)[j + 8 * c];
     if (NEWKV) {
 #pragma unroll
         for (int h = 0; h < G; ++h) attn_rope16(qv[h], nk.rope_row, j, nk.rope_type);
     }
     const uint32_t new_pos = seq_len - 1;   // NEWKV: the position whose K/V are not in the cache yet
 
-    float4 acc[G][4];
-    float m[G], l[G];
 #pragma unroll
     for (int h = 0; h < G; ++h) {
         m[h] = -__builtin_inff();
@@ -109,24 +102,21 @@ __global__ __launch_bounds__(256) void attn_decode_partial_kernel(
         for (int c = 0; c < 4; ++c) acc[h][c] = make_float4(0.f, 0.f, 0.f, 0.f);
     }
 
-    const float* kbase = kc + static_cast<uint64_t>(kvh) * max_seq * ATTN_HD;
-    const float* vbase = vc + static_cast<uint64_t>(kvh) * max_seq * ATTN_HD;
     constexpr uint32_t CHUNK = 8 * S;
     constexpr bool PREFETCH_V = S <= 2;  // small chunks: V loads issued together with K
-    const uint32_t t_begin = part * chunks_per_part * CHUNK;
-    const uint32_t t_end = min(seq_len, t_begin + chunks_per_part * CHUNK);
-
-    for (uint32_t t0 = t_begin; t0 < t_end; t0 += CHUNK) {
+    // a lane past t_end re-reads the range's first position (from the cache, or the new row if
+    // that is the one not stored yet) and gets a dead score
+    for (uint32_t t0 = t_begin; t0 < t_end; t0 += t_step) {
         float4 vpre[PREFETCH_V ? S : 1][4];
         if (PREFETCH_V) {
 #pragma unroll
             for (int s = 0; s < S; ++s) {
-                uint32_t t = t0 + 8 * s + pg;
-                const float4* vp = reinterpret_cast<const float4*>(vbase + static_cast<uint64_t>(t < t_end ? t : t_begin) * ATTN_HD);
-                if (NEWKV && t == new_pos) vp = reinterpret_cast<const float4*>(nk.v_new + kvh * ATTN_HD);
+                const uint32_t t = t0 + 8 * s + pg, tt = t < t_end ? t : t_begin;
+                const float4* vp = reinterpret_cast<const float4*>(vbase + static_cast<uint64_t>(tt) * ATTN_HD);
+                if (NEWKV && tt == new_pos) vp = reinterpret_cast<const float4*>(nk.v_new + kvh * ATTN_HD);
 #pragma unroll
                 for (int c = 0; c < 4; ++c) vpre[s][c] = vp[j + 8 * c];
-                if (NEWKV && t == new_pos) {
+                if (NEWKV && t == new_pos && write_new) {
                     float4* dst = reinterpret_cast<float4*>(nk.vc_w + (static_cast<uint64_t>(kvh) * max_seq + t) * ATTN_HD);
 #pragma unroll
                     for (int c = 0; c < 4; ++c) dst[j + 8 * c] = vpre[s][c];
@@ -137,18 +127,21 @@ __global__ __launch_bounds__(256) void attn_decode_partial_kernel(
         float sc[G][S];
 #pragma unroll
         for (int s = 0; s < S; ++s) {
-            uint32_t t = t0 + 8 * s + pg;
-            bool live = t < t_end;
-            const float4* kp = reinterpret_cast<const float4*>(kbase + static_cast<uint64_t>(live ? t : t_begin) * ATTN_HD);
-            if (NEWKV && t == new_pos) kp = reinterpret_cast<const float4*>(nk.k_new + kvh * ATTN_HD);
+            const uint32_t t = t0 + 8 * s + pg;
+            const bool live = t < t_end;
+            const uint32_t tt = live ? t : t_begin;
+            const float4* kp = reinterpret_cast<const float4*>(kbase + static_cast<uint64_t>(tt) * ATTN_HD);
+            if (NEWKV && tt == new_pos) kp = reinterpret_cast<const float4*>(nk.k_new + kvh * ATTN_HD);
             float4 kv[4];
 #pragma unroll
             for (int c = 0; c < 4; ++c) kv[c] = kp[j + 8 * c];
             if (NEWKV && t == new_pos) {
                 attn_rope16(kv, nk.rope_row, j, nk.rope_type);
-                float4* dst = reinterpret_cast<float4*>(nk.kc_w + (static_cast<uint64_t>(kvh) * max_seq + t) * ATTN_HD);
+                if (write_new) {
+                    float4* dst = reinterpret_cast<float4*>(nk.kc_w + (static_cast<uint64_t>(kvh) * max_seq + t) * ATTN_HD);
 #pragma unroll
-                for (int c = 0; c < 4; ++c) dst[j + 8 * c] = kv[c];
+                    for (int c = 0; c < 4; ++c) dst[j + 8 * c] = kv[c];
+                }
             }
 #pragma unroll
             for (int h = 0; h < G; ++h) {
@@ -192,12 +185,12 @@ __global__ __launch_bounds__(256) void attn_decode_partial_kernel(
 #pragma unroll
                 for (int c = 0; c < 4; ++c) vv[c] = vpre[s][c];
             } else {
-                uint32_t t = t0 + 8 * s + pg;
-                const float4* vp = reinterpret_cast<const float4*>(vbase + static_cast<uint64_t>(t < t_end ? t : t_begin) * ATTN_HD);
-                if (NEWKV && t == new_pos) vp = reinterpret_cast<const float4*>(nk.v_new + kvh * ATTN_HD);
+                const uint32_t t = t0 + 8 * s + pg, tt = t < t_end ? t : t_begin;
+                const float4* vp = reinterpret_cast<const float4*>(vbase + static_cast<uint64_t>(tt) * ATTN_HD);
+                if (NEWKV && tt == new_pos) vp = reinterpret_cast<const float4*>(nk.v_new + kvh * ATTN_HD);
 #pragma unroll
                 for (int c = 0; c < 4; ++c) vv[c] = vp[j + 8 * c];
-                if (NEWKV && t == new_pos) {
+                if (NEWKV && t == new_pos && write_new) {
                     float4* dst = reinterpret_cast<float4*>(nk.vc_w + (static_cast<uint64_t>(kvh) * max_seq + t) * ATTN_HD);
 #pragma unroll
                     for (int c = 0; c < 4; ++c) dst[j + 8 * c] = vv[c];
@@ -236,6 +229,34 @@ __global__ __launch_bounds__(256) void attn_decode_partial_kernel(
             }
         }
     }
+}
+
+template <int G, int S, bool NEWKV>
+__global__ __launch_bounds__(256) void attn_decode_partial_kernel(
+    const float* __restrict__ q,       // [n_heads][128]
+    const float* __restrict__ kc,      // [n_kv][max_seq][128]
+    const float* __restrict__ vc,
+    uint32_t seq_len, uint32_t max_seq, float scale, uint32_t chunks_per_part, uint32_t n_parts,
+    uint32_t q_stride,                 // floats between consecutive queries (prefill batches queries on grid.z)
+    float* __restrict__ part_acc,      // [n_queries][n_kv][n_parts][G][128]
+    float* __restrict__ part_ml,       // [n_queries][n_kv][n_parts][G][2]
+    AttnNewKV nk) {
+    const uint32_t lane = threadIdx.x & 63;
+    const uint32_t part = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    const uint32_t kvh = blockIdx.y, qi = blockIdx.z;
+    if (part >= n_parts) return;
+    // causal prefill: query qi sits at position seq_len - 1 + qi and sees seq_len + qi keys
+    seq_len += qi;
+    q += static_cast<uint64_t>(qi) * q_stride + kvh * G * ATTN_HD;
+    const uint32_t j = lane & 7, pg = lane >> 3;
+    constexpr uint32_t CHUNK = 8 * S;
+    const uint32_t t_begin = part * chunks_per_part * CHUNK;
+    const uint32_t t_end = min(seq_len, t_begin + chunks_per_part * CHUNK);
+    float4 acc[G][4];
+    float m[G], l[G];
+    attn_decode_range<G, S, NEWKV>(q, kc + static_cast<uint64_t>(kvh) * max_seq * ATTN_HD,
+                                   vc + static_cast<uint64_t>(kvh) * max_seq * ATTN_HD, kvh, max_seq, seq_len, t_begin,
+                                   t_end, CHUNK, scale, nk, true, lane, acc, m, l);
     if (pg == 0) {
         uint64_t base = ((static_cast<uint64_t>(qi) * gridDim.y + kvh) * n_parts + part) * G;
 #pragma unroll
@@ -423,6 +444,14 @@ __global__ __launch_bounds__(256) void attn_decode_merge_kernel(const float* __r
     const uint32_t head = blockIdx.x, tid = threadIdx.x, c = tid & 31, grp = tid >> 5, wave = tid >> 6;
     const uint32_t kvh = head / G, hg = head % G, qi = blockIdx.y, n_kv = n_heads / G;
     const uint64_t pbase = (static_cast<uint64_t>(qi) * n_kv + kvh) * n_parts;
+    // the first ATTN_MERGE_PF parts of this group are requested before anything depends on them
+    float4 pre[ATTN_MERGE_PF];
+#pragma unroll
+    for (int i = 0; i < ATTN_MERGE_PF; ++i) {
+        const uint32_t p = grp + 8 * i;
+        pre[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (p < n_parts) pre[i] = reinterpret_cast<const float4*>(part_acc + ((pbase + p) * G + hg) * ATTN_HD)[c];
+    }
     float M = -__builtin_inff();
     for (uint32_t p = tid; p < n_parts; p += 256) M = fmaxf(M, part_ml[((pbase + p) * G + hg) * 2]);
     M = wave_max(M);
@@ -441,8 +470,15 @@ __global__ __launch_bounds__(256) void attn_decode_merge_kernel(const float* __r
     __syncthreads();
     L = (red[4] + red[5]) + (red[6] + red[7]);
     float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+    for (int i = 0; i < ATTN_MERGE_PF; ++i) {
+        const uint32_t p = grp + 8 * i;
+        const float w = p < n_parts ? wbuf[p] : 0.0f;
+        acc.x = fmaf(w, pre[i].x, acc.x); acc.y = fmaf(w, pre[i].y, acc.y);
+        acc.z = fmaf(w, pre[i].z, acc.z); acc.w = fmaf(w, pre[i].w, acc.w);
+    }
 #pragma unroll 2
-    for (uint32_t p = grp; p < n_parts; p += 8) {
+    for (uint32_t p = grp + 8 * ATTN_MERGE_PF; p < n_parts; p += 8) {
         const float w = wbuf[p];
         const float4 a = reinterpret_cast<const float4*>(part_acc + ((pbase + p) * G + hg) * ATTN_HD)[c];
         acc.x = fmaf(w, a.x, acc.x); acc.y = fmaf(w, a.y, acc.y);

@@ -166,6 +166,9 @@ extern "C" cera_hip_status cera_hip_model_create(cera_hip_ctx* ctx, const cera_h
             }
             CERA_TRY(dev_alloc_t(ctx, kv_elems, &D.kc, tot));
             CERA_TRY(dev_alloc_t(ctx, kv_elems, &D.vc, tot));
+            // lanes past the end of a key range re-read a cached row with weight 0: keep every row finite
+            HIP_TRY(ctx, hipMemsetAsync(D.kc, 0, kv_elems * sizeof(float), ctx->stream));
+            HIP_TRY(ctx, hipMemsetAsync(D.vc, 0, kv_elems * sizeof(float), ctx->stream));
         }
         std::vector<float> table;
         cera_build_rope_table(c.max_seq_len, c.head_dim, c.rope_theta, cfg->rope_freqs, table);

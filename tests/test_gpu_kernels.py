@@ -259,6 +259,21 @@ def test_attn_decode_split_invariance(hip, orc, splits):
     assert np.abs(out - ref).max() <= ATTN_TOL * util.rms(ref)
 
 
+@pytest.mark.parametrize("L", [1, 9, 127, 640, 1024, 1025])
+def test_attn_decode_auto_matches_explicit_split(hip, L):
+    """The automatic split (one 8- or 16-key chunk per wavefront at these lengths) and an explicit
+    5-way split give the same result."""
+    nh, nkv, hd = 32, 8, 128
+    _say(f"attn_decode auto vs 5 splits L={L}")
+    q = util.make_x(nh * hd, 75)
+    k = util.make_x(L * nkv * hd, 76 + L)
+    v = util.make_x(L * nkv * hd, 77 + L)
+    auto = hip.attn_decode(q, k, v, nh, nkv, hd, L, 0.09)
+    split = hip.attn_decode(q, k, v, nh, nkv, hd, L, 0.09, n_splits=5)
+    assert np.isfinite(auto).all()
+    assert np.abs(auto - split).max() <= 1e-5 * max(1.0, float(np.abs(split).max()))
+
+
 def test_attn_decode_peaked_softmax(hip, orc):
     """One dominant key (large logit) and large-magnitude scores: online softmax must not overflow."""
     nh, nkv, hd, L = 8, 2, 128, 300
