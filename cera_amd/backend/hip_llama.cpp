@@ -281,6 +281,53 @@ void HipLlamaModel::truncate_kv(InferenceState& state, size_t len) {
     state.seq_len = len;
 }
 
+// The trait defaults panic with unimplemented!(): a backend without device-resident state has
+// nothing to snapshot (cera/src/model/mod.rs:521-533).
+StateSnapshot Model::snapshot_state() { throw BackendError("snapshot_state not supported by this backend"); }
+void Model::restore_state(const StateSnapshot&) { throw BackendError("restore_state not supported by this backend"); }
+
+void HipLlamaModel::shift_kv(InferenceState& state, size_t n_keep, size_t shift) {
+    // the reference asserts these in all builds (cera/src/kv_cache.rs:1110-1116)
+    if (shift == 0) bail("shift_kv: shift must be > 0");
+    if (n_keep + shift > state.seq_len)
+        bail("shift range out of bounds: n_keep=" + std::to_string(n_keep) + " + shift=" + std::to_string(shift) +
+             " > seq_len=" + std::to_string(state.seq_len));
+    if (cera_hip_shift_kv(model_, static_cast<uint32_t>(n_keep), static_cast<uint32_t>(shift)) != CERA_HIP_OK)
+        device_panic("shift_kv");
+    state.seq_len = cera_hip_seq_len(model_);
+}
+
+StateSnapshot HipLlamaModel::snapshot_state() {
+    StateSnapshot snap;
+    snap.seq_len = cera_hip_seq_len(model_);
+    const size_t bytes = snap.seq_len * config_.n_kv_heads * config_.head_dim * sizeof(float);
+    snap.layers.resize(config_.n_layers);
+    for (size_t l = 0; l < config_.n_layers; ++l) {
+        snap.layers[l].k_data.resize(bytes);
+        snap.layers[l].v_data.resize(bytes);
+        if (bytes && cera_hip_read_kv(model_, static_cast<uint32_t>(l), reinterpret_cast<float*>(snap.layers[l].k_data.data()),
+                                      reinterpret_cast<float*>(snap.layers[l].v_data.data())) != CERA_HIP_OK)
+            device_panic("snapshot_state");
+    }
+    return snap;
+}
+
+void HipLlamaModel::restore_state(const StateSnapshot& snap) {
+    const size_t bytes = snap.seq_len * config_.n_kv_heads * config_.head_dim * sizeof(float);
+    if (snap.layers.size() != config_.n_layers) bail("restore_state: snapshot has " + std::to_string(snap.layers.size()) +
+                                                     " layers, model has " + std::to_string(config_.n_layers));
+    if (snap.seq_len > config_.max_seq_len) bail("restore_state: snapshot is longer than the context");
+    for (const LayerSnapshot& L : snap.layers)
+        if (L.k_data.size() != bytes || L.v_data.size() != bytes)
+            bail("restore_state: layer byte length does not match seq_len * kv_dim * 4 (an f16 or compressed snapshot?)");
+    for (size_t l = 0; l < config_.n_layers; ++l)
+        if (cera_hip_write_kv(model_, static_cast<uint32_t>(l), reinterpret_cast<const float*>(snap.layers[l].k_data.data()),
+                              reinterpret_cast<const float*>(snap.layers[l].v_data.data()),
+                              static_cast<uint32_t>(snap.seq_len)) != CERA_HIP_OK)
+            device_panic("restore_state");
+    if (cera_hip_set_seq_len(model_, static_cast<uint32_t>(snap.seq_len)) != CERA_HIP_OK) device_panic("restore_state");
+}
+
 uint64_t HipLlamaModel::gpu_memory_bytes() const { return cera_hip_memory_bytes(model_); }
 
 std::string HipLlamaModel::device_name() const {

@@ -57,6 +57,16 @@ struct InferenceState {
     size_t seq_len = 0;
 };
 
+// cera/src/kv_cache.rs:1382-1396: per attention layer the raw f32 K and V bytes of rows
+// [0, seq_len), time-major [pos][kv_dim] (LayerSnapshot::Attention).
+struct LayerSnapshot {
+    std::vector<uint8_t> k_data, v_data;
+};
+struct StateSnapshot {
+    std::vector<LayerSnapshot> layers;
+    size_t seq_len = 0;
+};
+
 // The subset of `trait Model` a text backend implements.
 class Model {
 public:
@@ -68,6 +78,11 @@ public:
     // logits of every position, row-major [n_tokens * vocab]; empty unless supports_all_logits()
     virtual std::vector<float> forward_prefill_logits_all(const uint32_t*, size_t, size_t, InferenceState&) { return {}; }
     virtual void truncate_kv(InferenceState& state, size_t len) = 0;
+    // n_keep context shift (cera/src/model/mod.rs:336-365): callers check supports_kv_shift() first
+    virtual void shift_kv(InferenceState&, size_t /*n_keep*/, size_t /*shift*/) {}
+    // prefix-cache snapshots (cera/src/model/mod.rs:507-533)
+    virtual struct StateSnapshot snapshot_state();
+    virtual void restore_state(const struct StateSnapshot&);
     // (tokens consumed, logits of the last processed chunk); chunks of `ubatch` (0 = one chunk),
     // `cancel` polled after each chunk.
     std::pair<size_t, std::optional<std::vector<float>>> forward_prefill_chunked(const uint32_t* tokens, size_t n_tokens,
@@ -100,6 +115,10 @@ public:
                                                   InferenceState& state) override;
     bool supports_all_logits() const override { return true; }
     void truncate_kv(InferenceState& state, size_t len) override;
+    bool supports_kv_shift() const override { return true; }
+    void shift_kv(InferenceState& state, size_t n_keep, size_t shift) override;
+    StateSnapshot snapshot_state() override;
+    void restore_state(const StateSnapshot& snapshot) override;
     const ModelConfig& config() const override { return config_; }
     uint64_t gpu_memory_bytes() const override;
 

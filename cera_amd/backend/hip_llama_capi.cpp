@@ -116,6 +116,39 @@ void cera_llama_set_cancel(cera_llama* h, int c) { h->cancel.store(c != 0); }
 int cera_llama_truncate_kv(cera_llama* h, uint64_t len) {
     return guarded(h, [&] { h->model->truncate_kv(h->state, len); });
 }
+int cera_llama_supports_kv_shift(const cera_llama* h) { return h && h->model->supports_kv_shift() ? 1 : 0; }
+int cera_llama_shift_kv(cera_llama* h, uint64_t n_keep, uint64_t shift) {
+    return guarded(h, [&] { h->model->shift_kv(h->state, n_keep, shift); });
+}
+struct cera_llama_snapshot {
+    cera::StateSnapshot snap;
+};
+cera_llama_snapshot* cera_llama_snapshot_state(cera_llama* h) {
+    cera_llama_snapshot* out = nullptr;
+    if (guarded(h, [&] {
+            out = new cera_llama_snapshot();
+            out->snap = h->model->snapshot_state();
+        }) != 0) {
+        delete out;
+        return nullptr;
+    }
+    return out;
+}
+uint64_t cera_llama_snapshot_seq_len(const cera_llama_snapshot* s) { return s ? s->snap.seq_len : 0; }
+uint64_t cera_llama_snapshot_bytes(const cera_llama_snapshot* s) {
+    uint64_t n = 0;
+    if (s)
+        for (const auto& L : s->snap.layers) n += L.k_data.size() + L.v_data.size();
+    return n;
+}
+int cera_llama_restore_state(cera_llama* h, const cera_llama_snapshot* s) {
+    if (!s) return -1;
+    return guarded(h, [&] {
+        h->model->restore_state(s->snap);
+        h->state.seq_len = s->snap.seq_len;
+    });
+}
+void cera_llama_snapshot_free(cera_llama_snapshot* s) { delete s; }
 
 int cera_llama_generate_greedy(cera_llama* h, const uint32_t* prompt, uint64_t n_prompt, uint64_t n_new,
                                uint64_t ubatch, uint32_t* out, double* prefill_s, double* decode_s) {

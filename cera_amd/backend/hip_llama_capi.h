@@ -41,6 +41,18 @@ CERA_LLAMA_API int cera_llama_forward_prefill_chunked(cera_llama*, const uint32_
                                                       float* last_logits);
 CERA_LLAMA_API void cera_llama_set_cancel(cera_llama*, int cancel);
 CERA_LLAMA_API int cera_llama_truncate_kv(cera_llama*, uint64_t len);
+/* Model::supports_kv_shift / shift_kv */
+CERA_LLAMA_API int cera_llama_supports_kv_shift(const cera_llama*);
+CERA_LLAMA_API int cera_llama_shift_kv(cera_llama*, uint64_t n_keep, uint64_t shift);
+/* Model::snapshot_state / restore_state.  A snapshot is an opaque handle owned by the caller
+ * (free it with cera_llama_snapshot_free); it can be restored into any model of the same shape.
+ * restore also sets the session's seq_len, as the trait method sets the model's. */
+typedef struct cera_llama_snapshot cera_llama_snapshot;
+CERA_LLAMA_API cera_llama_snapshot* cera_llama_snapshot_state(cera_llama*);
+CERA_LLAMA_API uint64_t cera_llama_snapshot_seq_len(const cera_llama_snapshot*);
+CERA_LLAMA_API uint64_t cera_llama_snapshot_bytes(const cera_llama_snapshot*);
+CERA_LLAMA_API int cera_llama_restore_state(cera_llama*, const cera_llama_snapshot*);
+CERA_LLAMA_API void cera_llama_snapshot_free(cera_llama_snapshot*);
 /* Greedy generation as Session drives it for temperature 0: prefill the prompt in `ubatch`
  * chunks, take argmax of its last logits as the first new token, then n_new-1
  * forward_greedy steps.  out_tokens[n_new]; timings in seconds (nullable). */

@@ -227,6 +227,55 @@ static __global__ void rope_kv_kernel(float* __restrict__ q, float* __restrict__
     }
 }
 
+// n_keep context shift (cera/src/kv_cache.rs:1091-1310): rows [src_row, src_row + n_rows) of every
+// kv head move to [dst_row, ...) of `dst` (the cache itself when the two ranges do not overlap,
+// a staging buffer otherwise), and K rows are rotated on the way by the constant delta rotation
+// R(-shift) -- `delta_cs` holds its head_dim/2 (cos, sin) pairs, built on the host with the
+// reference's recurrence (cera/src/backend/cpu.rs:5065-5086 NEOX, :5145-5180 NORM); null = plain
+// copy (V, and the copy back from staging).  head_dim = 128; 16 threads per row, each owning
+// float4 j and float4 j + 16.  grid = (ceil(n_rows * 16 / 256), n_kv_heads).
+static __global__ __launch_bounds__(256) void kv_shift_kernel(const float* __restrict__ src, float* __restrict__ dst,
+                                                              uint32_t src_row, uint32_t dst_row, uint32_t n_rows,
+                                                              uint64_t src_head_stride, uint64_t dst_head_stride,
+                                                              const float* __restrict__ delta_cs, uint32_t rope_type) {
+    const uint32_t t = (blockIdx.x * 256 + threadIdx.x) >> 4, j = threadIdx.x & 15;
+    if (t >= n_rows) return;
+    const float4* sp = reinterpret_cast<const float4*>(src + blockIdx.y * src_head_stride + static_cast<uint64_t>(src_row + t) * 128);
+    float4* dp = reinterpret_cast<float4*>(dst + blockIdx.y * dst_head_stride + static_cast<uint64_t>(dst_row + t) * 128);
+    float4 a = sp[j], b = sp[j + 16];
+    if (delta_cs) {
+        const float4* cs = reinterpret_cast<const float4*>(delta_cs);
+        if (rope_type == 1) {   // NORM: pairs (2i, 2i+1): pair i uses cs[i]; float4 j holds pairs 2j, 2j+1
+            const float4 ca = cs[j], cb = cs[j + 16];
+            float4 r;
+            r.x = __fsub_rn(__fmul_rn(a.x, ca.x), __fmul_rn(a.y, ca.y));
+            r.y = __fadd_rn(__fmul_rn(a.x, ca.y), __fmul_rn(a.y, ca.x));
+            r.z = __fsub_rn(__fmul_rn(a.z, ca.z), __fmul_rn(a.w, ca.w));
+            r.w = __fadd_rn(__fmul_rn(a.z, ca.w), __fmul_rn(a.w, ca.z));
+            a = r;
+            r.x = __fsub_rn(__fmul_rn(b.x, cb.x), __fmul_rn(b.y, cb.y));
+            r.y = __fadd_rn(__fmul_rn(b.x, cb.y), __fmul_rn(b.y, cb.x));
+            r.z = __fsub_rn(__fmul_rn(b.z, cb.z), __fmul_rn(b.w, cb.w));
+            r.w = __fadd_rn(__fmul_rn(b.z, cb.w), __fmul_rn(b.w, cb.z));
+            b = r;
+        } else {                // NEOX: pairs (i, i + 64): element 4j + e of a with the same of b, cs[4j + e]
+            const float4 c01 = cs[2 * j], c23 = cs[2 * j + 1];
+            float4 ra, rb;
+            ra.x = __fsub_rn(__fmul_rn(a.x, c01.x), __fmul_rn(b.x, c01.y));
+            rb.x = __fadd_rn(__fmul_rn(a.x, c01.y), __fmul_rn(b.x, c01.x));
+            ra.y = __fsub_rn(__fmul_rn(a.y, c01.z), __fmul_rn(b.y, c01.w));
+            rb.y = __fadd_rn(__fmul_rn(a.y, c01.w), __fmul_rn(b.y, c01.z));
+            ra.z = __fsub_rn(__fmul_rn(a.z, c23.x), __fmul_rn(b.z, c23.y));
+            rb.z = __fadd_rn(__fmul_rn(a.z, c23.y), __fmul_rn(b.z, c23.x));
+            ra.w = __fsub_rn(__fmul_rn(a.w, c23.z), __fmul_rn(b.w, c23.w));
+            rb.w = __fadd_rn(__fmul_rn(a.w, c23.w), __fmul_rn(b.w, c23.z));
+            a = ra; b = rb;
+        }
+    }
+    dp[j] = a;
+    dp[j + 16] = b;
+}
+
 // out = a + b (cera/src/backend/cpu.rs:5223-5228), optional scale on b first.
 static __global__ void add_kernel(const float* __restrict__ a, const float* __restrict__ b, float bscale, uint32_t n,
                            float* __restrict__ out) {

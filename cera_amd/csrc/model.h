@@ -24,6 +24,8 @@ struct cera_hip_model {
     float* output_norm = nullptr;
     std::vector<LayerDev> layers;
     float* rope_table = nullptr;  // [max_seq_len][head_dim/2] (cos, sin)
+    std::vector<float> rope_ff;   // host copy of the per-pair frequency factors (empty: none)
+    float* shift_cs = nullptr;    // [head_dim/2] (cos, sin) of the last context shift's delta rotation
     // single-token activations
     float *hidden = nullptr, *normed = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *attn_out = nullptr,
           *proj = nullptr, *act = nullptr, *up = nullptr, *xs = nullptr, *logits = nullptr;

@@ -170,6 +170,9 @@ extern "C" cera_hip_status cera_hip_model_create(cera_hip_ctx* ctx, const cera_h
             HIP_TRY(ctx, hipMemsetAsync(D.kc, 0, kv_elems * sizeof(float), ctx->stream));
             HIP_TRY(ctx, hipMemsetAsync(D.vc, 0, kv_elems * sizeof(float), ctx->stream));
         }
+        if (cfg->rope_freqs) m->rope_ff.assign(cfg->rope_freqs, cfg->rope_freqs + c.head_dim / 2);
+        CERA_TRY(dev_alloc_t(ctx, c.head_dim, &tmp, tot));
+        m->shift_cs = tmp; m->owned.push_back(tmp);
         std::vector<float> table;
         cera_build_rope_table(c.max_seq_len, c.head_dim, c.rope_theta, cfg->rope_freqs, table);
         CERA_TRY(upload_f32(ctx, table.data(), table.size(), &tmp, tot));
@@ -217,6 +220,101 @@ extern "C" cera_hip_status cera_hip_truncate_kv(cera_hip_model* m, uint32_t len)
     if (!m) return CERA_HIP_ERR_ARGUMENT;
     std::lock_guard<std::mutex> lk(m->infer_lock);
     if (len < m->seq_len) m->seq_len = len;  // rows past len are simply overwritten later
+    return CERA_HIP_OK;
+}
+
+// LlamaModel::shift_kv -> InferenceState::shift_kv_with_rope (cera/src/model/llama.rs:1727-1738,
+// cera/src/kv_cache.rs:1091-1310): drop cache cells [n_keep, n_keep + shift), move the tail down
+// and re-rotate its K rows by R(-shift) so their encoded position matches their new index.
+extern "C" cera_hip_status cera_hip_shift_kv(cera_hip_model* m, uint32_t n_keep, uint32_t shift) {
+    if (!m) return CERA_HIP_ERR_ARGUMENT;
+    std::lock_guard<std::mutex> lk(m->infer_lock);
+    cera_hip_ctx* ctx = m->ctx;
+    const cera_hip_config& c = m->cfg;
+    if (shift == 0) return cera_fail(ctx, CERA_HIP_ERR_ARGUMENT, "shift_kv: shift must be > 0");
+    if (static_cast<uint64_t>(n_keep) + shift > m->seq_len)
+        return cera_fail(ctx, CERA_HIP_ERR_POSITION, "shift_kv: n_keep=" + std::to_string(n_keep) + " + shift=" +
+                                                         std::to_string(shift) + " > seq_len=" + std::to_string(m->seq_len));
+    if (c.head_dim != 128) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "shift_kv: head_dim must be 128");
+    const uint32_t new_len = m->seq_len - shift, tail = new_len - n_keep, src_row = n_keep + shift;
+    if (tail) {
+        // delta rotation: theta_0 = -(shift) as f32, the forward pass's recurrence and factors
+        std::vector<float> row;
+        {
+            const uint32_t half = c.head_dim / 2;
+            row.resize(2 * half);
+            const float theta_scale = powf(c.rope_theta, -2.0f / static_cast<float>(c.head_dim));
+            float theta = static_cast<float>(-static_cast<int32_t>(shift));
+            for (uint32_t i = 0; i < half; ++i) {
+                // NEOX never divides by frequency factors (cera/src/backend/cpu.rs:5065-5086)
+                const float ang = (c.rope_type == 1 && !m->rope_ff.empty()) ? theta / m->rope_ff[i] : theta;
+                row[2 * i] = cosf(ang);
+                row[2 * i + 1] = sinf(ang);
+                theta *= theta_scale;
+            }
+        }
+        CERA_TRY(cera_hip_upload(ctx, m->shift_cs, row.data(), row.size() * 4));
+        const uint64_t head_stride = static_cast<uint64_t>(c.max_seq_len) * c.head_dim;
+        const dim3 grid((tail * 16 + 255) / 256, c.n_kv_heads), block(256);
+        const bool overlap = tail > shift;   // source and destination rows intersect: go through staging
+        float* stage = nullptr;
+        const uint64_t stage_stride = static_cast<uint64_t>(tail) * c.head_dim;
+        if (overlap) {
+            void* p = nullptr;
+            CERA_TRY(cera_scratch(ctx, 5, stage_stride * c.n_kv_heads * sizeof(float), &p));
+            stage = static_cast<float*>(p);
+        }
+        for (LayerDev& L : m->layers) {
+            for (int is_v = 0; is_v < 2; ++is_v) {
+                float* cache = is_v ? L.vc : L.kc;
+                const float* cs = is_v ? nullptr : m->shift_cs;
+                if (!overlap) {
+                    hipLaunchKernelGGL(kv_shift_kernel, grid, block, 0, ctx->stream, cache, cache, src_row, n_keep, tail,
+                                       head_stride, head_stride, cs, c.rope_type);
+                } else {
+                    hipLaunchKernelGGL(kv_shift_kernel, grid, block, 0, ctx->stream, cache, stage, src_row, 0u, tail,
+                                       head_stride, stage_stride, cs, c.rope_type);
+                    hipLaunchKernelGGL(kv_shift_kernel, grid, block, 0, ctx->stream, stage, cache, 0u, n_keep, tail,
+                                       stage_stride, head_stride, static_cast<const float*>(nullptr), c.rope_type);
+                }
+            }
+        }
+        HIP_TRY(ctx, hipGetLastError());
+        HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    }
+    m->seq_len = new_len;
+    return CERA_HIP_OK;
+}
+
+// Prefix-cache snapshots (Model::snapshot_state / restore_state, cera/src/model/mod.rs:507-533;
+// layer layout LayerSnapshot::Attention, cera/src/kv_cache.rs:1382-1396): a layer's K and V as
+// time-major [n_pos][kv_dim] f32, the CPU state's own layout.  cera_hip_read_kv is the snapshot
+// side; this is the restore side.  Call it for every layer, then cera_hip_set_seq_len.
+extern "C" cera_hip_status cera_hip_write_kv(cera_hip_model* m, uint32_t layer, const float* k, const float* v,
+                                             uint32_t n_pos) {
+    if (!m || (n_pos && (!k || !v)) || layer >= m->cfg.n_layers) return CERA_HIP_ERR_ARGUMENT;
+    std::lock_guard<std::mutex> lk(m->infer_lock);
+    const cera_hip_config& c = m->cfg;
+    if (n_pos > c.max_seq_len) return cera_fail(m->ctx, CERA_HIP_ERR_POSITION, "write_kv: more positions than max_seq_len");
+    const uint64_t per_head = static_cast<uint64_t>(c.max_seq_len) * c.head_dim;
+    const uint64_t kv_dim = static_cast<uint64_t>(c.n_kv_heads) * c.head_dim;
+    std::vector<float> hk(static_cast<uint64_t>(n_pos) * c.head_dim), hv(hk.size());
+    for (uint32_t h = 0; h < c.n_kv_heads && n_pos; ++h) {
+        for (uint32_t t = 0; t < n_pos; ++t) {
+            std::memcpy(hk.data() + static_cast<uint64_t>(t) * c.head_dim, k + t * kv_dim + h * c.head_dim, c.head_dim * 4);
+            std::memcpy(hv.data() + static_cast<uint64_t>(t) * c.head_dim, v + t * kv_dim + h * c.head_dim, c.head_dim * 4);
+        }
+        CERA_TRY(cera_hip_upload(m->ctx, m->layers[layer].kc + h * per_head, hk.data(), hk.size() * 4));
+        CERA_TRY(cera_hip_upload(m->ctx, m->layers[layer].vc + h * per_head, hv.data(), hv.size() * 4));
+    }
+    return CERA_HIP_OK;
+}
+
+extern "C" cera_hip_status cera_hip_set_seq_len(cera_hip_model* m, uint32_t len) {
+    if (!m) return CERA_HIP_ERR_ARGUMENT;
+    std::lock_guard<std::mutex> lk(m->infer_lock);
+    if (len > m->cfg.max_seq_len) return cera_fail(m->ctx, CERA_HIP_ERR_POSITION, "set_seq_len: beyond max_seq_len");
+    m->seq_len = len;
     return CERA_HIP_OK;
 }
 

@@ -27,7 +27,7 @@ SYMBOLS = [
     "cera_hip_quantize_q8_0_dev", "cera_hip_gemv_q8_dev", "cera_hip_gemv_seq_dev", "cera_hip_attn_decode_dev",
     "cera_hip_gemm_dev",
     "cera_hip_model_create", "cera_hip_model_destroy", "cera_hip_forward", "cera_hip_forward_greedy",
-    "cera_hip_forward_prefill", "cera_hip_forward_prefill_logits_all", "cera_hip_truncate_kv", "cera_hip_seq_len", "cera_hip_memory_bytes",
+    "cera_hip_forward_prefill", "cera_hip_forward_prefill_logits_all", "cera_hip_truncate_kv", "cera_hip_shift_kv", "cera_hip_write_kv", "cera_hip_set_seq_len", "cera_hip_seq_len", "cera_hip_memory_bytes",
     "cera_hip_read_kv", "cera_hip_read_hidden",
 ]
 
@@ -115,6 +115,9 @@ def load_library() -> C.CDLL:
         "cera_hip_forward_prefill": (i32, [vp, vp, u32, u32, vp]),
         "cera_hip_forward_prefill_logits_all": (i32, [vp, vp, u32, u32, vp]),
         "cera_hip_truncate_kv": (i32, [vp, u32]),
+        "cera_hip_shift_kv": (i32, [vp, u32, u32]),
+        "cera_hip_write_kv": (i32, [vp, u32, vp, vp, u32]),
+        "cera_hip_set_seq_len": (i32, [vp, u32]),
         "cera_hip_seq_len": (u32, [vp]), "cera_hip_memory_bytes": (u64, [vp]),
         "cera_hip_read_kv": (i32, [vp, u32, vp, vp]), "cera_hip_read_hidden": (i32, [vp, vp]),
     }
@@ -396,6 +399,19 @@ class Model:
         self.ctx.check(self.ctx.lib.cera_hip_forward_prefill_logits_all(self.h, _p(t) if t.size else None, t.size, start_pos,
                                                                         _p(out)))
         return out
+
+    def shift_kv(self, n_keep: int, shift: int):
+        self.ctx.check(self.ctx.lib.cera_hip_shift_kv(self.h, n_keep, shift))
+
+    def write_kv(self, layer: int, k: np.ndarray, v: np.ndarray):
+        k = np.ascontiguousarray(k, np.float32); v = np.ascontiguousarray(v, np.float32)
+        kv_dim = self.cfg["n_kv_heads"] * self.cfg["head_dim"]
+        assert k.size == v.size and k.size % kv_dim == 0
+        self.ctx.check(self.ctx.lib.cera_hip_write_kv(self.h, layer, _p(k) if k.size else None,
+                                                      _p(v) if v.size else None, k.size // kv_dim))
+
+    def set_seq_len(self, n: int):
+        self.ctx.check(self.ctx.lib.cera_hip_set_seq_len(self.h, n))
 
     def truncate_kv(self, n: int):
         self.ctx.check(self.ctx.lib.cera_hip_truncate_kv(self.h, n))

@@ -14,7 +14,9 @@ from . import _build
 LLAMA_SYMBOLS = ["cera_llama_open", "cera_llama_close", "cera_llama_last_error", "cera_llama_get_config",
                  "cera_llama_seq_len", "cera_llama_gpu_memory_bytes", "cera_llama_forward",
                  "cera_llama_forward_greedy", "cera_llama_forward_prefill", "cera_llama_forward_prefill_logits_all", "cera_llama_forward_prefill_chunked",
-                 "cera_llama_set_cancel", "cera_llama_truncate_kv", "cera_llama_generate_greedy"]
+                 "cera_llama_set_cancel", "cera_llama_truncate_kv", "cera_llama_supports_kv_shift", "cera_llama_shift_kv",
+                 "cera_llama_snapshot_state", "cera_llama_snapshot_seq_len", "cera_llama_snapshot_bytes",
+                 "cera_llama_restore_state", "cera_llama_snapshot_free", "cera_llama_generate_greedy"]
 
 
 class LlamaConfigC(C.Structure):
@@ -47,6 +49,13 @@ def lib() -> C.CDLL:
             "cera_llama_forward_prefill_chunked": (C.c_int, [vp, vp, u64, u64, u64, C.POINTER(u64), vp]),
             "cera_llama_set_cancel": (None, [vp, C.c_int]),
             "cera_llama_truncate_kv": (C.c_int, [vp, u64]),
+            "cera_llama_supports_kv_shift": (C.c_int, [vp]),
+            "cera_llama_shift_kv": (C.c_int, [vp, u64, u64]),
+            "cera_llama_snapshot_state": (vp, [vp]),
+            "cera_llama_snapshot_seq_len": (u64, [vp]),
+            "cera_llama_snapshot_bytes": (u64, [vp]),
+            "cera_llama_restore_state": (C.c_int, [vp, vp]),
+            "cera_llama_snapshot_free": (None, [vp]),
             "cera_llama_generate_greedy": (C.c_int, [vp, vp, u64, u64, u64, vp, C.POINTER(C.c_double),
                                                      C.POINTER(C.c_double)]),
         }
@@ -59,6 +68,29 @@ def lib() -> C.CDLL:
 
 class BackendError(RuntimeError):
     pass
+
+
+class Snapshot:
+    """Opaque KV snapshot (Model::snapshot_state); restorable into any model of the same shape."""
+
+    def __init__(self, handle):
+        self.h = handle
+
+    @property
+    def seq_len(self) -> int:
+        return lib().cera_llama_snapshot_seq_len(self.h)
+
+    @property
+    def nbytes(self) -> int:
+        return lib().cera_llama_snapshot_bytes(self.h)
+
+    def close(self):
+        if self.h:
+            lib().cera_llama_snapshot_free(self.h)
+            self.h = None
+
+    def __del__(self):
+        self.close()
 
 
 class HipLlama:
@@ -130,6 +162,22 @@ class HipLlama:
 
     def truncate_kv(self, n: int):
         self._check(lib().cera_llama_truncate_kv(self.h, n))
+
+    @property
+    def supports_kv_shift(self) -> bool:
+        return bool(lib().cera_llama_supports_kv_shift(self.h))
+
+    def shift_kv(self, n_keep: int, shift: int):
+        self._check(lib().cera_llama_shift_kv(self.h, n_keep, shift))
+
+    def snapshot_state(self) -> "Snapshot":
+        s = lib().cera_llama_snapshot_state(self.h)
+        if not s:
+            raise BackendError(lib().cera_llama_last_error(self.h).decode())
+        return Snapshot(s)
+
+    def restore_state(self, snap: "Snapshot"):
+        self._check(lib().cera_llama_restore_state(self.h, snap.h))
 
     def generate_greedy(self, prompt, n_new: int, ubatch: int = 512):
         p = np.ascontiguousarray(prompt, np.uint32)

@@ -249,9 +249,23 @@ CERA_HIP_API cera_hip_status cera_hip_truncate_kv(cera_hip_model*, uint32_t len)
 CERA_HIP_API uint32_t cera_hip_seq_len(const cera_hip_model*);
 /* Model::gpu_memory_bytes. */
 CERA_HIP_API uint64_t cera_hip_memory_bytes(const cera_hip_model*);
-/* Test hook: copies layer `layer`'s K and V cache rows [0, seq_len) to host in
- * the reference's time-major [pos][kv_dim] order. */
+/* Model::shift_kv for a RoPE model (cera/src/model/llama.rs:1727-1738 ->
+ * InferenceState::shift_kv_with_rope, cera/src/kv_cache.rs:1091-1310): drops cache cells
+ * [n_keep, n_keep + shift), moves the tail down and re-rotates its K rows by R(-shift)
+ * (cera/src/backend/cpu.rs:5065-5086, 5145-5180); V rows only move.  seq_len -= shift.
+ * shift == 0 -> CERA_HIP_ERR_ARGUMENT, n_keep + shift > seq_len -> CERA_HIP_ERR_POSITION
+ * (the reference asserts both). */
+CERA_HIP_API cera_hip_status cera_hip_shift_kv(cera_hip_model*, uint32_t n_keep, uint32_t shift);
+/* Model::snapshot_state, one layer (cera/src/model/mod.rs:507-524; LayerSnapshot::Attention,
+ * cera/src/kv_cache.rs:1382-1396): K and V cache rows [0, seq_len) to host in the reference's
+ * time-major [pos][kv_dim] f32 order.  Also the parity tests' view of the cache. */
 CERA_HIP_API cera_hip_status cera_hip_read_kv(cera_hip_model*, uint32_t layer, float* k_out, float* v_out);
+/* Model::restore_state, one layer (cera/src/model/mod.rs:526-533): the inverse of
+ * cera_hip_read_kv for rows [0, n_pos).  After the last layer call cera_hip_set_seq_len(n_pos),
+ * which "sets internal seq_len" as the trait method does. */
+CERA_HIP_API cera_hip_status cera_hip_write_kv(cera_hip_model*, uint32_t layer, const float* k, const float* v,
+                                               uint32_t n_pos);
+CERA_HIP_API cera_hip_status cera_hip_set_seq_len(cera_hip_model*, uint32_t len);
 /* Test hook: final normed hidden state of the last forward (f32[hidden]). */
 CERA_HIP_API cera_hip_status cera_hip_read_hidden(cera_hip_model*, float* hidden_out);
 

@@ -97,6 +97,10 @@ def lib() -> C.CDLL:
         "orc_llama_forward_prefill_batched": (i32, [vp, vp, u32, u32, vp, vp]),
         "orc_flash_attention_head": (None, [vp, vp, vp, vp, u64, u64, u64, u32, f32, u64]),
         "orc_llama_kcache": (vp, [vp, u32]), "orc_llama_vcache": (vp, [vp, u32]),
+        "orc_rope_delta_head": (None, [vp, i32, u32, f32, u32, vp]),
+        "orc_llama_shift_kv": (i32, [vp, u32, u32]),
+        "orc_llama_restore_kv": (i32, [vp, u32, vp, vp, u32]),
+        "orc_llama_set_seq_len": (None, [vp, u32]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(L, name, None)
@@ -236,6 +240,15 @@ def rope(q: np.ndarray, k: np.ndarray, pos: int, n_heads: int, n_kv_heads: int, 
     return q2, k2
 
 
+def rope_delta_head(head: np.ndarray, delta_pos: int, head_dim: int, base: float, norm: bool = True,
+                    freq_factors: np.ndarray | None = None) -> np.ndarray:
+    """apply_rope_delta_to_head / apply_rope_norm_delta_to_head on one head."""
+    h = np.array(head, np.float32, copy=True).reshape(-1)
+    ff = None if freq_factors is None else np.ascontiguousarray(freq_factors, np.float32)
+    lib().orc_rope_delta_head(_p(h), delta_pos, head_dim, base, 1 if norm else 0, None if ff is None else _p(ff))
+    return h
+
+
 def argmax(logits: np.ndarray) -> int:
     l = np.ascontiguousarray(logits, np.float32)
     return int(lib().orc_argmax(_p(l) if l.size else None, l.size))
@@ -353,6 +366,17 @@ class Llama:
 
     def truncate(self, n: int):
         lib().orc_llama_truncate(self.h, n)
+
+    def shift_kv(self, n_keep: int, shift: int) -> int:
+        """0, or -1 where the reference asserts."""
+        return lib().orc_llama_shift_kv(self.h, n_keep, shift)
+
+    def restore(self, layers_kv, n_pos: int):
+        """layers_kv: per layer (k, v) time-major [n_pos][kv_dim]; sets seq_len."""
+        for i, (k, v) in enumerate(layers_kv):
+            k = np.ascontiguousarray(k, np.float32); v = np.ascontiguousarray(v, np.float32)
+            assert lib().orc_llama_restore_kv(self.h, i, _p(k), _p(v), n_pos) == 0
+        lib().orc_llama_set_seq_len(self.h, n_pos)
 
     def forward(self, token: int, pos: int, want_hidden: bool = False):
         logits = np.empty(self.vocab, np.float32)

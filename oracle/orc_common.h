@@ -109,6 +109,8 @@ ORC_API void  orc_rope_norm(float* q, float* k, uint64_t pos, uint32_t n_heads,
                             const float* freq_factors);
 ORC_API void  orc_rope_neox(float* q, float* k, uint64_t pos, uint32_t n_heads,
                             uint32_t n_kv_heads, uint32_t head_dim, float freq_base);
+ORC_API void  orc_rope_delta_head(float* head, int32_t delta_pos, uint32_t head_dim, float freq_base,
+                                  uint32_t rope_type /*0 neox, 1 norm*/, const float* freq_factors);
 ORC_API uint32_t orc_argmax(const float* logits, uint64_t n);
 
 // ---- attention ------------------------------------------------------------

@@ -52,6 +52,41 @@ void orc_llama_truncate(OrcLlama* m, uint32_t len) {
     m->seq_len = len;
 }
 
+// LlamaModel::shift_kv (llama.rs:1727-1738) -> InferenceState::shift_kv_with_rope, f32 path
+// (kv_cache.rs:1091-1160, 1233-1310): drain rows [n_keep, n_keep + shift) of every layer's K and
+// V, then delta-rotate the K heads of the rows now at [n_keep, new_seq_len) by -shift.
+// Returns -1 where the reference asserts (shift == 0, range past seq_len).
+int orc_llama_shift_kv(OrcLlama* m, uint32_t n_keep, uint32_t shift) {
+    const OrcLlamaConfig& c = m->cfg;
+    if (shift == 0 || uint64_t(n_keep) + shift > m->seq_len) return -1;
+    const uint64_t kv_dim = uint64_t(c.n_kv_heads) * c.head_dim;
+    const uint32_t new_len = m->seq_len - shift;
+    for (uint32_t l = 0; l < c.n_layers; ++l) {
+        auto& kc = m->kc[l];
+        auto& vc = m->vc[l];
+        if (kc.empty() && vc.empty()) continue;
+        kc.erase(kc.begin() + n_keep * kv_dim, kc.begin() + (uint64_t(n_keep) + shift) * kv_dim);
+        vc.erase(vc.begin() + n_keep * kv_dim, vc.begin() + (uint64_t(n_keep) + shift) * kv_dim);
+        for (uint32_t t = n_keep; t < new_len; ++t)
+            for (uint32_t h = 0; h < c.n_kv_heads; ++h)
+                orc_rope_delta_head(kc.data() + t * kv_dim + h * c.head_dim, -int32_t(shift), c.head_dim, c.rope_theta,
+                                    c.rope_type, c.rope_freqs);
+    }
+    m->seq_len = new_len;
+    return 0;
+}
+
+// Prefix-cache restore (InferenceState::restore, the CPU twin of Model::restore_state,
+// mod.rs:526-533): replace every layer's K/V with n_pos rows and set seq_len.
+int orc_llama_restore_kv(OrcLlama* m, uint32_t layer, const float* k, const float* v, uint32_t n_pos) {
+    if (layer >= m->cfg.n_layers) return -1;
+    const uint64_t n = uint64_t(n_pos) * m->cfg.n_kv_heads * m->cfg.head_dim;
+    m->kc[layer].assign(k, k + n);
+    m->vc[layer].assign(v, v + n);
+    return 0;
+}
+void orc_llama_set_seq_len(OrcLlama* m, uint32_t len) { m->seq_len = len; }
+
 // llama.rs:1585-1605 + :468-597.  Writes vocab logits; optionally the final
 // normed hidden state (for intermediate-value checks).
 int orc_llama_forward(OrcLlama* m, uint32_t token, uint32_t pos, float* logits, float* hidden_out) {

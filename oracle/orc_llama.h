@@ -42,5 +42,8 @@ ORC_API int      orc_llama_forward_prefill_per_token(OrcLlama*, const uint32_t* 
 // receives the per-token final-normed hidden states [n][hidden].
 ORC_API int      orc_llama_forward_prefill_batched(OrcLlama*, const uint32_t* tokens, uint32_t n,
                                                    uint32_t start_pos, float* last_logits, float* all_hidden);
+ORC_API int      orc_llama_shift_kv(OrcLlama*, uint32_t n_keep, uint32_t shift);
+ORC_API int      orc_llama_restore_kv(OrcLlama*, uint32_t layer, const float* k, const float* v, uint32_t n_pos);
+ORC_API void     orc_llama_set_seq_len(OrcLlama*, uint32_t len);
 ORC_API const float* orc_llama_kcache(const OrcLlama*, uint32_t layer);
 ORC_API const float* orc_llama_vcache(const OrcLlama*, uint32_t layer);

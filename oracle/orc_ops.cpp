@@ -123,6 +123,16 @@ void orc_rope_neox(float* q, float* k, uint64_t pos, uint32_t n_heads, uint32_t 
     for (uint32_t h = 0; h < n_kv_heads; ++h) rope_neox_head(k + h * head_dim, float(pos), head_dim, freq_base);
 }
 
+// cpu.rs:5065-5086 (apply_rope_delta_to_head, NEOX) and :5145-5153
+// (apply_rope_norm_delta_to_head): compose a further rotation of delta_pos onto an
+// already-rotated head; the same recurrences with theta_start = delta_pos as f32.
+// NEOX takes no frequency factors.
+void orc_rope_delta_head(float* head, int32_t delta_pos, uint32_t head_dim, float freq_base, uint32_t rope_type,
+                         const float* freq_factors) {
+    if (rope_type == 0) rope_neox_head(head, float(delta_pos), head_dim, freq_base);
+    else rope_norm_head(head, float(delta_pos), head_dim, freq_base, freq_factors);
+}
+
 // sampler.rs:20-30 -- strict >, lowest index on ties, NaN never wins.
 uint32_t orc_argmax(const float* logits, uint64_t n) {
     uint32_t best_i = 0;

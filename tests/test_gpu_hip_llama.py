@@ -243,3 +243,39 @@ def test_truncate_restores_the_cache(tiny_llama):
     got = gm.forward_prefill(toks[4:], 4)
     assert gm.seq_len == 8
     assert int(np.argmax(ref)) == int(np.argmax(got)) and float(np.abs(ref - got).max()) < 1e-3
+
+
+def test_shift_and_snapshot_through_the_model_layer(tiny_llama, tmp_path):
+    """Model::shift_kv keeps the session's seq_len in step; snapshot_state / restore_state
+    (cera/src/model/mod.rs:507-533) bring a second model to the same state: the next logits
+    are bit-identical to the snapshotted model's."""
+    path, cfg, gm, om = tiny_llama
+    assert gm.supports_kv_shift
+    toks = [int(t) for t in util.rng(41).integers(0, cfg["vocab"], 30)]
+    gm.truncate_kv(0); om.truncate(0)
+    gm.forward_prefill(toks, 0)
+    om.forward_prefill_batched(toks, 0)
+    snap = gm.snapshot_state()
+    assert snap.seq_len == 30
+    assert snap.nbytes == cfg["n_layers"] * 2 * 30 * cfg["n_kv_heads"] * cfg["head_dim"] * 4
+    other = llama_api.HipLlama(path, context_size=64)
+    other.restore_state(snap)
+    assert other.seq_len == 30
+    a, b = gm.forward(9, 30), other.forward(9, 30)
+    assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+    # restoring rewinds: the snapshot predates token 9
+    gm.restore_state(snap)
+    assert gm.seq_len == 30
+    c = gm.forward(9, 30)
+    assert np.array_equal(a.view(np.uint32), c.view(np.uint32))
+    other.close(); snap.close()
+    # shift through the Model layer, against the oracle
+    gm.truncate_kv(30); om.truncate(30)
+    gm.shift_kv(2, 10); om.shift_kv(2, 10)
+    assert gm.seq_len == om.seq_len == 20
+    _close(gm.forward(5, 20), om.forward(5, 20), "after shift")
+    with pytest.raises(llama_api.BackendError):
+        gm.shift_kv(20, 5)
+    with pytest.raises(llama_api.BackendError):
+        gm.shift_kv(1, 0)
+    assert gm.seq_len == 21

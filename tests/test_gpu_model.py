@@ -147,3 +147,75 @@ def test_model_create_refuses_bad_shapes(hip):
     with pytest.raises(hip_api.HipError) as e:
         hip_api.Model(hip, cfg, bad)
     assert e.value.status == 3
+
+
+# ---- n_keep context shift, snapshots ---------------------------------------------------
+@pytest.mark.parametrize("rope_type,seq_len,n_keep,shift", [(1, 24, 5, 7), (0, 24, 5, 7), (1, 60, 4, 10), (0, 40, 0, 30),
+                                                             (1, 33, 32, 1), (1, 20, 3, 17)])
+def test_shift_kv_matches_oracle_bitwise(hip, orc, rope_type, seq_len, n_keep, shift):
+    """The reference's shift fixture (cera/tests/n_keep_shift.rs:95-245) loaded into both caches:
+    the delta rotation is the same correctly rounded f32 arithmetic on the same host-built
+    cos/sin row, so K and V after the shift are bit-identical to the oracle's.  Covers tails
+    longer than the shift (rows move through staging), shorter, and empty."""
+    from test_oracle_kv_shift import rope_filled_cache
+    cfg = dict(synth.TINY, rope_type=rope_type)
+    weights = synth.make_llama(cfg, seed=5, sigma=0.05)
+    _say(f"shift_kv rope_type={rope_type} seq_len={seq_len} n_keep={n_keep} shift={shift}")
+    gm = hip_api.Model(hip, cfg, weights)
+    om = orc.Llama(cfg, weights)
+    layers, _ = rope_filled_cache(orc, cfg, seq_len, rope_type == 1)
+    om.restore(layers, seq_len)
+    for i, (k, v) in enumerate(layers):
+        gm.write_kv(i, k, v)
+    gm.set_seq_len(seq_len)
+    kg, vg = gm.read_kv(1)
+    assert np.array_equal(kg, layers[1][0]) and np.array_equal(vg, layers[1][1])   # write/read round trip
+    gm.shift_kv(n_keep, shift)
+    assert om.shift_kv(n_keep, shift) == 0
+    assert gm.seq_len == om.seq_len == seq_len - shift
+    for layer in range(cfg["n_layers"]):
+        kg, vg = gm.read_kv(layer)
+        ko, vo = om.kv(layer)
+        assert np.array_equal(kg.view(np.uint32), ko.view(np.uint32)), layer
+        assert np.array_equal(vg.view(np.uint32), vo.view(np.uint32)), layer
+    gm.close(); om.close()
+
+
+def test_shift_kv_with_frequency_factors_and_errors(hip, orc):
+    from test_oracle_kv_shift import rope_filled_cache
+    ff = (1.0 + 0.05 * np.arange(64)).astype(np.float32)
+    cfg = dict(synth.TINY)
+    weights = dict(synth.make_llama(cfg, seed=5, sigma=0.05))
+    weights["rope_freqs.weight"] = ff
+    gm = hip_api.Model(hip, cfg, weights)
+    om = orc.Llama(cfg, weights)
+    layers, _ = rope_filled_cache(orc, cfg, 20, True, ff)
+    om.restore(layers, 20)
+    for i, (k, v) in enumerate(layers):
+        gm.write_kv(i, k, v)
+    gm.set_seq_len(20)
+    with pytest.raises(hip_api.HipError) as e:
+        gm.shift_kv(3, 0)
+    assert e.value.status == 6  # CERA_HIP_ERR_ARGUMENT
+    with pytest.raises(hip_api.HipError):
+        gm.shift_kv(15, 6)
+    assert gm.seq_len == 20
+    gm.shift_kv(2, 6); om.shift_kv(2, 6)
+    kg, _ = gm.read_kv(0)
+    ko, _ = om.kv(0)
+    assert np.array_equal(kg.view(np.uint32), ko.view(np.uint32))
+    gm.close(); om.close()
+
+
+def test_decode_continues_after_a_shift(tiny):
+    """Prefill, shift the context, keep decoding: logits track the oracle doing the same."""
+    cfg, weights, gm, om = tiny
+    gm.truncate_kv(0); om.truncate(0)
+    toks = [int(t) for t in util.rng(31).integers(0, cfg["vocab"], 40)]
+    gm.forward_prefill(toks, 0)
+    om.forward_prefill_batched(toks, 0)
+    gm.shift_kv(4, 12); om.shift_kv(4, 12)
+    assert gm.seq_len == om.seq_len == 28
+    for i, t in enumerate([7, 300, 12, 99]):
+        lg, lo = gm.forward(t, 28 + i), om.forward(t, 28 + i)
+        assert _cos(lg, lo) > 0.999, i
