@@ -1,6 +1,8 @@
 // HipLlamaModel over the C-ABI of cera_hip.h.  Reference lines: see hip_llama.h.
 #include "hip_llama.h"
 
+#include "cera_host.h"
+
 #include <algorithm>
 #include <cmath>
 #include <cstring>
@@ -297,34 +299,79 @@ void HipLlamaModel::shift_kv(InferenceState& state, size_t n_keep, size_t shift)
     state.seq_len = cera_hip_seq_len(model_);
 }
 
+void HipLlamaModel::configure_kv_compression(KvCompression mode) {
+    // a second call with a different mode is CeraError::KvCompressionConflict in the reference
+    if (cera_hip_configure_kv(model_, mode == KvCompression::F16 ? CERA_HIP_KV_F16 : CERA_HIP_KV_F32) != CERA_HIP_OK)
+        bail(std::string("configure_kv_compression: ") + cera_hip_last_error(ctx_));
+}
+KvCompression HipLlamaModel::kv_compression() const {
+    return cera_hip_kv_type(model_) == CERA_HIP_KV_F16 ? KvCompression::F16 : KvCompression::None;
+}
+
+// the integer-only converters of the host library (the reference's, cera/src/quant.rs:48-164)
+static uint16_t half_bits(float v) { return cera_f32_to_f16(v); }
+static float half_value(uint16_t b) { return cera_f16_to_f32(b); }
+
 StateSnapshot HipLlamaModel::snapshot_state() {
     StateSnapshot snap;
     snap.seq_len = cera_hip_seq_len(model_);
-    const size_t bytes = snap.seq_len * config_.n_kv_heads * config_.head_dim * sizeof(float);
+    const bool f16 = kv_compression() == KvCompression::F16;
+    const size_t elems = snap.seq_len * config_.n_kv_heads * config_.head_dim;
+    std::vector<float> k(elems), v(elems);
     snap.layers.resize(config_.n_layers);
     for (size_t l = 0; l < config_.n_layers; ++l) {
-        snap.layers[l].k_data.resize(bytes);
-        snap.layers[l].v_data.resize(bytes);
-        if (bytes && cera_hip_read_kv(model_, static_cast<uint32_t>(l), reinterpret_cast<float*>(snap.layers[l].k_data.data()),
-                                      reinterpret_cast<float*>(snap.layers[l].v_data.data())) != CERA_HIP_OK)
+        LayerSnapshot& L = snap.layers[l];
+        L.f16 = f16;
+        if (elems && cera_hip_read_kv(model_, static_cast<uint32_t>(l), k.data(), v.data()) != CERA_HIP_OK)
             device_panic("snapshot_state");
+        if (!f16) {
+            L.k_data.assign(reinterpret_cast<uint8_t*>(k.data()), reinterpret_cast<uint8_t*>(k.data() + elems));
+            L.v_data.assign(reinterpret_cast<uint8_t*>(v.data()), reinterpret_cast<uint8_t*>(v.data() + elems));
+        } else {  // the cache's own half bits: read_kv widened them exactly
+            L.k_data.resize(elems * 2);
+            L.v_data.resize(elems * 2);
+            for (size_t i = 0; i < elems; ++i) {
+                const uint16_t kb = half_bits(k[i]), vb = half_bits(v[i]);
+                std::memcpy(L.k_data.data() + 2 * i, &kb, 2);
+                std::memcpy(L.v_data.data() + 2 * i, &vb, 2);
+            }
+        }
     }
     return snap;
 }
 
 void HipLlamaModel::restore_state(const StateSnapshot& snap) {
-    const size_t bytes = snap.seq_len * config_.n_kv_heads * config_.head_dim * sizeof(float);
+    const bool f16 = kv_compression() == KvCompression::F16;
+    const size_t elems = snap.seq_len * config_.n_kv_heads * config_.head_dim;
+    const size_t bytes = elems * (f16 ? 2 : 4);
     if (snap.layers.size() != config_.n_layers) bail("restore_state: snapshot has " + std::to_string(snap.layers.size()) +
                                                      " layers, model has " + std::to_string(config_.n_layers));
     if (snap.seq_len > config_.max_seq_len) bail("restore_state: snapshot is longer than the context");
-    for (const LayerSnapshot& L : snap.layers)
+    for (const LayerSnapshot& L : snap.layers) {
+        // the cross-mode gate: an f16 snapshot never loads into an f32 cache or the reverse
+        if (L.f16 != f16) bail("restore_state: snapshot and model disagree on the KV cache element type");
         if (L.k_data.size() != bytes || L.v_data.size() != bytes)
-            bail("restore_state: layer byte length does not match seq_len * kv_dim * 4 (an f16 or compressed snapshot?)");
-    for (size_t l = 0; l < config_.n_layers; ++l)
-        if (cera_hip_write_kv(model_, static_cast<uint32_t>(l), reinterpret_cast<const float*>(snap.layers[l].k_data.data()),
-                              reinterpret_cast<const float*>(snap.layers[l].v_data.data()),
-                              static_cast<uint32_t>(snap.seq_len)) != CERA_HIP_OK)
+            bail("restore_state: layer byte length does not match seq_len * kv_dim * element size");
+    }
+    std::vector<float> k(elems), v(elems);
+    for (size_t l = 0; l < config_.n_layers; ++l) {
+        const LayerSnapshot& L = snap.layers[l];
+        if (!f16) {
+            std::memcpy(k.data(), L.k_data.data(), bytes);
+            std::memcpy(v.data(), L.v_data.data(), bytes);
+        } else {
+            for (size_t i = 0; i < elems; ++i) {
+                uint16_t kb, vb;
+                std::memcpy(&kb, L.k_data.data() + 2 * i, 2);
+                std::memcpy(&vb, L.v_data.data() + 2 * i, 2);
+                k[i] = half_value(kb);
+                v[i] = half_value(vb);
+            }
+        }
+        if (cera_hip_write_kv(model_, static_cast<uint32_t>(l), k.data(), v.data(), static_cast<uint32_t>(snap.seq_len)) !=
+            CERA_HIP_OK)
             device_panic("restore_state");
+    }
     if (cera_hip_set_seq_len(model_, static_cast<uint32_t>(snap.seq_len)) != CERA_HIP_OK) device_panic("restore_state");
 }
 

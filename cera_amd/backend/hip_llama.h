@@ -59,13 +59,19 @@ struct InferenceState {
 
 // cera/src/kv_cache.rs:1382-1396: per attention layer the raw f32 K and V bytes of rows
 // [0, seq_len), time-major [pos][kv_dim] (LayerSnapshot::Attention).
+// With an f16 cache the bytes are the raw little-endian half bits (LayerSnapshot::AttentionF16,
+// cera/src/kv_cache.rs:1411-1421); `f16` is the variant tag restore checks.
 struct LayerSnapshot {
     std::vector<uint8_t> k_data, v_data;
+    bool f16 = false;
 };
 struct StateSnapshot {
     std::vector<LayerSnapshot> layers;
     size_t seq_len = 0;
 };
+
+// cera/src/kv_cache.rs:88-110, the modes a dense transformer on this backend honours
+enum class KvCompression { None = 0, F16 = 1 };
 
 // The subset of `trait Model` a text backend implements.
 class Model {
@@ -97,6 +103,8 @@ public:
     virtual bool supports_hidden_states() const { return false; }
     virtual bool turboquant_supported() const { return false; }
     virtual bool f16_kv_supported() const { return false; }
+    // cera/src/model/mod.rs:557-592: called before any forward pass; first call wins
+    virtual void configure_kv_compression(KvCompression) {}
 };
 
 class HipLlamaModel final : public Model {
@@ -116,6 +124,9 @@ public:
     bool supports_all_logits() const override { return true; }
     void truncate_kv(InferenceState& state, size_t len) override;
     bool supports_kv_shift() const override { return true; }
+    bool f16_kv_supported() const override { return true; }
+    void configure_kv_compression(KvCompression mode) override;
+    KvCompression kv_compression() const;
     void shift_kv(InferenceState& state, size_t n_keep, size_t shift) override;
     StateSnapshot snapshot_state() override;
     void restore_state(const StateSnapshot& snapshot) override;

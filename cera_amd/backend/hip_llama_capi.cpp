@@ -116,6 +116,13 @@ void cera_llama_set_cancel(cera_llama* h, int c) { h->cancel.store(c != 0); }
 int cera_llama_truncate_kv(cera_llama* h, uint64_t len) {
     return guarded(h, [&] { h->model->truncate_kv(h->state, len); });
 }
+int cera_llama_f16_kv_supported(const cera_llama* h) { return h && h->model->f16_kv_supported() ? 1 : 0; }
+int cera_llama_configure_kv_compression(cera_llama* h, int kind) {
+    return guarded(h, [&] {
+        if (kind != 0 && kind != 1) throw cera::BackendError("configure_kv_compression: kind must be 0 (none) or 1 (f16)");
+        h->model->configure_kv_compression(kind == 1 ? cera::KvCompression::F16 : cera::KvCompression::None);
+    });
+}
 int cera_llama_supports_kv_shift(const cera_llama* h) { return h && h->model->supports_kv_shift() ? 1 : 0; }
 int cera_llama_shift_kv(cera_llama* h, uint64_t n_keep, uint64_t shift) {
     return guarded(h, [&] { h->model->shift_kv(h->state, n_keep, shift); });

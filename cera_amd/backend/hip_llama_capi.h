@@ -41,6 +41,10 @@ CERA_LLAMA_API int cera_llama_forward_prefill_chunked(cera_llama*, const uint32_
                                                       float* last_logits);
 CERA_LLAMA_API void cera_llama_set_cancel(cera_llama*, int cancel);
 CERA_LLAMA_API int cera_llama_truncate_kv(cera_llama*, uint64_t len);
+/* Model::f16_kv_supported / configure_kv_compression: kind 0 = KvCompression::None (f32 cache),
+ * 1 = KvCompression::F16.  Before the first forward pass; the first call wins. */
+CERA_LLAMA_API int cera_llama_f16_kv_supported(const cera_llama*);
+CERA_LLAMA_API int cera_llama_configure_kv_compression(cera_llama*, int kind);
 /* Model::supports_kv_shift / shift_kv */
 CERA_LLAMA_API int cera_llama_supports_kv_shift(const cera_llama*);
 CERA_LLAMA_API int cera_llama_shift_kv(cera_llama*, uint64_t n_keep, uint64_t shift);

@@ -400,10 +400,61 @@ cera_hip_status cera_launch_gemv_q5k_f32(cera_hip_ctx* ctx, const cera_hip_dtens
     return CERA_HIP_OK;
 }
 
-cera_hip_status cera_launch_attn(cera_hip_ctx* ctx, const float* q, const float* kc, const float* vc,
+struct AttnLaunch {
+    const float* q;
+    uint32_t seq_len, max_seq;
+    float scale;
+    uint32_t n_heads, n_kv_heads, n_queries, q_stride, G, S, n_parts, part_keys, chunks_per_part;
+    bool batch, fused_new_kv;
+    AttnNewKV nk;
+};
+
+template <int G, typename KV>
+static void attn_launch_decode_g(cera_hip_ctx* ctx, const AttnLaunch& a, const KV* kc, const KV* vc) {
+    const dim3 grid((a.n_parts + 3) / 4, a.n_kv_heads, a.n_queries), block(256);
+#define ATTN_LAUNCH_S(SS)                                                                                            \
+    do {                                                                                                             \
+        if (a.fused_new_kv)                                                                                          \
+            hipLaunchKernelGGL((attn_decode_partial_kernel<G, SS, true, KV>), grid, block, 0, ctx->stream, a.q, kc,  \
+                               vc, a.seq_len, a.max_seq, a.scale, a.chunks_per_part, a.n_parts, a.q_stride,          \
+                               ctx->attn_acc, ctx->attn_ml, a.nk);                                                   \
+        else                                                                                                         \
+            hipLaunchKernelGGL((attn_decode_partial_kernel<G, SS, false, KV>), grid, block, 0, ctx->stream, a.q, kc, \
+                               vc, a.seq_len, a.max_seq, a.scale, a.chunks_per_part, a.n_parts, a.q_stride,          \
+                               ctx->attn_acc, ctx->attn_ml, a.nk);                                                   \
+    } while (0)
+    switch (a.S) {
+        case 1: ATTN_LAUNCH_S(1); break;
+        case 2: ATTN_LAUNCH_S(2); break;
+        case 4: ATTN_LAUNCH_S(4); break;
+        default: ATTN_LAUNCH_S(8); break;
+    }
+#undef ATTN_LAUNCH_S
+}
+
+template <typename KV>
+static void attn_launch_partials(cera_hip_ctx* ctx, const AttnLaunch& a, const KV* kc, const KV* vc) {
+    if (a.batch) {
+        // heaviest query blocks (most visible keys) first
+        const dim3 pgrid((a.n_queries + 31) / 32, a.n_heads, a.n_parts);
+        hipLaunchKernelGGL(attn_prefill_partial_kernel<KV>, pgrid, dim3(64), 0, ctx->stream, a.q, kc, vc, a.seq_len,
+                           a.n_queries, a.max_seq, a.scale, a.part_keys, a.n_parts, a.q_stride, a.G, ctx->attn_acc,
+                           ctx->attn_ml);
+        return;
+    }
+    switch (a.G) {
+        case 1: attn_launch_decode_g<1, KV>(ctx, a, kc, vc); break;
+        case 2: attn_launch_decode_g<2, KV>(ctx, a, kc, vc); break;
+        case 4: attn_launch_decode_g<4, KV>(ctx, a, kc, vc); break;
+        default: attn_launch_decode_g<8, KV>(ctx, a, kc, vc); break;
+    }
+}
+
+cera_hip_status cera_launch_attn(cera_hip_ctx* ctx, const float* q, const void* kc, const void* vc,
                                  uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, uint64_t seq_len,
                                  uint64_t max_seq, float scale, uint32_t n_splits, uint32_t n_queries, float* out,
-                                 float* out_scales, int8_t* out_quants, float* out_bsum, const AttnNewKV* new_kv) {
+                                 float* out_scales, int8_t* out_quants, float* out_bsum, const AttnNewKV* new_kv,
+                                 bool kv_f16) {
     if (head_dim != ATTN_HD) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "attention: head_dim must be 128");
     if (n_kv_heads == 0 || n_heads % n_kv_heads) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "attention: n_heads must be a multiple of n_kv_heads");
     uint32_t G = n_heads / n_kv_heads;
@@ -452,40 +503,10 @@ cera_hip_status cera_launch_attn(cera_hip_ctx* ctx, const float* q, const float*
         HIP_TRY(ctx, hipMalloc(reinterpret_cast<void**>(&ctx->attn_ml), ml_bytes));
         ctx->attn_ml_bytes = ml_bytes;
     }
-    uint32_t sl = static_cast<uint32_t>(seq_len), ms = static_cast<uint32_t>(max_seq);
-    uint32_t q_stride = n_heads * head_dim;
-    if (batch) {
-        // heaviest query blocks (most visible keys) first
-        dim3 pgrid((n_queries + 31) / 32, n_heads, n_parts);
-        hipLaunchKernelGGL(attn_prefill_partial_kernel, pgrid, dim3(64), 0, ctx->stream, q, kc, vc, sl, n_queries, ms, scale,
-                           part_keys, n_parts, q_stride, G, ctx->attn_acc, ctx->attn_ml);
-    } else {
-    dim3 grid((n_parts + 3) / 4, n_kv_heads, n_queries);
-#define ATTN_LAUNCH_S(GG, SS)                                                                                         \
-    do {                                                                                                              \
-        if (new_kv)                                                                                                   \
-            hipLaunchKernelGGL((attn_decode_partial_kernel<GG, SS, true>), grid, dim3(256), 0, ctx->stream, q, kc, vc, \
-                               sl, ms, scale, chunks_per_part, n_parts, q_stride, ctx->attn_acc, ctx->attn_ml, nk);   \
-        else                                                                                                          \
-            hipLaunchKernelGGL((attn_decode_partial_kernel<GG, SS, false>), grid, dim3(256), 0, ctx->stream, q, kc, vc, \
-                               sl, ms, scale, chunks_per_part, n_parts, q_stride, ctx->attn_acc, ctx->attn_ml, nk);   \
-    } while (0)
-#define ATTN_LAUNCH(GG)                              \
-    switch (S) {                                     \
-        case 1: ATTN_LAUNCH_S(GG, 1); break;         \
-        case 2: ATTN_LAUNCH_S(GG, 2); break;         \
-        case 4: ATTN_LAUNCH_S(GG, 4); break;         \
-        default: ATTN_LAUNCH_S(GG, 8); break;        \
-    }
-    switch (G) {
-        case 1: ATTN_LAUNCH(1); break;
-        case 2: ATTN_LAUNCH(2); break;
-        case 4: ATTN_LAUNCH(4); break;
-        default: ATTN_LAUNCH(8); break;
-    }
-#undef ATTN_LAUNCH_S
-#undef ATTN_LAUNCH
-    }
+    AttnLaunch a{q, static_cast<uint32_t>(seq_len), static_cast<uint32_t>(max_seq), scale, n_heads, n_kv_heads, n_queries,
+                 n_heads * head_dim, G, S, n_parts, part_keys, chunks_per_part, batch, new_kv != nullptr, nk};
+    if (kv_f16) attn_launch_partials<kv_half>(ctx, a, static_cast<const kv_half*>(kc), static_cast<const kv_half*>(vc));
+    else attn_launch_partials<float>(ctx, a, static_cast<const float*>(kc), static_cast<const float*>(vc));
     HIP_TRY(ctx, hipGetLastError());
     dim3 mgrid(n_heads, n_queries);
     if (out_quants)
@@ -499,12 +520,12 @@ cera_hip_status cera_launch_attn(cera_hip_ctx* ctx, const float* q, const float*
     return CERA_HIP_OK;
 }
 
-cera_hip_status cera_launch_attn_decode(cera_hip_ctx* ctx, const float* q, const float* kc, const float* vc,
+cera_hip_status cera_launch_attn_decode(cera_hip_ctx* ctx, const float* q, const void* kc, const void* vc,
                                         uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, uint64_t seq_len,
                                         uint64_t max_seq, float scale, uint32_t n_splits, float* out,
-                                        float* out_scales, int8_t* out_quants, const AttnNewKV* new_kv) {
+                                        float* out_scales, int8_t* out_quants, const AttnNewKV* new_kv, bool kv_f16) {
     return cera_launch_attn(ctx, q, kc, vc, n_heads, n_kv_heads, head_dim, seq_len, max_seq, scale, n_splits, 1, out,
-                            out_scales, out_quants, nullptr, new_kv);
+                            out_scales, out_quants, nullptr, new_kv, kv_f16);
 }
 
 // ---------------------------------------------------------------------------
@@ -597,49 +618,29 @@ cera_hip_status cera_hip_attn_decode_dev(cera_hip_ctx* ctx, const float* q, cons
     return cera_launch_attn_decode(ctx, q, k, v, n_heads, n_kv_heads, head_dim, seq_len, max_seq, scale, n_splits, out, nullptr, nullptr);
 }
 
-cera_hip_status cera_hip_attn_decode(cera_hip_ctx* ctx, const float* q, const float* k, const float* v,
-                                     uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, uint64_t seq_len,
-                                     float scale, uint32_t n_splits, float* out) {
-    if (!ctx || !q || !k || !v || !out) return CERA_HIP_ERR_ARGUMENT;
-    if (seq_len == 0 || n_kv_heads == 0 || head_dim == 0) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "attn_decode: empty input");
-    const uint64_t kv_dim = static_cast<uint64_t>(n_kv_heads) * head_dim;
-    const uint64_t kv_bytes = seq_len * kv_dim * 4;
-    // time-major [pos][kv_dim] (reference layout) -> head-major [kv_head][pos][head_dim]
-    std::vector<float> hk(seq_len * kv_dim), hv(seq_len * kv_dim);
-    for (uint64_t t = 0; t < seq_len; ++t)
-        for (uint32_t h = 0; h < n_kv_heads; ++h) {
-            std::memcpy(&hk[(h * seq_len + t) * head_dim], k + t * kv_dim + h * head_dim, head_dim * 4);
-            std::memcpy(&hv[(h * seq_len + t) * head_dim], v + t * kv_dim + h * head_dim, head_dim * 4);
-        }
-    void *dq, *dk, *dv, *dout;
-    CERA_TRY(cera_scratch(ctx, 0, static_cast<uint64_t>(n_heads) * head_dim * 4, &dq));
-    CERA_TRY(cera_scratch(ctx, 5, kv_bytes, &dk));
-    CERA_TRY(cera_scratch(ctx, 6, kv_bytes, &dv));
-    CERA_TRY(cera_scratch(ctx, 3, static_cast<uint64_t>(n_heads) * head_dim * 4, &dout));
-    CERA_TRY(cera_hip_upload(ctx, dq, q, static_cast<uint64_t>(n_heads) * head_dim * 4));
-    CERA_TRY(cera_hip_upload(ctx, dk, hk.data(), kv_bytes));
-    CERA_TRY(cera_hip_upload(ctx, dv, hv.data(), kv_bytes));
-    CERA_TRY(cera_launch_attn_decode(ctx, static_cast<float*>(dq), static_cast<float*>(dk), static_cast<float*>(dv),
-                                     n_heads, n_kv_heads, head_dim, seq_len, seq_len, scale, n_splits,
-                                     static_cast<float*>(dout), nullptr, nullptr));
-    CERA_TRY(cera_hip_download(ctx, out, dout, static_cast<uint64_t>(n_heads) * head_dim * 4));
-    return CERA_HIP_OK;
-}
-
-cera_hip_status cera_hip_attn_prefill(cera_hip_ctx* ctx, const float* q, const float* k, const float* v,
-                                      uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, uint64_t start_pos,
-                                      uint32_t n_queries, float scale, float* out) {
-    if (!ctx || !q || !k || !v || !out) return CERA_HIP_ERR_ARGUMENT;
-    if (n_queries == 0 || n_kv_heads == 0 || head_dim == 0) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "attn_prefill: empty input");
+// Shared body of the host-pointer attention entries: n_queries consecutive queries whose first
+// sees start_pos + 1 keys; K/V arrive time-major [pos][kv_dim] f32 (the reference layout) and
+// are laid out head-major on the device, narrowed to half first when kv_f16.
+static cera_hip_status attn_host(cera_hip_ctx* ctx, const float* q, const float* k, const float* v, uint32_t n_heads,
+                                 uint32_t n_kv_heads, uint32_t head_dim, uint64_t start_pos, uint32_t n_queries,
+                                 float scale, uint32_t n_splits, float* out, bool kv_f16) {
     const uint64_t seq_len = start_pos + n_queries;
     const uint64_t kv_dim = static_cast<uint64_t>(n_kv_heads) * head_dim, q_dim = static_cast<uint64_t>(n_heads) * head_dim;
-    const uint64_t kv_bytes = seq_len * kv_dim * 4, q_bytes = n_queries * q_dim * 4;
-    // time-major [pos][kv_dim] (reference layout) -> head-major [kv_head][pos][head_dim]
-    std::vector<float> hk(seq_len * kv_dim), hv(seq_len * kv_dim);
+    const uint64_t esz = kv_f16 ? sizeof(kv_half) : sizeof(float);
+    const uint64_t kv_bytes = seq_len * kv_dim * esz, q_bytes = n_queries * q_dim * 4;
+    std::vector<char> hk(kv_bytes), hv(kv_bytes);
     for (uint64_t t = 0; t < seq_len; ++t)
         for (uint32_t h = 0; h < n_kv_heads; ++h) {
-            std::memcpy(&hk[(h * seq_len + t) * head_dim], k + t * kv_dim + h * head_dim, head_dim * 4);
-            std::memcpy(&hv[(h * seq_len + t) * head_dim], v + t * kv_dim + h * head_dim, head_dim * 4);
+            const uint64_t dst = (h * seq_len + t) * head_dim, src = t * kv_dim + h * head_dim;
+            if (kv_f16) {
+                for (uint32_t d = 0; d < head_dim; ++d) {
+                    reinterpret_cast<kv_half*>(hk.data())[dst + d] = static_cast<kv_half>(k[src + d]);
+                    reinterpret_cast<kv_half*>(hv.data())[dst + d] = static_cast<kv_half>(v[src + d]);
+                }
+            } else {
+                std::memcpy(hk.data() + dst * 4, k + src, head_dim * 4);
+                std::memcpy(hv.data() + dst * 4, v + src, head_dim * 4);
+            }
         }
     void *dq, *dk, *dv, *dout;
     CERA_TRY(cera_scratch(ctx, 0, q_bytes, &dq));
@@ -649,10 +650,42 @@ cera_hip_status cera_hip_attn_prefill(cera_hip_ctx* ctx, const float* q, const f
     CERA_TRY(cera_hip_upload(ctx, dq, q, q_bytes));
     CERA_TRY(cera_hip_upload(ctx, dk, hk.data(), kv_bytes));
     CERA_TRY(cera_hip_upload(ctx, dv, hv.data(), kv_bytes));
-    CERA_TRY(cera_launch_attn(ctx, static_cast<float*>(dq), static_cast<float*>(dk), static_cast<float*>(dv), n_heads,
-                              n_kv_heads, head_dim, start_pos + 1, seq_len, scale, 0, n_queries, static_cast<float*>(dout),
-                              nullptr, nullptr, nullptr));
+    CERA_TRY(cera_launch_attn(ctx, static_cast<float*>(dq), dk, dv, n_heads, n_kv_heads, head_dim, start_pos + 1, seq_len,
+                              scale, n_splits, n_queries, static_cast<float*>(dout), nullptr, nullptr, nullptr, nullptr,
+                              kv_f16));
     return cera_hip_download(ctx, out, dout, q_bytes);
+}
+
+cera_hip_status cera_hip_attn_decode(cera_hip_ctx* ctx, const float* q, const float* k, const float* v,
+                                     uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, uint64_t seq_len,
+                                     float scale, uint32_t n_splits, float* out) {
+    if (!ctx || !q || !k || !v || !out) return CERA_HIP_ERR_ARGUMENT;
+    if (seq_len == 0 || n_kv_heads == 0 || head_dim == 0) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "attn_decode: empty input");
+    return attn_host(ctx, q, k, v, n_heads, n_kv_heads, head_dim, seq_len - 1, 1, scale, n_splits, out, false);
+}
+
+cera_hip_status cera_hip_attn_prefill(cera_hip_ctx* ctx, const float* q, const float* k, const float* v,
+                                      uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, uint64_t start_pos,
+                                      uint32_t n_queries, float scale, float* out) {
+    if (!ctx || !q || !k || !v || !out) return CERA_HIP_ERR_ARGUMENT;
+    if (n_queries == 0 || n_kv_heads == 0 || head_dim == 0) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "attn_prefill: empty input");
+    return attn_host(ctx, q, k, v, n_heads, n_kv_heads, head_dim, start_pos, n_queries, scale, 0, out, false);
+}
+
+cera_hip_status cera_hip_attn_f16kv(cera_hip_ctx* ctx, const float* q, const float* k, const float* v, uint32_t n_heads,
+                                    uint32_t n_kv_heads, uint32_t head_dim, uint64_t start_pos, uint32_t n_queries,
+                                    float scale, uint32_t n_splits, float* out) {
+    if (!ctx || !q || !k || !v || !out) return CERA_HIP_ERR_ARGUMENT;
+    if (n_queries == 0 || n_kv_heads == 0 || head_dim == 0) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "attn_f16kv: empty input");
+    return attn_host(ctx, q, k, v, n_heads, n_kv_heads, head_dim, start_pos, n_queries, scale, n_splits, out, true);
+}
+
+cera_hip_status cera_hip_attn_decode_f16_dev(cera_hip_ctx* ctx, const float* q, const void* k16, const void* v16,
+                                             uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, uint64_t seq_len,
+                                             uint64_t max_seq, float scale, uint32_t n_splits, float* out) {
+    if (!ctx || !q || !k16 || !v16 || !out) return CERA_HIP_ERR_ARGUMENT;
+    return cera_launch_attn_decode(ctx, q, k16, v16, n_heads, n_kv_heads, head_dim, seq_len, max_seq, scale, n_splits, out,
+                                   nullptr, nullptr, nullptr, true);
 }
 
 cera_hip_status cera_hip_rmsnorm(cera_hip_ctx* ctx, const float* x, const float* weight, uint64_t n, float eps, float* y) {

@@ -68,14 +68,36 @@ __device__ __forceinline__ void attn_rope16(float4 (&x)[4], const float* __restr
     }
 }
 
+// This lane's 16 columns of the V row of position tt; the token's own row comes from the
+// projection output (narrowed like a cached row) and is stored into the cache by the one
+// caller that owns the append.
+template <bool NEWKV, typename KV>
+__device__ __forceinline__ void attn_load_v(float4 (&vv)[4], const KV* __restrict__ vbase, uint32_t t, uint32_t tt,
+                                            uint32_t new_pos, uint32_t kvh, uint32_t max_seq, uint32_t j,
+                                            const AttnNewKV& nk, bool store) {
+    if (NEWKV && tt == new_pos) {
+        const float4* vp = reinterpret_cast<const float4*>(nk.v_new + kvh * ATTN_HD);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) vv[c] = KvOps<KV>::rnd4(vp[j + 8 * c]);
+        if (store) {
+            KV* dst = static_cast<KV*>(nk.vc_w) + (static_cast<uint64_t>(kvh) * max_seq + t) * ATTN_HD;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) KvOps<KV>::st4(dst, j + 8 * c, vv[c]);
+        }
+    } else {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) vv[c] = KvOps<KV>::ld4(vbase + static_cast<uint64_t>(tt) * ATTN_HD, j + 8 * c);
+    }
+}
+
 // One wavefront's share of the keys: chunks of 8*S positions at t_begin, t_begin + t_step, ...
 // below t_end, for the G query heads of one kv head.  Returns the online-softmax state with
 // the eight position groups already folded: every lane holds its 16 columns of acc and the
 // wavefront-wide m and l.  `q` points at the first of the G heads; `write_new` says whether
 // this caller stores the new position's K/V row into the cache (NEWKV only).
-template <int G, int S, bool NEWKV>
-__device__ __forceinline__ void attn_decode_range(const float* __restrict__ q, const float* __restrict__ kbase,
-                                                  const float* __restrict__ vbase, uint32_t kvh, uint32_t max_seq,
+template <int G, int S, bool NEWKV, typename KV>
+__device__ __forceinline__ void attn_decode_range(const float* __restrict__ q, const KV* __restrict__ kbase,
+                                                  const KV* __restrict__ vbase, uint32_t kvh, uint32_t max_seq,
                                                   uint32_t seq_len, uint32_t t_begin, uint32_t t_end, uint32_t t_step,
                                                   float scale, const AttnNewKV& nk, bool write_new, uint32_t lane,
                                                   float4 (&acc)[G][4], float (&m)[G], float (&l)[G]) {
@@ -111,16 +133,9 @@ __device__ __forceinline__ void attn_decode_range(const float* __restrict__ q, c
         if (PREFETCH_V) {
 #pragma unroll
             for (int s = 0; s < S; ++s) {
-                const uint32_t t = t0 + 8 * s + pg, tt = t < t_end ? t : t_begin;
-                const float4* vp = reinterpret_cast<const float4*>(vbase + static_cast<uint64_t>(tt) * ATTN_HD);
-                if (NEWKV && tt == new_pos) vp = reinterpret_cast<const float4*>(nk.v_new + kvh * ATTN_HD);
-#pragma unroll
-                for (int c = 0; c < 4; ++c) vpre[s][c] = vp[j + 8 * c];
-                if (NEWKV && t == new_pos && write_new) {
-                    float4* dst = reinterpret_cast<float4*>(nk.vc_w + (static_cast<uint64_t>(kvh) * max_seq + t) * ATTN_HD);
-#pragma unroll
-                    for (int c = 0; c < 4; ++c) dst[j + 8 * c] = vpre[s][c];
-                }
+                const uint32_t t = t0 + 8 * s + pg;
+                attn_load_v<NEWKV, KV>(vpre[s], vbase, t, t < t_end ? t : t_begin, new_pos, kvh, max_seq, j, nk,
+                                       write_new && t == new_pos);
             }
         }
         // ---- scores: step s covers positions t0 + 8s + pg
@@ -130,18 +145,23 @@ __device__ __forceinline__ void attn_decode_range(const float* __restrict__ q, c
             const uint32_t t = t0 + 8 * s + pg;
             const bool live = t < t_end;
             const uint32_t tt = live ? t : t_begin;
-            const float4* kp = reinterpret_cast<const float4*>(kbase + static_cast<uint64_t>(tt) * ATTN_HD);
-            if (NEWKV && tt == new_pos) kp = reinterpret_cast<const float4*>(nk.k_new + kvh * ATTN_HD);
             float4 kv[4];
+            if (NEWKV && tt == new_pos) {
+                // the token's own key: from the projection output, rotated here, narrowed like a cached row
+                const float4* kp = reinterpret_cast<const float4*>(nk.k_new + kvh * ATTN_HD);
 #pragma unroll
-            for (int c = 0; c < 4; ++c) kv[c] = kp[j + 8 * c];
-            if (NEWKV && t == new_pos) {
+                for (int c = 0; c < 4; ++c) kv[c] = kp[j + 8 * c];
                 attn_rope16(kv, nk.rope_row, j, nk.rope_type);
-                if (write_new) {
-                    float4* dst = reinterpret_cast<float4*>(nk.kc_w + (static_cast<uint64_t>(kvh) * max_seq + t) * ATTN_HD);
 #pragma unroll
-                    for (int c = 0; c < 4; ++c) dst[j + 8 * c] = kv[c];
+                for (int c = 0; c < 4; ++c) kv[c] = KvOps<KV>::rnd4(kv[c]);
+                if (write_new && live) {
+                    KV* dst = static_cast<KV*>(nk.kc_w) + (static_cast<uint64_t>(kvh) * max_seq + t) * ATTN_HD;
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) KvOps<KV>::st4(dst, j + 8 * c, kv[c]);
                 }
+            } else {
+#pragma unroll
+                for (int c = 0; c < 4; ++c) kv[c] = KvOps<KV>::ld4(kbase + static_cast<uint64_t>(tt) * ATTN_HD, j + 8 * c);
             }
 #pragma unroll
             for (int h = 0; h < G; ++h) {
@@ -185,16 +205,9 @@ __device__ __forceinline__ void attn_decode_range(const float* __restrict__ q, c
 #pragma unroll
                 for (int c = 0; c < 4; ++c) vv[c] = vpre[s][c];
             } else {
-                const uint32_t t = t0 + 8 * s + pg, tt = t < t_end ? t : t_begin;
-                const float4* vp = reinterpret_cast<const float4*>(vbase + static_cast<uint64_t>(tt) * ATTN_HD);
-                if (NEWKV && tt == new_pos) vp = reinterpret_cast<const float4*>(nk.v_new + kvh * ATTN_HD);
-#pragma unroll
-                for (int c = 0; c < 4; ++c) vv[c] = vp[j + 8 * c];
-                if (NEWKV && t == new_pos && write_new) {
-                    float4* dst = reinterpret_cast<float4*>(nk.vc_w + (static_cast<uint64_t>(kvh) * max_seq + t) * ATTN_HD);
-#pragma unroll
-                    for (int c = 0; c < 4; ++c) dst[j + 8 * c] = vv[c];
-                }
+                const uint32_t t = t0 + 8 * s + pg;
+                attn_load_v<NEWKV, KV>(vv, vbase, t, t < t_end ? t : t_begin, new_pos, kvh, max_seq, j, nk,
+                                       write_new && t == new_pos);
             }
 #pragma unroll
             for (int h = 0; h < G; ++h) {
@@ -231,11 +244,11 @@ __device__ __forceinline__ void attn_decode_range(const float* __restrict__ q, c
     }
 }
 
-template <int G, int S, bool NEWKV>
+template <int G, int S, bool NEWKV, typename KV>
 __global__ __launch_bounds__(256) void attn_decode_partial_kernel(
     const float* __restrict__ q,       // [n_heads][128]
-    const float* __restrict__ kc,      // [n_kv][max_seq][128]
-    const float* __restrict__ vc,
+    const KV* __restrict__ kc,         // [n_kv][max_seq][128]
+    const KV* __restrict__ vc,
     uint32_t seq_len, uint32_t max_seq, float scale, uint32_t chunks_per_part, uint32_t n_parts,
     uint32_t q_stride,                 // floats between consecutive queries (prefill batches queries on grid.z)
     float* __restrict__ part_acc,      // [n_queries][n_kv][n_parts][G][128]
@@ -254,7 +267,7 @@ __global__ __launch_bounds__(256) void attn_decode_partial_kernel(
     const uint32_t t_end = min(seq_len, t_begin + chunks_per_part * CHUNK);
     float4 acc[G][4];
     float m[G], l[G];
-    attn_decode_range<G, S, NEWKV>(q, kc + static_cast<uint64_t>(kvh) * max_seq * ATTN_HD,
+    attn_decode_range<G, S, NEWKV, KV>(q, kc + static_cast<uint64_t>(kvh) * max_seq * ATTN_HD,
                                    vc + static_cast<uint64_t>(kvh) * max_seq * ATTN_HD, kvh, max_seq, seq_len, t_begin,
                                    t_end, CHUNK, scale, nk, true, lane, acc, m, l);
     if (pg == 0) {
@@ -300,10 +313,11 @@ __global__ __launch_bounds__(256) void attn_decode_partial_kernel(
 #define ATTN_PF_LD 33  // words per LDS row of the transposed K tile (32 + 1 pad)
 typedef float attn_v16f __attribute__((ext_vector_type(16)));
 
+template <typename KV>
 __global__ __launch_bounds__(64) void attn_prefill_partial_kernel(
     const float* __restrict__ q,       // [n_queries][q_stride]
-    const float* __restrict__ kc,      // [n_kv][max_seq][128], already holding the batch's keys
-    const float* __restrict__ vc,
+    const KV* __restrict__ kc,         // [n_kv][max_seq][128], already holding the batch's keys
+    const KV* __restrict__ vc,
     uint32_t first_len,                // keys visible to query 0; query i sees first_len + i
     uint32_t n_queries, uint32_t max_seq, float scale, uint32_t part_keys, uint32_t n_parts, uint32_t q_stride,
     uint32_t G,
@@ -321,8 +335,8 @@ __global__ __launch_bounds__(64) void attn_prefill_partial_kernel(
     const uint32_t key_lo = part * part_keys;
     const uint32_t key_hi = min(key_lo + part_keys, block_len);
 
-    const float* kbase = kc + static_cast<uint64_t>(kvh) * max_seq * ATTN_HD;
-    const float* vbase = vc + static_cast<uint64_t>(kvh) * max_seq * ATTN_HD;
+    const KV* kbase = kc + static_cast<uint64_t>(kvh) * max_seq * ATTN_HD;
+    const KV* vbase = vc + static_cast<uint64_t>(kvh) * max_seq * ATTN_HD;
 
     // this lane's query, the dims of its half: d = 2s + half
     float qreg[64];
@@ -345,7 +359,7 @@ __global__ __launch_bounds__(64) void attn_prefill_partial_kernel(
         for (int i = 0; i < 16; ++i) {
             const uint32_t f = lane + 64 * i, key = f >> 5, c4 = f & 31;
             float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (k0 + key < key_hi) v = reinterpret_cast<const float4*>(kbase + static_cast<uint64_t>(k0 + key) * ATTN_HD)[c4];
+            if (k0 + key < key_hi) v = KvOps<KV>::ld4(kbase + static_cast<uint64_t>(k0 + key) * ATTN_HD, c4);
             sKt[(4 * c4 + 0) * ATTN_PF_LD + key] = v.x;
             sKt[(4 * c4 + 1) * ATTN_PF_LD + key] = v.y;
             sKt[(4 * c4 + 2) * ATTN_PF_LD + key] = v.z;
@@ -396,10 +410,10 @@ __global__ __launch_bounds__(64) void attn_prefill_partial_kernel(
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
             const uint32_t kg = min(k0 + 8 * (e >> 2) + 4 * half + (e & 3), key_hi - 1);   // masked keys have p = 0
-            const float* vrow = vbase + static_cast<uint64_t>(kg) * ATTN_HD + col;
+            const KV* vrow = vbase + static_cast<uint64_t>(kg) * ATTN_HD + col;
 #pragma unroll
             for (int dt = 0; dt < 4; ++dt)
-                acc[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(c[e], vrow[32 * dt], acc[dt], 0, 0, 0);
+                acc[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(c[e], KvOps<KV>::ld1(vrow + 32 * dt), acc[dt], 0, 0, 0);
         }
         __syncthreads();   // sKt and sX are rewritten by the next tile
     }

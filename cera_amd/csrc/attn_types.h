@@ -11,6 +11,6 @@ struct AttnNewKV {
     uint32_t rope_type;      // 0 NEOX, 1 NORM
     const float* k_new;      // [n_kv][128], unrotated
     const float* v_new;      // [n_kv][128]
-    float* kc_w;             // the caches, writable
-    float* vc_w;
+    void* kc_w;              // the caches, writable (f32 or half, as the kernel is instantiated)
+    void* vc_w;
 };

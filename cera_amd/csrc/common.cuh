@@ -32,6 +32,32 @@ __device__ __forceinline__ uint32_t f2h(float v) {
     return __builtin_bit_cast(uint16_t, static_cast<_Float16>(v));
 }
 
+// KV cache element access.  The cache holds f32, or IEEE half when the session asks for an f16
+// KV cache (cera/src/kv_cache.rs:93-98): values are narrowed with round-to-nearest-even when a
+// row is appended and widened exactly on every read, accumulation stays f32
+// (cera/src/model/transformer.rs:1424-1447, 1170-1196).
+typedef _Float16 kv_half;
+template <typename KV> struct KvOps;
+template <> struct KvOps<float> {
+    __device__ static __forceinline__ float4 ld4(const float* row, uint32_t i) { return reinterpret_cast<const float4*>(row)[i]; }
+    __device__ static __forceinline__ void st4(float* row, uint32_t i, float4 v) { reinterpret_cast<float4*>(row)[i] = v; }
+    __device__ static __forceinline__ float4 rnd4(float4 v) { return v; }
+    __device__ static __forceinline__ float ld1(const float* p) { return *p; }
+};
+template <> struct KvOps<kv_half> {
+    __device__ static __forceinline__ float4 ld4(const kv_half* row, uint32_t i) {
+        const uint2 r = reinterpret_cast<const uint2*>(row)[i];
+        return make_float4(h2f(r.x & 0xFFFF), h2f(r.x >> 16), h2f(r.y & 0xFFFF), h2f(r.y >> 16));
+    }
+    __device__ static __forceinline__ void st4(kv_half* row, uint32_t i, float4 v) {
+        reinterpret_cast<uint2*>(row)[i] = make_uint2(f2h(v.x) | (f2h(v.y) << 16), f2h(v.z) | (f2h(v.w) << 16));
+    }
+    __device__ static __forceinline__ float4 rnd4(float4 v) {
+        return make_float4(h2f(f2h(v.x)), h2f(f2h(v.y)), h2f(f2h(v.z)), h2f(f2h(v.w)));
+    }
+    __device__ static __forceinline__ float ld1(const kv_half* p) { return static_cast<float>(*p); }
+};
+
 // 4 x int8 dot with int32 accumulate (v_dot4_i32_i8).
 __device__ __forceinline__ int dot4(uint32_t a, uint32_t b, int c) {
     return __builtin_amdgcn_sdot4(static_cast<int>(a), static_cast<int>(b), c, false);

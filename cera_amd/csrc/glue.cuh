@@ -194,10 +194,11 @@ static __global__ __launch_bounds__(1024) void rmsnorm_row_kernel(const float* _
 // threads: blocks [0, n_heads) rotate q; the next n_kv_heads rotate k and
 // store it; the last n_kv_heads copy v.
 // KV cache layout: [kv_head][max_seq][head_dim] f32.
+template <typename KV>
 static __global__ void rope_kv_kernel(float* __restrict__ q, float* __restrict__ k, const float* v,
                                const float* __restrict__ cs_table, const uint32_t* __restrict__ pos_ptr,
                                uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, uint32_t rope_type,
-                               float* __restrict__ k_cache, float* __restrict__ v_cache, uint32_t max_seq) {
+                               KV* __restrict__ k_cache, KV* __restrict__ v_cache, uint32_t max_seq) {
     // grid.y = tokens of a prefill batch: token t sits at position *pos_ptr + t and its
     // q/k/v rows follow each other ([n][n_heads*head_dim], [n][n_kv_heads*head_dim])
     const uint32_t pos = *pos_ptr + blockIdx.y;
@@ -215,15 +216,15 @@ static __global__ void rope_kv_kernel(float* __restrict__ q, float* __restrict__
         head[i0] = r0;
         head[i1] = r1;
         if (b >= n_heads && k_cache) {
-            float* dst = k_cache + (static_cast<uint64_t>(b - n_heads) * max_seq + pos) * head_dim;
-            dst[i0] = r0;
-            dst[i1] = r1;
+            KV* dst = k_cache + (static_cast<uint64_t>(b - n_heads) * max_seq + pos) * head_dim;
+            dst[i0] = static_cast<KV>(r0);   // half cache: round to nearest even
+            dst[i1] = static_cast<KV>(r1);
         }
     } else if (v_cache) {
         uint32_t h = b - n_heads - n_kv_heads;
-        float* dst = v_cache + (static_cast<uint64_t>(h) * max_seq + pos) * head_dim;
-        dst[2 * i] = v[h * head_dim + 2 * i];
-        dst[2 * i + 1] = v[h * head_dim + 2 * i + 1];
+        KV* dst = v_cache + (static_cast<uint64_t>(h) * max_seq + pos) * head_dim;
+        dst[2 * i] = static_cast<KV>(v[h * head_dim + 2 * i]);
+        dst[2 * i + 1] = static_cast<KV>(v[h * head_dim + 2 * i + 1]);
     }
 }
 
@@ -234,15 +235,17 @@ static __global__ void rope_kv_kernel(float* __restrict__ q, float* __restrict__
 // reference's recurrence (cera/src/backend/cpu.rs:5065-5086 NEOX, :5145-5180 NORM); null = plain
 // copy (V, and the copy back from staging).  head_dim = 128; 16 threads per row, each owning
 // float4 j and float4 j + 16.  grid = (ceil(n_rows * 16 / 256), n_kv_heads).
-static __global__ __launch_bounds__(256) void kv_shift_kernel(const float* __restrict__ src, float* __restrict__ dst,
+template <typename KV>
+static __global__ __launch_bounds__(256) void kv_shift_kernel(const KV* __restrict__ src, KV* __restrict__ dst,
                                                               uint32_t src_row, uint32_t dst_row, uint32_t n_rows,
                                                               uint64_t src_head_stride, uint64_t dst_head_stride,
                                                               const float* __restrict__ delta_cs, uint32_t rope_type) {
     const uint32_t t = (blockIdx.x * 256 + threadIdx.x) >> 4, j = threadIdx.x & 15;
     if (t >= n_rows) return;
-    const float4* sp = reinterpret_cast<const float4*>(src + blockIdx.y * src_head_stride + static_cast<uint64_t>(src_row + t) * 128);
-    float4* dp = reinterpret_cast<float4*>(dst + blockIdx.y * dst_head_stride + static_cast<uint64_t>(dst_row + t) * 128);
-    float4 a = sp[j], b = sp[j + 16];
+    const KV* sp = src + blockIdx.y * src_head_stride + static_cast<uint64_t>(src_row + t) * 128;
+    KV* dp = dst + blockIdx.y * dst_head_stride + static_cast<uint64_t>(dst_row + t) * 128;
+    // a half cache is widened, rotated in f32 and narrowed again (cera/src/kv_cache.rs:1196-1230)
+    float4 a = KvOps<KV>::ld4(sp, j), b = KvOps<KV>::ld4(sp, j + 16);
     if (delta_cs) {
         const float4* cs = reinterpret_cast<const float4*>(delta_cs);
         if (rope_type == 1) {   // NORM: pairs (2i, 2i+1): pair i uses cs[i]; float4 j holds pairs 2j, 2j+1
@@ -272,8 +275,8 @@ static __global__ __launch_bounds__(256) void kv_shift_kernel(const float* __res
             a = ra; b = rb;
         }
     }
-    dp[j] = a;
-    dp[j + 16] = b;
+    KvOps<KV>::st4(dp, j, a);
+    KvOps<KV>::st4(dp, j + 16, b);
 }
 
 // out = a + b (cera/src/backend/cpu.rs:5223-5228), optional scale on b first.

@@ -68,17 +68,19 @@ cera_hip_status cera_launch_gemv(cera_hip_ctx* ctx, const cera_hip_dtensor* w, c
 // index of the maximum of x[0, n) into *out_dev (device); uses scratch slot 8 of the context
 cera_hip_status cera_launch_argmax(cera_hip_ctx* ctx, const float* x, uint32_t n, uint32_t* out_dev);
 cera_hip_status cera_launch_gemv_q5k_f32(cera_hip_ctx* ctx, const cera_hip_dtensor* w, const float* x, float* y);
-cera_hip_status cera_launch_attn_decode(cera_hip_ctx* ctx, const float* q, const float* kc, const float* vc,
+// kc / vc: [n_kv_heads][max_seq][head_dim], f32 or IEEE half (kv_f16)
+cera_hip_status cera_launch_attn_decode(cera_hip_ctx* ctx, const float* q, const void* kc, const void* vc,
                                         uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, uint64_t seq_len,
                                         uint64_t max_seq, float scale, uint32_t n_splits, float* out,
-                                        float* out_scales, int8_t* out_quants, const AttnNewKV* new_kv = nullptr);
+                                        float* out_scales, int8_t* out_quants, const AttnNewKV* new_kv = nullptr,
+                                        bool kv_f16 = false);
 // n_queries consecutive queries (causal): query i sees seq_len + i keys; q and the outputs are
 // [n_queries][n_heads*head_dim]
-cera_hip_status cera_launch_attn(cera_hip_ctx* ctx, const float* q, const float* kc, const float* vc,
+cera_hip_status cera_launch_attn(cera_hip_ctx* ctx, const float* q, const void* kc, const void* vc,
                                  uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, uint64_t seq_len,
                                  uint64_t max_seq, float scale, uint32_t n_splits, uint32_t n_queries, float* out,
                                  float* out_scales, int8_t* out_quants, float* out_bsum,
-                                 const AttnNewKV* new_kv = nullptr);
+                                 const AttnNewKV* new_kv = nullptr, bool kv_f16 = false);
 // One allocation holding the rows of several same-type, same-k matrices back to back
 // (`fused`), plus a non-owning view per part.  Lets the decode step run Q|K(|V) as one GEMV.
 cera_hip_status cera_tensor_upload_concat(cera_hip_ctx* ctx, const cera_hip_tensor* const* parts, int n_parts,

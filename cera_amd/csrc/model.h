@@ -14,7 +14,7 @@ struct LayerDev {
     uint32_t qkv_rows = 0;  // rows covered by the fused launch (0: not fused)
     float *attn_norm = nullptr, *ffn_norm = nullptr;
     float *q_bias = nullptr, *k_bias = nullptr, *v_bias = nullptr, *q_norm = nullptr, *k_norm = nullptr;
-    float *kc = nullptr, *vc = nullptr;  // [n_kv_heads][max_seq_len][head_dim] f32
+    void *kc = nullptr, *vc = nullptr;  // [n_kv_heads][max_seq_len][head_dim], f32 or half (model->kv_f16)
 };
 
 struct cera_hip_model {
@@ -42,6 +42,8 @@ struct cera_hip_model {
     uint32_t pf_logits_cap = 0;
     std::vector<void*> pf_owned;
     uint32_t seq_len = 0;
+    bool kv_f16 = false;          // KV caches hold IEEE half instead of f32
+    bool kv_configured = false;   // cera_hip_configure_kv was called: a different mode is a conflict
     uint64_t bytes = 0;
     // every trait call is serialised, like the reference GPU backends' infer_lock
     // (cera/src/model/mod.rs:184-199)

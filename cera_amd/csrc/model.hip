@@ -7,6 +7,8 @@
 #include <cstring>
 #include <new>
 
+#include <type_traits>
+
 #include "glue.cuh"
 #include "host_common.h"
 #include "model.h"
@@ -26,6 +28,13 @@ static cera_hip_status upload_f32(cera_hip_ctx* ctx, const float* host, uint64_t
     if (!host) { *out = nullptr; return CERA_HIP_OK; }
     CERA_TRY(dev_alloc_t(ctx, n, out, total));
     return cera_hip_upload(ctx, *out, host, n * 4);
+}
+
+// lanes past the end of a key range re-read a cached row with weight 0: keep every row finite
+static cera_hip_status alloc_kv_cache(cera_hip_ctx* ctx, uint64_t bytes, void** out, uint64_t* total) {
+    CERA_TRY(dev_alloc(ctx, bytes, out, total));
+    HIP_TRY(ctx, hipMemsetAsync(*out, 0, bytes, ctx->stream));
+    return CERA_HIP_OK;
 }
 
 // cos/sin table [max_seq][head_dim/2] built with the CPU path's own recurrence:
@@ -55,8 +64,10 @@ static void free_model(cera_hip_model* m) {
     auto ft = [&](cera_hip_dtensor* t) { if (t) cera_hip_tensor_free(ctx, t); };
     for (auto& L : m->layers) {
         ft(L.q); ft(L.k); ft(L.v); ft(L.o); ft(L.gate); ft(L.up); ft(L.down); ft(L.qkv);
-        for (float* p : {L.attn_norm, L.ffn_norm, L.q_bias, L.k_bias, L.v_bias, L.q_norm, L.k_norm, L.kc, L.vc})
+        for (float* p : {L.attn_norm, L.ffn_norm, L.q_bias, L.k_bias, L.v_bias, L.q_norm, L.k_norm})
             if (p) (void)hipFree(p);
+        if (L.kc) (void)hipFree(L.kc);
+        if (L.vc) (void)hipFree(L.vc);
     }
     ft(m->embd);
     ft(m->output);
@@ -164,11 +175,8 @@ extern "C" cera_hip_status cera_hip_model_create(cera_hip_ctx* ctx, const cera_h
                 CERA_TRY(upload_f32(ctx, L.q_norm, c.head_dim, &D.q_norm, tot));
                 CERA_TRY(upload_f32(ctx, L.k_norm, c.head_dim, &D.k_norm, tot));
             }
-            CERA_TRY(dev_alloc_t(ctx, kv_elems, &D.kc, tot));
-            CERA_TRY(dev_alloc_t(ctx, kv_elems, &D.vc, tot));
-            // lanes past the end of a key range re-read a cached row with weight 0: keep every row finite
-            HIP_TRY(ctx, hipMemsetAsync(D.kc, 0, kv_elems * sizeof(float), ctx->stream));
-            HIP_TRY(ctx, hipMemsetAsync(D.vc, 0, kv_elems * sizeof(float), ctx->stream));
+            CERA_TRY(alloc_kv_cache(ctx, kv_elems * sizeof(float), &D.kc, tot));
+            CERA_TRY(alloc_kv_cache(ctx, kv_elems * sizeof(float), &D.vc, tot));
         }
         if (cfg->rope_freqs) m->rope_ff.assign(cfg->rope_freqs, cfg->rope_freqs + c.head_dim / 2);
         CERA_TRY(dev_alloc_t(ctx, c.head_dim, &tmp, tot));
@@ -257,28 +265,32 @@ extern "C" cera_hip_status cera_hip_shift_kv(cera_hip_model* m, uint32_t n_keep,
         const uint64_t head_stride = static_cast<uint64_t>(c.max_seq_len) * c.head_dim;
         const dim3 grid((tail * 16 + 255) / 256, c.n_kv_heads), block(256);
         const bool overlap = tail > shift;   // source and destination rows intersect: go through staging
-        float* stage = nullptr;
+        void* stage = nullptr;
         const uint64_t stage_stride = static_cast<uint64_t>(tail) * c.head_dim;
         if (overlap) {
-            void* p = nullptr;
-            CERA_TRY(cera_scratch(ctx, 5, stage_stride * c.n_kv_heads * sizeof(float), &p));
-            stage = static_cast<float*>(p);
+            CERA_TRY(cera_scratch(ctx, 5, stage_stride * c.n_kv_heads * sizeof(float), &stage));
         }
-        for (LayerDev& L : m->layers) {
-            for (int is_v = 0; is_v < 2; ++is_v) {
-                float* cache = is_v ? L.vc : L.kc;
-                const float* cs = is_v ? nullptr : m->shift_cs;
-                if (!overlap) {
-                    hipLaunchKernelGGL(kv_shift_kernel, grid, block, 0, ctx->stream, cache, cache, src_row, n_keep, tail,
-                                       head_stride, head_stride, cs, c.rope_type);
-                } else {
-                    hipLaunchKernelGGL(kv_shift_kernel, grid, block, 0, ctx->stream, cache, stage, src_row, 0u, tail,
-                                       head_stride, stage_stride, cs, c.rope_type);
-                    hipLaunchKernelGGL(kv_shift_kernel, grid, block, 0, ctx->stream, stage, cache, 0u, n_keep, tail,
-                                       stage_stride, head_stride, static_cast<const float*>(nullptr), c.rope_type);
+        auto run = [&](auto* tag) {
+            using KV = std::remove_pointer_t<decltype(tag)>;
+            for (LayerDev& L : m->layers) {
+                for (int is_v = 0; is_v < 2; ++is_v) {
+                    KV* cache = static_cast<KV*>(is_v ? L.vc : L.kc);
+                    const float* cs = is_v ? nullptr : m->shift_cs;
+                    if (!overlap) {
+                        hipLaunchKernelGGL(kv_shift_kernel<KV>, grid, block, 0, ctx->stream, cache, cache, src_row, n_keep,
+                                           tail, head_stride, head_stride, cs, c.rope_type);
+                    } else {
+                        hipLaunchKernelGGL(kv_shift_kernel<KV>, grid, block, 0, ctx->stream, cache, static_cast<KV*>(stage),
+                                           src_row, 0u, tail, head_stride, stage_stride, cs, c.rope_type);
+                        hipLaunchKernelGGL(kv_shift_kernel<KV>, grid, block, 0, ctx->stream, static_cast<KV*>(stage), cache,
+                                           0u, n_keep, tail, stage_stride, head_stride, static_cast<const float*>(nullptr),
+                                           c.rope_type);
+                    }
                 }
             }
-        }
+        };
+        if (m->kv_f16) run(static_cast<kv_half*>(nullptr));
+        else run(static_cast<float*>(nullptr));
         HIP_TRY(ctx, hipGetLastError());
         HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
     }
@@ -299,13 +311,22 @@ extern "C" cera_hip_status cera_hip_write_kv(cera_hip_model* m, uint32_t layer, 
     const uint64_t per_head = static_cast<uint64_t>(c.max_seq_len) * c.head_dim;
     const uint64_t kv_dim = static_cast<uint64_t>(c.n_kv_heads) * c.head_dim;
     std::vector<float> hk(static_cast<uint64_t>(n_pos) * c.head_dim), hv(hk.size());
+    std::vector<kv_half> h16;
+    const uint64_t esz = m->kv_f16 ? sizeof(kv_half) : sizeof(float);
+    auto put = [&](void* cache, uint32_t h, const std::vector<float>& rows) -> cera_hip_status {
+        char* dst = static_cast<char*>(cache) + h * per_head * esz;
+        if (!m->kv_f16) return cera_hip_upload(m->ctx, dst, rows.data(), rows.size() * 4);
+        h16.resize(rows.size());
+        for (size_t i = 0; i < rows.size(); ++i) h16[i] = static_cast<kv_half>(rows[i]);   // round to nearest even
+        return cera_hip_upload(m->ctx, dst, h16.data(), h16.size() * sizeof(kv_half));
+    };
     for (uint32_t h = 0; h < c.n_kv_heads && n_pos; ++h) {
         for (uint32_t t = 0; t < n_pos; ++t) {
             std::memcpy(hk.data() + static_cast<uint64_t>(t) * c.head_dim, k + t * kv_dim + h * c.head_dim, c.head_dim * 4);
             std::memcpy(hv.data() + static_cast<uint64_t>(t) * c.head_dim, v + t * kv_dim + h * c.head_dim, c.head_dim * 4);
         }
-        CERA_TRY(cera_hip_upload(m->ctx, m->layers[layer].kc + h * per_head, hk.data(), hk.size() * 4));
-        CERA_TRY(cera_hip_upload(m->ctx, m->layers[layer].vc + h * per_head, hv.data(), hv.size() * 4));
+        CERA_TRY(put(m->layers[layer].kc, h, hk));
+        CERA_TRY(put(m->layers[layer].vc, h, hv));
     }
     return CERA_HIP_OK;
 }
@@ -317,6 +338,40 @@ extern "C" cera_hip_status cera_hip_set_seq_len(cera_hip_model* m, uint32_t len)
     m->seq_len = len;
     return CERA_HIP_OK;
 }
+
+// Model::configure_kv_compression for the modes this backend has (cera/src/model/mod.rs:557-592,
+// KvCompression::{None, F16}, cera/src/kv_cache.rs:88-98): called before the first forward pass;
+// the first call wins, the same mode again is a no-op, a different one a conflict.  Switching
+// re-allocates the (still empty) caches at the new element width.
+extern "C" cera_hip_status cera_hip_configure_kv(cera_hip_model* m, uint32_t kv_type) {
+    if (!m) return CERA_HIP_ERR_ARGUMENT;
+    std::lock_guard<std::mutex> lk(m->infer_lock);
+    cera_hip_ctx* ctx = m->ctx;
+    if (kv_type > CERA_HIP_KV_F16) return cera_fail(ctx, CERA_HIP_ERR_ARGUMENT, "configure_kv: unknown cache type");
+    const bool want_f16 = kv_type == CERA_HIP_KV_F16;
+    if (m->kv_configured && want_f16 != m->kv_f16)
+        return cera_fail(ctx, CERA_HIP_ERR_ARGUMENT, "configure_kv: the KV cache is already configured for another mode");
+    m->kv_configured = true;
+    if (want_f16 == m->kv_f16) return CERA_HIP_OK;
+    if (m->seq_len != 0) return cera_fail(ctx, CERA_HIP_ERR_POSITION, "configure_kv: the cache already holds positions");
+    const cera_hip_config& c = m->cfg;
+    const uint64_t kv_elems = static_cast<uint64_t>(c.n_kv_heads) * c.max_seq_len * c.head_dim;
+    const uint64_t old_bytes = kv_elems * (m->kv_f16 ? sizeof(kv_half) : sizeof(float));
+    const uint64_t new_bytes = kv_elems * (want_f16 ? sizeof(kv_half) : sizeof(float));
+    HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    for (LayerDev& L : m->layers) {
+        for (void** cache : {&L.kc, &L.vc}) {
+            if (*cache) HIP_TRY(ctx, hipFree(*cache));
+            *cache = nullptr;
+            m->bytes -= old_bytes;
+            CERA_TRY(alloc_kv_cache(ctx, new_bytes, cache, &m->bytes));
+        }
+    }
+    m->kv_f16 = want_f16;
+    return CERA_HIP_OK;
+}
+
+extern "C" uint32_t cera_hip_kv_type(const cera_hip_model* m) { return m && m->kv_f16 ? CERA_HIP_KV_F16 : CERA_HIP_KV_F32; }
 
 // ---------------------------------------------------------------------------
 // One projection: int8 kernels read the quantized activations, Q5_K the f32 ones.
@@ -401,7 +456,7 @@ static cera_hip_status decode_step(cera_hip_model* m, uint32_t pos, bool want_lo
         nk.kc_w = L.kc;
         nk.vc_w = L.vc;
         CERA_TRY(cera_launch_attn_decode(ctx, m->q, L.kc, L.vc, c.n_heads, c.n_kv_heads, c.head_dim, pos + 1,
-                                         c.max_seq_len, scale, 0, m->attn_out, m->xs, m->xq, &nk));
+                                         c.max_seq_len, scale, 0, m->attn_out, m->xs, m->xq, &nk, m->kv_f16));
         CERA_TRY(project(m, L.o, m->attn_out, m->hidden, m->hidden));
 
         CERA_TRY(norm_quant(m, m->hidden, L.ffn_norm, c.hidden, 1, m->normed));
@@ -535,9 +590,20 @@ extern "C" cera_hip_status cera_hip_read_kv(cera_hip_model* m, uint32_t layer, f
     const uint64_t per_head = static_cast<uint64_t>(c.max_seq_len) * c.head_dim;
     std::vector<float> hk(static_cast<uint64_t>(m->seq_len) * c.head_dim), hv(hk.size());
     const uint64_t kv_dim = static_cast<uint64_t>(c.n_kv_heads) * c.head_dim;
+    std::vector<kv_half> h16;
+    const uint64_t esz = m->kv_f16 ? sizeof(kv_half) : sizeof(float);
+    // a half cache is widened (exactly) to the f32 the caller sees
+    auto get = [&](const void* cache, uint32_t h, std::vector<float>& rows) -> cera_hip_status {
+        const char* src = static_cast<const char*>(cache) + h * per_head * esz;
+        if (!m->kv_f16) return cera_hip_download(m->ctx, rows.data(), src, rows.size() * 4);
+        h16.resize(rows.size());
+        CERA_TRY(cera_hip_download(m->ctx, h16.data(), src, h16.size() * sizeof(kv_half)));
+        for (size_t i = 0; i < rows.size(); ++i) rows[i] = static_cast<float>(h16[i]);
+        return CERA_HIP_OK;
+    };
     for (uint32_t h = 0; h < c.n_kv_heads; ++h) {
-        CERA_TRY(cera_hip_download(m->ctx, hk.data(), m->layers[layer].kc + h * per_head, hk.size() * 4));
-        CERA_TRY(cera_hip_download(m->ctx, hv.data(), m->layers[layer].vc + h * per_head, hv.size() * 4));
+        CERA_TRY(get(m->layers[layer].kc, h, hk));
+        CERA_TRY(get(m->layers[layer].vc, h, hv));
         for (uint32_t t = 0; t < m->seq_len; ++t) {
             std::memcpy(k_out + t * kv_dim + h * c.head_dim, hk.data() + static_cast<uint64_t>(t) * c.head_dim, c.head_dim * 4);
             std::memcpy(v_out + t * kv_dim + h * c.head_dim, hv.data() + static_cast<uint64_t>(t) * c.head_dim, c.head_dim * 4);
@@ -571,7 +637,7 @@ extern "C" cera_hip_status cera_hip_rope(cera_hip_ctx* ctx, float* q, float* k, 
     CERA_TRY(cera_hip_upload(ctx, dk, k, static_cast<uint64_t>(n_kv_heads) * head_dim * 4));
     CERA_TRY(cera_hip_upload(ctx, dt, table.data() + static_cast<uint64_t>(pos) * half * 2, half * 8));
     CERA_TRY(cera_hip_upload(ctx, dp, &zero, 4));
-    hipLaunchKernelGGL(rope_kv_kernel, dim3(n_heads + n_kv_heads), dim3(head_dim / 2), 0, ctx->stream,
+    hipLaunchKernelGGL(rope_kv_kernel<float>, dim3(n_heads + n_kv_heads), dim3(head_dim / 2), 0, ctx->stream,
                        static_cast<float*>(dq), static_cast<float*>(dk), static_cast<const float*>(nullptr),
                        static_cast<float*>(dt), static_cast<uint32_t*>(dp), n_heads, n_kv_heads, head_dim, rope_type,
                        static_cast<float*>(nullptr), static_cast<float*>(nullptr), 1u);

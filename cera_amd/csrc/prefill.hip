@@ -196,13 +196,18 @@ static cera_hip_status prefill_chunk(cera_hip_model* m, const uint32_t* tokens, 
             hipLaunchKernelGGL((rmsnorm_kernel<false>), dim3(n * c.n_kv_heads), dim3(256), 0, s, m->pf_k, L.k_norm, c.head_dim,
                                c.rms_eps, m->pf_k, nullptr, nullptr, nullptr);
         }
-        hipLaunchKernelGGL(rope_kv_kernel, dim3(c.n_heads + 2 * c.n_kv_heads, n), dim3(c.head_dim / 2), 0, s, m->pf_q, m->pf_k,
-                           m->pf_v, m->rope_table, m->scalars + 1, c.n_heads, c.n_kv_heads, c.head_dim, c.rope_type, L.kc, L.vc,
-                           c.max_seq_len);
+        if (m->kv_f16)
+            hipLaunchKernelGGL(rope_kv_kernel<kv_half>, dim3(c.n_heads + 2 * c.n_kv_heads, n), dim3(c.head_dim / 2), 0, s,
+                               m->pf_q, m->pf_k, m->pf_v, m->rope_table, m->scalars + 1, c.n_heads, c.n_kv_heads, c.head_dim,
+                               c.rope_type, static_cast<kv_half*>(L.kc), static_cast<kv_half*>(L.vc), c.max_seq_len);
+        else
+            hipLaunchKernelGGL(rope_kv_kernel<float>, dim3(c.n_heads + 2 * c.n_kv_heads, n), dim3(c.head_dim / 2), 0, s,
+                               m->pf_q, m->pf_k, m->pf_v, m->rope_table, m->scalars + 1, c.n_heads, c.n_kv_heads, c.head_dim,
+                               c.rope_type, static_cast<float*>(L.kc), static_cast<float*>(L.vc), c.max_seq_len);
         HIP_TRY(ctx, hipGetLastError());
         // causal attention: query t sees positions 0 .. start_pos + t
         CERA_TRY(cera_launch_attn(ctx, m->pf_q, L.kc, L.vc, c.n_heads, c.n_kv_heads, c.head_dim, start_pos + 1ull,
-                                  c.max_seq_len, scale, 0, n, m->pf_attn, m->pf_xs, m->pf_xq, m->pf_bsum));
+                                  c.max_seq_len, scale, 0, n, m->pf_attn, m->pf_xs, m->pf_xq, m->pf_bsum, nullptr, m->kv_f16));
         CERA_TRY(gemm(L.o, m->pf_hidden, m->pf_hidden));
 
         CERA_TRY(norm_rows(m->pf_hidden, L.ffn_norm, m->pf_normed));

@@ -27,7 +27,8 @@ SYMBOLS = [
     "cera_hip_quantize_q8_0_dev", "cera_hip_gemv_q8_dev", "cera_hip_gemv_seq_dev", "cera_hip_attn_decode_dev",
     "cera_hip_gemm_dev",
     "cera_hip_model_create", "cera_hip_model_destroy", "cera_hip_forward", "cera_hip_forward_greedy",
-    "cera_hip_forward_prefill", "cera_hip_forward_prefill_logits_all", "cera_hip_truncate_kv", "cera_hip_shift_kv", "cera_hip_write_kv", "cera_hip_set_seq_len", "cera_hip_seq_len", "cera_hip_memory_bytes",
+    "cera_hip_forward_prefill", "cera_hip_forward_prefill_logits_all", "cera_hip_truncate_kv", "cera_hip_configure_kv", "cera_hip_kv_type", "cera_hip_attn_f16kv",
+    "cera_hip_attn_decode_f16_dev", "cera_hip_shift_kv", "cera_hip_write_kv", "cera_hip_set_seq_len", "cera_hip_seq_len", "cera_hip_memory_bytes",
     "cera_hip_read_kv", "cera_hip_read_hidden",
 ]
 
@@ -115,6 +116,10 @@ def load_library() -> C.CDLL:
         "cera_hip_forward_prefill": (i32, [vp, vp, u32, u32, vp]),
         "cera_hip_forward_prefill_logits_all": (i32, [vp, vp, u32, u32, vp]),
         "cera_hip_truncate_kv": (i32, [vp, u32]),
+        "cera_hip_configure_kv": (i32, [vp, u32]),
+        "cera_hip_kv_type": (u32, [vp]),
+        "cera_hip_attn_f16kv": (i32, [vp, vp, vp, vp, u32, u32, u32, u64, u32, f32, u32, vp]),
+        "cera_hip_attn_decode_f16_dev": (i32, [vp, vp, vp, vp, u32, u32, u32, u64, u64, f32, u32, vp]),
         "cera_hip_shift_kv": (i32, [vp, u32, u32]),
         "cera_hip_write_kv": (i32, [vp, u32, vp, vp, u32]),
         "cera_hip_set_seq_len": (i32, [vp, u32]),
@@ -273,6 +278,16 @@ class Context:
                                                   n_queries, scale, _p(out)))
         return out.reshape(n_queries, n_heads * head_dim)
 
+    def attn_f16kv(self, q, k, v, n_heads, n_kv_heads, head_dim, start_pos, n_queries, scale, n_splits=0) -> np.ndarray:
+        """Attention over an f16 KV cache: k, v (f32) are narrowed to half before the upload."""
+        q = np.ascontiguousarray(q, np.float32)
+        k = np.ascontiguousarray(k, np.float32)
+        v = np.ascontiguousarray(v, np.float32)
+        out = np.empty(n_queries * n_heads * head_dim, np.float32)
+        self.check(self.lib.cera_hip_attn_f16kv(self.h, _p(q), _p(k), _p(v), n_heads, n_kv_heads, head_dim, start_pos,
+                                                n_queries, scale, n_splits, _p(out)))
+        return out.reshape(n_queries, n_heads * head_dim)
+
     def rmsnorm(self, x, w, eps) -> np.ndarray:
         x = np.ascontiguousarray(x, np.float32)
         w = np.ascontiguousarray(w, np.float32)
@@ -399,6 +414,13 @@ class Model:
         self.ctx.check(self.ctx.lib.cera_hip_forward_prefill_logits_all(self.h, _p(t) if t.size else None, t.size, start_pos,
                                                                         _p(out)))
         return out
+
+    def configure_kv(self, f16: bool):
+        self.ctx.check(self.ctx.lib.cera_hip_configure_kv(self.h, 1 if f16 else 0))
+
+    @property
+    def kv_f16(self) -> bool:
+        return self.ctx.lib.cera_hip_kv_type(self.h) == 1
 
     def shift_kv(self, n_keep: int, shift: int):
         self.ctx.check(self.ctx.lib.cera_hip_shift_kv(self.h, n_keep, shift))

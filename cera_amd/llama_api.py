@@ -14,7 +14,7 @@ from . import _build
 LLAMA_SYMBOLS = ["cera_llama_open", "cera_llama_close", "cera_llama_last_error", "cera_llama_get_config",
                  "cera_llama_seq_len", "cera_llama_gpu_memory_bytes", "cera_llama_forward",
                  "cera_llama_forward_greedy", "cera_llama_forward_prefill", "cera_llama_forward_prefill_logits_all", "cera_llama_forward_prefill_chunked",
-                 "cera_llama_set_cancel", "cera_llama_truncate_kv", "cera_llama_supports_kv_shift", "cera_llama_shift_kv",
+                 "cera_llama_set_cancel", "cera_llama_truncate_kv", "cera_llama_supports_kv_shift", "cera_llama_f16_kv_supported", "cera_llama_configure_kv_compression", "cera_llama_shift_kv",
                  "cera_llama_snapshot_state", "cera_llama_snapshot_seq_len", "cera_llama_snapshot_bytes",
                  "cera_llama_restore_state", "cera_llama_snapshot_free", "cera_llama_generate_greedy"]
 
@@ -50,6 +50,8 @@ def lib() -> C.CDLL:
             "cera_llama_set_cancel": (None, [vp, C.c_int]),
             "cera_llama_truncate_kv": (C.c_int, [vp, u64]),
             "cera_llama_supports_kv_shift": (C.c_int, [vp]),
+            "cera_llama_f16_kv_supported": (C.c_int, [vp]),
+            "cera_llama_configure_kv_compression": (C.c_int, [vp, C.c_int]),
             "cera_llama_shift_kv": (C.c_int, [vp, u64, u64]),
             "cera_llama_snapshot_state": (vp, [vp]),
             "cera_llama_snapshot_seq_len": (u64, [vp]),
@@ -162,6 +164,13 @@ class HipLlama:
 
     def truncate_kv(self, n: int):
         self._check(lib().cera_llama_truncate_kv(self.h, n))
+
+    @property
+    def f16_kv_supported(self) -> bool:
+        return bool(lib().cera_llama_f16_kv_supported(self.h))
+
+    def configure_kv_compression(self, f16: bool):
+        self._check(lib().cera_llama_configure_kv_compression(self.h, 1 if f16 else 0))
 
     @property
     def supports_kv_shift(self) -> bool:

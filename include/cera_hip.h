@@ -173,6 +173,16 @@ CERA_HIP_API cera_hip_status cera_hip_attn_prefill(cera_hip_ctx*, const float* q
                                                    uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim,
                                                    uint64_t start_pos, uint32_t n_queries, float scale, float* out);
 
+/* The same two operations over an f16 KV cache (KvCompression::F16; the kernels
+ * cpu::attn_scores_f16 / attn_values_f16 widen on read, cera/src/model/transformer.rs:1170-1196):
+ * k and v arrive as f32 in the layout above and are narrowed to IEEE half (round to nearest
+ * even, as the cache append does, transformer.rs:1435-1446) before the upload.  n_queries = 1 is
+ * the decode step with start_pos + 1 visible keys; n_splits as in cera_hip_attn_decode. */
+CERA_HIP_API cera_hip_status cera_hip_attn_f16kv(cera_hip_ctx*, const float* q, const float* k, const float* v,
+                                                 uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim,
+                                                 uint64_t start_pos, uint32_t n_queries, float scale,
+                                                 uint32_t n_splits, float* out);
+
 /* cpu::rmsnorm (cera/src/backend/cpu.rs:2479-2496), out of place: y = x*inv_rms*w. */
 CERA_HIP_API cera_hip_status cera_hip_rmsnorm(cera_hip_ctx*, const float* x, const float* weight, uint64_t n,
                                               float eps, float* y);
@@ -213,6 +223,12 @@ CERA_HIP_API cera_hip_status cera_hip_attn_decode_dev(cera_hip_ctx*, const float
                                                       const float* v_headmajor, uint32_t n_heads,
                                                       uint32_t n_kv_heads, uint32_t head_dim, uint64_t seq_len,
                                                       uint64_t max_seq, float scale, uint32_t n_splits, float* out);
+/* k, v: device, head-major IEEE half [n_kv_heads][max_seq][head_dim] */
+CERA_HIP_API cera_hip_status cera_hip_attn_decode_f16_dev(cera_hip_ctx*, const float* q, const void* k_headmajor_f16,
+                                                          const void* v_headmajor_f16, uint32_t n_heads,
+                                                          uint32_t n_kv_heads, uint32_t head_dim, uint64_t seq_len,
+                                                          uint64_t max_seq, float scale, uint32_t n_splits,
+                                                          float* out);
 /* out[m][n] = W . quantize(x[n][k]) with x, out on the device. */
 CERA_HIP_API cera_hip_status cera_hip_gemm_dev(cera_hip_ctx*, const cera_hip_dtensor* w, const float* x, uint64_t n,
                                                float* out);
@@ -244,6 +260,16 @@ CERA_HIP_API cera_hip_status cera_hip_forward_prefill(cera_hip_model*, const uin
  * (cera/src/model/mod.rs:221-249).  The LM head is read once for all n positions. */
 CERA_HIP_API cera_hip_status cera_hip_forward_prefill_logits_all(cera_hip_model*, const uint32_t* tokens, uint32_t n,
                                                                  uint32_t start_pos, float* logits_all);
+/* Model::configure_kv_compression for KvCompression::None / ::F16 (cera/src/model/mod.rs:557-592,
+ * cera/src/kv_cache.rs:88-98; f16_kv_supported, mod.rs:594-603): an f16 cache stores K and V as
+ * IEEE half (round to nearest even on append, exact widening on read, f32 accumulation --
+ * cera/src/model/transformer.rs:1424-1447, 1170-1196), halving the bytes decode attention
+ * streams.  Call before the first forward pass: the first call wins, the same mode again is a
+ * no-op, a different mode is CERA_HIP_ERR_ARGUMENT, a non-empty cache CERA_HIP_ERR_POSITION. */
+#define CERA_HIP_KV_F32 0u
+#define CERA_HIP_KV_F16 1u
+CERA_HIP_API cera_hip_status cera_hip_configure_kv(cera_hip_model*, uint32_t kv_type);
+CERA_HIP_API uint32_t cera_hip_kv_type(const cera_hip_model*);
 /* Model::truncate_kv (cera/src/model/mod.rs:251-283). */
 CERA_HIP_API cera_hip_status cera_hip_truncate_kv(cera_hip_model*, uint32_t len);
 CERA_HIP_API uint32_t cera_hip_seq_len(const cera_hip_model*);

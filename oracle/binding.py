@@ -99,6 +99,7 @@ def lib() -> C.CDLL:
         "orc_llama_kcache": (vp, [vp, u32]), "orc_llama_vcache": (vp, [vp, u32]),
         "orc_rope_delta_head": (None, [vp, i32, u32, f32, u32, vp]),
         "orc_llama_shift_kv": (i32, [vp, u32, u32]),
+        "orc_llama_set_kv_f16": (None, [vp, i32]),
         "orc_llama_restore_kv": (i32, [vp, u32, vp, vp, u32]),
         "orc_llama_set_seq_len": (None, [vp, u32]),
     }
@@ -366,6 +367,10 @@ class Llama:
 
     def truncate(self, n: int):
         lib().orc_llama_truncate(self.h, n)
+
+    def set_kv_f16(self, on: bool = True):
+        """KvCompression::F16: K/V rows are rounded through IEEE half when appended."""
+        lib().orc_llama_set_kv_f16(self.h, 1 if on else 0)
 
     def shift_kv(self, n_keep: int, shift: int) -> int:
         """0, or -1 where the reference asserts."""

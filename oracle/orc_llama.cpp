@@ -19,6 +19,10 @@ struct OrcLlama {
     // state (kv_cache.rs:201-221): per layer time-major f32 K and V, [pos][kv_dim]
     std::vector<std::vector<float>> kc, vc;
     uint32_t seq_len = 0;
+    // KvCompression::F16 (kv_cache.rs:93-98): rows are narrowed to half on append and widened on
+    // every read (transformer.rs:1424-1447, llama.rs:1134-1170).  Widening is exact, so the
+    // caches here keep the widened values: same numbers, one code path.
+    bool kv_f16 = false;
     int variant = 0;
     void* pool = nullptr;  // optional worker pool for the GEMVs (timing only)
 };
@@ -43,6 +47,11 @@ OrcLlama* orc_llama_create(const OrcLlamaConfig* cfg, const OrcTensor* embd, con
 }
 void orc_llama_destroy(OrcLlama* m) { delete m; }
 void orc_llama_set_pool(OrcLlama* m, void* pool) { m->pool = pool; }
+void orc_llama_set_kv_f16(OrcLlama* m, int on) { m->kv_f16 = on != 0; }
+static void append_kv(const OrcLlama* m, std::vector<float>& cache, const float* row, uint64_t n) {
+    if (!m->kv_f16) { cache.insert(cache.end(), row, row + n); return; }
+    for (uint64_t i = 0; i < n; ++i) cache.push_back(orc_f16_to_f32(orc_f32_to_f16(row[i])));
+}
 uint32_t orc_llama_seq_len(const OrcLlama* m) { return m->seq_len; }
 void orc_llama_truncate(OrcLlama* m, uint32_t len) {
     if (len >= m->seq_len) return;
@@ -69,8 +78,13 @@ int orc_llama_shift_kv(OrcLlama* m, uint32_t n_keep, uint32_t shift) {
         vc.erase(vc.begin() + n_keep * kv_dim, vc.begin() + (uint64_t(n_keep) + shift) * kv_dim);
         for (uint32_t t = n_keep; t < new_len; ++t)
             for (uint32_t h = 0; h < c.n_kv_heads; ++h)
-                orc_rope_delta_head(kc.data() + t * kv_dim + h * c.head_dim, -int32_t(shift), c.head_dim, c.rope_theta,
-                                    c.rope_type, c.rope_freqs);
+            {
+                float* head = kc.data() + t * kv_dim + h * c.head_dim;
+                orc_rope_delta_head(head, -int32_t(shift), c.head_dim, c.rope_theta, c.rope_type, c.rope_freqs);
+                // f16 cache: widened, rotated, narrowed back (kv_cache.rs:1196-1230)
+                if (m->kv_f16)
+                    for (uint32_t d = 0; d < c.head_dim; ++d) head[d] = orc_f16_to_f32(orc_f32_to_f16(head[d]));
+            }
     }
     m->seq_len = new_len;
     return 0;
@@ -81,8 +95,10 @@ int orc_llama_shift_kv(OrcLlama* m, uint32_t n_keep, uint32_t shift) {
 int orc_llama_restore_kv(OrcLlama* m, uint32_t layer, const float* k, const float* v, uint32_t n_pos) {
     if (layer >= m->cfg.n_layers) return -1;
     const uint64_t n = uint64_t(n_pos) * m->cfg.n_kv_heads * m->cfg.head_dim;
-    m->kc[layer].assign(k, k + n);
-    m->vc[layer].assign(v, v + n);
+    m->kc[layer].clear();
+    m->vc[layer].clear();
+    append_kv(m, m->kc[layer], k, n);
+    append_kv(m, m->vc[layer], v, n);
     return 0;
 }
 void orc_llama_set_seq_len(OrcLlama* m, uint32_t len) { m->seq_len = len; }
@@ -121,8 +137,8 @@ int orc_llama_forward(OrcLlama* m, uint32_t token, uint32_t pos, float* logits, 
         }
         if (c.rope_type == 0) orc_rope_neox(q.data(), k.data(), pos, c.n_heads, c.n_kv_heads, hd, c.rope_theta);
         else orc_rope_norm(q.data(), k.data(), pos, c.n_heads, c.n_kv_heads, hd, c.rope_theta, c.rope_freqs);
-        m->kc[l].insert(m->kc[l].end(), k.begin(), k.end());
-        m->vc[l].insert(m->vc[l].end(), v.begin(), v.end());
+        append_kv(m, m->kc[l], k.data(), k.size());
+        append_kv(m, m->vc[l], v.data(), v.size());
         uint64_t L_ctx = m->kc[l].size() / kv_dim;
         orc_decode_attention(q.data(), m->kc[l].data(), m->vc[l].data(), c.n_heads, c.n_kv_heads, hd,
                              scale, L_ctx, attn_out.data(), m->variant);
@@ -253,8 +269,8 @@ int orc_llama_forward_prefill_batched(OrcLlama* m, const uint32_t* tokens, uint3
             }
             if (c.rope_type == 0) orc_rope_neox(q, k, start_pos + j, c.n_heads, c.n_kv_heads, hd, c.rope_theta);
             else orc_rope_norm(q, k, start_pos + j, c.n_heads, c.n_kv_heads, hd, c.rope_theta, c.rope_freqs);
-            m->kc[l].insert(m->kc[l].end(), k, k + kv_dim);
-            m->vc[l].insert(m->vc[l].end(), v, v + kv_dim);
+            append_kv(m, m->kc[l], k, kv_dim);
+            append_kv(m, m->vc[l], v, kv_dim);
         }
         const float* kcache = m->kc[l].data();
         const float* vcache = m->vc[l].data();

@@ -279,3 +279,31 @@ def test_shift_and_snapshot_through_the_model_layer(tiny_llama, tmp_path):
     with pytest.raises(llama_api.BackendError):
         gm.shift_kv(1, 0)
     assert gm.seq_len == 21
+
+
+def test_f16_kv_through_the_model_layer(tiny_llama, orc):
+    """f16_kv_supported + configure_kv_compression (cera/src/model/mod.rs:557-603), an f16
+    snapshot at half the bytes, and the cross-mode restore gate (cera/src/kv_cache.rs:1411-1421)."""
+    path, cfg, gm32, om32 = tiny_llama
+    gm = llama_api.HipLlama(path, context_size=64)
+    assert gm.f16_kv_supported
+    gm.configure_kv_compression(True)
+    with pytest.raises(llama_api.BackendError):
+        gm.configure_kv_compression(False)
+    _, weights = H.Gguf(path).llama_weights()
+    om = orc.Llama(cfg, weights)
+    om.set_kv_f16(True)
+    toks = [int(t) for t in util.rng(61).integers(0, cfg["vocab"], 18)]
+    _close(gm.forward_prefill(toks, 0), om.forward_prefill_batched(toks, 0), "f16 prefill")
+    _close(gm.forward(4, 18), om.forward(4, 18), "f16 decode")
+    snap = gm.snapshot_state()
+    assert snap.seq_len == 19
+    assert snap.nbytes == cfg["n_layers"] * 2 * 19 * cfg["n_kv_heads"] * cfg["head_dim"] * 2
+    a = gm.forward(8, 19)
+    gm.restore_state(snap)
+    b = gm.forward(8, 19)
+    assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+    gm32.truncate_kv(0)
+    with pytest.raises(llama_api.BackendError):
+        gm32.restore_state(snap)          # an f16 snapshot does not load into an f32 cache
+    gm.close(); om.close(); snap.close()

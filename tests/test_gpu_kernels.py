@@ -327,3 +327,50 @@ def test_attn_decode_config4_long_contexts(hip, orc, L):
     same = hip.attn_decode(q, k, vconst, nh, nkv, hd, L, scale).reshape(nh, hd)
     want = row.reshape(nkv, hd).repeat(nh // nkv, axis=0)
     assert np.abs(same - want).max() <= 2e-6 * float(np.abs(want).max())
+
+
+# ---- attention over an f16 KV cache ----------------------------------------------------
+def _through_half(x):
+    return x.astype(np.float16).astype(np.float32)
+
+
+@pytest.mark.parametrize("L", [1, 9, 65, 512, 1000, 4096, 20000])
+def test_attn_decode_f16_kv_vs_oracle(hip, orc, L):
+    """KvCompression::F16: rows are narrowed to half on append and widened on read
+    (cera/src/model/transformer.rs:1170-1196, 1424-1447), so the reference result is the f32
+    attention of the half-rounded K and V."""
+    nh, nkv, hd = 32, 8, 128
+    _say(f"attn_decode f16 kv L={L}")
+    q = util.make_x(nh * hd, 160)
+    k = util.make_x(L * nkv * hd, 161 + L)
+    v = util.make_x(L * nkv * hd, 162 + L)
+    scale = 1.0 / math.sqrt(hd)
+    out = hip.attn_f16kv(q, k, v, nh, nkv, hd, L - 1, 1, scale).reshape(-1)
+    ref = orc.decode_attention(q, _through_half(k), _through_half(v), nh, nkv, hd, scale, L)
+    err = np.abs(out.astype(np.float64) - ref).max()
+    assert err <= ATTN_TOL * util.rms(ref), (err, util.rms(ref))
+    if L >= 65:
+        # the rounding is really applied: closer to the half-rounded reference than to the f32 one
+        ref32 = orc.decode_attention(q, k, v, nh, nkv, hd, scale, L)
+        assert err < np.abs(out.astype(np.float64) - ref32).max()
+        other = hip.attn_f16kv(q, k, v, nh, nkv, hd, L - 1, 1, scale, n_splits=3).reshape(-1)
+        assert np.abs(other - out).max() <= 1e-5 * max(1.0, float(np.abs(out).max()))
+
+
+@pytest.mark.parametrize("nh,nkv,start,n", [(32, 8, 0, 96), (8, 2, 300, 40), (16, 2, 1000, 33), (4, 4, 5, 3)])
+def test_attn_prefill_f16_kv_vs_oracle(hip, orc, nh, nkv, start, n):
+    hd = 128
+    _say(f"attn_prefill f16 kv nh={nh} nkv={nkv} start={start} n={n}")
+    r = util.rng(11 * n + start)
+    L = start + n
+    q = r.standard_normal((n, nh * hd), dtype=np.float32)
+    k = r.standard_normal(L * nkv * hd, dtype=np.float32)
+    v = r.standard_normal(L * nkv * hd, dtype=np.float32)
+    scale = 1.0 / np.sqrt(hd)
+    out = hip.attn_f16kv(q, k, v, nh, nkv, hd, start, n, scale)
+    kh, vh = _through_half(k), _through_half(v)
+    for i in sorted(set([0, 1, n // 2, n - 1])):
+        Li = start + i + 1
+        ref = orc.decode_attention(q[i], kh[:Li * nkv * hd], vh[:Li * nkv * hd], nh, nkv, hd, scale, Li)
+        err = np.abs(out[i].astype(np.float64) - ref).max()
+        assert err <= ATTN_TOL * util.rms(ref), (i, err, util.rms(ref))

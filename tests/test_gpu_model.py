@@ -219,3 +219,80 @@ def test_decode_continues_after_a_shift(tiny):
     for i, t in enumerate([7, 300, 12, 99]):
         lg, lo = gm.forward(t, 28 + i), om.forward(t, 28 + i)
         assert _cos(lg, lo) > 0.999, i
+
+
+# ---- f16 KV cache -------------------------------------------------------------------------
+def test_f16_kv_cache_model_parity(hip, orc):
+    """configure_kv(F16) before the first forward: prefill, decode and the cache contents track
+    the oracle in the same mode; every cached value is exactly representable in half."""
+    cfg = dict(synth.TINY)
+    weights = synth.make_llama(cfg, seed=1234, sigma=0.05, norm_jitter=0.1)
+    gm = hip_api.Model(hip, cfg, weights)
+    om = orc.Llama(cfg, weights)
+    before = gm.memory_bytes
+    gm.configure_kv(True)
+    om.set_kv_f16(True)
+    assert gm.kv_f16
+    kv_f32 = cfg["n_layers"] * 2 * cfg["n_kv_heads"] * cfg["max_seq_len"] * cfg["head_dim"] * 4
+    assert gm.memory_bytes == before - kv_f32 // 2
+    gm.configure_kv(True)                                  # same mode again: no-op
+    with pytest.raises(hip_api.HipError):
+        gm.configure_kv(False)                             # a different mode: conflict
+    toks = [int(t) for t in util.rng(51).integers(0, cfg["vocab"], 20)]
+    _say("f16 kv: batched prefill 20 + 10 decode steps")
+    lg, lo = gm.forward_prefill(toks, 0), om.forward_prefill_batched(toks, 0)
+    assert _cos(lg, lo) > 0.999
+    for i in range(10):
+        t = int(orc_argmax(lo))
+        lg, lo = gm.forward(t, 20 + i), om.forward(t, 20 + i)
+        assert _cos(lg, lo) > 0.999, i
+    for layer in range(cfg["n_layers"]):
+        kg, vg = gm.read_kv(layer)
+        ko, vo = om.kv(layer)
+        assert np.array_equal(kg, kg.astype(np.float16).astype(np.float32))
+        assert np.array_equal(vg, vg.astype(np.float16).astype(np.float32))
+        tol = 3e-3 if layer == 0 else 5e-2     # one half ulp on top of the f32 bar
+        assert np.abs(kg - ko).max() <= tol * util.rms(ko), layer
+        assert np.abs(vg - vo).max() <= tol * util.rms(vo), layer
+    # per-token prefill (decode kernels appending to the half cache) agrees with the batched route
+    gm.truncate_kv(0)
+    for pos, t in enumerate(toks):
+        lb = gm.forward(t, pos)
+    gm.truncate_kv(0)
+    la = gm.forward_prefill(toks, 0)
+    assert _cos(la, lb) > 0.999
+    gm.close(); om.close()
+
+
+def test_f16_kv_cache_cannot_switch_when_in_use(tiny):
+    cfg, weights, gm, om = tiny
+    gm.truncate_kv(0); om.truncate(0)
+    gm.forward(3, 0); om.forward(3, 0)
+    with pytest.raises(hip_api.HipError) as e:
+        gm.configure_kv(True)
+    assert e.value.status == 5  # CERA_HIP_ERR_POSITION: the cache already holds positions
+    assert not gm.kv_f16
+
+
+@pytest.mark.parametrize("rope_type,seq_len,n_keep,shift", [(1, 24, 5, 7), (0, 40, 3, 10)])
+def test_shift_kv_f16_matches_oracle_bitwise(hip, orc, rope_type, seq_len, n_keep, shift):
+    """f16 caches are widened, delta-rotated in f32 and narrowed back (cera/src/kv_cache.rs:1196-1230)."""
+    from test_oracle_kv_shift import rope_filled_cache
+    cfg = dict(synth.TINY, rope_type=rope_type)
+    weights = synth.make_llama(cfg, seed=5, sigma=0.05)
+    gm = hip_api.Model(hip, cfg, weights)
+    om = orc.Llama(cfg, weights)
+    gm.configure_kv(True); om.set_kv_f16(True)
+    layers, _ = rope_filled_cache(orc, cfg, seq_len, rope_type == 1)
+    om.restore(layers, seq_len)
+    for i, (k, v) in enumerate(layers):
+        gm.write_kv(i, k, v)
+    gm.set_seq_len(seq_len)
+    gm.shift_kv(n_keep, shift)
+    assert om.shift_kv(n_keep, shift) == 0
+    for layer in range(cfg["n_layers"]):
+        kg, vg = gm.read_kv(layer)
+        ko, vo = om.kv(layer)
+        assert np.array_equal(kg.view(np.uint32), ko.view(np.uint32)), layer
+        assert np.array_equal(vg.view(np.uint32), vo.view(np.uint32)), layer
+    gm.close(); om.close()
