@@ -87,7 +87,30 @@ def measure_attention(ctx, hip_api, rng):
         out.append({"context": L, "us_per_call": round(us, 2), "GB/s": round(nbytes / us / 1e3, 1),
                     "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
                     "cache_resident": 2 * n_kv * L * hd * 4 <= 256 << 20})
-    for d in (dk, dv, dchunk, dq, dout):
+    # the same contexts over an f16 KV cache (KvCompression::F16): half the bytes per position
+    chunk16 = chunk.astype(np.float16)
+    dchunk16 = ctx.to_device(chunk16.view(np.uint16))
+    for off in range(0, kv_bytes // 2, chunk16.nbytes):
+        ctx.check(ctx.lib.cera_hip_copy_dev(ctx.h, dk + off, dchunk16, chunk16.nbytes))
+        ctx.check(ctx.lib.cera_hip_copy_dev(ctx.h, dv + off, dchunk16, chunk16.nbytes))
+    for L in (4096, 32768, 131072):
+        call = lambda: ctx.check(ctx.lib.cera_hip_attn_decode_f16_dev(ctx.h, dq, dk, dv, n_heads, n_kv, hd, L, L,
+                                                                      C.c_float(scale), 0, dout))
+        iters = 200 if L <= 4096 else 50
+        for _ in range(5):
+            call()
+        e0, e1 = ctx.event(), ctx.event()
+        ctx.record(e0)
+        for _ in range(iters):
+            call()
+        ctx.record(e1)
+        ctx.sync()
+        us = ctx.elapsed_ms(e0, e1) * 1e3 / iters
+        nbytes = 2 * n_kv * L * hd * 2 + 2 * n_heads * hd * 4
+        out.append({"context": L, "kv": "f16", "us_per_call": round(us, 2), "GB/s": round(nbytes / us / 1e3, 1),
+                    "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
+                    "cache_resident": 2 * n_kv * L * hd * 2 <= 256 << 20})
+    for d in (dk, dv, dchunk, dchunk16, dq, dout):
         ctx.free(d)
     return out
 

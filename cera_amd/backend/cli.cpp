@@ -4,6 +4,7 @@
 //   cera-hip inspect --model m.gguf
 //   cera-hip run     --model m.gguf [--prompt-len 512] [--n-predict 256] [--seed S]
 //                    [--ubatch 512] [--ctx 1024] [--device 0] [--tokens-out FILE] [--per-token-prefill]
+//                    [--kv f32|f16]
 //
 // `run` is the workload `cera bench` times (cera-cli/src/main.rs:932-938 for the
 // protocol): a prompt of uniform random token ids is prefilled in `ubatch`
@@ -123,6 +124,17 @@ int cmd_run(const Args& a) {
         std::fprintf(stderr, "load failed: %s\n", e.what());
         return 1;
     }
+    const std::string kv = a.str("kv", "f32");
+    if (kv != "f32" && kv != "f16") { std::fprintf(stderr, "--kv must be f32 or f16\n"); return 1; }
+    try {
+        if (kv == "f16") {
+            if (!model->f16_kv_supported()) { std::fprintf(stderr, "this backend has no f16 KV cache\n"); return 1; }
+            model->configure_kv_compression(cera::KvCompression::F16);
+        }
+    } catch (const std::exception& e) {
+        std::fprintf(stderr, "configure failed: %s\n", e.what());
+        return 1;
+    }
     double load_s = now_s() - t0;
     const cera::ModelConfig& c = model->config();
     std::vector<uint32_t> prompt(n_prompt);
@@ -164,10 +176,10 @@ int cmd_run(const Args& a) {
     }
     const double decode_steps = n_predict > 1 ? double(n_predict - 1) : 0.0;
     std::printf("{\"arch\": \"%s\", \"n_layers\": %zu, \"hidden\": %zu, \"vocab\": %zu, \"prompt_len\": %zu, "
-                "\"n_predict\": %zu, \"ubatch\": %zu, \"load_s\": %.3f, \"gpu_memory_bytes\": %llu, "
+                "\"n_predict\": %zu, \"ubatch\": %zu, \"kv\": \"%s\", \"load_s\": %.3f, \"gpu_memory_bytes\": %llu, "
                 "\"prefill_s\": %.6f, \"prefill_tok_s\": %.2f, \"decode_s\": %.6f, \"decode_tok_s\": %.2f, "
                 "\"first_tokens\": [%u, %u, %u, %u]}\n",
-                c.architecture.c_str(), c.n_layers, c.hidden_size, c.vocab_size, n_prompt, n_predict, ubatch, load_s,
+                c.architecture.c_str(), c.n_layers, c.hidden_size, c.vocab_size, n_prompt, n_predict, ubatch, kv.c_str(), load_s,
                 static_cast<unsigned long long>(model->gpu_memory_bytes()), prefill_s, n_prompt / prefill_s, decode_s,
                 decode_s > 0 ? decode_steps / decode_s : 0.0, out.size() > 0 ? out[0] : 0, out.size() > 1 ? out[1] : 0,
                 out.size() > 2 ? out[2] : 0, out.size() > 3 ? out[3] : 0);

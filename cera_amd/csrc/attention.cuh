@@ -14,8 +14,9 @@
 // passes for Llama-3's 32/8 heads).
 //
 // Work split: part = one wavefront = `chunks_per_part` chunks of 64 positions.
-// Eight lanes share a position (16 floats each, as four float4 spaced 128 B
-// apart so every load instruction covers whole 128-byte lines); a wavefront
+// Eight lanes share a position (16 values each: of an f32 row four float4 spaced
+// 128 B apart, of a half row two 16-byte runs spaced 128 B apart, so every load
+// instruction covers whole 128-byte lines); a wavefront
 // covers 8 positions per step and 64 per chunk.  The P.V accumulation keeps
 // positions lane-local (lane group g accumulates positions == g mod 8), so the
 // only cross-lane traffic is the 3-step reduction of the q.k partials and one
@@ -37,24 +38,27 @@ struct AttnPart {  // per (part, query head): running max, sum and unnormalised 
 // every wavefront has a single memory round trip (all its K and V loads in
 // flight at once) and there are enough wavefronts to cover the chip; long
 // contexts use 64-position chunks to amortise the softmax bookkeeping.
-// In-place RoPE of the 16 values a lane holds of one 128-wide head (float4 c sits at float4
-// index j + 8c), same arithmetic as rope_kv_kernel.  rope_row = the position's 64 (cos, sin).
+// In-place RoPE of the 16 values a lane holds of one 128-wide head (register quad c is float4
+// column KvOps<KV>::col4(j, c)), same arithmetic as rope_kv_kernel.  rope_row = the position's
+// 64 (cos, sin).
+template <typename KV>
 __device__ __forceinline__ void attn_rope16(float4 (&x)[4], const float* __restrict__ rope_row, uint32_t j, uint32_t rope_type) {
     if (rope_type == 1) {   // NORM: pairs (2i, 2i+1) = (x, y) and (z, w) of each float4
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
-            const float4 cs = reinterpret_cast<const float4*>(rope_row)[j + 8 * c];
+            const float4 cs = reinterpret_cast<const float4*>(rope_row)[KvOps<KV>::col4(j, c)];
             const float4 v = x[c];
             x[c].x = __fsub_rn(__fmul_rn(v.x, cs.x), __fmul_rn(v.y, cs.y));
             x[c].y = __fadd_rn(__fmul_rn(v.x, cs.y), __fmul_rn(v.y, cs.x));
             x[c].z = __fsub_rn(__fmul_rn(v.z, cs.z), __fmul_rn(v.w, cs.w));
             x[c].w = __fadd_rn(__fmul_rn(v.z, cs.w), __fmul_rn(v.w, cs.z));
         }
-    } else {                // NEOX: pairs (i, i + 64): float4 c with float4 c + 2
+    } else {                // NEOX: pairs (i, i + 64); in both layouts quad c + 2 sits 64 columns after quad c
 #pragma unroll
         for (int c = 0; c < 2; ++c) {
-            const float4 c01 = reinterpret_cast<const float4*>(rope_row)[2 * (j + 8 * c)];
-            const float4 c23 = reinterpret_cast<const float4*>(rope_row)[2 * (j + 8 * c) + 1];
+            const uint32_t f = KvOps<KV>::col4(j, c);
+            const float4 c01 = reinterpret_cast<const float4*>(rope_row)[2 * f];
+            const float4 c23 = reinterpret_cast<const float4*>(rope_row)[2 * f + 1];
             const float4 a = x[c], b = x[c + 2];
             x[c].x = __fsub_rn(__fmul_rn(a.x, c01.x), __fmul_rn(b.x, c01.y));
             x[c + 2].x = __fadd_rn(__fmul_rn(a.x, c01.y), __fmul_rn(b.x, c01.x));
@@ -78,15 +82,14 @@ __device__ __forceinline__ void attn_load_v(float4 (&vv)[4], const KV* __restric
     if (NEWKV && tt == new_pos) {
         const float4* vp = reinterpret_cast<const float4*>(nk.v_new + kvh * ATTN_HD);
 #pragma unroll
-        for (int c = 0; c < 4; ++c) vv[c] = KvOps<KV>::rnd4(vp[j + 8 * c]);
+        for (int c = 0; c < 4; ++c) vv[c] = KvOps<KV>::rnd4(vp[KvOps<KV>::col4(j, c)]);
         if (store) {
             KV* dst = static_cast<KV*>(nk.vc_w) + (static_cast<uint64_t>(kvh) * max_seq + t) * ATTN_HD;
 #pragma unroll
-            for (int c = 0; c < 4; ++c) KvOps<KV>::st4(dst, j + 8 * c, vv[c]);
+            for (int c = 0; c < 4; ++c) KvOps<KV>::st4(dst, KvOps<KV>::col4(j, c), vv[c]);
         }
     } else {
-#pragma unroll
-        for (int c = 0; c < 4; ++c) vv[c] = KvOps<KV>::ld4(vbase + static_cast<uint64_t>(tt) * ATTN_HD, j + 8 * c);
+        KvOps<KV>::ld16(vbase + static_cast<uint64_t>(tt) * ATTN_HD, j, vv);
     }
 }
 
@@ -109,10 +112,10 @@ __device__ __forceinline__ void attn_decode_range(const float* __restrict__ q, c
     for (int h = 0; h < G; ++h)
 #pragma unroll
         for (int c = 0; c < 4; ++c)
-            qv[h][c] = reinterpret_cast<const float4*>(q + h * ATTN_HD)[j + 8 * c];
+            qv[h][c] = reinterpret_cast<const float4*>(q + h * ATTN_HD)[KvOps<KV>::col4(j, c)];
     if (NEWKV) {
 #pragma unroll
-        for (int h = 0; h < G; ++h) attn_rope16(qv[h], nk.rope_row, j, nk.rope_type);
+        for (int h = 0; h < G; ++h) attn_rope16<KV>(qv[h], nk.rope_row, j, nk.rope_type);
     }
     const uint32_t new_pos = seq_len - 1;   // NEWKV: the position whose K/V are not in the cache yet
 
@@ -150,18 +153,17 @@ __device__ __forceinline__ void attn_decode_range(const float* __restrict__ q, c
                 // the token's own key: from the projection output, rotated here, narrowed like a cached row
                 const float4* kp = reinterpret_cast<const float4*>(nk.k_new + kvh * ATTN_HD);
 #pragma unroll
-                for (int c = 0; c < 4; ++c) kv[c] = kp[j + 8 * c];
-                attn_rope16(kv, nk.rope_row, j, nk.rope_type);
+                for (int c = 0; c < 4; ++c) kv[c] = kp[KvOps<KV>::col4(j, c)];
+                attn_rope16<KV>(kv, nk.rope_row, j, nk.rope_type);
 #pragma unroll
                 for (int c = 0; c < 4; ++c) kv[c] = KvOps<KV>::rnd4(kv[c]);
                 if (write_new && live) {
                     KV* dst = static_cast<KV*>(nk.kc_w) + (static_cast<uint64_t>(kvh) * max_seq + t) * ATTN_HD;
 #pragma unroll
-                    for (int c = 0; c < 4; ++c) KvOps<KV>::st4(dst, j + 8 * c, kv[c]);
+                    for (int c = 0; c < 4; ++c) KvOps<KV>::st4(dst, KvOps<KV>::col4(j, c), kv[c]);
                 }
             } else {
-#pragma unroll
-                for (int c = 0; c < 4; ++c) kv[c] = KvOps<KV>::ld4(kbase + static_cast<uint64_t>(tt) * ATTN_HD, j + 8 * c);
+                KvOps<KV>::ld16(kbase + static_cast<uint64_t>(tt) * ATTN_HD, j, kv);
             }
 #pragma unroll
             for (int h = 0; h < G; ++h) {
@@ -276,7 +278,7 @@ __global__ __launch_bounds__(256) void attn_decode_partial_kernel(
         for (int h = 0; h < G; ++h) {
             float4* dst = reinterpret_cast<float4*>(part_acc + (base + h) * ATTN_HD);
 #pragma unroll
-            for (int c = 0; c < 4; ++c) dst[j + 8 * c] = acc[h][c];
+            for (int c = 0; c < 4; ++c) dst[KvOps<KV>::col4(j, c)] = acc[h][c];
             if (j == 0) {
                 part_ml[(base + h) * 2] = m[h];
                 part_ml[(base + h) * 2 + 1] = l[h];

@@ -37,17 +37,28 @@ __device__ __forceinline__ uint32_t f2h(float v) {
 // row is appended and widened exactly on every read, accumulation stays f32
 // (cera/src/model/transformer.rs:1424-1447, 1170-1196).
 typedef _Float16 kv_half;
+// col4(j, c) is the float4 column (of the 32 in a 128-wide row) that lane j of an 8-lane group
+// holds as its c-th register quad in the decode attention kernels: chosen per element type so
+// that a lane's loads are 16 bytes wide and the 8 lanes of a load cover whole 128-byte lines.
 template <typename KV> struct KvOps;
 template <> struct KvOps<float> {
     __device__ static __forceinline__ float4 ld4(const float* row, uint32_t i) { return reinterpret_cast<const float4*>(row)[i]; }
     __device__ static __forceinline__ void st4(float* row, uint32_t i, float4 v) { reinterpret_cast<float4*>(row)[i] = v; }
     __device__ static __forceinline__ float4 rnd4(float4 v) { return v; }
     __device__ static __forceinline__ float ld1(const float* p) { return *p; }
+    __device__ static __forceinline__ uint32_t col4(uint32_t j, int c) { return j + 8 * c; }
+    __device__ static __forceinline__ void ld16(const float* row, uint32_t j, float4 (&v)[4]) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) v[c] = reinterpret_cast<const float4*>(row)[j + 8 * c];
+    }
 };
 template <> struct KvOps<kv_half> {
+    __device__ static __forceinline__ float4 cvt4(uint32_t lo, uint32_t hi) {
+        return make_float4(h2f(lo & 0xFFFF), h2f(lo >> 16), h2f(hi & 0xFFFF), h2f(hi >> 16));
+    }
     __device__ static __forceinline__ float4 ld4(const kv_half* row, uint32_t i) {
         const uint2 r = reinterpret_cast<const uint2*>(row)[i];
-        return make_float4(h2f(r.x & 0xFFFF), h2f(r.x >> 16), h2f(r.y & 0xFFFF), h2f(r.y >> 16));
+        return cvt4(r.x, r.y);
     }
     __device__ static __forceinline__ void st4(kv_half* row, uint32_t i, float4 v) {
         reinterpret_cast<uint2*>(row)[i] = make_uint2(f2h(v.x) | (f2h(v.y) << 16), f2h(v.z) | (f2h(v.w) << 16));
@@ -56,6 +67,16 @@ template <> struct KvOps<kv_half> {
         return make_float4(h2f(f2h(v.x)), h2f(f2h(v.y)), h2f(f2h(v.z)), h2f(f2h(v.w)));
     }
     __device__ static __forceinline__ float ld1(const kv_half* p) { return static_cast<float>(*p); }
+    // quads 2c', 2c'+1 are the two halves of one 16-byte load: float4 columns 2(j + 8c'), +1
+    __device__ static __forceinline__ uint32_t col4(uint32_t j, int c) { return 2 * (j + 8 * (c >> 1)) + (c & 1); }
+    __device__ static __forceinline__ void ld16(const kv_half* row, uint32_t j, float4 (&v)[4]) {
+#pragma unroll
+        for (int cc = 0; cc < 2; ++cc) {
+            const uint4 r = reinterpret_cast<const uint4*>(row)[j + 8 * cc];
+            v[2 * cc] = cvt4(r.x, r.y);
+            v[2 * cc + 1] = cvt4(r.z, r.w);
+        }
+    }
 };
 
 // 4 x int8 dot with int32 accumulate (v_dot4_i32_i8).
