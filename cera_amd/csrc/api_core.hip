@@ -409,17 +409,17 @@ struct AttnLaunch {
     AttnNewKV nk;
 };
 
-template <int G, typename KV>
+template <int G, typename KV, int HD>
 static void attn_launch_decode_g(cera_hip_ctx* ctx, const AttnLaunch& a, const KV* kc, const KV* vc) {
     const dim3 grid((a.n_parts + 3) / 4, a.n_kv_heads, a.n_queries), block(256);
 #define ATTN_LAUNCH_S(SS)                                                                                            \
     do {                                                                                                             \
         if (a.fused_new_kv)                                                                                          \
-            hipLaunchKernelGGL((attn_decode_partial_kernel<G, SS, true, KV>), grid, block, 0, ctx->stream, a.q, kc,  \
+            hipLaunchKernelGGL((attn_decode_partial_kernel<G, SS, true, KV, HD>), grid, block, 0, ctx->stream, a.q, kc,  \
                                vc, a.seq_len, a.max_seq, a.scale, a.chunks_per_part, a.n_parts, a.q_stride,          \
                                ctx->attn_acc, ctx->attn_ml, a.nk);                                                   \
         else                                                                                                         \
-            hipLaunchKernelGGL((attn_decode_partial_kernel<G, SS, false, KV>), grid, block, 0, ctx->stream, a.q, kc, \
+            hipLaunchKernelGGL((attn_decode_partial_kernel<G, SS, false, KV, HD>), grid, block, 0, ctx->stream, a.q, kc, \
                                vc, a.seq_len, a.max_seq, a.scale, a.chunks_per_part, a.n_parts, a.q_stride,          \
                                ctx->attn_acc, ctx->attn_ml, a.nk);                                                   \
     } while (0)
@@ -432,21 +432,21 @@ static void attn_launch_decode_g(cera_hip_ctx* ctx, const AttnLaunch& a, const K
 #undef ATTN_LAUNCH_S
 }
 
-template <typename KV>
+template <typename KV, int HD>
 static void attn_launch_partials(cera_hip_ctx* ctx, const AttnLaunch& a, const KV* kc, const KV* vc) {
     if (a.batch) {
         // heaviest query blocks (most visible keys) first
         const dim3 pgrid((a.n_queries + 31) / 32, a.n_heads, a.n_parts);
-        hipLaunchKernelGGL(attn_prefill_partial_kernel<KV>, pgrid, dim3(64), 0, ctx->stream, a.q, kc, vc, a.seq_len,
+        hipLaunchKernelGGL((attn_prefill_partial_kernel<KV, HD>), pgrid, dim3(64), 0, ctx->stream, a.q, kc, vc, a.seq_len,
                            a.n_queries, a.max_seq, a.scale, a.part_keys, a.n_parts, a.q_stride, a.G, ctx->attn_acc,
                            ctx->attn_ml);
         return;
     }
     switch (a.G) {
-        case 1: attn_launch_decode_g<1, KV>(ctx, a, kc, vc); break;
-        case 2: attn_launch_decode_g<2, KV>(ctx, a, kc, vc); break;
-        case 4: attn_launch_decode_g<4, KV>(ctx, a, kc, vc); break;
-        default: attn_launch_decode_g<8, KV>(ctx, a, kc, vc); break;
+        case 1: attn_launch_decode_g<1, KV, HD>(ctx, a, kc, vc); break;
+        case 2: attn_launch_decode_g<2, KV, HD>(ctx, a, kc, vc); break;
+        case 4: attn_launch_decode_g<4, KV, HD>(ctx, a, kc, vc); break;
+        default: attn_launch_decode_g<8, KV, HD>(ctx, a, kc, vc); break;
     }
 }
 
@@ -455,7 +455,7 @@ cera_hip_status cera_launch_attn(cera_hip_ctx* ctx, const float* q, const void* 
                                  uint64_t max_seq, float scale, uint32_t n_splits, uint32_t n_queries, float* out,
                                  float* out_scales, int8_t* out_quants, float* out_bsum, const AttnNewKV* new_kv,
                                  bool kv_f16) {
-    if (head_dim != ATTN_HD) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "attention: head_dim must be 128");
+    if (head_dim != 64 && head_dim != 128) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "attention: head_dim must be 64 or 128");
     if (n_kv_heads == 0 || n_heads % n_kv_heads) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "attention: n_heads must be a multiple of n_kv_heads");
     uint32_t G = n_heads / n_kv_heads;
     if (G != 1 && G != 2 && G != 4 && G != 8) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "attention: group size must be 1, 2, 4 or 8");
@@ -487,7 +487,7 @@ cera_hip_status cera_launch_attn(cera_hip_ctx* ctx, const float* q, const void* 
         chunks_per_part = std::max(1u, (n_chunks + want_parts - 1) / want_parts);
         n_parts = (n_chunks + chunks_per_part - 1) / chunks_per_part;
     }
-    uint64_t acc_bytes = static_cast<uint64_t>(n_queries) * n_kv_heads * n_parts * G * ATTN_HD * sizeof(float);
+    uint64_t acc_bytes = static_cast<uint64_t>(n_queries) * n_kv_heads * n_parts * G * head_dim * sizeof(float);
     uint64_t ml_bytes = static_cast<uint64_t>(n_queries) * n_kv_heads * n_parts * G * 2 * sizeof(float);
     if (ctx->attn_acc_bytes < acc_bytes) {
         HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
@@ -505,17 +505,23 @@ cera_hip_status cera_launch_attn(cera_hip_ctx* ctx, const float* q, const void* 
     }
     AttnLaunch a{q, static_cast<uint32_t>(seq_len), static_cast<uint32_t>(max_seq), scale, n_heads, n_kv_heads, n_queries,
                  n_heads * head_dim, G, S, n_parts, part_keys, chunks_per_part, batch, new_kv != nullptr, nk};
-    if (kv_f16) attn_launch_partials<kv_half>(ctx, a, static_cast<const kv_half*>(kc), static_cast<const kv_half*>(vc));
-    else attn_launch_partials<float>(ctx, a, static_cast<const float*>(kc), static_cast<const float*>(vc));
+    const kv_half *kh = static_cast<const kv_half*>(kc), *vh = static_cast<const kv_half*>(vc);
+    const float *kf = static_cast<const float*>(kc), *vf = static_cast<const float*>(vc);
+    if (head_dim == 128) {
+        if (kv_f16) attn_launch_partials<kv_half, 128>(ctx, a, kh, vh);
+        else attn_launch_partials<float, 128>(ctx, a, kf, vf);
+    } else {
+        if (kv_f16) attn_launch_partials<kv_half, 64>(ctx, a, kh, vh);
+        else attn_launch_partials<float, 64>(ctx, a, kf, vf);
+    }
     HIP_TRY(ctx, hipGetLastError());
     dim3 mgrid(n_heads, n_queries);
-    if (out_quants)
-        hipLaunchKernelGGL((attn_decode_merge_kernel<true>), mgrid, dim3(256), 0, ctx->stream, ctx->attn_acc,
-                           ctx->attn_ml, n_parts, G, n_heads, out, out_scales, out_quants, out_bsum);
-    else
-        hipLaunchKernelGGL((attn_decode_merge_kernel<false>), mgrid, dim3(256), 0, ctx->stream, ctx->attn_acc,
-                           ctx->attn_ml, n_parts, G, n_heads, out, static_cast<float*>(nullptr),
-                           static_cast<int8_t*>(nullptr), static_cast<float*>(nullptr));
+#define ATTN_MERGE(QQ, HH)                                                                                              \
+    hipLaunchKernelGGL((attn_decode_merge_kernel<QQ, HH>), mgrid, dim3(256), 0, ctx->stream, ctx->attn_acc, ctx->attn_ml, \
+                       n_parts, G, n_heads, out, out_scales, out_quants, out_bsum)
+    if (out_quants) { if (head_dim == 128) ATTN_MERGE(true, 128); else ATTN_MERGE(true, 64); }
+    else            { if (head_dim == 128) ATTN_MERGE(false, 128); else ATTN_MERGE(false, 64); }
+#undef ATTN_MERGE
     HIP_TRY(ctx, hipGetLastError());
     return CERA_HIP_OK;
 }

@@ -26,7 +26,6 @@
 #include "attn_types.h"
 #include "quantize.cuh"
 
-#define ATTN_HD 128
 #define ATTN_MAX_PARTS 1024  // the merge kernel keeps one weight per part in LDS
 #define ATTN_MERGE_PF 4       // parts per lane group the merge kernel requests up front (x8 groups)
 
@@ -34,40 +33,68 @@ struct AttnPart {  // per (part, query head): running max, sum and unnormalised 
     float m, l;
 };
 
+// Which columns of a head_dim-wide row a lane of an 8-lane position group holds, and how it loads
+// them.  A lane keeps NQ = head_dim / 32 register quads; quad c is float4 column col4(j, c).  The
+// mapping is chosen per (element type, head_dim) so that loads are as wide as possible, the 8
+// lanes of a load cover whole 128-byte lines, and the NEOX partner of quad c (head_dim / 2
+// columns on) is quad c + NQ / 2 of the same lane.
+template <typename KV, int HD> struct AttnLay {   // f32 rows, and half rows of 64
+    static constexpr int NQ = HD / 32;
+    __device__ static __forceinline__ uint32_t col4(uint32_t j, int c) { return j + 8 * c; }
+    __device__ static __forceinline__ void ld(const KV* row, uint32_t j, float4 (&v)[NQ]) {
+#pragma unroll
+        for (int c = 0; c < NQ; ++c) v[c] = KvOps<KV>::ld4(row, j + 8 * c);
+    }
+};
+template <> struct AttnLay<kv_half, 128> {         // two 16-byte loads per row: quads 2c', 2c'+1 together
+    static constexpr int NQ = 4;
+    __device__ static __forceinline__ uint32_t col4(uint32_t j, int c) { return 2 * (j + 8 * (c >> 1)) + (c & 1); }
+    __device__ static __forceinline__ void ld(const kv_half* row, uint32_t j, float4 (&v)[4]) {
+#pragma unroll
+        for (int cc = 0; cc < 2; ++cc) {
+            const uint4 r = reinterpret_cast<const uint4*>(row)[j + 8 * cc];
+            v[2 * cc] = KvOps<kv_half>::cvt4(r.x, r.y);
+            v[2 * cc + 1] = KvOps<kv_half>::cvt4(r.z, r.w);
+        }
+    }
+};
+
 // S = steps of 8 positions per chunk.  Short contexts use small chunks so that
 // every wavefront has a single memory round trip (all its K and V loads in
 // flight at once) and there are enough wavefronts to cover the chip; long
 // contexts use 64-position chunks to amortise the softmax bookkeeping.
-// In-place RoPE of the 16 values a lane holds of one 128-wide head (register quad c is float4
-// column KvOps<KV>::col4(j, c)), same arithmetic as rope_kv_kernel.  rope_row = the position's
-// 64 (cos, sin).
-template <typename KV>
-__device__ __forceinline__ void attn_rope16(float4 (&x)[4], const float* __restrict__ rope_row, uint32_t j, uint32_t rope_type) {
+// In-place RoPE of the values a lane holds of one head (register quad c is float4 column
+// Lay::col4(j, c)), same arithmetic as rope_kv_kernel.  rope_row = the position's head_dim / 2
+// (cos, sin) pairs.
+template <typename Lay>
+__device__ __forceinline__ void attn_rope16(float4 (&x)[Lay::NQ], const float* __restrict__ rope_row, uint32_t j, uint32_t rope_type) {
+    constexpr int NQ = Lay::NQ;
     if (rope_type == 1) {   // NORM: pairs (2i, 2i+1) = (x, y) and (z, w) of each float4
 #pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            const float4 cs = reinterpret_cast<const float4*>(rope_row)[KvOps<KV>::col4(j, c)];
+        for (int c = 0; c < NQ; ++c) {
+            const float4 cs = reinterpret_cast<const float4*>(rope_row)[Lay::col4(j, c)];
             const float4 v = x[c];
             x[c].x = __fsub_rn(__fmul_rn(v.x, cs.x), __fmul_rn(v.y, cs.y));
             x[c].y = __fadd_rn(__fmul_rn(v.x, cs.y), __fmul_rn(v.y, cs.x));
             x[c].z = __fsub_rn(__fmul_rn(v.z, cs.z), __fmul_rn(v.w, cs.w));
             x[c].w = __fadd_rn(__fmul_rn(v.z, cs.w), __fmul_rn(v.w, cs.z));
         }
-    } else {                // NEOX: pairs (i, i + 64); in both layouts quad c + 2 sits 64 columns after quad c
+    } else {                // NEOX: pairs (i, i + head_dim / 2): quad c with quad c + NQ / 2
+        constexpr int H2 = NQ / 2;
 #pragma unroll
-        for (int c = 0; c < 2; ++c) {
-            const uint32_t f = KvOps<KV>::col4(j, c);
+        for (int c = 0; c < H2; ++c) {
+            const uint32_t f = Lay::col4(j, c);
             const float4 c01 = reinterpret_cast<const float4*>(rope_row)[2 * f];
             const float4 c23 = reinterpret_cast<const float4*>(rope_row)[2 * f + 1];
-            const float4 a = x[c], b = x[c + 2];
+            const float4 a = x[c], b = x[c + H2];
             x[c].x = __fsub_rn(__fmul_rn(a.x, c01.x), __fmul_rn(b.x, c01.y));
-            x[c + 2].x = __fadd_rn(__fmul_rn(a.x, c01.y), __fmul_rn(b.x, c01.x));
+            x[c + H2].x = __fadd_rn(__fmul_rn(a.x, c01.y), __fmul_rn(b.x, c01.x));
             x[c].y = __fsub_rn(__fmul_rn(a.y, c01.z), __fmul_rn(b.y, c01.w));
-            x[c + 2].y = __fadd_rn(__fmul_rn(a.y, c01.w), __fmul_rn(b.y, c01.z));
+            x[c + H2].y = __fadd_rn(__fmul_rn(a.y, c01.w), __fmul_rn(b.y, c01.z));
             x[c].z = __fsub_rn(__fmul_rn(a.z, c23.x), __fmul_rn(b.z, c23.y));
-            x[c + 2].z = __fadd_rn(__fmul_rn(a.z, c23.y), __fmul_rn(b.z, c23.x));
+            x[c + H2].z = __fadd_rn(__fmul_rn(a.z, c23.y), __fmul_rn(b.z, c23.x));
             x[c].w = __fsub_rn(__fmul_rn(a.w, c23.z), __fmul_rn(b.w, c23.w));
-            x[c + 2].w = __fadd_rn(__fmul_rn(a.w, c23.w), __fmul_rn(b.w, c23.z));
+            x[c + H2].w = __fadd_rn(__fmul_rn(a.w, c23.w), __fmul_rn(b.w, c23.z));
         }
     }
 }
@@ -75,21 +102,23 @@ __device__ __forceinline__ void attn_rope16(float4 (&x)[4], const float* __restr
 // This lane's 16 columns of the V row of position tt; the token's own row comes from the
 // projection output (narrowed like a cached row) and is stored into the cache by the one
 // caller that owns the append.
-template <bool NEWKV, typename KV>
-__device__ __forceinline__ void attn_load_v(float4 (&vv)[4], const KV* __restrict__ vbase, uint32_t t, uint32_t tt,
+template <bool NEWKV, typename KV, int HD>
+__device__ __forceinline__ void attn_load_v(float4 (&vv)[HD / 32], const KV* __restrict__ vbase, uint32_t t, uint32_t tt,
                                             uint32_t new_pos, uint32_t kvh, uint32_t max_seq, uint32_t j,
                                             const AttnNewKV& nk, bool store) {
+    using Lay = AttnLay<KV, HD>;
+    constexpr int NQ = Lay::NQ;
     if (NEWKV && tt == new_pos) {
-        const float4* vp = reinterpret_cast<const float4*>(nk.v_new + kvh * ATTN_HD);
+        const float4* vp = reinterpret_cast<const float4*>(nk.v_new + kvh * HD);
 #pragma unroll
-        for (int c = 0; c < 4; ++c) vv[c] = KvOps<KV>::rnd4(vp[KvOps<KV>::col4(j, c)]);
+        for (int c = 0; c < NQ; ++c) vv[c] = KvOps<KV>::rnd4(vp[Lay::col4(j, c)]);
         if (store) {
-            KV* dst = static_cast<KV*>(nk.vc_w) + (static_cast<uint64_t>(kvh) * max_seq + t) * ATTN_HD;
+            KV* dst = static_cast<KV*>(nk.vc_w) + (static_cast<uint64_t>(kvh) * max_seq + t) * HD;
 #pragma unroll
-            for (int c = 0; c < 4; ++c) KvOps<KV>::st4(dst, KvOps<KV>::col4(j, c), vv[c]);
+            for (int c = 0; c < NQ; ++c) KvOps<KV>::st4(dst, Lay::col4(j, c), vv[c]);
         }
     } else {
-        KvOps<KV>::ld16(vbase + static_cast<uint64_t>(tt) * ATTN_HD, j, vv);
+        Lay::ld(vbase + static_cast<uint64_t>(tt) * HD, j, vv);
     }
 }
 
@@ -98,24 +127,26 @@ __device__ __forceinline__ void attn_load_v(float4 (&vv)[4], const KV* __restric
 // the eight position groups already folded: every lane holds its 16 columns of acc and the
 // wavefront-wide m and l.  `q` points at the first of the G heads; `write_new` says whether
 // this caller stores the new position's K/V row into the cache (NEWKV only).
-template <int G, int S, bool NEWKV, typename KV>
+template <int G, int S, bool NEWKV, typename KV, int HD>
 __device__ __forceinline__ void attn_decode_range(const float* __restrict__ q, const KV* __restrict__ kbase,
                                                   const KV* __restrict__ vbase, uint32_t kvh, uint32_t max_seq,
                                                   uint32_t seq_len, uint32_t t_begin, uint32_t t_end, uint32_t t_step,
                                                   float scale, const AttnNewKV& nk, bool write_new, uint32_t lane,
-                                                  float4 (&acc)[G][4], float (&m)[G], float (&l)[G]) {
+                                                  float4 (&acc)[G][HD / 32], float (&m)[G], float (&l)[G]) {
+    using Lay = AttnLay<KV, HD>;
+    constexpr int NQ = Lay::NQ;
     const uint32_t j = lane & 7, pg = lane >> 3;  // float4 column group, position group
 
     // this lane's 16 q values for each of the G heads
-    float4 qv[G][4];
+    float4 qv[G][NQ];
 #pragma unroll
     for (int h = 0; h < G; ++h)
 #pragma unroll
-        for (int c = 0; c < 4; ++c)
-            qv[h][c] = reinterpret_cast<const float4*>(q + h * ATTN_HD)[KvOps<KV>::col4(j, c)];
+        for (int c = 0; c < NQ; ++c)
+            qv[h][c] = reinterpret_cast<const float4*>(q + h * HD)[Lay::col4(j, c)];
     if (NEWKV) {
 #pragma unroll
-        for (int h = 0; h < G; ++h) attn_rope16<KV>(qv[h], nk.rope_row, j, nk.rope_type);
+        for (int h = 0; h < G; ++h) attn_rope16<Lay>(qv[h], nk.rope_row, j, nk.rope_type);
     }
     const uint32_t new_pos = seq_len - 1;   // NEWKV: the position whose K/V are not in the cache yet
 
@@ -124,7 +155,7 @@ __device__ __forceinline__ void attn_decode_range(const float* __restrict__ q, c
         m[h] = -__builtin_inff();
         l[h] = 0.0f;
 #pragma unroll
-        for (int c = 0; c < 4; ++c) acc[h][c] = make_float4(0.f, 0.f, 0.f, 0.f);
+        for (int c = 0; c < NQ; ++c) acc[h][c] = make_float4(0.f, 0.f, 0.f, 0.f);
     }
 
     constexpr uint32_t CHUNK = 8 * S;
@@ -132,12 +163,12 @@ __device__ __forceinline__ void attn_decode_range(const float* __restrict__ q, c
     // a lane past t_end re-reads the range's first position (from the cache, or the new row if
     // that is the one not stored yet) and gets a dead score
     for (uint32_t t0 = t_begin; t0 < t_end; t0 += t_step) {
-        float4 vpre[PREFETCH_V ? S : 1][4];
+        float4 vpre[PREFETCH_V ? S : 1][NQ];
         if (PREFETCH_V) {
 #pragma unroll
             for (int s = 0; s < S; ++s) {
                 const uint32_t t = t0 + 8 * s + pg;
-                attn_load_v<NEWKV, KV>(vpre[s], vbase, t, t < t_end ? t : t_begin, new_pos, kvh, max_seq, j, nk,
+                attn_load_v<NEWKV, KV, HD>(vpre[s], vbase, t, t < t_end ? t : t_begin, new_pos, kvh, max_seq, j, nk,
                                        write_new && t == new_pos);
             }
         }
@@ -148,28 +179,28 @@ __device__ __forceinline__ void attn_decode_range(const float* __restrict__ q, c
             const uint32_t t = t0 + 8 * s + pg;
             const bool live = t < t_end;
             const uint32_t tt = live ? t : t_begin;
-            float4 kv[4];
+            float4 kv[NQ];
             if (NEWKV && tt == new_pos) {
                 // the token's own key: from the projection output, rotated here, narrowed like a cached row
-                const float4* kp = reinterpret_cast<const float4*>(nk.k_new + kvh * ATTN_HD);
+                const float4* kp = reinterpret_cast<const float4*>(nk.k_new + kvh * HD);
 #pragma unroll
-                for (int c = 0; c < 4; ++c) kv[c] = kp[KvOps<KV>::col4(j, c)];
-                attn_rope16<KV>(kv, nk.rope_row, j, nk.rope_type);
+                for (int c = 0; c < NQ; ++c) kv[c] = kp[Lay::col4(j, c)];
+                attn_rope16<Lay>(kv, nk.rope_row, j, nk.rope_type);
 #pragma unroll
-                for (int c = 0; c < 4; ++c) kv[c] = KvOps<KV>::rnd4(kv[c]);
+                for (int c = 0; c < NQ; ++c) kv[c] = KvOps<KV>::rnd4(kv[c]);
                 if (write_new && live) {
-                    KV* dst = static_cast<KV*>(nk.kc_w) + (static_cast<uint64_t>(kvh) * max_seq + t) * ATTN_HD;
+                    KV* dst = static_cast<KV*>(nk.kc_w) + (static_cast<uint64_t>(kvh) * max_seq + t) * HD;
 #pragma unroll
-                    for (int c = 0; c < 4; ++c) KvOps<KV>::st4(dst, KvOps<KV>::col4(j, c), kv[c]);
+                    for (int c = 0; c < NQ; ++c) KvOps<KV>::st4(dst, Lay::col4(j, c), kv[c]);
                 }
             } else {
-                KvOps<KV>::ld16(kbase + static_cast<uint64_t>(tt) * ATTN_HD, j, kv);
+                Lay::ld(kbase + static_cast<uint64_t>(tt) * HD, j, kv);
             }
 #pragma unroll
             for (int h = 0; h < G; ++h) {
                 float d = 0.0f;
 #pragma unroll
-                for (int c = 0; c < 4; ++c) {
+                for (int c = 0; c < NQ; ++c) {
                     d = fmaf(qv[h][c].x, kv[c].x, d);
                     d = fmaf(qv[h][c].y, kv[c].y, d);
                     d = fmaf(qv[h][c].z, kv[c].z, d);
@@ -194,7 +225,7 @@ __device__ __forceinline__ void attn_decode_range(const float* __restrict__ q, c
             m[h] = m_new;
             l[h] *= corr[h];
 #pragma unroll
-            for (int c = 0; c < 4; ++c) {
+            for (int c = 0; c < NQ; ++c) {
                 acc[h][c].x *= corr[h]; acc[h][c].y *= corr[h];
                 acc[h][c].z *= corr[h]; acc[h][c].w *= corr[h];
             }
@@ -202,13 +233,13 @@ __device__ __forceinline__ void attn_decode_range(const float* __restrict__ q, c
         // ---- P.V: this lane's positions, its 16 columns
 #pragma unroll
         for (int s = 0; s < S; ++s) {
-            float4 vv[4];
+            float4 vv[NQ];
             if (PREFETCH_V) {
 #pragma unroll
-                for (int c = 0; c < 4; ++c) vv[c] = vpre[s][c];
+                for (int c = 0; c < NQ; ++c) vv[c] = vpre[s][c];
             } else {
                 const uint32_t t = t0 + 8 * s + pg;
-                attn_load_v<NEWKV, KV>(vv, vbase, t, t < t_end ? t : t_begin, new_pos, kvh, max_seq, j, nk,
+                attn_load_v<NEWKV, KV, HD>(vv, vbase, t, t < t_end ? t : t_begin, new_pos, kvh, max_seq, j, nk,
                                        write_new && t == new_pos);
             }
 #pragma unroll
@@ -217,7 +248,7 @@ __device__ __forceinline__ void attn_decode_range(const float* __restrict__ q, c
                 // all 8 lanes of a position add the same p; count it once (lane j == 0)
                 l[h] += (j == 0) ? p : 0.0f;
 #pragma unroll
-                for (int c = 0; c < 4; ++c) {
+                for (int c = 0; c < NQ; ++c) {
                     acc[h][c].x = fmaf(p, vv[c].x, acc[h][c].x);
                     acc[h][c].y = fmaf(p, vv[c].y, acc[h][c].y);
                     acc[h][c].z = fmaf(p, vv[c].z, acc[h][c].z);
@@ -232,7 +263,7 @@ __device__ __forceinline__ void attn_decode_range(const float* __restrict__ q, c
     for (int h = 0; h < G; ++h) {
         l[h] = wave_sum(l[h]);
 #pragma unroll
-        for (int c = 0; c < 4; ++c) {
+        for (int c = 0; c < NQ; ++c) {
             float* f = reinterpret_cast<float*>(&acc[h][c]);
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
@@ -246,7 +277,7 @@ __device__ __forceinline__ void attn_decode_range(const float* __restrict__ q, c
     }
 }
 
-template <int G, int S, bool NEWKV, typename KV>
+template <int G, int S, bool NEWKV, typename KV, int HD>
 __global__ __launch_bounds__(256) void attn_decode_partial_kernel(
     const float* __restrict__ q,       // [n_heads][128]
     const KV* __restrict__ kc,         // [n_kv][max_seq][128]
@@ -262,23 +293,25 @@ __global__ __launch_bounds__(256) void attn_decode_partial_kernel(
     if (part >= n_parts) return;
     // causal prefill: query qi sits at position seq_len - 1 + qi and sees seq_len + qi keys
     seq_len += qi;
-    q += static_cast<uint64_t>(qi) * q_stride + kvh * G * ATTN_HD;
+    q += static_cast<uint64_t>(qi) * q_stride + kvh * G * HD;
+    using Lay = AttnLay<KV, HD>;
+    constexpr int NQ = Lay::NQ;
     const uint32_t j = lane & 7, pg = lane >> 3;
     constexpr uint32_t CHUNK = 8 * S;
     const uint32_t t_begin = part * chunks_per_part * CHUNK;
     const uint32_t t_end = min(seq_len, t_begin + chunks_per_part * CHUNK);
-    float4 acc[G][4];
+    float4 acc[G][NQ];
     float m[G], l[G];
-    attn_decode_range<G, S, NEWKV, KV>(q, kc + static_cast<uint64_t>(kvh) * max_seq * ATTN_HD,
-                                   vc + static_cast<uint64_t>(kvh) * max_seq * ATTN_HD, kvh, max_seq, seq_len, t_begin,
+    attn_decode_range<G, S, NEWKV, KV, HD>(q, kc + static_cast<uint64_t>(kvh) * max_seq * HD,
+                                   vc + static_cast<uint64_t>(kvh) * max_seq * HD, kvh, max_seq, seq_len, t_begin,
                                    t_end, CHUNK, scale, nk, true, lane, acc, m, l);
     if (pg == 0) {
         uint64_t base = ((static_cast<uint64_t>(qi) * gridDim.y + kvh) * n_parts + part) * G;
 #pragma unroll
         for (int h = 0; h < G; ++h) {
-            float4* dst = reinterpret_cast<float4*>(part_acc + (base + h) * ATTN_HD);
+            float4* dst = reinterpret_cast<float4*>(part_acc + (base + h) * HD);
 #pragma unroll
-            for (int c = 0; c < 4; ++c) dst[KvOps<KV>::col4(j, c)] = acc[h][c];
+            for (int c = 0; c < NQ; ++c) dst[Lay::col4(j, c)] = acc[h][c];
             if (j == 0) {
                 part_ml[(base + h) * 2] = m[h];
                 part_ml[(base + h) * 2 + 1] = l[h];
@@ -315,7 +348,7 @@ __global__ __launch_bounds__(256) void attn_decode_partial_kernel(
 #define ATTN_PF_LD 33  // words per LDS row of the transposed K tile (32 + 1 pad)
 typedef float attn_v16f __attribute__((ext_vector_type(16)));
 
-template <typename KV>
+template <typename KV, int HD>
 __global__ __launch_bounds__(64) void attn_prefill_partial_kernel(
     const float* __restrict__ q,       // [n_queries][q_stride]
     const KV* __restrict__ kc,         // [n_kv][max_seq][128], already holding the batch's keys
@@ -325,7 +358,7 @@ __global__ __launch_bounds__(64) void attn_prefill_partial_kernel(
     uint32_t G,
     float* __restrict__ part_acc,      // [n_queries][n_kv][n_parts][G][128]
     float* __restrict__ part_ml) {     // [n_queries][n_kv][n_parts][G][2]
-    __shared__ float sKt[ATTN_HD * ATTN_PF_LD];
+    __shared__ float sKt[HD * ATTN_PF_LD];
     __shared__ __attribute__((aligned(16))) float sX[32];
     const uint32_t lane = threadIdx.x, col = lane & 31, half = lane >> 5;
     const uint32_t head = blockIdx.y, kvh = head / G, hg = head % G, n_kv = gridDim.y / G;
@@ -337,31 +370,32 @@ __global__ __launch_bounds__(64) void attn_prefill_partial_kernel(
     const uint32_t key_lo = part * part_keys;
     const uint32_t key_hi = min(key_lo + part_keys, block_len);
 
-    const KV* kbase = kc + static_cast<uint64_t>(kvh) * max_seq * ATTN_HD;
-    const KV* vbase = vc + static_cast<uint64_t>(kvh) * max_seq * ATTN_HD;
+    const KV* kbase = kc + static_cast<uint64_t>(kvh) * max_seq * HD;
+    const KV* vbase = vc + static_cast<uint64_t>(kvh) * max_seq * HD;
 
     // this lane's query, the dims of its half: d = 2s + half
-    float qreg[64];
+    float qreg[HD / 2];
     {
-        const float* qp = q + static_cast<uint64_t>(min(qidx, n_queries - 1)) * q_stride + head * ATTN_HD + half;
+        const float* qp = q + static_cast<uint64_t>(min(qidx, n_queries - 1)) * q_stride + head * HD + half;
 #pragma unroll
-        for (int s = 0; s < 64; ++s) qreg[s] = qp[2 * s];
+        for (int s = 0; s < HD / 2; ++s) qreg[s] = qp[2 * s];
     }
-    attn_v16f acc[4];
+    constexpr int NDT = HD / 32;   // 32-column output tiles
+    attn_v16f acc[NDT];
 #pragma unroll
-    for (int dt = 0; dt < 4; ++dt)
+    for (int dt = 0; dt < NDT; ++dt)
 #pragma unroll
         for (int e = 0; e < 16; ++e) acc[dt][e] = 0.0f;
     float m = -__builtin_inff();
     double l = 0.0;
 
     for (uint32_t k0 = key_lo; k0 < key_hi; k0 += 32) {
-        // ---- K tile -> LDS, transposed: 32 keys x 32 float4, 16 per lane
+        // ---- K tile -> LDS, transposed: 32 keys x HD/4 float4, HD/8 per lane
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const uint32_t f = lane + 64 * i, key = f >> 5, c4 = f & 31;
+        for (int i = 0; i < HD / 8; ++i) {
+            const uint32_t f = lane + 64 * i, key = f / (HD / 4), c4 = f % (HD / 4);
             float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (k0 + key < key_hi) v = KvOps<KV>::ld4(kbase + static_cast<uint64_t>(k0 + key) * ATTN_HD, c4);
+            if (k0 + key < key_hi) v = KvOps<KV>::ld4(kbase + static_cast<uint64_t>(k0 + key) * HD, c4);
             sKt[(4 * c4 + 0) * ATTN_PF_LD + key] = v.x;
             sKt[(4 * c4 + 1) * ATTN_PF_LD + key] = v.y;
             sKt[(4 * c4 + 2) * ATTN_PF_LD + key] = v.z;
@@ -373,7 +407,7 @@ __global__ __launch_bounds__(64) void attn_prefill_partial_kernel(
 #pragma unroll
         for (int e = 0; e < 16; ++e) c[e] = 0.0f;
 #pragma unroll
-        for (int s = 0; s < 64; ++s)
+        for (int s = 0; s < HD / 2; ++s)
             c = __builtin_amdgcn_mfma_f32_32x32x2f32(sKt[(2 * s + half) * ATTN_PF_LD + col], qreg[s], c, 0, 0, 0);
         float mx = -__builtin_inff();
 #pragma unroll
@@ -404,7 +438,7 @@ __global__ __launch_bounds__(64) void attn_prefill_partial_kernel(
             const float4 cr = *reinterpret_cast<const float4*>(sX + 8 * blk + 4 * half);
             const float crv[4] = {cr.x, cr.y, cr.z, cr.w};
 #pragma unroll
-            for (int dt = 0; dt < 4; ++dt)
+            for (int dt = 0; dt < NDT; ++dt)
 #pragma unroll
                 for (int r = 0; r < 4; ++r) acc[dt][4 * blk + r] *= crv[r];
         }
@@ -412,9 +446,9 @@ __global__ __launch_bounds__(64) void attn_prefill_partial_kernel(
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
             const uint32_t kg = min(k0 + 8 * (e >> 2) + 4 * half + (e & 3), key_hi - 1);   // masked keys have p = 0
-            const KV* vrow = vbase + static_cast<uint64_t>(kg) * ATTN_HD + col;
+            const KV* vrow = vbase + static_cast<uint64_t>(kg) * HD + col;
 #pragma unroll
-            for (int dt = 0; dt < 4; ++dt)
+            for (int dt = 0; dt < NDT; ++dt)
                 acc[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(c[e], KvOps<KV>::ld1(vrow + 32 * dt), acc[dt], 0, 0, 0);
         }
         __syncthreads();   // sKt and sX are rewritten by the next tile
@@ -427,9 +461,9 @@ __global__ __launch_bounds__(64) void attn_prefill_partial_kernel(
         for (int r = 0; r < 4; ++r) {
             const uint32_t qi = q0 + 8 * blk + 4 * half + r;
             if (qi < n_queries) {
-                float* dst = part_acc + (((static_cast<uint64_t>(qi) * n_kv + kvh) * n_parts + part) * G + hg) * ATTN_HD + col;
+                float* dst = part_acc + (((static_cast<uint64_t>(qi) * n_kv + kvh) * n_parts + part) * G + hg) * HD + col;
 #pragma unroll
-                for (int dt = 0; dt < 4; ++dt) dst[32 * dt] = acc[dt][4 * blk + r];
+                for (int dt = 0; dt < NDT; ++dt) dst[32 * dt] = acc[dt][4 * blk + r];
             }
         }
     if (half == 0 && q_live) {
@@ -442,11 +476,11 @@ __global__ __launch_bounds__(64) void attn_prefill_partial_kernel(
 // Merge the parts of one query head: out = sum_p e^{m_p - M} acc_p / sum_p e^{m_p - M} l_p.
 // One workgroup of 256 threads per (head, query): the maxima and weights are
 // computed with the parts spread over all threads, the weighted accumulation
-// with the parts spread over 8 groups of 32 lanes (a float4 of the 128 columns
-// per lane), so the dependent-load chain is n_parts / 8 long.  Group 0 folds
+// with the parts spread over 8 groups of 32 lanes (a float4 of the head's columns
+// per lane; half of each group idles when head_dim is 64), so the dependent-load chain is n_parts / 8 long.  Group 0 folds
 // the groups together and optionally writes the Q8_0 quantisation of the
 // result for the output projection.
-template <bool QUANT>
+template <bool QUANT, int HD>
 __global__ __launch_bounds__(256) void attn_decode_merge_kernel(const float* __restrict__ part_acc,
                                                                 const float* __restrict__ part_ml,
                                                                 uint32_t n_parts, uint32_t G, uint32_t n_heads,
@@ -460,13 +494,15 @@ __global__ __launch_bounds__(256) void attn_decode_merge_kernel(const float* __r
     const uint32_t head = blockIdx.x, tid = threadIdx.x, c = tid & 31, grp = tid >> 5, wave = tid >> 6;
     const uint32_t kvh = head / G, hg = head % G, qi = blockIdx.y, n_kv = n_heads / G;
     const uint64_t pbase = (static_cast<uint64_t>(qi) * n_kv + kvh) * n_parts;
+    constexpr uint32_t C4 = HD / 4;          // float4 columns of a head; lanes c >= C4 of a group idle
+    const bool live = c < C4;
     // the first ATTN_MERGE_PF parts of this group are requested before anything depends on them
     float4 pre[ATTN_MERGE_PF];
 #pragma unroll
     for (int i = 0; i < ATTN_MERGE_PF; ++i) {
         const uint32_t p = grp + 8 * i;
         pre[i] = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (p < n_parts) pre[i] = reinterpret_cast<const float4*>(part_acc + ((pbase + p) * G + hg) * ATTN_HD)[c];
+        if (p < n_parts && live) pre[i] = reinterpret_cast<const float4*>(part_acc + ((pbase + p) * G + hg) * HD)[c];
     }
     float M = -__builtin_inff();
     for (uint32_t p = tid; p < n_parts; p += 256) M = fmaxf(M, part_ml[((pbase + p) * G + hg) * 2]);
@@ -496,7 +532,8 @@ __global__ __launch_bounds__(256) void attn_decode_merge_kernel(const float* __r
 #pragma unroll 2
     for (uint32_t p = grp + 8 * ATTN_MERGE_PF; p < n_parts; p += 8) {
         const float w = wbuf[p];
-        const float4 a = reinterpret_cast<const float4*>(part_acc + ((pbase + p) * G + hg) * ATTN_HD)[c];
+        float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (live) a = reinterpret_cast<const float4*>(part_acc + ((pbase + p) * G + hg) * HD)[c];
         acc.x = fmaf(w, a.x, acc.x); acc.y = fmaf(w, a.y, acc.y);
         acc.z = fmaf(w, a.z, acc.z); acc.w = fmaf(w, a.w, acc.w);
     }
@@ -510,16 +547,19 @@ __global__ __launch_bounds__(256) void attn_decode_merge_kernel(const float* __r
         }
         float inv = 1.0f / L;
         float4 o = make_float4(acc.x * inv, acc.y * inv, acc.z * inv, acc.w * inv);
-        const uint64_t row = static_cast<uint64_t>(qi) * n_heads + head;  // outputs are [n_queries][n_heads][128]
-        reinterpret_cast<float4*>(out + row * ATTN_HD)[c] = o;
+        const uint64_t row = static_cast<uint64_t>(qi) * n_heads + head;  // outputs are [n_queries][n_heads][HD]
+        if (live) reinterpret_cast<float4*>(out + row * HD)[c] = o;
         if (QUANT) {
+            // every lane takes part in the 8-lane exchanges; whole groups of 8 are live or idle together
             float sc;
             uint32_t packed = q8_quantize_quad(o, sc);
             float ssum = bsum ? q8_block_scaled_sum(packed, sc) : 0.0f;
-            reinterpret_cast<uint32_t*>(quants)[row * 32 + c] = packed;
-            if ((c & 7) == 0) {
-                scales[row * 4 + (c >> 3)] = sc;
-                if (bsum) bsum[row * 4 + (c >> 3)] = ssum;
+            if (live) {
+                reinterpret_cast<uint32_t*>(quants)[row * C4 + c] = packed;
+                if ((c & 7) == 0) {
+                    scales[row * (HD / 32) + (c >> 3)] = sc;
+                    if (bsum) bsum[row * (HD / 32) + (c >> 3)] = ssum;
+                }
             }
         }
     }

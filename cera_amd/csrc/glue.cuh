@@ -233,23 +233,24 @@ static __global__ void rope_kv_kernel(float* __restrict__ q, float* __restrict__
 // a staging buffer otherwise), and K rows are rotated on the way by the constant delta rotation
 // R(-shift) -- `delta_cs` holds its head_dim/2 (cos, sin) pairs, built on the host with the
 // reference's recurrence (cera/src/backend/cpu.rs:5065-5086 NEOX, :5145-5180 NORM); null = plain
-// copy (V, and the copy back from staging).  head_dim = 128; 16 threads per row, each owning
-// float4 j and float4 j + 16.  grid = (ceil(n_rows * 16 / 256), n_kv_heads).
-template <typename KV>
+// copy (V, and the copy back from staging).  HD / 8 threads per row, each owning float4 j and
+// float4 j + HD / 8 (its NEOX partner).  grid = (ceil(n_rows * HD / 8 / 256), n_kv_heads).
+template <typename KV, int HD>
 static __global__ __launch_bounds__(256) void kv_shift_kernel(const KV* __restrict__ src, KV* __restrict__ dst,
                                                               uint32_t src_row, uint32_t dst_row, uint32_t n_rows,
                                                               uint64_t src_head_stride, uint64_t dst_head_stride,
                                                               const float* __restrict__ delta_cs, uint32_t rope_type) {
-    const uint32_t t = (blockIdx.x * 256 + threadIdx.x) >> 4, j = threadIdx.x & 15;
+    constexpr uint32_t TPR = HD / 8;
+    const uint32_t t = (blockIdx.x * 256 + threadIdx.x) / TPR, j = threadIdx.x % TPR;
     if (t >= n_rows) return;
-    const KV* sp = src + blockIdx.y * src_head_stride + static_cast<uint64_t>(src_row + t) * 128;
-    KV* dp = dst + blockIdx.y * dst_head_stride + static_cast<uint64_t>(dst_row + t) * 128;
+    const KV* sp = src + blockIdx.y * src_head_stride + static_cast<uint64_t>(src_row + t) * HD;
+    KV* dp = dst + blockIdx.y * dst_head_stride + static_cast<uint64_t>(dst_row + t) * HD;
     // a half cache is widened, rotated in f32 and narrowed again (cera/src/kv_cache.rs:1196-1230)
-    float4 a = KvOps<KV>::ld4(sp, j), b = KvOps<KV>::ld4(sp, j + 16);
+    float4 a = KvOps<KV>::ld4(sp, j), b = KvOps<KV>::ld4(sp, j + TPR);
     if (delta_cs) {
         const float4* cs = reinterpret_cast<const float4*>(delta_cs);
         if (rope_type == 1) {   // NORM: pairs (2i, 2i+1): pair i uses cs[i]; float4 j holds pairs 2j, 2j+1
-            const float4 ca = cs[j], cb = cs[j + 16];
+            const float4 ca = cs[j], cb = cs[j + TPR];
             float4 r;
             r.x = __fsub_rn(__fmul_rn(a.x, ca.x), __fmul_rn(a.y, ca.y));
             r.y = __fadd_rn(__fmul_rn(a.x, ca.y), __fmul_rn(a.y, ca.x));
@@ -261,7 +262,7 @@ static __global__ __launch_bounds__(256) void kv_shift_kernel(const KV* __restri
             r.z = __fsub_rn(__fmul_rn(b.z, cb.z), __fmul_rn(b.w, cb.w));
             r.w = __fadd_rn(__fmul_rn(b.z, cb.w), __fmul_rn(b.w, cb.z));
             b = r;
-        } else {                // NEOX: pairs (i, i + 64): element 4j + e of a with the same of b, cs[4j + e]
+        } else {                // NEOX: pairs (i, i + HD/2): element 4j + e of a with the same of b, cs[4j + e]
             const float4 c01 = cs[2 * j], c23 = cs[2 * j + 1];
             float4 ra, rb;
             ra.x = __fsub_rn(__fmul_rn(a.x, c01.x), __fmul_rn(b.x, c01.y));
@@ -276,7 +277,7 @@ static __global__ __launch_bounds__(256) void kv_shift_kernel(const KV* __restri
         }
     }
     KvOps<KV>::st4(dp, j, a);
-    KvOps<KV>::st4(dp, j + 16, b);
+    KvOps<KV>::st4(dp, j + TPR, b);
 }
 
 // out = a + b (cera/src/backend/cpu.rs:5223-5228), optional scale on b first.

@@ -94,7 +94,7 @@ extern "C" cera_hip_status cera_hip_model_create(cera_hip_ctx* ctx, const cera_h
     if (c.n_layers == 0 || c.hidden == 0 || c.ffn == 0 || c.n_heads == 0 || c.n_kv_heads == 0 || c.vocab == 0 ||
         c.max_seq_len == 0)
         return cera_fail(ctx, CERA_HIP_ERR_ARGUMENT, "model_create: zero dimension in config");
-    if (c.head_dim != 128) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "model_create: head_dim must be 128");
+    if (c.head_dim != 64 && c.head_dim != 128) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "model_create: head_dim must be 64 or 128");
     if (c.n_heads % c.n_kv_heads) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "model_create: n_heads % n_kv_heads != 0");
     if (c.hidden % 32 || c.ffn % 32) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "model_create: hidden and ffn must be multiples of 32");
     if (c.rope_type > 1) return cera_fail(ctx, CERA_HIP_ERR_ARGUMENT, "model_create: rope_type must be 0 (neox) or 1 (norm)");
@@ -243,7 +243,6 @@ extern "C" cera_hip_status cera_hip_shift_kv(cera_hip_model* m, uint32_t n_keep,
     if (static_cast<uint64_t>(n_keep) + shift > m->seq_len)
         return cera_fail(ctx, CERA_HIP_ERR_POSITION, "shift_kv: n_keep=" + std::to_string(n_keep) + " + shift=" +
                                                          std::to_string(shift) + " > seq_len=" + std::to_string(m->seq_len));
-    if (c.head_dim != 128) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "shift_kv: head_dim must be 128");
     const uint32_t new_len = m->seq_len - shift, tail = new_len - n_keep, src_row = n_keep + shift;
     if (tail) {
         // delta rotation: theta_0 = -(shift) as f32, the forward pass's recurrence and factors
@@ -263,34 +262,43 @@ extern "C" cera_hip_status cera_hip_shift_kv(cera_hip_model* m, uint32_t n_keep,
         }
         CERA_TRY(cera_hip_upload(ctx, m->shift_cs, row.data(), row.size() * 4));
         const uint64_t head_stride = static_cast<uint64_t>(c.max_seq_len) * c.head_dim;
-        const dim3 grid((tail * 16 + 255) / 256, c.n_kv_heads), block(256);
+        const dim3 grid((tail * (c.head_dim / 8) + 255) / 256, c.n_kv_heads), block(256);
         const bool overlap = tail > shift;   // source and destination rows intersect: go through staging
         void* stage = nullptr;
         const uint64_t stage_stride = static_cast<uint64_t>(tail) * c.head_dim;
         if (overlap) {
             CERA_TRY(cera_scratch(ctx, 5, stage_stride * c.n_kv_heads * sizeof(float), &stage));
         }
-        auto run = [&](auto* tag) {
+        auto run = [&](auto* tag, auto hd_tag) {
             using KV = std::remove_pointer_t<decltype(tag)>;
+            constexpr int HD = decltype(hd_tag)::value;
             for (LayerDev& L : m->layers) {
                 for (int is_v = 0; is_v < 2; ++is_v) {
                     KV* cache = static_cast<KV*>(is_v ? L.vc : L.kc);
                     const float* cs = is_v ? nullptr : m->shift_cs;
                     if (!overlap) {
-                        hipLaunchKernelGGL(kv_shift_kernel<KV>, grid, block, 0, ctx->stream, cache, cache, src_row, n_keep,
-                                           tail, head_stride, head_stride, cs, c.rope_type);
+                        hipLaunchKernelGGL((kv_shift_kernel<KV, HD>), grid, block, 0, ctx->stream, cache, cache, src_row,
+                                           n_keep, tail, head_stride, head_stride, cs, c.rope_type);
                     } else {
-                        hipLaunchKernelGGL(kv_shift_kernel<KV>, grid, block, 0, ctx->stream, cache, static_cast<KV*>(stage),
-                                           src_row, 0u, tail, head_stride, stage_stride, cs, c.rope_type);
-                        hipLaunchKernelGGL(kv_shift_kernel<KV>, grid, block, 0, ctx->stream, static_cast<KV*>(stage), cache,
-                                           0u, n_keep, tail, stage_stride, head_stride, static_cast<const float*>(nullptr),
+                        hipLaunchKernelGGL((kv_shift_kernel<KV, HD>), grid, block, 0, ctx->stream, cache,
+                                           static_cast<KV*>(stage), src_row, 0u, tail, head_stride, stage_stride, cs,
                                            c.rope_type);
+                        hipLaunchKernelGGL((kv_shift_kernel<KV, HD>), grid, block, 0, ctx->stream, static_cast<KV*>(stage),
+                                           cache, 0u, n_keep, tail, stage_stride, head_stride,
+                                           static_cast<const float*>(nullptr), c.rope_type);
                     }
                 }
             }
         };
-        if (m->kv_f16) run(static_cast<kv_half*>(nullptr));
-        else run(static_cast<float*>(nullptr));
+        using HD128 = std::integral_constant<int, 128>;
+        using HD64 = std::integral_constant<int, 64>;
+        if (c.head_dim == 128) {
+            if (m->kv_f16) run(static_cast<kv_half*>(nullptr), HD128{});
+            else run(static_cast<float*>(nullptr), HD128{});
+        } else {
+            if (m->kv_f16) run(static_cast<kv_half*>(nullptr), HD64{});
+            else run(static_cast<float*>(nullptr), HD64{});
+        }
         HIP_TRY(ctx, hipGetLastError());
         HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
     }

@@ -307,3 +307,23 @@ def test_f16_kv_through_the_model_layer(tiny_llama, orc):
     with pytest.raises(llama_api.BackendError):
         gm32.restore_state(snap)          # an f16 snapshot does not load into an f32 cache
     gm.close(); om.close(); snap.close()
+
+
+@pytest.mark.parametrize("arch,explicit", [("llama", False), ("qwen3", True)])
+def test_head_dim_64_file(tmp_path, orc, hip, arch, explicit):
+    """Llama-3.2-1B / Granite-2B shape class: head_dim 64, implied by hidden / n_heads (llama) or
+    given by attention.key_length and decoupled from it (qwen3: 8 heads x 64 over hidden 256)."""
+    cfg0 = dict(synth.TINY, n_heads=8 if explicit else 4, n_kv_heads=2, head_dim=64)
+    path = str(tmp_path / "hd64.gguf")
+    H.synth_llama_gguf(path, cfg0, seed=15, sigma=0.05, norm_jitter=0.1, arch=arch, qk_norm=(arch == "qwen3"),
+                       explicit_head_dim=explicit)
+    cfg, weights = H.Gguf(path).llama_weights()
+    assert cfg["head_dim"] == 64
+    gm = llama_api.HipLlama(path, context_size=64)
+    om = orc.Llama(cfg, weights)
+    try:
+        assert gm.config["head_dim"] == 64
+        _say(f"hip_llama: head_dim 64 {arch} file")
+        _teacher_forced(gm, om, orc, [11, 22, 33, 44, 55, 66, 77], 14, 12)
+    finally:
+        gm.close(); om.close()

@@ -374,3 +374,23 @@ def test_attn_prefill_f16_kv_vs_oracle(hip, orc, nh, nkv, start, n):
         ref = orc.decode_attention(q[i], kh[:Li * nkv * hd], vh[:Li * nkv * hd], nh, nkv, hd, scale, Li)
         err = np.abs(out[i].astype(np.float64) - ref).max()
         assert err <= ATTN_TOL * util.rms(ref), (i, err, util.rms(ref))
+
+
+# ---- head_dim 64 (Llama-3.2-1B, Granite-2B, Qwen2 < 7B) ---------------------------------
+@pytest.mark.parametrize("kv_f16", [False, True])
+@pytest.mark.parametrize("nh,nkv,L", [(32, 8, 1), (32, 8, 777), (8, 8, 130), (16, 2, 5000), (4, 1, 64)])
+def test_attn_decode_head_dim_64(hip, orc, kv_f16, nh, nkv, L):
+    hd = 64
+    _say(f"attn_decode hd=64 nh={nh} nkv={nkv} L={L} f16={kv_f16}")
+    q = util.make_x(nh * hd, 260)
+    k = util.make_x(L * nkv * hd, 261 + L)
+    v = util.make_x(L * nkv * hd, 262 + L)
+    scale = 1.0 / math.sqrt(hd)
+    if kv_f16:
+        out = hip.attn_f16kv(q, k, v, nh, nkv, hd, L - 1, 1, scale).reshape(-1)
+        k, v = _through_half(k), _through_half(v)
+    else:
+        out = hip.attn_decode(q, k, v, nh, nkv, hd, L, scale)
+    ref = orc.decode_attention(q, k, v, nh, nkv, hd, scale, L)
+    err = np.abs(out.astype(np.float64) - ref).max()
+    assert err <= ATTN_TOL * util.rms(ref), (err, util.rms(ref))

@@ -296,3 +296,58 @@ def test_shift_kv_f16_matches_oracle_bitwise(hip, orc, rope_type, seq_len, n_kee
         assert np.array_equal(kg.view(np.uint32), ko.view(np.uint32)), layer
         assert np.array_equal(vg.view(np.uint32), vo.view(np.uint32)), layer
     gm.close(); om.close()
+
+
+# ---- head_dim 64 --------------------------------------------------------------------------
+TINY64 = dict(synth.TINY, n_heads=8, n_kv_heads=2, head_dim=64)   # q_dim 512 != hidden 256, group of 4
+
+
+@pytest.mark.parametrize("rope_type,kv_f16", [(1, False), (0, False), (1, True)])
+def test_head_dim_64_model_parity(hip, orc, rope_type, kv_f16):
+    cfg = dict(TINY64, rope_type=rope_type)
+    weights = synth.make_llama(cfg, seed=91, sigma=0.05, norm_jitter=0.1)
+    gm = hip_api.Model(hip, cfg, weights)
+    om = orc.Llama(cfg, weights)
+    if kv_f16:
+        gm.configure_kv(True); om.set_kv_f16(True)
+    _say(f"head_dim 64 model: rope_type={rope_type} f16={kv_f16}")
+    toks = [int(t) for t in util.rng(92).integers(0, cfg["vocab"], 24)]
+    lg, lo = gm.forward_prefill(toks, 0), om.forward_prefill_batched(toks, 0)
+    assert _cos(lg, lo) > 0.999
+    same = 0
+    for i in range(12):
+        tg, to = int(orc_argmax(lg)), int(orc_argmax(lo))
+        same += tg == to
+        lg, lo = gm.forward(to, 24 + i), om.forward(to, 24 + i)
+        assert _cos(lg, lo) > 0.999, i
+    assert same >= 10
+    kg, vg = gm.read_kv(0)
+    ko, vo = om.kv(0)
+    assert np.abs(kg - ko).max() <= 3e-3 * util.rms(ko) and np.abs(vg - vo).max() <= 3e-3 * util.rms(vo)
+    # context shift on the 64-wide cache, bit for bit
+    gm.shift_kv(3, 9); om.shift_kv(3, 9)
+    assert gm.seq_len == om.seq_len == 27
+    lg, lo = gm.forward(5, 27), om.forward(5, 27)
+    assert _cos(lg, lo) > 0.999
+    gm.close(); om.close()
+
+
+def test_head_dim_64_shift_bitwise(hip, orc):
+    from test_oracle_kv_shift import rope_filled_cache
+    for rope_type in (0, 1):
+        cfg = dict(TINY64, rope_type=rope_type)
+        weights = synth.make_llama(cfg, seed=5, sigma=0.05)
+        gm = hip_api.Model(hip, cfg, weights)
+        om = orc.Llama(cfg, weights)
+        layers, _ = rope_filled_cache(orc, cfg, 30, rope_type == 1)
+        om.restore(layers, 30)
+        for i, (k, v) in enumerate(layers):
+            gm.write_kv(i, k, v)
+        gm.set_seq_len(30)
+        gm.shift_kv(4, 6); om.shift_kv(4, 6)       # tail 20 > shift 6: through staging
+        for layer in range(cfg["n_layers"]):
+            kg, vg = gm.read_kv(layer)
+            ko, vo = om.kv(layer)
+            assert np.array_equal(kg.view(np.uint32), ko.view(np.uint32)), (rope_type, layer)
+            assert np.array_equal(vg.view(np.uint32), vo.view(np.uint32)), (rope_type, layer)
+        gm.close(); om.close()

@@ -148,3 +148,26 @@ def test_attn_prefill_batch_vs_oracle(hip, orc, nh, nkv, start, n):
         err = np.abs(out[i].astype(np.float64) - ref).max()
         assert err <= 2e-3 * util.rms(ref), (i, err, util.rms(ref))
     assert np.isfinite(out).all()
+
+
+@pytest.mark.parametrize("kv_f16", [False, True])
+@pytest.mark.parametrize("nh,nkv,start,n", [(32, 8, 0, 200), (8, 2, 300, 40), (4, 4, 1000, 33)])
+def test_attn_prefill_batch_head_dim_64(hip, orc, kv_f16, nh, nkv, start, n):
+    hd = 64
+    _say(f"attn_prefill hd=64 nh={nh} nkv={nkv} start={start} n={n} f16={kv_f16}")
+    r = util.rng(13 * n + start)
+    L = start + n
+    q = r.standard_normal((n, nh * hd), dtype=np.float32)
+    k = r.standard_normal(L * nkv * hd, dtype=np.float32)
+    v = r.standard_normal(L * nkv * hd, dtype=np.float32)
+    scale = 1.0 / np.sqrt(hd)
+    if kv_f16:
+        out = hip.attn_f16kv(q, k, v, nh, nkv, hd, start, n, scale)
+        k = k.astype(np.float16).astype(np.float32); v = v.astype(np.float16).astype(np.float32)
+    else:
+        out = hip.attn_prefill(q, k, v, nh, nkv, hd, start, n, scale)
+    for i in sorted(set([0, 1, 31, 32, n // 2, n - 1]) & set(range(n))):
+        Li = start + i + 1
+        ref = orc.decode_attention(q[i], k[:Li * nkv * hd], v[:Li * nkv * hd], nh, nkv, hd, scale, Li)
+        err = np.abs(out[i].astype(np.float64) - ref).max()
+        assert err <= 2e-3 * util.rms(ref), (i, err, util.rms(ref))
