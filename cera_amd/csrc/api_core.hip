@@ -10,6 +10,7 @@
 #include "quantize.cuh"
 
 bool cera_gemv_launch_q4k(const GemvArgs&, const GemvPlan&, int, bool, hipStream_t);
+bool cera_gemv_launch_pair_q4k_q6k(const GemvPairArgs& a, const GemvPlan& pa, const GemvPlan& pb, hipStream_t s);
 bool cera_gemv_launch_q6k(const GemvArgs&, const GemvPlan&, int, bool, hipStream_t);
 bool cera_gemv_launch_q4_0(const GemvArgs&, const GemvPlan&, int, bool, hipStream_t);
 bool cera_gemv_launch_q4_1(const GemvArgs&, const GemvPlan&, int, bool, hipStream_t);
@@ -380,6 +381,34 @@ cera_hip_status cera_launch_gemv(cera_hip_ctx* ctx, const cera_hip_dtensor* w, c
     return CERA_HIP_OK;
 }
 
+// Two projections of the same quantized activations in one launch (plain store epilogue).
+// *launched is false when no paired kernel instance covers the two shapes: the caller then
+// launches them one after the other.
+cera_hip_status cera_launch_gemv_pair(cera_hip_ctx* ctx, const cera_hip_dtensor* wa, const cera_hip_dtensor* wb,
+                                      const float* xs, const int8_t* xq, float* ya, float* yb, bool* launched) {
+    *launched = false;
+    if (wa->dtype != CERA_HIP_Q4_K || wb->dtype != CERA_HIP_Q6_K || wa->k != wb->k) return CERA_HIP_OK;
+    auto fill = [&](const cera_hip_dtensor* w, float* y, uint32_t n_units, GemvArgs* a) {
+        a->w = w->dev; a->w2 = nullptr; a->xq = xq; a->xs = xs; a->y = y; a->resid = nullptr;
+        a->m = static_cast<uint32_t>(w->m); a->n_units = n_units; a->row_bytes = static_cast<uint32_t>(w->row_bytes);
+        a->dbg_dots = nullptr; a->dbg_asums = nullptr; a->dbg_stride = 0;
+    };
+    GemvPairArgs p;
+    GemvPlan pa, pb;
+    const uint32_t ua = static_cast<uint32_t>(wa->k / 32), ub = static_cast<uint32_t>(wb->k / Q6K::ELEMS_PER_UNIT);
+    if (!gemv_plan(static_cast<uint32_t>(wa->m), ua, ctx->n_cu, false, 4, &pa)) return CERA_HIP_OK;
+    if (!gemv_plan(static_cast<uint32_t>(wb->m), ub, ctx->n_cu, false, 2, &pb)) return CERA_HIP_OK;
+    fill(wa, ya, ua, &p.a);
+    fill(wb, yb, ub, &p.b);
+    p.a.rows_per_wave = pa.rows_per_block;
+    p.b.rows_per_wave = pb.rows_per_block;
+    p.n_blocks_a = pa.n_blocks;
+    if (!cera_gemv_launch_pair_q4k_q6k(p, pa, pb, ctx->stream)) return CERA_HIP_OK;
+    HIP_TRY(ctx, hipGetLastError());
+    *launched = true;
+    return CERA_HIP_OK;
+}
+
 cera_hip_status cera_launch_argmax(cera_hip_ctx* ctx, const float* x, uint32_t n, uint32_t* out_dev) {
     void* part;
     CERA_TRY(cera_scratch(ctx, 8, ARGMAX_PARTS * 8, &part));
@@ -614,6 +643,36 @@ cera_hip_status cera_hip_gemv(cera_hip_ctx* ctx, const cera_hip_tensor* t, const
     };
     st = run();
     cera_hip_tensor_free(ctx, w);
+    return st;
+}
+
+cera_hip_status cera_hip_gemv_pair(cera_hip_ctx* ctx, const cera_hip_tensor* ta, const cera_hip_tensor* tb, const float* x,
+                                   float* ya, float* yb) {
+    if (!ctx || !ta || !tb || !x || !ya || !yb) return CERA_HIP_ERR_ARGUMENT;
+    if (ta->k != tb->k || ta->k == 0 || ta->k % 256) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "gemv_pair: the two matrices must share k, a multiple of 256");
+    cera_hip_dtensor *wa = nullptr, *wb = nullptr;
+    CERA_TRY(cera_hip_tensor_upload(ctx, ta, &wa));
+    cera_hip_status st = cera_hip_tensor_upload(ctx, tb, &wb);
+    if (st != CERA_HIP_OK) { cera_hip_tensor_free(ctx, wa); return st; }
+    auto run = [&]() -> cera_hip_status {
+        const uint64_t k = wa->k;
+        void *dx, *ds, *dq, *dy;
+        CERA_TRY(cera_scratch(ctx, 0, k * 4, &dx));
+        CERA_TRY(cera_scratch(ctx, 1, k / 32 * 4, &ds));
+        CERA_TRY(cera_scratch(ctx, 2, k, &dq));
+        CERA_TRY(cera_scratch(ctx, 3, (wa->m + wb->m) * 4, &dy));
+        CERA_TRY(cera_hip_upload(ctx, dx, x, k * 4));
+        CERA_TRY(cera_launch_quantize(ctx, static_cast<float*>(dx), k, static_cast<float*>(ds), static_cast<int8_t*>(dq)));
+        bool launched = false;
+        float *da = static_cast<float*>(dy), *db = da + wa->m;
+        CERA_TRY(cera_launch_gemv_pair(ctx, wa, wb, static_cast<float*>(ds), static_cast<int8_t*>(dq), da, db, &launched));
+        if (!launched) return cera_fail(ctx, CERA_HIP_ERR_UNSUPPORTED_DTYPE, "gemv_pair: no paired kernel instance for these types / shapes");
+        CERA_TRY(cera_hip_download(ctx, ya, da, wa->m * 4));
+        return cera_hip_download(ctx, yb, db, wb->m * 4);
+    };
+    st = run();
+    cera_hip_tensor_free(ctx, wa);
+    cera_hip_tensor_free(ctx, wb);
     return st;
 }
 

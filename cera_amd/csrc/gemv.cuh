@@ -368,13 +368,13 @@ __device__ __forceinline__ void gemv_compute(const GemvArgs& p, const GemvTile<T
     }
 }
 
+// The work of workgroup `block` (KS wavefronts; this wavefront is number kw, this lane `lane`).
+// `part` is the workgroup's LDS combine buffer (unused when KS == 1, which also has no barrier).
 template <class T, int U, int KS, int RB, int EPI, bool DBG>
-static __global__ __launch_bounds__(64 * KS) void gemv_kernel(GemvArgs p) {
+__device__ __forceinline__ void gemv_body(const GemvArgs& p, uint32_t block, uint32_t lane, uint32_t kw,
+                                          float (*part)[EPI == EPI_SILU_MUL ? 2 : 1][RB][KS * 4]) {
     constexpr int NM = EPI == EPI_SILU_MUL ? 2 : 1;
-    // two LDS buffers: a buffer is rewritten two row groups later, after another barrier
-    __shared__ float part[2][NM][RB][KS * 4];
-    const uint32_t lane = threadIdx.x & 63, kw = threadIdx.x >> 6;
-    uint32_t r = blockIdx.x * p.rows_per_wave;  // rows per workgroup
+    uint32_t r = block * p.rows_per_wave;  // rows per workgroup
     if (r >= p.m) return;
     const uint32_t r1 = min(p.m, r + p.rows_per_wave);
 
@@ -393,27 +393,57 @@ static __global__ __launch_bounds__(64 * KS) void gemv_kernel(GemvArgs p) {
 #pragma unroll
     for (int i = 0; i < U; ++i) {
         T::load_act(act[i], p.xq, p.xs, unit[i], live[i]);
-        if (DBG && blockIdx.x == 0 && live[i] && p.dbg_asums) T::dbg_asum(act[i], unit[i], p.dbg_asums);
+        if (DBG && block == 0 && live[i] && p.dbg_asums) T::dbg_asum(act[i], unit[i], p.dbg_asums);
     }
 
     // Each prefetch sits in the same straight-line block as the compute it overlaps, so the
     // compiler can wait for exactly the older tile's loads (a prefetch under its own
     // condition would force a wait for everything at the join).
+    float (*part0)[RB][KS * 4] = KS == 1 ? nullptr : part[0];
+    float (*part1)[RB][KS * 4] = KS == 1 ? nullptr : part[1];
     for (;;) {
         if (r + RB >= r1) {
-            gemv_compute<T, U, KS, RB, EPI, DBG>(p, ta, act, unit, live, lane, kw, r, r1, part[0]);
+            gemv_compute<T, U, KS, RB, EPI, DBG>(p, ta, act, unit, live, lane, kw, r, r1, part0);
             break;
         }
         tb.load(p, unit, r + RB, r1);
-        gemv_compute<T, U, KS, RB, EPI, DBG>(p, ta, act, unit, live, lane, kw, r, r1, part[0]);
+        gemv_compute<T, U, KS, RB, EPI, DBG>(p, ta, act, unit, live, lane, kw, r, r1, part0);
         r += RB;
         if (r + RB >= r1) {
-            gemv_compute<T, U, KS, RB, EPI, DBG>(p, tb, act, unit, live, lane, kw, r, r1, part[1]);
+            gemv_compute<T, U, KS, RB, EPI, DBG>(p, tb, act, unit, live, lane, kw, r, r1, part1);
             break;
         }
         ta.load(p, unit, r + RB, r1);
-        gemv_compute<T, U, KS, RB, EPI, DBG>(p, tb, act, unit, live, lane, kw, r, r1, part[1]);
+        gemv_compute<T, U, KS, RB, EPI, DBG>(p, tb, act, unit, live, lane, kw, r, r1, part1);
         r += RB;
+    }
+}
+
+template <class T, int U, int KS, int RB, int EPI, bool DBG>
+static __global__ __launch_bounds__(64 * KS) void gemv_kernel(GemvArgs p) {
+    constexpr int NM = EPI == EPI_SILU_MUL ? 2 : 1;
+    // two LDS buffers: a buffer is rewritten two row groups later, after another barrier
+    __shared__ float part[2][NM][RB][KS * 4];
+    gemv_body<T, U, KS, RB, EPI, DBG>(p, blockIdx.x, threadIdx.x & 63, threadIdx.x >> 6, part);
+}
+
+// Two independent GEMVs over the same activations in one launch: workgroups [0, n_blocks_a) run
+// matrix A (KSA wavefronts split its K), the rest run matrix B, whose K fits one wavefront, so each
+// of their KSA wavefronts is a workgroup of B on its own (no LDS, no barrier on that side).
+// For a layer whose V projection has another block type than Q and K: one launch instead of two.
+struct GemvPairArgs {
+    GemvArgs a, b;
+    uint32_t n_blocks_a;
+};
+template <class TA, int KSA, int RBA, class TB, int RBB>
+static __global__ __launch_bounds__(64 * KSA) void gemv_pair_kernel(GemvPairArgs p) {
+    __shared__ float part[2][1][RBA][KSA * 4];
+    const uint32_t lane = threadIdx.x & 63, kw = threadIdx.x >> 6;
+    if (blockIdx.x < p.n_blocks_a) {
+        gemv_body<TA, 1, KSA, RBA, EPI_STORE, false>(p.a, blockIdx.x, lane, kw, part);
+    } else {
+        gemv_body<TB, 1, 1, RBB, EPI_STORE, false>(p.b, (blockIdx.x - p.n_blocks_a) * KSA + kw, lane, 0,
+                                                   static_cast<float(*)[1][RBB][4]>(nullptr));
     }
 }
 

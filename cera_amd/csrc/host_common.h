@@ -65,6 +65,8 @@ cera_hip_status cera_launch_quantize(cera_hip_ctx* ctx, const float* x, uint64_t
 cera_hip_status cera_launch_gemv(cera_hip_ctx* ctx, const cera_hip_dtensor* w, const cera_hip_dtensor* w2,
                                  const float* xs, const int8_t* xq, float* y, const float* resid, int epi,
                                  int32_t* dbg_dots = nullptr, int32_t* dbg_asums = nullptr);
+cera_hip_status cera_launch_gemv_pair(cera_hip_ctx* ctx, const cera_hip_dtensor* wa, const cera_hip_dtensor* wb,
+                                      const float* xs, const int8_t* xq, float* ya, float* yb, bool* launched);
 // index of the maximum of x[0, n) into *out_dev (device); uses scratch slot 8 of the context
 cera_hip_status cera_launch_argmax(cera_hip_ctx* ctx, const float* x, uint32_t n, uint32_t* out_dev);
 cera_hip_status cera_launch_gemv_q5k_f32(cera_hip_ctx* ctx, const cera_hip_dtensor* w, const float* x, float* y);

@@ -435,8 +435,15 @@ static cera_hip_status decode_step(cera_hip_model* m, uint32_t pos, bool want_lo
         LayerDev& L = m->layers[i];
         CERA_TRY(norm_quant(m, m->hidden, L.attn_norm, c.hidden, 1, m->normed));
         if (L.qkv) {
-            CERA_TRY(project(m, L.qkv, m->normed, m->q, nullptr));
-            if (L.qkv_rows == q_dim + kv_dim) CERA_TRY(project(m, L.v, m->normed, m->v, nullptr));
+            bool paired = false;
+            // Q|K in one block type and V in another (the Q4_K_M mix): still one launch where a
+            // paired kernel instance exists
+            if (L.qkv_rows == q_dim + kv_dim)
+                CERA_TRY(cera_launch_gemv_pair(ctx, L.qkv, L.v, m->xs, m->xq, m->q, m->v, &paired));
+            if (!paired) {
+                CERA_TRY(project(m, L.qkv, m->normed, m->q, nullptr));
+                if (L.qkv_rows == q_dim + kv_dim) CERA_TRY(project(m, L.v, m->normed, m->v, nullptr));
+            }
         } else {
             CERA_TRY(project(m, L.q, m->normed, m->q, nullptr));
             CERA_TRY(project(m, L.k, m->normed, m->k, nullptr));

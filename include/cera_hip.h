@@ -145,6 +145,15 @@ CERA_HIP_API cera_hip_status cera_hip_quantize_q8_0(cera_hip_ctx*, const float* 
 CERA_HIP_API cera_hip_status cera_hip_gemv(cera_hip_ctx*, const cera_hip_tensor* w, const float* x, float* y,
                                            int32_t* dbg_block_dots, int32_t* dbg_block_asums);
 
+/* Two projections of the same activation vector in one launch: what the decode step does for a
+ * layer whose attn_q|attn_k (Q4_K, stored back to back) and attn_v (Q6_K) differ in block type
+ * (the Q4_K_M mix, cera/src/convert/quantize.rs:102-113); each result is exactly that of
+ * cera_hip_gemv on its own matrix (same kernel body, same row grouping).  Kernel instances
+ * exist for a Q4_K matrix with 2048 < k <= 4096 next to a Q6_K one; any other combination is
+ * CERA_HIP_ERR_UNSUPPORTED_DTYPE (the model then launches the two one after the other). */
+CERA_HIP_API cera_hip_status cera_hip_gemv_pair(cera_hip_ctx*, const cera_hip_tensor* a, const cera_hip_tensor* b,
+                                                const float* x, float* ya, float* yb);
+
 /* transformer::gemm_preq over quantize_columns (cera/src/model/transformer.rs:
  * 710-788, 865-946; kernels cera/src/backend/cpu.rs:1437-1557).
  * x is [n][k] row-major f32 (one activation row per token), each row is

@@ -12,6 +12,7 @@ import pytest
 
 import util
 from util import Q4_0, Q4_1, Q8_0, Q4_K, Q5_K, Q6_K
+from cera_amd import hip_api
 
 pytestmark = pytest.mark.gpu
 
@@ -394,3 +395,32 @@ def test_attn_decode_head_dim_64(hip, orc, kv_f16, nh, nkv, L):
     ref = orc.decode_attention(q, k, v, nh, nkv, hd, scale, L)
     err = np.abs(out.astype(np.float64) - ref).max()
     assert err <= ATTN_TOL * util.rms(ref), (err, util.rms(ref))
+
+
+# ---- two projections in one launch --------------------------------------------------------
+@pytest.mark.parametrize("ma,mb,k", [(5120, 1024, 4096), (4096, 4096, 4096), (1027, 515, 4096), (6, 3, 3072)])
+def test_gemv_pair_is_bitwise_the_two_single_launches(hip, orc, ma, mb, k):
+    """attn_q|attn_k (Q4_K) and attn_v (Q6_K) of one layer in a single launch: the same kernel
+    body per matrix, so each output equals cera_hip_gemv's bit for bit (and the oracle to the bar)."""
+    _say(f"gemv_pair ma={ma} mb={mb} k={k}")
+    wa, _ = util.make_weights(Q4_K, ma, k, seed=301)
+    wb, _ = util.make_weights(Q6_K, mb, k, seed=302)
+    x = util.make_x(k, 303)
+    ya, yb = hip.gemv_pair(Q4_K, wa, ma, Q6_K, wb, mb, x, k)
+    sa, sb = hip.gemv(Q4_K, wa, x, ma, k), hip.gemv(Q6_K, wb, x, mb, k)
+    assert np.array_equal(ya.view(np.uint32), sa.view(np.uint32))
+    assert np.array_equal(yb.view(np.uint32), sb.view(np.uint32))
+    ref = orc.gemv(Q6_K, wb, x, mb, k)
+    assert np.abs(yb - ref).max() <= 1e-3 * util.rms(ref)
+
+
+def test_gemv_pair_refuses_what_it_has_no_instance_for(hip):
+    k = 1024   # one wavefront covers a Q4_K row of 1024: no paired instance
+    wa, _ = util.make_weights(Q4_K, 8, k, seed=1)
+    wb, _ = util.make_weights(Q6_K, 8, k, seed=2)
+    with pytest.raises(hip_api.HipError) as e:
+        hip.gemv_pair(Q4_K, wa, 8, Q6_K, wb, 8, util.make_x(k, 3), k)
+    assert e.value.status == 3
+    with pytest.raises(hip_api.HipError) as e:   # types the other way round
+        hip.gemv_pair(Q6_K, wb, 8, Q4_K, wa, 8, util.make_x(k, 3), k)
+    assert e.value.status == 3
