@@ -63,29 +63,38 @@ template <> struct AttnLay<kv_half, 128> {         // two 16-byte loads per row:
 // every wavefront has a single memory round trip (all its K and V loads in
 // flight at once) and there are enough wavefronts to cover the chip; long
 // contexts use 64-position chunks to amortise the softmax bookkeeping.
-// In-place RoPE of the values a lane holds of one head (register quad c is float4 column
-// Lay::col4(j, c)), same arithmetic as rope_kv_kernel.  rope_row = the position's head_dim / 2
-// (cos, sin) pairs.
+// RoPE of the values a lane holds of one head (register quad c is float4 column Lay::col4(j, c)),
+// same arithmetic as rope_kv_kernel.  The lane's (cos, sin) values are loaded once
+// (attn_rope_load: NQ float4 of the position's head_dim / 2 pairs) and applied to as many heads
+// as needed.  NORM rotates pairs (2i, 2i+1) = (x, y) and (z, w) of each float4 with the float4 of
+// the table at the same column; NEOX rotates pairs (i, i + head_dim / 2) = quad c with quad
+// c + NQ / 2, whose four pairs take two float4 of the table.
 template <typename Lay>
-__device__ __forceinline__ void attn_rope16(float4 (&x)[Lay::NQ], const float* __restrict__ rope_row, uint32_t j, uint32_t rope_type) {
+__device__ __forceinline__ void attn_rope_load(float4 (&cs)[Lay::NQ], const float* __restrict__ rope_row, uint32_t j,
+                                               uint32_t rope_type) {
+#pragma unroll
+    for (int i = 0; i < Lay::NQ; ++i) {
+        const uint32_t idx = rope_type == 1 ? Lay::col4(j, i) : 2 * Lay::col4(j, i >> 1) + (i & 1);
+        cs[i] = reinterpret_cast<const float4*>(rope_row)[idx];
+    }
+}
+template <typename Lay>
+__device__ __forceinline__ void attn_rope_apply(float4 (&x)[Lay::NQ], const float4 (&cs)[Lay::NQ], uint32_t rope_type) {
     constexpr int NQ = Lay::NQ;
-    if (rope_type == 1) {   // NORM: pairs (2i, 2i+1) = (x, y) and (z, w) of each float4
+    if (rope_type == 1) {
 #pragma unroll
         for (int c = 0; c < NQ; ++c) {
-            const float4 cs = reinterpret_cast<const float4*>(rope_row)[Lay::col4(j, c)];
-            const float4 v = x[c];
-            x[c].x = __fsub_rn(__fmul_rn(v.x, cs.x), __fmul_rn(v.y, cs.y));
-            x[c].y = __fadd_rn(__fmul_rn(v.x, cs.y), __fmul_rn(v.y, cs.x));
-            x[c].z = __fsub_rn(__fmul_rn(v.z, cs.z), __fmul_rn(v.w, cs.w));
-            x[c].w = __fadd_rn(__fmul_rn(v.z, cs.w), __fmul_rn(v.w, cs.z));
+            const float4 v = x[c], t = cs[c];
+            x[c].x = __fsub_rn(__fmul_rn(v.x, t.x), __fmul_rn(v.y, t.y));
+            x[c].y = __fadd_rn(__fmul_rn(v.x, t.y), __fmul_rn(v.y, t.x));
+            x[c].z = __fsub_rn(__fmul_rn(v.z, t.z), __fmul_rn(v.w, t.w));
+            x[c].w = __fadd_rn(__fmul_rn(v.z, t.w), __fmul_rn(v.w, t.z));
         }
-    } else {                // NEOX: pairs (i, i + head_dim / 2): quad c with quad c + NQ / 2
+    } else {
         constexpr int H2 = NQ / 2;
 #pragma unroll
         for (int c = 0; c < H2; ++c) {
-            const uint32_t f = Lay::col4(j, c);
-            const float4 c01 = reinterpret_cast<const float4*>(rope_row)[2 * f];
-            const float4 c23 = reinterpret_cast<const float4*>(rope_row)[2 * f + 1];
+            const float4 c01 = cs[2 * c], c23 = cs[2 * c + 1];
             const float4 a = x[c], b = x[c + H2];
             x[c].x = __fsub_rn(__fmul_rn(a.x, c01.x), __fmul_rn(b.x, c01.y));
             x[c + H2].x = __fadd_rn(__fmul_rn(a.x, c01.y), __fmul_rn(b.x, c01.x));
@@ -99,46 +108,83 @@ __device__ __forceinline__ void attn_rope16(float4 (&x)[Lay::NQ], const float* _
     }
 }
 
-// This lane's 16 columns of the V row of position tt; the token's own row comes from the
-// projection output (narrowed like a cached row) and is stored into the cache by the one
-// caller that owns the append.
+// The K or V values a lane needs of position tt: from the cache, or -- for the position whose
+// row is not stored yet -- raw from the projection output.  Loads only, nothing waits here.
+template <bool NEWKV, typename KV, int HD>
+__device__ __forceinline__ void attn_issue_row(float4 (&r)[HD / 32], const KV* __restrict__ base, const float* fresh,
+                                               uint32_t tt, uint32_t new_pos, uint32_t kvh, uint32_t j) {
+    using Lay = AttnLay<KV, HD>;
+    if (NEWKV && tt == new_pos) {
+        const float4* p = reinterpret_cast<const float4*>(fresh + kvh * HD);
+#pragma unroll
+        for (int c = 0; c < Lay::NQ; ++c) r[c] = p[Lay::col4(j, c)];
+    } else {
+        Lay::ld(base + static_cast<uint64_t>(tt) * HD, j, r);
+    }
+}
+// The position's own row once its loads are in: rotate (K only), narrow like a cached row, and
+// store it into the cache if this caller owns the append.
+template <bool ROTATE, typename KV, int HD>
+__device__ __forceinline__ void attn_finish_new_row(float4 (&r)[HD / 32], const float4 (&cs)[HD / 32], uint32_t rope_type,
+                                                    void* cache, uint64_t row, uint32_t j, bool store) {
+    using Lay = AttnLay<KV, HD>;
+    if (ROTATE) attn_rope_apply<Lay>(r, cs, rope_type);
+#pragma unroll
+    for (int c = 0; c < Lay::NQ; ++c) r[c] = KvOps<KV>::rnd4(r[c]);
+    if (store) {
+        KV* dst = static_cast<KV*>(cache) + row * HD;
+#pragma unroll
+        for (int c = 0; c < Lay::NQ; ++c) KvOps<KV>::st4(dst, Lay::col4(j, c), r[c]);
+    }
+}
+
+// Load-and-finish in one go (the long-chunk path, which loads V after the scores).
 template <bool NEWKV, typename KV, int HD>
 __device__ __forceinline__ void attn_load_v(float4 (&vv)[HD / 32], const KV* __restrict__ vbase, uint32_t t, uint32_t tt,
                                             uint32_t new_pos, uint32_t kvh, uint32_t max_seq, uint32_t j,
                                             const AttnNewKV& nk, bool store) {
-    using Lay = AttnLay<KV, HD>;
-    constexpr int NQ = Lay::NQ;
-    if (NEWKV && tt == new_pos) {
-        const float4* vp = reinterpret_cast<const float4*>(nk.v_new + kvh * HD);
-#pragma unroll
-        for (int c = 0; c < NQ; ++c) vv[c] = KvOps<KV>::rnd4(vp[Lay::col4(j, c)]);
-        if (store) {
-            KV* dst = static_cast<KV*>(nk.vc_w) + (static_cast<uint64_t>(kvh) * max_seq + t) * HD;
-#pragma unroll
-            for (int c = 0; c < NQ; ++c) KvOps<KV>::st4(dst, Lay::col4(j, c), vv[c]);
-        }
-    } else {
-        Lay::ld(vbase + static_cast<uint64_t>(tt) * HD, j, vv);
-    }
+    attn_issue_row<NEWKV, KV, HD>(vv, vbase, nk.v_new, tt, new_pos, kvh, j);
+    if (NEWKV && tt == new_pos)
+        attn_finish_new_row<false, KV, HD>(vv, vv, 0, nk.vc_w, static_cast<uint64_t>(kvh) * max_seq + t, j, store);
 }
 
 // One wavefront's share of the keys: chunks of 8*S positions at t_begin, t_begin + t_step, ...
 // below t_end, for the G query heads of one kv head.  Returns the online-softmax state with
-// the eight position groups already folded: every lane holds its 16 columns of acc and the
-// wavefront-wide m and l.  `q` points at the first of the G heads; `write_new` says whether
+// the eight position groups folded: the wavefront-wide m and l in every lane, and of the
+// unnormalised output each lane's head_dim / 64 consecutive columns from attn_fold_column.  `q` points at the first of the G heads; `write_new` says whether
 // this caller stores the new position's K/V row into the cache (NEWKV only).
 template <int G, int S, bool NEWKV, typename KV, int HD>
 __device__ __forceinline__ void attn_decode_range(const float* __restrict__ q, const KV* __restrict__ kbase,
                                                   const KV* __restrict__ vbase, uint32_t kvh, uint32_t max_seq,
                                                   uint32_t seq_len, uint32_t t_begin, uint32_t t_end, uint32_t t_step,
                                                   float scale, const AttnNewKV& nk, bool write_new, uint32_t lane,
-                                                  float4 (&acc)[G][HD / 32], float (&m)[G], float (&l)[G]) {
+                                                  float (&out)[G][HD / 64], float (&m)[G], float (&l)[G]) {
     using Lay = AttnLay<KV, HD>;
     constexpr int NQ = Lay::NQ;
     const uint32_t j = lane & 7, pg = lane >> 3;  // float4 column group, position group
+    float4 acc[G][NQ];
 
-    // this lane's 16 q values for each of the G heads
-    float4 qv[G][NQ];
+    const uint32_t new_pos = seq_len - 1;   // NEWKV: the position whose K/V are not in the cache yet
+    constexpr uint32_t CHUNK = 8 * S;
+    constexpr bool PREFETCH_V = S <= 2;  // small chunks: V loads issued together with K
+    // Short chunks are latency-bound, so their first chunk's K/V loads go out before anything
+    // else: one memory round trip covers the cache rows, q and the RoPE row together.
+    float4 kbuf[PREFETCH_V ? S : 1][NQ], vpre[PREFETCH_V ? S : 1][NQ];
+    // a lane past t_end re-reads the range's first position (from the cache, or the new row if
+    // that is the one not stored yet) and gets a dead score
+    auto issue_chunk = [&](uint32_t t0) {
+#pragma unroll
+        for (int s = 0; s < S; ++s) {
+            const uint32_t t = t0 + 8 * s + pg, tt = t < t_end ? t : t_begin;
+            attn_issue_row<NEWKV, KV, HD>(kbuf[s], kbase, nk.k_new, tt, new_pos, kvh, j);
+            attn_issue_row<NEWKV, KV, HD>(vpre[s], vbase, nk.v_new, tt, new_pos, kvh, j);
+        }
+    };
+    if (PREFETCH_V && t_begin < t_end) issue_chunk(t_begin);
+
+    // this lane's 16 q values for each of the G heads, and its part of the position's RoPE row
+    float4 qv[G][NQ], cs[NQ];
+    if (NEWKV) attn_rope_load<Lay>(cs, nk.rope_row, j, nk.rope_type);
 #pragma unroll
     for (int h = 0; h < G; ++h)
 #pragma unroll
@@ -146,9 +192,8 @@ __device__ __forceinline__ void attn_decode_range(const float* __restrict__ q, c
             qv[h][c] = reinterpret_cast<const float4*>(q + h * HD)[Lay::col4(j, c)];
     if (NEWKV) {
 #pragma unroll
-        for (int h = 0; h < G; ++h) attn_rope16<Lay>(qv[h], nk.rope_row, j, nk.rope_type);
+        for (int h = 0; h < G; ++h) attn_rope_apply<Lay>(qv[h], cs, nk.rope_type);
     }
-    const uint32_t new_pos = seq_len - 1;   // NEWKV: the position whose K/V are not in the cache yet
 
 #pragma unroll
     for (int h = 0; h < G; ++h) {
@@ -158,18 +203,20 @@ __device__ __forceinline__ void attn_decode_range(const float* __restrict__ q, c
         for (int c = 0; c < NQ; ++c) acc[h][c] = make_float4(0.f, 0.f, 0.f, 0.f);
     }
 
-    constexpr uint32_t CHUNK = 8 * S;
-    constexpr bool PREFETCH_V = S <= 2;  // small chunks: V loads issued together with K
-    // a lane past t_end re-reads the range's first position (from the cache, or the new row if
-    // that is the one not stored yet) and gets a dead score
     for (uint32_t t0 = t_begin; t0 < t_end; t0 += t_step) {
-        float4 vpre[PREFETCH_V ? S : 1][NQ];
         if (PREFETCH_V) {
+            if (t0 != t_begin) issue_chunk(t0);
+            if (NEWKV) {
 #pragma unroll
-            for (int s = 0; s < S; ++s) {
-                const uint32_t t = t0 + 8 * s + pg;
-                attn_load_v<NEWKV, KV, HD>(vpre[s], vbase, t, t < t_end ? t : t_begin, new_pos, kvh, max_seq, j, nk,
-                                       write_new && t == new_pos);
+                for (int s = 0; s < S; ++s) {
+                    const uint32_t t = t0 + 8 * s + pg, tt = t < t_end ? t : t_begin;
+                    if (tt == new_pos) {
+                        const uint64_t row = static_cast<uint64_t>(kvh) * max_seq + tt;
+                        const bool store = write_new && t < t_end;
+                        attn_finish_new_row<true, KV, HD>(kbuf[s], cs, nk.rope_type, nk.kc_w, row, j, store);
+                        attn_finish_new_row<false, KV, HD>(vpre[s], cs, 0, nk.vc_w, row, j, store);
+                    }
+                }
             }
         }
         // ---- scores: step s covers positions t0 + 8s + pg
@@ -180,21 +227,14 @@ __device__ __forceinline__ void attn_decode_range(const float* __restrict__ q, c
             const bool live = t < t_end;
             const uint32_t tt = live ? t : t_begin;
             float4 kv[NQ];
-            if (NEWKV && tt == new_pos) {
-                // the token's own key: from the projection output, rotated here, narrowed like a cached row
-                const float4* kp = reinterpret_cast<const float4*>(nk.k_new + kvh * HD);
+            if (PREFETCH_V) {
 #pragma unroll
-                for (int c = 0; c < NQ; ++c) kv[c] = kp[Lay::col4(j, c)];
-                attn_rope16<Lay>(kv, nk.rope_row, j, nk.rope_type);
-#pragma unroll
-                for (int c = 0; c < NQ; ++c) kv[c] = KvOps<KV>::rnd4(kv[c]);
-                if (write_new && live) {
-                    KV* dst = static_cast<KV*>(nk.kc_w) + (static_cast<uint64_t>(kvh) * max_seq + t) * HD;
-#pragma unroll
-                    for (int c = 0; c < NQ; ++c) KvOps<KV>::st4(dst, Lay::col4(j, c), kv[c]);
-                }
+                for (int c = 0; c < NQ; ++c) kv[c] = kbuf[s][c];
             } else {
-                Lay::ld(kbase + static_cast<uint64_t>(tt) * HD, j, kv);
+                attn_issue_row<NEWKV, KV, HD>(kv, kbase, nk.k_new, tt, new_pos, kvh, j);
+                if (NEWKV && tt == new_pos)
+                    attn_finish_new_row<true, KV, HD>(kv, cs, nk.rope_type, nk.kc_w, static_cast<uint64_t>(kvh) * max_seq + tt,
+                                                      j, write_new && live);
             }
 #pragma unroll
             for (int h = 0; h < G; ++h) {
@@ -220,6 +260,12 @@ __device__ __forceinline__ void attn_decode_range(const float* __restrict__ q, c
 #pragma unroll
             for (int s = 1; s < S; ++s) mx = fmaxf(mx, sc[h][s]);
             mx = wave_max(mx);
+            // short chunks (latency-bound, usually one per wavefront): nothing is accumulated yet on
+            // the first one, so skip the rescale; long chunks keep straight-line code for the scheduler
+            if (PREFETCH_V && t0 == t_begin) {
+                m[h] = mx;
+                continue;
+            }
             float m_new = fmaxf(m[h], mx);
             corr[h] = cera_expf(m[h] - m_new);  // 0 on the first chunk (m = -inf)
             m[h] = m_new;
@@ -258,23 +304,47 @@ __device__ __forceinline__ void attn_decode_range(const float* __restrict__ q, c
         }
     }
 
-    // ---- fold the 8 position groups (lanes differing in bits 3..5) together
+    // ---- fold the 8 position groups (lanes differing in bits 3..5) together: a reduce-scatter.
+    // Each exchange halves what a lane keeps (half its quads with the lane 32 away, half of those
+    // with the lane 16 away, half of that with the lane 8 away), so a lane ends with
+    // 4 * NQ / 8 consecutive floats of the sum: out[h][e], columns attn_fold_column(lane) + e.
+    const bool b5 = lane & 32, b4 = lane & 16, b3 = lane & 8;
 #pragma unroll
     for (int h = 0; h < G; ++h) {
         l[h] = wave_sum(l[h]);
+        float v[4 * NQ];
 #pragma unroll
         for (int c = 0; c < NQ; ++c) {
-            float* f = reinterpret_cast<float*>(&acc[h][c]);
+            v[4 * c] = acc[h][c].x; v[4 * c + 1] = acc[h][c].y; v[4 * c + 2] = acc[h][c].z; v[4 * c + 3] = acc[h][c].w;
+        }
+        constexpr int N1 = 2 * NQ, N2 = NQ, N3 = NQ / 2;
+        float w1[N1], w2[N2];
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                float v = f[e];
-                v += __shfl_xor(v, 8, 64);
-                v += __shfl_xor(v, 16, 64);
-                v += __shfl_xor(v, 32, 64);
-                f[e] = v;
-            }
+        for (int i = 0; i < N1; ++i) {
+            const float keep = b5 ? v[N1 + i] : v[i], send = b5 ? v[i] : v[N1 + i];
+            w1[i] = keep + __shfl_xor(send, 32, 64);
+        }
+#pragma unroll
+        for (int i = 0; i < N2; ++i) {
+            const float keep = b4 ? w1[N2 + i] : w1[i], send = b4 ? w1[i] : w1[N2 + i];
+            w2[i] = keep + __shfl_xor(send, 16, 64);
+        }
+#pragma unroll
+        for (int i = 0; i < N3; ++i) {
+            const float keep = b3 ? w2[N3 + i] : w2[i], send = b3 ? w2[i] : w2[N3 + i];
+            out[h][i] = keep + __shfl_xor(send, 8, 64);
         }
     }
+}
+
+// First float column (of head_dim) of the NQ / 2 a lane holds after the fold above.
+template <typename Lay>
+__device__ __forceinline__ uint32_t attn_fold_column(uint32_t lane) {
+    constexpr int NQ = Lay::NQ;
+    const uint32_t j = lane & 7, b5 = (lane >> 5) & 1, b4 = (lane >> 4) & 1, b3 = (lane >> 3) & 1;
+    // floats kept: index range [f0, f0 + NQ/2) of the lane's 4*NQ values, f0 = b5*2NQ + b4*NQ + b3*NQ/2
+    const uint32_t f0 = b5 * 2 * NQ + b4 * NQ + b3 * (NQ / 2);
+    return 4 * Lay::col4(j, f0 >> 2) + (f0 & 3);
 }
 
 template <int G, int S, bool NEWKV, typename KV, int HD>
@@ -300,22 +370,21 @@ __global__ __launch_bounds__(256) void attn_decode_partial_kernel(
     constexpr uint32_t CHUNK = 8 * S;
     const uint32_t t_begin = part * chunks_per_part * CHUNK;
     const uint32_t t_end = min(seq_len, t_begin + chunks_per_part * CHUNK);
-    float4 acc[G][NQ];
+    float out[G][NQ / 2];
     float m[G], l[G];
     attn_decode_range<G, S, NEWKV, KV, HD>(q, kc + static_cast<uint64_t>(kvh) * max_seq * HD,
                                    vc + static_cast<uint64_t>(kvh) * max_seq * HD, kvh, max_seq, seq_len, t_begin,
-                                   t_end, CHUNK, scale, nk, true, lane, acc, m, l);
-    if (pg == 0) {
-        uint64_t base = ((static_cast<uint64_t>(qi) * gridDim.y + kvh) * n_parts + part) * G;
+                                   t_end, CHUNK, scale, nk, true, lane, out, m, l);
+    const uint64_t base = ((static_cast<uint64_t>(qi) * gridDim.y + kvh) * n_parts + part) * G;
+    const uint32_t col = attn_fold_column<Lay>(lane);
 #pragma unroll
-        for (int h = 0; h < G; ++h) {
-            float4* dst = reinterpret_cast<float4*>(part_acc + (base + h) * HD);
-#pragma unroll
-            for (int c = 0; c < NQ; ++c) dst[Lay::col4(j, c)] = acc[h][c];
-            if (j == 0) {
-                part_ml[(base + h) * 2] = m[h];
-                part_ml[(base + h) * 2 + 1] = l[h];
-            }
+    for (int h = 0; h < G; ++h) {
+        float* dst = part_acc + (base + h) * HD + col;
+        if (NQ == 4) *reinterpret_cast<float2*>(dst) = make_float2(out[h][0], out[h][NQ / 2 - 1]);
+        else dst[0] = out[h][0];
+        if (lane == 0) {
+            part_ml[(base + h) * 2] = m[h];
+            part_ml[(base + h) * 2 + 1] = l[h];
         }
     }
 }
