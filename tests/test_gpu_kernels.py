@@ -93,6 +93,19 @@ def test_gemv_small_shapes(hip, orc, dtype, m, k):
     _check_gemv(hip, orc, dtype, m, k, seed=dtype * 100 + m)
 
 
+@pytest.mark.parametrize("dtype", util.INT8_TYPES)
+def test_gemv_seeded_shape_sweep(hip, orc, dtype):
+    """Seeded random shapes across every K-split width the planner can choose (1..8 wavefronts,
+    one and two units per lane), ragged row counts, and -- for the 32-element block types -- K
+    that is not a multiple of 256.  Integer dots bit-exact on the smaller ones, floats to the bar."""
+    r = util.rng(4000 + dtype)
+    step = 256 if dtype in (Q4_K, Q6_K) else 32
+    ks = [step * int(v) for v in r.integers(1, 8192 // step + 1, 6)] + [16384 // step * step, 28672 // step * step, 32768]
+    for i, k in enumerate(ks):
+        m = int(r.integers(1, 300))
+        _check_gemv(hip, orc, dtype, m, k, seed=dtype * 1000 + i, debug=(m * k <= 1 << 20))
+
+
 def test_gemv_config1_q4_0_4096(hip, orc):
     # BASELINE config 1: single Q4_0 GEMV, 4096 x 4096
     rel = _check_gemv(hip, orc, Q4_0, 4096, 4096, seed=11)

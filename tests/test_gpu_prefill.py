@@ -36,6 +36,23 @@ def test_gemm_small_shapes(hip, orc, dtype, m, n, k):
     assert err <= GEMM_TOL * util.rms(ref), (err, util.rms(ref))
 
 
+@pytest.mark.parametrize("dtype", util.INT8_TYPES)
+def test_gemm_seeded_shape_sweep(hip, orc, dtype):
+    """Seeded random (rows, tokens, k): ragged tiles on both sides, and few output tiles with a long
+    K so the split-K route and its fixed-order reduction are exercised."""
+    r = util.rng(5000 + dtype)
+    shapes = [(int(r.integers(1, 400)), int(r.integers(1, 200)), 256 * int(r.integers(1, 17))) for _ in range(5)]
+    shapes += [(64, 48, 8192), (130, 17, 14336), (256, 64, 4096)]
+    for m, n, k in shapes:
+        _say(f"gemm sweep {util.NAMES[dtype]} m={m} n={n} k={k}")
+        w, _ = util.make_weights(dtype, m, k, seed=dtype * 7 + m)
+        x = util.rng(m + n).standard_normal((n, k)).astype(np.float32)
+        out = hip.gemm(dtype, w, x, m, n, k)
+        ref = _oracle_gemm(orc, dtype, w, x, m, n, k)
+        err = np.abs(out.astype(np.float64) - ref).max()
+        assert err <= GEMM_TOL * util.rms(ref), (m, n, k, err, util.rms(ref))
+
+
 @pytest.mark.parametrize("dtype,m,k", [(Q4_K, 4096, 4096), (Q6_K, 4096, 14336)])
 @pytest.mark.parametrize("n", [128, 512, 2048])
 def test_gemm_config3_shapes_row_sample(hip, orc, dtype, m, k, n):
