@@ -9,7 +9,8 @@ batch 1 -- per layer fused QKV 6144x4096, O 4096x4096, gate and up 14336x4096
 4.8 GB working set rotates far past the 256 MB last-level cache.  Activations
 (Q8_0-quantized x ~ N(0,1)) and weights are resident in HBM before timing.
 
-Prints ONE JSON line (see README / DESIGN.md for the fields).
+Prints ONE JSON line: metric / value / unit, the roofline of the dominant kernel, the CPU baseline,
+and (unless disabled) end-to-end, flash-decode and prefill-GEMM measurements.
 """
 from __future__ import annotations
 
