@@ -506,12 +506,14 @@ cera_hip_status cera_launch_attn(cera_hip_ctx* ctx, const float* q, const void* 
     } else {
         // positions per chunk: small chunks while the context is short (one memory round
         // trip per wavefront, many wavefronts), 64 once there is plenty of work
-        S = last_len >= 16384 ? 8 : (last_len >= 4096 ? 4 : (last_len >= 1024 ? 2 : 1));
+        S = last_len >= 16384 ? 8 : (last_len >= 4096 ? 4 : (last_len >= ATTN_FUSED_NEW_KV_MAX_KEYS ? 2 : 1));
         if (G == 8 && S == 8) S = 4;   // eight heads x 64 positions per chunk does not fit the register file
         uint32_t n_chunks = static_cast<uint32_t>((last_len + 8 * S - 1) / (8 * S));
-        // parts (wavefronts) per (query, kv head): enough to fill the chip ~8 waves per CU
-        // deep, but at least one chunk each and at most ATTN_MAX_PARTS
-        uint32_t want_parts = n_splits ? n_splits : std::max(1u, ctx->n_cu * 8 / (n_kv_heads * n_queries));
+        // parts (wavefronts) per (query, kv head): enough to fill the chip ~4 waves per CU deep
+        // (more parts make the partial kernel shorter but the merge longer: measured best from 2k
+        // to 128k keys with an f32 cache), but at least one chunk each and at most ATTN_MAX_PARTS
+        const uint32_t waves_per_cu = kv_f16 ? 8 : 4;   // a half cache is nearer VALU-bound: more wavefronts help
+        uint32_t want_parts = n_splits ? n_splits : std::max(1u, ctx->n_cu * waves_per_cu / (n_kv_heads * n_queries));
         want_parts = std::min<uint32_t>(want_parts, ATTN_MAX_PARTS);
         chunks_per_part = std::max(1u, (n_chunks + want_parts - 1) / want_parts);
         n_parts = (n_chunks + chunks_per_part - 1) / chunks_per_part;

@@ -27,7 +27,7 @@
 #include "quantize.cuh"
 
 #define ATTN_MAX_PARTS 1024  // the merge kernel keeps one weight per part in LDS
-#define ATTN_MERGE_PF 4       // parts per lane group the merge kernel requests up front (x8 groups)
+#define ATTN_MERGE_PF 8       // parts per lane group the merge kernel requests per round trip (x8 groups)
 
 struct AttnPart {  // per (part, query head): running max, sum and unnormalised output
     float m, l;
@@ -108,24 +108,18 @@ __device__ __forceinline__ void attn_rope_apply(float4 (&x)[Lay::NQ], const floa
     }
 }
 
-// The K or V values a lane needs of position tt: from the cache, or -- for the position whose
-// row is not stored yet -- raw from the projection output.  Loads only, nothing waits here.
-template <bool NEWKV, typename KV, int HD>
-__device__ __forceinline__ void attn_issue_row(float4 (&r)[HD / 32], const KV* __restrict__ base, const float* fresh,
-                                               uint32_t tt, uint32_t new_pos, uint32_t kvh, uint32_t j) {
+// The token's own K or V row, not in the cache yet: its loads (raw projection output, this lane's
+// columns) are issued first; once they are in, the row is rotated (K only), narrowed like a
+// cached row and stored into the cache if this caller owns the append.
+template <typename KV, int HD>
+__device__ __forceinline__ void attn_new_row_load(float4 (&r)[HD / 32], const float* fresh, uint32_t kvh, uint32_t j) {
     using Lay = AttnLay<KV, HD>;
-    if (NEWKV && tt == new_pos) {
-        const float4* p = reinterpret_cast<const float4*>(fresh + kvh * HD);
+    const float4* p = reinterpret_cast<const float4*>(fresh + kvh * HD);
 #pragma unroll
-        for (int c = 0; c < Lay::NQ; ++c) r[c] = p[Lay::col4(j, c)];
-    } else {
-        Lay::ld(base + static_cast<uint64_t>(tt) * HD, j, r);
-    }
+    for (int c = 0; c < Lay::NQ; ++c) r[c] = p[Lay::col4(j, c)];
 }
-// The position's own row once its loads are in: rotate (K only), narrow like a cached row, and
-// store it into the cache if this caller owns the append.
 template <bool ROTATE, typename KV, int HD>
-__device__ __forceinline__ void attn_finish_new_row(float4 (&r)[HD / 32], const float4 (&cs)[HD / 32], uint32_t rope_type,
+__device__ __forceinline__ void attn_new_row_finish(float4 (&r)[HD / 32], const float4 (&cs)[HD / 32], uint32_t rope_type,
                                                     void* cache, uint64_t row, uint32_t j, bool store) {
     using Lay = AttnLay<KV, HD>;
     if (ROTATE) attn_rope_apply<Lay>(r, cs, rope_type);
@@ -136,16 +130,6 @@ __device__ __forceinline__ void attn_finish_new_row(float4 (&r)[HD / 32], const 
 #pragma unroll
         for (int c = 0; c < Lay::NQ; ++c) KvOps<KV>::st4(dst, Lay::col4(j, c), r[c]);
     }
-}
-
-// Load-and-finish in one go (the long-chunk path, which loads V after the scores).
-template <bool NEWKV, typename KV, int HD>
-__device__ __forceinline__ void attn_load_v(float4 (&vv)[HD / 32], const KV* __restrict__ vbase, uint32_t t, uint32_t tt,
-                                            uint32_t new_pos, uint32_t kvh, uint32_t max_seq, uint32_t j,
-                                            const AttnNewKV& nk, bool store) {
-    attn_issue_row<NEWKV, KV, HD>(vv, vbase, nk.v_new, tt, new_pos, kvh, j);
-    if (NEWKV && tt == new_pos)
-        attn_finish_new_row<false, KV, HD>(vv, vv, 0, nk.vc_w, static_cast<uint64_t>(kvh) * max_seq + t, j, store);
 }
 
 // One wavefront's share of the keys: chunks of 8*S positions at t_begin, t_begin + t_step, ...
@@ -164,23 +148,31 @@ __device__ __forceinline__ void attn_decode_range(const float* __restrict__ q, c
     const uint32_t j = lane & 7, pg = lane >> 3;  // float4 column group, position group
     float4 acc[G][NQ];
 
-    const uint32_t new_pos = seq_len - 1;   // NEWKV: the position whose K/V are not in the cache yet
-    constexpr uint32_t CHUNK = 8 * S;
+    // NEWKV: the last position's K/V are not in the cache yet.  The chunk loop below only walks
+    // cached positions, so it is the same straight-line code with or without NEWKV; the wavefront
+    // whose range holds the new position takes it as one extra step afterwards.
+    const uint32_t new_pos = seq_len - 1;
+    const bool own_new = NEWKV && t_begin <= new_pos && new_pos < t_end;   // wavefront-uniform
+    if (NEWKV) t_end = min(t_end, new_pos);
     constexpr bool PREFETCH_V = S <= 2;  // small chunks: V loads issued together with K
     // Short chunks are latency-bound, so their first chunk's K/V loads go out before anything
     // else: one memory round trip covers the cache rows, q and the RoPE row together.
     float4 kbuf[PREFETCH_V ? S : 1][NQ], vpre[PREFETCH_V ? S : 1][NQ];
-    // a lane past t_end re-reads the range's first position (from the cache, or the new row if
-    // that is the one not stored yet) and gets a dead score
+    // a lane past t_end re-reads the range's first position and gets a dead score
     auto issue_chunk = [&](uint32_t t0) {
 #pragma unroll
         for (int s = 0; s < S; ++s) {
             const uint32_t t = t0 + 8 * s + pg, tt = t < t_end ? t : t_begin;
-            attn_issue_row<NEWKV, KV, HD>(kbuf[s], kbase, nk.k_new, tt, new_pos, kvh, j);
-            attn_issue_row<NEWKV, KV, HD>(vpre[s], vbase, nk.v_new, tt, new_pos, kvh, j);
+            Lay::ld(kbase + static_cast<uint64_t>(tt) * HD, j, kbuf[s]);
+            Lay::ld(vbase + static_cast<uint64_t>(tt) * HD, j, vpre[s]);
         }
     };
     if (PREFETCH_V && t_begin < t_end) issue_chunk(t_begin);
+    float4 kn[NQ], vn[NQ];
+    if (own_new) {
+        attn_new_row_load<KV, HD>(kn, nk.k_new, kvh, j);
+        attn_new_row_load<KV, HD>(vn, nk.v_new, kvh, j);
+    }
 
     // this lane's 16 q values for each of the G heads, and its part of the position's RoPE row
     float4 qv[G][NQ], cs[NQ];
@@ -204,37 +196,19 @@ __device__ __forceinline__ void attn_decode_range(const float* __restrict__ q, c
     }
 
     for (uint32_t t0 = t_begin; t0 < t_end; t0 += t_step) {
-        if (PREFETCH_V) {
-            if (t0 != t_begin) issue_chunk(t0);
-            if (NEWKV) {
-#pragma unroll
-                for (int s = 0; s < S; ++s) {
-                    const uint32_t t = t0 + 8 * s + pg, tt = t < t_end ? t : t_begin;
-                    if (tt == new_pos) {
-                        const uint64_t row = static_cast<uint64_t>(kvh) * max_seq + tt;
-                        const bool store = write_new && t < t_end;
-                        attn_finish_new_row<true, KV, HD>(kbuf[s], cs, nk.rope_type, nk.kc_w, row, j, store);
-                        attn_finish_new_row<false, KV, HD>(vpre[s], cs, 0, nk.vc_w, row, j, store);
-                    }
-                }
-            }
-        }
+        if (PREFETCH_V && t0 != t_begin) issue_chunk(t0);
         // ---- scores: step s covers positions t0 + 8s + pg
         float sc[G][S];
 #pragma unroll
         for (int s = 0; s < S; ++s) {
             const uint32_t t = t0 + 8 * s + pg;
             const bool live = t < t_end;
-            const uint32_t tt = live ? t : t_begin;
             float4 kv[NQ];
             if (PREFETCH_V) {
 #pragma unroll
                 for (int c = 0; c < NQ; ++c) kv[c] = kbuf[s][c];
             } else {
-                attn_issue_row<NEWKV, KV, HD>(kv, kbase, nk.k_new, tt, new_pos, kvh, j);
-                if (NEWKV && tt == new_pos)
-                    attn_finish_new_row<true, KV, HD>(kv, cs, nk.rope_type, nk.kc_w, static_cast<uint64_t>(kvh) * max_seq + tt,
-                                                      j, write_new && live);
+                Lay::ld(kbase + static_cast<uint64_t>(live ? t : t_begin) * HD, j, kv);
             }
 #pragma unroll
             for (int h = 0; h < G; ++h) {
@@ -285,8 +259,7 @@ __device__ __forceinline__ void attn_decode_range(const float* __restrict__ q, c
                 for (int c = 0; c < NQ; ++c) vv[c] = vpre[s][c];
             } else {
                 const uint32_t t = t0 + 8 * s + pg;
-                attn_load_v<NEWKV, KV, HD>(vv, vbase, t, t < t_end ? t : t_begin, new_pos, kvh, max_seq, j, nk,
-                                       write_new && t == new_pos);
+                Lay::ld(vbase + static_cast<uint64_t>(t < t_end ? t : t_begin) * HD, j, vv);
             }
 #pragma unroll
             for (int h = 0; h < G; ++h) {
@@ -300,6 +273,43 @@ __device__ __forceinline__ void attn_decode_range(const float* __restrict__ q, c
                     acc[h][c].z = fmaf(p, vv[c].z, acc[h][c].z);
                     acc[h][c].w = fmaf(p, vv[c].w, acc[h][c].w);
                 }
+            }
+        }
+    }
+
+    // ---- the token's own position: every position group holds the same row, so the score is the
+    // same in all lanes; group 0 alone accumulates it and (if this caller owns the append) stores
+    // the row into the cache
+    if (own_new) {
+        const uint64_t row = static_cast<uint64_t>(kvh) * max_seq + new_pos;
+        attn_new_row_finish<true, KV, HD>(kn, cs, nk.rope_type, nk.kc_w, row, j, write_new && pg == 0);
+        attn_new_row_finish<false, KV, HD>(vn, cs, 0, nk.vc_w, row, j, write_new && pg == 0);
+#pragma unroll
+        for (int h = 0; h < G; ++h) {
+            float d = 0.0f;
+#pragma unroll
+            for (int c = 0; c < NQ; ++c) {
+                d = fmaf(qv[h][c].x, kn[c].x, d);
+                d = fmaf(qv[h][c].y, kn[c].y, d);
+                d = fmaf(qv[h][c].z, kn[c].z, d);
+                d = fmaf(qv[h][c].w, kn[c].w, d);
+            }
+            d += dpp_f<0xB1>(d);
+            d += dpp_f<0x4E>(d);
+            d += dpp_f<0x141>(d);
+            const float sn = d * scale;
+            const float m_new = fmaxf(m[h], sn);
+            const float corr = cera_expf(m[h] - m_new);   // 0 when nothing came before (m = -inf)
+            m[h] = m_new;
+            l[h] *= corr;
+            const float p = pg == 0 ? cera_expf(sn - m_new) : 0.0f;
+            l[h] += (j == 0) ? p : 0.0f;
+#pragma unroll
+            for (int c = 0; c < NQ; ++c) {
+                acc[h][c].x = fmaf(p, vn[c].x, acc[h][c].x * corr);
+                acc[h][c].y = fmaf(p, vn[c].y, acc[h][c].y * corr);
+                acc[h][c].z = fmaf(p, vn[c].z, acc[h][c].z * corr);
+                acc[h][c].w = fmaf(p, vn[c].w, acc[h][c].w * corr);
             }
         }
     }
@@ -598,13 +608,21 @@ __global__ __launch_bounds__(256) void attn_decode_merge_kernel(const float* __r
         acc.x = fmaf(w, pre[i].x, acc.x); acc.y = fmaf(w, pre[i].y, acc.y);
         acc.z = fmaf(w, pre[i].z, acc.z); acc.w = fmaf(w, pre[i].w, acc.w);
     }
-#pragma unroll 2
-    for (uint32_t p = grp + 8 * ATTN_MERGE_PF; p < n_parts; p += 8) {
-        const float w = wbuf[p];
-        float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (live) a = reinterpret_cast<const float4*>(part_acc + ((pbase + p) * G + hg) * HD)[c];
-        acc.x = fmaf(w, a.x, acc.x); acc.y = fmaf(w, a.y, acc.y);
-        acc.z = fmaf(w, a.z, acc.z); acc.w = fmaf(w, a.w, acc.w);
+    // further parts in batches of ATTN_MERGE_PF per group, each batch one memory round trip
+    for (uint32_t base = 8 * ATTN_MERGE_PF; base < n_parts; base += 8 * ATTN_MERGE_PF) {
+#pragma unroll
+        for (int i = 0; i < ATTN_MERGE_PF; ++i) {
+            const uint32_t p = base + grp + 8 * i;
+            pre[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (p < n_parts && live) pre[i] = reinterpret_cast<const float4*>(part_acc + ((pbase + p) * G + hg) * HD)[c];
+        }
+#pragma unroll
+        for (int i = 0; i < ATTN_MERGE_PF; ++i) {
+            const uint32_t p = base + grp + 8 * i;
+            const float w = p < n_parts ? wbuf[p] : 0.0f;
+            acc.x = fmaf(w, pre[i].x, acc.x); acc.y = fmaf(w, pre[i].y, acc.y);
+            acc.z = fmaf(w, pre[i].z, acc.z); acc.w = fmaf(w, pre[i].w, acc.w);
+        }
     }
     sacc[grp][c] = acc;
     __syncthreads();

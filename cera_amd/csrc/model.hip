@@ -460,9 +460,9 @@ static cera_hip_status decode_step(cera_hip_model* m, uint32_t pos, bool want_lo
             hipLaunchKernelGGL((rmsnorm_kernel<false>), dim3(c.n_kv_heads), dim3(256), 0, s, m->k, L.k_norm, c.head_dim,
                                c.rms_eps, m->k, nullptr, nullptr, nullptr);
         }
-        // attention over positions [0, pos]: the kernel rotates q on load, takes the new token's
-        // K/V rows from the projections (rotating K) and appends them to the cache itself; the
-        // merge also quantizes for the O projection
+        // attention over positions [0, pos]; the merge also quantizes for the O projection.  While the
+        // context is short the kernel rotates q on load, takes the new token's K/V rows from the
+        // projections (rotating K) and appends them to the cache itself
         AttnNewKV nk;
         nk.rope_row = m->rope_table + static_cast<uint64_t>(pos) * c.head_dim;
         nk.rope_type = c.rope_type;
@@ -470,8 +470,24 @@ static cera_hip_status decode_step(cera_hip_model* m, uint32_t pos, bool want_lo
         nk.v_new = m->v;
         nk.kc_w = L.kc;
         nk.vc_w = L.vc;
-        CERA_TRY(cera_launch_attn_decode(ctx, m->q, L.kc, L.vc, c.n_heads, c.n_kv_heads, c.head_dim, pos + 1,
-                                         c.max_seq_len, scale, 0, m->attn_out, m->xs, m->xq, &nk, m->kv_f16));
+        if (pos + 1 < ATTN_FUSED_NEW_KV_MAX_KEYS) {
+            CERA_TRY(cera_launch_attn_decode(ctx, m->q, L.kc, L.vc, c.n_heads, c.n_kv_heads, c.head_dim, pos + 1,
+                                             c.max_seq_len, scale, 0, m->attn_out, m->xs, m->xq, &nk, m->kv_f16));
+        } else {
+            // longer contexts: RoPE + cache append as their own launch, then plain attention
+            const dim3 rgrid(c.n_heads + 2 * c.n_kv_heads, 1), rblock(c.head_dim / 2);
+            if (m->kv_f16)
+                hipLaunchKernelGGL(rope_kv_kernel<kv_half>, rgrid, rblock, 0, s, m->q, m->k, m->v, m->rope_table,
+                                   m->scalars + 1, c.n_heads, c.n_kv_heads, c.head_dim, c.rope_type,
+                                   static_cast<kv_half*>(L.kc), static_cast<kv_half*>(L.vc), c.max_seq_len);
+            else
+                hipLaunchKernelGGL(rope_kv_kernel<float>, rgrid, rblock, 0, s, m->q, m->k, m->v, m->rope_table,
+                                   m->scalars + 1, c.n_heads, c.n_kv_heads, c.head_dim, c.rope_type,
+                                   static_cast<float*>(L.kc), static_cast<float*>(L.vc), c.max_seq_len);
+            HIP_TRY(ctx, hipGetLastError());
+            CERA_TRY(cera_launch_attn_decode(ctx, m->q, L.kc, L.vc, c.n_heads, c.n_kv_heads, c.head_dim, pos + 1,
+                                             c.max_seq_len, scale, 0, m->attn_out, m->xs, m->xq, nullptr, m->kv_f16));
+        }
         CERA_TRY(project(m, L.o, m->attn_out, m->hidden, m->hidden));
 
         CERA_TRY(norm_quant(m, m->hidden, L.ffn_norm, c.hidden, 1, m->normed));

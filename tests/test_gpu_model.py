@@ -351,3 +351,32 @@ def test_head_dim_64_shift_bitwise(hip, orc):
             assert np.array_equal(kg.view(np.uint32), ko.view(np.uint32)), (rope_type, layer)
             assert np.array_equal(vg.view(np.uint32), vo.view(np.uint32)), (rope_type, layer)
         gm.close(); om.close()
+
+
+@pytest.mark.parametrize("kv_f16", [False, True])
+def test_decode_across_the_fused_append_window(hip, orc, kv_f16):
+    """Below 1024 keys the attention kernel rotates q and appends the token's K/V itself; from there
+    on a RoPE/append launch precedes plain attention.  Decode across the switch tracks the oracle,
+    and the rows appended on either side of it land in the cache alike."""
+    cfg = dict(synth.TINY, max_seq_len=1100)
+    weights = synth.make_llama(cfg, seed=77, sigma=0.05, norm_jitter=0.1)
+    gm = hip_api.Model(hip, cfg, weights)
+    om = orc.Llama(cfg, weights)
+    if kv_f16:
+        gm.configure_kv(True); om.set_kv_f16(True)
+    toks = [int(t) for t in util.rng(71).integers(0, cfg["vocab"], 1018)]
+    _say(f"decode across 1024 keys, f16={kv_f16}")
+    lg, lo = gm.forward_prefill(toks, 0), om.forward_prefill_batched(toks, 0)
+    assert _cos(lg, lo) > 0.999
+    for i in range(12):                      # positions 1018 .. 1029
+        t = int(orc_argmax(lo))
+        lg, lo = gm.forward(t, 1018 + i), om.forward(t, 1018 + i)
+        assert _cos(lg, lo) > 0.999, i
+    assert gm.seq_len == om.seq_len == 1030
+    kvd = cfg["n_kv_heads"] * cfg["head_dim"]
+    kg, vg = gm.read_kv(0)
+    ko, vo = om.kv(0)
+    rows = slice(1016 * kvd, 1030 * kvd)
+    assert np.abs(kg[rows] - ko[rows]).max() <= 3e-3 * util.rms(ko[rows])
+    assert np.abs(vg[rows] - vo[rows]).max() <= 3e-3 * util.rms(vo[rows])
+    gm.close(); om.close()
