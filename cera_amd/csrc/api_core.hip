@@ -5,12 +5,18 @@
 
 #include "attention.cuh"
 #include "gemv_launch.cuh"
+#include "gemv_nb.cuh"
 #include "glue.cuh"
 #include "host_common.h"
 #include "quantize.cuh"
 
 bool cera_gemv_launch_q4k(const GemvArgs&, const GemvPlan&, int, bool, hipStream_t);
 bool cera_gemv_launch_pair_q4k_q6k(const GemvPairArgs& a, const GemvPlan& pa, const GemvPlan& pb, hipStream_t s);
+bool cera_gemv_nb_launch_q4k(const GemvNbArgs&, int, int, int, bool, uint32_t, hipStream_t);
+bool cera_gemv_nb_launch_q6k(const GemvNbArgs&, int, int, int, bool, uint32_t, hipStream_t);
+bool cera_gemv_nb_launch_q4_0(const GemvNbArgs&, int, int, int, bool, uint32_t, hipStream_t);
+bool cera_gemv_nb_launch_q4_1(const GemvNbArgs&, int, int, int, bool, uint32_t, hipStream_t);
+bool cera_gemv_nb_launch_q8_0(const GemvNbArgs&, int, int, int, bool, uint32_t, hipStream_t);
 bool cera_gemv_launch_q6k(const GemvArgs&, const GemvPlan&, int, bool, hipStream_t);
 bool cera_gemv_launch_q4_0(const GemvArgs&, const GemvPlan&, int, bool, hipStream_t);
 bool cera_gemv_launch_q4_1(const GemvArgs&, const GemvPlan&, int, bool, hipStream_t);
@@ -381,6 +387,51 @@ cera_hip_status cera_launch_gemv(cera_hip_ctx* ctx, const cera_hip_dtensor* w, c
     return CERA_HIP_OK;
 }
 
+// A short batch of tokens through one matrix with the weights streamed once per 8 tokens:
+// y[t][row] (row stride 1, token stride y_stride) = W . x_t (+ resid, same layout).  *launched is
+// false when the shape has no multi-token instance (two units per lane, i.e. very long rows):
+// the caller then takes the GEMM route.
+cera_hip_status cera_launch_gemv_nb(cera_hip_ctx* ctx, const cera_hip_dtensor* w, const float* xs, const int8_t* xq,
+                                    uint32_t xs_stride, uint32_t xq_stride, uint32_t n_tok, float* y, uint32_t y_stride,
+                                    const float* resid, bool* launched) {
+    *launched = false;
+    if (!is_int8_type(w->dtype) || n_tok == 0) return CERA_HIP_OK;
+    const uint32_t n_units = static_cast<uint32_t>(w->k / (w->dtype == CERA_HIP_Q6_K ? Q6K::ELEMS_PER_UNIT : 32));
+    GemvPlan p;
+    if (!gemv_plan(static_cast<uint32_t>(w->m), n_units, ctx->n_cu, false, 2, &p) || p.U != 1) return CERA_HIP_OK;
+    const int KS = p.KS == 7 ? 8 : p.KS;   // instantiated widths: 1, 2, 4, 8 (surplus lanes carry zero activations)
+    GemvNbArgs a;
+    a.w = w->dev;
+    a.m = static_cast<uint32_t>(w->m);
+    a.n_units = n_units;
+    a.row_bytes = static_cast<uint32_t>(w->row_bytes);
+    a.rows_per_block = p.rows_per_block;
+    a.xq_stride = xq_stride;
+    a.xs_stride = xs_stride;
+    a.y_stride = y_stride;
+    for (uint32_t t0 = 0; t0 < n_tok; t0 += 8) {
+        const uint32_t nt = std::min(8u, n_tok - t0);
+        const int NB = nt <= 2 ? 2 : (nt <= 4 ? 4 : 8);
+        a.n_tok = nt;
+        a.xq = xq + static_cast<uint64_t>(t0) * xq_stride;
+        a.xs = xs + static_cast<uint64_t>(t0) * xs_stride;
+        a.y = y + static_cast<uint64_t>(t0) * y_stride;
+        a.resid = resid ? resid + static_cast<uint64_t>(t0) * y_stride : nullptr;
+        bool ok = false;
+        switch (w->dtype) {
+            case CERA_HIP_Q4_K: ok = cera_gemv_nb_launch_q4k(a, KS, p.RB, NB, resid != nullptr, p.n_blocks, ctx->stream); break;
+            case CERA_HIP_Q6_K: ok = cera_gemv_nb_launch_q6k(a, KS, p.RB, NB, resid != nullptr, p.n_blocks, ctx->stream); break;
+            case CERA_HIP_Q4_0: ok = cera_gemv_nb_launch_q4_0(a, KS, p.RB, NB, resid != nullptr, p.n_blocks, ctx->stream); break;
+            case CERA_HIP_Q4_1: ok = cera_gemv_nb_launch_q4_1(a, KS, p.RB, NB, resid != nullptr, p.n_blocks, ctx->stream); break;
+            case CERA_HIP_Q8_0: ok = cera_gemv_nb_launch_q8_0(a, KS, p.RB, NB, resid != nullptr, p.n_blocks, ctx->stream); break;
+        }
+        if (!ok) return t0 == 0 ? CERA_HIP_OK : cera_fail(ctx, CERA_HIP_ERR_SHAPE, "gemv_nb: no kernel instance for this shape");
+        HIP_TRY(ctx, hipGetLastError());
+    }
+    *launched = true;
+    return CERA_HIP_OK;
+}
+
 // Two projections of the same quantized activations in one launch (plain store epilogue).
 // *launched is false when no paired kernel instance covers the two shapes: the caller then
 // launches them one after the other.
@@ -644,6 +695,33 @@ cera_hip_status cera_hip_gemv(cera_hip_ctx* ctx, const cera_hip_tensor* t, const
         return CERA_HIP_OK;
     };
     st = run();
+    cera_hip_tensor_free(ctx, w);
+    return st;
+}
+
+cera_hip_status cera_hip_gemv_nb(cera_hip_ctx* ctx, const cera_hip_tensor* t, const float* x, uint32_t n, float* y) {
+    if (!ctx || !t || !x || !y) return CERA_HIP_ERR_ARGUMENT;
+    if (n == 0 || t->k == 0 || t->k % 32) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "gemv_nb: need n > 0 and k a multiple of 32");
+    cera_hip_dtensor* w = nullptr;
+    CERA_TRY(cera_hip_tensor_upload(ctx, t, &w));
+    auto run = [&]() -> cera_hip_status {
+        const uint64_t k = w->k, m = w->m;
+        void *dx, *ds, *dq, *dy;
+        CERA_TRY(cera_scratch(ctx, 0, n * k * 4, &dx));
+        CERA_TRY(cera_scratch(ctx, 1, n * (k / 32) * 4, &ds));
+        CERA_TRY(cera_scratch(ctx, 2, n * k, &dq));
+        CERA_TRY(cera_scratch(ctx, 3, n * m * 4, &dy));
+        CERA_TRY(cera_hip_upload(ctx, dx, x, n * k * 4));
+        // rows are multiples of 32 long, so quantizing the n rows as one vector is row by row
+        CERA_TRY(cera_launch_quantize(ctx, static_cast<float*>(dx), n * k, static_cast<float*>(ds), static_cast<int8_t*>(dq)));
+        bool launched = false;
+        CERA_TRY(cera_launch_gemv_nb(ctx, w, static_cast<float*>(ds), static_cast<int8_t*>(dq), static_cast<uint32_t>(k / 32),
+                                     static_cast<uint32_t>(k), n, static_cast<float*>(dy), static_cast<uint32_t>(m), nullptr,
+                                     &launched));
+        if (!launched) return cera_fail(ctx, CERA_HIP_ERR_UNSUPPORTED_DTYPE, "gemv_nb: no multi-token kernel instance for this type / shape");
+        return cera_hip_download(ctx, y, dy, n * m * 4);
+    };
+    cera_hip_status st = run();
     cera_hip_tensor_free(ctx, w);
     return st;
 }

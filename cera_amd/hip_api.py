@@ -27,7 +27,7 @@ SYMBOLS = [
     "cera_hip_quantize_q8_0_dev", "cera_hip_gemv_q8_dev", "cera_hip_gemv_seq_dev", "cera_hip_attn_decode_dev",
     "cera_hip_gemm_dev",
     "cera_hip_model_create", "cera_hip_model_destroy", "cera_hip_forward", "cera_hip_forward_greedy",
-    "cera_hip_forward_prefill", "cera_hip_forward_prefill_logits_all", "cera_hip_truncate_kv", "cera_hip_gemv_pair", "cera_hip_configure_kv", "cera_hip_kv_type", "cera_hip_attn_f16kv",
+    "cera_hip_forward_prefill", "cera_hip_forward_prefill_logits_all", "cera_hip_truncate_kv", "cera_hip_gemv_pair", "cera_hip_gemv_nb", "cera_hip_configure_kv", "cera_hip_kv_type", "cera_hip_attn_f16kv",
     "cera_hip_attn_decode_f16_dev", "cera_hip_shift_kv", "cera_hip_write_kv", "cera_hip_set_seq_len", "cera_hip_seq_len", "cera_hip_memory_bytes",
     "cera_hip_read_kv", "cera_hip_read_hidden",
 ]
@@ -117,6 +117,7 @@ def load_library() -> C.CDLL:
         "cera_hip_forward_prefill_logits_all": (i32, [vp, vp, u32, u32, vp]),
         "cera_hip_truncate_kv": (i32, [vp, u32]),
         "cera_hip_gemv_pair": (i32, [vp, vp, vp, vp, vp, vp]),
+        "cera_hip_gemv_nb": (i32, [vp, vp, vp, u32, vp]),
         "cera_hip_configure_kv": (i32, [vp, u32]),
         "cera_hip_kv_type": (u32, [vp]),
         "cera_hip_attn_f16kv": (i32, [vp, vp, vp, vp, u32, u32, u32, u64, u32, f32, u32, vp]),
@@ -278,6 +279,14 @@ class Context:
         self.check(self.lib.cera_hip_attn_prefill(self.h, _p(q), _p(k), _p(v), n_heads, n_kv_heads, head_dim, start_pos,
                                                   n_queries, scale, _p(out)))
         return out.reshape(n_queries, n_heads * head_dim)
+
+    def gemv_nb(self, ggml_type: int, blocks: np.ndarray, x: np.ndarray, m: int, k: int) -> np.ndarray:
+        """x [n][k] -> y [n][m] through the multi-token GEMV."""
+        t = make_tensor(ggml_type, m, k, blocks)
+        x = np.ascontiguousarray(x, np.float32).reshape(-1, k)
+        y = np.empty((x.shape[0], m), np.float32)
+        self.check(self.lib.cera_hip_gemv_nb(self.h, C.byref(t), _p(x), x.shape[0], _p(y)))
+        return y
 
     def gemv_pair(self, type_a, wa, ma, type_b, wb, mb, x, k):
         ta, tb = make_tensor(type_a, ma, k, wa), make_tensor(type_b, mb, k, wb)

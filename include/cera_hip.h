@@ -145,6 +145,15 @@ CERA_HIP_API cera_hip_status cera_hip_quantize_q8_0(cera_hip_ctx*, const float* 
 CERA_HIP_API cera_hip_status cera_hip_gemv(cera_hip_ctx*, const cera_hip_tensor* w, const float* x, float* y,
                                            int32_t* dbg_block_dots, int32_t* dbg_block_asums);
 
+/* The same product for a short batch of n activation vectors (x f32 [n][k], y f32 [n][m]) with
+ * the weights streamed once per 8 vectors: what the prefill path runs instead of the int8 GEMM
+ * while a batch is at most 16 tokens (a few new tokens of a chat turn, the verification pass of
+ * speculative decoding, cera/src/model/mod.rs:221-249).  Row t of y is bit-identical to
+ * cera_hip_gemv on x[t].  CERA_HIP_ERR_UNSUPPORTED_DTYPE for Q5_K and for k beyond one unit per
+ * lane (k > 16384, Q6_K 32768). */
+CERA_HIP_API cera_hip_status cera_hip_gemv_nb(cera_hip_ctx*, const cera_hip_tensor* w, const float* x, uint32_t n,
+                                              float* y);
+
 /* Two projections of the same activation vector in one launch: what the decode step does for a
  * layer whose attn_q|attn_k (Q4_K, stored back to back) and attn_v (Q6_K) differ in block type
  * (the Q4_K_M mix, cera/src/convert/quantize.rs:102-113); each result is exactly that of

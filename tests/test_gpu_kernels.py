@@ -437,3 +437,28 @@ def test_gemv_pair_refuses_what_it_has_no_instance_for(hip):
     with pytest.raises(hip_api.HipError) as e:   # types the other way round
         hip.gemv_pair(Q6_K, wb, 8, Q4_K, wa, 8, util.make_x(k, 3), k)
     assert e.value.status == 3
+
+
+# ---- a few tokens per weight pass ------------------------------------------------------
+@pytest.mark.parametrize("dtype", util.INT8_TYPES)
+@pytest.mark.parametrize("n", [1, 2, 3, 5, 8, 11, 16])
+def test_gemv_multi_token_is_bitwise_per_token_gemv(hip, orc, dtype, n):
+    """Short batches go through the multi-token GEMV: every row of the result equals the
+    single-vector kernel on that token bit for bit, for every K-split width."""
+    for m, k in [(37, 256), (130, 4096), (9, 14336), (260, 1024)]:
+        _say(f"gemv_nb {util.NAMES[dtype]} n={n} m={m} k={k}")
+        w, _ = util.make_weights(dtype, m, k, seed=dtype * 31 + n)
+        x = util.rng(900 + n).standard_normal((n, k)).astype(np.float32)
+        y = hip.gemv_nb(dtype, w, x, m, k)
+        for t in range(n):
+            one = hip.gemv(dtype, w, x[t], m, k)
+            assert np.array_equal(y[t].view(np.uint32), one.view(np.uint32)), (m, k, t)
+        ref = orc.gemv(dtype, w, x[n - 1], m, k)
+        assert np.abs(y[n - 1] - ref).max() <= GEMV_TOL * util.rms(ref)
+
+
+def test_gemv_multi_token_refusals(hip):
+    with pytest.raises(hip_api.HipError) as e:   # two units per lane: no multi-token instance
+        w, _ = util.make_weights(Q4_K, 4, 28672, seed=1)
+        hip.gemv_nb(Q4_K, w, np.zeros((2, 28672), np.float32), 4, 28672)
+    assert e.value.status == 3
