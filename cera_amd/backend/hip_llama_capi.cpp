@@ -1,5 +1,8 @@
 #include "hip_llama_capi.h"
 
+#include <algorithm>
+#include "spec.h"
+
 #include <chrono>
 #include <cmath>
 #include <cstring>
@@ -175,6 +178,31 @@ int cera_llama_generate_greedy(cera_llama* h, const uint32_t* prompt, uint64_t n
         double t2 = now_s();
         if (prefill_s) *prefill_s = t1 - t0;
         if (decode_s) *decode_s = t2 - t1;
+    });
+}
+
+uint64_t cera_spec_prompt_lookup_draft(const uint32_t* tokens, uint64_t n, uint64_t ngram, uint64_t k, uint32_t* out,
+                                       uint64_t cap) {
+    if ((!tokens && n) || (!out && cap)) return 0;
+    const std::vector<uint32_t> d = cera::prompt_lookup_draft(tokens, n, ngram, k);
+    const uint64_t m = std::min<uint64_t>(d.size(), cap);
+    std::copy(d.begin(), d.begin() + m, out);
+    return m;
+}
+
+int cera_llama_generate_spec(cera_llama* h, const uint32_t* prompt, uint64_t n_prompt, uint64_t max_new, const uint32_t* eos,
+                             uint64_t n_eos, uint64_t ngram, uint64_t k, uint32_t* out, uint64_t* n_out, uint64_t stats[3],
+                             double* seconds) {
+    return guarded(h, [&] {
+        if (!out || !n_out) throw cera::BackendError("generate_spec: null output");
+        const std::vector<uint32_t> p(prompt, prompt + n_prompt), e(eos, eos + (eos ? n_eos : 0));
+        cera::SpecStats st;
+        const double t0 = now_s();
+        const std::vector<uint32_t> toks = cera::greedy_generate_spec(*h->model, h->state, p, max_new, e, ngram, k, &st);
+        if (seconds) *seconds = now_s() - t0;
+        std::copy(toks.begin(), toks.end(), out);
+        *n_out = toks.size();
+        if (stats) { stats[0] = st.drafted; stats[1] = st.accepted; stats[2] = st.rounds; }
     });
 }
 

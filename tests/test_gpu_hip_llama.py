@@ -327,3 +327,45 @@ def test_head_dim_64_file(tmp_path, orc, hip, arch, explicit):
         _teacher_forced(gm, om, orc, [11, 22, 33, 44, 55, 66, 77], 14, 12)
     finally:
         gm.close(); om.close()
+
+
+# ---- speculative decoding (the caller of forward_prefill_logits_all / truncate_kv) ---------
+def _plain_greedy(path, prompt, n_new):
+    gm = llama_api.HipLlama(path, context_size=64)
+    try:
+        return gm.generate_greedy(prompt, n_new)[0]
+    finally:
+        gm.close()
+
+
+def test_speculative_greedy_is_a_greedy_decode(tiny_llama):
+    """cera/tests/spec_decode_logits.rs:212-330 in spirit: every emitted token is the target's own
+    argmax, so the stream equals the sequential greedy loop (on this small model, token for
+    token); a drafter that never matches (ngram 999) runs no verification round at all; EOS is
+    not emitted; the budget cap is exact."""
+    path, cfg, _, _ = tiny_llama
+    prompt = [5, 6, 7, 8] * 5
+    plain = [int(t) for t in _plain_greedy(path, prompt, 30)]
+    gm = llama_api.HipLlama(path, context_size=64)
+    try:
+        spec, st = gm.generate_spec(prompt, 30, ngram=2, k=4)
+        _say(f"spec: drafted {st['drafted']} accepted {st['accepted']} rounds {st['rounds']}")
+        assert spec == plain
+        assert st["rounds"] > 0 and 0 <= st["accepted"] <= st["drafted"]
+        assert gm.seq_len <= len(prompt) + 30
+        with pytest.raises(llama_api.BackendError):
+            gm.generate_spec(prompt, 4)                      # the session is no longer fresh
+        gm.truncate_kv(0)
+        none, st0 = gm.generate_spec(prompt, 30, ngram=999, k=4)
+        assert none == plain and st0["rounds"] == 0 and st0["drafted"] == 0
+        gm.truncate_kv(0)
+        stop_at = 11
+        eos = [plain[stop_at]]
+        first = plain.index(eos[0])
+        cut, _ = gm.generate_spec(prompt, 30, eos=eos, ngram=2, k=4)
+        assert cut == plain[:first]                           # the EOS token itself is not emitted
+        gm.truncate_kv(0)
+        capped, _ = gm.generate_spec(prompt, 7, ngram=2, k=4)
+        assert capped == plain[:7]
+    finally:
+        gm.close()
