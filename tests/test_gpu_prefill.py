@@ -188,3 +188,27 @@ def test_attn_prefill_batch_head_dim_64(hip, orc, kv_f16, nh, nkv, start, n):
         ref = orc.decode_attention(q[i], k[:Li * nkv * hd], v[:Li * nkv * hd], nh, nkv, hd, scale, Li)
         err = np.abs(out[i].astype(np.float64) - ref).max()
         assert err <= 2e-3 * util.rms(ref), (i, err, util.rms(ref))
+
+
+def test_prefill_longer_than_one_pass(hip, orc):
+    """A prompt beyond the 2048-token pass size is cut into passes; logits and the cache rows on
+    both sides of the cut track the oracle's single batched prefill."""
+    cfg = dict(synth.TINY, max_seq_len=2200)
+    weights = synth.make_llama(cfg, seed=79, sigma=0.05, norm_jitter=0.1)
+    gm = hip_api.Model(hip, cfg, weights)
+    om = orc.Llama(cfg, weights)
+    toks = [int(t) for t in util.rng(9).integers(0, cfg["vocab"], 2100)]
+    _say("model: prefill 2100 tokens (two passes)")
+    lg = gm.forward_prefill(toks, 0)
+    lo = om.forward_prefill_batched(toks, 0)
+    assert gm.seq_len == om.seq_len == 2100
+    assert _cos(lg, lo) > 0.999
+    kvd = cfg["n_kv_heads"] * cfg["head_dim"]
+    kg, vg = gm.read_kv(0)
+    ko, vo = om.kv(0)
+    rows = slice(2040 * kvd, 2060 * kvd)
+    assert np.abs(kg[rows] - ko[rows]).max() <= 2e-3 * util.rms(ko[rows])
+    assert np.abs(vg[rows] - vo[rows]).max() <= 2e-3 * util.rms(vo[rows])
+    lg2, lo2 = gm.forward(3, 2100), om.forward(3, 2100)
+    assert _cos(lg2, lo2) > 0.999
+    gm.close(); om.close()
