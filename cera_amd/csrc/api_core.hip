@@ -371,7 +371,7 @@ cera_hip_status cera_launch_gemv(cera_hip_ctx* ctx, const cera_hip_dtensor* w, c
     a.dbg_stride = static_cast<uint32_t>(w->dtype == CERA_HIP_Q6_K ? w->k / 16 : w->k / 32);
     const bool dbg = dbg_dots != nullptr;
     GemvPlan p;
-    if (!gemv_plan(a.m, n_units, ctx->n_cu, dbg, w->dtype == CERA_HIP_Q6_K ? 2 : 4, &p))
+    if (!gemv_plan(a.m, n_units, ctx->n_cu, dbg, w->dtype == CERA_HIP_Q6_K ? 2 : 4, &p, epi == CERA_EPI_SILU_MUL))
         return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "gemv: k=" + std::to_string(w->k) + " exceeds the 32768 supported by the register-resident kernel");
     a.rows_per_wave = p.rows_per_block;
     bool ok = false;

@@ -23,11 +23,15 @@ static inline bool gemv_pick_split(uint32_t n_units, int* U, int* KS) {
 
 // Measured on MI355X: ~32 wavefronts per CU in flight, four rows per workgroup
 // step for the 16-byte-unit formats and two for Q6_K (15 registers per row).
-static inline bool gemv_plan(uint32_t m, uint32_t n_units, uint32_t n_cu, bool dbg, int max_rb, GemvPlan* p) {
+static inline bool gemv_plan(uint32_t m, uint32_t n_units, uint32_t n_cu, bool dbg, int max_rb, GemvPlan* p,
+                             bool dual = false) {
     if (!gemv_pick_split(n_units, &p->U, &p->KS)) return false;
     // very tall matrices (the vocabulary head) do better with few long-lived workgroups that
     // stream row groups through the two register buffers; everything else with many short ones
-    const uint32_t per_cu = m >= 65536 ? 4 : 32;
+    // (wavefronts per CU the launch aims at; the fused gate+up pair, whose workgroups carry two
+    // matrices' rows, likes 32, plain two-wavefront splits 24, the wide K splits of long rows 16:
+    // measured 2-3 % apart on the Llama-3-8B shapes)
+    const uint32_t per_cu = m >= 65536 ? 4 : (dual ? 32 : (p->KS >= 4 ? 16 : 24));
     const uint32_t target_blocks = std::max(1u, n_cu * per_cu / static_cast<uint32_t>(p->KS));
     uint32_t rpb = (m + target_blocks - 1) / target_blocks;
     p->RB = rpb >= 4 ? 4 : (rpb >= 2 ? 2 : 1);
