@@ -183,7 +183,7 @@ static cera_hip_status prefill_chunk(cera_hip_model* m, const uint32_t* tokens, 
     auto gemm = [&](const cera_hip_dtensor* w, float* out, const float* resid) -> cera_hip_status {
         // a short batch streams the weights once per 8 tokens through the multi-token GEMV (an
         // int8-MFMA tile would be mostly empty); its residual add is unscaled
-        if (n <= PREFILL_SMALL_BATCH && (!resid || c.residual_scale == 1.0f)) {
+        if ((n <= PREFILL_SMALL_BATCH || !cera_gemm_supports(w->dtype, w->k)) && (!resid || c.residual_scale == 1.0f)) {
             bool launched = false;
             CERA_TRY(cera_launch_gemv_nb(ctx, w, m->pf_xs, m->pf_xq, static_cast<uint32_t>(w->k / 32),
                                          static_cast<uint32_t>(w->k), n, out, static_cast<uint32_t>(w->m), resid, &launched));
@@ -285,10 +285,21 @@ static cera_hip_status prefill_chunk(cera_hip_model* m, const uint32_t* tokens, 
     return CERA_HIP_OK;
 }
 
+// A matrix can take a batch of tokens either through the int8 GEMM (K in whole 256-element
+// steps) or, any int8 type with one unit per lane, through the multi-token GEMV in passes of 8
+// tokens (unscaled residual add only) -- e.g. the Q4_0 / Q8_0 files of small models whose hidden
+// size is not a multiple of 256.
+static bool batched_supports(const cera_hip_model* m, const cera_hip_dtensor* w) {
+    if (cera_gemm_supports(w->dtype, w->k)) return true;
+    const bool int8_type = w->dtype == CERA_HIP_Q4_0 || w->dtype == CERA_HIP_Q4_1 || w->dtype == CERA_HIP_Q8_0 ||
+                           w->dtype == CERA_HIP_Q4_K || w->dtype == CERA_HIP_Q6_K;
+    const uint64_t unit = w->dtype == CERA_HIP_Q6_K ? 64 : 32;
+    return int8_type && w->k % unit == 0 && w->k / unit <= 512 && m->cfg.residual_scale == 1.0f;
+}
 static bool prefill_batchable(const cera_hip_model* m) {
     for (const LayerDev& L : m->layers)
         for (const cera_hip_dtensor* w : {L.q, L.k, L.v, L.o, L.gate, L.up, L.down})
-            if (!cera_gemm_supports(w->dtype, w->k)) return false;
+            if (!batched_supports(m, w)) return false;
     return true;
 }
 
@@ -298,7 +309,7 @@ cera_hip_status cera_model_prefill_logits_all(cera_hip_model* m, const uint32_t*
     const uint64_t vocab = m->cfg.vocab;
     // single token, or a weight / head type without an int8 GEMM: each forward returns that
     // position's logits (the reference's fallback, cera/src/model/llama.rs:1712-1720)
-    if (n == 1 || !prefill_batchable(m) || !cera_gemm_supports(head->dtype, head->k)) {
+    if (n == 1 || !prefill_batchable(m) || !batched_supports(m, head)) {
         for (uint32_t i = 0; i < n; ++i)
             CERA_TRY(cera_model_decode_logits(m, tokens[i], start_pos + i, logits_all + i * vocab));
         return CERA_HIP_OK;
@@ -312,14 +323,10 @@ cera_hip_status cera_model_prefill_logits_all(cera_hip_model* m, const uint32_t*
 
 cera_hip_status cera_model_prefill(cera_hip_model* m, const uint32_t* tokens, uint32_t n, uint32_t start_pos,
                                    float* last_logits) {
-    // A single token, or a weight type without an int8 GEMM, takes the per-token
+    // A single token, or a weight type with no batched kernel (Q5_K), takes the per-token
     // route -- the same decision LlamaModel::forward_prefill makes (llama.rs:1643,
     // 762-795); it is still the HIP path, only slower.
-    bool batched = n > 1;
-    for (const LayerDev& L : m->layers)
-        for (const cera_hip_dtensor* w : {L.q, L.k, L.v, L.o, L.gate, L.up, L.down})
-            if (!cera_gemm_supports(w->dtype, w->k)) batched = false;
-    if (!batched) return cera_model_prefill_per_token(m, tokens, n, start_pos, last_logits);
+    if (n == 1 || !prefill_batchable(m)) return cera_model_prefill_per_token(m, tokens, n, start_pos, last_logits);
     for (uint32_t off = 0; off < n; off += PREFILL_CHUNK) {
         uint32_t len = std::min(PREFILL_CHUNK, n - off);
         CERA_TRY(prefill_chunk(m, tokens + off, len, start_pos + off, off + len == n));

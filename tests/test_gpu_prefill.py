@@ -212,3 +212,28 @@ def test_prefill_longer_than_one_pass(hip, orc):
     lg2, lo2 = gm.forward(3, 2100), om.forward(3, 2100)
     assert _cos(lg2, lo2) > 0.999
     gm.close(); om.close()
+
+
+@pytest.mark.parametrize("n", [5, 40])
+def test_batched_prefill_when_k_is_not_a_multiple_of_256(hip, orc, n):
+    """Small models' hidden sizes (896, 1536 ...) have no int8-GEMM form; their Q4_0 / Q8_0 matrices
+    still take a batch through the multi-token GEMV (8 tokens per weight pass) instead of one decode
+    step per token.  hidden 288, ffn 480: every K is a multiple of 32 only."""
+    cfg = dict(synth.TINY, hidden=288, ffn=480, n_heads=4, n_kv_heads=2, head_dim=64)
+    type_of = lambda name: Q8_0 if ("attn_v" in name or "ffn_down" in name or "token_embd" in name) else Q4_0
+    weights = synth.make_llama(cfg, seed=83, sigma=0.05, type_of=type_of, norm_jitter=0.1)
+    gm = hip_api.Model(hip, cfg, weights)
+    om = orc.Llama(cfg, weights)
+    toks = [int(t) for t in util.rng(19 + n).integers(0, cfg["vocab"], n)]
+    _say(f"model: hidden 288, batched prefill of {n} tokens over Q4_0 / Q8_0")
+    lg = gm.forward_prefill(toks, 0)
+    lo = om.forward_prefill_per_token(toks, 0)
+    assert gm.seq_len == om.seq_len == n
+    assert _cos(lg, lo) > 0.999
+    kg, vg = gm.read_kv(1)
+    ko, vo = om.kv(1)
+    assert np.abs(kg - ko).max() <= 5e-2 * util.rms(ko) and np.abs(vg - vo).max() <= 5e-2 * util.rms(vo)
+    rows = gm.forward_prefill_logits_all([3, 4, 5], n)
+    for i, t in enumerate([3, 4, 5]):
+        assert _cos(rows[i], om.forward(t, n + i)) > 0.999, i
+    gm.close(); om.close()
