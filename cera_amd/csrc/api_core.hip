@@ -516,8 +516,8 @@ template <typename KV, int HD>
 static void attn_launch_partials(cera_hip_ctx* ctx, const AttnLaunch& a, const KV* kc, const KV* vc) {
     if (a.batch) {
         // heaviest query blocks (most visible keys) first
-        const dim3 pgrid((a.n_queries + 31) / 32, a.n_heads, a.n_parts);
-        hipLaunchKernelGGL((attn_prefill_partial_kernel<KV, HD>), pgrid, dim3(64), 0, ctx->stream, a.q, kc, vc, a.seq_len,
+        const dim3 pgrid((a.n_queries + 31) / 32, a.n_kv_heads, a.n_parts);
+        hipLaunchKernelGGL((attn_prefill_partial_kernel<KV, HD>), pgrid, dim3(64 * a.G), 0, ctx->stream, a.q, kc, vc, a.seq_len,
                            a.n_queries, a.max_seq, a.scale, a.part_keys, a.n_parts, a.q_stride, a.G, ctx->attn_acc,
                            ctx->attn_ml);
         return;

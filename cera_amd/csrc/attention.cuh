@@ -423,12 +423,16 @@ __global__ __launch_bounds__(256) void attn_decode_partial_kernel(
 // produces the (m, l, acc) partial of one (query block, head, part) in the layout
 // the merge kernel below consumes, so long prompts spread over the chip and the
 // merge (and its fused Q8_0 quantisation) is shared with the decode path.
-// grid = (query blocks, heads, parts), 64 threads.
+// A workgroup is the G query heads of one KV head, one wavefront each: the K tile
+// (transposed) and the V tile are staged in LDS once, by all G wavefronts together,
+// and every head of the group reads them from there.
+// grid = (query blocks, KV heads, parts), 64 * G threads.
 #define ATTN_PF_LD 33  // words per LDS row of the transposed K tile (32 + 1 pad)
 typedef float attn_v16f __attribute__((ext_vector_type(16)));
 
+#define ATTN_PF_VLD(HD) ((HD) + 8)   // words per LDS row of the V tile: the halves' rows (4 apart) fall in different banks
 template <typename KV, int HD>
-__global__ __launch_bounds__(64) void attn_prefill_partial_kernel(
+__global__ __launch_bounds__(512) void attn_prefill_partial_kernel(
     const float* __restrict__ q,       // [n_queries][q_stride]
     const KV* __restrict__ kc,         // [n_kv][max_seq][128], already holding the batch's keys
     const KV* __restrict__ vc,
@@ -437,10 +441,13 @@ __global__ __launch_bounds__(64) void attn_prefill_partial_kernel(
     uint32_t G,
     float* __restrict__ part_acc,      // [n_queries][n_kv][n_parts][G][128]
     float* __restrict__ part_ml) {     // [n_queries][n_kv][n_parts][G][2]
+    constexpr int VLD = ATTN_PF_VLD(HD);
     __shared__ float sKt[HD * ATTN_PF_LD];
-    __shared__ __attribute__((aligned(16))) float sX[32];
-    const uint32_t lane = threadIdx.x, col = lane & 31, half = lane >> 5;
-    const uint32_t head = blockIdx.y, kvh = head / G, hg = head % G, n_kv = gridDim.y / G;
+    __shared__ __attribute__((aligned(16))) float sV[32 * VLD];
+    __shared__ __attribute__((aligned(16))) float sXall[8 * 32];
+    const uint32_t tid = threadIdx.x, lane = tid & 63, col = lane & 31, half = lane >> 5;
+    const uint32_t kvh = blockIdx.y, hg = tid >> 6, head = kvh * G + hg, n_kv = gridDim.y;
+    float* sX = sXall + 32 * hg;
     const uint32_t part = blockIdx.z;
     const uint32_t q0 = blockIdx.x * 32, qidx = q0 + col;
     const bool q_live = qidx < n_queries;
@@ -469,16 +476,20 @@ __global__ __launch_bounds__(64) void attn_prefill_partial_kernel(
     double l = 0.0;
 
     for (uint32_t k0 = key_lo; k0 < key_hi; k0 += 32) {
-        // ---- K tile -> LDS, transposed: 32 keys x HD/4 float4, HD/8 per lane
-#pragma unroll
-        for (int i = 0; i < HD / 8; ++i) {
-            const uint32_t f = lane + 64 * i, key = f / (HD / 4), c4 = f % (HD / 4);
-            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (k0 + key < key_hi) v = KvOps<KV>::ld4(kbase + static_cast<uint64_t>(k0 + key) * HD, c4);
+        // ---- K tile -> LDS transposed, V tile -> LDS as it lies: 32 keys x HD/4 float4 each, spread
+        // over the workgroup; keys past the part's end are zeros (their weights are zero too)
+        for (uint32_t f = tid; f < 32 * (HD / 4); f += blockDim.x) {
+            const uint32_t key = f / (HD / 4), c4 = f % (HD / 4);
+            float4 v = make_float4(0.f, 0.f, 0.f, 0.f), w = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (k0 + key < key_hi) {
+                v = KvOps<KV>::ld4(kbase + static_cast<uint64_t>(k0 + key) * HD, c4);
+                w = KvOps<KV>::ld4(vbase + static_cast<uint64_t>(k0 + key) * HD, c4);
+            }
             sKt[(4 * c4 + 0) * ATTN_PF_LD + key] = v.x;
             sKt[(4 * c4 + 1) * ATTN_PF_LD + key] = v.y;
             sKt[(4 * c4 + 2) * ATTN_PF_LD + key] = v.z;
             sKt[(4 * c4 + 3) * ATTN_PF_LD + key] = v.w;
+            *reinterpret_cast<float4*>(sV + key * VLD + 4 * c4) = w;
         }
         __syncthreads();
         // ---- scores, transposed: c[4blk + r] = <K[k0 + 8blk + 4half + r], Q[qidx]>
@@ -511,7 +522,7 @@ __global__ __launch_bounds__(64) void attn_prefill_partial_kernel(
         m = m_new;
         // ---- the correction factors, re-laid out by output row (query 8blk + 4half + r)
         if (half == 0) sX[col] = corr;
-        __syncthreads();
+        __builtin_amdgcn_wave_barrier();   // sX is this wavefront's own: LDS operations of one wavefront complete in order
 #pragma unroll
         for (int blk = 0; blk < 4; ++blk) {
             const float4 cr = *reinterpret_cast<const float4*>(sX + 8 * blk + 4 * half);
@@ -524,13 +535,12 @@ __global__ __launch_bounds__(64) void attn_prefill_partial_kernel(
         // ---- O += P . V
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
-            const uint32_t kg = min(k0 + 8 * (e >> 2) + 4 * half + (e & 3), key_hi - 1);   // masked keys have p = 0
-            const KV* vrow = vbase + static_cast<uint64_t>(kg) * HD + col;
+            const float* vrow = sV + (8 * (e >> 2) + 4 * half + (e & 3)) * VLD + col;
 #pragma unroll
             for (int dt = 0; dt < NDT; ++dt)
-                acc[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(c[e], KvOps<KV>::ld1(vrow + 32 * dt), acc[dt], 0, 0, 0);
+                acc[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(c[e], vrow[32 * dt], acc[dt], 0, 0, 0);
         }
-        __syncthreads();   // sKt and sX are rewritten by the next tile
+        __syncthreads();   // sKt and sV are rewritten by the next tile
     }
 
     // ---- partial out: rows of acc are queries 8blk + 4half + r, columns 32dt + col
