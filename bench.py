@@ -53,6 +53,28 @@ def algorithmic_bytes(H, tname, m, k):
     return m * H.row_bytes(H.TYPE_IDS[tname], k) + k + k // 32 * 4 + m * 4
 
 
+def host_cpu_info():
+    """CPU model and physical / logical core counts of the host the CPU baseline ran on."""
+    model, cores = "unknown", set()
+    try:
+        phys = core = None
+        for line in open("/proc/cpuinfo"):
+            key, _, val = line.partition(":")
+            key, val = key.strip(), val.strip()
+            if key == "model name":
+                model = val
+            elif key == "physical id":
+                phys = val
+            elif key == "core id":
+                core = val
+            elif not key and phys is not None:
+                cores.add((phys, core))
+                phys = core = None
+    except OSError:
+        pass
+    return {"cpu_model": model, "physical_cores": len(cores) or None, "logical_cores": os.cpu_count()}
+
+
 def measure_attention(ctx, hip_api, rng):
     """BASELINE.json configs[3]: GQA flash-decode, 32 q heads / 8 kv heads / head_dim 128, f32 KV
     resident in HBM in the kernel's head-major layout; bytes = K + V read once."""
@@ -330,6 +352,29 @@ def main() -> int:
     per_group = {g: {"GB/s": round(grp_bytes[g] / (grp_ms[g] / args.steps * 1e-3) / 1e9, 1),
                      "ms_per_step": round(grp_ms[g] / args.steps, 4)} for g, _ in groups}
 
+    # ---- the Q8_0 activation quantizer on its own (the reference re-quantizes per GEMV call,
+    # cpu.rs:787-790): kernel time per call, and the set's rate with one quantize per GEMV folded in
+    quant_us = {}
+    for kk in (4096, 14336):
+        dxf = ctx.to_device(acts[kk][2])
+        qcall = lambda: ctx.check(ctx.lib.cera_hip_quantize_q8_0_dev(ctx.h, dxf, kk, acts[kk][0], acts[kk][1]))
+        for _ in range(5):
+            qcall()
+        e0, e1 = ctx.event(), ctx.event()
+        ctx.record(e0)
+        for _ in range(200):
+            qcall()
+        ctx.record(e1)
+        ctx.sync()
+        quant_us[kk] = ctx.elapsed_ms(e0, e1) * 1e3 / 200
+        ctx.free(dxf)
+    quant_ms_per_step = (N_LAYERS * (4 * quant_us[4096] + quant_us[14336]) + quant_us[4096]) * 1e-3
+    quantize = {"k4096_us_per_call": round(quant_us[4096], 2), "k14336_us_per_call": round(quant_us[14336], 2),
+                "calls_per_step": N_LAYERS * 5 + 1,
+                "set_incl_quantize_GB/s": round(step_bytes / ((ms_per_step + quant_ms_per_step) * 1e-3) / 1e9, 1),
+                "note": "back-to-back launches of the standalone kernel; the decode path fuses three of the "
+                        "five per-layer quantizations into the producing kernels"}
+
     # ---- correctness spot check of what was just timed (oracle is only the checker)
     cpu_baseline = None
     if not args.no_cpu_baseline:
@@ -364,7 +409,7 @@ def main() -> int:
                         "sample": f"{done_layers} decode-layer GEMV sets (QKV, O, gate, up Q4_K; down Q6_K; "
                                   f"{layer_bytes} B each) in {cpu_s:.1f} s, restated cera AVX2 int8 path "
                                   f"incl. per-call Q8_0 quantize, {n_copies} rotating weight copies",
-                        "avx2": bool(orc.lib().orc_have_avx2())}
+                        "avx2": bool(orc.lib().orc_have_avx2()), **host_cpu_info()}
 
     extras = {}
     if not args.no_extras:
@@ -385,6 +430,7 @@ def main() -> int:
         "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2),
         "gemv_only_tok_s_equiv": round(1e3 / ms_per_step, 1),
         "per_group": per_group,
+        "quantize": quantize,
         "roofline": roofline,
         "cpu_baseline": cpu_baseline,
         "e2e": e2e,
