@@ -11,17 +11,18 @@
 // of one 32-element block for 32 weight rows x 32 tokens (Q6_K uses the
 // 32x32x16 form, one per 16-element scale run).  Every block carries its own
 // pair of scales (weight side x activation side), so the int32 tile is folded
-// into f32 accumulators after each block; that VALU work (convert, scale,
-// accumulate: three to four instructions per output per block against 32 matrix-core
-// cycles per 1024 outputs) is the throughput limit of this kernel, not the matrix
-// core.  Two things keep it down:
+// into f32 accumulators after each block: a convert and an FMA per output per block
+// on the VALU.  Everything else about the scales runs on the matrix core:
+//   * the per-output scale  rs[row][b] * xs[token][b]  is a rank-1 matrix per block;
+//     one v_mfma_f32_32x32x1_2b_f32 produces it for two blocks (Q6_K: for the two
+//     16-element groups of one block) from ONE scalar LDS read per lane per operand,
+//     already in the accumulator layout.  Reading the sixteen row scales a lane needs
+//     straight from LDS costs a full-width read for data every lane of a half shares,
+//     and that broadcast traffic, not the fragments, was what kept the LDS busy;
 //   * the min terms  dmin*mn[row][b] * (xs*sum a)[tok][b]  (Q4_K, Q4_1) are a small
-//     f32 contraction over blocks of their own; they run on the matrix core too
-//     (v_mfma_f32_32x32x2_f32, two blocks per instruction) instead of one FMA per
-//     output per block;
-//   * Q6_K's int8 group scales are applied in integer (dot16_a*sc_a + dot16_b*sc_b,
-//     24-bit multiplies) so a 32-block costs one convert and one FMA with the
-//     activation scale; the f16 super-block scale d is applied once per 256.
+//     f32 contraction over blocks of their own: v_mfma_f32_32x32x2_f32, two blocks
+//     per instruction, accumulated (negated) into the same f32 tile as the dots;
+//   * Q6_K's f16 super-block scale d is applied once per 256.
 //
 // Workgroup: 256 threads = 4 wavefronts as 2 (M) x 2 (N); block tile 128 rows x
 // 64 tokens; each wavefront owns 64 x 32 (two MFMA row tiles).  K advances in
@@ -46,6 +47,7 @@
 
 typedef int v16i __attribute__((ext_vector_type(16)));
 typedef float v16f __attribute__((ext_vector_type(16)));
+typedef float v32f __attribute__((ext_vector_type(32)));
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v2i __attribute__((ext_vector_type(2)));
 
@@ -73,6 +75,7 @@ struct GemmArgs {
 // scales() writes the row's per-sub-block scales.  NSUB = MFMA steps per tile,
 // KSTEP = elements per MFMA.
 struct GemmQ4K {
+    static constexpr int WAVES_PER_SIMD = 3;   // register budget the kernel is compiled for
     static constexpr int NSUB = 4, KSTEP = 32;
     static constexpr bool HAS_MIN = true, INT_SCALE = false;
     static constexpr int BLOCK_BYTES = 144;
@@ -114,6 +117,7 @@ struct GemmQ4K {
 };
 
 struct GemmQ6K {
+    static constexpr int WAVES_PER_SIMD = 2;   // register budget the kernel is compiled for
     static constexpr int NSUB = 8, KSTEP = 16;
     static constexpr bool HAS_MIN = false, INT_SCALE = true;
     static constexpr int BLOCK_BYTES = 210;
@@ -164,6 +168,7 @@ struct GemmQ6K {
 
 // 32-element block formats: a tile is 4 blocks; word w = block index within the tile.
 struct GemmQ4_0 {
+    static constexpr int WAVES_PER_SIMD = 3;   // register budget the kernel is compiled for
     static constexpr int NSUB = 4, KSTEP = 32;
     static constexpr bool HAS_MIN = false, INT_SCALE = false;
     static constexpr int BLOCK_BYTES = 18 * 8;  // bytes per 256 elements
@@ -198,6 +203,7 @@ struct GemmQ4_0 {
     }
 };
 struct GemmQ4_1 {
+    static constexpr int WAVES_PER_SIMD = 3;   // register budget the kernel is compiled for
     static constexpr int NSUB = 4, KSTEP = 32;
     static constexpr bool HAS_MIN = true, INT_SCALE = false;   // rm holds -m so that out = rs*dot - rm*sum(a) covers q*d + m
     static constexpr int BLOCK_BYTES = 20 * 8;
@@ -229,6 +235,7 @@ struct GemmQ4_1 {
     }
 };
 struct GemmQ8_0 {
+    static constexpr int WAVES_PER_SIMD = 2;   // register budget the kernel is compiled for
     static constexpr int NSUB = 4, KSTEP = 32;
     static constexpr bool HAS_MIN = false, INT_SCALE = false;
     static constexpr int BLOCK_BYTES = 34 * 8;
@@ -256,7 +263,7 @@ struct GemmQ8_0 {
 };
 
 template <class T>
-static __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
+static __global__ __launch_bounds__(256, T::WAVES_PER_SIMD) void gemm_kernel(GemmArgs p) {
     constexpr int NB = GEMM_KT / 32;  // 32-blocks per tile
     __shared__ __attribute__((aligned(16))) int8_t sA[GEMM_BM * GEMM_LDA];
     __shared__ __attribute__((aligned(16))) int8_t sB[GEMM_BN * GEMM_LDA];
@@ -272,12 +279,13 @@ static __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
     const uint32_t col = lane & 31, half = lane >> 5;
     const uint32_t nb32 = p.k / 32;
 
-    float acc[2][16], accsb[2][16];
-    v16f macc[2];
+    // acc takes the scaled block dots (VALU) and, negated, the min terms (matrix core)
+    v16f acc[2];
+    float accsb[2][16];
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) { acc[t][r] = 0.0f; accsb[t][r] = 0.0f; macc[t][r] = 0.0f; }
+        for (int r = 0; r < 16; ++r) { acc[t][r] = 0.0f; accsb[t][r] = 0.0f; }
 
     // per-thread staging assignments, fixed for the whole K loop: AI weight words, one row's
     // scales (threads 0..127), two activation words, one activation scale
@@ -341,34 +349,63 @@ static __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
 
         // ---- MFMA over the K tile
         const int8_t* bRow = sB + (wn * 32 + col) * GEMM_LDA;
+        if (!T::INT_SCALE) {
+            // Blocks in pairs.  The per-output scale  rs[row][b] * xs[token][b]  of both blocks of a
+            // pair is one two-block outer product on the matrix core (each lane supplies the scale
+            // of row `col` and of token `col` for the block of its half): one scalar LDS read per
+            // lane per operand instead of the same sixteen row scales re-read by every lane of a
+            // half, which made the LDS the limit of this kernel, and no multiply on the VALU.
 #pragma unroll
-        for (int b = 0; b < NB; ++b) {
-            const float xs = sCS[b * GEMM_BN + wn * 32 + col];
-            if (!T::INT_SCALE) {
-                const v4i bf = *reinterpret_cast<const v4i*>(bRow + b * 32 + half * 16);
+            for (int pr = 0; pr < NB / 2; ++pr) {
+                v4i bf[2];
+#pragma unroll
+                for (int jb = 0; jb < 2; ++jb) bf[jb] = *reinterpret_cast<const v4i*>(bRow + (2 * pr + jb) * 32 + half * 16);
+                const float xsl = sCS[(2 * pr + half) * GEMM_BN + wn * 32 + col];
 #pragma unroll
                 for (int t = 0; t < 2; ++t) {
+                    const float rsl = sRS[(2 * pr + half) * GEMM_BM + wm * 64 + t * 32 + col];
+                    v32f z32;
+#pragma unroll
+                    for (int e = 0; e < 32; ++e) z32[e] = 0.0f;
+                    const v32f sc = __builtin_amdgcn_mfma_f32_32x32x1f32(rsl, xsl, z32, 0, 0, 0);
                     const int8_t* aRow = sA + (wm * 64 + t * 32 + col) * GEMM_LDA;
-                    const v4i af = *reinterpret_cast<const v4i*>(aRow + b * 32 + half * 16);
-                    v16i c = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-                    c = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, bf, c, 0, 0, 0);
-                    // rows held by this lane: 8*blk + 4*half + r, blk = 0..3, r = 0..3
 #pragma unroll
-                    for (int blk = 0; blk < 4; ++blk) {
-                        const uint32_t rbase = wm * 64 + t * 32 + blk * 8 + half * 4;
-                        const float4 rs = *reinterpret_cast<const float4*>(sRS + b * GEMM_BM + rbase);
-                        const float rsv[4] = {rs.x, rs.y, rs.z, rs.w};
+                    for (int jb = 0; jb < 2; ++jb) {
+                        const v4i af = *reinterpret_cast<const v4i*>(aRow + (2 * pr + jb) * 32 + half * 16);
+                        v16i c = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+                        c = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, bf[jb], c, 0, 0, 0);
+                        // rows held by this lane: 8*blk + 4*half + r, blk = 0..3, r = 0..3
 #pragma unroll
-                        for (int r = 0; r < 4; ++r)
-                            acc[t][blk * 4 + r] = fmaf(static_cast<float>(c[blk * 4 + r]), rsv[r] * xs, acc[t][blk * 4 + r]);
+                        for (int e = 0; e < 16; ++e) acc[t][e] = fmaf(static_cast<float>(c[e]), sc[16 * jb + e], acc[t][e]);
                     }
                 }
-            } else {
-                // two 16-element scale groups share this block's activation scale
+                if (T::HAS_MIN) {
+                    // min terms of the pair's blocks: a rank-2 f32 update on the matrix core
+                    const float xm = sCM[(2 * pr + half) * GEMM_BN + wn * 32 + col];
+#pragma unroll
+                    for (int t = 0; t < 2; ++t) {
+                        const float rm = -sRM[(2 * pr + half) * GEMM_BM + wm * 64 + t * 32 + col];
+                        acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(rm, xm, acc[t], 0, 0, 0);
+                    }
+                }
+            }
+        } else {
+#pragma unroll
+            for (int b = 0; b < NB; ++b) {
+                // two 16-element scale groups share this block's activation scale.  Their per-output
+                // scales  sc[row][group] * xs[token]  (an 8-bit integer times an f16 value: exact in
+                // f32) are the two blocks of one outer-product MFMA, as above.
+                const float xs = sCS[b * GEMM_BN + wn * 32 + col];
                 const long bf0 = *reinterpret_cast<const long*>(bRow + b * 32 + half * 8);
                 const long bf1 = *reinterpret_cast<const long*>(bRow + b * 32 + 16 + half * 8);
 #pragma unroll
                 for (int t = 0; t < 2; ++t) {
+                    const float rsl = static_cast<float>(
+                        __builtin_bit_cast(int, sRS[(2 * b + half) * GEMM_BM + wm * 64 + t * 32 + col]));
+                    v32f z32;
+#pragma unroll
+                    for (int e = 0; e < 32; ++e) z32[e] = 0.0f;
+                    const v32f sc = __builtin_amdgcn_mfma_f32_32x32x1f32(rsl, xs, z32, 0, 0, 0);
                     const int8_t* aRow = sA + (wm * 64 + t * 32 + col) * GEMM_LDA;
                     const long af0 = *reinterpret_cast<const long*>(aRow + b * 32 + half * 8);
                     const long af1 = *reinterpret_cast<const long*>(aRow + b * 32 + 16 + half * 8);
@@ -376,26 +413,10 @@ static __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
                     v16i c0 = __builtin_amdgcn_mfma_i32_32x32x16_i8(af0, bf0, z, 0, 0, 0);
                     v16i c1 = __builtin_amdgcn_mfma_i32_32x32x16_i8(af1, bf1, z, 0, 0, 0);
 #pragma unroll
-                    for (int blk = 0; blk < 4; ++blk) {
-                        const uint32_t rbase = wm * 64 + t * 32 + blk * 8 + half * 4;
-                        const v4i s0 = *reinterpret_cast<const v4i*>(sRS + (2 * b) * GEMM_BM + rbase);
-                        const v4i s1 = *reinterpret_cast<const v4i*>(sRS + (2 * b + 1) * GEMM_BM + rbase);
-#pragma unroll
-                        for (int r = 0; r < 4; ++r) {
-                            // |dot16| <= 16*32*127 and |scale| <= 128: 24-bit operands, 32-bit result
-                            const int iv = __mul24(c0[blk * 4 + r], s0[r]) + __mul24(c1[blk * 4 + r], s1[r]);
-                            accsb[t][blk * 4 + r] = fmaf(static_cast<float>(iv), xs, accsb[t][blk * 4 + r]);
-                        }
+                    for (int e = 0; e < 16; ++e) {
+                        accsb[t][e] = fmaf(static_cast<float>(c0[e]), sc[e], accsb[t][e]);
+                        accsb[t][e] = fmaf(static_cast<float>(c1[e]), sc[16 + e], accsb[t][e]);
                     }
-                }
-            }
-            if (T::HAS_MIN && (b & 1)) {
-                // min terms of blocks b-1, b: a rank-2 f32 update on the matrix core
-                const float xm = sCM[(b - 1 + half) * GEMM_BN + wn * 32 + col];
-#pragma unroll
-                for (int t = 0; t < 2; ++t) {
-                    const float rm = sRM[(b - 1 + half) * GEMM_BM + wm * 64 + t * 32 + col];
-                    macc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(rm, xm, macc[t], 0, 0, 0);
                 }
             }
         }
@@ -427,7 +448,7 @@ static __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
                 for (int r = 0; r < 4; ++r) {
                     uint32_t row = m0 + wm * 64 + t * 32 + blk * 8 + half * 4 + r;
                     if (row < p.m) {
-                        float v = acc[t][blk * 4 + r] - (T::HAS_MIN ? macc[t][blk * 4 + r] : 0.0f);
+                        float v = acc[t][blk * 4 + r];
                         uint64_t idx = row * p.ld_m + tok * p.ld_n;
                         if (p.resid) v = p.resid[idx] + (p.resid_scale != 1.0f ? v * p.resid_scale : v);
                         p.out[idx + blockIdx.z * p.part_stride] = v;
