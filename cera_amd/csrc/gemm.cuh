@@ -22,7 +22,8 @@
 //   * the min terms  dmin*mn[row][b] * (xs*sum a)[tok][b]  (Q4_K, Q4_1) are a small
 //     f32 contraction over blocks of their own: v_mfma_f32_32x32x2_f32, two blocks
 //     per instruction, accumulated (negated) into the same f32 tile as the dots;
-//   * Q6_K's f16 super-block scale d is applied once per 256.
+//   * Q6_K's f16 super-block scale d rides on the row operand of the outer product
+//     (sc * d is exact), so there is no per-super-block stage.
 //
 // Workgroup: 256 threads = 4 wavefronts as 2 (M) x 2 (N); block tile 128 rows x
 // 64 tokens; each wavefront owns 64 x 32 (two MFMA row tiles).  K advances in
@@ -281,11 +282,10 @@ static __global__ __launch_bounds__(256, T::WAVES_PER_SIMD) void gemm_kernel(Gem
 
     // acc takes the scaled block dots (VALU) and, negated, the min terms (matrix core)
     v16f acc[2];
-    float accsb[2][16];
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) { acc[t][r] = 0.0f; accsb[t][r] = 0.0f; }
+        for (int r = 0; r < 16; ++r) acc[t][r] = 0.0f;
 
     // per-thread staging assignments, fixed for the whole K loop: AI weight words, one row's
     // scales (threads 0..127), two activation words, one activation scale
@@ -400,8 +400,11 @@ static __global__ __launch_bounds__(256, T::WAVES_PER_SIMD) void gemm_kernel(Gem
                 const long bf1 = *reinterpret_cast<const long*>(bRow + b * 32 + 16 + half * 8);
 #pragma unroll
                 for (int t = 0; t < 2; ++t) {
-                    const float rsl = static_cast<float>(
-                        __builtin_bit_cast(int, sRS[(2 * b + half) * GEMM_BM + wm * 64 + t * 32 + col]));
+                    // (sc * d) is exact (8 x 11 bits); times xs it rounds once, as the reference's
+                    // own  ([sc0, sc1] * d) * xs  does
+                    const float rsl = static_cast<float>(__builtin_bit_cast(
+                                          int, sRS[(2 * b + half) * GEMM_BM + wm * 64 + t * 32 + col])) *
+                                      sRD[wm * 64 + t * 32 + col];
                     v32f z32;
 #pragma unroll
                     for (int e = 0; e < 32; ++e) z32[e] = 0.0f;
@@ -414,26 +417,11 @@ static __global__ __launch_bounds__(256, T::WAVES_PER_SIMD) void gemm_kernel(Gem
                     v16i c1 = __builtin_amdgcn_mfma_i32_32x32x16_i8(af1, bf1, z, 0, 0, 0);
 #pragma unroll
                     for (int e = 0; e < 16; ++e) {
-                        accsb[t][e] = fmaf(static_cast<float>(c0[e]), sc[e], accsb[t][e]);
-                        accsb[t][e] = fmaf(static_cast<float>(c1[e]), sc[16 + e], accsb[t][e]);
+                        acc[t][e] = fmaf(static_cast<float>(c0[e]), sc[e], acc[t][e]);
+                        acc[t][e] = fmaf(static_cast<float>(c1[e]), sc[16 + e], acc[t][e]);
                     }
                 }
             }
-        }
-        if (T::INT_SCALE && hs == 1) {
-            // the super-block's f16 scale, once per 256 elements
-#pragma unroll
-            for (int t = 0; t < 2; ++t)
-#pragma unroll
-                for (int blk = 0; blk < 4; ++blk) {
-                    const float4 d = *reinterpret_cast<const float4*>(sRD + wm * 64 + t * 32 + blk * 8 + half * 4);
-                    const float dv[4] = {d.x, d.y, d.z, d.w};
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        acc[t][blk * 4 + r] = fmaf(dv[r], accsb[t][blk * 4 + r], acc[t][blk * 4 + r]);
-                        accsb[t][blk * 4 + r] = 0.0f;
-                    }
-                }
         }
         __syncthreads();
     }
