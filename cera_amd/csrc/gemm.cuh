@@ -67,6 +67,12 @@ struct GemmArgs {
     // sums to out + z*part_stride (k_chunk == k, part_stride == 0 when not split)
     uint32_t k_chunk;
     uint64_t part_stride;
+    // optional second matrix of the same type and k sharing the launch (and the activations):
+    // row tiles [tiles1, gridDim.y) belong to it.  No residual, no split-K for a pair.
+    const uint8_t* w2;
+    float* out2;
+    uint32_t m2, tiles1;
+    uint64_t ld_n2;
 };
 
 // ---- per-type staging of one 128-element K tile of one row -------------------
@@ -276,7 +282,12 @@ static __global__ __launch_bounds__(256, T::WAVES_PER_SIMD) void gemm_kernel(Gem
 
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const uint32_t wm = wave >> 1, wn = wave & 1;           // wavefront position in the 2 x 2 grid
-    const uint32_t m0 = blockIdx.y * GEMM_BM, n0 = blockIdx.x * GEMM_BN;
+    const bool second = p.w2 != nullptr && blockIdx.y >= p.tiles1;
+    const uint8_t* const wmat = second ? p.w2 : p.w;
+    float* const omat = second ? p.out2 : p.out;
+    const uint32_t mrows = second ? p.m2 : p.m;
+    const uint64_t ldn = second ? p.ld_n2 : p.ld_n;
+    const uint32_t m0 = (second ? blockIdx.y - p.tiles1 : blockIdx.y) * GEMM_BM, n0 = blockIdx.x * GEMM_BN;
     const uint32_t col = lane & 31, half = lane >> 5;
     const uint32_t nb32 = p.k / 32;
 
@@ -297,10 +308,10 @@ static __global__ __launch_bounds__(256, T::WAVES_PER_SIMD) void gemm_kernel(Gem
     for (int i = 0; i < AI; ++i) {
         const uint32_t it = tid + 256 * i, r = it / T::WORDS;
         a_w[i] = it % T::WORDS;
-        a_src[i] = p.w + static_cast<uint64_t>(min(m0 + r, p.m - 1)) * p.row_bytes;
+        a_src[i] = wmat + static_cast<uint64_t>(min(m0 + r, mrows - 1)) * p.row_bytes;
         a_dst[i] = sA + r * GEMM_LDA;
     }
-    const uint8_t* s_src = p.w + static_cast<uint64_t>(min(m0 + (tid & (GEMM_BM - 1)), p.m - 1)) * p.row_bytes;
+    const uint8_t* s_src = wmat + static_cast<uint64_t>(min(m0 + (tid & (GEMM_BM - 1)), mrows - 1)) * p.row_bytes;
     const int8_t* b_src[2];
     int8_t* b_dst[2];
     bool b_live[2];
@@ -435,11 +446,11 @@ static __global__ __launch_bounds__(256, T::WAVES_PER_SIMD) void gemm_kernel(Gem
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     uint32_t row = m0 + wm * 64 + t * 32 + blk * 8 + half * 4 + r;
-                    if (row < p.m) {
+                    if (row < mrows) {
                         float v = acc[t][blk * 4 + r];
-                        uint64_t idx = row * p.ld_m + tok * p.ld_n;
+                        uint64_t idx = row * p.ld_m + tok * ldn;
                         if (p.resid) v = p.resid[idx] + (p.resid_scale != 1.0f ? v * p.resid_scale : v);
-                        p.out[idx + blockIdx.z * p.part_stride] = v;
+                        omat[idx + blockIdx.z * p.part_stride] = v;
                     }
                 }
     }

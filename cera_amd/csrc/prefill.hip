@@ -18,9 +18,13 @@ static bool gemm_type_ok(uint32_t t) {
 bool cera_gemm_supports(uint32_t dtype, uint64_t k) { return gemm_type_ok(dtype) && k % GEMM_KSUPER == 0 && k > 0; }
 
 // out[i*ld_m + j*ld_n] = (W . B)[i][j] (+ resid)
+// w2 / out2 (nullable): a second matrix of the same type and k multiplied by the same activations
+// in the same launch, out2[i*ld_m + j*ld_n2]; *paired says whether that happened (if not, the
+// caller launches the second matrix on its own)
 cera_hip_status cera_launch_gemm(cera_hip_ctx* ctx, const cera_hip_dtensor* w, const float* bs, const int8_t* bq,
                                  const float* bsum, uint32_t n, float* out, uint64_t ld_m, uint64_t ld_n,
-                                 const float* resid, float resid_scale) {
+                                 const float* resid, float resid_scale, const cera_hip_dtensor* w2 = nullptr,
+                                 float* out2 = nullptr, uint64_t ld_n2 = 0, bool* paired = nullptr) {
     if (!cera_gemm_supports(w->dtype, w->k))
         return cera_fail(ctx, CERA_HIP_ERR_UNSUPPORTED_DTYPE,
                          "gemm: no int8 GEMM for ggml type " + std::to_string(w->dtype) + " with k=" + std::to_string(w->k));
@@ -31,6 +35,15 @@ cera_hip_status cera_launch_gemm(cera_hip_ctx* ctx, const cera_hip_dtensor* w, c
     a.row_bytes = static_cast<uint32_t>(w->row_bytes);
     a.ld_m = ld_m; a.ld_n = ld_n; a.resid = resid; a.resid_scale = resid_scale;
     dim3 grid((n + GEMM_BN - 1) / GEMM_BN, (a.m + GEMM_BM - 1) / GEMM_BM);
+    a.w2 = nullptr; a.out2 = nullptr; a.m2 = 0; a.tiles1 = grid.y; a.ld_n2 = 0;
+    if (paired) *paired = false;
+    // a pair is taken when both outputs are token-major and dense (what the split-K reduction needs)
+    if (w2 && !resid && w2->dtype == w->dtype && w2->k == w->k && w2->row_bytes == w->row_bytes && ld_m == 1 &&
+        ld_n == w->m && ld_n2 == w2->m && (w->m * n) % 4 == 0 && (w2->m * n) % 4 == 0) {
+        a.w2 = w2->dev; a.out2 = out2; a.m2 = static_cast<uint32_t>(w2->m); a.ld_n2 = ld_n2;
+        grid.y += static_cast<uint32_t>((w2->m + GEMM_BM - 1) / GEMM_BM);
+        if (paired) *paired = true;
+    }
     // Few output tiles and a long K (the down projection at a few hundred tokens): split K over
     // grid.z so the chip is filled, partial sums to scratch, then one fixed-order reduction.
     // The outputs must be dense in m*n floats for the elementwise reduction.
@@ -45,12 +58,14 @@ cera_hip_status cera_launch_gemm(cera_hip_ctx* ctx, const cera_hip_dtensor* w, c
     }
     a.k_chunk = a.k / split;
     a.part_stride = 0;
-    const uint64_t mn = static_cast<uint64_t>(a.m) * n;
+    // a pair's partials lie side by side: [split][m*n | m2*n]
+    const uint64_t mn = static_cast<uint64_t>(a.m) * n, mn2 = static_cast<uint64_t>(a.m2) * n;
     if (split > 1) {
         void* part;
-        CERA_TRY(cera_scratch(ctx, 9, split * mn * sizeof(float), &part));
+        CERA_TRY(cera_scratch(ctx, 9, split * (mn + mn2) * sizeof(float), &part));
         a.out = static_cast<float*>(part);
-        a.part_stride = mn;
+        if (a.w2) a.out2 = a.out + mn;
+        a.part_stride = mn + mn2;
         a.resid = nullptr;
         grid.z = split;
     }
@@ -61,9 +76,14 @@ cera_hip_status cera_launch_gemm(cera_hip_ctx* ctx, const cera_hip_dtensor* w, c
         case CERA_HIP_Q4_1: hipLaunchKernelGGL((gemm_kernel<GemmQ4_1>), grid, dim3(256), 0, ctx->stream, a); break;
         default: hipLaunchKernelGGL((gemm_kernel<GemmQ8_0>), grid, dim3(256), 0, ctx->stream, a); break;
     }
-    if (split > 1)
+    if (split > 1) {
         hipLaunchKernelGGL(gemm_reduce_kernel, dim3(static_cast<uint32_t>((mn / 4 + 255) / 256)), dim3(256), 0, ctx->stream,
-                           a.out, split, mn, mn / 4, out, resid, resid_scale);
+                           a.out, split, a.part_stride, mn / 4, out, resid, resid_scale);
+        if (a.w2)
+            hipLaunchKernelGGL(gemm_reduce_kernel, dim3(static_cast<uint32_t>((mn2 / 4 + 255) / 256)), dim3(256), 0,
+                               ctx->stream, a.out2, split, a.part_stride, mn2 / 4, out2, static_cast<const float*>(nullptr),
+                               1.0f);
+    }
     HIP_TRY(ctx, hipGetLastError());
     return CERA_HIP_OK;
 }
@@ -192,11 +212,25 @@ static cera_hip_status prefill_chunk(cera_hip_model* m, const uint32_t* tokens, 
         return cera_launch_gemm(ctx, w, m->pf_xs, m->pf_xq, m->pf_bsum, n, out, 1, w->m, resid, c.residual_scale);
     };
 
+    // two projections of the same activations: one launch when both have an int8 GEMM of the same
+    // type (the tail of one matrix's workgroups then overlaps the other's, and a short K-split
+    // matrix like K shares Q's launch), else one after the other
+    auto gemm2 = [&](const cera_hip_dtensor* wa, float* outa, const cera_hip_dtensor* wb, float* outb) -> cera_hip_status {
+        if (n > PREFILL_SMALL_BATCH && cera_gemm_supports(wa->dtype, wa->k) && cera_gemm_supports(wb->dtype, wb->k)) {
+            bool paired = false;
+            CERA_TRY(cera_launch_gemm(ctx, wa, m->pf_xs, m->pf_xq, m->pf_bsum, n, outa, 1, wa->m, nullptr, 1.0f, wb, outb,
+                                      wb->m, &paired));
+            if (paired) return CERA_HIP_OK;
+            return cera_launch_gemm(ctx, wb, m->pf_xs, m->pf_xq, m->pf_bsum, n, outb, 1, wb->m, nullptr, 1.0f);
+        }
+        CERA_TRY(gemm(wa, outa, nullptr));
+        return gemm(wb, outb, nullptr);
+    };
+
     for (uint32_t i = 0; i < c.n_layers; ++i) {
         LayerDev& L = m->layers[i];
         CERA_TRY(norm_rows(m->pf_hidden, L.attn_norm, m->pf_normed));
-        CERA_TRY(gemm(L.q, m->pf_q, nullptr));
-        CERA_TRY(gemm(L.k, m->pf_k, nullptr));
+        CERA_TRY(gemm2(L.q, m->pf_q, L.k, m->pf_k));
         CERA_TRY(gemm(L.v, m->pf_v, nullptr));
         if (L.q_bias) {
             // bias rows: one launch per token keeps the kernel trivial; models with biases are rare here
@@ -227,8 +261,7 @@ static cera_hip_status prefill_chunk(cera_hip_model* m, const uint32_t* tokens, 
         CERA_TRY(gemm(L.o, m->pf_hidden, m->pf_hidden));
 
         CERA_TRY(norm_rows(m->pf_hidden, L.ffn_norm, m->pf_normed));
-        CERA_TRY(gemm(L.gate, m->pf_gate, nullptr));
-        CERA_TRY(gemm(L.up, m->pf_up, nullptr));
+        CERA_TRY(gemm2(L.gate, m->pf_gate, L.up, m->pf_up));
         const uint64_t tot = static_cast<uint64_t>(n) * c.ffn;
         hipLaunchKernelGGL((silu_mul_kernel<true>), dim3(static_cast<uint32_t>((tot / 4 + 255) / 256)), dim3(256), 0, s,
                            m->pf_gate, m->pf_up, tot, m->pf_gate, m->pf_xs, m->pf_xq, m->pf_bsum);
