@@ -130,6 +130,45 @@ extern "C" cera_hip_status cera_hip_gemm(cera_hip_ctx* ctx, const cera_hip_tenso
     return st;
 }
 
+extern "C" cera_hip_status cera_hip_gemm_pair(cera_hip_ctx* ctx, const cera_hip_tensor* ta, const cera_hip_tensor* tb,
+                                              const float* x, uint64_t n, float* out_a, float* out_b) {
+    if (!ctx || !ta || !tb || !x || !out_a || !out_b) return CERA_HIP_ERR_ARGUMENT;
+    if (n == 0 || n > 0x7FFFFFFFull) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "gemm_pair: bad n");
+    cera_hip_dtensor *wa = nullptr, *wb = nullptr;
+    CERA_TRY(cera_hip_tensor_upload(ctx, ta, &wa));
+    cera_hip_status st = cera_hip_tensor_upload(ctx, tb, &wb);
+    if (st != CERA_HIP_OK) { cera_hip_tensor_free(ctx, wa); return st; }
+    auto run = [&]() -> cera_hip_status {
+        if (!cera_gemm_supports(wa->dtype, wa->k) || wa->dtype != wb->dtype || wa->k != wb->k)
+            return cera_fail(ctx, CERA_HIP_ERR_UNSUPPORTED_DTYPE,
+                             "gemm_pair: the matrices must share a type with an int8 GEMM and k");
+        const uint64_t k = wa->k;
+        void *dx, *ds, *dq, *db, *dya, *dyb;
+        CERA_TRY(cera_scratch(ctx, 0, n * k * 4, &dx));
+        CERA_TRY(cera_scratch(ctx, 1, n * (k / 32) * 4, &ds));
+        CERA_TRY(cera_scratch(ctx, 2, n * k, &dq));
+        CERA_TRY(cera_scratch(ctx, 7, n * (k / 32) * 4, &db));
+        CERA_TRY(cera_scratch(ctx, 3, n * wa->m * 4, &dya));
+        CERA_TRY(cera_scratch(ctx, 4, n * wb->m * 4, &dyb));
+        CERA_TRY(cera_hip_upload(ctx, dx, x, n * k * 4));
+        CERA_TRY(quantize_rows(ctx, static_cast<float*>(dx), n, k, static_cast<float*>(ds), static_cast<int8_t*>(dq),
+                               static_cast<float*>(db)));
+        bool paired = false;
+        CERA_TRY(cera_launch_gemm(ctx, wa, static_cast<float*>(ds), static_cast<int8_t*>(dq), static_cast<float*>(db),
+                                  static_cast<uint32_t>(n), static_cast<float*>(dya), 1, wa->m, nullptr, 1.0f, wb,
+                                  static_cast<float*>(dyb), wb->m, &paired));
+        if (!paired)   // rows x tokens not a multiple of 4: one after the other, as the forward pass does
+            CERA_TRY(cera_launch_gemm(ctx, wb, static_cast<float*>(ds), static_cast<int8_t*>(dq), static_cast<float*>(db),
+                                      static_cast<uint32_t>(n), static_cast<float*>(dyb), 1, wb->m, nullptr, 1.0f));
+        CERA_TRY(cera_hip_download(ctx, out_a, dya, n * wa->m * 4));
+        return cera_hip_download(ctx, out_b, dyb, n * wb->m * 4);
+    };
+    st = run();
+    cera_hip_tensor_free(ctx, wa);
+    cera_hip_tensor_free(ctx, wb);
+    return st;
+}
+
 // ---------------------------------------------------------------------------
 // Batched prefill of one chunk of n <= CHUNK tokens.
 // Largest batch one pass takes; longer prompts are cut into passes of this size.  A caller that

@@ -27,7 +27,7 @@ SYMBOLS = [
     "cera_hip_quantize_q8_0_dev", "cera_hip_gemv_q8_dev", "cera_hip_gemv_seq_dev", "cera_hip_attn_decode_dev",
     "cera_hip_gemm_dev",
     "cera_hip_model_create", "cera_hip_model_destroy", "cera_hip_forward", "cera_hip_forward_greedy",
-    "cera_hip_forward_prefill", "cera_hip_forward_prefill_logits_all", "cera_hip_truncate_kv", "cera_hip_gemv_pair", "cera_hip_gemv_nb", "cera_hip_configure_kv", "cera_hip_kv_type", "cera_hip_attn_f16kv",
+    "cera_hip_forward_prefill", "cera_hip_forward_prefill_logits_all", "cera_hip_truncate_kv", "cera_hip_gemv_pair", "cera_hip_gemm_pair", "cera_hip_gemv_nb", "cera_hip_configure_kv", "cera_hip_kv_type", "cera_hip_attn_f16kv",
     "cera_hip_attn_decode_f16_dev", "cera_hip_shift_kv", "cera_hip_write_kv", "cera_hip_set_seq_len", "cera_hip_seq_len", "cera_hip_memory_bytes",
     "cera_hip_read_kv", "cera_hip_read_hidden",
 ]
@@ -117,6 +117,7 @@ def load_library() -> C.CDLL:
         "cera_hip_forward_prefill_logits_all": (i32, [vp, vp, u32, u32, vp]),
         "cera_hip_truncate_kv": (i32, [vp, u32]),
         "cera_hip_gemv_pair": (i32, [vp, vp, vp, vp, vp, vp]),
+        "cera_hip_gemm_pair": (i32, [vp, vp, vp, vp, u64, vp, vp]),
         "cera_hip_gemv_nb": (i32, [vp, vp, vp, u32, vp]),
         "cera_hip_configure_kv": (i32, [vp, u32]),
         "cera_hip_kv_type": (u32, [vp]),
@@ -294,6 +295,14 @@ class Context:
         ya, yb = np.empty(ma, np.float32), np.empty(mb, np.float32)
         self.check(self.lib.cera_hip_gemv_pair(self.h, C.byref(ta), C.byref(tb), _p(x), _p(ya), _p(yb)))
         return ya, yb
+
+    def gemm_pair(self, type_a, wa, ma, type_b, wb, mb, x, n, k):
+        """Two matrices of one type against the same n activation rows in one launch; token-major outputs."""
+        ta, tb = make_tensor(type_a, ma, k, wa), make_tensor(type_b, mb, k, wb)
+        x = np.ascontiguousarray(x, np.float32).reshape(n, k)
+        oa, ob = np.empty((n, ma), np.float32), np.empty((n, mb), np.float32)
+        self.check(self.lib.cera_hip_gemm_pair(self.h, C.byref(ta), C.byref(tb), _p(x), n, _p(oa), _p(ob)))
+        return oa, ob
 
     def attn_f16kv(self, q, k, v, n_heads, n_kv_heads, head_dim, start_pos, n_queries, scale, n_splits=0) -> np.ndarray:
         """Attention over an f16 KV cache: k, v (f32) are narrowed to half before the upload."""

@@ -171,6 +171,16 @@ CERA_HIP_API cera_hip_status cera_hip_gemv_pair(cera_hip_ctx*, const cera_hip_te
 CERA_HIP_API cera_hip_status cera_hip_gemm(cera_hip_ctx*, const cera_hip_tensor* w, const float* x, uint64_t n,
                                            float* out);
 
+/* Two gemm_preq calls on the same quantized activations in one launch, the way the prefill pass
+ * issues attn_q | attn_k and ffn_gate | ffn_up (LlamaModel::forward_prefill_batched,
+ * cera/src/model/llama.rs:738-1523, multiplies them one after the other): one grid over both
+ * matrices' row tiles, split-K partials side by side when the tiles are few.  The matrices must
+ * share a type that has an int8 GEMM and k.  Outputs are token-major, out_a[n][m_a] and
+ * out_b[n][m_b] (the layout the batched forward pass keeps), each equal to cera_hip_gemm on its
+ * own matrix up to the order of the split-K partial sums. */
+CERA_HIP_API cera_hip_status cera_hip_gemm_pair(cera_hip_ctx*, const cera_hip_tensor* a, const cera_hip_tensor* b,
+                                                const float* x, uint64_t n, float* out_a, float* out_b);
+
 /* transformer::decode_attention (cera/src/model/transformer.rs:1249-1305) with
  * cpu::attn_scores / softmax_inplace / attn_values (cera/src/backend/cpu.rs:
  * 3222-3363, 2617-2633).  q f32[n_heads*head_dim]; k, v f32 time-major

@@ -82,6 +82,35 @@ def test_gemm_equals_gemv_per_column(hip, orc):
             assert np.abs(out[:, j] - y).max() <= 2e-5 * max(util.rms(y), 1e-6) * 10
 
 
+@pytest.mark.parametrize("dtype", [Q4_K, Q6_K, Q4_0])
+@pytest.mark.parametrize("ma,mb,n,k", [(256, 128, 40, 512), (4096, 1024, 512, 4096), (300, 77, 33, 2048),
+                                       (1024, 1024, 1100, 256)])
+def test_gemm_pair_matches_single_launches(hip, orc, dtype, ma, mb, n, k):
+    """Q|K and gate|up share a launch in the prefill pass: each output equals the matrix's own GEMM
+    (bit for bit where neither launch splits K; to the order of the partial sums where they do,
+    as at 4096 x 4096 | 1024 x 4096 with 512 tokens), and a row sample agrees with the oracle."""
+    _say(f"gemm pair {util.NAMES[dtype]} ma={ma} mb={mb} n={n} k={k}")
+    wa, _ = util.make_weights(dtype, ma, k, seed=31)
+    wb, _ = util.make_weights(dtype, mb, k, seed=32)
+    x = util.rng(n + k).standard_normal((n, k)).astype(np.float32)
+    oa, ob = hip.gemm_pair(dtype, wa, ma, dtype, wb, mb, x, n, k)
+    sa, sb = hip.gemm(dtype, wa, x, ma, n, k).T, hip.gemm(dtype, wb, x, mb, n, k).T
+    for got, single in ((oa, sa), (ob, sb)):
+        assert np.abs(got - single).max() <= 2e-5 * util.rms(single)
+    rows = np.unique(np.concatenate([np.arange(4), np.arange(mb - 4, mb)]))
+    rb = util.H.row_bytes(dtype, k)
+    wr = np.ascontiguousarray(wb.reshape(mb, rb)[rows]).reshape(-1)
+    ref = _oracle_gemm(orc, dtype, wr, x, rows.size, n, k)
+    assert np.abs(ob[:, rows].T.astype(np.float64) - ref).max() <= GEMM_TOL * util.rms(ref)
+
+
+def test_gemm_pair_refuses_mixed_types(hip):
+    with pytest.raises(hip_api.HipError) as e:
+        hip.gemm_pair(Q4_K, np.zeros(144 * 4, np.uint8), 4, Q6_K, np.zeros(210 * 4, np.uint8), 4,
+                      np.zeros((4, 256), np.float32), 4, 256)
+    assert e.value.status == 3
+
+
 def test_gemm_refuses_unsupported(hip):
     with pytest.raises(hip_api.HipError) as e:
         hip.gemm(Q5_K, np.zeros(176, np.uint8), np.zeros((1, 256), np.float32), 1, 1, 256)
