@@ -1,40 +1,38 @@
 // Prefill GEMM: out[m][n] = W[m, k] . B[k, n] with W in native GGUF blocks and
-// B the Q8_0-quantized activations of n tokens, on the int8 matrix cores.
+// B the Q8_0-quantized activations of n tokens, on the int8 matrix cores
+// (Q4_K, Q4_0, Q4_1, Q8_0; Q6_K has a kernel of its own in gemm_q6k_f16.cuh).
 //
 // Arithmetic contract (cera's batched int8 path, cera/src/backend/simd.rs:
-// 5693-5878 Q4_K, :5988-6195 Q6_K, :5893-5976 Q4_1, :4718-5010 Q4_0/Q8_0;
+// 5693-5878 Q4_K, :5893-5976 Q4_1, :4718-5010 Q4_0/Q8_0;
 // cera/src/model/transformer.rs:710-788, 865-946): exact int32 dots of weight
-// codes with int8 activations per 32-element block (16 for Q6_K), then an f32
+// codes with int8 activations per 32-element block, then an f32
 // epilogue  sum_b xs[j][b] * (d*sc * dot - dmin*mn * sum a).
 //
 // Mapping to gfx950: one v_mfma_i32_32x32x32_i8 computes the 32x32 int32 dots
-// of one 32-element block for 32 weight rows x 32 tokens (Q6_K uses the
-// 32x32x16 form, one per 16-element scale run).  Every block carries its own
+// of one 32-element block for 32 weight rows x 32 tokens.  Every block carries its own
 // pair of scales (weight side x activation side), so the int32 tile is folded
 // into f32 accumulators after each block: a convert and an FMA per output per block
 // on the VALU.  Everything else about the scales runs on the matrix core:
 //   * the per-output scale  rs[row][b] * xs[token][b]  is a rank-1 matrix per block;
-//     one v_mfma_f32_32x32x1_2b_f32 produces it for two blocks (Q6_K: for the two
-//     16-element groups of one block) from ONE scalar LDS read per lane per operand,
-//     already in the accumulator layout.  Reading the sixteen row scales a lane needs
-//     straight from LDS costs a full-width read for data every lane of a half shares,
-//     and that broadcast traffic, not the fragments, was what kept the LDS busy;
+//     one v_mfma_f32_32x32x1_2b_f32 produces it for two blocks from ONE scalar LDS
+//     read per lane per operand, already in the accumulator layout.  Reading the
+//     sixteen row scales a lane needs straight from LDS costs a full-width read for
+//     data every lane of a half shares, and that broadcast traffic, not the fragments,
+//     was what kept the LDS busy;
 //   * the min terms  dmin*mn[row][b] * (xs*sum a)[tok][b]  (Q4_K, Q4_1) are a small
 //     f32 contraction over blocks of their own: v_mfma_f32_32x32x2_f32, two blocks
-//     per instruction, accumulated (negated) into the same f32 tile as the dots;
-//   * Q6_K's f16 super-block scale d rides on the row operand of the outer product
-//     (sc * d is exact), so there is no per-super-block stage.
+//     per instruction, accumulated (negated) into the same f32 tile as the dots.
 //
 // Workgroup: 256 threads = 4 wavefronts as 2 (M) x 2 (N); block tile 128 rows x
 // 64 tokens; each wavefront owns 64 x 32 (two MFMA row tiles).  K advances in
 // steps of 128 elements (half a K-quant super-block): the LDS footprint stays
 // near 32 KB, so several workgroups share a CU and one's global loads and
 // unpacking overlap another's MFMA/VALU phase.  Per step the workgroup stages
-//   A: 128 rows x 128 weight codes unpacked to int8 (Q6_K/Q4_0 re-centred to
+//   A: 128 rows x 128 weight codes unpacked to int8 (Q4_0 re-centred to
 //      signed so no activation-sum correction is needed), row stride 144 B so
 //      16-byte fragment reads of 16 consecutive rows fall in distinct banks;
-//   rs/rm: per-row scale (d*sc, or the int8 scale for Q6_K) and min (dmin*mn) per
-//      sub-block, stored [sub][row] so a lane fetches four consecutive rows with one b128;
+//   rs/rm: per-row scale (d*sc) and min (dmin*mn) per
+//      sub-block, stored [sub][row];
 //   B: 64 tokens x 128 int8 activations, cs/cm: activation scale and
 //      scale*sum(a) per 32-block.
 #pragma once
@@ -57,6 +55,7 @@ struct GemmArgs {
     const int8_t* bq;   // [n][k] int8 activations
     const float* bs;    // [n][k/32] activation scales
     const float* bsum;  // [n][k/32] scale * sum(a) per block (exact product)
+    const void* bh;     // [n][k] the quants as f16, K in 0,2,1,3 order within fours (Q6_K kernel only)
     float* out;
     uint32_t m, n, k;
     uint32_t row_bytes;
@@ -84,7 +83,7 @@ struct GemmArgs {
 struct GemmQ4K {
     static constexpr int WAVES_PER_SIMD = 3;   // register budget the kernel is compiled for
     static constexpr int NSUB = 4, KSTEP = 32;
-    static constexpr bool HAS_MIN = true, INT_SCALE = false;
+    static constexpr bool HAS_MIN = true;
     static constexpr int BLOCK_BYTES = 144;
     static constexpr int WORDS = 4;
     struct Raw { uint4 q; };
@@ -101,7 +100,7 @@ struct GemmQ4K {
         *reinterpret_cast<uint4*>(dst + 64 * g + 16 * h) = lo;
         *reinterpret_cast<uint4*>(dst + 64 * g + 32 + 16 * h) = hi;
     }
-    __device__ static void scales(const RawS& raw, uint32_t hs, float* rs, float* rm, float* rd, uint32_t ld) {
+    __device__ static void scales(const RawS& raw, uint32_t hs, float* rs, float* rm, uint32_t ld) {
         const uint4 h = raw.h;
         float d = h2f(h.x & 0xFFFF), dmin = h2f(h.x >> 16);
         const uint32_t s[3] = {h.y, h.z, h.w};
@@ -119,57 +118,6 @@ struct GemmQ4K {
             rs[jj * ld] = d * static_cast<float>(sc);
             rm[jj * ld] = dmin * static_cast<float>(mn);
         }
-        (void)rd;
-    }
-};
-
-struct GemmQ6K {
-    static constexpr int WAVES_PER_SIMD = 2;   // register budget the kernel is compiled for
-    static constexpr int NSUB = 8, KSTEP = 16;
-    static constexpr bool HAS_MIN = false, INT_SCALE = true;
-    static constexpr int BLOCK_BYTES = 210;
-    static constexpr int WORDS = 2;  // j: 16 positions l0..l0+15 of the half -> 64 codes
-    struct Raw { uint4 qa, qb, qh; };
-    struct RawS { uint2 sc; uint32_t d; };
-    __device__ static void load(Raw& r, const uint8_t* blk, uint32_t nh, uint32_t j) {
-        r.qa = ld_u128_a2(blk + nh * 64 + j * 16);
-        r.qb = ld_u128_a2(blk + nh * 64 + 32 + j * 16);
-        r.qh = ld_u128_a2(blk + 128 + nh * 32 + j * 16);
-    }
-    __device__ static void load_scales(RawS& r, const uint8_t* blk, uint32_t nh) {
-        r.sc = ld_u64_a2(blk + 192 + nh * 8);
-        r.d = ld_u16(blk + 208);
-    }
-    __device__ static void unpack(const Raw& raw, uint32_t j, int8_t* dst) {
-        const uint4 qa = raw.qa, qb = raw.qb, qh = raw.qh;
-        const uint32_t a[4] = {qa.x, qa.y, qa.z, qa.w}, b[4] = {qb.x, qb.y, qb.z, qb.w}, h[4] = {qh.x, qh.y, qh.z, qh.w};
-        uint32_t o[4][4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            uint32_t q0 = (a[i] & 0x0F0F0F0Fu) | ((h[i] << 4) & 0x30303030u);
-            uint32_t q1 = (b[i] & 0x0F0F0F0Fu) | ((h[i] << 2) & 0x30303030u);
-            uint32_t q2 = ((a[i] >> 4) & 0x0F0F0F0Fu) | (h[i] & 0x30303030u);
-            uint32_t q3 = ((b[i] >> 4) & 0x0F0F0F0Fu) | ((h[i] >> 2) & 0x30303030u);
-            // q - 32 per byte: codes are 0..63, so flipping bit 5 gives the 6-bit two's
-            // complement; replicate it into bits 6 and 7 to sign-extend to int8
-            uint32_t s;
-            s = q0 ^ 0x20202020u; o[0][i] = s | ((s & 0x20202020u) << 1) | ((s & 0x20202020u) << 2);
-            s = q1 ^ 0x20202020u; o[1][i] = s | ((s & 0x20202020u) << 1) | ((s & 0x20202020u) << 2);
-            s = q2 ^ 0x20202020u; o[2][i] = s | ((s & 0x20202020u) << 1) | ((s & 0x20202020u) << 2);
-            s = q3 ^ 0x20202020u; o[3][i] = s | ((s & 0x20202020u) << 1) | ((s & 0x20202020u) << 2);
-        }
-#pragma unroll
-        for (int t = 0; t < 4; ++t)
-            *reinterpret_cast<uint4*>(dst + 32 * t + 16 * j) = make_uint4(o[t][0], o[t][1], o[t][2], o[t][3]);
-    }
-    // rs holds the int8 group scales as int32 (bit pattern), rd the super-block scale
-    __device__ static void scales(const RawS& raw, uint32_t, float* rs, float* rm, float* rd, uint32_t ld) {
-        const uint32_t s[2] = {raw.sc.x, raw.sc.y};
-#pragma unroll
-        for (int h = 0; h < 8; ++h)
-            rs[h * ld] = __builtin_bit_cast(float, static_cast<int>(static_cast<int8_t>((s[h >> 2] >> (8 * (h & 3))) & 0xFF)));
-        *rd = h2f(raw.d);
-        (void)rm;
     }
 };
 
@@ -177,7 +125,7 @@ struct GemmQ6K {
 struct GemmQ4_0 {
     static constexpr int WAVES_PER_SIMD = 3;   // register budget the kernel is compiled for
     static constexpr int NSUB = 4, KSTEP = 32;
-    static constexpr bool HAS_MIN = false, INT_SCALE = false;
+    static constexpr bool HAS_MIN = false;
     static constexpr int BLOCK_BYTES = 18 * 8;  // bytes per 256 elements
     static constexpr int WORDS = 4;
     struct Raw { uint4 q; };
@@ -203,16 +151,16 @@ struct GemmQ4_0 {
         *reinterpret_cast<uint4*>(dst + 32 * w) = lo;
         *reinterpret_cast<uint4*>(dst + 32 * w + 16) = hi;
     }
-    __device__ static void scales(const RawS& raw, uint32_t, float* rs, float* rm, float* rd, uint32_t ld) {
+    __device__ static void scales(const RawS& raw, uint32_t, float* rs, float* rm, uint32_t ld) {
 #pragma unroll
         for (int b = 0; b < 4; ++b) rs[b * ld] = h2f(raw.d[b]);
-        (void)rm; (void)rd;
+        (void)rm;
     }
 };
 struct GemmQ4_1 {
     static constexpr int WAVES_PER_SIMD = 3;   // register budget the kernel is compiled for
     static constexpr int NSUB = 4, KSTEP = 32;
-    static constexpr bool HAS_MIN = true, INT_SCALE = false;   // rm holds -m so that out = rs*dot - rm*sum(a) covers q*d + m
+    static constexpr bool HAS_MIN = true;   // rm holds -m so that out = rs*dot - rm*sum(a) covers q*d + m
     static constexpr int BLOCK_BYTES = 20 * 8;
     static constexpr int WORDS = 4;
     struct Raw { uint4 q; };
@@ -231,20 +179,19 @@ struct GemmQ4_1 {
         *reinterpret_cast<uint4*>(dst + 32 * w) = lo;
         *reinterpret_cast<uint4*>(dst + 32 * w + 16) = hi;
     }
-    __device__ static void scales(const RawS& raw, uint32_t, float* rs, float* rm, float* rd, uint32_t ld) {
+    __device__ static void scales(const RawS& raw, uint32_t, float* rs, float* rm, uint32_t ld) {
 #pragma unroll
         for (int b = 0; b < 4; ++b) {
             uint32_t dm = raw.dm[b];
             rs[b * ld] = h2f(dm & 0xFFFF);
             rm[b * ld] = -h2f(dm >> 16);
         }
-        (void)rd;
     }
 };
 struct GemmQ8_0 {
     static constexpr int WAVES_PER_SIMD = 2;   // register budget the kernel is compiled for
     static constexpr int NSUB = 4, KSTEP = 32;
-    static constexpr bool HAS_MIN = false, INT_SCALE = false;
+    static constexpr bool HAS_MIN = false;
     static constexpr int BLOCK_BYTES = 34 * 8;
     static constexpr int WORDS = 4;
     struct Raw { uint4 q0, q1; };
@@ -262,10 +209,10 @@ struct GemmQ8_0 {
         *reinterpret_cast<uint4*>(dst + 32 * w) = raw.q0;
         *reinterpret_cast<uint4*>(dst + 32 * w + 16) = raw.q1;
     }
-    __device__ static void scales(const RawS& raw, uint32_t, float* rs, float* rm, float* rd, uint32_t ld) {
+    __device__ static void scales(const RawS& raw, uint32_t, float* rs, float* rm, uint32_t ld) {
 #pragma unroll
         for (int b = 0; b < 4; ++b) rs[b * ld] = h2f(raw.d[b]);
-        (void)rm; (void)rd;
+        (void)rm;
     }
 };
 
@@ -275,7 +222,6 @@ static __global__ __launch_bounds__(256, T::WAVES_PER_SIMD) void gemm_kernel(Gem
     __shared__ __attribute__((aligned(16))) int8_t sA[GEMM_BM * GEMM_LDA];
     __shared__ __attribute__((aligned(16))) int8_t sB[GEMM_BN * GEMM_LDA];
     __shared__ __attribute__((aligned(16))) float sRS[T::NSUB * GEMM_BM];
-    __shared__ __attribute__((aligned(16))) float sRD[T::INT_SCALE ? GEMM_BM : 4];
     __shared__ __attribute__((aligned(16))) float sRM[T::HAS_MIN ? NB * GEMM_BM : 4];
     __shared__ __attribute__((aligned(16))) float sCS[NB * GEMM_BN];
     __shared__ __attribute__((aligned(16))) float sCM[T::HAS_MIN ? NB * GEMM_BN : 4];
@@ -350,7 +296,7 @@ static __global__ __launch_bounds__(256, T::WAVES_PER_SIMD) void gemm_kernel(Gem
         // ---- registers -> LDS: A 128 rows x WORDS words (unpacked), B 64 tokens x 8 words
 #pragma unroll
         for (int i = 0; i < AI; ++i) T::unpack(ra[i], a_w[i], a_dst[i]);
-        if (tid < GEMM_BM) T::scales(rsc, hs, sRS + tid, sRM + tid, sRD + tid, GEMM_BM);
+        if (tid < GEMM_BM) T::scales(rsc, hs, sRS + tid, sRM + tid, GEMM_BM);
 #pragma unroll
         for (int i = 0; i < 2; ++i) *reinterpret_cast<uint4*>(b_dst[i]) = b_live[i] ? rb[i] : make_uint4(0, 0, 0, 0);
         sCS[c_b * GEMM_BN + c_tok] = c_live ? rcs : 0.0f;
@@ -360,7 +306,7 @@ static __global__ __launch_bounds__(256, T::WAVES_PER_SIMD) void gemm_kernel(Gem
 
         // ---- MFMA over the K tile
         const int8_t* bRow = sB + (wn * 32 + col) * GEMM_LDA;
-        if (!T::INT_SCALE) {
+        {
             // Blocks in pairs.  The per-output scale  rs[row][b] * xs[token][b]  of both blocks of a
             // pair is one two-block outer product on the matrix core (each lane supplies the scale
             // of row `col` and of token `col` for the block of its half): one scalar LDS read per
@@ -397,39 +343,6 @@ static __global__ __launch_bounds__(256, T::WAVES_PER_SIMD) void gemm_kernel(Gem
                     for (int t = 0; t < 2; ++t) {
                         const float rm = -sRM[(2 * pr + half) * GEMM_BM + wm * 64 + t * 32 + col];
                         acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(rm, xm, acc[t], 0, 0, 0);
-                    }
-                }
-            }
-        } else {
-#pragma unroll
-            for (int b = 0; b < NB; ++b) {
-                // two 16-element scale groups share this block's activation scale.  Their per-output
-                // scales  sc[row][group] * xs[token]  (an 8-bit integer times an f16 value: exact in
-                // f32) are the two blocks of one outer-product MFMA, as above.
-                const float xs = sCS[b * GEMM_BN + wn * 32 + col];
-                const long bf0 = *reinterpret_cast<const long*>(bRow + b * 32 + half * 8);
-                const long bf1 = *reinterpret_cast<const long*>(bRow + b * 32 + 16 + half * 8);
-#pragma unroll
-                for (int t = 0; t < 2; ++t) {
-                    // (sc * d) is exact (8 x 11 bits); times xs it rounds once, as the reference's
-                    // own  ([sc0, sc1] * d) * xs  does
-                    const float rsl = static_cast<float>(__builtin_bit_cast(
-                                          int, sRS[(2 * b + half) * GEMM_BM + wm * 64 + t * 32 + col])) *
-                                      sRD[wm * 64 + t * 32 + col];
-                    v32f z32;
-#pragma unroll
-                    for (int e = 0; e < 32; ++e) z32[e] = 0.0f;
-                    const v32f sc = __builtin_amdgcn_mfma_f32_32x32x1f32(rsl, xs, z32, 0, 0, 0);
-                    const int8_t* aRow = sA + (wm * 64 + t * 32 + col) * GEMM_LDA;
-                    const long af0 = *reinterpret_cast<const long*>(aRow + b * 32 + half * 8);
-                    const long af1 = *reinterpret_cast<const long*>(aRow + b * 32 + 16 + half * 8);
-                    v16i z = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-                    v16i c0 = __builtin_amdgcn_mfma_i32_32x32x16_i8(af0, bf0, z, 0, 0, 0);
-                    v16i c1 = __builtin_amdgcn_mfma_i32_32x32x16_i8(af1, bf1, z, 0, 0, 0);
-#pragma unroll
-                    for (int e = 0; e < 16; ++e) {
-                        acc[t][e] = fmaf(static_cast<float>(c0[e]), sc[e], acc[t][e]);
-                        acc[t][e] = fmaf(static_cast<float>(c1[e]), sc[16 + e], acc[t][e]);
                     }
                 }
             }

@@ -27,8 +27,8 @@ struct cera_hip_ctx {
     std::string err;
     uint32_t n_cu = 0;
     // grow-only device scratch for the host-pointer entry points
-    void* scratch[10] = {nullptr};
-    uint64_t scratch_bytes[10] = {0};
+    void* scratch[12] = {nullptr};
+    uint64_t scratch_bytes[12] = {0};
     // attention split-K workspace
     float* attn_acc = nullptr;
     float* attn_ml = nullptr;

@@ -5,7 +5,7 @@
 #include <cmath>
 #include <cstring>
 
-#include "gemm.cuh"
+#include "gemm_q6k_f16.cuh"
 #include "glue.cuh"
 #include "model.h"
 
@@ -24,7 +24,8 @@ bool cera_gemm_supports(uint32_t dtype, uint64_t k) { return gemm_type_ok(dtype)
 cera_hip_status cera_launch_gemm(cera_hip_ctx* ctx, const cera_hip_dtensor* w, const float* bs, const int8_t* bq,
                                  const float* bsum, uint32_t n, float* out, uint64_t ld_m, uint64_t ld_n,
                                  const float* resid, float resid_scale, const cera_hip_dtensor* w2 = nullptr,
-                                 float* out2 = nullptr, uint64_t ld_n2 = 0, bool* paired = nullptr) {
+                                 float* out2 = nullptr, uint64_t ld_n2 = 0, bool* paired = nullptr, void* bh_ws = nullptr,
+                                 bool* staged = nullptr) {
     if (!cera_gemm_supports(w->dtype, w->k))
         return cera_fail(ctx, CERA_HIP_ERR_UNSUPPORTED_DTYPE,
                          "gemm: no int8 GEMM for ggml type " + std::to_string(w->dtype) + " with k=" + std::to_string(w->k));
@@ -34,6 +35,22 @@ cera_hip_status cera_launch_gemm(cera_hip_ctx* ctx, const cera_hip_dtensor* w, c
     a.m = static_cast<uint32_t>(w->m); a.n = n; a.k = static_cast<uint32_t>(w->k);
     a.row_bytes = static_cast<uint32_t>(w->row_bytes);
     a.ld_m = ld_m; a.ld_n = ld_n; a.resid = resid; a.resid_scale = resid_scale;
+    // Q6_K runs its block dots on the f16 matrix cores and reads the quants as f16: converted here
+    // unless the caller says its workspace (bh_ws) still holds these activations (*staged)
+    a.bh = nullptr;
+    if (w->dtype == CERA_HIP_Q6_K) {
+        if (!bh_ws) {
+            CERA_TRY(cera_scratch(ctx, 10, static_cast<uint64_t>(n) * a.k * 2, &bh_ws));
+            staged = nullptr;
+        }
+        if (!staged || !*staged) {
+            const uint64_t words = static_cast<uint64_t>(n) * a.k / 16;
+            hipLaunchKernelGGL(gemm_act_f16_kernel, dim3(static_cast<uint32_t>((words + 255) / 256)), dim3(256), 0,
+                               ctx->stream, reinterpret_cast<const uint4*>(bq), static_cast<uint4*>(bh_ws), words);
+            if (staged) *staged = true;
+        }
+        a.bh = bh_ws;
+    }
     dim3 grid((n + GEMM_BN - 1) / GEMM_BN, (a.m + GEMM_BM - 1) / GEMM_BM);
     a.w2 = nullptr; a.out2 = nullptr; a.m2 = 0; a.tiles1 = grid.y; a.ld_n2 = 0;
     if (paired) *paired = false;
@@ -71,7 +88,7 @@ cera_hip_status cera_launch_gemm(cera_hip_ctx* ctx, const cera_hip_dtensor* w, c
     }
     switch (w->dtype) {
         case CERA_HIP_Q4_K: hipLaunchKernelGGL((gemm_kernel<GemmQ4K>), grid, dim3(256), 0, ctx->stream, a); break;
-        case CERA_HIP_Q6_K: hipLaunchKernelGGL((gemm_kernel<GemmQ6K>), grid, dim3(256), 0, ctx->stream, a); break;
+        case CERA_HIP_Q6_K: hipLaunchKernelGGL(gemm_q6k_f16_kernel, grid, dim3(256), 0, ctx->stream, a); break;
         case CERA_HIP_Q4_0: hipLaunchKernelGGL((gemm_kernel<GemmQ4_0>), grid, dim3(256), 0, ctx->stream, a); break;
         case CERA_HIP_Q4_1: hipLaunchKernelGGL((gemm_kernel<GemmQ4_1>), grid, dim3(256), 0, ctx->stream, a); break;
         default: hipLaunchKernelGGL((gemm_kernel<GemmQ8_0>), grid, dim3(256), 0, ctx->stream, a); break;
@@ -207,6 +224,7 @@ static cera_hip_status ensure_prefill_buffers(cera_hip_model* m, uint32_t n) {
     CERA_TRY(alloc(cap * c.ffn * 4ull, reinterpret_cast<void**>(&m->pf_gate)));
     CERA_TRY(alloc(cap * c.ffn * 4ull, reinterpret_cast<void**>(&m->pf_up)));
     CERA_TRY(alloc(cap * maxk, reinterpret_cast<void**>(&m->pf_xq)));
+    CERA_TRY(alloc(cap * maxk * 2, &m->pf_xh));
     CERA_TRY(alloc(cap * (maxk / 32) * 4, reinterpret_cast<void**>(&m->pf_xs)));
     CERA_TRY(alloc(cap * (maxk / 32) * 4, reinterpret_cast<void**>(&m->pf_bsum)));
     CERA_TRY(alloc(cap * 4ull, reinterpret_cast<void**>(&m->pf_tokens)));
@@ -232,7 +250,10 @@ static cera_hip_status prefill_chunk(cera_hip_model* m, const uint32_t* tokens, 
                        m->embd->row_bytes, m->pf_tokens, hs, c.embed_scale, m->pf_hidden);
     HIP_TRY(ctx, hipGetLastError());
 
+    // whether pf_xh holds the f16 form of the quants now in pf_xq; cleared wherever those are rewritten
+    bool staged = false;
     auto norm_rows = [&](const float* x, const float* w, float* y) -> cera_hip_status {
+        staged = false;
         hipLaunchKernelGGL((rmsnorm_kernel<true>), dim3(n), dim3(256), 0, s, x, w, hs, c.rms_eps, y, m->pf_xs, m->pf_xq,
                            m->pf_bsum);
         HIP_TRY(ctx, hipGetLastError());
@@ -248,7 +269,8 @@ static cera_hip_status prefill_chunk(cera_hip_model* m, const uint32_t* tokens, 
                                          static_cast<uint32_t>(w->k), n, out, static_cast<uint32_t>(w->m), resid, &launched));
             if (launched) return CERA_HIP_OK;
         }
-        return cera_launch_gemm(ctx, w, m->pf_xs, m->pf_xq, m->pf_bsum, n, out, 1, w->m, resid, c.residual_scale);
+        return cera_launch_gemm(ctx, w, m->pf_xs, m->pf_xq, m->pf_bsum, n, out, 1, w->m, resid, c.residual_scale, nullptr,
+                                nullptr, 0, nullptr, m->pf_xh, &staged);
     };
 
     // two projections of the same activations: one launch when both have an int8 GEMM of the same
@@ -258,9 +280,10 @@ static cera_hip_status prefill_chunk(cera_hip_model* m, const uint32_t* tokens, 
         if (n > PREFILL_SMALL_BATCH && cera_gemm_supports(wa->dtype, wa->k) && cera_gemm_supports(wb->dtype, wb->k)) {
             bool paired = false;
             CERA_TRY(cera_launch_gemm(ctx, wa, m->pf_xs, m->pf_xq, m->pf_bsum, n, outa, 1, wa->m, nullptr, 1.0f, wb, outb,
-                                      wb->m, &paired));
+                                      wb->m, &paired, m->pf_xh, &staged));
             if (paired) return CERA_HIP_OK;
-            return cera_launch_gemm(ctx, wb, m->pf_xs, m->pf_xq, m->pf_bsum, n, outb, 1, wb->m, nullptr, 1.0f);
+            return cera_launch_gemm(ctx, wb, m->pf_xs, m->pf_xq, m->pf_bsum, n, outb, 1, wb->m, nullptr, 1.0f, nullptr,
+                                    nullptr, 0, nullptr, m->pf_xh, &staged);
         }
         CERA_TRY(gemm(wa, outa, nullptr));
         return gemm(wb, outb, nullptr);
@@ -297,6 +320,7 @@ static cera_hip_status prefill_chunk(cera_hip_model* m, const uint32_t* tokens, 
         // causal attention: query t sees positions 0 .. start_pos + t
         CERA_TRY(cera_launch_attn(ctx, m->pf_q, L.kc, L.vc, c.n_heads, c.n_kv_heads, c.head_dim, start_pos + 1ull,
                                   c.max_seq_len, scale, 0, n, m->pf_attn, m->pf_xs, m->pf_xq, m->pf_bsum, nullptr, m->kv_f16));
+        staged = false;   // the attention merge rewrote the quants
         CERA_TRY(gemm(L.o, m->pf_hidden, m->pf_hidden));
 
         CERA_TRY(norm_rows(m->pf_hidden, L.ffn_norm, m->pf_normed));
@@ -305,6 +329,7 @@ static cera_hip_status prefill_chunk(cera_hip_model* m, const uint32_t* tokens, 
         hipLaunchKernelGGL((silu_mul_kernel<true>), dim3(static_cast<uint32_t>((tot / 4 + 255) / 256)), dim3(256), 0, s,
                            m->pf_gate, m->pf_up, tot, m->pf_gate, m->pf_xs, m->pf_xq, m->pf_bsum);
         HIP_TRY(ctx, hipGetLastError());
+        staged = false;   // ... and so did the SwiGLU
         CERA_TRY(gemm(L.down, m->pf_hidden, m->pf_hidden));
     }
     m->seq_len = start_pos + n;
