@@ -598,9 +598,17 @@ cera_hip_status cera_launch_attn(cera_hip_ctx* ctx, const float* q, const void* 
     }
     HIP_TRY(ctx, hipGetLastError());
     dim3 mgrid(n_heads, n_queries);
+    const uint32_t n_pairs = n_heads * n_queries;
 #define ATTN_MERGE(QQ, HH)                                                                                              \
-    hipLaunchKernelGGL((attn_decode_merge_kernel<QQ, HH>), mgrid, dim3(256), 0, ctx->stream, ctx->attn_acc, ctx->attn_ml, \
-                       n_parts, G, n_heads, out, out_scales, out_quants, out_bsum)
+    do {                                                                                                                \
+        if (batch)                                                                                                      \
+            hipLaunchKernelGGL((attn_prefill_merge_kernel<QQ, HH>), dim3((n_pairs + 7) / 8), dim3(256), 0, ctx->stream,  \
+                               ctx->attn_acc, ctx->attn_ml, n_parts, G, n_heads, n_pairs, out, out_scales, out_quants,  \
+                               out_bsum);                                                                               \
+        else                                                                                                            \
+            hipLaunchKernelGGL((attn_decode_merge_kernel<QQ, HH>), mgrid, dim3(256), 0, ctx->stream, ctx->attn_acc,      \
+                               ctx->attn_ml, n_parts, G, n_heads, out, out_scales, out_quants, out_bsum);               \
+    } while (0)
     if (out_quants) { if (head_dim == 128) ATTN_MERGE(true, 128); else ATTN_MERGE(true, 64); }
     else            { if (head_dim == 128) ATTN_MERGE(false, 128); else ATTN_MERGE(false, 64); }
 #undef ATTN_MERGE

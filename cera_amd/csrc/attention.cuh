@@ -661,3 +661,55 @@ __global__ __launch_bounds__(256) void attn_decode_merge_kernel(const float* __r
         }
     }
 }
+
+// Merge for a batch of queries (prefill): the same formula as above over the few parts a prefill
+// pass makes (8 at most), but eight (query, head) pairs per workgroup, 32 lanes each (a float4 of
+// the head's columns per lane), the parts walked in order by every lane.  The decode merge spends
+// a 256-thread workgroup and two barriers on one pair, which for 512 queries x 32 heads x 4 parts
+// cost more than the attention itself.
+template <bool QUANT, int HD>
+__global__ __launch_bounds__(256) void attn_prefill_merge_kernel(const float* __restrict__ part_acc,
+                                                                 const float* __restrict__ part_ml,
+                                                                 uint32_t n_parts, uint32_t G, uint32_t n_heads,
+                                                                 uint32_t n_pairs, float* __restrict__ out,
+                                                                 float* __restrict__ scales, int8_t* __restrict__ quants,
+                                                                 float* __restrict__ bsum) {
+    const uint32_t pair = blockIdx.x * 8 + (threadIdx.x >> 5), c = threadIdx.x & 31;
+    if (pair >= n_pairs) return;   // whole 32-lane groups leave together
+    const uint32_t qi = pair / n_heads, head = pair % n_heads;
+    const uint32_t kvh = head / G, hg = head % G, n_kv = n_heads / G;
+    const uint64_t pbase = (static_cast<uint64_t>(qi) * n_kv + kvh) * n_parts;
+    constexpr uint32_t C4 = HD / 4;
+    const bool live = c < C4;
+    float M = -__builtin_inff();
+    for (uint32_t p = 0; p < n_parts; ++p) M = fmaxf(M, part_ml[((pbase + p) * G + hg) * 2]);
+    float L = 0.0f;
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (uint32_t p = 0; p < n_parts; ++p) {
+        const float2 ml = *reinterpret_cast<const float2*>(part_ml + ((pbase + p) * G + hg) * 2);
+        const float w = cera_expf(ml.x - M);
+        L = fmaf(w, ml.y, L);
+        float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (live) a = reinterpret_cast<const float4*>(part_acc + ((pbase + p) * G + hg) * HD)[c];
+        acc.x = fmaf(w, a.x, acc.x); acc.y = fmaf(w, a.y, acc.y);
+        acc.z = fmaf(w, a.z, acc.z); acc.w = fmaf(w, a.w, acc.w);
+    }
+    const float inv = 1.0f / L;
+    const float4 o = make_float4(acc.x * inv, acc.y * inv, acc.z * inv, acc.w * inv);
+    const uint64_t row = static_cast<uint64_t>(qi) * n_heads + head;   // outputs are [n_queries][n_heads][HD]
+    if (live) reinterpret_cast<float4*>(out + row * HD)[c] = o;
+    if (QUANT) {
+        // every lane of the pair takes part in the 8-lane exchanges; whole groups of 8 are live or idle together
+        float sc;
+        const uint32_t packed = q8_quantize_quad(o, sc);
+        const float ssum = bsum ? q8_block_scaled_sum(packed, sc) : 0.0f;
+        if (live) {
+            reinterpret_cast<uint32_t*>(quants)[row * C4 + c] = packed;
+            if ((c & 7) == 0) {
+                scales[row * (HD / 32) + (c >> 3)] = sc;
+                if (bsum) bsum[row * (HD / 32) + (c >> 3)] = ssum;
+            }
+        }
+    }
+}
+
