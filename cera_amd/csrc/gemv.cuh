@@ -83,14 +83,16 @@ struct Q4K {
     }
     __device__ static float dot(const Wt& w, const Act& a, uint32_t u, int32_t* dbg) {
         uint32_t g = (u >> 1) & 3;
-        // 6-bit scales/mins of sub-blocks 2g, 2g+1 (get_scale_min_k4)
-        uint32_t sh = 16 * (g & 1);
-        uint32_t y2 = (w.h.y >> sh) & 0xFFFF, z2 = (w.h.z >> sh) & 0xFFFF, w2 = (w.h.w >> sh) & 0xFFFF;
-        // branch-free select between the two packings (low sub-blocks keep 6 bits in
-        // place; high ones splice a nibble of bytes 8..11 with the top two bits)
-        const uint32_t low = g < 2 ? 0xFFFFFFFFu : 0u;
-        uint32_t sc2 = ((y2 & 0x3F3F) & low) | (((w2 & 0x0F0F) | ((y2 >> 2) & 0x3030)) & ~low);
-        uint32_t mn2 = ((z2 & 0x3F3F) & low) | ((((w2 >> 4) & 0x0F0F) | ((z2 >> 2) & 0x3030)) & ~low);
+        // 6-bit scales/mins of sub-blocks 2g, 2g+1 (get_scale_min_k4), two per 16-bit pair.  Low
+        // sub-blocks keep their 6 bits in place in bytes 0..3 / 4..7; high ones splice a nibble of
+        // bytes 8..11 with the top two bits of those bytes.  Which packing applies depends on the
+        // lane's unit only, so it is folded into shift counts and masks that stay in registers
+        // across the rows: two shifts, an AND and an AND-OR per pair instead of a select.
+        const uint32_t sh = 16 * (g & 1);
+        const bool low = g < 2;
+        const uint32_t sh_a = low ? sh : sh + 2, m_a = low ? 0x3F3Fu : 0x3030u, m_b = low ? 0u : 0x0F0Fu;
+        const uint32_t sc2 = ((w.h.y >> sh_a) & m_a) | ((w.h.w >> sh) & m_b);
+        const uint32_t mn2 = ((w.h.z >> sh_a) & m_a) | ((w.h.w >> (sh + 4)) & m_b);
         float d = h2f(w.h.x & 0xFFFF), dmin = h2f(w.h.x >> 16);
         int dl = 0, dh = 0;
         const uint32_t q[4] = {w.q.x, w.q.y, w.q.z, w.q.w};
