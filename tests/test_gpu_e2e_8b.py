@@ -4,8 +4,10 @@ mix), 512-token prefill of uniform random ids, then 256 greedy tokens -- the GPU
 backend through HipLlamaModel against the CPU oracle on the same file.
 
 The oracle side takes a few minutes of CPU time (and the file is 5.2 GB), so
-the test only runs when CERA_E2E_8B=1; a smaller number of layers can be chosen
-with CERA_E2E_LAYERS for a quicker pass over the same per-layer shapes.
+the full test only runs when CERA_E2E_8B=1; a smaller number of layers can be chosen
+with CERA_E2E_LAYERS for a quicker pass over the same per-layer shapes.  A cut of the
+same architecture (4 layers, the full-width embedding and head, 128-token prefill,
+32 greedy tokens; 1.4 GB, seconds of CPU time) runs with every GPU test run.
 """
 import os
 import time
@@ -16,18 +18,26 @@ import pytest
 import util
 from cera_amd import host_api as H, llama_api, synth
 
-pytestmark = [pytest.mark.gpu,
-              pytest.mark.skipif(os.environ.get("CERA_E2E_8B") != "1", reason="set CERA_E2E_8B=1 (minutes of CPU time)")]
+pytestmark = pytest.mark.gpu
 
 
 def _say(msg):
     print(msg, flush=True)
 
 
+@pytest.mark.skipif(os.environ.get("CERA_E2E_8B") != "1", reason="set CERA_E2E_8B=1 (minutes of CPU time)")
 def test_llama3_8b_prefill_512_greedy_256(tmp_path, orc, hip):
+    n_layers = int(os.environ.get("CERA_E2E_LAYERS", synth.LLAMA3_8B["n_layers"]))
+    _run(tmp_path, orc, n_layers, 512, int(os.environ.get("CERA_E2E_NEW", 256)))
+
+
+def test_llama3_8b_shapes_4_layers_prefill_128_greedy_32(tmp_path, orc, hip):
+    _run(tmp_path, orc, 4, 128, 32)
+
+
+def _run(tmp_path, orc, n_layers, n_prompt, n_new):
     cfg = dict(synth.LLAMA3_8B, max_seq_len=1024)
-    cfg["n_layers"] = int(os.environ.get("CERA_E2E_LAYERS", cfg["n_layers"]))
-    n_prompt, n_new = 512, int(os.environ.get("CERA_E2E_NEW", 256))
+    cfg["n_layers"] = n_layers
     threads = min(16, os.cpu_count() or 1)
     path = str(tmp_path / "llama3_8b_synth.gguf")
     t0 = time.time()
