@@ -174,7 +174,7 @@ def test_prefill_equals_decode_on_gpu(hip):
 
 
 @pytest.mark.parametrize("nh,nkv,start,n", [(32, 8, 0, 512), (8, 2, 0, 40), (8, 8, 300, 100), (16, 2, 1000, 33),
-                                             (4, 1, 0, 16), (32, 8, 4000, 96)])
+                                             (4, 1, 0, 16), (32, 8, 4000, 96), (32, 8, 2048, 2048)])
 def test_attn_prefill_batch_vs_oracle(hip, orc, nh, nkv, start, n):
     """Causal attention of a batch of queries (the tiled MFMA kernel) against the oracle's
     decode_attention evaluated query by query: query i sees positions 0 .. start + i."""
