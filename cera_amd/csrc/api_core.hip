@@ -517,9 +517,16 @@ static void attn_launch_partials(cera_hip_ctx* ctx, const AttnLaunch& a, const K
     if (a.batch) {
         // heaviest query blocks (most visible keys) first
         const dim3 pgrid((a.n_queries + 31) / 32, a.n_kv_heads, a.n_parts);
-        hipLaunchKernelGGL((attn_prefill_partial_kernel<KV, HD>), pgrid, dim3(64 * a.G), 0, ctx->stream, a.q, kc, vc, a.seq_len,
-                           a.n_queries, a.max_seq, a.scale, a.part_keys, a.n_parts, a.q_stride, a.G, ctx->attn_acc,
-                           ctx->attn_ml);
+#define ATTN_PF(GG)                                                                                                        \
+    hipLaunchKernelGGL((attn_prefill_partial_kernel<KV, HD, GG>), pgrid, dim3(64 * GG), 0, ctx->stream, a.q, kc, vc, a.seq_len, \
+                       a.n_queries, a.max_seq, a.scale, a.part_keys, a.n_parts, a.q_stride, ctx->attn_acc, ctx->attn_ml)
+        switch (a.G) {
+            case 1: ATTN_PF(1); break;
+            case 2: ATTN_PF(2); break;
+            case 4: ATTN_PF(4); break;
+            default: ATTN_PF(8); break;
+        }
+#undef ATTN_PF
         return;
     }
     switch (a.G) {
@@ -548,6 +555,7 @@ cera_hip_status cera_launch_attn(cera_hip_ctx* ctx, const float* q, const void* 
     // eight parts per query block beyond that.
     if (new_kv && n_queries != 1) return cera_fail(ctx, CERA_HIP_ERR_ARGUMENT, "attention: fused RoPE/append is for single-token decode");
     const bool batch = n_queries >= 16;
+    if (batch && (reinterpret_cast<uintptr_t>(q) & 15)) return cera_fail(ctx, CERA_HIP_ERR_ARGUMENT, "attention: a query batch must be 16-byte aligned");
     const AttnNewKV nk = new_kv ? *new_kv : AttnNewKV{};
     uint32_t n_parts, part_keys = 0, chunks_per_part = 0;
     uint32_t S = 1;

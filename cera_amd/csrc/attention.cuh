@@ -400,51 +400,84 @@ __global__ __launch_bounds__(256) void attn_decode_partial_kernel(
 }
 
 // ---------------------------------------------------------------------------
-// Causal attention for a batch of queries (prefill) on the f32 matrix cores.
+// Causal attention for a batch of queries (prefill) on the f16 matrix cores, at f32
+// accuracy.
 //
 // The decode kernel above reads the whole visible K/V range once per query; for a
 // prompt of n tokens that is n passes over the cache.  Here one wavefront owns a
 // block of 32 consecutive queries of one head and walks the keys in tiles of 32, so
-// a K/V tile is read once per 32 queries, and both contractions run as
-// v_mfma_f32_32x32x2_f32 (f32 products, f32 accumulation: the same arithmetic class
-// as the reference's f32 dot products, cera/src/backend/cpu.rs:4028-4241).
+// a K/V tile is read once per 32 queries.  Both contractions run as
+// v_mfma_f32_32x32x16_f16 on operands split in two: every f32 value x is staged as
+// the f16 pair (hi, lo), hi = x truncated to f16 and lo = (x - hi) truncated, so
+// x = hi + lo up to 2^-21 |x|, and a product x.y is the three MFMAs hi.hi + hi.lo + lo.hi
+// (each f16 product is exact in the f32 accumulator; the dropped lo.lo term is below
+// 2^-22 |x.y|).  That keeps the arithmetic class of the reference's f32 dot products
+// (cera/src/backend/cpu.rs:4028-4241) at a fifth of the f32 MFMA's cycles.  A half
+// cache has no low parts and takes two MFMAs per product.
 //
-//   S^T = K . Q^T   A = K tile (row = key, from LDS, transposed there so the lanes
-//                   of one step read consecutive words), B = the lane's query
-//                   (registers).  A lane ends up with 16 keys of ONE query, so the
+//   S^T = K . Q^T   A = K tile (row = key; the lane of key `col` reads 8 consecutive
+//                   dims of its half from LDS), B = the lane's query (registers, the
+//                   same dims).  A lane ends up with 16 keys of ONE query, so the
 //                   softmax reduction over keys is over registers plus one exchange
 //                   between the wavefront halves.
-//   O  += P . V     A = P straight from those registers (the MFMA step (blk, r) pairs
-//                   key 8blk+r of the lower half with key 8blk+4+r of the upper half,
-//                   exactly the rows the two halves hold), B = V rows from HBM/L2.
+//   O  += P . V     A = P straight from those registers: the lanes of half h hold keys
+//                   8blk + 4h + r, and the MFMA over keys 16kk .. 16kk+15 takes its
+//                   eight K slots of half h from blk = 2kk, 2kk+1.  B = the V tile,
+//                   staged TRANSPOSED in LDS with the keys of each 16 in that slot order
+//                   (position 8h + 4(blk&1) + r), so a lane reads its eight keys of one
+//                   output column as one 16-byte word.
 //
-// Online softmax per key tile with the reference's polynomial expf and an f64
-// running sum.  The key range is cut into parts of `part_keys`; a workgroup
+// Online softmax per key tile in the base-2 domain (v_exp_f32 on scores pre-multiplied by
+// log2 e; the reference's polynomial expf agrees with it to a few ulp, far inside this
+// kernel's tolerance) with an f64 running sum.  The key range is cut into parts of `part_keys`; a workgroup
 // produces the (m, l, acc) partial of one (query block, head, part) in the layout
 // the merge kernel below consumes, so long prompts spread over the chip and the
 // merge (and its fused Q8_0 quantisation) is shared with the decode path.
-// A workgroup is the G query heads of one KV head, one wavefront each: the K tile
-// (transposed) and the V tile are staged in LDS once, by all G wavefronts together,
-// and every head of the group reads them from there.
+// A workgroup is the G query heads of one KV head, one wavefront each: the K and V
+// tiles are split and staged in LDS once, by all G wavefronts together, and every
+// head of the group reads them from there.
 // grid = (query blocks, KV heads, parts), 64 * G threads.
-#define ATTN_PF_LD 33  // words per LDS row of the transposed K tile (32 + 1 pad)
 typedef float attn_v16f __attribute__((ext_vector_type(16)));
+typedef _Float16 attn_v8h __attribute__((ext_vector_type(8)));
+typedef _Float16 attn_v2h __attribute__((ext_vector_type(2)));
+#define ATTN_PF_KLD(HD) ((HD) + 8)   // halves per LDS row of the K tile: 16-byte reads of 16 rows cover all banks
+#define ATTN_PF_VTLD 40              // halves per LDS row of the transposed V tile (32 keys + 8 pad), same property
 
-#define ATTN_PF_VLD(HD) ((HD) + 8)   // words per LDS row of the V tile: the halves' rows (4 apart) fall in different banks
-template <typename KV, int HD>
-__global__ __launch_bounds__(512) void attn_prefill_partial_kernel(
-    const float* __restrict__ q,       // [n_queries][q_stride]
+// (a, b) -> packed f16 high parts and packed f16 low parts
+__device__ __forceinline__ void attn_split2(float a, float b, uint32_t& hi, uint32_t& lo) {
+    const attn_v2h h = __builtin_bit_cast(attn_v2h, __builtin_amdgcn_cvt_pkrtz(a, b));
+    hi = __builtin_bit_cast(uint32_t, h);
+    lo = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(a - static_cast<float>(h[0]), b - static_cast<float>(h[1])));
+}
+__device__ __forceinline__ attn_v16f attn_mfma(const uint4& a, const uint4& b, attn_v16f c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(attn_v8h, a), __builtin_bit_cast(attn_v8h, b), c, 0, 0, 0);
+}
+
+template <typename KV, int HD, int G>
+__global__ __launch_bounds__(64 * G) void attn_prefill_partial_kernel(
+    const float* __restrict__ q,       // [n_queries][q_stride], rows 16-byte aligned
     const KV* __restrict__ kc,         // [n_kv][max_seq][128], already holding the batch's keys
     const KV* __restrict__ vc,
     uint32_t first_len,                // keys visible to query 0; query i sees first_len + i
     uint32_t n_queries, uint32_t max_seq, float scale, uint32_t part_keys, uint32_t n_parts, uint32_t q_stride,
-    uint32_t G,
     float* __restrict__ part_acc,      // [n_queries][n_kv][n_parts][G][128]
     float* __restrict__ part_ml) {     // [n_queries][n_kv][n_parts][G][2]
-    constexpr int VLD = ATTN_PF_VLD(HD);
-    __shared__ float sKt[HD * ATTN_PF_LD];
-    __shared__ __attribute__((aligned(16))) float sV[32 * VLD];
-    __shared__ __attribute__((aligned(16))) float sXall[8 * 32];
+    constexpr bool LOW = sizeof(KV) == 4;   // an f32 cache has low parts, a half cache is its own high part
+    constexpr int KLD = ATTN_PF_KLD(HD), VTLD = ATTN_PF_VTLD;
+    constexpr int NJ = HD / 16;    // MFMA steps over the head dimension
+    constexpr int NDT = HD / 32;   // 32-column output tiles
+    constexpr int NT = 64 * G;     // threads
+    // staging items per thread: K quads (32 keys x HD/4), V quad pairs (16 key pairs x HD/4)
+    constexpr int K_ITEMS = 32 * (HD / 4), V_ITEMS = 16 * (HD / 4);
+    constexpr int KI = (K_ITEMS + NT - 1) / NT, VI = (V_ITEMS + NT - 1) / NT;
+    // the next tile's global loads stay in flight (in registers) while this one is multiplied,
+    // where a thread's share of a tile is small enough to hold
+    constexpr bool PREFETCH = KI + 2 * VI <= 10;
+    __shared__ __attribute__((aligned(16))) _Float16 sKh[32 * KLD];
+    __shared__ __attribute__((aligned(16))) _Float16 sKl[LOW ? 32 * KLD : 8];
+    __shared__ __attribute__((aligned(16))) _Float16 sVh[HD * VTLD];
+    __shared__ __attribute__((aligned(16))) _Float16 sVl[LOW ? HD * VTLD : 8];
+    __shared__ __attribute__((aligned(16))) float sXall[G * 32];
     const uint32_t tid = threadIdx.x, lane = tid & 63, col = lane & 31, half = lane >> 5;
     const uint32_t kvh = blockIdx.y, hg = tid >> 6, head = kvh * G + hg, n_kv = gridDim.y;
     float* sX = sXall + 32 * hg;
@@ -459,88 +492,167 @@ __global__ __launch_bounds__(512) void attn_prefill_partial_kernel(
     const KV* kbase = kc + static_cast<uint64_t>(kvh) * max_seq * HD;
     const KV* vbase = vc + static_cast<uint64_t>(kvh) * max_seq * HD;
 
-    // this lane's query, the dims of its half: d = 2s + half
-    float qreg[HD / 2];
+    // this lane's query, split: step j holds dims 16j + 8half .. +7
+    uint4 qh[NJ], ql[NJ];
     {
-        const float* qp = q + static_cast<uint64_t>(min(qidx, n_queries - 1)) * q_stride + head * HD + half;
+        const float* qp = q + static_cast<uint64_t>(min(qidx, n_queries - 1)) * q_stride + head * HD + 8 * half;
 #pragma unroll
-        for (int s = 0; s < HD / 2; ++s) qreg[s] = qp[2 * s];
+        for (int j = 0; j < NJ; ++j) {
+            const float4 a = *reinterpret_cast<const float4*>(qp + 16 * j), b = *reinterpret_cast<const float4*>(qp + 16 * j + 4);
+            attn_split2(a.x, a.y, qh[j].x, ql[j].x);
+            attn_split2(a.z, a.w, qh[j].y, ql[j].y);
+            attn_split2(b.x, b.y, qh[j].z, ql[j].z);
+            attn_split2(b.z, b.w, qh[j].w, ql[j].w);
+        }
     }
-    constexpr int NDT = HD / 32;   // 32-column output tiles
     attn_v16f acc[NDT];
 #pragma unroll
     for (int dt = 0; dt < NDT; ++dt)
 #pragma unroll
         for (int e = 0; e < 16; ++e) acc[dt][e] = 0.0f;
-    float m = -__builtin_inff();
+    float m = -__builtin_inff();   // running maximum, base-2 domain
     double l = 0.0;
+    const float scale2 = scale * 1.44269504088896340736f;
 
-    for (uint32_t k0 = key_lo; k0 < key_hi; k0 += 32) {
-        // ---- K tile -> LDS transposed, V tile -> LDS as it lies: 32 keys x HD/4 float4 each, spread
-        // over the workgroup; keys past the part's end are zeros (their weights are zero too)
-        for (uint32_t f = tid; f < 32 * (HD / 4); f += blockDim.x) {
-            const uint32_t key = f / (HD / 4), c4 = f % (HD / 4);
-            float4 v = make_float4(0.f, 0.f, 0.f, 0.f), w = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (k0 + key < key_hi) {
-                v = KvOps<KV>::ld4(kbase + static_cast<uint64_t>(k0 + key) * HD, c4);
-                w = KvOps<KV>::ld4(vbase + static_cast<uint64_t>(k0 + key) * HD, c4);
-            }
-            sKt[(4 * c4 + 0) * ATTN_PF_LD + key] = v.x;
-            sKt[(4 * c4 + 1) * ATTN_PF_LD + key] = v.y;
-            sKt[(4 * c4 + 2) * ATTN_PF_LD + key] = v.z;
-            sKt[(4 * c4 + 3) * ATTN_PF_LD + key] = v.w;
-            *reinterpret_cast<float4*>(sV + key * VLD + 4 * c4) = w;
+    // ---- staging.  K tile -> LDS by rows, an item is one key x one quad of dims.  V tile -> LDS
+    // transposed: an item is two neighbouring keys (neighbours in slot order too) x one quad of
+    // dims; consecutive lanes take consecutive key pairs, so the 4-byte stores of a wavefront fall
+    // in different banks.  Keys past the part's end are zeros (their weights are zero too).
+    float4 kreg[KI], v0reg[VI], v1reg[VI];
+    auto fetch = [&](uint32_t k0) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < KI; ++i) {
+            const uint32_t f = tid + NT * i, key = f / (HD / 4), c4 = f % (HD / 4);
+            kreg[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (f < K_ITEMS && k0 + key < key_hi) kreg[i] = KvOps<KV>::ld4(kbase + static_cast<uint64_t>(k0 + key) * HD, c4);
         }
+#pragma unroll
+        for (int i = 0; i < VI; ++i) {
+            const uint32_t f = tid + NT * i, key = 2 * (f & 15), c4 = f >> 4;
+            v0reg[i] = v1reg[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (f < V_ITEMS && k0 + key < key_hi) v0reg[i] = KvOps<KV>::ld4(vbase + static_cast<uint64_t>(k0 + key) * HD, c4);
+            if (f < V_ITEMS && k0 + key + 1 < key_hi) v1reg[i] = KvOps<KV>::ld4(vbase + static_cast<uint64_t>(k0 + key + 1) * HD, c4);
+        }
+    };
+    auto stage = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < KI; ++i) {
+            const uint32_t f = tid + NT * i, key = f / (HD / 4), c4 = f % (HD / 4);
+            uint2 hi, lo;
+            attn_split2(kreg[i].x, kreg[i].y, hi.x, lo.x);
+            attn_split2(kreg[i].z, kreg[i].w, hi.y, lo.y);
+            if (f < K_ITEMS) {
+                *reinterpret_cast<uint2*>(sKh + key * KLD + 4 * c4) = hi;
+                if (LOW) *reinterpret_cast<uint2*>(sKl + key * KLD + 4 * c4) = lo;
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < VI; ++i) {
+            const uint32_t f = tid + NT * i, key = 2 * (f & 15), c4 = f >> 4;
+            // slot of key: 16 (key / 16) + 8 h + 4 (blk & 1) + r  with  key % 16 = 8 (blk & 1) + 4 h + r
+            const uint32_t slot = (key & 16) + ((key & 4) << 1) + ((key & 8) >> 1) + (key & 3);
+            const float a[4] = {v0reg[i].x, v0reg[i].y, v0reg[i].z, v0reg[i].w};
+            const float b[4] = {v1reg[i].x, v1reg[i].y, v1reg[i].z, v1reg[i].w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                uint32_t hi, lo;
+                attn_split2(a[e], b[e], hi, lo);
+                if (f < V_ITEMS) {
+                    *reinterpret_cast<uint32_t*>(sVh + (4 * c4 + e) * VTLD + slot) = hi;
+                    if (LOW) *reinterpret_cast<uint32_t*>(sVl + (4 * c4 + e) * VTLD + slot) = lo;
+                }
+            }
+        }
+    };
+
+    if (PREFETCH && key_lo < key_hi) fetch(key_lo);
+    for (uint32_t k0 = key_lo; k0 < key_hi; k0 += 32) {
+        if (!PREFETCH) fetch(k0);
+        stage();
         __syncthreads();
-        // ---- scores, transposed: c[4blk + r] = <K[k0 + 8blk + 4half + r], Q[qidx]>
-        attn_v16f c;
+        if (PREFETCH && k0 + 32 < key_hi) fetch(k0 + 32);
+        // ---- scores, transposed: c[4blk + r] = <K[k0 + 8blk + 4half + r], Q[qidx]>, two chains
+        attn_v16f c, c2;
 #pragma unroll
-        for (int e = 0; e < 16; ++e) c[e] = 0.0f;
+        for (int e = 0; e < 16; ++e) c[e] = c2[e] = 0.0f;
 #pragma unroll
-        for (int s = 0; s < HD / 2; ++s)
-            c = __builtin_amdgcn_mfma_f32_32x32x2f32(sKt[(2 * s + half) * ATTN_PF_LD + col], qreg[s], c, 0, 0, 0);
+        for (int j = 0; j < NJ; ++j) {
+            const uint4 kh = *reinterpret_cast<const uint4*>(sKh + col * KLD + 16 * j + 8 * half);
+            c = attn_mfma(kh, qh[j], c);
+            c2 = attn_mfma(kh, ql[j], c2);
+            if (LOW) {
+                const uint4 kl = *reinterpret_cast<const uint4*>(sKl + col * KLD + 16 * j + 8 * half);
+                c2 = attn_mfma(kl, qh[j], c2);
+            }
+        }
+        // scores in the base-2 domain (scale * log2 e folded into one factor); a tile that every
+        // query of the block sees whole skips the masking
         float mx = -__builtin_inff();
+        if (k0 + 32 <= min(key_hi, first_len + q0)) {
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
-            const uint32_t kg = k0 + 8 * (e >> 2) + 4 * half + (e & 3);
-            const bool ok = q_live && kg < my_len && kg < key_hi;
-            c[e] = ok ? c[e] * scale : -__builtin_inff();
-            mx = fmaxf(mx, c[e]);
+            for (int e = 0; e < 16; ++e) {
+                c[e] = (c[e] + c2[e]) * scale2;
+                mx = fmaxf(mx, c[e]);
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const uint32_t kg = k0 + 8 * (e >> 2) + 4 * half + (e & 3);
+                const bool ok = q_live && kg < my_len && kg < key_hi;
+                c[e] = ok ? (c[e] + c2[e]) * scale2 : -__builtin_inff();
+                mx = fmaxf(mx, c[e]);
+            }
         }
         mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
         const float m_new = fmaxf(m, mx);
         // a query with nothing visible yet keeps m = -inf: weights and correction are then 0 / 1
-        const float corr = m_new == -__builtin_inff() ? 1.0f : cera_expf(m - m_new);
+        const float corr = m_new == -__builtin_inff() ? 1.0f : __builtin_amdgcn_exp2f(m - m_new);
         float ps = 0.0f;
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
-            c[e] = c[e] == -__builtin_inff() ? 0.0f : cera_expf(c[e] - m_new);
+            c[e] = c[e] == -__builtin_inff() ? 0.0f : __builtin_amdgcn_exp2f(c[e] - m_new);
             ps += c[e];
         }
         ps += __shfl_xor(ps, 32, 64);
         l = l * static_cast<double>(corr) + static_cast<double>(ps);
         m = m_new;
-        // ---- the correction factors, re-laid out by output row (query 8blk + 4half + r)
-        if (half == 0) sX[col] = corr;
-        __builtin_amdgcn_wave_barrier();   // sX is this wavefront's own: LDS operations of one wavefront complete in order
+        // ---- the correction factors, re-laid out by output row (query 8blk + 4half + r); once the
+        // running maxima have settled they are all exactly 1
+        if (__builtin_amdgcn_ballot_w64(corr != 1.0f) != 0) {
+            if (half == 0) sX[col] = corr;
+            __builtin_amdgcn_wave_barrier();   // sX is this wavefront's own: LDS operations of one wavefront complete in order
 #pragma unroll
-        for (int blk = 0; blk < 4; ++blk) {
-            const float4 cr = *reinterpret_cast<const float4*>(sX + 8 * blk + 4 * half);
-            const float crv[4] = {cr.x, cr.y, cr.z, cr.w};
+            for (int blk = 0; blk < 4; ++blk) {
+                const float4 cr = *reinterpret_cast<const float4*>(sX + 8 * blk + 4 * half);
+                const float crv[4] = {cr.x, cr.y, cr.z, cr.w};
 #pragma unroll
-            for (int dt = 0; dt < NDT; ++dt)
+                for (int dt = 0; dt < NDT; ++dt)
 #pragma unroll
-                for (int r = 0; r < 4; ++r) acc[dt][4 * blk + r] *= crv[r];
+                    for (int r = 0; r < 4; ++r) acc[dt][4 * blk + r] *= crv[r];
+            }
         }
-        // ---- O += P . V
+        // ---- O += P . V: the weights split like everything else; slot s of step kk is c[8kk + s]
+        uint4 ph[2], pl[2];
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
-            const float* vrow = sV + (8 * (e >> 2) + 4 * half + (e & 3)) * VLD + col;
-#pragma unroll
-            for (int dt = 0; dt < NDT; ++dt)
-                acc[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(c[e], vrow[32 * dt], acc[dt], 0, 0, 0);
+        for (int kk = 0; kk < 2; ++kk) {
+            attn_split2(c[8 * kk + 0], c[8 * kk + 1], ph[kk].x, pl[kk].x);
+            attn_split2(c[8 * kk + 2], c[8 * kk + 3], ph[kk].y, pl[kk].y);
+            attn_split2(c[8 * kk + 4], c[8 * kk + 5], ph[kk].z, pl[kk].z);
+            attn_split2(c[8 * kk + 6], c[8 * kk + 7], ph[kk].w, pl[kk].w);
         }
-        __syncthreads();   // sKt and sV are rewritten by the next tile
+#pragma unroll
+        for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+            for (int dt = 0; dt < NDT; ++dt) {
+                const uint4 vh = *reinterpret_cast<const uint4*>(sVh + (32 * dt + col) * VTLD + 16 * kk + 8 * half);
+                acc[dt] = attn_mfma(ph[kk], vh, acc[dt]);
+                acc[dt] = attn_mfma(pl[kk], vh, acc[dt]);
+                if (LOW) {
+                    const uint4 vl = *reinterpret_cast<const uint4*>(sVl + (32 * dt + col) * VTLD + 16 * kk + 8 * half);
+                    acc[dt] = attn_mfma(ph[kk], vl, acc[dt]);
+                }
+            }
+        __syncthreads();   // the K and V tiles are rewritten by the next tile
     }
 
     // ---- partial out: rows of acc are queries 8blk + 4half + r, columns 32dt + col
@@ -557,7 +669,7 @@ __global__ __launch_bounds__(512) void attn_prefill_partial_kernel(
         }
     if (half == 0 && q_live) {
         float* ml = part_ml + (((static_cast<uint64_t>(qidx) * n_kv + kvh) * n_parts + part) * G + hg) * 2;
-        ml[0] = m;
+        ml[0] = m * 0.69314718055994530942f;   // back to the natural-log domain the merge works in
         ml[1] = static_cast<float>(l);
     }
 }
