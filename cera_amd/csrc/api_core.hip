@@ -560,7 +560,8 @@ cera_hip_status cera_launch_attn(cera_hip_ctx* ctx, const float* q, const void* 
     uint32_t n_parts, part_keys = 0, chunks_per_part = 0;
     uint32_t S = 1;
     if (batch) {
-        part_keys = last_len <= 1024 ? 128u : static_cast<uint32_t>(((last_len + 7) / 8 + 31) / 32 * 32);
+        const uint64_t want = n_queries >= 1024 ? 4 : 8;   // many query blocks fill the chip with fewer parts
+        part_keys = last_len <= 1024 ? 128u : static_cast<uint32_t>(((last_len + want - 1) / want + 31) / 32 * 32);
         n_parts = static_cast<uint32_t>((last_len + part_keys - 1) / part_keys);
     } else {
         // positions per chunk: small chunks while the context is short (one memory round

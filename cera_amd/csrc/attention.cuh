@@ -411,7 +411,9 @@ __global__ __launch_bounds__(256) void attn_decode_partial_kernel(
 // the f16 pair (hi, lo), hi = x truncated to f16 and lo = (x - hi) truncated, so
 // x = hi + lo up to 2^-21 |x|, and a product x.y is the three MFMAs hi.hi + hi.lo + lo.hi
 // (each f16 product is exact in the f32 accumulator; the dropped lo.lo term is below
-// 2^-22 |x.y|).  That keeps the arithmetic class of the reference's f32 dot products
+// 2^-22 |x.y|; the low parts of Q and K are carried times 2^11 and their two cross products
+// collect in an accumulator of their own, so that they stay in f16's normal range and a
+// large Q element cannot magnify a subnormal's absolute rounding).  That keeps the arithmetic class of the reference's f32 dot products
 // (cera/src/backend/cpu.rs:4028-4241) at a fifth of the f32 MFMA's cycles.  A half
 // cache has no low parts and takes two MFMAs per product.
 //
@@ -443,11 +445,18 @@ typedef _Float16 attn_v2h __attribute__((ext_vector_type(2)));
 #define ATTN_PF_KLD(HD) ((HD) + 8)   // halves per LDS row of the K tile: 16-byte reads of 16 rows cover all banks
 #define ATTN_PF_VTLD 40              // halves per LDS row of the transposed V tile (32 keys + 8 pad), same property
 
-// (a, b) -> packed f16 high parts and packed f16 low parts
+// (a, b) -> packed f16 high parts and packed f16 low parts.  SCALED: the low parts times 2^11,
+// which keeps them in the f16 normal range whenever the high part is (an unscaled low part of a
+// value below 1/8 is subnormal, i.e. absolute instead of relative precision: harmless against
+// an operand of ordinary size, not against a very large one).
+#define ATTN_LO_SCALE 2048.0f
+template <bool SCALED>
 __device__ __forceinline__ void attn_split2(float a, float b, uint32_t& hi, uint32_t& lo) {
     const attn_v2h h = __builtin_bit_cast(attn_v2h, __builtin_amdgcn_cvt_pkrtz(a, b));
     hi = __builtin_bit_cast(uint32_t, h);
-    lo = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(a - static_cast<float>(h[0]), b - static_cast<float>(h[1])));
+    float ra = a - static_cast<float>(h[0]), rb = b - static_cast<float>(h[1]);
+    if (SCALED) { ra *= ATTN_LO_SCALE; rb *= ATTN_LO_SCALE; }
+    lo = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(ra, rb));
 }
 __device__ __forceinline__ attn_v16f attn_mfma(const uint4& a, const uint4& b, attn_v16f c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(attn_v8h, a), __builtin_bit_cast(attn_v8h, b), c, 0, 0, 0);
@@ -499,10 +508,10 @@ __global__ __launch_bounds__(64 * G) void attn_prefill_partial_kernel(
 #pragma unroll
         for (int j = 0; j < NJ; ++j) {
             const float4 a = *reinterpret_cast<const float4*>(qp + 16 * j), b = *reinterpret_cast<const float4*>(qp + 16 * j + 4);
-            attn_split2(a.x, a.y, qh[j].x, ql[j].x);
-            attn_split2(a.z, a.w, qh[j].y, ql[j].y);
-            attn_split2(b.x, b.y, qh[j].z, ql[j].z);
-            attn_split2(b.z, b.w, qh[j].w, ql[j].w);
+            attn_split2<true>(a.x, a.y, qh[j].x, ql[j].x);
+            attn_split2<true>(a.z, a.w, qh[j].y, ql[j].y);
+            attn_split2<true>(b.x, b.y, qh[j].z, ql[j].z);
+            attn_split2<true>(b.z, b.w, qh[j].w, ql[j].w);
         }
     }
     attn_v16f acc[NDT];
@@ -539,8 +548,8 @@ __global__ __launch_bounds__(64 * G) void attn_prefill_partial_kernel(
         for (int i = 0; i < KI; ++i) {
             const uint32_t f = tid + NT * i, key = f / (HD / 4), c4 = f % (HD / 4);
             uint2 hi, lo;
-            attn_split2(kreg[i].x, kreg[i].y, hi.x, lo.x);
-            attn_split2(kreg[i].z, kreg[i].w, hi.y, lo.y);
+            attn_split2<true>(kreg[i].x, kreg[i].y, hi.x, lo.x);
+            attn_split2<true>(kreg[i].z, kreg[i].w, hi.y, lo.y);
             if (f < K_ITEMS) {
                 *reinterpret_cast<uint2*>(sKh + key * KLD + 4 * c4) = hi;
                 if (LOW) *reinterpret_cast<uint2*>(sKl + key * KLD + 4 * c4) = lo;
@@ -556,7 +565,7 @@ __global__ __launch_bounds__(64 * G) void attn_prefill_partial_kernel(
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 uint32_t hi, lo;
-                attn_split2(a[e], b[e], hi, lo);
+                attn_split2<false>(a[e], b[e], hi, lo);
                 if (f < V_ITEMS) {
                     *reinterpret_cast<uint32_t*>(sVh + (4 * c4 + e) * VTLD + slot) = hi;
                     if (LOW) *reinterpret_cast<uint32_t*>(sVl + (4 * c4 + e) * VTLD + slot) = lo;
@@ -571,7 +580,8 @@ __global__ __launch_bounds__(64 * G) void attn_prefill_partial_kernel(
         stage();
         __syncthreads();
         if (PREFETCH && k0 + 32 < key_hi) fetch(k0 + 32);
-        // ---- scores, transposed: c[4blk + r] = <K[k0 + 8blk + 4half + r], Q[qidx]>, two chains
+        // ---- scores, transposed: c[4blk + r] = <K[k0 + 8blk + 4half + r], Q[qidx]>; the cross terms
+        // (scaled low parts) collect in c2
         attn_v16f c, c2;
 #pragma unroll
         for (int e = 0; e < 16; ++e) c[e] = c2[e] = 0.0f;
@@ -591,7 +601,7 @@ __global__ __launch_bounds__(64 * G) void attn_prefill_partial_kernel(
         if (k0 + 32 <= min(key_hi, first_len + q0)) {
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
-                c[e] = (c[e] + c2[e]) * scale2;
+                c[e] = fmaf(c2[e], 1.0f / ATTN_LO_SCALE, c[e]) * scale2;
                 mx = fmaxf(mx, c[e]);
             }
         } else {
@@ -599,7 +609,7 @@ __global__ __launch_bounds__(64 * G) void attn_prefill_partial_kernel(
             for (int e = 0; e < 16; ++e) {
                 const uint32_t kg = k0 + 8 * (e >> 2) + 4 * half + (e & 3);
                 const bool ok = q_live && kg < my_len && kg < key_hi;
-                c[e] = ok ? (c[e] + c2[e]) * scale2 : -__builtin_inff();
+                c[e] = ok ? fmaf(c2[e], 1.0f / ATTN_LO_SCALE, c[e]) * scale2 : -__builtin_inff();
                 mx = fmaxf(mx, c[e]);
             }
         }
@@ -635,10 +645,10 @@ __global__ __launch_bounds__(64 * G) void attn_prefill_partial_kernel(
         uint4 ph[2], pl[2];
 #pragma unroll
         for (int kk = 0; kk < 2; ++kk) {
-            attn_split2(c[8 * kk + 0], c[8 * kk + 1], ph[kk].x, pl[kk].x);
-            attn_split2(c[8 * kk + 2], c[8 * kk + 3], ph[kk].y, pl[kk].y);
-            attn_split2(c[8 * kk + 4], c[8 * kk + 5], ph[kk].z, pl[kk].z);
-            attn_split2(c[8 * kk + 6], c[8 * kk + 7], ph[kk].w, pl[kk].w);
+            attn_split2<false>(c[8 * kk + 0], c[8 * kk + 1], ph[kk].x, pl[kk].x);
+            attn_split2<false>(c[8 * kk + 2], c[8 * kk + 3], ph[kk].y, pl[kk].y);
+            attn_split2<false>(c[8 * kk + 4], c[8 * kk + 5], ph[kk].z, pl[kk].z);
+            attn_split2<false>(c[8 * kk + 6], c[8 * kk + 7], ph[kk].w, pl[kk].w);
         }
 #pragma unroll
         for (int kk = 0; kk < 2; ++kk)

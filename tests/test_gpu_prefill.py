@@ -196,6 +196,41 @@ def test_attn_prefill_batch_vs_oracle(hip, orc, nh, nkv, start, n):
     assert np.isfinite(out).all()
 
 
+@pytest.mark.parametrize("case", ["plain", "wide_range", "sink"])
+def test_attn_prefill_split_f16_keeps_f32_accuracy(hip, orc, case):
+    """The batch kernel multiplies on the f16 matrix cores with every operand split into an f16
+    high and low part.  Its error against the f32 reference must stay at f32 level (far inside
+    the 2e-3 bar a plain f16 product would only just meet), also when the operands span many
+    binades and when the weights are one dominant key (an attention sink) plus thousands of
+    keys at 1e-4 of it, where f16 alone would round the small weights coarsely."""
+    nh, nkv, hd, start, n = 8, 2, 128, 3000, 64
+    _say(f"attn_prefill split-f16 accuracy case={case}")
+    r = util.rng(1234)
+    L = start + n
+    q = r.standard_normal((n, nh * hd), dtype=np.float32)
+    k = r.standard_normal((L, nkv * hd), dtype=np.float32)
+    v = r.standard_normal((L, nkv * hd), dtype=np.float32)
+    if case == "wide_range":
+        # per-dimension magnitudes from 2^-12 to 2^6: f16 subnormal low parts and large values
+        mag = np.exp2(r.integers(-12, 7, hd)).astype(np.float32)
+        k *= np.tile(mag, nkv); q /= np.tile(mag, nh); v *= np.tile(mag[::-1], nkv)
+    if case == "sink":
+        # key 0 lines up with every query: one weight of 1 against thousands near exp(-9)
+        k *= 0.05
+        k[0] = 0.0
+        k[0, ::hd] = 60.0          # dim 0 of every KV head
+        q[:, ::hd] = np.abs(q[:, ::hd]) + 2.0
+    scale = 1.0 / np.sqrt(hd)
+    out = hip.attn_prefill(q, k.reshape(-1), v.reshape(-1), nh, nkv, hd, start, n, scale)
+    worst = 0.0
+    for i in (0, 31, 32, n - 1):
+        Li = start + i + 1
+        ref = orc.decode_attention(q[i], k[:Li].reshape(-1), v[:Li].reshape(-1), nh, nkv, hd, scale, Li)
+        worst = max(worst, np.abs(out[i].astype(np.float64) - ref).max() / util.rms(ref))
+    _say(f"  max|err| / rms = {worst:.3e}")
+    assert worst <= 5e-5
+
+
 @pytest.mark.parametrize("kv_f16", [False, True])
 @pytest.mark.parametrize("nh,nkv,start,n", [(32, 8, 0, 200), (8, 2, 300, 40), (4, 4, 1000, 33)])
 def test_attn_prefill_batch_head_dim_64(hip, orc, kv_f16, nh, nkv, start, n):
