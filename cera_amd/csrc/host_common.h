@@ -33,6 +33,10 @@ struct cera_hip_ctx {
     float* attn_acc = nullptr;
     float* attn_ml = nullptr;
     uint64_t attn_acc_bytes = 0, attn_ml_bytes = 0;
+    // two pinned chunks + events: staging for device-to-host copies into pageable memory
+    std::mutex pin_mu;
+    void* pin[2] = {nullptr, nullptr};
+    hipEvent_t pin_ev[2] = {nullptr, nullptr};
 };
 
 void cera_set_global_error(const std::string& s);

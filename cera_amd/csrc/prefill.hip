@@ -358,10 +358,9 @@ static cera_hip_status prefill_chunk(cera_hip_model* m, const uint32_t* tokens, 
             HIP_TRY(ctx, hipGetLastError());
         }
         if (rows == c.vocab)   // no pad rows: one contiguous copy
-            HIP_TRY(ctx, hipMemcpyAsync(all_logits, m->pf_logits, static_cast<size_t>(n) * rows * 4, hipMemcpyDeviceToHost, s));
-        else
-            HIP_TRY(ctx, hipMemcpy2DAsync(all_logits, static_cast<size_t>(c.vocab) * 4, m->pf_logits, rows * 4,
-                                          static_cast<size_t>(c.vocab) * 4, n, hipMemcpyDeviceToHost, s));
+            return cera_hip_download(ctx, all_logits, m->pf_logits, static_cast<uint64_t>(n) * rows * 4);
+        HIP_TRY(ctx, hipMemcpy2DAsync(all_logits, static_cast<size_t>(c.vocab) * 4, m->pf_logits, rows * 4,
+                                      static_cast<size_t>(c.vocab) * 4, n, hipMemcpyDeviceToHost, s));
         HIP_TRY(ctx, hipStreamSynchronize(s));
         return CERA_HIP_OK;
     }
