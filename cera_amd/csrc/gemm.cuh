@@ -37,6 +37,7 @@
 //      scale*sum(a) per 32-block.
 #pragma once
 #include "common.cuh"
+#include "quantize.cuh"
 
 #define GEMM_BM 128
 #define GEMM_BN 64
@@ -72,6 +73,11 @@ struct GemmArgs {
     float* out2;
     uint32_t m2, tiles1;
     uint64_t ld_n2;
+    // SwiGLU form of the kernel (w = gate, w2 = up, both m x k): nothing goes to out; the Q8_0
+    // quantization of silu(gate.x) * (up.x) goes to hq [n][m], hs and hbsum [n][m/32]
+    int8_t* hq;
+    float* hs;
+    float* hbsum;
 };
 
 // ---- per-type staging of one 128-element K tile of one row -------------------
@@ -216,7 +222,12 @@ struct GemmQ8_0 {
     }
 };
 
-template <class T>
+// SWIGLU: the workgroup's 128 staged rows are 64 rows of the gate matrix and the same 64 rows of
+// the up matrix, and a wavefront's two row tiles are 32 gate rows and the same 32 up rows: both
+// factors of an output of the FFN's first half then sit in the same lane and register index, a
+// 32-row Q8_0 block of one token in the two lanes of a column, and the activation of the down
+// projection is quantized straight from the accumulators.
+template <class T, bool SWIGLU = false>
 static __global__ __launch_bounds__(256, T::WAVES_PER_SIMD) void gemm_kernel(GemmArgs p) {
     constexpr int NB = GEMM_KT / 32;  // 32-blocks per tile
     __shared__ __attribute__((aligned(16))) int8_t sA[GEMM_BM * GEMM_LDA];
@@ -228,12 +239,18 @@ static __global__ __launch_bounds__(256, T::WAVES_PER_SIMD) void gemm_kernel(Gem
 
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const uint32_t wm = wave >> 1, wn = wave & 1;           // wavefront position in the 2 x 2 grid
-    const bool second = p.w2 != nullptr && blockIdx.y >= p.tiles1;
+    const bool second = !SWIGLU && p.w2 != nullptr && blockIdx.y >= p.tiles1;
     const uint8_t* const wmat = second ? p.w2 : p.w;
     float* const omat = second ? p.out2 : p.out;
     const uint32_t mrows = second ? p.m2 : p.m;
     const uint64_t ldn = second ? p.ld_n2 : p.ld_n;
-    const uint32_t m0 = (second ? blockIdx.y - p.tiles1 : blockIdx.y) * GEMM_BM, n0 = blockIdx.x * GEMM_BN;
+    const uint32_t m0 = (second ? blockIdx.y - p.tiles1 : blockIdx.y) * (SWIGLU ? GEMM_BM / 2 : GEMM_BM), n0 = blockIdx.x * GEMM_BN;
+    // staged row r of the tile -> matrix and row; row tile t of wavefront row wm -> first staged row
+    auto row_ptr = [&](uint32_t r) __attribute__((always_inline)) {
+        if (SWIGLU) return (r < GEMM_BM / 2 ? p.w : p.w2) + static_cast<uint64_t>(min(m0 + (r & (GEMM_BM / 2 - 1)), mrows - 1)) * p.row_bytes;
+        return wmat + static_cast<uint64_t>(min(m0 + r, mrows - 1)) * p.row_bytes;
+    };
+    const uint32_t arow0 = SWIGLU ? wm * 32 : wm * 64, arow_step = SWIGLU ? GEMM_BM / 2 : 32;
     const uint32_t col = lane & 31, half = lane >> 5;
     const uint32_t nb32 = p.k / 32;
 
@@ -254,10 +271,10 @@ static __global__ __launch_bounds__(256, T::WAVES_PER_SIMD) void gemm_kernel(Gem
     for (int i = 0; i < AI; ++i) {
         const uint32_t it = tid + 256 * i, r = it / T::WORDS;
         a_w[i] = it % T::WORDS;
-        a_src[i] = wmat + static_cast<uint64_t>(min(m0 + r, mrows - 1)) * p.row_bytes;
+        a_src[i] = row_ptr(r);
         a_dst[i] = sA + r * GEMM_LDA;
     }
-    const uint8_t* s_src = wmat + static_cast<uint64_t>(min(m0 + (tid & (GEMM_BM - 1)), mrows - 1)) * p.row_bytes;
+    const uint8_t* s_src = row_ptr(tid & (GEMM_BM - 1));
     const int8_t* b_src[2];
     int8_t* b_dst[2];
     bool b_live[2];
@@ -320,12 +337,12 @@ static __global__ __launch_bounds__(256, T::WAVES_PER_SIMD) void gemm_kernel(Gem
                 const float xsl = sCS[(2 * pr + half) * GEMM_BN + wn * 32 + col];
 #pragma unroll
                 for (int t = 0; t < 2; ++t) {
-                    const float rsl = sRS[(2 * pr + half) * GEMM_BM + wm * 64 + t * 32 + col];
+                    const float rsl = sRS[(2 * pr + half) * GEMM_BM + arow0 + t * arow_step + col];
                     v32f z32;
 #pragma unroll
                     for (int e = 0; e < 32; ++e) z32[e] = 0.0f;
                     const v32f sc = __builtin_amdgcn_mfma_f32_32x32x1f32(rsl, xsl, z32, 0, 0, 0);
-                    const int8_t* aRow = sA + (wm * 64 + t * 32 + col) * GEMM_LDA;
+                    const int8_t* aRow = sA + (arow0 + t * arow_step + col) * GEMM_LDA;
 #pragma unroll
                     for (int jb = 0; jb < 2; ++jb) {
                         const v4i af = *reinterpret_cast<const v4i*>(aRow + (2 * pr + jb) * 32 + half * 16);
@@ -341,7 +358,7 @@ static __global__ __launch_bounds__(256, T::WAVES_PER_SIMD) void gemm_kernel(Gem
                     const float xm = sCM[(2 * pr + half) * GEMM_BN + wn * 32 + col];
 #pragma unroll
                     for (int t = 0; t < 2; ++t) {
-                        const float rm = -sRM[(2 * pr + half) * GEMM_BM + wm * 64 + t * 32 + col];
+                        const float rm = -sRM[(2 * pr + half) * GEMM_BM + arow0 + t * arow_step + col];
                         acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(rm, xm, acc[t], 0, 0, 0);
                     }
                 }
@@ -351,6 +368,47 @@ static __global__ __launch_bounds__(256, T::WAVES_PER_SIMD) void gemm_kernel(Gem
     }
     // ---- store: lane holds token n0 + wn*32 + col, 32 rows
     const uint32_t tok = n0 + wn * 32 + col;
+    if (SWIGLU) {
+        // h = silu(gate) * up (cera/src/backend/cpu.rs:2570-2575), then the Q8_0 block of this token's
+        // rows m0 + 32 wm .. +31 (cpu.rs:942-958): this lane holds 16 of them, lane ^ 32 the others
+        float h[16];
+        float amax = 0.0f;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            const float g = acc[0][e];
+            h[e] = __fmul_rn(__fdiv_rn(g, __fadd_rn(1.0f, cera_expf(-g))), acc[1][e]);
+            amax = fmaxf(amax, fabsf(h[e]));   // fmaxf drops a NaN operand, as f32::max does
+        }
+        amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
+        const float d = __fdiv_rn(amax, 127.0f), r = __fdiv_rn(1.0f, d);
+        const float id = (d != 0.0f && fabsf(r) != __builtin_inff() && r == r) ? r : 0.0f;
+        const float scale = h2f(f2h(d));
+        uint32_t packed[4];
+        int sum = 0;
+#pragma unroll
+        for (int blk = 0; blk < 4; ++blk) {
+            packed[blk] = 0;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int v = q8_round(h[4 * blk + q], id);
+                sum += v;
+                packed[blk] |= (static_cast<uint32_t>(v) & 0xFF) << (8 * q);
+            }
+        }
+        sum += __shfl_xor(sum, 32, 64);
+        const uint32_t row0 = m0 + wm * 32;   // m % 32 == 0: the block is whole or absent
+        if (tok < p.n && row0 < mrows) {
+#pragma unroll
+            for (int blk = 0; blk < 4; ++blk)
+                *reinterpret_cast<uint32_t*>(p.hq + static_cast<uint64_t>(tok) * mrows + row0 + 8 * blk + 4 * half) = packed[blk];
+            if (half == 0) {
+                const uint64_t b = static_cast<uint64_t>(tok) * (mrows / 32) + row0 / 32;
+                p.hs[b] = scale;
+                p.hbsum[b] = scale * static_cast<float>(sum);
+            }
+        }
+        return;
+    }
     if (tok < p.n) {
 #pragma unroll
         for (int t = 0; t < 2; ++t)

@@ -105,6 +105,36 @@ cera_hip_status cera_launch_gemm(cera_hip_ctx* ctx, const cera_hip_dtensor* w, c
     return CERA_HIP_OK;
 }
 
+// First half of the FFN in one launch: hq/hs/hbsum [n][m] = Q8_0(silu(gate.B) * (up.B)), the
+// activation of the down projection, quantized in the GEMM's epilogue.  *fused = false (nothing
+// launched) when the pair is not two int8-GEMM matrices of one shape or when the launch would
+// need a K split to fill the chip; the caller then takes the GEMM pair and the SwiGLU kernel.
+cera_hip_status cera_launch_gemm_swiglu(cera_hip_ctx* ctx, const cera_hip_dtensor* gate, const cera_hip_dtensor* up,
+                                        const float* bs, const int8_t* bq, const float* bsum, uint32_t n, int8_t* hq,
+                                        float* hs, float* hbsum, bool* fused) {
+    *fused = false;
+    if (!cera_gemm_supports(gate->dtype, gate->k) || gate->dtype == CERA_HIP_Q6_K || up->dtype != gate->dtype ||
+        up->k != gate->k || up->m != gate->m || up->row_bytes != gate->row_bytes || gate->m % 32 || n == 0)
+        return CERA_HIP_OK;
+    GemmArgs a{};
+    a.w = gate->dev; a.w2 = up->dev; a.bq = bq; a.bs = bs; a.bsum = bsum;
+    a.m = static_cast<uint32_t>(gate->m); a.n = n; a.k = static_cast<uint32_t>(gate->k);
+    a.row_bytes = static_cast<uint32_t>(gate->row_bytes);
+    a.k_chunk = a.k;
+    a.hq = hq; a.hs = hs; a.hbsum = hbsum;
+    const dim3 grid((n + GEMM_BN - 1) / GEMM_BN, (a.m + GEMM_BM / 2 - 1) / (GEMM_BM / 2));
+    if (grid.x * grid.y < 2 * ctx->n_cu) return CERA_HIP_OK;
+    switch (gate->dtype) {
+        case CERA_HIP_Q4_K: hipLaunchKernelGGL((gemm_kernel<GemmQ4K, true>), grid, dim3(256), 0, ctx->stream, a); break;
+        case CERA_HIP_Q4_0: hipLaunchKernelGGL((gemm_kernel<GemmQ4_0, true>), grid, dim3(256), 0, ctx->stream, a); break;
+        case CERA_HIP_Q4_1: hipLaunchKernelGGL((gemm_kernel<GemmQ4_1, true>), grid, dim3(256), 0, ctx->stream, a); break;
+        default: hipLaunchKernelGGL((gemm_kernel<GemmQ8_0, true>), grid, dim3(256), 0, ctx->stream, a); break;
+    }
+    HIP_TRY(ctx, hipGetLastError());
+    *fused = true;
+    return CERA_HIP_OK;
+}
+
 // quantize n rows of k floats: quants [n][k], scales and bsum [n][k/32]
 static cera_hip_status quantize_rows(cera_hip_ctx* ctx, const float* x, uint64_t n, uint64_t k, float* scales,
                                      int8_t* quants, float* bsum) {
@@ -183,6 +213,57 @@ extern "C" cera_hip_status cera_hip_gemm_pair(cera_hip_ctx* ctx, const cera_hip_
     st = run();
     cera_hip_tensor_free(ctx, wa);
     cera_hip_tensor_free(ctx, wb);
+    return st;
+}
+
+extern "C" cera_hip_status cera_hip_gemm_swiglu(cera_hip_ctx* ctx, const cera_hip_tensor* tg, const cera_hip_tensor* tu,
+                                                const float* x, uint64_t n, int8_t* quants, float* scales, int* fused_out) {
+    if (!ctx || !tg || !tu || !x || !quants || !scales) return CERA_HIP_ERR_ARGUMENT;
+    if (n == 0 || n > 0x7FFFFFFFull) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "gemm_swiglu: bad n");
+    cera_hip_dtensor *wg = nullptr, *wu = nullptr;
+    CERA_TRY(cera_hip_tensor_upload(ctx, tg, &wg));
+    cera_hip_status st = cera_hip_tensor_upload(ctx, tu, &wu);
+    if (st != CERA_HIP_OK) { cera_hip_tensor_free(ctx, wg); return st; }
+    auto run = [&]() -> cera_hip_status {
+        if (!cera_gemm_supports(wg->dtype, wg->k) || wg->dtype != wu->dtype || wg->k != wu->k || wg->m != wu->m || wg->m % 32)
+            return cera_fail(ctx, CERA_HIP_ERR_UNSUPPORTED_DTYPE,
+                             "gemm_swiglu: gate and up must share a type with an int8 GEMM, k and m (a multiple of 32)");
+        const uint64_t k = wg->k, mm = wg->m;
+        void *dx, *ds, *dq, *db, *dg, *du, *hq, *hs, *hb;
+        CERA_TRY(cera_scratch(ctx, 0, n * k * 4, &dx));
+        CERA_TRY(cera_scratch(ctx, 1, n * (k / 32) * 4, &ds));
+        CERA_TRY(cera_scratch(ctx, 2, n * k, &dq));
+        CERA_TRY(cera_scratch(ctx, 7, n * (k / 32) * 4, &db));
+        CERA_TRY(cera_scratch(ctx, 3, n * mm * 4, &dg));
+        CERA_TRY(cera_scratch(ctx, 4, n * mm * 4, &du));
+        CERA_TRY(cera_scratch(ctx, 5, n * mm, &hq));
+        CERA_TRY(cera_scratch(ctx, 6, n * (mm / 32) * 4, &hs));
+        CERA_TRY(cera_scratch(ctx, 8, n * (mm / 32) * 4, &hb));
+        CERA_TRY(cera_hip_upload(ctx, dx, x, n * k * 4));
+        CERA_TRY(quantize_rows(ctx, static_cast<float*>(dx), n, k, static_cast<float*>(ds), static_cast<int8_t*>(dq),
+                               static_cast<float*>(db)));
+        bool fused = false;
+        CERA_TRY(cera_launch_gemm_swiglu(ctx, wg, wu, static_cast<float*>(ds), static_cast<int8_t*>(dq), static_cast<float*>(db),
+                                         static_cast<uint32_t>(n), static_cast<int8_t*>(hq), static_cast<float*>(hs),
+                                         static_cast<float*>(hb), &fused));
+        if (!fused) {   // the forward pass's other route: the two GEMMs, then the SwiGLU + quantize kernel
+            CERA_TRY(cera_launch_gemm(ctx, wg, static_cast<float*>(ds), static_cast<int8_t*>(dq), static_cast<float*>(db),
+                                      static_cast<uint32_t>(n), static_cast<float*>(dg), 1, mm, nullptr, 1.0f));
+            CERA_TRY(cera_launch_gemm(ctx, wu, static_cast<float*>(ds), static_cast<int8_t*>(dq), static_cast<float*>(db),
+                                      static_cast<uint32_t>(n), static_cast<float*>(du), 1, mm, nullptr, 1.0f));
+            const uint64_t tot = n * mm;
+            hipLaunchKernelGGL((silu_mul_kernel<true>), dim3(static_cast<uint32_t>((tot / 4 + 255) / 256)), dim3(256), 0,
+                               ctx->stream, static_cast<float*>(dg), static_cast<float*>(du), tot, static_cast<float*>(nullptr),
+                               static_cast<float*>(hs), static_cast<int8_t*>(hq), static_cast<float*>(hb));
+            HIP_TRY(ctx, hipGetLastError());
+        }
+        if (fused_out) *fused_out = fused ? 1 : 0;
+        CERA_TRY(cera_hip_download(ctx, quants, hq, n * mm));
+        return cera_hip_download(ctx, scales, hs, n * (mm / 32) * 4);
+    };
+    st = run();
+    cera_hip_tensor_free(ctx, wg);
+    cera_hip_tensor_free(ctx, wu);
     return st;
 }
 
@@ -324,12 +405,32 @@ static cera_hip_status prefill_chunk(cera_hip_model* m, const uint32_t* tokens, 
         CERA_TRY(gemm(L.o, m->pf_hidden, m->pf_hidden));
 
         CERA_TRY(norm_rows(m->pf_hidden, L.ffn_norm, m->pf_normed));
-        CERA_TRY(gemm2(L.gate, m->pf_gate, L.up, m->pf_up));
-        const uint64_t tot = static_cast<uint64_t>(n) * c.ffn;
-        hipLaunchKernelGGL((silu_mul_kernel<true>), dim3(static_cast<uint32_t>((tot / 4 + 255) / 256)), dim3(256), 0, s,
-                           m->pf_gate, m->pf_up, tot, m->pf_gate, m->pf_xs, m->pf_xq, m->pf_bsum);
-        HIP_TRY(ctx, hipGetLastError());
-        staged = false;   // ... and so did the SwiGLU
+        // gate, up, SwiGLU and the quantization for the down projection in one launch where the
+        // batch fills the chip; the quantized activations then lie in the (otherwise unused) gate
+        // and up buffers, since the launch still reads its own input from pf_xq
+        bool fused = false;
+        int8_t* const hq = reinterpret_cast<int8_t*>(m->pf_gate);
+        float *const hs = m->pf_up, *const hb = m->pf_up + static_cast<uint64_t>(n) * (c.ffn / 32);
+        if (n > PREFILL_SMALL_BATCH)
+            CERA_TRY(cera_launch_gemm_swiglu(ctx, L.gate, L.up, m->pf_xs, m->pf_xq, m->pf_bsum, n, hq, hs, hb, &fused));
+        staged = false;   // the down projection's activations are new either way
+        if (fused && cera_gemm_supports(L.down->dtype, L.down->k)) {
+            CERA_TRY(cera_launch_gemm(ctx, L.down, hs, hq, hb, n, m->pf_hidden, 1, L.down->m, m->pf_hidden, c.residual_scale,
+                                      nullptr, nullptr, 0, nullptr, m->pf_xh, &staged));
+            staged = false;   // pf_xh now mirrors hq, not pf_xq
+            continue;
+        }
+        if (fused) {   // a down projection without a GEMM reads pf_xq: move the quantized activations there
+            HIP_TRY(ctx, hipMemcpyAsync(m->pf_xq, hq, static_cast<uint64_t>(n) * c.ffn, hipMemcpyDeviceToDevice, s));
+            HIP_TRY(ctx, hipMemcpyAsync(m->pf_xs, hs, static_cast<uint64_t>(n) * (c.ffn / 32) * 4, hipMemcpyDeviceToDevice, s));
+            HIP_TRY(ctx, hipMemcpyAsync(m->pf_bsum, hb, static_cast<uint64_t>(n) * (c.ffn / 32) * 4, hipMemcpyDeviceToDevice, s));
+        } else {
+            CERA_TRY(gemm2(L.gate, m->pf_gate, L.up, m->pf_up));
+            const uint64_t tot = static_cast<uint64_t>(n) * c.ffn;
+            hipLaunchKernelGGL((silu_mul_kernel<true>), dim3(static_cast<uint32_t>((tot / 4 + 255) / 256)), dim3(256), 0, s,
+                               m->pf_gate, m->pf_up, tot, m->pf_gate, m->pf_xs, m->pf_xq, m->pf_bsum);
+            HIP_TRY(ctx, hipGetLastError());
+        }
         CERA_TRY(gemm(L.down, m->pf_hidden, m->pf_hidden));
     }
     m->seq_len = start_pos + n;

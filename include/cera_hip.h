@@ -181,6 +181,17 @@ CERA_HIP_API cera_hip_status cera_hip_gemm(cera_hip_ctx*, const cera_hip_tensor*
 CERA_HIP_API cera_hip_status cera_hip_gemm_pair(cera_hip_ctx*, const cera_hip_tensor* a, const cera_hip_tensor* b,
                                                 const float* x, uint64_t n, float* out_a, float* out_b);
 
+/* The first half of the FFN of the batched forward pass in one launch (LlamaModel::
+ * forward_prefill_batched, cera/src/model/llama.rs:738-1523: gemm_preq on ffn_gate and ffn_up,
+ * cpu::silu_mul_inplace, cera/src/backend/cpu.rs:2570-2575, then quantize_columns for the down
+ * projection, cera/src/model/transformer.rs:865-946): quants[n][m] / scales[n][m/32] =
+ * Q8_0(silu(gate.x) * (up.x)) per token row, quantized in the GEMM's epilogue.  gate and up must
+ * share a type with an int8 GEMM (not Q6_K), k and m, m a multiple of 32.  Small batches, which
+ * need a K split to fill the chip, take the two GEMMs and the SwiGLU kernel instead (*fused = 0,
+ * nullable); both routes give identical bytes. */
+CERA_HIP_API cera_hip_status cera_hip_gemm_swiglu(cera_hip_ctx*, const cera_hip_tensor* gate, const cera_hip_tensor* up,
+                                                  const float* x, uint64_t n, int8_t* quants, float* scales, int* fused);
+
 /* transformer::decode_attention (cera/src/model/transformer.rs:1249-1305) with
  * cpu::attn_scores / softmax_inplace / attn_values (cera/src/backend/cpu.rs:
  * 3222-3363, 2617-2633).  q f32[n_heads*head_dim]; k, v f32 time-major

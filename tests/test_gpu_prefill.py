@@ -104,6 +104,27 @@ def test_gemm_pair_matches_single_launches(hip, orc, dtype, ma, mb, n, k):
     assert np.abs(ob[:, rows].T.astype(np.float64) - ref).max() <= GEMM_TOL * util.rms(ref)
 
 
+@pytest.mark.parametrize("dtype", [Q4_K, Q4_0, Q4_1, Q8_0])
+@pytest.mark.parametrize("m,k,n,want_fused", [(2048, 512, 1040, True), (1056, 256, 2000, True), (512, 256, 70, False)])
+def test_gemm_swiglu_epilogue_matches_separate_kernels(hip, orc, dtype, m, k, n, want_fused):
+    """gate | up | SwiGLU | Q8_0 in one launch: the quants and scales must be, byte for byte, the
+    oracle's quantization of the oracle's SwiGLU of the two GEMM outputs the pair launch gives
+    (silu_mul_inplace cpu.rs:2570-2575, quantize_columns transformer.rs:865-946).  Row counts
+    that are not a multiple of the 64-row tile, ragged token tiles, and a batch too small to
+    fill the chip (which takes the separate kernels) are covered."""
+    _say(f"gemm_swiglu {util.NAMES[dtype]} m={m} k={k} n={n}")
+    wg, _ = util.make_weights(dtype, m, k, seed=41)
+    wu, _ = util.make_weights(dtype, m, k, seed=42)
+    x = util.rng(m + 3 * n).standard_normal((n, k)).astype(np.float32)
+    q, sc, fused = hip.gemm_swiglu(dtype, wg, wu, m, x, n, k)
+    assert fused == want_fused
+    g, u = hip.gemm_pair(dtype, wg, m, dtype, wu, m, x, n, k)
+    h = orc.silu_mul(g.reshape(-1), u.reshape(-1))
+    ref_s, ref_q = orc.quantize_q8_0(h)
+    assert np.array_equal(q.reshape(-1), ref_q)
+    assert np.array_equal(sc.reshape(-1).view(np.uint32), ref_s.view(np.uint32))
+
+
 def test_gemm_pair_refuses_mixed_types(hip):
     with pytest.raises(hip_api.HipError) as e:
         hip.gemm_pair(Q4_K, np.zeros(144 * 4, np.uint8), 4, Q6_K, np.zeros(210 * 4, np.uint8), 4,
