@@ -107,9 +107,9 @@ def build_backend(verbose: bool = False) -> Path:
     b = PKG / "backend"
     gguf = str(PKG / "host" / "gguf.cpp")  # C++ classes are not exported by the host library: compile them in
     cmds = [
-        [*common, "-shared", str(b / "hip_llama.cpp"), str(b / "hip_llama_capi.cpp"), str(b / "spec.cpp"), gguf, "-o", str(LLAMA_LIB),
+        [*common, "-shared", str(b / "hip_llama.cpp"), str(b / "hip_llama_capi.cpp"), gguf, "-o", str(LLAMA_LIB),
          *link],
-        [*common, str(b / "cli.cpp"), str(b / "hip_llama.cpp"), str(b / "spec.cpp"), gguf, "-o", str(CLI_BIN), *link],
+        [*common, str(b / "cli.cpp"), str(b / "hip_llama.cpp"), gguf, "-o", str(CLI_BIN), *link],
     ]
     for cmd in cmds:
         r = subprocess.run(cmd, capture_output=True, text=True)

@@ -133,6 +133,9 @@ public:
     const ModelConfig& config() const override { return config_; }
     uint64_t gpu_memory_bytes() const override;
 
+    // verification hook: run every forward on the reference-order kernels (bit-identical to the
+    // CPU AVX2 path, many times slower); only with an empty cache
+    void set_reference_order(bool on);
     RopeType rope_type() const { return rope_type_; }
     std::string device_name() const;
 

@@ -1,7 +1,6 @@
 #include "hip_llama_capi.h"
 
 #include <algorithm>
-#include "spec.h"
 
 #include <chrono>
 #include <cmath>
@@ -34,6 +33,11 @@ int guarded(cera_llama* h, F&& f) {
         h->err = "unknown error";
     }
     return -1;
+}
+// The handle carries one InferenceState for the caller's convenience.  A call at position 0 is a
+// caller arriving with a new state (every generate() in the reference makes one): start over.
+void fresh_at(cera_llama* h, uint64_t pos) {
+    if (pos == 0) h->state = cera::InferenceState{};
 }
 double now_s() {
     return std::chrono::duration<double>(std::chrono::steady_clock::now().time_since_epoch()).count();
@@ -87,15 +91,20 @@ uint64_t cera_llama_gpu_memory_bytes(const cera_llama* h) { return h->model->gpu
 
 int cera_llama_forward(cera_llama* h, uint32_t token, uint64_t pos, float* logits) {
     return guarded(h, [&] {
+        fresh_at(h, pos);
         std::vector<float> l = h->model->forward(&token, 1, pos, h->state);
         std::memcpy(logits, l.data(), l.size() * sizeof(float));
     });
 }
 int cera_llama_forward_greedy(cera_llama* h, uint32_t token, uint64_t pos, uint32_t* next) {
-    return guarded(h, [&] { *next = h->model->forward_greedy(&token, 1, pos, h->state); });
+    return guarded(h, [&] {
+        fresh_at(h, pos);
+        *next = h->model->forward_greedy(&token, 1, pos, h->state);
+    });
 }
 int cera_llama_forward_prefill(cera_llama* h, const uint32_t* tokens, uint64_t n, uint64_t start_pos, float* logits) {
     return guarded(h, [&] {
+        fresh_at(h, start_pos);
         std::vector<float> l = h->model->forward_prefill(tokens, n, start_pos, h->state);
         std::memcpy(logits, l.data(), l.size() * sizeof(float));
     });
@@ -103,6 +112,7 @@ int cera_llama_forward_prefill(cera_llama* h, const uint32_t* tokens, uint64_t n
 int cera_llama_forward_prefill_logits_all(cera_llama* h, const uint32_t* tokens, uint64_t n, uint64_t start_pos,
                                           float* logits) {
     return guarded(h, [&] {
+        fresh_at(h, start_pos);
         std::vector<float> l = h->model->forward_prefill_logits_all(tokens, n, start_pos, h->state);
         std::memcpy(logits, l.data(), l.size() * sizeof(float));
     });
@@ -110,6 +120,7 @@ int cera_llama_forward_prefill_logits_all(cera_llama* h, const uint32_t* tokens,
 int cera_llama_forward_prefill_chunked(cera_llama* h, const uint32_t* tokens, uint64_t n, uint64_t start_pos,
                                        uint64_t ubatch, uint64_t* consumed, float* logits) {
     return guarded(h, [&] {
+        fresh_at(h, start_pos);
         auto r = h->model->forward_prefill_chunked(tokens, n, start_pos, h->state, ubatch, h->cancel);
         if (consumed) *consumed = r.first;
         if (r.second && logits) std::memcpy(logits, r.second->data(), r.second->size() * sizeof(float));
@@ -165,8 +176,9 @@ int cera_llama_generate_greedy(cera_llama* h, const uint32_t* prompt, uint64_t n
     return guarded(h, [&] {
         if (!n_prompt || !n_new) throw cera::BackendError("generate_greedy needs a prompt and n_new > 0");
         std::atomic<bool> never{false};
+        h->state = cera::InferenceState{};   // a generation starts with a new state, as Session::generate does
         double t0 = now_s();
-        auto r = h->model->forward_prefill_chunked(prompt, n_prompt, h->state.seq_len, h->state, ubatch, never);
+        auto r = h->model->forward_prefill_chunked(prompt, n_prompt, 0, h->state, ubatch, never);
         const std::vector<float>& l = *r.second;
         size_t best = 0;
         float bv = -INFINITY;
@@ -181,28 +193,11 @@ int cera_llama_generate_greedy(cera_llama* h, const uint32_t* prompt, uint64_t n
     });
 }
 
-uint64_t cera_spec_prompt_lookup_draft(const uint32_t* tokens, uint64_t n, uint64_t ngram, uint64_t k, uint32_t* out,
-                                       uint64_t cap) {
-    if ((!tokens && n) || (!out && cap)) return 0;
-    const std::vector<uint32_t> d = cera::prompt_lookup_draft(tokens, n, ngram, k);
-    const uint64_t m = std::min<uint64_t>(d.size(), cap);
-    std::copy(d.begin(), d.begin() + m, out);
-    return m;
-}
-
-int cera_llama_generate_spec(cera_llama* h, const uint32_t* prompt, uint64_t n_prompt, uint64_t max_new, const uint32_t* eos,
-                             uint64_t n_eos, uint64_t ngram, uint64_t k, uint32_t* out, uint64_t* n_out, uint64_t stats[3],
-                             double* seconds) {
+int cera_llama_set_reference_order(cera_llama* h, int on) {
     return guarded(h, [&] {
-        if (!out || !n_out) throw cera::BackendError("generate_spec: null output");
-        const std::vector<uint32_t> p(prompt, prompt + n_prompt), e(eos, eos + (eos ? n_eos : 0));
-        cera::SpecStats st;
-        const double t0 = now_s();
-        const std::vector<uint32_t> toks = cera::greedy_generate_spec(*h->model, h->state, p, max_new, e, ngram, k, &st);
-        if (seconds) *seconds = now_s() - t0;
-        std::copy(toks.begin(), toks.end(), out);
-        *n_out = toks.size();
-        if (stats) { stats[0] = st.drafted; stats[1] = st.accepted; stats[2] = st.rounds; }
+        auto* hm = dynamic_cast<cera::HipLlamaModel*>(h->model.get());
+        if (!hm) throw cera::BackendError("set_reference_order: not a hip model");
+        hm->set_reference_order(on != 0);
     });
 }
 

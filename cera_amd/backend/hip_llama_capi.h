@@ -64,15 +64,11 @@ CERA_LLAMA_API int cera_llama_generate_greedy(cera_llama*, const uint32_t* promp
                                               uint64_t ubatch, uint32_t* out_tokens, double* prefill_s,
                                               double* decode_s);
 
-/* cera/src/spec.rs: prompt-lookup draft (model-free; returns the draft length, at most k and cap)
- * and the greedy speculative driver.  generate_spec resets nothing: the session must be fresh
- * (seq_len 0).  out receives at most max_new tokens, *n_out how many; stats = {drafted,
- * accepted, rounds}. */
-CERA_LLAMA_API uint64_t cera_spec_prompt_lookup_draft(const uint32_t* tokens, uint64_t n, uint64_t ngram, uint64_t k,
-                                                      uint32_t* out, uint64_t cap);
-CERA_LLAMA_API int cera_llama_generate_spec(cera_llama*, const uint32_t* prompt, uint64_t n_prompt, uint64_t max_new,
-                                            const uint32_t* eos, uint64_t n_eos, uint64_t ngram, uint64_t k,
-                                            uint32_t* out, uint64_t* n_out, uint64_t stats[3], double* seconds);
+/* Verification hook (no counterpart in the trait): switches the model to the reference-order
+ * route of cera_hip_set_reference_order (logits bit-identical to the CPU AVX2 path, many times
+ * slower); the session must be empty. */
+CERA_LLAMA_API int cera_llama_set_reference_order(cera_llama*, int on);
+
 #ifdef __cplusplus
 }
 #endif

@@ -670,11 +670,13 @@ extern "C" {
 
 cera_hip_status cera_hip_quantize_q8_0_dev(cera_hip_ctx* ctx, const float* x, uint64_t k, float* scales, int8_t* quants) {
     if (!ctx || !x || !scales || !quants) return CERA_HIP_ERR_ARGUMENT;
+    std::lock_guard<std::recursive_mutex> op_lk(ctx->op_mu);
     return cera_launch_quantize(ctx, x, k, scales, quants);
 }
 
 cera_hip_status cera_hip_quantize_q8_0(cera_hip_ctx* ctx, const float* x, uint64_t k, float* scales, int8_t* quants) {
     if (!ctx || !x || !scales || !quants) return CERA_HIP_ERR_ARGUMENT;
+    std::lock_guard<std::recursive_mutex> op_lk(ctx->op_mu);
     if (k == 0 || k % 32) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "quantize_q8_0: k must be a positive multiple of 32");
     void *dx, *ds, *dq;
     CERA_TRY(cera_scratch(ctx, 0, k * 4, &dx));
@@ -689,11 +691,13 @@ cera_hip_status cera_hip_quantize_q8_0(cera_hip_ctx* ctx, const float* x, uint64
 
 cera_hip_status cera_hip_gemv_q8_dev(cera_hip_ctx* ctx, const cera_hip_dtensor* w, const float* xs, const int8_t* xq, float* y) {
     if (!ctx || !w || !xs || !xq || !y) return CERA_HIP_ERR_ARGUMENT;
+    std::lock_guard<std::recursive_mutex> op_lk(ctx->op_mu);
     return cera_launch_gemv(ctx, w, nullptr, xs, xq, y, nullptr, CERA_EPI_STORE);
 }
 
 cera_hip_status cera_hip_gemv_seq_dev(cera_hip_ctx* ctx, const cera_hip_gemv_op* ops, uint32_t n) {
     if (!ctx || (!ops && n)) return CERA_HIP_ERR_ARGUMENT;
+    std::lock_guard<std::recursive_mutex> op_lk(ctx->op_mu);
     for (uint32_t i = 0; i < n; ++i) {
         if (!ops[i].w || !ops[i].xs || !ops[i].xq || !ops[i].y) return cera_fail(ctx, CERA_HIP_ERR_ARGUMENT, "gemv_seq: null field in op " + std::to_string(i));
         CERA_TRY(cera_launch_gemv(ctx, ops[i].w, ops[i].w2, ops[i].xs, ops[i].xq, ops[i].y, nullptr,
@@ -705,6 +709,7 @@ cera_hip_status cera_hip_gemv_seq_dev(cera_hip_ctx* ctx, const cera_hip_gemv_op*
 cera_hip_status cera_hip_gemv(cera_hip_ctx* ctx, const cera_hip_tensor* t, const float* x, float* y,
                               int32_t* dbg_dots, int32_t* dbg_asums) {
     if (!ctx || !x || !y) return CERA_HIP_ERR_ARGUMENT;
+    std::lock_guard<std::recursive_mutex> op_lk(ctx->op_mu);
     cera_hip_dtensor* w = nullptr;
     CERA_TRY(cera_hip_tensor_upload(ctx, t, &w));
     cera_hip_status st = CERA_HIP_OK;
@@ -749,6 +754,7 @@ cera_hip_status cera_hip_gemv(cera_hip_ctx* ctx, const cera_hip_tensor* t, const
 
 cera_hip_status cera_hip_gemv_nb(cera_hip_ctx* ctx, const cera_hip_tensor* t, const float* x, uint32_t n, float* y) {
     if (!ctx || !t || !x || !y) return CERA_HIP_ERR_ARGUMENT;
+    std::lock_guard<std::recursive_mutex> op_lk(ctx->op_mu);
     if (n == 0 || t->k == 0 || t->k % 32) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "gemv_nb: need n > 0 and k a multiple of 32");
     cera_hip_dtensor* w = nullptr;
     CERA_TRY(cera_hip_tensor_upload(ctx, t, &w));
@@ -777,6 +783,7 @@ cera_hip_status cera_hip_gemv_nb(cera_hip_ctx* ctx, const cera_hip_tensor* t, co
 cera_hip_status cera_hip_gemv_pair(cera_hip_ctx* ctx, const cera_hip_tensor* ta, const cera_hip_tensor* tb, const float* x,
                                    float* ya, float* yb) {
     if (!ctx || !ta || !tb || !x || !ya || !yb) return CERA_HIP_ERR_ARGUMENT;
+    std::lock_guard<std::recursive_mutex> op_lk(ctx->op_mu);
     if (ta->k != tb->k || ta->k == 0 || ta->k % 256) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "gemv_pair: the two matrices must share k, a multiple of 256");
     cera_hip_dtensor *wa = nullptr, *wb = nullptr;
     CERA_TRY(cera_hip_tensor_upload(ctx, ta, &wa));
@@ -808,6 +815,7 @@ cera_hip_status cera_hip_attn_decode_dev(cera_hip_ctx* ctx, const float* q, cons
                                          uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, uint64_t seq_len,
                                          uint64_t max_seq, float scale, uint32_t n_splits, float* out) {
     if (!ctx || !q || !k || !v || !out) return CERA_HIP_ERR_ARGUMENT;
+    std::lock_guard<std::recursive_mutex> op_lk(ctx->op_mu);
     return cera_launch_attn_decode(ctx, q, k, v, n_heads, n_kv_heads, head_dim, seq_len, max_seq, scale, n_splits, out, nullptr, nullptr);
 }
 
@@ -853,6 +861,7 @@ cera_hip_status cera_hip_attn_decode(cera_hip_ctx* ctx, const float* q, const fl
                                      uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, uint64_t seq_len,
                                      float scale, uint32_t n_splits, float* out) {
     if (!ctx || !q || !k || !v || !out) return CERA_HIP_ERR_ARGUMENT;
+    std::lock_guard<std::recursive_mutex> op_lk(ctx->op_mu);
     if (seq_len == 0 || n_kv_heads == 0 || head_dim == 0) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "attn_decode: empty input");
     return attn_host(ctx, q, k, v, n_heads, n_kv_heads, head_dim, seq_len - 1, 1, scale, n_splits, out, false);
 }
@@ -861,6 +870,7 @@ cera_hip_status cera_hip_attn_prefill(cera_hip_ctx* ctx, const float* q, const f
                                       uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, uint64_t start_pos,
                                       uint32_t n_queries, float scale, float* out) {
     if (!ctx || !q || !k || !v || !out) return CERA_HIP_ERR_ARGUMENT;
+    std::lock_guard<std::recursive_mutex> op_lk(ctx->op_mu);
     if (n_queries == 0 || n_kv_heads == 0 || head_dim == 0) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "attn_prefill: empty input");
     return attn_host(ctx, q, k, v, n_heads, n_kv_heads, head_dim, start_pos, n_queries, scale, 0, out, false);
 }
@@ -869,6 +879,7 @@ cera_hip_status cera_hip_attn_f16kv(cera_hip_ctx* ctx, const float* q, const flo
                                     uint32_t n_kv_heads, uint32_t head_dim, uint64_t start_pos, uint32_t n_queries,
                                     float scale, uint32_t n_splits, float* out) {
     if (!ctx || !q || !k || !v || !out) return CERA_HIP_ERR_ARGUMENT;
+    std::lock_guard<std::recursive_mutex> op_lk(ctx->op_mu);
     if (n_queries == 0 || n_kv_heads == 0 || head_dim == 0) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "attn_f16kv: empty input");
     return attn_host(ctx, q, k, v, n_heads, n_kv_heads, head_dim, start_pos, n_queries, scale, n_splits, out, true);
 }
@@ -877,12 +888,14 @@ cera_hip_status cera_hip_attn_decode_f16_dev(cera_hip_ctx* ctx, const float* q, 
                                              uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, uint64_t seq_len,
                                              uint64_t max_seq, float scale, uint32_t n_splits, float* out) {
     if (!ctx || !q || !k16 || !v16 || !out) return CERA_HIP_ERR_ARGUMENT;
+    std::lock_guard<std::recursive_mutex> op_lk(ctx->op_mu);
     return cera_launch_attn_decode(ctx, q, k16, v16, n_heads, n_kv_heads, head_dim, seq_len, max_seq, scale, n_splits, out,
                                    nullptr, nullptr, nullptr, true);
 }
 
 cera_hip_status cera_hip_rmsnorm(cera_hip_ctx* ctx, const float* x, const float* weight, uint64_t n, float eps, float* y) {
     if (!ctx || !x || !weight || !y) return CERA_HIP_ERR_ARGUMENT;
+    std::lock_guard<std::recursive_mutex> op_lk(ctx->op_mu);
     if (n == 0 || n % 4 || n > 0xFFFFFFFFull) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "rmsnorm: n must be a positive multiple of 4");
     void *dx, *dw, *dy;
     CERA_TRY(cera_scratch(ctx, 0, n * 4, &dx));
@@ -898,6 +911,7 @@ cera_hip_status cera_hip_rmsnorm(cera_hip_ctx* ctx, const float* x, const float*
 
 cera_hip_status cera_hip_silu_mul(cera_hip_ctx* ctx, const float* gate, const float* up, uint64_t n, float* out) {
     if (!ctx || !gate || !up || !out) return CERA_HIP_ERR_ARGUMENT;
+    std::lock_guard<std::recursive_mutex> op_lk(ctx->op_mu);
     if (n == 0 || n % 4) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "silu_mul: n must be a positive multiple of 4");
     void *dg, *du, *dy;
     CERA_TRY(cera_scratch(ctx, 0, n * 4, &dg));
@@ -914,6 +928,7 @@ cera_hip_status cera_hip_silu_mul(cera_hip_ctx* ctx, const float* gate, const fl
 
 cera_hip_status cera_hip_argmax(cera_hip_ctx* ctx, const float* logits, uint64_t n, uint32_t* index) {
     if (!ctx || !index || (!logits && n)) return CERA_HIP_ERR_ARGUMENT;
+    std::lock_guard<std::recursive_mutex> op_lk(ctx->op_mu);
     if (n > 0xFFFFFFFFull) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "argmax: n exceeds 2^32");
     if (n == 0) { *index = 0; return CERA_HIP_OK; }
     void *dx, *di;
@@ -926,6 +941,7 @@ cera_hip_status cera_hip_argmax(cera_hip_ctx* ctx, const float* logits, uint64_t
 
 cera_hip_status cera_hip_dequantize_row(cera_hip_ctx* ctx, const cera_hip_tensor* t, uint64_t row, float* out) {
     if (!ctx || !out) return CERA_HIP_ERR_ARGUMENT;
+    std::lock_guard<std::recursive_mutex> op_lk(ctx->op_mu);
     uint64_t rb;
     CERA_TRY(check_tensor(ctx, t, &rb));
     if (row >= t->m) return cera_fail(ctx, CERA_HIP_ERR_ARGUMENT, "dequantize_row: row index out of range");

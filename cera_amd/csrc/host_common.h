@@ -26,6 +26,9 @@ struct cera_hip_ctx {
     hipStream_t stream = nullptr;
     std::string err;
     uint32_t n_cu = 0;
+    // serialises every call that uses the stream's workspaces below (kernel-level entry points
+    // with host buffers, and every model-level call of any model on this context)
+    std::recursive_mutex op_mu;
     // grow-only device scratch for the host-pointer entry points
     void* scratch[12] = {nullptr};
     uint64_t scratch_bytes[12] = {0};

@@ -34,6 +34,7 @@ struct cera_hip_model {
     std::vector<void*> owned;     // plain device allocations freed with the model
     // batched-prefill activations, token-major [n][dim], allocated on first use
     uint32_t pf_cap = 0;
+    uint64_t pf_bytes = 0;        // bytes held by pf_owned (part of `bytes`)
     float *pf_hidden = nullptr, *pf_normed = nullptr, *pf_q = nullptr, *pf_k = nullptr, *pf_v = nullptr,
           *pf_attn = nullptr, *pf_gate = nullptr, *pf_up = nullptr, *pf_xs = nullptr, *pf_bsum = nullptr;
     int8_t* pf_xq = nullptr;
@@ -43,12 +44,26 @@ struct cera_hip_model {
     uint32_t pf_logits_cap = 0;
     std::vector<void*> pf_owned;
     uint32_t seq_len = 0;
+    // reference-order verification route (reforder.hip): every f32 operation in the CPU path's
+    // order, bit-identical logits; slow, never the default
+    bool ref_order = false;
+    float* ref_scores = nullptr;  // [n_heads][max_seq_len] attention scores of that route
     bool kv_f16 = false;          // KV caches hold IEEE half instead of f32
     bool kv_configured = false;   // cera_hip_configure_kv was called: a different mode is a conflict
+    bool kv_broken = false;       // a cache re-allocation failed part-way: every later call fails
     uint64_t bytes = 0;
     // every trait call is serialised, like the reference GPU backends' infer_lock
     // (cera/src/model/mod.rs:184-199)
     std::mutex infer_lock;
+};
+
+// Held for the length of a model-level call: the model's own lock, then the lock of the context
+// whose stream and workspaces (scratch slots, attention partials) the call uses -- two models on
+// one context may be driven from two threads.
+struct ModelLock {
+    std::lock_guard<std::mutex> model;
+    std::lock_guard<std::recursive_mutex> ctx;
+    explicit ModelLock(cera_hip_model* m) : model(m->infer_lock), ctx(m->ctx->op_mu) {}
 };
 
 void cera_build_rope_table(uint32_t max_seq, uint32_t head_dim, float base, const float* ff, std::vector<float>& out);
@@ -61,4 +76,7 @@ cera_hip_status cera_model_prefill(cera_hip_model* m, const uint32_t* tokens, ui
 // same, logits of every position into logits_all[n][vocab] (host)
 cera_hip_status cera_model_prefill_logits_all(cera_hip_model* m, const uint32_t* tokens, uint32_t n, uint32_t start_pos,
                                               float* logits_all);
+// one token through the reference-order kernels (reforder.hip)
+cera_hip_status cera_model_decode_step_ref(cera_hip_model* m, uint32_t pos, bool want_logits);
+bool cera_model_ref_order_supported(const cera_hip_model* m, std::string* why);
 cera_hip_status cera_model_decode_logits(cera_hip_model* m, uint32_t token, uint32_t pos, float* logits);

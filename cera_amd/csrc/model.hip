@@ -60,6 +60,7 @@ void cera_build_rope_table(uint32_t max_seq, uint32_t head_dim, float base, cons
 static void free_model(cera_hip_model* m) {
     if (!m) return;
     cera_hip_ctx* ctx = m->ctx;
+    std::lock_guard<std::recursive_mutex> op_lk(ctx->op_mu);
     (void)hipStreamSynchronize(ctx->stream);
     auto ft = [&](cera_hip_dtensor* t) { if (t) cera_hip_tensor_free(ctx, t); };
     for (auto& L : m->layers) {
@@ -89,6 +90,7 @@ extern "C" cera_hip_status cera_hip_model_create(cera_hip_ctx* ctx, const cera_h
                                                  const float* output_norm, const cera_hip_layer* layers,
                                                  cera_hip_model** out) {
     if (!ctx || !cfg || !token_embd || !output_norm || !layers || !out) return CERA_HIP_ERR_ARGUMENT;
+    std::lock_guard<std::recursive_mutex> op_lk(ctx->op_mu);
     *out = nullptr;
     const cera_hip_config& c = *cfg;
     if (c.n_layers == 0 || c.hidden == 0 || c.ffn == 0 || c.n_heads == 0 || c.n_kv_heads == 0 || c.vocab == 0 ||
@@ -111,8 +113,20 @@ extern "C" cera_hip_status cera_hip_model_create(cera_hip_ctx* ctx, const cera_h
                              std::string(name) + ": no hip GEMV kernel for ggml type " + std::to_string(t.ggml_type));
         return CERA_HIP_OK;
     };
-    CERA_TRY(expect(*token_embd, c.vocab, c.hidden, "token_embd", output == nullptr));
-    if (output) CERA_TRY(expect(*output, c.vocab, c.hidden, "output", true));
+    // The embedding / head tables may carry pad rows past vocab_size (the reference bounds token
+    // ids and logits by vocab_size, not by the row count, cera/src/model/llama.rs:839-846): only
+    // the first vocab rows are ever read, so only those are uploaded.
+    auto vocab_rows = [&](const cera_hip_tensor& t, const char* name, bool matmul, cera_hip_tensor* cut) -> cera_hip_status {
+        *cut = t;
+        if (t.m > c.vocab && t.m != 0 && t.nbytes % t.m == 0) {
+            cut->nbytes = t.nbytes / t.m * c.vocab;
+            cut->m = c.vocab;
+        }
+        return expect(*cut, c.vocab, c.hidden, name, matmul);
+    };
+    cera_hip_tensor embd_cut, output_cut;
+    CERA_TRY(vocab_rows(*token_embd, "token_embd", output == nullptr, &embd_cut));
+    if (output) CERA_TRY(vocab_rows(*output, "output", true, &output_cut));
     for (uint32_t i = 0; i < c.n_layers; ++i) {
         const cera_hip_layer& L = layers[i];
         if (!L.attn_norm || !L.ffn_norm) return cera_fail(ctx, CERA_HIP_ERR_ARGUMENT, "layer norm weights missing");
@@ -133,10 +147,10 @@ extern "C" cera_hip_status cera_hip_model_create(cera_hip_ctx* ctx, const cera_h
     m->layers.resize(c.n_layers);
     uint64_t* tot = &m->bytes;
     auto build = [&]() -> cera_hip_status {
-        CERA_TRY(cera_hip_tensor_upload(ctx, token_embd, &m->embd));
+        CERA_TRY(cera_hip_tensor_upload(ctx, &embd_cut, &m->embd));
         *tot += m->embd->nbytes;
         if (output) {
-            CERA_TRY(cera_hip_tensor_upload(ctx, output, &m->output));
+            CERA_TRY(cera_hip_tensor_upload(ctx, &output_cut, &m->output));
             *tot += m->output->nbytes;
         }
         float* tmp;
@@ -178,11 +192,14 @@ extern "C" cera_hip_status cera_hip_model_create(cera_hip_ctx* ctx, const cera_h
             CERA_TRY(alloc_kv_cache(ctx, kv_elems * sizeof(float), &D.kc, tot));
             CERA_TRY(alloc_kv_cache(ctx, kv_elems * sizeof(float), &D.vc, tot));
         }
-        if (cfg->rope_freqs) m->rope_ff.assign(cfg->rope_freqs, cfg->rope_freqs + c.head_dim / 2);
+        // frequency factors belong to the interleaved-pair layout only: the split-half rotation
+        // never divides by them (cera/src/backend/cpu.rs:5031-5045, transformer.rs:1411)
+        const float* ff = c.rope_type == 1 ? cfg->rope_freqs : nullptr;
+        if (ff) m->rope_ff.assign(ff, ff + c.head_dim / 2);
         CERA_TRY(dev_alloc_t(ctx, c.head_dim, &tmp, tot));
         m->shift_cs = tmp; m->owned.push_back(tmp);
         std::vector<float> table;
-        cera_build_rope_table(c.max_seq_len, c.head_dim, c.rope_theta, cfg->rope_freqs, table);
+        cera_build_rope_table(c.max_seq_len, c.head_dim, c.rope_theta, ff, table);
         CERA_TRY(upload_f32(ctx, table.data(), table.size(), &tmp, tot));
         m->rope_table = tmp; m->owned.push_back(tmp);
 
@@ -226,7 +243,7 @@ extern "C" uint64_t cera_hip_memory_bytes(const cera_hip_model* m) { return m ? 
 
 extern "C" cera_hip_status cera_hip_truncate_kv(cera_hip_model* m, uint32_t len) {
     if (!m) return CERA_HIP_ERR_ARGUMENT;
-    std::lock_guard<std::mutex> lk(m->infer_lock);
+    ModelLock lk(m);
     if (len < m->seq_len) m->seq_len = len;  // rows past len are simply overwritten later
     return CERA_HIP_OK;
 }
@@ -236,7 +253,7 @@ extern "C" cera_hip_status cera_hip_truncate_kv(cera_hip_model* m, uint32_t len)
 // and re-rotate its K rows by R(-shift) so their encoded position matches their new index.
 extern "C" cera_hip_status cera_hip_shift_kv(cera_hip_model* m, uint32_t n_keep, uint32_t shift) {
     if (!m) return CERA_HIP_ERR_ARGUMENT;
-    std::lock_guard<std::mutex> lk(m->infer_lock);
+    ModelLock lk(m);
     cera_hip_ctx* ctx = m->ctx;
     const cera_hip_config& c = m->cfg;
     if (shift == 0) return cera_fail(ctx, CERA_HIP_ERR_ARGUMENT, "shift_kv: shift must be > 0");
@@ -313,7 +330,7 @@ extern "C" cera_hip_status cera_hip_shift_kv(cera_hip_model* m, uint32_t n_keep,
 extern "C" cera_hip_status cera_hip_write_kv(cera_hip_model* m, uint32_t layer, const float* k, const float* v,
                                              uint32_t n_pos) {
     if (!m || (n_pos && (!k || !v)) || layer >= m->cfg.n_layers) return CERA_HIP_ERR_ARGUMENT;
-    std::lock_guard<std::mutex> lk(m->infer_lock);
+    ModelLock lk(m);
     const cera_hip_config& c = m->cfg;
     if (n_pos > c.max_seq_len) return cera_fail(m->ctx, CERA_HIP_ERR_POSITION, "write_kv: more positions than max_seq_len");
     const uint64_t per_head = static_cast<uint64_t>(c.max_seq_len) * c.head_dim;
@@ -341,7 +358,7 @@ extern "C" cera_hip_status cera_hip_write_kv(cera_hip_model* m, uint32_t layer, 
 
 extern "C" cera_hip_status cera_hip_set_seq_len(cera_hip_model* m, uint32_t len) {
     if (!m) return CERA_HIP_ERR_ARGUMENT;
-    std::lock_guard<std::mutex> lk(m->infer_lock);
+    ModelLock lk(m);
     if (len > m->cfg.max_seq_len) return cera_fail(m->ctx, CERA_HIP_ERR_POSITION, "set_seq_len: beyond max_seq_len");
     m->seq_len = len;
     return CERA_HIP_OK;
@@ -353,31 +370,51 @@ extern "C" cera_hip_status cera_hip_set_seq_len(cera_hip_model* m, uint32_t len)
 // re-allocates the (still empty) caches at the new element width.
 extern "C" cera_hip_status cera_hip_configure_kv(cera_hip_model* m, uint32_t kv_type) {
     if (!m) return CERA_HIP_ERR_ARGUMENT;
-    std::lock_guard<std::mutex> lk(m->infer_lock);
+    ModelLock lk(m);
     cera_hip_ctx* ctx = m->ctx;
     if (kv_type > CERA_HIP_KV_F16) return cera_fail(ctx, CERA_HIP_ERR_ARGUMENT, "configure_kv: unknown cache type");
     const bool want_f16 = kv_type == CERA_HIP_KV_F16;
+    if (m->kv_broken) return cera_fail(ctx, CERA_HIP_ERR_DEVICE, "configure_kv: an earlier cache re-allocation failed; the model is unusable");
     if (m->kv_configured && want_f16 != m->kv_f16)
         return cera_fail(ctx, CERA_HIP_ERR_ARGUMENT, "configure_kv: the KV cache is already configured for another mode");
-    m->kv_configured = true;
-    if (want_f16 == m->kv_f16) return CERA_HIP_OK;
+    if (want_f16 == m->kv_f16) { m->kv_configured = true; return CERA_HIP_OK; }
     if (m->seq_len != 0) return cera_fail(ctx, CERA_HIP_ERR_POSITION, "configure_kv: the cache already holds positions");
     const cera_hip_config& c = m->cfg;
     const uint64_t kv_elems = static_cast<uint64_t>(c.n_kv_heads) * c.max_seq_len * c.head_dim;
     const uint64_t old_bytes = kv_elems * (m->kv_f16 ? sizeof(kv_half) : sizeof(float));
     const uint64_t new_bytes = kv_elems * (want_f16 ? sizeof(kv_half) : sizeof(float));
     HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
-    for (LayerDev& L : m->layers) {
-        for (void** cache : {&L.kc, &L.vc}) {
-            if (*cache) HIP_TRY(ctx, hipFree(*cache));
-            *cache = nullptr;
-            m->bytes -= old_bytes;
-            CERA_TRY(alloc_kv_cache(ctx, new_bytes, cache, &m->bytes));
+    // A failure part-way leaves layers with caches of different widths: the model is then marked
+    // unusable (every later forward / configure call fails) instead of running on them.
+    auto swap_all = [&]() -> cera_hip_status {
+        for (LayerDev& L : m->layers) {
+            for (void** cache : {&L.kc, &L.vc}) {
+                if (*cache) HIP_TRY(ctx, hipFree(*cache));
+                *cache = nullptr;
+                m->bytes -= old_bytes;
+                CERA_TRY(alloc_kv_cache(ctx, new_bytes, cache, &m->bytes));
+            }
         }
-    }
+        return CERA_HIP_OK;
+    };
+    const cera_hip_status st = swap_all();
+    if (st != CERA_HIP_OK) { m->kv_broken = true; return st; }
     m->kv_f16 = want_f16;
+    m->kv_configured = true;
     return CERA_HIP_OK;
 }
+
+extern "C" cera_hip_status cera_hip_set_reference_order(cera_hip_model* m, uint32_t on) {
+    if (!m) return CERA_HIP_ERR_ARGUMENT;
+    ModelLock lk(m);
+    if (m->seq_len != 0) return cera_fail(m->ctx, CERA_HIP_ERR_POSITION, "set_reference_order: the cache already holds positions");
+    std::string why;
+    if (on && !cera_model_ref_order_supported(m, &why))
+        return cera_fail(m->ctx, CERA_HIP_ERR_UNSUPPORTED_DTYPE, "set_reference_order: " + why);
+    m->ref_order = on != 0;
+    return CERA_HIP_OK;
+}
+extern "C" uint32_t cera_hip_reference_order(const cera_hip_model* m) { return m && m->ref_order ? 1u : 0u; }
 
 extern "C" uint32_t cera_hip_kv_type(const cera_hip_model* m) { return m && m->kv_f16 ? CERA_HIP_KV_F16 : CERA_HIP_KV_F32; }
 
@@ -421,6 +458,7 @@ static cera_hip_status norm_quant(cera_hip_model* m, const float* x, const float
 // The per-token layer stack: LlamaModel::run_layers + project_logits.  The
 // token id and position are read by the kernels from m->scalars[0..1].
 static cera_hip_status decode_step(cera_hip_model* m, uint32_t pos, bool want_logits) {
+    if (m->ref_order) return cera_model_decode_step_ref(m, pos, want_logits);
     cera_hip_ctx* ctx = m->ctx;
     const cera_hip_config& c = m->cfg;
     hipStream_t s = ctx->stream;
@@ -518,7 +556,18 @@ static cera_hip_status decode_step(cera_hip_model* m, uint32_t pos, bool want_lo
     return CERA_HIP_OK;
 }
 
+// A call at position 0 starts a fresh sequence: callers hand a new InferenceState to every
+// generate(), and a device-resident backend resets its own counter then, as the reference's do
+// (cera/src/model/metal_lfm2.rs:4091-4096, gpu_lfm2.rs:3755-3762).  Cached rows are simply
+// overwritten.
+static cera_hip_status begin_at(cera_hip_model* m, uint32_t pos) {
+    if (m->kv_broken) return cera_fail(m->ctx, CERA_HIP_ERR_DEVICE, "the model's KV cache is unusable (a cache re-allocation failed)");
+    if (pos == 0) m->seq_len = 0;
+    return CERA_HIP_OK;
+}
+
 static cera_hip_status check_step(cera_hip_model* m, uint32_t token, uint32_t pos) {
+    CERA_TRY(begin_at(m, pos));
     if (token >= m->cfg.vocab)
         return cera_fail(m->ctx, CERA_HIP_ERR_ARGUMENT, "token id " + std::to_string(token) + " out of range (vocab " + std::to_string(m->cfg.vocab) + ")");
     if (pos != m->seq_len)
@@ -542,7 +591,7 @@ static cera_hip_status set_token_pos(cera_hip_model* m, uint32_t token, uint32_t
 
 extern "C" cera_hip_status cera_hip_forward(cera_hip_model* m, uint32_t token, uint32_t pos, float* logits) {
     if (!m || !logits) return CERA_HIP_ERR_ARGUMENT;
-    std::lock_guard<std::mutex> lk(m->infer_lock);
+    ModelLock lk(m);
     CERA_TRY(check_step(m, token, pos));
     CERA_TRY(set_token_pos(m, token, pos));
     CERA_TRY(decode_step(m, pos, true));
@@ -553,7 +602,7 @@ extern "C" cera_hip_status cera_hip_forward(cera_hip_model* m, uint32_t token, u
 
 extern "C" cera_hip_status cera_hip_forward_greedy(cera_hip_model* m, uint32_t token, uint32_t pos, uint32_t* next) {
     if (!m || !next) return CERA_HIP_ERR_ARGUMENT;
-    std::lock_guard<std::mutex> lk(m->infer_lock);
+    ModelLock lk(m);
     CERA_TRY(check_step(m, token, pos));
     CERA_TRY(set_token_pos(m, token, pos));
     CERA_TRY(decode_step(m, pos, true));
@@ -567,7 +616,8 @@ extern "C" cera_hip_status cera_hip_forward_prefill(cera_hip_model* m, const uin
                                                     uint32_t start_pos, float* last_logits) {
     if (!m || !tokens || !last_logits) return CERA_HIP_ERR_ARGUMENT;
     if (n == 0) return cera_fail(m->ctx, CERA_HIP_ERR_ARGUMENT, "forward_prefill requires at least one token");
-    std::lock_guard<std::mutex> lk(m->infer_lock);
+    ModelLock lk(m);
+    CERA_TRY(begin_at(m, start_pos));
     if (start_pos != m->seq_len)
         return cera_fail(m->ctx, CERA_HIP_ERR_POSITION, "forward_prefill: start_pos " + std::to_string(start_pos) +
                                                             " must equal seq_len " + std::to_string(m->seq_len));
@@ -582,7 +632,8 @@ extern "C" cera_hip_status cera_hip_forward_prefill_logits_all(cera_hip_model* m
                                                                uint32_t start_pos, float* logits_all) {
     if (!m || !tokens || !logits_all) return CERA_HIP_ERR_ARGUMENT;
     if (n == 0) return cera_fail(m->ctx, CERA_HIP_ERR_ARGUMENT, "forward_prefill_logits_all requires at least one token");
-    std::lock_guard<std::mutex> lk(m->infer_lock);
+    ModelLock lk(m);
+    CERA_TRY(begin_at(m, start_pos));
     if (start_pos != m->seq_len)
         return cera_fail(m->ctx, CERA_HIP_ERR_POSITION, "forward_prefill_logits_all: start_pos " + std::to_string(start_pos) +
                                                             " must equal seq_len " + std::to_string(m->seq_len));
@@ -616,7 +667,7 @@ cera_hip_status cera_model_prefill_per_token(cera_hip_model* m, const uint32_t* 
 
 extern "C" cera_hip_status cera_hip_read_kv(cera_hip_model* m, uint32_t layer, float* k_out, float* v_out) {
     if (!m || !k_out || !v_out || layer >= m->cfg.n_layers) return CERA_HIP_ERR_ARGUMENT;
-    std::lock_guard<std::mutex> lk(m->infer_lock);
+    ModelLock lk(m);
     const cera_hip_config& c = m->cfg;
     const uint64_t per_head = static_cast<uint64_t>(c.max_seq_len) * c.head_dim;
     std::vector<float> hk(static_cast<uint64_t>(m->seq_len) * c.head_dim), hv(hk.size());
@@ -645,7 +696,7 @@ extern "C" cera_hip_status cera_hip_read_kv(cera_hip_model* m, uint32_t layer, f
 
 extern "C" cera_hip_status cera_hip_read_hidden(cera_hip_model* m, float* hidden_out) {
     if (!m || !hidden_out) return CERA_HIP_ERR_ARGUMENT;
-    std::lock_guard<std::mutex> lk(m->infer_lock);
+    ModelLock lk(m);
     return cera_hip_download(m->ctx, hidden_out, m->hidden, static_cast<uint64_t>(m->cfg.hidden) * 4);
 }
 
@@ -655,8 +706,9 @@ extern "C" cera_hip_status cera_hip_rope(cera_hip_ctx* ctx, float* q, float* k, 
                                          const float* freq_factors) {
     if (!ctx || !q || !k) return CERA_HIP_ERR_ARGUMENT;
     if (head_dim == 0 || head_dim % 2 || head_dim > 2048 || rope_type > 1) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "rope: bad head_dim or rope_type");
+    std::lock_guard<std::recursive_mutex> lk(ctx->op_mu);
     std::vector<float> table;
-    cera_build_rope_table(pos + 1, head_dim, freq_base, freq_factors, table);
+    cera_build_rope_table(pos + 1, head_dim, freq_base, rope_type == 1 ? freq_factors : nullptr, table);
     const uint64_t half = head_dim / 2;
     void *dq, *dk, *dt, *dp;
     CERA_TRY(cera_scratch(ctx, 0, static_cast<uint64_t>(n_heads) * head_dim * 4, &dq));

@@ -144,6 +144,7 @@ static cera_hip_status quantize_rows(cera_hip_ctx* ctx, const float* x, uint64_t
 extern "C" cera_hip_status cera_hip_gemm_dev(cera_hip_ctx* ctx, const cera_hip_dtensor* w, const float* x, uint64_t n,
                                              float* out) {
     if (!ctx || !w || !x || !out) return CERA_HIP_ERR_ARGUMENT;
+    std::lock_guard<std::recursive_mutex> op_lk(ctx->op_mu);
     if (n == 0 || n > 0x7FFFFFFFull) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "gemm: bad n");
     if (!cera_gemm_supports(w->dtype, w->k))
         return cera_fail(ctx, CERA_HIP_ERR_UNSUPPORTED_DTYPE,
@@ -161,6 +162,7 @@ extern "C" cera_hip_status cera_hip_gemm_dev(cera_hip_ctx* ctx, const cera_hip_d
 extern "C" cera_hip_status cera_hip_gemm(cera_hip_ctx* ctx, const cera_hip_tensor* t, const float* x, uint64_t n,
                                          float* out) {
     if (!ctx || !x || !out) return CERA_HIP_ERR_ARGUMENT;
+    std::lock_guard<std::recursive_mutex> op_lk(ctx->op_mu);
     if (n == 0 || n > 0x7FFFFFFFull) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "gemm: bad n");
     cera_hip_dtensor* w = nullptr;
     CERA_TRY(cera_hip_tensor_upload(ctx, t, &w));
@@ -180,6 +182,7 @@ extern "C" cera_hip_status cera_hip_gemm(cera_hip_ctx* ctx, const cera_hip_tenso
 extern "C" cera_hip_status cera_hip_gemm_pair(cera_hip_ctx* ctx, const cera_hip_tensor* ta, const cera_hip_tensor* tb,
                                               const float* x, uint64_t n, float* out_a, float* out_b) {
     if (!ctx || !ta || !tb || !x || !out_a || !out_b) return CERA_HIP_ERR_ARGUMENT;
+    std::lock_guard<std::recursive_mutex> op_lk(ctx->op_mu);
     if (n == 0 || n > 0x7FFFFFFFull) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "gemm_pair: bad n");
     cera_hip_dtensor *wa = nullptr, *wb = nullptr;
     CERA_TRY(cera_hip_tensor_upload(ctx, ta, &wa));
@@ -219,6 +222,7 @@ extern "C" cera_hip_status cera_hip_gemm_pair(cera_hip_ctx* ctx, const cera_hip_
 extern "C" cera_hip_status cera_hip_gemm_swiglu(cera_hip_ctx* ctx, const cera_hip_tensor* tg, const cera_hip_tensor* tu,
                                                 const float* x, uint64_t n, int8_t* quants, float* scales, int* fused_out) {
     if (!ctx || !tg || !tu || !x || !quants || !scales) return CERA_HIP_ERR_ARGUMENT;
+    std::lock_guard<std::recursive_mutex> op_lk(ctx->op_mu);
     if (n == 0 || n > 0x7FFFFFFFull) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "gemm_swiglu: bad n");
     cera_hip_dtensor *wg = nullptr, *wu = nullptr;
     CERA_TRY(cera_hip_tensor_upload(ctx, tg, &wg));
@@ -288,12 +292,15 @@ static cera_hip_status ensure_prefill_buffers(cera_hip_model* m, uint32_t n) {
     HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
     for (void* p : m->pf_owned) (void)hipFree(p);
     m->pf_owned.clear();
+    m->bytes -= m->pf_bytes;
+    m->pf_bytes = 0;
     m->pf_cap = 0;
     const uint32_t cap = std::min<uint32_t>(PREFILL_CHUNK, std::max<uint32_t>(n, 64));
     auto alloc = [&](uint64_t bytes, void** p) -> cera_hip_status {
         HIP_TRY(ctx, hipMalloc(p, bytes));
         m->pf_owned.push_back(*p);
         m->bytes += bytes;
+        m->pf_bytes += bytes;
         return CERA_HIP_OK;
     };
     CERA_TRY(alloc(cap * c.hidden * 4ull, reinterpret_cast<void**>(&m->pf_hidden)));
@@ -436,7 +443,7 @@ static cera_hip_status prefill_chunk(cera_hip_model* m, const uint32_t* tokens, 
     m->seq_len = start_pos + n;
     if (all_logits) {
         const cera_hip_dtensor* o = m->output ? m->output : m->embd;
-        const uint64_t rows = o->m;   // >= vocab; pad rows of a tied table are computed and dropped
+        const uint64_t rows = o->m;   // == vocab: pad rows of a table are cut off at load
         if (m->pf_logits_cap < n) {
             HIP_TRY(ctx, hipStreamSynchronize(s));
             if (m->pf_logits) {
@@ -458,12 +465,7 @@ static cera_hip_status prefill_chunk(cera_hip_model* m, const uint32_t* tokens, 
                                1.0f / c.logit_scale, static_cast<uint32_t>(tot));
             HIP_TRY(ctx, hipGetLastError());
         }
-        if (rows == c.vocab)   // no pad rows: one contiguous copy
-            return cera_hip_download(ctx, all_logits, m->pf_logits, static_cast<uint64_t>(n) * rows * 4);
-        HIP_TRY(ctx, hipMemcpy2DAsync(all_logits, static_cast<size_t>(c.vocab) * 4, m->pf_logits, rows * 4,
-                                      static_cast<size_t>(c.vocab) * 4, n, hipMemcpyDeviceToHost, s));
-        HIP_TRY(ctx, hipStreamSynchronize(s));
-        return CERA_HIP_OK;
+        return cera_hip_download(ctx, all_logits, m->pf_logits, static_cast<uint64_t>(n) * rows * 4);
     }
     if (want_logits) {
         // last token: final norm then the decode-style GEMV (project_logits)
@@ -494,6 +496,7 @@ static bool batched_supports(const cera_hip_model* m, const cera_hip_dtensor* w)
     return int8_type && w->k % unit == 0 && w->k / unit <= 512 && m->cfg.residual_scale == 1.0f;
 }
 static bool prefill_batchable(const cera_hip_model* m) {
+    if (m->ref_order) return false;   // the verification route prefills token by token, as its CPU twin does
     for (const LayerDev& L : m->layers)
         for (const cera_hip_dtensor* w : {L.q, L.k, L.v, L.o, L.gate, L.up, L.down})
             if (!batched_supports(m, w)) return false;

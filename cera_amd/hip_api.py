@@ -30,6 +30,8 @@ SYMBOLS = [
     "cera_hip_forward_prefill", "cera_hip_forward_prefill_logits_all", "cera_hip_truncate_kv", "cera_hip_gemv_pair", "cera_hip_gemm_pair", "cera_hip_gemm_swiglu", "cera_hip_gemv_nb", "cera_hip_configure_kv", "cera_hip_kv_type", "cera_hip_attn_f16kv",
     "cera_hip_attn_decode_f16_dev", "cera_hip_shift_kv", "cera_hip_write_kv", "cera_hip_set_seq_len", "cera_hip_seq_len", "cera_hip_memory_bytes",
     "cera_hip_read_kv", "cera_hip_read_hidden",
+    "cera_hip_gemv_reference_order", "cera_hip_attn_decode_reference_order", "cera_hip_rmsnorm_reference_order",
+    "cera_hip_set_reference_order", "cera_hip_reference_order",
 ]
 
 
@@ -129,6 +131,10 @@ def load_library() -> C.CDLL:
         "cera_hip_set_seq_len": (i32, [vp, u32]),
         "cera_hip_seq_len": (u32, [vp]), "cera_hip_memory_bytes": (u64, [vp]),
         "cera_hip_read_kv": (i32, [vp, u32, vp, vp]), "cera_hip_read_hidden": (i32, [vp, vp]),
+        "cera_hip_gemv_reference_order": (i32, [vp, C.POINTER(Tensor), vp, vp]),
+        "cera_hip_attn_decode_reference_order": (i32, [vp, vp, vp, vp, u32, u32, u32, u64, f32, vp]),
+        "cera_hip_rmsnorm_reference_order": (i32, [vp, vp, vp, u64, f32, vp]),
+        "cera_hip_set_reference_order": (i32, [vp, u32]), "cera_hip_reference_order": (u32, [vp]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(L, name)
@@ -324,6 +330,30 @@ class Context:
                                                 n_queries, scale, n_splits, _p(out)))
         return out.reshape(n_queries, n_heads * head_dim)
 
+    # -- reference-order verification kernels (bit-identical to the CPU AVX2 path)
+    def gemv_reference_order(self, ggml_type: int, blocks: np.ndarray, x: np.ndarray, m: int, k: int) -> np.ndarray:
+        t = make_tensor(ggml_type, m, k, blocks)
+        x = np.ascontiguousarray(x, np.float32)
+        y = np.empty(m, np.float32)
+        self.check(self.lib.cera_hip_gemv_reference_order(self.h, C.byref(t), _p(x), _p(y)))
+        return y
+
+    def attn_decode_reference_order(self, q, k, v, n_heads, n_kv_heads, head_dim, seq_len, scale) -> np.ndarray:
+        q = np.ascontiguousarray(q, np.float32)
+        k = np.ascontiguousarray(k, np.float32)
+        v = np.ascontiguousarray(v, np.float32)
+        out = np.empty(n_heads * head_dim, np.float32)
+        self.check(self.lib.cera_hip_attn_decode_reference_order(self.h, _p(q), _p(k), _p(v), n_heads, n_kv_heads, head_dim,
+                                                                 seq_len, scale, _p(out)))
+        return out
+
+    def rmsnorm_reference_order(self, x, w, eps) -> np.ndarray:
+        x = np.ascontiguousarray(x, np.float32)
+        w = np.ascontiguousarray(w, np.float32)
+        y = np.empty_like(x)
+        self.check(self.lib.cera_hip_rmsnorm_reference_order(self.h, _p(x), _p(w), x.size, eps, _p(y)))
+        return y
+
     def rmsnorm(self, x, w, eps) -> np.ndarray:
         x = np.ascontiguousarray(x, np.float32)
         w = np.ascontiguousarray(w, np.float32)
@@ -450,6 +480,14 @@ class Model:
         self.ctx.check(self.ctx.lib.cera_hip_forward_prefill_logits_all(self.h, _p(t) if t.size else None, t.size, start_pos,
                                                                         _p(out)))
         return out
+
+    def set_reference_order(self, on: bool = True):
+        """Switch to (or from) the reference-order verification route; needs an empty cache."""
+        self.ctx.check(self.ctx.lib.cera_hip_set_reference_order(self.h, 1 if on else 0))
+
+    @property
+    def reference_order(self) -> bool:
+        return self.ctx.lib.cera_hip_reference_order(self.h) == 1
 
     def configure_kv(self, f16: bool):
         self.ctx.check(self.ctx.lib.cera_hip_configure_kv(self.h, 1 if f16 else 0))

@@ -16,8 +16,8 @@ LLAMA_SYMBOLS = ["cera_llama_open", "cera_llama_close", "cera_llama_last_error",
                  "cera_llama_forward_greedy", "cera_llama_forward_prefill", "cera_llama_forward_prefill_logits_all", "cera_llama_forward_prefill_chunked",
                  "cera_llama_set_cancel", "cera_llama_truncate_kv", "cera_llama_supports_kv_shift", "cera_llama_f16_kv_supported", "cera_llama_configure_kv_compression", "cera_llama_shift_kv",
                  "cera_llama_snapshot_state", "cera_llama_snapshot_seq_len", "cera_llama_snapshot_bytes",
-                 "cera_llama_restore_state", "cera_llama_snapshot_free", "cera_llama_generate_greedy", "cera_spec_prompt_lookup_draft",
-                 "cera_llama_generate_spec"]
+                 "cera_llama_restore_state", "cera_llama_snapshot_free", "cera_llama_generate_greedy",
+                 "cera_llama_set_reference_order"]
 
 
 class LlamaConfigC(C.Structure):
@@ -59,8 +59,7 @@ def lib() -> C.CDLL:
             "cera_llama_snapshot_bytes": (u64, [vp]),
             "cera_llama_restore_state": (C.c_int, [vp, vp]),
             "cera_llama_snapshot_free": (None, [vp]),
-            "cera_spec_prompt_lookup_draft": (u64, [vp, u64, u64, u64, vp, u64]),
-            "cera_llama_generate_spec": (C.c_int, [vp, vp, u64, u64, vp, u64, u64, u64, vp, vp, vp, vp]),
+            "cera_llama_set_reference_order": (C.c_int, [vp, C.c_int]),
             "cera_llama_generate_greedy": (C.c_int, [vp, vp, u64, u64, u64, vp, C.POINTER(C.c_double),
                                                      C.POINTER(C.c_double)]),
         }
@@ -73,14 +72,6 @@ def lib() -> C.CDLL:
 
 class BackendError(RuntimeError):
     pass
-
-
-def prompt_lookup_draft(tokens, ngram: int, k: int) -> list:
-    """cera/src/spec.rs:23-40 through the C face (model-free, needs no GPU)."""
-    t = np.ascontiguousarray(tokens, np.uint32)
-    out = np.empty(max(k, 1), np.uint32)
-    n = lib().cera_spec_prompt_lookup_draft(t.ctypes.data if t.size else None, t.size, ngram, k, out.ctypes.data, out.size)
-    return [int(v) for v in out[:n]]
 
 
 class Snapshot:
@@ -162,20 +153,9 @@ class HipLlama:
                                                                 start_pos, out.ctypes.data))
         return out
 
-    def generate_spec(self, prompt, max_new: int, eos=(), ngram: int = 3, k: int = 7):
-        """Greedy speculative decoding with prompt-lookup drafting on a fresh session:
-        (tokens, {drafted, accepted, rounds, seconds})."""
-        p = np.ascontiguousarray(prompt, np.uint32)
-        e = np.ascontiguousarray(list(eos), np.uint32)
-        out = np.empty(max(max_new, 1), np.uint32)
-        n_out = C.c_uint64(0)
-        stats = (C.c_uint64 * 3)()
-        secs = C.c_double(0)
-        self._check(lib().cera_llama_generate_spec(self.h, p.ctypes.data if p.size else None, p.size, max_new,
-                                                   e.ctypes.data if e.size else None, e.size, ngram, k, out.ctypes.data,
-                                                   C.byref(n_out), stats, C.byref(secs)))
-        return [int(v) for v in out[:n_out.value]], dict(drafted=int(stats[0]), accepted=int(stats[1]),
-                                                          rounds=int(stats[2]), seconds=secs.value)
+    def set_reference_order(self, on: bool = True):
+        """Verification hook: reference-order kernels (bit-identical to the CPU AVX2 path)."""
+        self._check(lib().cera_llama_set_reference_order(self.h, 1 if on else 0))
 
     def forward_prefill_chunked(self, tokens, start_pos: int, ubatch: int):
         t = np.ascontiguousarray(tokens, np.uint32)

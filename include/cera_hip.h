@@ -12,7 +12,9 @@
  *  - "host" pointers are ordinary CPU memory owned by the caller and only
  *    borrowed for the duration of the call; "dev" pointers come from
  *    cera_hip_malloc() on the same context;
- *  - all work of a context runs on that context's single HIP stream;
+ *  - all work of a context runs on that context's single HIP stream; calls on one context are
+ *    serialised by the library (a model is additionally serialised by its own lock), so models
+ *    sharing a context may be driven from different threads, one call at a time;
  *  - weights stay in their native GGUF block layout in device memory.
  */
 #ifndef CERA_HIP_H
@@ -239,6 +241,24 @@ CERA_HIP_API cera_hip_status cera_hip_argmax(cera_hip_ctx*, const float* logits,
 CERA_HIP_API cera_hip_status cera_hip_dequantize_row(cera_hip_ctx*, const cera_hip_tensor* w, uint64_t row,
                                                      float* out);
 
+/* ---- reference-order verification route (never the default, never timed) -- */
+/* The same three operations with every f32 operation performed exactly as the CPU AVX2 path
+ * performs it, in its order, so the results are bit-identical to that path (not merely within
+ * the float tolerance): gemm_q4_k_q8_0 / gemm_q6_k_q8_0 at n == 1 with their eight-lane
+ * four-accumulator FMA chains, tree add and hsum256_ps (cera/src/backend/simd.rs:5742-5795,
+ * 6025-6093, 4546-4554), row_dot_q4_0 / row_dot_q8_0 (:4593-4637), gemm_q4_1_q8_0 (:5893-5976);
+ * attn_scores / softmax_inplace / attn_values of the AVX2 tier (cera/src/backend/cpu.rs:3503-3589,
+ * 2617-2633); cpu::rmsnorm with its serial f64 sum (:2479-2496).  Arguments as the fast entry
+ * points of the same name.  Q5_K is CERA_HIP_ERR_UNSUPPORTED_DTYPE here. */
+CERA_HIP_API cera_hip_status cera_hip_gemv_reference_order(cera_hip_ctx*, const cera_hip_tensor* w, const float* x,
+                                                           float* y);
+CERA_HIP_API cera_hip_status cera_hip_attn_decode_reference_order(cera_hip_ctx*, const float* q, const float* k,
+                                                                  const float* v, uint32_t n_heads, uint32_t n_kv_heads,
+                                                                  uint32_t head_dim, uint64_t seq_len, float scale,
+                                                                  float* out);
+CERA_HIP_API cera_hip_status cera_hip_rmsnorm_reference_order(cera_hip_ctx*, const float* x, const float* weight,
+                                                              uint64_t n, float eps, float* y);
+
 /* ---- kernel-level entry points, device buffers (timing) ----------------- */
 CERA_HIP_API cera_hip_status cera_hip_quantize_q8_0_dev(cera_hip_ctx*, const float* x, uint64_t k, float* scales,
                                                         int8_t* quants);
@@ -284,7 +304,11 @@ CERA_HIP_API cera_hip_status cera_hip_model_create(cera_hip_ctx*, const cera_hip
                                                    cera_hip_model** out);
 CERA_HIP_API void cera_hip_model_destroy(cera_hip_model*);
 /* Model::forward (cera/src/model/mod.rs:200-606; LlamaModel::forward,
- * cera/src/model/llama.rs:1585-1605): one token at `pos` -> vocab logits. */
+ * cera/src/model/llama.rs:1585-1605): one token at `pos` -> vocab logits.
+ * pos must equal cera_hip_seq_len, except that pos == 0 always starts a fresh sequence (the
+ * device-side counter is reset, as the reference's device-resident backends do when a caller
+ * arrives with a new InferenceState, cera/src/model/metal_lfm2.rs:4091-4096); the same holds
+ * for start_pos of the prefill calls. */
 CERA_HIP_API cera_hip_status cera_hip_forward(cera_hip_model*, uint32_t token, uint32_t pos, float* logits);
 /* Model::forward_greedy (cera/src/model/mod.rs:494-497): forward + argmax on
  * the device, 4-byte readback. */
@@ -309,6 +333,16 @@ CERA_HIP_API cera_hip_status cera_hip_forward_prefill_logits_all(cera_hip_model*
 #define CERA_HIP_KV_F16 1u
 CERA_HIP_API cera_hip_status cera_hip_configure_kv(cera_hip_model*, uint32_t kv_type);
 CERA_HIP_API uint32_t cera_hip_kv_type(const cera_hip_model*);
+/* Switches a model to the reference-order verification route (on != 0) or back: forward,
+ * forward_greedy and forward_prefill then run LlamaModel::forward's operations one by one
+ * (cera/src/model/llama.rs:468-597, 1585-1649; prefill token by token, as :1643-1648) on the
+ * reference-order kernels above, and logits are bit-identical to the CPU AVX2 path's -- the
+ * harness of cera/tests/gpu_transformer_parity.rs:75-103 then sees the identical greedy token
+ * stream.  Many times slower than the default route; meant for verification only.  Only with an
+ * empty cache (CERA_HIP_ERR_POSITION otherwise); CERA_HIP_ERR_UNSUPPORTED_DTYPE if a matrix is
+ * Q5_K. */
+CERA_HIP_API cera_hip_status cera_hip_set_reference_order(cera_hip_model*, uint32_t on);
+CERA_HIP_API uint32_t cera_hip_reference_order(const cera_hip_model*);
 /* Model::truncate_kv (cera/src/model/mod.rs:251-283). */
 CERA_HIP_API cera_hip_status cera_hip_truncate_kv(cera_hip_model*, uint32_t len);
 CERA_HIP_API uint32_t cera_hip_seq_len(const cera_hip_model*);

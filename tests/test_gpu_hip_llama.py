@@ -329,7 +329,7 @@ def test_head_dim_64_file(tmp_path, orc, hip, arch, explicit):
         gm.close(); om.close()
 
 
-# ---- speculative decoding (the caller of forward_prefill_logits_all / truncate_kv) ---------
+# ---- a speculative-decoding caller as the harness of forward_prefill_logits_all / truncate_kv ----
 def _plain_greedy(path, prompt, n_new):
     gm = llama_api.HipLlama(path, context_size=64)
     try:
@@ -338,34 +338,79 @@ def _plain_greedy(path, prompt, n_new):
         gm.close()
 
 
+def _draft(tokens, ngram, k):
+    """Continuation of the most recent earlier occurrence of the last `ngram` tokens, at most k long."""
+    n = len(tokens)
+    if ngram == 0 or k == 0 or n <= ngram:
+        return []
+    tail = tokens[n - ngram:]
+    for start in range(n - ngram - 1, -1, -1):
+        if tokens[start:start + ngram] == tail:
+            return tokens[start + ngram:start + ngram + k]
+    return []
+
+
+def _speculative_greedy(gm, prompt, max_new, ngram, k):
+    """Draft from the token history, verify the draft in ONE all-logits pass, keep the longest
+    prefix the model itself would have produced, roll the cache back past the rejected rest."""
+    seq = list(prompt)
+    logits = gm.forward_prefill(prompt, 0)
+    out, rounds, drafted, accepted = [], 0, 0, 0
+    nxt = int(np.argmax(logits))
+    while len(out) < max_new:
+        out.append(nxt); seq.append(nxt)
+        if len(out) == max_new:
+            break
+        d = _draft(seq, ngram, min(k, max_new - len(out) - 1))
+        base = gm.seq_len
+        rows = gm.forward_prefill_logits_all([nxt] + d, base)      # row i = logits after token i of the batch
+        rounds += bool(d); drafted += len(d)
+        keep = 0
+        while keep < len(d) and int(np.argmax(rows[keep])) == d[keep]:
+            keep += 1
+        accepted += keep
+        out.extend(d[:keep]); seq.extend(d[:keep])
+        gm.truncate_kv(base + 1 + keep)
+        nxt = int(np.argmax(rows[keep]))
+    return out[:max_new], dict(rounds=rounds, drafted=drafted, accepted=accepted)
+
+
 def test_speculative_greedy_is_a_greedy_decode(tiny_llama):
     """cera/tests/spec_decode_logits.rs:212-330 in spirit: every emitted token is the target's own
-    argmax, so the stream equals the sequential greedy loop (on this small model, token for
-    token); a drafter that never matches (ngram 999) runs no verification round at all; EOS is
-    not emitted; the budget cap is exact."""
+    argmax over a row of forward_prefill_logits_all, so the stream equals the sequential greedy
+    loop token for token on this small model; a drafter that never matches runs no verification
+    batch longer than one token; the budget cap is exact."""
     path, cfg, _, _ = tiny_llama
     prompt = [5, 6, 7, 8] * 5
     plain = [int(t) for t in _plain_greedy(path, prompt, 30)]
     gm = llama_api.HipLlama(path, context_size=64)
     try:
-        spec, st = gm.generate_spec(prompt, 30, ngram=2, k=4)
+        spec, st = _speculative_greedy(gm, prompt, 30, ngram=2, k=4)
         _say(f"spec: drafted {st['drafted']} accepted {st['accepted']} rounds {st['rounds']}")
         assert spec == plain
         assert st["rounds"] > 0 and 0 <= st["accepted"] <= st["drafted"]
         assert gm.seq_len <= len(prompt) + 30
-        with pytest.raises(llama_api.BackendError):
-            gm.generate_spec(prompt, 4)                      # the session is no longer fresh
-        gm.truncate_kv(0)
-        none, st0 = gm.generate_spec(prompt, 30, ngram=999, k=4)
+        none, st0 = _speculative_greedy(gm, prompt, 30, ngram=999, k=4)   # fresh sequence at position 0
         assert none == plain and st0["rounds"] == 0 and st0["drafted"] == 0
-        gm.truncate_kv(0)
-        stop_at = 11
-        eos = [plain[stop_at]]
-        first = plain.index(eos[0])
-        cut, _ = gm.generate_spec(prompt, 30, eos=eos, ngram=2, k=4)
-        assert cut == plain[:first]                           # the EOS token itself is not emitted
-        gm.truncate_kv(0)
-        capped, _ = gm.generate_spec(prompt, 7, ngram=2, k=4)
+        capped, _ = _speculative_greedy(gm, prompt, 7, ngram=2, k=4)
         assert capped == plain[:7]
+    finally:
+        gm.close()
+
+
+def test_two_generations_with_fresh_states_and_no_truncate(tiny_llama):
+    """A caller hands a new InferenceState to every generate(): position 0 starts a fresh
+    sequence on the device too, without a truncate_kv in between."""
+    path, cfg, _, _ = tiny_llama
+    gm = llama_api.HipLlama(path, context_size=64)
+    try:
+        a = [int(t) for t in gm.generate_greedy([9, 8, 7], 12)[0]]
+        assert gm.seq_len == 3 + 11
+        b = [int(t) for t in gm.generate_greedy([9, 8, 7], 12)[0]]     # no truncate_kv(0) between the two
+        assert a == b
+        l1 = gm.forward(5, 0)                                           # single-token entry at position 0 as well
+        assert gm.seq_len == 1
+        l2 = gm.forward(5, 0)
+        assert np.array_equal(l1, l2)
     finally:
         gm.close()

@@ -121,8 +121,11 @@ def test_position_contract(tiny):
         gm.forward(1, 5)          # pos must equal seq_len
     assert e.value.status == 5
     with pytest.raises(hip_api.HipError) as e:
-        gm.forward_prefill([1, 2], 0)
+        gm.forward_prefill([1, 2], 3)   # start_pos must equal seq_len
     assert e.value.status == 5
+    gm.forward_prefill([1, 2], 0)       # ... except position 0, which starts a fresh sequence
+    assert gm.seq_len == 2
+    gm.forward(1, 0)
     with pytest.raises(hip_api.HipError) as e:
         gm.forward(cfg["vocab"], 1)   # token out of range
     assert e.value.status == 6

@@ -1,0 +1,194 @@
+"""The reference-order verification route: the GPU performs exactly the f32 operations of cera's
+CPU AVX2 path, in its order, so results are BIT-identical to the oracle (not merely within the
+float tolerance) -- kernel by kernel, and for whole models token after token.
+
+GEMV: gemm_q4_k_q8_0 / gemm_q6_k_q8_0 at n == 1 (cera/src/backend/simd.rs:5742-5795, 6025-6093),
+row_dot_q4_0 / row_dot_q8_0 (:4593-4637), gemm_q4_1_q8_0 (:5893-5976).  Attention: attn_scores /
+softmax_inplace / attn_values, AVX2 tier (cera/src/backend/cpu.rs:3503-3589, 2617-2633).
+rmsnorm: cera/src/backend/cpu.rs:2479-2496.  Model: LlamaModel::forward (llama.rs:468-597).
+"""
+import math
+
+import numpy as np
+import pytest
+
+import util
+from cera_amd import hip_api, host_api as H, synth
+
+pytestmark = pytest.mark.gpu
+
+
+def _say(msg):
+    print(msg, flush=True)
+
+
+def _same_bits(a, b):
+    a = np.ascontiguousarray(a, np.float32).view(np.uint32)
+    b = np.ascontiguousarray(b, np.float32).view(np.uint32)
+    return np.array_equal(a, b)
+
+
+@pytest.mark.parametrize("dtype,m,k", [
+    (util.Q4_K, 96, 4096), (util.Q4_K, 37, 256), (util.Q4_K, 64, 14336), (util.Q4_K, 33, 512),
+    (util.Q6_K, 96, 4096), (util.Q6_K, 64, 14336), (util.Q6_K, 5, 256),
+    (util.Q4_0, 96, 4096), (util.Q4_0, 7, 96), (util.Q8_0, 64, 4096), (util.Q8_0, 3, 32),
+    (util.Q4_1, 64, 4096), (util.Q4_1, 9, 128),
+])
+def test_gemv_reference_order_is_bit_identical(hip, orc, dtype, m, k):
+    _say(f"ref-order gemv {util.NAMES[dtype]} {m}x{k}")
+    w, _ = util.make_weights(dtype, m, k, seed=m + k)
+    for seed, scale in ((1, 1.0), (2, 30.0), (3, 1e-3)):
+        x = util.make_x(k, seed) * np.float32(scale)
+        got = hip.gemv_reference_order(dtype, w, x, m, k)
+        ref = orc.gemv(dtype, w, x, m, k)            # AVX2 twin where the host has it, else the lane emulation: same bits
+        assert _same_bits(got, ref), (util.NAMES[dtype], m, k, seed, float(np.abs(got - ref).max()))
+    # and the fast kernel agrees with it to the float bar
+    fast = hip.gemv(dtype, w, x, m, k)
+    assert np.abs(fast - got).max() <= 1e-3 * util.rms(got) + 1e-12
+
+
+def test_gemv_reference_order_config2_rows(hip, orc):
+    """Row samples of the Llama-3-8B decode shapes (config 2): down 4096x14336 Q6_K and the
+    head's 4096-wide Q6_K rows, gate 14336x4096 Q4_K."""
+    for dtype, m, k in ((util.Q4_K, 512, 4096), (util.Q6_K, 256, 14336), (util.Q6_K, 1024, 4096)):
+        w, _ = util.make_weights(dtype, m, k, seed=17)
+        x = util.make_x(k, 5)
+        assert _same_bits(hip.gemv_reference_order(dtype, w, x, m, k), orc.gemv(dtype, w, x, m, k)), (dtype, m, k)
+
+
+def test_gemv_reference_order_refuses_q5_k(hip):
+    w, _ = util.make_weights(util.Q5_K, 8, 256, seed=1)
+    with pytest.raises(hip_api.HipError) as e:
+        hip.gemv_reference_order(util.Q5_K, w, util.make_x(256, 1), 8, 256)
+    assert e.value.status == 3
+
+
+@pytest.mark.parametrize("n_heads,n_kv,hd,L", [(32, 8, 128, 1), (32, 8, 128, 7), (32, 8, 128, 300), (8, 2, 64, 33),
+                                               (4, 4, 128, 1000), (8, 1, 64, 257), (2, 1, 72, 40)])
+def test_attention_reference_order_is_bit_identical(hip, orc, n_heads, n_kv, hd, L):
+    if not orc.lib().orc_have_avx2():
+        pytest.fail("the oracle's AVX2 attention twin needs an x86-64-v3 host")
+    _say(f"ref-order attention heads {n_heads}/{n_kv} hd {hd} L {L}")
+    q = util.make_x(n_heads * hd, 1)
+    k = util.make_x(L * n_kv * hd, 2)
+    v = util.make_x(L * n_kv * hd, 3)
+    scale = 1.0 / math.sqrt(hd)
+    got = hip.attn_decode_reference_order(q, k, v, n_heads, n_kv, hd, L, scale)
+    ref = orc.decode_attention(q, k, v, n_heads, n_kv, hd, scale, L, variant=1)
+    assert _same_bits(got, ref), float(np.abs(got - ref).max())
+    if hd in (64, 128) and n_heads // n_kv in (1, 2, 4, 8):
+        fast = hip.attn_decode(q, k, v, n_heads, n_kv, hd, L, scale)
+        assert np.abs(fast - got).max() <= 2e-3 * max(util.rms(got), 1e-6)
+
+
+@pytest.mark.parametrize("n", [128, 256, 4096, 14336, 100, 4100])
+def test_rmsnorm_reference_order_is_bit_identical(hip, orc, n):
+    x = util.make_x(n, n) * np.float32(3.0)
+    w = (1.0 + 0.1 * util.make_x(n, n + 1)).astype(np.float32)
+    assert _same_bits(hip.rmsnorm_reference_order(x, w, 1e-5), orc.rmsnorm(x, w, 1e-5))
+
+
+# ---- whole models ------------------------------------------------------------------------------
+def _extras(cfg, w, seed, bias=False, qk_norm=False, freqs=False):
+    w = dict(w)
+    r = util.rng(seed)
+    q_dim, kv_dim = cfg["n_heads"] * cfg["head_dim"], cfg["n_kv_heads"] * cfg["head_dim"]
+    for i in range(cfg["n_layers"]):
+        if bias:
+            w[f"blk.{i}.attn_q.bias"] = (r.standard_normal(q_dim) * 0.5).astype(np.float32)
+            w[f"blk.{i}.attn_k.bias"] = (r.standard_normal(kv_dim) * 0.5).astype(np.float32)
+            w[f"blk.{i}.attn_v.bias"] = (r.standard_normal(kv_dim) * 0.5).astype(np.float32)
+        if qk_norm:
+            w[f"blk.{i}.attn_q_norm.weight"] = (1.0 + 0.3 * r.standard_normal(cfg["head_dim"])).astype(np.float32)
+            w[f"blk.{i}.attn_k_norm.weight"] = (1.0 + 0.3 * r.standard_normal(cfg["head_dim"])).astype(np.float32)
+    if freqs:
+        w["rope_freqs.weight"] = (1.0 + 0.25 * np.arange(cfg["head_dim"] // 2)).astype(np.float32)
+    return w
+
+
+MODELS = {
+    "llama_q4_k_m": (dict(), dict(), dict()),
+    "llama3_rope_freqs": (dict(), dict(), dict(freqs=True)),
+    "qwen2_neox_bias": (dict(rope_type=0), dict(), dict(bias=True)),
+    "qwen3_qknorm_hd64": (dict(rope_type=0, n_heads=8, n_kv_heads=2, head_dim=64), dict(), dict(qk_norm=True)),
+    "granite_scalars": (dict(embed_scale=12.0, residual_scale=0.22, attn_scale=0.0078125, logit_scale=8.0), dict(), dict()),
+    "tied_q8_0": (dict(), dict(type_of=lambda name: H.Q8_0, tied_output=True), dict()),
+    "q4_0": (dict(), dict(type_of=lambda name: H.Q4_0), dict()),
+}
+
+
+@pytest.mark.parametrize("name", list(MODELS))
+def test_model_reference_order_logits_bit_identical(hip, orc, name):
+    """Prefill + free-running greedy decode: every step's logits carry the oracle's bits, so the
+    token streams are identical by construction (asserted anyway)."""
+    over, mk, ex = MODELS[name]
+    cfg = dict(synth.TINY, **over)
+    weights = _extras(cfg, synth.make_llama(cfg, seed=321, sigma=0.05, norm_jitter=0.1, **mk), 7, **ex)
+    gm = hip_api.Model(hip, cfg, weights)
+    om = orc.Llama(cfg, weights)
+    gm.set_reference_order(True)
+    assert gm.reference_order
+    prompt = [int(t) for t in util.rng(5).integers(0, cfg["vocab"], 9)]
+    _say(f"ref-order model {name}: prefill 9 + 20 greedy")
+    lg, lo = gm.forward_prefill(prompt, 0), om.forward_prefill_per_token(prompt, 0)
+    for i in range(20):
+        assert _same_bits(lg, lo), (name, i, float(np.abs(lg - lo).max()))
+        tg, to = int(orc.argmax(lg)), int(orc.argmax(lo))
+        assert tg == to
+        lg, lo = gm.forward(tg, 9 + i), om.forward(to, 9 + i)
+    for layer in range(cfg["n_layers"]):
+        kg, vg = gm.read_kv(layer)
+        ko, vo = om.kv(layer)
+        assert _same_bits(kg, ko) and _same_bits(vg, vo), (name, layer)
+    # forward_greedy on this route is the same stream
+    gm.truncate_kv(0); om.truncate(0)
+    tg = to = 11
+    for pos in range(12):
+        to = int(orc.argmax(om.forward(to, pos)))
+        tg = gm.forward_greedy(tg, pos)
+        assert tg == to, (name, pos)
+    gm.close(); om.close()
+
+
+def test_model_reference_order_f16_kv(hip, orc):
+    cfg = dict(synth.TINY)
+    weights = synth.make_llama(cfg, seed=44, sigma=0.05, norm_jitter=0.1)
+    gm = hip_api.Model(hip, cfg, weights)
+    om = orc.Llama(cfg, weights)
+    gm.configure_kv(True); om.set_kv_f16(True)
+    gm.set_reference_order(True)
+    tok = 3
+    for pos in range(16):
+        lg, lo = gm.forward(tok, pos), om.forward(tok, pos)
+        assert _same_bits(lg, lo), pos
+        tok = int(orc.argmax(lo))
+    gm.close(); om.close()
+
+
+def test_reference_order_switch_rules(hip, orc):
+    cfg = dict(synth.TINY)
+    weights = synth.make_llama(cfg, seed=44, sigma=0.05)
+    gm = hip_api.Model(hip, cfg, weights)
+    om = orc.Llama(cfg, weights)
+    fast = gm.forward(7, 0)
+    with pytest.raises(hip_api.HipError) as e:
+        gm.set_reference_order(True)            # the cache holds a position
+    assert e.value.status == 5 and not gm.reference_order
+    gm.truncate_kv(0)
+    gm.set_reference_order(True)
+    ref = gm.forward(7, 0)
+    assert _same_bits(ref, om.forward(7, 0))
+    # the default route computes the same thing up to re-quantization noise
+    a, b = fast.astype(np.float64), ref.astype(np.float64)
+    assert float(a @ b / np.sqrt((a @ a) * (b @ b))) > 0.9995
+    gm.truncate_kv(0)
+    gm.set_reference_order(False)
+    assert _same_bits(gm.forward(7, 0), fast)   # and is unchanged by the round trip
+    gm.close(); om.close()
+    # a Q5_K matrix has no reference-order kernel: refused, never skipped
+    w5 = synth.make_llama(cfg, seed=1, sigma=0.05, type_of=lambda name: H.Q5_K if "ffn_up" in name else H.Q8_0)
+    g5 = hip_api.Model(hip, cfg, w5)
+    with pytest.raises(hip_api.HipError) as e:
+        g5.set_reference_order(True)
+    assert e.value.status == 3
+    g5.close()
