@@ -66,6 +66,10 @@ struct ModelLock {
     explicit ModelLock(cera_hip_model* m) : model(m->infer_lock), ctx(m->ctx->op_mu) {}
 };
 
+cera_hip_status cera_attn_step(cera_hip_ctx* ctx, float* q, float* k_new, const float* v_new, void* kc, void* vc,
+                               const float* rope_table, const uint32_t* pos_dev, uint32_t pos, uint32_t n_heads,
+                               uint32_t n_kv_heads, uint32_t head_dim, uint32_t max_seq, uint32_t rope_type, float scale,
+                               bool kv_f16, float* out, float* out_scales, int8_t* out_quants);
 void cera_build_rope_table(uint32_t max_seq, uint32_t head_dim, float base, const float* ff, std::vector<float>& out);
 cera_hip_status cera_model_prefill_per_token(cera_hip_model* m, const uint32_t* tokens, uint32_t n, uint32_t start_pos,
                                              float* last_logits);

@@ -444,15 +444,55 @@ static cera_hip_status project(cera_hip_model* m, const cera_hip_dtensor* w, con
     return cera_launch_gemv(ctx, w, nullptr, m->xs, m->xq, y, resid, resid ? CERA_EPI_ADD : CERA_EPI_STORE);
 }
 
-static cera_hip_status norm_quant(cera_hip_model* m, const float* x, const float* w, uint32_t n, uint32_t rows, float* y) {
+// rmsnorm of `rows` rows of n elements with the Q8_0 quantization of the result fused in
+// (cpu::rmsnorm then quantize_f32_to_q8_0, cera/src/backend/cpu.rs:2479-2496, 942-958).  A single
+// row of up to 16384 elements (the decode step) runs the register-resident one-pass kernel.
+static cera_hip_status launch_norm_quant(cera_hip_ctx* ctx, const float* x, const float* w, uint32_t n, uint32_t rows,
+                                         float eps, float* y, float* xs, int8_t* xq) {
     if (rows == 1 && n <= 16384)
-        hipLaunchKernelGGL((rmsnorm_row_kernel<true>), dim3(1), dim3(1024), 0, m->ctx->stream, x, w, n, m->cfg.rms_eps, y,
-                           m->xs, m->xq);
+        hipLaunchKernelGGL((rmsnorm_row_kernel<true>), dim3(1), dim3(1024), 0, ctx->stream, x, w, n, eps, y, xs, xq);
     else
-        hipLaunchKernelGGL((rmsnorm_kernel<true>), dim3(rows), dim3(256), 0, m->ctx->stream, x, w, n, m->cfg.rms_eps, y,
-                           m->xs, m->xq, static_cast<float*>(nullptr));
-    HIP_TRY(m->ctx, hipGetLastError());
+        hipLaunchKernelGGL((rmsnorm_kernel<true>), dim3(rows), dim3(256), 0, ctx->stream, x, w, n, eps, y, xs, xq,
+                           static_cast<float*>(nullptr));
+    HIP_TRY(ctx, hipGetLastError());
     return CERA_HIP_OK;
+}
+static cera_hip_status norm_quant(cera_hip_model* m, const float* x, const float* w, uint32_t n, uint32_t rows, float* y) {
+    return launch_norm_quant(m->ctx, x, w, n, rows, m->cfg.rms_eps, y, m->xs, m->xq);
+}
+
+// The attention step of one decode layer: RoPE on q and the new K row, append of the new K/V rows
+// to the cache at `pos`, attention over positions [0, pos], and the Q8_0 quantization of the
+// result for the O projection (the merge kernel writes both).  While the context is short the
+// attention kernel rotates q on load, takes the new token's K/V rows from the projections
+// (rotating K) and appends them to the cache itself; longer contexts run RoPE + append as their
+// own launch, then plain attention.  q / k_new are rotated in place only on the second route.
+cera_hip_status cera_attn_step(cera_hip_ctx* ctx, float* q, float* k_new, const float* v_new, void* kc, void* vc,
+                               const float* rope_table, const uint32_t* pos_dev, uint32_t pos, uint32_t n_heads,
+                               uint32_t n_kv_heads, uint32_t head_dim, uint32_t max_seq, uint32_t rope_type, float scale,
+                               bool kv_f16, float* out, float* out_scales, int8_t* out_quants) {
+    hipStream_t s = ctx->stream;
+    if (pos + 1 < ATTN_FUSED_NEW_KV_MAX_KEYS) {
+        AttnNewKV nk;
+        nk.rope_row = rope_table + static_cast<uint64_t>(pos) * head_dim;
+        nk.rope_type = rope_type;
+        nk.k_new = k_new;
+        nk.v_new = v_new;
+        nk.kc_w = kc;
+        nk.vc_w = vc;
+        return cera_launch_attn_decode(ctx, q, kc, vc, n_heads, n_kv_heads, head_dim, pos + 1, max_seq, scale, 0, out,
+                                       out_scales, out_quants, &nk, kv_f16);
+    }
+    const dim3 rgrid(n_heads + 2 * n_kv_heads, 1), rblock(head_dim / 2);
+    if (kv_f16)
+        hipLaunchKernelGGL(rope_kv_kernel<kv_half>, rgrid, rblock, 0, s, q, k_new, v_new, rope_table, pos_dev, n_heads,
+                           n_kv_heads, head_dim, rope_type, static_cast<kv_half*>(kc), static_cast<kv_half*>(vc), max_seq);
+    else
+        hipLaunchKernelGGL(rope_kv_kernel<float>, rgrid, rblock, 0, s, q, k_new, v_new, rope_table, pos_dev, n_heads,
+                           n_kv_heads, head_dim, rope_type, static_cast<float*>(kc), static_cast<float*>(vc), max_seq);
+    HIP_TRY(ctx, hipGetLastError());
+    return cera_launch_attn_decode(ctx, q, kc, vc, n_heads, n_kv_heads, head_dim, pos + 1, max_seq, scale, 0, out, out_scales,
+                                   out_quants, nullptr, kv_f16);
 }
 
 // The per-token layer stack: LlamaModel::run_layers + project_logits.  The
@@ -498,34 +538,8 @@ static cera_hip_status decode_step(cera_hip_model* m, uint32_t pos, bool want_lo
             hipLaunchKernelGGL((rmsnorm_kernel<false>), dim3(c.n_kv_heads), dim3(256), 0, s, m->k, L.k_norm, c.head_dim,
                                c.rms_eps, m->k, nullptr, nullptr, nullptr);
         }
-        // attention over positions [0, pos]; the merge also quantizes for the O projection.  While the
-        // context is short the kernel rotates q on load, takes the new token's K/V rows from the
-        // projections (rotating K) and appends them to the cache itself
-        AttnNewKV nk;
-        nk.rope_row = m->rope_table + static_cast<uint64_t>(pos) * c.head_dim;
-        nk.rope_type = c.rope_type;
-        nk.k_new = m->k;
-        nk.v_new = m->v;
-        nk.kc_w = L.kc;
-        nk.vc_w = L.vc;
-        if (pos + 1 < ATTN_FUSED_NEW_KV_MAX_KEYS) {
-            CERA_TRY(cera_launch_attn_decode(ctx, m->q, L.kc, L.vc, c.n_heads, c.n_kv_heads, c.head_dim, pos + 1,
-                                             c.max_seq_len, scale, 0, m->attn_out, m->xs, m->xq, &nk, m->kv_f16));
-        } else {
-            // longer contexts: RoPE + cache append as their own launch, then plain attention
-            const dim3 rgrid(c.n_heads + 2 * c.n_kv_heads, 1), rblock(c.head_dim / 2);
-            if (m->kv_f16)
-                hipLaunchKernelGGL(rope_kv_kernel<kv_half>, rgrid, rblock, 0, s, m->q, m->k, m->v, m->rope_table,
-                                   m->scalars + 1, c.n_heads, c.n_kv_heads, c.head_dim, c.rope_type,
-                                   static_cast<kv_half*>(L.kc), static_cast<kv_half*>(L.vc), c.max_seq_len);
-            else
-                hipLaunchKernelGGL(rope_kv_kernel<float>, rgrid, rblock, 0, s, m->q, m->k, m->v, m->rope_table,
-                                   m->scalars + 1, c.n_heads, c.n_kv_heads, c.head_dim, c.rope_type,
-                                   static_cast<float*>(L.kc), static_cast<float*>(L.vc), c.max_seq_len);
-            HIP_TRY(ctx, hipGetLastError());
-            CERA_TRY(cera_launch_attn_decode(ctx, m->q, L.kc, L.vc, c.n_heads, c.n_kv_heads, c.head_dim, pos + 1,
-                                             c.max_seq_len, scale, 0, m->attn_out, m->xs, m->xq, nullptr, m->kv_f16));
-        }
+        CERA_TRY(cera_attn_step(ctx, m->q, m->k, m->v, L.kc, L.vc, m->rope_table, m->scalars + 1, pos, c.n_heads, c.n_kv_heads,
+                                c.head_dim, c.max_seq_len, c.rope_type, scale, m->kv_f16, m->attn_out, m->xs, m->xq));
         CERA_TRY(project(m, L.o, m->attn_out, m->hidden, m->hidden));
 
         CERA_TRY(norm_quant(m, m->hidden, L.ffn_norm, c.hidden, 1, m->normed));
@@ -727,4 +741,93 @@ extern "C" cera_hip_status cera_hip_rope(cera_hip_ctx* ctx, float* q, float* k, 
     HIP_TRY(ctx, hipGetLastError());
     CERA_TRY(cera_hip_download(ctx, q, dq, static_cast<uint64_t>(n_heads) * head_dim * 4));
     return cera_hip_download(ctx, k, dk, static_cast<uint64_t>(n_kv_heads) * head_dim * 4);
+}
+
+// ---- kernel-level entry points for the decode step's fused kernels (host buffers) ------------
+extern "C" cera_hip_status cera_hip_rmsnorm_q8_0(cera_hip_ctx* ctx, const float* x, const float* weight, uint64_t n, float eps,
+                                                 float* y, float* scales, int8_t* quants) {
+    if (!ctx || !x || !weight || !y || !scales || !quants) return CERA_HIP_ERR_ARGUMENT;
+    if (n == 0 || n % 32 || n > 0xFFFFFFFFull) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "rmsnorm_q8_0: n must be a positive multiple of 32");
+    std::lock_guard<std::recursive_mutex> lk(ctx->op_mu);
+    void *dx, *dw, *dy, *ds, *dq;
+    CERA_TRY(cera_scratch(ctx, 0, n * 4, &dx));
+    CERA_TRY(cera_scratch(ctx, 1, n * 4, &dw));
+    CERA_TRY(cera_scratch(ctx, 3, n * 4, &dy));
+    CERA_TRY(cera_scratch(ctx, 4, n / 32 * 4, &ds));
+    CERA_TRY(cera_scratch(ctx, 2, n, &dq));
+    CERA_TRY(cera_hip_upload(ctx, dx, x, n * 4));
+    CERA_TRY(cera_hip_upload(ctx, dw, weight, n * 4));
+    CERA_TRY(launch_norm_quant(ctx, static_cast<float*>(dx), static_cast<float*>(dw), static_cast<uint32_t>(n), 1, eps,
+                               static_cast<float*>(dy), static_cast<float*>(ds), static_cast<int8_t*>(dq)));
+    CERA_TRY(cera_hip_download(ctx, y, dy, n * 4));
+    CERA_TRY(cera_hip_download(ctx, scales, ds, n / 32 * 4));
+    return cera_hip_download(ctx, quants, dq, n);
+}
+
+extern "C" cera_hip_status cera_hip_attn_decode_step(cera_hip_ctx* ctx, const float* q, const float* k_new, const float* v_new,
+                                                     const float* k_cache, const float* v_cache, uint32_t n_heads,
+                                                     uint32_t n_kv_heads, uint32_t head_dim, uint32_t pos, float rope_base,
+                                                     uint32_t rope_type, const float* freq_factors, float scale,
+                                                     uint32_t kv_type, float* out, float* out_scales, int8_t* out_quants,
+                                                     float* k_row, float* v_row) {
+    if (!ctx || !q || !k_new || !v_new || (pos && (!k_cache || !v_cache)) || !out || !out_scales || !out_quants || !k_row || !v_row)
+        return CERA_HIP_ERR_ARGUMENT;
+    if ((head_dim != 64 && head_dim != 128) || rope_type > 1 || kv_type > CERA_HIP_KV_F16 || n_kv_heads == 0 || n_heads % n_kv_heads)
+        return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "attn_decode_step: bad shape");
+    std::lock_guard<std::recursive_mutex> lk(ctx->op_mu);
+    const bool f16 = kv_type == CERA_HIP_KV_F16;
+    const uint32_t max_seq = pos + 1;
+    const uint64_t kv_dim = static_cast<uint64_t>(n_kv_heads) * head_dim, q_dim = static_cast<uint64_t>(n_heads) * head_dim;
+    const uint64_t esz = f16 ? sizeof(kv_half) : sizeof(float), cache_bytes = kv_dim * max_seq * esz;
+    // caches: head-major [kv_head][max_seq][head_dim], rows [0, pos) from the caller, row pos zero
+    std::vector<char> hk(cache_bytes, 0), hv(cache_bytes, 0);
+    for (uint64_t t = 0; t < pos; ++t)
+        for (uint32_t h = 0; h < n_kv_heads; ++h)
+            for (uint32_t d = 0; d < head_dim; ++d) {
+                const uint64_t dst = (static_cast<uint64_t>(h) * max_seq + t) * head_dim + d, src = t * kv_dim + h * head_dim + d;
+                if (f16) {
+                    reinterpret_cast<kv_half*>(hk.data())[dst] = static_cast<kv_half>(k_cache[src]);
+                    reinterpret_cast<kv_half*>(hv.data())[dst] = static_cast<kv_half>(v_cache[src]);
+                } else {
+                    reinterpret_cast<float*>(hk.data())[dst] = k_cache[src];
+                    reinterpret_cast<float*>(hv.data())[dst] = v_cache[src];
+                }
+            }
+    std::vector<float> table;
+    cera_build_rope_table(max_seq, head_dim, rope_base, rope_type == 1 ? freq_factors : nullptr, table);
+    void *dq, *dk, *dv, *dkc, *dvc, *dt, *dp, *dout, *dsc, *dqq;
+    CERA_TRY(cera_scratch(ctx, 0, q_dim * 4, &dq));
+    CERA_TRY(cera_scratch(ctx, 1, kv_dim * 4, &dk));
+    CERA_TRY(cera_scratch(ctx, 2, kv_dim * 4, &dv));
+    CERA_TRY(cera_scratch(ctx, 5, cache_bytes, &dkc));
+    CERA_TRY(cera_scratch(ctx, 6, cache_bytes, &dvc));
+    CERA_TRY(cera_scratch(ctx, 4, table.size() * 4, &dt));
+    CERA_TRY(cera_scratch(ctx, 7, 4, &dp));
+    CERA_TRY(cera_scratch(ctx, 3, q_dim * 4, &dout));
+    CERA_TRY(cera_scratch(ctx, 9, q_dim / 32 * 4, &dsc));
+    CERA_TRY(cera_scratch(ctx, 10, q_dim, &dqq));
+    CERA_TRY(cera_hip_upload(ctx, dq, q, q_dim * 4));
+    CERA_TRY(cera_hip_upload(ctx, dk, k_new, kv_dim * 4));
+    CERA_TRY(cera_hip_upload(ctx, dv, v_new, kv_dim * 4));
+    CERA_TRY(cera_hip_upload(ctx, dkc, hk.data(), cache_bytes));
+    CERA_TRY(cera_hip_upload(ctx, dvc, hv.data(), cache_bytes));
+    CERA_TRY(cera_hip_upload(ctx, dt, table.data(), table.size() * 4));
+    CERA_TRY(cera_hip_upload(ctx, dp, &pos, 4));
+    CERA_TRY(cera_attn_step(ctx, static_cast<float*>(dq), static_cast<float*>(dk), static_cast<float*>(dv), dkc, dvc,
+                            static_cast<float*>(dt), static_cast<uint32_t*>(dp), pos, n_heads, n_kv_heads, head_dim, max_seq,
+                            rope_type, scale, f16, static_cast<float*>(dout), static_cast<float*>(dsc), static_cast<int8_t*>(dqq)));
+    CERA_TRY(cera_hip_download(ctx, out, dout, q_dim * 4));
+    CERA_TRY(cera_hip_download(ctx, out_scales, dsc, q_dim / 32 * 4));
+    CERA_TRY(cera_hip_download(ctx, out_quants, dqq, q_dim));
+    // the rows the step appended at `pos`, widened exactly when the cache holds halves
+    std::vector<char> row(head_dim * esz);
+    for (int is_v = 0; is_v < 2; ++is_v)
+        for (uint32_t h = 0; h < n_kv_heads; ++h) {
+            const char* src = static_cast<const char*>(is_v ? dvc : dkc) + (static_cast<uint64_t>(h) * max_seq + pos) * head_dim * esz;
+            CERA_TRY(cera_hip_download(ctx, row.data(), src, row.size()));
+            float* dst = (is_v ? v_row : k_row) + h * head_dim;
+            for (uint32_t d = 0; d < head_dim; ++d)
+                dst[d] = f16 ? static_cast<float>(reinterpret_cast<const kv_half*>(row.data())[d]) : reinterpret_cast<const float*>(row.data())[d];
+        }
+    return CERA_HIP_OK;
 }

@@ -32,6 +32,7 @@ SYMBOLS = [
     "cera_hip_read_kv", "cera_hip_read_hidden",
     "cera_hip_gemv_reference_order", "cera_hip_attn_decode_reference_order", "cera_hip_rmsnorm_reference_order",
     "cera_hip_set_reference_order", "cera_hip_reference_order",
+    "cera_hip_rmsnorm_q8_0", "cera_hip_attn_decode_step",
 ]
 
 
@@ -135,6 +136,9 @@ def load_library() -> C.CDLL:
         "cera_hip_attn_decode_reference_order": (i32, [vp, vp, vp, vp, u32, u32, u32, u64, f32, vp]),
         "cera_hip_rmsnorm_reference_order": (i32, [vp, vp, vp, u64, f32, vp]),
         "cera_hip_set_reference_order": (i32, [vp, u32]), "cera_hip_reference_order": (u32, [vp]),
+        "cera_hip_rmsnorm_q8_0": (i32, [vp, vp, vp, u64, f32, vp, vp, vp]),
+        "cera_hip_attn_decode_step": (i32, [vp, vp, vp, vp, vp, vp, u32, u32, u32, u32, f32, u32, vp, f32, u32,
+                                            vp, vp, vp, vp, vp]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(L, name)
@@ -329,6 +333,34 @@ class Context:
         self.check(self.lib.cera_hip_attn_f16kv(self.h, _p(q), _p(k), _p(v), n_heads, n_kv_heads, head_dim, start_pos,
                                                 n_queries, scale, n_splits, _p(out)))
         return out.reshape(n_queries, n_heads * head_dim)
+
+    # -- the decode step's fused kernels
+    def rmsnorm_q8_0(self, x, w, eps):
+        """(normed f32, Q8_0 scales, Q8_0 quants) from the decode step's one-launch norm + quantize."""
+        x = np.ascontiguousarray(x, np.float32)
+        w = np.ascontiguousarray(w, np.float32)
+        y = np.empty_like(x)
+        scales = np.empty(x.size // 32, np.float32)
+        quants = np.empty(x.size, np.int8)
+        self.check(self.lib.cera_hip_rmsnorm_q8_0(self.h, _p(x), _p(w), x.size, eps, _p(y), _p(scales), _p(quants)))
+        return y, scales, quants
+
+    def attn_decode_step(self, q, k_new, v_new, k_cache, v_cache, n_heads, n_kv_heads, head_dim, pos, rope_base,
+                         norm=True, freq_factors=None, scale=None, kv_f16=False):
+        """One decode layer's attention step: (out, out_scales, out_quants, appended k row, appended v row)."""
+        q = np.ascontiguousarray(q, np.float32); k_new = np.ascontiguousarray(k_new, np.float32)
+        v_new = np.ascontiguousarray(v_new, np.float32)
+        kc = np.ascontiguousarray(k_cache, np.float32); vc = np.ascontiguousarray(v_cache, np.float32)
+        ff = None if freq_factors is None else np.ascontiguousarray(freq_factors, np.float32)
+        q_dim, kv_dim = n_heads * head_dim, n_kv_heads * head_dim
+        out = np.empty(q_dim, np.float32); sc = np.empty(q_dim // 32, np.float32); qq = np.empty(q_dim, np.int8)
+        k_row = np.empty(kv_dim, np.float32); v_row = np.empty(kv_dim, np.float32)
+        scale = float(scale if scale is not None else 1.0 / np.sqrt(head_dim))
+        self.check(self.lib.cera_hip_attn_decode_step(
+            self.h, _p(q), _p(k_new), _p(v_new), _p(kc) if kc.size else None, _p(vc) if vc.size else None, n_heads,
+            n_kv_heads, head_dim, pos, rope_base, 1 if norm else 0, None if ff is None else _p(ff), scale,
+            1 if kv_f16 else 0, _p(out), _p(sc), _p(qq), _p(k_row), _p(v_row)))
+        return out, sc, qq, k_row, v_row
 
     # -- reference-order verification kernels (bit-identical to the CPU AVX2 path)
     def gemv_reference_order(self, ggml_type: int, blocks: np.ndarray, x: np.ndarray, m: int, k: int) -> np.ndarray:

@@ -241,6 +241,30 @@ CERA_HIP_API cera_hip_status cera_hip_argmax(cera_hip_ctx*, const float* logits,
 CERA_HIP_API cera_hip_status cera_hip_dequantize_row(cera_hip_ctx*, const cera_hip_tensor* w, uint64_t row,
                                                      float* out);
 
+/* ---- the decode step's fused kernels, host buffers (parity tests) -------- */
+/* cpu::rmsnorm followed by quantize_f32_to_q8_0 of its result (cera/src/backend/cpu.rs:2479-2496,
+ * 942-958), as ONE launch: what the decode step runs before the Q/K/V and gate/up projections.
+ * n % 32 == 0.  y f32[n], scales f32[n/32], quants i8[n]. */
+CERA_HIP_API cera_hip_status cera_hip_rmsnorm_q8_0(cera_hip_ctx*, const float* x, const float* weight, uint64_t n,
+                                                   float eps, float* y, float* scales, int8_t* quants);
+/* The attention step of one decode layer exactly as the model's decode step issues it
+ * (transformer::forward_attn_block from the RoPE on, cera/src/model/transformer.rs:1399-1470, with
+ * cpu::rope / rope_norm, cera/src/backend/cpu.rs:5008-5180, and decode_attention,
+ * transformer.rs:1249-1305): q [n_heads*head_dim] and k_new [n_kv_heads*head_dim] arrive unrotated,
+ * v_new [n_kv_heads*head_dim]; k_cache / v_cache hold positions [0, pos) time-major
+ * [pos][n_kv_heads*head_dim] f32 (narrowed to half first when kv_type is CERA_HIP_KV_F16).  Below
+ * 1024 keys one attention launch rotates q, rotates and appends the new K/V rows and attends;
+ * beyond, a RoPE/append launch precedes it.  Returns the attention output out [n_heads*head_dim],
+ * its Q8_0 quantization (the O projection's input, written by the merge kernel) and the rows the
+ * step appended to the cache at `pos` (k_row rotated; widened exactly from a half cache). */
+CERA_HIP_API cera_hip_status cera_hip_attn_decode_step(cera_hip_ctx*, const float* q, const float* k_new,
+                                                       const float* v_new, const float* k_cache, const float* v_cache,
+                                                       uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim,
+                                                       uint32_t pos, float rope_base, uint32_t rope_type,
+                                                       const float* freq_factors, float scale, uint32_t kv_type,
+                                                       float* out, float* out_scales, int8_t* out_quants, float* k_row,
+                                                       float* v_row);
+
 /* ---- reference-order verification route (never the default, never timed) -- */
 /* The same three operations with every f32 operation performed exactly as the CPU AVX2 path
  * performs it, in its order, so the results are bit-identical to that path (not merely within

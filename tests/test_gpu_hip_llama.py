@@ -131,7 +131,7 @@ def test_contract_violations_fail_loudly(tiny_llama):
     path, cfg, gm, om = tiny_llama
     gm.truncate_kv(0)
     gm.forward(1, 0)
-    for call, needle in ((lambda: gm.forward(1, 5), "pos"), (lambda: gm.forward_prefill([1, 2], 0), "start_pos"),
+    for call, needle in ((lambda: gm.forward(1, 5), "pos"), (lambda: gm.forward_prefill([1, 2], 3), "start_pos"),
                          (lambda: gm.forward(cfg["vocab"], 1), "out of range"),
                          (lambda: gm.truncate_kv(3), "exceeds"),
                          (lambda: gm.forward_prefill(list(range(70)), 1), "")):

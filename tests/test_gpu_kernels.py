@@ -462,3 +462,55 @@ def test_gemv_multi_token_refusals(hip):
         w, _ = util.make_weights(Q4_K, 4, 28672, seed=1)
         hip.gemv_nb(Q4_K, w, np.zeros((2, 28672), np.float32), 4, 28672)
     assert e.value.status == 3
+
+
+# ---- the decode step's fused kernels, one by one --------------------------------------------------
+@pytest.mark.parametrize("n", [4096, 256, 14336, 16384, 32768, 96])
+def test_decode_rmsnorm_q8_0_fused_bit_exact(hip, orc, n):
+    """The one-launch rmsnorm + Q8_0 quantization of the decode step (the register-resident
+    single-row kernel up to 16384 elements, the looping one beyond): normed values, int8 quants and
+    scales all carry the bits of cpu::rmsnorm followed by quantize_f32_to_q8_0
+    (cera/src/backend/cpu.rs:2479-2496, 942-958)."""
+    _say(f"decode rmsnorm+q8_0 n={n}")
+    for seed, mag in ((1, 1.0), (2, 40.0), (3, 1e-4)):
+        x = util.make_x(n, seed + n) * np.float32(mag)
+        w = (1.0 + 0.2 * util.make_x(n, seed + 7)).astype(np.float32)
+        y, sc, qq = hip.rmsnorm_q8_0(x, w, 1e-5)
+        ref = orc.rmsnorm(x, w, 1e-5)
+        rs, rq = orc.quantize_q8_0(ref)
+        assert np.array_equal(y.view(np.uint32), ref.view(np.uint32)), (n, seed)
+        assert np.array_equal(qq, rq), (n, seed, int(np.count_nonzero(qq != rq)))
+        assert np.array_equal(sc.view(np.uint32), rs.view(np.uint32)), (n, seed)
+
+
+@pytest.mark.parametrize("norm", [True, False])
+@pytest.mark.parametrize("kv_f16", [False, True])
+@pytest.mark.parametrize("n_heads,n_kv,hd,pos", [(32, 8, 128, 0), (32, 8, 128, 5), (32, 8, 128, 640), (32, 8, 128, 1022),
+                                                 (32, 8, 128, 1023), (32, 8, 128, 1500), (8, 2, 64, 37), (8, 8, 64, 1100)])
+def test_decode_attention_step_fused_append_and_q8_0(hip, orc, norm, kv_f16, n_heads, n_kv, hd, pos):
+    """One decode layer's attention step through the model's own dispatch: the K row it appends
+    at `pos` carries the bits of cpu::rope / rope_norm on the new key (cera/src/backend/cpu.rs:
+    5008-5180; rounded to half for an f16 cache), the V row those of the new value, whether the
+    attention kernel did the rotation and the append itself (below 1024 keys) or a RoPE/append
+    launch did; the attention output meets the 2e-3 bar against decode_attention on the rotated
+    query and the completed cache; and the Q8_0 output the merge kernel writes for the O
+    projection is bit for bit the quantization of that output."""
+    _say(f"decode attention step heads {n_heads}/{n_kv} hd {hd} pos {pos} norm={norm} f16={kv_f16}")
+    kv_dim = n_kv * hd
+    q = util.make_x(n_heads * hd, 11 + pos)
+    k_new, v_new = util.make_x(kv_dim, 12 + pos), util.make_x(kv_dim, 13 + pos)
+    kc, vc = util.make_x(pos * kv_dim, 14), util.make_x(pos * kv_dim, 15)
+    ff = (1.0 + 0.1 * np.arange(hd // 2)).astype(np.float32) if norm and pos % 2 else None
+    out, sc, qq, k_row, v_row = hip.attn_decode_step(q, k_new, v_new, kc, vc, n_heads, n_kv, hd, pos, 500000.0, norm=norm,
+                                                     freq_factors=ff, kv_f16=kv_f16)
+    q_rot, k_rot = orc.rope(q, k_new, pos, n_heads, n_kv, hd, 500000.0, norm=norm, freq_factors=ff)
+    half = lambda a: a.astype(np.float16).astype(np.float32)
+    k_want, v_want = (half(k_rot), half(v_new)) if kv_f16 else (k_rot, v_new)
+    assert np.array_equal(k_row.view(np.uint32), k_want.view(np.uint32)), "appended K row"
+    assert np.array_equal(v_row.view(np.uint32), v_want.view(np.uint32)), "appended V row"
+    kc_full = np.concatenate([half(kc) if kv_f16 else kc, k_want])
+    vc_full = np.concatenate([half(vc) if kv_f16 else vc, v_want])
+    ref = orc.decode_attention(q_rot, kc_full, vc_full, n_heads, n_kv, hd, 1.0 / np.sqrt(hd), pos + 1)
+    assert np.abs(out - ref).max() <= 2e-3 * util.rms(ref)
+    rs, rq = orc.quantize_q8_0(out)
+    assert np.array_equal(qq, rq) and np.array_equal(sc.view(np.uint32), rs.view(np.uint32)), "fused Q8_0 of the merge kernel"

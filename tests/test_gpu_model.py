@@ -383,3 +383,102 @@ def test_decode_across_the_fused_append_window(hip, orc, kv_f16):
     assert np.abs(kg[rows] - ko[rows]).max() <= 3e-3 * util.rms(ko[rows])
     assert np.abs(vg[rows] - vo[rows]).max() <= 3e-3 * util.rms(vo[rows])
     gm.close(); om.close()
+
+
+# ---- Granite scalars, NEOX with frequency factors ------------------------------------------------
+def test_granite_scalars_model_parity(hip, orc):
+    """embedding / residual / attention / logit multipliers all different from their identities
+    (cera/src/model/llama.rs:513-520, 590-593; mod.rs:52-113): decode (separate scaled residual
+    add, logit scaling launch), batched prefill and a short batch track the oracle, in direction
+    and in magnitude."""
+    cfg = dict(synth.TINY, embed_scale=12.0, residual_scale=0.22, attn_scale=0.0078125, logit_scale=8.0)
+    weights = synth.make_llama(cfg, seed=77, sigma=0.05, norm_jitter=0.1)
+    gm = hip_api.Model(hip, cfg, weights)
+    om = orc.Llama(cfg, weights)
+    plain = orc.Llama(dict(synth.TINY), weights)
+    toks = [int(t) for t in util.rng(3).integers(0, cfg["vocab"], 20)]
+    _say("granite scalars: batched prefill 20 + 12 decode steps")
+    lg, lo = gm.forward_prefill(toks, 0), om.forward_prefill_batched(toks, 0)
+    lp = plain.forward_prefill_batched(toks, 0)
+    assert _cos(lo, lp) < 0.99, "the scalars must matter for this test to mean anything"
+    assert _cos(lg, lo) > 0.999 and abs(util.rms(lg) / util.rms(lo) - 1) < 0.02
+    same = 0
+    for i in range(12):
+        t = int(orc_argmax(lo))
+        same += int(orc_argmax(lg)) == t
+        lg, lo = gm.forward(t, 20 + i), om.forward(t, 20 + i)
+        assert _cos(lg, lo) > 0.999 and abs(util.rms(lg) / util.rms(lo) - 1) < 0.02, i
+    assert same >= 10
+    for layer in range(cfg["n_layers"]):
+        kg, vg = gm.read_kv(layer)
+        ko, vo = om.kv(layer)
+        assert np.abs(kg - ko).max() <= 3e-2 * util.rms(ko) and np.abs(vg - vo).max() <= 3e-2 * util.rms(vo)
+    # a 5-token batch (multi-token GEMV or per-token route) and all-position logits
+    gm.truncate_kv(0); om.truncate(0)
+    rows = gm.forward_prefill_logits_all(toks[:5], 0)
+    for i, t in enumerate(toks[:5]):
+        lo = om.forward(t, i)
+        assert _cos(rows[i], lo) > 0.999 and abs(util.rms(rows[i]) / util.rms(lo) - 1) < 0.02, i
+    gm.close(); om.close(); plain.close()
+
+
+def test_neox_ignores_frequency_factors(hip, orc):
+    """A split-half (NEOX) model whose file carries rope_freqs.weight: the rotation never divides
+    by the factors (cera/src/backend/cpu.rs:5031-5045; cera/src/model/transformer.rs:1411), in the
+    forward pass and in the context shift alike -- cached K rows equal the oracle's to the float
+    bar of the K projection, and equal those of the same model without the tensor bit for bit."""
+    cfg = dict(synth.TINY, rope_type=0)
+    base = synth.make_llama(cfg, seed=15, sigma=0.05, norm_jitter=0.1)
+    withf = dict(base)
+    withf["rope_freqs.weight"] = (1.0 + 0.5 * np.arange(cfg["head_dim"] // 2)).astype(np.float32)
+    ga, gb = hip_api.Model(hip, cfg, withf), hip_api.Model(hip, cfg, base)
+    om = orc.Llama(cfg, withf)
+    toks = [int(t) for t in util.rng(8).integers(0, cfg["vocab"], 18)]
+    la, lb, lo = ga.forward_prefill(toks, 0), gb.forward_prefill(toks, 0), om.forward_prefill_batched(toks, 0)
+    assert np.array_equal(la.view(np.uint32), lb.view(np.uint32))
+    assert _cos(la, lo) > 0.999
+    for t in (4, 9):
+        pos = ga.seq_len
+        la, lb, lo = ga.forward(t, pos), gb.forward(t, pos), om.forward(t, pos)
+        assert np.array_equal(la.view(np.uint32), lb.view(np.uint32)) and _cos(la, lo) > 0.999
+    ka, _ = ga.read_kv(0)
+    kb, _ = gb.read_kv(0)
+    ko, _ = om.kv(0)
+    assert np.array_equal(ka.view(np.uint32), kb.view(np.uint32))
+    assert np.abs(ka - ko).max() <= 3e-3 * util.rms(ko)
+    ga.shift_kv(3, 5); gb.shift_kv(3, 5); om.shift_kv(3, 5)
+    ka, _ = ga.read_kv(1)
+    kb, _ = gb.read_kv(1)
+    assert np.array_equal(ka.view(np.uint32), kb.view(np.uint32))
+    ga.close(); gb.close(); om.close()
+
+
+def test_two_models_on_one_context_from_two_threads(hip, orc):
+    """Workspaces (scratch slots, attention partials) belong to the context: calls of different
+    models sharing it are serialised by the library, so two threads may drive them."""
+    import threading
+    cfg = dict(synth.TINY)
+    wa, wb = synth.make_llama(cfg, seed=1, sigma=0.05), synth.make_llama(cfg, seed=2, sigma=0.05)
+    ga, gb = hip_api.Model(hip, cfg, wa), hip_api.Model(hip, cfg, wb)
+    toks = [int(t) for t in util.rng(8).integers(0, cfg["vocab"], 40)]
+    want = []
+    for g in (ga, gb):
+        want.append([g.forward_prefill(toks, 0)] + [g.forward(7, 40 + i) for i in range(6)])
+    got = [None, None]
+    errs = []
+
+    def run(i, g):
+        try:
+            for _ in range(3):
+                got[i] = [g.forward_prefill(toks, 0)] + [g.forward(7, 40 + j) for j in range(6)]
+        except Exception as e:   # surfaced below: an exception in a thread would otherwise be lost
+            errs.append(e)
+
+    th = [threading.Thread(target=run, args=(i, g)) for i, g in enumerate((ga, gb))]
+    for t in th: t.start()
+    for t in th: t.join()
+    assert not errs, errs
+    for i in range(2):
+        for a, b in zip(got[i], want[i]):
+            assert np.array_equal(a.view(np.uint32), b.view(np.uint32)), i
+    ga.close(); gb.close()
