@@ -518,6 +518,7 @@ struct AttnLaunch {
     uint32_t n_heads, n_kv_heads, n_queries, q_stride, G, S, n_parts, part_keys, chunks_per_part;
     bool batch, fused_new_kv;
     AttnNewKV nk;
+    float *acc, *ml;   // split-K partials: (o) and (m, l) per (query, head, part)
 };
 
 template <int G, typename KV, int HD>
@@ -528,11 +529,11 @@ static void attn_launch_decode_g(cera_hip_ctx* ctx, const AttnLaunch& a, const K
         if (a.fused_new_kv)                                                                                          \
             hipLaunchKernelGGL((attn_decode_partial_kernel<G, SS, true, KV, HD>), grid, block, 0, ctx->stream, a.q, kc,  \
                                vc, a.seq_len, a.max_seq, a.scale, a.chunks_per_part, a.n_parts, a.q_stride,          \
-                               ctx->attn_acc, ctx->attn_ml, a.nk);                                                   \
+                               a.acc, a.ml, a.nk);                                                                   \
         else                                                                                                         \
             hipLaunchKernelGGL((attn_decode_partial_kernel<G, SS, false, KV, HD>), grid, block, 0, ctx->stream, a.q, kc, \
                                vc, a.seq_len, a.max_seq, a.scale, a.chunks_per_part, a.n_parts, a.q_stride,          \
-                               ctx->attn_acc, ctx->attn_ml, a.nk);                                                   \
+                               a.acc, a.ml, a.nk);                                                                   \
     } while (0)
     switch (a.S) {
         case 1: ATTN_LAUNCH_S(1); break;
@@ -550,7 +551,7 @@ static void attn_launch_partials(cera_hip_ctx* ctx, const AttnLaunch& a, const K
         const dim3 pgrid((a.n_queries + 31) / 32, a.n_kv_heads, a.n_parts);
 #define ATTN_PF(GG)                                                                                                        \
     hipLaunchKernelGGL((attn_prefill_partial_kernel<KV, HD, GG>), pgrid, dim3(64 * GG), 0, ctx->stream, a.q, kc, vc, a.seq_len, \
-                       a.n_queries, a.max_seq, a.scale, a.part_keys, a.n_parts, a.q_stride, ctx->attn_acc, ctx->attn_ml)
+                       a.n_queries, a.max_seq, a.scale, a.part_keys, a.n_parts, a.q_stride, a.acc, a.ml)
         switch (a.G) {
             case 1: ATTN_PF(1); break;
             case 2: ATTN_PF(2); break;
@@ -572,7 +573,7 @@ cera_hip_status cera_launch_attn(cera_hip_ctx* ctx, const float* q, const void* 
                                  uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, uint64_t seq_len,
                                  uint64_t max_seq, float scale, uint32_t n_splits, uint32_t n_queries, float* out,
                                  float* out_scales, int8_t* out_quants, float* out_bsum, const AttnNewKV* new_kv,
-                                 bool kv_f16) {
+                                 bool kv_f16, const AttnWorkspace* ws) {
     if (head_dim != 64 && head_dim != 128) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "attention: head_dim must be 64 or 128");
     if (n_kv_heads == 0 || n_heads % n_kv_heads) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "attention: n_heads must be a multiple of n_kv_heads");
     uint32_t G = n_heads / n_kv_heads;
@@ -611,22 +612,36 @@ cera_hip_status cera_launch_attn(cera_hip_ctx* ctx, const float* q, const void* 
     }
     uint64_t acc_bytes = static_cast<uint64_t>(n_queries) * n_kv_heads * n_parts * G * head_dim * sizeof(float);
     uint64_t ml_bytes = static_cast<uint64_t>(n_queries) * n_kv_heads * n_parts * G * 2 * sizeof(float);
-    if (ctx->attn_acc_bytes < acc_bytes) {
-        HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
-        if (ctx->attn_acc) HIP_TRY(ctx, hipFree(ctx->attn_acc));
-        ctx->attn_acc = nullptr; ctx->attn_acc_bytes = 0;
-        HIP_TRY(ctx, hipMalloc(reinterpret_cast<void**>(&ctx->attn_acc), acc_bytes));
-        ctx->attn_acc_bytes = acc_bytes;
-    }
-    if (ctx->attn_ml_bytes < ml_bytes) {
-        HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
-        if (ctx->attn_ml) HIP_TRY(ctx, hipFree(ctx->attn_ml));
-        ctx->attn_ml = nullptr; ctx->attn_ml_bytes = 0;
-        HIP_TRY(ctx, hipMalloc(reinterpret_cast<void**>(&ctx->attn_ml), ml_bytes));
-        ctx->attn_ml_bytes = ml_bytes;
+    float *acc, *ml;
+    if (ws) {
+        // caller-provided workspace: nothing is allocated, a request that does not fit is refused
+        if (acc_bytes > ws->acc_bytes || ml_bytes > ws->ml_bytes)
+            return cera_fail(ctx, CERA_HIP_ERR_SHAPE,
+                             "attention: the split-K partials need " + std::to_string(acc_bytes) + " + " + std::to_string(ml_bytes) +
+                                 " bytes, the fixed workspace holds " + std::to_string(ws->acc_bytes) + " + " +
+                                 std::to_string(ws->ml_bytes));
+        acc = ws->acc;
+        ml = ws->ml;
+    } else {
+        if (ctx->attn_acc_bytes < acc_bytes) {
+            HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+            if (ctx->attn_acc) HIP_TRY(ctx, hipFree(ctx->attn_acc));
+            ctx->attn_acc = nullptr; ctx->attn_acc_bytes = 0;
+            HIP_TRY(ctx, hipMalloc(reinterpret_cast<void**>(&ctx->attn_acc), acc_bytes));
+            ctx->attn_acc_bytes = acc_bytes;
+        }
+        if (ctx->attn_ml_bytes < ml_bytes) {
+            HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+            if (ctx->attn_ml) HIP_TRY(ctx, hipFree(ctx->attn_ml));
+            ctx->attn_ml = nullptr; ctx->attn_ml_bytes = 0;
+            HIP_TRY(ctx, hipMalloc(reinterpret_cast<void**>(&ctx->attn_ml), ml_bytes));
+            ctx->attn_ml_bytes = ml_bytes;
+        }
+        acc = ctx->attn_acc;
+        ml = ctx->attn_ml;
     }
     AttnLaunch a{q, static_cast<uint32_t>(seq_len), static_cast<uint32_t>(max_seq), scale, n_heads, n_kv_heads, n_queries,
-                 n_heads * head_dim, G, S, n_parts, part_keys, chunks_per_part, batch, new_kv != nullptr, nk};
+                 n_heads * head_dim, G, S, n_parts, part_keys, chunks_per_part, batch, new_kv != nullptr, nk, acc, ml};
     const kv_half *kh = static_cast<const kv_half*>(kc), *vh = static_cast<const kv_half*>(vc);
     const float *kf = static_cast<const float*>(kc), *vf = static_cast<const float*>(vc);
     if (head_dim == 128) {
@@ -643,11 +658,11 @@ cera_hip_status cera_launch_attn(cera_hip_ctx* ctx, const float* q, const void* 
     do {                                                                                                                \
         if (batch)                                                                                                      \
             hipLaunchKernelGGL((attn_prefill_merge_kernel<QQ, HH>), dim3((n_pairs + 7) / 8), dim3(256), 0, ctx->stream,  \
-                               ctx->attn_acc, ctx->attn_ml, n_parts, G, n_heads, n_pairs, out, out_scales, out_quants,  \
+                               acc, ml, n_parts, G, n_heads, n_pairs, out, out_scales, out_quants,                      \
                                out_bsum);                                                                               \
         else                                                                                                            \
-            hipLaunchKernelGGL((attn_decode_merge_kernel<QQ, HH>), mgrid, dim3(256), 0, ctx->stream, ctx->attn_acc,      \
-                               ctx->attn_ml, n_parts, G, n_heads, out, out_scales, out_quants, out_bsum);               \
+            hipLaunchKernelGGL((attn_decode_merge_kernel<QQ, HH>), mgrid, dim3(256), 0, ctx->stream, acc,                \
+                               ml, n_parts, G, n_heads, out, out_scales, out_quants, out_bsum);                         \
     } while (0)
     if (out_quants) { if (head_dim == 128) ATTN_MERGE(true, 128); else ATTN_MERGE(true, 64); }
     else            { if (head_dim == 128) ATTN_MERGE(false, 128); else ATTN_MERGE(false, 64); }

@@ -86,13 +86,20 @@ cera_hip_status cera_launch_attn_decode(cera_hip_ctx* ctx, const float* q, const
                                         uint64_t max_seq, float scale, uint32_t n_splits, float* out,
                                         float* out_scales, int8_t* out_quants, const AttnNewKV* new_kv = nullptr,
                                         bool kv_f16 = false);
+// where the split-K partials of an attention launch go when the caller provides the memory
+struct AttnWorkspace {
+    float* acc;   // [query][kv head][part][group][head_dim]
+    float* ml;    // [query][kv head][part][group][2]
+    uint64_t acc_bytes, ml_bytes;
+};
 // n_queries consecutive queries (causal): query i sees seq_len + i keys; q and the outputs are
-// [n_queries][n_heads*head_dim]
+// [n_queries][n_heads*head_dim].  ws == null: the context's own grow-on-demand workspace.
 cera_hip_status cera_launch_attn(cera_hip_ctx* ctx, const float* q, const void* kc, const void* vc,
                                  uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, uint64_t seq_len,
                                  uint64_t max_seq, float scale, uint32_t n_splits, uint32_t n_queries, float* out,
                                  float* out_scales, int8_t* out_quants, float* out_bsum,
-                                 const AttnNewKV* new_kv = nullptr, bool kv_f16 = false);
+                                 const AttnNewKV* new_kv = nullptr, bool kv_f16 = false,
+                                 const AttnWorkspace* ws = nullptr);
 // One allocation holding the rows of several same-type, same-k matrices back to back
 // (`fused`), plus a non-owning view per part.  Lets the decode step run Q|K(|V) as one GEMV.
 cera_hip_status cera_tensor_upload_concat(cera_hip_ctx* ctx, const cera_hip_tensor* const* parts, int n_parts,
