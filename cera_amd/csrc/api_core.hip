@@ -23,6 +23,29 @@ bool cera_gemv_launch_q4_1(const GemvArgs&, const GemvPlan&, int, bool, hipStrea
 bool cera_gemv_launch_q8_0(const GemvArgs&, const GemvPlan&, int, bool, hipStream_t);
 
 // ---------------------------------------------------------------------------
+// Fixed workspace of the allocation-free attention entry (cera_hip_attn_decode_dev_noalloc): the
+// split-K partials of one decode-attention call.  The array's name is only a host-side handle;
+// its device address is resolved once per device at context creation and that pointer is what
+// kernels receive.  Every GPU holds its own copy until the process ends.
+static __device__ __align__(256) unsigned char scratch[CERA_HIP_NOALLOC_WORKSPACE_BYTES];
+static constexpr uint64_t NOALLOC_ML_BYTES = 128u << 10;   // (m, l) pairs in front, the accumulators behind
+static constexpr int MAX_DEVICES = 64;
+static std::mutex g_scratch_mu;
+static void* g_scratch_ptr[MAX_DEVICES] = {nullptr};
+
+// with `device` current: the address of this device's copy of `scratch`
+static hipError_t resolve_static_scratch(int device, void** out) {
+    std::lock_guard<std::mutex> lk(g_scratch_mu);
+    if (!g_scratch_ptr[device]) {
+        void* p = nullptr;
+        hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return e;
+        g_scratch_ptr[device] = p;
+    }
+    *out = g_scratch_ptr[device];
+    return hipSuccess;
+}
+
 static std::mutex g_err_mu;
 static std::string g_err;
 
@@ -77,12 +100,13 @@ cera_hip_status cera_hip_ctx_create(int device, cera_hip_ctx** out) {
     if (e != hipSuccess || n == 0)
         return cera_fail(nullptr, CERA_HIP_ERR_DEVICE,
                          std::string("no HIP device available: ") + (e != hipSuccess ? hipGetErrorString(e) : "count is 0"));
-    if (device < 0 || device >= n) return cera_fail(nullptr, CERA_HIP_ERR_ARGUMENT, "device index out of range");
+    if (device < 0 || device >= n || device >= MAX_DEVICES) return cera_fail(nullptr, CERA_HIP_ERR_ARGUMENT, "device index out of range");
     cera_hip_ctx* ctx = new (std::nothrow) cera_hip_ctx();
     if (!ctx) return cera_fail(nullptr, CERA_HIP_ERR_OOM, "host allocation failed");
     ctx->device = device;
     hipDeviceProp_t prop;
     if ((e = hipSetDevice(device)) != hipSuccess || (e = hipGetDeviceProperties(&prop, device)) != hipSuccess ||
+        (e = resolve_static_scratch(device, &ctx->static_scratch)) != hipSuccess ||
         (e = hipStreamCreate(&ctx->stream)) != hipSuccess) {
         delete ctx;
         return cera_fail(nullptr, CERA_HIP_ERR_DEVICE, std::string("device init: ") + hipGetErrorString(e));
@@ -897,6 +921,23 @@ cera_hip_status cera_hip_attn_f16kv(cera_hip_ctx* ctx, const float* q, const flo
     std::lock_guard<std::recursive_mutex> op_lk(ctx->op_mu);
     if (n_queries == 0 || n_kv_heads == 0 || head_dim == 0) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "attn_f16kv: empty input");
     return attn_host(ctx, q, k, v, n_heads, n_kv_heads, head_dim, start_pos, n_queries, scale, n_splits, out, true);
+}
+
+// cera_hip_attn_decode_dev without any allocation: the partials go to this device's copy of the
+// static array above, through the pointer resolved at context creation.  Nothing in it has to
+// start at zero (every part writes its (m, l, o) before the merge reads them), so nothing is
+// cleared; calls that overlap on one GPU would share the array and race.
+cera_hip_status cera_hip_attn_decode_dev_noalloc(cera_hip_ctx* ctx, const float* q, const float* k, const float* v,
+                                                 uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, uint64_t seq_len,
+                                                 uint64_t max_seq, float scale, uint32_t n_splits, float* out) {
+    if (!ctx || !q || !k || !v || !out) return CERA_HIP_ERR_ARGUMENT;
+    std::lock_guard<std::recursive_mutex> op_lk(ctx->op_mu);
+    if (!ctx->static_scratch) return cera_fail(ctx, CERA_HIP_ERR_DEVICE, "attn_decode_dev_noalloc: the static workspace was not resolved");
+    unsigned char* base = static_cast<unsigned char*>(ctx->static_scratch);
+    const AttnWorkspace ws{reinterpret_cast<float*>(base + NOALLOC_ML_BYTES), reinterpret_cast<float*>(base),
+                           CERA_HIP_NOALLOC_WORKSPACE_BYTES - NOALLOC_ML_BYTES, NOALLOC_ML_BYTES};
+    return cera_launch_attn(ctx, q, k, v, n_heads, n_kv_heads, head_dim, seq_len, max_seq, scale, n_splits, 1, out, nullptr,
+                            nullptr, nullptr, nullptr, false, &ws);
 }
 
 cera_hip_status cera_hip_attn_decode_f16_dev(cera_hip_ctx* ctx, const float* q, const void* k16, const void* v16,

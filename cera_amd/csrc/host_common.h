@@ -32,6 +32,7 @@ struct cera_hip_ctx {
     // grow-only device scratch for the host-pointer entry points
     void* scratch[12] = {nullptr};
     uint64_t scratch_bytes[12] = {0};
+    void* static_scratch = nullptr;   // this device's copy of the library's fixed workspace (resolved at creation)
     // attention split-K workspace
     float* attn_acc = nullptr;
     float* attn_ml = nullptr;

@@ -32,7 +32,7 @@ SYMBOLS = [
     "cera_hip_read_kv", "cera_hip_read_hidden",
     "cera_hip_gemv_reference_order", "cera_hip_attn_decode_reference_order", "cera_hip_rmsnorm_reference_order",
     "cera_hip_set_reference_order", "cera_hip_reference_order",
-    "cera_hip_rmsnorm_q8_0", "cera_hip_attn_decode_step",
+    "cera_hip_rmsnorm_q8_0", "cera_hip_attn_decode_step", "cera_hip_attn_decode_dev_noalloc",
 ]
 
 
@@ -136,6 +136,7 @@ def load_library() -> C.CDLL:
         "cera_hip_attn_decode_reference_order": (i32, [vp, vp, vp, vp, u32, u32, u32, u64, f32, vp]),
         "cera_hip_rmsnorm_reference_order": (i32, [vp, vp, vp, u64, f32, vp]),
         "cera_hip_set_reference_order": (i32, [vp, u32]), "cera_hip_reference_order": (u32, [vp]),
+        "cera_hip_attn_decode_dev_noalloc": (i32, [vp, vp, vp, vp, u32, u32, u32, u64, u64, f32, u32, vp]),
         "cera_hip_rmsnorm_q8_0": (i32, [vp, vp, vp, u64, f32, vp, vp, vp]),
         "cera_hip_attn_decode_step": (i32, [vp, vp, vp, vp, vp, vp, u32, u32, u32, u32, f32, u32, vp, f32, u32,
                                             vp, vp, vp, vp, vp]),

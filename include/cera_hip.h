@@ -306,6 +306,21 @@ CERA_HIP_API cera_hip_status cera_hip_attn_decode_dev(cera_hip_ctx*, const float
                                                       const float* v_headmajor, uint32_t n_heads,
                                                       uint32_t n_kv_heads, uint32_t head_dim, uint64_t seq_len,
                                                       uint64_t max_seq, float scale, uint32_t n_splits, float* out);
+/* cera_hip_attn_decode_dev for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid it).  No counterpart in the reference.  The
+ * split-K partials go to a fixed CERA_HIP_NOALLOC_WORKSPACE_BYTES array inside the library (one
+ * per GPU, held until the process ends) instead of the context's grow-on-demand workspace, and
+ * the call allocates and frees nothing.  Same arguments and the same result, bit for bit, as
+ * cera_hip_attn_decode_dev.  A shape whose partials do not fit -- n_heads * parts * head_dim * 4
+ * bytes beyond the array less 128 KiB, parts being n_splits or the library's choice (about
+ * 4 * CUs / n_kv_heads, at most one per 8 keys) -- is CERA_HIP_ERR_SHAPE.  Every call on a GPU
+ * shares that GPU's array: calls that overlap on one GPU (two contexts, two streams) race. */
+#define CERA_HIP_NOALLOC_WORKSPACE_BYTES (4u << 20)
+CERA_HIP_API cera_hip_status cera_hip_attn_decode_dev_noalloc(cera_hip_ctx*, const float* q, const float* k_headmajor,
+                                                              const float* v_headmajor, uint32_t n_heads,
+                                                              uint32_t n_kv_heads, uint32_t head_dim, uint64_t seq_len,
+                                                              uint64_t max_seq, float scale, uint32_t n_splits,
+                                                              float* out);
 /* k, v: device, head-major IEEE half [n_kv_heads][max_seq][head_dim] */
 CERA_HIP_API cera_hip_status cera_hip_attn_decode_f16_dev(cera_hip_ctx*, const float* q, const void* k_headmajor_f16,
                                                           const void* v_headmajor_f16, uint32_t n_heads,
