@@ -322,3 +322,77 @@ def test_batched_prefill_when_k_is_not_a_multiple_of_256(hip, orc, n):
     for i, t in enumerate([3, 4, 5]):
         assert _cos(rows[i], om.forward(t, n + i)) > 0.999, i
     gm.close(); om.close()
+
+
+# ---- config 3 at the shapes the benchmark times ---------------------------------------------------
+def _row_sample_check(hip, orc, dtype, w, m, k, x, n, rows):
+    out = hip.gemm(dtype, w, x, m, n, k)
+    rb = util.H.row_bytes(dtype, k)
+    wr = np.ascontiguousarray(w.reshape(m, rb)[rows]).reshape(-1)
+    ref = _oracle_gemm(orc, dtype, wr, x, rows.size, n, k)
+    err = np.abs(out[rows].astype(np.float64) - ref).max()
+    assert err <= GEMM_TOL * util.rms(ref), (err, util.rms(ref))
+    return out
+
+
+@pytest.mark.parametrize("dtype,m,k", [(Q4_K, 14336, 4096), (Q4_K, 6144, 4096)])
+@pytest.mark.parametrize("n", [128, 512, 2048])
+def test_gemm_config3_gate_and_qkv_shapes(hip, orc, dtype, m, k, n):
+    """The gate/up projection (the shape the benchmark times) and the fused QKV height."""
+    _say(f"gemm config 3 {util.NAMES[dtype]} m={m} n={n} k={k}")
+    w, _ = util.make_weights(dtype, m, k, seed=11)
+    x = util.rng(n + 1).standard_normal((n, k)).astype(np.float32)
+    rows = np.unique(np.concatenate([np.arange(8), util.rng(2).integers(0, m, 48), np.arange(m - 8, m)]))
+    _row_sample_check(hip, orc, dtype, w, m, k, x, n, rows)
+
+
+@pytest.fixture(scope="module")
+def head_q6k():
+    m, k = 128256, 4096
+    w, _ = util.make_weights(Q6_K, m, k, seed=12)
+    return w, m, k
+
+
+@pytest.mark.parametrize("n", [128, 512, 2048])
+def test_gemm_config3_vocabulary_head(hip, orc, head_q6k, n):
+    """The Q6_K output head 128256 x 4096 (the all-position logits GEMM), row-sampled."""
+    w, m, k = head_q6k
+    _say(f"gemm config 3 Q6_K head m={m} n={n} k={k}")
+    x = util.rng(n + 2).standard_normal((n, k)).astype(np.float32)
+    rows = np.unique(np.concatenate([np.arange(4), util.rng(3).integers(0, m, 40), np.arange(m - 4, m)]))
+    _row_sample_check(hip, orc, Q6_K, w, m, k, x, n, rows)
+
+
+@pytest.mark.parametrize("n", [128, 512, 2048])
+def test_gemm_swiglu_at_ffn_shape_against_the_oracle(hip, orc, n):
+    """The prefill pass's fused gate | up | SwiGLU | Q8_0 launch at 14336 x 4096, against the
+    oracle's own chain gemm_preq -> silu_mul_inplace -> quantize_columns (transformer.rs:710-788,
+    cpu.rs:2570-2575, transformer.rs:865-946) on a sample of 32-row quantization blocks.  The GEMM
+    outputs agree with the oracle's to the float bar only, so a value that sits on a rounding
+    boundary may land one int8 step away and a block maximum may round to the neighbouring f16
+    scale: the dequantized result must meet the oracle's SwiGLU output within one quantization
+    step, codes may differ by at most one step and only rarely, scales by at most one f16 ulp."""
+    m, k = 14336, 4096
+    _say(f"gemm_swiglu 14336x4096 vs oracle n={n}")
+    wg, _ = util.make_weights(Q4_K, m, k, seed=51)
+    wu, _ = util.make_weights(Q4_K, m, k, seed=52)
+    x = util.rng(53 + n).standard_normal((n, k)).astype(np.float32)
+    q, sc, fused = hip.gemm_swiglu(Q4_K, wg, wu, m, x, n, k)
+    assert fused == (n >= 512), "small batches take the pair + SwiGLU kernels, large ones the fused launch"
+    blocks = np.unique(np.concatenate([[0, 1, m // 32 - 1], util.rng(4).integers(0, m // 32, 5)]))
+    rows = (blocks[:, None] * 32 + np.arange(32)[None, :]).reshape(-1)
+    rb = util.H.row_bytes(Q4_K, k)
+    g = _oracle_gemm(orc, Q4_K, np.ascontiguousarray(wg.reshape(m, rb)[rows]).reshape(-1), x, rows.size, n, k)
+    u = _oracle_gemm(orc, Q4_K, np.ascontiguousarray(wu.reshape(m, rb)[rows]).reshape(-1), x, rows.size, n, k)
+    h = orc.silu_mul(np.ascontiguousarray(g.T).reshape(-1), np.ascontiguousarray(u.T).reshape(-1)).reshape(n, rows.size)
+    rs, rq = orc.quantize_q8_0(h.reshape(-1))
+    rs, rq = rs.reshape(n, blocks.size), rq.reshape(n, rows.size)
+    gq, gs = q[:, rows], sc[:, blocks]
+    dq = np.abs(gq.astype(np.int32) - rq.astype(np.int32))
+    assert dq.max() <= 1, int(dq.max())
+    assert np.count_nonzero(dq) <= 0.02 * dq.size, np.count_nonzero(dq) / dq.size
+    ulp = np.abs(gs.astype(np.float16).view(np.int16).astype(np.int32) - rs.astype(np.float16).view(np.int16).astype(np.int32))
+    assert np.array_equal(gs, gs.astype(np.float16).astype(np.float32)) and ulp.max() <= 1
+    deq = gq.astype(np.float32).reshape(n, blocks.size, 32) * gs[:, :, None]
+    step = rs[:, :, None]
+    assert (np.abs(deq - h.reshape(n, blocks.size, 32)) <= 1.01 * step + 1e-9).all()
