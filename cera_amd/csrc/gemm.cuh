@@ -78,6 +78,9 @@ struct GemmArgs {
     int8_t* hq;
     float* hs;
     float* hbsum;
+    // debug instances only: the integer dot of every (row, token, block) as the matrix core
+    // delivered it, [m][n][k/32] int32 (Q6_K: [m][n][k/16], f32 bit patterns of the f16 MFMA's result)
+    int32_t* dbg_dots;
 };
 
 // ---- per-type staging of one 128-element K tile of one row -------------------
@@ -227,7 +230,7 @@ struct GemmQ8_0 {
 // factors of an output of the FFN's first half then sit in the same lane and register index, a
 // 32-row Q8_0 block of one token in the two lanes of a column, and the activation of the down
 // projection is quantized straight from the accumulators.
-template <class T, bool SWIGLU = false>
+template <class T, bool SWIGLU = false, bool DBG = false>
 static __global__ __launch_bounds__(256, T::WAVES_PER_SIMD) void gemm_kernel(GemmArgs p) {
     constexpr int NB = GEMM_KT / 32;  // 32-blocks per tile
     __shared__ __attribute__((aligned(16))) int8_t sA[GEMM_BM * GEMM_LDA];
@@ -349,6 +352,15 @@ static __global__ __launch_bounds__(256, T::WAVES_PER_SIMD) void gemm_kernel(Gem
                         v16i c = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
                         c = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, bf[jb], c, 0, 0, 0);
                         // rows held by this lane: 8*blk + 4*half + r, blk = 0..3, r = 0..3
+                        if (DBG) {
+                            const uint32_t dtok = n0 + wn * 32 + col, dblk = k0 / 32 + 2 * pr + jb;
+#pragma unroll
+                            for (int e = 0; e < 16; ++e) {
+                                const uint32_t drow = m0 + arow0 + t * arow_step + (e >> 2) * 8 + half * 4 + (e & 3);
+                                if (drow < mrows && dtok < p.n)
+                                    p.dbg_dots[(static_cast<uint64_t>(drow) * p.n + dtok) * nb32 + dblk] = c[e];
+                            }
+                        }
 #pragma unroll
                         for (int e = 0; e < 16; ++e) acc[t][e] = fmaf(static_cast<float>(c[e]), sc[16 * jb + e], acc[t][e]);
                     }

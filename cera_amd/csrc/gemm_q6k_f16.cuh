@@ -55,6 +55,7 @@ static __global__ __launch_bounds__(256) void gemm_act_f16_kernel(const uint4* _
 // byte offset of 16-byte chunk `chunk` of staged row `row`
 __device__ __forceinline__ uint32_t gq_off(uint32_t row, uint32_t chunk) { return row * GQ_LD + (chunk << 4); }
 
+template <bool DBG = false>
 static __global__ __launch_bounds__(256, 2) void gemm_q6k_f16_kernel(GemmArgs p) {
     constexpr int NB = GEMM_KT / 32;
     __shared__ __attribute__((aligned(16))) uint8_t sA[GEMM_BM * GQ_LD];
@@ -177,6 +178,19 @@ static __global__ __launch_bounds__(256, 2) void gemm_q6k_f16_kernel(GemmArgs p)
                 v16f z = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
                 const v16f c0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(af0, bf0, z, 0, 0, 0);
                 const v16f c1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(af1, bf1, z, 0, 0, 0);
+                if (DBG) {
+                    const uint32_t dtok = n0 + wn * 32 + col, dgrp = 2 * (k0 / 32 + b);
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) {
+                        const uint32_t drow = m0 + wm * 64 + t * 32 + (e >> 2) * 8 + half * 4 + (e & 3);
+                        if (drow < mrows && dtok < p.n) {
+                            int32_t* d = p.dbg_dots + (static_cast<uint64_t>(drow) * p.n + dtok) * (2 * nb32) + dgrp;
+                            const float v0 = c0[e], v1 = c1[e];   // (a bit_cast of the element expression itself reads element 0)
+                            d[0] = __float_as_int(v0);
+                            d[1] = __float_as_int(v1);
+                        }
+                    }
+                }
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {
                     acc[t][e] = fmaf(c0[e], sc[e], acc[t][e]);

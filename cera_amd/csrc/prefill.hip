@@ -25,7 +25,7 @@ cera_hip_status cera_launch_gemm(cera_hip_ctx* ctx, const cera_hip_dtensor* w, c
                                  const float* bsum, uint32_t n, float* out, uint64_t ld_m, uint64_t ld_n,
                                  const float* resid, float resid_scale, const cera_hip_dtensor* w2 = nullptr,
                                  float* out2 = nullptr, uint64_t ld_n2 = 0, bool* paired = nullptr, void* bh_ws = nullptr,
-                                 bool* staged = nullptr) {
+                                 bool* staged = nullptr, int32_t* dbg_dots = nullptr) {
     if (!cera_gemm_supports(w->dtype, w->k))
         return cera_fail(ctx, CERA_HIP_ERR_UNSUPPORTED_DTYPE,
                          "gemm: no int8 GEMM for ggml type " + std::to_string(w->dtype) + " with k=" + std::to_string(w->k));
@@ -35,6 +35,7 @@ cera_hip_status cera_launch_gemm(cera_hip_ctx* ctx, const cera_hip_dtensor* w, c
     a.m = static_cast<uint32_t>(w->m); a.n = n; a.k = static_cast<uint32_t>(w->k);
     a.row_bytes = static_cast<uint32_t>(w->row_bytes);
     a.ld_m = ld_m; a.ld_n = ld_n; a.resid = resid; a.resid_scale = resid_scale;
+    a.hq = nullptr; a.hs = nullptr; a.hbsum = nullptr; a.dbg_dots = dbg_dots;
     // Q6_K runs its block dots on the f16 matrix cores and reads the quants as f16: converted here
     // unless the caller says its workspace (bh_ws) still holds these activations (*staged)
     a.bh = nullptr;
@@ -67,7 +68,7 @@ cera_hip_status cera_launch_gemm(cera_hip_ctx* ctx, const cera_hip_dtensor* w, c
     uint32_t split = 1;
     const uint32_t wgs = grid.x * grid.y, nsb = a.k / GEMM_KSUPER;
     const bool dense = (ld_m == 1 && ld_n == a.m) || (ld_n == 1 && ld_m == n);
-    if (wgs < 2 * ctx->n_cu && nsb >= 8 && dense && (static_cast<uint64_t>(a.m) * n) % 4 == 0) {
+    if (!dbg_dots && wgs < 2 * ctx->n_cu && nsb >= 8 && dense && (static_cast<uint64_t>(a.m) * n) % 4 == 0) {
         // smallest divisor of the super-block count that gives at least two workgroups per CU
         const uint32_t want = std::min<uint32_t>(8, (2 * ctx->n_cu + wgs - 1) / wgs);
         for (uint32_t d = 2; d <= 8 && split < want; ++d)
@@ -86,9 +87,21 @@ cera_hip_status cera_launch_gemm(cera_hip_ctx* ctx, const cera_hip_dtensor* w, c
         a.resid = nullptr;
         grid.z = split;
     }
+    if (dbg_dots) {
+        // the same kernels, compiled to also store every block's integer tile (no K split, no pair)
+        switch (w->dtype) {
+            case CERA_HIP_Q4_K: hipLaunchKernelGGL((gemm_kernel<GemmQ4K, false, true>), grid, dim3(256), 0, ctx->stream, a); break;
+            case CERA_HIP_Q6_K: hipLaunchKernelGGL(gemm_q6k_f16_kernel<true>, grid, dim3(256), 0, ctx->stream, a); break;
+            case CERA_HIP_Q4_0: hipLaunchKernelGGL((gemm_kernel<GemmQ4_0, false, true>), grid, dim3(256), 0, ctx->stream, a); break;
+            case CERA_HIP_Q4_1: hipLaunchKernelGGL((gemm_kernel<GemmQ4_1, false, true>), grid, dim3(256), 0, ctx->stream, a); break;
+            default: hipLaunchKernelGGL((gemm_kernel<GemmQ8_0, false, true>), grid, dim3(256), 0, ctx->stream, a); break;
+        }
+        HIP_TRY(ctx, hipGetLastError());
+        return CERA_HIP_OK;
+    }
     switch (w->dtype) {
         case CERA_HIP_Q4_K: hipLaunchKernelGGL((gemm_kernel<GemmQ4K>), grid, dim3(256), 0, ctx->stream, a); break;
-        case CERA_HIP_Q6_K: hipLaunchKernelGGL(gemm_q6k_f16_kernel, grid, dim3(256), 0, ctx->stream, a); break;
+        case CERA_HIP_Q6_K: hipLaunchKernelGGL(gemm_q6k_f16_kernel<false>, grid, dim3(256), 0, ctx->stream, a); break;
         case CERA_HIP_Q4_0: hipLaunchKernelGGL((gemm_kernel<GemmQ4_0>), grid, dim3(256), 0, ctx->stream, a); break;
         case CERA_HIP_Q4_1: hipLaunchKernelGGL((gemm_kernel<GemmQ4_1>), grid, dim3(256), 0, ctx->stream, a); break;
         default: hipLaunchKernelGGL((gemm_kernel<GemmQ8_0>), grid, dim3(256), 0, ctx->stream, a); break;
@@ -173,6 +186,44 @@ extern "C" cera_hip_status cera_hip_gemm(cera_hip_ctx* ctx, const cera_hip_tenso
         CERA_TRY(cera_hip_upload(ctx, dx, x, n * w->k * 4));
         CERA_TRY(cera_hip_gemm_dev(ctx, w, static_cast<float*>(dx), n, static_cast<float*>(dy)));
         return cera_hip_download(ctx, out, dy, n * w->m * 4);
+    };
+    cera_hip_status st = run();
+    cera_hip_tensor_free(ctx, w);
+    return st;
+}
+
+// The GEMM's integer block dots as the matrix cores deliver them (debug instances of the same
+// kernels): dots [m][n][k/32] int32 -- Q4_0 sum (q-8)a, Q8_0 sum w a, Q4_1 / Q4_K sum q a -- and
+// for Q6_K [m][n][k/16], each the f32 result of the f16 MFMA for one 16-element scale group,
+// sum (q-32)a, returned as f32 so that a test can see it is an exact integer.  out (nullable)
+// receives the float result of the same launch.
+extern "C" cera_hip_status cera_hip_gemm_block_dots(cera_hip_ctx* ctx, const cera_hip_tensor* t, const float* x, uint64_t n,
+                                                    int32_t* dots, float* out) {
+    if (!ctx || !t || !x || !dots) return CERA_HIP_ERR_ARGUMENT;
+    std::lock_guard<std::recursive_mutex> op_lk(ctx->op_mu);
+    if (n == 0 || n > 0x7FFFFFFFull) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "gemm_block_dots: bad n");
+    const uint64_t per = t->ggml_type == CERA_HIP_Q6_K ? t->k / 16 : t->k / 32;
+    if (t->m * n * per > (64ull << 20)) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "gemm_block_dots: more than 64 Mi block dots; use a smaller shape");
+    cera_hip_dtensor* w = nullptr;
+    CERA_TRY(cera_hip_tensor_upload(ctx, t, &w));
+    auto run = [&]() -> cera_hip_status {
+        if (!cera_gemm_supports(w->dtype, w->k))
+            return cera_fail(ctx, CERA_HIP_ERR_UNSUPPORTED_DTYPE, "gemm_block_dots: no int8 GEMM for this type / k");
+        void *dx, *dy, *ds, *dq, *db, *dd;
+        CERA_TRY(cera_scratch(ctx, 0, n * w->k * 4, &dx));
+        CERA_TRY(cera_scratch(ctx, 3, n * w->m * 4, &dy));
+        CERA_TRY(cera_scratch(ctx, 1, n * (w->k / 32) * 4, &ds));
+        CERA_TRY(cera_scratch(ctx, 2, n * w->k, &dq));
+        CERA_TRY(cera_scratch(ctx, 7, n * (w->k / 32) * 4, &db));
+        CERA_TRY(cera_scratch(ctx, 4, w->m * n * per * 4, &dd));
+        CERA_TRY(cera_hip_upload(ctx, dx, x, n * w->k * 4));
+        CERA_TRY(quantize_rows(ctx, static_cast<float*>(dx), n, w->k, static_cast<float*>(ds), static_cast<int8_t*>(dq), static_cast<float*>(db)));
+        CERA_TRY(cera_launch_gemm(ctx, w, static_cast<float*>(ds), static_cast<int8_t*>(dq), static_cast<float*>(db),
+                                  static_cast<uint32_t>(n), static_cast<float*>(dy), n, 1, nullptr, 1.0f, nullptr, nullptr, 0,
+                                  nullptr, nullptr, nullptr, static_cast<int32_t*>(dd)));
+        CERA_TRY(cera_hip_download(ctx, dots, dd, w->m * n * per * 4));
+        if (out) CERA_TRY(cera_hip_download(ctx, out, dy, n * w->m * 4));
+        return CERA_HIP_OK;
     };
     cera_hip_status st = run();
     cera_hip_tensor_free(ctx, w);

@@ -32,7 +32,7 @@ SYMBOLS = [
     "cera_hip_read_kv", "cera_hip_read_hidden",
     "cera_hip_gemv_reference_order", "cera_hip_attn_decode_reference_order", "cera_hip_rmsnorm_reference_order",
     "cera_hip_set_reference_order", "cera_hip_reference_order",
-    "cera_hip_rmsnorm_q8_0", "cera_hip_attn_decode_step", "cera_hip_attn_decode_dev_noalloc",
+    "cera_hip_rmsnorm_q8_0", "cera_hip_attn_decode_step", "cera_hip_attn_decode_dev_noalloc", "cera_hip_gemm_block_dots",
 ]
 
 
@@ -137,6 +137,7 @@ def load_library() -> C.CDLL:
         "cera_hip_rmsnorm_reference_order": (i32, [vp, vp, vp, u64, f32, vp]),
         "cera_hip_set_reference_order": (i32, [vp, u32]), "cera_hip_reference_order": (u32, [vp]),
         "cera_hip_attn_decode_dev_noalloc": (i32, [vp, vp, vp, vp, u32, u32, u32, u64, u64, f32, u32, vp]),
+        "cera_hip_gemm_block_dots": (i32, [vp, C.POINTER(Tensor), vp, u64, vp, vp]),
         "cera_hip_rmsnorm_q8_0": (i32, [vp, vp, vp, u64, f32, vp, vp, vp]),
         "cera_hip_attn_decode_step": (i32, [vp, vp, vp, vp, vp, vp, u32, u32, u32, u32, f32, u32, vp, f32, u32,
                                             vp, vp, vp, vp, vp]),
@@ -274,6 +275,16 @@ class Context:
         out = np.empty((m, n), np.float32)
         self.check(self.lib.cera_hip_gemm(self.h, C.byref(t), _p(x), n, _p(out)))
         return out
+
+    def gemm_block_dots(self, ggml_type: int, blocks: np.ndarray, x: np.ndarray, m: int, n: int, k: int):
+        """(dots, out): dots int32 [m][n][k/32], or for Q6_K float32 [m][n][k/16] (the f16 MFMA's results)."""
+        t = make_tensor(ggml_type, m, k, blocks)
+        x = np.ascontiguousarray(x, np.float32).reshape(n, k)
+        per = k // 16 if ggml_type == Q6_K else k // 32
+        dots = np.zeros((m, n, per), np.int32)
+        out = np.empty((m, n), np.float32)
+        self.check(self.lib.cera_hip_gemm_block_dots(self.h, C.byref(t), _p(x), n, _p(dots), _p(out)))
+        return (dots.view(np.float32) if ggml_type == Q6_K else dots), out
 
     def attn_decode(self, q, k, v, n_heads, n_kv_heads, head_dim, seq_len, scale, n_splits=0) -> np.ndarray:
         q = np.ascontiguousarray(q, np.float32)

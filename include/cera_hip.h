@@ -173,6 +173,16 @@ CERA_HIP_API cera_hip_status cera_hip_gemv_pair(cera_hip_ctx*, const cera_hip_te
 CERA_HIP_API cera_hip_status cera_hip_gemm(cera_hip_ctx*, const cera_hip_tensor* w, const float* x, uint64_t n,
                                            float* out);
 
+/* cera_hip_gemm with the integer block dots its matrix-core instructions produced, from debug
+ * instances of the same kernels (the integer quantities cera's own test reference defines,
+ * cera/src/backend/simd.rs:6609-6629): dots [m][n][k/32] int32 -- Q4_0 sum (q-8)a, Q8_0 sum w a,
+ * Q4_1 / Q4_K sum q a, q in 0..15.  Q6_K forms its dots per 16-element scale group on the f16
+ * matrix cores: dots [m][n][k/16], each the f32 bit pattern of that instruction's result,
+ * sum (q-32)a -- an exact integer, which a test can check because it sees the float.  out
+ * (nullable) receives the [m][n] result of the same launch.  At most 64 Mi dots per call. */
+CERA_HIP_API cera_hip_status cera_hip_gemm_block_dots(cera_hip_ctx*, const cera_hip_tensor* w, const float* x, uint64_t n,
+                                                      int32_t* dots, float* out);
+
 /* Two gemm_preq calls on the same quantized activations in one launch, the way the prefill pass
  * issues attn_q | attn_k and ffn_gate | ffn_up (LlamaModel::forward_prefill_batched,
  * cera/src/model/llama.rs:738-1523, multiplies them one after the other): one grid over both

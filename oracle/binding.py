@@ -76,6 +76,12 @@ def lib() -> C.CDLL:
         "orc_block_dots": (i32, [u32, vp, u64, u64, vp, vp, vp]),
         "orc_gemm_preq": (i32, [u32, vp, vp, vp, vp, u64, u64, u64, i32]),
         "orc_gemv": (i32, [u32, vp, vp, vp, u64, u64, i32]),
+        "orc_repack_q4_0_8x8": (i32, [vp, u64, u64, vp, vp]),
+        "orc_repack_q4_k_8x8": (i32, [vp, u64, u64, vp, vp, vp]),
+        "orc_gemm_q4_0_8x8_q8_0": (i32, [vp, vp, vp, vp, vp, u64, u64, u64]),
+        "orc_gemm_q4_k_8x8_q8_0": (i32, [vp, vp, vp, vp, vp, vp, u64, u64, u64]),
+        "orc_gemm_preq_x86": (i32, [u32, vp, vp, vp, vp, u64, u64, u64, i32]),
+        "orc_llama_set_x86_repack": (None, [vp, i32]),
         "orc_gemv_f64ref": (i32, [u32, vp, vp, vp, u64, u64]),
         "orc_have_avx2": (i32, []),
         "orc_pool_create": (vp, [i32]), "orc_pool_destroy": (None, [vp]), "orc_pool_threads": (i32, [vp]),
@@ -200,6 +206,43 @@ def gemm_preq(dtype: int, w: np.ndarray, b_scales: np.ndarray, b_quants: np.ndar
     out = np.empty((m, n), np.float32)
     v = default_variant() if variant is None else variant
     rc = lib().orc_gemm_preq(dtype, _p(w), _p(bs), _p(bq), _p(out), m, n, k, v)
+    assert rc == 0, rc
+    return out
+
+
+def gemm_preq_x86(dtype: int, w: np.ndarray, bs: np.ndarray, bq: np.ndarray, m: int, n: int, k: int,
+                  variant: int | None = None) -> np.ndarray:
+    """transformer::gemm_preq as an x86 host runs it: repacked 8x8 kernels for Q4_0 / Q4_K weights
+    with m % 8 == 0, the standard layout otherwise.  out [m][n]."""
+    w = np.ascontiguousarray(w.reshape(-1).view(np.uint8))
+    bs = np.ascontiguousarray(bs, np.float32); bq = np.ascontiguousarray(bq, np.int8)
+    out = np.empty((m, n), np.float32)
+    v = default_variant() if variant is None else variant
+    rc = lib().orc_gemm_preq_x86(dtype, _p(w), _p(bs), _p(bq), _p(out), m, n, k, v)
+    assert rc == 0, rc
+    return out
+
+
+def repack_8x8(dtype: int, w: np.ndarray, m: int, k: int):
+    """(packed, scales) for Q4_0, (packed, dsc, dmn) for Q4_K."""
+    w = np.ascontiguousarray(w.reshape(-1).view(np.uint8))
+    packed = np.empty((m // 8) * (k // 32) * 128, np.uint8)
+    a = np.empty((m // 8) * (k // 32) * 8, np.float32)
+    if dtype == Q4_0:
+        assert lib().orc_repack_q4_0_8x8(_p(w), m, k, _p(packed), _p(a)) == 0
+        return packed, a
+    b = np.empty_like(a)
+    assert lib().orc_repack_q4_k_8x8(_p(w), m, k, _p(packed), _p(a), _p(b)) == 0
+    return packed, a, b
+
+
+def gemm_8x8(dtype: int, repacked, bs: np.ndarray, bq: np.ndarray, m: int, n: int, k: int) -> np.ndarray:
+    bs = np.ascontiguousarray(bs, np.float32); bq = np.ascontiguousarray(bq, np.int8)
+    out = np.empty((m, n), np.float32)
+    if dtype == Q4_0:
+        rc = lib().orc_gemm_q4_0_8x8_q8_0(_p(repacked[0]), _p(repacked[1]), _p(bs), _p(bq), _p(out), m, n, k)
+    else:
+        rc = lib().orc_gemm_q4_k_8x8_q8_0(_p(repacked[0]), _p(repacked[1]), _p(repacked[2]), _p(bs), _p(bq), _p(out), m, n, k)
     assert rc == 0, rc
     return out
 
@@ -367,6 +410,10 @@ class Llama:
 
     def truncate(self, n: int):
         lib().orc_llama_truncate(self.h, n)
+
+    def set_x86_repack(self, on: bool = True):
+        """Batched prefill GEMMs through the repacked 8x8 kernels where cera's x86 build uses them."""
+        lib().orc_llama_set_x86_repack(self.h, 1 if on else 0)
 
     def set_kv_f16(self, on: bool = True):
         """KvCompression::F16: K/V rows are rounded through IEEE half when appended."""

@@ -78,6 +78,17 @@ ORC_API int orc_block_dots(uint32_t dtype, const void* w, uint64_t m, uint64_t k
 ORC_API int orc_gemm_preq(uint32_t dtype, const void* w, const float* b_scales,
                           const int8_t* b_quants, float* out, uint64_t m, uint64_t n,
                           uint64_t k, int variant);
+// The x86 prefill route for repacked weights (orc_repack.cpp): repack_q4_0_8x8 / repack_q4_k_8x8
+// (cpu.rs:1145-1196, 1282-1358), gemm_q4_0_8x8_q8_0 / gemm_q4_k_8x8_q8_0 (simd.rs:5215-5518), and
+// transformer::gemm_preq's choice between them and the standard layout (transformer.rs:758-775).
+ORC_API int orc_repack_q4_0_8x8(const uint8_t* src, uint64_t m, uint64_t k, uint8_t* packed, float* scales);
+ORC_API int orc_repack_q4_k_8x8(const uint8_t* src, uint64_t m, uint64_t k, uint8_t* packed, float* dsc, float* dmn);
+ORC_API int orc_gemm_q4_0_8x8_q8_0(const uint8_t* packed, const float* scales, const float* b_scales, const int8_t* b_quants,
+                                   float* out, uint64_t m, uint64_t n, uint64_t k);
+ORC_API int orc_gemm_q4_k_8x8_q8_0(const uint8_t* packed, const float* dsc, const float* dmn, const float* b_scales,
+                                   const int8_t* b_quants, float* out, uint64_t m, uint64_t n, uint64_t k);
+ORC_API int orc_gemm_preq_x86(uint32_t dtype, const void* w, const float* b_scales, const int8_t* b_quants, float* out,
+                              uint64_t m, uint64_t n, uint64_t k, int variant);
 // cpu::gemv_dispatch (cpu.rs:2360): quantizes x to Q8_0 then runs the int8
 // kernel; Q5_K/F32/F16/BF16 take the scalar f32 route on unquantized x.
 ORC_API int orc_gemv(uint32_t dtype, const void* w, const float* x, float* y, uint64_t m,

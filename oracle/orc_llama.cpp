@@ -24,6 +24,9 @@ struct OrcLlama {
     // caches here keep the widened values: same numbers, one code path.
     bool kv_f16 = false;
     int variant = 0;
+    // batched prefill GEMMs through transformer::gemm_preq's x86 route: Q4_0 / Q4_K weights that
+    // cera repacks at load take the 8-row-interleaved kernels (orc_repack.cpp)
+    bool x86_repack = false;
     void* pool = nullptr;  // optional worker pool for the GEMVs (timing only)
 };
 
@@ -48,6 +51,7 @@ OrcLlama* orc_llama_create(const OrcLlamaConfig* cfg, const OrcTensor* embd, con
 void orc_llama_destroy(OrcLlama* m) { delete m; }
 void orc_llama_set_pool(OrcLlama* m, void* pool) { m->pool = pool; }
 void orc_llama_set_kv_f16(OrcLlama* m, int on) { m->kv_f16 = on != 0; }
+void orc_llama_set_x86_repack(OrcLlama* m, int on) { m->x86_repack = on != 0; }
 static void append_kv(const OrcLlama* m, std::vector<float>& cache, const float* row, uint64_t n) {
     if (!m->kv_f16) { cache.insert(cache.end(), row, row + n); return; }
     for (uint64_t i = 0; i < n; ++i) cache.push_back(orc_f16_to_f32(orc_f32_to_f16(row[i])));
@@ -214,13 +218,16 @@ static int gemm_rows(OrcLlama* m, const OrcTensor& t, const std::vector<float>& 
             uint64_t r0 = std::min<uint64_t>(j.t->m, tiles * uint64_t(tid) / uint64_t(nt) * 8);
             uint64_t r1 = std::min<uint64_t>(j.t->m, tiles * uint64_t(tid + 1) / uint64_t(nt) * 8);
             if (r1 <= r0) return;
-            int e = orc_gemm_preq(j.t->dtype, static_cast<const uint8_t*>(j.t->data) + r0 * j.rb, j.bs, j.bq,
-                                  j.tmp + r0 * j.n, r1 - r0, j.n, j.t->k, j.m->variant);
+            // a weight is repacked as a whole (m % 8 == 0); the ranges here are whole 8-row tiles
+            auto fn = (j.m->x86_repack && j.t->m % 8 == 0) ? orc_gemm_preq_x86 : orc_gemm_preq;
+            int e = fn(j.t->dtype, static_cast<const uint8_t*>(j.t->data) + r0 * j.rb, j.bs, j.bq,
+                       j.tmp + r0 * j.n, r1 - r0, j.n, j.t->k, j.m->variant);
             if (e) j.rc = e;
         }, &job);
         rc = job.rc;
     } else {
-        rc = orc_gemm_preq(t.dtype, t.data, bs.data(), bq.data(), tmp.data(), t.m, n, t.k, m->variant);
+        auto fn = m->x86_repack ? orc_gemm_preq_x86 : orc_gemm_preq;
+        rc = fn(t.dtype, t.data, bs.data(), bq.data(), tmp.data(), t.m, n, t.k, m->variant);
     }
     if (rc) return rc;
     out_rows.resize(size_t(n) * t.m);

@@ -32,6 +32,8 @@ ORC_API OrcLlama* orc_llama_create(const OrcLlamaConfig* cfg, const OrcTensor* e
 ORC_API void     orc_llama_destroy(OrcLlama*);
 ORC_API void     orc_llama_set_pool(OrcLlama*, void* pool);
 ORC_API void     orc_llama_set_kv_f16(OrcLlama*, int on);  // KvCompression::F16; set before the first forward
+// batched prefill through the x86 route of transformer::gemm_preq (repacked Q4_0 / Q4_K weights)
+ORC_API void     orc_llama_set_x86_repack(OrcLlama*, int on);
 ORC_API uint32_t orc_llama_seq_len(const OrcLlama*);
 ORC_API void     orc_llama_truncate(OrcLlama*, uint32_t len);
 ORC_API int      orc_llama_forward(OrcLlama*, uint32_t token, uint32_t pos, float* logits /*nullable*/,

@@ -396,3 +396,48 @@ def test_gemm_swiglu_at_ffn_shape_against_the_oracle(hip, orc, n):
     deq = gq.astype(np.float32).reshape(n, blocks.size, 32) * gs[:, :, None]
     step = rs[:, :, None]
     assert (np.abs(deq - h.reshape(n, blocks.size, 32)) <= 1.01 * step + 1e-9).all()
+
+
+# ---- the GEMM's integer block dots, and the route an x86 host really runs ------------------------
+@pytest.mark.parametrize("dtype", util.INT8_TYPES)
+@pytest.mark.parametrize("m,n,k", [(130, 70, 512), (64, 33, 1024), (9, 1, 256), (200, 5, 2048)])
+def test_gemm_integer_block_dots_bit_exact(hip, orc, dtype, m, n, k):
+    """Every (row, token, block) integer dot the matrix cores produce inside the prefill GEMM equals
+    the brute-force integer reference (the quantities of simd.rs:6609-6629): int32 tiles of the
+    int8 MFMA for Q4_0 / Q8_0 / Q4_1 / Q4_K, and for Q6_K the f32 results of the f16 MFMA, one per
+    16-element scale group, which must be exact integers sum (q - 32) a."""
+    _say(f"gemm block dots {util.NAMES[dtype]} m={m} n={n} k={k}")
+    w, _ = util.make_weights(dtype, m, k, seed=dtype + m)
+    x = util.rng(n + k).standard_normal((n, k)).astype(np.float32) * np.float32(3.0)
+    dots, out = hip.gemm_block_dots(dtype, w, x, m, n, k)
+    for j in range(n):
+        _, xq = orc.quantize_q8_0(x[j])
+        ref, asums = orc.block_dots(dtype, w, m, k, xq)
+        if dtype == Q6_K:
+            want = (ref - 32 * asums[None, :]).astype(np.float32)     # the kernel recentres the codes
+            assert np.array_equal(dots[:, j, :], want), j
+        else:
+            assert np.array_equal(dots[:, j, :], ref), j
+    ref_out = _oracle_gemm(orc, dtype, w, x, m, n, k)
+    assert np.abs(out.astype(np.float64) - ref_out).max() <= GEMM_TOL * util.rms(ref_out)
+
+
+@pytest.mark.parametrize("dtype,m,k,n", [(Q4_K, 14336, 4096, 512), (Q4_K, 4096, 4096, 128), (Q4_K, 6144, 4096, 2048),
+                                         (Q4_0, 4096, 4096, 512)])
+def test_gemm_against_the_x86_repacked_route(hip, orc, dtype, m, k, n):
+    """cera on an x86 host multiplies repacked Q4_0 / Q4_K weights with the 8-row-interleaved
+    kernels (gemm_q4_k_8x8_q8_0, cera/src/backend/simd.rs:5392-5518), not the standard-layout
+    ones: the HIP GEMM meets the float bar against that route too (whole 8-row super-rows sampled)."""
+    _say(f"gemm vs x86 8x8 route {util.NAMES[dtype]} m={m} n={n} k={k}")
+    w, _ = util.make_weights(dtype, m, k, seed=21)
+    x = util.rng(n + 9).standard_normal((n, k)).astype(np.float32)
+    out = hip.gemm(dtype, w, x, m, n, k)
+    srs = np.unique(np.concatenate([[0, m // 8 - 1], util.rng(6).integers(0, m // 8, 6)]))
+    rows = (srs[:, None] * 8 + np.arange(8)[None, :]).reshape(-1)
+    rb = util.H.row_bytes(dtype, k)
+    wr = np.ascontiguousarray(w.reshape(m, rb)[rows]).reshape(-1)
+    bs = np.empty((n, k // 32), np.float32); bq = np.empty((n, k), np.int8)
+    for j in range(n):
+        bs[j], bq[j] = orc.quantize_q8_0(x[j])
+    ref = orc.gemm_preq_x86(dtype, wr, bs, bq, rows.size, n, k)
+    assert np.abs(out[rows].astype(np.float64) - ref).max() <= GEMM_TOL * util.rms(ref)
