@@ -395,6 +395,9 @@ cera_hip_status cera_launch_quantize(cera_hip_ctx* ctx, const float* x, uint64_t
     return CERA_HIP_OK;
 }
 
+// weights per lane unit of the decode GEMV kernels
+static uint32_t cera_gemv_unit_elems(uint32_t dtype) { return (dtype == CERA_HIP_Q6_K || dtype == CERA_HIP_Q4_K) ? 64 : 32; }
+
 static bool is_int8_type(uint32_t t) {
     return t == CERA_HIP_Q4_0 || t == CERA_HIP_Q4_1 || t == CERA_HIP_Q8_0 || t == CERA_HIP_Q4_K || t == CERA_HIP_Q6_K;
 }
@@ -409,8 +412,8 @@ cera_hip_status cera_launch_gemv(cera_hip_ctx* ctx, const cera_hip_dtensor* w, c
             return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "fused gate/up gemv needs two matrices of identical type and shape");
     }
     if (epi == CERA_EPI_ADD && !resid) return cera_fail(ctx, CERA_HIP_ERR_ARGUMENT, "residual pointer is null");
-    // unit = 32 weights, except Q6_K whose lanes take 64
-    uint32_t n_units = static_cast<uint32_t>(w->k / (w->dtype == CERA_HIP_Q6_K ? Q6K::ELEMS_PER_UNIT : 32));
+    // unit = 32 weights, except the K-quants whose lanes take 64
+    uint32_t n_units = static_cast<uint32_t>(w->k / cera_gemv_unit_elems(w->dtype));
     GemvArgs a;
     a.w = w->dev;
     a.w2 = w2 ? w2->dev : nullptr;
@@ -426,7 +429,9 @@ cera_hip_status cera_launch_gemv(cera_hip_ctx* ctx, const cera_hip_dtensor* w, c
     a.dbg_stride = static_cast<uint32_t>(w->dtype == CERA_HIP_Q6_K ? w->k / 16 : w->k / 32);
     const bool dbg = dbg_dots != nullptr;
     GemvPlan p;
-    if (!gemv_plan(a.m, n_units, ctx->n_cu, dbg, w->dtype == CERA_HIP_Q6_K ? 2 : 4, &p, epi == CERA_EPI_SILU_MUL))
+    // rows in flight: a K-quant row unit is 12-15 registers (two matrices in the fused pair)
+    const int max_rb = w->dtype == CERA_HIP_Q4_K ? (epi == CERA_EPI_SILU_MUL ? 1 : 2) : (w->dtype == CERA_HIP_Q6_K ? 2 : 4);
+    if (!gemv_plan(a.m, n_units, ctx->n_cu, dbg, max_rb, &p, epi == CERA_EPI_SILU_MUL))
         return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "gemv: k=" + std::to_string(w->k) + " exceeds the 32768 supported by the register-resident kernel");
     a.rows_per_wave = p.rows_per_block;
     bool ok = false;
@@ -451,7 +456,7 @@ cera_hip_status cera_launch_gemv_nb(cera_hip_ctx* ctx, const cera_hip_dtensor* w
                                     const float* resid, bool* launched) {
     *launched = false;
     if (!is_int8_type(w->dtype) || n_tok == 0) return CERA_HIP_OK;
-    const uint32_t n_units = static_cast<uint32_t>(w->k / (w->dtype == CERA_HIP_Q6_K ? Q6K::ELEMS_PER_UNIT : 32));
+    const uint32_t n_units = static_cast<uint32_t>(w->k / cera_gemv_unit_elems(w->dtype));
     GemvPlan p;
     if (!gemv_plan(static_cast<uint32_t>(w->m), n_units, ctx->n_cu, false, 2, &p) || p.U != 1) return CERA_HIP_OK;
     const int KS = p.KS == 7 ? 8 : p.KS;   // instantiated widths: 1, 2, 4, 8 (surplus lanes carry zero activations)
@@ -501,8 +506,8 @@ cera_hip_status cera_launch_gemv_pair(cera_hip_ctx* ctx, const cera_hip_dtensor*
     };
     GemvPairArgs p;
     GemvPlan pa, pb;
-    const uint32_t ua = static_cast<uint32_t>(wa->k / 32), ub = static_cast<uint32_t>(wb->k / Q6K::ELEMS_PER_UNIT);
-    if (!gemv_plan(static_cast<uint32_t>(wa->m), ua, ctx->n_cu, false, 4, &pa)) return CERA_HIP_OK;
+    const uint32_t ua = static_cast<uint32_t>(wa->k / Q4K::ELEMS_PER_UNIT), ub = static_cast<uint32_t>(wb->k / Q6K::ELEMS_PER_UNIT);
+    if (!gemv_plan(static_cast<uint32_t>(wa->m), ua, ctx->n_cu, false, 2, &pa)) return CERA_HIP_OK;
     if (!gemv_plan(static_cast<uint32_t>(wb->m), ub, ctx->n_cu, false, 2, &pb)) return CERA_HIP_OK;
     fill(wa, ya, ua, &p.a);
     fill(wb, yb, ub, &p.b);

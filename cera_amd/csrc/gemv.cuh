@@ -10,7 +10,7 @@
 // the CPU's eight-lane FMA chains.
 //
 // Design: "activation-stationary lanes".  The K dimension is cut into
-// fixed-size *units* (16 B of Q4_K nibbles, 24 B of Q6_K codes, one Q4_0 /
+// fixed-size *units* (32 B of Q4_K nibbles, 48 B of Q6_K codes, one Q4_0 /
 // Q4_1 / Q8_0 block).  A workgroup is KS wavefronts that split K between them:
 // wavefront kw owns units kw*64 .. kw*64+63 (+ 64*KS*i for i < U), one per
 // lane, so a lane keeps the int8 activations, activation scales and activation
@@ -42,68 +42,68 @@ struct GemvArgs {
 enum { EPI_STORE = 0, EPI_ADD = 1, EPI_SILU_MUL = 2 };
 
 // ---------------------------------------------------------------------------
-// Q4_K: unit = 16 bytes of qs (32 nibbles): 16 codes of sub-block 2g (low
-// nibbles) and 16 of sub-block 2g+1 (high nibbles); 8 units per 144-byte block.
+// Q4_K: unit = 32 bytes of qs -- one whole chunk g of a 144-byte block, i.e. ALL 32 codes of
+// sub-block 2g (low nibbles) and all 32 of sub-block 2g+1 (high nibbles); 4 units per block.
+// The per-sub-block work (6-bit scale/min decode, the f32 scale algebra, the row reduction and
+// the header load) is paid once per 64 weights: a unit of 16 bytes (half of each sub-block, the
+// two halves in neighbouring lanes) needed about half as many VALU instructions again per byte
+// and streamed 8 % slower (5.3 against 5.8 TB/s on long matrices).  A 4096-wide row is exactly
+// one wavefront: no LDS combine, no barrier.
 struct Q4K {
-    static constexpr int ELEMS_PER_UNIT = 32;
-    struct Act { uint32_t lo[4], hi[4]; float xs0, xs1, c0, c1; int s0, s1; };
-    struct Wt { uint4 q; uint4 h; };
+    static constexpr int ELEMS_PER_UNIT = 64;
+    struct Act { uint32_t lo[8], hi[8]; float xs0, xs1, c0, c1; int s0, s1; };
+    struct Wt { uint4 q0, q1; uint4 h; };
     __device__ static void dbg_asum(const Act& a, uint32_t u, int32_t* out) {
-        atomicAdd(out + (u >> 3) * 8 + ((u >> 1) & 3) * 2, a.s0);
-        atomicAdd(out + (u >> 3) * 8 + ((u >> 1) & 3) * 2 + 1, a.s1);
+        out[(u >> 2) * 8 + (u & 3) * 2] = a.s0;
+        out[(u >> 2) * 8 + (u & 3) * 2 + 1] = a.s1;
     }
-    // `u` is always a valid unit (dead lanes pass unit 0); `live` zeroes the result,
-    // so the loads themselves are unconditional 16-byte loads.
     __device__ static void load_act(Act& a, const int8_t* xq, const float* xs, uint32_t u, bool live) {
-        uint32_t b = u >> 3, w8 = u & 7, g = w8 >> 1, h = w8 & 1;
-        const uint4 lo = *reinterpret_cast<const uint4*>(xq + b * 256 + g * 64 + h * 16);
-        const uint4 hi = *reinterpret_cast<const uint4*>(xq + b * 256 + g * 64 + h * 16 + 32);
+        const uint32_t b = u >> 2, g = u & 3;
+        const uint4* p = reinterpret_cast<const uint4*>(xq + b * 256 + g * 64);
+        const uint4 l0 = p[0], l1 = p[1], h0 = p[2], h1 = p[3];
         const float2 sc = *reinterpret_cast<const float2*>(xs + b * 8 + 2 * g);
         const uint32_t keep = live ? 0xFFFFFFFFu : 0u;
-        a.lo[0] = lo.x & keep; a.lo[1] = lo.y & keep; a.lo[2] = lo.z & keep; a.lo[3] = lo.w & keep;
-        a.hi[0] = hi.x & keep; a.hi[1] = hi.y & keep; a.hi[2] = hi.z & keep; a.hi[3] = hi.w & keep;
+        const uint32_t lv[8] = {l0.x, l0.y, l0.z, l0.w, l1.x, l1.y, l1.z, l1.w};
+        const uint32_t hv[8] = {h0.x, h0.y, h0.z, h0.w, h1.x, h1.y, h1.z, h1.w};
         int s0 = 0, s1 = 0;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        for (int i = 0; i < 8; ++i) {
+            a.lo[i] = lv[i] & keep;
+            a.hi[i] = hv[i] & keep;
             s0 = sum4(a.lo[i], s0);
             s1 = sum4(a.hi[i], s1);
         }
         a.xs0 = live ? sc.x : 0.0f;
         a.xs1 = live ? sc.y : 0.0f;
-        // xs has an 11-bit significand and |s| <= 16*127: the products are exact.
-        a.c0 = a.xs0 * static_cast<float>(s0);
+        a.c0 = a.xs0 * static_cast<float>(s0);   // exact: 11-bit significand x |s| <= 32*127
         a.c1 = a.xs1 * static_cast<float>(s1);
         a.s0 = s0;
         a.s1 = s1;
     }
     __device__ static void load_w(Wt& w, const uint8_t* row, uint32_t u) {
-        const uint8_t* blk = row + (u >> 3) * 144;
+        const uint8_t* blk = row + (u >> 2) * 144;
         w.h = ld_u128(blk);
-        w.q = ld_u128(blk + 16 + (u & 7) * 16);
+        w.q0 = ld_u128(blk + 16 + (u & 3) * 32);
+        w.q1 = ld_u128(blk + 32 + (u & 3) * 32);
     }
     __device__ static float dot(const Wt& w, const Act& a, uint32_t u, int32_t* dbg) {
-        uint32_t g = (u >> 1) & 3;
-        // 6-bit scales/mins of sub-blocks 2g, 2g+1 (get_scale_min_k4), two per 16-bit pair.  Low
-        // sub-blocks keep their 6 bits in place in bytes 0..3 / 4..7; high ones splice a nibble of
-        // bytes 8..11 with the top two bits of those bytes.  Which packing applies depends on the
-        // lane's unit only, so it is folded into shift counts and masks that stay in registers
-        // across the rows: two shifts, an AND and an AND-OR per pair instead of a select.
+        const uint32_t g = u & 3;
         const uint32_t sh = 16 * (g & 1);
         const bool low = g < 2;
         const uint32_t sh_a = low ? sh : sh + 2, m_a = low ? 0x3F3Fu : 0x3030u, m_b = low ? 0u : 0x0F0Fu;
         const uint32_t sc2 = ((w.h.y >> sh_a) & m_a) | ((w.h.w >> sh) & m_b);
         const uint32_t mn2 = ((w.h.z >> sh_a) & m_a) | ((w.h.w >> (sh + 4)) & m_b);
-        float d = h2f(w.h.x & 0xFFFF), dmin = h2f(w.h.x >> 16);
+        const float d = h2f(w.h.x & 0xFFFF), dmin = h2f(w.h.x >> 16);
         int dl = 0, dh = 0;
-        const uint32_t q[4] = {w.q.x, w.q.y, w.q.z, w.q.w};
+        const uint32_t q[8] = {w.q0.x, w.q0.y, w.q0.z, w.q0.w, w.q1.x, w.q1.y, w.q1.z, w.q1.w};
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        for (int i = 0; i < 8; ++i) {
             dl = dot4(q[i] & 0x0F0F0F0Fu, a.lo[i], dl);
             dh = dot4((q[i] >> 4) & 0x0F0F0F0Fu, a.hi[i], dh);
         }
         if (dbg) {
-            atomicAdd(dbg + (u >> 3) * 8 + 2 * g, dl);
-            atomicAdd(dbg + (u >> 3) * 8 + 2 * g + 1, dh);
+            dbg[(u >> 2) * 8 + 2 * g] = dl;
+            dbg[(u >> 2) * 8 + 2 * g + 1] = dh;
         }
         float s = (static_cast<float>(sc2 & 0xFF) * a.xs0) * static_cast<float>(dl);
         s = fmaf(static_cast<float>(sc2 >> 8) * a.xs1, static_cast<float>(dh), s);

@@ -1,0 +1,313 @@
+// Decode GEMVs with the neighbouring small operations folded in, for rows that fit one wavefront
+// (k <= 4096 with 64-weight units: the hidden size of the 7-8B models).
+//
+// A decode step is a chain of dependent launches, and on this hardware a launch costs about 3 us
+// before its first byte arrives, whatever it does.  rmsnorm + Q8_0 quantization of a 4096-vector
+// and the Q8_0 quantization of the SwiGLU output are such launches: 16 KB of work each.  Here
+//   * the consumer does the norm: every workgroup of the Q|K|V and gate|up projections reads the
+//     f32 hidden vector and the norm weights itself (32 KB from L2), reduces the sum of squares,
+//     normalizes and quantizes into LDS -- exactly rmsnorm_row_kernel's arithmetic
+//     (cpu::rmsnorm + quantize_f32_to_q8_0, cera/src/backend/cpu.rs:2479-2496, 942-958) -- while its
+//     first weight rows are already in flight, and its wavefronts take their activations from LDS;
+//   * the producer does the SwiGLU quantization: a workgroup owns 32 consecutive rows of gate and
+//     up, i.e. one whole Q8_0 block of the down projection's input, and writes its int8 codes and
+//     scale (silu_mul_inplace cpu.rs:2570-2575, then cpu.rs:942-958); the f32 vector is never stored.
+// A wavefront owns whole rows (one 64-weight unit per lane), walks its rows one at a time with
+// the next row's loads in flight, and reduces with DPP only: no LDS combine, no barrier in the
+// row loop.  Per-row arithmetic is gemv.cuh's (T::dot), so results meet the same bars.
+#include "gemv.cuh"
+#include "host_common.h"
+#include "quantize.cuh"
+
+enum { FEPI_STORE = 0, FEPI_ADD = 1, FEPI_SILU_Q8 = 2 };
+
+struct RowGemvArgs {
+    const uint8_t* w;       // [m] rows
+    const uint8_t* w2;      // second matrix, same shape (SILU_Q8: w = gate, w2 = up)
+    uint32_t m, k, row_bytes, rows_per_wave;
+    const int8_t* xq;       // NORM == false: quantized activations
+    const float* xs;
+    const float* x;         // NORM == true: f32 vector [k] and norm weights [k]
+    const float* norm_w;
+    float eps;
+    float* y;               // STORE / ADD
+    const float* resid;
+    int8_t* out_q;          // SILU_Q8: [m] int8, [m/32] scales
+    float* out_s;
+};
+struct RowGemvPairArgs {
+    RowGemvArgs a, b;       // two matrices over the same activations: workgroups [0, n_blocks_a) take a
+    uint32_t n_blocks_a;
+};
+
+// rmsnorm + Q8_0 of x[0, k) into LDS; all 64 * NW threads take part (k % 32 == 0, k <= 4096)
+template <int NW>
+__device__ __forceinline__ void norm_quant_to_lds(const float* __restrict__ x, const float* __restrict__ w, uint32_t k, float eps,
+                                                  uint32_t* s_xq, float* s_xs, double* s_part) {
+    constexpr int NT = 64 * NW, MAXIT = 1024 / NT;
+    float4 v[MAXIT], g[MAXIT];
+    double s = 0.0;
+#pragma unroll
+    for (int it = 0; it < MAXIT; ++it) {
+        const uint32_t i = (threadIdx.x + NT * it) * 4;
+        if (i < k) {
+            v[it] = *reinterpret_cast<const float4*>(x + i);
+            g[it] = *reinterpret_cast<const float4*>(w + i);
+            s += static_cast<double>(v[it].x) * v[it].x;
+            s += static_cast<double>(v[it].y) * v[it].y;
+            s += static_cast<double>(v[it].z) * v[it].z;
+            s += static_cast<double>(v[it].w) * v[it].w;
+        }
+    }
+    for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
+    if ((threadIdx.x & 63) == 0) s_part[threadIdx.x >> 6] = s;
+    __syncthreads();
+    double tot = 0.0;
+#pragma unroll
+    for (int i = 0; i < NW; ++i) tot += s_part[i];
+    const float inv = static_cast<float>(1.0 / sqrt(tot / static_cast<double>(k) + static_cast<double>(eps)));
+#pragma unroll
+    for (int it = 0; it < MAXIT; ++it) {
+        const uint32_t i = (threadIdx.x + NT * it) * 4;
+        if (i < k) {   // k % 32 == 0: the eight lanes of a block are live together
+            float4 o;
+            o.x = __fmul_rn(__fmul_rn(v[it].x, inv), g[it].x);
+            o.y = __fmul_rn(__fmul_rn(v[it].y, inv), g[it].y);
+            o.z = __fmul_rn(__fmul_rn(v[it].z, inv), g[it].z);
+            o.w = __fmul_rn(__fmul_rn(v[it].w, inv), g[it].w);
+            float sc;
+            const uint32_t packed = q8_quantize_quad(o, sc);
+            s_xq[i >> 2] = packed;
+            if ((threadIdx.x & 7) == 0) s_xs[i >> 5] = sc;
+        }
+    }
+    __syncthreads();
+}
+
+template <class T, int NM>
+struct RowTile {
+    typename T::Wt w[NM];
+    __device__ __forceinline__ void load(const RowGemvArgs& p, uint32_t unit, uint32_t row) {
+        T::load_w(w[0], p.w + static_cast<uint64_t>(row) * p.row_bytes, unit);
+        if (NM == 2) T::load_w(w[NM - 1], p.w2 + static_cast<uint64_t>(row) * p.row_bytes, unit);
+    }
+};
+
+// The work of workgroup `block` on matrix p.  Every thread of the workgroup must call this (it
+// contains barriers when NORM or SILU_Q8), including wavefronts whose row range is empty.
+template <class T, int NW, bool NORM, int EPI>
+__device__ __forceinline__ void row_gemv_body(const RowGemvArgs& p, uint32_t block, uint32_t* s_xq, float* s_xs, double* s_part,
+                                              float* s_out) {
+    constexpr int NM = EPI == FEPI_SILU_Q8 ? 2 : 1;
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t n_units = p.k / T::ELEMS_PER_UNIT;
+    const bool live = lane < n_units;
+    const uint32_t unit = live ? lane : 0;
+    uint32_t r = (block * NW + wave) * p.rows_per_wave;
+    const uint32_t r1 = min(p.m, r + p.rows_per_wave);
+    const bool has_rows = r < p.m;
+
+    RowTile<T, NM> ta, tb;
+    if (has_rows) ta.load(p, unit, r);   // in flight while the activations are prepared
+
+    typename T::Act act;
+    if (NORM) {
+        norm_quant_to_lds<NW>(p.x, p.norm_w, p.k, p.eps, s_xq, s_xs, s_part);
+        T::load_act(act, reinterpret_cast<const int8_t*>(s_xq), s_xs, unit, live);
+    } else {
+        T::load_act(act, p.xq, p.xs, unit, live);
+    }
+
+    auto finish = [&](const RowTile<T, NM>& t, uint32_t row) {
+        float tot[NM];
+#pragma unroll
+        for (int mi = 0; mi < NM; ++mi) tot[mi] = wave_sum(T::dot(t.w[mi], act, unit, nullptr));
+        if (lane == 0) {
+            if (EPI == FEPI_SILU_Q8) {
+                // cera/src/backend/cpu.rs:2570-2575: g / (1 + expf(-g)) * u
+                const float g = tot[0];
+                s_out[row - block * NW * p.rows_per_wave] = __fmul_rn(__fdiv_rn(g, __fadd_rn(1.0f, cera_expf(-g))), tot[NM - 1]);
+            } else {
+                p.y[row] = EPI == FEPI_ADD ? p.resid[row] + tot[0] : tot[0];
+            }
+        }
+    };
+    if (has_rows) {
+        for (;;) {
+            if (r + 1 >= r1) { finish(ta, r); break; }
+            tb.load(p, unit, r + 1);
+            finish(ta, r);
+            ++r;
+            if (r + 1 >= r1) { finish(tb, r); break; }
+            ta.load(p, unit, r + 1);
+            finish(tb, r);
+            ++r;
+        }
+    }
+    if (EPI == FEPI_SILU_Q8) {
+        // the workgroup's NW * rows_per_wave = 32 rows are one Q8_0 block of the next projection's input
+        __syncthreads();
+        if (wave == 0) {
+            const uint32_t row0 = block * NW * p.rows_per_wave;
+            const bool q_live = lane < 8 && row0 < p.m;   // m % 32 == 0: the block is whole or absent
+            const float4 h = q_live ? reinterpret_cast<const float4*>(s_out)[lane] : make_float4(0.f, 0.f, 0.f, 0.f);
+            float sc;
+            const uint32_t packed = q8_quantize_quad(h, sc);
+            if (q_live) {
+                reinterpret_cast<uint32_t*>(p.out_q + row0)[lane] = packed;
+                if (lane == 0) p.out_s[row0 >> 5] = sc;
+            }
+        }
+    }
+}
+
+template <class T, int NW, bool NORM, int EPI>
+static __global__ __launch_bounds__(64 * NW) void row_gemv_kernel(RowGemvArgs p) {
+    __shared__ uint32_t s_xq[NORM ? 1024 : 1];
+    __shared__ float s_xs[NORM ? 128 : 1];
+    __shared__ double s_part[NW];
+    __shared__ __attribute__((aligned(16))) float s_out[EPI == FEPI_SILU_Q8 ? 32 : 4];
+    row_gemv_body<T, NW, NORM, EPI>(p, blockIdx.x, s_xq, s_xs, s_part, s_out);
+}
+
+template <class TA, class TB, int NW, bool NORM>
+static __global__ __launch_bounds__(64 * NW) void row_gemv_pair_kernel(RowGemvPairArgs p) {
+    __shared__ uint32_t s_xq[NORM ? 1024 : 1];
+    __shared__ float s_xs[NORM ? 128 : 1];
+    __shared__ double s_part[NW];
+    if (blockIdx.x < p.n_blocks_a) row_gemv_body<TA, NW, NORM, FEPI_STORE>(p.a, blockIdx.x, s_xq, s_xs, s_part, nullptr);
+    else row_gemv_body<TB, NW, NORM, FEPI_STORE>(p.b, blockIdx.x - p.n_blocks_a, s_xq, s_xs, s_part, nullptr);
+}
+
+// ---------------------------------------------------------------------------
+static constexpr int FUSED_NW = 8;
+
+static bool fused_type(uint32_t t) { return t == CERA_HIP_Q4_K || t == CERA_HIP_Q6_K; }
+// rows that fit one wavefront of 64-weight units, whole super-blocks
+static bool fused_k(uint64_t k) { return k % 256 == 0 && k <= 4096 && k > 0; }
+
+static void fill(RowGemvArgs& a, const cera_hip_dtensor* w, const cera_hip_dtensor* w2, uint32_t rows_per_wave) {
+    a = RowGemvArgs{};
+    a.w = w->dev;
+    a.w2 = w2 ? w2->dev : nullptr;
+    a.m = static_cast<uint32_t>(w->m);
+    a.k = static_cast<uint32_t>(w->k);
+    a.row_bytes = static_cast<uint32_t>(w->row_bytes);
+    a.rows_per_wave = rows_per_wave;
+}
+static uint32_t blocks_for(uint64_t m, uint32_t rows_per_wave) {
+    const uint64_t per = static_cast<uint64_t>(FUSED_NW) * rows_per_wave;
+    return static_cast<uint32_t>((m + per - 1) / per);
+}
+
+// ffn first half: Q8_0(silu(gate . n) * (up . n)) with n = Q8_0(rmsnorm(x, norm_w)); out_q [m], out_s [m/32].
+// *launched = false (nothing done) when the shapes / types have no fused instance.
+cera_hip_status cera_launch_ffn_gate_up_fused(cera_hip_ctx* ctx, const cera_hip_dtensor* gate, const cera_hip_dtensor* up,
+                                              const float* x, const float* norm_w, float eps, int8_t* out_q, float* out_s,
+                                              bool* launched) {
+    *launched = false;
+    if (gate->dtype != CERA_HIP_Q4_K || up->dtype != CERA_HIP_Q4_K || gate->m != up->m || gate->k != up->k || !fused_k(gate->k) ||
+        gate->m % 32)
+        return CERA_HIP_OK;
+    RowGemvArgs a;
+    fill(a, gate, up, 32 / FUSED_NW);   // 32 rows per workgroup: one Q8_0 block of the output
+    a.x = x; a.norm_w = norm_w; a.eps = eps; a.out_q = out_q; a.out_s = out_s;
+    hipLaunchKernelGGL((row_gemv_kernel<Q4K, FUSED_NW, true, FEPI_SILU_Q8>), dim3(blocks_for(a.m, a.rows_per_wave)),
+                       dim3(64 * FUSED_NW), 0, ctx->stream, a);
+    HIP_TRY(ctx, hipGetLastError());
+    *launched = true;
+    return CERA_HIP_OK;
+}
+
+// attention projections: ya = A . n, yb = B . n (b nullable) with n = Q8_0(rmsnorm(x, norm_w)).
+cera_hip_status cera_launch_qkv_fused(cera_hip_ctx* ctx, const cera_hip_dtensor* wa, const cera_hip_dtensor* wb, const float* x,
+                                      const float* norm_w, float eps, float* ya, float* yb, bool* launched) {
+    *launched = false;
+    if (!fused_type(wa->dtype) || !fused_k(wa->k) || (wb && (!fused_type(wb->dtype) || wb->k != wa->k))) return CERA_HIP_OK;
+    // about 12 wavefronts per CU over both matrices, at least one row per wavefront
+    const uint64_t rows = wa->m + (wb ? wb->m : 0);
+    const uint32_t rpw = static_cast<uint32_t>(std::max<uint64_t>(1, rows / (static_cast<uint64_t>(ctx->n_cu) * 12)));
+    RowGemvPairArgs p;
+    fill(p.a, wa, nullptr, rpw);
+    p.a.x = x; p.a.norm_w = norm_w; p.a.eps = eps; p.a.y = ya;
+    p.n_blocks_a = blocks_for(wa->m, rpw);
+    uint32_t n_blocks = p.n_blocks_a;
+    if (wb) {
+        fill(p.b, wb, nullptr, rpw);
+        p.b.x = x; p.b.norm_w = norm_w; p.b.eps = eps; p.b.y = yb;
+        n_blocks += blocks_for(wb->m, rpw);
+    } else {
+        p.b = p.a;
+    }
+    const dim3 grid(n_blocks), block(64 * FUSED_NW);
+    const uint32_t ta = wa->dtype, tb = wb ? wb->dtype : wa->dtype;
+    if (ta == CERA_HIP_Q4_K && tb == CERA_HIP_Q6_K) hipLaunchKernelGGL((row_gemv_pair_kernel<Q4K, Q6K, FUSED_NW, true>), grid, block, 0, ctx->stream, p);
+    else if (ta == CERA_HIP_Q4_K && tb == CERA_HIP_Q4_K) hipLaunchKernelGGL((row_gemv_pair_kernel<Q4K, Q4K, FUSED_NW, true>), grid, block, 0, ctx->stream, p);
+    else if (ta == CERA_HIP_Q6_K && tb == CERA_HIP_Q6_K) hipLaunchKernelGGL((row_gemv_pair_kernel<Q6K, Q6K, FUSED_NW, true>), grid, block, 0, ctx->stream, p);
+    else hipLaunchKernelGGL((row_gemv_pair_kernel<Q6K, Q4K, FUSED_NW, true>), grid, block, 0, ctx->stream, p);
+    HIP_TRY(ctx, hipGetLastError());
+    *launched = true;
+    return CERA_HIP_OK;
+}
+
+// ---- kernel-level entry points (host buffers) --------------------------------------------------
+extern "C" cera_hip_status cera_hip_ffn_gate_up_fused(cera_hip_ctx* ctx, const cera_hip_tensor* gate, const cera_hip_tensor* up,
+                                                      const float* x, const float* norm_w, float eps, int8_t* quants,
+                                                      float* scales) {
+    if (!ctx || !gate || !up || !x || !norm_w || !quants || !scales) return CERA_HIP_ERR_ARGUMENT;
+    std::lock_guard<std::recursive_mutex> lk(ctx->op_mu);
+    cera_hip_dtensor *wg = nullptr, *wu = nullptr;
+    CERA_TRY(cera_hip_tensor_upload(ctx, gate, &wg));
+    cera_hip_status st = cera_hip_tensor_upload(ctx, up, &wu);
+    if (st != CERA_HIP_OK) { cera_hip_tensor_free(ctx, wg); return st; }
+    auto run = [&]() -> cera_hip_status {
+        const uint64_t k = wg->k, m = wg->m;
+        void *dx, *dw, *dq, *ds;
+        CERA_TRY(cera_scratch(ctx, 0, k * 4, &dx));
+        CERA_TRY(cera_scratch(ctx, 1, k * 4, &dw));
+        CERA_TRY(cera_scratch(ctx, 2, m, &dq));
+        CERA_TRY(cera_scratch(ctx, 3, m / 32 * 4 + 4, &ds));
+        CERA_TRY(cera_hip_upload(ctx, dx, x, k * 4));
+        CERA_TRY(cera_hip_upload(ctx, dw, norm_w, k * 4));
+        bool launched = false;
+        CERA_TRY(cera_launch_ffn_gate_up_fused(ctx, wg, wu, static_cast<float*>(dx), static_cast<float*>(dw), eps,
+                                               static_cast<int8_t*>(dq), static_cast<float*>(ds), &launched));
+        if (!launched) return cera_fail(ctx, CERA_HIP_ERR_UNSUPPORTED_DTYPE, "ffn_gate_up_fused: needs two Q4_K matrices of one shape, k <= 4096 in whole super-blocks, m a multiple of 32");
+        CERA_TRY(cera_hip_download(ctx, quants, dq, m));
+        return cera_hip_download(ctx, scales, ds, m / 32 * 4);
+    };
+    st = run();
+    cera_hip_tensor_free(ctx, wg);
+    cera_hip_tensor_free(ctx, wu);
+    return st;
+}
+
+extern "C" cera_hip_status cera_hip_qkv_fused(cera_hip_ctx* ctx, const cera_hip_tensor* a, const cera_hip_tensor* b, const float* x,
+                                              const float* norm_w, float eps, float* ya, float* yb) {
+    if (!ctx || !a || !x || !norm_w || !ya || (b && !yb)) return CERA_HIP_ERR_ARGUMENT;
+    std::lock_guard<std::recursive_mutex> lk(ctx->op_mu);
+    cera_hip_dtensor *wa = nullptr, *wb = nullptr;
+    CERA_TRY(cera_hip_tensor_upload(ctx, a, &wa));
+    cera_hip_status st = b ? cera_hip_tensor_upload(ctx, b, &wb) : CERA_HIP_OK;
+    if (st != CERA_HIP_OK) { cera_hip_tensor_free(ctx, wa); return st; }
+    auto run = [&]() -> cera_hip_status {
+        const uint64_t k = wa->k;
+        void *dx, *dw, *dy;
+        CERA_TRY(cera_scratch(ctx, 0, k * 4, &dx));
+        CERA_TRY(cera_scratch(ctx, 1, k * 4, &dw));
+        CERA_TRY(cera_scratch(ctx, 3, (wa->m + (wb ? wb->m : 0)) * 4, &dy));
+        CERA_TRY(cera_hip_upload(ctx, dx, x, k * 4));
+        CERA_TRY(cera_hip_upload(ctx, dw, norm_w, k * 4));
+        float *da = static_cast<float*>(dy), *db = da + wa->m;
+        bool launched = false;
+        CERA_TRY(cera_launch_qkv_fused(ctx, wa, wb, static_cast<float*>(dx), static_cast<float*>(dw), eps, da, db, &launched));
+        if (!launched) return cera_fail(ctx, CERA_HIP_ERR_UNSUPPORTED_DTYPE, "qkv_fused: needs Q4_K / Q6_K matrices with k <= 4096 in whole super-blocks");
+        CERA_TRY(cera_hip_download(ctx, ya, da, wa->m * 4));
+        if (wb) CERA_TRY(cera_hip_download(ctx, yb, db, wb->m * 4));
+        return CERA_HIP_OK;
+    };
+    st = run();
+    cera_hip_tensor_free(ctx, wa);
+    if (wb) cera_hip_tensor_free(ctx, wb);
+    return st;
+}

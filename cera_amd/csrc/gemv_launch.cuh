@@ -10,8 +10,8 @@ struct GemvPlan {
     uint32_t rows_per_block, n_blocks;
 };
 
-// n_units = K / 32.  One unit per lane while K <= 16384 (KS up to 8 wavefronts),
-// two per lane up to 32768.  KS is rounded up to an instantiated width; surplus
+// n_units = K / elements per unit (64 for the K-quants, 32 for the block formats).  One unit per
+// lane up to 512 units (KS up to 8 wavefronts), two per lane up to 1024.  KS is rounded up to an instantiated width; surplus
 // lanes carry zeroed activations.
 static inline bool gemv_pick_split(uint32_t n_units, int* U, int* KS) {
     const int widths[] = {1, 2, 4, 7, 8};
@@ -21,8 +21,8 @@ static inline bool gemv_pick_split(uint32_t n_units, int* U, int* KS) {
     return false;
 }
 
-// Measured on MI355X: ~32 wavefronts per CU in flight, four rows per workgroup
-// step for the 16-byte-unit formats and two for Q6_K (15 registers per row).
+// Measured on MI355X: ~32 wavefronts per CU in flight; rows in flight per workgroup step are
+// capped by the caller (max_rb) by the registers a row of the type takes.
 static inline bool gemv_plan(uint32_t m, uint32_t n_units, uint32_t n_cu, bool dbg, int max_rb, GemvPlan* p,
                              bool dual = false) {
     if (!gemv_pick_split(n_units, &p->U, &p->KS)) return false;
@@ -35,6 +35,7 @@ static inline bool gemv_plan(uint32_t m, uint32_t n_units, uint32_t n_cu, bool d
     const uint32_t target_blocks = std::max(1u, n_cu * per_cu / static_cast<uint32_t>(p->KS));
     uint32_t rpb = (m + target_blocks - 1) / target_blocks;
     p->RB = rpb >= 4 ? 4 : (rpb >= 2 ? 2 : 1);
+
     if (p->RB > max_rb) p->RB = max_rb;
     if (dbg) p->RB = 1;
     rpb = (rpb + p->RB - 1) / p->RB * p->RB;

@@ -78,6 +78,15 @@ cera_hip_status cera_launch_gemv_nb(cera_hip_ctx* ctx, const cera_hip_dtensor* w
                                     const float* resid, bool* launched);
 cera_hip_status cera_launch_gemv_pair(cera_hip_ctx* ctx, const cera_hip_dtensor* wa, const cera_hip_dtensor* wb,
                                       const float* xs, const int8_t* xq, float* ya, float* yb, bool* launched);
+// Decode projections with the neighbouring small kernels folded in (gemv_fused.hip); *launched =
+// false when the shapes / types have no fused instance and the caller takes the separate launches.
+//   gate|up: out_q / out_s = Q8_0(silu(gate . n) * (up . n)), n = Q8_0(rmsnorm(x, norm_w))
+//   q|k|v:   ya = A . n, yb = B . n (wb nullable)
+cera_hip_status cera_launch_ffn_gate_up_fused(cera_hip_ctx* ctx, const cera_hip_dtensor* gate, const cera_hip_dtensor* up,
+                                              const float* x, const float* norm_w, float eps, int8_t* out_q, float* out_s,
+                                              bool* launched);
+cera_hip_status cera_launch_qkv_fused(cera_hip_ctx* ctx, const cera_hip_dtensor* wa, const cera_hip_dtensor* wb, const float* x,
+                                      const float* norm_w, float eps, float* ya, float* yb, bool* launched);
 // index of the maximum of x[0, n) into *out_dev (device); uses scratch slot 8 of the context
 cera_hip_status cera_launch_argmax(cera_hip_ctx* ctx, const float* x, uint32_t n, uint32_t* out_dev);
 cera_hip_status cera_launch_gemv_q5k_f32(cera_hip_ctx* ctx, const cera_hip_dtensor* w, const float* x, float* y);

@@ -4,6 +4,7 @@
 // layer graph of LlamaModel (cera/src/model/llama.rs:468-597, 1585-1649;
 // cera/src/model/transformer.rs:1313-1652).
 #include <cmath>
+#include <cstdlib>
 #include <cstring>
 #include <new>
 
@@ -511,8 +512,16 @@ static cera_hip_status decode_step(cera_hip_model* m, uint32_t pos, bool want_lo
 
     for (uint32_t i = 0; i < c.n_layers; ++i) {
         LayerDev& L = m->layers[i];
-        CERA_TRY(norm_quant(m, m->hidden, L.attn_norm, c.hidden, 1, m->normed));
-        if (L.qkv) {
+        static const bool tmp_nofuse = getenv("CERA_TMP_NOFUSE") != nullptr;   // TMP experiment hook
+        // Q|K|V with the attention norm and its Q8_0 quantization done by the projection's own
+        // workgroups (one launch instead of two), where the shapes allow
+        bool qkv_done = false;
+        if (L.qkv && !tmp_nofuse)
+            CERA_TRY(cera_launch_qkv_fused(ctx, L.qkv, L.qkv_rows == q_dim + kv_dim ? L.v : nullptr, m->hidden, L.attn_norm,
+                                           c.rms_eps, m->q, m->v, &qkv_done));
+        if (qkv_done) {
+        } else if (L.qkv) {
+            CERA_TRY(norm_quant(m, m->hidden, L.attn_norm, c.hidden, 1, m->normed));
             bool paired = false;
             // Q|K in one block type and V in another (the Q4_K_M mix): still one launch where a
             // paired kernel instance exists
@@ -523,6 +532,7 @@ static cera_hip_status decode_step(cera_hip_model* m, uint32_t pos, bool want_lo
                 if (L.qkv_rows == q_dim + kv_dim) CERA_TRY(project(m, L.v, m->normed, m->v, nullptr));
             }
         } else {
+            CERA_TRY(norm_quant(m, m->hidden, L.attn_norm, c.hidden, 1, m->normed));
             CERA_TRY(project(m, L.q, m->normed, m->q, nullptr));
             CERA_TRY(project(m, L.k, m->normed, m->k, nullptr));
             CERA_TRY(project(m, L.v, m->normed, m->v, nullptr));
@@ -542,9 +552,15 @@ static cera_hip_status decode_step(cera_hip_model* m, uint32_t pos, bool want_lo
                                 c.head_dim, c.max_seq_len, c.rope_type, scale, m->kv_f16, m->attn_out, m->xs, m->xq));
         CERA_TRY(project(m, L.o, m->attn_out, m->hidden, m->hidden));
 
-        CERA_TRY(norm_quant(m, m->hidden, L.ffn_norm, c.hidden, 1, m->normed));
+        // gate | up with the FFN norm in front and SwiGLU + the down projection's Q8_0 quantization
+        // behind, all in one launch instead of three, where the shapes allow
+        bool ffn_done = false;
+        if (!tmp_nofuse)
+            CERA_TRY(cera_launch_ffn_gate_up_fused(ctx, L.gate, L.up, m->hidden, L.ffn_norm, c.rms_eps, m->xq, m->xs, &ffn_done));
         const bool fuse = L.gate->dtype == L.up->dtype && L.gate->dtype != CERA_HIP_Q5_K;
-        if (fuse) {
+        if (!ffn_done) CERA_TRY(norm_quant(m, m->hidden, L.ffn_norm, c.hidden, 1, m->normed));
+        if (ffn_done) {
+        } else if (fuse) {
             CERA_TRY(cera_launch_gemv(ctx, L.gate, L.up, m->xs, m->xq, m->act, nullptr, CERA_EPI_SILU_MUL));
             CERA_TRY(cera_launch_quantize(ctx, m->act, c.ffn, m->xs, m->xq));
         } else {

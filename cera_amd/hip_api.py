@@ -33,6 +33,7 @@ SYMBOLS = [
     "cera_hip_gemv_reference_order", "cera_hip_attn_decode_reference_order", "cera_hip_rmsnorm_reference_order",
     "cera_hip_set_reference_order", "cera_hip_reference_order",
     "cera_hip_rmsnorm_q8_0", "cera_hip_attn_decode_step", "cera_hip_attn_decode_dev_noalloc", "cera_hip_gemm_block_dots",
+    "cera_hip_ffn_gate_up_fused", "cera_hip_qkv_fused",
 ]
 
 
@@ -137,6 +138,8 @@ def load_library() -> C.CDLL:
         "cera_hip_rmsnorm_reference_order": (i32, [vp, vp, vp, u64, f32, vp]),
         "cera_hip_set_reference_order": (i32, [vp, u32]), "cera_hip_reference_order": (u32, [vp]),
         "cera_hip_attn_decode_dev_noalloc": (i32, [vp, vp, vp, vp, u32, u32, u32, u64, u64, f32, u32, vp]),
+        "cera_hip_ffn_gate_up_fused": (i32, [vp, vp, vp, vp, vp, f32, vp, vp]),
+        "cera_hip_qkv_fused": (i32, [vp, vp, vp, vp, vp, f32, vp, vp]),
         "cera_hip_gemm_block_dots": (i32, [vp, C.POINTER(Tensor), vp, u64, vp, vp]),
         "cera_hip_rmsnorm_q8_0": (i32, [vp, vp, vp, u64, f32, vp, vp, vp]),
         "cera_hip_attn_decode_step": (i32, [vp, vp, vp, vp, vp, vp, u32, u32, u32, u32, f32, u32, vp, f32, u32,
@@ -345,6 +348,23 @@ class Context:
         self.check(self.lib.cera_hip_attn_f16kv(self.h, _p(q), _p(k), _p(v), n_heads, n_kv_heads, head_dim, start_pos,
                                                 n_queries, scale, n_splits, _p(out)))
         return out.reshape(n_queries, n_heads * head_dim)
+
+    def ffn_gate_up_fused(self, w_gate, w_up, m, k, x, norm_w, eps):
+        """Q8_0(silu(gate.n) * (up.n)), n = Q8_0(rmsnorm(x, norm_w)): (quants [m], scales [m/32])."""
+        tg, tu = make_tensor(Q4_K, m, k, w_gate), make_tensor(Q4_K, m, k, w_up)
+        x = np.ascontiguousarray(x, np.float32); nw = np.ascontiguousarray(norm_w, np.float32)
+        q, sc = np.empty(m, np.int8), np.empty(m // 32, np.float32)
+        self.check(self.lib.cera_hip_ffn_gate_up_fused(self.h, C.byref(tg), C.byref(tu), _p(x), _p(nw), eps, _p(q), _p(sc)))
+        return q, sc
+
+    def qkv_fused(self, type_a, wa, ma, type_b, wb, mb, k, x, norm_w, eps):
+        ta = make_tensor(type_a, ma, k, wa)
+        tb = make_tensor(type_b, mb, k, wb) if wb is not None else None
+        x = np.ascontiguousarray(x, np.float32); nw = np.ascontiguousarray(norm_w, np.float32)
+        ya = np.empty(ma, np.float32); yb = np.empty(mb, np.float32) if wb is not None else None
+        self.check(self.lib.cera_hip_qkv_fused(self.h, C.byref(ta), C.byref(tb) if tb is not None else None, _p(x), _p(nw), eps,
+                                               _p(ya), _p(yb) if yb is not None else None))
+        return ya, yb
 
     # -- the decode step's fused kernels
     def rmsnorm_q8_0(self, x, w, eps):

@@ -152,7 +152,7 @@ CERA_HIP_API cera_hip_status cera_hip_gemv(cera_hip_ctx*, const cera_hip_tensor*
  * while a batch is at most 16 tokens (a few new tokens of a chat turn, the verification pass of
  * speculative decoding, cera/src/model/mod.rs:221-249).  Row t of y is bit-identical to
  * cera_hip_gemv on x[t].  CERA_HIP_ERR_UNSUPPORTED_DTYPE for Q5_K and for k beyond one unit per
- * lane (k > 16384, Q6_K 32768). */
+ * lane (k > 16384; Q4_K and Q6_K 32768). */
 CERA_HIP_API cera_hip_status cera_hip_gemv_nb(cera_hip_ctx*, const cera_hip_tensor* w, const float* x, uint32_t n,
                                               float* y);
 
@@ -160,7 +160,7 @@ CERA_HIP_API cera_hip_status cera_hip_gemv_nb(cera_hip_ctx*, const cera_hip_tens
  * layer whose attn_q|attn_k (Q4_K, stored back to back) and attn_v (Q6_K) differ in block type
  * (the Q4_K_M mix, cera/src/convert/quantize.rs:102-113); each result is exactly that of
  * cera_hip_gemv on its own matrix (same kernel body, same row grouping).  Kernel instances
- * exist for a Q4_K matrix with 2048 < k <= 4096 next to a Q6_K one; any other combination is
+ * exist for a Q4_K matrix with k <= 4096 next to a Q6_K one; any other combination is
  * CERA_HIP_ERR_UNSUPPORTED_DTYPE (the model then launches the two one after the other). */
 CERA_HIP_API cera_hip_status cera_hip_gemv_pair(cera_hip_ctx*, const cera_hip_tensor* a, const cera_hip_tensor* b,
                                                 const float* x, float* ya, float* yb);
@@ -274,6 +274,23 @@ CERA_HIP_API cera_hip_status cera_hip_attn_decode_step(cera_hip_ctx*, const floa
                                                        const float* freq_factors, float scale, uint32_t kv_type,
                                                        float* out, float* out_scales, int8_t* out_quants, float* k_row,
                                                        float* v_row);
+
+/* The two fused launches of the decode step, for parity tests.  gate | up: cpu::rmsnorm(x, norm_w),
+ * its Q8_0 quantization, the two projections of transformer::forward_ffn_block
+ * (cera/src/model/transformer.rs:1541), cpu::silu_mul_inplace (cera/src/backend/cpu.rs:2570-2575)
+ * and the Q8_0 quantization of the result for the down projection (cpu.rs:942-958) in ONE launch:
+ * quants i8[m], scales f32[m/32].  Two Q4_K matrices of one shape, k <= 4096 in whole
+ * 256-element super-blocks, m a multiple of 32; anything else is CERA_HIP_ERR_UNSUPPORTED_DTYPE
+ * (the decode step then issues the separate launches). */
+CERA_HIP_API cera_hip_status cera_hip_ffn_gate_up_fused(cera_hip_ctx*, const cera_hip_tensor* gate,
+                                                        const cera_hip_tensor* up, const float* x, const float* norm_w,
+                                                        float eps, int8_t* quants, float* scales);
+/* q | k | v: cpu::rmsnorm(x, norm_w), its Q8_0 quantization and the projections of
+ * transformer::forward_attn_block (cera/src/model/transformer.rs:1340-1373) in one launch:
+ * ya = A . n, yb = B . n (b / yb nullable).  Q4_K or Q6_K matrices with k <= 4096 in whole
+ * super-blocks. */
+CERA_HIP_API cera_hip_status cera_hip_qkv_fused(cera_hip_ctx*, const cera_hip_tensor* a, const cera_hip_tensor* b,
+                                                const float* x, const float* norm_w, float eps, float* ya, float* yb);
 
 /* ---- reference-order verification route (never the default, never timed) -- */
 /* The same three operations with every f32 operation performed exactly as the CPU AVX2 path

@@ -411,7 +411,7 @@ def test_attn_decode_head_dim_64(hip, orc, kv_f16, nh, nkv, L):
 
 
 # ---- two projections in one launch --------------------------------------------------------
-@pytest.mark.parametrize("ma,mb,k", [(5120, 1024, 4096), (4096, 4096, 4096), (1027, 515, 4096), (6, 3, 3072)])
+@pytest.mark.parametrize("ma,mb,k", [(5120, 1024, 4096), (4096, 4096, 4096), (1027, 515, 4096), (6, 3, 3072), (70, 30, 1024)])
 def test_gemv_pair_is_bitwise_the_two_single_launches(hip, orc, ma, mb, k):
     """attn_q|attn_k (Q4_K) and attn_v (Q6_K) of one layer in a single launch: the same kernel
     body per matrix, so each output equals cera_hip_gemv's bit for bit (and the oracle to the bar)."""
@@ -428,7 +428,7 @@ def test_gemv_pair_is_bitwise_the_two_single_launches(hip, orc, ma, mb, k):
 
 
 def test_gemv_pair_refuses_what_it_has_no_instance_for(hip):
-    k = 1024   # one wavefront covers a Q4_K row of 1024: no paired instance
+    k = 8192   # a Q4_K row of 8192 takes two wavefronts: no paired instance
     wa, _ = util.make_weights(Q4_K, 8, k, seed=1)
     wb, _ = util.make_weights(Q6_K, 8, k, seed=2)
     with pytest.raises(hip_api.HipError) as e:
@@ -459,8 +459,8 @@ def test_gemv_multi_token_is_bitwise_per_token_gemv(hip, orc, dtype, n):
 
 def test_gemv_multi_token_refusals(hip):
     with pytest.raises(hip_api.HipError) as e:   # two units per lane: no multi-token instance
-        w, _ = util.make_weights(Q4_K, 4, 28672, seed=1)
-        hip.gemv_nb(Q4_K, w, np.zeros((2, 28672), np.float32), 4, 28672)
+        w, _ = util.make_weights(Q4_0, 4, 28672, seed=1)
+        hip.gemv_nb(Q4_0, w, np.zeros((2, 28672), np.float32), 4, 28672)
     assert e.value.status == 3
 
 
@@ -514,3 +514,73 @@ def test_decode_attention_step_fused_append_and_q8_0(hip, orc, norm, kv_f16, n_h
     assert np.abs(out - ref).max() <= 2e-3 * util.rms(ref)
     rs, rq = orc.quantize_q8_0(out)
     assert np.array_equal(qq, rq) and np.array_equal(sc.view(np.uint32), rs.view(np.uint32)), "fused Q8_0 of the merge kernel"
+
+
+# ---- the decode step's fused projection launches ----------------------------------------------------
+@pytest.mark.parametrize("ma,mb,k,tb", [(5120, 1024, 4096, Q6_K), (640, 128, 512, Q6_K), (768, None, 256, None),
+                                       (96, 64, 2048, Q4_K), (40, 24, 4096, Q6_K)])
+def test_qkv_fused_norm_projection(hip, orc, ma, mb, k, tb):
+    """attention norm + its Q8_0 quantization + the Q|K (Q4_K) and V projections in one launch:
+    every output within the GEMV float bar of the oracle's rmsnorm -> gemv chain
+    (cera/src/backend/cpu.rs:2479-2496; cera/src/model/transformer.rs:1340-1373)."""
+    _say(f"qkv fused ma={ma} mb={mb} k={k}")
+    wa, _ = util.make_weights(Q4_K, ma, k, seed=61)
+    wb = util.make_weights(tb, mb, k, seed=62)[0] if mb else None
+    x = util.make_x(k, 63) * np.float32(2.5)
+    nw = (1.0 + 0.2 * util.make_x(k, 64)).astype(np.float32)
+    ya, yb = hip.qkv_fused(Q4_K, wa, ma, tb, wb, mb, k, x, nw, 1e-5)
+    n = orc.rmsnorm(x, nw, 1e-5)
+    ra = orc.gemv(Q4_K, wa, n, ma, k)
+    assert np.abs(ya - ra).max() <= 1e-3 * util.rms(ra)
+    if mb:
+        rb = orc.gemv(tb, wb, n, mb, k)
+        assert np.abs(yb - rb).max() <= 1e-3 * util.rms(rb)
+
+
+@pytest.mark.parametrize("m,k", [(14336, 4096), (512, 256), (96, 2048), (32, 4096)])
+def test_ffn_gate_up_fused_against_the_oracle(hip, orc, m, k):
+    """FFN norm + Q8_0 + gate | up + SwiGLU + Q8_0 of the result in one launch, against the oracle's
+    chain rmsnorm -> gemv x 2 -> silu_mul -> quantize.  The projections agree with the oracle's to
+    the float bar only, so a value on a rounding boundary may land one int8 step away and a block
+    maximum may round to the neighbouring f16 scale: the dequantized result must meet the oracle's
+    SwiGLU output within one quantization step, codes differ by at most one step and rarely."""
+    _say(f"ffn gate|up fused m={m} k={k}")
+    wg, _ = util.make_weights(Q4_K, m, k, seed=71, sigma=0.05)
+    wu, _ = util.make_weights(Q4_K, m, k, seed=72, sigma=0.05)
+    x = util.make_x(k, 73) * np.float32(1.7)
+    nw = (1.0 + 0.2 * util.make_x(k, 74)).astype(np.float32)
+    q, sc = hip.ffn_gate_up_fused(wg, wu, m, k, x, nw, 1e-5)
+    n = orc.rmsnorm(x, nw, 1e-5)
+    h = orc.silu_mul(orc.gemv(Q4_K, wg, n, m, k), orc.gemv(Q4_K, wu, n, m, k))
+    rs, rq = orc.quantize_q8_0(h)
+    dq = np.abs(q.astype(np.int32) - rq.astype(np.int32))
+    assert dq.max() <= 1 and np.count_nonzero(dq) <= max(2, 0.02 * dq.size), (int(dq.max()), np.count_nonzero(dq))
+    ulp = np.abs(sc.astype(np.float16).view(np.int16).astype(np.int32) - rs.astype(np.float16).view(np.int16).astype(np.int32))
+    assert np.array_equal(sc, sc.astype(np.float16).astype(np.float32)) and ulp.max() <= 1
+    deq = q.astype(np.float32).reshape(-1, 32) * sc[:, None]
+    assert (np.abs(deq - h.reshape(-1, 32)) <= 1.01 * rs[:, None] + 1e-9).all()
+
+
+def test_fused_launches_refuse_what_they_do_not_cover(hip):
+    w = np.zeros(8 * 32 * 144, np.uint8)
+    with pytest.raises(hip_api.HipError) as e:     # k beyond one wavefront of 64-weight units
+        hip.qkv_fused(Q4_K, w, 8, None, None, None, 8192, np.zeros(8192, np.float32), np.ones(8192, np.float32), 1e-5)
+    assert e.value.status == 3
+    with pytest.raises(hip_api.HipError) as e:     # m not a whole number of 32-row Q8_0 blocks
+        hip.ffn_gate_up_fused(w[:8 * 144], w[:8 * 144], 8, 256, np.zeros(256, np.float32), np.ones(256, np.float32), 1e-5)
+    assert e.value.status == 3
+
+
+def test_ffn_gate_up_fused_is_bitwise_the_separate_launches(hip, orc):
+    """The fused launch computes what rmsnorm+Q8_0 -> fused gate|up GEMV -> Q8_0 compute as three
+    launches: same activation bytes, same per-row arithmetic, so the same int8 codes and scales."""
+    m, k = 2048, 4096
+    wg, _ = util.make_weights(Q4_K, m, k, seed=81)
+    wu, _ = util.make_weights(Q4_K, m, k, seed=82)
+    x = util.make_x(k, 83)
+    nw = (1.0 + 0.1 * util.make_x(k, 84)).astype(np.float32)
+    q, sc = hip.ffn_gate_up_fused(wg, wu, m, k, x, nw, 1e-5)
+    n, _, _ = hip.rmsnorm_q8_0(x, nw, 1e-5)
+    h = hip.silu_mul(hip.gemv(Q4_K, wg, n, m, k), hip.gemv(Q4_K, wu, n, m, k))
+    rs, rq = hip.quantize_q8_0(h)
+    assert np.array_equal(q, rq) and np.array_equal(sc.view(np.uint32), rs.view(np.uint32))
