@@ -79,6 +79,16 @@ template <> struct KvOps<kv_half> {
     }
 };
 
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also fences global memory, which
+// on this target means waiting for every outstanding global load of the wavefront -- including
+// prefetched weight rows that nothing behind the barrier needs yet.  Use this where the data
+// exchanged across the barrier lives in LDS.
+__device__ __forceinline__ void lds_barrier() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
 // 4 x int8 dot with int32 accumulate (v_dot4_i32_i8).
 __device__ __forceinline__ int dot4(uint32_t a, uint32_t b, int c) {
     return __builtin_amdgcn_sdot4(static_cast<int>(a), static_cast<int>(b), c, false);

@@ -352,7 +352,7 @@ __device__ __forceinline__ void gemv_compute(const GemvArgs& p, const GemvTile<T
         }
     }
     if (KS > 1) {
-        __syncthreads();
+        lds_barrier();
         if (threadIdx.x < RB && r + threadIdx.x < r1) {
             float v[NM];
 #pragma unroll

@@ -40,49 +40,60 @@ struct RowGemvPairArgs {
     uint32_t n_blocks_a;
 };
 
-// rmsnorm + Q8_0 of x[0, k) into LDS; all 64 * NW threads take part (k % 32 == 0, k <= 4096)
+// rmsnorm + Q8_0 of x[0, k) into LDS by all 64 * NW threads (k % 32 == 0, k <= 4096), in two steps:
+// load() issues the loads of x and the norm weights, finish() does the rest.  The caller issues
+// its weight-row loads between the two: the hardware counts outstanding loads in order, so a wait
+// for x placed behind the weight loads would wait for every weight row as well.
 template <int NW>
-__device__ __forceinline__ void norm_quant_to_lds(const float* __restrict__ x, const float* __restrict__ w, uint32_t k, float eps,
-                                                  uint32_t* s_xq, float* s_xs, double* s_part) {
-    constexpr int NT = 64 * NW, MAXIT = 1024 / NT;
+struct NormQuant {
+    static constexpr int NT = 64 * NW, MAXIT = 1024 / NT;
     float4 v[MAXIT], g[MAXIT];
-    double s = 0.0;
+    __device__ __forceinline__ void load(const float* __restrict__ x, const float* __restrict__ w, uint32_t k) {
 #pragma unroll
-    for (int it = 0; it < MAXIT; ++it) {
-        const uint32_t i = (threadIdx.x + NT * it) * 4;
-        if (i < k) {
-            v[it] = *reinterpret_cast<const float4*>(x + i);
-            g[it] = *reinterpret_cast<const float4*>(w + i);
+        for (int it = 0; it < MAXIT; ++it) {
+            const uint32_t i = (threadIdx.x + NT * it) * 4;
+            v[it] = make_float4(0.f, 0.f, 0.f, 0.f);
+            g[it] = v[it];
+            if (i < k) {
+                v[it] = *reinterpret_cast<const float4*>(x + i);
+                g[it] = *reinterpret_cast<const float4*>(w + i);
+            }
+        }
+    }
+    __device__ __forceinline__ void finish(uint32_t k, float eps, uint32_t* s_xq, float* s_xs, double* s_part) {
+        double s = 0.0;
+#pragma unroll
+        for (int it = 0; it < MAXIT; ++it) {   // elements past k are zero
             s += static_cast<double>(v[it].x) * v[it].x;
             s += static_cast<double>(v[it].y) * v[it].y;
             s += static_cast<double>(v[it].z) * v[it].z;
             s += static_cast<double>(v[it].w) * v[it].w;
         }
-    }
-    for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
-    if ((threadIdx.x & 63) == 0) s_part[threadIdx.x >> 6] = s;
-    __syncthreads();
-    double tot = 0.0;
+        for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
+        if ((threadIdx.x & 63) == 0) s_part[threadIdx.x >> 6] = s;
+        lds_barrier();
+        double tot = 0.0;
 #pragma unroll
-    for (int i = 0; i < NW; ++i) tot += s_part[i];
-    const float inv = static_cast<float>(1.0 / sqrt(tot / static_cast<double>(k) + static_cast<double>(eps)));
+        for (int i = 0; i < NW; ++i) tot += s_part[i];
+        const float inv = static_cast<float>(1.0 / sqrt(tot / static_cast<double>(k) + static_cast<double>(eps)));
 #pragma unroll
-    for (int it = 0; it < MAXIT; ++it) {
-        const uint32_t i = (threadIdx.x + NT * it) * 4;
-        if (i < k) {   // k % 32 == 0: the eight lanes of a block are live together
-            float4 o;
-            o.x = __fmul_rn(__fmul_rn(v[it].x, inv), g[it].x);
-            o.y = __fmul_rn(__fmul_rn(v[it].y, inv), g[it].y);
-            o.z = __fmul_rn(__fmul_rn(v[it].z, inv), g[it].z);
-            o.w = __fmul_rn(__fmul_rn(v[it].w, inv), g[it].w);
-            float sc;
-            const uint32_t packed = q8_quantize_quad(o, sc);
-            s_xq[i >> 2] = packed;
-            if ((threadIdx.x & 7) == 0) s_xs[i >> 5] = sc;
+        for (int it = 0; it < MAXIT; ++it) {
+            const uint32_t i = (threadIdx.x + NT * it) * 4;
+            if (i < k) {   // k % 32 == 0: the eight lanes of a block are live together
+                float4 o;
+                o.x = __fmul_rn(__fmul_rn(v[it].x, inv), g[it].x);
+                o.y = __fmul_rn(__fmul_rn(v[it].y, inv), g[it].y);
+                o.z = __fmul_rn(__fmul_rn(v[it].z, inv), g[it].z);
+                o.w = __fmul_rn(__fmul_rn(v[it].w, inv), g[it].w);
+                float sc;
+                const uint32_t packed = q8_quantize_quad(o, sc);
+                s_xq[i >> 2] = packed;
+                if ((threadIdx.x & 7) == 0) s_xs[i >> 5] = sc;
+            }
         }
+        lds_barrier();
     }
-    __syncthreads();
-}
+};
 
 template <class T, int NM>
 struct RowTile {
@@ -93,9 +104,13 @@ struct RowTile {
     }
 };
 
-// The work of workgroup `block` on matrix p.  Every thread of the workgroup must call this (it
-// contains barriers when NORM or SILU_Q8), including wavefronts whose row range is empty.
-template <class T, int NW, bool NORM, int EPI>
+// The work of workgroup `block` on matrix p: wavefront w owns rows (block * NW + w) * ROWS .. + ROWS.
+// ALL of a wavefront's weight loads are issued first, so the whole matrix is in flight across the
+// chip while the activations are being prepared (NORM: a memory round trip for x and the norm
+// weights, an f64 reduction, two barriers), and what is left afterwards is arithmetic on
+// registers.  Every thread of the workgroup must call this (it contains barriers when NORM or
+// SILU_Q8), including wavefronts whose row range is empty.
+template <class T, int NW, int ROWS, bool NORM, int EPI>
 __device__ __forceinline__ void row_gemv_body(const RowGemvArgs& p, uint32_t block, uint32_t* s_xq, float* s_xs, double* s_part,
                                               float* s_out) {
     constexpr int NM = EPI == FEPI_SILU_Q8 ? 2 : 1;
@@ -103,52 +118,52 @@ __device__ __forceinline__ void row_gemv_body(const RowGemvArgs& p, uint32_t blo
     const uint32_t n_units = p.k / T::ELEMS_PER_UNIT;
     const bool live = lane < n_units;
     const uint32_t unit = live ? lane : 0;
-    uint32_t r = (block * NW + wave) * p.rows_per_wave;
-    const uint32_t r1 = min(p.m, r + p.rows_per_wave);
-    const bool has_rows = r < p.m;
+    const uint32_t r0 = (block * NW + wave) * ROWS;
 
-    RowTile<T, NM> ta, tb;
-    if (has_rows) ta.load(p, unit, r);   // in flight while the activations are prepared
+    NormQuant<NW> nq;
+    if (NORM) {
+        nq.load(p.x, p.norm_w, p.k);
+        __builtin_amdgcn_sched_barrier(0);   // x and the norm weights first: they are waited for first
+    }
+    // DEPTH rows in flight per wavefront: their loads are issued before the activations are
+    // prepared, and each finished row's buffer is refilled with the row DEPTH further on
+    constexpr int DEPTH = ROWS < 2 ? ROWS : 2;
+    RowTile<T, NM> t[DEPTH];
+#pragma unroll
+    for (int i = 0; i < DEPTH; ++i) t[i].load(p, unit, min(r0 + i, p.m - 1));   // rows past the end re-read the last row
+    __builtin_amdgcn_sched_barrier(0);   // the loads are issued here, not wherever their first use would pull them
 
     typename T::Act act;
     if (NORM) {
-        norm_quant_to_lds<NW>(p.x, p.norm_w, p.k, p.eps, s_xq, s_xs, s_part);
+        nq.finish(p.k, p.eps, s_xq, s_xs, s_part);
         T::load_act(act, reinterpret_cast<const int8_t*>(s_xq), s_xs, unit, live);
     } else {
         T::load_act(act, p.xq, p.xs, unit, live);
     }
 
-    auto finish = [&](const RowTile<T, NM>& t, uint32_t row) {
+#pragma unroll
+    for (int i = 0; i < ROWS; ++i) {
+        const uint32_t row = r0 + i;
         float tot[NM];
 #pragma unroll
-        for (int mi = 0; mi < NM; ++mi) tot[mi] = wave_sum(T::dot(t.w[mi], act, unit, nullptr));
-        if (lane == 0) {
+        for (int mi = 0; mi < NM; ++mi) tot[mi] = wave_sum(T::dot(t[i % DEPTH].w[mi], act, unit, nullptr));
+        if (i + DEPTH < ROWS) t[i % DEPTH].load(p, unit, min(r0 + i + DEPTH, p.m - 1));
+        if (lane == 0 && row < p.m) {
             if (EPI == FEPI_SILU_Q8) {
                 // cera/src/backend/cpu.rs:2570-2575: g / (1 + expf(-g)) * u
                 const float g = tot[0];
-                s_out[row - block * NW * p.rows_per_wave] = __fmul_rn(__fdiv_rn(g, __fadd_rn(1.0f, cera_expf(-g))), tot[NM - 1]);
+                s_out[row - block * NW * ROWS] = __fmul_rn(__fdiv_rn(g, __fadd_rn(1.0f, cera_expf(-g))), tot[NM - 1]);
             } else {
                 p.y[row] = EPI == FEPI_ADD ? p.resid[row] + tot[0] : tot[0];
             }
         }
-    };
-    if (has_rows) {
-        for (;;) {
-            if (r + 1 >= r1) { finish(ta, r); break; }
-            tb.load(p, unit, r + 1);
-            finish(ta, r);
-            ++r;
-            if (r + 1 >= r1) { finish(tb, r); break; }
-            ta.load(p, unit, r + 1);
-            finish(tb, r);
-            ++r;
-        }
     }
     if (EPI == FEPI_SILU_Q8) {
-        // the workgroup's NW * rows_per_wave = 32 rows are one Q8_0 block of the next projection's input
-        __syncthreads();
+        // the workgroup's NW * ROWS = 32 rows are one Q8_0 block of the next projection's input
+        static_assert(EPI != FEPI_SILU_Q8 || NW * ROWS == 32, "a workgroup must own exactly one Q8_0 block of output rows");
+        lds_barrier();
         if (wave == 0) {
-            const uint32_t row0 = block * NW * p.rows_per_wave;
+            const uint32_t row0 = block * NW * ROWS;
             const bool q_live = lane < 8 && row0 < p.m;   // m % 32 == 0: the block is whole or absent
             const float4 h = q_live ? reinterpret_cast<const float4*>(s_out)[lane] : make_float4(0.f, 0.f, 0.f, 0.f);
             float sc;
@@ -161,22 +176,22 @@ __device__ __forceinline__ void row_gemv_body(const RowGemvArgs& p, uint32_t blo
     }
 }
 
-template <class T, int NW, bool NORM, int EPI>
-static __global__ __launch_bounds__(64 * NW) void row_gemv_kernel(RowGemvArgs p) {
+template <class T, int NW, int ROWS, bool NORM, int EPI>
+static __global__ __launch_bounds__(64 * NW, 2) void row_gemv_kernel(RowGemvArgs p) {
     __shared__ uint32_t s_xq[NORM ? 1024 : 1];
     __shared__ float s_xs[NORM ? 128 : 1];
     __shared__ double s_part[NW];
     __shared__ __attribute__((aligned(16))) float s_out[EPI == FEPI_SILU_Q8 ? 32 : 4];
-    row_gemv_body<T, NW, NORM, EPI>(p, blockIdx.x, s_xq, s_xs, s_part, s_out);
+    row_gemv_body<T, NW, ROWS, NORM, EPI>(p, blockIdx.x, s_xq, s_xs, s_part, s_out);
 }
 
-template <class TA, class TB, int NW, bool NORM>
-static __global__ __launch_bounds__(64 * NW) void row_gemv_pair_kernel(RowGemvPairArgs p) {
+template <class TA, class TB, int NW, int ROWS, bool NORM>
+static __global__ __launch_bounds__(64 * NW, 2) void row_gemv_pair_kernel(RowGemvPairArgs p) {
     __shared__ uint32_t s_xq[NORM ? 1024 : 1];
     __shared__ float s_xs[NORM ? 128 : 1];
     __shared__ double s_part[NW];
-    if (blockIdx.x < p.n_blocks_a) row_gemv_body<TA, NW, NORM, FEPI_STORE>(p.a, blockIdx.x, s_xq, s_xs, s_part, nullptr);
-    else row_gemv_body<TB, NW, NORM, FEPI_STORE>(p.b, blockIdx.x - p.n_blocks_a, s_xq, s_xs, s_part, nullptr);
+    if (blockIdx.x < p.n_blocks_a) row_gemv_body<TA, NW, ROWS, NORM, FEPI_STORE>(p.a, blockIdx.x, s_xq, s_xs, s_part, nullptr);
+    else row_gemv_body<TB, NW, ROWS, NORM, FEPI_STORE>(p.b, blockIdx.x - p.n_blocks_a, s_xq, s_xs, s_part, nullptr);
 }
 
 // ---------------------------------------------------------------------------
@@ -210,9 +225,10 @@ cera_hip_status cera_launch_ffn_gate_up_fused(cera_hip_ctx* ctx, const cera_hip_
         gate->m % 32)
         return CERA_HIP_OK;
     RowGemvArgs a;
-    fill(a, gate, up, 32 / FUSED_NW);   // 32 rows per workgroup: one Q8_0 block of the output
+    constexpr int ROWS = 32 / FUSED_NW;   // 32 rows per workgroup: one Q8_0 block of the output
+    fill(a, gate, up, ROWS);
     a.x = x; a.norm_w = norm_w; a.eps = eps; a.out_q = out_q; a.out_s = out_s;
-    hipLaunchKernelGGL((row_gemv_kernel<Q4K, FUSED_NW, true, FEPI_SILU_Q8>), dim3(blocks_for(a.m, a.rows_per_wave)),
+    hipLaunchKernelGGL((row_gemv_kernel<Q4K, FUSED_NW, ROWS, true, FEPI_SILU_Q8>), dim3(blocks_for(a.m, ROWS)),
                        dim3(64 * FUSED_NW), 0, ctx->stream, a);
     HIP_TRY(ctx, hipGetLastError());
     *launched = true;
@@ -224,9 +240,9 @@ cera_hip_status cera_launch_qkv_fused(cera_hip_ctx* ctx, const cera_hip_dtensor*
                                       const float* norm_w, float eps, float* ya, float* yb, bool* launched) {
     *launched = false;
     if (!fused_type(wa->dtype) || !fused_k(wa->k) || (wb && (!fused_type(wb->dtype) || wb->k != wa->k))) return CERA_HIP_OK;
-    // about 12 wavefronts per CU over both matrices, at least one row per wavefront
+    // two rows per wavefront (12 wavefronts per CU on the 8B shapes), one for short matrices
     const uint64_t rows = wa->m + (wb ? wb->m : 0);
-    const uint32_t rpw = static_cast<uint32_t>(std::max<uint64_t>(1, rows / (static_cast<uint64_t>(ctx->n_cu) * 12)));
+    const uint32_t rpw = rows >= static_cast<uint64_t>(ctx->n_cu) * 8 ? 2 : 1;
     RowGemvPairArgs p;
     fill(p.a, wa, nullptr, rpw);
     p.a.x = x; p.a.norm_w = norm_w; p.a.eps = eps; p.a.y = ya;
@@ -241,10 +257,16 @@ cera_hip_status cera_launch_qkv_fused(cera_hip_ctx* ctx, const cera_hip_dtensor*
     }
     const dim3 grid(n_blocks), block(64 * FUSED_NW);
     const uint32_t ta = wa->dtype, tb = wb ? wb->dtype : wa->dtype;
-    if (ta == CERA_HIP_Q4_K && tb == CERA_HIP_Q6_K) hipLaunchKernelGGL((row_gemv_pair_kernel<Q4K, Q6K, FUSED_NW, true>), grid, block, 0, ctx->stream, p);
-    else if (ta == CERA_HIP_Q4_K && tb == CERA_HIP_Q4_K) hipLaunchKernelGGL((row_gemv_pair_kernel<Q4K, Q4K, FUSED_NW, true>), grid, block, 0, ctx->stream, p);
-    else if (ta == CERA_HIP_Q6_K && tb == CERA_HIP_Q6_K) hipLaunchKernelGGL((row_gemv_pair_kernel<Q6K, Q6K, FUSED_NW, true>), grid, block, 0, ctx->stream, p);
-    else hipLaunchKernelGGL((row_gemv_pair_kernel<Q6K, Q4K, FUSED_NW, true>), grid, block, 0, ctx->stream, p);
+#define QKV_LAUNCH(TA_, TB_)                                                                                                  \
+    do {                                                                                                                      \
+        if (rpw == 2) hipLaunchKernelGGL((row_gemv_pair_kernel<TA_, TB_, FUSED_NW, 2, true>), grid, block, 0, ctx->stream, p); \
+        else hipLaunchKernelGGL((row_gemv_pair_kernel<TA_, TB_, FUSED_NW, 1, true>), grid, block, 0, ctx->stream, p);          \
+    } while (0)
+    if (ta == CERA_HIP_Q4_K && tb == CERA_HIP_Q6_K) QKV_LAUNCH(Q4K, Q6K);
+    else if (ta == CERA_HIP_Q4_K && tb == CERA_HIP_Q4_K) QKV_LAUNCH(Q4K, Q4K);
+    else if (ta == CERA_HIP_Q6_K && tb == CERA_HIP_Q6_K) QKV_LAUNCH(Q6K, Q6K);
+    else QKV_LAUNCH(Q6K, Q4K);
+#undef QKV_LAUNCH
     HIP_TRY(ctx, hipGetLastError());
     *launched = true;
     return CERA_HIP_OK;

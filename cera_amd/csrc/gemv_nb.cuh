@@ -65,7 +65,7 @@ static __global__ __launch_bounds__(64 * KS) void gemv_nb_kernel(GemvNbArgs p) {
             }
         }
         if (KS > 1) {
-            __syncthreads();
+            lds_barrier();
             if (threadIdx.x < RB * NB) {
                 const uint32_t rb = threadIdx.x / NB, b = threadIdx.x % NB;
                 if (rr + rb < r1 && b < p.n_tok) {
