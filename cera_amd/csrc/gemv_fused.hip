@@ -159,29 +159,30 @@ __device__ __forceinline__ void row_gemv_body(const RowGemvArgs& p, uint32_t blo
         }
     }
     if (EPI == FEPI_SILU_Q8) {
-        // the workgroup's NW * ROWS = 32 rows are one Q8_0 block of the next projection's input
-        static_assert(EPI != FEPI_SILU_Q8 || NW * ROWS == 32, "a workgroup must own exactly one Q8_0 block of output rows");
+        // the workgroup's NW * ROWS rows are whole Q8_0 blocks of the next projection's input
+        static_assert(EPI != FEPI_SILU_Q8 || (NW * ROWS) % 32 == 0, "a workgroup must own whole Q8_0 blocks of output rows");
         lds_barrier();
         if (wave == 0) {
+            constexpr uint32_t NQ = NW * ROWS / 4;   // float4 groups of the workgroup's rows, 8 per Q8_0 block
             const uint32_t row0 = block * NW * ROWS;
-            const bool q_live = lane < 8 && row0 < p.m;   // m % 32 == 0: the block is whole or absent
+            const bool q_live = lane < NQ && row0 + 4 * lane < p.m;   // m % 32 == 0: a block is whole or absent
             const float4 h = q_live ? reinterpret_cast<const float4*>(s_out)[lane] : make_float4(0.f, 0.f, 0.f, 0.f);
             float sc;
             const uint32_t packed = q8_quantize_quad(h, sc);
             if (q_live) {
                 reinterpret_cast<uint32_t*>(p.out_q + row0)[lane] = packed;
-                if (lane == 0) p.out_s[row0 >> 5] = sc;
+                if ((lane & 7) == 0) p.out_s[(row0 >> 5) + (lane >> 3)] = sc;
             }
         }
     }
 }
 
 template <class T, int NW, int ROWS, bool NORM, int EPI>
-static __global__ __launch_bounds__(64 * NW, 2) void row_gemv_kernel(RowGemvArgs p) {
+static __global__ __launch_bounds__(64 * NW, NW <= 8 ? 2 : 1) void row_gemv_kernel(RowGemvArgs p) {
     __shared__ uint32_t s_xq[NORM ? 1024 : 1];
     __shared__ float s_xs[NORM ? 128 : 1];
     __shared__ double s_part[NW];
-    __shared__ __attribute__((aligned(16))) float s_out[EPI == FEPI_SILU_Q8 ? 32 : 4];
+    __shared__ __attribute__((aligned(16))) float s_out[EPI == FEPI_SILU_Q8 ? NW * ROWS : 4];
     row_gemv_body<T, NW, ROWS, NORM, EPI>(p, blockIdx.x, s_xq, s_xs, s_part, s_out);
 }
 
@@ -225,11 +226,14 @@ cera_hip_status cera_launch_ffn_gate_up_fused(cera_hip_ctx* ctx, const cera_hip_
         gate->m % 32)
         return CERA_HIP_OK;
     RowGemvArgs a;
-    constexpr int ROWS = 32 / FUSED_NW;   // 32 rows per workgroup: one Q8_0 block of the output
+    // 16 wavefronts x 4 rows: a workgroup owns two Q8_0 blocks of the output, and 14336 rows make
+    // 224 workgroups -- one per CU in a single wave of the launch (448 eight-wavefront workgroups
+    // leave a quarter of the CUs with half the others' share: 1 % slower end to end)
+    constexpr int GATE_UP_NW = 16, ROWS = 4;
     fill(a, gate, up, ROWS);
     a.x = x; a.norm_w = norm_w; a.eps = eps; a.out_q = out_q; a.out_s = out_s;
-    hipLaunchKernelGGL((row_gemv_kernel<Q4K, FUSED_NW, ROWS, true, FEPI_SILU_Q8>), dim3(blocks_for(a.m, ROWS)),
-                       dim3(64 * FUSED_NW), 0, ctx->stream, a);
+    hipLaunchKernelGGL((row_gemv_kernel<Q4K, GATE_UP_NW, ROWS, true, FEPI_SILU_Q8>), dim3((a.m + GATE_UP_NW * ROWS - 1) / (GATE_UP_NW * ROWS)),
+                       dim3(64 * GATE_UP_NW), 0, ctx->stream, a);
     HIP_TRY(ctx, hipGetLastError());
     *launched = true;
     return CERA_HIP_OK;

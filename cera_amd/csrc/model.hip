@@ -512,11 +512,10 @@ static cera_hip_status decode_step(cera_hip_model* m, uint32_t pos, bool want_lo
 
     for (uint32_t i = 0; i < c.n_layers; ++i) {
         LayerDev& L = m->layers[i];
-        static const bool tmp_nofuse = getenv("CERA_TMP_NOFUSE") != nullptr;   // TMP experiment hook
         // Q|K|V with the attention norm and its Q8_0 quantization done by the projection's own
         // workgroups (one launch instead of two), where the shapes allow
         bool qkv_done = false;
-        if (L.qkv && !tmp_nofuse)
+        if (L.qkv)
             CERA_TRY(cera_launch_qkv_fused(ctx, L.qkv, L.qkv_rows == q_dim + kv_dim ? L.v : nullptr, m->hidden, L.attn_norm,
                                            c.rms_eps, m->q, m->v, &qkv_done));
         if (qkv_done) {
@@ -555,8 +554,7 @@ static cera_hip_status decode_step(cera_hip_model* m, uint32_t pos, bool want_lo
         // gate | up with the FFN norm in front and SwiGLU + the down projection's Q8_0 quantization
         // behind, all in one launch instead of three, where the shapes allow
         bool ffn_done = false;
-        if (!tmp_nofuse)
-            CERA_TRY(cera_launch_ffn_gate_up_fused(ctx, L.gate, L.up, m->hidden, L.ffn_norm, c.rms_eps, m->xq, m->xs, &ffn_done));
+        CERA_TRY(cera_launch_ffn_gate_up_fused(ctx, L.gate, L.up, m->hidden, L.ffn_norm, c.rms_eps, m->xq, m->xs, &ffn_done));
         const bool fuse = L.gate->dtype == L.up->dtype && L.gate->dtype != CERA_HIP_Q5_K;
         if (!ffn_done) CERA_TRY(norm_quant(m, m->hidden, L.ffn_norm, c.hidden, 1, m->normed));
         if (ffn_done) {
