@@ -3,12 +3,12 @@
 #include <cstring>
 #include <new>
 
-#include "attention.cuh"
-#include "gemv_launch.cuh"
-#include "gemv_nb.cuh"
-#include "glue.cuh"
+#include "attention.hip.h"
+#include "gemv_launch.hip.h"
+#include "gemv_nb.hip.h"
+#include "glue.hip.h"
 #include "host_common.h"
-#include "quantize.cuh"
+#include "quantize.hip.h"
 
 bool cera_gemv_launch_q4k(const GemvArgs&, const GemvPlan&, int, bool, hipStream_t);
 bool cera_gemv_launch_pair_q4k_q6k(const GemvPairArgs& a, const GemvPlan& pa, const GemvPlan& pb, hipStream_t s);

@@ -22,9 +22,9 @@
 // only cross-lane traffic is the 3-step reduction of the q.k partials and one
 // reduction at the end of the part.
 #pragma once
-#include "common.cuh"
+#include "common.hip.h"
 #include "attn_types.h"
-#include "quantize.cuh"
+#include "quantize.hip.h"
 
 #define ATTN_MAX_PARTS 1024  // the merge kernel keeps one weight per part in LDS
 #define ATTN_MERGE_PF 8       // parts per lane group the merge kernel requests per round trip (x8 groups)

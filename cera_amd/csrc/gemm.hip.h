@@ -1,6 +1,6 @@
 // Prefill GEMM: out[m][n] = W[m, k] . B[k, n] with W in native GGUF blocks and
 // B the Q8_0-quantized activations of n tokens, on the int8 matrix cores
-// (Q4_K, Q4_0, Q4_1, Q8_0; Q6_K has a kernel of its own in gemm_q6k_f16.cuh).
+// (Q4_K, Q4_0, Q4_1, Q8_0; Q6_K has a kernel of its own in gemm_q6k_f16.hip.h).
 //
 // Arithmetic contract (cera's batched int8 path, cera/src/backend/simd.rs:
 // 5693-5878 Q4_K, :5893-5976 Q4_1, :4718-5010 Q4_0/Q8_0;
@@ -36,8 +36,8 @@
 //   B: 64 tokens x 128 int8 activations, cs/cm: activation scale and
 //      scale*sum(a) per 32-block.
 #pragma once
-#include "common.cuh"
-#include "quantize.cuh"
+#include "common.hip.h"
+#include "quantize.hip.h"
 
 #define GEMM_BM 128
 #define GEMM_BN 64

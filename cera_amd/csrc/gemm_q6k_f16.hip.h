@@ -1,6 +1,6 @@
 // Prefill GEMM for Q6_K with the block dots on the f16 matrix cores.
 //
-// Same arithmetic contract as gemm.cuh (cera's batched int8 path for Q6_K,
+// Same arithmetic contract as gemm.hip.h (cera's batched int8 path for Q6_K,
 // cera/src/backend/simd.rs:5988-6195): exact integer dots of the 6-bit codes (minus 32) with
 // the int8 activations per 16-element scale group, then  sum_g (sc[g]*d) * xs[b] * dot[g].
 // The int8 kernel is VALU-bound for this type: two groups per 32-block, each needing a convert
@@ -10,7 +10,7 @@
 // integer dot (|dot| <= 16*32*127, far below 2^24): no convert, and no sign extension (the
 // -32 is one packed f16 add on the 1024 + q form the unpack produces anyway).  The per-output
 // scales (sc*d)[row] x xs[token] of the two groups of a block come from one two-block
-// outer-product MFMA as in gemm.cuh.  VALU work per output per 32-block: two FMAs.
+// outer-product MFMA as in gemm.hip.h.  VALU work per output per 32-block: two FMAs.
 //
 // 6-bit codes become f16 without a convert: the low nibble and the two high bits are OR-ed into
 // the mantissa of 1024.0 (ulp 1), giving 1024 + q.  That pairs bytes (0, 2) and (1, 3) of each
@@ -18,12 +18,12 @@
 // staged in the same order (gemm_act_f16_kernel) -- the order inside a scale group does not
 // matter to its dot product.
 //
-// Tiles as gemm.cuh: 256 threads = 2 x 2 wavefronts, 128 rows x 64 tokens, K in steps of 128
+// Tiles as gemm.hip.h: 256 threads = 2 x 2 wavefronts, 128 rows x 64 tokens, K in steps of 128
 // (one half of a super-block); LDS rows are 256 B + 16 B pad (57 KB a workgroup, two per CU: an
 // unpadded, XOR-swizzled layout that fits three was tried and spilled on its sixteen distinct
 // fragment addresses).
 #pragma once
-#include "gemm.cuh"
+#include "gemm.hip.h"
 
 typedef _Float16 gq_v8h __attribute__((ext_vector_type(8)));
 typedef _Float16 gq_h2 __attribute__((ext_vector_type(2)));

@@ -21,7 +21,7 @@
 // its 64 partial sums with DPP; the KS per-wavefront sums meet in LDS and are
 // added in wavefront order (deterministic, no atomics).
 #pragma once
-#include "common.cuh"
+#include "common.hip.h"
 
 struct GemvArgs {
     const uint8_t* w;    // [m] rows of native blocks

@@ -14,10 +14,10 @@
 //     scale (silu_mul_inplace cpu.rs:2570-2575, then cpu.rs:942-958); the f32 vector is never stored.
 // A wavefront owns whole rows (one 64-weight unit per lane), walks its rows one at a time with
 // the next row's loads in flight, and reduces with DPP only: no LDS combine, no barrier in the
-// row loop.  Per-row arithmetic is gemv.cuh's (T::dot), so results meet the same bars.
-#include "gemv.cuh"
+// row loop.  Per-row arithmetic is gemv.hip.h's (T::dot), so results meet the same bars.
+#include "gemv.hip.h"
 #include "host_common.h"
-#include "quantize.cuh"
+#include "quantize.hip.h"
 
 enum { FEPI_STORE = 0, FEPI_ADD = 1, FEPI_SILU_Q8 = 2 };
 

@@ -2,7 +2,7 @@
 // values of the K split (KS wavefronts per workgroup, U units per lane), RB
 // (rows in flight) and the epilogue.
 #pragma once
-#include "gemv.cuh"
+#include "gemv.hip.h"
 #include "host_common.h"
 
 struct GemvPlan {

@@ -5,7 +5,7 @@
 // the prefill path for short batches (a few new tokens, speculative-decoding verification),
 // where an int8-MFMA tile would be mostly empty and one GEMV per token would re-read the weights.
 #pragma once
-#include "gemv.cuh"
+#include "gemv.hip.h"
 
 struct GemvNbArgs {
     const uint8_t* w;     // [m] rows of native blocks

@@ -1,6 +1,6 @@
 // gemv_pair_kernel instantiations: a Q4_K matrix and a Q6_K matrix whose rows each fit one wavefront
 // (k <= 4096) -- Q|K and V of a Q4_K_M-style layer in one launch.
-#include "gemv_launch.cuh"
+#include "gemv_launch.hip.h"
 
 bool cera_gemv_launch_pair_q4k_q6k(const GemvPairArgs& a, const GemvPlan& pa, const GemvPlan& pb, hipStream_t s) {
     if (pa.U != 1 || pa.KS != 1 || pb.U != 1 || pb.KS != 1) return false;

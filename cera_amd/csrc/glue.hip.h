@@ -4,8 +4,8 @@
 // (cera/src/backend/cpu.rs) so that their f32 outputs match it bit for bit
 // wherever the CPU order is a plain elementwise expression.
 #pragma once
-#include "common.cuh"
-#include "quantize.cuh"
+#include "common.hip.h"
+#include "quantize.hip.h"
 
 // ---------------------------------------------------------------------------
 // Row dequantisation (cera/src/quant.rs:364-886 via

@@ -10,7 +10,7 @@
 
 #include <type_traits>
 
-#include "glue.cuh"
+#include "glue.hip.h"
 #include "host_common.h"
 #include "model.h"
 

@@ -5,8 +5,8 @@
 #include <cmath>
 #include <cstring>
 
-#include "gemm_q6k_f16.cuh"
-#include "glue.cuh"
+#include "gemm_q6k_f16.hip.h"
+#include "glue.hip.h"
 #include "model.h"
 
 static bool gemm_type_ok(uint32_t t) {

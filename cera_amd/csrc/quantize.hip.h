@@ -8,7 +8,7 @@
 // Eight lanes own one block (a float4 each): loads and stores are fully
 // coalesced, the block maximum is a three-step DPP reduction.
 #pragma once
-#include "common.cuh"
+#include "common.hip.h"
 
 __device__ __forceinline__ int q8_round(float v, float id) {
     float r = rintf(__fmul_rn(v, id));  // v_rndne_f32

@@ -21,7 +21,7 @@
 //          f64 softmax sum in key order, one FMA chain per output column in key order.
 #include <cmath>
 
-#include "glue.cuh"
+#include "glue.hip.h"
 #include "host_common.h"
 #include "model.h"
 
