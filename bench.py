@@ -4,10 +4,12 @@
 Workload (BASELINE.json configs[1]): the Llama-3-8B decode-layer GEMV set at
 batch 1 -- per layer fused QKV 6144x4096, O 4096x4096, gate and up 14336x4096
 (Q4_K), down 4096x14336 (Q6_K), plus the output head 128256x4096 (Q6_K).  One
-"step" is one token's worth: 32 layers + head (129 launches: QKV, O, fused gate+up, down per layer) over
-4 841 250 816 bytes of weights, every layer in its own HBM allocation so the
-4.8 GB working set rotates far past the 256 MB last-level cache.  Activations
-(Q8_0-quantized x ~ N(0,1)) and weights are resident in HBM before timing.
+"step" is one token's worth, in the order and with the launches the decode path issues: per
+layer Q|K|V (rmsnorm + Q8_0 of its input inside the launch), O (+ residual), gate|up (rmsnorm +
+Q8_0 in, SwiGLU + Q8_0 out), down (+ residual); then rmsnorm + Q8_0 and the head: 130 launches
+over 4 841 250 816 bytes of weights, every layer in its own HBM allocation so the 4.8 GB
+working set rotates far past the 256 MB last-level cache.  Weights and the f32 / Q8_0 inputs
+(x ~ N(0,1)) are resident in HBM before timing.
 
 Prints ONE JSON line: metric / value / unit, the roofline of the dominant kernel, the CPU baseline,
 and (unless disabled) end-to-end, flash-decode and prefill-GEMM measurements.
@@ -33,7 +35,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 # `bench.py --pmc-probe` under rocprofv3 --pmc, summary in profiles/gemv_q4k_gate_up_hbm_traffic_pmc.txt).
 # It is a recorded measurement of this kernel configuration, not taken live: counters need the profiler.
 GATE_UP_TRAFFIC_BYTES = 66_328_548
-GATE_UP_TRAFFIC_KERNEL = "gemv_kernel<Q4K,1,2,4,2,false>"
+GATE_UP_KERNEL = "row_gemv_kernel<Q4K,16,4,true,2>"
 
 # (name, ggml type name, m, k, copies per step)
 LAYER_SET = [
@@ -44,6 +46,7 @@ LAYER_SET = [
     ("ffn_down", "Q6_K", 4096, 14336),
 ]
 HEAD = ("output", "Q6_K", 128256, 4096)
+CONFIG1 = ("config1_q4_0", "Q4_0", 4096, 4096)   # BASELINE.json configs[0]: the reference's CPU-runnable GEMV case
 N_LAYERS = 32
 
 
@@ -75,9 +78,24 @@ def host_cpu_info():
     return {"cpu_model": model, "physical_cores": len(cores) or None, "logical_cores": os.cpu_count()}
 
 
+def _time_calls(ctx, calls, iters, warm=3):
+    """Average microseconds per call of `calls[i % len(calls)]()` over `iters` calls (HIP events)."""
+    for i in range(warm):
+        calls[i % len(calls)]()
+    e0, e1 = ctx.event(), ctx.event()
+    ctx.record(e0)
+    for i in range(iters):
+        calls[i % len(calls)]()
+    ctx.record(e1)
+    ctx.sync()
+    return ctx.elapsed_ms(e0, e1) * 1e3 / iters
+
+
 def measure_attention(ctx, hip_api, rng):
-    """BASELINE.json configs[3]: GQA flash-decode, 32 q heads / 8 kv heads / head_dim 128, f32 KV
-    resident in HBM in the kernel's head-major layout; bytes = K + V read once."""
+    """BASELINE.json configs[3]: GQA flash-decode, 32 q heads / 8 kv heads / head_dim 128, KV resident in
+    HBM in the kernel's head-major layout; bytes = K + V read once.  Every context length rotates over
+    distinct caches (about 1 GiB in all) so each call streams from HBM, not from the 256 MB last-level
+    cache; the back-to-back rate on ONE cache is kept beside it where that cache fits the LLC."""
     n_heads, n_kv, hd = 32, 8, 128
     out = []
     max_l = 131072
@@ -91,48 +109,37 @@ def measure_attention(ctx, hip_api, rng):
     dq = ctx.to_device(rng.standard_normal(n_heads * hd, dtype=np.float32))
     dout = ctx.malloc(n_heads * hd * 4)
     scale = 1.0 / np.sqrt(hd)
-    for L in (512, 4096, 32768, 131072):
-        # each context length gets its own cache stride = L, as a model with max_seq_len = L would
-        call = lambda: ctx.check(ctx.lib.cera_hip_attn_decode_dev(ctx.h, dq, dk, dv, n_heads, n_kv, hd, L, L,
-                                                                  C.c_float(scale), 0, dout))
-        iters = 200 if L <= 4096 else 50
-        for _ in range(5):
-            call()
-        e0, e1 = ctx.event(), ctx.event()
-        ctx.record(e0)
-        for _ in range(iters):
-            call()
-        ctx.record(e1)
-        ctx.sync()
-        us = ctx.elapsed_ms(e0, e1) * 1e3 / iters
-        nbytes = 2 * n_kv * L * hd * 4 + 2 * n_heads * hd * 4
-        # below ~32k the K/V working set fits the 256 MB last-level cache when launched back to back
-        out.append({"context": L, "us_per_call": round(us, 2), "GB/s": round(nbytes / us / 1e3, 1),
-                    "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
-                    "cache_resident": 2 * n_kv * L * hd * 4 <= 256 << 20})
+
+    def rows(fn, esz, lengths, tag):
+        for L in lengths:
+            # each context length gets its own cache stride = L, as a model with max_seq_len = L would;
+            # cache i of the rotation starts i * (bytes of one cache) into the two big buffers
+            one = n_kv * L * hd * esz
+            n_rot = max(1, min(kv_bytes // one, -(-(1 << 30) // (2 * one))))
+            calls = [(lambda o=i * one: ctx.check(fn(ctx.h, dq, dk + o, dv + o, n_heads, n_kv, hd, L, L, C.c_float(scale), 0, dout)))
+                     for i in range(n_rot)]
+            iters = 256 if L <= 4096 else 48
+            us = _time_calls(ctx, calls, iters, warm=4)
+            nbytes = 2 * one + 2 * n_heads * hd * 4
+            row = {"context": L, "us_per_call": round(us, 2), "GB/s": round(nbytes / us / 1e3, 1),
+                   "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
+                   "rotating_caches": n_rot, "working_set_MB": round(2 * one * n_rot / 1e6, 1),
+                   "hbm_streamed": 2 * one * n_rot > (256 << 20)}
+            if tag:
+                row["kv"] = tag
+            if 2 * one <= 256 << 20 and n_rot > 1:
+                us1 = _time_calls(ctx, calls[:1], iters, warm=4)
+                row["one_cache_back_to_back_GB/s"] = round(nbytes / us1 / 1e3, 1)
+            out.append(row)
+
+    rows(ctx.lib.cera_hip_attn_decode_dev, 4, (512, 4096, 32768, 131072), None)
     # the same contexts over an f16 KV cache (KvCompression::F16): half the bytes per position
     chunk16 = chunk.astype(np.float16)
     dchunk16 = ctx.to_device(chunk16.view(np.uint16))
-    for off in range(0, kv_bytes // 2, chunk16.nbytes):
+    for off in range(0, kv_bytes, chunk16.nbytes):
         ctx.check(ctx.lib.cera_hip_copy_dev(ctx.h, dk + off, dchunk16, chunk16.nbytes))
         ctx.check(ctx.lib.cera_hip_copy_dev(ctx.h, dv + off, dchunk16, chunk16.nbytes))
-    for L in (4096, 32768, 131072):
-        call = lambda: ctx.check(ctx.lib.cera_hip_attn_decode_f16_dev(ctx.h, dq, dk, dv, n_heads, n_kv, hd, L, L,
-                                                                      C.c_float(scale), 0, dout))
-        iters = 200 if L <= 4096 else 50
-        for _ in range(5):
-            call()
-        e0, e1 = ctx.event(), ctx.event()
-        ctx.record(e0)
-        for _ in range(iters):
-            call()
-        ctx.record(e1)
-        ctx.sync()
-        us = ctx.elapsed_ms(e0, e1) * 1e3 / iters
-        nbytes = 2 * n_kv * L * hd * 2 + 2 * n_heads * hd * 4
-        out.append({"context": L, "kv": "f16", "us_per_call": round(us, 2), "GB/s": round(nbytes / us / 1e3, 1),
-                    "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
-                    "cache_resident": 2 * n_kv * L * hd * 2 <= 256 << 20})
+    rows(ctx.lib.cera_hip_attn_decode_f16_dev, 2, (4096, 32768, 131072), "f16")
     for d in (dk, dv, dchunk, dchunk16, dq, dout):
         ctx.free(d)
     return out
@@ -219,21 +226,33 @@ def measure_e2e(seed: int, n_thr: int):
             "all_logits_short_batch": short}
 
 
+def reference_decode_threads(physical, logical):
+    """The decode pool width cera picks for a bandwidth-bound model (more than 2.5 MB of weights per pool
+    dispatch, which an 8B model is): physical + physical / 4 capped at 24, never above the detected
+    logical count (cera README.md "How the decode thread count is chosen", CERA_DECODE_WIDE)."""
+    if not physical:
+        return max(1, min(12, logical or 1))   # the flat cap the sizing falls back to
+    return max(1, min(24, physical + physical // 4, logical or physical))
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--seed", type=int, default=20250)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    ap.add_argument("--cpu-threads", type=int, default=0,
+                    help="CPU-baseline pool width (default: the reference's own decode sizing rule for this host, "
+                         "capped at the 16 cores a one-GPU box gives a job)")
     ap.add_argument("--weight-copies", type=int, default=N_LAYERS,
                     help="distinct HBM copies of the layer weights the step rotates over (default: one per layer; "
                          "fewer lets the last-level cache hold them, which is NOT the reported configuration)")
     ap.add_argument("--no-e2e", action="store_true", help="skip the end-to-end model run (prefill 512 + greedy 256)")
     ap.add_argument("--no-extras", action="store_true", help="skip the flash-decode and prefill-GEMM side measurements")
     ap.add_argument("--pmc-probe", action="store_true",
-                    help="run only a 1 GiB copy kernel and one step of the fused gate+up GEMVs, for a "
+                    help="run only a 1 GiB copy kernel and a few launches of each per-layer GEMV kernel, for a "
                          "hardware-counter pass under rocprofv3 --pmc; prints no JSON")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -242,64 +261,118 @@ def main() -> int:
         return 2
 
     from cera_amd import hip_api, host_api as H
+    Op = hip_api.DecodeOp
 
     ctx = hip_api.Context(0)
     dev_name, n_cu, hbm = ctx.device_info()
     rng = np.random.default_rng(args.seed)
     n_thr = min(16, os.cpu_count() or 1)
+    eps = 1e-5
 
     # ---- synthetic weights: one properly quantized layer + head, cloned on device
     t0 = time.time()
     host = {}
-    for name, tname, m, k in LAYER_SET + [HEAD]:
+    for name, tname, m, k in LAYER_SET + [HEAD] + [CONFIG1]:
         w = rng.standard_normal((m, k), dtype=np.float32)
         w *= np.float32(0.02)
         host[name] = H.quantize(H.TYPE_IDS[tname], w, n_thr)
         del w
+    n_copies = max(1, min(N_LAYERS, args.weight_copies))
     dts = {}   # name -> list of device tensor handles (one per layer)
-    for name, tname, m, k in LAYER_SET:
+    for name, tname, m, k in LAYER_SET + [CONFIG1]:
         first = ctx.tensor_upload(H.TYPE_IDS[tname], m, k, host[name])
-        copies = [first] + [ctx.tensor_clone(first) for _ in range(max(1, min(N_LAYERS, args.weight_copies)) - 1)]
+        copies = [first] + [ctx.tensor_clone(first) for _ in range(n_copies - 1)]
         dts[name] = [copies[l % len(copies)] for l in range(N_LAYERS)]
     name, tname, m, k = HEAD
     dts[name] = [ctx.tensor_upload(H.TYPE_IDS[tname], m, k, host[name])]
     gen_s = time.time() - t0
 
-    # ---- activations, quantized on the device, resident before timing
+    # ---- inputs resident before timing: the f32 hidden state and norm weight the fused launches
+    # read, and Q8_0-quantized activations for the projections whose input arrives quantized
+    x_host = {kk: rng.standard_normal(kk, dtype=np.float32) for kk in (4096, 14336)}
+    norm_host = (1.0 + 0.1 * rng.standard_normal(4096)).astype(np.float32)
+    d_x = {kk: ctx.to_device(x_host[kk]) for kk in x_host}
+    d_norm = ctx.to_device(norm_host)
     acts = {}
     for kk in (4096, 14336):
-        x = rng.standard_normal(kk, dtype=np.float32)
-        dx = ctx.to_device(x)
         dxs, dxq = ctx.malloc(kk // 32 * 4), ctx.malloc(kk)
-        ctx.check(ctx.lib.cera_hip_quantize_q8_0_dev(ctx.h, dx, kk, dxs, dxq))
-        acts[kk] = (dxs, dxq, x)
-    outs = {name: ctx.malloc(m * 4) for name, _, m, _ in LAYER_SET + [HEAD]}
+        ctx.check(ctx.lib.cera_hip_quantize_q8_0_dev(ctx.h, d_x[kk], kk, dxs, dxq))
+        acts[kk] = (dxs, dxq)
+    outs = {name: ctx.malloc(m * 4) for name, _, m, _ in LAYER_SET + [HEAD] + [CONFIG1]}
+    d_ffn_q, d_ffn_s = ctx.malloc(14336), ctx.malloc(14336 // 32 * 4)     # the gate|up launch's Q8_0 output
+    d_head_in = ctx.malloc(4096 * 4)
+    d_head_q, d_head_s = ctx.malloc(4096), ctx.malloc(4096 // 32 * 4)
+    d_oq, d_os = ctx.malloc(4096), ctx.malloc(4096 // 32 * 4)
     ctx.sync()
 
-    def make_ops(entries):
-        arr = (hip_api.GemvOp * len(entries))()
-        for i, (name, layer, k) in enumerate(entries):
-            if isinstance(name, tuple):   # fused FFN pair: silu(gate.x) * (up.x) in one launch
-                arr[i] = hip_api.GemvOp(dts[name[0]][layer], dts[name[1]][layer], acts[k][0], acts[k][1], outs[name[0]])
-            else:
-                arr[i] = hip_api.GemvOp(dts[name][layer], None, acts[k][0], acts[k][1], outs[name])
+    def op_qkv(l):
+        return Op(kind=Op.NORM_GEMV, w=dts["attn_qkv"][l], x=d_x[4096], norm_w=d_norm, eps=eps, y=outs["attn_qkv"])
+
+    def op_o(l, xs=None, xq=None):
+        return Op(kind=Op.GEMV, w=dts["attn_output"][l], xs=xs or acts[4096][0], xq=xq or acts[4096][1], resid=d_x[4096],
+                  y=outs["attn_output"])
+
+    def op_gate_up(l):
+        return Op(kind=Op.NORM_GATE_UP, w=dts["ffn_gate"][l], w2=dts["ffn_up"][l], x=d_x[4096], norm_w=d_norm, eps=eps,
+                  out_q=d_ffn_q, out_s=d_ffn_s)
+
+    def op_down(l, fused_input=True):
+        xs, xq = (d_ffn_s, d_ffn_q) if fused_input else acts[14336]
+        return Op(kind=Op.GEMV, w=dts["ffn_down"][l], xs=xs, xq=xq, resid=d_x[4096], y=outs["ffn_down"])
+
+    op_head_norm = Op(kind=Op.NORM_QUANT, n=4096, x=d_x[4096], norm_w=d_norm, eps=eps, y=d_head_in, out_q=d_head_q, out_s=d_head_s)
+    op_head = Op(kind=Op.GEMV, w=dts["output"][0], xs=d_head_s, xq=d_head_q, y=outs["output"])
+    op_quant_o = Op(kind=Op.QUANT, n=4096, x=d_x[4096], out_q=d_oq, out_s=d_os)
+
+    def ops_array(ops):
+        arr = (Op * len(ops))()
+        for i, o in enumerate(ops):
+            arr[i] = o
         return arr
 
-    # group A: the dominant kernel (Q4_K 14336x4096 gate/up), B: other Q4_K, C: Q6_K
-    # (gate and up run as the fused pair the decode path uses: one launch, both matrices)
-    grp_a = make_ops([(("ffn_gate", "ffn_up"), l, 4096) for l in range(N_LAYERS)])
-    grp_b = make_ops([(n, l, 4096) for l in range(N_LAYERS) for n in ("attn_qkv", "attn_output")])
-    grp_c = make_ops([("ffn_down", l, 14336) for l in range(N_LAYERS)] + [("output", 0, 4096)])
-    groups = [("q4k_gate_up", grp_a), ("q4k_qkv_o", grp_b), ("q6k_down_head", grp_c)]
-    shape = {n: (t, m, k) for n, t, m, k in LAYER_SET + [HEAD]}
-    bytes_of = {n: algorithmic_bytes(H, *shape[n]) for n in shape}
-    grp_bytes = {
-        "q4k_gate_up": N_LAYERS * (bytes_of["ffn_gate"] + bytes_of["ffn_up"] - 4096 - 512 - 14336 * 4),
-        "q4k_qkv_o": N_LAYERS * (bytes_of["attn_qkv"] + bytes_of["attn_output"]),
-        "q6k_down_head": N_LAYERS * bytes_of["ffn_down"] + bytes_of["output"],
+    # one token: the decode path's launches in its order (attention itself is not part of the set)
+    step_ops = []
+    for l in range(N_LAYERS):
+        step_ops += [op_qkv(l), op_o(l), op_gate_up(l), op_down(l)]
+    step_ops += [op_head_norm, op_head]
+    step_arr = ops_array(step_ops)
+    # the same with the one quantization the decode path gets from its attention kernel done as a
+    # launch of its own: every Q8_0 quantization the reference performs per GEMV call is then inside
+    step_q_ops = []
+    for l in range(N_LAYERS):
+        step_q_ops += [op_qkv(l), op_quant_o, op_o(l, d_os, d_oq), op_gate_up(l), op_down(l)]
+    step_q_ops += [op_head_norm, op_head]
+    step_q_arr = ops_array(step_q_ops)
+
+    shape = {n: (t, m, k) for n, t, m, k in LAYER_SET + [HEAD] + [CONFIG1]}
+    wbytes = {n: shape[n][1] * H.row_bytes(H.TYPE_IDS[shape[n][0]], shape[n][2]) for n in shape}
+    # algorithmic bytes per launch: weights once, every input and output vector once
+    launch_bytes = {
+        "attn_qkv": wbytes["attn_qkv"] + 2 * 4096 * 4 + 6144 * 4,
+        "attn_output": wbytes["attn_output"] + 4096 + 4096 // 32 * 4 + 2 * 4096 * 4,
+        "ffn_gate_up": wbytes["ffn_gate"] + wbytes["ffn_up"] + 2 * 4096 * 4 + 14336 + 14336 // 32 * 4,
+        "ffn_down": wbytes["ffn_down"] + 14336 + 14336 // 32 * 4 + 2 * 4096 * 4,
+        "head_norm_quant": 3 * 4096 * 4 + 4096 + 4096 // 32 * 4,
+        "output": wbytes["output"] + 4096 + 4096 // 32 * 4 + 128256 * 4,
+        "config1_q4_0": algorithmic_bytes(H, *shape["config1_q4_0"]),
     }
-    step_bytes = sum(grp_bytes.values())
+    step_bytes = N_LAYERS * sum(launch_bytes[n] for n in ("attn_qkv", "attn_output", "ffn_gate_up", "ffn_down")) \
+        + launch_bytes["head_norm_quant"] + launch_bytes["output"]
     weight_bytes = sum(N_LAYERS * len(host[n]) for n, *_ in LAYER_SET) + len(host["output"])
+
+    def run(arr):
+        ctx.check(ctx.lib.cera_hip_decode_ops_dev(ctx.h, arr, len(arr)))
+
+    # per-kernel groups: 32 back-to-back launches of one kind over the rotating layer copies
+    groups = {
+        "attn_qkv": ops_array([op_qkv(l) for l in range(N_LAYERS)]),
+        "attn_output": ops_array([op_o(l) for l in range(N_LAYERS)]),
+        "ffn_gate_up": ops_array([op_gate_up(l) for l in range(N_LAYERS)]),
+        "ffn_down": ops_array([op_down(l, fused_input=False) for l in range(N_LAYERS)]),
+        "output": ops_array([op_head]),
+        "config1_q4_0": ops_array([Op(kind=Op.GEMV, w=dts["config1_q4_0"][l], xs=acts[4096][0], xq=acts[4096][1],
+                                      y=outs["config1_q4_0"]) for l in range(N_LAYERS)]),
+    }
 
     if args.pmc_probe:
         n = 1 << 30
@@ -308,75 +381,79 @@ def main() -> int:
         for _ in range(3):
             ctx.check(ctx.lib.cera_hip_copy_kernel(ctx.h, dst, src, n))
         for _ in range(2):
-            ctx.check(ctx.lib.cera_hip_gemv_seq_dev(ctx.h, grp_a, len(grp_a)))
-            ctx.check(ctx.lib.cera_hip_gemv_seq_dev(ctx.h, grp_c, len(grp_c)))
+            for g in ("ffn_gate_up", "ffn_down", "attn_qkv", "attn_output"):
+                run(groups[g])
         ctx.sync()
-        print(f"pmc probe done: copy kernel {n} B read + {n} B written per launch; fused gate+up "
-              f"{grp_bytes['q4k_gate_up'] // N_LAYERS} algorithmic B per launch", file=sys.stderr)
+        print(f"pmc probe done: copy kernel {n} B read + {n} B written per launch; algorithmic B per launch: "
+              + ", ".join(f"{g} {launch_bytes[g]}" for g in ("ffn_gate_up", "ffn_down", "attn_qkv", "attn_output")),
+              file=sys.stderr)
         return 0
 
-    def run_step(events=None):
-        for gi, (_, ops) in enumerate(groups):
-            ctx.check(ctx.lib.cera_hip_gemv_seq_dev(ctx.h, ops, len(ops)))
-            if events is not None:
-                ctx.record(events[gi + 1])
-
     for _ in range(args.warmup):
-        run_step()
+        run(step_arr)
     ctx.sync()
 
-    # ---- timed region: exactly --steps steps, bracketed by synchronisation
-    evs = [[ctx.event() for _ in range(4)] for _ in range(args.steps)]
+    # ---- timed region: exactly --steps steps, bracketed by synchronisation; an event pair per step
+    evs = [(ctx.event(), ctx.event()) for _ in range(args.steps)]
     ctx.sync()
     t_start = time.perf_counter()
     for s in range(args.steps):
         ctx.record(evs[s][0])
-        run_step(evs[s])
+        run(step_arr)
+        ctx.record(evs[s][1])
     ctx.sync()
     wall = time.perf_counter() - t_start
-    grp_ms = {g: 0.0 for g, _ in groups}
-    for s in range(args.steps):
-        for gi, (g, _) in enumerate(groups):
-            grp_ms[g] += ctx.elapsed_ms(evs[s][gi], evs[s][gi + 1])
+    step_ms = sorted(ctx.elapsed_ms(a, b) for a, b in evs)
     ms_per_step = wall * 1e3 / args.steps
     value = step_bytes / (wall / args.steps) / 1e9
+    p50 = step_ms[len(step_ms) // 2]
+    p10, p90 = step_ms[len(step_ms) // 10], step_ms[min(len(step_ms) - 1, len(step_ms) * 9 // 10)]
 
-    # dominant kernel: the fused Q4_K gate+up GEMV, 2 x (14336 x 4096) per launch, 32 launches per step
-    n_launch = len(grp_a) * args.steps
-    avg_launch_ms = grp_ms["q4k_gate_up"] / n_launch
-    pair_bytes = bytes_of["ffn_gate"] + bytes_of["ffn_up"] - 4096 - 512 - 14336 * 4   # x and y counted once
-    ach = pair_bytes / (avg_launch_ms * 1e-3) / 1e9
-    roofline = {"bound": "hbm", "kernel": "gemv_kernel<Q4K,1,2,4,2,false> (Q4_K gate+up, 2 x 14336x4096)",
-                "achieved": round(ach, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": GATE_UP_TRAFFIC_BYTES,
-                "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE passes over bench.py --pmc-probe, "
-                                  "calibrated on a 1 GiB copy kernel (recorded, see profiles/)",
-                "bytes_per_launch": pair_bytes, "avg_launch_us": round(avg_launch_ms * 1e3, 2)}
-    per_group = {g: {"GB/s": round(grp_bytes[g] / (grp_ms[g] / args.steps * 1e-3) / 1e9, 1),
-                     "ms_per_step": round(grp_ms[g] / args.steps, 4)} for g, _ in groups}
+    # ---- the set with every per-call Q8_0 quantization of the reference inside (cpu.rs:787-790)
+    q_steps = max(10, args.steps // 2)
+    for _ in range(2):
+        run(step_q_arr)
+    ctx.sync()
+    t_q = time.perf_counter()
+    for _ in range(q_steps):
+        run(step_q_arr)
+    ctx.sync()
+    ms_q = (time.perf_counter() - t_q) * 1e3 / q_steps
+    bytes_q = step_bytes + N_LAYERS * (4096 * 4 + 4096 + 4096 // 32 * 4)
 
-    # ---- the Q8_0 activation quantizer on its own (the reference re-quantizes per GEMV call,
-    # cpu.rs:787-790): kernel time per call, and the set's rate with one quantize per GEMV folded in
-    quant_us = {}
-    for kk in (4096, 14336):
-        dxf = ctx.to_device(acts[kk][2])
-        qcall = lambda: ctx.check(ctx.lib.cera_hip_quantize_q8_0_dev(ctx.h, dxf, kk, acts[kk][0], acts[kk][1]))
-        for _ in range(5):
-            qcall()
+    # ---- per matrix: HIP events around 32 back-to-back launches of one kernel, rotating copies
+    per_matrix = {}
+    reps = 8
+    for g, arr in groups.items():
+        for _ in range(2):
+            run(arr)
         e0, e1 = ctx.event(), ctx.event()
+        n_rep = reps * (8 if len(arr) == 1 else 1)
         ctx.record(e0)
-        for _ in range(200):
-            qcall()
+        for _ in range(n_rep):
+            run(arr)
         ctx.record(e1)
         ctx.sync()
-        quant_us[kk] = ctx.elapsed_ms(e0, e1) * 1e3 / 200
-        ctx.free(dxf)
-    quant_ms_per_step = (N_LAYERS * (4 * quant_us[4096] + quant_us[14336]) + quant_us[4096]) * 1e-3
-    quantize = {"k4096_us_per_call": round(quant_us[4096], 2), "k14336_us_per_call": round(quant_us[14336], 2),
-                "calls_per_step": N_LAYERS * 5 + 1,
-                "set_incl_quantize_GB/s": round(step_bytes / ((ms_per_step + quant_ms_per_step) * 1e-3) / 1e9, 1),
-                "note": "back-to-back launches of the standalone kernel; the decode path fuses three of the "
-                        "five per-layer quantizations into the producing kernels"}
+        us = ctx.elapsed_ms(e0, e1) * 1e3 / (n_rep * len(arr))
+        tname, m, k = shape["ffn_gate" if g == "ffn_gate_up" else g]
+        per_matrix[g] = {"weights": ("2 x " if g == "ffn_gate_up" else "") + f"{tname} {m}x{k}", "us_per_launch": round(us, 2),
+                         "bytes_per_launch": launch_bytes[g], "GB/s": round(launch_bytes[g] / us / 1e3, 1),
+                         "frac_of_hbm_peak": round(launch_bytes[g] / us / 1e3 / HBM_PEAK_GBS, 4),
+                         "cache_resident": len(arr) == 1 and False}
+    per_matrix["output"]["note"] = "one 431 MB matrix launched back to back: larger than the 256 MB last-level cache"
+    for g in per_matrix:
+        per_matrix[g].pop("cache_resident")
+
+    # dominant kernel: the fused Q4_K gate|up launch, 2 x (14336 x 4096) per launch, 32 launches per step
+    gu = per_matrix["ffn_gate_up"]
+    roofline = {"bound": "hbm", "kernel": GATE_UP_KERNEL + " (rmsnorm + Q8_0 in, Q4_K gate | up 2 x 14336x4096, SwiGLU + Q8_0 out)",
+                "achieved": gu["GB/s"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(gu["GB/s"] / HBM_PEAK_GBS, 4), "traffic": GATE_UP_TRAFFIC_BYTES,
+                "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE passes over bench.py --pmc-probe, "
+                                  "calibrated on a 1 GiB copy kernel (recorded, see profiles/)",
+                "bytes_per_launch": launch_bytes["ffn_gate_up"], "avg_launch_us": gu["us_per_launch"],
+                "avg_launch_source": f"HIP events on the launch stream around {reps} x 32 back-to-back launches over "
+                                     f"{n_copies} rotating layer copies, taken right after the timed region"}
 
     # ---- correctness spot check of what was just timed (oracle is only the checker)
     cpu_baseline = None
@@ -385,34 +462,46 @@ def main() -> int:
         name = "attn_output"
         tname, m, k = shape[name]
         y = ctx.download(outs[name], (m,), np.float32)
-        ref = orc.gemv(H.TYPE_IDS[tname], host[name], acts[k][2], m, k)
+        ref = x_host[4096] + orc.gemv(H.TYPE_IDS[tname], host[name], x_host[k], m, k)
         rel = float(np.abs(y - ref).max() / np.sqrt(np.mean(ref.astype(np.float64) ** 2)))
         assert rel <= 1e-3, f"GPU result of the timed GEMV deviates from the oracle: {rel}"
+        fq = ctx.download(d_ffn_q, (14336,), np.int8)
+        normed = orc.rmsnorm(x_host[4096], norm_host, eps)
+        act = orc.silu_mul(orc.gemv(H.TYPE_IDS["Q4_K"], host["ffn_gate"], normed, 14336, 4096),
+                           orc.gemv(H.TYPE_IDS["Q4_K"], host["ffn_up"], normed, 14336, 4096))
+        _, want_q = orc.quantize_q8_0(act)
+        off = np.abs(fq.astype(np.int32) - want_q.astype(np.int32))
+        assert off.max() <= 1 and np.count_nonzero(off) <= 14336 // 50, "fused gate|up output deviates from the oracle"
         # CPU baseline: the restated cera AVX2 int8 path on a bounded sample --
         # whole layers' GEMV sets (QKV, O, gate, up, down), rotating over distinct
         # weight copies so the host LLC does not hold them.
-        pool = orc.Pool(n_thr)
-        n_copies = 8
+        info = host_cpu_info()
+        policy = reference_decode_threads(info["physical_cores"], info["logical_cores"])
+        cpu_thr = args.cpu_threads or max(1, min(policy, 16))
+        pool = orc.Pool(cpu_thr)
+        n_cp = 8
         layer_sets = []
-        for c in range(n_copies):
+        for c in range(n_cp):
             layer_sets.append({n: (host[n] if c == 0 else host[n].copy()) for n, *_ in LAYER_SET})
         ybuf = {n: np.empty(shape[n][1], np.float32) for n, *_ in LAYER_SET}
-        layer_bytes = sum(bytes_of[n] for n, *_ in LAYER_SET)
+        layer_bytes = sum(algorithmic_bytes(H, *shape[n]) for n, *_ in LAYER_SET)
         done_layers = 0
         t_cpu = time.perf_counter()
         while time.perf_counter() - t_cpu < args.cpu_seconds or done_layers < 2:
-            ws = layer_sets[done_layers % n_copies]
+            ws = layer_sets[done_layers % n_cp]
             for n, tname, m, k in LAYER_SET:
-                pool.gemv(H.TYPE_IDS[tname], ws[n], acts[k][2], m, k, ybuf[n])
+                pool.gemv(H.TYPE_IDS[tname], ws[n], x_host[k], m, k, ybuf[n])
             done_layers += 1
         cpu_s = time.perf_counter() - t_cpu
         pool.close()
         cpu_baseline = {"value": round(done_layers * layer_bytes / cpu_s / 1e9, 2), "unit": "GB/s",
-                        "cores": n_thr, "kind": "port",
+                        "cores": cpu_thr, "kind": "port",
                         "sample": f"{done_layers} decode-layer GEMV sets (QKV, O, gate, up Q4_K; down Q6_K; "
                                   f"{layer_bytes} B each) in {cpu_s:.1f} s, restated cera AVX2 int8 path "
-                                  f"incl. per-call Q8_0 quantize, {n_copies} rotating weight copies",
-                        "avx2": bool(orc.lib().orc_have_avx2()), **host_cpu_info()}
+                                  f"incl. per-call Q8_0 quantize, {n_cp} rotating weight copies",
+                        "threads_policy": f"cera's decode sizing for a bandwidth-bound model: physical + physical/4 <= 24 "
+                                          f"= {policy} on this host, capped at the 16 cores of a one-GPU job",
+                        "avx2": bool(orc.lib().orc_have_avx2()), **info}
 
     extras = {}
     if not args.no_extras:
@@ -425,15 +514,22 @@ def main() -> int:
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "int8", "data": "synthetic",
-        "config": {"workload": "Llama-3-8B decode-layer GEMV set, batch 1: 32 x (QKV 6144x4096, O 4096x4096, "
-                               "gate+up 14336x4096 Q4_K; down 4096x14336 Q6_K) + head 128256x4096 Q6_K",
-                   "launches_per_step": sum(len(o) for _, o in groups), "weight_bytes_per_step": weight_bytes,
+        "config": {"workload": "Llama-3-8B decode-layer GEMV set, batch 1, decode order: 32 x (QKV 6144x4096 with rmsnorm+Q8_0 "
+                               "inside, O 4096x4096, gate|up 2 x 14336x4096 Q4_K with rmsnorm+Q8_0 in and SwiGLU+Q8_0 out; "
+                               "down 4096x14336 Q6_K) + rmsnorm+Q8_0 + head 128256x4096 Q6_K",
+                   "launches_per_step": len(step_ops), "weight_bytes_per_step": weight_bytes,
                    "algorithmic_bytes_per_step": step_bytes, "w_sigma": 0.02, "seed": args.seed,
-                   "distinct_weight_copies": max(1, min(N_LAYERS, args.weight_copies))},
+                   "distinct_weight_copies": n_copies},
         "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2),
+        "ms_per_step_p50": round(p50, 4), "ms_per_step_p10": round(p10, 4), "ms_per_step_p90": round(p90, 4),
+        "value_p50_GB/s": round(step_bytes / (p50 * 1e-3) / 1e9, 1),
+        "set_incl_quantize_GB/s": round(bytes_q / (ms_q * 1e-3) / 1e9, 1),
+        "set_incl_quantize": {"ms_per_step": round(ms_q, 4), "steps": q_steps, "launches_per_step": len(step_q_ops),
+                              "what": "the same step with O's input quantized by a launch of its own: all five per-layer "
+                                      "Q8_0 quantizations and the head's, which the reference performs per GEMV call, "
+                                      "are inside the timed step (the decode path gets O's from its attention kernel)"},
         "gemv_only_tok_s_equiv": round(1e3 / ms_per_step, 1),
-        "per_group": per_group,
-        "quantize": quantize,
+        "per_matrix": per_matrix,
         "roofline": roofline,
         "cpu_baseline": cpu_baseline,
         "e2e": e2e,

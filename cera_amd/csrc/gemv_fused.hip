@@ -98,17 +98,20 @@ struct NormQuant {
 template <class T, int NM>
 struct RowTile {
     typename T::Wt w[NM];
+    __device__ __forceinline__ void load_one(const RowGemvArgs& p, int mi, uint32_t unit, uint32_t row) {
+        T::load_w(w[mi], (mi == 0 ? p.w : p.w2) + static_cast<uint64_t>(row) * p.row_bytes, unit);
+    }
     __device__ __forceinline__ void load(const RowGemvArgs& p, uint32_t unit, uint32_t row) {
-        T::load_w(w[0], p.w + static_cast<uint64_t>(row) * p.row_bytes, unit);
-        if (NM == 2) T::load_w(w[NM - 1], p.w2 + static_cast<uint64_t>(row) * p.row_bytes, unit);
+#pragma unroll
+        for (int mi = 0; mi < NM; ++mi) load_one(p, mi, unit, row);
     }
 };
 
 // The work of workgroup `block` on matrix p: wavefront w owns rows (block * NW + w) * ROWS .. + ROWS.
-// ALL of a wavefront's weight loads are issued first, so the whole matrix is in flight across the
-// chip while the activations are being prepared (NORM: a memory round trip for x and the norm
-// weights, an f64 reduction, two barriers), and what is left afterwards is arithmetic on
-// registers.  Every thread of the workgroup must call this (it contains barriers when NORM or
+// The first two rows' weight loads are issued before the activations are prepared (NORM: a memory
+// round trip for x and the norm weights, an f64 reduction, two barriers), every buffer is
+// refilled as soon as its dot product is formed, and the per-row epilogue runs once per
+// wavefront with lane i finishing row i.  Every thread of the workgroup must call this (it contains barriers when NORM or
 // SILU_Q8), including wavefronts whose row range is empty.
 template <class T, int NW, int ROWS, bool NORM, int EPI>
 __device__ __forceinline__ void row_gemv_body(const RowGemvArgs& p, uint32_t block, uint32_t* s_xq, float* s_xs, double* s_part,
@@ -118,7 +121,9 @@ __device__ __forceinline__ void row_gemv_body(const RowGemvArgs& p, uint32_t blo
     const uint32_t n_units = p.k / T::ELEMS_PER_UNIT;
     const bool live = lane < n_units;
     const uint32_t unit = live ? lane : 0;
+    constexpr int DEPTH = ROWS < 2 ? ROWS : 2;
     const uint32_t r0 = (block * NW + wave) * ROWS;
+    auto row_of = [&](int i) -> uint32_t { return r0 + i; };
 
     NormQuant<NW> nq;
     if (NORM) {
@@ -127,10 +132,9 @@ __device__ __forceinline__ void row_gemv_body(const RowGemvArgs& p, uint32_t blo
     }
     // DEPTH rows in flight per wavefront: their loads are issued before the activations are
     // prepared, and each finished row's buffer is refilled with the row DEPTH further on
-    constexpr int DEPTH = ROWS < 2 ? ROWS : 2;
     RowTile<T, NM> t[DEPTH];
 #pragma unroll
-    for (int i = 0; i < DEPTH; ++i) t[i].load(p, unit, min(r0 + i, p.m - 1));   // rows past the end re-read the last row
+    for (int i = 0; i < DEPTH; ++i) t[i].load(p, unit, min(row_of(i), p.m - 1));   // rows past the end re-read the last row
     __builtin_amdgcn_sched_barrier(0);   // the loads are issued here, not wherever their first use would pull them
 
     typename T::Act act;
@@ -141,20 +145,42 @@ __device__ __forceinline__ void row_gemv_body(const RowGemvArgs& p, uint32_t blo
         T::load_act(act, p.xq, p.xs, unit, live);
     }
 
+    float tot[ROWS][NM];   // wave-uniform row totals
 #pragma unroll
     for (int i = 0; i < ROWS; ++i) {
-        const uint32_t row = r0 + i;
-        float tot[NM];
 #pragma unroll
-        for (int mi = 0; mi < NM; ++mi) tot[mi] = wave_sum(T::dot(t[i % DEPTH].w[mi], act, unit, nullptr));
-        if (i + DEPTH < ROWS) t[i % DEPTH].load(p, unit, min(r0 + i + DEPTH, p.m - 1));
-        if (lane == 0 && row < p.m) {
+        for (int mi = 0; mi < NM; ++mi) {
+            const float part = T::dot(t[i % DEPTH].w[mi], act, unit, nullptr);
+            // the buffer is free as soon as its dot is formed: refill it before the reduction
+            if (i + DEPTH < ROWS) {
+                __builtin_amdgcn_sched_barrier(0);
+                t[i % DEPTH].load_one(p, mi, unit, min(row_of(i + DEPTH), p.m - 1));
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            tot[i][mi] = wave_sum(part);
+        }
+    }
+    // epilogue once per wavefront: lane i finishes row i
+    {
+        float mine[NM];
+        uint32_t row = row_of(0);
+#pragma unroll
+        for (int mi = 0; mi < NM; ++mi) mine[mi] = tot[0][mi];
+#pragma unroll
+        for (int i = 1; i < ROWS; ++i) {
+            if (lane == i) {
+                row = row_of(i);
+#pragma unroll
+                for (int mi = 0; mi < NM; ++mi) mine[mi] = tot[i][mi];
+            }
+        }
+        if (lane < ROWS && row < p.m) {
             if (EPI == FEPI_SILU_Q8) {
                 // cera/src/backend/cpu.rs:2570-2575: g / (1 + expf(-g)) * u
-                const float g = tot[0];
-                s_out[row - block * NW * ROWS] = __fmul_rn(__fdiv_rn(g, __fadd_rn(1.0f, cera_expf(-g))), tot[NM - 1]);
+                const float g = mine[0];
+                s_out[wave * ROWS + lane] = __fmul_rn(__fdiv_rn(g, __fadd_rn(1.0f, cera_expf(-g))), mine[NM - 1]);
             } else {
-                p.y[row] = EPI == FEPI_ADD ? p.resid[row] + tot[0] : tot[0];
+                p.y[row] = EPI == FEPI_ADD ? p.resid[row] + mine[0] : mine[0];
             }
         }
     }
@@ -171,7 +197,7 @@ __device__ __forceinline__ void row_gemv_body(const RowGemvArgs& p, uint32_t blo
             const uint32_t packed = q8_quantize_quad(h, sc);
             if (q_live) {
                 reinterpret_cast<uint32_t*>(p.out_q + row0)[lane] = packed;
-                if ((lane & 7) == 0) p.out_s[(row0 >> 5) + (lane >> 3)] = sc;
+                if ((lane & 7) == 0) p.out_s[(row0 + 4 * lane) >> 5] = sc;
             }
         }
     }

@@ -757,6 +757,45 @@ extern "C" cera_hip_status cera_hip_rope(cera_hip_ctx* ctx, float* q, float* k, 
     return cera_hip_download(ctx, k, dk, static_cast<uint64_t>(n_kv_heads) * head_dim * 4);
 }
 
+// ---- one token's projection launches on device operands (benchmarks, profiling) ---------------
+extern "C" cera_hip_status cera_hip_decode_ops_dev(cera_hip_ctx* ctx, const cera_hip_decode_op* ops, uint32_t n) {
+    if (!ctx || (!ops && n)) return CERA_HIP_ERR_ARGUMENT;
+    std::lock_guard<std::recursive_mutex> lk(ctx->op_mu);
+    for (uint32_t i = 0; i < n; ++i) {
+        const cera_hip_decode_op& o = ops[i];
+        auto bad = [&](const char* what) {
+            return cera_fail(ctx, CERA_HIP_ERR_ARGUMENT, "decode_ops: op " + std::to_string(i) + ": " + what);
+        };
+        bool done = false;
+        switch (o.kind) {
+            case CERA_HIP_OP_GEMV:
+                if (!o.w || !o.xs || !o.xq || !o.y) return bad("GEMV needs w, xs, xq, y");
+                CERA_TRY(cera_launch_gemv(ctx, o.w, nullptr, o.xs, o.xq, o.y, o.resid, o.resid ? CERA_EPI_ADD : CERA_EPI_STORE));
+                break;
+            case CERA_HIP_OP_NORM_GEMV:
+                if (!o.w || !o.x || !o.norm_w || !o.y || (o.w2 && !o.y2)) return bad("NORM_GEMV needs w, x, norm_w, y (and y2 with w2)");
+                CERA_TRY(cera_launch_qkv_fused(ctx, o.w, o.w2, o.x, o.norm_w, o.eps, o.y, o.y2, &done));
+                if (!done) return cera_fail(ctx, CERA_HIP_ERR_UNSUPPORTED_DTYPE, "decode_ops: no fused norm + projection launch for this shape");
+                break;
+            case CERA_HIP_OP_NORM_GATE_UP:
+                if (!o.w || !o.w2 || !o.x || !o.norm_w || !o.out_q || !o.out_s) return bad("NORM_GATE_UP needs w, w2, x, norm_w, out_q, out_s");
+                CERA_TRY(cera_launch_ffn_gate_up_fused(ctx, o.w, o.w2, o.x, o.norm_w, o.eps, o.out_q, o.out_s, &done));
+                if (!done) return cera_fail(ctx, CERA_HIP_ERR_UNSUPPORTED_DTYPE, "decode_ops: no fused gate | up launch for this shape");
+                break;
+            case CERA_HIP_OP_NORM_QUANT:
+                if (!o.x || !o.norm_w || !o.y || !o.out_q || !o.out_s || o.n == 0 || o.n % 32) return bad("NORM_QUANT needs x, norm_w, y, out_q, out_s and n % 32 == 0");
+                CERA_TRY(launch_norm_quant(ctx, o.x, o.norm_w, o.n, 1, o.eps, o.y, o.out_s, o.out_q));
+                break;
+            case CERA_HIP_OP_QUANT:
+                if (!o.x || !o.out_q || !o.out_s || o.n == 0 || o.n % 32) return bad("QUANT needs x, out_q, out_s and n % 32 == 0");
+                CERA_TRY(cera_launch_quantize(ctx, o.x, o.n, o.out_s, o.out_q));
+                break;
+            default: return bad("unknown kind");
+        }
+    }
+    return CERA_HIP_OK;
+}
+
 // ---- kernel-level entry points for the decode step's fused kernels (host buffers) ------------
 extern "C" cera_hip_status cera_hip_rmsnorm_q8_0(cera_hip_ctx* ctx, const float* x, const float* weight, uint64_t n, float eps,
                                                  float* y, float* scales, int8_t* quants) {

@@ -24,7 +24,7 @@ SYMBOLS = [
     "cera_hip_tensor_upload", "cera_hip_tensor_clone", "cera_hip_tensor_free", "cera_hip_tensor_nbytes",
     "cera_hip_quantize_q8_0", "cera_hip_gemv", "cera_hip_gemm", "cera_hip_attn_decode", "cera_hip_attn_prefill", "cera_hip_rmsnorm",
     "cera_hip_silu_mul", "cera_hip_rope", "cera_hip_argmax", "cera_hip_dequantize_row",
-    "cera_hip_quantize_q8_0_dev", "cera_hip_gemv_q8_dev", "cera_hip_gemv_seq_dev", "cera_hip_attn_decode_dev",
+    "cera_hip_quantize_q8_0_dev", "cera_hip_gemv_q8_dev", "cera_hip_gemv_seq_dev", "cera_hip_decode_ops_dev", "cera_hip_attn_decode_dev",
     "cera_hip_gemm_dev",
     "cera_hip_model_create", "cera_hip_model_destroy", "cera_hip_forward", "cera_hip_forward_greedy",
     "cera_hip_forward_prefill", "cera_hip_forward_prefill_logits_all", "cera_hip_truncate_kv", "cera_hip_gemv_pair", "cera_hip_gemm_pair", "cera_hip_gemm_swiglu", "cera_hip_gemv_nb", "cera_hip_configure_kv", "cera_hip_kv_type", "cera_hip_attn_f16kv",
@@ -70,6 +70,14 @@ class GemvOp(C.Structure):
     _fields_ = [("w", C.c_void_p), ("w2", C.c_void_p), ("xs", C.c_void_p), ("xq", C.c_void_p), ("y", C.c_void_p)]
 
 
+class DecodeOp(C.Structure):
+    """cera_hip_decode_op (include/cera_hip.h)."""
+    GEMV, NORM_GEMV, NORM_GATE_UP, NORM_QUANT, QUANT = range(5)
+    _fields_ = [("kind", C.c_uint32), ("n", C.c_uint32), ("w", C.c_void_p), ("w2", C.c_void_p), ("x", C.c_void_p),
+                ("norm_w", C.c_void_p), ("eps", C.c_float), ("xs", C.c_void_p), ("xq", C.c_void_p), ("resid", C.c_void_p),
+                ("y", C.c_void_p), ("y2", C.c_void_p), ("out_s", C.c_void_p), ("out_q", C.c_void_p)]
+
+
 _lib = None
 
 
@@ -110,6 +118,7 @@ def load_library() -> C.CDLL:
         "cera_hip_quantize_q8_0_dev": (i32, [vp, vp, u64, vp, vp]),
         "cera_hip_gemv_q8_dev": (i32, [vp, vp, vp, vp, vp]),
         "cera_hip_gemv_seq_dev": (i32, [vp, C.POINTER(GemvOp), u32]),
+        "cera_hip_decode_ops_dev": (i32, [vp, C.POINTER(DecodeOp), u32]),
         "cera_hip_attn_decode_dev": (i32, [vp, vp, vp, vp, u32, u32, u32, u64, u64, f32, u32, vp]),
         "cera_hip_gemm_dev": (i32, [vp, vp, vp, u64, vp]),
         "cera_hip_model_create": (i32, [vp, C.POINTER(Config), C.POINTER(Tensor), C.POINTER(Tensor), vp,

@@ -329,6 +329,37 @@ typedef struct {
 /* Launches ops[0..n) back to back on the context's stream (one decode token's
  * worth of GEMVs without per-call host overhead). */
 CERA_HIP_API cera_hip_status cera_hip_gemv_seq_dev(cera_hip_ctx*, const cera_hip_gemv_op* ops, uint32_t n);
+/* One decode token's projection launches on device-resident operands, issued back to back on the
+ * context's stream exactly as cera_hip_forward issues them (benchmarks and profiling; the
+ * operations are those of LlamaModel::forward, cera/src/model/llama.rs:468-597):
+ *   CERA_HIP_OP_GEMV           y = w . (xs, xq) [+ resid]                  (O and down projections, head)
+ *   CERA_HIP_OP_NORM_GEMV      y = w . Q8_0(rmsnorm(x, norm_w)), y2 = w2 . same (w2 / y2 nullable)
+ *                              (the Q|K|V launch; refused with CERA_HIP_ERR_UNSUPPORTED_DTYPE where
+ *                              cera_hip_qkv_fused is)
+ *   CERA_HIP_OP_NORM_GATE_UP   (out_q, out_s) = Q8_0(silu(w . n) * (w2 . n)), n = Q8_0(rmsnorm(x, norm_w))
+ *   CERA_HIP_OP_NORM_QUANT     y = rmsnorm(x, norm_w), (out_q, out_s) = Q8_0(y), n elements (before the head)
+ *   CERA_HIP_OP_QUANT          (out_q, out_s) = Q8_0(x), n elements (quantize_f32_to_q8_0,
+ *                              cera/src/backend/cpu.rs:942-958)
+ * All pointers are device pointers; fields an op does not use are ignored. */
+enum { CERA_HIP_OP_GEMV = 0, CERA_HIP_OP_NORM_GEMV = 1, CERA_HIP_OP_NORM_GATE_UP = 2, CERA_HIP_OP_NORM_QUANT = 3,
+       CERA_HIP_OP_QUANT = 4 };
+typedef struct {
+    uint32_t kind;
+    uint32_t n;               /* NORM_QUANT / QUANT: element count (multiple of 32) */
+    const cera_hip_dtensor* w;
+    const cera_hip_dtensor* w2;
+    const float* x;           /* f32 input of the NORM_* and QUANT kinds */
+    const float* norm_w;
+    float eps;
+    const float* xs;          /* GEMV: Q8_0 scales f32[k/32] */
+    const int8_t* xq;         /* GEMV: Q8_0 quants i8[k] */
+    const float* resid;       /* GEMV: nullable residual f32[m] */
+    float* y;
+    float* y2;
+    float* out_s;
+    int8_t* out_q;
+} cera_hip_decode_op;
+CERA_HIP_API cera_hip_status cera_hip_decode_ops_dev(cera_hip_ctx*, const cera_hip_decode_op* ops, uint32_t n);
 CERA_HIP_API cera_hip_status cera_hip_attn_decode_dev(cera_hip_ctx*, const float* q, const float* k_headmajor,
                                                       const float* v_headmajor, uint32_t n_heads,
                                                       uint32_t n_kv_heads, uint32_t head_dim, uint64_t seq_len,
