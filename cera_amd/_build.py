@@ -19,6 +19,7 @@ HIP_LIB = LIB_DIR / "libcera_hip.so"
 HOST_LIB = LIB_DIR / "libcera_host.so"
 LLAMA_LIB = LIB_DIR / "libcera_hip_llama.so"
 CLI_BIN = LIB_DIR / "cera-hip"
+HSACO = LIB_DIR / "cera_hip_gfx950.hsaco"
 
 HIP_SRCS = sorted((PKG / "csrc").glob("*.hip"))
 HOST_SRCS = sorted((PKG / "host").glob("*.cpp"))
@@ -82,6 +83,21 @@ def build_hip(verbose: bool = False, jobs: int = 8) -> Path:
     return HIP_LIB
 
 
+def build_hsaco(verbose: bool = False) -> Path:
+    """The standalone gfx950 code object of the lower ABI (include/cera_hip_kernels.h)."""
+    LIB_DIR.mkdir(exist_ok=True)
+    flags = [f for f in HIPCC_FLAGS if f not in ("-shared", "-fPIC")]
+    cmd = [hipcc_path(), "--genco", "--no-gpu-bundle-output", *flags, f"-I{ROOT / 'include'}", f"-I{PKG / 'csrc'}",
+           str(PKG / "csrc" / "lower" / "cera_hip_gfx950.hip"), "-o", str(HSACO)]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if verbose or r.returncode:
+        print(" ".join(cmd))
+        print(r.stdout + r.stderr)
+    if r.returncode:
+        raise RuntimeError("hipcc --genco failed")
+    return HSACO
+
+
 def build_host(verbose: bool = False) -> Path:
     LIB_DIR.mkdir(exist_ok=True)
     srcs = sorted((PKG / "host").glob("*.cpp"))
@@ -124,6 +140,7 @@ def build_backend(verbose: bool = False) -> Path:
 def build_all(verbose: bool = False) -> None:
     build_host(verbose)
     build_hip(verbose)
+    build_hsaco(verbose)
     build_backend(verbose)
 
 

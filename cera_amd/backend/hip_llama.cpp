@@ -211,7 +211,7 @@ std::unique_ptr<HipLlamaModel> HipLlamaModel::from_gguf(const GgufFile& g, size_
     hc.logit_scale = c.scalars.logit;
     hc.rope_freqs = rope_freqs.empty() ? nullptr : rope_freqs.data();
 
-    if (cera_hip_ctx_create(device, &self->ctx_) != CERA_HIP_OK)
+    if (cera_hip_ctx_create(device, nullptr, &self->ctx_) != CERA_HIP_OK)
         bail(std::string("hip context: ") + cera_hip_last_error(nullptr));
     if (cera_hip_model_create(self->ctx_, &hc, &embd, untied ? &output : nullptr, output_norm.data(), layers.data(),
                               &self->model_) != CERA_HIP_OK)

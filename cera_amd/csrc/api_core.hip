@@ -7,6 +7,7 @@
 #include "gemv_launch.hip.h"
 #include "gemv_nb.hip.h"
 #include "glue.hip.h"
+#include "cera_hip_kernels.h"
 #include "host_common.h"
 #include "quantize.hip.h"
 
@@ -90,9 +91,28 @@ cera_hip_status cera_scratch(cera_hip_ctx* ctx, int slot, uint64_t nbytes, void*
     return CERA_HIP_OK;
 }
 
+hipFunction_t cera_module_fn(cera_hip_ctx* ctx, const std::string& name) {
+    if (!ctx->module) return nullptr;
+    auto it = ctx->module_fns.find(name);
+    if (it != ctx->module_fns.end()) return it->second;
+    hipFunction_t f = nullptr;
+    if (hipModuleGetFunction(&f, ctx->module, name.c_str()) != hipSuccess) {
+        f = nullptr;
+        (void)hipGetLastError();   // "not found" is an answer, not a sticky error
+    }
+    ctx->module_fns.emplace(name, f);
+    return f;
+}
+
+cera_hip_status cera_module_launch(cera_hip_ctx* ctx, hipFunction_t f, uint32_t grid, uint32_t block, void* args) {
+    void* params[] = {args};
+    HIP_TRY(ctx, hipModuleLaunchKernel(f, grid, 1, 1, block, 1, 1, 0, ctx->stream, params, nullptr));
+    return CERA_HIP_OK;
+}
+
 extern "C" {
 
-cera_hip_status cera_hip_ctx_create(int device, cera_hip_ctx** out) {
+cera_hip_status cera_hip_ctx_create(int device, const char* hsaco_path, cera_hip_ctx** out) {
     if (!out) return cera_fail(nullptr, CERA_HIP_ERR_ARGUMENT, "cera_hip_ctx_create: out is null");
     *out = nullptr;
     int n = 0;
@@ -118,6 +138,19 @@ cera_hip_status cera_hip_ctx_create(int device, cera_hip_ctx** out) {
         return cera_fail(nullptr, CERA_HIP_ERR_DEVICE, "kernels are built for gfx950 only; device is " + arch);
     }
     ctx->n_cu = static_cast<uint32_t>(prop.multiProcessorCount);
+    if (hsaco_path) {
+        if ((e = hipModuleLoad(&ctx->module, hsaco_path)) != hipSuccess) {
+            hipStreamDestroy(ctx->stream);
+            delete ctx;
+            return cera_fail(nullptr, CERA_HIP_ERR_DEVICE, std::string("hipModuleLoad(") + hsaco_path + "): " + hipGetErrorString(e));
+        }
+        if (!cera_module_fn(ctx, "cera_k_quantize_q8_0")) {
+            hipModuleUnload(ctx->module);
+            hipStreamDestroy(ctx->stream);
+            delete ctx;
+            return cera_fail(nullptr, CERA_HIP_ERR_ARGUMENT, std::string(hsaco_path) + " is not this library's code object (no cera_k_quantize_q8_0)");
+        }
+    }
     *out = ctx;
     return CERA_HIP_OK;
 }
@@ -134,6 +167,7 @@ void cera_hip_ctx_destroy(cera_hip_ctx* ctx) {
         if (ctx->pin[i]) (void)hipHostFree(ctx->pin[i]);
         if (ctx->pin_ev[i]) (void)hipEventDestroy(ctx->pin_ev[i]);
     }
+    if (ctx->module) (void)hipModuleUnload(ctx->module);
     (void)hipStreamDestroy(ctx->stream);
     delete ctx;
 }
@@ -390,6 +424,10 @@ cera_hip_status cera_launch_quantize(cera_hip_ctx* ctx, const float* x, uint64_t
     if (k == 0 || k % 32) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "quantize_q8_0: k must be a positive multiple of 32");
     uint64_t threads = k / 4;
     dim3 grid(static_cast<uint32_t>((threads + 255) / 256));
+    if (hipFunction_t f = cera_module_fn(ctx, "cera_k_quantize_q8_0")) {
+        cera_k_quantize_q8_0_args a{x, k, scales, quants, bsum};
+        return cera_module_launch(ctx, f, grid.x, 256, &a);
+    }
     hipLaunchKernelGGL(quantize_q8_0_kernel, grid, dim3(256), 0, ctx->stream, x, k, scales, quants, bsum);
     HIP_TRY(ctx, hipGetLastError());
     return CERA_HIP_OK;
@@ -434,6 +472,18 @@ cera_hip_status cera_launch_gemv(cera_hip_ctx* ctx, const cera_hip_dtensor* w, c
     if (!gemv_plan(a.m, n_units, ctx->n_cu, dbg, max_rb, &p, epi == CERA_EPI_SILU_MUL))
         return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "gemv: k=" + std::to_string(w->k) + " exceeds the 32768 supported by the register-resident kernel");
     a.rows_per_wave = p.rows_per_block;
+    // with a loaded code object, the instances it exports (one unit per lane, K split 1/2/4/8, two
+    // rows in flight, store / add epilogue) are launched from it; everything else is embedded
+    if (ctx->module && !dbg && p.U == 1 && p.KS != 7 && epi != CERA_EPI_SILU_MUL) {
+        static const char* const tn[] = {"q4_0", "q4_1", "q8_0", "q4_k", "q6_k"};
+        const int ti = w->dtype == CERA_HIP_Q4_0 ? 0 : w->dtype == CERA_HIP_Q4_1 ? 1 : w->dtype == CERA_HIP_Q8_0 ? 2 : w->dtype == CERA_HIP_Q4_K ? 3 : 4;
+        const std::string name = std::string("cera_k_gemv_") + tn[ti] + "_ks" + std::to_string(p.KS) + (epi == CERA_EPI_ADD ? "_add" : "_store");
+        if (hipFunction_t f = cera_module_fn(ctx, name)) {
+            a.rows_per_wave = (p.rows_per_block + 1) / 2 * 2;
+            const uint32_t n_blocks = (a.m + a.rows_per_wave - 1) / a.rows_per_wave;
+            return cera_module_launch(ctx, f, n_blocks, 64 * p.KS, &a);
+        }
+    }
     bool ok = false;
     switch (w->dtype) {
         case CERA_HIP_Q4_K: ok = cera_gemv_launch_q4k(a, p, epi, dbg, ctx->stream); break;

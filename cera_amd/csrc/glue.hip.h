@@ -140,10 +140,9 @@ static __global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __rest
 // keep the row in registers, so the row is read once and the whole kernel is
 // one memory round trip plus the reduction.  Same arithmetic as rmsnorm_kernel.
 template <bool QUANT>
-static __global__ __launch_bounds__(1024) void rmsnorm_row_kernel(const float* __restrict__ x, const float* __restrict__ w,
-                                                                  uint32_t n, float eps, float* __restrict__ y,
-                                                                  float* __restrict__ scales, int8_t* __restrict__ quants) {
-    __shared__ double part[16];
+__device__ __forceinline__ void rmsnorm_row_body(const float* __restrict__ x, const float* __restrict__ w, uint32_t n, float eps,
+                                                 float* __restrict__ y, float* __restrict__ scales, int8_t* __restrict__ quants,
+                                                 double* part /* LDS, 16 */) {
     float4 v[4], g[4];
     double s = 0.0;
 #pragma unroll
@@ -183,6 +182,13 @@ static __global__ __launch_bounds__(1024) void rmsnorm_row_kernel(const float* _
             }
         }
     }
+}
+template <bool QUANT>
+static __global__ __launch_bounds__(1024) void rmsnorm_row_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                                                                  uint32_t n, float eps, float* __restrict__ y,
+                                                                  float* __restrict__ scales, int8_t* __restrict__ quants) {
+    __shared__ double part[16];
+    rmsnorm_row_body<QUANT>(x, w, n, eps, y, scales, quants, part);
 }
 
 // ---------------------------------------------------------------------------

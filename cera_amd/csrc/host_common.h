@@ -4,6 +4,7 @@
 
 #include <mutex>
 #include <string>
+#include <unordered_map>
 #include <vector>
 
 #include "attn_types.h"
@@ -33,6 +34,10 @@ struct cera_hip_ctx {
     void* scratch[12] = {nullptr};
     uint64_t scratch_bytes[12] = {0};
     void* static_scratch = nullptr;   // this device's copy of the library's fixed workspace (resolved at creation)
+    // optional standalone code object (cera_hip_ctx_create with an hsaco_path): the quantizer and the
+    // GEMV instances it exports are then launched from it with hipModuleLaunchKernel
+    hipModule_t module = nullptr;
+    std::unordered_map<std::string, hipFunction_t> module_fns;   // name -> function, nullptr = not exported
     // attention split-K workspace
     float* attn_acc = nullptr;
     float* attn_ml = nullptr;
@@ -63,6 +68,10 @@ cera_hip_status cera_fail(cera_hip_ctx* ctx, cera_hip_status st, const std::stri
 // element / byte geometry of a GGML type; false when there is no kernel for it
 bool cera_type_geometry(uint32_t t, uint32_t* block_elems, uint32_t* block_bytes);
 cera_hip_status cera_scratch(cera_hip_ctx* ctx, int slot, uint64_t nbytes, void** out);
+// kernel `name` of the context's loaded code object, nullptr when there is no module or no such kernel
+hipFunction_t cera_module_fn(cera_hip_ctx* ctx, const std::string& name);
+// launch a one-struct-argument kernel of the loaded code object
+cera_hip_status cera_module_launch(cera_hip_ctx* ctx, hipFunction_t f, uint32_t grid, uint32_t block, void* args);
 
 // ---- launchers (defined next to their kernels) --------------------------------
 enum CeraEpilogue { CERA_EPI_STORE = 0, CERA_EPI_ADD = 1, CERA_EPI_SILU_MUL = 2 };

@@ -52,10 +52,8 @@ __device__ __forceinline__ float q8_block_scaled_sum(uint32_t packed, float scal
 
 // grid: ceil(k/4 / 256) blocks of 256 threads; thread t owns x[4t .. 4t+3].
 // bsum (nullable): per-block scale * sum(quants), consumed by the prefill GEMM.
-static __global__ __launch_bounds__(256) void quantize_q8_0_kernel(const float* __restrict__ x, uint64_t k,
-                                                            float* __restrict__ scales,
-                                                            int8_t* __restrict__ quants,
-                                                            float* __restrict__ bsum) {
+__device__ __forceinline__ void quantize_q8_0_body(const float* __restrict__ x, uint64_t k, float* __restrict__ scales,
+                                                   int8_t* __restrict__ quants, float* __restrict__ bsum) {
     uint64_t t = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     bool live = 4 * t < k;
     // k % 32 == 0, so a whole 8-lane group is live or dead together.
@@ -70,4 +68,10 @@ static __global__ __launch_bounds__(256) void quantize_q8_0_kernel(const float* 
             if (bsum) bsum[t >> 3] = ssum;
         }
     }
+}
+static __global__ __launch_bounds__(256) void quantize_q8_0_kernel(const float* __restrict__ x, uint64_t k,
+                                                            float* __restrict__ scales,
+                                                            int8_t* __restrict__ quants,
+                                                            float* __restrict__ bsum) {
+    quantize_q8_0_body(x, k, scales, quants, bsum);
 }

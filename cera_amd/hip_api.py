@@ -92,7 +92,7 @@ def load_library() -> C.CDLL:
     vp, u32, u64, f32, i32 = C.c_void_p, C.c_uint32, C.c_uint64, C.c_float, C.c_int
     pp = C.POINTER(C.c_void_p)
     sig = {
-        "cera_hip_ctx_create": (i32, [i32, pp]), "cera_hip_ctx_destroy": (None, [vp]),
+        "cera_hip_ctx_create": (i32, [i32, C.c_char_p, pp]), "cera_hip_ctx_destroy": (None, [vp]),
         "cera_hip_last_error": (C.c_char_p, [vp]), "cera_hip_sync": (i32, [vp]),
         "cera_hip_device_info": (i32, [vp, C.c_char_p, C.POINTER(u32), C.POINTER(u64)]),
         "cera_hip_malloc": (i32, [vp, u64, pp]), "cera_hip_free": (i32, [vp, vp]),
@@ -176,10 +176,12 @@ def make_tensor(ggml_type: int, m: int, k: int, blocks: np.ndarray) -> Tensor:
 class Context:
     """One HIP device + stream (cera_hip_ctx)."""
 
-    def __init__(self, device: int = 0):
+    def __init__(self, device: int = 0, hsaco_path: str | None = None):
+        """hsaco_path: the standalone code object (``_build.HSACO``) to launch the quantizer and the
+        GEMV instances from with hipModuleLaunchKernel; None = the kernels embedded in the library."""
         self.lib = load_library()
         h = C.c_void_p()
-        st = self.lib.cera_hip_ctx_create(device, C.byref(h))
+        st = self.lib.cera_hip_ctx_create(device, hsaco_path.encode() if hsaco_path else None, C.byref(h))
         if st != 0:
             raise HipError(st, (self.lib.cera_hip_last_error(None) or b"").decode())
         self.h = h

@@ -86,10 +86,15 @@ typedef struct {
 
 /* ---- context ------------------------------------------------------------ */
 
-/* Create a context on HIP device `device` (kernels are embedded in this
- * library as a gfx950 code object).  Stands where a GPU backend's context
- * constructor does (cera/src/model/mod.rs:672-703 builds one per load). */
-CERA_HIP_API cera_hip_status cera_hip_ctx_create(int device, cera_hip_ctx** out);
+/* Create a context on HIP device `device`.  Stands where a GPU backend's context constructor
+ * does (cera/src/model/mod.rs:672-703 builds one per load).  hsaco_path NULL: every kernel comes
+ * from the gfx950 code object embedded in this library.  hsaco_path = path of the standalone
+ * code object cera_hip_gfx950.hsaco (built beside this library; include/cera_hip_kernels.h): it
+ * is loaded with hipModuleLoad and the Q8_0 quantizer and the GEMV instances it exports are
+ * launched from it with hipModuleLaunchKernel -- the same code, results bit-identical; kernels
+ * it does not export still come from the embedded object.  A file that cannot be loaded or is
+ * not that code object fails the call. */
+CERA_HIP_API cera_hip_status cera_hip_ctx_create(int device, const char* hsaco_path, cera_hip_ctx** out);
 CERA_HIP_API void cera_hip_ctx_destroy(cera_hip_ctx*);
 /* Message of the most recent failure on `ctx` (ctx may be NULL for a failed
  * cera_hip_ctx_create: then the process-wide last message).  Valid until the

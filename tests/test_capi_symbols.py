@@ -30,7 +30,7 @@ def test_library_exports_every_declared_symbol():
 def test_no_gpu_is_a_loud_error_not_a_fallback():
     lib = hip_api.load_library()
     h = ctypes.c_void_p()
-    st = lib.cera_hip_ctx_create(0, ctypes.byref(h))
+    st = lib.cera_hip_ctx_create(0, None, ctypes.byref(h))
     if st == 0:          # running on a GPU box: nothing to check here
         lib.cera_hip_ctx_destroy(h)
         pytest.skip("a GPU is present")

@@ -1,0 +1,91 @@
+"""The lower ABI: the standalone gfx950 code object, driven with nothing but hipModuleLoad /
+hipModuleLaunchKernel (cera_amd/hsaco_api.py never touches libcera_hip.so), must reproduce the
+library's results bit for bit -- they are the same kernels -- and the library itself must give the
+same bits when told to launch from the code object (cera_hip_ctx_create with an hsaco_path)."""
+import numpy as np
+import pytest
+
+import util
+from cera_amd import _build, hip_api, hsaco_api
+
+pytestmark = pytest.mark.gpu
+
+
+def _bits(a):
+    return np.ascontiguousarray(a).view(np.uint8)
+
+
+@pytest.fixture(scope="module")
+def host():
+    h = hsaco_api.Host()
+    yield h
+    h.close()
+
+
+def test_quantizer_from_the_code_object(hip, orc, host):
+    print("hsaco: quantize_q8_0 via hipModuleLaunchKernel", flush=True)
+    for k, seed in ((32, 1), (4096, 2), (14336, 3)):
+        x = util.make_x(k, seed) * np.float32(3.0)
+        s, q, _ = host.quantize_q8_0(x)
+        rs, rq = hip.quantize_q8_0(x)
+        os_, oq = orc.quantize_q8_0(x)
+        assert np.array_equal(q, rq) and np.array_equal(_bits(s), _bits(rs))
+        assert np.array_equal(q, oq) and np.array_equal(_bits(s), _bits(os_))
+
+
+def test_rmsnorm_q8_0_from_the_code_object(hip, host):
+    x = util.make_x(4096, 5) * np.float32(2.0)
+    w = (1.0 + 0.1 * util.make_x(4096, 6)).astype(np.float32)
+    y, s, q = host.rmsnorm_q8_0(x, w, 1e-5)
+    ry, rs, rq = hip.rmsnorm_q8_0(x, w, 1e-5)
+    assert np.array_equal(_bits(y), _bits(ry)) and np.array_equal(_bits(s), _bits(rs)) and np.array_equal(q, rq)
+
+
+@pytest.mark.parametrize("dtype,m,k", [(util.Q4_K, 512, 4096), (util.Q4_K, 96, 14336), (util.Q6_K, 256, 4096),
+                                       (util.Q6_K, 64, 14336), (util.Q4_0, 128, 4096), (util.Q4_1, 64, 2048),
+                                       (util.Q8_0, 64, 4096), (util.Q4_K, 37, 256)])
+def test_gemv_from_the_code_object(hip, orc, host, dtype, m, k):
+    print(f"hsaco: gemv {util.NAMES[dtype]} {m}x{k} via hipModuleLaunchKernel", flush=True)
+    w, _ = util.make_weights(dtype, m, k, seed=m + k)
+    x = util.make_x(k, 9)
+    got = host.gemv(dtype, w, m, k, x)
+    lib = hip.gemv(dtype, w, x, m, k)
+    assert np.array_equal(_bits(got), _bits(lib)), float(np.abs(got - lib).max())
+    ref = orc.gemv(dtype, w, x, m, k)
+    assert np.abs(got - ref).max() <= 1e-3 * util.rms(ref) + 1e-12
+    r = util.make_x(m, 10)
+    got_add = host.gemv(dtype, w, m, k, x, resid=r)
+    assert np.abs(got_add - (r + ref)).max() <= 1e-3 * util.rms(ref) + 1e-6
+
+
+def test_library_launching_from_the_code_object(hip, orc):
+    """cera_hip_ctx_create(device, hsaco_path): same results as the embedded kernels, kernel level
+    and through a whole model."""
+    from cera_amd import synth
+    mod = hip_api.Context(0, hsaco_path=str(_build.HSACO))
+    try:
+        for dtype, m, k in ((util.Q4_K, 512, 4096), (util.Q6_K, 128, 14336), (util.Q4_0, 96, 4096), (util.Q8_0, 64, 1024)):
+            w, _ = util.make_weights(dtype, m, k, seed=3)
+            x = util.make_x(k, 4)
+            assert np.array_equal(_bits(mod.gemv(dtype, w, x, m, k)), _bits(hip.gemv(dtype, w, x, m, k))), (dtype, m, k)
+        cfg = dict(synth.TINY)
+        weights = synth.make_llama(cfg, seed=12, sigma=0.05)
+        ga, gb = hip_api.Model(hip, cfg, weights), hip_api.Model(mod, cfg, weights)
+        tok = 5
+        for pos in range(6):
+            la, lb = ga.forward(tok, pos), gb.forward(tok, pos)
+            assert np.array_equal(_bits(la), _bits(lb)), pos
+            tok = int(orc.argmax(la))
+        ga.close(); gb.close()
+    finally:
+        mod.close()
+
+
+def test_a_wrong_code_object_is_refused(tmp_path):
+    bad = tmp_path / "not_a_code_object.hsaco"
+    bad.write_bytes(b"\x7fELF" + bytes(200))
+    with pytest.raises(hip_api.HipError):
+        hip_api.Context(0, hsaco_path=str(bad))
+    with pytest.raises(hip_api.HipError):
+        hip_api.Context(0, hsaco_path=str(tmp_path / "missing.hsaco"))
+    hip_api.Context(0).close()   # and the runtime is still usable afterwards
