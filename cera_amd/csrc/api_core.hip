@@ -140,6 +140,7 @@ cera_hip_status cera_hip_ctx_create(int device, const char* hsaco_path, cera_hip
     ctx->n_cu = static_cast<uint32_t>(prop.multiProcessorCount);
     if (hsaco_path) {
         if ((e = hipModuleLoad(&ctx->module, hsaco_path)) != hipSuccess) {
+            (void)hipGetLastError();   // the failed load must not surface as a later call's error
             hipStreamDestroy(ctx->stream);
             delete ctx;
             return cera_fail(nullptr, CERA_HIP_ERR_DEVICE, std::string("hipModuleLoad(") + hsaco_path + "): " + hipGetErrorString(e));
