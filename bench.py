@@ -34,7 +34,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 # each scaled by what the same counter reads for this library's 1 GiB copy kernel; the two passes run
 # `bench.py --pmc-probe` under rocprofv3 --pmc, summary in profiles/gemv_q4k_gate_up_hbm_traffic_pmc.txt).
 # It is a recorded measurement of this kernel configuration, not taken live: counters need the profiler.
-GATE_UP_TRAFFIC_BYTES = 66_328_548
+GATE_UP_TRAFFIC_BYTES = 66_479_331
 GATE_UP_KERNEL = "row_gemv_kernel<Q4K,16,4,true,2>"
 
 # (name, ggml type name, m, k, copies per step)
@@ -252,8 +252,8 @@ def main() -> int:
     ap.add_argument("--no-e2e", action="store_true", help="skip the end-to-end model run (prefill 512 + greedy 256)")
     ap.add_argument("--no-extras", action="store_true", help="skip the flash-decode and prefill-GEMM side measurements")
     ap.add_argument("--pmc-probe", action="store_true",
-                    help="run only a 1 GiB copy kernel and a few launches of each per-layer GEMV kernel, for a "
-                         "hardware-counter pass under rocprofv3 --pmc; prints no JSON")
+                    help="run only a 1 GiB copy kernel, a few launches of each per-layer GEMV kernel and the two "
+                         "prefill GEMMs at 2048 tokens, for a hardware-counter pass under rocprofv3 --pmc; prints no JSON")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the hot path has no multi-GPU part); "
@@ -383,6 +383,17 @@ def main() -> int:
         for _ in range(2):
             for g in ("ffn_gate_up", "ffn_down", "attn_qkv", "attn_output"):
                 run(groups[g])
+        # the prefill GEMMs at 2048 tokens: Q4_K gate (int8 matrix core) and Q6_K down (f16 matrix core)
+        m_tok = 2048
+        for name in ("ffn_gate", "ffn_down"):
+            _, n_out, kk = shape[name]
+            dxg = ctx.to_device(rng.standard_normal((m_tok, kk), dtype=np.float32))
+            dog = ctx.malloc(n_out * m_tok * 4)
+            for _ in range(3):
+                ctx.check(ctx.lib.cera_hip_gemm_dev(ctx.h, dts[name][0], dxg, m_tok, dog))
+            ctx.sync()
+            ctx.free(dxg)
+            ctx.free(dog)
         ctx.sync()
         print(f"pmc probe done: copy kernel {n} B read + {n} B written per launch; algorithmic B per launch: "
               + ", ".join(f"{g} {launch_bytes[g]}" for g in ("ffn_gate_up", "ffn_down", "attn_qkv", "attn_output")),
