@@ -114,6 +114,28 @@ __device__ __forceinline__ float wave_sum(float v) {
     float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 48));
     return (r0 + r1) + (r2 + r3);
 }
+// The same for a double: each step moves the two halves of the value with a DPP move apiece
+// (a wave shuffle of a 64-bit value is two LDS-pipe permutes, ~10x the latency).
+template <int CTRL>
+__device__ __forceinline__ double dpp_d(double v) {
+    const uint64_t b = __builtin_bit_cast(uint64_t, v);
+    const uint32_t lo = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(static_cast<uint32_t>(b)), CTRL, 0xF, 0xF, true));
+    const uint32_t hi = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(static_cast<uint32_t>(b >> 32)), CTRL, 0xF, 0xF, true));
+    return __builtin_bit_cast(double, (static_cast<uint64_t>(hi) << 32) | lo);
+}
+__device__ __forceinline__ double readlane_d(double v, int lane) {
+    const uint64_t b = __builtin_bit_cast(uint64_t, v);
+    const uint32_t lo = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(static_cast<uint32_t>(b)), lane));
+    const uint32_t hi = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(static_cast<uint32_t>(b >> 32)), lane));
+    return __builtin_bit_cast(double, (static_cast<uint64_t>(hi) << 32) | lo);
+}
+__device__ __forceinline__ double wave_sum_f64(double v) {
+    v += dpp_d<0xB1>(v);
+    v += dpp_d<0x4E>(v);
+    v += dpp_d<0x141>(v);
+    v += dpp_d<0x140>(v);
+    return (readlane_d(v, 0) + readlane_d(v, 16)) + (readlane_d(v, 32) + readlane_d(v, 48));
+}
 // sum over each 16-lane row; every lane of a row ends up with its row's sum
 __device__ __forceinline__ float wave_row_sum(float v) {
     v += dpp_f<0xB1>(v);

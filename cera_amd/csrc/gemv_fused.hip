@@ -69,7 +69,7 @@ struct NormQuant {
             s += static_cast<double>(v[it].z) * v[it].z;
             s += static_cast<double>(v[it].w) * v[it].w;
         }
-        for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
+        s = wave_sum_f64(s);
         if ((threadIdx.x & 63) == 0) s_part[threadIdx.x >> 6] = s;
         lds_barrier();
         double tot = 0.0;

@@ -106,7 +106,7 @@ static __global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __rest
         s += static_cast<double>(v.z) * v.z;
         s += static_cast<double>(v.w) * v.w;
     }
-    for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
+    s = wave_sum_f64(s);
     if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = s;
     __syncthreads();
     double tot = (part[0] + part[1]) + (part[2] + part[3]);
@@ -157,7 +157,7 @@ __device__ __forceinline__ void rmsnorm_row_body(const float* __restrict__ x, co
             s += static_cast<double>(v[it].w) * v[it].w;
         }
     }
-    for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
+    s = wave_sum_f64(s);
     if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = s;
     __syncthreads();
     double tot = 0.0;
