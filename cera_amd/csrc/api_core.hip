@@ -601,18 +601,19 @@ struct AttnLaunch {
     float *acc, *ml;   // split-K partials: (o) and (m, l) per (query, head, part)
 };
 
+// G = heads per wavefront; a.G = heads per kv head (G or 2 G)
 template <int G, typename KV, int HD>
 static void attn_launch_decode_g(cera_hip_ctx* ctx, const AttnLaunch& a, const KV* kc, const KV* vc) {
-    const dim3 grid((a.n_parts + 3) / 4, a.n_kv_heads, a.n_queries), block(256);
+    const dim3 grid((a.n_parts + 3) / 4, a.n_kv_heads * (a.G / G), a.n_queries), block(256);
 #define ATTN_LAUNCH_S(SS)                                                                                            \
     do {                                                                                                             \
         if (a.fused_new_kv)                                                                                          \
             hipLaunchKernelGGL((attn_decode_partial_kernel<G, SS, true, KV, HD>), grid, block, 0, ctx->stream, a.q, kc,  \
-                               vc, a.seq_len, a.max_seq, a.scale, a.chunks_per_part, a.n_parts, a.q_stride,          \
+                               vc, a.seq_len, a.max_seq, a.scale, a.chunks_per_part, a.n_parts, a.q_stride, a.G,     \
                                a.acc, a.ml, a.nk);                                                                   \
         else                                                                                                         \
             hipLaunchKernelGGL((attn_decode_partial_kernel<G, SS, false, KV, HD>), grid, block, 0, ctx->stream, a.q, kc, \
-                               vc, a.seq_len, a.max_seq, a.scale, a.chunks_per_part, a.n_parts, a.q_stride,          \
+                               vc, a.seq_len, a.max_seq, a.scale, a.chunks_per_part, a.n_parts, a.q_stride, a.G,     \
                                a.acc, a.ml, a.nk);                                                                   \
     } while (0)
     switch (a.S) {
@@ -641,11 +642,22 @@ static void attn_launch_partials(cera_hip_ctx* ctx, const AttnLaunch& a, const K
 #undef ATTN_PF
         return;
     }
+    // Short contexts (one 8-key chunk per wavefront): a wavefront's time is its own instruction
+    // stream, which grows with the heads it serves, so groups of 4 and 8 heads are split over two
+    // wavefronts (the K/V rows they both read are a few KB and come from cache the second time).
+    // One head per wavefront gains nothing over two (590 tok/s either way on the 8B model, 580 unsplit).
+    const bool split_heads = a.S == 1 && a.G >= 4;
     switch (a.G) {
         case 1: attn_launch_decode_g<1, KV, HD>(ctx, a, kc, vc); break;
         case 2: attn_launch_decode_g<2, KV, HD>(ctx, a, kc, vc); break;
-        case 4: attn_launch_decode_g<4, KV, HD>(ctx, a, kc, vc); break;
-        default: attn_launch_decode_g<8, KV, HD>(ctx, a, kc, vc); break;
+        case 4:
+            if (split_heads) attn_launch_decode_g<2, KV, HD>(ctx, a, kc, vc);
+            else attn_launch_decode_g<4, KV, HD>(ctx, a, kc, vc);
+            break;
+        default:
+            if (split_heads) attn_launch_decode_g<4, KV, HD>(ctx, a, kc, vc);
+            else attn_launch_decode_g<8, KV, HD>(ctx, a, kc, vc);
+            break;
     }
 }
 

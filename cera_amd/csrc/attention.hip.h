@@ -357,6 +357,10 @@ __device__ __forceinline__ uint32_t attn_fold_column(uint32_t lane) {
     return 4 * Lay::col4(j, f0 >> 2) + (f0 & 3);
 }
 
+// G = query heads one wavefront serves (all of a kv head's group, or -- short contexts, where the
+// kernel is bound by a wavefront's own instruction stream, not by bytes -- half of it: grid.y is
+// then n_kv * 2 and the two halves of a group run as separate wavefronts, re-reading the same few
+// K/V rows from cache).  g_total = heads per kv head, the stride of the partials.
 template <int G, int S, bool NEWKV, typename KV, int HD>
 __global__ __launch_bounds__(256) void attn_decode_partial_kernel(
     const float* __restrict__ q,       // [n_heads][128]
@@ -364,28 +368,30 @@ __global__ __launch_bounds__(256) void attn_decode_partial_kernel(
     const KV* __restrict__ vc,
     uint32_t seq_len, uint32_t max_seq, float scale, uint32_t chunks_per_part, uint32_t n_parts,
     uint32_t q_stride,                 // floats between consecutive queries (prefill batches queries on grid.z)
-    float* __restrict__ part_acc,      // [n_queries][n_kv][n_parts][G][128]
-    float* __restrict__ part_ml,       // [n_queries][n_kv][n_parts][G][2]
+    uint32_t g_total,                  // query heads per kv head (a multiple of G)
+    float* __restrict__ part_acc,      // [n_queries][n_kv][n_parts][g_total][128]
+    float* __restrict__ part_ml,       // [n_queries][n_kv][n_parts][g_total][2]
     AttnNewKV nk) {
     const uint32_t lane = threadIdx.x & 63;
     const uint32_t part = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
-    const uint32_t kvh = blockIdx.y, qi = blockIdx.z;
+    const uint32_t subs = g_total / G, n_kv = gridDim.y / subs;
+    const uint32_t kvh = blockIdx.y / subs, sub = blockIdx.y % subs, qi = blockIdx.z;
     if (part >= n_parts) return;
     // causal prefill: query qi sits at position seq_len - 1 + qi and sees seq_len + qi keys
     seq_len += qi;
-    q += static_cast<uint64_t>(qi) * q_stride + kvh * G * HD;
+    q += static_cast<uint64_t>(qi) * q_stride + (kvh * g_total + sub * G) * HD;
     using Lay = AttnLay<KV, HD>;
     constexpr int NQ = Lay::NQ;
-    const uint32_t j = lane & 7, pg = lane >> 3;
     constexpr uint32_t CHUNK = 8 * S;
     const uint32_t t_begin = part * chunks_per_part * CHUNK;
     const uint32_t t_end = min(seq_len, t_begin + chunks_per_part * CHUNK);
     float out[G][NQ / 2];
     float m[G], l[G];
+    // the first sub-group's wavefront appends the token's K/V rows to the cache
     attn_decode_range<G, S, NEWKV, KV, HD>(q, kc + static_cast<uint64_t>(kvh) * max_seq * HD,
                                    vc + static_cast<uint64_t>(kvh) * max_seq * HD, kvh, max_seq, seq_len, t_begin,
-                                   t_end, CHUNK, scale, nk, true, lane, out, m, l);
-    const uint64_t base = ((static_cast<uint64_t>(qi) * gridDim.y + kvh) * n_parts + part) * G;
+                                   t_end, CHUNK, scale, nk, sub == 0, lane, out, m, l);
+    const uint64_t base = ((static_cast<uint64_t>(qi) * n_kv + kvh) * n_parts + part) * g_total + sub * G;
     const uint32_t col = attn_fold_column<Lay>(lane);
 #pragma unroll
     for (int h = 0; h < G; ++h) {
