@@ -27,7 +27,7 @@
 #include "quantize.hip.h"
 
 #define ATTN_MAX_PARTS 1024  // the merge kernel keeps one weight per part in LDS
-#define ATTN_MERGE_PF 8       // parts per lane group the merge kernel requests per round trip (x8 groups)
+#define ATTN_MERGE_PF 16      // parts per lane group the merge kernel requests per round trip (x8 groups: 128 parts, every short-context split)
 
 struct AttnPart {  // per (part, query head): running max, sum and unnormalised output
     float m, l;
