@@ -150,6 +150,31 @@ def test_model_reference_order_logits_bit_identical(hip, orc, name):
     gm.close(); om.close()
 
 
+def test_final_hidden_state_matches_the_oracle(hip, orc):
+    """cera_hip_read_hidden: the final normed hidden state of the last forward (what the LM head
+    reads).  Bit-identical to the oracle's on the reference-order route; on the default route it
+    carries the re-quantization noise of the layers below and is compared by cosine."""
+    cfg = dict(synth.TINY)
+    weights = synth.make_llama(cfg, seed=77, sigma=0.05, norm_jitter=0.1)
+    gm = hip_api.Model(hip, cfg, weights)
+    om = orc.Llama(cfg, weights)
+    fast = []
+    tok = 4
+    for pos in range(5):
+        gm.forward(tok, pos)
+        fast.append(gm.read_hidden())
+    gm.truncate_kv(0)
+    gm.set_reference_order(True)
+    for pos in range(5):
+        gm.forward(tok, pos)
+        _, ho = om.forward(tok, pos, want_hidden=True)
+        hg = gm.read_hidden()
+        assert _same_bits(hg, ho), pos
+        a, b = fast[pos].astype(np.float64), ho.astype(np.float64)
+        assert float(a @ b / np.sqrt((a @ a) * (b @ b))) > 0.9995, pos
+    gm.close(); om.close()
+
+
 def test_model_reference_order_f16_kv(hip, orc):
     cfg = dict(synth.TINY)
     weights = synth.make_llama(cfg, seed=44, sigma=0.05, norm_jitter=0.1)
