@@ -642,11 +642,11 @@ static void attn_launch_partials(cera_hip_ctx* ctx, const AttnLaunch& a, const K
 #undef ATTN_PF
         return;
     }
-    // Short contexts (one 8-key chunk per wavefront): a wavefront's time is its own instruction
-    // stream, which grows with the heads it serves, so groups of 4 and 8 heads are split over two
-    // wavefronts (the K/V rows they both read are a few KB and come from cache the second time).
-    // One head per wavefront gains nothing over two (590 tok/s either way on the 8B model, 580 unsplit).
-    const bool split_heads = a.S == 1 && a.G >= 4;
+    // A wavefront's time is largely its own instruction stream, which grows with the heads it
+    // serves, so groups of 4 and 8 heads are split over two wavefronts (the K/V rows both read come
+    // from cache the second time): 580 -> 590 tok/s on the 8B model at ~640 keys, 5-15 % per call
+    // from 1k to 16k keys.  One head per wavefront gains nothing over two.
+    const bool split_heads = a.G >= 4;
     switch (a.G) {
         case 1: attn_launch_decode_g<1, KV, HD>(ctx, a, kc, vc); break;
         case 2: attn_launch_decode_g<2, KV, HD>(ctx, a, kc, vc); break;
@@ -690,7 +690,9 @@ cera_hip_status cera_launch_attn(cera_hip_ctx* ctx, const float* q, const void* 
     } else {
         // positions per chunk: small chunks while the context is short (one memory round
         // trip per wavefront, many wavefronts), 64 once there is plenty of work
-        S = last_len >= 16384 ? 8 : (last_len >= 4096 ? 4 : (last_len >= ATTN_FUSED_NEW_KV_MAX_KEYS ? 2 : 1));
+        // (thresholds measured on the 32/8/128 shape over rotating caches: 2048 keys 12.0 -> 10.2 us,
+        // 3072 keys 14.9 -> 12.4 us, 8192 keys 18.8 -> 18.2 us against the 4096 / 16384 ones used before)
+        S = last_len >= 8192 ? 8 : (last_len >= 2048 ? 4 : (last_len >= ATTN_FUSED_NEW_KV_MAX_KEYS ? 2 : 1));
         if (G == 8 && S == 8) S = 4;   // eight heads x 64 positions per chunk does not fit the register file
         uint32_t n_chunks = static_cast<uint32_t>((last_len + 8 * S - 1) / (8 * S));
         // parts (wavefronts) per (query, kv head): enough to fill the chip ~4 waves per CU deep

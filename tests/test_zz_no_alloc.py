@@ -52,8 +52,9 @@ def test_no_alloc_attention_matches_the_allocating_entry(hip, orc):
 
 
 def test_no_alloc_attention_refuses_what_does_not_fit(hip):
-    # 32 heads x 1024 parts x 128 x 4 bytes = 16 MiB of partials: beyond the fixed 4 MiB array
-    L, n_kv, hd = 8192, 8, 128
+    # 32768 keys in 64-key chunks, one part each = 512 parts: 32 heads x 512 x 128 x 4 bytes = 8 MiB of
+    # partials, beyond the fixed 4 MiB array
+    L, n_kv, hd = 32768, 8, 128
     dq, dk = hip.to_device(np.zeros(32 * hd, np.float32)), hip.to_device(np.zeros((n_kv, L, hd), np.float32))
     d_out = hip.malloc(32 * hd * 4)
     st = hip.lib.cera_hip_attn_decode_dev_noalloc(hip.h, dq, dk, dk, 32, n_kv, hd, L, L, 0.1, 1024, d_out)
