@@ -82,6 +82,9 @@ cera_hip_status cera_launch_quantize(cera_hip_ctx* ctx, const float* x, uint64_t
 cera_hip_status cera_launch_gemv(cera_hip_ctx* ctx, const cera_hip_dtensor* w, const cera_hip_dtensor* w2,
                                  const float* xs, const int8_t* xq, float* y, const float* resid, int epi,
                                  int32_t* dbg_dots = nullptr, int32_t* dbg_asums = nullptr);
+// y = resid + W.(xs,xq) with one wavefront per row; *launched = false when the shape has no such instance
+cera_hip_status cera_launch_row_gemv_add(cera_hip_ctx* ctx, const cera_hip_dtensor* w, const float* xs, const int8_t* xq,
+                                         float* y, const float* resid, bool* launched);
 cera_hip_status cera_launch_gemv_nb(cera_hip_ctx* ctx, const cera_hip_dtensor* w, const float* xs, const int8_t* xq,
                                     uint32_t xs_stride, uint32_t xq_stride, uint32_t n_tok, float* y, uint32_t y_stride,
                                     const float* resid, bool* launched);

@@ -442,6 +442,11 @@ static cera_hip_status project(cera_hip_model* m, const cera_hip_dtensor* w, con
         HIP_TRY(ctx, hipGetLastError());
         return CERA_HIP_OK;
     }
+    if (resid) {
+        bool done = false;
+        CERA_TRY(cera_launch_row_gemv_add(ctx, w, m->xs, m->xq, y, resid, &done));
+        if (done) return CERA_HIP_OK;
+    }
     return cera_launch_gemv(ctx, w, nullptr, m->xs, m->xq, y, resid, resid ? CERA_EPI_ADD : CERA_EPI_STORE);
 }
 
