@@ -133,7 +133,7 @@ cera_hip_status cera_hip_ctx_create(int device, const char* hsaco_path, cera_hip
     }
     if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0) {
         std::string arch = prop.gcnArchName;
-        hipStreamDestroy(ctx->stream);
+        (void)hipStreamDestroy(ctx->stream);
         delete ctx;
         return cera_fail(nullptr, CERA_HIP_ERR_DEVICE, "kernels are built for gfx950 only; device is " + arch);
     }
@@ -141,13 +141,13 @@ cera_hip_status cera_hip_ctx_create(int device, const char* hsaco_path, cera_hip
     if (hsaco_path) {
         if ((e = hipModuleLoad(&ctx->module, hsaco_path)) != hipSuccess) {
             (void)hipGetLastError();   // the failed load must not surface as a later call's error
-            hipStreamDestroy(ctx->stream);
+            (void)hipStreamDestroy(ctx->stream);
             delete ctx;
             return cera_fail(nullptr, CERA_HIP_ERR_DEVICE, std::string("hipModuleLoad(") + hsaco_path + "): " + hipGetErrorString(e));
         }
         if (!cera_module_fn(ctx, "cera_k_quantize_q8_0")) {
-            hipModuleUnload(ctx->module);
-            hipStreamDestroy(ctx->stream);
+            (void)hipModuleUnload(ctx->module);
+            (void)hipStreamDestroy(ctx->stream);
             delete ctx;
             return cera_fail(nullptr, CERA_HIP_ERR_ARGUMENT, std::string(hsaco_path) + " is not this library's code object (no cera_k_quantize_q8_0)");
         }

@@ -221,6 +221,67 @@ static __global__ __launch_bounds__(64 * NW, 2) void row_gemv_pair_kernel(RowGem
     else row_gemv_body<TB, NW, ROWS, NORM, FEPI_STORE>(p.b, blockIdx.x - p.n_blocks_a, s_xq, s_xs, s_part, nullptr);
 }
 
+// Long rows (4096 < k <= 16384: the down projection): still one wavefront per row, walking the
+// row in TILES passes of 64 units with every pass's weights requested up front and the activations
+// read from LDS pass by pass (a lane cannot keep four passes' activations in registers).  There is
+// no K split across wavefronts, so no combine and no barrier after the activations are staged:
+// a wavefront's only dependencies are its own loads.  The K-split kernel's workgroup meets at a
+// barrier per row group, which costs it most when the weights come from HBM (12.3 us against
+// 9.6 us from the last-level cache).  Pass t sees exactly the units wavefront t of the K-split
+// kernel sees, and the pass totals are added in wavefront order, so the result has the same bits.
+template <class T, int NW, int TILES, int EPI>
+static __global__ __launch_bounds__(64 * NW) void row_gemv_long_kernel(RowGemvArgs p) {
+    constexpr uint32_t MAX_K = TILES * 64 * T::ELEMS_PER_UNIT;
+    __shared__ __attribute__((aligned(16))) int8_t s_xq[MAX_K];
+    __shared__ __attribute__((aligned(16))) float s_xs[MAX_K / 32];
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint32_t n_units = p.k / T::ELEMS_PER_UNIT;
+    const uint32_t row = blockIdx.x * NW + wave;
+    const uint8_t* rp = p.w + static_cast<uint64_t>(min(row, p.m - 1)) * p.row_bytes;
+    // activations first (they are waited for first: the load counter is in order), then all weights
+    constexpr int XI = (MAX_K / 16 + 64 * NW - 1) / (64 * NW);
+    uint4 xv[XI];
+#pragma unroll
+    for (int i = 0; i < XI; ++i) {
+        const uint32_t o = (tid + 64 * NW * i) * 16;
+        xv[i] = o < p.k ? *reinterpret_cast<const uint4*>(p.xq + o) : make_uint4(0, 0, 0, 0);
+    }
+    const uint32_t n_sc = p.k / 32;
+    constexpr int SI = (MAX_K / 32 + 64 * NW - 1) / (64 * NW);
+    float sv[SI];
+#pragma unroll
+    for (int i = 0; i < SI; ++i) sv[i] = tid + 64 * NW * i < n_sc ? p.xs[tid + 64 * NW * i] : 0.0f;
+    __builtin_amdgcn_sched_barrier(0);
+    typename T::Wt w[TILES];
+    bool live[TILES];
+    uint32_t unit[TILES];
+#pragma unroll
+    for (int t = 0; t < TILES; ++t) {
+        const uint32_t u = 64 * t + lane;
+        live[t] = u < n_units;
+        unit[t] = live[t] ? u : 0;   // dead lanes re-read unit 0 with zeroed activations
+        T::load_w(w[t], rp, unit[t]);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < XI; ++i) {
+        const uint32_t o = (tid + 64 * NW * i) * 16;
+        if (o < MAX_K) *reinterpret_cast<uint4*>(s_xq + o) = xv[i];
+    }
+#pragma unroll
+    for (int i = 0; i < SI; ++i)
+        if (tid + 64 * NW * i < MAX_K / 32) s_xs[tid + 64 * NW * i] = sv[i];
+    lds_barrier();
+    float s = 0.0f;
+#pragma unroll
+    for (int t = 0; t < TILES; ++t) {
+        typename T::Act act;
+        T::load_act(act, s_xq, s_xs, unit[t], live[t]);
+        s += wave_sum(T::dot(w[t], act, unit[t], nullptr));
+    }
+    if (lane == 0 && row < p.m) p.y[row] = EPI == FEPI_ADD ? p.resid[row] + s : s;
+}
+
 // ---------------------------------------------------------------------------
 static constexpr int FUSED_NW = 8;
 
@@ -316,6 +377,34 @@ cera_hip_status cera_launch_row_gemv_add(cera_hip_ctx* ctx, const cera_hip_dtens
     const dim3 grid((a.m + NW * ROWS - 1) / (NW * ROWS)), block(64 * NW);
     if (w->dtype == CERA_HIP_Q4_K) hipLaunchKernelGGL((row_gemv_kernel<Q4K, NW, ROWS, false, FEPI_ADD>), grid, block, 0, ctx->stream, a);
     else hipLaunchKernelGGL((row_gemv_kernel<Q6K, NW, ROWS, false, FEPI_ADD>), grid, block, 0, ctx->stream, a);
+    HIP_TRY(ctx, hipGetLastError());
+    *launched = true;
+    return CERA_HIP_OK;
+}
+
+// y = resid + W . (xs, xq) for long rows (see row_gemv_long_kernel); *launched = false when the
+// shape has no instance.
+cera_hip_status cera_launch_row_gemv_long_add(cera_hip_ctx* ctx, const cera_hip_dtensor* w, const float* xs, const int8_t* xq,
+                                              float* y, const float* resid, bool* launched) {
+    *launched = false;
+    if (!fused_type(w->dtype) || w->k % 256 || w->k <= 4096 || w->k > 16384 || !resid || w->m > (1u << 20)) return CERA_HIP_OK;
+    // four rows per workgroup: small workgroups start and retire independently, which measured
+    // faster end to end than 8 or 16 rows sharing one staged copy of the activations
+    constexpr int NW = 4;
+    RowGemvArgs a;
+    fill(a, w, nullptr, 1);
+    a.xq = xq; a.xs = xs; a.y = y; a.resid = resid;
+    const uint32_t tiles = static_cast<uint32_t>((w->k / 64 + 63) / 64);   // both types: 64 weights per unit
+    const dim3 grid((a.m + NW - 1) / NW), block(64 * NW);
+#define LONG_LAUNCH(TT)                                                                                                  \
+    do {                                                                                                                 \
+        if (tiles == 2) hipLaunchKernelGGL((row_gemv_long_kernel<TT, NW, 2, FEPI_ADD>), grid, block, 0, ctx->stream, a);  \
+        else if (tiles == 3) hipLaunchKernelGGL((row_gemv_long_kernel<TT, NW, 3, FEPI_ADD>), grid, block, 0, ctx->stream, a); \
+        else hipLaunchKernelGGL((row_gemv_long_kernel<TT, NW, 4, FEPI_ADD>), grid, block, 0, ctx->stream, a);             \
+    } while (0)
+    if (w->dtype == CERA_HIP_Q4_K) LONG_LAUNCH(Q4K);
+    else LONG_LAUNCH(Q6K);
+#undef LONG_LAUNCH
     HIP_TRY(ctx, hipGetLastError());
     *launched = true;
     return CERA_HIP_OK;

@@ -85,6 +85,8 @@ cera_hip_status cera_launch_gemv(cera_hip_ctx* ctx, const cera_hip_dtensor* w, c
 // y = resid + W.(xs,xq) with one wavefront per row; *launched = false when the shape has no such instance
 cera_hip_status cera_launch_row_gemv_add(cera_hip_ctx* ctx, const cera_hip_dtensor* w, const float* xs, const int8_t* xq,
                                          float* y, const float* resid, bool* launched);
+cera_hip_status cera_launch_row_gemv_long_add(cera_hip_ctx* ctx, const cera_hip_dtensor* w, const float* xs, const int8_t* xq,
+                                              float* y, const float* resid, bool* launched);
 cera_hip_status cera_launch_gemv_nb(cera_hip_ctx* ctx, const cera_hip_dtensor* w, const float* xs, const int8_t* xq,
                                     uint32_t xs_stride, uint32_t xq_stride, uint32_t n_tok, float* y, uint32_t y_stride,
                                     const float* resid, bool* launched);

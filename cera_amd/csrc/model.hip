@@ -421,6 +421,17 @@ extern "C" uint32_t cera_hip_kv_type(const cera_hip_model* m) { return m && m->k
 
 // ---------------------------------------------------------------------------
 // One projection: int8 kernels read the quantized activations, Q5_K the f32 ones.
+// y = resid + W . (xs, xq): one wavefront per row where a row fits one (the O projection) or a few
+// passes of one (the down projection), the K-split kernel otherwise.  All three give the same bits.
+static cera_hip_status launch_proj_add(cera_hip_ctx* ctx, const cera_hip_dtensor* w, const float* xs, const int8_t* xq, float* y,
+                                       const float* resid) {
+    bool done = false;
+    CERA_TRY(cera_launch_row_gemv_add(ctx, w, xs, xq, y, resid, &done));
+    if (!done) CERA_TRY(cera_launch_row_gemv_long_add(ctx, w, xs, xq, y, resid, &done));
+    if (done) return CERA_HIP_OK;
+    return cera_launch_gemv(ctx, w, nullptr, xs, xq, y, resid, CERA_EPI_ADD);
+}
+
 static cera_hip_status project(cera_hip_model* m, const cera_hip_dtensor* w, const float* x_f32, float* y,
                                const float* resid) {
     cera_hip_ctx* ctx = m->ctx;
@@ -442,12 +453,8 @@ static cera_hip_status project(cera_hip_model* m, const cera_hip_dtensor* w, con
         HIP_TRY(ctx, hipGetLastError());
         return CERA_HIP_OK;
     }
-    if (resid) {
-        bool done = false;
-        CERA_TRY(cera_launch_row_gemv_add(ctx, w, m->xs, m->xq, y, resid, &done));
-        if (done) return CERA_HIP_OK;
-    }
-    return cera_launch_gemv(ctx, w, nullptr, m->xs, m->xq, y, resid, resid ? CERA_EPI_ADD : CERA_EPI_STORE);
+    if (resid) return launch_proj_add(ctx, w, m->xs, m->xq, y, resid);
+    return cera_launch_gemv(ctx, w, nullptr, m->xs, m->xq, y, nullptr, CERA_EPI_STORE);
 }
 
 // rmsnorm of `rows` rows of n elements with the Q8_0 quantization of the result fused in
@@ -775,7 +782,8 @@ extern "C" cera_hip_status cera_hip_decode_ops_dev(cera_hip_ctx* ctx, const cera
         switch (o.kind) {
             case CERA_HIP_OP_GEMV:
                 if (!o.w || !o.xs || !o.xq || !o.y) return bad("GEMV needs w, xs, xq, y");
-                CERA_TRY(cera_launch_gemv(ctx, o.w, nullptr, o.xs, o.xq, o.y, o.resid, o.resid ? CERA_EPI_ADD : CERA_EPI_STORE));
+                if (o.resid) CERA_TRY(launch_proj_add(ctx, o.w, o.xs, o.xq, o.y, o.resid));
+                else CERA_TRY(cera_launch_gemv(ctx, o.w, nullptr, o.xs, o.xq, o.y, nullptr, CERA_EPI_STORE));
                 break;
             case CERA_HIP_OP_NORM_GEMV:
                 if (!o.w || !o.x || !o.norm_w || !o.y || (o.w2 && !o.y2)) return bad("NORM_GEMV needs w, x, norm_w, y (and y2 with w2)");

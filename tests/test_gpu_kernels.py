@@ -584,3 +584,19 @@ def test_ffn_gate_up_fused_is_bitwise_the_separate_launches(hip, orc):
     h = hip.silu_mul(hip.gemv(Q4_K, wg, n, m, k), hip.gemv(Q4_K, wu, n, m, k))
     rs, rq = hip.quantize_q8_0(h)
     assert np.array_equal(q, rq) and np.array_equal(sc.view(np.uint32), rs.view(np.uint32))
+
+
+@pytest.mark.parametrize("dtype,m,k", [(Q6_K, 4096, 14336), (Q4_K, 512, 14336), (Q6_K, 77, 8192), (Q4_K, 100, 11008 // 256 * 256),
+                                       (Q4_K, 4096, 4096), (Q6_K, 130, 4096), (Q4_K, 33, 256), (Q4_0, 64, 4096)])
+def test_projection_with_residual_is_bitwise_the_plain_gemv(hip, dtype, m, k):
+    """The decode step's residual projections (O, down) run one wavefront per row where the row
+    length allows; whichever kernel a shape takes, y = resid + W.x carries the bits of the plain
+    GEMV's W.x added to resid."""
+    print(f"projection + residual {util.NAMES[dtype]} {m}x{k}", flush=True)
+    w, _ = util.make_weights(dtype, m, k, seed=m + k + 1)
+    x = util.make_x(k, 3)
+    r = util.make_x(m, 4)
+    plain = hip.gemv(dtype, w, x, m, k)
+    got = hip.gemv_add_dev(dtype, w, x, r, m, k)
+    want = (r + plain).astype(np.float32)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), float(np.abs(got - want).max())
