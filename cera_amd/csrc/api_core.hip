@@ -645,8 +645,10 @@ static void attn_launch_partials(cera_hip_ctx* ctx, const AttnLaunch& a, const K
     // A wavefront's time is largely its own instruction stream, which grows with the heads it
     // serves, so groups of 4 and 8 heads are split over two wavefronts (the K/V rows both read come
     // from cache the second time): 580 -> 590 tok/s on the 8B model at ~640 keys, 5-15 % per call
-    // from 1k to 16k keys.  One head per wavefront gains nothing over two.
-    const bool split_heads = a.G >= 4;
+    // from 1k to 16k keys.  One head per wavefront gains nothing over two.  From 32k keys on the
+    // kernel is bound by bytes and the second reader costs more than it saves (131072 keys:
+    // 5.85 TB/s unsplit against 5.50 split), so long contexts keep one wavefront per group.
+    const bool split_heads = a.G >= 4 && a.seq_len < 32768;
     switch (a.G) {
         case 1: attn_launch_decode_g<1, KV, HD>(ctx, a, kc, vc); break;
         case 2: attn_launch_decode_g<2, KV, HD>(ctx, a, kc, vc); break;
