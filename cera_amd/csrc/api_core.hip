@@ -605,23 +605,35 @@ struct AttnLaunch {
 template <int G, typename KV, int HD>
 static void attn_launch_decode_g(cera_hip_ctx* ctx, const AttnLaunch& a, const KV* kc, const KV* vc) {
     const dim3 grid((a.n_parts + 3) / 4, a.n_kv_heads * (a.G / G), a.n_queries), block(256);
-#define ATTN_LAUNCH_S(SS)                                                                                            \
+    // one query and one wavefront per kv head and key range: every K/V row is read exactly once,
+    // which is what the non-temporal instances want (long chunks only: short ones prefetch V
+    // with K and are latency-bound)
+    const bool nt = a.G == G && a.n_queries == 1 && a.S >= 4;
+#define ATTN_LAUNCH_SN(SS, NT)                                                                                       \
     do {                                                                                                             \
         if (a.fused_new_kv)                                                                                          \
-            hipLaunchKernelGGL((attn_decode_partial_kernel<G, SS, true, KV, HD>), grid, block, 0, ctx->stream, a.q, kc,  \
-                               vc, a.seq_len, a.max_seq, a.scale, a.chunks_per_part, a.n_parts, a.q_stride, a.G,     \
+            hipLaunchKernelGGL((attn_decode_partial_kernel<G, SS, true, KV, HD, NT>), grid, block, 0, ctx->stream, a.q,  \
+                               kc, vc, a.seq_len, a.max_seq, a.scale, a.chunks_per_part, a.n_parts, a.q_stride, a.G, \
                                a.acc, a.ml, a.nk);                                                                   \
         else                                                                                                         \
-            hipLaunchKernelGGL((attn_decode_partial_kernel<G, SS, false, KV, HD>), grid, block, 0, ctx->stream, a.q, kc, \
-                               vc, a.seq_len, a.max_seq, a.scale, a.chunks_per_part, a.n_parts, a.q_stride, a.G,     \
+            hipLaunchKernelGGL((attn_decode_partial_kernel<G, SS, false, KV, HD, NT>), grid, block, 0, ctx->stream, a.q, \
+                               kc, vc, a.seq_len, a.max_seq, a.scale, a.chunks_per_part, a.n_parts, a.q_stride, a.G, \
                                a.acc, a.ml, a.nk);                                                                   \
     } while (0)
+#define ATTN_LAUNCH_S(SS) ATTN_LAUNCH_SN(SS, false)
     switch (a.S) {
         case 1: ATTN_LAUNCH_S(1); break;
         case 2: ATTN_LAUNCH_S(2); break;
-        case 4: ATTN_LAUNCH_S(4); break;
-        default: ATTN_LAUNCH_S(8); break;
+        case 4:
+            if (nt) ATTN_LAUNCH_SN(4, true);
+            else ATTN_LAUNCH_S(4);
+            break;
+        default:
+            if (nt) ATTN_LAUNCH_SN(8, true);
+            else ATTN_LAUNCH_S(8);
+            break;
     }
+#undef ATTN_LAUNCH_SN
 #undef ATTN_LAUNCH_S
 }
 
@@ -645,10 +657,11 @@ static void attn_launch_partials(cera_hip_ctx* ctx, const AttnLaunch& a, const K
     // A wavefront's time is largely its own instruction stream, which grows with the heads it
     // serves, so groups of 4 and 8 heads are split over two wavefronts (the K/V rows both read come
     // from cache the second time): 580 -> 590 tok/s on the 8B model at ~640 keys, 5-15 % per call
-    // from 1k to 16k keys.  One head per wavefront gains nothing over two.  From 32k keys on the
-    // kernel is bound by bytes and the second reader costs more than it saves (131072 keys:
-    // 5.85 TB/s unsplit against 5.50 split), so long contexts keep one wavefront per group.
-    const bool split_heads = a.G >= 4 && a.seq_len < 32768;
+    // from 1k to 16k keys.  One head per wavefront gains nothing over two.  From 16k keys on the
+    // kernel is bound by bytes: a group keeps one wavefront, every K/V row is then read exactly
+    // once and the loads carry the non-temporal hint (131072 keys: 5.50 TB/s split, 5.85 unsplit,
+    // 6.42 unsplit and non-temporal; 16384 keys: the same time either way).
+    const bool split_heads = a.G >= 4 && a.seq_len < 16384;
     switch (a.G) {
         case 1: attn_launch_decode_g<1, KV, HD>(ctx, a, kc, vc); break;
         case 2: attn_launch_decode_g<2, KV, HD>(ctx, a, kc, vc); break;

@@ -41,18 +41,20 @@ struct AttnPart {  // per (part, query head): running max, sum and unnormalised 
 template <typename KV, int HD> struct AttnLay {   // f32 rows, and half rows of 64
     static constexpr int NQ = HD / 32;
     __device__ static __forceinline__ uint32_t col4(uint32_t j, int c) { return j + 8 * c; }
+    template <bool NT = false>
     __device__ static __forceinline__ void ld(const KV* row, uint32_t j, float4 (&v)[NQ]) {
 #pragma unroll
-        for (int c = 0; c < NQ; ++c) v[c] = KvOps<KV>::ld4(row, j + 8 * c);
+        for (int c = 0; c < NQ; ++c) v[c] = NT ? KvOps<KV>::ld4nt(row, j + 8 * c) : KvOps<KV>::ld4(row, j + 8 * c);
     }
 };
 template <> struct AttnLay<kv_half, 128> {         // two 16-byte loads per row: quads 2c', 2c'+1 together
     static constexpr int NQ = 4;
     __device__ static __forceinline__ uint32_t col4(uint32_t j, int c) { return 2 * (j + 8 * (c >> 1)) + (c & 1); }
+    template <bool NT = false>
     __device__ static __forceinline__ void ld(const kv_half* row, uint32_t j, float4 (&v)[4]) {
 #pragma unroll
         for (int cc = 0; cc < 2; ++cc) {
-            const uint4 r = reinterpret_cast<const uint4*>(row)[j + 8 * cc];
+            const uint4 r = NT ? ld_u128_nt(reinterpret_cast<const uint4*>(row) + j + 8 * cc) : reinterpret_cast<const uint4*>(row)[j + 8 * cc];
             v[2 * cc] = KvOps<kv_half>::cvt4(r.x, r.y);
             v[2 * cc + 1] = KvOps<kv_half>::cvt4(r.z, r.w);
         }
@@ -137,7 +139,7 @@ __device__ __forceinline__ void attn_new_row_finish(float4 (&r)[HD / 32], const 
 // the eight position groups folded: the wavefront-wide m and l in every lane, and of the
 // unnormalised output each lane's head_dim / 64 consecutive columns from attn_fold_column.  `q` points at the first of the G heads; `write_new` says whether
 // this caller stores the new position's K/V row into the cache (NEWKV only).
-template <int G, int S, bool NEWKV, typename KV, int HD>
+template <int G, int S, bool NEWKV, typename KV, int HD, bool NT>
 __device__ __forceinline__ void attn_decode_range(const float* __restrict__ q, const KV* __restrict__ kbase,
                                                   const KV* __restrict__ vbase, uint32_t kvh, uint32_t max_seq,
                                                   uint32_t seq_len, uint32_t t_begin, uint32_t t_end, uint32_t t_step,
@@ -208,7 +210,7 @@ __device__ __forceinline__ void attn_decode_range(const float* __restrict__ q, c
 #pragma unroll
                 for (int c = 0; c < NQ; ++c) kv[c] = kbuf[s][c];
             } else {
-                Lay::ld(kbase + static_cast<uint64_t>(live ? t : t_begin) * HD, j, kv);
+                Lay::template ld<NT>(kbase + static_cast<uint64_t>(live ? t : t_begin) * HD, j, kv);
             }
 #pragma unroll
             for (int h = 0; h < G; ++h) {
@@ -259,7 +261,7 @@ __device__ __forceinline__ void attn_decode_range(const float* __restrict__ q, c
                 for (int c = 0; c < NQ; ++c) vv[c] = vpre[s][c];
             } else {
                 const uint32_t t = t0 + 8 * s + pg;
-                Lay::ld(vbase + static_cast<uint64_t>(t < t_end ? t : t_begin) * HD, j, vv);
+                Lay::template ld<NT>(vbase + static_cast<uint64_t>(t < t_end ? t : t_begin) * HD, j, vv);
             }
 #pragma unroll
             for (int h = 0; h < G; ++h) {
@@ -361,7 +363,9 @@ __device__ __forceinline__ uint32_t attn_fold_column(uint32_t lane) {
 // kernel is bound by a wavefront's own instruction stream, not by bytes -- half of it: grid.y is
 // then n_kv * 2 and the two halves of a group run as separate wavefronts, re-reading the same few
 // K/V rows from cache).  g_total = heads per kv head, the stride of the partials.
-template <int G, int S, bool NEWKV, typename KV, int HD>
+// NT: every K/V row is read once, by this wavefront only (one query, the group not split):
+// non-temporal loads.
+template <int G, int S, bool NEWKV, typename KV, int HD, bool NT = false>
 __global__ __launch_bounds__(256) void attn_decode_partial_kernel(
     const float* __restrict__ q,       // [n_heads][128]
     const KV* __restrict__ kc,         // [n_kv][max_seq][128]
@@ -388,7 +392,7 @@ __global__ __launch_bounds__(256) void attn_decode_partial_kernel(
     float out[G][NQ / 2];
     float m[G], l[G];
     // the first sub-group's wavefront appends the token's K/V rows to the cache
-    attn_decode_range<G, S, NEWKV, KV, HD>(q, kc + static_cast<uint64_t>(kvh) * max_seq * HD,
+    attn_decode_range<G, S, NEWKV, KV, HD, NT>(q, kc + static_cast<uint64_t>(kvh) * max_seq * HD,
                                    vc + static_cast<uint64_t>(kvh) * max_seq * HD, kvh, max_seq, seq_len, t_begin,
                                    t_end, CHUNK, scale, nk, sub == 0, lane, out, m, l);
     const uint64_t base = ((static_cast<uint64_t>(qi) * n_kv + kvh) * n_parts + part) * g_total + sub * G;
