@@ -104,15 +104,6 @@ __device__ __forceinline__ void lds_barrier() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
 
-// Orders one wavefront's own LDS traffic for the compiler (lane a's store, then lane b's load of
-// the same bytes): the hardware executes a wavefront's LDS instructions in order, so this costs
-// a wait for the LDS counter and no barrier.
-__device__ __forceinline__ void wave_lds_sync() {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");
-}
-
 // 4 x int8 dot with int32 accumulate (v_dot4_i32_i8).
 __device__ __forceinline__ int dot4(uint32_t a, uint32_t b, int c) {
     return __builtin_amdgcn_sdot4(static_cast<int>(a), static_cast<int>(b), c, false);
