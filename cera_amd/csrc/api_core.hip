@@ -187,6 +187,13 @@ cera_hip_status cera_hip_sync(cera_hip_ctx* ctx) {
     return CERA_HIP_OK;
 }
 
+cera_hip_status cera_hip_ctx_set_decode_copies(cera_hip_ctx* ctx, int enabled) {
+    if (!ctx) return CERA_HIP_ERR_ARGUMENT;
+    std::lock_guard<std::recursive_mutex> lk(ctx->op_mu);
+    ctx->decode_copies = enabled != 0;
+    return CERA_HIP_OK;
+}
+
 cera_hip_status cera_hip_device_info(cera_hip_ctx* ctx, char* name256, uint32_t* n_cu, uint64_t* hbm) {
     if (!ctx) return CERA_HIP_ERR_ARGUMENT;
     hipDeviceProp_t prop;
@@ -378,6 +385,7 @@ void cera_hip_tensor_free(cera_hip_ctx* ctx, cera_hip_dtensor* d) {
     if (!d) return;
     if (ctx) (void)hipStreamSynchronize(ctx->stream);
     if (d->dev && d->owns) (void)hipFree(d->dev);
+    if (d->dev_stream) (void)hipFree(d->dev_stream);
     delete d;
 }
 uint64_t cera_hip_tensor_nbytes(const cera_hip_dtensor* d) { return d ? d->nbytes : 0; }

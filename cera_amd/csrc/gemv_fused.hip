@@ -95,11 +95,15 @@ struct NormQuant {
     }
 };
 
-template <class T, int NM>
+// STREAM: p.w / p.w2 point at the matrices' decode copies (T::load_w_stream), p.row_bytes is
+// their row stride.
+template <class T, int NM, bool STREAM>
 struct RowTile {
     typename T::Wt w[NM];
     __device__ __forceinline__ void load_one(const RowGemvArgs& p, int mi, uint32_t unit, uint32_t row) {
-        T::load_w(w[mi], (mi == 0 ? p.w : p.w2) + static_cast<uint64_t>(row) * p.row_bytes, unit);
+        const uint8_t* r = (mi == 0 ? p.w : p.w2) + static_cast<uint64_t>(row) * p.row_bytes;
+        if (STREAM) T::load_w_stream(w[mi], r, unit, p.k / T::ELEMS_PER_UNIT);
+        else T::load_w(w[mi], r, unit);
     }
     __device__ __forceinline__ void load(const RowGemvArgs& p, uint32_t unit, uint32_t row) {
 #pragma unroll
@@ -113,7 +117,7 @@ struct RowTile {
 // refilled as soon as its dot product is formed, and the per-row epilogue runs once per
 // wavefront with lane i finishing row i.  Every thread of the workgroup must call this (it contains barriers when NORM or
 // SILU_Q8), including wavefronts whose row range is empty.
-template <class T, int NW, int ROWS, bool NORM, int EPI>
+template <class T, int NW, int ROWS, bool NORM, int EPI, bool STREAM>
 __device__ __forceinline__ void row_gemv_body(const RowGemvArgs& p, uint32_t block, uint32_t* s_xq, float* s_xs, double* s_part,
                                               float* s_out) {
     constexpr int NM = EPI == FEPI_SILU_Q8 ? 2 : 1;
@@ -132,7 +136,7 @@ __device__ __forceinline__ void row_gemv_body(const RowGemvArgs& p, uint32_t blo
     }
     // DEPTH rows in flight per wavefront: their loads are issued before the activations are
     // prepared, and each finished row's buffer is refilled with the row DEPTH further on
-    RowTile<T, NM> t[DEPTH];
+    RowTile<T, NM, STREAM> t[DEPTH];
 #pragma unroll
     for (int i = 0; i < DEPTH; ++i) t[i].load(p, unit, min(row_of(i), p.m - 1));   // rows past the end re-read the last row
     __builtin_amdgcn_sched_barrier(0);   // the loads are issued here, not wherever their first use would pull them
@@ -203,22 +207,22 @@ __device__ __forceinline__ void row_gemv_body(const RowGemvArgs& p, uint32_t blo
     }
 }
 
-template <class T, int NW, int ROWS, bool NORM, int EPI>
+template <class T, int NW, int ROWS, bool NORM, int EPI, bool STREAM>
 static __global__ __launch_bounds__(64 * NW, NW <= 8 ? 2 : 1) void row_gemv_kernel(RowGemvArgs p) {
     __shared__ uint32_t s_xq[NORM ? 1024 : 1];
     __shared__ float s_xs[NORM ? 128 : 1];
     __shared__ double s_part[NW];
     __shared__ __attribute__((aligned(16))) float s_out[EPI == FEPI_SILU_Q8 ? NW * ROWS : 4];
-    row_gemv_body<T, NW, ROWS, NORM, EPI>(p, blockIdx.x, s_xq, s_xs, s_part, s_out);
+    row_gemv_body<T, NW, ROWS, NORM, EPI, STREAM>(p, blockIdx.x, s_xq, s_xs, s_part, s_out);
 }
 
-template <class TA, class TB, int NW, int ROWS, bool NORM>
+template <class TA, class TB, int NW, int ROWS, bool NORM, bool STREAM>
 static __global__ __launch_bounds__(64 * NW, 2) void row_gemv_pair_kernel(RowGemvPairArgs p) {
     __shared__ uint32_t s_xq[NORM ? 1024 : 1];
     __shared__ float s_xs[NORM ? 128 : 1];
     __shared__ double s_part[NW];
-    if (blockIdx.x < p.n_blocks_a) row_gemv_body<TA, NW, ROWS, NORM, FEPI_STORE>(p.a, blockIdx.x, s_xq, s_xs, s_part, nullptr);
-    else row_gemv_body<TB, NW, ROWS, NORM, FEPI_STORE>(p.b, blockIdx.x - p.n_blocks_a, s_xq, s_xs, s_part, nullptr);
+    if (blockIdx.x < p.n_blocks_a) row_gemv_body<TA, NW, ROWS, NORM, FEPI_STORE, STREAM>(p.a, blockIdx.x, s_xq, s_xs, s_part, nullptr);
+    else row_gemv_body<TB, NW, ROWS, NORM, FEPI_STORE, STREAM>(p.b, blockIdx.x - p.n_blocks_a, s_xq, s_xs, s_part, nullptr);
 }
 
 // Long rows (4096 < k <= 16384: the down projection): still one wavefront per row, walking the
@@ -229,7 +233,7 @@ static __global__ __launch_bounds__(64 * NW, 2) void row_gemv_pair_kernel(RowGem
 // barrier per row group, which costs it most when the weights come from HBM (12.3 us against
 // 9.6 us from the last-level cache).  Pass t sees exactly the units wavefront t of the K-split
 // kernel sees, and the pass totals are added in wavefront order, so the result has the same bits.
-template <class T, int NW, int TILES, int EPI>
+template <class T, int NW, int TILES, int EPI, bool STREAM>
 static __global__ __launch_bounds__(64 * NW) void row_gemv_long_kernel(RowGemvArgs p) {
     constexpr uint32_t MAX_K = TILES * 64 * T::ELEMS_PER_UNIT;
     __shared__ __attribute__((aligned(16))) int8_t s_xq[MAX_K];
@@ -260,7 +264,8 @@ static __global__ __launch_bounds__(64 * NW) void row_gemv_long_kernel(RowGemvAr
         const uint32_t u = 64 * t + lane;
         live[t] = u < n_units;
         unit[t] = live[t] ? u : 0;   // dead lanes re-read unit 0 with zeroed activations
-        T::load_w(w[t], rp, unit[t]);
+        if (STREAM) T::load_w_stream(w[t], rp, unit[t], n_units);
+        else T::load_w(w[t], rp, unit[t]);
     }
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -289,14 +294,60 @@ static bool fused_type(uint32_t t) { return t == CERA_HIP_Q4_K || t == CERA_HIP_
 // rows that fit one wavefront of 64-weight units, whole super-blocks
 static bool fused_k(uint64_t k) { return k % 256 == 0 && k <= 4096 && k > 0; }
 
-static void fill(RowGemvArgs& a, const cera_hip_dtensor* w, const cera_hip_dtensor* w2, uint32_t rows_per_wave) {
+static void fill(RowGemvArgs& a, const cera_hip_dtensor* w, const cera_hip_dtensor* w2, uint32_t rows_per_wave, bool stream = false) {
     a = RowGemvArgs{};
-    a.w = w->dev;
-    a.w2 = w2 ? w2->dev : nullptr;
+    a.w = stream ? w->dev_stream : w->dev;
+    a.w2 = w2 ? (stream ? w2->dev_stream : w2->dev) : nullptr;
     a.m = static_cast<uint32_t>(w->m);
     a.k = static_cast<uint32_t>(w->k);
-    a.row_bytes = static_cast<uint32_t>(w->row_bytes);
+    a.row_bytes = static_cast<uint32_t>(stream ? w->stream_row_bytes : w->row_bytes);
     a.rows_per_wave = rows_per_wave;
+}
+
+// ---- decode copies ------------------------------------------------------------------------------
+// One thread per unit of a row: the unit's bytes from the native block layout to their places in
+// the decode copy (T::to_stream).
+template <class T>
+static __global__ __launch_bounds__(256) void stream_rows_kernel(const uint8_t* __restrict__ src, uint8_t* __restrict__ dst, uint32_t m,
+                                                                 uint32_t n_units, uint32_t row_bytes, uint32_t stream_row_bytes) {
+    const uint32_t row = blockIdx.x;
+    for (uint32_t u = threadIdx.x; u < n_units; u += blockDim.x)
+        T::to_stream(src + static_cast<uint64_t>(row) * row_bytes, dst + static_cast<uint64_t>(row) * stream_row_bytes, u, n_units);
+}
+
+// Gives a Q4_K / Q6_K matrix its decode copy (a second allocation of about the same size, kept
+// until the tensor is freed): the per-row permutation that lets the one-wavefront-per-row
+// kernels stream it with non-temporal loads.  A load-time re-layout for the kernel that reads
+// it, as the reference's own x86 path does with repack_q4_k_8x8 (cera/src/backend/cpu.rs:1282-1358);
+// the native bytes stay for every other reader (prefill GEMM, embedding lookup, verification
+// route).  Shapes without whole-line planes, other types and views are left alone.
+cera_hip_status cera_tensor_prepare_stream(cera_hip_ctx* ctx, cera_hip_dtensor* w) {
+    if (!ctx->decode_copies) return CERA_HIP_OK;
+    if (!w || w->dev_stream || !w->owns || !fused_type(w->dtype) || w->k == 0 || w->k > 16384 || w->m == 0 || w->m > 0x7FFFFFFFull) return CERA_HIP_OK;
+    const uint32_t k = static_cast<uint32_t>(w->k);
+    const bool q4 = w->dtype == CERA_HIP_Q4_K;
+    if (!(q4 ? Q4K::stream_ok(k) : Q6K::stream_ok(k)) || (reinterpret_cast<uintptr_t>(w->dev) & 15)) return CERA_HIP_OK;
+    const uint64_t srb = q4 ? Q4K::stream_row_bytes(k) : Q6K::stream_row_bytes(k);
+    void* p = nullptr;
+    const hipError_t e = hipMalloc(&p, srb * w->m);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        return cera_fail(ctx, e == hipErrorOutOfMemory ? CERA_HIP_ERR_OOM : CERA_HIP_ERR_DEVICE,
+                         std::string("hipMalloc(decode copy): ") + hipGetErrorString(e));
+    }
+    const dim3 grid(static_cast<uint32_t>(w->m)), block(256);
+    if (q4) hipLaunchKernelGGL(stream_rows_kernel<Q4K>, grid, block, 0, ctx->stream, w->dev, static_cast<uint8_t*>(p), grid.x, k / 64,
+                               static_cast<uint32_t>(w->row_bytes), static_cast<uint32_t>(srb));
+    else hipLaunchKernelGGL(stream_rows_kernel<Q6K>, grid, block, 0, ctx->stream, w->dev, static_cast<uint8_t*>(p), grid.x, k / 64,
+                            static_cast<uint32_t>(w->row_bytes), static_cast<uint32_t>(srb));
+    const hipError_t le = hipGetLastError();
+    if (le != hipSuccess) {
+        (void)hipFree(p);
+        return cera_fail(ctx, CERA_HIP_ERR_DEVICE, std::string("decode copy: ") + hipGetErrorString(le));
+    }
+    w->dev_stream = static_cast<uint8_t*>(p);
+    w->stream_row_bytes = srb;
+    return CERA_HIP_OK;
 }
 static uint32_t blocks_for(uint64_t m, uint32_t rows_per_wave) {
     const uint64_t per = static_cast<uint64_t>(FUSED_NW) * rows_per_wave;
@@ -317,10 +368,12 @@ cera_hip_status cera_launch_ffn_gate_up_fused(cera_hip_ctx* ctx, const cera_hip_
     // 224 workgroups -- one per CU in a single wave of the launch (448 eight-wavefront workgroups
     // leave a quarter of the CUs with half the others' share: 1 % slower end to end)
     constexpr int GATE_UP_NW = 16, ROWS = 4;
-    fill(a, gate, up, ROWS);
+    const bool stream = gate->dev_stream && up->dev_stream;
+    fill(a, gate, up, ROWS, stream);
     a.x = x; a.norm_w = norm_w; a.eps = eps; a.out_q = out_q; a.out_s = out_s;
-    hipLaunchKernelGGL((row_gemv_kernel<Q4K, GATE_UP_NW, ROWS, true, FEPI_SILU_Q8>), dim3((a.m + GATE_UP_NW * ROWS - 1) / (GATE_UP_NW * ROWS)),
-                       dim3(64 * GATE_UP_NW), 0, ctx->stream, a);
+    const dim3 grid((a.m + GATE_UP_NW * ROWS - 1) / (GATE_UP_NW * ROWS)), block(64 * GATE_UP_NW);
+    if (stream) hipLaunchKernelGGL((row_gemv_kernel<Q4K, GATE_UP_NW, ROWS, true, FEPI_SILU_Q8, true>), grid, block, 0, ctx->stream, a);
+    else hipLaunchKernelGGL((row_gemv_kernel<Q4K, GATE_UP_NW, ROWS, true, FEPI_SILU_Q8, false>), grid, block, 0, ctx->stream, a);
     HIP_TRY(ctx, hipGetLastError());
     *launched = true;
     return CERA_HIP_OK;
@@ -335,12 +388,13 @@ cera_hip_status cera_launch_qkv_fused(cera_hip_ctx* ctx, const cera_hip_dtensor*
     const uint64_t rows = wa->m + (wb ? wb->m : 0);
     const uint32_t rpw = rows >= static_cast<uint64_t>(ctx->n_cu) * 8 ? 2 : 1;
     RowGemvPairArgs p;
-    fill(p.a, wa, nullptr, rpw);
+    const bool stream = wa->dev_stream && (!wb || wb->dev_stream);
+    fill(p.a, wa, nullptr, rpw, stream);
     p.a.x = x; p.a.norm_w = norm_w; p.a.eps = eps; p.a.y = ya;
     p.n_blocks_a = blocks_for(wa->m, rpw);
     uint32_t n_blocks = p.n_blocks_a;
     if (wb) {
-        fill(p.b, wb, nullptr, rpw);
+        fill(p.b, wb, nullptr, rpw, stream);
         p.b.x = x; p.b.norm_w = norm_w; p.b.eps = eps; p.b.y = yb;
         n_blocks += blocks_for(wb->m, rpw);
     } else {
@@ -348,16 +402,22 @@ cera_hip_status cera_launch_qkv_fused(cera_hip_ctx* ctx, const cera_hip_dtensor*
     }
     const dim3 grid(n_blocks), block(64 * FUSED_NW);
     const uint32_t ta = wa->dtype, tb = wb ? wb->dtype : wa->dtype;
-#define QKV_LAUNCH(TA_, TB_)                                                                                                  \
-    do {                                                                                                                      \
-        if (rpw == 2) hipLaunchKernelGGL((row_gemv_pair_kernel<TA_, TB_, FUSED_NW, 2, true>), grid, block, 0, ctx->stream, p); \
-        else hipLaunchKernelGGL((row_gemv_pair_kernel<TA_, TB_, FUSED_NW, 1, true>), grid, block, 0, ctx->stream, p);          \
+#define QKV_LAUNCH_S(TA_, TB_, ST_)                                                                                                \
+    do {                                                                                                                           \
+        if (rpw == 2) hipLaunchKernelGGL((row_gemv_pair_kernel<TA_, TB_, FUSED_NW, 2, true, ST_>), grid, block, 0, ctx->stream, p); \
+        else hipLaunchKernelGGL((row_gemv_pair_kernel<TA_, TB_, FUSED_NW, 1, true, ST_>), grid, block, 0, ctx->stream, p);          \
+    } while (0)
+#define QKV_LAUNCH(TA_, TB_)                    \
+    do {                                        \
+        if (stream) QKV_LAUNCH_S(TA_, TB_, true); \
+        else QKV_LAUNCH_S(TA_, TB_, false);     \
     } while (0)
     if (ta == CERA_HIP_Q4_K && tb == CERA_HIP_Q6_K) QKV_LAUNCH(Q4K, Q6K);
     else if (ta == CERA_HIP_Q4_K && tb == CERA_HIP_Q4_K) QKV_LAUNCH(Q4K, Q4K);
     else if (ta == CERA_HIP_Q6_K && tb == CERA_HIP_Q6_K) QKV_LAUNCH(Q6K, Q6K);
     else QKV_LAUNCH(Q6K, Q4K);
 #undef QKV_LAUNCH
+#undef QKV_LAUNCH_S
     HIP_TRY(ctx, hipGetLastError());
     *launched = true;
     return CERA_HIP_OK;
@@ -372,11 +432,38 @@ cera_hip_status cera_launch_row_gemv_add(cera_hip_ctx* ctx, const cera_hip_dtens
     if (!fused_type(w->dtype) || !fused_k(w->k) || !resid || w->m > 65535) return CERA_HIP_OK;
     constexpr int NW = 4, ROWS = 2;
     RowGemvArgs a;
-    fill(a, w, nullptr, ROWS);
+    const bool stream = w->dev_stream != nullptr;
+    fill(a, w, nullptr, ROWS, stream);
     a.xq = xq; a.xs = xs; a.y = y; a.resid = resid;
     const dim3 grid((a.m + NW * ROWS - 1) / (NW * ROWS)), block(64 * NW);
-    if (w->dtype == CERA_HIP_Q4_K) hipLaunchKernelGGL((row_gemv_kernel<Q4K, NW, ROWS, false, FEPI_ADD>), grid, block, 0, ctx->stream, a);
-    else hipLaunchKernelGGL((row_gemv_kernel<Q6K, NW, ROWS, false, FEPI_ADD>), grid, block, 0, ctx->stream, a);
+#define ADD_LAUNCH(TT)                                                                                                     \
+    do {                                                                                                                   \
+        if (stream) hipLaunchKernelGGL((row_gemv_kernel<TT, NW, ROWS, false, FEPI_ADD, true>), grid, block, 0, ctx->stream, a); \
+        else hipLaunchKernelGGL((row_gemv_kernel<TT, NW, ROWS, false, FEPI_ADD, false>), grid, block, 0, ctx->stream, a);    \
+    } while (0)
+    if (w->dtype == CERA_HIP_Q4_K) ADD_LAUNCH(Q4K);
+    else ADD_LAUNCH(Q6K);
+#undef ADD_LAUNCH
+    HIP_TRY(ctx, hipGetLastError());
+    *launched = true;
+    return CERA_HIP_OK;
+}
+
+// y = W . (xs, xq) from a decode copy with a wavefront per row (k <= 4096): the vocabulary head.
+// Only taken when the matrix has a decode copy -- from the native bytes the K-split kernel is as
+// fast.  Same per-row arithmetic, same bits; 73.6 -> 62.3 us on the 128256 x 4096 Q6_K head
+// (6.9 TB/s).
+cera_hip_status cera_launch_row_gemv_store(cera_hip_ctx* ctx, const cera_hip_dtensor* w, const float* xs, const int8_t* xq,
+                                           float* y, bool* launched) {
+    *launched = false;
+    if (!fused_type(w->dtype) || !fused_k(w->k) || !w->dev_stream || w->m > (1u << 24)) return CERA_HIP_OK;
+    constexpr int NW = 4, ROWS = 2;   // four rows per wavefront measured the same
+    RowGemvArgs a;
+    fill(a, w, nullptr, ROWS, true);
+    a.xq = xq; a.xs = xs; a.y = y;
+    const dim3 grid((a.m + NW * ROWS - 1) / (NW * ROWS)), block(64 * NW);
+    if (w->dtype == CERA_HIP_Q4_K) hipLaunchKernelGGL((row_gemv_kernel<Q4K, NW, ROWS, false, FEPI_STORE, true>), grid, block, 0, ctx->stream, a);
+    else hipLaunchKernelGGL((row_gemv_kernel<Q6K, NW, ROWS, false, FEPI_STORE, true>), grid, block, 0, ctx->stream, a);
     HIP_TRY(ctx, hipGetLastError());
     *launched = true;
     return CERA_HIP_OK;
@@ -392,19 +479,26 @@ cera_hip_status cera_launch_row_gemv_long_add(cera_hip_ctx* ctx, const cera_hip_
     // faster end to end than 8 or 16 rows sharing one staged copy of the activations
     constexpr int NW = 4;
     RowGemvArgs a;
-    fill(a, w, nullptr, 1);
+    const bool stream = w->dev_stream != nullptr;
+    fill(a, w, nullptr, 1, stream);
     a.xq = xq; a.xs = xs; a.y = y; a.resid = resid;
     const uint32_t tiles = static_cast<uint32_t>((w->k / 64 + 63) / 64);   // both types: 64 weights per unit
     const dim3 grid((a.m + NW - 1) / NW), block(64 * NW);
-#define LONG_LAUNCH(TT)                                                                                                  \
-    do {                                                                                                                 \
-        if (tiles == 2) hipLaunchKernelGGL((row_gemv_long_kernel<TT, NW, 2, FEPI_ADD>), grid, block, 0, ctx->stream, a);  \
-        else if (tiles == 3) hipLaunchKernelGGL((row_gemv_long_kernel<TT, NW, 3, FEPI_ADD>), grid, block, 0, ctx->stream, a); \
-        else hipLaunchKernelGGL((row_gemv_long_kernel<TT, NW, 4, FEPI_ADD>), grid, block, 0, ctx->stream, a);             \
+#define LONG_LAUNCH_S(TT, ST_)                                                                                                 \
+    do {                                                                                                                       \
+        if (tiles == 2) hipLaunchKernelGGL((row_gemv_long_kernel<TT, NW, 2, FEPI_ADD, ST_>), grid, block, 0, ctx->stream, a);   \
+        else if (tiles == 3) hipLaunchKernelGGL((row_gemv_long_kernel<TT, NW, 3, FEPI_ADD, ST_>), grid, block, 0, ctx->stream, a); \
+        else hipLaunchKernelGGL((row_gemv_long_kernel<TT, NW, 4, FEPI_ADD, ST_>), grid, block, 0, ctx->stream, a);              \
+    } while (0)
+#define LONG_LAUNCH(TT)                      \
+    do {                                     \
+        if (stream) LONG_LAUNCH_S(TT, true); \
+        else LONG_LAUNCH_S(TT, false);       \
     } while (0)
     if (w->dtype == CERA_HIP_Q4_K) LONG_LAUNCH(Q4K);
     else LONG_LAUNCH(Q6K);
 #undef LONG_LAUNCH
+#undef LONG_LAUNCH_S
     HIP_TRY(ctx, hipGetLastError());
     *launched = true;
     return CERA_HIP_OK;
@@ -421,6 +515,8 @@ extern "C" cera_hip_status cera_hip_ffn_gate_up_fused(cera_hip_ctx* ctx, const c
     cera_hip_status st = cera_hip_tensor_upload(ctx, up, &wu);
     if (st != CERA_HIP_OK) { cera_hip_tensor_free(ctx, wg); return st; }
     auto run = [&]() -> cera_hip_status {
+        CERA_TRY(cera_tensor_prepare_stream(ctx, wg));
+        CERA_TRY(cera_tensor_prepare_stream(ctx, wu));
         const uint64_t k = wg->k, m = wg->m;
         void *dx, *dw, *dq, *ds;
         CERA_TRY(cera_scratch(ctx, 0, k * 4, &dx));
@@ -451,6 +547,8 @@ extern "C" cera_hip_status cera_hip_qkv_fused(cera_hip_ctx* ctx, const cera_hip_
     cera_hip_status st = b ? cera_hip_tensor_upload(ctx, b, &wb) : CERA_HIP_OK;
     if (st != CERA_HIP_OK) { cera_hip_tensor_free(ctx, wa); return st; }
     auto run = [&]() -> cera_hip_status {
+        CERA_TRY(cera_tensor_prepare_stream(ctx, wa));
+        if (wb) CERA_TRY(cera_tensor_prepare_stream(ctx, wb));
         const uint64_t k = wa->k;
         void *dx, *dw, *dy;
         CERA_TRY(cera_scratch(ctx, 0, k * 4, &dx));

@@ -20,6 +20,10 @@ struct cera_hip_dtensor {
     uint64_t row_bytes = 0, nbytes = 0;
     uint8_t* dev = nullptr;
     bool owns = true;  // false: a row-range view into another tensor's allocation
+    // optional decode copy (cera_tensor_prepare_stream): the rows permuted for streaming reads,
+    // row stride stream_row_bytes; owned by this tensor
+    uint8_t* dev_stream = nullptr;
+    uint64_t stream_row_bytes = 0;
 };
 
 struct cera_hip_ctx {
@@ -27,6 +31,7 @@ struct cera_hip_ctx {
     hipStream_t stream = nullptr;
     std::string err;
     uint32_t n_cu = 0;
+    bool decode_copies = true;   // cera_hip_ctx_set_decode_copies
     // serialises every call that uses the stream's workspaces below (kernel-level entry points
     // with host buffers, and every model-level call of any model on this context)
     std::recursive_mutex op_mu;
@@ -85,6 +90,9 @@ cera_hip_status cera_launch_gemv(cera_hip_ctx* ctx, const cera_hip_dtensor* w, c
 // y = resid + W.(xs,xq) with one wavefront per row; *launched = false when the shape has no such instance
 cera_hip_status cera_launch_row_gemv_add(cera_hip_ctx* ctx, const cera_hip_dtensor* w, const float* xs, const int8_t* xq,
                                          float* y, const float* resid, bool* launched);
+cera_hip_status cera_tensor_prepare_stream(cera_hip_ctx* ctx, cera_hip_dtensor* w);
+cera_hip_status cera_launch_row_gemv_store(cera_hip_ctx* ctx, const cera_hip_dtensor* w, const float* xs, const int8_t* xq,
+                                           float* y, bool* launched);
 cera_hip_status cera_launch_row_gemv_long_add(cera_hip_ctx* ctx, const cera_hip_dtensor* w, const float* xs, const int8_t* xq,
                                               float* y, const float* resid, bool* launched);
 cera_hip_status cera_launch_gemv_nb(cera_hip_ctx* ctx, const cera_hip_dtensor* w, const float* xs, const int8_t* xq,

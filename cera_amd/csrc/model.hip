@@ -154,6 +154,11 @@ extern "C" cera_hip_status cera_hip_model_create(cera_hip_ctx* ctx, const cera_h
             CERA_TRY(cera_hip_tensor_upload(ctx, &output_cut, &m->output));
             *tot += m->output->nbytes;
         }
+        {   // the vocabulary head streams a decode copy too (a tied head: the embedding table's)
+            cera_hip_dtensor* head = m->output ? m->output : m->embd;
+            CERA_TRY(cera_tensor_prepare_stream(ctx, head));
+            if (head->dev_stream) *tot += head->stream_row_bytes * head->m;
+        }
         float* tmp;
         CERA_TRY(upload_f32(ctx, output_norm, c.hidden, &tmp, tot));
         m->output_norm = tmp; m->owned.push_back(tmp);
@@ -178,6 +183,12 @@ extern "C" cera_hip_status cera_hip_model_create(cera_hip_ctx* ctx, const cera_h
             for (int t = fuse; t < 7; ++t) {
                 CERA_TRY(cera_hip_tensor_upload(ctx, src[t], dst[t]));
                 *tot += (*dst[t])->nbytes;
+            }
+            // decode copies of what the one-wavefront-per-row kernels stream
+            for (cera_hip_dtensor* w : {D.qkv, D.v, D.o, D.gate, D.up, D.down}) {
+                if (!w || w->dev_stream) continue;
+                CERA_TRY(cera_tensor_prepare_stream(ctx, w));
+                if (w->dev_stream) *tot += w->stream_row_bytes * w->m;
             }
             CERA_TRY(upload_f32(ctx, L.attn_norm, c.hidden, &D.attn_norm, tot));
             CERA_TRY(upload_f32(ctx, L.ffn_norm, c.hidden, &D.ffn_norm, tot));
@@ -432,6 +443,14 @@ static cera_hip_status launch_proj_add(cera_hip_ctx* ctx, const cera_hip_dtensor
     return cera_launch_gemv(ctx, w, nullptr, xs, xq, y, resid, CERA_EPI_ADD);
 }
 
+// y = W . (xs, xq): from the decode copy where the matrix has one, else the K-split kernel.
+static cera_hip_status launch_proj_store(cera_hip_ctx* ctx, const cera_hip_dtensor* w, const float* xs, const int8_t* xq, float* y) {
+    bool done = false;
+    CERA_TRY(cera_launch_row_gemv_store(ctx, w, xs, xq, y, &done));
+    if (done) return CERA_HIP_OK;
+    return cera_launch_gemv(ctx, w, nullptr, xs, xq, y, nullptr, CERA_EPI_STORE);
+}
+
 static cera_hip_status project(cera_hip_model* m, const cera_hip_dtensor* w, const float* x_f32, float* y,
                                const float* resid) {
     cera_hip_ctx* ctx = m->ctx;
@@ -454,7 +473,7 @@ static cera_hip_status project(cera_hip_model* m, const cera_hip_dtensor* w, con
         return CERA_HIP_OK;
     }
     if (resid) return launch_proj_add(ctx, w, m->xs, m->xq, y, resid);
-    return cera_launch_gemv(ctx, w, nullptr, m->xs, m->xq, y, nullptr, CERA_EPI_STORE);
+    return launch_proj_store(ctx, w, m->xs, m->xq, y);
 }
 
 // rmsnorm of `rows` rows of n elements with the Q8_0 quantization of the result fused in
@@ -773,6 +792,13 @@ extern "C" cera_hip_status cera_hip_rope(cera_hip_ctx* ctx, float* q, float* k, 
 extern "C" cera_hip_status cera_hip_decode_ops_dev(cera_hip_ctx* ctx, const cera_hip_decode_op* ops, uint32_t n) {
     if (!ctx || (!ops && n)) return CERA_HIP_ERR_ARGUMENT;
     std::lock_guard<std::recursive_mutex> lk(ctx->op_mu);
+    // the launches below are the decode step's, so their matrices get decode copies as a model's do
+    // (on first use; the handles are this library's own objects)
+    for (uint32_t i = 0; i < n; ++i) {
+        if (ops[i].kind > CERA_HIP_OP_NORM_GATE_UP) continue;
+        CERA_TRY(cera_tensor_prepare_stream(ctx, const_cast<cera_hip_dtensor*>(ops[i].w)));
+        CERA_TRY(cera_tensor_prepare_stream(ctx, const_cast<cera_hip_dtensor*>(ops[i].w2)));
+    }
     for (uint32_t i = 0; i < n; ++i) {
         const cera_hip_decode_op& o = ops[i];
         auto bad = [&](const char* what) {
@@ -783,7 +809,7 @@ extern "C" cera_hip_status cera_hip_decode_ops_dev(cera_hip_ctx* ctx, const cera
             case CERA_HIP_OP_GEMV:
                 if (!o.w || !o.xs || !o.xq || !o.y) return bad("GEMV needs w, xs, xq, y");
                 if (o.resid) CERA_TRY(launch_proj_add(ctx, o.w, o.xs, o.xq, o.y, o.resid));
-                else CERA_TRY(cera_launch_gemv(ctx, o.w, nullptr, o.xs, o.xq, o.y, nullptr, CERA_EPI_STORE));
+                else CERA_TRY(launch_proj_store(ctx, o.w, o.xs, o.xq, o.y));
                 break;
             case CERA_HIP_OP_NORM_GEMV:
                 if (!o.w || !o.x || !o.norm_w || !o.y || (o.w2 && !o.y2)) return bad("NORM_GEMV needs w, x, norm_w, y (and y2 with w2)");

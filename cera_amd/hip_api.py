@@ -18,7 +18,7 @@ STATUS = {0: "OK", 1: "ERR_DEVICE", 2: "ERR_OOM", 3: "ERR_UNSUPPORTED_DTYPE", 4:
 
 # every symbol include/cera_hip.h declares
 SYMBOLS = [
-    "cera_hip_ctx_create", "cera_hip_ctx_destroy", "cera_hip_last_error", "cera_hip_sync", "cera_hip_device_info",
+    "cera_hip_ctx_create", "cera_hip_ctx_destroy", "cera_hip_ctx_set_decode_copies", "cera_hip_last_error", "cera_hip_sync", "cera_hip_device_info",
     "cera_hip_malloc", "cera_hip_free", "cera_hip_upload", "cera_hip_download", "cera_hip_copy_dev", "cera_hip_copy_kernel",
     "cera_hip_event_create", "cera_hip_event_destroy", "cera_hip_event_record", "cera_hip_event_elapsed_ms",
     "cera_hip_tensor_upload", "cera_hip_tensor_clone", "cera_hip_tensor_free", "cera_hip_tensor_nbytes",
@@ -93,6 +93,7 @@ def load_library() -> C.CDLL:
     pp = C.POINTER(C.c_void_p)
     sig = {
         "cera_hip_ctx_create": (i32, [i32, C.c_char_p, pp]), "cera_hip_ctx_destroy": (None, [vp]),
+        "cera_hip_ctx_set_decode_copies": (i32, [vp, i32]),
         "cera_hip_last_error": (C.c_char_p, [vp]), "cera_hip_sync": (i32, [vp]),
         "cera_hip_device_info": (i32, [vp, C.c_char_p, C.POINTER(u32), C.POINTER(u64)]),
         "cera_hip_malloc": (i32, [vp, u64, pp]), "cera_hip_free": (i32, [vp, vp]),
@@ -198,6 +199,10 @@ class Context:
 
     def sync(self):
         self.check(self.lib.cera_hip_sync(self.h))
+
+    def set_decode_copies(self, enabled: bool):
+        """Whether matrices prepared from now on get the permuted second copy the decode GEMVs stream."""
+        self.check(self.lib.cera_hip_ctx_set_decode_copies(self.h, 1 if enabled else 0))
 
     def device_info(self):
         name = C.create_string_buffer(256)

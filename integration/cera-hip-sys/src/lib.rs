@@ -175,6 +175,7 @@ pub fn cera_hip_ctx_create(
         out: *mut *mut cera_hip_ctx,
     ) -> cera_hip_status;
     pub fn cera_hip_ctx_destroy(ctx: *mut cera_hip_ctx);
+    pub fn cera_hip_ctx_set_decode_copies(ctx: *mut cera_hip_ctx, enabled: c_int) -> cera_hip_status;
     pub fn cera_hip_last_error(ctx: *const cera_hip_ctx) -> *const c_char;
     pub fn cera_hip_sync(ctx: *mut cera_hip_ctx) -> cera_hip_status;
     pub fn cera_hip_device_info(

@@ -600,3 +600,50 @@ def test_projection_with_residual_is_bitwise_the_plain_gemv(hip, dtype, m, k):
     got = hip.gemv_add_dev(dtype, w, x, r, m, k)
     want = (r + plain).astype(np.float32)
     assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), float(np.abs(got - want).max())
+
+
+@pytest.fixture
+def no_decode_copies(hip):
+    """Runs the body with decode copies switched off on the shared context, then on again."""
+    def run(fn):
+        hip.set_decode_copies(False)
+        try:
+            return fn()
+        finally:
+            hip.set_decode_copies(True)
+    return run
+
+
+@pytest.mark.parametrize("dtype,m,k", [(Q6_K, 1024, 14336), (Q4_K, 512, 14336), (Q6_K, 77, 8192), (Q4_K, 100, 6144), (Q4_K, 130, 16384),
+                                       (Q4_K, 1030, 4096), (Q6_K, 130, 4096), (Q6_K, 40, 2048), (Q4_K, 33, 1024)])
+def test_residual_projection_streams_the_decode_copy_to_the_same_bits(hip, no_decode_copies, dtype, m, k):
+    """A matrix's decode copy is a permutation of its bytes, read by the same arithmetic: the
+    residual projections give identical bits with the copy (the default) and from the native
+    bytes.  k = 1024 has no copy either way (its planes would not start on 128-byte lines)."""
+    print(f"decode copy on/off {util.NAMES[dtype]} {m}x{k}", flush=True)
+    w, _ = util.make_weights(dtype, m, k, seed=m + k + 7)
+    x = util.make_x(k, 5)
+    r = util.make_x(m, 6)
+    with_copy = hip.gemv_add_dev(dtype, w, x, r, m, k)
+    native = no_decode_copies(lambda: hip.gemv_add_dev(dtype, w, x, r, m, k))
+    assert np.array_equal(with_copy.view(np.uint32), native.view(np.uint32))
+    plain = hip.gemv(dtype, w, x, m, k)
+    assert np.array_equal(with_copy.view(np.uint32), (r + plain).astype(np.float32).view(np.uint32))
+
+
+def test_fused_launches_stream_the_decode_copy_to_the_same_bits(hip, no_decode_copies):
+    """The Q|K|V launch (Q4_K and Q6_K matrices in one grid) and the gate|up launch, with and
+    without decode copies."""
+    k = 4096
+    wa, _ = util.make_weights(Q4_K, 1280, k, seed=91)
+    wb, _ = util.make_weights(Q6_K, 256, k, seed=92)
+    wg, _ = util.make_weights(Q4_K, 1024, k, seed=93)
+    wu, _ = util.make_weights(Q4_K, 1024, k, seed=94)
+    x = util.make_x(k, 95) * np.float32(1.3)
+    nw = (1.0 + 0.1 * util.make_x(k, 96)).astype(np.float32)
+    ya, yb = hip.qkv_fused(Q4_K, wa, 1280, Q6_K, wb, 256, k, x, nw, 1e-5)
+    q, sc = hip.ffn_gate_up_fused(wg, wu, 1024, k, x, nw, 1e-5)
+    ya0, yb0 = no_decode_copies(lambda: hip.qkv_fused(Q4_K, wa, 1280, Q6_K, wb, 256, k, x, nw, 1e-5))
+    q0, sc0 = no_decode_copies(lambda: hip.ffn_gate_up_fused(wg, wu, 1024, k, x, nw, 1e-5))
+    assert np.array_equal(ya.view(np.uint32), ya0.view(np.uint32)) and np.array_equal(yb.view(np.uint32), yb0.view(np.uint32))
+    assert np.array_equal(q, q0) and np.array_equal(sc.view(np.uint32), sc0.view(np.uint32))

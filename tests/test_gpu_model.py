@@ -482,3 +482,31 @@ def test_two_models_on_one_context_from_two_threads(hip, orc):
         for a, b in zip(got[i], want[i]):
             assert np.array_equal(a.view(np.uint32), b.view(np.uint32)), i
     ga.close(); gb.close()
+
+
+def test_decode_copies_do_not_change_a_logit(hip):
+    """A model whose widths are multiples of 2048 decodes through the permuted second copies of its
+    projection matrices (the default); the same model built without them reads the native bytes.
+    Same arithmetic on the same values: every logit of every step is bit-identical."""
+    cfg = dict(n_layers=2, hidden=2048, ffn=6144, n_heads=16, n_kv_heads=4, head_dim=128, vocab=768,
+               max_seq_len=64, rope_type=1, rope_theta=10000.0, rms_eps=1e-5)
+    weights = synth.make_llama(cfg, seed=4321, sigma=0.03, norm_jitter=0.1)
+    _say("model: decode copies on")
+    with_copies = hip_api.Model(hip, cfg, weights)
+    hip.set_decode_copies(False)
+    try:
+        _say("model: decode copies off")
+        native = hip_api.Model(hip, cfg, weights)
+    finally:
+        hip.set_decode_copies(True)
+    try:
+        assert with_copies.memory_bytes > native.memory_bytes * 1.5
+        tok = 5
+        for pos in range(6):
+            a = with_copies.forward(tok, pos)
+            b = native.forward(tok, pos)
+            assert np.array_equal(a.view(np.uint32), b.view(np.uint32)), pos
+            tok = int(np.argmax(a))
+    finally:
+        with_copies.close()
+        native.close()
