@@ -106,7 +106,8 @@ CERA_HIP_API cera_hip_status cera_hip_sync(cera_hip_ctx*);
  * about the same size in which each row's bytes are permuted so that the decode GEMV kernels read
  * it in whole 128-byte lines with non-temporal loads (+6 % decode rate on the 8B model for about
  * twice those matrices' memory); every other reader keeps the native GGUF bytes.  Results are
- * bit-identical either way.  Applies to matrices prepared after the call.  A load-time re-layout
+ * bit-identical either way; a copy that does not fit in device memory is skipped.  Applies to
+ * matrices prepared after the call.  A load-time re-layout
  * for one kernel, as the reference's x86 path does with repack_q4_k_8x8
  * (cera/src/backend/cpu.rs:1282-1358); it has no switch there. */
 CERA_HIP_API cera_hip_status cera_hip_ctx_set_decode_copies(cera_hip_ctx* ctx, int enabled);
@@ -354,7 +355,9 @@ CERA_HIP_API cera_hip_status cera_hip_gemv_seq_dev(cera_hip_ctx*, const cera_hip
  *   CERA_HIP_OP_NORM_QUANT     y = rmsnorm(x, norm_w), (out_q, out_s) = Q8_0(y), n elements (before the head)
  *   CERA_HIP_OP_QUANT          (out_q, out_s) = Q8_0(x), n elements (quantize_f32_to_q8_0,
  *                              cera/src/backend/cpu.rs:942-958)
- * All pointers are device pointers; fields an op does not use are ignored. */
+ * All pointers are device pointers; fields an op does not use are ignored.  With decode copies on
+ * (cera_hip_ctx_set_decode_copies), a matrix's first use here allocates and builds its copy, as
+ * cera_hip_model_create does for a model's: time the second call, not the first. */
 enum { CERA_HIP_OP_GEMV = 0, CERA_HIP_OP_NORM_GEMV = 1, CERA_HIP_OP_NORM_GATE_UP = 2, CERA_HIP_OP_NORM_QUANT = 3,
        CERA_HIP_OP_QUANT = 4 };
 typedef struct {
