@@ -530,7 +530,9 @@ def main() -> int:
                                "down 4096x14336 Q6_K) + rmsnorm+Q8_0 + head 128256x4096 Q6_K",
                    "launches_per_step": len(step_ops), "weight_bytes_per_step": weight_bytes,
                    "algorithmic_bytes_per_step": step_bytes, "w_sigma": 0.02, "seed": args.seed,
-                   "distinct_weight_copies": n_copies},
+                   "distinct_weight_copies": n_copies,
+                   "weight_layout": "each matrix read from its decode copy (per-row permutation of the GGUF bytes, the "
+                                    "library's default, built before the timed region); same bytes per step"},
         "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2),
         "ms_per_step_p50": round(p50, 4), "ms_per_step_p10": round(p10, 4), "ms_per_step_p90": round(p90, 4),
         "value_p50_GB/s": round(step_bytes / (p50 * 1e-3) / 1e9, 1),
