@@ -86,22 +86,24 @@ struct Q4K {
         w.q0 = ld_u128(blk + 16 + (u & 3) * 32);
         w.q1 = ld_u128(blk + 32 + (u & 3) * 32);
     }
-    // The decode copy of a row (see stream_rows_kernel): the same 144 * n_units / 4 bytes permuted
-    // into planes -- every block's 16-byte header, then every unit's first 16 quant bytes, then
-    // every unit's second 16 -- so that each of the three loads of a wavefront reads consecutive
-    // bytes, whole 128-byte lines, once: the shape the non-temporal hint needs.
-    static constexpr uint32_t stream_row_bytes(uint32_t k) { return k / 256 * 144; }
-    static constexpr bool stream_ok(uint32_t k) { return k % 2048 == 0; }   // planes and rows start on 128-byte lines
+    // The decode copy of a row (see stream_rows_kernel): the row's bytes permuted into planes --
+    // every block's 16-byte header, then every unit's first 16 quant bytes, then every unit's
+    // second 16, each plane padded to whole 128-byte lines -- so that each of the three loads of a
+    // wavefront reads consecutive bytes, whole lines, once: the shape the non-temporal hint needs.
+    static constexpr uint32_t up128(uint32_t b) { return (b + 127u) & ~127u; }
+    static constexpr uint32_t stream_q0(uint32_t n_units) { return up128(4 * n_units); }
+    static constexpr uint32_t stream_q1(uint32_t n_units) { return stream_q0(n_units) + up128(16 * n_units); }
+    static constexpr uint32_t stream_row_bytes(uint32_t k) { return stream_q1(k / 64) + up128(16 * (k / 64)); }
     __device__ static void load_w_stream(Wt& w, const uint8_t* row, uint32_t u, uint32_t n_units) {
         w.h = ld_u128_nt(row + (u >> 2) * 16);
-        w.q0 = ld_u128_nt(row + 4 * n_units + u * 16);
-        w.q1 = ld_u128_nt(row + 20 * n_units + u * 16);
+        w.q0 = ld_u128_nt(row + stream_q0(n_units) + u * 16);
+        w.q1 = ld_u128_nt(row + stream_q1(n_units) + u * 16);
     }
     __device__ static void to_stream(const uint8_t* row, uint8_t* dst, uint32_t u, uint32_t n_units) {
         const uint8_t* blk = row + (u >> 2) * 144;
         if ((u & 3) == 0) *reinterpret_cast<uint4*>(dst + (u >> 2) * 16) = ld_u128(blk);
-        *reinterpret_cast<uint4*>(dst + 4 * n_units + u * 16) = ld_u128(blk + 16 + (u & 3) * 32);
-        *reinterpret_cast<uint4*>(dst + 20 * n_units + u * 16) = ld_u128(blk + 32 + (u & 3) * 32);
+        *reinterpret_cast<uint4*>(dst + stream_q0(n_units) + u * 16) = ld_u128(blk + 16 + (u & 3) * 32);
+        *reinterpret_cast<uint4*>(dst + stream_q1(n_units) + u * 16) = ld_u128(blk + 32 + (u & 3) * 32);
     }
     __device__ static float dot(const Wt& w, const Act& a, uint32_t u, int32_t* dbg) {
         const uint32_t g = u & 3;
@@ -169,26 +171,29 @@ struct Q6K {
         w.d = ld_u16(blk + 208);
     }
     // The decode copy of a row: planes of the units' three 16-byte runs (ql low, ql + 32, qh),
-    // then the scales (8 bytes per half block) and the block scales d, the row padded to whole
-    // 128-byte lines.  The three big planes are read once, non-temporally; the small ones are
-    // shared by neighbouring lanes and passes and stay ordinary loads.
-    static constexpr uint32_t stream_row_bytes(uint32_t k) { return (k / 256 * 210 + 127) / 128 * 128; }
-    static constexpr bool stream_ok(uint32_t k) { return k % 2048 == 0; }
+    // then the scales (8 bytes per half block) and the block scales d, every plane padded to
+    // whole 128-byte lines.  The three big planes are read once, non-temporally; the small ones
+    // are shared by neighbouring lanes and passes and stay ordinary loads.
+    static constexpr uint32_t up128(uint32_t b) { return (b + 127u) & ~127u; }
+    static constexpr uint32_t stream_sc(uint32_t n_units) { return 3 * up128(16 * n_units); }
+    static constexpr uint32_t stream_d(uint32_t n_units) { return stream_sc(n_units) + up128(4 * n_units); }
+    static constexpr uint32_t stream_row_bytes(uint32_t k) { return stream_d(k / 64) + up128(k / 64 / 2); }
     __device__ static void load_w_stream(Wt& w, const uint8_t* row, uint32_t u, uint32_t n_units) {
+        const uint32_t plane = up128(16 * n_units);
         w.qa = ld_u128_nt(row + u * 16);
-        w.qb = ld_u128_nt(row + 16 * n_units + u * 16);
-        w.qh = ld_u128_nt(row + 32 * n_units + u * 16);
-        w.sc = *reinterpret_cast<const uint2*>(row + 48 * n_units + (u >> 1) * 8);
-        w.d = ld_u16(row + 52 * n_units + (u >> 2) * 2);
+        w.qb = ld_u128_nt(row + plane + u * 16);
+        w.qh = ld_u128_nt(row + 2 * plane + u * 16);
+        w.sc = *reinterpret_cast<const uint2*>(row + stream_sc(n_units) + (u >> 1) * 8);
+        w.d = ld_u16(row + stream_d(n_units) + (u >> 2) * 2);
     }
     __device__ static void to_stream(const uint8_t* row, uint8_t* dst, uint32_t u, uint32_t n_units) {
         const uint8_t* blk = row + (u >> 2) * 210;
-        const uint32_t nh = (u >> 1) & 1, j = u & 1;
+        const uint32_t nh = (u >> 1) & 1, j = u & 1, plane = up128(16 * n_units);
         *reinterpret_cast<uint4*>(dst + u * 16) = ld_u128_a2(blk + nh * 64 + j * 16);
-        *reinterpret_cast<uint4*>(dst + 16 * n_units + u * 16) = ld_u128_a2(blk + nh * 64 + 32 + j * 16);
-        *reinterpret_cast<uint4*>(dst + 32 * n_units + u * 16) = ld_u128_a2(blk + 128 + nh * 32 + j * 16);
-        if (j == 0) *reinterpret_cast<uint2*>(dst + 48 * n_units + (u >> 1) * 8) = ld_u64_a2(blk + 192 + nh * 8);
-        if ((u & 3) == 0) *reinterpret_cast<uint16_t*>(dst + 52 * n_units + (u >> 2) * 2) = static_cast<uint16_t>(ld_u16(blk + 208));
+        *reinterpret_cast<uint4*>(dst + plane + u * 16) = ld_u128_a2(blk + nh * 64 + 32 + j * 16);
+        *reinterpret_cast<uint4*>(dst + 2 * plane + u * 16) = ld_u128_a2(blk + 128 + nh * 32 + j * 16);
+        if (j == 0) *reinterpret_cast<uint2*>(dst + stream_sc(n_units) + (u >> 1) * 8) = ld_u64_a2(blk + 192 + nh * 8);
+        if ((u & 3) == 0) *reinterpret_cast<uint16_t*>(dst + stream_d(n_units) + (u >> 2) * 2) = static_cast<uint16_t>(ld_u16(blk + 208));
     }
     __device__ static float dot(const Wt& w, const Act& a, uint32_t u, int32_t* dbg) {
         uint32_t is = u & 1;  // l0 / 16

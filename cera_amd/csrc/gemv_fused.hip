@@ -320,13 +320,13 @@ static __global__ __launch_bounds__(256) void stream_rows_kernel(const uint8_t* 
 // kernels stream it with non-temporal loads.  A load-time re-layout for the kernel that reads
 // it, as the reference's own x86 path does with repack_q4_k_8x8 (cera/src/backend/cpu.rs:1282-1358);
 // the native bytes stay for every other reader (prefill GEMM, embedding lookup, verification
-// route).  Shapes without whole-line planes, other types and views are left alone.
+// route).  Other types and views are left alone.
 cera_hip_status cera_tensor_prepare_stream(cera_hip_ctx* ctx, cera_hip_dtensor* w) {
     if (!ctx->decode_copies) return CERA_HIP_OK;
     if (!w || w->dev_stream || !w->owns || !fused_type(w->dtype) || w->k == 0 || w->k > 16384 || w->m == 0 || w->m > 0x7FFFFFFFull) return CERA_HIP_OK;
     const uint32_t k = static_cast<uint32_t>(w->k);
     const bool q4 = w->dtype == CERA_HIP_Q4_K;
-    if (!(q4 ? Q4K::stream_ok(k) : Q6K::stream_ok(k)) || (reinterpret_cast<uintptr_t>(w->dev) & 15)) return CERA_HIP_OK;
+    if (k % 256 || (reinterpret_cast<uintptr_t>(w->dev) & 15)) return CERA_HIP_OK;
     const uint64_t srb = q4 ? Q4K::stream_row_bytes(k) : Q6K::stream_row_bytes(k);
     void* p = nullptr;
     const hipError_t e = hipMalloc(&p, srb * w->m);

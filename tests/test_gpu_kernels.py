@@ -615,11 +615,13 @@ def no_decode_copies(hip):
 
 
 @pytest.mark.parametrize("dtype,m,k", [(Q6_K, 1024, 14336), (Q4_K, 512, 14336), (Q6_K, 77, 8192), (Q4_K, 100, 6144), (Q4_K, 130, 16384),
-                                       (Q4_K, 1030, 4096), (Q6_K, 130, 4096), (Q6_K, 40, 2048), (Q4_K, 33, 1024)])
+                                       (Q4_K, 1030, 4096), (Q6_K, 130, 4096), (Q6_K, 40, 2048), (Q4_K, 33, 1024),
+                                       (Q4_K, 70, 3584), (Q6_K, 50, 11008), (Q4_K, 64, 5120), (Q6_K, 40, 256), (Q4_K, 9, 256),
+                                       (Q6_K, 35, 3584), (Q4_K, 48, 11008)])
 def test_residual_projection_streams_the_decode_copy_to_the_same_bits(hip, no_decode_copies, dtype, m, k):
     """A matrix's decode copy is a permutation of its bytes, read by the same arithmetic: the
     residual projections give identical bits with the copy (the default) and from the native
-    bytes.  k = 1024 has no copy either way (its planes would not start on 128-byte lines)."""
+    bytes, whatever the row length (planes are padded to whole 128-byte lines)."""
     print(f"decode copy on/off {util.NAMES[dtype]} {m}x{k}", flush=True)
     w, _ = util.make_weights(dtype, m, k, seed=m + k + 7)
     x = util.make_x(k, 5)
