@@ -264,6 +264,20 @@ struct Q4_0 {  // 18 B: d, qs[16]; byte i = element i (low nibble), element i+16
         w.d = ld_u16(blk);
         w.q = ld_u128_a2(blk + 2);
     }
+    // decode copy of a row: every block's scale, then every block's 16 quant bytes, each plane
+    // padded to whole 128-byte lines (see Q4K::load_w_stream)
+    static constexpr uint32_t up128(uint32_t b) { return (b + 127u) & ~127u; }
+    static constexpr uint32_t stream_q(uint32_t n_units) { return up128(2 * n_units); }
+    static constexpr uint32_t stream_row_bytes(uint32_t k) { return stream_q(k / 32) + up128(16 * (k / 32)); }
+    __device__ static void load_w_stream(Wt& w, const uint8_t* row, uint32_t u, uint32_t n_units) {
+        w.d = *reinterpret_cast<const uint16_t*>(row + 2 * u);
+        w.q = ld_u128_nt(row + stream_q(n_units) + u * 16);
+    }
+    __device__ static void to_stream(const uint8_t* row, uint8_t* dst, uint32_t u, uint32_t n_units) {
+        const uint8_t* blk = row + u * 18;
+        *reinterpret_cast<uint16_t*>(dst + 2 * u) = static_cast<uint16_t>(ld_u16(blk));
+        *reinterpret_cast<uint4*>(dst + stream_q(n_units) + u * 16) = ld_u128_a2(blk + 2);
+    }
     __device__ static float dot(const Wt& w, const Act& a, uint32_t u, int32_t* dbg) {
         int acc = -8 * a.asum;
         const uint32_t q[4] = {w.q.x, w.q.y, w.q.z, w.q.w};
@@ -289,6 +303,19 @@ struct Q4_1 {  // 20 B: d, m, qs[16]; value = q*d + m
         const uint8_t* blk = row + u * 20;
         w.dm = *reinterpret_cast<const uint32_t*>(blk);
         w.q = ld_u128_a4(blk + 4);
+    }
+    // decode copy of a row: every block's (d, m), then every block's 16 quant bytes
+    static constexpr uint32_t up128(uint32_t b) { return (b + 127u) & ~127u; }
+    static constexpr uint32_t stream_q(uint32_t n_units) { return up128(4 * n_units); }
+    static constexpr uint32_t stream_row_bytes(uint32_t k) { return stream_q(k / 32) + up128(16 * (k / 32)); }
+    __device__ static void load_w_stream(Wt& w, const uint8_t* row, uint32_t u, uint32_t n_units) {
+        w.dm = *reinterpret_cast<const uint32_t*>(row + 4 * u);
+        w.q = ld_u128_nt(row + stream_q(n_units) + u * 16);
+    }
+    __device__ static void to_stream(const uint8_t* row, uint8_t* dst, uint32_t u, uint32_t n_units) {
+        const uint8_t* blk = row + u * 20;
+        *reinterpret_cast<uint32_t*>(dst + 4 * u) = *reinterpret_cast<const uint32_t*>(blk);
+        *reinterpret_cast<uint4*>(dst + stream_q(n_units) + u * 16) = ld_u128_a4(blk + 4);
     }
     __device__ static float dot(const Wt& w, const Act& a, uint32_t u, int32_t* dbg) {
         int acc = 0;
@@ -317,6 +344,21 @@ struct Q8_0 {  // 34 B: d, int8[32]
         w.d = ld_u16(blk);
         w.q0 = ld_u128_a2(blk + 2);
         w.q1 = ld_u128_a2(blk + 18);
+    }
+    // decode copy of a row: every block's scale, then every block's first and second 16 codes
+    static constexpr uint32_t up128(uint32_t b) { return (b + 127u) & ~127u; }
+    static constexpr uint32_t stream_q(uint32_t n_units) { return up128(2 * n_units); }
+    static constexpr uint32_t stream_row_bytes(uint32_t k) { return stream_q(k / 32) + 2 * up128(16 * (k / 32)); }
+    __device__ static void load_w_stream(Wt& w, const uint8_t* row, uint32_t u, uint32_t n_units) {
+        w.d = *reinterpret_cast<const uint16_t*>(row + 2 * u);
+        w.q0 = ld_u128_nt(row + stream_q(n_units) + u * 16);
+        w.q1 = ld_u128_nt(row + stream_q(n_units) + up128(16 * n_units) + u * 16);
+    }
+    __device__ static void to_stream(const uint8_t* row, uint8_t* dst, uint32_t u, uint32_t n_units) {
+        const uint8_t* blk = row + u * 34;
+        *reinterpret_cast<uint16_t*>(dst + 2 * u) = static_cast<uint16_t>(ld_u16(blk));
+        *reinterpret_cast<uint4*>(dst + stream_q(n_units) + u * 16) = ld_u128_a2(blk + 2);
+        *reinterpret_cast<uint4*>(dst + stream_q(n_units) + up128(16 * n_units) + u * 16) = ld_u128_a2(blk + 18);
     }
     __device__ static float dot(const Wt& w, const Act& a, uint32_t u, int32_t* dbg) {
         int acc = 0;

@@ -97,15 +97,18 @@ struct NormQuant {
 
 // STREAM: p.w / p.w2 point at the matrices' decode copies (T::load_w_stream), p.row_bytes is
 // their row stride.
-template <class T, int NM, bool STREAM>
+template <class T, int NM, bool STREAM, int TILES>
 struct RowTile {
-    typename T::Wt w[NM];
-    __device__ __forceinline__ void load_one(const RowGemvArgs& p, int mi, uint32_t unit, uint32_t row) {
+    typename T::Wt w[NM][TILES];
+    __device__ __forceinline__ void load_one(const RowGemvArgs& p, int mi, const uint32_t (&unit)[TILES], uint32_t row) {
         const uint8_t* r = (mi == 0 ? p.w : p.w2) + static_cast<uint64_t>(row) * p.row_bytes;
-        if (STREAM) T::load_w_stream(w[mi], r, unit, p.k / T::ELEMS_PER_UNIT);
-        else T::load_w(w[mi], r, unit);
+#pragma unroll
+        for (int tt = 0; tt < TILES; ++tt) {
+            if (STREAM) T::load_w_stream(w[mi][tt], r, unit[tt], p.k / T::ELEMS_PER_UNIT);
+            else T::load_w(w[mi][tt], r, unit[tt]);
+        }
     }
-    __device__ __forceinline__ void load(const RowGemvArgs& p, uint32_t unit, uint32_t row) {
+    __device__ __forceinline__ void load(const RowGemvArgs& p, const uint32_t (&unit)[TILES], uint32_t row) {
 #pragma unroll
         for (int mi = 0; mi < NM; ++mi) load_one(p, mi, unit, row);
     }
@@ -117,14 +120,22 @@ struct RowTile {
 // refilled as soon as its dot product is formed, and the per-row epilogue runs once per
 // wavefront with lane i finishing row i.  Every thread of the workgroup must call this (it contains barriers when NORM or
 // SILU_Q8), including wavefronts whose row range is empty.
-template <class T, int NW, int ROWS, bool NORM, int EPI, bool STREAM>
+// TILES: units per lane (a row is TILES passes of 64 units: 1 for the K-quants' 64-weight units up
+// to k = 4096, 2 for the 32-weight blocks of Q4_0 / Q8_0 beyond k = 2048).  Pass t holds the units
+// wavefront t of the K-split kernel holds and the pass totals are added in that order: same bits.
+template <class T, int NW, int ROWS, bool NORM, int EPI, bool STREAM, int TILES>
 __device__ __forceinline__ void row_gemv_body(const RowGemvArgs& p, uint32_t block, uint32_t* s_xq, float* s_xs, double* s_part,
                                               float* s_out) {
     constexpr int NM = EPI == FEPI_SILU_Q8 ? 2 : 1;
     const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const uint32_t n_units = p.k / T::ELEMS_PER_UNIT;
-    const bool live = lane < n_units;
-    const uint32_t unit = live ? lane : 0;
+    bool live[TILES];
+    uint32_t unit[TILES];
+#pragma unroll
+    for (int tt = 0; tt < TILES; ++tt) {
+        live[tt] = 64 * tt + lane < n_units;
+        unit[tt] = live[tt] ? 64 * tt + lane : 0;   // dead lanes re-read unit 0 with zeroed activations
+    }
     constexpr int DEPTH = ROWS < 2 ? ROWS : 2;
     const uint32_t r0 = (block * NW + wave) * ROWS;
     auto row_of = [&](int i) -> uint32_t { return r0 + i; };
@@ -136,17 +147,17 @@ __device__ __forceinline__ void row_gemv_body(const RowGemvArgs& p, uint32_t blo
     }
     // DEPTH rows in flight per wavefront: their loads are issued before the activations are
     // prepared, and each finished row's buffer is refilled with the row DEPTH further on
-    RowTile<T, NM, STREAM> t[DEPTH];
+    RowTile<T, NM, STREAM, TILES> t[DEPTH];
 #pragma unroll
     for (int i = 0; i < DEPTH; ++i) t[i].load(p, unit, min(row_of(i), p.m - 1));   // rows past the end re-read the last row
     __builtin_amdgcn_sched_barrier(0);   // the loads are issued here, not wherever their first use would pull them
 
-    typename T::Act act;
-    if (NORM) {
-        nq.finish(p.k, p.eps, s_xq, s_xs, s_part);
-        T::load_act(act, reinterpret_cast<const int8_t*>(s_xq), s_xs, unit, live);
-    } else {
-        T::load_act(act, p.xq, p.xs, unit, live);
+    typename T::Act act[TILES];
+    if (NORM) nq.finish(p.k, p.eps, s_xq, s_xs, s_part);
+#pragma unroll
+    for (int tt = 0; tt < TILES; ++tt) {
+        if (NORM) T::load_act(act[tt], reinterpret_cast<const int8_t*>(s_xq), s_xs, unit[tt], live[tt]);
+        else T::load_act(act[tt], p.xq, p.xs, unit[tt], live[tt]);
     }
 
     float tot[ROWS][NM];   // wave-uniform row totals
@@ -154,14 +165,23 @@ __device__ __forceinline__ void row_gemv_body(const RowGemvArgs& p, uint32_t blo
     for (int i = 0; i < ROWS; ++i) {
 #pragma unroll
         for (int mi = 0; mi < NM; ++mi) {
-            const float part = T::dot(t[i % DEPTH].w[mi], act, unit, nullptr);
-            // the buffer is free as soon as its dot is formed: refill it before the reduction
+            float part[TILES];
+#pragma unroll
+            for (int tt = 0; tt < TILES; ++tt) part[tt] = T::dot(t[i % DEPTH].w[mi][tt], act[tt], unit[tt], nullptr);
+            // the buffer is free as soon as its dots are formed: refill it before the reduction
             if (i + DEPTH < ROWS) {
                 __builtin_amdgcn_sched_barrier(0);
                 t[i % DEPTH].load_one(p, mi, unit, min(row_of(i + DEPTH), p.m - 1));
                 __builtin_amdgcn_sched_barrier(0);
             }
-            tot[i][mi] = wave_sum(part);
+            if (TILES == 1) {
+                tot[i][mi] = wave_sum(part[0]);
+            } else {
+                float sum = 0.0f;
+#pragma unroll
+                for (int tt = 0; tt < TILES; ++tt) sum += wave_sum(part[tt]);
+                tot[i][mi] = sum;
+            }
         }
     }
     // epilogue once per wavefront: lane i finishes row i
@@ -207,22 +227,22 @@ __device__ __forceinline__ void row_gemv_body(const RowGemvArgs& p, uint32_t blo
     }
 }
 
-template <class T, int NW, int ROWS, bool NORM, int EPI, bool STREAM>
+template <class T, int NW, int ROWS, bool NORM, int EPI, bool STREAM, int TILES = 1>
 static __global__ __launch_bounds__(64 * NW, NW <= 8 ? 2 : 1) void row_gemv_kernel(RowGemvArgs p) {
     __shared__ uint32_t s_xq[NORM ? 1024 : 1];
     __shared__ float s_xs[NORM ? 128 : 1];
     __shared__ double s_part[NW];
     __shared__ __attribute__((aligned(16))) float s_out[EPI == FEPI_SILU_Q8 ? NW * ROWS : 4];
-    row_gemv_body<T, NW, ROWS, NORM, EPI, STREAM>(p, blockIdx.x, s_xq, s_xs, s_part, s_out);
+    row_gemv_body<T, NW, ROWS, NORM, EPI, STREAM, TILES>(p, blockIdx.x, s_xq, s_xs, s_part, s_out);
 }
 
-template <class TA, class TB, int NW, int ROWS, bool NORM, bool STREAM>
+template <class TA, class TB, int NW, int ROWS, bool NORM, bool STREAM, int TILES = 1>
 static __global__ __launch_bounds__(64 * NW, 2) void row_gemv_pair_kernel(RowGemvPairArgs p) {
     __shared__ uint32_t s_xq[NORM ? 1024 : 1];
     __shared__ float s_xs[NORM ? 128 : 1];
     __shared__ double s_part[NW];
-    if (blockIdx.x < p.n_blocks_a) row_gemv_body<TA, NW, ROWS, NORM, FEPI_STORE, STREAM>(p.a, blockIdx.x, s_xq, s_xs, s_part, nullptr);
-    else row_gemv_body<TB, NW, ROWS, NORM, FEPI_STORE, STREAM>(p.b, blockIdx.x - p.n_blocks_a, s_xq, s_xs, s_part, nullptr);
+    if (blockIdx.x < p.n_blocks_a) row_gemv_body<TA, NW, ROWS, NORM, FEPI_STORE, STREAM, TILES>(p.a, blockIdx.x, s_xq, s_xs, s_part, nullptr);
+    else row_gemv_body<TB, NW, ROWS, NORM, FEPI_STORE, STREAM, TILES>(p.b, blockIdx.x - p.n_blocks_a, s_xq, s_xs, s_part, nullptr);
 }
 
 // Long rows (4096 < k <= 16384: the down projection): still one wavefront per row, walking the
@@ -290,9 +310,21 @@ static __global__ __launch_bounds__(64 * NW) void row_gemv_long_kernel(RowGemvAr
 // ---------------------------------------------------------------------------
 static constexpr int FUSED_NW = 8;
 
-static bool fused_type(uint32_t t) { return t == CERA_HIP_Q4_K || t == CERA_HIP_Q6_K; }
-// rows that fit one wavefront of 64-weight units, whole super-blocks
-static bool fused_k(uint64_t k) { return k % 256 == 0 && k <= 4096 && k > 0; }
+static bool kquant_type(uint32_t t) { return t == CERA_HIP_Q4_K || t == CERA_HIP_Q6_K; }
+static bool block32_type(uint32_t t) { return t == CERA_HIP_Q4_0 || t == CERA_HIP_Q8_0; }
+static bool fused_type(uint32_t t) { return kquant_type(t) || block32_type(t); }
+static uint32_t unit_elems(uint32_t t) { return kquant_type(t) ? 64 : 32; }
+// Passes of 64 units a row of k weights of this type takes in the one-wavefront-per-row kernels
+// (0: the type or the row length has no such kernel).
+static uint32_t row_tiles(uint32_t type, uint64_t k) {
+    if (!fused_type(type) || k == 0 || k % (kquant_type(type) ? 256 : 32)) return 0;
+    return static_cast<uint32_t>((k / unit_elems(type) + 63) / 64);
+}
+// rows short enough for the kernels that keep a row's activations in registers
+static uint32_t short_tiles(uint32_t type, uint64_t k) {
+    const uint32_t t = k <= 4096 ? row_tiles(type, k) : 0;
+    return t <= (kquant_type(type) ? 1u : 2u) ? t : 0;
+}
 
 static void fill(RowGemvArgs& a, const cera_hip_dtensor* w, const cera_hip_dtensor* w2, uint32_t rows_per_wave, bool stream = false) {
     a = RowGemvArgs{};
@@ -323,11 +355,16 @@ static __global__ __launch_bounds__(256) void stream_rows_kernel(const uint8_t* 
 // route).  Other types and views are left alone.
 cera_hip_status cera_tensor_prepare_stream(cera_hip_ctx* ctx, cera_hip_dtensor* w) {
     if (!ctx->decode_copies) return CERA_HIP_OK;
-    if (!w || w->dev_stream || !w->owns || !fused_type(w->dtype) || w->k == 0 || w->k > 16384 || w->m == 0 || w->m > 0x7FFFFFFFull) return CERA_HIP_OK;
+    if (!w || w->dev_stream || !w->owns || w->k > 16384 || w->m == 0 || w->m > 0x7FFFFFFFull) return CERA_HIP_OK;
+    if (row_tiles(w->dtype, w->k) == 0 || (reinterpret_cast<uintptr_t>(w->dev) & 15)) return CERA_HIP_OK;
     const uint32_t k = static_cast<uint32_t>(w->k);
-    const bool q4 = w->dtype == CERA_HIP_Q4_K;
-    if (k % 256 || (reinterpret_cast<uintptr_t>(w->dev) & 15)) return CERA_HIP_OK;
-    const uint64_t srb = q4 ? Q4K::stream_row_bytes(k) : Q6K::stream_row_bytes(k);
+    uint64_t srb = 0;
+    switch (w->dtype) {
+        case CERA_HIP_Q4_K: srb = Q4K::stream_row_bytes(k); break;
+        case CERA_HIP_Q6_K: srb = Q6K::stream_row_bytes(k); break;
+        case CERA_HIP_Q4_0: srb = Q4_0::stream_row_bytes(k); break;
+        default: srb = Q8_0::stream_row_bytes(k); break;
+    }
     void* p = nullptr;
     const hipError_t e = hipMalloc(&p, srb * w->m);
     if (e != hipSuccess) {
@@ -337,10 +374,14 @@ cera_hip_status cera_tensor_prepare_stream(cera_hip_ctx* ctx, cera_hip_dtensor* 
         return cera_fail(ctx, CERA_HIP_ERR_DEVICE, std::string("hipMalloc(decode copy): ") + hipGetErrorString(e));
     }
     const dim3 grid(static_cast<uint32_t>(w->m)), block(256);
-    if (q4) hipLaunchKernelGGL(stream_rows_kernel<Q4K>, grid, block, 0, ctx->stream, w->dev, static_cast<uint8_t*>(p), grid.x, k / 64,
-                               static_cast<uint32_t>(w->row_bytes), static_cast<uint32_t>(srb));
-    else hipLaunchKernelGGL(stream_rows_kernel<Q6K>, grid, block, 0, ctx->stream, w->dev, static_cast<uint8_t*>(p), grid.x, k / 64,
-                            static_cast<uint32_t>(w->row_bytes), static_cast<uint32_t>(srb));
+    const uint32_t n_units = k / unit_elems(w->dtype), rb = static_cast<uint32_t>(w->row_bytes);
+    uint8_t* dst = static_cast<uint8_t*>(p);
+    switch (w->dtype) {
+        case CERA_HIP_Q4_K: hipLaunchKernelGGL(stream_rows_kernel<Q4K>, grid, block, 0, ctx->stream, w->dev, dst, grid.x, n_units, rb, static_cast<uint32_t>(srb)); break;
+        case CERA_HIP_Q6_K: hipLaunchKernelGGL(stream_rows_kernel<Q6K>, grid, block, 0, ctx->stream, w->dev, dst, grid.x, n_units, rb, static_cast<uint32_t>(srb)); break;
+        case CERA_HIP_Q4_0: hipLaunchKernelGGL(stream_rows_kernel<Q4_0>, grid, block, 0, ctx->stream, w->dev, dst, grid.x, n_units, rb, static_cast<uint32_t>(srb)); break;
+        default: hipLaunchKernelGGL(stream_rows_kernel<Q8_0>, grid, block, 0, ctx->stream, w->dev, dst, grid.x, n_units, rb, static_cast<uint32_t>(srb)); break;
+    }
     const hipError_t le = hipGetLastError();
     if (le != hipSuccess) {
         (void)hipFree(p);
@@ -361,8 +402,8 @@ cera_hip_status cera_launch_ffn_gate_up_fused(cera_hip_ctx* ctx, const cera_hip_
                                               const float* x, const float* norm_w, float eps, int8_t* out_q, float* out_s,
                                               bool* launched) {
     *launched = false;
-    if (gate->dtype != CERA_HIP_Q4_K || up->dtype != CERA_HIP_Q4_K || gate->m != up->m || gate->k != up->k || !fused_k(gate->k) ||
-        gate->m % 32)
+    const uint32_t tiles = short_tiles(gate->dtype, gate->k);
+    if (tiles == 0 || gate->dtype == CERA_HIP_Q6_K || up->dtype != gate->dtype || gate->m != up->m || gate->k != up->k || gate->m % 32)
         return CERA_HIP_OK;
     RowGemvArgs a;
     // 16 wavefronts x 4 rows: a workgroup owns two Q8_0 blocks of the output, and 14336 rows make
@@ -373,8 +414,21 @@ cera_hip_status cera_launch_ffn_gate_up_fused(cera_hip_ctx* ctx, const cera_hip_
     fill(a, gate, up, ROWS, stream);
     a.x = x; a.norm_w = norm_w; a.eps = eps; a.out_q = out_q; a.out_s = out_s;
     const dim3 grid((a.m + GATE_UP_NW * ROWS - 1) / (GATE_UP_NW * ROWS)), block(64 * GATE_UP_NW);
-    if (stream) hipLaunchKernelGGL((row_gemv_kernel<Q4K, GATE_UP_NW, ROWS, true, FEPI_SILU_Q8, true>), grid, block, 0, ctx->stream, a);
-    else hipLaunchKernelGGL((row_gemv_kernel<Q4K, GATE_UP_NW, ROWS, true, FEPI_SILU_Q8, false>), grid, block, 0, ctx->stream, a);
+#define GATE_UP_LAUNCH(TT, TL)                                                                                                          \
+    do {                                                                                                                                \
+        if (stream) hipLaunchKernelGGL((row_gemv_kernel<TT, GATE_UP_NW, ROWS, true, FEPI_SILU_Q8, true, TL>), grid, block, 0, ctx->stream, a); \
+        else hipLaunchKernelGGL((row_gemv_kernel<TT, GATE_UP_NW, ROWS, true, FEPI_SILU_Q8, false, TL>), grid, block, 0, ctx->stream, a);   \
+    } while (0)
+#define GATE_UP_LAUNCH_B32(TT)            \
+    do {                                  \
+        if (tiles == 1) GATE_UP_LAUNCH(TT, 1); \
+        else GATE_UP_LAUNCH(TT, 2);       \
+    } while (0)
+    if (gate->dtype == CERA_HIP_Q4_K) GATE_UP_LAUNCH(Q4K, 1);
+    else if (gate->dtype == CERA_HIP_Q4_0) GATE_UP_LAUNCH_B32(Q4_0);
+    else GATE_UP_LAUNCH_B32(Q8_0);
+#undef GATE_UP_LAUNCH_B32
+#undef GATE_UP_LAUNCH
     HIP_TRY(ctx, hipGetLastError());
     *launched = true;
     return CERA_HIP_OK;
@@ -384,7 +438,11 @@ cera_hip_status cera_launch_ffn_gate_up_fused(cera_hip_ctx* ctx, const cera_hip_
 cera_hip_status cera_launch_qkv_fused(cera_hip_ctx* ctx, const cera_hip_dtensor* wa, const cera_hip_dtensor* wb, const float* x,
                                       const float* norm_w, float eps, float* ya, float* yb, bool* launched) {
     *launched = false;
-    if (!fused_type(wa->dtype) || !fused_k(wa->k) || (wb && (!fused_type(wb->dtype) || wb->k != wa->k))) return CERA_HIP_OK;
+    const uint32_t tiles = short_tiles(wa->dtype, wa->k);
+    if (tiles == 0 || (wb && (wb->k != wa->k || short_tiles(wb->dtype, wb->k) != tiles))) return CERA_HIP_OK;
+    // the 32-weight-block types pair with their own kind only
+    if (wb && block32_type(wa->dtype) != block32_type(wb->dtype)) return CERA_HIP_OK;
+    if (wb && block32_type(wa->dtype) && wb->dtype != wa->dtype) return CERA_HIP_OK;
     // two rows per wavefront (12 wavefronts per CU on the 8B shapes), one for short matrices
     const uint64_t rows = wa->m + (wb ? wb->m : 0);
     const uint32_t rpw = rows >= static_cast<uint64_t>(ctx->n_cu) * 8 ? 2 : 1;
@@ -403,20 +461,28 @@ cera_hip_status cera_launch_qkv_fused(cera_hip_ctx* ctx, const cera_hip_dtensor*
     }
     const dim3 grid(n_blocks), block(64 * FUSED_NW);
     const uint32_t ta = wa->dtype, tb = wb ? wb->dtype : wa->dtype;
-#define QKV_LAUNCH_S(TA_, TB_, ST_)                                                                                                \
-    do {                                                                                                                           \
-        if (rpw == 2) hipLaunchKernelGGL((row_gemv_pair_kernel<TA_, TB_, FUSED_NW, 2, true, ST_>), grid, block, 0, ctx->stream, p); \
-        else hipLaunchKernelGGL((row_gemv_pair_kernel<TA_, TB_, FUSED_NW, 1, true, ST_>), grid, block, 0, ctx->stream, p);          \
+#define QKV_LAUNCH_S(TA_, TB_, ST_, TL_)                                                                                                \
+    do {                                                                                                                                \
+        if (rpw == 2) hipLaunchKernelGGL((row_gemv_pair_kernel<TA_, TB_, FUSED_NW, 2, true, ST_, TL_>), grid, block, 0, ctx->stream, p); \
+        else hipLaunchKernelGGL((row_gemv_pair_kernel<TA_, TB_, FUSED_NW, 1, true, ST_, TL_>), grid, block, 0, ctx->stream, p);          \
     } while (0)
-#define QKV_LAUNCH(TA_, TB_)                    \
-    do {                                        \
-        if (stream) QKV_LAUNCH_S(TA_, TB_, true); \
-        else QKV_LAUNCH_S(TA_, TB_, false);     \
+#define QKV_LAUNCH(TA_, TB_, TL_)                    \
+    do {                                             \
+        if (stream) QKV_LAUNCH_S(TA_, TB_, true, TL_); \
+        else QKV_LAUNCH_S(TA_, TB_, false, TL_);     \
     } while (0)
-    if (ta == CERA_HIP_Q4_K && tb == CERA_HIP_Q6_K) QKV_LAUNCH(Q4K, Q6K);
-    else if (ta == CERA_HIP_Q4_K && tb == CERA_HIP_Q4_K) QKV_LAUNCH(Q4K, Q4K);
-    else if (ta == CERA_HIP_Q6_K && tb == CERA_HIP_Q6_K) QKV_LAUNCH(Q6K, Q6K);
-    else QKV_LAUNCH(Q6K, Q4K);
+#define QKV_LAUNCH_B32(TT)                  \
+    do {                                    \
+        if (tiles == 1) QKV_LAUNCH(TT, TT, 1); \
+        else QKV_LAUNCH(TT, TT, 2);         \
+    } while (0)
+    if (ta == CERA_HIP_Q4_0) QKV_LAUNCH_B32(Q4_0);
+    else if (ta == CERA_HIP_Q8_0) QKV_LAUNCH_B32(Q8_0);
+    else if (ta == CERA_HIP_Q4_K && tb == CERA_HIP_Q6_K) QKV_LAUNCH(Q4K, Q6K, 1);
+    else if (ta == CERA_HIP_Q4_K && tb == CERA_HIP_Q4_K) QKV_LAUNCH(Q4K, Q4K, 1);
+    else if (ta == CERA_HIP_Q6_K && tb == CERA_HIP_Q6_K) QKV_LAUNCH(Q6K, Q6K, 1);
+    else QKV_LAUNCH(Q6K, Q4K, 1);
+#undef QKV_LAUNCH_B32
 #undef QKV_LAUNCH
 #undef QKV_LAUNCH_S
     HIP_TRY(ctx, hipGetLastError());
@@ -430,20 +496,29 @@ cera_hip_status cera_launch_qkv_fused(cera_hip_ctx* ctx, const cera_hip_dtensor*
 cera_hip_status cera_launch_row_gemv_add(cera_hip_ctx* ctx, const cera_hip_dtensor* w, const float* xs, const int8_t* xq,
                                          float* y, const float* resid, bool* launched) {
     *launched = false;
-    if (!fused_type(w->dtype) || !fused_k(w->k) || !resid || w->m > 65535) return CERA_HIP_OK;
+    const uint32_t tiles = short_tiles(w->dtype, w->k);
+    if (tiles == 0 || !resid || w->m > 65535) return CERA_HIP_OK;
     constexpr int NW = 4, ROWS = 2;
     RowGemvArgs a;
     const bool stream = w->dev_stream != nullptr;
     fill(a, w, nullptr, ROWS, stream);
     a.xq = xq; a.xs = xs; a.y = y; a.resid = resid;
     const dim3 grid((a.m + NW * ROWS - 1) / (NW * ROWS)), block(64 * NW);
-#define ADD_LAUNCH(TT)                                                                                                     \
-    do {                                                                                                                   \
-        if (stream) hipLaunchKernelGGL((row_gemv_kernel<TT, NW, ROWS, false, FEPI_ADD, true>), grid, block, 0, ctx->stream, a); \
-        else hipLaunchKernelGGL((row_gemv_kernel<TT, NW, ROWS, false, FEPI_ADD, false>), grid, block, 0, ctx->stream, a);    \
+#define ADD_LAUNCH(TT, TL)                                                                                                     \
+    do {                                                                                                                       \
+        if (stream) hipLaunchKernelGGL((row_gemv_kernel<TT, NW, ROWS, false, FEPI_ADD, true, TL>), grid, block, 0, ctx->stream, a); \
+        else hipLaunchKernelGGL((row_gemv_kernel<TT, NW, ROWS, false, FEPI_ADD, false, TL>), grid, block, 0, ctx->stream, a);    \
     } while (0)
-    if (w->dtype == CERA_HIP_Q4_K) ADD_LAUNCH(Q4K);
-    else ADD_LAUNCH(Q6K);
+#define ADD_LAUNCH_B32(TT)            \
+    do {                              \
+        if (tiles == 1) ADD_LAUNCH(TT, 1); \
+        else ADD_LAUNCH(TT, 2);       \
+    } while (0)
+    if (w->dtype == CERA_HIP_Q4_K) ADD_LAUNCH(Q4K, 1);
+    else if (w->dtype == CERA_HIP_Q6_K) ADD_LAUNCH(Q6K, 1);
+    else if (w->dtype == CERA_HIP_Q4_0) ADD_LAUNCH_B32(Q4_0);
+    else ADD_LAUNCH_B32(Q8_0);
+#undef ADD_LAUNCH_B32
 #undef ADD_LAUNCH
     HIP_TRY(ctx, hipGetLastError());
     *launched = true;
@@ -457,14 +532,21 @@ cera_hip_status cera_launch_row_gemv_add(cera_hip_ctx* ctx, const cera_hip_dtens
 cera_hip_status cera_launch_row_gemv_store(cera_hip_ctx* ctx, const cera_hip_dtensor* w, const float* xs, const int8_t* xq,
                                            float* y, bool* launched) {
     *launched = false;
-    if (!fused_type(w->dtype) || !fused_k(w->k) || !w->dev_stream || w->m > (1u << 24)) return CERA_HIP_OK;
+    const uint32_t tiles = short_tiles(w->dtype, w->k);
+    if (tiles == 0 || !w->dev_stream || w->m > (1u << 24)) return CERA_HIP_OK;
     constexpr int NW = 4, ROWS = 2;   // four rows per wavefront measured the same
     RowGemvArgs a;
     fill(a, w, nullptr, ROWS, true);
     a.xq = xq; a.xs = xs; a.y = y;
     const dim3 grid((a.m + NW * ROWS - 1) / (NW * ROWS)), block(64 * NW);
-    if (w->dtype == CERA_HIP_Q4_K) hipLaunchKernelGGL((row_gemv_kernel<Q4K, NW, ROWS, false, FEPI_STORE, true>), grid, block, 0, ctx->stream, a);
-    else hipLaunchKernelGGL((row_gemv_kernel<Q6K, NW, ROWS, false, FEPI_STORE, true>), grid, block, 0, ctx->stream, a);
+#define STORE_LAUNCH(TT, TL) hipLaunchKernelGGL((row_gemv_kernel<TT, NW, ROWS, false, FEPI_STORE, true, TL>), grid, block, 0, ctx->stream, a)
+    if (w->dtype == CERA_HIP_Q4_K) STORE_LAUNCH(Q4K, 1);
+    else if (w->dtype == CERA_HIP_Q6_K) STORE_LAUNCH(Q6K, 1);
+    else if (w->dtype == CERA_HIP_Q4_0 && tiles == 1) STORE_LAUNCH(Q4_0, 1);
+    else if (w->dtype == CERA_HIP_Q4_0) STORE_LAUNCH(Q4_0, 2);
+    else if (tiles == 1) STORE_LAUNCH(Q8_0, 1);
+    else STORE_LAUNCH(Q8_0, 2);
+#undef STORE_LAUNCH
     HIP_TRY(ctx, hipGetLastError());
     *launched = true;
     return CERA_HIP_OK;
@@ -475,7 +557,9 @@ cera_hip_status cera_launch_row_gemv_store(cera_hip_ctx* ctx, const cera_hip_dte
 cera_hip_status cera_launch_row_gemv_long_add(cera_hip_ctx* ctx, const cera_hip_dtensor* w, const float* xs, const int8_t* xq,
                                               float* y, const float* resid, bool* launched) {
     *launched = false;
-    if (!fused_type(w->dtype) || w->k % 256 || w->k <= 4096 || w->k > 16384 || !resid || w->m > (1u << 20)) return CERA_HIP_OK;
+    const uint32_t tiles = row_tiles(w->dtype, w->k);
+    const bool b32 = block32_type(w->dtype);
+    if (tiles == 0 || short_tiles(w->dtype, w->k) != 0 || tiles > (b32 ? 8u : 4u) || !resid || w->m > (1u << 20)) return CERA_HIP_OK;
     // four rows per workgroup: small workgroups start and retire independently, which measured
     // faster end to end than 8 or 16 rows sharing one staged copy of the activations
     constexpr int NW = 4;
@@ -483,7 +567,6 @@ cera_hip_status cera_launch_row_gemv_long_add(cera_hip_ctx* ctx, const cera_hip_
     const bool stream = w->dev_stream != nullptr;
     fill(a, w, nullptr, 1, stream);
     a.xq = xq; a.xs = xs; a.y = y; a.resid = resid;
-    const uint32_t tiles = static_cast<uint32_t>((w->k / 64 + 63) / 64);   // both types: 64 weights per unit
     const dim3 grid((a.m + NW - 1) / NW), block(64 * NW);
 #define LONG_LAUNCH_S(TT, ST_)                                                                                                 \
     do {                                                                                                                       \
@@ -496,8 +579,19 @@ cera_hip_status cera_launch_row_gemv_long_add(cera_hip_ctx* ctx, const cera_hip_
         if (stream) LONG_LAUNCH_S(TT, true); \
         else LONG_LAUNCH_S(TT, false);       \
     } while (0)
+    // the 32-weight-block types take 4 or 8 passes (a surplus pass re-reads unit 0 against zeroed activations)
+#define LONG_LAUNCH_B32(TT)                                                                                                     \
+    do {                                                                                                                        \
+        if (tiles <= 4 && stream) hipLaunchKernelGGL((row_gemv_long_kernel<TT, NW, 4, FEPI_ADD, true>), grid, block, 0, ctx->stream, a);  \
+        else if (tiles <= 4) hipLaunchKernelGGL((row_gemv_long_kernel<TT, NW, 4, FEPI_ADD, false>), grid, block, 0, ctx->stream, a);      \
+        else if (stream) hipLaunchKernelGGL((row_gemv_long_kernel<TT, NW, 8, FEPI_ADD, true>), grid, block, 0, ctx->stream, a);           \
+        else hipLaunchKernelGGL((row_gemv_long_kernel<TT, NW, 8, FEPI_ADD, false>), grid, block, 0, ctx->stream, a);                      \
+    } while (0)
     if (w->dtype == CERA_HIP_Q4_K) LONG_LAUNCH(Q4K);
-    else LONG_LAUNCH(Q6K);
+    else if (w->dtype == CERA_HIP_Q6_K) LONG_LAUNCH(Q6K);
+    else if (w->dtype == CERA_HIP_Q4_0) LONG_LAUNCH_B32(Q4_0);
+    else LONG_LAUNCH_B32(Q8_0);
+#undef LONG_LAUNCH_B32
 #undef LONG_LAUNCH
 #undef LONG_LAUNCH_S
     HIP_TRY(ctx, hipGetLastError());

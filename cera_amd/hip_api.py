@@ -381,9 +381,9 @@ class Context:
                                                 n_queries, scale, n_splits, _p(out)))
         return out.reshape(n_queries, n_heads * head_dim)
 
-    def ffn_gate_up_fused(self, w_gate, w_up, m, k, x, norm_w, eps):
+    def ffn_gate_up_fused(self, w_gate, w_up, m, k, x, norm_w, eps, ggml_type: int = Q4_K):
         """Q8_0(silu(gate.n) * (up.n)), n = Q8_0(rmsnorm(x, norm_w)): (quants [m], scales [m/32])."""
-        tg, tu = make_tensor(Q4_K, m, k, w_gate), make_tensor(Q4_K, m, k, w_up)
+        tg, tu = make_tensor(ggml_type, m, k, w_gate), make_tensor(ggml_type, m, k, w_up)
         x = np.ascontiguousarray(x, np.float32); nw = np.ascontiguousarray(norm_w, np.float32)
         q, sc = np.empty(m, np.int8), np.empty(m // 32, np.float32)
         self.check(self.lib.cera_hip_ffn_gate_up_fused(self.h, C.byref(tg), C.byref(tu), _p(x), _p(nw), eps, _p(q), _p(sc)))

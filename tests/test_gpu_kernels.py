@@ -617,7 +617,10 @@ def no_decode_copies(hip):
 @pytest.mark.parametrize("dtype,m,k", [(Q6_K, 1024, 14336), (Q4_K, 512, 14336), (Q6_K, 77, 8192), (Q4_K, 100, 6144), (Q4_K, 130, 16384),
                                        (Q4_K, 1030, 4096), (Q6_K, 130, 4096), (Q6_K, 40, 2048), (Q4_K, 33, 1024),
                                        (Q4_K, 70, 3584), (Q6_K, 50, 11008), (Q4_K, 64, 5120), (Q6_K, 40, 256), (Q4_K, 9, 256),
-                                       (Q6_K, 35, 3584), (Q4_K, 48, 11008)])
+                                       (Q6_K, 35, 3584), (Q4_K, 48, 11008),
+                                       (Q4_0, 1030, 4096), (Q8_0, 130, 4096), (Q4_0, 70, 2048), (Q8_0, 33, 1024), (Q4_0, 9, 32),
+                                       (Q4_0, 512, 14336), (Q8_0, 200, 14336), (Q4_0, 64, 8192), (Q8_0, 40, 6144), (Q4_0, 50, 11008),
+                                       (Q8_0, 24, 4128), (Q4_0, 24, 16384)])
 def test_residual_projection_streams_the_decode_copy_to_the_same_bits(hip, no_decode_copies, dtype, m, k):
     """A matrix's decode copy is a permutation of its bytes, read by the same arithmetic: the
     residual projections give identical bits with the copy (the default) and from the native
@@ -649,3 +652,30 @@ def test_fused_launches_stream_the_decode_copy_to_the_same_bits(hip, no_decode_c
     q0, sc0 = no_decode_copies(lambda: hip.ffn_gate_up_fused(wg, wu, 1024, k, x, nw, 1e-5))
     assert np.array_equal(ya.view(np.uint32), ya0.view(np.uint32)) and np.array_equal(yb.view(np.uint32), yb0.view(np.uint32))
     assert np.array_equal(q, q0) and np.array_equal(sc.view(np.uint32), sc0.view(np.uint32))
+
+
+@pytest.mark.parametrize("dtype,k", [(Q4_0, 4096), (Q8_0, 4096), (Q4_0, 2048), (Q8_0, 1536)])
+def test_fused_launches_for_the_32_block_types(hip, orc, no_decode_copies, dtype, k):
+    """Q4_0 and Q8_0 matrices take the same fused decode launches as the K-quants (a lane holds two
+    32-weight blocks of a 4096-wide row): Q|K|V with the norm inside and gate|up with norm, SwiGLU and
+    Q8_0 -- bitwise what the separate launches compute, with and without decode copies."""
+    _say(f"fused launches {util.NAMES[dtype]} k={k}")
+    m = 1024
+    wa, _ = util.make_weights(dtype, 1280, k, seed=101)
+    wg, _ = util.make_weights(dtype, m, k, seed=103)
+    wu, _ = util.make_weights(dtype, m, k, seed=104)
+    x = util.make_x(k, 105) * np.float32(1.3)
+    nw = (1.0 + 0.1 * util.make_x(k, 106)).astype(np.float32)
+    ya, _ = hip.qkv_fused(dtype, wa, 1280, None, None, None, k, x, nw, 1e-5)
+    q, sc = hip.ffn_gate_up_fused(wg, wu, m, k, x, nw, 1e-5, dtype)
+    n, _, _ = hip.rmsnorm_q8_0(x, nw, 1e-5)
+    assert np.array_equal(ya.view(np.uint32), hip.gemv(dtype, wa, n, 1280, k).view(np.uint32))
+    h = hip.silu_mul(hip.gemv(dtype, wg, n, m, k), hip.gemv(dtype, wu, n, m, k))
+    rs, rq = hip.quantize_q8_0(h)
+    assert np.array_equal(q, rq) and np.array_equal(sc.view(np.uint32), rs.view(np.uint32))
+    ya0, _ = no_decode_copies(lambda: hip.qkv_fused(dtype, wa, 1280, None, None, None, k, x, nw, 1e-5))
+    q0, sc0 = no_decode_copies(lambda: hip.ffn_gate_up_fused(wg, wu, m, k, x, nw, 1e-5, dtype))
+    assert np.array_equal(ya.view(np.uint32), ya0.view(np.uint32))
+    assert np.array_equal(q, q0) and np.array_equal(sc.view(np.uint32), sc0.view(np.uint32))
+    ref = orc.gemv(dtype, wa, orc.rmsnorm(x, nw, 1e-5), 1280, k)
+    assert np.abs(ya - ref).max() <= 1e-3 * util.rms(ref)
