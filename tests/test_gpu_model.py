@@ -510,3 +510,35 @@ def test_decode_copies_do_not_change_a_logit(hip):
     finally:
         with_copies.close()
         native.close()
+
+
+@pytest.mark.parametrize("wtype", ["q4_0", "q8_0"])
+def test_wide_32_block_model_decodes_through_the_fused_launches(hip, orc, wtype):
+    """A one-layer model of the 8B width whose matrices are all Q4_0 (or Q8_0): decode runs the six
+    fused launches with two blocks per lane (4096-wide rows) and four passes (the 8192-wide down
+    projection), over decode copies.  Logits against the oracle's per-token forward, and -- same
+    arithmetic -- bit-identical to the same model without decode copies."""
+    from cera_amd import host_api as H
+    t = H.Q4_0 if wtype == "q4_0" else H.Q8_0
+    cfg = dict(n_layers=1, hidden=4096, ffn=8192, n_heads=32, n_kv_heads=8, head_dim=128, vocab=512,
+               max_seq_len=32, rope_type=1, rope_theta=10000.0, rms_eps=1e-5)
+    weights = synth.make_llama(cfg, seed=99, sigma=0.02, type_of=lambda name: t, norm_jitter=0.1)
+    _say(f"model: one {wtype} layer at width 4096")
+    gm = hip_api.Model(hip, cfg, weights)
+    hip.set_decode_copies(False)
+    try:
+        native = hip_api.Model(hip, cfg, weights)
+    finally:
+        hip.set_decode_copies(True)
+    om = orc.Llama(cfg, weights)
+    try:
+        tok = 3
+        for pos in range(5):
+            lg, ln, lo = gm.forward(tok, pos), native.forward(tok, pos), om.forward(tok, pos)
+            assert np.array_equal(lg.view(np.uint32), ln.view(np.uint32)), pos
+            assert _cos(lg, lo) > 0.9999, (pos, _cos(lg, lo))
+            # re-quantization noise of the activations between the layers' matrices: the other model tests' bound
+            assert np.abs(lg - lo).max() <= 0.1 * util.rms(lo), (pos, float(np.abs(lg - lo).max()), util.rms(lo))
+            tok = int(np.argmax(lo))
+    finally:
+        gm.close(); native.close(); om.close()
