@@ -591,14 +591,6 @@ cera_hip_status cera_launch_argmax(cera_hip_ctx* ctx, const float* x, uint32_t n
     return CERA_HIP_OK;
 }
 
-cera_hip_status cera_launch_gemv_q5k_f32(cera_hip_ctx* ctx, const cera_hip_dtensor* w, const float* x, float* y) {
-    dim3 grid(static_cast<uint32_t>((w->m + 3) / 4));
-    hipLaunchKernelGGL(gemv_q5k_f32_kernel, grid, dim3(256), 0, ctx->stream, w->dev, x, y,
-                       static_cast<uint32_t>(w->m), static_cast<uint32_t>(w->k));
-    HIP_TRY(ctx, hipGetLastError());
-    return CERA_HIP_OK;
-}
-
 struct AttnLaunch {
     const float* q;
     uint32_t seq_len, max_seq;

@@ -141,14 +141,18 @@ def test_gemv_config2_head_rows_sampled(hip, orc):
 
 
 def test_gemv_q5k_f32_activation_path(hip, orc):
-    # Q5_K dots against unquantized f32 x on both sides (cpu.rs:1830-1854)
-    for m, k in [(9, 512), (64, 4096)]:
+    # Q5_K dots against unquantized f32 x on both sides (cpu.rs:1830-1854); row widths that take one,
+    # two and four wavefronts per row group, ragged row counts, and a row beyond the K split (20480)
+    for m, k in [(9, 512), (64, 4096), (1, 256), (131, 2048), (77, 8192), (100, 14336), (33, 11008), (5, 16384), (6, 20480)]:
         _say(f"gemv Q5_K m={m} k={k}")
-        w, _ = util.make_weights(Q5_K, m, k, seed=31)
+        w, _ = util.make_weights(Q5_K, m, k, seed=31 + m)
         x = util.make_x(k, 32)
         y = hip.gemv(Q5_K, w, x, m, k)
         ref = orc.gemv(Q5_K, w, x, m, k)
         assert np.abs(y.astype(np.float64) - ref).max() <= GEMV_TOL * util.rms(ref)
+        # and against the exact value: dequantized weights . x in f64
+        exact = util.dequant_np(Q5_K, w, m, k).astype(np.float64) @ x.astype(np.float64)
+        assert np.abs(y.astype(np.float64) - exact).max() <= GEMV_TOL * util.rms(exact)
 
 
 def test_gemv_weight_extremes(hip, orc):
