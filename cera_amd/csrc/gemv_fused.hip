@@ -311,7 +311,7 @@ static __global__ __launch_bounds__(64 * NW) void row_gemv_long_kernel(RowGemvAr
 static constexpr int FUSED_NW = 8;
 
 static bool kquant_type(uint32_t t) { return t == CERA_HIP_Q4_K || t == CERA_HIP_Q6_K; }
-static bool block32_type(uint32_t t) { return t == CERA_HIP_Q4_0 || t == CERA_HIP_Q8_0; }
+static bool block32_type(uint32_t t) { return t == CERA_HIP_Q4_0 || t == CERA_HIP_Q4_1 || t == CERA_HIP_Q8_0; }
 static bool fused_type(uint32_t t) { return kquant_type(t) || block32_type(t); }
 static uint32_t unit_elems(uint32_t t) { return kquant_type(t) ? 64 : 32; }
 // Passes of 64 units a row of k weights of this type takes in the one-wavefront-per-row kernels
@@ -363,6 +363,7 @@ cera_hip_status cera_tensor_prepare_stream(cera_hip_ctx* ctx, cera_hip_dtensor* 
         case CERA_HIP_Q4_K: srb = Q4K::stream_row_bytes(k); break;
         case CERA_HIP_Q6_K: srb = Q6K::stream_row_bytes(k); break;
         case CERA_HIP_Q4_0: srb = Q4_0::stream_row_bytes(k); break;
+        case CERA_HIP_Q4_1: srb = Q4_1::stream_row_bytes(k); break;
         default: srb = Q8_0::stream_row_bytes(k); break;
     }
     void* p = nullptr;
@@ -380,6 +381,7 @@ cera_hip_status cera_tensor_prepare_stream(cera_hip_ctx* ctx, cera_hip_dtensor* 
         case CERA_HIP_Q4_K: hipLaunchKernelGGL(stream_rows_kernel<Q4K>, grid, block, 0, ctx->stream, w->dev, dst, grid.x, n_units, rb, static_cast<uint32_t>(srb)); break;
         case CERA_HIP_Q6_K: hipLaunchKernelGGL(stream_rows_kernel<Q6K>, grid, block, 0, ctx->stream, w->dev, dst, grid.x, n_units, rb, static_cast<uint32_t>(srb)); break;
         case CERA_HIP_Q4_0: hipLaunchKernelGGL(stream_rows_kernel<Q4_0>, grid, block, 0, ctx->stream, w->dev, dst, grid.x, n_units, rb, static_cast<uint32_t>(srb)); break;
+        case CERA_HIP_Q4_1: hipLaunchKernelGGL(stream_rows_kernel<Q4_1>, grid, block, 0, ctx->stream, w->dev, dst, grid.x, n_units, rb, static_cast<uint32_t>(srb)); break;
         default: hipLaunchKernelGGL(stream_rows_kernel<Q8_0>, grid, block, 0, ctx->stream, w->dev, dst, grid.x, n_units, rb, static_cast<uint32_t>(srb)); break;
     }
     const hipError_t le = hipGetLastError();
@@ -426,6 +428,7 @@ cera_hip_status cera_launch_ffn_gate_up_fused(cera_hip_ctx* ctx, const cera_hip_
     } while (0)
     if (gate->dtype == CERA_HIP_Q4_K) GATE_UP_LAUNCH(Q4K, 1);
     else if (gate->dtype == CERA_HIP_Q4_0) GATE_UP_LAUNCH_B32(Q4_0);
+    else if (gate->dtype == CERA_HIP_Q4_1) GATE_UP_LAUNCH_B32(Q4_1);
     else GATE_UP_LAUNCH_B32(Q8_0);
 #undef GATE_UP_LAUNCH_B32
 #undef GATE_UP_LAUNCH
@@ -477,6 +480,7 @@ cera_hip_status cera_launch_qkv_fused(cera_hip_ctx* ctx, const cera_hip_dtensor*
         else QKV_LAUNCH(TT, TT, 2);         \
     } while (0)
     if (ta == CERA_HIP_Q4_0) QKV_LAUNCH_B32(Q4_0);
+    else if (ta == CERA_HIP_Q4_1) QKV_LAUNCH_B32(Q4_1);
     else if (ta == CERA_HIP_Q8_0) QKV_LAUNCH_B32(Q8_0);
     else if (ta == CERA_HIP_Q4_K && tb == CERA_HIP_Q6_K) QKV_LAUNCH(Q4K, Q6K, 1);
     else if (ta == CERA_HIP_Q4_K && tb == CERA_HIP_Q4_K) QKV_LAUNCH(Q4K, Q4K, 1);
@@ -517,6 +521,7 @@ cera_hip_status cera_launch_row_gemv_add(cera_hip_ctx* ctx, const cera_hip_dtens
     if (w->dtype == CERA_HIP_Q4_K) ADD_LAUNCH(Q4K, 1);
     else if (w->dtype == CERA_HIP_Q6_K) ADD_LAUNCH(Q6K, 1);
     else if (w->dtype == CERA_HIP_Q4_0) ADD_LAUNCH_B32(Q4_0);
+    else if (w->dtype == CERA_HIP_Q4_1) ADD_LAUNCH_B32(Q4_1);
     else ADD_LAUNCH_B32(Q8_0);
 #undef ADD_LAUNCH_B32
 #undef ADD_LAUNCH
@@ -544,6 +549,8 @@ cera_hip_status cera_launch_row_gemv_store(cera_hip_ctx* ctx, const cera_hip_dte
     else if (w->dtype == CERA_HIP_Q6_K) STORE_LAUNCH(Q6K, 1);
     else if (w->dtype == CERA_HIP_Q4_0 && tiles == 1) STORE_LAUNCH(Q4_0, 1);
     else if (w->dtype == CERA_HIP_Q4_0) STORE_LAUNCH(Q4_0, 2);
+    else if (w->dtype == CERA_HIP_Q4_1 && tiles == 1) STORE_LAUNCH(Q4_1, 1);
+    else if (w->dtype == CERA_HIP_Q4_1) STORE_LAUNCH(Q4_1, 2);
     else if (tiles == 1) STORE_LAUNCH(Q8_0, 1);
     else STORE_LAUNCH(Q8_0, 2);
 #undef STORE_LAUNCH
@@ -590,6 +597,7 @@ cera_hip_status cera_launch_row_gemv_long_add(cera_hip_ctx* ctx, const cera_hip_
     if (w->dtype == CERA_HIP_Q4_K) LONG_LAUNCH(Q4K);
     else if (w->dtype == CERA_HIP_Q6_K) LONG_LAUNCH(Q6K);
     else if (w->dtype == CERA_HIP_Q4_0) LONG_LAUNCH_B32(Q4_0);
+    else if (w->dtype == CERA_HIP_Q4_1) LONG_LAUNCH_B32(Q4_1);
     else LONG_LAUNCH_B32(Q8_0);
 #undef LONG_LAUNCH_B32
 #undef LONG_LAUNCH

@@ -102,7 +102,7 @@ CERA_HIP_API void cera_hip_ctx_destroy(cera_hip_ctx*);
 CERA_HIP_API const char* cera_hip_last_error(const cera_hip_ctx*);
 CERA_HIP_API cera_hip_status cera_hip_sync(cera_hip_ctx*);
 /* Decode copies (on by default).  When on, cera_hip_model_create and cera_hip_decode_ops_dev give
- * every Q4_K / Q6_K / Q4_0 / Q8_0 projection matrix (k at most 16384) a second copy of
+ * every Q4_K / Q6_K / Q4_0 / Q4_1 / Q8_0 projection matrix (k at most 16384) a second copy of
  * about the same size in which each row's bytes are permuted so that the decode GEMV kernels read
  * it in whole 128-byte lines with non-temporal loads (+6 % decode rate on the 8B model for about
  * twice those matrices' memory); every other reader keeps the native GGUF bytes.  Results are

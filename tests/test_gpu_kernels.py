@@ -624,7 +624,8 @@ def no_decode_copies(hip):
                                        (Q6_K, 35, 3584), (Q4_K, 48, 11008),
                                        (Q4_0, 1030, 4096), (Q8_0, 130, 4096), (Q4_0, 70, 2048), (Q8_0, 33, 1024), (Q4_0, 9, 32),
                                        (Q4_0, 512, 14336), (Q8_0, 200, 14336), (Q4_0, 64, 8192), (Q8_0, 40, 6144), (Q4_0, 50, 11008),
-                                       (Q8_0, 24, 4128), (Q4_0, 24, 16384)])
+                                       (Q8_0, 24, 4128), (Q4_0, 24, 16384),
+                                       (Q4_1, 130, 4096), (Q4_1, 70, 2048), (Q4_1, 64, 14336), (Q4_1, 40, 6144), (Q4_1, 9, 96)])
 def test_residual_projection_streams_the_decode_copy_to_the_same_bits(hip, no_decode_copies, dtype, m, k):
     """A matrix's decode copy is a permutation of its bytes, read by the same arithmetic: the
     residual projections give identical bits with the copy (the default) and from the native
@@ -658,9 +659,9 @@ def test_fused_launches_stream_the_decode_copy_to_the_same_bits(hip, no_decode_c
     assert np.array_equal(q, q0) and np.array_equal(sc.view(np.uint32), sc0.view(np.uint32))
 
 
-@pytest.mark.parametrize("dtype,k", [(Q4_0, 4096), (Q8_0, 4096), (Q4_0, 2048), (Q8_0, 1536)])
+@pytest.mark.parametrize("dtype,k", [(Q4_0, 4096), (Q8_0, 4096), (Q4_0, 2048), (Q8_0, 1536), (Q4_1, 4096), (Q4_1, 1024)])
 def test_fused_launches_for_the_32_block_types(hip, orc, no_decode_copies, dtype, k):
-    """Q4_0 and Q8_0 matrices take the same fused decode launches as the K-quants (a lane holds two
+    """Q4_0, Q4_1 and Q8_0 matrices take the same fused decode launches as the K-quants (a lane holds two
     32-weight blocks of a 4096-wide row): Q|K|V with the norm inside and gate|up with norm, SwiGLU and
     Q8_0 -- bitwise what the separate launches compute, with and without decode copies."""
     _say(f"fused launches {util.NAMES[dtype]} k={k}")
