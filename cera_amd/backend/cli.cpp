@@ -77,17 +77,16 @@ int cmd_gen(const Args& a) {
     c.type_token_embd = CERA_TYPE_Q4_K; c.type_output = CERA_TYPE_Q6_K;
     c.type_attn_q = c.type_attn_k = c.type_attn_output = c.type_ffn_gate = c.type_ffn_up = CERA_TYPE_Q4_K;
     c.type_attn_v = c.type_ffn_down = CERA_TYPE_Q6_K;
-    // --quant q5_k_m: Q5_K in place of Q4_K; q4_0 | q8_0 | q4_1: every matrix in that 32-block type (the head stays Q6_K as llama.cpp's
-    // converters leave it for q4_0 / q4_1, and follows for q8_0)
+    // --quant q5_k_m: Q5_K in place of Q4_K; q4_0 | q8_0: every matrix in that 32-block type (the head stays Q6_K as
+    // llama.cpp's converters leave it for q4_0, and follows for q8_0)
     const std::string quant = a.str("quant", "q4_k_m");
     if (quant == "q5_k_m") {   // Q5_K where Q4_K_M has Q4_K
         c.type_token_embd = c.type_attn_q = c.type_attn_k = c.type_attn_output = c.type_ffn_gate = c.type_ffn_up = CERA_TYPE_Q5_K;
     } else if (quant != "q4_k_m") {
         int t;
         if (quant == "q4_0") t = CERA_TYPE_Q4_0;
-        else if (quant == "q4_1") t = CERA_TYPE_Q4_1;
         else if (quant == "q8_0") t = CERA_TYPE_Q8_0;
-        else { std::fprintf(stderr, "gen: --quant must be q4_k_m, q5_k_m, q4_0, q4_1 or q8_0\n"); return 2; }
+        else { std::fprintf(stderr, "gen: --quant must be q4_k_m, q5_k_m, q4_0 or q8_0\n"); return 2; }
         c.type_token_embd = c.type_attn_q = c.type_attn_k = c.type_attn_v = c.type_attn_output = t;
         c.type_ffn_gate = c.type_ffn_up = c.type_ffn_down = t;
         if (quant == "q8_0") c.type_output = t;
