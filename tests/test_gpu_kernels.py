@@ -251,7 +251,7 @@ def test_dequantize_row_bit_exact(hip, orc, dtype):
 
 
 # ---- decode attention ----------------------------------------------------------------
-@pytest.mark.parametrize("L", [1, 2, 63, 64, 65, 512, 1000, 4096])
+@pytest.mark.parametrize("L", [1, 2, 63, 64, 65, 512, 1000, 4096, 2560, 5120, 10240, 12289, 16384, 20481])
 def test_attn_decode_vs_oracle(hip, orc, L):
     nh, nkv, hd = 32, 8, 128
     _say(f"attn_decode L={L}")
