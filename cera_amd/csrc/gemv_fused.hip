@@ -347,7 +347,7 @@ static __global__ __launch_bounds__(256) void stream_rows_kernel(const uint8_t* 
         T::to_stream(src + static_cast<uint64_t>(row) * row_bytes, dst + static_cast<uint64_t>(row) * stream_row_bytes, u, n_units);
 }
 
-// Gives a Q4_K / Q6_K matrix its decode copy (a second allocation of about the same size, kept
+// Gives a Q4_K / Q6_K / Q4_0 / Q4_1 / Q8_0 matrix its decode copy (a second allocation of about the same size, kept
 // until the tensor is freed): the per-row permutation that lets the one-wavefront-per-row
 // kernels stream it with non-temporal loads.  A load-time re-layout for the kernel that reads
 // it, as the reference's own x86 path does with repack_q4_k_8x8 (cera/src/backend/cpu.rs:1282-1358);
