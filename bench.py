@@ -34,7 +34,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 # each scaled by what the same counter reads for this library's 1 GiB copy kernel; the two passes run
 # `bench.py --pmc-probe` under rocprofv3 --pmc, summary in profiles/gemv_q4k_gate_up_hbm_traffic_pmc.txt).
 # It is a recorded measurement of this kernel configuration, not taken live: counters need the profiler.
-GATE_UP_TRAFFIC_BYTES = 66_478_845
+GATE_UP_TRAFFIC_BYTES = 66_481_099
 GATE_UP_KERNEL = "row_gemv_kernel<Q4K,16,4,true,2,true,1>"
 
 # (name, ggml type name, m, k, copies per step)
@@ -252,8 +252,9 @@ def main() -> int:
     ap.add_argument("--no-e2e", action="store_true", help="skip the end-to-end model run (prefill 512 + greedy 256)")
     ap.add_argument("--no-extras", action="store_true", help="skip the flash-decode and prefill-GEMM side measurements")
     ap.add_argument("--pmc-probe", action="store_true",
-                    help="run only a 1 GiB copy kernel, a few launches of each per-layer GEMV kernel and the two "
-                         "prefill GEMMs at 2048 tokens, for a hardware-counter pass under rocprofv3 --pmc; prints no JSON")
+                    help="run only a 1 GiB copy kernel, a few launches of each per-layer GEMV kernel, decode attention at "
+                         "131072 and 8192 keys and the two prefill GEMMs at 2048 tokens, for a hardware-counter pass under "
+                         "rocprofv3 --pmc; prints no JSON")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the hot path has no multi-GPU part); "
@@ -383,6 +384,18 @@ def main() -> int:
         for _ in range(2):
             for g in ("ffn_gate_up", "ffn_down", "attn_qkv", "attn_output"):
                 run(groups[g])
+        # decode attention, 32/8/128 heads, f32 cache (the values do not matter to the counters): 131072 keys take
+        # one wavefront per head group and non-temporal reads, 8192 keys two wavefronts per group and cached reads
+        import ctypes as C
+        kv_b = 8 * 131072 * 128 * 4
+        dkp, dvp = ctx.malloc(kv_b), ctx.malloc(kv_b)
+        dqp, dop = ctx.to_device(rng.standard_normal(32 * 128, dtype=np.float32)), ctx.malloc(32 * 128 * 4)
+        for L in (131072, 8192):
+            for _ in range(4):
+                ctx.check(ctx.lib.cera_hip_attn_decode_dev(ctx.h, dqp, dkp, dvp, 32, 8, 128, L, L, C.c_float(1.0 / np.sqrt(128.0)), 0, dop))
+        ctx.sync()
+        for d in (dkp, dvp, dqp, dop):
+            ctx.free(d)
         # the prefill GEMMs at 2048 tokens: Q4_K gate (int8 matrix core) and Q6_K down (f16 matrix core)
         m_tok = 2048
         for name in ("ffn_gate", "ffn_down"):
