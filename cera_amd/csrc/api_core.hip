@@ -596,7 +596,7 @@ struct AttnLaunch {
     uint32_t seq_len, max_seq;
     float scale;
     uint32_t n_heads, n_kv_heads, n_queries, q_stride, G, S, n_parts, part_keys, chunks_per_part;
-    bool batch, fused_new_kv;
+    bool batch, fused_new_kv, split_heads;
     AttnNewKV nk;
     float *acc, *ml;   // split-K partials: (o) and (m, l) per (query, head, part)
 };
@@ -604,7 +604,10 @@ struct AttnLaunch {
 // G = heads per wavefront; a.G = heads per kv head (G or 2 G)
 template <int G, typename KV, int HD>
 static void attn_launch_decode_g(cera_hip_ctx* ctx, const AttnLaunch& a, const KV* kc, const KV* vc) {
-    const dim3 grid((a.n_parts + 3) / 4, a.n_kv_heads * (a.G / G), a.n_queries), block(256);
+    // a workgroup is four wavefronts = four consecutive parts of one (kv head, sub-group, query);
+    // the kernel maps launch indices to them XCD by XCD, so the count is rounded up to whole eights
+    const uint32_t groups = (a.n_parts + 3) / 4 * a.n_kv_heads, reps = (a.G / G) * a.n_queries;
+    const dim3 grid((groups + 7) / 8 * 8 * reps), block(256);
     // one query and one wavefront per kv head and key range: every K/V row is read exactly once,
     // which is what the non-temporal instances want (long chunks only: short ones prefetch V
     // with K and are latency-bound)
@@ -614,11 +617,11 @@ static void attn_launch_decode_g(cera_hip_ctx* ctx, const AttnLaunch& a, const K
         if (a.fused_new_kv)                                                                                          \
             hipLaunchKernelGGL((attn_decode_partial_kernel<G, SS, true, KV, HD, NT>), grid, block, 0, ctx->stream, a.q,  \
                                kc, vc, a.seq_len, a.max_seq, a.scale, a.chunks_per_part, a.n_parts, a.q_stride, a.G, \
-                               a.acc, a.ml, a.nk);                                                                   \
+                               a.n_kv_heads, a.n_queries, a.acc, a.ml, a.nk);                                        \
         else                                                                                                         \
             hipLaunchKernelGGL((attn_decode_partial_kernel<G, SS, false, KV, HD, NT>), grid, block, 0, ctx->stream, a.q, \
                                kc, vc, a.seq_len, a.max_seq, a.scale, a.chunks_per_part, a.n_parts, a.q_stride, a.G, \
-                               a.acc, a.ml, a.nk);                                                                   \
+                               a.n_kv_heads, a.n_queries, a.acc, a.ml, a.nk);                                        \
     } while (0)
 #define ATTN_LAUNCH_S(SS) ATTN_LAUNCH_SN(SS, false)
     switch (a.S) {
@@ -656,12 +659,14 @@ static void attn_launch_partials(cera_hip_ctx* ctx, const AttnLaunch& a, const K
     }
     // A wavefront's time is largely its own instruction stream, which grows with the heads it
     // serves, so groups of 4 and 8 heads are split over two wavefronts (the K/V rows both read come
-    // from cache the second time): 580 -> 590 tok/s on the 8B model at ~640 keys, 5-15 % per call
-    // from 1k to 16k keys.  One head per wavefront gains nothing over two.  From 16k keys on the
-    // kernel is bound by bytes: a group keeps one wavefront, every K/V row is then read exactly
-    // once and the loads carry the non-temporal hint (131072 keys: 5.50 TB/s split, 5.85 unsplit,
-    // 6.42 unsplit and non-temporal; 16384 keys: the same time either way).
-    const bool split_heads = a.G >= 4 && a.seq_len < 16384;
+    // from cache the second time: the kernel places them on one XCD): 580 -> 590 tok/s on the 8B
+    // model at ~640 keys, 5-15 % per call from 1k to 16k keys.  One head per wavefront gains nothing
+    // over two.  From 16k keys on an f32 cache is bound by bytes: a group keeps one wavefront, every
+    // K/V row is then read exactly once and the loads carry the non-temporal hint (131072 keys:
+    // 5.50 TB/s split, 5.85 unsplit, 6.42 unsplit and non-temporal; 16384 keys: the same time either
+    // way).  An f16 cache moves half the bytes for the same arithmetic and keeps the split up to 32k
+    // keys (20000 keys: 30.4 -> 24.3 us; 65536: 58.4 unsplit, 62.0 split).
+    const bool split_heads = a.split_heads;
     switch (a.G) {
         case 1: attn_launch_decode_g<1, KV, HD>(ctx, a, kc, vc); break;
         case 2: attn_launch_decode_g<2, KV, HD>(ctx, a, kc, vc); break;
@@ -698,16 +703,20 @@ cera_hip_status cera_launch_attn(cera_hip_ctx* ctx, const float* q, const void* 
     const AttnNewKV nk = new_kv ? *new_kv : AttnNewKV{};
     uint32_t n_parts, part_keys = 0, chunks_per_part = 0;
     uint32_t S = 1;
+    bool split_heads = false;
     if (batch) {
         const uint64_t want = n_queries >= 1024 ? 4 : 8;   // many query blocks fill the chip with fewer parts
         part_keys = last_len <= 1024 ? 128u : static_cast<uint32_t>(((last_len + want - 1) / want + 31) / 32 * 32);
         n_parts = static_cast<uint32_t>((last_len + part_keys - 1) / part_keys);
     } else {
-        // positions per chunk: small chunks while the context is short (one memory round
-        // trip per wavefront, many wavefronts), 64 once there is plenty of work
-        // (thresholds measured on the 32/8/128 shape over rotating caches: 2048 keys 12.0 -> 10.2 us,
-        // 3072 keys 14.9 -> 12.4 us, 8192 keys 18.8 -> 18.2 us against the 4096 / 16384 ones used before)
-        S = last_len >= 8192 ? 8 : (last_len >= 2048 ? 4 : (last_len >= ATTN_FUSED_NEW_KV_MAX_KEYS ? 2 : 1));
+        // positions per chunk (8 S): one 8-key chunk per wavefront while the context is short (a single
+        // memory round trip, many wavefronts), longer chunks once there is plenty of work.  Measured on
+        // the 32/8/128 shape over rotating caches; with a kv head's query heads split over two
+        // wavefronts (attn_launch_partials) 32-key chunks are best from 1024 keys up to where the split
+        // ends: 64-key chunks take one wavefront per SIMD (registers) and lose 2-3 us from 8k to 16k keys.
+        split_heads = G >= 4 && last_len < (kv_f16 ? 32768u : 16384u);   // attn_launch_partials has the reasons
+        if (split_heads) S = last_len >= ATTN_FUSED_NEW_KV_MAX_KEYS ? 4 : 1;
+        else S = last_len >= 8192 ? 8 : (last_len >= 2048 ? 4 : (last_len >= ATTN_FUSED_NEW_KV_MAX_KEYS ? 2 : 1));
         if (G == 8 && S == 8) S = 4;   // eight heads x 64 positions per chunk does not fit the register file
         uint32_t n_chunks = static_cast<uint32_t>((last_len + 8 * S - 1) / (8 * S));
         // parts (wavefronts) per (query, kv head): enough to fill the chip ~4 waves per CU deep
@@ -719,18 +728,24 @@ cera_hip_status cera_launch_attn(cera_hip_ctx* ctx, const float* q, const void* 
         chunks_per_part = std::max(1u, (n_chunks + want_parts - 1) / want_parts);
         if (!n_splits) {
             // Between the lengths where that divides evenly the chip runs a ragged last round.  A
-            // wavefront's time goes with its chunks, a SIMD's with its wavefronts: take the chunks per
-            // part that minimise chunks x rounds, and of equals the one with fewer parts (a cheaper
-            // merge).  5120 keys: 20.5 -> 16.6 us, 10240: 33.2 -> 25.1; no length measured slower.
-            const uint32_t subs = (G >= 4 && last_len < 16384) ? 2 : 1;   // see attn_launch_partials
-            const uint64_t slots = static_cast<uint64_t>(ctx->n_cu) * 4;
+            // wavefront's time goes with its chunks, the launch's with the rounds of workgroups a CU
+            // runs (one workgroup per CU and round with an f32 cache, which is bound by bytes; two with
+            // an f16 cache): from the nominal count down to a quarter of it, take the parts that
+            // minimise chunks x rounds.  Of equals an f32 cache takes the one with more parts, an f16
+            // cache the one with fewer -- either way the one nearer two workgroups per CU.
+            // 9216 keys, f32: 31.2 -> 21.9 us together with the kernel's launch-index mapping, 13824:
+            // 37.2 -> 27.9; f16: 8192 keys 16.3 -> 13.9.  Within 4 % of the best (chunk, parts) pair
+            // of a sweep at every length from 1k to 16k keys (f32) and of a parts sweep (f16).
+            const uint32_t subs = split_heads ? 2 : 1;
             uint64_t best = ~0ull;
-            const uint32_t lo = std::max(1u, (n_chunks + ATTN_MAX_PARTS - 1) / ATTN_MAX_PARTS);
-            for (uint32_t cpp = chunks_per_part; cpp >= lo; --cpp) {
+            const uint32_t first = chunks_per_part;
+            for (uint32_t cpp = first; cpp <= n_chunks; ++cpp) {
                 const uint64_t parts = (n_chunks + cpp - 1) / cpp;
-                const uint64_t waves = parts * n_kv_heads * subs * n_queries;
-                const uint64_t cost = cpp * ((waves + slots - 1) / slots);
-                if (cost < best) { best = cost; chunks_per_part = cpp; }
+                if (cpp > first && parts * 4 < want_parts) break;
+                const uint64_t groups = (parts + 3) / 4 * n_kv_heads * subs * n_queries;   // workgroups
+                const uint64_t round = static_cast<uint64_t>(ctx->n_cu) * (waves_per_cu / 4);   // workgroups of four wavefronts
+                const uint64_t cost = cpp * ((groups + round - 1) / round);
+                if (cost < best || (kv_f16 && cost == best)) { best = cost; chunks_per_part = cpp; }
             }
         }
         n_parts = (n_chunks + chunks_per_part - 1) / chunks_per_part;
@@ -766,7 +781,7 @@ cera_hip_status cera_launch_attn(cera_hip_ctx* ctx, const float* q, const void* 
         ml = ctx->attn_ml;
     }
     AttnLaunch a{q, static_cast<uint32_t>(seq_len), static_cast<uint32_t>(max_seq), scale, n_heads, n_kv_heads, n_queries,
-                 n_heads * head_dim, G, S, n_parts, part_keys, chunks_per_part, batch, new_kv != nullptr, nk, acc, ml};
+                 n_heads * head_dim, G, S, n_parts, part_keys, chunks_per_part, batch, new_kv != nullptr, split_heads, nk, acc, ml};
     const kv_half *kh = static_cast<const kv_half*>(kc), *vh = static_cast<const kv_half*>(vc);
     const float *kf = static_cast<const float*>(kc), *vf = static_cast<const float*>(vc);
     if (head_dim == 128) {

@@ -373,13 +373,23 @@ __global__ __launch_bounds__(256) void attn_decode_partial_kernel(
     uint32_t seq_len, uint32_t max_seq, float scale, uint32_t chunks_per_part, uint32_t n_parts,
     uint32_t q_stride,                 // floats between consecutive queries (prefill batches queries on grid.z)
     uint32_t g_total,                  // query heads per kv head (a multiple of G)
+    uint32_t n_kv, uint32_t n_queries,
     float* __restrict__ part_acc,      // [n_queries][n_kv][n_parts][g_total][128]
     float* __restrict__ part_ml,       // [n_queries][n_kv][n_parts][g_total][2]
     AttnNewKV nk) {
     const uint32_t lane = threadIdx.x & 63;
-    const uint32_t part = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
-    const uint32_t subs = g_total / G, n_kv = gridDim.y / subs;
-    const uint32_t kvh = blockIdx.y / subs, sub = blockIdx.y % subs, qi = blockIdx.z;
+    // Workgroups are handed to the eight XCDs round-robin in launch order and every XCD has an L2 of
+    // its own.  The workgroups that read the same K/V rows (the sub-groups of a kv head's query heads,
+    // the queries of a small batch) therefore take launch indices 8 apart: same XCD, consecutive
+    // there, so all but the first find the rows in that L2 whatever the number of parts is.
+    // grid = attn_decode_grid(): index = (slot * reps + rep) * 8 + xcd, key-range group = slot * 8 + xcd.
+    const uint32_t subs = g_total / G, reps = subs * n_queries;
+    const uint32_t xcd = blockIdx.x & 7, t = blockIdx.x >> 3;
+    const uint32_t group = (t / reps) * 8 + xcd, rep = t % reps;
+    const uint32_t part_groups = (n_parts + 3) >> 2;
+    if (group >= part_groups * n_kv) return;
+    const uint32_t kvh = group / part_groups, sub = rep % subs, qi = rep / subs;
+    const uint32_t part = (group % part_groups) * 4 + (threadIdx.x >> 6);
     if (part >= n_parts) return;
     // causal prefill: query qi sits at position seq_len - 1 + qi and sees seq_len + qi keys
     seq_len += qi;

@@ -320,6 +320,32 @@ def test_attn_decode_gqa_groupings(hip, orc):
         assert np.abs(out - ref).max() <= ATTN_TOL * util.rms(ref)
 
 
+@pytest.mark.parametrize("nh,nkv,L,n", [(32, 8, 1100, 1), (32, 8, 4200, 1), (32, 8, 9000, 1), (24, 3, 1500, 1), (40, 5, 2300, 1),
+                                         (16, 2, 700, 1), (8, 1, 3000, 1), (14, 7, 900, 1), (32, 8, 1200, 5), (24, 3, 2100, 3),
+                                         (8, 8, 333, 7), (64, 8, 5000, 2)])
+def test_attn_decode_workgroup_mapping_covers_every_part(hip, orc, nh, nkv, L, n):
+    """The partial kernel maps launch indices to (kv head, key range, sub-group of heads, query)
+    XCD by XCD and rounds the launch up to whole eights: kv-head counts that do not divide eight,
+    part counts that are not multiples of four, both head sub-groups and small query batches must
+    all reach every (head, query), against the oracle query by query."""
+    hd = 128
+    _say(f"attn workgroup mapping nh={nh} nkv={nkv} L={L} n={n}")
+    r = util.rng(31 * L + nh + n)
+    q = r.standard_normal((n, nh * hd), dtype=np.float32)
+    k = r.standard_normal(L * nkv * hd, dtype=np.float32)
+    v = r.standard_normal(L * nkv * hd, dtype=np.float32)
+    scale = 1.0 / math.sqrt(hd)
+    if n == 1:
+        out = hip.attn_decode(q[0], k, v, nh, nkv, hd, L, scale).reshape(1, -1)
+    else:
+        out = hip.attn_prefill(q, k, v, nh, nkv, hd, L - n, n, scale)
+    for i in range(n):
+        Li = L - n + i + 1
+        ref = orc.decode_attention(q[i], k[:Li * nkv * hd], v[:Li * nkv * hd], nh, nkv, hd, scale, Li)
+        err = np.abs(out[i].astype(np.float64) - ref).max()
+        assert err <= ATTN_TOL * util.rms(ref), (i, err, util.rms(ref))
+
+
 @pytest.mark.parametrize("L", [32768, 131072])
 def test_attn_decode_config4_long_contexts(hip, orc, L):
     """The long contexts of the flash-decode configuration, against the oracle, plus two
@@ -352,7 +378,7 @@ def _through_half(x):
     return x.astype(np.float16).astype(np.float32)
 
 
-@pytest.mark.parametrize("L", [1, 9, 65, 512, 1000, 4096, 20000])
+@pytest.mark.parametrize("L", [1, 9, 65, 512, 1000, 4096, 9000, 20000, 33000])
 def test_attn_decode_f16_kv_vs_oracle(hip, orc, L):
     """KvCompression::F16: rows are narrowed to half on append and widened on read
     (cera/src/model/transformer.rs:1170-1196, 1424-1447), so the reference result is the f32
