@@ -6,6 +6,7 @@
 
 #include "cera_hip_kernels.h"
 #include "gemv.hip.h"
+#include "gemv_rows.hip.h"
 #include "glue.hip.h"
 #include "quantize.hip.h"
 
@@ -45,3 +46,108 @@ CERA_K_GEMV_TYPE(q4_1, Q4_1)
 CERA_K_GEMV_TYPE(q8_0, Q8_0)
 CERA_K_GEMV_TYPE(q4_k, Q4K)
 CERA_K_GEMV_TYPE(q6_k, Q6K)
+
+// ---- the one-wavefront-per-row decode kernels and the decode copies ----------------------------
+static_assert(sizeof(cera_k_row_gemv_args) == sizeof(RowGemvArgs) && offsetof(cera_k_row_gemv_args, row_bytes) == offsetof(RowGemvArgs, row_bytes) &&
+                  offsetof(cera_k_row_gemv_args, xq) == offsetof(RowGemvArgs, xq) && offsetof(cera_k_row_gemv_args, x) == offsetof(RowGemvArgs, x) &&
+                  offsetof(cera_k_row_gemv_args, eps) == offsetof(RowGemvArgs, eps) && offsetof(cera_k_row_gemv_args, y) == offsetof(RowGemvArgs, y) &&
+                  offsetof(cera_k_row_gemv_args, resid) == offsetof(RowGemvArgs, resid) &&
+                  offsetof(cera_k_row_gemv_args, out_q) == offsetof(RowGemvArgs, out_q) &&
+                  offsetof(cera_k_row_gemv_args, out_s) == offsetof(RowGemvArgs, out_s),
+              "row gemv args");
+static_assert(sizeof(cera_k_row_gemv_pair_args) == sizeof(RowGemvPairArgs) &&
+                  offsetof(cera_k_row_gemv_pair_args, b) == offsetof(RowGemvPairArgs, b) &&
+                  offsetof(cera_k_row_gemv_pair_args, n_blocks_a) == offsetof(RowGemvPairArgs, n_blocks_a),
+              "row gemv pair args");
+#define CERA_K_COPY_BYTES_OK(GT, T, K) (CERA_K_DECODE_COPY_ROW_BYTES(GT, K) == T::stream_row_bytes(K))
+static_assert(CERA_K_COPY_BYTES_OK(12, Q4K, 256) && CERA_K_COPY_BYTES_OK(12, Q4K, 4096) && CERA_K_COPY_BYTES_OK(12, Q4K, 14336), "Q4_K copy row bytes");
+static_assert(CERA_K_COPY_BYTES_OK(14, Q6K, 256) && CERA_K_COPY_BYTES_OK(14, Q6K, 4096) && CERA_K_COPY_BYTES_OK(14, Q6K, 14336), "Q6_K copy row bytes");
+static_assert(CERA_K_COPY_BYTES_OK(2, Q4_0, 32) && CERA_K_COPY_BYTES_OK(2, Q4_0, 4096) && CERA_K_COPY_BYTES_OK(2, Q4_0, 11008), "Q4_0 copy row bytes");
+static_assert(CERA_K_COPY_BYTES_OK(3, Q4_1, 32) && CERA_K_COPY_BYTES_OK(3, Q4_1, 4096) && CERA_K_COPY_BYTES_OK(3, Q4_1, 11008), "Q4_1 copy row bytes");
+static_assert(CERA_K_COPY_BYTES_OK(8, Q8_0, 32) && CERA_K_COPY_BYTES_OK(8, Q8_0, 4096) && CERA_K_COPY_BYTES_OK(8, Q8_0, 11008), "Q8_0 copy row bytes");
+
+#define CERA_K_DECODE_COPY(TN, T)                                                                        \
+    extern "C" __global__ __launch_bounds__(256) void cera_k_decode_copy_##TN(cera_k_decode_copy_args a) { \
+        stream_rows_body<T>(a.src, a.dst, a.n_units, a.row_bytes, a.copy_row_bytes);                     \
+    }
+CERA_K_DECODE_COPY(q4_0, Q4_0)
+CERA_K_DECODE_COPY(q4_1, Q4_1)
+CERA_K_DECODE_COPY(q8_0, Q8_0)
+CERA_K_DECODE_COPY(q4_k, Q4K)
+CERA_K_DECODE_COPY(q6_k, Q6K)
+
+// the launch bounds are those of the library's instances (gemv_rows.hip.h)
+#define CERA_K_ROW(NAME, T, P, EPI)                                                              \
+    extern "C" __global__ __launch_bounds__(256, 2) void NAME(RowGemvArgs p) {                   \
+        __shared__ uint32_t s_xq[1];                                                             \
+        __shared__ float s_xs[1];                                                                \
+        __shared__ double s_part[4];                                                             \
+        __shared__ __attribute__((aligned(16))) float s_out[4];                                  \
+        row_gemv_body<T, 4, 2, false, EPI, true, P>(p, blockIdx.x, s_xq, s_xs, s_part, s_out);   \
+    }
+#define CERA_K_ROW_BOTH(TN, T, P)                                \
+    CERA_K_ROW(cera_k_row_gemv_##TN##_p##P##_store, T, P, FEPI_STORE) \
+    CERA_K_ROW(cera_k_row_gemv_##TN##_p##P##_add, T, P, FEPI_ADD)
+CERA_K_ROW_BOTH(q4_k, Q4K, 1)
+CERA_K_ROW_BOTH(q6_k, Q6K, 1)
+CERA_K_ROW_BOTH(q4_0, Q4_0, 1)
+CERA_K_ROW_BOTH(q4_0, Q4_0, 2)
+CERA_K_ROW_BOTH(q4_1, Q4_1, 1)
+CERA_K_ROW_BOTH(q4_1, Q4_1, 2)
+CERA_K_ROW_BOTH(q8_0, Q8_0, 1)
+CERA_K_ROW_BOTH(q8_0, Q8_0, 2)
+
+#define CERA_K_ROW_LONG(TN, T, P)                                                                        \
+    extern "C" __global__ __launch_bounds__(256) void cera_k_row_gemv_long_##TN##_p##P##_add(RowGemvArgs p) { \
+        __shared__ __attribute__((aligned(16))) int8_t s_xq[P * 64 * T::ELEMS_PER_UNIT];                 \
+        __shared__ __attribute__((aligned(16))) float s_xs[P * 64 * T::ELEMS_PER_UNIT / 32];             \
+        row_gemv_long_body<T, 4, P, FEPI_ADD, true>(p, s_xq, s_xs);                                      \
+    }
+CERA_K_ROW_LONG(q4_k, Q4K, 2)
+CERA_K_ROW_LONG(q4_k, Q4K, 3)
+CERA_K_ROW_LONG(q4_k, Q4K, 4)
+CERA_K_ROW_LONG(q6_k, Q6K, 2)
+CERA_K_ROW_LONG(q6_k, Q6K, 3)
+CERA_K_ROW_LONG(q6_k, Q6K, 4)
+CERA_K_ROW_LONG(q4_0, Q4_0, 4)
+CERA_K_ROW_LONG(q4_0, Q4_0, 8)
+CERA_K_ROW_LONG(q4_1, Q4_1, 4)
+CERA_K_ROW_LONG(q4_1, Q4_1, 8)
+CERA_K_ROW_LONG(q8_0, Q8_0, 4)
+CERA_K_ROW_LONG(q8_0, Q8_0, 8)
+
+#define CERA_K_GATE_UP(TN, T, P)                                                                         \
+    extern "C" __global__ __launch_bounds__(1024, 1) void cera_k_norm_gate_up_##TN##_p##P(RowGemvArgs p) { \
+        __shared__ uint32_t s_xq[1024];                                                                  \
+        __shared__ float s_xs[128];                                                                      \
+        __shared__ double s_part[16];                                                                    \
+        __shared__ __attribute__((aligned(16))) float s_out[64];                                         \
+        row_gemv_body<T, 16, 4, true, FEPI_SILU_Q8, true, P>(p, blockIdx.x, s_xq, s_xs, s_part, s_out);  \
+    }
+CERA_K_GATE_UP(q4_k, Q4K, 1)
+CERA_K_GATE_UP(q4_0, Q4_0, 1)
+CERA_K_GATE_UP(q4_0, Q4_0, 2)
+CERA_K_GATE_UP(q4_1, Q4_1, 1)
+CERA_K_GATE_UP(q4_1, Q4_1, 2)
+CERA_K_GATE_UP(q8_0, Q8_0, 1)
+CERA_K_GATE_UP(q8_0, Q8_0, 2)
+
+#define CERA_K_QKV(TNA, TNB, TA, TB, P, R)                                                                                  \
+    extern "C" __global__ __launch_bounds__(512, 2) void cera_k_norm_qkv_##TNA##_##TNB##_p##P##_r##R(RowGemvPairArgs p) {     \
+        __shared__ uint32_t s_xq[1024];                                                                                     \
+        __shared__ float s_xs[128];                                                                                         \
+        __shared__ double s_part[8];                                                                                        \
+        if (blockIdx.x < p.n_blocks_a) row_gemv_body<TA, 8, R, true, FEPI_STORE, true, P>(p.a, blockIdx.x, s_xq, s_xs, s_part, nullptr); \
+        else row_gemv_body<TB, 8, R, true, FEPI_STORE, true, P>(p.b, blockIdx.x - p.n_blocks_a, s_xq, s_xs, s_part, nullptr); \
+    }
+#define CERA_K_QKV_R(TNA, TNB, TA, TB, P) CERA_K_QKV(TNA, TNB, TA, TB, P, 1) CERA_K_QKV(TNA, TNB, TA, TB, P, 2)
+CERA_K_QKV_R(q4_k, q4_k, Q4K, Q4K, 1)
+CERA_K_QKV_R(q4_k, q6_k, Q4K, Q6K, 1)
+CERA_K_QKV_R(q6_k, q4_k, Q6K, Q4K, 1)
+CERA_K_QKV_R(q6_k, q6_k, Q6K, Q6K, 1)
+CERA_K_QKV_R(q4_0, q4_0, Q4_0, Q4_0, 1)
+CERA_K_QKV_R(q4_0, q4_0, Q4_0, Q4_0, 2)
+CERA_K_QKV_R(q4_1, q4_1, Q4_1, Q4_1, 1)
+CERA_K_QKV_R(q4_1, q4_1, Q4_1, Q4_1, 2)
+CERA_K_QKV_R(q8_0, q8_0, Q8_0, Q8_0, 1)
+CERA_K_QKV_R(q8_0, q8_0, Q8_0, Q8_0, 2)

@@ -58,6 +58,57 @@ def test_gemv_from_the_code_object(hip, orc, host, dtype, m, k):
     assert np.abs(got_add - (r + ref)).max() <= 1e-3 * util.rms(ref) + 1e-6
 
 
+@pytest.mark.parametrize("dtype,m,k", [(util.Q4_K, 512, 4096), (util.Q4_K, 37, 256), (util.Q6_K, 264, 4096), (util.Q6_K, 1030, 2048),
+                                       (util.Q4_0, 128, 4096), (util.Q4_0, 77, 2048), (util.Q4_1, 64, 2080), (util.Q8_0, 96, 4096),
+                                       (util.Q8_0, 40, 160)])
+def test_row_gemv_on_a_decode_copy_from_the_code_object(hip, host, dtype, m, k):
+    """cera_k_decode_copy_* + cera_k_row_gemv_*: the bits of the library's GEMV on the native bytes."""
+    print(f"hsaco: row gemv {util.NAMES[dtype]} {m}x{k} on a decode copy", flush=True)
+    w, _ = util.make_weights(dtype, m, k, seed=m + k)
+    x, r = util.make_x(k, 19), util.make_x(m, 20)
+    lib = hip.gemv(dtype, w, x, m, k)
+    assert np.array_equal(_bits(host.row_gemv(dtype, w, m, k, x)), _bits(lib))
+    assert np.array_equal(_bits(host.row_gemv(dtype, w, m, k, x, resid=r)), _bits(hip.gemv_add_dev(dtype, w, x, r, m, k)))
+
+
+@pytest.mark.parametrize("dtype,m,k", [(util.Q6_K, 260, 14336), (util.Q4_K, 130, 14336), (util.Q4_K, 64, 8192), (util.Q6_K, 33, 11008),
+                                       (util.Q4_0, 70, 11008), (util.Q4_0, 64, 6144), (util.Q4_1, 48, 8192), (util.Q8_0, 36, 14336)])
+def test_long_row_gemv_on_a_decode_copy_from_the_code_object(hip, host, dtype, m, k):
+    print(f"hsaco: long row gemv {util.NAMES[dtype]} {m}x{k} on a decode copy", flush=True)
+    w, _ = util.make_weights(dtype, m, k, seed=m + k)
+    x, r = util.make_x(k, 21), util.make_x(m, 22)
+    got = host.row_gemv(dtype, w, m, k, x, resid=r)
+    assert np.array_equal(_bits(got), _bits(hip.gemv_add_dev(dtype, w, x, r, m, k)))
+
+
+@pytest.mark.parametrize("dtype,m,k", [(util.Q4_K, 14336, 4096), (util.Q4_K, 96, 2048), (util.Q4_0, 224, 4096), (util.Q4_1, 64, 1024),
+                                       (util.Q8_0, 160, 4096)])
+def test_norm_gate_up_from_the_code_object(hip, host, dtype, m, k):
+    print(f"hsaco: norm + gate|up {util.NAMES[dtype]} {m}x{k}", flush=True)
+    g, _ = util.make_weights(dtype, m, k, seed=3 * m + k)
+    u, _ = util.make_weights(dtype, m, k, seed=5 * m + k)
+    x = util.make_x(k, 23) * np.float32(2.0)
+    nw = (1.0 + 0.1 * util.make_x(k, 24)).astype(np.float32)
+    q, s = host.norm_gate_up(dtype, g, u, m, k, x, nw, 1e-5)
+    lq, ls = hip.ffn_gate_up_fused(g, u, m, k, x, nw, 1e-5, ggml_type=dtype)
+    assert np.array_equal(q, lq) and np.array_equal(_bits(s), _bits(ls))
+
+
+@pytest.mark.parametrize("ta,ma,tb,mb,k,rpw", [(util.Q4_K, 5120, util.Q6_K, 1024, 4096, 2), (util.Q4_K, 6144, util.Q4_K, 8, 4096, 2),
+                                                (util.Q6_K, 100, util.Q4_K, 52, 2048, 1), (util.Q6_K, 64, util.Q6_K, 64, 1024, 1),
+                                                (util.Q4_0, 640, util.Q4_0, 128, 4096, 2), (util.Q8_0, 96, util.Q8_0, 32, 2048, 1),
+                                                (util.Q4_1, 72, util.Q4_1, 24, 3072, 1)])
+def test_norm_qkv_from_the_code_object(hip, host, ta, ma, tb, mb, k, rpw):
+    print(f"hsaco: norm + qkv {util.NAMES[ta]} {ma} | {util.NAMES[tb]} {mb} x {k} r{rpw}", flush=True)
+    wa, _ = util.make_weights(ta, ma, k, seed=ma + k)
+    wb, _ = util.make_weights(tb, mb, k, seed=mb + k + 1)
+    x = util.make_x(k, 25) * np.float32(1.5)
+    nw = (1.0 + 0.1 * util.make_x(k, 26)).astype(np.float32)
+    ya, yb = host.norm_qkv(ta, wa, ma, tb, wb, mb, k, x, nw, 1e-5, rows_per_wave=rpw)
+    la, lb = hip.qkv_fused(ta, wa, ma, tb, wb, mb, k, x, nw, 1e-5)
+    assert np.array_equal(_bits(ya), _bits(la)) and np.array_equal(_bits(yb), _bits(lb))
+
+
 def test_library_launching_from_the_code_object(hip, orc):
     """cera_hip_ctx_create(device, hsaco_path): same results as the embedded kernels, kernel level
     and through a whole model."""
