@@ -385,12 +385,13 @@ def main() -> int:
             for g in ("ffn_gate_up", "ffn_down", "attn_qkv", "attn_output"):
                 run(groups[g])
         # decode attention, 32/8/128 heads, f32 cache (the values do not matter to the counters): 131072 keys take
-        # one wavefront per head group and non-temporal reads, 8192 keys two wavefronts per group and cached reads
+        # one wavefront per head group and non-temporal reads, 8192 and 9216 keys two wavefronts per group and
+        # cached reads (9216 keys make 15 workgroups per kv head and sub-group, not a multiple of the 8 XCDs)
         import ctypes as C
         kv_b = 8 * 131072 * 128 * 4
         dkp, dvp = ctx.malloc(kv_b), ctx.malloc(kv_b)
         dqp, dop = ctx.to_device(rng.standard_normal(32 * 128, dtype=np.float32)), ctx.malloc(32 * 128 * 4)
-        for L in (131072, 8192):
+        for L in (131072, 8192, 9216):
             for _ in range(4):
                 ctx.check(ctx.lib.cera_hip_attn_decode_dev(ctx.h, dqp, dkp, dvp, 32, 8, 128, L, L, C.c_float(1.0 / np.sqrt(128.0)), 0, dop))
         ctx.sync()
