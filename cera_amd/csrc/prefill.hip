@@ -5,6 +5,7 @@
 #include <cmath>
 #include <cstring>
 
+#include "gemm_q5k_f16.hip.h"
 #include "gemm_q6k_f16.hip.h"
 #include "glue.hip.h"
 #include "model.h"
@@ -16,6 +17,10 @@ static bool gemm_type_ok(uint32_t t) {
 // batched_gemm_supports (cera/src/model/transformer.rs:536-565): the int8 GEMM
 // takes K in whole 256-element steps.
 bool cera_gemm_supports(uint32_t dtype, uint64_t k) { return gemm_type_ok(dtype) && k % GEMM_KSUPER == 0 && k > 0; }
+// Q5_K has a batched kernel of its own that reads the f32 activations (gemm_q5k_f16.hip.h), as its
+// GEMV does: the reference never quantizes the input of a Q5_K projection (cera/src/backend/cpu.rs:1830-1854).
+static bool gemm_f32_supports(uint32_t dtype, uint64_t k) { return dtype == CERA_HIP_Q5_K && k % GEMM_KSUPER == 0 && k > 0; }
+static bool gemm_batched(uint32_t dtype, uint64_t k) { return cera_gemm_supports(dtype, k) || gemm_f32_supports(dtype, k); }
 
 // out[i*ld_m + j*ld_n] = (W . B)[i][j] (+ resid)
 // w2 / out2 (nullable): a second matrix of the same type and k multiplied by the same activations
@@ -25,10 +30,16 @@ cera_hip_status cera_launch_gemm(cera_hip_ctx* ctx, const cera_hip_dtensor* w, c
                                  const float* bsum, uint32_t n, float* out, uint64_t ld_m, uint64_t ld_n,
                                  const float* resid, float resid_scale, const cera_hip_dtensor* w2 = nullptr,
                                  float* out2 = nullptr, uint64_t ld_n2 = 0, bool* paired = nullptr, void* bh_ws = nullptr,
-                                 bool* staged = nullptr, int32_t* dbg_dots = nullptr) {
-    if (!cera_gemm_supports(w->dtype, w->k))
+                                 bool* staged = nullptr, int32_t* dbg_dots = nullptr, const float* x_f32 = nullptr,
+                                 bool* staged_f32 = nullptr) {
+    // Q5_K: x_f32 [n][k] are the activations (bs / bq / bsum are not read); *staged_f32 (nullable)
+    // says whether the context's split copy still holds exactly these activations
+    const bool q5 = gemm_f32_supports(w->dtype, w->k);
+    if (!q5 && !cera_gemm_supports(w->dtype, w->k))
         return cera_fail(ctx, CERA_HIP_ERR_UNSUPPORTED_DTYPE,
-                         "gemm: no int8 GEMM for ggml type " + std::to_string(w->dtype) + " with k=" + std::to_string(w->k));
+                         "gemm: no batched kernel for ggml type " + std::to_string(w->dtype) + " with k=" + std::to_string(w->k));
+    if (q5 && (!x_f32 || dbg_dots || (reinterpret_cast<uintptr_t>(w->dev) & 15) || (reinterpret_cast<uintptr_t>(x_f32) & 15)))
+        return cera_fail(ctx, CERA_HIP_ERR_ARGUMENT, "gemm: a Q5_K matrix takes 16-byte aligned f32 activations and has no integer block dots");
     if (n == 0) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "gemm: n must be positive");
     GemmArgs a;
     a.w = w->dev; a.bq = bq; a.bs = bs; a.bsum = bsum; a.out = out;
@@ -51,6 +62,24 @@ cera_hip_status cera_launch_gemm(cera_hip_ctx* ctx, const cera_hip_dtensor* w, c
             if (staged) *staged = true;
         }
         a.bh = bh_ws;
+    }
+    if (q5) {
+        // hi | lo f16 halves of x and its f32 block sums, in one scratch allocation
+        const uint64_t nk = static_cast<uint64_t>(n) * a.k;
+        void* ws;
+        CERA_TRY(cera_scratch(ctx, 11, nk * 4 + nk / 32 * 4 + static_cast<uint64_t>(n) * 4, &ws));
+        uint8_t* base = static_cast<uint8_t*>(ws);
+        float* xsum = reinterpret_cast<float*>(base + nk * 4);
+        float* unscale = xsum + nk / 32;   // 2^-e per token
+        if (!staged_f32 || !*staged_f32) {
+            hipLaunchKernelGGL(gemm_act_split_kernel, dim3(n), dim3(256), 0, ctx->stream, x_f32, reinterpret_cast<uint4*>(base),
+                               reinterpret_cast<uint4*>(base + nk * 2), xsum, unscale, a.k);
+            if (staged_f32) *staged_f32 = true;
+        }
+        a.bh = base;
+        a.bq = reinterpret_cast<const int8_t*>(base + nk * 2);
+        a.bs = unscale;
+        a.bsum = xsum;
     }
     dim3 grid((n + GEMM_BN - 1) / GEMM_BN, (a.m + GEMM_BM - 1) / GEMM_BM);
     a.w2 = nullptr; a.out2 = nullptr; a.m2 = 0; a.tiles1 = grid.y; a.ld_n2 = 0;
@@ -102,6 +131,7 @@ cera_hip_status cera_launch_gemm(cera_hip_ctx* ctx, const cera_hip_dtensor* w, c
     switch (w->dtype) {
         case CERA_HIP_Q4_K: hipLaunchKernelGGL((gemm_kernel<GemmQ4K>), grid, dim3(256), 0, ctx->stream, a); break;
         case CERA_HIP_Q6_K: hipLaunchKernelGGL(gemm_q6k_f16_kernel<false>, grid, dim3(256), 0, ctx->stream, a); break;
+        case CERA_HIP_Q5_K: hipLaunchKernelGGL(gemm_q5k_f16_kernel, grid, dim3(256), 0, ctx->stream, a); break;
         case CERA_HIP_Q4_0: hipLaunchKernelGGL((gemm_kernel<GemmQ4_0>), grid, dim3(256), 0, ctx->stream, a); break;
         case CERA_HIP_Q4_1: hipLaunchKernelGGL((gemm_kernel<GemmQ4_1>), grid, dim3(256), 0, ctx->stream, a); break;
         default: hipLaunchKernelGGL((gemm_kernel<GemmQ8_0>), grid, dim3(256), 0, ctx->stream, a); break;
@@ -159,9 +189,12 @@ extern "C" cera_hip_status cera_hip_gemm_dev(cera_hip_ctx* ctx, const cera_hip_d
     if (!ctx || !w || !x || !out) return CERA_HIP_ERR_ARGUMENT;
     std::lock_guard<std::recursive_mutex> op_lk(ctx->op_mu);
     if (n == 0 || n > 0x7FFFFFFFull) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "gemm: bad n");
+    if (gemm_f32_supports(w->dtype, w->k))   // f32 activations, no quantization (the reference's Q5_K semantics)
+        return cera_launch_gemm(ctx, w, nullptr, nullptr, nullptr, static_cast<uint32_t>(n), out, n, 1, nullptr, 1.0f, nullptr,
+                                nullptr, 0, nullptr, nullptr, nullptr, nullptr, x);
     if (!cera_gemm_supports(w->dtype, w->k))
         return cera_fail(ctx, CERA_HIP_ERR_UNSUPPORTED_DTYPE,
-                         "gemm: no int8 GEMM for ggml type " + std::to_string(w->dtype) + " with k=" + std::to_string(w->k));
+                         "gemm: no batched kernel for ggml type " + std::to_string(w->dtype) + " with k=" + std::to_string(w->k));
     void *ds, *dq, *db;
     CERA_TRY(cera_scratch(ctx, 1, n * (w->k / 32) * 4, &ds));
     CERA_TRY(cera_scratch(ctx, 2, n * w->k, &dq));
@@ -391,48 +424,56 @@ static cera_hip_status prefill_chunk(cera_hip_model* m, const uint32_t* tokens, 
 
     // whether pf_xh holds the f16 form of the quants now in pf_xq; cleared wherever those are rewritten
     bool staged = false;
+    // the f32 activations whose hi / lo split (Q5_K GEMMs) the context's workspace holds now
+    const float* split_of = nullptr;
     auto norm_rows = [&](const float* x, const float* w, float* y) -> cera_hip_status {
         staged = false;
+        split_of = nullptr;
         hipLaunchKernelGGL((rmsnorm_kernel<true>), dim3(n), dim3(256), 0, s, x, w, hs, c.rms_eps, y, m->pf_xs, m->pf_xq,
                            m->pf_bsum);
         HIP_TRY(ctx, hipGetLastError());
         return CERA_HIP_OK;
     };
     // out[n][w->m] (token-major rows) = B . W^T, optionally added onto resid
-    auto gemm = [&](const cera_hip_dtensor* w, float* out, const float* resid) -> cera_hip_status {
+    // xf: the f32 activations the quantized ones in pf_xs / pf_xq were made from (what a Q5_K matrix reads)
+    auto gemm = [&](const cera_hip_dtensor* w, float* out, const float* resid, const float* xf) -> cera_hip_status {
         // a short batch streams the weights once per 8 tokens through the multi-token GEMV (an
         // int8-MFMA tile would be mostly empty); its residual add is unscaled
-        if ((n <= PREFILL_SMALL_BATCH || !cera_gemm_supports(w->dtype, w->k)) && (!resid || c.residual_scale == 1.0f)) {
+        if ((n <= PREFILL_SMALL_BATCH || !gemm_batched(w->dtype, w->k)) && (!resid || c.residual_scale == 1.0f)) {
             bool launched = false;
             CERA_TRY(cera_launch_gemv_nb(ctx, w, m->pf_xs, m->pf_xq, static_cast<uint32_t>(w->k / 32),
                                          static_cast<uint32_t>(w->k), n, out, static_cast<uint32_t>(w->m), resid, &launched));
             if (launched) return CERA_HIP_OK;
         }
-        return cera_launch_gemm(ctx, w, m->pf_xs, m->pf_xq, m->pf_bsum, n, out, 1, w->m, resid, c.residual_scale, nullptr,
-                                nullptr, 0, nullptr, m->pf_xh, &staged);
+        bool split_held = split_of == xf;
+        CERA_TRY(cera_launch_gemm(ctx, w, m->pf_xs, m->pf_xq, m->pf_bsum, n, out, 1, w->m, resid, c.residual_scale, nullptr,
+                                  nullptr, 0, nullptr, m->pf_xh, &staged, nullptr, xf, &split_held));
+        if (w->dtype == CERA_HIP_Q5_K) split_of = xf;
+        return CERA_HIP_OK;
     };
 
     // two projections of the same activations: one launch when both have an int8 GEMM of the same
     // type (the tail of one matrix's workgroups then overlaps the other's, and a short K-split
     // matrix like K shares Q's launch), else one after the other
-    auto gemm2 = [&](const cera_hip_dtensor* wa, float* outa, const cera_hip_dtensor* wb, float* outb) -> cera_hip_status {
-        if (n > PREFILL_SMALL_BATCH && cera_gemm_supports(wa->dtype, wa->k) && cera_gemm_supports(wb->dtype, wb->k)) {
+    auto gemm2 = [&](const cera_hip_dtensor* wa, float* outa, const cera_hip_dtensor* wb, float* outb, const float* xf) -> cera_hip_status {
+        if (n > PREFILL_SMALL_BATCH && gemm_batched(wa->dtype, wa->k) && gemm_batched(wb->dtype, wb->k)) {
             bool paired = false;
+            bool split_held = split_of == xf;
             CERA_TRY(cera_launch_gemm(ctx, wa, m->pf_xs, m->pf_xq, m->pf_bsum, n, outa, 1, wa->m, nullptr, 1.0f, wb, outb,
-                                      wb->m, &paired, m->pf_xh, &staged));
+                                      wb->m, &paired, m->pf_xh, &staged, nullptr, xf, &split_held));
+            if (wa->dtype == CERA_HIP_Q5_K) split_of = xf;
             if (paired) return CERA_HIP_OK;
-            return cera_launch_gemm(ctx, wb, m->pf_xs, m->pf_xq, m->pf_bsum, n, outb, 1, wb->m, nullptr, 1.0f, nullptr,
-                                    nullptr, 0, nullptr, m->pf_xh, &staged);
+            return gemm(wb, outb, nullptr, xf);
         }
-        CERA_TRY(gemm(wa, outa, nullptr));
-        return gemm(wb, outb, nullptr);
+        CERA_TRY(gemm(wa, outa, nullptr, xf));
+        return gemm(wb, outb, nullptr, xf);
     };
 
     for (uint32_t i = 0; i < c.n_layers; ++i) {
         LayerDev& L = m->layers[i];
         CERA_TRY(norm_rows(m->pf_hidden, L.attn_norm, m->pf_normed));
-        CERA_TRY(gemm2(L.q, m->pf_q, L.k, m->pf_k));
-        CERA_TRY(gemm(L.v, m->pf_v, nullptr));
+        CERA_TRY(gemm2(L.q, m->pf_q, L.k, m->pf_k, m->pf_normed));
+        CERA_TRY(gemm(L.v, m->pf_v, nullptr, m->pf_normed));
         if (L.q_bias) {
             // bias rows: one launch per token keeps the kernel trivial; models with biases are rare here
             for (uint32_t t = 0; t < n; ++t) {
@@ -460,7 +501,8 @@ static cera_hip_status prefill_chunk(cera_hip_model* m, const uint32_t* tokens, 
         CERA_TRY(cera_launch_attn(ctx, m->pf_q, L.kc, L.vc, c.n_heads, c.n_kv_heads, c.head_dim, start_pos + 1ull,
                                   c.max_seq_len, scale, 0, n, m->pf_attn, m->pf_xs, m->pf_xq, m->pf_bsum, nullptr, m->kv_f16));
         staged = false;   // the attention merge rewrote the quants
-        CERA_TRY(gemm(L.o, m->pf_hidden, m->pf_hidden));
+        split_of = nullptr;
+        CERA_TRY(gemm(L.o, m->pf_hidden, m->pf_hidden, m->pf_attn));
 
         CERA_TRY(norm_rows(m->pf_hidden, L.ffn_norm, m->pf_normed));
         // gate, up, SwiGLU and the quantization for the down projection in one launch where the
@@ -469,7 +511,7 @@ static cera_hip_status prefill_chunk(cera_hip_model* m, const uint32_t* tokens, 
         bool fused = false;
         int8_t* const hq = reinterpret_cast<int8_t*>(m->pf_gate);
         float *const hs = m->pf_up, *const hb = m->pf_up + static_cast<uint64_t>(n) * (c.ffn / 32);
-        if (n > PREFILL_SMALL_BATCH)
+        if (n > PREFILL_SMALL_BATCH && L.down->dtype != CERA_HIP_Q5_K)   // a Q5_K down projection reads the f32 SwiGLU output
             CERA_TRY(cera_launch_gemm_swiglu(ctx, L.gate, L.up, m->pf_xs, m->pf_xq, m->pf_bsum, n, hq, hs, hb, &fused));
         staged = false;   // the down projection's activations are new either way
         if (fused && cera_gemm_supports(L.down->dtype, L.down->k)) {
@@ -483,13 +525,14 @@ static cera_hip_status prefill_chunk(cera_hip_model* m, const uint32_t* tokens, 
             HIP_TRY(ctx, hipMemcpyAsync(m->pf_xs, hs, static_cast<uint64_t>(n) * (c.ffn / 32) * 4, hipMemcpyDeviceToDevice, s));
             HIP_TRY(ctx, hipMemcpyAsync(m->pf_bsum, hb, static_cast<uint64_t>(n) * (c.ffn / 32) * 4, hipMemcpyDeviceToDevice, s));
         } else {
-            CERA_TRY(gemm2(L.gate, m->pf_gate, L.up, m->pf_up));
+            CERA_TRY(gemm2(L.gate, m->pf_gate, L.up, m->pf_up, m->pf_normed));
             const uint64_t tot = static_cast<uint64_t>(n) * c.ffn;
             hipLaunchKernelGGL((silu_mul_kernel<true>), dim3(static_cast<uint32_t>((tot / 4 + 255) / 256)), dim3(256), 0, s,
                                m->pf_gate, m->pf_up, tot, m->pf_gate, m->pf_xs, m->pf_xq, m->pf_bsum);
             HIP_TRY(ctx, hipGetLastError());
+            split_of = nullptr;
         }
-        CERA_TRY(gemm(L.down, m->pf_hidden, m->pf_hidden));
+        CERA_TRY(gemm(L.down, m->pf_hidden, m->pf_hidden, m->pf_gate));
     }
     m->seq_len = start_pos + n;
     if (all_logits) {
@@ -509,7 +552,7 @@ static cera_hip_status prefill_chunk(cera_hip_model* m, const uint32_t* tokens, 
         }
         // final norm of every row (+ Q8_0), then logits[n][rows] = normed . head^T
         CERA_TRY(norm_rows(m->pf_hidden, m->output_norm, m->pf_normed));
-        CERA_TRY(gemm(o, m->pf_logits, nullptr));
+        CERA_TRY(gemm(o, m->pf_logits, nullptr, m->pf_normed));
         if (c.logit_scale != 1.0f) {
             const uint64_t tot = static_cast<uint64_t>(n) * rows;
             hipLaunchKernelGGL(scale_kernel, dim3(static_cast<uint32_t>((tot + 255) / 256)), dim3(256), 0, s, m->pf_logits,
@@ -540,7 +583,7 @@ static cera_hip_status prefill_chunk(cera_hip_model* m, const uint32_t* tokens, 
 // tokens (unscaled residual add only) -- e.g. the Q4_0 / Q8_0 files of small models whose hidden
 // size is not a multiple of 256.
 static bool batched_supports(const cera_hip_model* m, const cera_hip_dtensor* w) {
-    if (cera_gemm_supports(w->dtype, w->k)) return true;
+    if (gemm_batched(w->dtype, w->k)) return true;
     const bool int8_type = w->dtype == CERA_HIP_Q4_0 || w->dtype == CERA_HIP_Q4_1 || w->dtype == CERA_HIP_Q8_0 ||
                            w->dtype == CERA_HIP_Q4_K || w->dtype == CERA_HIP_Q6_K;
     const uint64_t unit = w->dtype == CERA_HIP_Q6_K ? 64 : 32;
@@ -574,9 +617,10 @@ cera_hip_status cera_model_prefill_logits_all(cera_hip_model* m, const uint32_t*
 
 cera_hip_status cera_model_prefill(cera_hip_model* m, const uint32_t* tokens, uint32_t n, uint32_t start_pos,
                                    float* last_logits) {
-    // A single token, or a weight type with no batched kernel (Q5_K), takes the per-token
+    // A single token, or a weight shape with no batched kernel, takes the per-token
     // route -- the same decision LlamaModel::forward_prefill makes (llama.rs:1643,
-    // 762-795); it is still the HIP path, only slower.
+    // 762-795); it is still the HIP path, only slower.  (Q5_K, which sends the reference down
+    // that route, has a batched kernel here.)
     if (n == 1 || !prefill_batchable(m)) return cera_model_prefill_per_token(m, tokens, n, start_pos, last_logits);
     for (uint32_t off = 0; off < n; off += PREFILL_CHUNK) {
         uint32_t len = std::min(PREFILL_CHUNK, n - off);

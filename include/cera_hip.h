@@ -184,7 +184,10 @@ CERA_HIP_API cera_hip_status cera_hip_gemv_pair(cera_hip_ctx*, const cera_hip_te
  * 710-788, 865-946; kernels cera/src/backend/cpu.rs:1437-1557).
  * x is [n][k] row-major f32 (one activation row per token), each row is
  * quantized to Q8_0; out is [m][n] row-major -- the reference's
- * out[m_out_features][n_tokens] layout (cera/src/backend/simd.rs:5130-5148). */
+ * out[m_out_features][n_tokens] layout (cera/src/backend/simd.rs:5130-5148).
+ * A Q5_K matrix (k a multiple of 256) is multiplied with the f32 rows as they are, to f32
+ * accuracy: the reference never quantizes the input of a Q5_K projection
+ * (gemv_q5km_f32, cera/src/backend/cpu.rs:1830-1854), it only has no batched form of it. */
 CERA_HIP_API cera_hip_status cera_hip_gemm(cera_hip_ctx*, const cera_hip_tensor* w, const float* x, uint64_t n,
                                            float* out);
 

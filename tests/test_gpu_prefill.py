@@ -133,12 +133,73 @@ def test_gemm_pair_refuses_mixed_types(hip):
 
 
 def test_gemm_refuses_unsupported(hip):
+    with pytest.raises(hip_api.HipError) as e:  # Q5_K has no Q8_0 route: no paired / SwiGLU / block-dot entry
+        hip.gemm_pair(Q5_K, np.zeros(176 * 4, np.uint8), 4, Q5_K, np.zeros(176 * 4, np.uint8), 4,
+                      np.zeros((4, 256), np.float32), 4, 256)
+    assert e.value.status == 3
     with pytest.raises(hip_api.HipError) as e:
-        hip.gemm(Q5_K, np.zeros(176, np.uint8), np.zeros((1, 256), np.float32), 1, 1, 256)
+        hip.gemm_block_dots(Q5_K, np.zeros(176, np.uint8), np.zeros((1, 256), np.float32), 1, 1, 256)
     assert e.value.status == 3
     with pytest.raises(hip_api.HipError) as e:  # k not a multiple of 256
         hip.gemm(Q4_0, np.zeros(18 * 4, np.uint8), np.zeros((1, 128), np.float32), 1, 1, 128)
     assert e.value.status == 3
+
+
+@pytest.mark.parametrize("m,n,k,amp", [(96, 5, 1024, 1.0), (300, 77, 2048, 1.0), (130, 17, 14336, 1.0), (512, 200, 4096, 1.0),
+                                         (257, 65, 512, 1e-3), (64, 130, 4096, 300.0), (1, 1, 256, 1.0), (4096, 512, 4096, 1.0)])
+def test_gemm_q5k_reads_f32_activations(hip, orc, m, n, k, amp):
+    """The Q5_K batched kernel dots the weights with the UNQUANTIZED activations, as cera does
+    (cpu.rs:1830-1854): against the exact product in f64 the error is f32-class -- far below
+    what a Q8_0 round trip of x would cost (~5e-3 rms) -- at every magnitude of x, with ragged
+    tiles, a split K and a lone element; and each column agrees with the Q5_K GEMV of that token."""
+    _say(f"gemm Q5_K m={m} n={n} k={k} amp={amp}")
+    w, _ = util.make_weights(Q5_K, m, k, seed=41 + m)
+    x = (util.rng(m + n + k).standard_normal((n, k)) * amp).astype(np.float32)
+    out = hip.gemm(Q5_K, w, x, m, n, k)
+    rows = np.arange(m) if m <= 600 else np.unique(np.concatenate([np.arange(8), util.rng(2).integers(0, m, 48), np.arange(m - 8, m)]))
+    rb = util.H.row_bytes(Q5_K, k)
+    wr = np.ascontiguousarray(w.reshape(m, rb)[rows]).reshape(-1)
+    exact = util.dequant_np(Q5_K, wr, rows.size, k).astype(np.float64) @ x.astype(np.float64).T
+    err = np.abs(out[rows].astype(np.float64) - exact).max()
+    _say(f"  max|err|={err:.3e} rms={util.rms(exact):.3e}")
+    assert err <= GEMM_TOL * util.rms(exact)
+    assert err <= 3e-5 * util.rms(exact), "not f32-class: the activations were rounded somewhere"
+    for j in sorted({0, n // 2, n - 1}):
+        y = hip.gemv(Q5_K, wr, x[j], rows.size, k)
+        assert np.abs(out[rows, j] - y).max() <= 3e-5 * util.rms(exact)
+
+
+def test_q5k_model_prefills_in_batches(hip, orc):
+    """A model whose Q4_K tensors are Q5_K (the Q5_K_M recipe) takes the batched prefill route:
+    logits and KV cache agree with the token-by-token decode of the same prompt, and with the
+    oracle's per-token forward (cera's own route for a Q5_K model, llama.rs:1643)."""
+    cfg = dict(synth.TINY)
+    q5 = lambda name: util.H.Q5_K if synth.q4_k_m_type(name) == util.H.Q4_K else synth.q4_k_m_type(name)
+    weights = synth.make_llama(cfg, seed=91, sigma=0.05, norm_jitter=0.1, type_of=q5)
+    assert weights["blk.0.attn_q.weight"][0] == util.H.Q5_K and weights["blk.0.ffn_down.weight"][0] == util.H.Q6_K
+    a, b = hip_api.Model(hip, cfg, weights), hip_api.Model(hip, cfg, weights)
+    om = orc.Llama(cfg, weights)
+    toks = [int(t) for t in util.rng(6).integers(0, cfg["vocab"], 37)]
+    _say("model: Q5_K_M batched prefill 37 tokens")
+    la = a.forward_prefill(toks, 0)
+    for pos, t in enumerate(toks):
+        lb = b.forward(t, pos)
+        lo = om.forward(t, pos)
+    _say(f"  batched vs per-token cos={_cos(la, lb):.8f}; vs oracle cos={_cos(la, lo):.8f}")
+    assert _cos(la, lb) > 0.999 and _cos(la, lo) > 0.999
+    ka, va = a.read_kv(0)
+    kb, vb = b.read_kv(0)
+    assert np.abs(ka - kb).max() <= 1e-4 * util.rms(kb)   # layer 0: Q5_K k-projection of identical f32 inputs
+    kl, _ = a.read_kv(cfg["n_layers"] - 1)
+    kr, _ = b.read_kv(cfg["n_layers"] - 1)
+    assert np.abs(kl - kr).max() <= 5e-2 * util.rms(kr)
+    # all-position logits through the batched head as well
+    c = hip_api.Model(hip, cfg, weights)
+    allg = c.forward_prefill_logits_all(toks[:12], 0)
+    assert _cos(allg[-1], hip_api.Model(hip, cfg, weights).forward_prefill(toks[:12], 0)) > 0.9999
+    for mdl in (a, b, c):
+        mdl.close()
+    om.close()
 
 
 def _cos(a, b):
