@@ -168,6 +168,7 @@ void cera_hip_ctx_destroy(cera_hip_ctx* ctx) {
         if (ctx->pin[i]) (void)hipHostFree(ctx->pin[i]);
         if (ctx->pin_ev[i]) (void)hipEventDestroy(ctx->pin_ev[i]);
     }
+    if (ctx->word_host) (void)hipHostFree(ctx->word_host);
     if (ctx->module) (void)hipModuleUnload(ctx->module);
     (void)hipStreamDestroy(ctx->stream);
     delete ctx;
@@ -579,14 +580,31 @@ cera_hip_status cera_launch_gemv_pair(cera_hip_ctx* ctx, const cera_hip_dtensor*
     return CERA_HIP_OK;
 }
 
-cera_hip_status cera_launch_argmax(cera_hip_ctx* ctx, const float* x, uint32_t n, uint32_t* out_dev) {
+cera_hip_status cera_pinned_word(cera_hip_ctx* ctx, uint32_t** host, uint32_t** dev) {
+    if (!ctx->word_host) {
+        void *h = nullptr, *d = nullptr;
+        HIP_TRY(ctx, hipHostMalloc(&h, 64, hipHostMallocMapped));
+        const hipError_t e = hipHostGetDevicePointer(&d, h, 0);
+        if (e != hipSuccess) {
+            (void)hipHostFree(h);
+            return cera_fail(ctx, CERA_HIP_ERR_DEVICE, std::string("hipHostGetDevicePointer: ") + hipGetErrorString(e));
+        }
+        ctx->word_host = static_cast<uint32_t*>(h);
+        ctx->word_dev = static_cast<uint32_t*>(d);
+    }
+    *host = ctx->word_host;
+    *dev = ctx->word_dev;
+    return CERA_HIP_OK;
+}
+
+cera_hip_status cera_launch_argmax(cera_hip_ctx* ctx, const float* x, uint32_t n, uint32_t* out_dev, uint32_t* out_host_mapped) {
     void* part;
     CERA_TRY(cera_scratch(ctx, 8, ARGMAX_PARTS * 8, &part));
     float* pv = static_cast<float*>(part);
     uint32_t* pi = reinterpret_cast<uint32_t*>(pv + ARGMAX_PARTS);
     const uint32_t np = std::max(1u, std::min<uint32_t>(ARGMAX_PARTS, (n + 1023) / 1024));
     hipLaunchKernelGGL(argmax_partial_kernel, dim3(np), dim3(256), 0, ctx->stream, x, n, pv, pi);
-    hipLaunchKernelGGL(argmax_final_kernel, dim3(1), dim3(256), 0, ctx->stream, pv, pi, np, out_dev);
+    hipLaunchKernelGGL(argmax_final_kernel, dim3(1), dim3(256), 0, ctx->stream, pv, pi, np, out_dev, out_host_mapped);
     HIP_TRY(ctx, hipGetLastError());
     return CERA_HIP_OK;
 }
@@ -1107,7 +1125,7 @@ cera_hip_status cera_hip_argmax(cera_hip_ctx* ctx, const float* logits, uint64_t
     CERA_TRY(cera_scratch(ctx, 0, n * 4, &dx));
     CERA_TRY(cera_scratch(ctx, 1, 4, &di));
     CERA_TRY(cera_hip_upload(ctx, dx, logits, n * 4));
-    CERA_TRY(cera_launch_argmax(ctx, static_cast<float*>(dx), static_cast<uint32_t>(n), static_cast<uint32_t*>(di)));
+    CERA_TRY(cera_launch_argmax(ctx, static_cast<float*>(dx), static_cast<uint32_t>(n), static_cast<uint32_t*>(di), nullptr));
     return cera_hip_download(ctx, index, di, 4);
 }
 

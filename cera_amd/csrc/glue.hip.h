@@ -83,6 +83,21 @@ static __global__ void embed_row_kernel(uint32_t dtype, const uint8_t* __restric
     out[static_cast<uint64_t>(blockIdx.y) * k + e] = scale != 1.0f ? __fmul_rn(v, scale) : v;
 }
 
+// The decode step's first launch: the token's embedding row, and the token id and position into
+// scalars[0..1] for the kernels behind it (one launch instead of a one-thread kernel plus the lookup).
+static __global__ void embed_token_kernel(uint32_t dtype, const uint8_t* __restrict__ w, uint64_t row_bytes, uint32_t token,
+                                          uint32_t pos, uint32_t* __restrict__ scalars, uint32_t k, float scale,
+                                          float* __restrict__ out) {
+    uint32_t e = blockIdx.x * blockDim.x + threadIdx.x;
+    if (e == 0) {
+        scalars[0] = token;
+        scalars[1] = pos;
+    }
+    if (e >= k) return;
+    float v = dequant_elem(dtype, w + static_cast<uint64_t>(token) * row_bytes, e);
+    out[e] = scale != 1.0f ? __fmul_rn(v, scale) : v;
+}
+
 // ---------------------------------------------------------------------------
 // RMSNorm (cera/src/backend/cpu.rs:2479-2496): f64 sum of squares,
 // inv = (1/sqrt(mean + eps)) as f32, y = (x*inv)*w.  One 256-thread block per
@@ -372,13 +387,19 @@ static __global__ __launch_bounds__(256) void argmax_partial_kernel(const float*
     argmax_block_reduce(bv, bi, sv, si);
     if (threadIdx.x == 0) { pv[blockIdx.x] = bv; pi[blockIdx.x] = bi; }
 }
+// out2 (nullable): a second place for the index -- host memory the device can write, so that the
+// greedy step needs no copy launch after this one
 static __global__ __launch_bounds__(256) void argmax_final_kernel(const float* __restrict__ pv, const uint32_t* __restrict__ pi,
-                                                           uint32_t np, uint32_t* __restrict__ out) {
+                                                           uint32_t np, uint32_t* __restrict__ out, uint32_t* __restrict__ out2) {
     __shared__ float sv[4];
     __shared__ uint32_t si[4];
     float bv = -__builtin_inff();
     uint32_t bi = 0xFFFFFFFFu;
     for (uint32_t i = threadIdx.x; i < np; i += 256) argmax_merge(bv, bi, pv[i], pi[i]);
     argmax_block_reduce(bv, bi, sv, si);
-    if (threadIdx.x == 0) *out = bi == 0xFFFFFFFFu ? 0u : bi;
+    if (threadIdx.x == 0) {
+        const uint32_t v = bi == 0xFFFFFFFFu ? 0u : bi;
+        *out = v;
+        if (out2) *out2 = v;
+    }
 }

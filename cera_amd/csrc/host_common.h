@@ -51,6 +51,9 @@ struct cera_hip_ctx {
     std::mutex pin_mu;
     void* pin[2] = {nullptr, nullptr};
     hipEvent_t pin_ev[2] = {nullptr, nullptr};
+    // one pinned word the device writes directly (the greedy step's token): host view and device view
+    uint32_t* word_host = nullptr;
+    uint32_t* word_dev = nullptr;
 };
 
 void cera_set_global_error(const std::string& s);
@@ -110,7 +113,10 @@ cera_hip_status cera_launch_ffn_gate_up_fused(cera_hip_ctx* ctx, const cera_hip_
 cera_hip_status cera_launch_qkv_fused(cera_hip_ctx* ctx, const cera_hip_dtensor* wa, const cera_hip_dtensor* wb, const float* x,
                                       const float* norm_w, float eps, float* ya, float* yb, bool* launched);
 // index of the maximum of x[0, n) into *out_dev (device); uses scratch slot 8 of the context
-cera_hip_status cera_launch_argmax(cera_hip_ctx* ctx, const float* x, uint32_t n, uint32_t* out_dev);
+// out_host_mapped (nullable): device view of pinned host memory that also receives the index
+cera_hip_status cera_launch_argmax(cera_hip_ctx* ctx, const float* x, uint32_t n, uint32_t* out_dev, uint32_t* out_host_mapped);
+// the context's pinned word (allocated at first use)
+cera_hip_status cera_pinned_word(cera_hip_ctx* ctx, uint32_t** host, uint32_t** dev);
 cera_hip_status cera_launch_gemv_q5k_f32(cera_hip_ctx* ctx, const cera_hip_dtensor* w, const float* x, float* y);
 // kc / vc: [n_kv_heads][max_seq][head_dim], f32 or IEEE half (kv_f16)
 cera_hip_status cera_launch_attn_decode(cera_hip_ctx* ctx, const float* q, const void* kc, const void* vc,

@@ -527,18 +527,23 @@ cera_hip_status cera_attn_step(cera_hip_ctx* ctx, float* q, float* k_new, const 
                                    out_quants, nullptr, kv_f16);
 }
 
-// The per-token layer stack: LlamaModel::run_layers + project_logits.  The
-// token id and position are read by the kernels from m->scalars[0..1].
-static cera_hip_status decode_step(cera_hip_model* m, uint32_t pos, bool want_logits) {
-    if (m->ref_order) return cera_model_decode_step_ref(m, pos, want_logits);
+// The per-token layer stack: LlamaModel::run_layers + project_logits.  The first launch puts the
+// token id and position into m->scalars[0..1], where the kernels behind it read the position.
+static cera_hip_status set_token_pos(cera_hip_model* m, uint32_t token, uint32_t pos);
+
+static cera_hip_status decode_step(cera_hip_model* m, uint32_t token, uint32_t pos, bool want_logits) {
+    if (m->ref_order) {
+        CERA_TRY(set_token_pos(m, token, pos));
+        return cera_model_decode_step_ref(m, pos, want_logits);
+    }
     cera_hip_ctx* ctx = m->ctx;
     const cera_hip_config& c = m->cfg;
     hipStream_t s = ctx->stream;
     const uint32_t q_dim = c.n_heads * c.head_dim, kv_dim = c.n_kv_heads * c.head_dim;
     const float scale = c.attn_scale != 0.0f ? c.attn_scale : 1.0f / std::sqrt(static_cast<float>(c.head_dim));
 
-    hipLaunchKernelGGL(embed_row_kernel, dim3((c.hidden + 255) / 256), dim3(256), 0, s, m->embd->dtype, m->embd->dev,
-                       m->embd->row_bytes, m->scalars, c.hidden, c.embed_scale, m->hidden);
+    hipLaunchKernelGGL(embed_token_kernel, dim3((c.hidden + 255) / 256), dim3(256), 0, s, m->embd->dtype, m->embd->dev,
+                       m->embd->row_bytes, token, pos, m->scalars, c.hidden, c.embed_scale, m->hidden);
     HIP_TRY(ctx, hipGetLastError());
 
     for (uint32_t i = 0; i < c.n_layers; ++i) {
@@ -652,8 +657,7 @@ extern "C" cera_hip_status cera_hip_forward(cera_hip_model* m, uint32_t token, u
     if (!m || !logits) return CERA_HIP_ERR_ARGUMENT;
     ModelLock lk(m);
     CERA_TRY(check_step(m, token, pos));
-    CERA_TRY(set_token_pos(m, token, pos));
-    CERA_TRY(decode_step(m, pos, true));
+    CERA_TRY(decode_step(m, token, pos, true));
     CERA_TRY(cera_hip_download(m->ctx, logits, m->logits, static_cast<uint64_t>(m->cfg.vocab) * 4));
     m->seq_len = pos + 1;
     return CERA_HIP_OK;
@@ -663,10 +667,13 @@ extern "C" cera_hip_status cera_hip_forward_greedy(cera_hip_model* m, uint32_t t
     if (!m || !next) return CERA_HIP_ERR_ARGUMENT;
     ModelLock lk(m);
     CERA_TRY(check_step(m, token, pos));
-    CERA_TRY(set_token_pos(m, token, pos));
-    CERA_TRY(decode_step(m, pos, true));
-    CERA_TRY(cera_launch_argmax(m->ctx, m->logits, m->cfg.vocab, m->scalars + 2));
-    CERA_TRY(cera_hip_download(m->ctx, next, m->scalars + 2, 4));
+    CERA_TRY(decode_step(m, token, pos, true));
+    // the argmax kernel writes the token into pinned host memory itself: no copy launch behind it
+    uint32_t *word_host, *word_dev;
+    CERA_TRY(cera_pinned_word(m->ctx, &word_host, &word_dev));
+    CERA_TRY(cera_launch_argmax(m->ctx, m->logits, m->cfg.vocab, m->scalars + 2, word_dev));
+    HIP_TRY(m->ctx, hipStreamSynchronize(m->ctx->stream));
+    *next = *static_cast<volatile uint32_t*>(word_host);
     m->seq_len = pos + 1;
     return CERA_HIP_OK;
 }
@@ -705,8 +712,7 @@ extern "C" cera_hip_status cera_hip_forward_prefill_logits_all(cera_hip_model* m
 
 // one decode step with the logits copied out (the per-token route of the all-logits call)
 cera_hip_status cera_model_decode_logits(cera_hip_model* m, uint32_t token, uint32_t pos, float* logits) {
-    CERA_TRY(set_token_pos(m, token, pos));
-    CERA_TRY(decode_step(m, pos, true));
+    CERA_TRY(decode_step(m, token, pos, true));
     m->seq_len = pos + 1;
     return cera_hip_download(m->ctx, logits, m->logits, static_cast<uint64_t>(m->cfg.vocab) * 4);
 }
@@ -717,8 +723,7 @@ cera_hip_status cera_model_decode_logits(cera_hip_model* m, uint32_t token, uint
 cera_hip_status cera_model_prefill_per_token(cera_hip_model* m, const uint32_t* tokens, uint32_t n,
                                              uint32_t start_pos, float* last_logits) {
     for (uint32_t i = 0; i < n; ++i) {
-        CERA_TRY(set_token_pos(m, tokens[i], start_pos + i));
-        CERA_TRY(decode_step(m, start_pos + i, i + 1 == n));
+        CERA_TRY(decode_step(m, tokens[i], start_pos + i, i + 1 == n));
         m->seq_len = start_pos + i + 1;
     }
     return cera_hip_download(m->ctx, last_logits, m->logits, static_cast<uint64_t>(m->cfg.vocab) * 4);
