@@ -382,7 +382,8 @@ __global__ __launch_bounds__(256) void attn_decode_partial_kernel(
     // its own.  The workgroups that read the same K/V rows (the sub-groups of a kv head's query heads,
     // the queries of a small batch) therefore take launch indices 8 apart: same XCD, consecutive
     // there, so all but the first find the rows in that L2 whatever the number of parts is.
-    // grid = attn_decode_grid(): index = (slot * reps + rep) * 8 + xcd, key-range group = slot * 8 + xcd.
+    // Launch index = (slot * reps + rep) * 8 + xcd, key-range group = slot * 8 + xcd; the launcher
+    // (attn_launch_decode_g) rounds the groups up to whole eights.
     const uint32_t subs = g_total / G, reps = subs * n_queries;
     const uint32_t xcd = blockIdx.x & 7, t = blockIdx.x >> 3;
     const uint32_t group = (t / reps) * 8 + xcd, rep = t % reps;
