@@ -113,6 +113,32 @@ def test_greedy_free_running_prefix(tiny):
     assert n_same >= 2
 
 
+def test_greedy_token_is_the_argmax_of_the_same_logits(hip):
+    """forward_greedy's second argmax stage writes the token into pinned host memory, which the host
+    reads after the stream has drained: step by step it must return exactly the argmax (strict >,
+    lowest index on ties, cera/src/sampler.rs:20-30) of the logits forward() returns for the same
+    token and position -- with a Q6_K head, a tied (Q4_K embedding) head, an odd vocabulary size,
+    and the decode copies off."""
+    for tied, vocab, copies in ((False, 512, True), (True, 500, True), (False, 331, False)):
+        cfg = dict(synth.TINY, vocab=vocab)
+        weights = synth.make_llama(cfg, seed=300 + vocab, sigma=0.05, norm_jitter=0.1, tied_output=tied)
+        if not copies:
+            hip.set_decode_copies(False)
+        try:
+            a, b = hip_api.Model(hip, cfg, weights), hip_api.Model(hip, cfg, weights)
+        finally:
+            hip.set_decode_copies(True)
+        _say(f"greedy vs argmax(logits): tied={tied} vocab={vocab} decode copies={copies}")
+        tok = 7
+        for pos in range(12):
+            logits = b.forward(tok, pos)
+            want = int(orc_argmax(logits))
+            got = a.forward_greedy(tok, pos)
+            assert got == want, (pos, got, want)
+            tok = got
+        a.close(); b.close()
+
+
 def test_position_contract(tiny):
     cfg, weights, gm, om = tiny
     gm.truncate_kv(0)
