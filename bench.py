@@ -145,13 +145,21 @@ def measure_attention(ctx, hip_api, rng):
     return out
 
 
-def measure_gemm(ctx, H, dts, shape, rng):
+def measure_gemm(ctx, H, dts, shape, rng, n_thr=16):
     """BASELINE.json configs[2]: prefill GEMM out[N][M] = W_q . Q8_0(X[M][K]) on the matrix cores, activation
-    quantization included in the timed call."""
+    quantization included in the timed call.  One extra row set, outside BASELINE: the gate shape in Q5_K, whose
+    batched kernel reads the f32 activations (as the reference's Q5_K dot does) as split f16 operands."""
     INT8_PEAK_TOPS = 5000.0  # MI355X published dense int8 MFMA rate
     F16_PEAK_TOPS = 2500.0   # ... and dense f16
     res = []
-    for name in ("ffn_gate", "ffn_down"):
+    shape = dict(shape)
+    dts = dict(dts)
+    _, n_gate, k_gate = shape["ffn_gate"]
+    w5 = rng.standard_normal((n_gate, k_gate), dtype=np.float32) * np.float32(0.02)
+    dts["ffn_gate_q5_k"] = [ctx.tensor_upload(H.TYPE_IDS["Q5_K"], n_gate, k_gate, H.quantize(H.TYPE_IDS["Q5_K"], w5, n_thr))]
+    shape["ffn_gate_q5_k"] = ("Q5_K", n_gate, k_gate)
+    del w5
+    for name in ("ffn_gate", "ffn_down", "ffn_gate_q5_k"):
         tname, n_out, k = shape[name]
         for m_tok in (128, 512, 2048):
             dx = ctx.to_device(rng.standard_normal((m_tok, k), dtype=np.float32))
@@ -169,11 +177,12 @@ def measure_gemm(ctx, H, dts, shape, rng):
             us = ctx.elapsed_ms(e0, e1) * 1e3 / iters
             tops = 2.0 * m_tok * n_out * k / us / 1e6
             # Q6_K's block dots run on the f16 matrix cores (2.5 PFLOP/s dense), the rest on int8 (5 POP/s)
-            peak_key, peak = ("frac_of_f16_mfma_peak", F16_PEAK_TOPS) if tname == "Q6_K" else ("frac_of_int8_mfma_peak", INT8_PEAK_TOPS)
+            peak_key, peak = ("frac_of_f16_mfma_peak", F16_PEAK_TOPS) if tname in ("Q6_K", "Q5_K") else ("frac_of_int8_mfma_peak", INT8_PEAK_TOPS)
             res.append({"weight": f"{name} {tname} {n_out}x{k}", "tokens": m_tok, "us_per_call": round(us, 1),
                         "TOP/s": round(tops, 1), peak_key: round(tops / peak, 4)})
             ctx.free(dx)
             ctx.free(dout)
+    ctx.tensor_free(dts["ffn_gate_q5_k"][0])
     return res
 
 
@@ -535,7 +544,7 @@ def main() -> int:
     extras = {}
     if not args.no_extras:
         extras["flash_decode"] = measure_attention(ctx, hip_api, rng)
-        extras["prefill_gemm"] = measure_gemm(ctx, H, dts, shape, rng)
+        extras["prefill_gemm"] = measure_gemm(ctx, H, dts, shape, rng, n_thr)
     e2e = None if args.no_e2e else measure_e2e(args.seed, n_thr)
 
     out = {
