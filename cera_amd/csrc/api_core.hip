@@ -683,7 +683,9 @@ static void attn_launch_partials(cera_hip_ctx* ctx, const AttnLaunch& a, const K
     // K/V row is then read exactly once and the loads carry the non-temporal hint (131072 keys:
     // 5.50 TB/s split, 5.85 unsplit, 6.42 unsplit and non-temporal; 16384 keys: the same time either
     // way).  An f16 cache moves half the bytes for the same arithmetic and keeps the split up to 32k
-    // keys (20000 keys: 30.4 -> 24.3 us; 65536: 58.4 unsplit, 62.0 split).
+    // keys (20000 keys: 30.4 -> 24.3 us; 65536: 58.4 unsplit, 62.0 split).  Groups of 8 heads do
+    // twice the arithmetic per K/V byte and are never bound by bytes: they keep the split at every
+    // length (64 / 8 heads, 131072 keys: 279.5 -> 207.3 us; f16 cache, 32768 keys: 91.0 -> 54.5).
     const bool split_heads = a.split_heads;
     switch (a.G) {
         case 1: attn_launch_decode_g<1, KV, HD>(ctx, a, kc, vc); break;
@@ -732,7 +734,7 @@ cera_hip_status cera_launch_attn(cera_hip_ctx* ctx, const float* q, const void* 
         // the 32/8/128 shape over rotating caches; with a kv head's query heads split over two
         // wavefronts (attn_launch_partials) 32-key chunks are best from 1024 keys up to where the split
         // ends: 64-key chunks take one wavefront per SIMD (registers) and lose 2-3 us from 8k to 16k keys.
-        split_heads = G >= 4 && last_len < (kv_f16 ? 32768u : 16384u);   // attn_launch_partials has the reasons
+        split_heads = G >= 4 && (G == 8 || last_len < (kv_f16 ? 32768u : 16384u));   // attn_launch_partials has the reasons
         if (split_heads) S = last_len >= ATTN_FUSED_NEW_KV_MAX_KEYS ? 4 : 1;
         else S = last_len >= 8192 ? 8 : (last_len >= 2048 ? 4 : (last_len >= ATTN_FUSED_NEW_KV_MAX_KEYS ? 2 : 1));
         if (G == 8 && S == 8) S = 4;   // eight heads x 64 positions per chunk does not fit the register file

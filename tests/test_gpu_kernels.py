@@ -322,12 +322,13 @@ def test_attn_decode_gqa_groupings(hip, orc):
 
 @pytest.mark.parametrize("nh,nkv,L,n", [(32, 8, 1100, 1), (32, 8, 4200, 1), (32, 8, 9000, 1), (24, 3, 1500, 1), (40, 5, 2300, 1),
                                          (16, 2, 700, 1), (8, 1, 3000, 1), (14, 7, 900, 1), (32, 8, 1200, 5), (24, 3, 2100, 3),
-                                         (8, 8, 333, 7), (64, 8, 5000, 2)])
+                                         (8, 8, 333, 7), (64, 8, 5000, 2), (16, 2, 17000, 1), (8, 1, 33000, 1)])
 def test_attn_decode_workgroup_mapping_covers_every_part(hip, orc, nh, nkv, L, n):
     """The partial kernel maps launch indices to (kv head, key range, sub-group of heads, query)
     XCD by XCD and rounds the launch up to whole eights: kv-head counts that do not divide eight,
-    part counts that are not multiples of four, both head sub-groups and small query batches must
-    all reach every (head, query), against the oracle query by query."""
+    part counts that are not multiples of four, both head sub-groups (groups of eight heads keep
+    them at every length) and small query batches must all reach every (head, query), against the
+    oracle query by query."""
     hd = 128
     _say(f"attn workgroup mapping nh={nh} nkv={nkv} L={L} n={n}")
     r = util.rng(31 * L + nh + n)
