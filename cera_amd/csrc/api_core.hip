@@ -750,7 +750,7 @@ cera_hip_status cera_launch_attn(cera_hip_ctx* ctx, const float* q, const void* 
             // Between the lengths where that divides evenly the chip runs a ragged last round.  A
             // wavefront's time goes with its chunks, the launch's with the rounds of workgroups a CU
             // runs (one workgroup per CU and round with an f32 cache, which is bound by bytes; two with
-            // an f16 cache): from the nominal count down to a quarter of it, take the parts that
+            // an f16 cache or eight heads per kv head): from the nominal count down to a quarter of it, take the parts that
             // minimise chunks x rounds.  Of equals an f32 cache takes the one with more parts, an f16
             // cache the one with fewer -- either way the one nearer two workgroups per CU.
             // 9216 keys, f32: 31.2 -> 21.9 us together with the kernel's launch-index mapping, 13824:
@@ -763,7 +763,9 @@ cera_hip_status cera_launch_attn(cera_hip_ctx* ctx, const float* q, const void* 
                 const uint64_t parts = (n_chunks + cpp - 1) / cpp;
                 if (cpp > first && parts * 4 < want_parts) break;
                 const uint64_t groups = (parts + 3) / 4 * n_kv_heads * subs * n_queries;   // workgroups
-                const uint64_t round = static_cast<uint64_t>(ctx->n_cu) * (waves_per_cu / 4);   // workgroups of four wavefronts
+                // workgroups a CU takes per round: two where the kernel is bound by its own instructions
+                // (an f16 cache, eight heads per kv head), one where it is bound by bytes
+                const uint64_t round = static_cast<uint64_t>(ctx->n_cu) * ((kv_f16 || G == 8) ? 2 : 1);
                 const uint64_t cost = cpp * ((groups + round - 1) / round);
                 if (cost < best || (kv_f16 && cost == best)) { best = cost; chunks_per_part = cpp; }
             }
