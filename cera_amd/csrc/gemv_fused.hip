@@ -17,9 +17,10 @@ static uint32_t row_tiles(uint32_t type, uint64_t k) {
     return static_cast<uint32_t>((k / unit_elems(type) + 63) / 64);
 }
 // rows short enough for the kernels that keep a row's activations in registers
+// (one or two passes per lane: k <= 8192 for the K-quants' 64-weight units, k <= 4096 for 32-weight blocks)
 static uint32_t short_tiles(uint32_t type, uint64_t k) {
-    const uint32_t t = k <= 4096 ? row_tiles(type, k) : 0;
-    return t <= (kquant_type(type) ? 1u : 2u) ? t : 0;
+    const uint32_t t = k <= (kquant_type(type) ? 8192u : 4096u) ? row_tiles(type, k) : 0;
+    return t <= 2u ? t : 0;
 }
 
 static void fill(RowGemvArgs& a, const cera_hip_dtensor* w, const cera_hip_dtensor* w2, uint32_t rows_per_wave, bool stream = false) {
@@ -41,7 +42,7 @@ static void fill(RowGemvArgs& a, const cera_hip_dtensor* w, const cera_hip_dtens
 // route).  Other types and views are left alone.
 cera_hip_status cera_tensor_prepare_stream(cera_hip_ctx* ctx, cera_hip_dtensor* w) {
     if (!ctx->decode_copies) return CERA_HIP_OK;
-    if (!w || w->dev_stream || !w->owns || w->k > 16384 || w->m == 0 || w->m > 0x7FFFFFFFull) return CERA_HIP_OK;
+    if (!w || w->dev_stream || !w->owns || w->k > 32768 || w->m == 0 || w->m > 0x7FFFFFFFull) return CERA_HIP_OK;
     if (row_tiles(w->dtype, w->k) == 0 || (reinterpret_cast<uintptr_t>(w->dev) & 15)) return CERA_HIP_OK;
     const uint32_t k = static_cast<uint32_t>(w->k);
     uint64_t srb = 0;
@@ -96,12 +97,16 @@ cera_hip_status cera_launch_ffn_gate_up_fused(cera_hip_ctx* ctx, const cera_hip_
     RowGemvArgs a;
     // 16 wavefronts x 4 rows: a workgroup owns two Q8_0 blocks of the output, and 14336 rows make
     // 224 workgroups -- one per CU in a single wave of the launch (448 eight-wavefront workgroups
-    // leave a quarter of the CUs with half the others' share: 1 % slower end to end)
-    constexpr int GATE_UP_NW = 16, ROWS = 4;
+    // leave a quarter of the CUs with half the others' share: 1 % slower end to end).  Q4_K rows of
+    // two passes per lane (4096 < k <= 8192) hold twice the weights and activations per lane and
+    // take 8 wavefronts (one Q8_0 block of the output per workgroup).
+    constexpr int GATE_UP_NW = 16, ROWS = 4, WIDE_NW = 8, WIDE_ROWS = 8;
     const bool stream = gate->dev_stream && up->dev_stream;
-    fill(a, gate, up, ROWS, stream);
+    const bool wide = gate->dtype == CERA_HIP_Q4_K && tiles == 2;
+    fill(a, gate, up, wide ? WIDE_ROWS : ROWS, stream);
     a.x = x; a.norm_w = norm_w; a.eps = eps; a.out_q = out_q; a.out_s = out_s;
-    const dim3 grid((a.m + GATE_UP_NW * ROWS - 1) / (GATE_UP_NW * ROWS)), block(64 * GATE_UP_NW);
+    const uint32_t nw = wide ? WIDE_NW : GATE_UP_NW, per_wg = wide ? WIDE_NW * WIDE_ROWS : GATE_UP_NW * ROWS;
+    const dim3 grid((a.m + per_wg - 1) / per_wg), block(64 * nw);
 #define GATE_UP_LAUNCH(TT, TL)                                                                                                          \
     do {                                                                                                                                \
         if (stream) hipLaunchKernelGGL((row_gemv_kernel<TT, GATE_UP_NW, ROWS, true, FEPI_SILU_Q8, true, TL>), grid, block, 0, ctx->stream, a); \
@@ -112,7 +117,10 @@ cera_hip_status cera_launch_ffn_gate_up_fused(cera_hip_ctx* ctx, const cera_hip_
         if (tiles == 1) GATE_UP_LAUNCH(TT, 1); \
         else GATE_UP_LAUNCH(TT, 2);       \
     } while (0)
-    if (gate->dtype == CERA_HIP_Q4_K) GATE_UP_LAUNCH(Q4K, 1);
+    if (wide) {
+        if (stream) hipLaunchKernelGGL((row_gemv_kernel<Q4K, WIDE_NW, WIDE_ROWS, true, FEPI_SILU_Q8, true, 2, 8192>), grid, block, 0, ctx->stream, a);
+        else hipLaunchKernelGGL((row_gemv_kernel<Q4K, WIDE_NW, WIDE_ROWS, true, FEPI_SILU_Q8, false, 2, 8192>), grid, block, 0, ctx->stream, a);
+    } else if (gate->dtype == CERA_HIP_Q4_K) GATE_UP_LAUNCH(Q4K, 1);
     else if (gate->dtype == CERA_HIP_Q4_0) GATE_UP_LAUNCH_B32(Q4_0);
     else if (gate->dtype == CERA_HIP_Q4_1) GATE_UP_LAUNCH_B32(Q4_1);
     else GATE_UP_LAUNCH_B32(Q8_0);
@@ -133,6 +141,7 @@ cera_hip_status cera_launch_qkv_fused(cera_hip_ctx* ctx, const cera_hip_dtensor*
     if (wb && block32_type(wa->dtype) != block32_type(wb->dtype)) return CERA_HIP_OK;
     if (wb && block32_type(wa->dtype) && wb->dtype != wa->dtype) return CERA_HIP_OK;
     // two rows per wavefront (12 wavefronts per CU on the 8B shapes), one for short matrices
+    // (four for the 10240 x 8192 matrix of a 70B-class layer, to fit one round: no faster)
     const uint64_t rows = wa->m + (wb ? wb->m : 0);
     const uint32_t rpw = rows >= static_cast<uint64_t>(ctx->n_cu) * 8 ? 2 : 1;
     RowGemvPairArgs p;
@@ -152,8 +161,8 @@ cera_hip_status cera_launch_qkv_fused(cera_hip_ctx* ctx, const cera_hip_dtensor*
     const uint32_t ta = wa->dtype, tb = wb ? wb->dtype : wa->dtype;
 #define QKV_LAUNCH_S(TA_, TB_, ST_, TL_)                                                                                                \
     do {                                                                                                                                \
-        if (rpw == 2) hipLaunchKernelGGL((row_gemv_pair_kernel<TA_, TB_, FUSED_NW, 2, true, ST_, TL_>), grid, block, 0, ctx->stream, p); \
-        else hipLaunchKernelGGL((row_gemv_pair_kernel<TA_, TB_, FUSED_NW, 1, true, ST_, TL_>), grid, block, 0, ctx->stream, p);          \
+        if (rpw == 2) hipLaunchKernelGGL((row_gemv_pair_kernel<TA_, TB_, FUSED_NW, 2, true, ST_, TL_, 4096 * TL_>), grid, block, 0, ctx->stream, p); \
+        else hipLaunchKernelGGL((row_gemv_pair_kernel<TA_, TB_, FUSED_NW, 1, true, ST_, TL_, 4096 * TL_>), grid, block, 0, ctx->stream, p);          \
     } while (0)
 #define QKV_LAUNCH(TA_, TB_, TL_)                    \
     do {                                             \
@@ -168,10 +177,16 @@ cera_hip_status cera_launch_qkv_fused(cera_hip_ctx* ctx, const cera_hip_dtensor*
     if (ta == CERA_HIP_Q4_0) QKV_LAUNCH_B32(Q4_0);
     else if (ta == CERA_HIP_Q4_1) QKV_LAUNCH_B32(Q4_1);
     else if (ta == CERA_HIP_Q8_0) QKV_LAUNCH_B32(Q8_0);
-    else if (ta == CERA_HIP_Q4_K && tb == CERA_HIP_Q6_K) QKV_LAUNCH(Q4K, Q6K, 1);
-    else if (ta == CERA_HIP_Q4_K && tb == CERA_HIP_Q4_K) QKV_LAUNCH(Q4K, Q4K, 1);
-    else if (ta == CERA_HIP_Q6_K && tb == CERA_HIP_Q6_K) QKV_LAUNCH(Q6K, Q6K, 1);
-    else QKV_LAUNCH(Q6K, Q4K, 1);
+#define QKV_LAUNCH_KQ(TA_, TB_)                \
+    do {                                       \
+        if (tiles == 1) QKV_LAUNCH(TA_, TB_, 1); \
+        else QKV_LAUNCH(TA_, TB_, 2);          \
+    } while (0)
+    else if (ta == CERA_HIP_Q4_K && tb == CERA_HIP_Q6_K) QKV_LAUNCH_KQ(Q4K, Q6K);
+    else if (ta == CERA_HIP_Q4_K && tb == CERA_HIP_Q4_K) QKV_LAUNCH_KQ(Q4K, Q4K);
+    else if (ta == CERA_HIP_Q6_K && tb == CERA_HIP_Q6_K) QKV_LAUNCH_KQ(Q6K, Q6K);
+    else QKV_LAUNCH_KQ(Q6K, Q4K);
+#undef QKV_LAUNCH_KQ
 #undef QKV_LAUNCH_B32
 #undef QKV_LAUNCH
 #undef QKV_LAUNCH_S
@@ -204,8 +219,8 @@ cera_hip_status cera_launch_row_gemv_add(cera_hip_ctx* ctx, const cera_hip_dtens
         if (tiles == 1) ADD_LAUNCH(TT, 1); \
         else ADD_LAUNCH(TT, 2);       \
     } while (0)
-    if (w->dtype == CERA_HIP_Q4_K) ADD_LAUNCH(Q4K, 1);
-    else if (w->dtype == CERA_HIP_Q6_K) ADD_LAUNCH(Q6K, 1);
+    if (w->dtype == CERA_HIP_Q4_K) ADD_LAUNCH_B32(Q4K);
+    else if (w->dtype == CERA_HIP_Q6_K) ADD_LAUNCH_B32(Q6K);
     else if (w->dtype == CERA_HIP_Q4_0) ADD_LAUNCH_B32(Q4_0);
     else if (w->dtype == CERA_HIP_Q4_1) ADD_LAUNCH_B32(Q4_1);
     else ADD_LAUNCH_B32(Q8_0);
@@ -231,8 +246,10 @@ cera_hip_status cera_launch_row_gemv_store(cera_hip_ctx* ctx, const cera_hip_dte
     a.xq = xq; a.xs = xs; a.y = y;
     const dim3 grid((a.m + NW * ROWS - 1) / (NW * ROWS)), block(64 * NW);
 #define STORE_LAUNCH(TT, TL) hipLaunchKernelGGL((row_gemv_kernel<TT, NW, ROWS, false, FEPI_STORE, true, TL>), grid, block, 0, ctx->stream, a)
-    if (w->dtype == CERA_HIP_Q4_K) STORE_LAUNCH(Q4K, 1);
-    else if (w->dtype == CERA_HIP_Q6_K) STORE_LAUNCH(Q6K, 1);
+    if (w->dtype == CERA_HIP_Q4_K && tiles == 1) STORE_LAUNCH(Q4K, 1);
+    else if (w->dtype == CERA_HIP_Q4_K) STORE_LAUNCH(Q4K, 2);
+    else if (w->dtype == CERA_HIP_Q6_K && tiles == 1) STORE_LAUNCH(Q6K, 1);
+    else if (w->dtype == CERA_HIP_Q6_K) STORE_LAUNCH(Q6K, 2);
     else if (w->dtype == CERA_HIP_Q4_0 && tiles == 1) STORE_LAUNCH(Q4_0, 1);
     else if (w->dtype == CERA_HIP_Q4_0) STORE_LAUNCH(Q4_0, 2);
     else if (w->dtype == CERA_HIP_Q4_1 && tiles == 1) STORE_LAUNCH(Q4_1, 1);
@@ -252,7 +269,7 @@ cera_hip_status cera_launch_row_gemv_long_add(cera_hip_ctx* ctx, const cera_hip_
     *launched = false;
     const uint32_t tiles = row_tiles(w->dtype, w->k);
     const bool b32 = block32_type(w->dtype);
-    if (tiles == 0 || short_tiles(w->dtype, w->k) != 0 || tiles > (b32 ? 8u : 4u) || !resid || w->m > (1u << 20)) return CERA_HIP_OK;
+    if (tiles == 0 || short_tiles(w->dtype, w->k) != 0 || tiles > 8u || !resid || w->m > (1u << 20)) return CERA_HIP_OK;
     // four rows per workgroup: small workgroups start and retire independently, which measured
     // faster end to end than 8 or 16 rows sharing one staged copy of the activations
     constexpr int NW = 4;
@@ -261,11 +278,14 @@ cera_hip_status cera_launch_row_gemv_long_add(cera_hip_ctx* ctx, const cera_hip_
     fill(a, w, nullptr, 1, stream);
     a.xq = xq; a.xs = xs; a.y = y; a.resid = resid;
     const dim3 grid((a.m + NW - 1) / NW), block(64 * NW);
+    // K-quant rows: 3 or 4 passes as they come (the 8B / 7B down projections), longer rows in 6 or 8
+    // (a surplus pass re-reads unit 0 against zeroed activations)
 #define LONG_LAUNCH_S(TT, ST_)                                                                                                 \
     do {                                                                                                                       \
-        if (tiles == 2) hipLaunchKernelGGL((row_gemv_long_kernel<TT, NW, 2, FEPI_ADD, ST_>), grid, block, 0, ctx->stream, a);   \
-        else if (tiles == 3) hipLaunchKernelGGL((row_gemv_long_kernel<TT, NW, 3, FEPI_ADD, ST_>), grid, block, 0, ctx->stream, a); \
-        else hipLaunchKernelGGL((row_gemv_long_kernel<TT, NW, 4, FEPI_ADD, ST_>), grid, block, 0, ctx->stream, a);              \
+        if (tiles <= 3) hipLaunchKernelGGL((row_gemv_long_kernel<TT, NW, 3, FEPI_ADD, ST_>), grid, block, 0, ctx->stream, a);   \
+        else if (tiles == 4) hipLaunchKernelGGL((row_gemv_long_kernel<TT, NW, 4, FEPI_ADD, ST_>), grid, block, 0, ctx->stream, a); \
+        else if (tiles <= 6) hipLaunchKernelGGL((row_gemv_long_kernel<TT, NW, 6, FEPI_ADD, ST_>), grid, block, 0, ctx->stream, a); \
+        else hipLaunchKernelGGL((row_gemv_long_kernel<TT, NW, 8, FEPI_ADD, ST_>), grid, block, 0, ctx->stream, a);              \
     } while (0)
 #define LONG_LAUNCH(TT)                      \
     do {                                     \
@@ -317,7 +337,7 @@ extern "C" cera_hip_status cera_hip_ffn_gate_up_fused(cera_hip_ctx* ctx, const c
         bool launched = false;
         CERA_TRY(cera_launch_ffn_gate_up_fused(ctx, wg, wu, static_cast<float*>(dx), static_cast<float*>(dw), eps,
                                                static_cast<int8_t*>(dq), static_cast<float*>(ds), &launched));
-        if (!launched) return cera_fail(ctx, CERA_HIP_ERR_UNSUPPORTED_DTYPE, "ffn_gate_up_fused: needs two Q4_K matrices of one shape, k <= 4096 in whole super-blocks, m a multiple of 32");
+        if (!launched) return cera_fail(ctx, CERA_HIP_ERR_UNSUPPORTED_DTYPE, "ffn_gate_up_fused: needs two matrices of one fused type and shape, k <= 8192 (Q4_K) or 4096 in whole blocks, m a multiple of 32");
         CERA_TRY(cera_hip_download(ctx, quants, dq, m));
         return cera_hip_download(ctx, scales, ds, m / 32 * 4);
     };
@@ -348,7 +368,7 @@ extern "C" cera_hip_status cera_hip_qkv_fused(cera_hip_ctx* ctx, const cera_hip_
         float *da = static_cast<float*>(dy), *db = da + wa->m;
         bool launched = false;
         CERA_TRY(cera_launch_qkv_fused(ctx, wa, wb, static_cast<float*>(dx), static_cast<float*>(dw), eps, da, db, &launched));
-        if (!launched) return cera_fail(ctx, CERA_HIP_ERR_UNSUPPORTED_DTYPE, "qkv_fused: needs Q4_K / Q6_K matrices with k <= 4096 in whole super-blocks");
+        if (!launched) return cera_fail(ctx, CERA_HIP_ERR_UNSUPPORTED_DTYPE, "qkv_fused: needs Q4_K / Q6_K matrices with k <= 8192 in whole super-blocks (or 32-block types of one kind, k <= 4096)");
         CERA_TRY(cera_hip_download(ctx, ya, da, wa->m * 4));
         if (wb) CERA_TRY(cera_hip_download(ctx, yb, db, wb->m * 4));
         return CERA_HIP_OK;

@@ -1,5 +1,5 @@
 // Decode GEMVs with the neighbouring small operations folded in, for rows that fit one wavefront
-// (k <= 4096 with 64-weight units: the hidden size of the 7-8B models).
+// (k <= 4096 with 64-weight units in one pass per lane: the hidden size of the 7-8B models; k <= 8192 in two).
 //
 // A decode step is a chain of dependent launches, and on this hardware a launch costs about 3 us
 // before its first byte arrives, whatever it does.  rmsnorm + Q8_0 quantization of a 4096-vector
@@ -43,13 +43,13 @@ struct RowGemvPairArgs {
     uint32_t n_blocks_a;
 };
 
-// rmsnorm + Q8_0 of x[0, k) into LDS by all 64 * NW threads (k % 32 == 0, k <= 4096), in two steps:
+// rmsnorm + Q8_0 of x[0, k) into LDS by all 64 * NW threads (k % 32 == 0, k <= MAXK), in two steps:
 // load() issues the loads of x and the norm weights, finish() does the rest.  The caller issues
 // its weight-row loads between the two: the hardware counts outstanding loads in order, so a wait
 // for x placed behind the weight loads would wait for every weight row as well.
-template <int NW>
+template <int NW, int MAXK = 4096>
 struct NormQuant {
-    static constexpr int NT = 64 * NW, MAXIT = 1024 / NT;
+    static constexpr int NT = 64 * NW, MAXIT = (MAXK / 4 + NT - 1) / NT;
     float4 v[MAXIT], g[MAXIT];
     __device__ __forceinline__ void load(const float* __restrict__ x, const float* __restrict__ w, uint32_t k) {
 #pragma unroll
@@ -126,7 +126,7 @@ struct RowTile {
 // TILES: units per lane (a row is TILES passes of 64 units: 1 for the K-quants' 64-weight units up
 // to k = 4096, 2 for the 32-weight blocks of Q4_0 / Q8_0 beyond k = 2048).  Pass t holds the units
 // wavefront t of the K-split kernel holds and the pass totals are added in that order: same bits.
-template <class T, int NW, int ROWS, bool NORM, int EPI, bool STREAM, int TILES>
+template <class T, int NW, int ROWS, bool NORM, int EPI, bool STREAM, int TILES, int MAXK = 4096>
 __device__ __forceinline__ void row_gemv_body(const RowGemvArgs& p, uint32_t block, uint32_t* s_xq, float* s_xs, double* s_part,
                                               float* s_out) {
     constexpr int NM = EPI == FEPI_SILU_Q8 ? 2 : 1;
@@ -143,7 +143,7 @@ __device__ __forceinline__ void row_gemv_body(const RowGemvArgs& p, uint32_t blo
     const uint32_t r0 = (block * NW + wave) * ROWS;
     auto row_of = [&](int i) -> uint32_t { return r0 + i; };
 
-    NormQuant<NW> nq;
+    NormQuant<NW, MAXK> nq;
     if (NORM) {
         nq.load(p.x, p.norm_w, p.k);
         __builtin_amdgcn_sched_barrier(0);   // x and the norm weights first: they are waited for first
@@ -230,25 +230,26 @@ __device__ __forceinline__ void row_gemv_body(const RowGemvArgs& p, uint32_t blo
     }
 }
 
-template <class T, int NW, int ROWS, bool NORM, int EPI, bool STREAM, int TILES = 1>
+// MAXK: the longest row the NORM form stages (LDS for its quantized activations)
+template <class T, int NW, int ROWS, bool NORM, int EPI, bool STREAM, int TILES = 1, int MAXK = 4096>
 static __global__ __launch_bounds__(64 * NW, NW <= 8 ? 2 : 1) void row_gemv_kernel(RowGemvArgs p) {
-    __shared__ uint32_t s_xq[NORM ? 1024 : 1];
-    __shared__ float s_xs[NORM ? 128 : 1];
+    __shared__ uint32_t s_xq[NORM ? MAXK / 4 : 1];
+    __shared__ float s_xs[NORM ? MAXK / 32 : 1];
     __shared__ double s_part[NW];
     __shared__ __attribute__((aligned(16))) float s_out[EPI == FEPI_SILU_Q8 ? NW * ROWS : 4];
-    row_gemv_body<T, NW, ROWS, NORM, EPI, STREAM, TILES>(p, blockIdx.x, s_xq, s_xs, s_part, s_out);
+    row_gemv_body<T, NW, ROWS, NORM, EPI, STREAM, TILES, MAXK>(p, blockIdx.x, s_xq, s_xs, s_part, s_out);
 }
 
-template <class TA, class TB, int NW, int ROWS, bool NORM, bool STREAM, int TILES = 1>
+template <class TA, class TB, int NW, int ROWS, bool NORM, bool STREAM, int TILES = 1, int MAXK = 4096>
 static __global__ __launch_bounds__(64 * NW, 2) void row_gemv_pair_kernel(RowGemvPairArgs p) {
-    __shared__ uint32_t s_xq[NORM ? 1024 : 1];
-    __shared__ float s_xs[NORM ? 128 : 1];
+    __shared__ uint32_t s_xq[NORM ? MAXK / 4 : 1];
+    __shared__ float s_xs[NORM ? MAXK / 32 : 1];
     __shared__ double s_part[NW];
-    if (blockIdx.x < p.n_blocks_a) row_gemv_body<TA, NW, ROWS, NORM, FEPI_STORE, STREAM, TILES>(p.a, blockIdx.x, s_xq, s_xs, s_part, nullptr);
-    else row_gemv_body<TB, NW, ROWS, NORM, FEPI_STORE, STREAM, TILES>(p.b, blockIdx.x - p.n_blocks_a, s_xq, s_xs, s_part, nullptr);
+    if (blockIdx.x < p.n_blocks_a) row_gemv_body<TA, NW, ROWS, NORM, FEPI_STORE, STREAM, TILES, MAXK>(p.a, blockIdx.x, s_xq, s_xs, s_part, nullptr);
+    else row_gemv_body<TB, NW, ROWS, NORM, FEPI_STORE, STREAM, TILES, MAXK>(p.b, blockIdx.x - p.n_blocks_a, s_xq, s_xs, s_part, nullptr);
 }
 
-// Long rows (4096 < k <= 16384: the down projection): still one wavefront per row, walking the
+// Long rows (beyond the short kernels, k <= 32768 for the K-quants: the down projection): still one wavefront per row, walking the
 // row in TILES passes of 64 units with every pass's weights requested up front and the activations
 // read from LDS pass by pass (a lane cannot keep four passes' activations in registers).  There is
 // no K split across wavefronts, so no combine and no barrier after the activations are staged:

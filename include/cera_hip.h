@@ -102,7 +102,7 @@ CERA_HIP_API void cera_hip_ctx_destroy(cera_hip_ctx*);
 CERA_HIP_API const char* cera_hip_last_error(const cera_hip_ctx*);
 CERA_HIP_API cera_hip_status cera_hip_sync(cera_hip_ctx*);
 /* Decode copies (on by default).  When on, cera_hip_model_create and cera_hip_decode_ops_dev give
- * every Q4_K / Q6_K / Q4_0 / Q4_1 / Q8_0 projection matrix (k at most 16384) a second copy of
+ * every Q4_K / Q6_K / Q4_0 / Q4_1 / Q8_0 projection matrix (k at most 32768; 16384 for the 32-weight blocks) a second copy of
  * about the same size in which each row's bytes are permuted so that the decode GEMV kernels read
  * it in whole 128-byte lines with non-temporal loads (+6 % decode rate on the 8B model for about
  * twice those matrices' memory); every other reader keeps the native GGUF bytes.  Results are
@@ -297,16 +297,16 @@ CERA_HIP_API cera_hip_status cera_hip_attn_decode_step(cera_hip_ctx*, const floa
  * its Q8_0 quantization, the two projections of transformer::forward_ffn_block
  * (cera/src/model/transformer.rs:1541), cpu::silu_mul_inplace (cera/src/backend/cpu.rs:2570-2575)
  * and the Q8_0 quantization of the result for the down projection (cpu.rs:942-958) in ONE launch:
- * quants i8[m], scales f32[m/32].  Two Q4_K matrices of one shape, k <= 4096 in whole
- * 256-element super-blocks, m a multiple of 32; anything else is CERA_HIP_ERR_UNSUPPORTED_DTYPE
+ * quants i8[m], scales f32[m/32].  Two Q4_K matrices of one shape, k <= 8192 in whole
+ * 256-element super-blocks (or two Q4_0 / Q4_1 / Q8_0 matrices, k <= 4096), m a multiple of 32; anything else is CERA_HIP_ERR_UNSUPPORTED_DTYPE
  * (the decode step then issues the separate launches). */
 CERA_HIP_API cera_hip_status cera_hip_ffn_gate_up_fused(cera_hip_ctx*, const cera_hip_tensor* gate,
                                                         const cera_hip_tensor* up, const float* x, const float* norm_w,
                                                         float eps, int8_t* quants, float* scales);
 /* q | k | v: cpu::rmsnorm(x, norm_w), its Q8_0 quantization and the projections of
  * transformer::forward_attn_block (cera/src/model/transformer.rs:1340-1373) in one launch:
- * ya = A . n, yb = B . n (b / yb nullable).  Q4_K or Q6_K matrices with k <= 4096 in whole
- * super-blocks. */
+ * ya = A . n, yb = B . n (b / yb nullable).  Q4_K or Q6_K matrices with k <= 8192 in whole
+ * super-blocks, or two matrices of one 32-weight-block type with k <= 4096. */
 CERA_HIP_API cera_hip_status cera_hip_qkv_fused(cera_hip_ctx*, const cera_hip_tensor* a, const cera_hip_tensor* b,
                                                 const float* x, const float* norm_w, float eps, float* ya, float* yb);
 

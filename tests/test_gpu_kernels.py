@@ -593,9 +593,9 @@ def test_ffn_gate_up_fused_against_the_oracle(hip, orc, m, k):
 
 
 def test_fused_launches_refuse_what_they_do_not_cover(hip):
-    w = np.zeros(8 * 32 * 144, np.uint8)
-    with pytest.raises(hip_api.HipError) as e:     # k beyond one wavefront of 64-weight units
-        hip.qkv_fused(Q4_K, w, 8, None, None, None, 8192, np.zeros(8192, np.float32), np.ones(8192, np.float32), 1e-5)
+    w = np.zeros(8 * 48 * 144, np.uint8)
+    with pytest.raises(hip_api.HipError) as e:     # k beyond two passes of a wavefront's 64-weight units
+        hip.qkv_fused(Q4_K, w, 8, None, None, None, 12288, np.zeros(12288, np.float32), np.ones(12288, np.float32), 1e-5)
     assert e.value.status == 3
     with pytest.raises(hip_api.HipError) as e:     # m not a whole number of 32-row Q8_0 blocks
         hip.ffn_gate_up_fused(w[:8 * 144], w[:8 * 144], 8, 256, np.zeros(256, np.float32), np.ones(256, np.float32), 1e-5)
@@ -652,7 +652,9 @@ def no_decode_copies(hip):
                                        (Q4_0, 1030, 4096), (Q8_0, 130, 4096), (Q4_0, 70, 2048), (Q8_0, 33, 1024), (Q4_0, 9, 32),
                                        (Q4_0, 512, 14336), (Q8_0, 200, 14336), (Q4_0, 64, 8192), (Q8_0, 40, 6144), (Q4_0, 50, 11008),
                                        (Q8_0, 24, 4128), (Q4_0, 24, 16384),
-                                       (Q4_1, 130, 4096), (Q4_1, 70, 2048), (Q4_1, 64, 14336), (Q4_1, 40, 6144), (Q4_1, 9, 96)])
+                                       (Q4_1, 130, 4096), (Q4_1, 70, 2048), (Q4_1, 64, 14336), (Q4_1, 40, 6144), (Q4_1, 9, 96),
+                                       (Q4_K, 130, 8192), (Q6_K, 66, 5120), (Q4_K, 40, 7168), (Q6_K, 70, 18944), (Q4_K, 36, 20480),
+                                       (Q6_K, 130, 28672), (Q4_K, 20, 32768), (Q6_K, 12, 24576)])
 def test_residual_projection_streams_the_decode_copy_to_the_same_bits(hip, no_decode_copies, dtype, m, k):
     """A matrix's decode copy is a permutation of its bytes, read by the same arithmetic: the
     residual projections give identical bits with the copy (the default) and from the native
@@ -684,6 +686,35 @@ def test_fused_launches_stream_the_decode_copy_to_the_same_bits(hip, no_decode_c
     q0, sc0 = no_decode_copies(lambda: hip.ffn_gate_up_fused(wg, wu, 1024, k, x, nw, 1e-5))
     assert np.array_equal(ya.view(np.uint32), ya0.view(np.uint32)) and np.array_equal(yb.view(np.uint32), yb0.view(np.uint32))
     assert np.array_equal(q, q0) and np.array_equal(sc.view(np.uint32), sc0.view(np.uint32))
+
+
+@pytest.mark.parametrize("k,tb", [(8192, Q6_K), (5120, Q4_K), (6144, Q6_K)])
+def test_fused_launches_for_rows_of_two_passes(hip, orc, no_decode_copies, k, tb):
+    """K-quant rows of 4096 < k <= 8192 (the hidden sizes of the 13B - 70B models) take the same fused
+    decode launches with two 64-weight units per lane: Q|K|V with the norm inside, gate|up with norm,
+    SwiGLU and Q8_0, the O projection with its residual and the head -- bitwise what the separate
+    launches compute, with and without decode copies."""
+    _say(f"fused launches, two passes per lane, k={k}")
+    m = 1024
+    wa, _ = util.make_weights(Q4_K, 1280, k, seed=111)
+    wb, _ = util.make_weights(tb, 256, k, seed=112)
+    wg, _ = util.make_weights(Q4_K, m, k, seed=113)
+    wu, _ = util.make_weights(Q4_K, m, k, seed=114)
+    x = util.make_x(k, 115) * np.float32(1.3)
+    nw = (1.0 + 0.1 * util.make_x(k, 116)).astype(np.float32)
+    n, _, _ = hip.rmsnorm_q8_0(x, nw, 1e-5)
+    ya, yb = hip.qkv_fused(Q4_K, wa, 1280, tb, wb, 256, k, x, nw, 1e-5)
+    assert np.array_equal(ya.view(np.uint32), hip.gemv(Q4_K, wa, n, 1280, k).view(np.uint32))
+    assert np.array_equal(yb.view(np.uint32), hip.gemv(tb, wb, n, 256, k).view(np.uint32))
+    q, sc = hip.ffn_gate_up_fused(wg, wu, m, k, x, nw, 1e-5)
+    rs, rq = hip.quantize_q8_0(hip.silu_mul(hip.gemv(Q4_K, wg, n, m, k), hip.gemv(Q4_K, wu, n, m, k)))
+    assert np.array_equal(q, rq) and np.array_equal(sc.view(np.uint32), rs.view(np.uint32))
+    ya0, yb0 = no_decode_copies(lambda: hip.qkv_fused(Q4_K, wa, 1280, tb, wb, 256, k, x, nw, 1e-5))
+    q0, sc0 = no_decode_copies(lambda: hip.ffn_gate_up_fused(wg, wu, m, k, x, nw, 1e-5))
+    assert np.array_equal(ya.view(np.uint32), ya0.view(np.uint32)) and np.array_equal(yb.view(np.uint32), yb0.view(np.uint32))
+    assert np.array_equal(q, q0) and np.array_equal(sc.view(np.uint32), sc0.view(np.uint32))
+    ref = orc.gemv(Q4_K, wa, orc.rmsnorm(x, nw, 1e-5), 1280, k)
+    assert np.abs(ya - ref).max() <= 1e-3 * util.rms(ref)
 
 
 @pytest.mark.parametrize("dtype,k", [(Q4_0, 4096), (Q8_0, 4096), (Q4_0, 2048), (Q8_0, 1536), (Q4_1, 4096), (Q4_1, 1024)])

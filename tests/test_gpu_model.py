@@ -113,6 +113,28 @@ def test_greedy_free_running_prefix(tiny):
     assert n_same >= 2
 
 
+def test_wide_model_decodes_through_the_two_pass_row_kernels(hip, orc):
+    """hidden 5120 (a 13B-class width: 80 units of 64 weights, two passes per lane) and a 13824-wide
+    feed-forward block (the long-row kernel's four passes): the decode step takes the same fused
+    launches as at 4096, its logits agree with the oracle's forward and carry the same bits with
+    and without decode copies."""
+    cfg = dict(synth.TINY, hidden=5120, ffn=13824, n_heads=8, n_kv_heads=2, head_dim=128, n_layers=1, vocab=384, max_seq_len=64)
+    weights = synth.make_llama(cfg, seed=77, sigma=0.03, norm_jitter=0.1, n_threads=16)
+    a = hip_api.Model(hip, cfg, weights)
+    hip.set_decode_copies(False)
+    try:
+        b = hip_api.Model(hip, cfg, weights)
+    finally:
+        hip.set_decode_copies(True)
+    om = orc.Llama(cfg, weights)
+    _say("model: hidden 5120, ffn 13824")
+    for pos, tok in enumerate([5, 17, 301, 42]):
+        la, lb, lo = a.forward(tok, pos), b.forward(tok, pos), om.forward(tok, pos)
+        assert np.array_equal(la.view(np.uint32), lb.view(np.uint32))
+        assert _cos(la, lo) > 0.9999 and np.abs(la - lo).max() <= 0.1 * util.rms(lo), (pos, _cos(la, lo))
+    a.close(); b.close(); om.close()
+
+
 def test_greedy_token_is_the_argmax_of_the_same_logits(hip):
     """forward_greedy's second argmax stage writes the token into pinned host memory, which the host
     reads after the stream has drained: step by step it must return exactly the argmax (strict >,
