@@ -614,7 +614,8 @@ struct AttnLaunch {
     uint32_t seq_len, max_seq;
     float scale;
     uint32_t n_heads, n_kv_heads, n_queries, q_stride, G, S, n_parts, part_keys, chunks_per_part;
-    bool batch, fused_new_kv, split_heads;
+    uint32_t Gw;   // query heads one decode wavefront serves (divides G); G / Gw wavefronts share a kv head's rows
+    bool batch, fused_new_kv;
     AttnNewKV nk;
     float *acc, *ml;   // split-K partials: (o) and (m, l) per (query, head, part)
 };
@@ -666,10 +667,14 @@ static void attn_launch_partials(cera_hip_ctx* ctx, const AttnLaunch& a, const K
 #define ATTN_PF(GG)                                                                                                        \
     hipLaunchKernelGGL((attn_prefill_partial_kernel<KV, HD, GG>), pgrid, dim3(64 * GG), 0, ctx->stream, a.q, kc, vc, a.seq_len, \
                        a.n_queries, a.max_seq, a.scale, a.part_keys, a.n_parts, a.q_stride, a.acc, a.ml)
-        switch (a.G) {
+        switch (a.G) {   // any group of up to eight heads: one wavefront per head, 64 G threads
             case 1: ATTN_PF(1); break;
             case 2: ATTN_PF(2); break;
+            case 3: ATTN_PF(3); break;
             case 4: ATTN_PF(4); break;
+            case 5: ATTN_PF(5); break;
+            case 6: ATTN_PF(6); break;
+            case 7: ATTN_PF(7); break;
             default: ATTN_PF(8); break;
         }
 #undef ATTN_PF
@@ -686,18 +691,14 @@ static void attn_launch_partials(cera_hip_ctx* ctx, const AttnLaunch& a, const K
     // keys (20000 keys: 30.4 -> 24.3 us; 65536: 58.4 unsplit, 62.0 split).  Groups of 8 heads do
     // twice the arithmetic per K/V byte and are never bound by bytes: they keep the split at every
     // length (64 / 8 heads, 131072 keys: 279.5 -> 207.3 us; f16 cache, 32768 keys: 91.0 -> 54.5).
-    const bool split_heads = a.split_heads;
-    switch (a.G) {
+    // Group sizes that are not powers of two (Qwen2's 28 / 4 and 12 / 2 heads) run the widest
+    // instance that divides them -- seven one-head wavefronts, three two-head ones -- sharing the
+    // kv head's rows the same way.
+    switch (a.Gw) {
         case 1: attn_launch_decode_g<1, KV, HD>(ctx, a, kc, vc); break;
         case 2: attn_launch_decode_g<2, KV, HD>(ctx, a, kc, vc); break;
-        case 4:
-            if (split_heads) attn_launch_decode_g<2, KV, HD>(ctx, a, kc, vc);
-            else attn_launch_decode_g<4, KV, HD>(ctx, a, kc, vc);
-            break;
-        default:
-            if (split_heads) attn_launch_decode_g<4, KV, HD>(ctx, a, kc, vc);
-            else attn_launch_decode_g<8, KV, HD>(ctx, a, kc, vc);
-            break;
+        case 4: attn_launch_decode_g<4, KV, HD>(ctx, a, kc, vc); break;
+        default: attn_launch_decode_g<8, KV, HD>(ctx, a, kc, vc); break;
     }
 }
 
@@ -709,7 +710,7 @@ cera_hip_status cera_launch_attn(cera_hip_ctx* ctx, const float* q, const void* 
     if (head_dim != 64 && head_dim != 128) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "attention: head_dim must be 64 or 128");
     if (n_kv_heads == 0 || n_heads % n_kv_heads) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "attention: n_heads must be a multiple of n_kv_heads");
     uint32_t G = n_heads / n_kv_heads;
-    if (G != 1 && G != 2 && G != 4 && G != 8) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "attention: group size must be 1, 2, 4 or 8");
+    if (G > 8) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "attention: at most 8 query heads per kv head");
     if (n_queries == 0 || n_queries > 65535) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "attention: 1..65535 queries per call");
     // seq_len = keys visible to the first query; the last query sees seq_len + n_queries - 1
     const uint64_t last_len = seq_len + n_queries - 1;
@@ -723,7 +724,7 @@ cera_hip_status cera_launch_attn(cera_hip_ctx* ctx, const float* q, const void* 
     const AttnNewKV nk = new_kv ? *new_kv : AttnNewKV{};
     uint32_t n_parts, part_keys = 0, chunks_per_part = 0;
     uint32_t S = 1;
-    bool split_heads = false;
+    uint32_t Gw = G;   // decode: heads per wavefront
     if (batch) {
         const uint64_t want = n_queries >= 1024 ? 4 : 8;   // many query blocks fill the chip with fewer parts
         part_keys = last_len <= 1024 ? 128u : static_cast<uint32_t>(((last_len + want - 1) / want + 31) / 32 * 32);
@@ -734,10 +735,14 @@ cera_hip_status cera_launch_attn(cera_hip_ctx* ctx, const float* q, const void* 
         // the 32/8/128 shape over rotating caches; with a kv head's query heads split over two
         // wavefronts (attn_launch_partials) 32-key chunks are best from 1024 keys up to where the split
         // ends: 64-key chunks take one wavefront per SIMD (registers) and lose 2-3 us from 8k to 16k keys.
-        split_heads = G >= 4 && (G == 8 || last_len < (kv_f16 ? 32768u : 16384u));   // attn_launch_partials has the reasons
+        // heads per wavefront: attn_launch_partials has the reasons
+        if (G == 8 || (G == 4 && last_len < (kv_f16 ? 32768u : 16384u))) Gw = G / 2;
+        else if (G == 6) Gw = 2;
+        else if (G == 3 || G == 5 || G == 7) Gw = 1;
+        const bool split_heads = Gw != G;
         if (split_heads) S = last_len >= ATTN_FUSED_NEW_KV_MAX_KEYS ? 4 : 1;
         else S = last_len >= 8192 ? 8 : (last_len >= 2048 ? 4 : (last_len >= ATTN_FUSED_NEW_KV_MAX_KEYS ? 2 : 1));
-        if (G == 8 && S == 8) S = 4;   // eight heads x 64 positions per chunk does not fit the register file
+        if (Gw == 8 && S == 8) S = 4;   // eight heads x 64 positions per chunk does not fit the register file
         uint32_t n_chunks = static_cast<uint32_t>((last_len + 8 * S - 1) / (8 * S));
         // parts (wavefronts) per (query, kv head): enough to fill the chip ~4 waves per CU deep
         // (more parts make the partial kernel shorter but the merge longer: measured best from 2k
@@ -756,7 +761,7 @@ cera_hip_status cera_launch_attn(cera_hip_ctx* ctx, const float* q, const void* 
             // 9216 keys, f32: 31.2 -> 21.9 us together with the kernel's launch-index mapping, 13824:
             // 37.2 -> 27.9; f16: 8192 keys 16.3 -> 13.9.  Within 4 % of the best (chunk, parts) pair
             // of a sweep at every length from 1k to 16k keys (f32) and of a parts sweep (f16).
-            const uint32_t subs = split_heads ? 2 : 1;
+            const uint32_t subs = G / Gw;
             uint64_t best = ~0ull;
             const uint32_t first = chunks_per_part;
             for (uint32_t cpp = first; cpp <= n_chunks; ++cpp) {
@@ -803,7 +808,7 @@ cera_hip_status cera_launch_attn(cera_hip_ctx* ctx, const float* q, const void* 
         ml = ctx->attn_ml;
     }
     AttnLaunch a{q, static_cast<uint32_t>(seq_len), static_cast<uint32_t>(max_seq), scale, n_heads, n_kv_heads, n_queries,
-                 n_heads * head_dim, G, S, n_parts, part_keys, chunks_per_part, batch, new_kv != nullptr, split_heads, nk, acc, ml};
+                 n_heads * head_dim, G, S, n_parts, part_keys, chunks_per_part, Gw, batch, new_kv != nullptr, nk, acc, ml};
     const kv_half *kh = static_cast<const kv_half*>(kc), *vh = static_cast<const kv_half*>(vc);
     const float *kf = static_cast<const float*>(kc), *vf = static_cast<const float*>(vc);
     if (head_dim == 128) {

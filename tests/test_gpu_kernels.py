@@ -308,10 +308,8 @@ def test_attn_decode_peaked_softmax(hip, orc):
 
 def test_attn_decode_gqa_groupings(hip, orc):
     hd, L = 128, 130
-    for nh, nkv in [(8, 8), (8, 4), (16, 2), (4, 1)]:
+    for nh, nkv in [(8, 8), (8, 4), (16, 2), (4, 1), (28, 4), (12, 2), (6, 2), (5, 1)]:
         _say(f"attn_decode nh={nh} nkv={nkv}")
-        if nh // nkv not in (1, 2, 4, 8):
-            continue
         q = util.make_x(nh * hd, 90)
         k = util.make_x(L * nkv * hd, 91)
         v = util.make_x(L * nkv * hd, 92)
@@ -322,13 +320,17 @@ def test_attn_decode_gqa_groupings(hip, orc):
 
 @pytest.mark.parametrize("nh,nkv,L,n", [(32, 8, 1100, 1), (32, 8, 4200, 1), (32, 8, 9000, 1), (24, 3, 1500, 1), (40, 5, 2300, 1),
                                          (16, 2, 700, 1), (8, 1, 3000, 1), (14, 7, 900, 1), (32, 8, 1200, 5), (24, 3, 2100, 3),
-                                         (8, 8, 333, 7), (64, 8, 5000, 2), (16, 2, 17000, 1), (8, 1, 33000, 1)])
+                                         (8, 8, 333, 7), (64, 8, 5000, 2), (16, 2, 17000, 1), (8, 1, 33000, 1),
+                                         (28, 4, 3000, 1), (28, 4, 700, 3), (12, 2, 9000, 1), (14, 2, 18000, 1), (6, 2, 1500, 5),
+                                         (5, 1, 2500, 1), (28, 4, 200, 40), (12, 2, 1000, 33)])
 def test_attn_decode_workgroup_mapping_covers_every_part(hip, orc, nh, nkv, L, n):
     """The partial kernel maps launch indices to (kv head, key range, sub-group of heads, query)
     XCD by XCD and rounds the launch up to whole eights: kv-head counts that do not divide eight,
     part counts that are not multiples of four, both head sub-groups (groups of eight heads keep
-    them at every length) and small query batches must all reach every (head, query), against the
-    oracle query by query."""
+    them at every length), group sizes that are not powers of two (Qwen2's 28 / 4 and 12 / 2 heads:
+    seven one-head or three two-head wavefronts per kv head; a batch of 16 or more queries takes the
+    tiled kernel with one wavefront per head) and small query batches must all reach every
+    (head, query), against the oracle query by query."""
     hd = 128
     _say(f"attn workgroup mapping nh={nh} nkv={nkv} L={L} n={n}")
     r = util.rng(31 * L + nh + n)

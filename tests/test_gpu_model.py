@@ -383,6 +383,31 @@ def test_head_dim_64_model_parity(hip, orc, rope_type, kv_f16):
     gm.close(); om.close()
 
 
+@pytest.mark.parametrize("n_heads,n_kv,hd", [(14, 2, 128), (12, 2, 128), (12, 4, 64), (28, 4, 64)])
+def test_odd_head_group_model_parity(hip, orc, n_heads, n_kv, hd):
+    """Qwen2-style head counts (28 / 4, 12 / 2, 14 / 2: seven or six query heads per kv head): a batched
+    prefill, greedy decode steps and the KV cache against the oracle."""
+    cfg = dict(synth.TINY, hidden=n_heads * hd, n_heads=n_heads, n_kv_heads=n_kv, head_dim=hd, ffn=768, rope_type=1)
+    weights = synth.make_llama(cfg, seed=131 + n_heads, sigma=0.05, norm_jitter=0.1)
+    gm = hip_api.Model(hip, cfg, weights)
+    om = orc.Llama(cfg, weights)
+    _say(f"model with {n_heads}/{n_kv} heads of {hd}")
+    toks = [int(t) for t in util.rng(132).integers(0, cfg["vocab"], 21)]
+    lg, lo = gm.forward_prefill(toks, 0), om.forward_prefill_batched(toks, 0)
+    assert _cos(lg, lo) > 0.999
+    same = 0
+    for i in range(10):
+        tg, to = int(orc_argmax(lg)), int(orc_argmax(lo))
+        same += tg == to
+        lg, lo = gm.forward(to, 21 + i), om.forward(to, 21 + i)
+        assert _cos(lg, lo) > 0.999, i
+    assert same >= 8
+    kg, vg = gm.read_kv(0)
+    ko, vo = om.kv(0)
+    assert np.abs(kg - ko).max() <= 3e-3 * util.rms(ko) and np.abs(vg - vo).max() <= 3e-3 * util.rms(vo)
+    gm.close(); om.close()
+
+
 def test_head_dim_64_shift_bitwise(hip, orc):
     from test_oracle_kv_shift import rope_filled_cache
     for rope_type in (0, 1):
