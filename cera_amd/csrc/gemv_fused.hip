@@ -97,21 +97,34 @@ cera_hip_status cera_launch_ffn_gate_up_fused(cera_hip_ctx* ctx, const cera_hip_
     RowGemvArgs a;
     // 16 wavefronts x 4 rows: a workgroup owns two Q8_0 blocks of the output, and 14336 rows make
     // 224 workgroups -- one per CU in a single wave of the launch (448 eight-wavefront workgroups
-    // leave a quarter of the CUs with half the others' share: 1 % slower end to end).  Q4_K rows of
-    // two passes per lane (4096 < k <= 8192) hold twice the weights and activations per lane and
-    // take 8 wavefronts (one Q8_0 block of the output per workgroup).
-    constexpr int GATE_UP_NW = 16, ROWS = 4, WIDE_NW = 8, WIDE_ROWS = 8;
+    // leave a quarter of the CUs with half the others' share: 1 % slower end to end).  A CU runs
+    // one of these workgroups at a time, so a matrix of more than 64 n_cu rows takes 6 or 8 rows per
+    // wavefront rather than a second round (Q4_K 18944 x 3584: 296 workgroups 23.0 us; 17408 rows
+    // the same, 16384 rows 13.8).  Q4_K rows of two passes per lane (4096 < k <= 8192) hold twice
+    // the weights and activations per lane and take 8 wavefronts of 8 rows.
+    constexpr int GATE_UP_NW = 16, WIDE_NW = 8, WIDE_ROWS = 8;
     const bool stream = gate->dev_stream && up->dev_stream;
     const bool wide = gate->dtype == CERA_HIP_Q4_K && tiles == 2;
-    fill(a, gate, up, wide ? WIDE_ROWS : ROWS, stream);
+    uint32_t rows = 4;
+    if (!wide && gate->dtype == CERA_HIP_Q4_K) {   // the instance with the fewest rows per wavefront x rounds
+        uint64_t best = ~0ull;
+        for (uint32_t r : {4u, 6u, 8u}) {
+            const uint64_t wgs = (gate->m + GATE_UP_NW * r - 1) / (GATE_UP_NW * r);
+            const uint64_t cost = r * ((wgs + ctx->n_cu - 1) / ctx->n_cu);
+            if (cost <= best) { best = cost; rows = r; }   // of equals the one with fewer rounds
+        }
+    }
+    if (wide) rows = WIDE_ROWS;
+    fill(a, gate, up, rows, stream);
     a.x = x; a.norm_w = norm_w; a.eps = eps; a.out_q = out_q; a.out_s = out_s;
-    const uint32_t nw = wide ? WIDE_NW : GATE_UP_NW, per_wg = wide ? WIDE_NW * WIDE_ROWS : GATE_UP_NW * ROWS;
+    const uint32_t nw = wide ? WIDE_NW : GATE_UP_NW, per_wg = nw * rows;
     const dim3 grid((a.m + per_wg - 1) / per_wg), block(64 * nw);
-#define GATE_UP_LAUNCH(TT, TL)                                                                                                          \
+#define GATE_UP_LAUNCH_R(TT, TL, RR)                                                                                                    \
     do {                                                                                                                                \
-        if (stream) hipLaunchKernelGGL((row_gemv_kernel<TT, GATE_UP_NW, ROWS, true, FEPI_SILU_Q8, true, TL>), grid, block, 0, ctx->stream, a); \
-        else hipLaunchKernelGGL((row_gemv_kernel<TT, GATE_UP_NW, ROWS, true, FEPI_SILU_Q8, false, TL>), grid, block, 0, ctx->stream, a);   \
+        if (stream) hipLaunchKernelGGL((row_gemv_kernel<TT, GATE_UP_NW, RR, true, FEPI_SILU_Q8, true, TL>), grid, block, 0, ctx->stream, a); \
+        else hipLaunchKernelGGL((row_gemv_kernel<TT, GATE_UP_NW, RR, true, FEPI_SILU_Q8, false, TL>), grid, block, 0, ctx->stream, a);   \
     } while (0)
+#define GATE_UP_LAUNCH(TT, TL) GATE_UP_LAUNCH_R(TT, TL, 4)
 #define GATE_UP_LAUNCH_B32(TT)            \
     do {                                  \
         if (tiles == 1) GATE_UP_LAUNCH(TT, 1); \
@@ -120,10 +133,15 @@ cera_hip_status cera_launch_ffn_gate_up_fused(cera_hip_ctx* ctx, const cera_hip_
     if (wide) {
         if (stream) hipLaunchKernelGGL((row_gemv_kernel<Q4K, WIDE_NW, WIDE_ROWS, true, FEPI_SILU_Q8, true, 2, 8192>), grid, block, 0, ctx->stream, a);
         else hipLaunchKernelGGL((row_gemv_kernel<Q4K, WIDE_NW, WIDE_ROWS, true, FEPI_SILU_Q8, false, 2, 8192>), grid, block, 0, ctx->stream, a);
-    } else if (gate->dtype == CERA_HIP_Q4_K) GATE_UP_LAUNCH(Q4K, 1);
+    } else if (gate->dtype == CERA_HIP_Q4_K) {
+        if (rows == 4) GATE_UP_LAUNCH_R(Q4K, 1, 4);
+        else if (rows == 6) GATE_UP_LAUNCH_R(Q4K, 1, 6);
+        else GATE_UP_LAUNCH_R(Q4K, 1, 8);
+    }
     else if (gate->dtype == CERA_HIP_Q4_0) GATE_UP_LAUNCH_B32(Q4_0);
     else if (gate->dtype == CERA_HIP_Q4_1) GATE_UP_LAUNCH_B32(Q4_1);
     else GATE_UP_LAUNCH_B32(Q8_0);
+#undef GATE_UP_LAUNCH_R
 #undef GATE_UP_LAUNCH_B32
 #undef GATE_UP_LAUNCH
     HIP_TRY(ctx, hipGetLastError());

@@ -570,7 +570,7 @@ def test_qkv_fused_norm_projection(hip, orc, ma, mb, k, tb):
         assert np.abs(yb - rb).max() <= 1e-3 * util.rms(rb)
 
 
-@pytest.mark.parametrize("m,k", [(14336, 4096), (512, 256), (96, 2048), (32, 4096)])
+@pytest.mark.parametrize("m,k", [(14336, 4096), (512, 256), (96, 2048), (32, 4096), (18944, 512), (28672, 256)])
 def test_ffn_gate_up_fused_against_the_oracle(hip, orc, m, k):
     """FFN norm + Q8_0 + gate | up + SwiGLU + Q8_0 of the result in one launch, against the oracle's
     chain rmsnorm -> gemv x 2 -> silu_mul -> quantize.  The projections agree with the oracle's to
