@@ -106,7 +106,7 @@ cera_hip_status cera_launch_ffn_gate_up_fused(cera_hip_ctx* ctx, const cera_hip_
     const bool stream = gate->dev_stream && up->dev_stream;
     const bool wide = gate->dtype == CERA_HIP_Q4_K && tiles == 2;
     uint32_t rows = 4;
-    if (!wide && gate->dtype == CERA_HIP_Q4_K) {   // the instance with the fewest rows per wavefront x rounds
+    if (!wide) {   // the instance with the fewest rows per wavefront x rounds
         uint64_t best = ~0ull;
         for (uint32_t r : {4u, 6u, 8u}) {
             const uint64_t wgs = (gate->m + GATE_UP_NW * r - 1) / (GATE_UP_NW * r);
@@ -124,7 +124,12 @@ cera_hip_status cera_launch_ffn_gate_up_fused(cera_hip_ctx* ctx, const cera_hip_
         if (stream) hipLaunchKernelGGL((row_gemv_kernel<TT, GATE_UP_NW, RR, true, FEPI_SILU_Q8, true, TL>), grid, block, 0, ctx->stream, a); \
         else hipLaunchKernelGGL((row_gemv_kernel<TT, GATE_UP_NW, RR, true, FEPI_SILU_Q8, false, TL>), grid, block, 0, ctx->stream, a);   \
     } while (0)
-#define GATE_UP_LAUNCH(TT, TL) GATE_UP_LAUNCH_R(TT, TL, 4)
+#define GATE_UP_LAUNCH(TT, TL)                     \
+    do {                                           \
+        if (rows == 4) GATE_UP_LAUNCH_R(TT, TL, 4); \
+        else if (rows == 6) GATE_UP_LAUNCH_R(TT, TL, 6); \
+        else GATE_UP_LAUNCH_R(TT, TL, 8);          \
+    } while (0)
 #define GATE_UP_LAUNCH_B32(TT)            \
     do {                                  \
         if (tiles == 1) GATE_UP_LAUNCH(TT, 1); \
@@ -133,11 +138,7 @@ cera_hip_status cera_launch_ffn_gate_up_fused(cera_hip_ctx* ctx, const cera_hip_
     if (wide) {
         if (stream) hipLaunchKernelGGL((row_gemv_kernel<Q4K, WIDE_NW, WIDE_ROWS, true, FEPI_SILU_Q8, true, 2, 8192>), grid, block, 0, ctx->stream, a);
         else hipLaunchKernelGGL((row_gemv_kernel<Q4K, WIDE_NW, WIDE_ROWS, true, FEPI_SILU_Q8, false, 2, 8192>), grid, block, 0, ctx->stream, a);
-    } else if (gate->dtype == CERA_HIP_Q4_K) {
-        if (rows == 4) GATE_UP_LAUNCH_R(Q4K, 1, 4);
-        else if (rows == 6) GATE_UP_LAUNCH_R(Q4K, 1, 6);
-        else GATE_UP_LAUNCH_R(Q4K, 1, 8);
-    }
+    } else if (gate->dtype == CERA_HIP_Q4_K) GATE_UP_LAUNCH(Q4K, 1);
     else if (gate->dtype == CERA_HIP_Q4_0) GATE_UP_LAUNCH_B32(Q4_0);
     else if (gate->dtype == CERA_HIP_Q4_1) GATE_UP_LAUNCH_B32(Q4_1);
     else GATE_UP_LAUNCH_B32(Q8_0);

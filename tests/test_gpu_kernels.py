@@ -690,6 +690,23 @@ def test_fused_launches_stream_the_decode_copy_to_the_same_bits(hip, no_decode_c
     assert np.array_equal(q, q0) and np.array_equal(sc.view(np.uint32), sc0.view(np.uint32))
 
 
+@pytest.mark.parametrize("dtype,k", [(Q4_K, 256), (Q4_0, 64), (Q4_1, 96), (Q8_0, 2080)])
+@pytest.mark.parametrize("m", [18944, 28672])
+def test_gate_up_fused_on_tall_matrices(hip, dtype, k, m):
+    """Beyond 64 rows x the CU count the gate|up launch takes 6 (18944 rows) or 8 (28672 rows) rows per
+    wavefront instead of a second round of workgroups: bitwise what the separate launches compute,
+    for every fused type and for one and two passes per lane."""
+    _say(f"gate|up on {m} rows {util.NAMES[dtype]} k={k}")
+    wg, _ = util.make_weights(dtype, m, k, seed=121)
+    wu, _ = util.make_weights(dtype, m, k, seed=122)
+    x = util.make_x(k, 123) * np.float32(1.3)
+    nw = (1.0 + 0.1 * util.make_x(k, 124)).astype(np.float32)
+    q, sc = hip.ffn_gate_up_fused(wg, wu, m, k, x, nw, 1e-5, dtype)
+    n, _, _ = hip.rmsnorm_q8_0(x, nw, 1e-5)
+    rs, rq = hip.quantize_q8_0(hip.silu_mul(hip.gemv(dtype, wg, n, m, k), hip.gemv(dtype, wu, n, m, k)))
+    assert np.array_equal(q, rq) and np.array_equal(sc.view(np.uint32), rs.view(np.uint32))
+
+
 @pytest.mark.parametrize("k,tb", [(8192, Q6_K), (5120, Q4_K), (6144, Q6_K)])
 def test_fused_launches_for_rows_of_two_passes(hip, orc, no_decode_copies, k, tb):
     """K-quant rows of 4096 < k <= 8192 (the hidden sizes of the 13B - 70B models) take the same fused
