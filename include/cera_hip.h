@@ -227,7 +227,10 @@ CERA_HIP_API cera_hip_status cera_hip_gemm_swiglu(cera_hip_ctx*, const cera_hip_
  * 3222-3363, 2617-2633).  q f32[n_heads*head_dim]; k, v f32 time-major
  * [seq_len][n_kv_heads*head_dim] (cera/src/kv_cache.rs:201-212);
  * out f32[n_heads*head_dim]; all seq_len positions visible.
- * n_splits = 0 lets the library choose the split-K factor. */
+ * n_splits = 0 lets the library choose the split-K factor.
+ * head_dim 64 or 128; n_heads a multiple of n_kv_heads, at most 8 query heads per kv head
+ * (any count: 28 / 4 and 12 / 2 included); anything else is CERA_HIP_ERR_SHAPE.  The same holds
+ * for every attention entry below. */
 CERA_HIP_API cera_hip_status cera_hip_attn_decode(cera_hip_ctx*, const float* q, const float* k, const float* v,
                                                   uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim,
                                                   uint64_t seq_len, float scale, uint32_t n_splits, float* out);
