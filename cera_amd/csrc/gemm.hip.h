@@ -443,7 +443,8 @@ static __global__ __launch_bounds__(256, T::WAVES_PER_SIMD) void gemm_kernel(Gem
 // Sums the split-K partials in a fixed order: out[e] = (resid[e] +) sum_z part[z][e].
 static __global__ __launch_bounds__(256) void gemm_reduce_kernel(const float* __restrict__ part, uint32_t n_split,
                                                           uint64_t stride, uint64_t n4, float* __restrict__ out,
-                                                          const float* resid, float resid_scale) {
+                                                          const float* resid, float resid_scale, uint64_t n4_first,
+                                                          float* __restrict__ out2) {
     const uint64_t e = static_cast<uint64_t>(blockIdx.x) * 256 + threadIdx.x;
     if (e >= n4) return;
     float4 s = reinterpret_cast<const float4*>(part)[e];
@@ -451,6 +452,8 @@ static __global__ __launch_bounds__(256) void gemm_reduce_kernel(const float* __
         const float4 v = reinterpret_cast<const float4*>(part + z * stride)[e];
         s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
     }
+    // a pair's partials lie side by side; the second matrix's sums go to its own output
+    if (e >= n4_first) { reinterpret_cast<float4*>(out2)[e - n4_first] = s; return; }
     if (resid) {
         const float4 r = reinterpret_cast<const float4*>(resid)[e];
         if (resid_scale != 1.0f) { s.x *= resid_scale; s.y *= resid_scale; s.z *= resid_scale; s.w *= resid_scale; }

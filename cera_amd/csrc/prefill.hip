@@ -100,8 +100,9 @@ cera_hip_status cera_launch_gemm(cera_hip_ctx* ctx, const cera_hip_dtensor* w, c
     if (!dbg_dots && wgs < 2 * ctx->n_cu && nsb >= 8 && dense && (static_cast<uint64_t>(a.m) * n) % 4 == 0) {
         // smallest divisor of the super-block count that gives at least two workgroups per CU
         const uint32_t want = std::min<uint32_t>(8, (2 * ctx->n_cu + wgs - 1) / wgs);
+        // (a slice keeps at least two super-blocks: below that the tile's prologue outweighs its K loop)
         for (uint32_t d = 2; d <= 8 && split < want; ++d)
-            if (nsb % d == 0 && nsb / d >= 4) split = d;
+            if (nsb % d == 0 && nsb / d >= 2) split = d;
     }
     a.k_chunk = a.k / split;
     a.part_stride = 0;
@@ -136,14 +137,9 @@ cera_hip_status cera_launch_gemm(cera_hip_ctx* ctx, const cera_hip_dtensor* w, c
         case CERA_HIP_Q4_1: hipLaunchKernelGGL((gemm_kernel<GemmQ4_1>), grid, dim3(256), 0, ctx->stream, a); break;
         default: hipLaunchKernelGGL((gemm_kernel<GemmQ8_0>), grid, dim3(256), 0, ctx->stream, a); break;
     }
-    if (split > 1) {
-        hipLaunchKernelGGL(gemm_reduce_kernel, dim3(static_cast<uint32_t>((mn / 4 + 255) / 256)), dim3(256), 0, ctx->stream,
-                           a.out, split, a.part_stride, mn / 4, out, resid, resid_scale);
-        if (a.w2)
-            hipLaunchKernelGGL(gemm_reduce_kernel, dim3(static_cast<uint32_t>((mn2 / 4 + 255) / 256)), dim3(256), 0,
-                               ctx->stream, a.out2, split, a.part_stride, mn2 / 4, out2, static_cast<const float*>(nullptr),
-                               1.0f);
-    }
+    if (split > 1)   // one launch reduces both matrices of a pair
+        hipLaunchKernelGGL(gemm_reduce_kernel, dim3(static_cast<uint32_t>(((mn + mn2) / 4 + 255) / 256)), dim3(256), 0,
+                           ctx->stream, a.out, split, a.part_stride, (mn + mn2) / 4, out, resid, resid_scale, mn / 4, out2);
     HIP_TRY(ctx, hipGetLastError());
     return CERA_HIP_OK;
 }
