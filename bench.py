@@ -35,7 +35,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 # `bench.py --pmc-probe` under rocprofv3 --pmc, summary in profiles/gemv_q4k_gate_up_hbm_traffic_pmc.txt).
 # It is a recorded measurement of this kernel configuration, not taken live: counters need the profiler.
 GATE_UP_TRAFFIC_BYTES = 66_481_099
-GATE_UP_KERNEL = "row_gemv_kernel<Q4K,16,4,true,2,true,1>"
+GATE_UP_KERNEL = "row_gemv_kernel<Q4K,16,4,true,2,true,1,4096>"
 
 # (name, ggml type name, m, k, copies per step)
 LAYER_SET = [
