@@ -81,6 +81,8 @@ struct GemmArgs {
     // debug instances only: the integer dot of every (row, token, block) as the matrix core
     // delivered it, [m][n][k/32] int32 (Q6_K: [m][n][k/16], f32 bit patterns of the f16 MFMA's result)
     int32_t* dbg_dots;
+    // fp8 kernel (gemm_fp8.hip.h) only: the activations' fragment-ordered split copy
+    const uint8_t* bf8;
 };
 
 // ---- per-type staging of one 128-element K tile of one row -------------------

@@ -36,8 +36,8 @@ struct cera_hip_ctx {
     // with host buffers, and every model-level call of any model on this context)
     std::recursive_mutex op_mu;
     // grow-only device scratch for the host-pointer entry points
-    void* scratch[12] = {nullptr};
-    uint64_t scratch_bytes[12] = {0};
+    void* scratch[16] = {nullptr};
+    uint64_t scratch_bytes[16] = {0};
     void* static_scratch = nullptr;   // this device's copy of the library's fixed workspace (resolved at creation)
     // optional standalone code object (cera_hip_ctx_create with an hsaco_path): the quantizer and the
     // GEMV instances it exports are then launched from it with hipModuleLaunchKernel

@@ -38,6 +38,7 @@ struct cera_hip_model {
     float *pf_hidden = nullptr, *pf_normed = nullptr, *pf_q = nullptr, *pf_k = nullptr, *pf_v = nullptr,
           *pf_attn = nullptr, *pf_gate = nullptr, *pf_up = nullptr, *pf_xs = nullptr, *pf_bsum = nullptr;
     int8_t* pf_xq = nullptr;
+    void* pf_x8 = nullptr;   // the same activations as the fragment-ordered fp8 split copy (Q4_K GEMMs)
     void* pf_xh = nullptr;   // the same quants as f16 (Q6_K GEMMs run their dots on the f16 matrix cores)
     uint32_t* pf_tokens = nullptr;
     float* pf_logits = nullptr;   // [pf_cap][head rows], allocated on the first all-logits call

@@ -7,6 +7,7 @@
 
 #include "gemm_q5k_f16.hip.h"
 #include "gemm_q6k_f16.hip.h"
+#include "gemm_fp8.hip.h"
 #include "glue.hip.h"
 #include "model.h"
 
@@ -22,6 +23,9 @@ bool cera_gemm_supports(uint32_t dtype, uint64_t k) { return gemm_type_ok(dtype)
 static bool gemm_f32_supports(uint32_t dtype, uint64_t k) { return dtype == CERA_HIP_Q5_K && k % GEMM_KSUPER == 0 && k > 0; }
 static bool gemm_batched(uint32_t dtype, uint64_t k) { return cera_gemm_supports(dtype, k) || gemm_f32_supports(dtype, k); }
 
+// bytes of the fragment-ordered fp8 split copy of n activation rows of k elements
+uint64_t cera_gemm_fp8_ws_bytes(uint64_t n, uint64_t k) { return (n + G8_BN - 1) / G8_BN * 2 * (k / 256) * G8_REC; }
+
 // out[i*ld_m + j*ld_n] = (W . B)[i][j] (+ resid)
 // w2 / out2 (nullable): a second matrix of the same type and k multiplied by the same activations
 // in the same launch, out2[i*ld_m + j*ld_n2]; *paired says whether that happened (if not, the
@@ -31,7 +35,7 @@ cera_hip_status cera_launch_gemm(cera_hip_ctx* ctx, const cera_hip_dtensor* w, c
                                  const float* resid, float resid_scale, const cera_hip_dtensor* w2 = nullptr,
                                  float* out2 = nullptr, uint64_t ld_n2 = 0, bool* paired = nullptr, void* bh_ws = nullptr,
                                  bool* staged = nullptr, int32_t* dbg_dots = nullptr, const float* x_f32 = nullptr,
-                                 bool* staged_f32 = nullptr) {
+                                 bool* staged_f32 = nullptr, void* b8_ws = nullptr, bool* staged8 = nullptr) {
     // Q5_K: x_f32 [n][k] are the activations (bs / bq / bsum are not read); *staged_f32 (nullable)
     // says whether the context's split copy still holds exactly these activations
     const bool q5 = gemm_f32_supports(w->dtype, w->k);
@@ -63,6 +67,25 @@ cera_hip_status cera_launch_gemm(cera_hip_ctx* ctx, const cera_hip_dtensor* w, c
         }
         a.bh = bh_ws;
     }
+    // Q4_K runs its block dots on the fp8 matrix cores and reads the activations from their
+    // fragment-ordered split copy (gemm_fp8.hip.h): built here unless the caller says its workspace
+    // (b8_ws) still holds these activations (*staged8)
+    const bool fp8 = w->dtype == CERA_HIP_Q4_K;
+    a.bf8 = nullptr;
+    if (fp8) {
+        const uint32_t tiles = (n + G8_BN - 1) / G8_BN * 2, nsb = a.k / 256;
+        if (!b8_ws) {
+            CERA_TRY(cera_scratch(ctx, 12, cera_gemm_fp8_ws_bytes(n, a.k), &b8_ws));
+            staged8 = nullptr;
+        }
+        if (!staged8 || !*staged8) {
+            hipLaunchKernelGGL(gemm_act_fp8_kernel, dim3(tiles * nsb), dim3(256), 0, ctx->stream, bq, bs, bsum,
+                               static_cast<uint8_t*>(b8_ws), n, a.k);
+            if (staged8) *staged8 = true;
+        }
+        a.bf8 = static_cast<const uint8_t*>(b8_ws);
+    }
+    const uint32_t BM = fp8 ? G8_BM : GEMM_BM, BN = fp8 ? G8_BN : GEMM_BN;
     if (q5) {
         // hi | lo f16 halves of x and its f32 block sums, in one scratch allocation
         const uint64_t nk = static_cast<uint64_t>(n) * a.k;
@@ -81,14 +104,14 @@ cera_hip_status cera_launch_gemm(cera_hip_ctx* ctx, const cera_hip_dtensor* w, c
         a.bs = unscale;
         a.bsum = xsum;
     }
-    dim3 grid((n + GEMM_BN - 1) / GEMM_BN, (a.m + GEMM_BM - 1) / GEMM_BM);
+    dim3 grid((n + BN - 1) / BN, (a.m + BM - 1) / BM);
     a.w2 = nullptr; a.out2 = nullptr; a.m2 = 0; a.tiles1 = grid.y; a.ld_n2 = 0;
     if (paired) *paired = false;
     // a pair is taken when both outputs are token-major and dense (what the split-K reduction needs)
     if (w2 && !resid && w2->dtype == w->dtype && w2->k == w->k && w2->row_bytes == w->row_bytes && ld_m == 1 &&
         ld_n == w->m && ld_n2 == w2->m && (w->m * n) % 4 == 0 && (w2->m * n) % 4 == 0) {
         a.w2 = w2->dev; a.out2 = out2; a.m2 = static_cast<uint32_t>(w2->m); a.ld_n2 = ld_n2;
-        grid.y += static_cast<uint32_t>((w2->m + GEMM_BM - 1) / GEMM_BM);
+        grid.y += static_cast<uint32_t>((w2->m + BM - 1) / BM);
         if (paired) *paired = true;
     }
     // Few output tiles and a long K (the down projection at a few hundred tokens): split K over
@@ -120,7 +143,7 @@ cera_hip_status cera_launch_gemm(cera_hip_ctx* ctx, const cera_hip_dtensor* w, c
     if (dbg_dots) {
         // the same kernels, compiled to also store every block's integer tile (no K split, no pair)
         switch (w->dtype) {
-            case CERA_HIP_Q4_K: hipLaunchKernelGGL((gemm_kernel<GemmQ4K, false, true>), grid, dim3(256), 0, ctx->stream, a); break;
+            case CERA_HIP_Q4_K: hipLaunchKernelGGL((gemm_q4k_fp8_kernel<false, true>), grid, dim3(256), 0, ctx->stream, a); break;
             case CERA_HIP_Q6_K: hipLaunchKernelGGL(gemm_q6k_f16_kernel<true>, grid, dim3(256), 0, ctx->stream, a); break;
             case CERA_HIP_Q4_0: hipLaunchKernelGGL((gemm_kernel<GemmQ4_0, false, true>), grid, dim3(256), 0, ctx->stream, a); break;
             case CERA_HIP_Q4_1: hipLaunchKernelGGL((gemm_kernel<GemmQ4_1, false, true>), grid, dim3(256), 0, ctx->stream, a); break;
@@ -130,7 +153,7 @@ cera_hip_status cera_launch_gemm(cera_hip_ctx* ctx, const cera_hip_dtensor* w, c
         return CERA_HIP_OK;
     }
     switch (w->dtype) {
-        case CERA_HIP_Q4_K: hipLaunchKernelGGL((gemm_kernel<GemmQ4K>), grid, dim3(256), 0, ctx->stream, a); break;
+        case CERA_HIP_Q4_K: hipLaunchKernelGGL((gemm_q4k_fp8_kernel<false, false>), grid, dim3(256), 0, ctx->stream, a); break;
         case CERA_HIP_Q6_K: hipLaunchKernelGGL(gemm_q6k_f16_kernel<false>, grid, dim3(256), 0, ctx->stream, a); break;
         case CERA_HIP_Q5_K: hipLaunchKernelGGL(gemm_q5k_f16_kernel, grid, dim3(256), 0, ctx->stream, a); break;
         case CERA_HIP_Q4_0: hipLaunchKernelGGL((gemm_kernel<GemmQ4_0>), grid, dim3(256), 0, ctx->stream, a); break;
@@ -150,7 +173,7 @@ cera_hip_status cera_launch_gemm(cera_hip_ctx* ctx, const cera_hip_dtensor* w, c
 // need a K split to fill the chip; the caller then takes the GEMM pair and the SwiGLU kernel.
 cera_hip_status cera_launch_gemm_swiglu(cera_hip_ctx* ctx, const cera_hip_dtensor* gate, const cera_hip_dtensor* up,
                                         const float* bs, const int8_t* bq, const float* bsum, uint32_t n, int8_t* hq,
-                                        float* hs, float* hbsum, bool* fused) {
+                                        float* hs, float* hbsum, bool* fused, void* b8_ws = nullptr, bool* staged8 = nullptr) {
     *fused = false;
     if (!cera_gemm_supports(gate->dtype, gate->k) || gate->dtype == CERA_HIP_Q6_K || up->dtype != gate->dtype ||
         up->k != gate->k || up->m != gate->m || up->row_bytes != gate->row_bytes || gate->m % 32 || n == 0)
@@ -161,10 +184,24 @@ cera_hip_status cera_launch_gemm_swiglu(cera_hip_ctx* ctx, const cera_hip_dtenso
     a.row_bytes = static_cast<uint32_t>(gate->row_bytes);
     a.k_chunk = a.k;
     a.hq = hq; a.hs = hs; a.hbsum = hbsum;
-    const dim3 grid((n + GEMM_BN - 1) / GEMM_BN, (a.m + GEMM_BM / 2 - 1) / (GEMM_BM / 2));
+    const bool fp8 = gate->dtype == CERA_HIP_Q4_K;
+    const uint32_t BM = fp8 ? G8_BM : GEMM_BM, BN = fp8 ? G8_BN : GEMM_BN;
+    const dim3 grid((n + BN - 1) / BN, (a.m + BM / 2 - 1) / (BM / 2));
     if (grid.x * grid.y < 2 * ctx->n_cu) return CERA_HIP_OK;
+    if (fp8) {
+        if (!b8_ws) {
+            CERA_TRY(cera_scratch(ctx, 12, cera_gemm_fp8_ws_bytes(n, a.k), &b8_ws));
+            staged8 = nullptr;
+        }
+        if (!staged8 || !*staged8) {
+            hipLaunchKernelGGL(gemm_act_fp8_kernel, dim3((n + G8_BN - 1) / G8_BN * 2 * (a.k / 256)), dim3(256), 0, ctx->stream, bq, bs,
+                               bsum, static_cast<uint8_t*>(b8_ws), n, a.k);
+            if (staged8) *staged8 = true;
+        }
+        a.bf8 = static_cast<const uint8_t*>(b8_ws);
+    }
     switch (gate->dtype) {
-        case CERA_HIP_Q4_K: hipLaunchKernelGGL((gemm_kernel<GemmQ4K, true>), grid, dim3(256), 0, ctx->stream, a); break;
+        case CERA_HIP_Q4_K: hipLaunchKernelGGL((gemm_q4k_fp8_kernel<true, false>), grid, dim3(256), 0, ctx->stream, a); break;
         case CERA_HIP_Q4_0: hipLaunchKernelGGL((gemm_kernel<GemmQ4_0, true>), grid, dim3(256), 0, ctx->stream, a); break;
         case CERA_HIP_Q4_1: hipLaunchKernelGGL((gemm_kernel<GemmQ4_1, true>), grid, dim3(256), 0, ctx->stream, a); break;
         default: hipLaunchKernelGGL((gemm_kernel<GemmQ8_0, true>), grid, dim3(256), 0, ctx->stream, a); break;
@@ -393,6 +430,7 @@ static cera_hip_status ensure_prefill_buffers(cera_hip_model* m, uint32_t n) {
     CERA_TRY(alloc(cap * c.ffn * 4ull, reinterpret_cast<void**>(&m->pf_up)));
     CERA_TRY(alloc(cap * maxk, reinterpret_cast<void**>(&m->pf_xq)));
     CERA_TRY(alloc(cap * maxk * 2, &m->pf_xh));
+    CERA_TRY(alloc(cera_gemm_fp8_ws_bytes(cap, maxk), &m->pf_x8));
     CERA_TRY(alloc(cap * (maxk / 32) * 4, reinterpret_cast<void**>(&m->pf_xs)));
     CERA_TRY(alloc(cap * (maxk / 32) * 4, reinterpret_cast<void**>(&m->pf_bsum)));
     CERA_TRY(alloc(cap * 4ull, reinterpret_cast<void**>(&m->pf_tokens)));
@@ -420,10 +458,13 @@ static cera_hip_status prefill_chunk(cera_hip_model* m, const uint32_t* tokens, 
 
     // whether pf_xh holds the f16 form of the quants now in pf_xq; cleared wherever those are rewritten
     bool staged = false;
+    // the same for pf_x8, the fp8 split copy the Q4_K GEMMs read
+    bool staged8 = false;
     // the f32 activations whose hi / lo split (Q5_K GEMMs) the context's workspace holds now
     const float* split_of = nullptr;
     auto norm_rows = [&](const float* x, const float* w, float* y) -> cera_hip_status {
         staged = false;
+        staged8 = false;
         split_of = nullptr;
         hipLaunchKernelGGL((rmsnorm_kernel<true>), dim3(n), dim3(256), 0, s, x, w, hs, c.rms_eps, y, m->pf_xs, m->pf_xq,
                            m->pf_bsum);
@@ -443,7 +484,7 @@ static cera_hip_status prefill_chunk(cera_hip_model* m, const uint32_t* tokens, 
         }
         bool split_held = split_of == xf;
         CERA_TRY(cera_launch_gemm(ctx, w, m->pf_xs, m->pf_xq, m->pf_bsum, n, out, 1, w->m, resid, c.residual_scale, nullptr,
-                                  nullptr, 0, nullptr, m->pf_xh, &staged, nullptr, xf, &split_held));
+                                  nullptr, 0, nullptr, m->pf_xh, &staged, nullptr, xf, &split_held, m->pf_x8, &staged8));
         if (w->dtype == CERA_HIP_Q5_K) split_of = xf;
         return CERA_HIP_OK;
     };
@@ -456,7 +497,7 @@ static cera_hip_status prefill_chunk(cera_hip_model* m, const uint32_t* tokens, 
             bool paired = false;
             bool split_held = split_of == xf;
             CERA_TRY(cera_launch_gemm(ctx, wa, m->pf_xs, m->pf_xq, m->pf_bsum, n, outa, 1, wa->m, nullptr, 1.0f, wb, outb,
-                                      wb->m, &paired, m->pf_xh, &staged, nullptr, xf, &split_held));
+                                      wb->m, &paired, m->pf_xh, &staged, nullptr, xf, &split_held, m->pf_x8, &staged8));
             if (wa->dtype == CERA_HIP_Q5_K) split_of = xf;
             if (paired) return CERA_HIP_OK;
             return gemm(wb, outb, nullptr, xf);
@@ -497,6 +538,7 @@ static cera_hip_status prefill_chunk(cera_hip_model* m, const uint32_t* tokens, 
         CERA_TRY(cera_launch_attn(ctx, m->pf_q, L.kc, L.vc, c.n_heads, c.n_kv_heads, c.head_dim, start_pos + 1ull,
                                   c.max_seq_len, scale, 0, n, m->pf_attn, m->pf_xs, m->pf_xq, m->pf_bsum, nullptr, m->kv_f16));
         staged = false;   // the attention merge rewrote the quants
+        staged8 = false;
         split_of = nullptr;
         CERA_TRY(gemm(L.o, m->pf_hidden, m->pf_hidden, m->pf_attn));
 
@@ -508,12 +550,14 @@ static cera_hip_status prefill_chunk(cera_hip_model* m, const uint32_t* tokens, 
         int8_t* const hq = reinterpret_cast<int8_t*>(m->pf_gate);
         float *const hs = m->pf_up, *const hb = m->pf_up + static_cast<uint64_t>(n) * (c.ffn / 32);
         if (n > PREFILL_SMALL_BATCH && L.down->dtype != CERA_HIP_Q5_K)   // a Q5_K down projection reads the f32 SwiGLU output
-            CERA_TRY(cera_launch_gemm_swiglu(ctx, L.gate, L.up, m->pf_xs, m->pf_xq, m->pf_bsum, n, hq, hs, hb, &fused));
+            CERA_TRY(cera_launch_gemm_swiglu(ctx, L.gate, L.up, m->pf_xs, m->pf_xq, m->pf_bsum, n, hq, hs, hb, &fused, m->pf_x8, &staged8));
         staged = false;   // the down projection's activations are new either way
+        if (fused) staged8 = false;
         if (fused && cera_gemm_supports(L.down->dtype, L.down->k)) {
             CERA_TRY(cera_launch_gemm(ctx, L.down, hs, hq, hb, n, m->pf_hidden, 1, L.down->m, m->pf_hidden, c.residual_scale,
-                                      nullptr, nullptr, 0, nullptr, m->pf_xh, &staged));
-            staged = false;   // pf_xh now mirrors hq, not pf_xq
+                                      nullptr, nullptr, 0, nullptr, m->pf_xh, &staged, nullptr, nullptr, nullptr, m->pf_x8, &staged8));
+            staged = false;   // pf_xh / pf_x8 now mirror hq, not pf_xq
+            staged8 = false;
             continue;
         }
         if (fused) {   // a down projection without a GEMM reads pf_xq: move the quantized activations there
@@ -528,6 +572,7 @@ static cera_hip_status prefill_chunk(cera_hip_model* m, const uint32_t* tokens, 
             HIP_TRY(ctx, hipGetLastError());
             split_of = nullptr;
         }
+        staged8 = false;   // pf_xq holds the SwiGLU output now
         CERA_TRY(gemm(L.down, m->pf_hidden, m->pf_hidden, m->pf_gate));
     }
     m->seq_len = start_pos + n;
