@@ -13,30 +13,41 @@
 //     partial sum an integer below 2^24: no int->float convert on the vector ALU, one FMA per
 //     output and block (the 2^18 rides on the row scale, a power of two, so the product
 //     xs * (d*sc) and the FMA round exactly as before);
-//   * the weights never touch LDS.  A wavefront owns 64 rows for the whole K loop and loads its
-//     own rows' quant bytes straight into registers (a lane = one row and one half of a 32-byte
-//     chunk = 16 codes of block 2g in the low nibbles and 16 of block 2g+1 in the high ones);
-//     two AND/shift passes make both A operands.  Only the activations are shared between the
-//     wavefronts of a workgroup, and they arrive in LDS by DMA (global_load_lds_dwordx4) from a
-//     copy that the activation split kernel below wrote in exactly the order the MFMA wants
-//     them, so staging costs neither registers nor vector instructions and fragment reads are
-//     lane-contiguous (no bank conflicts);
+//   * nothing is unpacked into LDS and nothing staged costs a vector instruction.  A wavefront owns 32
+//     rows for the whole K loop; the bytes of its rows and the activations both reach LDS by DMA
+//     (global_load_lds_dwordx4, inline assembly with scalar addresses: two scalar instructions and
+//     the load per KB).  The weights arrive as 16-byte pieces in row order (consecutive lanes on
+//     consecutive pieces of a row: every cache line is fetched once) and a lane picks its row's header
+//     and its half of each 32-byte chunk (16 codes of block 2g in the low nibbles, 16 of block 2g+1
+//     in the high ones) out of the wavefront's private copy; two AND/shift passes make both A
+//     operands.  The activations come from a copy that the split kernel below wrote in exactly the
+//     order the MFMA wants them, so fragment reads are lane-contiguous (no bank conflicts);
 //   * the min terms run on the bf16 matrix core once per 256-element super-block: dmin*mn (17
 //     significant bits) and xs*sum(a) (24) are split exactly into three bf16 pieces each and the
 //     six products above 2^-24 of the term take six K slots per block, 48 per super-block, three
 //     v_mfma_f32_32x32x16_bf16 accumulating (negated) into the same tile as the dots.
 //
 // Workgroup: 256 threads = 4 wavefronts stacked along M; tile 128 rows x 64 tokens; a wavefront
-// owns 32 rows x 64 tokens (two MFMA tiles, 32 accumulator registers) and three workgroups share
-// a CU, so one wavefront's vector work overlaps another's matrix-core work on each SIMD.
-// K advances in stages of 128 elements, double-buffered in LDS with one barrier per stage.
+// owns 32 rows x 64 tokens (two MFMA tiles, 32 accumulator registers); two workgroups share a CU.
+// K advances in stages of 128 elements, double-buffered in LDS with one barrier per stage, and the
+// K loop is software-pipelined inside the wavefront (see the kernel).
+//
+// What bounds it: on this chip the matrix core and the vector ALU of a SIMD do not run at the same
+// time in a kernel of this kind (matrix-core busy + vector-ALU busy = 100 % of the dispatch, here as
+// in the int8 kernel), so the cost of a 32 x 32 x 32 tile step is the SUM of its MFMA clocks (64 dot +
+// 32 scale tile + 12 min terms) and its vector instructions (16 FMAs + about 12 of unpacking and
+// scale decoding, ~3 clocks each).  Against the int8 form (32 + 32 + 32 MFMA clocks, 16 converts + 16
+// FMAs + staging) that sum is what the fp8 dot lowers.
 #pragma once
 #include "gemm.hip.h"
 
 typedef int v8i __attribute__((ext_vector_type(8)));
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 
-#define G8_BM 128                 // rows per workgroup
+#ifndef G8_NW
+#define G8_NW 4                   // wavefronts per workgroup
+#endif
+#define G8_BM (32 * G8_NW)        // rows per workgroup
 #define G8_BN 64                  // tokens per workgroup
 #define G8_REC 21504              // bytes of the activation copy per (32-token tile, 256-element super-block)
 #define G8_REC_XS 16384           //   offset of the activation scales  [8 blocks][32 tokens] f32
@@ -118,17 +129,21 @@ static __global__ __launch_bounds__(256) void gemm_act_fp8_kernel(const int8_t* 
     }
 }
 
-// global -> LDS copy of 1 KB (64 lanes x 16 B) without passing through registers; dst is
-// wavefront-uniform, lane i's 16 bytes land at dst + 16 i
-__device__ __forceinline__ void g8_dma_1k(const uint8_t* src_lane, uint8_t* dst_uniform) {
-    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src_lane),
-                                     (__attribute__((address_space(3))) void*)(dst_uniform), 16, 0, 0);
+// global -> LDS copy of 1 KB (64 lanes x 16 B) without passing through registers: lane i's 16 bytes
+// at base + off_lane land at LDS address lds + 16 i.  base and lds are wavefront-uniform (scalar
+// registers), so a copy costs two scalar instructions and the load itself.  Written as inline
+// assembly: the compiler's own form of this load makes it treat every later wait on an LDS read or
+// a global load as a wait for everything in flight.
+__device__ __forceinline__ void g8_dma_1k(const uint8_t* base, uint32_t off_lane, uint32_t lds) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(off_lane), "s"(base), "s"(lds) : "memory", "m0");
 }
-
 // the same for 256 B (64 lanes x 4 B)
-__device__ __forceinline__ void g8_dma_256(const uint8_t* src_lane, uint8_t* dst_uniform) {
-    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src_lane),
-                                     (__attribute__((address_space(3))) void*)(dst_uniform), 4, 0, 0);
+__device__ __forceinline__ void g8_dma_256(const uint8_t* base, uint32_t off_lane, uint32_t lds) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1" ::"v"(off_lane), "s"(base), "s"(lds) : "memory", "m0");
+}
+// LDS byte address of a __shared__ object
+__device__ __forceinline__ uint32_t g8_lds_addr(const void* p) {
+    return static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) void*)(p)));
 }
 
 struct G8Stage {
@@ -139,15 +154,18 @@ struct G8Mins {
     uint8_t b[2][4096];       // [token tile][j][lane][16], the last KB unused
 };
 
-template <bool SWIGLU = false, bool DBG = false>
-static __global__ __launch_bounds__(256, 2) void gemm_q4k_fp8_kernel(GemmArgs p) {
+template <bool SWIGLU = false, bool DBG = false, int NW = G8_NW>
+static __global__ __launch_bounds__(64 * NW, 8 / NW) void gemm_q4k_fp8_kernel(GemmArgs p) {
+    constexpr uint32_t BM = 32 * NW;   // rows per workgroup
     // the two stage buffers are separate variables so that the compiler can tell the DMA into one
     // from the fragment reads of the other (a shared array would make every LDS read wait for
     // the DMA in flight)
     __shared__ __attribute__((aligned(16))) G8Stage st0;
     __shared__ __attribute__((aligned(16))) G8Stage st1;
-    __shared__ __attribute__((aligned(16))) G8Mins mn0;   // even super-blocks
-    __shared__ __attribute__((aligned(16))) G8Mins mn1;   // odd super-blocks
+    __shared__ __attribute__((aligned(16))) G8Mins mnb_lds;   // min operands of the super-block in progress
+    // each wavefront's own rows of the next super-block, 32 x 144 bytes as 16-byte pieces in row order
+    // (+ 32 unused pieces: the fifth copy instruction runs with all lanes)
+    __shared__ __attribute__((aligned(16))) uint8_t wts[NW][320 * 16];
     const uint32_t tid = threadIdx.x, lane = tid & 63;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wavefront-uniform: a scalar register
     const uint32_t col = lane & 31, half = lane >> 5;
@@ -156,35 +174,58 @@ static __global__ __launch_bounds__(256, 2) void gemm_q4k_fp8_kernel(GemmArgs p)
     float* const omat = second ? p.out2 : p.out;
     const uint32_t mrows = second ? p.m2 : p.m;
     const uint64_t ldn = second ? p.ld_n2 : p.ld_n;
-    const uint32_t m0 = (second ? blockIdx.y - p.tiles1 : blockIdx.y) * (SWIGLU ? G8_BM / 2 : G8_BM);
+    const uint32_t m0 = (second ? blockIdx.y - p.tiles1 : blockIdx.y) * (SWIGLU ? BM / 2 : BM);
     const uint32_t n0 = blockIdx.x * G8_BN;
     const uint32_t nsb_all = p.k / 256;
-    // this wavefront's 32 rows.  SwiGLU: wavefronts 0, 1 take 64 rows of the gate matrix and
-    // wavefronts 2, 3 the same 64 rows of the up matrix.
-    const uint32_t row0 = SWIGLU ? m0 + 32 * (wave & 1) : m0 + 32 * wave;
+    // this wavefront's 32 rows.  SwiGLU: the first half of the wavefronts take rows of the gate
+    // matrix and the second half the same rows of the up matrix.
+    const uint32_t row0 = SWIGLU ? m0 + 32 * (wave % (NW / 2)) : m0 + 32 * wave;
     // uniform base + 32-bit lane offset: one address register per lane instead of a pointer
-    const uint8_t* const wbase = (SWIGLU ? (wave < 2 ? p.w : p.w2) : wmat) + static_cast<uint64_t>(m0) * p.row_bytes;
-    const uint32_t wlane = (min(row0 + col, mrows - 1) - m0) * p.row_bytes + half * 16;
+    const uint8_t* const wbase = (SWIGLU ? (wave < NW / 2 ? p.w : p.w2) : wmat) + static_cast<uint64_t>(m0) * p.row_bytes;
+    // Weights reach the lanes through LDS as well.  A lane that loaded its own row's bytes from
+    // global memory made every load instruction touch 32 rows = 32 cache lines for 16 bytes each, and a
+    // row's two lines were fetched again by each of the five loads of a super-block (they do not survive
+    // in the 16 KB first-level cache between them): the loads alone took a fifth of the kernel.  Instead
+    // five DMA instructions copy the wavefront's 32 x 144 bytes with consecutive lanes on consecutive
+    // 16-byte pieces of a row (every line fetched once), and each lane then picks its row's header and
+    // its half of the four chunks out of LDS.
+    uint32_t wpiece[5];   // global offset (from wbase, without the super-block) of piece 64 j + lane
+#pragma unroll
+    for (int j = 0; j < 5; ++j) {
+        const uint32_t q = min(64u * j + lane, 287u), r = q / 9, part = q - 9 * r;
+        wpiece[j] = (min(row0 + r, mrows - 1) - m0) * p.row_bytes + part * 16;
+    }
+    const uint32_t wts_lds = g8_lds_addr(&wts[0][0]) + wave * (320 * 16);
+    const uint8_t* const wts_row = &wts[0][0] + wave * (320 * 16) + col * 144;   // this lane's row in the staged copy
     const uint32_t sb_begin = blockIdx.z * (p.k_chunk / 256), sb_end = sb_begin + p.k_chunk / 256;
     const uint8_t* const rec0 = p.bf8 + static_cast<uint64_t>(blockIdx.x * 2) * nsb_all * G8_REC;   // token tile 2*blockIdx.x
     const uint64_t rec_tile = static_cast<uint64_t>(nsb_all) * G8_REC;
+    const uint32_t lane16 = lane * 16, lane4 = lane * 4;
 
-    // stage (sb, s) -> LDS buffer, every wavefront the same share: 4 of the 16 KB of fragments, a
-    // quarter of the 1 KB of scales, and with s == 0 two of the 8 KB of min operands
-    auto stage_in = [&](uint32_t sb, uint32_t s, G8Stage& dst) {
-        const uint8_t* const r = rec0 + (wave >> 1) * rec_tile + static_cast<uint64_t>(sb) * G8_REC;   // token tile wave / 2
-        const uint32_t hw = wave & 1;
+    // stage (sb, s) -> LDS buffer, every wavefront the same share of the 16 KB of fragments; 1 KB of
+    // scales in four quarters; with_mins: also the 8 KB of min operands of super-block sb_mins
+    auto stage_in = [&](uint32_t sb, uint32_t s, G8Stage& dst, bool with_mins, uint32_t sb_mins) {
+        constexpr int CW = 16 / NW;   // fragment chunks of 1 KB per wavefront
+        const uint32_t c0 = wave * CW, tn = c0 >> 3;
+        const uint8_t* const r = rec0 + tn * rec_tile + static_cast<uint64_t>(sb) * G8_REC + s * 8192 + (c0 & 7) * 1024;
+        const uint32_t l = g8_lds_addr(&dst.bf[tn][0][0]) + (c0 & 7) * 1024;
 #pragma unroll
-        for (int i = 0; i < 4; ++i)   // chunks 4 hw .. 4 hw + 3 of the tile's 8
-            g8_dma_1k(r + s * 8192 + (hw * 4 + i) * 1024 + lane * 16, &dst.bf[wave >> 1][0][0] + (hw * 4 + i) * 1024);
-        g8_dma_256(r + G8_REC_XS + s * 512 + hw * 256 + lane * 4, reinterpret_cast<uint8_t*>(&dst.xs[wave >> 1][0][0]) + hw * 256);
-        if (s == 0) {
+        for (int i = 0; i < CW; ++i) g8_dma_1k(r + i * 1024, lane16, l + i * 1024);
+        if (wave < 4) {
+            const uint8_t* const rx = rec0 + (wave >> 1) * rec_tile + static_cast<uint64_t>(sb) * G8_REC + G8_REC_XS + s * 512 + (wave & 1) * 256;
+            g8_dma_256(rx, lane4, g8_lds_addr(&dst.xs[wave >> 1][0][0]) + (wave & 1) * 256);
+        }
+        if (with_mins) {
+            constexpr int MW = 8 / NW;   // min-operand chunks per wavefront
+            const uint32_t q0 = wave * MW, tm = q0 >> 2;
+            const uint8_t* const rm = rec0 + tm * rec_tile + static_cast<uint64_t>(sb_mins) * G8_REC + G8_REC_MIN + (q0 & 3) * 1024;
+            const uint32_t lm = g8_lds_addr(mnb_lds.b[tm]) + (q0 & 3) * 1024;
 #pragma unroll
-            for (int j = 0; j < 2; ++j)
-                g8_dma_1k(r + G8_REC_MIN + (hw * 2 + j) * 1024 + lane * 16, ((sb & 1) ? mn1 : mn0).b[wave >> 1] + (hw * 2 + j) * 1024);
+            for (int j = 0; j < MW; ++j) g8_dma_1k(rm + j * 1024, lane16, lm + j * 1024);
         }
     };
 
+    // acc takes the scaled block dots (vector ALU) and, negated, the min terms (matrix core)
     v16f acc[2];
 #pragma unroll
     for (int tn = 0; tn < 2; ++tn)
@@ -192,25 +233,30 @@ static __global__ __launch_bounds__(256, 2) void gemm_q4k_fp8_kernel(GemmArgs p)
         for (int e = 0; e < 16; ++e) acc[tn][e] = 0.0f;
 
     // The K loop is software-pipelined inside the wavefront.  A step is one (pair g, token tile tn,
-    // block jb of the pair): 16 per super-block.  Tick t reads the fragments of step t+2 from LDS,
-    // issues the matrix-core work of step t+1 and then runs the 16 FMAs of step t while that work
+    // block jb of the pair): 16 per super-block.  Tick t issues the matrix-core work of step t+1, reads
+    // the fragments of step t+3 from LDS and then runs the 16 FMAs of step t while that work
     // executes: on this hardware a SIMD overlaps matrix-core and vector instructions of the SAME
     // wavefront, not those of two different wavefronts.
     //
-    // Weight prefetch: the 144 bytes of a row's next super-block are requested in one burst of five
-    // loads (header + this lane's half of the four chunks) right behind the barrier of tick 6, so the
-    // row's two cache lines come from L2 once and the barrier's wait never covers a young load.
-    // Pairs 2, 3 of the current super-block are still unread then: theirs land in spare registers and
-    // move over behind the barrier of tick 14.
-    uint4 hdr, raw[4], rawx[2];
-    auto load_hdr = [&](uint32_t sb) { hdr = ld_u128(wbase + (wlane - half * 16 + sb * 144)); };
-    auto load_raw = [&](uint32_t sb, int g) { return ld_u128(wbase + (wlane + sb * 144 + 16 + g * 32)); };
+    // Weight prefetch: a super-block's rows are copied to LDS one super-block ahead (behind the barrier
+    // of tick 13) and read into registers at tick 13 of the super-block before theirs.
+    uint4 hdr, raw[4];
+    // global -> this wavefront's LDS rows, super-block sb
+    auto weights_in = [&](uint32_t sb) {
+        const uint8_t* const b = wbase + static_cast<uint64_t>(sb) * 144;
+#pragma unroll
+        for (int j = 0; j < 5; ++j) g8_dma_1k(b, wpiece[j], wts_lds + j * 1024);
+    };
+    // LDS -> registers: header and this lane's half of the four chunks
+    auto weights_read = [&]() {
+        hdr = *reinterpret_cast<const uint4*>(wts_row);
+#pragma unroll
+        for (int g = 0; g < 4; ++g) raw[g] = *reinterpret_cast<const uint4*>(wts_row + 16 + g * 32 + half * 16);
+    };
 
     // per super-block row state (lane = row col), decoded from the header
     float d18 = 0.0f, ndmin = 0.0f;   // d * 2^18, -dmin
     uint32_t scb = 0, mnb = 0;        // 6-bit scales of blocks 2g + half (g = 0..3) / mins of blocks 4*half .. +3, one per byte
-    float ndmin_prev = 0.0f;          // the same of the super-block whose min terms are still to come
-    uint32_t mnb_prev = 0;
     auto decode_hdr = [&]() {
         const uint4 h = hdr;
         d18 = h2f(h.x & 0xFFFF) * 262144.0f;
@@ -225,7 +271,7 @@ static __global__ __launch_bounds__(256, 2) void gemm_q4k_fp8_kernel(GemmArgs p)
 
     v8i af[2];          // A operands of the pair being issued: low-nibble block, high-nibble block
     float rsl = 0.0f;   // this lane's row scale for the pair's scale-tile MFMA
-    v8i bfr[2];         // B fragments, by step parity
+    v8i bfr[4];         // B fragments, by step % 4 (read three steps ahead of the FMAs)
     float xsl[2];       // scale operand (token col, block 2pr + half), by (step / 2) parity
     v32f sct[2];        // scale tiles of a (pair, token tile), by (step / 2) parity
     v16f dot[2];        // block dots, by step parity
@@ -236,12 +282,24 @@ static __global__ __launch_bounds__(256, 2) void gemm_q4k_fp8_kernel(GemmArgs p)
         const int pr = (t >> 2) & 1, tn = (t >> 1) & 1, jb = t & 1;
         const uint8_t* f = &st.bf[tn][2 * pr + jb][0] + lane * 16;
         const v4i lo = *reinterpret_cast<const v4i*>(f), hi = *reinterpret_cast<const v4i*>(f + 1024);
-        bfr[t & 1] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        bfr[t & 3] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
         if (jb == 0) xsl[(t >> 1) & 1] = st.xs[tn][2 * pr + half][col];
     };
-    // matrix-core work of step t: at a pair's first step the A operands, at a (pair, token tile)'s
-    // first step the scale tile, always the block dot
-    auto issue = [&](int t) {
+    // matrix-core work of step t in two parts, so that other work can sit between them (behind the
+    // scale-tile MFMA, whose 64 clocks are otherwise spent waiting to issue the dot): at a (pair,
+    // token tile)'s first step the scale tile ...
+    auto issue_s = [&](int t) {
+        const int g = t >> 2;
+        if ((t & 3) == 0) rsl = d18 * static_cast<float>((scb >> (8 * g)) & 0xFF);
+        if ((t & 1) == 0) {
+            v32f z32;
+#pragma unroll
+            for (int e = 0; e < 32; ++e) z32[e] = 0.0f;
+            sct[(t >> 1) & 1] = __builtin_amdgcn_mfma_f32_32x32x1f32(rsl, xsl[(t >> 1) & 1], z32, 0, 0, 0);
+        }
+    };
+    // ... and, after the A operands at a pair's first step, the block dot
+    auto issue_d = [&](int t) {
         const int g = t >> 2, jb = t & 1;
         if ((t & 3) == 0) {
             const uint4 q = raw[g];
@@ -250,18 +308,11 @@ static __global__ __launch_bounds__(256, 2) void gemm_q4k_fp8_kernel(GemmArgs p)
                       h3 = (q.w >> 4) & 0x0F0F0F0F;
             af[0] = v8i{l0, l1, l2, l3, l0, l1, l2, l3};
             af[1] = v8i{h0, h1, h2, h3, h0, h1, h2, h3};
-            rsl = d18 * static_cast<float>((scb >> (8 * g)) & 0xFF);
-        }
-        if (jb == 0) {
-            v32f z32;
-#pragma unroll
-            for (int e = 0; e < 32; ++e) z32[e] = 0.0f;
-            sct[(t >> 1) & 1] = __builtin_amdgcn_mfma_f32_32x32x1f32(rsl, xsl[(t >> 1) & 1], z32, 0, 0, 0);
         }
         v16f z16;
 #pragma unroll
         for (int e = 0; e < 16; ++e) z16[e] = 0.0f;
-        dot[t & 1] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(af[jb], bfr[t & 1], z16, 0, 0, 0, 0, 0, 0);
+        dot[t & 1] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(af[jb], bfr[t & 3], z16, 0, 0, 0, 0, 0, 0);
     };
     auto fma_step = [&](int t, uint32_t sb) {
         const int tn = (t >> 1) & 1, jb = t & 1;
@@ -280,12 +331,12 @@ static __global__ __launch_bounds__(256, 2) void gemm_q4k_fp8_kernel(GemmArgs p)
         // super-block and every matrix-core result is spilled on the way
         asm volatile("" : "+v"(acc[tn]));
     };
-    // min terms of a finished super-block: acc -= sum_b (dmin*mn)[row][b] * (xs*sum a)[tok][b]
-    auto mins = [&](uint32_t sb) {
+    // min terms of the super-block in progress: acc -= sum_b (dmin*mn)[row][b] * (xs*sum a)[tok][b]
+    auto mins = [&]() {
         uint32_t aw[12];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const float rm = ndmin_prev * static_cast<float>((mnb_prev >> (8 * i)) & 0xFF);
+            const float rm = ndmin * static_cast<float>((mnb >> (8 * i)) & 0xFF);
             const uint32_t r0 = __builtin_bit_cast(uint32_t, rm) & 0xFFFF0000u;
             const float e1 = rm - __builtin_bit_cast(float, r0);
             const uint32_t r1 = __builtin_bit_cast(uint32_t, e1) & 0xFFFF0000u;
@@ -300,66 +351,68 @@ static __global__ __launch_bounds__(256, 2) void gemm_q4k_fp8_kernel(GemmArgs p)
         for (int tn = 0; tn < 2; ++tn)
 #pragma unroll
             for (int j = 0; j < 3; ++j) {
-                const uint4 b = *reinterpret_cast<const uint4*>(((sb & 1) ? mn1 : mn0).b[tn] + j * 1024 + lane * 16);
+                const uint4 b = *reinterpret_cast<const uint4*>(mnb_lds.b[tn] + j * 1024 + lane * 16);
                 const uint4 a = make_uint4(aw[4 * j], aw[4 * j + 1], aw[4 * j + 2], aw[4 * j + 3]);
                 acc[tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, a), __builtin_bit_cast(v8bf, b), acc[tn], 0, 0, 0);
             }
     };
 
-    // ---- prologue: stage 0 and the weights of the first super-block, then steps 0 (issued) and 1 (read)
-    stage_in(sb_begin, 0, st0);
-    load_hdr(sb_begin);
-#pragma unroll
-    for (int g = 0; g < 4; ++g) raw[g] = load_raw(sb_begin, g);
+    // ---- prologue: stage 0 (with the first super-block's min operands) and the weights of the first
+    // super-block, then steps 0 (issued), 1 and 2 (read)
+    stage_in(sb_begin, 0, st0, true, sb_begin);
+    weights_in(sb_begin);
     __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
     __syncthreads();
-    stage_in(sb_begin, 1, st1);
+    stage_in(sb_begin, 1, st1, false, 0);
+    weights_read();
+    __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(0): the staged rows are in registers, their LDS copy is free
+    weights_in(min(sb_begin + 1, sb_end - 1));
     decode_hdr();
     lds_read(0);
     lds_read(1);
-    issue(0);
+    lds_read(2);
+    issue_s(0);
+    issue_d(0);
 
     for (uint32_t sb = sb_begin; sb < sb_end; ++sb) {
         const uint32_t sb_next = min(sb + 1, sb_end - 1);   // the last super-block re-requests itself: no branch around the loads
 #pragma unroll
         for (int t = 0; t < 16; ++t) {
-            // matrix-core work of step t+1 first.  (While a DMA into LDS is in flight the compiler makes
-            // every wait for an LDS read a wait for ALL LDS reads, so the reads of step t+2 are
-            // requested behind these instructions, not in front of them.)
-            if (t == 15) {
-                // step 0 of the next super-block: its header
-                ndmin_prev = ndmin;
-                mnb_prev = mnb;
-                decode_hdr();
+            // matrix-core work of step t+1 first, everything else behind it.  (While a DMA into LDS is
+            // in flight the compiler makes every wait for an LDS read a wait for ALL LDS reads, so the
+            // reads of step t+3 are requested behind these instructions, not in front of them.)
+            if (t == 15) decode_hdr();   // step 0 of the next super-block: its header
+            __builtin_amdgcn_sched_barrier(0);
+            issue_s((t + 1) & 15);
+            __builtin_amdgcn_sched_barrier(0);
+            if (t == 11) {
+                // the min terms go here: their operands are read before the barrier of tick 13 lets the
+                // next super-block's overwrite them
+                mins();
+                __builtin_amdgcn_sched_barrier(0);
             }
-            __builtin_amdgcn_sched_barrier(0);
-            issue((t + 1) & 15);
-            __builtin_amdgcn_sched_barrier(0);
-            // ---- the barrier that publishes the stage step t+2 starts, and the DMA of the stage after it
-            if (t == 6 || t == 14) {
+            // ---- the barrier that publishes the stage step t+3 starts, and the DMA of the stage after it
+            if (t == 5 || t == 13) {
                 __builtin_amdgcn_s_waitcnt(0x0F70);   // this wavefront's DMA of that stage has landed
                 __syncthreads();
-                if (t == 6) {
-                    if (sb + 1 < sb_end) stage_in(sb + 1, 0, st0);
-                    load_hdr(sb_next);
-                    raw[0] = load_raw(sb_next, 0);
-                    raw[1] = load_raw(sb_next, 1);
-                    rawx[0] = load_raw(sb_next, 2);
-                    rawx[1] = load_raw(sb_next, 3);
+                if (t == 5) {
+                    if (sb + 1 < sb_end) stage_in(sb + 1, 0, st0, false, 0);
                 } else {
-                    if (sb + 1 < sb_end) stage_in(sb + 1, 1, st1);
-                    raw[2] = rawx[0];
-                    raw[3] = rawx[1];
+                    if (sb + 1 < sb_end) stage_in(sb + 1, 1, st1, true, sb + 1);
+                    // the next super-block's rows into registers (landed: waited for above; every pair of this
+                    // one is unpacked), then their LDS copy is free for the super-block after it
+                    weights_read();
+                    __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(0)
+                    weights_in(min(sb + 2, sb_end - 1));
                 }
+                __builtin_amdgcn_sched_barrier(0);
             }
-            lds_read((t + 2) & 15);
+            issue_d((t + 1) & 15);
+            __builtin_amdgcn_sched_barrier(0);
+            lds_read((t + 3) & 15);
             __builtin_amdgcn_sched_barrier(0);
             fma_step(t, sb);
             __builtin_amdgcn_sched_barrier(0);
-            if (t == 15) {
-                mins(sb);
-                __builtin_amdgcn_sched_barrier(0);
-            }
         }
     }
 
@@ -367,15 +420,19 @@ static __global__ __launch_bounds__(256, 2) void gemm_q4k_fp8_kernel(GemmArgs p)
     if (SWIGLU) {
         // The up wavefronts hand their tiles to the gate wavefronts through LDS (the stage buffers are
         // free after the last barrier): same lane, same register positions.
-        float* const xch = reinterpret_cast<float*>(&st0);   // [wave & 1][tn][e][lane] = 16 KB
-        if (wave >= 2) {
+        float* const xch = reinterpret_cast<float*>(&st0);   // [wave % (NW/2)][tn][e][lane], 8 KB per wavefront
+        static_assert(sizeof(G8Stage) >= (NW / 2) * 8192 || NW == 8, "exchange area");
+        float* const xch2 = NW == 8 ? reinterpret_cast<float*>(&st1) : xch;   // waves 2, 3 of four pairs use the second buffer
+        const uint32_t xw = wave % (NW / 2);
+        float* const myx = (xw >= 2 ? xch2 : xch) + (xw & 1) * 2048;
+        if (wave >= NW / 2) {
 #pragma unroll
             for (int tn = 0; tn < 2; ++tn)
 #pragma unroll
-                for (int e = 0; e < 16; ++e) xch[(((wave & 1) * 2 + tn) * 16 + e) * 64 + lane] = acc[tn][e];
+                for (int e = 0; e < 16; ++e) myx[(tn * 16 + e) * 64 + lane] = acc[tn][e];
         }
         __syncthreads();
-        if (wave >= 2) return;
+        if (wave >= NW / 2) return;
         // h = silu(gate) * up (cera/src/backend/cpu.rs:2570-2575), then the Q8_0 block of this token's
         // rows row0 .. row0+31 (cpu.rs:942-958): this lane holds 16 of them, lane ^ 32 the others
 #pragma unroll
@@ -385,7 +442,7 @@ static __global__ __launch_bounds__(256, 2) void gemm_q4k_fp8_kernel(GemmArgs p)
             float amax = 0.0f;
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
-                const float g = acc[tn][e], u = xch[((wave * 2 + tn) * 16 + e) * 64 + lane];
+                const float g = acc[tn][e], u = myx[(tn * 16 + e) * 64 + lane];
                 hv[e] = __fmul_rn(__fdiv_rn(g, __fadd_rn(1.0f, cera_expf(-g))), u);
                 amax = fmaxf(amax, fabsf(hv[e]));   // fmaxf drops a NaN operand, as f32::max does
             }
