@@ -375,8 +375,8 @@ void HipLlamaModel::restore_state(const StateSnapshot& snap) {
     if (cera_hip_set_seq_len(model_, static_cast<uint32_t>(snap.seq_len)) != CERA_HIP_OK) device_panic("restore_state");
 }
 
-void HipLlamaModel::set_reference_order(bool on) {
-    if (cera_hip_set_reference_order(model_, on ? 1u : 0u) != CERA_HIP_OK)
+void HipLlamaModel::set_reference_order(uint32_t mode) {
+    if (cera_hip_set_reference_order(model_, mode) != CERA_HIP_OK)
         bail(std::string("set_reference_order: ") + cera_hip_last_error(ctx_));
 }
 

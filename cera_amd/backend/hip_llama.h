@@ -135,7 +135,8 @@ public:
 
     // verification hook: run every forward on the reference-order kernels (bit-identical to the
     // CPU AVX2 path, many times slower); only with an empty cache
-    void set_reference_order(bool on);
+    // 0 off, 1 reference order with per-token prefill, 2 with the x86 host's batched prefill (cera_hip.h)
+    void set_reference_order(uint32_t mode);
     RopeType rope_type() const { return rope_type_; }
     std::string device_name() const;
 

@@ -197,7 +197,7 @@ int cera_llama_set_reference_order(cera_llama* h, int on) {
     return guarded(h, [&] {
         auto* hm = dynamic_cast<cera::HipLlamaModel*>(h->model.get());
         if (!hm) throw cera::BackendError("set_reference_order: not a hip model");
-        hm->set_reference_order(on != 0);
+        hm->set_reference_order(on < 0 ? 0u : static_cast<uint32_t>(on));
     });
 }
 

@@ -47,7 +47,7 @@ struct cera_hip_model {
     uint32_t seq_len = 0;
     // reference-order verification route (reforder.hip): every f32 operation in the CPU path's
     // order, bit-identical logits; slow, never the default
-    bool ref_order = false;
+    uint32_t ref_order = 0;   // 0 fast route; 1 reference order, per-token prefill; 2 reference order, the x86 host's batched prefill
     float* ref_scores = nullptr;  // [n_heads][max_seq_len] attention scores of that route
     bool kv_f16 = false;          // KV caches hold IEEE half instead of f32
     bool kv_configured = false;   // cera_hip_configure_kv was called: a different mode is a conflict
@@ -83,5 +83,11 @@ cera_hip_status cera_model_prefill_logits_all(cera_hip_model* m, const uint32_t*
                                               float* logits_all);
 // one token through the reference-order kernels (reforder.hip)
 cera_hip_status cera_model_decode_step_ref(cera_hip_model* m, uint32_t pos, bool want_logits);
+// n tokens in one pass in the order of the x86 host's forward_prefill_batched (reforder.hip); the
+// last row's logits are left in m->logits when want_logits
+cera_hip_status cera_model_prefill_ref_batched(cera_hip_model* m, const uint32_t* tokens, uint32_t n, uint32_t start_pos,
+                                               bool want_logits);
+// (re)allocates the prefill pass buffers for n tokens (at most one pass's capacity, m->pf_cap)
+cera_hip_status cera_model_ensure_prefill_buffers(cera_hip_model* m, uint32_t n);
 bool cera_model_ref_order_supported(const cera_hip_model* m, std::string* why);
 cera_hip_status cera_model_decode_logits(cera_hip_model* m, uint32_t token, uint32_t pos, float* logits);

@@ -423,10 +423,10 @@ extern "C" cera_hip_status cera_hip_set_reference_order(cera_hip_model* m, uint3
     std::string why;
     if (on && !cera_model_ref_order_supported(m, &why))
         return cera_fail(m->ctx, CERA_HIP_ERR_UNSUPPORTED_DTYPE, "set_reference_order: " + why);
-    m->ref_order = on != 0;
+    m->ref_order = on >= 2 ? 2u : on;
     return CERA_HIP_OK;
 }
-extern "C" uint32_t cera_hip_reference_order(const cera_hip_model* m) { return m && m->ref_order ? 1u : 0u; }
+extern "C" uint32_t cera_hip_reference_order(const cera_hip_model* m) { return m ? m->ref_order : 0u; }
 
 extern "C" uint32_t cera_hip_kv_type(const cera_hip_model* m) { return m && m->kv_f16 ? CERA_HIP_KV_F16 : CERA_HIP_KV_F32; }
 

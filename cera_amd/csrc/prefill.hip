@@ -400,7 +400,7 @@ static constexpr uint32_t PREFILL_CHUNK = 2048;
 // 10.7 against 9.4 -- the per-token dots grow with the batch while the GEMM's tile fills up)
 static constexpr uint32_t PREFILL_SMALL_BATCH = 8;
 
-static cera_hip_status ensure_prefill_buffers(cera_hip_model* m, uint32_t n) {
+cera_hip_status cera_model_ensure_prefill_buffers(cera_hip_model* m, uint32_t n) {
     if (m->pf_cap >= n) return CERA_HIP_OK;
     cera_hip_ctx* ctx = m->ctx;
     const cera_hip_config& c = m->cfg;
@@ -449,7 +449,7 @@ static cera_hip_status prefill_chunk(cera_hip_model* m, const uint32_t* tokens, 
     hipStream_t s = ctx->stream;
     const uint32_t hs = c.hidden, q_dim = c.n_heads * c.head_dim, kv_dim = c.n_kv_heads * c.head_dim;
     const float scale = c.attn_scale != 0.0f ? c.attn_scale : 1.0f / std::sqrt(static_cast<float>(c.head_dim));
-    CERA_TRY(ensure_prefill_buffers(m, n));
+    CERA_TRY(cera_model_ensure_prefill_buffers(m, n));
     CERA_TRY(cera_hip_upload(ctx, m->pf_tokens, tokens, n * 4ull));
     hipLaunchKernelGGL(set_pos_kernel, dim3(1), dim3(1), 0, s, m->scalars, start_pos);
     hipLaunchKernelGGL(embed_row_kernel, dim3((hs + 255) / 256, n), dim3(256), 0, s, m->embd->dtype, m->embd->dev,
@@ -662,6 +662,16 @@ cera_hip_status cera_model_prefill(cera_hip_model* m, const uint32_t* tokens, ui
     // route -- the same decision LlamaModel::forward_prefill makes (llama.rs:1643,
     // 762-795); it is still the HIP path, only slower.  (Q5_K, which sends the reference down
     // that route, has a batched kernel here.)
+    if (m->ref_order == 2 && n > 1) {
+        // the verification route in the x86 host's batched order (forward_prefill takes
+        // forward_prefill_batched for n > 1, cera/src/model/llama.rs:1639-1641); one pass holds
+        // PREFILL_CHUNK tokens, the reference's callers split at ubatch = 512 (model/mod.rs:303-332)
+        for (uint32_t off = 0; off < n; off += PREFILL_CHUNK) {
+            uint32_t len = std::min(PREFILL_CHUNK, n - off);
+            CERA_TRY(cera_model_prefill_ref_batched(m, tokens + off, len, start_pos + off, off + len == n));
+        }
+        return cera_hip_download(m->ctx, last_logits, m->logits, static_cast<uint64_t>(m->cfg.vocab) * 4);
+    }
     if (n == 1 || !prefill_batchable(m)) return cera_model_prefill_per_token(m, tokens, n, start_pos, last_logits);
     for (uint32_t off = 0; off < n; off += PREFILL_CHUNK) {
         uint32_t len = std::min(PREFILL_CHUNK, n - off);

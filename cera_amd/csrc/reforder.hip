@@ -52,6 +52,10 @@ struct RefGemvArgs {
 };
 
 // One row, one lane of its group.  Every lane carries the scalar chains (macc) redundantly.
+// NACC = 4: the n == 1 (decode) branch with its four round-robin accumulators; NACC = 1: the
+// KQ_COLS-tiled branch every column of a batch (n > 1) takes (cera/src/backend/simd.rs:5796-5851,
+// 6094-6168), one accumulator.
+template <int NACC = 4>
 __device__ __forceinline__ float ref_row_q4_k(const uint8_t* row, const int8_t* xq, const float* xs, uint32_t k, uint32_t j) {
     float facc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
     float macc = 0.0f;
@@ -81,13 +85,14 @@ __device__ __forceinline__ float ref_row_q4_k(const uint8_t* row, const int8_t* 
             const float dmn = __fmul_rn(dmin, static_cast<float>(mn));
             facc[slot] = fmaf(lanes, __fmul_rn(x, dsc), facc[slot]);
             macc = __fadd_rn(macc, __fmul_rn(__fmul_rn(x, dmn), static_cast<float>(sx)));
-            slot = (slot + 1) & 3;
+            slot = (slot + 1) & (NACC - 1);
         }
     }
-    const float f = __fadd_rn(__fadd_rn(facc[0], facc[1]), __fadd_rn(facc[2], facc[3]));
+    const float f = NACC == 4 ? __fadd_rn(__fadd_rn(facc[0], facc[1]), __fadd_rn(facc[2], facc[3])) : facc[0];
     return __fsub_rn(grp_hsum(f), macc);
 }
 
+template <int NACC = 4>
 __device__ __forceinline__ float ref_row_q6_k(const uint8_t* row, const int8_t* xq, const float* xs, uint32_t k, uint32_t j) {
     float facc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
     float macc = 0.0f;
@@ -120,11 +125,11 @@ __device__ __forceinline__ float ref_row_q6_k(const uint8_t* row, const int8_t* 
                 const float sx0 = static_cast<float>(j < 4 ? s16 : other), sx1 = static_cast<float>(j < 4 ? other : s16);
                 const float mins = __fadd_rn(__fmul_rn(sc0, sx0), __fmul_rn(sc1, sx1));
                 macc = __fadd_rn(macc, __fmul_rn(__fmul_rn(x, d32), mins));
-                slot = (slot + 1) & 3;
+                slot = (slot + 1) & (NACC - 1);
             }
         }
     }
-    const float f = __fadd_rn(__fadd_rn(facc[0], facc[1]), __fadd_rn(facc[2], facc[3]));
+    const float f = NACC == 4 ? __fadd_rn(__fadd_rn(facc[0], facc[1]), __fadd_rn(facc[2], facc[3])) : facc[0];
     return __fsub_rn(grp_hsum(f), macc);
 }
 
@@ -170,6 +175,155 @@ __global__ __launch_bounds__(256) void gemv_ref_kernel(RefGemvArgs p) {
     else v = ref_row_b32<TYPE>(rp, p.xq, p.xs, p.k, j);
     if (j == 0 && row < p.m) p.y[row] = v;
 }
+
+// ---- batched prefill in the order of cera's x86 host ---------------------------------------
+// transformer::gemm_preq (cera/src/model/transformer.rs:710-788) sends a Q4_K / Q4_0 weight
+// that was repacked at load (m % 8 == 0; cpu.rs:1204-1206, 1364-1366) to the 8-row-interleaved
+// kernels gemm_q4_k_8x8_q8_0 / gemm_q4_0_8x8_q8_0 (cera/src/backend/simd.rs:5392-5518, 5215-5366).
+// There the eight lanes of a vector are eight output ROWS of one column, so every output
+// element has an f32 chain of its own: per 32-block one FMA with the exact integer block dot
+// (Q4_K: and one FNMADD with the exact activation sum).  Integer sums are order-free, so the
+// eight lanes of a group only share the integer work; the float chain is the same in each.
+__device__ __forceinline__ float ref_elem_q4_k_8x8(const uint8_t* row, const int8_t* xq, const float* xs, uint32_t k, uint32_t j) {
+    float facc = 0.0f;
+    for (uint32_t bi = 0; bi < k / 256; ++bi) {
+        const uint8_t* blk = row + 144 * bi;
+        const float d = h2f(ld_u16(blk)), dmin = h2f(ld_u16(blk + 2));
+        const uint8_t* s12 = blk + 4;
+#pragma unroll
+        for (int s = 0; s < 8; ++s) {
+            uint32_t sc, mn;
+            if (s < 4) {
+                sc = s12[s] & 63;
+                mn = s12[s + 4] & 63;
+            } else {
+                sc = (s12[s + 4] & 0xF) | ((s12[s - 4] >> 6) << 4);
+                mn = (s12[s + 4] >> 4) | ((s12[s] >> 6) << 4);
+            }
+            const uint32_t xb = bi * 8 + s;
+            const uint32_t wq = *reinterpret_cast<const uint32_t*>(blk + 16 + 32 * (s >> 1) + 4 * j);
+            const uint32_t w4 = (s & 1) ? ((wq >> 4) & 0x0F0F0F0Fu) : (wq & 0x0F0F0F0Fu);
+            const uint32_t a4 = *reinterpret_cast<const uint32_t*>(xq + 32 * xb + 4 * j);
+            const int acc = grp_isum(dot4(w4, a4, 0));
+            const int sx = grp_isum(sum4(a4, 0));
+            const float x = xs[xb];
+            const float dsc = __fmul_rn(d, static_cast<float>(sc));     // baked at repack time (cpu.rs:1282-1358)
+            const float dmn = __fmul_rn(dmin, static_cast<float>(mn));
+            facc = fmaf(static_cast<float>(acc), __fmul_rn(dsc, x), facc);
+            facc = fmaf(-dmn, __fmul_rn(x, static_cast<float>(sx)), facc);   // _mm256_fnmadd_ps
+        }
+    }
+    return facc;
+}
+__device__ __forceinline__ float ref_elem_q4_0_8x8(const uint8_t* row, const int8_t* xq, const float* xs, uint32_t k, uint32_t j) {
+    float facc = 0.0f;
+    for (uint32_t b = 0; b < k / 32; ++b) {
+        const uint8_t* blk = row + 18 * b;
+        const uint32_t wq = ld_u32_a2(blk + 2 + 4 * (j & 3));
+        const uint32_t w4 = j < 4 ? (wq & 0x0F0F0F0Fu) : ((wq >> 4) & 0x0F0F0F0Fu);   // raw codes 0..15
+        const uint32_t a4 = *reinterpret_cast<const uint32_t*>(xq + 32 * b + 4 * j);
+        const int acc = grp_isum(dot4(w4, a4, 0));
+        const int cs = grp_isum(sum4(a4, 0));
+        const float eff = __fsub_rn(static_cast<float>(acc), __fmul_rn(8.0f, static_cast<float>(cs)));
+        facc = fmaf(eff, __fmul_rn(h2f(ld_u16(blk)), xs[b]), facc);
+    }
+    return facc;
+}
+
+struct RefGemmArgs {
+    const uint8_t* w;
+    const int8_t* xq;   // [n][k]
+    const float* xs;    // [n][k/32]
+    float* out;         // out[j * ld_n + i * ld_m]
+    uint32_t m, n, k, row_bytes;
+    uint64_t ld_m, ld_n;
+};
+// One 8-lane group per (row, token): grid = (ceil(m / 32), n).  REPACK: the 8x8 kernels' order.
+template <int TYPE, bool REPACK>
+__global__ __launch_bounds__(256) void gemm_ref_kernel(RefGemmArgs p) {
+    const uint32_t row = blockIdx.x * 32 + (threadIdx.x >> 3), j = threadIdx.x & 7, tok = blockIdx.y;
+    const uint8_t* rp = p.w + static_cast<uint64_t>(min(row, p.m - 1)) * p.row_bytes;
+    const int8_t* xq = p.xq + static_cast<uint64_t>(tok) * p.k;
+    const float* xs = p.xs + static_cast<uint64_t>(tok) * (p.k / 32);
+    float v;
+    if (TYPE == 12) v = REPACK ? ref_elem_q4_k_8x8(rp, xq, xs, p.k, j) : ref_row_q4_k<1>(rp, xq, xs, p.k, j);
+    else if (TYPE == 14) v = ref_row_q6_k<1>(rp, xq, xs, p.k, j);
+    else if (TYPE == 2 && REPACK) v = ref_elem_q4_0_8x8(rp, xq, xs, p.k, j);
+    else v = ref_row_b32<TYPE>(rp, xq, xs, p.k, j);
+    if (j == 0 && row < p.m) p.out[tok * p.ld_n + row * p.ld_m] = v;
+}
+
+// flash_attention_gqa_avx2 (cera/src/backend/cpu.rs:4261-4412), one wavefront per (query, head):
+// keys in tiles of 32; a score is two 8-lane FMA chains over the even / odd 8-wide slices of the
+// head, added, folded with hsum256 (cpu.rs:3489) and scaled; the online softmax is the scalar
+// bookkeeping of the CPU kernel (tile maximum with `>`, ggml expf, f64 tile sum in key order,
+// running sum in f64); every output column is one FMA chain over the keys in order.
+// q: [n][n_heads * hd] rotated queries; out the same shape.  Caches head-major.
+template <typename KV>
+__global__ __launch_bounds__(64) void flash_ref_kernel(const float* __restrict__ q, const KV* __restrict__ kc,
+                                                       const KV* __restrict__ vc, uint32_t n_heads, uint32_t group, uint32_t hd,
+                                                       uint32_t max_seq, uint32_t start_pos, float scale, float* __restrict__ out) {
+    __shared__ float sc_sh[32];
+    const uint32_t jq = blockIdx.x, h = blockIdx.y, kvh = h / group, lane = threadIdx.x;
+    const uint32_t grp = lane >> 3, j = lane & 7, nq = hd / 8;
+    const float* qh = q + (static_cast<uint64_t>(jq) * n_heads + h) * hd;
+    const KV* kbase = kc + static_cast<uint64_t>(kvh) * max_seq * hd;
+    const KV* vbase = vc + static_cast<uint64_t>(kvh) * max_seq * hd;
+    const uint32_t max_kv = start_pos + jq + 1;
+    float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};   // columns lane + 64 c, hd <= 256
+    float running_max = -__builtin_inff();
+    double running_sum = 0.0;
+    for (uint32_t kv_start = 0; kv_start < max_kv; kv_start += 32) {
+        const uint32_t tile_len = min(32u, max_kv - kv_start);
+        // scores: group grp takes keys grp, grp + 8, grp + 16, grp + 24 of the tile
+        for (uint32_t r = 0; r < 4; ++r) {
+            const uint32_t ti = grp + 8 * r;
+            const KV* kp = kbase + static_cast<uint64_t>(kv_start + min(ti, tile_len - 1)) * hd;
+            float s0 = 0.0f, s1 = 0.0f;
+            uint32_t i = 0;
+            for (; i + 2 <= nq; i += 2) {
+                s0 = fmaf(qh[8 * i + j], KvOps<KV>::ld1(kp + 8 * i + j), s0);
+                s1 = fmaf(qh[8 * (i + 1) + j], KvOps<KV>::ld1(kp + 8 * (i + 1) + j), s1);
+            }
+            if (i < nq) s0 = fmaf(qh[8 * i + j], KvOps<KV>::ld1(kp + 8 * i + j), s0);
+            const float v = grp_hsum(__fadd_rn(s0, s1));
+            if (j == 0 && ti < tile_len) sc_sh[ti] = __fmul_rn(v, scale);
+        }
+        __syncthreads();
+        float tile_max = -__builtin_inff();
+        for (uint32_t ti = 0; ti < tile_len; ++ti)
+            if (sc_sh[ti] > tile_max) tile_max = sc_sh[ti];
+        const float new_max = fmaxf(running_max, tile_max);   // f32::max
+        const float rescale = running_max > -__builtin_inff() ? cera_expf(__fsub_rn(running_max, new_max)) : 0.0f;
+        // every lane keeps the whole bookkeeping (identical values in all lanes); lane ti < 32 makes p[ti]
+        float p_mine = 0.0f;
+        if (lane < tile_len) p_mine = cera_expf(__fsub_rn(sc_sh[lane], new_max));
+        __syncthreads();
+        if (lane < tile_len) sc_sh[lane] = p_mine;
+        __syncthreads();
+        double tile_sum = 0.0;
+        for (uint32_t ti = 0; ti < tile_len; ++ti) tile_sum += static_cast<double>(sc_sh[ti]);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) acc[c] = __fmul_rn(acc[c], rescale);
+        for (uint32_t ti = 0; ti < tile_len; ++ti) {
+            const float pv = sc_sh[ti];
+            const KV* vp = vbase + static_cast<uint64_t>(kv_start + ti) * hd;
+#pragma unroll
+            for (int c = 0; c < 4; ++c)
+                if (lane + 64 * c < hd) acc[c] = fmaf(pv, KvOps<KV>::ld1(vp + lane + 64 * c), acc[c]);
+        }
+        running_sum = running_sum * static_cast<double>(rescale) + tile_sum;
+        running_max = new_max;
+        __syncthreads();
+    }
+    const float inv_sum = static_cast<float>(1.0 / running_sum);
+    float* oh = out + (static_cast<uint64_t>(jq) * n_heads + h) * hd;
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+        if (lane + 64 * c < hd) oh[lane + 64 * c] = __fmul_rn(acc[c], inv_sum);
+}
+
+__global__ void ref_set_pos_kernel(uint32_t* scalars, uint32_t pos) { scalars[1] = pos; }
 
 // cpu::rmsnorm with the CPU's serial f64 chain: squares are formed in parallel (exact in f64),
 // staged through LDS 256 at a time and added by one thread in index order.  In place is fine
@@ -311,6 +465,55 @@ cera_hip_status launch_attn_ref(cera_hip_ctx* ctx, const float* q, const void* k
     return CERA_HIP_OK;
 }
 
+// out[j * ld_n + i * ld_m] = (W . B)[i][j] for n quantized activation rows, every element in the
+// order of the x86 host's batched route: the 8x8 kernels for a weight cera repacks at load when
+// x86_repack is set, the KQ_COLS-tiled / strip kernels otherwise.
+cera_hip_status launch_gemm_ref(cera_hip_ctx* ctx, const cera_hip_dtensor* w, const float* xs, const int8_t* xq, uint32_t n,
+                                bool x86_repack, float* out, uint64_t ld_m, uint64_t ld_n) {
+    if (!ref_type_ok(w->dtype))
+        return cera_fail(ctx, CERA_HIP_ERR_UNSUPPORTED_DTYPE,
+                         "reference-order gemm: no kernel for ggml type " + std::to_string(w->dtype));
+    if (n == 0 || n > 65535) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "reference-order gemm: 1 .. 65535 activation rows");
+    RefGemmArgs a{w->dev, xq, xs, out, static_cast<uint32_t>(w->m), n, static_cast<uint32_t>(w->k),
+                  static_cast<uint32_t>(w->row_bytes), ld_m, ld_n};
+    const dim3 grid(static_cast<uint32_t>((w->m + 31) / 32), n), block(256);
+    // repack_supported: Q4_0 with m % 8 == 0, Q4_K with m % 8 == 0 and whole super-blocks
+    const bool rp = x86_repack && w->m % 8 == 0 && (w->dtype == CERA_HIP_Q4_0 || (w->dtype == CERA_HIP_Q4_K && w->k % 256 == 0));
+    switch (w->dtype) {
+        case CERA_HIP_Q4_K:
+            if (rp) hipLaunchKernelGGL((gemm_ref_kernel<12, true>), grid, block, 0, ctx->stream, a);
+            else hipLaunchKernelGGL((gemm_ref_kernel<12, false>), grid, block, 0, ctx->stream, a);
+            break;
+        case CERA_HIP_Q6_K: hipLaunchKernelGGL((gemm_ref_kernel<14, false>), grid, block, 0, ctx->stream, a); break;
+        case CERA_HIP_Q4_0:
+            if (rp) hipLaunchKernelGGL((gemm_ref_kernel<2, true>), grid, block, 0, ctx->stream, a);
+            else hipLaunchKernelGGL((gemm_ref_kernel<2, false>), grid, block, 0, ctx->stream, a);
+            break;
+        case CERA_HIP_Q4_1: hipLaunchKernelGGL((gemm_ref_kernel<3, false>), grid, block, 0, ctx->stream, a); break;
+        default: hipLaunchKernelGGL((gemm_ref_kernel<8, false>), grid, block, 0, ctx->stream, a); break;
+    }
+    HIP_TRY(ctx, hipGetLastError());
+    return CERA_HIP_OK;
+}
+
+cera_hip_status launch_flash_ref(cera_hip_ctx* ctx, const float* q, const void* kc, const void* vc, uint32_t n_queries,
+                                 uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, uint32_t max_seq, uint32_t start_pos,
+                                 float scale, float* out, bool kv_f16) {
+    if (head_dim % 8 || head_dim > 256 || n_queries == 0 || n_queries > 65535 || start_pos + n_queries > max_seq ||
+        n_kv_heads == 0 || n_heads % n_kv_heads)
+        return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "reference-order flash attention: bad shape");
+    const dim3 grid(n_queries, n_heads);
+    const uint32_t group = n_heads / n_kv_heads;
+    if (kv_f16)
+        hipLaunchKernelGGL(flash_ref_kernel<kv_half>, grid, dim3(64), 0, ctx->stream, q, static_cast<const kv_half*>(kc),
+                           static_cast<const kv_half*>(vc), n_heads, group, head_dim, max_seq, start_pos, scale, out);
+    else
+        hipLaunchKernelGGL(flash_ref_kernel<float>, grid, dim3(64), 0, ctx->stream, q, static_cast<const float*>(kc),
+                           static_cast<const float*>(vc), n_heads, group, head_dim, max_seq, start_pos, scale, out);
+    HIP_TRY(ctx, hipGetLastError());
+    return CERA_HIP_OK;
+}
+
 }  // namespace
 
 // ---------------------------------------------------------------------------
@@ -390,6 +593,112 @@ cera_hip_status cera_model_decode_step_ref(cera_hip_model* m, uint32_t pos, bool
         if (c.logit_scale != 1.0f) {
             hipLaunchKernelGGL(scale_kernel, dim3((c.vocab + 255) / 256), dim3(256), 0, s, m->logits, 1.0f / c.logit_scale,
                                c.vocab);
+            HIP_TRY(ctx, hipGetLastError());
+        }
+    }
+    return CERA_HIP_OK;
+}
+
+// LlamaModel::forward_prefill_batched (cera/src/model/llama.rs:738-1523) as an x86 host without
+// `blas` runs it, every operation a launch of its own in the CPU path's order: rmsnorm per row,
+// quantize_columns (transformer.rs:865-946), gemm_preq with the repacked 8x8 kernels where cera
+// repacks (transformer.rs:710-788), RoPE + cache append per token, flash_attention_gqa_avx2 from
+// 256 tokens on (llama.rs:885) and the per-token attn_scores / softmax / attn_values below that,
+// SwiGLU, residual adds; then project_logits of the last row through the n == 1 GEMV branch.
+// n tokens in one pass (n <= the prefill buffers' capacity; the caller splits longer prompts).
+cera_hip_status cera_model_prefill_ref_batched(cera_hip_model* m, const uint32_t* tokens, uint32_t n, uint32_t start_pos,
+                                               bool want_logits) {
+    cera_hip_ctx* ctx = m->ctx;
+    const cera_hip_config& c = m->cfg;
+    hipStream_t s = ctx->stream;
+    const uint32_t hs = c.hidden, q_dim = c.n_heads * c.head_dim, kv_dim = c.n_kv_heads * c.head_dim;
+    const float scale = c.attn_scale != 0.0f ? c.attn_scale : 1.0f / std::sqrt(static_cast<float>(c.head_dim));
+    CERA_TRY(cera_model_ensure_prefill_buffers(m, n));
+    if (n > m->pf_cap) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "reference-order prefill: more tokens than one pass holds");
+    if (!m->ref_scores) {
+        const uint64_t bytes = static_cast<uint64_t>(c.n_heads) * c.max_seq_len * sizeof(float);
+        HIP_TRY(ctx, hipMalloc(reinterpret_cast<void**>(&m->ref_scores), bytes));
+        m->owned.push_back(m->ref_scores);
+        m->bytes += bytes;
+    }
+    CERA_TRY(cera_hip_upload(ctx, m->pf_tokens, tokens, n * 4ull));
+    hipLaunchKernelGGL(ref_set_pos_kernel, dim3(1), dim3(1), 0, s, m->scalars, start_pos);
+    hipLaunchKernelGGL(embed_row_kernel, dim3((hs + 255) / 256, n), dim3(256), 0, s, m->embd->dtype, m->embd->dev,
+                       m->embd->row_bytes, m->pf_tokens, hs, c.embed_scale, m->pf_hidden);
+    HIP_TRY(ctx, hipGetLastError());
+    const bool repack = m->ref_order == 2;
+    // quantize_columns + gemm_preq: out[n][w->m]
+    auto gemm = [&](const cera_hip_dtensor* w, const float* x_f32, float* out) -> cera_hip_status {
+        CERA_TRY(cera_launch_quantize(ctx, x_f32, static_cast<uint64_t>(n) * w->k, m->pf_xs, m->pf_xq));
+        return launch_gemm_ref(ctx, w, m->pf_xs, m->pf_xq, n, repack, out, 1, w->m);
+    };
+    auto add_rows = [&](const float* block_out) -> cera_hip_status {
+        const uint32_t tot = n * hs;
+        hipLaunchKernelGGL(add_kernel, dim3((tot + 255) / 256), dim3(256), 0, s, m->pf_hidden, block_out, c.residual_scale, tot,
+                           m->pf_hidden);
+        HIP_TRY(ctx, hipGetLastError());
+        return CERA_HIP_OK;
+    };
+    for (uint32_t i = 0; i < c.n_layers; ++i) {
+        LayerDev& L = m->layers[i];
+        CERA_TRY(launch_rmsnorm_ref(ctx, m->pf_hidden, L.attn_norm, hs, n, c.rms_eps, m->pf_normed));
+        CERA_TRY(gemm(L.q, m->pf_normed, m->pf_q));
+        CERA_TRY(launch_gemm_ref(ctx, L.k, m->pf_xs, m->pf_xq, n, repack, m->pf_k, 1, L.k->m));   // the same quantized columns
+        CERA_TRY(launch_gemm_ref(ctx, L.v, m->pf_xs, m->pf_xq, n, repack, m->pf_v, 1, L.v->m));
+        if (L.q_bias) {
+            for (uint32_t t = 0; t < n; ++t) {
+                hipLaunchKernelGGL(bias_kernel, dim3((q_dim + 255) / 256), dim3(256), 0, s, m->pf_q + static_cast<uint64_t>(t) * q_dim, L.q_bias, q_dim);
+                hipLaunchKernelGGL(bias_kernel, dim3((kv_dim + 255) / 256), dim3(256), 0, s, m->pf_k + static_cast<uint64_t>(t) * kv_dim, L.k_bias, kv_dim);
+                hipLaunchKernelGGL(bias_kernel, dim3((kv_dim + 255) / 256), dim3(256), 0, s, m->pf_v + static_cast<uint64_t>(t) * kv_dim, L.v_bias, kv_dim);
+            }
+        }
+        if (L.q_norm) {
+            CERA_TRY(launch_rmsnorm_ref(ctx, m->pf_q, L.q_norm, c.head_dim, n * c.n_heads, c.rms_eps, m->pf_q));
+            CERA_TRY(launch_rmsnorm_ref(ctx, m->pf_k, L.k_norm, c.head_dim, n * c.n_kv_heads, c.rms_eps, m->pf_k));
+        }
+        const dim3 rgrid(c.n_heads + 2 * c.n_kv_heads, n), rblock(c.head_dim / 2);
+        if (m->kv_f16)
+            hipLaunchKernelGGL(rope_kv_kernel<kv_half>, rgrid, rblock, 0, s, m->pf_q, m->pf_k, m->pf_v, m->rope_table, m->scalars + 1,
+                               c.n_heads, c.n_kv_heads, c.head_dim, c.rope_type, static_cast<kv_half*>(L.kc),
+                               static_cast<kv_half*>(L.vc), c.max_seq_len);
+        else
+            hipLaunchKernelGGL(rope_kv_kernel<float>, rgrid, rblock, 0, s, m->pf_q, m->pf_k, m->pf_v, m->rope_table, m->scalars + 1,
+                               c.n_heads, c.n_kv_heads, c.head_dim, c.rope_type, static_cast<float*>(L.kc),
+                               static_cast<float*>(L.vc), c.max_seq_len);
+        HIP_TRY(ctx, hipGetLastError());
+        if (n >= 256) {   // FLASH_ATTN_THRESHOLD
+            CERA_TRY(launch_flash_ref(ctx, m->pf_q, L.kc, L.vc, n, c.n_heads, c.n_kv_heads, c.head_dim, c.max_seq_len, start_pos,
+                                      scale, m->pf_attn, m->kv_f16));
+        } else {
+            for (uint32_t t = 0; t < n; ++t)
+                CERA_TRY(launch_attn_ref(ctx, m->pf_q + static_cast<uint64_t>(t) * q_dim, L.kc, L.vc, c.n_heads, c.n_kv_heads,
+                                         c.head_dim, start_pos + t + 1, c.max_seq_len, scale, m->ref_scores,
+                                         m->pf_attn + static_cast<uint64_t>(t) * q_dim, m->kv_f16));
+        }
+        CERA_TRY(gemm(L.o, m->pf_attn, m->pf_normed));   // pf_normed is free here: block_out
+        CERA_TRY(add_rows(m->pf_normed));
+
+        CERA_TRY(launch_rmsnorm_ref(ctx, m->pf_hidden, L.ffn_norm, hs, n, c.rms_eps, m->pf_normed));
+        CERA_TRY(gemm(L.gate, m->pf_normed, m->pf_gate));
+        CERA_TRY(launch_gemm_ref(ctx, L.up, m->pf_xs, m->pf_xq, n, repack, m->pf_up, 1, L.up->m));
+        const uint64_t tot = static_cast<uint64_t>(n) * c.ffn;
+        hipLaunchKernelGGL((silu_mul_kernel<false>), dim3(static_cast<uint32_t>((tot / 4 + 255) / 256)), dim3(256), 0, s, m->pf_gate,
+                           m->pf_up, tot, m->pf_gate, static_cast<float*>(nullptr), static_cast<int8_t*>(nullptr),
+                           static_cast<float*>(nullptr));
+        HIP_TRY(ctx, hipGetLastError());
+        CERA_TRY(gemm(L.down, m->pf_gate, m->pf_normed));
+        CERA_TRY(add_rows(m->pf_normed));
+    }
+    m->seq_len = start_pos + n;
+    if (want_logits) {
+        // project_logits on the last row: the per-token path's norm and n == 1 GEMV
+        const float* last = m->pf_hidden + static_cast<uint64_t>(n - 1) * hs;
+        CERA_TRY(launch_rmsnorm_ref(ctx, last, m->output_norm, hs, 1, c.rms_eps, m->hidden));
+        const cera_hip_dtensor* o = m->output ? m->output : m->embd;
+        CERA_TRY(cera_launch_quantize(ctx, m->hidden, hs, m->xs, m->xq));
+        CERA_TRY(launch_gemv_ref(ctx, o, m->xs, m->xq, m->logits));
+        if (c.logit_scale != 1.0f) {
+            hipLaunchKernelGGL(scale_kernel, dim3((c.vocab + 255) / 256), dim3(256), 0, s, m->logits, 1.0f / c.logit_scale, c.vocab);
             HIP_TRY(ctx, hipGetLastError());
         }
     }
@@ -477,4 +786,63 @@ extern "C" cera_hip_status cera_hip_rmsnorm_reference_order(cera_hip_ctx* ctx, c
     CERA_TRY(launch_rmsnorm_ref(ctx, static_cast<float*>(dx), static_cast<float*>(dw), static_cast<uint32_t>(n), 1, eps,
                                 static_cast<float*>(dy)));
     return cera_hip_download(ctx, y, dy, n * 4);
+}
+
+// out[m][n] (the reference's layout, simd.rs:5130-5148) = W . Q8_0(x[n][k]) in the order of the x86
+// host's batched route; x86_repack != 0: the 8x8 kernels for the weights cera repacks at load.
+extern "C" cera_hip_status cera_hip_gemm_reference_order(cera_hip_ctx* ctx, const cera_hip_tensor* t, const float* x, uint64_t n,
+                                                         uint32_t x86_repack, float* out) {
+    if (!ctx || !t || !x || !out) return CERA_HIP_ERR_ARGUMENT;
+    if (n == 0 || n > 65535) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "gemm_reference_order: 1 .. 65535 activation rows");
+    std::lock_guard<std::recursive_mutex> lk(ctx->op_mu);
+    cera_hip_dtensor* w = nullptr;
+    CERA_TRY(cera_hip_tensor_upload(ctx, t, &w));
+    auto run = [&]() -> cera_hip_status {
+        const uint64_t k = w->k, mm = w->m;
+        void *dx, *ds, *dq, *dy;
+        CERA_TRY(cera_scratch(ctx, 0, n * k * 4, &dx));
+        CERA_TRY(cera_scratch(ctx, 1, n * (k / 32) * 4, &ds));
+        CERA_TRY(cera_scratch(ctx, 2, n * k, &dq));
+        CERA_TRY(cera_scratch(ctx, 3, mm * n * 4, &dy));
+        CERA_TRY(cera_hip_upload(ctx, dx, x, n * k * 4));
+        CERA_TRY(cera_launch_quantize(ctx, static_cast<float*>(dx), n * k, static_cast<float*>(ds), static_cast<int8_t*>(dq)));
+        CERA_TRY(launch_gemm_ref(ctx, w, static_cast<float*>(ds), static_cast<int8_t*>(dq), static_cast<uint32_t>(n), x86_repack != 0,
+                                 static_cast<float*>(dy), n, 1));
+        return cera_hip_download(ctx, out, dy, mm * n * 4);
+    };
+    cera_hip_status st = run();
+    cera_hip_tensor_free(ctx, w);
+    return st;
+}
+
+// flash_attention_gqa_avx2 for n_queries queries at positions start_pos .. start_pos + n_queries - 1:
+// q, out [n_queries][n_heads * head_dim]; k, v the reference's time-major caches
+// [start_pos + n_queries][n_kv_heads * head_dim].
+extern "C" cera_hip_status cera_hip_flash_attn_reference_order(cera_hip_ctx* ctx, const float* q, const float* k, const float* v,
+                                                               uint32_t n_queries, uint32_t n_heads, uint32_t n_kv_heads,
+                                                               uint32_t head_dim, uint32_t start_pos, float scale, float* out) {
+    if (!ctx || !q || !k || !v || !out) return CERA_HIP_ERR_ARGUMENT;
+    if (n_queries == 0 || n_kv_heads == 0 || head_dim == 0)
+        return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "flash_attn_reference_order: empty input");
+    std::lock_guard<std::recursive_mutex> lk(ctx->op_mu);
+    const uint64_t seq = static_cast<uint64_t>(start_pos) + n_queries, kv_dim = static_cast<uint64_t>(n_kv_heads) * head_dim;
+    const uint64_t q_bytes = static_cast<uint64_t>(n_queries) * n_heads * head_dim * 4;
+    std::vector<float> hk(seq * kv_dim), hv(seq * kv_dim);   // time-major -> head-major
+    for (uint64_t t = 0; t < seq; ++t)
+        for (uint32_t h = 0; h < n_kv_heads; ++h)
+            for (uint32_t d = 0; d < head_dim; ++d) {
+                hk[(h * seq + t) * head_dim + d] = k[t * kv_dim + h * head_dim + d];
+                hv[(h * seq + t) * head_dim + d] = v[t * kv_dim + h * head_dim + d];
+            }
+    void *dq, *dk, *dv, *dout;
+    CERA_TRY(cera_scratch(ctx, 0, q_bytes, &dq));
+    CERA_TRY(cera_scratch(ctx, 5, hk.size() * 4, &dk));
+    CERA_TRY(cera_scratch(ctx, 6, hv.size() * 4, &dv));
+    CERA_TRY(cera_scratch(ctx, 3, q_bytes, &dout));
+    CERA_TRY(cera_hip_upload(ctx, dq, q, q_bytes));
+    CERA_TRY(cera_hip_upload(ctx, dk, hk.data(), hk.size() * 4));
+    CERA_TRY(cera_hip_upload(ctx, dv, hv.data(), hv.size() * 4));
+    CERA_TRY(launch_flash_ref(ctx, static_cast<float*>(dq), dk, dv, n_queries, n_heads, n_kv_heads, head_dim,
+                              static_cast<uint32_t>(seq), start_pos, scale, static_cast<float*>(dout), false));
+    return cera_hip_download(ctx, out, dout, q_bytes);
 }

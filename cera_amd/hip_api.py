@@ -31,6 +31,7 @@ SYMBOLS = [
     "cera_hip_attn_decode_f16_dev", "cera_hip_shift_kv", "cera_hip_write_kv", "cera_hip_set_seq_len", "cera_hip_seq_len", "cera_hip_memory_bytes",
     "cera_hip_read_kv", "cera_hip_read_hidden",
     "cera_hip_gemv_reference_order", "cera_hip_attn_decode_reference_order", "cera_hip_rmsnorm_reference_order",
+    "cera_hip_gemm_reference_order", "cera_hip_flash_attn_reference_order",
     "cera_hip_set_reference_order", "cera_hip_reference_order",
     "cera_hip_rmsnorm_q8_0", "cera_hip_attn_decode_step", "cera_hip_attn_decode_dev_noalloc", "cera_hip_gemm_block_dots",
     "cera_hip_ffn_gate_up_fused", "cera_hip_qkv_fused",
@@ -146,6 +147,8 @@ def load_library() -> C.CDLL:
         "cera_hip_gemv_reference_order": (i32, [vp, C.POINTER(Tensor), vp, vp]),
         "cera_hip_attn_decode_reference_order": (i32, [vp, vp, vp, vp, u32, u32, u32, u64, f32, vp]),
         "cera_hip_rmsnorm_reference_order": (i32, [vp, vp, vp, u64, f32, vp]),
+        "cera_hip_gemm_reference_order": (i32, [vp, C.POINTER(Tensor), vp, u64, u32, vp]),
+        "cera_hip_flash_attn_reference_order": (i32, [vp, vp, vp, vp, u32, u32, u32, u32, u32, f32, vp]),
         "cera_hip_set_reference_order": (i32, [vp, u32]), "cera_hip_reference_order": (u32, [vp]),
         "cera_hip_attn_decode_dev_noalloc": (i32, [vp, vp, vp, vp, u32, u32, u32, u64, u64, f32, u32, vp]),
         "cera_hip_ffn_gate_up_fused": (i32, [vp, vp, vp, vp, vp, f32, vp, vp]),
@@ -443,6 +446,25 @@ class Context:
                                                                  seq_len, scale, _p(out)))
         return out
 
+    def gemm_reference_order(self, ggml_type: int, blocks: np.ndarray, x: np.ndarray, m: int, k: int,
+                             x86_repack: bool = True) -> np.ndarray:
+        """out[m][n] = W . Q8_0(x[n][k]) in the order of the x86 host's batched prefill route."""
+        t = make_tensor(ggml_type, m, k, blocks)
+        x = np.ascontiguousarray(x, np.float32).reshape(-1, k)
+        out = np.empty((m, x.shape[0]), np.float32)
+        self.check(self.lib.cera_hip_gemm_reference_order(self.h, C.byref(t), _p(x), x.shape[0], 1 if x86_repack else 0, _p(out)))
+        return out
+
+    def flash_attn_reference_order(self, q, k, v, n_heads, n_kv_heads, head_dim, start_pos, scale) -> np.ndarray:
+        """q [n][n_heads * head_dim]; k, v time-major [start_pos + n][n_kv_heads * head_dim]."""
+        q = np.ascontiguousarray(q, np.float32).reshape(-1, n_heads * head_dim)
+        k = np.ascontiguousarray(k, np.float32)
+        v = np.ascontiguousarray(v, np.float32)
+        out = np.empty_like(q)
+        self.check(self.lib.cera_hip_flash_attn_reference_order(self.h, _p(q), _p(k), _p(v), q.shape[0], n_heads, n_kv_heads,
+                                                                head_dim, start_pos, scale, _p(out)))
+        return out
+
     def rmsnorm_reference_order(self, x, w, eps) -> np.ndarray:
         x = np.ascontiguousarray(x, np.float32)
         w = np.ascontiguousarray(w, np.float32)
@@ -577,13 +599,16 @@ class Model:
                                                                         _p(out)))
         return out
 
-    def set_reference_order(self, on: bool = True):
-        """Switch to (or from) the reference-order verification route; needs an empty cache."""
-        self.ctx.check(self.ctx.lib.cera_hip_set_reference_order(self.h, 1 if on else 0))
+    def set_reference_order(self, on=True):
+        """Switch to (or from) the reference-order verification route; needs an empty cache.
+        True / 1: prefill token by token; 2: prompts of more than one token in the x86 host's
+        batched order (forward_prefill_batched with the repacked 8x8 kernels and the AVX2 flash
+        attention)."""
+        self.ctx.check(self.ctx.lib.cera_hip_set_reference_order(self.h, int(on)))
 
     @property
-    def reference_order(self) -> bool:
-        return self.ctx.lib.cera_hip_reference_order(self.h) == 1
+    def reference_order(self) -> int:
+        return int(self.ctx.lib.cera_hip_reference_order(self.h))
 
     def configure_kv(self, f16: bool):
         self.ctx.check(self.ctx.lib.cera_hip_configure_kv(self.h, 1 if f16 else 0))

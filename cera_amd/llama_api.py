@@ -155,7 +155,7 @@ class HipLlama:
 
     def set_reference_order(self, on: bool = True):
         """Verification hook: reference-order kernels (bit-identical to the CPU AVX2 path)."""
-        self._check(lib().cera_llama_set_reference_order(self.h, 1 if on else 0))
+        self._check(lib().cera_llama_set_reference_order(self.h, int(on)))
 
     def forward_prefill_chunked(self, tokens, start_pos: int, ubatch: int):
         t = np.ascontiguousarray(tokens, np.uint32)

@@ -330,6 +330,20 @@ CERA_HIP_API cera_hip_status cera_hip_attn_decode_reference_order(cera_hip_ctx*,
                                                                   float* out);
 CERA_HIP_API cera_hip_status cera_hip_rmsnorm_reference_order(cera_hip_ctx*, const float* x, const float* weight,
                                                               uint64_t n, float eps, float* y);
+/* The batched prefill's two kernels in the order of an x86 host (transformer::gemm_preq,
+ * cera/src/model/transformer.rs:710-788): out[m][n] = W . Q8_0(x[n][k]) with every element's f32
+ * chain that of gemm_q4_k_8x8_q8_0 / gemm_q4_0_8x8_q8_0 (cera/src/backend/simd.rs:5392-5518,
+ * 5215-5366) for a weight cera repacks at load (x86_repack != 0, m % 8 == 0), of the KQ_COLS-tiled
+ * K-quant kernels (:5796-5851, :6094-6168) and the strip kernels otherwise; and
+ * flash_attention_gqa_avx2 (cera/src/backend/cpu.rs:4261-4412) for n_queries queries at positions
+ * start_pos .., q / out [n_queries][n_heads * head_dim], k / v time-major
+ * [start_pos + n_queries][n_kv_heads * head_dim].  Bit-identical to the CPU kernels. */
+CERA_HIP_API cera_hip_status cera_hip_gemm_reference_order(cera_hip_ctx*, const cera_hip_tensor* w, const float* x, uint64_t n,
+                                                           uint32_t x86_repack, float* out);
+CERA_HIP_API cera_hip_status cera_hip_flash_attn_reference_order(cera_hip_ctx*, const float* q, const float* k,
+                                                                 const float* v, uint32_t n_queries, uint32_t n_heads,
+                                                                 uint32_t n_kv_heads, uint32_t head_dim, uint32_t start_pos,
+                                                                 float scale, float* out);
 
 /* ---- kernel-level entry points, device buffers (timing) ----------------- */
 CERA_HIP_API cera_hip_status cera_hip_quantize_q8_0_dev(cera_hip_ctx*, const float* x, uint64_t k, float* scales,
@@ -455,12 +469,23 @@ CERA_HIP_API cera_hip_status cera_hip_configure_kv(cera_hip_model*, uint32_t kv_
 CERA_HIP_API uint32_t cera_hip_kv_type(const cera_hip_model*);
 /* Switches a model to the reference-order verification route (on != 0) or back: forward,
  * forward_greedy and forward_prefill then run LlamaModel::forward's operations one by one
- * (cera/src/model/llama.rs:468-597, 1585-1649; prefill token by token, as :1643-1648) on the
- * reference-order kernels above, and logits are bit-identical to the CPU AVX2 path's -- the
- * harness of cera/tests/gpu_transformer_parity.rs:75-103 then sees the identical greedy token
- * stream.  Many times slower than the default route; meant for verification only.  Only with an
+ * (cera/src/model/llama.rs:468-597, 1585-1649) on the reference-order kernels above, and logits
+ * are bit-identical to the CPU AVX2 path's -- the harness of
+ * cera/tests/gpu_transformer_parity.rs:75-103 then sees the identical greedy token stream.
+ *   CERA_HIP_REF_ORDER_PER_TOKEN   forward_prefill runs token by token (llama.rs:1643-1648);
+ *   CERA_HIP_REF_ORDER_X86_BATCHED a prompt of more than one token takes
+ *       LlamaModel::forward_prefill_batched as an x86 host runs it (llama.rs:1639-1641, 738-1523):
+ *       quantize_columns, the repacked gemm_q4_k_8x8_q8_0 / gemm_q4_0_8x8_q8_0 for the weights
+ *       cera repacks at load and the tiled kernels for the rest (cera/src/backend/simd.rs:5392-5518,
+ *       5215-5366, 5796-5851, 6094-6168), flash_attention_gqa_avx2 from 256 tokens on
+ *       (cera/src/backend/cpu.rs:4261-4412), per-token attention below; one call = one batch, as
+ *       one call of the reference is (callers split prompts at their ubatch).
+ * Many times slower than the default route; meant for verification only.  Only with an
  * empty cache (CERA_HIP_ERR_POSITION otherwise); CERA_HIP_ERR_UNSUPPORTED_DTYPE if a matrix is
  * Q5_K. */
+#define CERA_HIP_REF_ORDER_OFF 0u
+#define CERA_HIP_REF_ORDER_PER_TOKEN 1u
+#define CERA_HIP_REF_ORDER_X86_BATCHED 2u
 CERA_HIP_API cera_hip_status cera_hip_set_reference_order(cera_hip_model*, uint32_t on);
 CERA_HIP_API uint32_t cera_hip_reference_order(const cera_hip_model*);
 /* Model::truncate_kv (cera/src/model/mod.rs:251-283). */

@@ -462,6 +462,27 @@ pub fn cera_hip_ctx_create(
         eps: f32,
         y: *mut f32,
     ) -> cera_hip_status;
+    pub fn cera_hip_gemm_reference_order(
+        ctx: *mut cera_hip_ctx,
+        w: *const cera_hip_tensor,
+        x: *const f32,
+        n: u64,
+        x86_repack: u32,
+        out: *mut f32,
+    ) -> cera_hip_status;
+    pub fn cera_hip_flash_attn_reference_order(
+        ctx: *mut cera_hip_ctx,
+        q: *const f32,
+        k: *const f32,
+        v: *const f32,
+        n_queries: u32,
+        n_heads: u32,
+        n_kv_heads: u32,
+        head_dim: u32,
+        start_pos: u32,
+        scale: f32,
+        out: *mut f32,
+    ) -> cera_hip_status;
     pub fn cera_hip_quantize_q8_0_dev(
         ctx: *mut cera_hip_ctx,
         x: *const f32,

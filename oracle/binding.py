@@ -102,6 +102,7 @@ def lib() -> C.CDLL:
         "orc_llama_forward_prefill_per_token": (i32, [vp, vp, u32, u32, vp]),
         "orc_llama_forward_prefill_batched": (i32, [vp, vp, u32, u32, vp, vp]),
         "orc_flash_attention_head": (None, [vp, vp, vp, vp, u64, u64, u64, u32, f32, u64]),
+        "orc_flash_attention_head_v": (None, [vp, vp, vp, vp, u64, u64, u64, u32, f32, u64, i32]),
         "orc_llama_kcache": (vp, [vp, u32]), "orc_llama_vcache": (vp, [vp, u32]),
         "orc_rope_delta_head": (None, [vp, i32, u32, f32, u32, vp]),
         "orc_llama_shift_kv": (i32, [vp, u32, u32]),
@@ -121,6 +122,11 @@ def lib() -> C.CDLL:
 def _p(a: np.ndarray) -> int:
     assert a.flags["C_CONTIGUOUS"], "array must be C contiguous"
     return a.ctypes.data
+
+
+def have_avx2() -> bool:
+    """Whether the AVX2 + FMA intrinsics twins (variant 1) can run on this host."""
+    return bool(lib().orc_have_avx2())
 
 
 def default_variant() -> int:
@@ -310,14 +316,19 @@ def decode_attention(q, k_cache, v_cache, n_heads, n_kv_heads, head_dim, scale, 
     return out
 
 
-def flash_attention_head(q, k_cache, v_cache, n_queries, kv_dim, kv_h_offset, head_dim, scale, start_pos):
-    """q [n_queries][head_dim] of one head; caches time-major [pos][kv_dim]."""
+def flash_attention_head(q, k_cache, v_cache, n_queries, kv_dim, kv_h_offset, head_dim, scale, start_pos, variant=None):
+    """q [n_queries][head_dim] of one head; caches time-major [pos][kv_dim].  variant None: the scalar
+    route; 1 / 2: flash_attention_gqa_avx2 as intrinsics / as plain C in the same order; 0 scalar."""
     q = np.ascontiguousarray(q, np.float32)
     kc = np.ascontiguousarray(k_cache, np.float32)
     vc = np.ascontiguousarray(v_cache, np.float32)
     out = np.empty((n_queries, head_dim), np.float32)
-    lib().orc_flash_attention_head(_p(q), _p(kc), _p(vc), _p(out), n_queries, kv_dim, kv_h_offset, head_dim, scale,
-                                   start_pos)
+    if variant is None:
+        lib().orc_flash_attention_head(_p(q), _p(kc), _p(vc), _p(out), n_queries, kv_dim, kv_h_offset, head_dim, scale,
+                                       start_pos)
+    else:
+        lib().orc_flash_attention_head_v(_p(q), _p(kc), _p(vc), _p(out), n_queries, kv_dim, kv_h_offset, head_dim, scale,
+                                         start_pos, variant)
     return out
 
 

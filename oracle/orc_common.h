@@ -140,3 +140,8 @@ ORC_API void orc_decode_attention(const float* q, const float* k_cache, const fl
 ORC_API void orc_flash_attention_head(const float* q, const float* k_cache, const float* v_cache, float* out,
                                       uint64_t n_queries, uint64_t kv_dim, uint64_t kv_h_offset,
                                       uint32_t head_dim, float scale, uint64_t start_pos);
+// The same head through the kernel an AVX2 host takes (flash_attention_gqa_avx2, cpu.rs:4261-4412):
+// variant 1 the intrinsics, 2 their lane algebra in plain C, 0 the scalar route above.
+ORC_API void orc_flash_attention_head_v(const float* q, const float* k_cache, const float* v_cache, float* out,
+                                        uint64_t n_queries, uint64_t kv_dim, uint64_t kv_h_offset,
+                                        uint32_t head_dim, float scale, uint64_t start_pos, int variant);

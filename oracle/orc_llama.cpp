@@ -282,8 +282,8 @@ int orc_llama_forward_prefill_batched(OrcLlama* m, const uint32_t* tokens, uint3
         const float* kcache = m->kc[l].data();
         const float* vcache = m->vc[l].data();
         if (use_flash) {
-            struct Job { const OrcLlamaConfig* c; const float *qm, *kc, *vc; float* attn; uint32_t n, start_pos, q_dim, kv_dim, group; float scale; };
-            Job job{&c, qm.data(), kcache, vcache, attn.data(), n, start_pos, q_dim, kv_dim, group, scale};
+            struct Job { const OrcLlamaConfig* c; const float *qm, *kc, *vc; float* attn; uint32_t n, start_pos, q_dim, kv_dim, group; float scale; int variant; };
+            Job job{&c, qm.data(), kcache, vcache, attn.data(), n, start_pos, q_dim, kv_dim, group, scale, m->variant};
             auto heads = [](int tid, int nt, void* a) {   // heads are independent: one range per worker
                 Job& j = *static_cast<Job*>(a);
                 const uint32_t hd = j.c->head_dim;
@@ -291,7 +291,7 @@ int orc_llama_forward_prefill_batched(OrcLlama* m, const uint32_t* tokens, uint3
                 for (uint32_t h = j.c->n_heads * uint32_t(tid) / uint32_t(nt); h < j.c->n_heads * uint32_t(tid + 1) / uint32_t(nt); ++h) {
                     for (uint32_t t = 0; t < j.n; ++t)
                         std::memcpy(qh.data() + size_t(t) * hd, j.qm + size_t(t) * j.q_dim + h * hd, hd * sizeof(float));
-                    orc_flash_attention_head(qh.data(), j.kc, j.vc, oh.data(), j.n, j.kv_dim, uint64_t(h / j.group) * hd, hd, j.scale, j.start_pos);
+                    orc_flash_attention_head_v(qh.data(), j.kc, j.vc, oh.data(), j.n, j.kv_dim, uint64_t(h / j.group) * hd, hd, j.scale, j.start_pos, j.variant);
                     for (uint32_t t = 0; t < j.n; ++t)
                         std::memcpy(j.attn + size_t(t) * j.q_dim + h * hd, oh.data() + size_t(t) * hd, hd * sizeof(float));
                 }

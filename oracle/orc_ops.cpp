@@ -289,3 +289,143 @@ void orc_flash_attention_head(const float* q, const float* k_cache, const float*
         for (uint32_t d = 0; d < head_dim; ++d) out[j * head_dim + d] = acc[d] * inv_sum;
     }
 }
+
+// ---------------------------------------------------------------------------
+// flash_attention_gqa_avx2 (cpu.rs:4261-4412), what flash_attention_gqa_cpu dispatches to on an
+// AVX2 host without AVX-512 (:4028-4140).  Same tiles and the same scalar online-softmax
+// bookkeeping as the scalar route; the QK dot is two 8-lane FMA chains over the even / odd
+// 8-wide slices of the head, added, folded by hsum256 (cpu.rs:3489) and scaled; the weighted-V
+// accumulate is one FMA per (key, column), keys in order.  The tile maximum uses `>`
+// (NaN never wins), the running maximum f32::max.
+//   variant 1: the intrinsics, operation for operation;
+//   variant 2: the same lane algebra in plain C (any host) -- bit-identical to variant 1;
+//   variant 0: the scalar route above.
+static void flash_head_avx2_order(const float* q, const float* k_cache, const float* v_cache, float* out,
+                                  uint64_t n_queries, uint64_t kv_dim, uint64_t kv_h_offset, uint32_t head_dim,
+                                  float scale, uint64_t start_pos) {
+    const int TILE = 32;
+    const uint32_t n_vecs = head_dim / 8;
+    std::vector<float> acc(head_dim);
+    float tile_scores[TILE];
+    for (uint64_t j = 0; j < n_queries; ++j) {
+        const uint64_t max_kv = start_pos + j + 1;
+        const float* ql = q + j * head_dim;
+        for (auto& a : acc) a = 0.0f;
+        float running_max = -INFINITY;
+        double running_sum = 0.0;
+        for (uint64_t kv_start = 0; kv_start < max_kv; kv_start += TILE) {
+            const uint64_t kv_end = kv_start + TILE < max_kv ? kv_start + TILE : max_kv;
+            const int tile_len = int(kv_end - kv_start);
+            for (int ti = 0; ti < tile_len; ++ti) {
+                const float* kp = k_cache + (kv_start + ti) * kv_dim + kv_h_offset;
+                float s0[8] = {0}, s1[8] = {0};
+                uint32_t i = 0;
+                while (i + 2 <= n_vecs) {
+                    for (int l = 0; l < 8; ++l) s0[l] = fmaf(ql[8 * i + l], kp[8 * i + l], s0[l]);
+                    for (int l = 0; l < 8; ++l) s1[l] = fmaf(ql[8 * (i + 1) + l], kp[8 * (i + 1) + l], s1[l]);
+                    i += 2;
+                }
+                if (i < n_vecs)
+                    for (int l = 0; l < 8; ++l) s0[l] = fmaf(ql[8 * i + l], kp[8 * i + l], s0[l]);
+                float v[8];
+                for (int l = 0; l < 8; ++l) v[l] = s0[l] + s1[l];
+                // hsum256: lo + hi, then movehl add, then lane 0 + lane 1
+                const float a0 = v[0] + v[4], a1 = v[1] + v[5], a2 = v[2] + v[6], a3 = v[3] + v[7];
+                const float b0 = a0 + a2, b1 = a1 + a3;
+                tile_scores[ti] = (b0 + b1) * scale;
+            }
+            float tile_max = -INFINITY;
+            for (int ti = 0; ti < tile_len; ++ti)
+                if (tile_scores[ti] > tile_max) tile_max = tile_scores[ti];
+            const float new_max = fmaxf(running_max, tile_max);
+            const float rescale = running_max > -INFINITY ? orc_expf(running_max - new_max) : 0.0f;
+            double tile_sum = 0.0;
+            for (int ti = 0; ti < tile_len; ++ti) {
+                tile_scores[ti] = orc_expf(tile_scores[ti] - new_max);
+                tile_sum += double(tile_scores[ti]);
+            }
+            for (uint32_t d = 0; d < head_dim; ++d) acc[d] = acc[d] * rescale;
+            for (int ti = 0; ti < tile_len; ++ti) {
+                const float sv = tile_scores[ti];
+                const float* vp = v_cache + (kv_start + ti) * kv_dim + kv_h_offset;
+                for (uint32_t d = 0; d < head_dim; ++d) acc[d] = fmaf(sv, vp[d], acc[d]);
+            }
+            running_sum = running_sum * double(rescale) + tile_sum;
+            running_max = new_max;
+        }
+        const float inv_sum = float(1.0 / running_sum);
+        for (uint32_t d = 0; d < head_dim; ++d) out[j * head_dim + d] = acc[d] * inv_sum;
+    }
+}
+#if ORC_X86
+ORC_AVX2 static void v_flash_head(const float* q, const float* k_cache, const float* v_cache, float* out,
+                                  uint64_t n_queries, uint64_t kv_dim, uint64_t kv_h_offset, uint32_t head_dim,
+                                  float scale, uint64_t start_pos) {
+    const int TILE = 32;
+    const uint32_t n_vecs = head_dim / 8;
+    __m256 q_vecs[32], acc_vecs[32];
+    float tile_scores[TILE];
+    for (uint64_t j = 0; j < n_queries; ++j) {
+        const uint64_t max_kv = start_pos + j + 1;
+        for (uint32_t i = 0; i < n_vecs; ++i) {
+            q_vecs[i] = _mm256_loadu_ps(q + j * head_dim + 8 * i);
+            acc_vecs[i] = _mm256_setzero_ps();
+        }
+        float running_max = -INFINITY;
+        double running_sum = 0.0;
+        for (uint64_t kv_start = 0; kv_start < max_kv; kv_start += TILE) {
+            const uint64_t kv_end = kv_start + TILE < max_kv ? kv_start + TILE : max_kv;
+            const int tile_len = int(kv_end - kv_start);
+            for (int ti = 0; ti < tile_len; ++ti) {
+                const float* kp = k_cache + (kv_start + ti) * kv_dim + kv_h_offset;
+                __m256 s0 = _mm256_setzero_ps(), s1 = _mm256_setzero_ps();
+                uint32_t i = 0;
+                while (i + 2 <= n_vecs) {
+                    s0 = _mm256_fmadd_ps(q_vecs[i], _mm256_loadu_ps(kp + 8 * i), s0);
+                    s1 = _mm256_fmadd_ps(q_vecs[i + 1], _mm256_loadu_ps(kp + 8 * i + 8), s1);
+                    i += 2;
+                }
+                if (i < n_vecs) s0 = _mm256_fmadd_ps(q_vecs[i], _mm256_loadu_ps(kp + 8 * i), s0);
+                tile_scores[ti] = v_hsum256(_mm256_add_ps(s0, s1)) * scale;
+            }
+            float tile_max = -INFINITY;
+            for (int ti = 0; ti < tile_len; ++ti)
+                if (tile_scores[ti] > tile_max) tile_max = tile_scores[ti];
+            const float new_max = fmaxf(running_max, tile_max);
+            const float rescale = running_max > -INFINITY ? orc_expf(running_max - new_max) : 0.0f;
+            double tile_sum = 0.0;
+            for (int ti = 0; ti < tile_len; ++ti) {
+                tile_scores[ti] = orc_expf(tile_scores[ti] - new_max);
+                tile_sum += double(tile_scores[ti]);
+            }
+            const __m256 rescale_v = _mm256_set1_ps(rescale);
+            for (uint32_t i = 0; i < n_vecs; ++i) acc_vecs[i] = _mm256_mul_ps(acc_vecs[i], rescale_v);
+            for (int ti = 0; ti < tile_len; ++ti) {
+                const __m256 sv = _mm256_set1_ps(tile_scores[ti]);
+                const float* vp = v_cache + (kv_start + ti) * kv_dim + kv_h_offset;
+                for (uint32_t i = 0; i < n_vecs; ++i) acc_vecs[i] = _mm256_fmadd_ps(sv, _mm256_loadu_ps(vp + 8 * i), acc_vecs[i]);
+            }
+            running_sum = running_sum * double(rescale) + tile_sum;
+            running_max = new_max;
+        }
+        const __m256 inv_sum_v = _mm256_set1_ps(float(1.0 / running_sum));
+        for (uint32_t i = 0; i < n_vecs; ++i) _mm256_storeu_ps(out + j * head_dim + 8 * i, _mm256_mul_ps(acc_vecs[i], inv_sum_v));
+    }
+}
+#endif
+void orc_flash_attention_head_v(const float* q, const float* k_cache, const float* v_cache, float* out,
+                                uint64_t n_queries, uint64_t kv_dim, uint64_t kv_h_offset, uint32_t head_dim,
+                                float scale, uint64_t start_pos, int variant) {
+    // the dispatcher takes the vector kernels only for head_dim % 8 == 0 and head_dim <= 256 (cpu.rs:4060-4140)
+    if (variant == 0 || head_dim % 8 != 0 || head_dim > 256) {
+        orc_flash_attention_head(q, k_cache, v_cache, out, n_queries, kv_dim, kv_h_offset, head_dim, scale, start_pos);
+        return;
+    }
+#if ORC_X86
+    if (variant == 1 && avx2_ok()) {
+        v_flash_head(q, k_cache, v_cache, out, n_queries, kv_dim, kv_h_offset, head_dim, scale, start_pos);
+        return;
+    }
+#endif
+    flash_head_avx2_order(q, k_cache, v_cache, out, n_queries, kv_dim, kv_h_offset, head_dim, scale, start_pos);
+}

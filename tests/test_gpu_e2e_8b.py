@@ -3,11 +3,16 @@
 mix), 512-token prefill of uniform random ids, then 256 greedy tokens -- the GPU
 backend through HipLlamaModel against the CPU oracle on the same file.
 
-Two GPU routes are checked, in the shape of the reference's own GPU-backend harness
+Three GPU routes are checked, in the shape of the reference's own GPU-backend harness
 (cera/tests/gpu_transformer_parity.rs:75-103, greedy_decode):
 
-* the reference-order verification route must reproduce the oracle's free-running greedy
-  stream token for token, with bit-identical logits at every step;
+* the reference-order verification route in its per-token mode must reproduce, token for token
+  and with bit-identical logits at every step, the free-running greedy stream of the oracle
+  that prefills token by token (LlamaModel::forward);
+* the same route in its x86-batched mode must do the same against the oracle that prefills the
+  way an x86 host runs this workload (cera/src/model/llama.rs forward_prefill_batched with the
+  8x8 repacked Q4_K GEMM and, from 256 prompt tokens, the AVX2 flash attention): one pass over
+  the whole prompt, bit-identical last-token logits, then the same free-running stream;
 * the default (fast) route, teacher-forced on that stream, must stay within the distance the
   reference algorithm keeps from itself (its batched-GEMM prefill route against its per-token
   route), and may pick another token only where the oracle's own margin is inside the measured
@@ -62,6 +67,9 @@ def _run(tmp_path, orc, n_layers, n_prompt, n_new):
     # the workload as a user runs it: batched prefill, free-running greedy decode
     toks_fast, tp, td = gm.generate_greedy(prompt, n_new, ubatch=512)
     _say(f"e2e: GPU prefill {n_prompt / tp:.0f} tok/s, decode {(n_new - 1) / td:.1f} tok/s")
+    gm.truncate_kv(0)
+    toks_again, _, _ = gm.generate_greedy(prompt, n_new, ubatch=512)
+    assert [int(t) for t in toks_again] == [int(t) for t in toks_fast], "GPU run is not reproducible"
 
     # ---- reference-order route, free running, every step's logits kept ----------------------
     gm.truncate_kv(0)
@@ -74,6 +82,17 @@ def _run(tmp_path, orc, n_layers, n_prompt, n_new):
         if i + 1 < n_new:
             r_logits.append(gm.forward(toks_ref[-1], n_prompt + i))
     _say(f"e2e: GPU reference-order route, {n_prompt + n_new - 1} tokens in {time.time() - t0:.0f} s")
+    # ---- reference-order route, x86-batched mode: the prompt in one pass, then free running ----
+    gm.truncate_kv(0)
+    gm.set_reference_order(2)
+    t0 = time.time()
+    x_logits = [gm.forward_prefill(prompt, 0)]
+    toks_x86 = []
+    for i in range(n_new):
+        toks_x86.append(int(orc.argmax(x_logits[-1])))
+        if i + 1 < n_new:
+            x_logits.append(gm.forward(toks_x86[-1], n_prompt + i))
+    _say(f"e2e: GPU reference-order route (x86 batched prefill), {n_prompt + n_new - 1} tokens in {time.time() - t0:.0f} s")
     gm.truncate_kv(0)
     gm.set_reference_order(False)
 
@@ -86,27 +105,33 @@ def _run(tmp_path, orc, n_layers, n_prompt, n_new):
     rcfg, weights = H.Gguf(path).llama_weights()
     rcfg["max_seq_len"] = 1024
     pool = orc.Pool(threads)
-    # Two oracle instances.  B prefills token by token (LlamaModel::forward, the route the
-    # reference-order kernels restate) and decodes free-running: the stream to reproduce.
-    # A prefills through the batched GEMM route (what the reference runs for n > 1) and follows
-    # B's tokens: the same algorithm up to how the K-quant partial sums are split over
-    # accumulators, so |A - B| is the distance the reference keeps from itself -- the floor the
-    # default route is measured against.
-    oa, ob = orc.Llama(rcfg, weights), orc.Llama(rcfg, weights)
-    oa.set_pool(pool); ob.set_pool(pool)
+    # Three oracle instances.  B prefills token by token (LlamaModel::forward, the route the
+    # per-token reference-order kernels restate) and decodes free-running: the stream the
+    # per-token mode reproduces.  A prefills through the batched GEMM route as an x86 host runs
+    # it (repacked 8x8 Q4_K GEMM, flash attention from 256 tokens) and then follows B's tokens:
+    # the same algorithm up to how the partial sums are ordered, so |A - B| is the distance the
+    # reference keeps from itself -- the floor the default route is measured against.  C starts
+    # from a copy of A's KV caches and prefill logits and decodes free-running: the stream the
+    # x86-batched mode reproduces.
+    oa, ob, oc = orc.Llama(rcfg, weights), orc.Llama(rcfg, weights), orc.Llama(rcfg, weights)
+    oa.set_pool(pool); ob.set_pool(pool); oc.set_pool(pool)
+    oa.set_x86_repack(True)
     t0 = time.time()
     lb = ob.forward_prefill_per_token(prompt, 0)
     _say(f"e2e: oracle per-token prefill {time.time() - t0:.0f} s on {threads} threads")
     t0 = time.time()
     la = oa.forward_prefill_batched(prompt, 0)
-    _say(f"e2e: oracle batched prefill {time.time() - t0:.0f} s")
+    _say(f"e2e: oracle batched prefill (x86 order) {time.time() - t0:.0f} s")
+    oc.restore([oa.kv(l) for l in range(n_layers)], n_prompt)
+    lc = la.copy()
 
     def cos(x, y):
         x, y = x.astype(np.float64), y.astype(np.float64)
         return float(x @ y / np.sqrt((x @ x) * (y @ y)))
 
-    same_ref = same_g = same_a = 0
-    bit_equal_steps = 0
+    same_ref = same_x86 = same_g = same_a = 0
+    bit_equal_steps = bit_equal_x86 = 0
+    first_tf = n_new   # first step at which the default route, teacher-forced, picks another token
     worst_g = 0.0   # largest margin of a default-route disagreement, in units of the per-logit noise rms
     rel_g, rel_a, cos_g, cos_a = [], [], [], []
     t0 = time.time()
@@ -119,6 +144,14 @@ def _run(tmp_path, orc, n_layers, n_prompt, n_new):
         bit_equal_steps += 1
         assert toks_ref[i] == tb, f"step {i}: reference-order token {toks_ref[i]} != oracle {tb}"
         same_ref += 1
+        # x86-batched mode against the oracle that prefilled in one pass the x86 way
+        tc = int(orc.argmax(lc))
+        diff = int(np.count_nonzero(_bits(x_logits[i]) != _bits(lc)))
+        assert diff == 0, (f"step {i}: x86-batched reference-order logits differ from the oracle's in {diff} of "
+                           f"{lc.size} entries, max |diff| {float(np.abs(x_logits[i] - lc).max()):.3e}")
+        bit_equal_x86 += 1
+        assert toks_x86[i] == tc, f"step {i}: x86-batched reference-order token {toks_x86[i]} != oracle {tc}"
+        same_x86 += 1
         # default route
         lg = g_logits[i]
         tg, ta = int(orc.argmax(lg)), int(orc.argmax(la))
@@ -136,23 +169,33 @@ def _run(tmp_path, orc, n_layers, n_prompt, n_new):
             m_b, m_g = float(lb[tb] - lb[tg]), float(lg[tg] - lg[tb])
             _say(f"  step {i}: default route {tg} vs oracle {tb}: margins {m_b:.3f} / {m_g:.3f}, logit noise rms {noise:.3f}")
             worst_g = max(worst_g, max(m_b, m_g) / noise)
+            first_tf = min(first_tf, i)
             assert m_b <= 7 * noise and m_g <= 7 * noise, f"step {i}: different token beyond the noise"
         if i + 1 < n_new:
             lb, la = ob.forward(tb, n_prompt + i), oa.forward(tb, n_prompt + i)
+            lc = oc.forward(tc, n_prompt + i)
     _say(f"e2e: oracle decode {time.time() - t0:.0f} s")
     _say(f"e2e: GPU reference-order route vs oracle: identical greedy tokens {same_ref}/{n_new} (free running), "
          f"logits bit-identical at {bit_equal_steps}/{n_new} steps")
+    _say(f"e2e: GPU reference-order route, x86-batched mode vs oracle(x86 batched prefill): identical greedy tokens "
+         f"{same_x86}/{n_new} (free running), logits bit-identical at {bit_equal_x86}/{n_new} steps "
+         f"(step 0 = last-token logits of the {n_prompt}-token one-pass prefill)")
     _say(f"e2e: GPU default route vs oracle (teacher-forced): identical greedy tokens {same_g}/{n_new}, "
          f"cosine min {min(cos_g):.5f} mean {np.mean(cos_g):.5f}, rms(diff)/rms mean {np.mean(rel_g):.4f}, "
          f"largest disagreement margin {worst_g:.1f} x noise")
     _say(f"e2e: oracle(batched) vs oracle(per-token): identical greedy tokens {same_a}/{n_new}, "
          f"cosine min {min(cos_a):.5f} mean {np.mean(cos_a):.5f}, rms(diff)/rms mean {np.mean(rel_a):.4f}")
-    _say(f"e2e: GPU default route free-running stream shares a prefix of "
-         f"{next((i for i, (a, b) in enumerate(zip(toks_fast, toks_ref)) if int(a) != b), n_new)}/{n_new} tokens with the oracle's")
-    oa.set_pool(None); ob.set_pool(None)
+    first_free = next((i for i, (a, b) in enumerate(zip(toks_fast, toks_ref)) if int(a) != b), n_new)
+    _say(f"e2e: GPU default route free-running stream shares a prefix of {first_free}/{n_new} tokens with the oracle's")
+    oa.set_pool(None); ob.set_pool(None); oc.set_pool(None)
     pool.close()
-    oa.close(); ob.close()
+    oa.close(); ob.close(); oc.close()
     assert same_ref == n_new and bit_equal_steps == n_new
+    assert same_x86 == n_new and bit_equal_x86 == n_new
+    # Up to its first disagreement the free-running default route has seen the same tokens as the
+    # teacher-forced one, so it leaves the oracle's stream exactly where that one first picks another
+    # token -- a step the margin rule above has already explained by the logit noise.
+    assert first_free == first_tf, f"free-running default route leaves the oracle's stream at {first_free}, teacher-forced at {first_tf}"
     # 0.99 is the floor the reference sets for its own flash-route (n >= 256) prefill comparison
     # (cera/tests/llama_batched_prefill_parity.rs:337-358)
     assert min(cos_g) >= 0.99

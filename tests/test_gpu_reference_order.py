@@ -6,6 +6,11 @@ GEMV: gemm_q4_k_q8_0 / gemm_q6_k_q8_0 at n == 1 (cera/src/backend/simd.rs:5742-5
 row_dot_q4_0 / row_dot_q8_0 (:4593-4637), gemm_q4_1_q8_0 (:5893-5976).  Attention: attn_scores /
 softmax_inplace / attn_values, AVX2 tier (cera/src/backend/cpu.rs:3503-3589, 2617-2633).
 rmsnorm: cera/src/backend/cpu.rs:2479-2496.  Model: LlamaModel::forward (llama.rs:468-597).
+
+Batched prefill as an x86 host runs it (LlamaModel::forward_prefill_batched, llama.rs:738-1523):
+transformer::gemm_preq with the repacked gemm_q4_k_8x8_q8_0 / gemm_q4_0_8x8_q8_0 (simd.rs:5392-5518,
+5215-5366) and the tiled K-quant / strip kernels (:5796-5851, :6094-6168), flash_attention_gqa_avx2
+(cpu.rs:4261-4412).
 """
 import math
 
@@ -88,6 +93,53 @@ def test_rmsnorm_reference_order_is_bit_identical(hip, orc, n):
     assert _same_bits(hip.rmsnorm_reference_order(x, w, 1e-5), orc.rmsnorm(x, w, 1e-5))
 
 
+# ---- the batched prefill's kernels ---------------------------------------------------------------
+@pytest.mark.parametrize("dtype,m,k,n", [
+    (util.Q4_K, 96, 4096, 5), (util.Q4_K, 64, 512, 9), (util.Q4_K, 36, 512, 3),      # 36 rows: not repacked (m % 8)
+    (util.Q6_K, 96, 4096, 5), (util.Q6_K, 5, 256, 4),
+    (util.Q4_0, 96, 4096, 3), (util.Q4_0, 7, 96, 2), (util.Q8_0, 64, 1024, 4), (util.Q4_1, 24, 256, 3),
+])
+def test_gemm_reference_order_is_bit_identical(hip, orc, dtype, m, k, n):
+    """Every output element carries the bits of the x86 host's batched route: the 8x8 kernels for the
+    weights cera repacks at load, the tiled (one-accumulator) K-quant kernels and the strip kernels
+    otherwise -- and, with the repack switched off, of the standard route for every weight."""
+    w, _ = util.make_weights(dtype, m, k, seed=m + n)
+    x = util.make_x(n * k, seed=k + n).reshape(n, k)
+    q = [orc.quantize_q8_0(x[j]) for j in range(n)]
+    bs = np.stack([a for a, _ in q]); bq = np.stack([b for _, b in q])
+    _say(f"ref-order gemm {util.NAMES[dtype]} {m}x{k} x {n}")
+    got = hip.gemm_reference_order(dtype, w, x, m, k, x86_repack=True)
+    assert _same_bits(got, orc.gemm_preq_x86(dtype, w, bs, bq, m, n, k)), (dtype, m, k, n)
+    got = hip.gemm_reference_order(dtype, w, x, m, k, x86_repack=False)
+    assert _same_bits(got, orc.gemm_preq(dtype, w, bs, bq, m, n, k)), (dtype, m, k, n)
+
+
+def test_gemm_reference_order_repack_changes_bits(hip, orc):
+    """The two routes really are different float chains (if they were not, the test above would pin
+    nothing about which one ran)."""
+    m, k, n = 64, 1024, 6
+    w, _ = util.make_weights(util.Q4_K, m, k, seed=3)
+    x = util.make_x(n * k, seed=4).reshape(n, k)
+    a = hip.gemm_reference_order(util.Q4_K, w, x, m, k, x86_repack=True)
+    b = hip.gemm_reference_order(util.Q4_K, w, x, m, k, x86_repack=False)
+    assert not _same_bits(a, b) and np.abs(a - b).max() <= 1e-4 * util.rms(a)
+
+
+@pytest.mark.parametrize("n_heads,n_kv,hd,n,start", [(8, 2, 128, 70, 300), (4, 4, 64, 33, 0), (6, 2, 72, 9, 40)])
+def test_flash_attention_reference_order_is_bit_identical(hip, orc, n_heads, n_kv, hd, n, start):
+    total = start + n
+    q = util.make_x(n * n_heads * hd, 1).reshape(n, n_heads, hd)
+    kc = util.make_x(total * n_kv * hd, 2)
+    vc = util.make_x(total * n_kv * hd, 3)
+    scale = 1.0 / math.sqrt(hd)
+    _say(f"ref-order flash attention {n_heads}/{n_kv}/{hd}, {n} queries from {start}")
+    got = hip.flash_attn_reference_order(q, kc, vc, n_heads, n_kv, hd, start, scale).reshape(n, n_heads, hd)
+    for h in range(n_heads):
+        off = (h // (n_heads // n_kv)) * hd
+        ref = orc.flash_attention_head(np.ascontiguousarray(q[:, h, :]), kc, vc, n, n_kv * hd, off, hd, scale, start, variant=2)
+        assert _same_bits(got[:, h, :], ref), (h,)
+
+
 # ---- whole models ------------------------------------------------------------------------------
 def _extras(cfg, w, seed, bias=False, qk_norm=False, freqs=False):
     w = dict(w)
@@ -147,6 +199,54 @@ def test_model_reference_order_logits_bit_identical(hip, orc, name):
         to = int(orc.argmax(om.forward(to, pos)))
         tg = gm.forward_greedy(tg, pos)
         assert tg == to, (name, pos)
+    gm.close(); om.close()
+
+
+@pytest.mark.parametrize("name", ["llama_q4_k_m", "qwen2_neox_bias", "qwen3_qknorm_hd64", "granite_scalars", "q4_0"])
+@pytest.mark.parametrize("n_prompt", [9, 260])
+def test_model_reference_order_x86_batched_prefill(hip, orc, name, n_prompt):
+    """Mode 2: a prompt of more than one token goes through forward_prefill_batched in the x86 host's
+    order (repacked 8x8 GEMMs; 260 tokens: the AVX2 flash attention, 9: per-token attention).  Last-row
+    logits, every cache row and the greedy continuation carry the oracle's bits -- the oracle here is
+    orc.Llama with set_x86_repack(True) and forward_prefill_batched."""
+    over, mk, ex = MODELS[name]
+    cfg = dict(synth.TINY, max_seq_len=320, **over)
+    weights = _extras(cfg, synth.make_llama(cfg, seed=123, sigma=0.05, norm_jitter=0.1, **mk), 9, **ex)
+    gm = hip_api.Model(hip, cfg, weights)
+    om = orc.Llama(cfg, weights)
+    om.set_x86_repack(True)
+    gm.set_reference_order(2)
+    assert gm.reference_order == 2
+    prompt = [int(t) for t in util.rng(8).integers(0, cfg["vocab"], n_prompt)]
+    _say(f"ref-order x86 batched prefill {name}: {n_prompt} tokens + 12 greedy")
+    lg, lo = gm.forward_prefill(prompt, 0), om.forward_prefill_batched(prompt, 0)
+    assert _same_bits(lg, lo), (name, float(np.abs(lg - lo).max()))
+    for layer in range(cfg["n_layers"]):
+        kg, vg = gm.read_kv(layer)
+        ko, vo = om.kv(layer)
+        assert _same_bits(kg, ko) and _same_bits(vg, vo), (name, layer)
+    for i in range(12):
+        tg, to = int(orc.argmax(lg)), int(orc.argmax(lo))
+        assert tg == to
+        lg, lo = gm.forward(tg, n_prompt + i), om.forward(to, n_prompt + i)
+        assert _same_bits(lg, lo), (name, i)
+    # a second batch appended behind the first (start_pos > 0)
+    more = [int(t) for t in util.rng(9).integers(0, cfg["vocab"], 7)]
+    pos = n_prompt + 12
+    assert _same_bits(gm.forward_prefill(more, pos), om.forward_prefill_batched(more, pos))
+    gm.close(); om.close()
+
+
+def test_model_reference_order_x86_batched_prefill_f16_kv(hip, orc):
+    cfg = dict(synth.TINY, max_seq_len=320)
+    weights = synth.make_llama(cfg, seed=45, sigma=0.05, norm_jitter=0.1)
+    gm = hip_api.Model(hip, cfg, weights)
+    om = orc.Llama(cfg, weights)
+    gm.configure_kv(True); om.set_kv_f16(True)
+    om.set_x86_repack(True)
+    gm.set_reference_order(2)
+    prompt = [int(t) for t in util.rng(10).integers(0, cfg["vocab"], 258)]
+    assert _same_bits(gm.forward_prefill(prompt, 0), om.forward_prefill_batched(prompt, 0))
     gm.close(); om.close()
 
 

@@ -48,6 +48,73 @@ def test_flash_matches_naive_reference_fixture(orc):
             assert np.abs(got[j] - p @ v).max() < 1e-4
 
 
+def _flash_fixture():
+    # cpu.rs:7091-7223: 4 heads, 2 kv heads, hd 64, n=8, start_pos 4, LCG seed 0xCAFEBABE
+    nh, nkv, hd, n, start = 4, 2, 64, 8, 4
+    state = [0xCAFEBABE]
+    mask = (1 << 64) - 1
+
+    def draw(count):
+        out = np.empty(count, np.float32)
+        for i in range(count):
+            state[0] = (state[0] * 6364136223846793005 + 1) & mask
+            v = (state[0] >> 33) & 0xFFFFFFFF
+            if v >= 1 << 31:
+                v -= 1 << 32
+            out[i] = np.float32(v) * np.float32(1e-9)
+        return out
+
+    total = start + n
+    return nh, nkv, hd, n, start, draw(n * nh * hd).reshape(n, nh, hd), draw(total * nkv * hd), draw(total * nkv * hd)
+
+
+def test_flash_avx2_order_matches_naive_reference_fixture(orc):
+    """flash_attention_gqa_avx2 (cpu.rs:4261-4412), the kernel an AVX2 host takes: pinned like the
+    scalar route on the reference's own fixture (max diff < 1e-4 against textbook attention), the
+    plain-C lane algebra (variant 2) bit-identical to the intrinsics (variant 1) where those run."""
+    nh, nkv, hd, n, start, q, kc, vc = _flash_fixture()
+    total = start + n
+    scale = 1.0 / math.sqrt(hd)
+    for h in range(nh):
+        off = (h // (nh // nkv)) * hd
+        got = orc.flash_attention_head(q[:, h, :], kc, vc, n, nkv * hd, off, hd, scale, start, variant=2)
+        for j in range(n):
+            L = start + j + 1
+            k = kc.reshape(total, nkv * hd)[:L, off:off + hd].astype(np.float64)
+            v = vc.reshape(total, nkv * hd)[:L, off:off + hd].astype(np.float64)
+            s = k @ q[j, h].astype(np.float64) * scale
+            p = np.exp(s - s.max()); p /= p.sum()
+            assert np.abs(got[j] - p @ v).max() < 1e-4
+        if orc.have_avx2():
+            twin = orc.flash_attention_head(q[:, h, :], kc, vc, n, nkv * hd, off, hd, scale, start, variant=1)
+            assert np.array_equal(got.view(np.uint32), twin.view(np.uint32))
+
+
+def test_flash_avx2_order_on_long_ragged_contexts(orc):
+    """Several tiles, a ragged last tile, head_dim 64 / 128 / 72 (an odd number of 8-wide slices: the
+    lone-slice tail of the QK loop), start_pos > 0: the two restatements of the AVX2 kernel agree bit for
+    bit, differ from the scalar route only by summation order, and a head_dim the vector kernel does not
+    take (not a multiple of 8) falls back to the scalar route as the dispatcher does (cpu.rs:4096-4100)."""
+    for hd, nkv, n, start in ((128, 2, 70, 300), (64, 1, 33, 95), (72, 1, 5, 40)):
+        total = start + n
+        q = util.make_x(n * hd, 1).reshape(n, hd)
+        kc = util.make_x(total * nkv * hd, 2)
+        vc = util.make_x(total * nkv * hd, 3)
+        scale = 1.0 / math.sqrt(hd)
+        off = (nkv - 1) * hd
+        a = orc.flash_attention_head(q, kc, vc, n, nkv * hd, off, hd, scale, start, variant=2)
+        s = orc.flash_attention_head(q, kc, vc, n, nkv * hd, off, hd, scale, start)
+        assert np.abs(a - s).max() < 2e-6 and not np.array_equal(a, s)
+        if orc.have_avx2():
+            b = orc.flash_attention_head(q, kc, vc, n, nkv * hd, off, hd, scale, start, variant=1)
+            assert np.array_equal(a.view(np.uint32), b.view(np.uint32)), hd
+    hd = 20
+    q = util.make_x(3 * hd, 4).reshape(3, hd)
+    kc = util.make_x(10 * hd, 5); vc = util.make_x(10 * hd, 6)
+    assert np.array_equal(orc.flash_attention_head(q, kc, vc, 3, hd, 0, hd, 0.3, 7, variant=2),
+                          orc.flash_attention_head(q, kc, vc, 3, hd, 0, hd, 0.3, 7))
+
+
 def test_flash_equals_decode_attention_on_long_context(orc):
     nkv, hd, n, start = 2, 128, 70, 300
     total = start + n
