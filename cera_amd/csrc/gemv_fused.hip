@@ -40,19 +40,35 @@ static void fill(RowGemvArgs& a, const cera_hip_dtensor* w, const cera_hip_dtens
 // it, as the reference's own x86 path does with repack_q4_k_8x8 (cera/src/backend/cpu.rs:1282-1358);
 // the native bytes stay for every other reader (prefill GEMM, embedding lookup, verification
 // route).  Other types and views are left alone.
-cera_hip_status cera_tensor_prepare_stream(cera_hip_ctx* ctx, cera_hip_dtensor* w) {
-    if (!ctx->decode_copies) return CERA_HIP_OK;
-    if (!w || w->dev_stream || !w->owns || w->k > 32768 || w->m == 0 || w->m > 0x7FFFFFFFull) return CERA_HIP_OK;
-    if (row_tiles(w->dtype, w->k) == 0 || (reinterpret_cast<uintptr_t>(w->dev) & 15)) return CERA_HIP_OK;
+static uint64_t stream_row_bytes_of(const cera_hip_ctx* ctx, const cera_hip_dtensor* w) {
+    if (!ctx->decode_copies) return 0;
+    if (!w || !w->owns || w->k > 32768 || w->m == 0 || w->m > 0x7FFFFFFFull) return 0;
+    if (row_tiles(w->dtype, w->k) == 0 || (reinterpret_cast<uintptr_t>(w->dev) & 15)) return 0;
     const uint32_t k = static_cast<uint32_t>(w->k);
-    uint64_t srb = 0;
     switch (w->dtype) {
-        case CERA_HIP_Q4_K: srb = Q4K::stream_row_bytes(k); break;
-        case CERA_HIP_Q6_K: srb = Q6K::stream_row_bytes(k); break;
-        case CERA_HIP_Q4_0: srb = Q4_0::stream_row_bytes(k); break;
-        case CERA_HIP_Q4_1: srb = Q4_1::stream_row_bytes(k); break;
-        default: srb = Q8_0::stream_row_bytes(k); break;
+        case CERA_HIP_Q4_K: return Q4K::stream_row_bytes(k);
+        case CERA_HIP_Q6_K: return Q6K::stream_row_bytes(k);
+        case CERA_HIP_Q4_0: return Q4_0::stream_row_bytes(k);
+        case CERA_HIP_Q4_1: return Q4_1::stream_row_bytes(k);
+        default: return Q8_0::stream_row_bytes(k);
     }
+}
+// bytes a decode copy of w would take; 0 when w gets none (copies off, a view, a type or shape
+// without a streaming kernel) or already has one
+uint64_t cera_tensor_stream_bytes(const cera_hip_ctx* ctx, const cera_hip_dtensor* w) {
+    return (w && w->dev_stream) ? 0 : stream_row_bytes_of(ctx, w) * (w ? w->m : 0);
+}
+void cera_tensor_drop_stream(cera_hip_dtensor* w) {
+    if (!w || !w->dev_stream) return;
+    (void)hipFree(w->dev_stream);
+    w->dev_stream = nullptr;
+    w->stream_row_bytes = 0;
+}
+cera_hip_status cera_tensor_prepare_stream(cera_hip_ctx* ctx, cera_hip_dtensor* w) {
+    if (!w || w->dev_stream) return CERA_HIP_OK;
+    const uint64_t srb = stream_row_bytes_of(ctx, w);
+    if (srb == 0) return CERA_HIP_OK;
+    const uint32_t k = static_cast<uint32_t>(w->k);
     void* p = nullptr;
     const hipError_t e = hipMalloc(&p, srb * w->m);
     if (e != hipSuccess) {

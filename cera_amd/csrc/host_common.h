@@ -94,6 +94,9 @@ cera_hip_status cera_launch_gemv(cera_hip_ctx* ctx, const cera_hip_dtensor* w, c
 cera_hip_status cera_launch_row_gemv_add(cera_hip_ctx* ctx, const cera_hip_dtensor* w, const float* xs, const int8_t* xq,
                                          float* y, const float* resid, bool* launched);
 cera_hip_status cera_tensor_prepare_stream(cera_hip_ctx* ctx, cera_hip_dtensor* w);
+// bytes a decode copy of w would take (0: none possible, or it has one); free an existing one
+uint64_t cera_tensor_stream_bytes(const cera_hip_ctx* ctx, const cera_hip_dtensor* w);
+void cera_tensor_drop_stream(cera_hip_dtensor* w);
 cera_hip_status cera_launch_row_gemv_store(cera_hip_ctx* ctx, const cera_hip_dtensor* w, const float* xs, const int8_t* xq,
                                            float* y, bool* launched);
 cera_hip_status cera_launch_row_gemv_long_add(cera_hip_ctx* ctx, const cera_hip_dtensor* w, const float* xs, const int8_t* xq,

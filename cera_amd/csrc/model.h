@@ -89,5 +89,9 @@ cera_hip_status cera_model_prefill_ref_batched(cera_hip_model* m, const uint32_t
                                                bool want_logits);
 // (re)allocates the prefill pass buffers for n tokens (at most one pass's capacity, m->pf_cap)
 cera_hip_status cera_model_ensure_prefill_buffers(cera_hip_model* m, uint32_t n);
+// hipMalloc for allocations made after model creation: out of memory -> the decode copies are
+// freed and the allocation is tried once more
+cera_hip_status cera_model_malloc(cera_hip_model* m, void** out, uint64_t bytes, const char* what);
+uint64_t cera_model_drop_decode_copies(cera_hip_model* m);
 bool cera_model_ref_order_supported(const cera_hip_model* m, std::string* why);
 cera_hip_status cera_model_decode_logits(cera_hip_model* m, uint32_t token, uint32_t pos, float* logits);

@@ -10,6 +10,7 @@
 
 #include <type_traits>
 
+#include "copy_budget.h"
 #include "glue.hip.h"
 #include "host_common.h"
 #include "model.h"
@@ -35,6 +36,71 @@ static cera_hip_status upload_f32(cera_hip_ctx* ctx, const float* host, uint64_t
 static cera_hip_status alloc_kv_cache(cera_hip_ctx* ctx, uint64_t bytes, void** out, uint64_t* total) {
     CERA_TRY(dev_alloc(ctx, bytes, out, total));
     HIP_TRY(ctx, hipMemsetAsync(*out, 0, bytes, ctx->stream));
+    return CERA_HIP_OK;
+}
+
+// The matrices the one-wavefront-per-row decode kernels stream, in the order copies are handed
+// out: the vocabulary head first (a tied head: the embedding table), then layer by layer.
+static std::vector<cera_hip_dtensor*> decode_copy_candidates(cera_hip_model* m) {
+    std::vector<cera_hip_dtensor*> v;
+    v.push_back(m->output ? m->output : m->embd);
+    for (LayerDev& D : m->layers)
+        for (cera_hip_dtensor* w : {D.qkv, D.v, D.o, D.gate, D.up, D.down})
+            if (w && w->owns) v.push_back(w);
+    return v;
+}
+
+// Decode copies come last -- after every native upload, the KV caches and the single-token
+// buffers -- and only from memory the model will not need later (copy_budget.h): a model that
+// loads and prefills with copies off must do so with copies on.
+static cera_hip_status build_decode_copies(cera_hip_model* m) {
+    cera_hip_ctx* ctx = m->ctx;
+    if (!ctx->decode_copies) return CERA_HIP_OK;
+    std::vector<cera_hip_dtensor*> cand = decode_copy_candidates(m);
+    std::vector<uint64_t> bytes(cand.size());
+    for (size_t i = 0; i < cand.size(); ++i) bytes[i] = cera_tensor_stream_bytes(ctx, cand[i]);
+    size_t free_b = 0, total_b = 0;
+    HIP_TRY(ctx, hipMemGetInfo(&free_b, &total_b));
+    std::vector<uint8_t> take(cand.size());
+    cera_plan_decode_copies(bytes.data(), bytes.size(), free_b, cera_copy_reserve_bytes(m->cfg), take.data());
+    for (size_t i = 0; i < cand.size(); ++i) {
+        if (!take[i]) continue;
+        CERA_TRY(cera_tensor_prepare_stream(ctx, cand[i]));
+        if (cand[i]->dev_stream) m->bytes += cand[i]->stream_row_bytes * cand[i]->m;
+    }
+    return CERA_HIP_OK;
+}
+
+// Frees every decode copy of the model (the kernels then read the native bytes); returns the bytes
+// given back.  The stream is drained first: a launched kernel may still be reading a copy.
+uint64_t cera_model_drop_decode_copies(cera_hip_model* m) {
+    uint64_t freed = 0;
+    (void)hipStreamSynchronize(m->ctx->stream);
+    for (cera_hip_dtensor* w : decode_copy_candidates(m)) {
+        if (!w->dev_stream) continue;
+        freed += w->stream_row_bytes * w->m;
+        cera_tensor_drop_stream(w);
+    }
+    m->bytes -= std::min(m->bytes, freed);
+    return freed;
+}
+
+// hipMalloc for a model's later allocations (prefill buffers, all-positions logits, re-typed KV
+// caches): when the device is out of memory the decode copies are given up and the allocation is
+// tried once more.
+cera_hip_status cera_model_malloc(cera_hip_model* m, void** out, uint64_t bytes, const char* what) {
+    *out = nullptr;
+    hipError_t e = hipMalloc(out, bytes ? bytes : 256);
+    if (e == hipErrorOutOfMemory) {
+        (void)hipGetLastError();
+        if (cera_model_drop_decode_copies(m) > 0) e = hipMalloc(out, bytes ? bytes : 256);
+    }
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        *out = nullptr;
+        return cera_fail(m->ctx, e == hipErrorOutOfMemory ? CERA_HIP_ERR_OOM : CERA_HIP_ERR_DEVICE,
+                         std::string("hipMalloc(") + what + ", " + std::to_string(bytes) + " bytes): " + hipGetErrorString(e));
+    }
     return CERA_HIP_OK;
 }
 
@@ -154,11 +220,6 @@ extern "C" cera_hip_status cera_hip_model_create(cera_hip_ctx* ctx, const cera_h
             CERA_TRY(cera_hip_tensor_upload(ctx, &output_cut, &m->output));
             *tot += m->output->nbytes;
         }
-        {   // the vocabulary head streams a decode copy too (a tied head: the embedding table's)
-            cera_hip_dtensor* head = m->output ? m->output : m->embd;
-            CERA_TRY(cera_tensor_prepare_stream(ctx, head));
-            if (head->dev_stream) *tot += head->stream_row_bytes * head->m;
-        }
         float* tmp;
         CERA_TRY(upload_f32(ctx, output_norm, c.hidden, &tmp, tot));
         m->output_norm = tmp; m->owned.push_back(tmp);
@@ -183,12 +244,6 @@ extern "C" cera_hip_status cera_hip_model_create(cera_hip_ctx* ctx, const cera_h
             for (int t = fuse; t < 7; ++t) {
                 CERA_TRY(cera_hip_tensor_upload(ctx, src[t], dst[t]));
                 *tot += (*dst[t])->nbytes;
-            }
-            // decode copies of what the one-wavefront-per-row kernels stream
-            for (cera_hip_dtensor* w : {D.qkv, D.v, D.o, D.gate, D.up, D.down}) {
-                if (!w || w->dev_stream) continue;
-                CERA_TRY(cera_tensor_prepare_stream(ctx, w));
-                if (w->dev_stream) *tot += w->stream_row_bytes * w->m;
             }
             CERA_TRY(upload_f32(ctx, L.attn_norm, c.hidden, &D.attn_norm, tot));
             CERA_TRY(upload_f32(ctx, L.ffn_norm, c.hidden, &D.ffn_norm, tot));
@@ -236,7 +291,8 @@ extern "C" cera_hip_status cera_hip_model_create(cera_hip_ctx* ctx, const cera_h
         m->owned.push_back(m->xq);
         CERA_TRY(dev_alloc_t(ctx, 4, &m->scalars, tot));  // [token, pos, argmax, spare]
         m->owned.push_back(m->scalars);
-        return CERA_HIP_OK;
+        // last, from what is left: the decode copies
+        return build_decode_copies(m);
     };
     cera_hip_status st = build();
     if (st != CERA_HIP_OK) {
@@ -250,6 +306,18 @@ extern "C" cera_hip_status cera_hip_model_create(cera_hip_ctx* ctx, const cera_h
 }
 
 extern "C" void cera_hip_model_destroy(cera_hip_model* m) { free_model(m); }
+extern "C" uint64_t cera_hip_decode_copy_reserve_bytes(const cera_hip_config* cfg) { return cfg ? cera_copy_reserve_bytes(*cfg) : 0; }
+extern "C" uint64_t cera_hip_decode_copy_plan(const uint64_t* copy_bytes, uint32_t n, uint64_t free_bytes, uint64_t reserve_bytes,
+                                              uint8_t* take) {
+    return copy_bytes ? cera_plan_decode_copies(copy_bytes, n, free_bytes, reserve_bytes, take) : 0;
+}
+extern "C" cera_hip_status cera_hip_drop_decode_copies(cera_hip_model* m, uint64_t* freed_bytes) {
+    if (!m) return CERA_HIP_ERR_ARGUMENT;
+    ModelLock lk(m);
+    const uint64_t f = cera_model_drop_decode_copies(m);
+    if (freed_bytes) *freed_bytes = f;
+    return CERA_HIP_OK;
+}
 extern "C" uint32_t cera_hip_seq_len(const cera_hip_model* m) { return m ? m->seq_len : 0; }
 extern "C" uint64_t cera_hip_memory_bytes(const cera_hip_model* m) { return m ? m->bytes : 0; }
 

@@ -5,6 +5,7 @@
 #include <cmath>
 #include <cstring>
 
+#include "copy_budget.h"
 #include "gemm_q5k_f16.hip.h"
 #include "gemm_q6k_f16.hip.h"
 #include "gemm_fp8.hip.h"
@@ -24,7 +25,8 @@ static bool gemm_f32_supports(uint32_t dtype, uint64_t k) { return dtype == CERA
 static bool gemm_batched(uint32_t dtype, uint64_t k) { return cera_gemm_supports(dtype, k) || gemm_f32_supports(dtype, k); }
 
 // bytes of the fragment-ordered fp8 split copy of n activation rows of k elements
-uint64_t cera_gemm_fp8_ws_bytes(uint64_t n, uint64_t k) { return (n + G8_BN - 1) / G8_BN * 2 * (k / 256) * G8_REC; }
+static_assert(G8_BN == 64 && G8_REC == 21504, "cera_fp8_split_bytes (copy_budget.h) restates this record geometry");
+uint64_t cera_gemm_fp8_ws_bytes(uint64_t n, uint64_t k) { return cera_fp8_split_bytes(n, k); }
 
 // out[i*ld_m + j*ld_n] = (W . B)[i][j] (+ resid)
 // w2 / out2 (nullable): a second matrix of the same type and k multiplied by the same activations
@@ -394,7 +396,7 @@ extern "C" cera_hip_status cera_hip_gemm_swiglu(cera_hip_ctx* ctx, const cera_hi
 // wants the reference Session's default ubatch of 512 (cera/src/model/mod.rs:303-332) gets it
 // through forward_prefill_chunked; given the whole prompt, 2048-token passes amortise the weight
 // staging of the GEMM better (+15 % tokens/s on an 8k prompt).
-static constexpr uint32_t PREFILL_CHUNK = 2048;
+static constexpr uint32_t PREFILL_CHUNK = CERA_PREFILL_CHUNK;
 // batches up to this many tokens run their projections on the multi-token GEMV instead of the GEMM
 // (measured on the 8B shapes: 2 tokens 2.8 ms against 7.7 ms, 8 tokens 5.4 against 7.9, 16 tokens
 // 10.7 against 9.4 -- the per-token dots grow with the batch while the GEMM's tile fills up)
@@ -404,36 +406,35 @@ cera_hip_status cera_model_ensure_prefill_buffers(cera_hip_model* m, uint32_t n)
     if (m->pf_cap >= n) return CERA_HIP_OK;
     cera_hip_ctx* ctx = m->ctx;
     const cera_hip_config& c = m->cfg;
-    const uint64_t q_dim = static_cast<uint64_t>(c.n_heads) * c.head_dim, kv_dim = static_cast<uint64_t>(c.n_kv_heads) * c.head_dim;
-    const uint64_t maxk = std::max<uint64_t>(std::max<uint64_t>(c.hidden, c.ffn), q_dim);
     HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
     for (void* p : m->pf_owned) (void)hipFree(p);
     m->pf_owned.clear();
     m->bytes -= m->pf_bytes;
     m->pf_bytes = 0;
     m->pf_cap = 0;
-    const uint32_t cap = std::min<uint32_t>(PREFILL_CHUNK, std::max<uint32_t>(n, 64));
+    const uint32_t cap = cera_prefill_cap(n);
+    const CeraPrefillSizes sz = cera_prefill_sizes(c, cap);
     auto alloc = [&](uint64_t bytes, void** p) -> cera_hip_status {
-        HIP_TRY(ctx, hipMalloc(p, bytes));
+        CERA_TRY(cera_model_malloc(m, p, bytes, "prefill buffer"));
         m->pf_owned.push_back(*p);
         m->bytes += bytes;
         m->pf_bytes += bytes;
         return CERA_HIP_OK;
     };
-    CERA_TRY(alloc(cap * c.hidden * 4ull, reinterpret_cast<void**>(&m->pf_hidden)));
-    CERA_TRY(alloc(cap * c.hidden * 4ull, reinterpret_cast<void**>(&m->pf_normed)));
-    CERA_TRY(alloc(cap * q_dim * 4, reinterpret_cast<void**>(&m->pf_q)));
-    CERA_TRY(alloc(cap * kv_dim * 4, reinterpret_cast<void**>(&m->pf_k)));
-    CERA_TRY(alloc(cap * kv_dim * 4, reinterpret_cast<void**>(&m->pf_v)));
-    CERA_TRY(alloc(cap * q_dim * 4, reinterpret_cast<void**>(&m->pf_attn)));
-    CERA_TRY(alloc(cap * c.ffn * 4ull, reinterpret_cast<void**>(&m->pf_gate)));
-    CERA_TRY(alloc(cap * c.ffn * 4ull, reinterpret_cast<void**>(&m->pf_up)));
-    CERA_TRY(alloc(cap * maxk, reinterpret_cast<void**>(&m->pf_xq)));
-    CERA_TRY(alloc(cap * maxk * 2, &m->pf_xh));
-    CERA_TRY(alloc(cera_gemm_fp8_ws_bytes(cap, maxk), &m->pf_x8));
-    CERA_TRY(alloc(cap * (maxk / 32) * 4, reinterpret_cast<void**>(&m->pf_xs)));
-    CERA_TRY(alloc(cap * (maxk / 32) * 4, reinterpret_cast<void**>(&m->pf_bsum)));
-    CERA_TRY(alloc(cap * 4ull, reinterpret_cast<void**>(&m->pf_tokens)));
+    CERA_TRY(alloc(sz.hidden, reinterpret_cast<void**>(&m->pf_hidden)));
+    CERA_TRY(alloc(sz.normed, reinterpret_cast<void**>(&m->pf_normed)));
+    CERA_TRY(alloc(sz.q, reinterpret_cast<void**>(&m->pf_q)));
+    CERA_TRY(alloc(sz.k, reinterpret_cast<void**>(&m->pf_k)));
+    CERA_TRY(alloc(sz.v, reinterpret_cast<void**>(&m->pf_v)));
+    CERA_TRY(alloc(sz.attn, reinterpret_cast<void**>(&m->pf_attn)));
+    CERA_TRY(alloc(sz.gate, reinterpret_cast<void**>(&m->pf_gate)));
+    CERA_TRY(alloc(sz.up, reinterpret_cast<void**>(&m->pf_up)));
+    CERA_TRY(alloc(sz.xq, reinterpret_cast<void**>(&m->pf_xq)));
+    CERA_TRY(alloc(sz.xh, &m->pf_xh));
+    CERA_TRY(alloc(sz.x8, &m->pf_x8));
+    CERA_TRY(alloc(sz.xs, reinterpret_cast<void**>(&m->pf_xs)));
+    CERA_TRY(alloc(sz.bsum, reinterpret_cast<void**>(&m->pf_bsum)));
+    CERA_TRY(alloc(sz.tokens, reinterpret_cast<void**>(&m->pf_tokens)));
     m->pf_cap = cap;
     return CERA_HIP_OK;
 }
@@ -587,7 +588,8 @@ static cera_hip_status prefill_chunk(cera_hip_model* m, const uint32_t* tokens, 
                 m->pf_logits = nullptr;
                 m->pf_logits_cap = 0;
             }
-            HIP_TRY(ctx, hipMalloc(reinterpret_cast<void**>(&m->pf_logits), static_cast<uint64_t>(m->pf_cap) * rows * 4));
+            CERA_TRY(cera_model_malloc(m, reinterpret_cast<void**>(&m->pf_logits), static_cast<uint64_t>(m->pf_cap) * rows * 4,
+                                       "all-positions logits"));
             m->pf_logits_cap = m->pf_cap;
             m->bytes += static_cast<uint64_t>(m->pf_cap) * rows * 4;
         }

@@ -18,7 +18,7 @@ STATUS = {0: "OK", 1: "ERR_DEVICE", 2: "ERR_OOM", 3: "ERR_UNSUPPORTED_DTYPE", 4:
 
 # every symbol include/cera_hip.h declares
 SYMBOLS = [
-    "cera_hip_ctx_create", "cera_hip_ctx_destroy", "cera_hip_ctx_set_decode_copies", "cera_hip_last_error", "cera_hip_sync", "cera_hip_device_info",
+    "cera_hip_ctx_create", "cera_hip_ctx_destroy", "cera_hip_ctx_set_decode_copies", "cera_hip_decode_copy_reserve_bytes", "cera_hip_decode_copy_plan", "cera_hip_drop_decode_copies", "cera_hip_last_error", "cera_hip_sync", "cera_hip_device_info",
     "cera_hip_malloc", "cera_hip_free", "cera_hip_upload", "cera_hip_download", "cera_hip_copy_dev", "cera_hip_copy_kernel",
     "cera_hip_event_create", "cera_hip_event_destroy", "cera_hip_event_record", "cera_hip_event_elapsed_ms",
     "cera_hip_tensor_upload", "cera_hip_tensor_clone", "cera_hip_tensor_free", "cera_hip_tensor_nbytes",
@@ -95,6 +95,9 @@ def load_library() -> C.CDLL:
     sig = {
         "cera_hip_ctx_create": (i32, [i32, C.c_char_p, pp]), "cera_hip_ctx_destroy": (None, [vp]),
         "cera_hip_ctx_set_decode_copies": (i32, [vp, i32]),
+        "cera_hip_decode_copy_reserve_bytes": (u64, [vp]),
+        "cera_hip_decode_copy_plan": (u64, [vp, u32, u64, u64, vp]),
+        "cera_hip_drop_decode_copies": (i32, [vp, vp]),
         "cera_hip_last_error": (C.c_char_p, [vp]), "cera_hip_sync": (i32, [vp]),
         "cera_hip_device_info": (i32, [vp, C.c_char_p, C.POINTER(u32), C.POINTER(u64)]),
         "cera_hip_malloc": (i32, [vp, u64, pp]), "cera_hip_free": (i32, [vp, vp]),
@@ -168,6 +171,35 @@ def load_library() -> C.CDLL:
 def _p(a: np.ndarray) -> int:
     assert a.flags["C_CONTIGUOUS"]
     return a.ctypes.data
+
+
+def make_config(cfg: dict) -> "Config":
+    c = Config()
+    for f in ("n_layers", "hidden", "ffn", "n_heads", "n_kv_heads", "head_dim", "vocab", "max_seq_len"):
+        setattr(c, f, int(cfg[f]))
+    c.rope_type = int(cfg.get("rope_type", 1))
+    c.rope_theta = float(cfg.get("rope_theta", 10000.0))
+    c.rms_eps = float(cfg.get("rms_eps", 1e-5))
+    c.embed_scale = float(cfg.get("embed_scale", 1.0))
+    c.residual_scale = float(cfg.get("residual_scale", 1.0))
+    c.attn_scale = float(cfg.get("attn_scale", 0.0))
+    c.logit_scale = float(cfg.get("logit_scale", 1.0))
+    c.rope_freqs = None
+    return c
+
+
+def decode_copy_reserve_bytes(cfg: dict) -> int:
+    """Bytes model_create keeps free when it hands out decode copies (plain arithmetic, no GPU)."""
+    c = make_config(cfg)
+    return int(load_library().cera_hip_decode_copy_reserve_bytes(C.addressof(c)))
+
+
+def decode_copy_plan(copy_bytes, free_bytes: int, reserve_bytes: int):
+    """(taken mask, bytes taken) of model_create's decode-copy rule (plain arithmetic, no GPU)."""
+    b = np.ascontiguousarray(copy_bytes, np.uint64)
+    take = np.zeros(b.size, np.uint8)
+    used = load_library().cera_hip_decode_copy_plan(_p(b), b.size, int(free_bytes), int(reserve_bytes), _p(take))
+    return take.astype(bool), int(used)
 
 
 def make_tensor(ggml_type: int, m: int, k: int, blocks: np.ndarray) -> Tensor:
@@ -516,17 +548,7 @@ class Model:
 
     def __init__(self, ctx: Context, cfg: dict, weights: dict):
         self.ctx = ctx
-        c = Config()
-        for f in ("n_layers", "hidden", "ffn", "n_heads", "n_kv_heads", "head_dim", "vocab", "max_seq_len"):
-            setattr(c, f, int(cfg[f]))
-        c.rope_type = int(cfg.get("rope_type", 1))
-        c.rope_theta = float(cfg.get("rope_theta", 10000.0))
-        c.rms_eps = float(cfg.get("rms_eps", 1e-5))
-        c.embed_scale = float(cfg.get("embed_scale", 1.0))
-        c.residual_scale = float(cfg.get("residual_scale", 1.0))
-        c.attn_scale = float(cfg.get("attn_scale", 0.0))
-        c.logit_scale = float(cfg.get("logit_scale", 1.0))
-        c.rope_freqs = None
+        c = make_config(cfg)
         self.cfg = dict(cfg)
         keep = []
         rf = weights.get("rope_freqs.weight")
@@ -575,6 +597,12 @@ class Model:
     @property
     def memory_bytes(self) -> int:
         return int(self.ctx.lib.cera_hip_memory_bytes(self.h))
+
+    def drop_decode_copies(self) -> int:
+        """Free every decode copy of the model; returns the bytes given back."""
+        freed = C.c_uint64()
+        self.ctx.check(self.ctx.lib.cera_hip_drop_decode_copies(self.h, C.addressof(freed)))
+        return int(freed.value)
 
     def forward(self, token: int, pos: int) -> np.ndarray:
         logits = np.empty(self.vocab, np.float32)

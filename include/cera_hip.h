@@ -111,6 +111,20 @@ CERA_HIP_API cera_hip_status cera_hip_sync(cera_hip_ctx*);
  * for one kernel, as the reference's x86 path does with repack_q4_k_8x8
  * (cera/src/backend/cpu.rs:1282-1358); it has no switch there. */
 CERA_HIP_API cera_hip_status cera_hip_ctx_set_decode_copies(cera_hip_ctx* ctx, int enabled);
+/* The rule by which cera_hip_model_create hands out decode copies, as plain arithmetic (no device
+ * is touched; callable without a GPU).  A model's copies are built last -- after every native
+ * upload, the KV caches and the single-token buffers -- and only while the device keeps
+ * cera_hip_decode_copy_reserve_bytes(cfg) free: the buffers of the largest batched prefill pass
+ * (2048 tokens, fewer when max_seq_len is shorter), that pass's all-positions logits, and 512 MiB
+ * for the context's workspaces.  Candidates are walked in priority order (the vocabulary head, then
+ * layer by layer); copy_bytes[i] == 0 marks a matrix that gets none; one that does not fit is
+ * skipped and later, smaller ones are still tried.  take[i] (nullable) receives 1 for each copy
+ * built; the return value is the bytes they take.  A model that loads and prefills with copies off
+ * therefore does so with copies on, with all, some or none of its matrices copied.  No counterpart
+ * in the reference (its repack replaces the native bytes instead of adding to them). */
+CERA_HIP_API uint64_t cera_hip_decode_copy_reserve_bytes(const cera_hip_config* cfg);
+CERA_HIP_API uint64_t cera_hip_decode_copy_plan(const uint64_t* copy_bytes, uint32_t n, uint64_t free_bytes,
+                                                uint64_t reserve_bytes, uint8_t* take);
 /* Device properties for reporting: name (<= 255 chars), CU count, bytes of HBM. */
 CERA_HIP_API cera_hip_status cera_hip_device_info(cera_hip_ctx*, char* name256, uint32_t* n_cu,
                                                   uint64_t* hbm_bytes);
@@ -493,6 +507,11 @@ CERA_HIP_API cera_hip_status cera_hip_truncate_kv(cera_hip_model*, uint32_t len)
 CERA_HIP_API uint32_t cera_hip_seq_len(const cera_hip_model*);
 /* Model::gpu_memory_bytes. */
 CERA_HIP_API uint64_t cera_hip_memory_bytes(const cera_hip_model*);
+/* Frees every decode copy of the model (second line of defence of the rule above: the library
+ * calls this itself and retries once when a prefill buffer does not fit).  Decode then reads the
+ * native bytes, with bit-identical results; *freed_bytes (nullable) receives what was given back,
+ * and cera_hip_memory_bytes drops by as much.  The copies are not rebuilt. */
+CERA_HIP_API cera_hip_status cera_hip_drop_decode_copies(cera_hip_model*, uint64_t* freed_bytes);
 /* Model::shift_kv for a RoPE model (cera/src/model/llama.rs:1727-1738 ->
  * InferenceState::shift_kv_with_rope, cera/src/kv_cache.rs:1091-1310): drops cache cells
  * [n_keep, n_keep + shift), moves the tail down and re-rotates its K rows by R(-shift)

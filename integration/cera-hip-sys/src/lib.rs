@@ -176,6 +176,14 @@ pub fn cera_hip_ctx_create(
     ) -> cera_hip_status;
     pub fn cera_hip_ctx_destroy(ctx: *mut cera_hip_ctx);
     pub fn cera_hip_ctx_set_decode_copies(ctx: *mut cera_hip_ctx, enabled: c_int) -> cera_hip_status;
+    pub fn cera_hip_decode_copy_reserve_bytes(cfg: *const cera_hip_config) -> u64;
+    pub fn cera_hip_decode_copy_plan(
+        copy_bytes: *const u64,
+        n: u32,
+        free_bytes: u64,
+        reserve_bytes: u64,
+        take: *mut u8,
+    ) -> u64;
     pub fn cera_hip_last_error(ctx: *const cera_hip_ctx) -> *const c_char;
     pub fn cera_hip_sync(ctx: *mut cera_hip_ctx) -> cera_hip_status;
     pub fn cera_hip_device_info(
@@ -599,6 +607,7 @@ pub fn cera_hip_ctx_create(
     pub fn cera_hip_truncate_kv(model: *mut cera_hip_model, len: u32) -> cera_hip_status;
     pub fn cera_hip_seq_len(model: *const cera_hip_model) -> u32;
     pub fn cera_hip_memory_bytes(model: *const cera_hip_model) -> u64;
+    pub fn cera_hip_drop_decode_copies(model: *mut cera_hip_model, freed_bytes: *mut u64) -> cera_hip_status;
     pub fn cera_hip_shift_kv(
         model: *mut cera_hip_model,
         n_keep: u32,
