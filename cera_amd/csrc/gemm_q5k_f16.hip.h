@@ -57,9 +57,14 @@ static __global__ __launch_bounds__(256) void gemm_act_split_kernel(const float*
 #pragma unroll
             for (int c = 0; c < 2; ++c) {
                 const float xs = v[2 * j + c] * scale;
-                const _Float16 hh = static_cast<_Float16>(fminf(fmaxf(xs, -65504.0f), 65504.0f));   // non-finite input stays finite here
+                // A NaN or an infinity goes through as itself (hi = the f16 NaN / infinity, lo = 0), so
+                // the token's outputs come out non-finite as the reference's f32 dot gives them
+                // (vec_dot_q5km_f32, cera/src/backend/cpu.rs:1830-1854).  The clamp only matters beside
+                // an infinity, where the row maximum gives no scale and a finite value may pass 65504.
+                const bool finite = (xs - xs) == 0.0f;
+                const _Float16 hh = static_cast<_Float16>(finite ? fminf(fmaxf(xs, -65504.0f), 65504.0f) : xs);
                 h[c] = hh;
-                l[c] = static_cast<_Float16>(xs - static_cast<float>(hh));
+                l[c] = finite ? static_cast<_Float16>(xs - static_cast<float>(hh)) : static_cast<_Float16>(0.0f);
             }
             oh[j] = __builtin_bit_cast(uint32_t, h);
             ol[j] = __builtin_bit_cast(uint32_t, l);

@@ -664,7 +664,13 @@ cera_hip_status cera_model_prefill(cera_hip_model* m, const uint32_t* tokens, ui
     // route -- the same decision LlamaModel::forward_prefill makes (llama.rs:1643,
     // 762-795); it is still the HIP path, only slower.  (Q5_K, which sends the reference down
     // that route, has a batched kernel here.)
-    if (m->ref_order == 2 && n > 1) {
+    // a layer projection the reference's batched GEMM cannot take (Q5_K) sends its whole prefill
+    // down the per-token route (cera/src/model/llama.rs:762-795); so does the verification route
+    bool ref_gemmable = true;
+    for (const LayerDev& L : m->layers)
+        for (const cera_hip_dtensor* w : {L.q, L.k, L.v, L.o, L.gate, L.up, L.down})
+            if (w->dtype == CERA_HIP_Q5_K) ref_gemmable = false;
+    if (m->ref_order == 2 && n > 1 && ref_gemmable) {
         // the verification route in the x86 host's batched order (forward_prefill takes
         // forward_prefill_batched for n > 1, cera/src/model/llama.rs:1639-1641); one pass holds
         // PREFILL_CHUNK tokens, the reference's callers split at ubatch = 512 (model/mod.rs:303-332)

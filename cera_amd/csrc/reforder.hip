@@ -176,6 +176,80 @@ __global__ __launch_bounds__(256) void gemv_ref_kernel(RefGemvArgs p) {
     if (j == 0 && row < p.m) p.y[row] = v;
 }
 
+// ---- Q5_K: f32 activations, scalar chains ----------------------------------------------------
+// gemv_q5km_f32 -> vec_dot_q5_k_f32_scalar (cera/src/backend/cpu.rs:1830-1854,
+// cera/src/quant.rs:892-937): the reference never quantizes the input of a Q5_K matrix; each
+// 256-weight block runs, per 64-weight pair j, four sequential 32-step chains with separate
+// multiply and add -- sum1 += q1*y, sum2 += q2*y', smn1 += y, smn2 += y' -- then
+// sumf += d*(sc1*sum1 + sc2*sum2) - dmin*(mn1*smn1 + mn2*smn2), and the row adds the block
+// results in order.  One wavefront per row: its 64 lanes are the 4 x 4 x 4 chains of four
+// consecutive blocks; the combination steps then run in the reference's order on one lane.
+struct RefGemvF32Args {
+    const uint8_t* w;
+    const float* x;
+    float* y;
+    uint32_t m, k, row_bytes;
+};
+__global__ __launch_bounds__(256) void gemv_q5k_ref_kernel(RefGemvF32Args p) {
+    const uint32_t lane = threadIdx.x & 63;
+    const uint32_t row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    // a wavefront past the last row recomputes it and drops the result (lanes stay together for the shuffles)
+    const uint8_t* rp = p.w + static_cast<uint64_t>(min(row, p.m - 1)) * p.row_bytes;
+    const uint32_t nb = p.k / 256;
+    const uint32_t bsel = lane >> 4, j = (lane >> 2) & 3, which = lane & 3;
+    float sum = 0.0f;
+    for (uint32_t b0 = 0; b0 < nb; b0 += 4) {
+        const uint32_t b = min(b0 + bsel, nb - 1);
+        const uint8_t* blk = rp + 176 * b;   // d, dmin, scales[12], qh[32], qs[128]
+        const uint8_t* qh = blk + 16;
+        const uint8_t* qs = blk + 48 + 32 * j;
+        const float* y = p.x + 256 * b + 64 * j + ((which & 1) ? 32 : 0);
+        const uint32_t bit = 1u << (2 * j + (which & 1));
+        float acc = 0.0f;
+        if (which < 2) {
+            for (int l = 0; l < 32; ++l) {
+                const uint32_t nib = (which & 1) ? (qs[l] >> 4) : (qs[l] & 0xF);
+                const float q = __fadd_rn(static_cast<float>(nib), (qh[l] & bit) ? 16.0f : 0.0f);
+                acc = __fadd_rn(acc, __fmul_rn(q, y[l]));
+            }
+        } else {
+            for (int l = 0; l < 32; ++l) acc = __fadd_rn(acc, y[l]);
+        }
+        // lanes 4q .. 4q+3 hold sum1, sum2, smn1, smn2 of one (block, j)
+        const uint32_t base = lane & ~3u;
+        const float sum1 = __shfl(acc, base), sum2 = __shfl(acc, base + 1), smn1 = __shfl(acc, base + 2), smn2 = __shfl(acc, base + 3);
+        const float d = h2f(ld_u16(blk)), dmin = h2f(ld_u16(blk + 2));
+        const uint8_t* s12 = blk + 4;
+        uint32_t sc[2], mn[2];
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            const uint32_t s = 2 * j + e;
+            if (s < 4) {
+                sc[e] = s12[s] & 63;
+                mn[e] = s12[s + 4] & 63;
+            } else {
+                sc[e] = (s12[s + 4] & 0xF) | ((s12[s - 4] >> 6) << 4);
+                mn[e] = (s12[s + 4] >> 4) | ((s12[s] >> 6) << 4);
+            }
+        }
+        const float pos = __fmul_rn(d, __fadd_rn(__fmul_rn(static_cast<float>(sc[0]), sum1), __fmul_rn(static_cast<float>(sc[1]), sum2)));
+        const float neg = __fmul_rn(dmin, __fadd_rn(__fmul_rn(static_cast<float>(mn[0]), smn1), __fmul_rn(static_cast<float>(mn[1]), smn2)));
+        const float term = __fsub_rn(pos, neg);
+        // block result: sumf = 0; sumf += term_j for j = 0..3 (lanes 16*bsel + 4*j hold term_j)
+        const uint32_t bl = lane & ~15u;
+        float sumf = 0.0f;
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj) sumf = __fadd_rn(sumf, __shfl(term, bl + 4 * jj));
+        // row: sum += block result, blocks in order (lanes 0, 16, 32, 48 hold them)
+#pragma unroll
+        for (int bb = 0; bb < 4; ++bb) {
+            const float v = __shfl(sumf, 16 * bb);
+            if (b0 + bb < nb) sum = __fadd_rn(sum, v);
+        }
+    }
+    if (lane == 0 && row < p.m) p.y[row] = sum;
+}
+
 // ---- batched prefill in the order of cera's x86 host ---------------------------------------
 // transformer::gemm_preq (cera/src/model/transformer.rs:710-788) sends a Q4_K / Q4_0 weight
 // that was repacked at load (m % 8 == 0; cpu.rs:1204-1206, 1364-1366) to the 8-row-interleaved
@@ -426,6 +500,16 @@ bool ref_type_ok(uint32_t t) {
     return t == CERA_HIP_Q4_0 || t == CERA_HIP_Q4_1 || t == CERA_HIP_Q8_0 || t == CERA_HIP_Q4_K || t == CERA_HIP_Q6_K;
 }
 
+// Q5_K reads the f32 activations themselves (no Q8_0 step on the reference's route)
+cera_hip_status launch_gemv_q5k_ref(cera_hip_ctx* ctx, const cera_hip_dtensor* w, const float* x_f32, float* y) {
+    if (w->dtype != CERA_HIP_Q5_K || w->k % 256 || w->k == 0)
+        return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "reference-order Q5_K gemv: k must be a positive multiple of 256");
+    RefGemvF32Args a{w->dev, x_f32, y, static_cast<uint32_t>(w->m), static_cast<uint32_t>(w->k), static_cast<uint32_t>(w->row_bytes)};
+    hipLaunchKernelGGL(gemv_q5k_ref_kernel, dim3(static_cast<uint32_t>((w->m + 3) / 4)), dim3(256), 0, ctx->stream, a);
+    HIP_TRY(ctx, hipGetLastError());
+    return CERA_HIP_OK;
+}
+
 cera_hip_status launch_gemv_ref(cera_hip_ctx* ctx, const cera_hip_dtensor* w, const float* xs, const int8_t* xq, float* y) {
     if (!ref_type_ok(w->dtype))
         return cera_fail(ctx, CERA_HIP_ERR_UNSUPPORTED_DTYPE,
@@ -532,6 +616,7 @@ cera_hip_status cera_model_decode_step_ref(cera_hip_model* m, uint32_t pos, bool
         m->bytes += bytes;
     }
     auto gemv = [&](const cera_hip_dtensor* w, const float* x_f32, uint32_t k, float* y) -> cera_hip_status {
+        if (w->dtype == CERA_HIP_Q5_K) return launch_gemv_q5k_ref(ctx, w, x_f32, y);
         // gemv_dispatch quantizes its input on every call (cera/src/backend/cpu.rs:787-790)
         CERA_TRY(cera_launch_quantize(ctx, x_f32, k, m->xs, m->xq));
         return launch_gemv_ref(ctx, w, m->xs, m->xq, y);
@@ -695,8 +780,12 @@ cera_hip_status cera_model_prefill_ref_batched(cera_hip_model* m, const uint32_t
         const float* last = m->pf_hidden + static_cast<uint64_t>(n - 1) * hs;
         CERA_TRY(launch_rmsnorm_ref(ctx, last, m->output_norm, hs, 1, c.rms_eps, m->hidden));
         const cera_hip_dtensor* o = m->output ? m->output : m->embd;
-        CERA_TRY(cera_launch_quantize(ctx, m->hidden, hs, m->xs, m->xq));
-        CERA_TRY(launch_gemv_ref(ctx, o, m->xs, m->xq, m->logits));
+        if (o->dtype == CERA_HIP_Q5_K) {
+            CERA_TRY(launch_gemv_q5k_ref(ctx, o, m->hidden, m->logits));
+        } else {
+            CERA_TRY(cera_launch_quantize(ctx, m->hidden, hs, m->xs, m->xq));
+            CERA_TRY(launch_gemv_ref(ctx, o, m->xs, m->xq, m->logits));
+        }
         if (c.logit_scale != 1.0f) {
             hipLaunchKernelGGL(scale_kernel, dim3((c.vocab + 255) / 256), dim3(256), 0, s, m->logits, 1.0f / c.logit_scale, c.vocab);
             HIP_TRY(ctx, hipGetLastError());
@@ -707,8 +796,8 @@ cera_hip_status cera_model_prefill_ref_batched(cera_hip_model* m, const uint32_t
 
 bool cera_model_ref_order_supported(const cera_hip_model* m, std::string* why) {
     auto ok = [&](const cera_hip_dtensor* w, const char* name) {
-        if (w && !ref_type_ok(w->dtype)) {
-            *why = std::string(name) + " has ggml type " + std::to_string(w->dtype) + " (the CPU path dots it against f32 activations)";
+        if (w && !ref_type_ok(w->dtype) && w->dtype != CERA_HIP_Q5_K) {
+            *why = std::string(name) + " has ggml type " + std::to_string(w->dtype) + " (no reference-order kernel)";
             return false;
         }
         return true;
@@ -734,6 +823,10 @@ extern "C" cera_hip_status cera_hip_gemv_reference_order(cera_hip_ctx* ctx, cons
         CERA_TRY(cera_scratch(ctx, 2, k, &dq));
         CERA_TRY(cera_scratch(ctx, 3, mm * 4, &dy));
         CERA_TRY(cera_hip_upload(ctx, dx, x, k * 4));
+        if (w->dtype == CERA_HIP_Q5_K) {
+            CERA_TRY(launch_gemv_q5k_ref(ctx, w, static_cast<float*>(dx), static_cast<float*>(dy)));
+            return cera_hip_download(ctx, y, dy, mm * 4);
+        }
         CERA_TRY(cera_launch_quantize(ctx, static_cast<float*>(dx), k, static_cast<float*>(ds), static_cast<int8_t*>(dq)));
         CERA_TRY(launch_gemv_ref(ctx, w, static_cast<float*>(ds), static_cast<int8_t*>(dq), static_cast<float*>(dy)));
         return cera_hip_download(ctx, y, dy, mm * 4);

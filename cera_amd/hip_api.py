@@ -339,6 +339,21 @@ class Context:
                 self.free(d)
             self.tensor_free(dt)
 
+    def gemv_store_dev(self, ggml_type: int, blocks: np.ndarray, x: np.ndarray, m: int, k: int) -> np.ndarray:
+        """W.Q8_0(x) the way the decode step launches its vocabulary head (a quantize op, then a GEMV op without a residual)."""
+        dt = self.tensor_upload(ggml_type, m, k, blocks)
+        d_x = self.to_device(np.ascontiguousarray(x, np.float32))
+        d_s, d_q, d_y = self.malloc(max(k // 32, 1) * 4), self.malloc(k), self.malloc(m * 4)
+        ops = (DecodeOp * 2)(DecodeOp(kind=DecodeOp.QUANT, n=k, x=d_x, out_q=d_q, out_s=d_s),
+                             DecodeOp(kind=DecodeOp.GEMV, w=dt, xs=d_s, xq=d_q, y=d_y))
+        try:
+            self.check(self.lib.cera_hip_decode_ops_dev(self.h, ops, 2))
+            return self.download(d_y, m, np.float32)
+        finally:
+            for d in (d_x, d_s, d_q, d_y):
+                self.free(d)
+            self.tensor_free(dt)
+
     def gemm(self, ggml_type: int, blocks: np.ndarray, x: np.ndarray, m: int, n: int, k: int) -> np.ndarray:
         t = make_tensor(ggml_type, m, k, blocks)
         x = np.ascontiguousarray(x, np.float32).reshape(n, k)

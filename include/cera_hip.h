@@ -334,8 +334,10 @@ CERA_HIP_API cera_hip_status cera_hip_qkv_fused(cera_hip_ctx*, const cera_hip_te
  * four-accumulator FMA chains, tree add and hsum256_ps (cera/src/backend/simd.rs:5742-5795,
  * 6025-6093, 4546-4554), row_dot_q4_0 / row_dot_q8_0 (:4593-4637), gemm_q4_1_q8_0 (:5893-5976);
  * attn_scores / softmax_inplace / attn_values of the AVX2 tier (cera/src/backend/cpu.rs:3503-3589,
- * 2617-2633); cpu::rmsnorm with its serial f64 sum (:2479-2496).  Arguments as the fast entry
- * points of the same name.  Q5_K is CERA_HIP_ERR_UNSUPPORTED_DTYPE here. */
+ * 2617-2633); cpu::rmsnorm with its serial f64 sum (:2479-2496).  A Q5_K matrix is dotted with the
+ * f32 activations themselves in the scalar order of vec_dot_q5_k_f32_scalar (cera/src/quant.rs:892-937,
+ * cera/src/backend/cpu.rs:1830-1854): per 64-weight pair four sequential 32-step chains with
+ * separate multiply and add.  Arguments as the fast entry points of the same name. */
 CERA_HIP_API cera_hip_status cera_hip_gemv_reference_order(cera_hip_ctx*, const cera_hip_tensor* w, const float* x,
                                                            float* y);
 CERA_HIP_API cera_hip_status cera_hip_attn_decode_reference_order(cera_hip_ctx*, const float* q, const float* k,
@@ -494,9 +496,10 @@ CERA_HIP_API uint32_t cera_hip_kv_type(const cera_hip_model*);
  *       5215-5366, 5796-5851, 6094-6168), flash_attention_gqa_avx2 from 256 tokens on
  *       (cera/src/backend/cpu.rs:4261-4412), per-token attention below; one call = one batch, as
  *       one call of the reference is (callers split prompts at their ubatch).
+ *       A model with a Q5_K layer projection prefills token by token in this mode too: the
+ *       reference's batched route hands such a model to its per-token path (llama.rs:762-795).
  * Many times slower than the default route; meant for verification only.  Only with an
- * empty cache (CERA_HIP_ERR_POSITION otherwise); CERA_HIP_ERR_UNSUPPORTED_DTYPE if a matrix is
- * Q5_K. */
+ * empty cache (CERA_HIP_ERR_POSITION otherwise). */
 #define CERA_HIP_REF_ORDER_OFF 0u
 #define CERA_HIP_REF_ORDER_PER_TOKEN 1u
 #define CERA_HIP_REF_ORDER_X86_BATCHED 2u

@@ -140,6 +140,39 @@ def test_gemv_config2_head_rows_sampled(hip, orc):
     assert err <= GEMV_TOL * util.rms(ref)
 
 
+def _head_matrix(dtype, m, k, seed):
+    """m x k rows built from a 2048-row quantized base, rolled per repetition so rows differ."""
+    r = util.rng(seed)
+    base = (r.standard_normal((2048, k)) * 0.02).astype(np.float32)
+    wb = util.H.quantize(dtype, base, 8).reshape(2048, -1)
+    reps = (m + 2047) // 2048
+    w = np.empty((m, wb.shape[1]), np.uint8)
+    for i in range(reps):
+        seg = w[i * 2048:min(m, (i + 1) * 2048)]
+        seg[:] = np.roll(wb, i * 7, axis=0)[:seg.shape[0]]
+    return w
+
+
+@pytest.mark.parametrize("dtype", [Q6_K, Q4_K])
+def test_head_row_kernel_on_the_decode_copy_at_full_size(hip, orc, no_decode_copies, dtype):
+    """The vocabulary head as the decode step launches it -- 128256 x 4096, one wavefront per row
+    streaming the decode copy (a Q6_K output.weight, or a tied Q4_K embedding table): every one of
+    the 128256 logits carries the bits of the K-split GEMV on the native bytes, the launch from the
+    native bytes (copies off) gives the same, and a row sample agrees with the oracle."""
+    m, k = 128256, 4096
+    _say(f"head row kernel {util.NAMES[dtype]} {m}x{k} on the decode copy")
+    w = _head_matrix(dtype, m, k, seed=15)
+    x = util.make_x(k, 16)
+    y = hip.gemv_store_dev(dtype, w.reshape(-1), x, m, k)
+    plain = hip.gemv(dtype, w.reshape(-1), x, m, k)
+    assert np.array_equal(y.view(np.uint32), plain.view(np.uint32)), int(np.count_nonzero(y != plain))
+    native = no_decode_copies(lambda: hip.gemv_store_dev(dtype, w.reshape(-1), x, m, k))
+    assert np.array_equal(y.view(np.uint32), native.view(np.uint32))
+    rows = np.unique(np.concatenate([np.arange(0, 64), util.rng(17).integers(0, m, 512), np.arange(m - 64, m)]))
+    ref = orc.gemv(dtype, np.ascontiguousarray(w[rows]).reshape(-1), x, rows.size, k)
+    assert np.abs(y[rows].astype(np.float64) - ref).max() <= GEMV_TOL * util.rms(ref)
+
+
 def test_gemv_q5k_f32_activation_path(hip, orc):
     # Q5_K dots against unquantized f32 x on both sides (cpu.rs:1830-1854); row widths that take one,
     # two and four wavefronts per row group, ragged row counts, and a row beyond the K split (20480)

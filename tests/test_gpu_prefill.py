@@ -169,6 +169,32 @@ def test_gemm_q5k_reads_f32_activations(hip, orc, m, n, k, amp):
         assert np.abs(out[rows, j] - y).max() <= 3e-5 * util.rms(exact)
 
 
+def test_gemm_q5k_lets_non_finite_activations_through(hip):
+    """One NaN among a token's activations makes every output of that token NaN, as the reference's
+    f32 dot does (vec_dot_q5km_f32, cera/src/backend/cpu.rs:1830-1854: NaN x weight is NaN for any
+    weight) and as the Q5_K GEMV of that token does; an infinity makes them non-finite; the other
+    tokens of the batch are untouched."""
+    m, n, k = 96, 40, 1024
+    w, _ = util.make_weights(Q5_K, m, k, seed=7)
+    x = util.rng(8).standard_normal((n, k)).astype(np.float32)
+    clean = hip.gemm(Q5_K, w, x, m, n, k)
+    bad = x.copy()
+    bad[3, 517] = np.nan
+    bad[29, 0] = np.inf
+    bad[31, 1023] = -np.inf
+    _say("gemm Q5_K with NaN / Inf activations")
+    out = hip.gemm(Q5_K, w, bad, m, n, k)
+    assert np.isnan(out[:, 3]).all()
+    assert not np.isfinite(out[:, 29]).any() and not np.isfinite(out[:, 31]).any()
+    others = [j for j in range(n) if j not in (3, 29, 31)]
+    assert np.array_equal(out[:, others].view(np.uint32), clean[:, others].view(np.uint32))
+    for j in (3, 29, 31):
+        y = hip.gemv(Q5_K, w, bad[j], m, k)
+        assert not np.isfinite(y).any()
+        if j == 3:
+            assert np.isnan(y).all()   # the same NaN positions as the batched kernel: all of them
+
+
 def test_q5k_model_prefills_in_batches(hip, orc):
     """A model whose Q4_K tensors are Q5_K (the Q5_K_M recipe) takes the batched prefill route:
     logits and KV cache agree with the token-by-token decode of the same prompt, and with the

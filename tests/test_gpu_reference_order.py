@@ -61,11 +61,22 @@ def test_gemv_reference_order_config2_rows(hip, orc):
         assert _same_bits(hip.gemv_reference_order(dtype, w, x, m, k), orc.gemv(dtype, w, x, m, k)), (dtype, m, k)
 
 
-def test_gemv_reference_order_refuses_q5_k(hip):
-    w, _ = util.make_weights(util.Q5_K, 8, 256, seed=1)
-    with pytest.raises(hip_api.HipError) as e:
-        hip.gemv_reference_order(util.Q5_K, w, util.make_x(256, 1), 8, 256)
-    assert e.value.status == 3
+@pytest.mark.parametrize("m,k", [(96, 4096), (5, 256), (33, 1280), (64, 14336), (1, 768)])
+def test_gemv_reference_order_q5_k_reads_f32_activations(hip, orc, m, k):
+    """Q5_K on the reference's route is a scalar f32 dot against the UNQUANTIZED activations
+    (gemv_q5km_f32 -> vec_dot_q5_k_f32_scalar, cera/src/backend/cpu.rs:1830-1854,
+    cera/src/quant.rs:892-937): four sequential 32-step chains per 64-weight pair with separate
+    multiplies and adds.  Same bits, at block counts that are and are not multiples of the four
+    blocks a wavefront takes per pass."""
+    _say(f"ref-order gemv Q5_K {m}x{k}")
+    w, _ = util.make_weights(util.Q5_K, m, k, seed=m + k)
+    for seed, scale in ((1, 1.0), (2, 30.0), (3, 1e-3)):
+        x = util.make_x(k, seed) * np.float32(scale)
+        got = hip.gemv_reference_order(util.Q5_K, w, x, m, k)
+        ref = orc.gemv(util.Q5_K, w, x, m, k)
+        assert _same_bits(got, ref), (m, k, seed, float(np.abs(got - ref).max()))
+    fast = hip.gemv(util.Q5_K, w, x, m, k)
+    assert np.abs(fast - got).max() <= 1e-4 * util.rms(got) + 1e-12
 
 
 @pytest.mark.parametrize("n_heads,n_kv,hd,L", [(32, 8, 128, 1), (32, 8, 128, 7), (32, 8, 128, 300), (8, 2, 64, 33),
@@ -166,6 +177,8 @@ MODELS = {
     "granite_scalars": (dict(embed_scale=12.0, residual_scale=0.22, attn_scale=0.0078125, logit_scale=8.0), dict(), dict()),
     "tied_q8_0": (dict(), dict(type_of=lambda name: H.Q8_0, tied_output=True), dict()),
     "q4_0": (dict(), dict(type_of=lambda name: H.Q4_0), dict()),
+    # the Q5_K_M recipe: Q5_K where Q4_K_M has Q4_K, f32 activations into those matrices
+    "llama_q5_k_m": (dict(), dict(type_of=lambda name: H.Q5_K if synth.q4_k_m_type(name) == H.Q4_K else synth.q4_k_m_type(name)), dict()),
 }
 
 
@@ -310,10 +323,22 @@ def test_reference_order_switch_rules(hip, orc):
     gm.set_reference_order(False)
     assert _same_bits(gm.forward(7, 0), fast)   # and is unchanged by the round trip
     gm.close(); om.close()
-    # a Q5_K matrix has no reference-order kernel: refused, never skipped
+
+
+def test_model_with_a_q5_k_matrix_prefills_token_by_token_in_both_modes(hip, orc):
+    """A layer projection the reference's batched GEMM cannot take sends its whole prefill down
+    the per-token route (cera/src/model/llama.rs:762-795): with one Q5_K matrix the x86-batched
+    mode gives the per-token mode's bits, which are the oracle's."""
+    cfg = dict(synth.TINY)
     w5 = synth.make_llama(cfg, seed=1, sigma=0.05, type_of=lambda name: H.Q5_K if "ffn_up" in name else H.Q8_0)
     g5 = hip_api.Model(hip, cfg, w5)
-    with pytest.raises(hip_api.HipError) as e:
-        g5.set_reference_order(True)
-    assert e.value.status == 3
-    g5.close()
+    om = orc.Llama(cfg, w5)
+    prompt = [int(t) for t in util.rng(6).integers(0, cfg["vocab"], 11)]
+    lo = om.forward_prefill_per_token(prompt, 0)
+    for mode in (1, 2):
+        g5.truncate_kv(0)
+        g5.set_reference_order(mode)
+        assert g5.reference_order == mode
+        assert _same_bits(g5.forward_prefill(prompt, 0), lo), mode
+    assert _same_bits(g5.forward(3, 11), om.forward(3, 11))
+    g5.close(); om.close()

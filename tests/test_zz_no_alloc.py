@@ -3,7 +3,9 @@ partials live in a fixed array inside the library instead of a workspace the con
 Checked through the C-ABI against cera_hip_attn_decode_dev on the same device buffers: the same
 kernels with the same split, so the outputs must be bit-identical -- on two calls in a row, the
 second on a smaller input (the array keeps the first call's contents), and again after a call
-of the allocating entry in between."""
+of the allocating entry in between.  And the property the entry exists for: on a context that has
+never run attention, a call leaves the device's free memory exactly where it was, while the
+allocating entry on the same context visibly takes its workspace."""
 import ctypes as C
 
 import numpy as np
@@ -49,6 +51,44 @@ def test_no_alloc_attention_matches_the_allocating_entry(hip, orc):
     assert np.array_equal(a2.view(np.uint32), b2.view(np.uint32))
     a3, b3, _ = _both(hip, 32, 8, 128, 700, 1024, seed=5, n_splits=16)           # explicit split
     assert np.array_equal(a3.view(np.uint32), b3.view(np.uint32))
+
+
+def _free_device_bytes():
+    rt = C.CDLL("libamdhip64.so")
+    free, total = C.c_size_t(), C.c_size_t()
+    assert rt.hipMemGetInfo(C.byref(free), C.byref(total)) == 0
+    return free.value
+
+
+def test_no_alloc_attention_allocates_nothing(hip):
+    from cera_amd import hip_api
+    fresh = hip_api.Context(0)     # no attention workspace, no scratch slot yet
+    try:
+        n_heads, n_kv, hd, L = 32, 8, 128, 8192         # 128 parts x 32 heads x 128 x 4 B = 2 MiB of partials
+        dq = fresh.to_device(util.make_x(n_heads * hd, 3))
+        dk = fresh.to_device(np.zeros((n_kv, L, hd), np.float32))
+        d_out = fresh.malloc(n_heads * hd * 4)
+        fresh.sync()
+        f0 = _free_device_bytes()
+        print(f"no-alloc attention on a fresh context: free {f0} bytes before", flush=True)
+        fresh.check(fresh.lib.cera_hip_attn_decode_dev_noalloc(fresh.h, dq, dk, dk, n_heads, n_kv, hd, L, L, 0.1, 128, d_out))
+        fresh.sync()
+        f1 = _free_device_bytes()
+        assert f1 == f0, f"the allocation-free entry changed free device memory by {f0 - f1} bytes"
+        # the probe is not blind: the allocating entry's first call on this context takes its workspace
+        fresh.check(fresh.lib.cera_hip_attn_decode_dev(fresh.h, dq, dk, dk, n_heads, n_kv, hd, L, L, 0.1, 128, d_out))
+        fresh.sync()
+        f2 = _free_device_bytes()
+        print(f"no-alloc attention: free after the allocating entry {f2} ({f1 - f2} bytes taken)", flush=True)
+        assert f1 - f2 >= n_heads * 128 * hd * 4
+        # and a second allocation-free call, with the context's workspace now present, still takes nothing
+        fresh.check(fresh.lib.cera_hip_attn_decode_dev_noalloc(fresh.h, dq, dk, dk, n_heads, n_kv, hd, L, L, 0.1, 128, d_out))
+        fresh.sync()
+        assert _free_device_bytes() == f2
+        for d in (dq, dk, d_out):
+            fresh.free(d)
+    finally:
+        fresh.close()
 
 
 def test_no_alloc_attention_refuses_what_does_not_fit(hip):
