@@ -36,6 +36,15 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 # It is a recorded measurement of this kernel configuration, not taken live: counters need the profiler.
 GATE_UP_TRAFFIC_BYTES = 66_481_099
 GATE_UP_KERNEL = "row_gemv_kernel<Q4K,16,4,true,2,true,1,4096>"
+# Average duration of that kernel among the other launches of a decode step, from the rocprofv3 kernel trace
+# of the whole default run (profiles/gemv_decode_set_llama3_8b_kernel_trace.txt): a recorded figure, kept
+# beside the live back-to-back one because events around a single launch inside a step would time the
+# launch gap, not the kernel.
+GATE_UP_IN_STEP_US = 13.99
+# Average duration rocprofv3 reports for the same kernel over `bench.py --roofline-probe` (back-to-back launches only,
+# profiles/gemv_gate_up_back_to_back_kernel_trace.txt).  Consecutive launches overlap by a ramp and a tail, so a
+# launch's own start-to-end duration is longer than the time per launch the events measure (wall time / launches).
+GATE_UP_TRACE_BACK_TO_BACK_US = 14.10
 
 # (name, ggml type name, m, k, copies per step)
 LAYER_SET = [
@@ -260,6 +269,10 @@ def main() -> int:
                          "fewer lets the last-level cache hold them, which is NOT the reported configuration)")
     ap.add_argument("--no-e2e", action="store_true", help="skip the end-to-end model run (prefill 512 + greedy 256)")
     ap.add_argument("--no-extras", action="store_true", help="skip the flash-decode and prefill-GEMM side measurements")
+    ap.add_argument("--roofline-probe", action="store_true",
+                    help="run only what roofline.avg_launch_us is taken from: the back-to-back launches of the fused "
+                         "gate|up kernel over the rotating layer copies, HIP events around them; prints that figure as "
+                         "JSON (the command whose rocprofv3 kernel trace is committed next to it)")
     ap.add_argument("--pmc-probe", action="store_true",
                     help="run only a 1 GiB copy kernel, a few launches of each per-layer GEMV kernel, decode attention at "
                          "131072 and 8192 keys and the two prefill GEMMs at 2048 tokens, for a hardware-counter pass under "
@@ -315,20 +328,20 @@ def main() -> int:
     d_oq, d_os = ctx.malloc(4096), ctx.malloc(4096 // 32 * 4)
     ctx.sync()
 
-    def op_qkv(l):
-        return Op(kind=Op.NORM_GEMV, w=dts["attn_qkv"][l], x=d_x[4096], norm_w=d_norm, eps=eps, y=outs["attn_qkv"])
+    def op_qkv(l, t=None):
+        return Op(kind=Op.NORM_GEMV, w=(t or dts)["attn_qkv"][l], x=d_x[4096], norm_w=d_norm, eps=eps, y=outs["attn_qkv"])
 
-    def op_o(l, xs=None, xq=None):
-        return Op(kind=Op.GEMV, w=dts["attn_output"][l], xs=xs or acts[4096][0], xq=xq or acts[4096][1], resid=d_x[4096],
+    def op_o(l, xs=None, xq=None, t=None):
+        return Op(kind=Op.GEMV, w=(t or dts)["attn_output"][l], xs=xs or acts[4096][0], xq=xq or acts[4096][1], resid=d_x[4096],
                   y=outs["attn_output"])
 
-    def op_gate_up(l):
-        return Op(kind=Op.NORM_GATE_UP, w=dts["ffn_gate"][l], w2=dts["ffn_up"][l], x=d_x[4096], norm_w=d_norm, eps=eps,
+    def op_gate_up(l, t=None):
+        return Op(kind=Op.NORM_GATE_UP, w=(t or dts)["ffn_gate"][l], w2=(t or dts)["ffn_up"][l], x=d_x[4096], norm_w=d_norm, eps=eps,
                   out_q=d_ffn_q, out_s=d_ffn_s)
 
-    def op_down(l, fused_input=True):
+    def op_down(l, fused_input=True, t=None):
         xs, xq = (d_ffn_s, d_ffn_q) if fused_input else acts[14336]
-        return Op(kind=Op.GEMV, w=dts["ffn_down"][l], xs=xs, xq=xq, resid=d_x[4096], y=outs["ffn_down"])
+        return Op(kind=Op.GEMV, w=(t or dts)["ffn_down"][l], xs=xs, xq=xq, resid=d_x[4096], y=outs["ffn_down"])
 
     op_head_norm = Op(kind=Op.NORM_QUANT, n=4096, x=d_x[4096], norm_w=d_norm, eps=eps, y=d_head_in, out_q=d_head_q, out_s=d_head_s)
     op_head = Op(kind=Op.GEMV, w=dts["output"][0], xs=d_head_s, xq=d_head_q, y=outs["output"])
@@ -427,6 +440,28 @@ def main() -> int:
     # permutation kernel per matrix), which belongs to loading the weights, not to a step
     run(step_arr)
     ctx.sync()
+
+    ROOFLINE_REPS = 8
+
+    def time_group(arr, reps):
+        """HIP events on the launch stream around reps back-to-back passes over arr: us per launch."""
+        for _ in range(2):
+            run(arr)
+        e0, e1 = ctx.event(), ctx.event()
+        ctx.record(e0)
+        for _ in range(reps):
+            run(arr)
+        ctx.record(e1)
+        ctx.sync()
+        return ctx.elapsed_ms(e0, e1) * 1e3 / (reps * len(arr))
+
+    if args.roofline_probe:
+        us = time_group(groups["ffn_gate_up"], ROOFLINE_REPS)
+        print(json.dumps({"kernel": GATE_UP_KERNEL, "launches": (ROOFLINE_REPS + 2) * N_LAYERS + N_LAYERS,
+                          "avg_launch_us_hip_events": round(us, 3), "bytes_per_launch": launch_bytes["ffn_gate_up"],
+                          "GB/s": round(launch_bytes["ffn_gate_up"] / us / 1e3, 1),
+                          "frac": round(launch_bytes["ffn_gate_up"] / us / 1e3 / HBM_PEAK_GBS, 4)}))
+        return 0
     for _ in range(args.warmup):
         run(step_arr)
     ctx.sync()
@@ -461,18 +496,9 @@ def main() -> int:
 
     # ---- per matrix: HIP events around 32 back-to-back launches of one kernel, rotating copies
     per_matrix = {}
-    reps = 8
+    reps = ROOFLINE_REPS
     for g, arr in groups.items():
-        for _ in range(2):
-            run(arr)
-        e0, e1 = ctx.event(), ctx.event()
-        n_rep = reps * (8 if len(arr) == 1 else 1)
-        ctx.record(e0)
-        for _ in range(n_rep):
-            run(arr)
-        ctx.record(e1)
-        ctx.sync()
-        us = ctx.elapsed_ms(e0, e1) * 1e3 / (n_rep * len(arr))
+        us = time_group(arr, reps * (8 if len(arr) == 1 else 1))
         tname, m, k = shape["ffn_gate" if g == "ffn_gate_up" else g]
         per_matrix[g] = {"weights": ("2 x " if g == "ffn_gate_up" else "") + f"{tname} {m}x{k}", "us_per_launch": round(us, 2),
                          "bytes_per_launch": launch_bytes[g], "GB/s": round(launch_bytes[g] / us / 1e3, 1),
@@ -491,7 +517,46 @@ def main() -> int:
                                   "calibrated on a 1 GiB copy kernel (recorded, see profiles/)",
                 "bytes_per_launch": launch_bytes["ffn_gate_up"], "avg_launch_us": gu["us_per_launch"],
                 "avg_launch_source": f"HIP events on the launch stream around {reps} x 32 back-to-back launches over "
-                                     f"{n_copies} rotating layer copies, taken right after the timed region"}
+                                     f"{n_copies} rotating layer copies, taken right after the timed region; "
+                                     "`bench.py --roofline-probe` runs exactly this loop, and its rocprofv3 kernel trace is "
+                                     "profiles/gemv_gate_up_back_to_back_kernel_trace.txt",
+                "trace_avg_launch_us_back_to_back": GATE_UP_TRACE_BACK_TO_BACK_US,
+                "frac_at_trace_avg_back_to_back": round(launch_bytes["ffn_gate_up"] / GATE_UP_TRACE_BACK_TO_BACK_US / 1e3 / HBM_PEAK_GBS, 4),
+                "avg_launch_us_in_decode_step": GATE_UP_IN_STEP_US,
+                "frac_in_decode_step": round(launch_bytes["ffn_gate_up"] / GATE_UP_IN_STEP_US / 1e3 / HBM_PEAK_GBS, 4),
+                "in_decode_step_source": "rocprofv3 --kernel-trace --stats over the whole default bench.py run "
+                                         "(recorded, profiles/gemv_decode_set_llama3_8b_kernel_trace.txt): between the other "
+                                         "kernels of a step the same launch averages longer than back to back"}
+
+    # ---- the same step on the native GGUF layout: decode copies off, freshly uploaded tensors
+    ctx.set_decode_copies(False)
+    try:
+        nat = {}
+        for name, tname, m, k in LAYER_SET:
+            first = ctx.tensor_upload(H.TYPE_IDS[tname], m, k, host[name])
+            copies = [first] + [ctx.tensor_clone(first) for _ in range(n_copies - 1)]
+            nat[name] = [copies[l % len(copies)] for l in range(N_LAYERS)]
+        name, tname, m, k = HEAD
+        nat_head = ctx.tensor_upload(H.TYPE_IDS[tname], m, k, host[name])
+        nat_ops = []
+        for l in range(N_LAYERS):
+            nat_ops += [op_qkv(l, nat), op_o(l, t=nat), op_gate_up(l, nat), op_down(l, t=nat)]
+        nat_ops += [op_head_norm, Op(kind=Op.GEMV, w=nat_head, xs=d_head_s, xq=d_head_q, y=outs["output"])]
+        nat_arr = ops_array(nat_ops)
+        for _ in range(max(2, args.warmup)):
+            run(nat_arr)
+        ctx.sync()
+        t_n = time.perf_counter()
+        for _ in range(args.steps):
+            run(nat_arr)
+        ctx.sync()
+        native_gbs = step_bytes / ((time.perf_counter() - t_n) / args.steps) / 1e9
+        for lst in nat.values():
+            for t in {id(x): x for x in lst}.values():
+                ctx.tensor_free(t)
+        ctx.tensor_free(nat_head)
+    finally:
+        ctx.set_decode_copies(True)
 
     # ---- correctness spot check of what was just timed (oracle is only the checker)
     cpu_baseline = None
@@ -546,6 +611,11 @@ def main() -> int:
         extras["flash_decode"] = measure_attention(ctx, hip_api, rng)
         extras["prefill_gemm"] = measure_gemm(ctx, H, dts, shape, rng, n_thr)
     e2e = None if args.no_e2e else measure_e2e(args.seed, n_thr)
+    # the metric names tok/s too: the end-to-end rates ride in `config`, next to the workload they belong to
+    e2e_cfg = None if e2e is None else {
+        "workload": "random-init Llama-3-8B arch GGUF (Q4_K_M-style mix) through HipLlamaModel: prefill 512 + greedy 256, batch 1",
+        "decode_tok_s": e2e["decode_tok_s"], "prefill_tok_s": e2e["prefill_tok_s"],
+        "decode_frac_of_hbm_peak": e2e["decode_frac_of_hbm_peak"]}
 
     out = {
         "metric": "Q4_K GEMV HBM GB/s (% of peak); Llama-3-8B-arch Q4_K decode tok/s, 1 GPU",
@@ -559,7 +629,11 @@ def main() -> int:
                    "algorithmic_bytes_per_step": step_bytes, "w_sigma": 0.02, "seed": args.seed,
                    "distinct_weight_copies": n_copies,
                    "weight_layout": "each matrix read from its decode copy (per-row permutation of the GGUF bytes, the "
-                                    "library's default, built before the timed region); same bytes per step"},
+                                    "library's default, built before the timed region); same bytes per step",
+                   "native_layout_GB/s": round(native_gbs, 1),
+                   "native_layout": "the same step with decode copies off: every matrix read from its GGUF bytes as uploaded",
+                   "e2e": e2e_cfg},
+        "native_layout_GB/s": round(native_gbs, 1),
         "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2),
         "ms_per_step_p50": round(p50, 4), "ms_per_step_p10": round(p10, 4), "ms_per_step_p90": round(p90, 4),
         "value_p50_GB/s": round(step_bytes / (p50 * 1e-3) / 1e9, 1),
