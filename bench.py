@@ -40,11 +40,11 @@ GATE_UP_KERNEL = "row_gemv_kernel<Q4K,16,4,true,2,true,1,4096>"
 # of the whole default run (profiles/gemv_decode_set_llama3_8b_kernel_trace.txt): a recorded figure, kept
 # beside the live back-to-back one because events around a single launch inside a step would time the
 # launch gap, not the kernel.
-GATE_UP_IN_STEP_US = 13.99
+GATE_UP_IN_STEP_US = 14.28
 # Average duration rocprofv3 reports for the same kernel over `bench.py --roofline-probe` (back-to-back launches only,
 # profiles/gemv_gate_up_back_to_back_kernel_trace.txt).  Consecutive launches overlap by a ramp and a tail, so a
 # launch's own start-to-end duration is longer than the time per launch the events measure (wall time / launches).
-GATE_UP_TRACE_BACK_TO_BACK_US = 14.10
+GATE_UP_TRACE_BACK_TO_BACK_US = 13.93
 
 # (name, ggml type name, m, k, copies per step)
 LAYER_SET = [
@@ -186,7 +186,9 @@ def measure_gemm(ctx, H, dts, shape, rng, n_thr=16):
             us = ctx.elapsed_ms(e0, e1) * 1e3 / iters
             tops = 2.0 * m_tok * n_out * k / us / 1e6
             # Q6_K's block dots run on the f16 matrix cores (2.5 PFLOP/s dense), the rest on int8 (5 POP/s)
-            peak_key, peak = ("frac_of_f16_mfma_peak", F16_PEAK_TOPS) if tname in ("Q6_K", "Q5_K") else ("frac_of_int8_mfma_peak", INT8_PEAK_TOPS)
+            # Q4_K runs on the fp8 matrix cores (exact small-integer operands), the other 4-/8-bit types on int8: both 5.0 P(FL)OP/s dense
+            peak_key, peak = (("frac_of_f16_mfma_peak", F16_PEAK_TOPS) if tname in ("Q6_K", "Q5_K") else
+                              ("frac_of_fp8_mfma_peak", INT8_PEAK_TOPS) if tname == "Q4_K" else ("frac_of_int8_mfma_peak", INT8_PEAK_TOPS))
             res.append({"weight": f"{name} {tname} {n_out}x{k}", "tokens": m_tok, "us_per_call": round(us, 1),
                         "TOP/s": round(tops, 1), peak_key: round(tops / peak, 4)})
             ctx.free(dx)
