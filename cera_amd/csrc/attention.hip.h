@@ -366,7 +366,7 @@ __device__ __forceinline__ uint32_t attn_fold_column(uint32_t lane) {
 // NT: every K/V row is read once, by this wavefront only (one query, the group not split):
 // non-temporal loads.
 template <int G, int S, bool NEWKV, typename KV, int HD, bool NT = false>
-__global__ __launch_bounds__(256) void attn_decode_partial_kernel(
+__device__ __forceinline__ void attn_decode_partial_body(
     const float* __restrict__ q,       // [n_heads][128]
     const KV* __restrict__ kc,         // [n_kv][max_seq][128]
     const KV* __restrict__ vc,
@@ -418,6 +418,20 @@ __global__ __launch_bounds__(256) void attn_decode_partial_kernel(
             part_ml[(base + h) * 2 + 1] = l[h];
         }
     }
+}
+template <int G, int S, bool NEWKV, typename KV, int HD, bool NT = false>
+__global__ __launch_bounds__(256) void attn_decode_partial_kernel(
+    const float* __restrict__ q,       // [n_heads][128]
+    const KV* __restrict__ kc,         // [n_kv][max_seq][128]
+    const KV* __restrict__ vc,
+    uint32_t seq_len, uint32_t max_seq, float scale, uint32_t chunks_per_part, uint32_t n_parts,
+    uint32_t q_stride,                 // floats between consecutive queries (prefill batches queries on grid.z)
+    uint32_t g_total,                  // query heads per kv head (a multiple of G)
+    uint32_t n_kv, uint32_t n_queries,
+    float* __restrict__ part_acc,      // [n_queries][n_kv][n_parts][g_total][128]
+    float* __restrict__ part_ml,       // [n_queries][n_kv][n_parts][g_total][2]
+    AttnNewKV nk) {
+    attn_decode_partial_body<G, S, NEWKV, KV, HD, NT>(q, kc, vc, seq_len, max_seq, scale, chunks_per_part, n_parts, q_stride, g_total, n_kv, n_queries, part_acc, part_ml, nk);
 }
 
 // ---------------------------------------------------------------------------
@@ -484,7 +498,7 @@ __device__ __forceinline__ attn_v16f attn_mfma(const uint4& a, const uint4& b, a
 }
 
 template <typename KV, int HD, int G>
-__global__ __launch_bounds__(64 * G) void attn_prefill_partial_kernel(
+__device__ __forceinline__ void attn_prefill_partial_body(
     const float* __restrict__ q,       // [n_queries][q_stride], rows 16-byte aligned
     const KV* __restrict__ kc,         // [n_kv][max_seq][128], already holding the batch's keys
     const KV* __restrict__ vc,
@@ -704,6 +718,17 @@ __global__ __launch_bounds__(64 * G) void attn_prefill_partial_kernel(
         ml[1] = static_cast<float>(l);
     }
 }
+template <typename KV, int HD, int G>
+__global__ __launch_bounds__(64 * G) void attn_prefill_partial_kernel(
+    const float* __restrict__ q,       // [n_queries][q_stride], rows 16-byte aligned
+    const KV* __restrict__ kc,         // [n_kv][max_seq][128], already holding the batch's keys
+    const KV* __restrict__ vc,
+    uint32_t first_len,                // keys visible to query 0; query i sees first_len + i
+    uint32_t n_queries, uint32_t max_seq, float scale, uint32_t part_keys, uint32_t n_parts, uint32_t q_stride,
+    float* __restrict__ part_acc,      // [n_queries][n_kv][n_parts][G][128]
+    float* __restrict__ part_ml) {
+    attn_prefill_partial_body<KV, HD, G>(q, kc, vc, first_len, n_queries, max_seq, scale, part_keys, n_parts, q_stride, part_acc, part_ml);
+}
 
 // Merge the parts of one query head: out = sum_p e^{m_p - M} acc_p / sum_p e^{m_p - M} l_p.
 // One workgroup of 256 threads per (head, query): the maxima and weights are
@@ -713,7 +738,7 @@ __global__ __launch_bounds__(64 * G) void attn_prefill_partial_kernel(
 // the groups together and optionally writes the Q8_0 quantisation of the
 // result for the output projection.
 template <bool QUANT, int HD>
-__global__ __launch_bounds__(256) void attn_decode_merge_kernel(const float* __restrict__ part_acc,
+__device__ __forceinline__ void attn_decode_merge_body(const float* __restrict__ part_acc,
                                                                 const float* __restrict__ part_ml,
                                                                 uint32_t n_parts, uint32_t G, uint32_t n_heads,
                                                                 float* __restrict__ out,
@@ -804,6 +829,16 @@ __global__ __launch_bounds__(256) void attn_decode_merge_kernel(const float* __r
         }
     }
 }
+template <bool QUANT, int HD>
+__global__ __launch_bounds__(256) void attn_decode_merge_kernel(const float* __restrict__ part_acc,
+                                                                const float* __restrict__ part_ml,
+                                                                uint32_t n_parts, uint32_t G, uint32_t n_heads,
+                                                                float* __restrict__ out,
+                                                                float* __restrict__ scales,
+                                                                int8_t* __restrict__ quants,
+                                                                float* __restrict__ bsum) {
+    attn_decode_merge_body<QUANT, HD>(part_acc, part_ml, n_parts, G, n_heads, out, scales, quants, bsum);
+}
 
 // Merge for a batch of queries (prefill): the same formula as above over the few parts a prefill
 // pass makes (8 at most), but eight (query, head) pairs per workgroup, 32 lanes each (a float4 of
@@ -811,7 +846,7 @@ __global__ __launch_bounds__(256) void attn_decode_merge_kernel(const float* __r
 // a 256-thread workgroup and two barriers on one pair, which for 512 queries x 32 heads x 4 parts
 // cost more than the attention itself.
 template <bool QUANT, int HD>
-__global__ __launch_bounds__(256) void attn_prefill_merge_kernel(const float* __restrict__ part_acc,
+__device__ __forceinline__ void attn_prefill_merge_body(const float* __restrict__ part_acc,
                                                                  const float* __restrict__ part_ml,
                                                                  uint32_t n_parts, uint32_t G, uint32_t n_heads,
                                                                  uint32_t n_pairs, float* __restrict__ out,
@@ -854,5 +889,14 @@ __global__ __launch_bounds__(256) void attn_prefill_merge_kernel(const float* __
             }
         }
     }
+}
+template <bool QUANT, int HD>
+__global__ __launch_bounds__(256) void attn_prefill_merge_kernel(const float* __restrict__ part_acc,
+                                                                 const float* __restrict__ part_ml,
+                                                                 uint32_t n_parts, uint32_t G, uint32_t n_heads,
+                                                                 uint32_t n_pairs, float* __restrict__ out,
+                                                                 float* __restrict__ scales, int8_t* __restrict__ quants,
+                                                                 float* __restrict__ bsum) {
+    attn_prefill_merge_body<QUANT, HD>(part_acc, part_ml, n_parts, G, n_heads, n_pairs, out, scales, quants, bsum);
 }
 

@@ -233,7 +233,7 @@ struct GemmQ8_0 {
 // 32-row Q8_0 block of one token in the two lanes of a column, and the activation of the down
 // projection is quantized straight from the accumulators.
 template <class T, bool SWIGLU = false, bool DBG = false>
-static __global__ __launch_bounds__(256, T::WAVES_PER_SIMD) void gemm_kernel(GemmArgs p) {
+__device__ __forceinline__ void gemm_body(GemmArgs p) {
     constexpr int NB = GEMM_KT / 32;  // 32-blocks per tile
     __shared__ __attribute__((aligned(16))) int8_t sA[GEMM_BM * GEMM_LDA];
     __shared__ __attribute__((aligned(16))) int8_t sB[GEMM_BN * GEMM_LDA];
@@ -440,10 +440,14 @@ static __global__ __launch_bounds__(256, T::WAVES_PER_SIMD) void gemm_kernel(Gem
                 }
     }
 }
+template <class T, bool SWIGLU = false, bool DBG = false>
+static __global__ __launch_bounds__(256, T::WAVES_PER_SIMD) void gemm_kernel(GemmArgs p) {
+    gemm_body<T, SWIGLU, DBG>(p);
+}
 
 
 // Sums the split-K partials in a fixed order: out[e] = (resid[e] +) sum_z part[z][e].
-static __global__ __launch_bounds__(256) void gemm_reduce_kernel(const float* __restrict__ part, uint32_t n_split,
+__device__ __forceinline__ void gemm_reduce_body(const float* __restrict__ part, uint32_t n_split,
                                                           uint64_t stride, uint64_t n4, float* __restrict__ out,
                                                           const float* resid, float resid_scale, uint64_t n4_first,
                                                           float* __restrict__ out2) {
@@ -462,4 +466,10 @@ static __global__ __launch_bounds__(256) void gemm_reduce_kernel(const float* __
         s.x = r.x + s.x; s.y = r.y + s.y; s.z = r.z + s.z; s.w = r.w + s.w;
     }
     reinterpret_cast<float4*>(out)[e] = s;
+}
+static __global__ __launch_bounds__(256) void gemm_reduce_kernel(const float* __restrict__ part, uint32_t n_split,
+                                                          uint64_t stride, uint64_t n4, float* __restrict__ out,
+                                                          const float* resid, float resid_scale, uint64_t n4_first,
+                                                          float* __restrict__ out2) {
+    gemm_reduce_body(part, n_split, stride, n4, out, resid, resid_scale, n4_first, out2);
 }

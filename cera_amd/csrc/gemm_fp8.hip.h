@@ -61,7 +61,7 @@ typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 //   [j 0..2][lane][8 bf16]                      xs*sum(a) of blocks 4*half .. 4*half+3 as three bf16 pieces
 //       b0, b1, b2 in slot order (b0, b1, b0, b2, b1, b0) per block, slots 8j .. 8j+7 of the lane's 24
 // Tokens at or beyond n are zero.
-static __global__ __launch_bounds__(256) void gemm_act_fp8_kernel(const int8_t* __restrict__ xq, const float* __restrict__ xs,
+__device__ __forceinline__ void gemm_act_fp8_body(const int8_t* __restrict__ xq, const float* __restrict__ xs,
                                                                   const float* __restrict__ bsum, uint8_t* __restrict__ rec,
                                                                   uint32_t n, uint32_t k) {
     const uint32_t nsb = k / 256, tile = blockIdx.x / nsb, sb = blockIdx.x % nsb, tid = threadIdx.x;
@@ -128,6 +128,11 @@ static __global__ __launch_bounds__(256) void gemm_act_fp8_kernel(const int8_t* 
         }
     }
 }
+static __global__ __launch_bounds__(256) void gemm_act_fp8_kernel(const int8_t* __restrict__ xq, const float* __restrict__ xs,
+                                                                  const float* __restrict__ bsum, uint8_t* __restrict__ rec,
+                                                                  uint32_t n, uint32_t k) {
+    gemm_act_fp8_body(xq, xs, bsum, rec, n, k);
+}
 
 // global -> LDS copy of 1 KB (64 lanes x 16 B) without passing through registers: lane i's 16 bytes
 // at base + off_lane land at LDS address lds + 16 i.  base and lds are wavefront-uniform (scalar
@@ -155,7 +160,7 @@ struct G8Mins {
 };
 
 template <bool SWIGLU = false, bool DBG = false, int NW = G8_NW>
-static __global__ __launch_bounds__(64 * NW, 8 / NW) void gemm_q4k_fp8_kernel(GemmArgs p) {
+__device__ __forceinline__ void gemm_q4k_fp8_body(GemmArgs p) {
     constexpr uint32_t BM = 32 * NW;   // rows per workgroup
     // the two stage buffers are separate variables so that the compiler can tell the DMA into one
     // from the fragment reads of the other (a shared array would make every LDS read wait for
@@ -506,4 +511,8 @@ static __global__ __launch_bounds__(64 * NW, 8 / NW) void gemm_q4k_fp8_kernel(Ge
             }
         }
     }
+}
+template <bool SWIGLU = false, bool DBG = false, int NW = G8_NW>
+static __global__ __launch_bounds__(64 * NW, 8 / NW) void gemm_q4k_fp8_kernel(GemmArgs p) {
+    gemm_q4k_fp8_body<SWIGLU, DBG, NW>(p);
 }

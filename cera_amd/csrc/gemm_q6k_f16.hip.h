@@ -32,7 +32,7 @@ typedef uint32_t gq_u4 __attribute__((ext_vector_type(4)));
 #define GQ_LD 272   // bytes per staged row: 128 f16 + 16 pad
 
 // int8 quants [n_words * 16] -> f16 in the 0,2,1,3 order, 16 per thread
-static __global__ __launch_bounds__(256) void gemm_act_f16_kernel(const uint4* __restrict__ q, uint4* __restrict__ out,
+__device__ __forceinline__ void gemm_act_f16_body(const uint4* __restrict__ q, uint4* __restrict__ out,
                                                                   uint64_t n_words) {
     const uint64_t i = static_cast<uint64_t>(blockIdx.x) * 256 + threadIdx.x;
     if (i >= n_words) return;
@@ -51,12 +51,16 @@ static __global__ __launch_bounds__(256) void gemm_act_f16_kernel(const uint4* _
     out[2 * i] = make_uint4(o[0], o[1], o[2], o[3]);
     out[2 * i + 1] = make_uint4(o[4], o[5], o[6], o[7]);
 }
+static __global__ __launch_bounds__(256) void gemm_act_f16_kernel(const uint4* __restrict__ q, uint4* __restrict__ out,
+                                                                  uint64_t n_words) {
+    gemm_act_f16_body(q, out, n_words);
+}
 
 // byte offset of 16-byte chunk `chunk` of staged row `row`
 __device__ __forceinline__ uint32_t gq_off(uint32_t row, uint32_t chunk) { return row * GQ_LD + (chunk << 4); }
 
 template <bool DBG = false>
-static __global__ __launch_bounds__(256, 2) void gemm_q6k_f16_kernel(GemmArgs p) {
+__device__ __forceinline__ void gemm_q6k_f16_body(GemmArgs p) {
     constexpr int NB = GEMM_KT / 32;
     __shared__ __attribute__((aligned(16))) uint8_t sA[GEMM_BM * GQ_LD];
     __shared__ __attribute__((aligned(16))) uint8_t sB[GEMM_BN * GQ_LD];
@@ -218,4 +222,8 @@ static __global__ __launch_bounds__(256, 2) void gemm_q6k_f16_kernel(GemmArgs p)
                     }
                 }
     }
+}
+template <bool DBG = false>
+static __global__ __launch_bounds__(256, 2) void gemm_q6k_f16_kernel(GemmArgs p) {
+    gemm_q6k_f16_body<DBG>(p);
 }

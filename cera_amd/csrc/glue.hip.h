@@ -74,7 +74,7 @@ __device__ __forceinline__ float dequant_elem(uint32_t dtype, const uint8_t* row
 // token comes from device memory so a graph-captured decode step can chain on
 // the previous step's argmax without a host round trip.
 // grid.y = number of tokens (prefill looks up a batch of rows: out is [n][k]).
-static __global__ void embed_row_kernel(uint32_t dtype, const uint8_t* __restrict__ w, uint64_t row_bytes,
+__device__ __forceinline__ void embed_row_body(uint32_t dtype, const uint8_t* __restrict__ w, uint64_t row_bytes,
                                  const uint32_t* __restrict__ token, uint32_t k, float scale,
                                  float* __restrict__ out) {
     uint32_t e = blockIdx.x * blockDim.x + threadIdx.x;
@@ -82,10 +82,15 @@ static __global__ void embed_row_kernel(uint32_t dtype, const uint8_t* __restric
     float v = dequant_elem(dtype, w + static_cast<uint64_t>(token[blockIdx.y]) * row_bytes, e);
     out[static_cast<uint64_t>(blockIdx.y) * k + e] = scale != 1.0f ? __fmul_rn(v, scale) : v;
 }
+static __global__ void embed_row_kernel(uint32_t dtype, const uint8_t* __restrict__ w, uint64_t row_bytes,
+                                 const uint32_t* __restrict__ token, uint32_t k, float scale,
+                                 float* __restrict__ out) {
+    embed_row_body(dtype, w, row_bytes, token, k, scale, out);
+}
 
 // The decode step's first launch: the token's embedding row, and the token id and position into
 // scalars[0..1] for the kernels behind it (one launch instead of a one-thread kernel plus the lookup).
-static __global__ void embed_token_kernel(uint32_t dtype, const uint8_t* __restrict__ w, uint64_t row_bytes, uint32_t token,
+__device__ __forceinline__ void embed_token_body(uint32_t dtype, const uint8_t* __restrict__ w, uint64_t row_bytes, uint32_t token,
                                           uint32_t pos, uint32_t* __restrict__ scalars, uint32_t k, float scale,
                                           float* __restrict__ out) {
     uint32_t e = blockIdx.x * blockDim.x + threadIdx.x;
@@ -97,6 +102,11 @@ static __global__ void embed_token_kernel(uint32_t dtype, const uint8_t* __restr
     float v = dequant_elem(dtype, w + static_cast<uint64_t>(token) * row_bytes, e);
     out[e] = scale != 1.0f ? __fmul_rn(v, scale) : v;
 }
+static __global__ void embed_token_kernel(uint32_t dtype, const uint8_t* __restrict__ w, uint64_t row_bytes, uint32_t token,
+                                          uint32_t pos, uint32_t* __restrict__ scalars, uint32_t k, float scale,
+                                          float* __restrict__ out) {
+    embed_token_body(dtype, w, row_bytes, token, pos, scalars, k, scale, out);
+}
 
 // ---------------------------------------------------------------------------
 // RMSNorm (cera/src/backend/cpu.rs:2479-2496): f64 sum of squares,
@@ -106,7 +116,7 @@ static __global__ void embed_token_kernel(uint32_t dtype, const uint8_t* __restr
 // differences (~1e-16 relative) vanish when inv is narrowed to f32 except in
 // astronomically rare double-rounding cases.
 template <bool QUANT>
-static __global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ x, const float* __restrict__ w,
+__device__ __forceinline__ void rmsnorm_body(const float* __restrict__ x, const float* __restrict__ w,
                                                       uint32_t n, float eps, float* __restrict__ y,
                                                       float* __restrict__ scales, int8_t* __restrict__ quants,
                                                       float* __restrict__ bsum) {
@@ -149,6 +159,13 @@ static __global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __rest
             }
         }
     }
+}
+template <bool QUANT>
+static __global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                                                      uint32_t n, float eps, float* __restrict__ y,
+                                                      float* __restrict__ scales, int8_t* __restrict__ quants,
+                                                      float* __restrict__ bsum) {
+    rmsnorm_body<QUANT>(x, w, n, eps, y, scales, quants, bsum);
 }
 
 // Single-pass variant for the decode step (one row, n <= 16384): 1024 threads
@@ -216,7 +233,7 @@ static __global__ __launch_bounds__(1024) void rmsnorm_row_kernel(const float* _
 // store it; the last n_kv_heads copy v.
 // KV cache layout: [kv_head][max_seq][head_dim] f32.
 template <typename KV>
-static __global__ void rope_kv_kernel(float* __restrict__ q, float* __restrict__ k, const float* v,
+__device__ __forceinline__ void rope_kv_body(float* __restrict__ q, float* __restrict__ k, const float* v,
                                const float* __restrict__ cs_table, const uint32_t* __restrict__ pos_ptr,
                                uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, uint32_t rope_type,
                                KV* __restrict__ k_cache, KV* __restrict__ v_cache, uint32_t max_seq) {
@@ -248,6 +265,13 @@ static __global__ void rope_kv_kernel(float* __restrict__ q, float* __restrict__
         dst[2 * i + 1] = static_cast<KV>(v[h * head_dim + 2 * i + 1]);
     }
 }
+template <typename KV>
+static __global__ void rope_kv_kernel(float* __restrict__ q, float* __restrict__ k, const float* v,
+                               const float* __restrict__ cs_table, const uint32_t* __restrict__ pos_ptr,
+                               uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, uint32_t rope_type,
+                               KV* __restrict__ k_cache, KV* __restrict__ v_cache, uint32_t max_seq) {
+    rope_kv_body<KV>(q, k, v, cs_table, pos_ptr, n_heads, n_kv_heads, head_dim, rope_type, k_cache, v_cache, max_seq);
+}
 
 // n_keep context shift (cera/src/kv_cache.rs:1091-1310): rows [src_row, src_row + n_rows) of every
 // kv head move to [dst_row, ...) of `dst` (the cache itself when the two ranges do not overlap,
@@ -257,7 +281,7 @@ static __global__ void rope_kv_kernel(float* __restrict__ q, float* __restrict__
 // copy (V, and the copy back from staging).  HD / 8 threads per row, each owning float4 j and
 // float4 j + HD / 8 (its NEOX partner).  grid = (ceil(n_rows * HD / 8 / 256), n_kv_heads).
 template <typename KV, int HD>
-static __global__ __launch_bounds__(256) void kv_shift_kernel(const KV* __restrict__ src, KV* __restrict__ dst,
+__device__ __forceinline__ void kv_shift_body(const KV* __restrict__ src, KV* __restrict__ dst,
                                                               uint32_t src_row, uint32_t dst_row, uint32_t n_rows,
                                                               uint64_t src_head_stride, uint64_t dst_head_stride,
                                                               const float* __restrict__ delta_cs, uint32_t rope_type) {
@@ -300,30 +324,47 @@ static __global__ __launch_bounds__(256) void kv_shift_kernel(const KV* __restri
     KvOps<KV>::st4(dp, j, a);
     KvOps<KV>::st4(dp, j + TPR, b);
 }
+template <typename KV, int HD>
+static __global__ __launch_bounds__(256) void kv_shift_kernel(const KV* __restrict__ src, KV* __restrict__ dst,
+                                                              uint32_t src_row, uint32_t dst_row, uint32_t n_rows,
+                                                              uint64_t src_head_stride, uint64_t dst_head_stride,
+                                                              const float* __restrict__ delta_cs, uint32_t rope_type) {
+    kv_shift_body<KV, HD>(src, dst, src_row, dst_row, n_rows, src_head_stride, dst_head_stride, delta_cs, rope_type);
+}
 
 // out = a + b (cera/src/backend/cpu.rs:5223-5228), optional scale on b first.
-static __global__ void add_kernel(const float* __restrict__ a, const float* __restrict__ b, float bscale, uint32_t n,
+__device__ __forceinline__ void add_body(const float* __restrict__ a, const float* __restrict__ b, float bscale, uint32_t n,
                            float* __restrict__ out) {
     uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
     float t = bscale != 1.0f ? __fmul_rn(b[i], bscale) : b[i];
     out[i] = __fadd_rn(a[i], t);
 }
+static __global__ void add_kernel(const float* __restrict__ a, const float* __restrict__ b, float bscale, uint32_t n,
+                           float* __restrict__ out) {
+    add_body(a, b, bscale, n, out);
+}
 
 // bias add in place: x[i] += b[i]
-static __global__ void bias_kernel(float* __restrict__ x, const float* __restrict__ b, uint32_t n) {
+__device__ __forceinline__ void bias_body(float* __restrict__ x, const float* __restrict__ b, uint32_t n) {
     uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) x[i] = __fadd_rn(x[i], b[i]);
 }
-static __global__ void scale_kernel(float* __restrict__ x, float s, uint32_t n) {
+static __global__ void bias_kernel(float* __restrict__ x, const float* __restrict__ b, uint32_t n) {
+    bias_body(x, b, n);
+}
+__device__ __forceinline__ void scale_body(float* __restrict__ x, float s, uint32_t n) {
     uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) x[i] = __fmul_rn(x[i], s);
+}
+static __global__ void scale_kernel(float* __restrict__ x, float s, uint32_t n) {
+    scale_body(x, s, n);
 }
 
 // SiLU(gate)*up (cera/src/backend/cpu.rs:2570-2575) with optional Q8_0
 // quantisation of the result (the activation of the down projection).
 template <bool QUANT>
-static __global__ __launch_bounds__(256) void silu_mul_kernel(const float* __restrict__ gate, const float* __restrict__ up,
+__device__ __forceinline__ void silu_mul_body(const float* __restrict__ gate, const float* __restrict__ up,
                                                        uint64_t n, float* __restrict__ out,
                                                        float* __restrict__ scales, int8_t* __restrict__ quants,
                                                        float* __restrict__ bsum) {
@@ -350,6 +391,13 @@ static __global__ __launch_bounds__(256) void silu_mul_kernel(const float* __res
     }
     if (live && out) reinterpret_cast<float4*>(out)[t] = o;
 }
+template <bool QUANT>
+static __global__ __launch_bounds__(256) void silu_mul_kernel(const float* __restrict__ gate, const float* __restrict__ up,
+                                                       uint64_t n, float* __restrict__ out,
+                                                       float* __restrict__ scales, int8_t* __restrict__ quants,
+                                                       float* __restrict__ bsum) {
+    silu_mul_body<QUANT>(gate, up, n, out, scales, quants, bsum);
+}
 
 // ---------------------------------------------------------------------------
 // argmax (cera/src/sampler.rs:20-30): strict >, lowest index on ties, NaN never
@@ -372,7 +420,7 @@ __device__ __forceinline__ void argmax_block_reduce(float& bv, uint32_t& bi, flo
     if (threadIdx.x == 0)
         for (uint32_t w = 1; w < blockDim.x / 64; ++w) argmax_merge(bv, bi, sv[w], si[w]);
 }
-static __global__ __launch_bounds__(256) void argmax_partial_kernel(const float* __restrict__ x, uint32_t n,
+__device__ __forceinline__ void argmax_partial_body(const float* __restrict__ x, uint32_t n,
                                                              float* __restrict__ pv, uint32_t* __restrict__ pi) {
     __shared__ float sv[4];
     __shared__ uint32_t si[4];
@@ -387,9 +435,13 @@ static __global__ __launch_bounds__(256) void argmax_partial_kernel(const float*
     argmax_block_reduce(bv, bi, sv, si);
     if (threadIdx.x == 0) { pv[blockIdx.x] = bv; pi[blockIdx.x] = bi; }
 }
+static __global__ __launch_bounds__(256) void argmax_partial_kernel(const float* __restrict__ x, uint32_t n,
+                                                             float* __restrict__ pv, uint32_t* __restrict__ pi) {
+    argmax_partial_body(x, n, pv, pi);
+}
 // out2 (nullable): a second place for the index -- host memory the device can write, so that the
 // greedy step needs no copy launch after this one
-static __global__ __launch_bounds__(256) void argmax_final_kernel(const float* __restrict__ pv, const uint32_t* __restrict__ pi,
+__device__ __forceinline__ void argmax_final_body(const float* __restrict__ pv, const uint32_t* __restrict__ pi,
                                                            uint32_t np, uint32_t* __restrict__ out, uint32_t* __restrict__ out2) {
     __shared__ float sv[4];
     __shared__ uint32_t si[4];
@@ -402,4 +454,8 @@ static __global__ __launch_bounds__(256) void argmax_final_kernel(const float* _
         *out = v;
         if (out2) *out2 = v;
     }
+}
+static __global__ __launch_bounds__(256) void argmax_final_kernel(const float* __restrict__ pv, const uint32_t* __restrict__ pi,
+                                                           uint32_t np, uint32_t* __restrict__ out, uint32_t* __restrict__ out2) {
+    argmax_final_body(pv, pi, np, out, out2);
 }

@@ -165,6 +165,235 @@ typedef struct {
     uint32_t n_blocks_a;
 } cera_k_row_gemv_pair_args;
 
+/* ==== the rest of a forward pass ===================================================================
+ * With the kernels below a host runs LlamaModel::forward and ::forward_prefill
+ * (cera/src/model/llama.rs:468-597, 738-1523) from the code object alone; cera_amd/hsaco_api.py does,
+ * and tests/test_gpu_hsaco.py compares its logits with the library's.  KV caches are head-major,
+ * [n_kv_heads][max_seq][head_dim], f32 (`f32` instances) or IEEE half (`f16`); head_dim 64 or 128. */
+
+/* ---- cera_k_embed_token / cera_k_embed_rows ---------------------------------------------------
+ * One row of the embedding table dequantized (dequantize_*_row, cera/src/quant.rs:318-539) and
+ * multiplied by `scale` when that is not 1.  ggml_type: 0 F32, 1 F16, 30 BF16, 2, 3, 8, 12, 13, 14.
+ * embed_token also writes scalars[0] = token, scalars[1] = pos (the position word rope_kv reads).
+ * grid = ceil(k / 256) workgroups of 256;  embed_rows: grid = (ceil(k / 256), n_tokens), out [n][k]. */
+typedef struct {
+    const uint8_t* w;
+    uint64_t row_bytes;
+    uint32_t ggml_type, token, pos, k;
+    uint32_t* scalars;
+    float scale;
+    float* out;
+} cera_k_embed_token_args;
+typedef struct {
+    const uint8_t* w;
+    uint64_t row_bytes;
+    const uint32_t* tokens;
+    uint32_t ggml_type, k;
+    float scale;
+    float* out;
+} cera_k_embed_rows_args;
+
+/* ---- cera_k_rmsnorm_rows / cera_k_rmsnorm_rows_q8_0 -------------------------------------------
+ * cpu::rmsnorm (cera/src/backend/cpu.rs:2479-2496) of `rows` rows of n elements (x and y may be
+ * the same buffer); _q8_0 also writes each row's Q8_0 quantization: scales [rows][n/32], quants
+ * [rows][n], bsum [rows][n/32] = scale * sum(quants) (nullable).  n % 32 == 0 for _q8_0.
+ * grid = rows workgroups of 256. */
+typedef struct {
+    const float* x;
+    const float* w;
+    uint32_t n;
+    float eps;
+    float* y;
+    float* scales;
+    int8_t* quants;
+    float* bsum;
+} cera_k_rmsnorm_rows_args;
+
+/* ---- cera_k_rope_kv_<f32|f16> -----------------------------------------------------------------
+ * RoPE on q and k in place and the append of k, v to the caches (rope_type 1: interleaved pairs,
+ * cera/src/backend/cpu.rs:5161-5180; 0: split halves, :5031-5045).  cs_table [max_seq][head_dim/2]
+ * of (cos, sin) built by the host with the reference's recurrence: theta_0 = pos as f32,
+ * theta_{i+1} = theta_i * base^(-2/head_dim) in f32, angle = theta_i (/ freq_factor_i for rope_type
+ * 1), libm cosf / sinf.  Token t of the batch sits at position *pos + t; q [n][n_heads*head_dim],
+ * k, v [n][n_kv_heads*head_dim].  grid = (n_heads + 2 n_kv_heads, n_tokens) of head_dim / 2 threads. */
+typedef struct {
+    float* q;
+    float* k;
+    const float* v;
+    const float* cs_table;
+    const uint32_t* pos;
+    uint32_t n_heads, n_kv_heads, head_dim, rope_type;
+    void* k_cache;
+    void* v_cache;
+    uint32_t max_seq;
+} cera_k_rope_kv_args;
+
+/* ---- cera_k_attn_decode_partial_<f32|f16>_hd<64|128>_g<1|2|4>_s<1|4> ---------------------------
+ * GQA flash-decode, split over the keys (decode_attention, cera/src/model/transformer.rs:1249-1305):
+ * wavefront (query, kv head, sub-group, part) scans chunks_per_part chunks of 8 S keys with an
+ * online softmax for g query heads and leaves an unnormalised partial.
+ *   g        query heads one wavefront serves; g_total = n_heads / n_kv_heads must be a multiple
+ *            (the library takes g = g_total / 2 for groups of 4 and 8 below 16k keys)
+ *   S        8 S keys per chunk (the library: 1 below 1024 keys, 4 beyond with split groups)
+ *   n_parts  = ceil(ceil(seq_len / (8 S)) / chunks_per_part), at most 1024; the library aims at
+ *            4 wavefronts per CU: chunks_per_part = max(1, ceil(chunks / (4 n_cu / n_kv)))
+ *   seq_len  keys visible to query 0; query i (n_queries > 1, q rows q_stride floats apart) sees
+ *            seq_len + i
+ *   part_acc [n_queries][n_kv][n_parts][g_total][head_dim], part_ml [...][g_total][2]
+ * grid = ceil(ceil(n_parts / 4) * n_kv / 8) * 8 * (g_total / g) * n_queries workgroups of 256
+ * (four consecutive parts per workgroup; the kernel maps launch indices to key ranges XCD by XCD
+ * and ignores the padding).
+ * ---- cera_k_attn_decode_merge_hd<64|128>[_q8_0] ------------------------------------------------
+ * out[head] = sum_p e^(m_p - M) acc_p / sum_p e^(m_p - M) l_p; _q8_0 also writes the Q8_0
+ * quantization of the n_heads * head_dim outputs (scales, quants, bsum nullable).
+ * grid = (n_heads, n_queries) workgroups of 256; out [n_queries][n_heads * head_dim]. */
+typedef struct {
+    const float* q;
+    const void* kc;
+    const void* vc;
+    uint32_t seq_len, max_seq;
+    float scale;
+    uint32_t chunks_per_part, n_parts, q_stride, g_total, n_kv, n_queries;
+    float* part_acc;
+    float* part_ml;
+} cera_k_attn_decode_args;
+typedef struct {
+    const float* part_acc;
+    const float* part_ml;
+    uint32_t n_parts, g_total, n_heads;
+    uint32_t n_pairs;          /* prefill merge: n_heads * n_queries; decode merge: unused */
+    float* out;
+    float* scales;
+    int8_t* quants;
+    float* bsum;
+} cera_k_attn_merge_args;
+
+/* ---- cera_k_attn_prefill_partial_<f32|f16>_hd<64|128>_g<1|2|4|8> ------------------------------
+ * Causal attention of a batch of queries (>= 16; fewer go through the decode kernel with
+ * n_queries) on the f16 matrix cores: a workgroup = 32 queries x one kv head x one key part,
+ * g = n_heads / n_kv_heads wavefronts.  The batch's own keys are already in the cache (rope_kv).
+ *   first_len  keys visible to query 0; query i sees first_len + i
+ *   part_keys  keys per part, a multiple of 32 (the library: 128 up to 1024 keys, else about an
+ *              eighth of the keys); n_parts = ceil((first_len + n_queries - 1) / part_keys) <= 1024
+ *   q rows 16-byte aligned, q_stride floats apart
+ * grid = (ceil(n_queries / 32), n_kv, n_parts) workgroups of 64 g.
+ * ---- cera_k_attn_prefill_merge_hd<64|128>[_q8_0] -----------------------------------------------
+ * The merge for a batch: eight (query, head) pairs per workgroup.  grid = ceil(n_pairs / 8) of 256. */
+typedef struct {
+    const float* q;
+    const void* kc;
+    const void* vc;
+    uint32_t first_len, n_queries, max_seq;
+    float scale;
+    uint32_t part_keys, n_parts, q_stride;
+    float* part_acc;
+    float* part_ml;
+} cera_k_attn_prefill_args;
+
+/* ---- cera_k_silu_mul[_q8_0], cera_k_add, cera_k_bias, cera_k_scale ----------------------------
+ * silu_mul: out = gate / (1 + expf(-gate)) * up (silu_mul_inplace, cera/src/backend/cpu.rs:2570-2575),
+ * n % 4 == 0 (_q8_0: n % 32 == 0, plus the Q8_0 quantization of out in rows of any length that
+ * is a multiple of 32); grid = ceil(n / 4 / 256) of 256.  add: out = a + b_scale * b.  bias: x += b.
+ * scale: x *= s.  grid = ceil(n / 256) of 256. */
+typedef struct {
+    const float* gate;
+    const float* up;
+    uint64_t n;
+    float* out;
+    float* scales;
+    int8_t* quants;
+    float* bsum;
+} cera_k_silu_mul_args;
+typedef struct { const float* a; const float* b; float b_scale; uint32_t n; float* out; } cera_k_add_args;
+typedef struct { float* x; const float* b; uint32_t n; } cera_k_bias_args;
+typedef struct { float* x; float s; uint32_t n; } cera_k_scale_args;
+
+/* ---- cera_k_argmax_partial / cera_k_argmax_final ----------------------------------------------
+ * Greedy sampling (cera/src/sampler.rs:20-30: strict >, lowest index on ties).  partial: workgroup
+ * b reduces its slice of x[0, n) to (pv[b], pi[b]); grid = np workgroups of 256 (the library:
+ * np = min(1024, ceil(n / 1024))).  final: one workgroup of 256 reduces the np candidates into
+ * *out (and *out2 when not null, e.g. a device view of pinned host memory). */
+typedef struct { const float* x; uint32_t n; float* pv; uint32_t* pi; } cera_k_argmax_partial_args;
+typedef struct { const float* pv; const uint32_t* pi; uint32_t np; uint32_t* out; uint32_t* out2; } cera_k_argmax_final_args;
+
+/* ---- cera_k_kv_shift_<f32|f16>_hd<64|128> -----------------------------------------------------
+ * The n_keep context shift (InferenceState::shift_kv_with_rope, cera/src/kv_cache.rs:1091-1310):
+ * rows [src_row, src_row + n_rows) of every kv head move to [dst_row, ...) of dst, K rows rotated
+ * on the way by R(-shift) whose head_dim / 2 (cos, sin) pairs the host builds with the recurrence
+ * above (theta_0 = -shift); delta_cs NULL = plain copy (V, and the copy back from staging when
+ * source and destination rows overlap).  head strides in elements.
+ * grid = (ceil(n_rows * head_dim / 8 / 256), n_kv_heads) of 256. */
+typedef struct {
+    const void* src;
+    void* dst;
+    uint32_t src_row, dst_row, n_rows;
+    uint64_t src_head_stride, dst_head_stride;
+    const float* delta_cs;
+    uint32_t rope_type;
+} cera_k_kv_shift_args;
+
+/* ==== batched (prefill) GEMMs: transformer::gemm_preq (cera/src/model/transformer.rs:710-788) =====
+ * out[i * ld_m + j * ld_n] = sum over k of W[i][k] * B[j][k] (+ resid), B = n token rows quantized
+ * to Q8_0 by cera_k_quantize_q8_0 / cera_k_rmsnorm_rows_q8_0 / a _q8_0 merge: bq [n][k], bs
+ * [n][k/32], bsum [n][k/32] (needed by q4_k and q4_1).  Exact integer block dots, then the
+ * reference's per-block float scales.  k % 256 == 0 for q4_k / q6_k, k % 128 == 0 otherwise.
+ *   cera_k_gemm_q4_k          fp8 matrix cores; reads bf8, the split copy cera_k_gemm_act_fp8 makes
+ *                             of (bq, bs, bsum): CERA_K_GEMM_FP8_ACT_BYTES(n, k) bytes,
+ *                             grid = ceil(n / 64) * 2 * (k / 256) workgroups of 256
+ *   cera_k_gemm_q4_k_swiglu   w = gate, w2 = up (both m x k, m % 32 == 0): nothing goes to out; hq [n][m], hs and
+ *                             hbsum [n][m/32] receive Q8_0(silu(gate.x) * (up.x)); a workgroup takes 64 gate and the
+ *                             same 64 up rows: grid = (ceil(n / 64), ceil(m / 64)), k_chunk = k
+ *   cera_k_gemm_q6_k          f16 matrix cores; reads bh, the quants as f16 made by
+ *                             cera_k_gemm_act_f16 (n * k * 2 bytes; n_words = n * k / 16,
+ *                             grid = ceil(n_words / 256) of 256)
+ *   cera_k_gemm_q4_0 | q4_1 | q8_0   int8 matrix cores
+ * grid = (ceil(n / 64), ceil(m / 128) [+ ceil(m2 / 128) for a pair], split) workgroups of 256.
+ * One matrix, no split: k_chunk = k, part_stride = 0, w2 = out2 = NULL, m2 = 0, tiles1 =
+ * ceil(m / 128), hq = hs = hbsum = dbg_dots = NULL.  Split K (grid.z = split, k_chunk = k / split
+ * a multiple of 512): every slice writes its partial to out + z * part_stride (out is then a
+ * scratch buffer, ld_m = 1, ld_n = m) and cera_k_gemm_reduce adds them in order.
+ * The library's results for a token-major output are ld_m = 1, ld_n = m. */
+#define CERA_K_GEMM_FP8_ACT_BYTES(n, k) ((uint64_t)(((n) + 63) / 64) * 2 * ((k) / 256) * 21504u)
+typedef struct {
+    const uint8_t* w;
+    const int8_t* bq;
+    const float* bs;
+    const float* bsum;
+    const void* bh;
+    float* out;
+    uint32_t m, n, k;
+    uint32_t row_bytes;
+    uint64_t ld_m, ld_n;
+    const float* resid;
+    float resid_scale;
+    uint32_t k_chunk;
+    uint64_t part_stride;
+    const uint8_t* w2;
+    float* out2;
+    uint32_t m2, tiles1;
+    uint64_t ld_n2;
+    int8_t* hq;
+    float* hs;
+    float* hbsum;
+    int32_t* dbg_dots;
+    const uint8_t* bf8;
+} cera_k_gemm_args;
+typedef struct { const int8_t* quants; const float* scales; const float* bsum; uint8_t* out; uint32_t n, k; } cera_k_gemm_act_fp8_args;
+typedef struct { const void* quants; void* out; uint64_t n_words; } cera_k_gemm_act_f16_args;
+/* out[e] = (resid[e] + resid_scale *) sum_z part[z * part_stride + e] over n4 float4s; for a pair
+ * float4s from n4_first on go to out2 (no pair: n4_first = n4, out2 = NULL).
+ * grid = ceil(n4 / 256) of 256. */
+typedef struct {
+    const float* part;
+    uint32_t n_split;
+    uint64_t part_stride, n4;
+    float* out;
+    const float* resid;
+    float resid_scale;
+    uint64_t n4_first;
+    float* out2;
+} cera_k_gemm_reduce_args;
+
 #ifdef __cplusplus
 }
 #endif

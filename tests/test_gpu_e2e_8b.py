@@ -35,17 +35,36 @@ from cera_amd import host_api as H, llama_api, synth
 pytestmark = pytest.mark.gpu
 
 
+_CAPSYS = None
+
+
 def _say(msg):
-    print(msg, flush=True)
+    """Progress lines go to the real stdout even when pytest captures output: the full-size case runs
+    for minutes, most of it inside the CPU oracle, and a harness watching for output must see it move."""
+    if _CAPSYS is not None:
+        with _CAPSYS.disabled():
+            print(msg, flush=True)
+    else:
+        print(msg, flush=True)
 
 
-def test_llama3_8b_shapes_4_layers_prefill_128_greedy_32(tmp_path, orc, hip):
-    _run(tmp_path, orc, 4, 128, 32)
+def test_llama3_8b_shapes_4_layers_prefill_128_greedy_32(tmp_path, orc, hip, capsys):
+    global _CAPSYS
+    _CAPSYS = capsys
+    try:
+        _run(tmp_path, orc, 4, 128, 32)
+    finally:
+        _CAPSYS = None
 
 
-def test_llama3_8b_prefill_512_greedy_256(tmp_path, orc, hip):
+def test_llama3_8b_prefill_512_greedy_256(tmp_path, orc, hip, capsys):
+    global _CAPSYS
+    _CAPSYS = capsys
     n_layers = int(os.environ.get("CERA_E2E_LAYERS", synth.LLAMA3_8B["n_layers"]))
-    _run(tmp_path, orc, n_layers, 512, int(os.environ.get("CERA_E2E_NEW", 256)))
+    try:
+        _run(tmp_path, orc, n_layers, 512, int(os.environ.get("CERA_E2E_NEW", 256)))
+    finally:
+        _CAPSYS = None
 
 
 def _bits(a):
@@ -174,6 +193,8 @@ def _run(tmp_path, orc, n_layers, n_prompt, n_new):
         if i + 1 < n_new:
             lb, la = ob.forward(tb, n_prompt + i), oa.forward(tb, n_prompt + i)
             lc = oc.forward(tc, n_prompt + i)
+            if (i + 1) % 64 == 0:
+                _say(f"e2e: oracle decode step {i + 1}/{n_new}")
     _say(f"e2e: oracle decode {time.time() - t0:.0f} s")
     _say(f"e2e: GPU reference-order route vs oracle: identical greedy tokens {same_ref}/{n_new} (free running), "
          f"logits bit-identical at {bit_equal_steps}/{n_new} steps")

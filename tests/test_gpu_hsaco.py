@@ -132,6 +132,58 @@ def test_library_launching_from_the_code_object(hip, orc):
         mod.close()
 
 
+def _host_model_cfg():
+    from cera_amd import synth
+    return dict(synth.TINY, n_layers=2, hidden=512, ffn=1024, n_heads=8, n_kv_heads=2, head_dim=128, vocab=640, max_seq_len=96)
+
+
+def test_whole_decode_step_from_the_code_object(hip, orc, host):
+    """A pure hipModuleLaunchKernel host (cera_amd/hsaco_api.Model: no libcera_hip.so) runs the decode
+    step of a small llama -- embedding, fused norm + Q|K|V, RoPE + cache append, split-K attention and
+    merge, O, fused norm + gate|up + SwiGLU, down, final norm, head, argmax -- and gets the library's
+    logits bit for bit, token after token (free-running greedy), and the oracle's within its bar."""
+    from cera_amd import synth
+    cfg = _host_model_cfg()
+    weights = synth.make_llama(cfg, seed=77, sigma=0.05, norm_jitter=0.1)
+    lib = hip_api.Model(hip, cfg, weights)
+    om = orc.Llama(cfg, weights)
+    hm = hsaco_api.Model(host, cfg, weights, n_cu=hip.device_info()[1])
+    print("hsaco: whole decode step, 12 greedy tokens", flush=True)
+    tok = 11
+    for pos in range(12):
+        a, b, o = hm.forward(tok, pos), lib.forward(tok, pos), om.forward(tok, pos)
+        assert np.array_equal(_bits(a), _bits(b)), (pos, float(np.abs(a - b).max()))
+        assert np.abs(a - o).max() <= 0.1 * util.rms(o)
+        assert hm.argmax() == int(orc.argmax(a))
+        tok = int(orc.argmax(a))
+    lib.close(); om.close()
+
+
+def test_batched_prefill_from_the_code_object(hip, orc, host):
+    """The same host prefills 32 tokens in one pass -- embedding rows, rmsnorm + Q8_0 per row, the
+    fp8 (Q4_K) and f16 (Q6_K) GEMMs with their activation-layout kernels, RoPE + append for the batch,
+    the MFMA prefill attention and its merge, SwiGLU + Q8_0, residual GEMMs -- then decodes on top of
+    the cache it built: logits equal to the library's (same kernels, same launch rules) and close to
+    the oracle's batched route."""
+    from cera_amd import synth
+    cfg = _host_model_cfg()
+    weights = synth.make_llama(cfg, seed=78, sigma=0.05, norm_jitter=0.1)
+    lib = hip_api.Model(hip, cfg, weights)
+    om = orc.Llama(cfg, weights)
+    hm = hsaco_api.Model(host, cfg, weights, n_cu=hip.device_info()[1])
+    prompt = [int(t) for t in util.rng(3).integers(0, cfg["vocab"], 32)]
+    print("hsaco: 32-token prefill + 4 decode steps", flush=True)
+    a, b, o = hm.forward_prefill(prompt, 0), lib.forward_prefill(prompt, 0), om.forward_prefill_batched(prompt, 0)
+    assert np.array_equal(_bits(a), _bits(b)), float(np.abs(a - b).max())
+    assert np.abs(a - o).max() <= 0.1 * util.rms(o)
+    tok = int(orc.argmax(b))
+    for i in range(4):
+        a, b = hm.forward(tok, 32 + i), lib.forward(tok, 32 + i)
+        assert np.array_equal(_bits(a), _bits(b)), (i, float(np.abs(a - b).max()))
+        tok = int(orc.argmax(b))
+    lib.close(); om.close()
+
+
 def test_a_wrong_code_object_is_refused(tmp_path):
     bad = tmp_path / "not_a_code_object.hsaco"
     bad.write_bytes(b"\x7fELF" + bytes(200))
