@@ -123,7 +123,11 @@ public:
                                                   InferenceState& state) override;
     bool supports_all_logits() const override { return true; }
     void truncate_kv(InferenceState& state, size_t len) override;
-    bool supports_kv_shift() const override { return true; }
+    // the shift kernel is instantiated for the head sizes models use
+    bool supports_kv_shift() const override {
+        const size_t hd = config_.head_dim;
+        return hd == 32 || hd == 64 || hd == 80 || hd == 96 || hd == 128 || hd == 256;
+    }
     bool f16_kv_supported() const override { return true; }
     void configure_kv_compression(KvCompression mode) override;
     KvCompression kv_compression() const;

@@ -707,11 +707,31 @@ cera_hip_status cera_launch_attn(cera_hip_ctx* ctx, const float* q, const void* 
                                  uint64_t max_seq, float scale, uint32_t n_splits, uint32_t n_queries, float* out,
                                  float* out_scales, int8_t* out_quants, float* out_bsum, const AttnNewKV* new_kv,
                                  bool kv_f16, const AttnWorkspace* ws) {
-    if (head_dim != 64 && head_dim != 128) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "attention: head_dim must be 64 or 128");
     if (n_kv_heads == 0 || n_heads % n_kv_heads) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "attention: n_heads must be a multiple of n_kv_heads");
-    uint32_t G = n_heads / n_kv_heads;
-    if (G > 8) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "attention: at most 8 query heads per kv head");
     if (n_queries == 0 || n_queries > 65535) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "attention: 1..65535 queries per call");
+    if (!cera_attn_shape_tuned(n_heads, n_kv_heads, head_dim)) {
+        // Any other head size (a multiple of 8 up to 256) or group size, as decode_attention takes them
+        // (cera/src/model/transformer.rs:1249-1305): one launch of the generic kernel per query, then the
+        // Q8_0 quantization of the outputs.  Correct and slow; no model of the benchmark configs comes here.
+        if (head_dim % 8 || head_dim > 256 || head_dim == 0)
+            return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "attention: head_dim must be a multiple of 8, at most 256");
+        if (new_kv) return cera_fail(ctx, CERA_HIP_ERR_ARGUMENT, "attention: fused RoPE/append needs head_dim 64 or 128 and at most 8 heads per kv head");
+        if (seq_len == 0 || seq_len + n_queries - 1 > max_seq || max_seq > 0x7FFFFFFFull)
+            return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "attention: need 0 < seq_len <= max_seq < 2^31");
+        void* scores;
+        CERA_TRY(cera_scratch(ctx, 13, static_cast<uint64_t>(n_heads) * max_seq * sizeof(float), &scores));
+        const uint64_t q_dim = static_cast<uint64_t>(n_heads) * head_dim;
+        for (uint32_t i = 0; i < n_queries; ++i)
+            CERA_TRY(cera_launch_attn_generic(ctx, q + i * q_dim, kc, vc, n_heads, n_kv_heads, head_dim,
+                                              static_cast<uint32_t>(seq_len) + i, static_cast<uint32_t>(max_seq), scale,
+                                              static_cast<float*>(scores), out + i * q_dim, kv_f16));
+        if (out_quants) {
+            if (q_dim % 32) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "attention: n_heads * head_dim must be a multiple of 32 to quantize the output");
+            CERA_TRY(cera_launch_quantize(ctx, out, q_dim * n_queries, out_scales, out_quants, out_bsum));
+        }
+        return CERA_HIP_OK;
+    }
+    uint32_t G = n_heads / n_kv_heads;
     // seq_len = keys visible to the first query; the last query sees seq_len + n_queries - 1
     const uint64_t last_len = seq_len + n_queries - 1;
     if (seq_len == 0 || last_len > max_seq || max_seq > 0x7FFFFFFFull) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "attention: need 0 < seq_len <= max_seq < 2^31");

@@ -286,7 +286,7 @@ __device__ __forceinline__ void kv_shift_body(const KV* __restrict__ src, KV* __
                                                               uint64_t src_head_stride, uint64_t dst_head_stride,
                                                               const float* __restrict__ delta_cs, uint32_t rope_type) {
     constexpr uint32_t TPR = HD / 8;
-    const uint32_t t = (blockIdx.x * 256 + threadIdx.x) / TPR, j = threadIdx.x % TPR;
+    const uint32_t gi = blockIdx.x * 256 + threadIdx.x, t = gi / TPR, j = gi % TPR;   // TPR need not divide 256
     if (t >= n_rows) return;
     const KV* sp = src + blockIdx.y * src_head_stride + static_cast<uint64_t>(src_row + t) * HD;
     KV* dp = dst + blockIdx.y * dst_head_stride + static_cast<uint64_t>(dst_row + t) * HD;

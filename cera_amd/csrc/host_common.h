@@ -115,6 +115,14 @@ cera_hip_status cera_launch_ffn_gate_up_fused(cera_hip_ctx* ctx, const cera_hip_
                                               bool* launched);
 cera_hip_status cera_launch_qkv_fused(cera_hip_ctx* ctx, const cera_hip_dtensor* wa, const cera_hip_dtensor* wb, const float* x,
                                       const float* norm_w, float eps, float* ya, float* yb, bool* launched);
+// one query, any head_dim % 8 == 0 up to 256, any heads per kv head (reforder.hip); scores: [n_heads][max_seq] floats
+cera_hip_status cera_launch_attn_generic(cera_hip_ctx* ctx, const float* q, const void* kc, const void* vc, uint32_t n_heads,
+                                         uint32_t n_kv_heads, uint32_t head_dim, uint32_t seq_len, uint32_t max_seq, float scale,
+                                         float* scores, float* out, bool kv_f16);
+// whether the tuned attention kernels cover the shape (else cera_launch_attn takes the generic kernel per query)
+static inline bool cera_attn_shape_tuned(uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim) {
+    return (head_dim == 64 || head_dim == 128) && n_kv_heads != 0 && n_heads % n_kv_heads == 0 && n_heads / n_kv_heads <= 8;
+}
 // index of the maximum of x[0, n) into *out_dev (device); uses scratch slot 8 of the context
 // out_host_mapped (nullable): device view of pinned host memory that also receives the index
 cera_hip_status cera_launch_argmax(cera_hip_ctx* ctx, const float* x, uint32_t n, uint32_t* out_dev, uint32_t* out_host_mapped);

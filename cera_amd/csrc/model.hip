@@ -163,7 +163,9 @@ extern "C" cera_hip_status cera_hip_model_create(cera_hip_ctx* ctx, const cera_h
     if (c.n_layers == 0 || c.hidden == 0 || c.ffn == 0 || c.n_heads == 0 || c.n_kv_heads == 0 || c.vocab == 0 ||
         c.max_seq_len == 0)
         return cera_fail(ctx, CERA_HIP_ERR_ARGUMENT, "model_create: zero dimension in config");
-    if (c.head_dim != 64 && c.head_dim != 128) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "model_create: head_dim must be 64 or 128");
+    // head sizes other than 64 / 128 and more than 8 query heads per kv head run on a generic attention kernel
+    if (c.head_dim == 0 || c.head_dim % 8 || c.head_dim > 256)
+        return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "model_create: head_dim must be a multiple of 8, at most 256");
     if (c.n_heads % c.n_kv_heads) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "model_create: n_heads % n_kv_heads != 0");
     if (c.hidden % 32 || c.ffn % 32) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "model_create: hidden and ffn must be multiples of 32");
     if (c.rope_type > 1) return cera_fail(ctx, CERA_HIP_ERR_ARGUMENT, "model_create: rope_type must be 0 (neox) or 1 (norm)");
@@ -387,14 +389,18 @@ extern "C" cera_hip_status cera_hip_shift_kv(cera_hip_model* m, uint32_t n_keep,
                 }
             }
         };
-        using HD128 = std::integral_constant<int, 128>;
-        using HD64 = std::integral_constant<int, 64>;
-        if (c.head_dim == 128) {
-            if (m->kv_f16) run(static_cast<kv_half*>(nullptr), HD128{});
-            else run(static_cast<float*>(nullptr), HD128{});
-        } else {
-            if (m->kv_f16) run(static_cast<kv_half*>(nullptr), HD64{});
-            else run(static_cast<float*>(nullptr), HD64{});
+        auto run_hd = [&](auto hd_tag) {
+            if (m->kv_f16) run(static_cast<kv_half*>(nullptr), hd_tag);
+            else run(static_cast<float*>(nullptr), hd_tag);
+        };
+        switch (c.head_dim) {
+            case 128: run_hd(std::integral_constant<int, 128>{}); break;
+            case 64: run_hd(std::integral_constant<int, 64>{}); break;
+            case 32: run_hd(std::integral_constant<int, 32>{}); break;
+            case 80: run_hd(std::integral_constant<int, 80>{}); break;
+            case 96: run_hd(std::integral_constant<int, 96>{}); break;
+            case 256: run_hd(std::integral_constant<int, 256>{}); break;
+            default: return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "shift_kv: head_dim must be one of 32, 64, 80, 96, 128, 256");
         }
         HIP_TRY(ctx, hipGetLastError());
         HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
@@ -572,7 +578,7 @@ cera_hip_status cera_attn_step(cera_hip_ctx* ctx, float* q, float* k_new, const 
                                uint32_t n_kv_heads, uint32_t head_dim, uint32_t max_seq, uint32_t rope_type, float scale,
                                bool kv_f16, float* out, float* out_scales, int8_t* out_quants) {
     hipStream_t s = ctx->stream;
-    if (pos + 1 < ATTN_FUSED_NEW_KV_MAX_KEYS) {
+    if (pos + 1 < ATTN_FUSED_NEW_KV_MAX_KEYS && cera_attn_shape_tuned(n_heads, n_kv_heads, head_dim)) {
         AttnNewKV nk;
         nk.rope_row = rope_table + static_cast<uint64_t>(pos) * head_dim;
         nk.rope_type = rope_type;

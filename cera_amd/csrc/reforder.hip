@@ -600,6 +600,15 @@ cera_hip_status launch_flash_ref(cera_hip_ctx* ctx, const float* q, const void* 
 
 }  // namespace
 
+// Attention of one query for any head_dim that is a multiple of 8 (at most 256) and any number of
+// query heads per kv head: the kernel of the verification route, which is what the default route
+// runs for shapes its tuned kernels (head_dim 64 / 128, groups of at most 8) do not cover.
+cera_hip_status cera_launch_attn_generic(cera_hip_ctx* ctx, const float* q, const void* kc, const void* vc, uint32_t n_heads,
+                                         uint32_t n_kv_heads, uint32_t head_dim, uint32_t seq_len, uint32_t max_seq, float scale,
+                                         float* scores, float* out, bool kv_f16) {
+    return launch_attn_ref(ctx, q, kc, vc, n_heads, n_kv_heads, head_dim, seq_len, max_seq, scale, scores, out, kv_f16);
+}
+
 // ---------------------------------------------------------------------------
 // LlamaModel::run_layers + project_logits (cera/src/model/llama.rs:468-597) with every
 // operation a launch of its own, in the CPU path's order.

@@ -242,9 +242,13 @@ CERA_HIP_API cera_hip_status cera_hip_gemm_swiglu(cera_hip_ctx*, const cera_hip_
  * [seq_len][n_kv_heads*head_dim] (cera/src/kv_cache.rs:201-212);
  * out f32[n_heads*head_dim]; all seq_len positions visible.
  * n_splits = 0 lets the library choose the split-K factor.
- * head_dim 64 or 128; n_heads a multiple of n_kv_heads, at most 8 query heads per kv head
- * (any count: 28 / 4 and 12 / 2 included); anything else is CERA_HIP_ERR_SHAPE.  The same holds
- * for every attention entry below. */
+ * n_heads a multiple of n_kv_heads.  The tuned kernels cover head_dim 64 and 128 with up to 8
+ * query heads per kv head (any count: 28 / 4 and 12 / 2 included); every other head_dim that is
+ * a multiple of 8 up to 256, and larger groups, run one launch per query of a generic kernel
+ * (the reference takes any shape: transformer.rs:1249-1305, cpu.rs:7075-7088) -- correct, not
+ * tuned, n_splits ignored.  Anything else is CERA_HIP_ERR_SHAPE.  The same holds for every
+ * attention entry below except the fused decode step and the allocation-free entry, which take
+ * the tuned shapes only. */
 CERA_HIP_API cera_hip_status cera_hip_attn_decode(cera_hip_ctx*, const float* q, const float* k, const float* v,
                                                   uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim,
                                                   uint64_t seq_len, float scale, uint32_t n_splits, float* out);

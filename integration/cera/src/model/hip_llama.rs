@@ -412,7 +412,8 @@ impl Model for HipLlamaModel {
     }
 
     fn supports_kv_shift(&self) -> bool {
-        true
+        // the shift kernel is instantiated for the head sizes models use
+        matches!(self.config.head_dim, 32 | 64 | 80 | 96 | 128 | 256)
     }
 
     fn shift_kv(&self, state: &mut InferenceState, n_keep: usize, shift: usize) {

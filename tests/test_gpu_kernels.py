@@ -477,6 +477,38 @@ def test_attn_decode_head_dim_64(hip, orc, kv_f16, nh, nkv, L):
 
 
 # ---- two projections in one launch --------------------------------------------------------
+@pytest.mark.parametrize("kv_f16,nh,nkv,hd,L", [(False, 4, 2, 96, 70), (False, 16, 1, 64, 130), (False, 6, 3, 40, 9), (False, 2, 2, 256, 33),
+                                               (True, 24, 2, 128, 77), (True, 4, 1, 80, 300)])
+def test_attn_decode_other_head_sizes_and_group_sizes(hip, orc, kv_f16, nh, nkv, hd, L):
+    """Head sizes other than 64 / 128 and more than 8 query heads per kv head -- which the reference's
+    decode_attention takes as it takes any shape (cera/src/model/transformer.rs:1249-1305, kernels
+    tested at head_dim 8 ... 256, cera/src/backend/cpu.rs:7075-7088) -- run on the generic kernel:
+    same bar against the oracle as the tuned shapes."""
+    _say(f"attn decode generic shape heads {nh}/{nkv} hd {hd} L {L} f16={kv_f16}")
+    q = util.make_x(nh * hd, 1)
+    k, v = util.make_x(L * nkv * hd, 2), util.make_x(L * nkv * hd, 3)
+    scale = 1.0 / np.sqrt(hd)
+    if kv_f16:
+        k, v = k.astype(np.float16).astype(np.float32), v.astype(np.float16).astype(np.float32)
+        out = hip.attn_f16kv(q, k, v, nh, nkv, hd, L - 1, 1, scale)[0]
+    else:
+        out = hip.attn_decode(q, k, v, nh, nkv, hd, L, scale)
+    ref = orc.decode_attention(q, k, v, nh, nkv, hd, scale, L)
+    assert np.abs(out - ref).max() <= 2e-3 * util.rms(ref)
+
+
+def test_attn_prefill_other_head_sizes(hip, orc):
+    nh, nkv, hd, start, n = 6, 2, 96, 5, 21
+    L = start + n
+    q = util.make_x(n * nh * hd, 4).reshape(n, nh * hd)
+    k, v = util.make_x(L * nkv * hd, 5), util.make_x(L * nkv * hd, 6)
+    scale = 1.0 / np.sqrt(hd)
+    out = hip.attn_prefill(q, k, v, nh, nkv, hd, start, n, scale)
+    for i in (0, 7, n - 1):
+        ref = orc.decode_attention(q[i], k, v, nh, nkv, hd, scale, start + i + 1)
+        assert np.abs(out[i] - ref).max() <= 2e-3 * util.rms(ref), i
+
+
 @pytest.mark.parametrize("ma,mb,k", [(5120, 1024, 4096), (4096, 4096, 4096), (1027, 515, 4096), (6, 3, 3072), (70, 30, 1024)])
 def test_gemv_pair_is_bitwise_the_two_single_launches(hip, orc, ma, mb, k):
     """attn_q|attn_k (Q4_K) and attn_v (Q6_K) of one layer in a single launch: the same kernel

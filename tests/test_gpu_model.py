@@ -191,6 +191,32 @@ def test_greedy_token_is_the_argmax_of_the_same_logits(hip):
         a.close(); b.close()
 
 
+@pytest.mark.parametrize("over", [dict(n_heads=8, n_kv_heads=2, head_dim=96), dict(n_heads=16, n_kv_heads=1, head_dim=64),
+                                  dict(n_heads=8, n_kv_heads=8, head_dim=32, rope_type=0), dict(n_heads=2, n_kv_heads=1, head_dim=256)])
+def test_models_with_other_head_sizes_and_group_sizes(hip, orc, over):
+    """A head size other than 64 / 128, or more than eight query heads per kv head: the model loads,
+    decodes, prefills in a batch and shifts its context, on the generic attention kernel, to the bars
+    of the tuned shapes (f32 and f16 cache)."""
+    cfg = dict(synth.TINY, hidden=256, max_seq_len=96, **over)
+    weights = synth.make_llama(cfg, seed=55 + over["head_dim"], sigma=0.05, norm_jitter=0.1)
+    _say(f"model: heads {cfg['n_heads']}/{cfg['n_kv_heads']} head_dim {cfg['head_dim']}")
+    for f16 in (False, True):
+        gm, om = hip_api.Model(hip, cfg, weights), orc.Llama(cfg, weights)
+        if f16:
+            gm.configure_kv(True); om.set_kv_f16(True)
+        prompt = [int(t) for t in util.rng(8).integers(0, cfg["vocab"], 19)]
+        lg, lo = gm.forward_prefill(prompt, 0), om.forward_prefill_per_token(prompt, 0)
+        for i in range(6):
+            assert _cos(lg, lo) > 0.999 and np.abs(lg - lo).max() <= 0.1 * util.rms(lo), (f16, i, _cos(lg, lo))
+            tok = int(orc_argmax(lo))
+            lg, lo = gm.forward(tok, 19 + i), om.forward(tok, 19 + i)
+        # n_keep shift: drop 5 cells after the first 4, then one more step on both sides
+        gm.shift_kv(4, 5); om.shift_kv(4, 5)
+        lg, lo = gm.forward(3, 20), om.forward(3, 20)
+        assert _cos(lg, lo) > 0.999 and np.abs(lg - lo).max() <= 0.1 * util.rms(lo), (f16, "after shift")
+        gm.close(); om.close()
+
+
 def test_position_contract(tiny):
     cfg, weights, gm, om = tiny
     gm.truncate_kv(0)
