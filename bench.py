@@ -222,7 +222,7 @@ def measure_e2e(seed: int, n_thr: int):
     # short batches (a few new tokens of a chat turn, the verification pass of speculative decoding):
     # all-position logits of n tokens on top of the 512-token context, weights streamed once per pass
     short = []
-    for n_tok in (1, 2, 4, 8):
+    for n_tok in (1, 2, 4, 8, 16, 32):
         toks_n = prompt[:n_tok]
         best = 1e9
         for _ in range(5):

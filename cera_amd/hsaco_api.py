@@ -521,9 +521,9 @@ class Model:
         self.L(f"cera_k_gemm_{GGML_NAMES[t]}", ((n + 63) // 64, (m + 127) // 128, 1), 256, a)
 
     def forward_prefill(self, tokens, start_pos: int) -> np.ndarray:
-        """More than 8 tokens at once (at most 1024 keys in all, hidden and ffn below 2048 so no K split): logits of the last."""
+        """16 tokens or more at once (at most 1024 keys in all, hidden and ffn below 2048 so the tile GEMMs need no K split): logits of the last."""
         n = len(tokens)
-        assert n > 8 and start_pos == self.seq_len and start_pos + n <= min(self.max_seq, 1024) and max(self.hs, self.ffn) < 2048
+        assert n >= 16 and start_pos == self.seq_len and start_pos + n <= min(self.max_seq, 1024) and max(self.hs, self.ffn) < 2048
         self._pf_buffers(n)
         P, e, G = self.pf, self.embd, self.nh // self.nkv
         self.h._ck(self.h.hip.hipMemcpy(C.c_void_p(P["tokens"]), C.c_void_p(np.ascontiguousarray(tokens, np.uint32).ctypes.data),

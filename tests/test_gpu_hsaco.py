@@ -160,11 +160,11 @@ def test_whole_decode_step_from_the_code_object(hip, orc, host):
 
 
 def test_batched_prefill_from_the_code_object(hip, orc, host):
-    """The same host prefills 32 tokens in one pass -- embedding rows, rmsnorm + Q8_0 per row, the
-    fp8 (Q4_K) and f16 (Q6_K) GEMMs with their activation-layout kernels, RoPE + append for the batch,
-    the MFMA prefill attention and its merge, SwiGLU + Q8_0, residual GEMMs -- then decodes on top of
-    the cache it built: logits equal to the library's (same kernels, same launch rules) and close to
-    the oracle's batched route."""
+    """The same host prefills 32 tokens in one pass and then 48 more on top -- embedding rows, rmsnorm +
+    Q8_0 per row, the fp8 (Q4_K) and f16 (Q6_K) GEMMs with their activation-layout kernels, RoPE + append
+    for the batch, the MFMA prefill attention and its merge, SwiGLU + Q8_0, residual GEMMs -- then decodes
+    on top of the cache it built: logits equal to the library's (same kernels, same launch rules) and
+    close to the oracle's batched route."""
     from cera_amd import synth
     cfg = _host_model_cfg()
     weights = synth.make_llama(cfg, seed=78, sigma=0.05, norm_jitter=0.1)
@@ -176,9 +176,13 @@ def test_batched_prefill_from_the_code_object(hip, orc, host):
     a, b, o = hm.forward_prefill(prompt, 0), lib.forward_prefill(prompt, 0), om.forward_prefill_batched(prompt, 0)
     assert np.array_equal(_bits(a), _bits(b)), float(np.abs(a - b).max())
     assert np.abs(a - o).max() <= 0.1 * util.rms(o)
+    more = [int(t) for t in util.rng(4).integers(0, cfg["vocab"], 48)]
+    a, b, o = hm.forward_prefill(more, 32), lib.forward_prefill(more, 32), om.forward_prefill_batched(more, 32)
+    assert np.array_equal(_bits(a), _bits(b)), float(np.abs(a - b).max())
+    assert np.abs(a - o).max() <= 0.1 * util.rms(o)
     tok = int(orc.argmax(b))
     for i in range(4):
-        a, b = hm.forward(tok, 32 + i), lib.forward(tok, 32 + i)
+        a, b = hm.forward(tok, 80 + i), lib.forward(tok, 80 + i)
         assert np.array_equal(_bits(a), _bits(b)), (i, float(np.abs(a - b).max()))
         tok = int(orc.argmax(b))
     lib.close(); om.close()
