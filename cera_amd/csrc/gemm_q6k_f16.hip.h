@@ -59,22 +59,31 @@ static __global__ __launch_bounds__(256) void gemm_act_f16_kernel(const uint4* _
 // byte offset of 16-byte chunk `chunk` of staged row `row`
 __device__ __forceinline__ uint32_t gq_off(uint32_t row, uint32_t chunk) { return row * GQ_LD + (chunk << 4); }
 
-template <bool DBG = false>
+// WIDE = 1: the tile above.  WIDE = 2: 512 threads = 2 x 4 wavefronts on 128 rows x 128 tokens, every
+// wavefront the same 64 x 32 share as before: the weight unpack (a quarter of the narrow tile's vector
+// instructions) is spread over twice the threads for twice the outputs, and a SIMD holds four
+// wavefronts instead of two.  76 KB of LDS a workgroup, still two per CU.
+template <bool DBG = false, int WIDE = 1>
 __device__ __forceinline__ void gemm_q6k_f16_body(GemmArgs p) {
     constexpr int NB = GEMM_KT / 32;
-    __shared__ __attribute__((aligned(16))) uint8_t sA[GEMM_BM * GQ_LD];
-    __shared__ __attribute__((aligned(16))) uint8_t sB[GEMM_BN * GQ_LD];
-    __shared__ __attribute__((aligned(16))) float sRS[2 * NB * GEMM_BM];   // (sc * d) per 16-group per row
-    __shared__ __attribute__((aligned(16))) float sCS[NB * GEMM_BN];
+    constexpr uint32_t BN = GEMM_BN * WIDE, NT = 256 * WIDE;   // tokens per workgroup, threads
+    constexpr int AW = 4 / WIDE;                               // 32-bit words of each code run a thread unpacks
+    // the wide tile has the CU to itself and stages K steps alternately into two buffers: one barrier per
+    // step (a buffer is rewritten two steps later, behind the barrier of the step between)
+    constexpr int NBUF = WIDE;
+    __shared__ __attribute__((aligned(16))) uint8_t sA_[NBUF][GEMM_BM * GQ_LD];
+    __shared__ __attribute__((aligned(16))) uint8_t sB_[NBUF][BN * GQ_LD];
+    __shared__ __attribute__((aligned(16))) float sRS_[NBUF][2 * NB * GEMM_BM];   // (sc * d) per 16-group per row
+    __shared__ __attribute__((aligned(16))) float sCS_[NBUF][NB * BN];
 
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const uint32_t wm = wave >> 1, wn = wave & 1;
+    const uint32_t wm = wave / (2 * WIDE), wn = wave % (2 * WIDE);
     const bool second = p.w2 != nullptr && blockIdx.y >= p.tiles1;
     const uint8_t* const wmat = second ? p.w2 : p.w;
     float* const omat = second ? p.out2 : p.out;
     const uint32_t mrows = second ? p.m2 : p.m;
     const uint64_t ldn = second ? p.ld_n2 : p.ld_n;
-    const uint32_t m0 = (second ? blockIdx.y - p.tiles1 : blockIdx.y) * GEMM_BM, n0 = blockIdx.x * GEMM_BN;
+    const uint32_t m0 = (second ? blockIdx.y - p.tiles1 : blockIdx.y) * GEMM_BM, n0 = blockIdx.x * BN;
     const uint32_t col = lane & 31, half = lane >> 5;
     const uint32_t nb32 = p.k / 32;
 
@@ -84,24 +93,25 @@ __device__ __forceinline__ void gemm_q6k_f16_body(GemmArgs p) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[t][r] = 0.0f;
 
-    // staging assignments, fixed for the whole K loop.  Weight item (row, j): positions 16j .. 16j+15
-    // of the 128-element half, four codes each; threads 0..127 also decode their row's scales.
+    // staging assignments, fixed for the whole K loop.  Weight item (row, j): positions 4 AW j ..
+    // 4 AW (j + 1) - 1 of each 32 of the 128-element half (AW words of ql[l], ql[32 + l] and qh[l]);
+    // threads 0..127 also decode their row's scales.
     // Rows and tokens past the edge are clamped: their products are computed and never stored.
-    const uint32_t a_row = tid >> 1, a_j = tid & 1;
+    const uint32_t a_row = tid / (2 * WIDE), a_j = tid % (2 * WIDE);
     const uint8_t* a_src = wmat + static_cast<uint64_t>(min(m0 + a_row, mrows - 1)) * p.row_bytes;
     const uint8_t* s_src = wmat + static_cast<uint64_t>(min(m0 + (tid & (GEMM_BM - 1)), mrows - 1)) * p.row_bytes;
     const uint8_t* b_src[4];
-    uint8_t* b_dst[4];
+    uint32_t b_dst[4];   // byte offset in sB
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        const uint32_t it = tid + 256 * i, c = it >> 4, wi = it & 15;
+        const uint32_t it = tid + NT * i, c = it >> 4, wi = it & 15;
         b_src[i] = static_cast<const uint8_t*>(p.bh) + static_cast<uint64_t>(min(n0 + c, p.n - 1)) * p.k * 2 + wi * 16;
-        b_dst[i] = sB + gq_off(c, wi);
+        b_dst[i] = gq_off(c, wi);
     }
     const uint32_t c_tok = tid >> 2, c_b = tid & 3;
     const uint64_t c_off = static_cast<uint64_t>(min(n0 + c_tok, p.n - 1)) * nb32 + c_b;
 
-    uint4 qa, qb, qh;   // prefetched codes of the item
+    uint32_t qa[AW], qb[AW], qh[AW];   // prefetched codes of the item
     uint2 rsc;          // the half's eight int8 group scales (threads 0..127)
     uint32_t rd;
     gq_u4 rb[4];
@@ -109,9 +119,19 @@ __device__ __forceinline__ void gemm_q6k_f16_body(GemmArgs p) {
     auto fetch = [&](uint32_t k0) __attribute__((always_inline)) {
         const uint32_t nh = (k0 / GEMM_KT) & 1;
         const uint8_t* blk = a_src + (k0 / 256) * 210;
-        qa = ld_u128_a2(blk + nh * 64 + a_j * 16);
-        qb = ld_u128_a2(blk + nh * 64 + 32 + a_j * 16);
-        qh = ld_u128_a2(blk + 128 + nh * 32 + a_j * 16);
+        if (WIDE == 1) {
+            const uint4 va = ld_u128_a2(blk + nh * 64 + a_j * 16), vb = ld_u128_a2(blk + nh * 64 + 32 + a_j * 16),
+                        vh = ld_u128_a2(blk + 128 + nh * 32 + a_j * 16);
+            qa[0] = va.x; qa[1] = va.y; qa[AW - 2] = va.z; qa[AW - 1] = va.w;
+            qb[0] = vb.x; qb[1] = vb.y; qb[AW - 2] = vb.z; qb[AW - 1] = vb.w;
+            qh[0] = vh.x; qh[1] = vh.y; qh[AW - 2] = vh.z; qh[AW - 1] = vh.w;
+        } else {
+            const uint2 va = ld_u64_a2(blk + nh * 64 + a_j * 8), vb = ld_u64_a2(blk + nh * 64 + 32 + a_j * 8),
+                        vh = ld_u64_a2(blk + 128 + nh * 32 + a_j * 8);
+            qa[0] = va.x; qa[1] = va.y;
+            qb[0] = vb.x; qb[1] = vb.y;
+            qh[0] = vh.x; qh[1] = vh.y;
+        }
         if (tid < GEMM_BM) {
             const uint8_t* sblk = s_src + (k0 / 256) * 210;
             rsc = ld_u64_a2(sblk + 192 + nh * 8);
@@ -126,15 +146,20 @@ __device__ __forceinline__ void gemm_q6k_f16_body(GemmArgs p) {
     const uint32_t k_begin = blockIdx.z * p.k_chunk, k_end = k_begin + p.k_chunk;
     fetch(k_begin);
     for (uint32_t k0 = k_begin; k0 < k_end; k0 += GEMM_KT) {
+        const uint32_t buf = NBUF == 2 ? ((k0 - k_begin) / GEMM_KT) & 1 : 0;
+        uint8_t* const sA = sA_[buf];
+        uint8_t* const sB = sB_[buf];
+        float* const sRS = sRS_[buf];
+        float* const sCS = sCS_[buf];
         // ---- registers -> LDS.  Element 32t + l of the half: low nibble of ql[l] (t = 0), of ql[32 + l]
         // (t = 1), high nibbles of the same (t = 2, 3); bits 2t, 2t+1 of qh[l] are its bits 4, 5.
         {
-            const uint32_t a[4] = {qa.x, qa.y, qa.z, qa.w}, b[4] = {qb.x, qb.y, qb.z, qb.w}, h[4] = {qh.x, qh.y, qh.z, qh.w};
+            const uint32_t *a = qa, *b = qb, *h = qh;
 #pragma unroll
             for (int t = 0; t < 4; ++t) {
-                uint32_t o[8];
+                uint32_t o[2 * AW];
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
+                for (int i = 0; i < AW; ++i) {
                     const uint32_t ql = (t & 1) ? b[i] : a[i];
                     const uint32_t lo = t >= 2 ? ql >> 4 : ql;          // the nibble of bytes 0, 2 at bits 0..3, 16..19
                     const uint32_t n02 = lo & 0x000F000Fu, n13 = (lo >> 8) & 0x000F000Fu;
@@ -144,8 +169,12 @@ __device__ __forceinline__ void gemm_q6k_f16_body(GemmArgs p) {
                     o[2 * i] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(gq_h2, n02 | h02 | 0x64006400u) + recentre);
                     o[2 * i + 1] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(gq_h2, n13 | h13 | 0x64006400u) + recentre);
                 }
-                *reinterpret_cast<gq_u4*>(sA + gq_off(a_row, 4 * t + 2 * a_j)) = gq_u4{o[0], o[1], o[2], o[3]};
-                *reinterpret_cast<gq_u4*>(sA + gq_off(a_row, 4 * t + 2 * a_j + 1)) = gq_u4{o[4], o[5], o[6], o[7]};
+                if (WIDE == 1) {
+                    *reinterpret_cast<gq_u4*>(sA + gq_off(a_row, 4 * t + 2 * a_j)) = gq_u4{o[0], o[1], o[2], o[3]};
+                    *reinterpret_cast<gq_u4*>(sA + gq_off(a_row, 4 * t + 2 * a_j + 1)) = gq_u4{o[2 * AW - 4], o[2 * AW - 3], o[2 * AW - 2], o[2 * AW - 1]};
+                } else {
+                    *reinterpret_cast<gq_u4*>(sA + gq_off(a_row, 4 * t + a_j)) = gq_u4{o[0], o[1], o[2], o[3]};
+                }
             }
         }
         if (tid < GEMM_BM) {
@@ -157,8 +186,8 @@ __device__ __forceinline__ void gemm_q6k_f16_body(GemmArgs p) {
                 sRS[g * GEMM_BM + tid] = d * static_cast<float>(static_cast<int>(static_cast<int8_t>((s[g >> 2] >> (8 * (g & 3))) & 0xFF)));
         }
 #pragma unroll
-        for (int i = 0; i < 4; ++i) *reinterpret_cast<gq_u4*>(b_dst[i]) = rb[i];
-        sCS[c_b * GEMM_BN + c_tok] = rcs;
+        for (int i = 0; i < 4; ++i) *reinterpret_cast<gq_u4*>(sB + b_dst[i]) = rb[i];
+        sCS[c_b * BN + c_tok] = rcs;
         __syncthreads();
         if (k0 + GEMM_KT < k_end) fetch(k0 + GEMM_KT);
 
@@ -166,7 +195,7 @@ __device__ __forceinline__ void gemm_q6k_f16_body(GemmArgs p) {
         const uint32_t bR = wn * 32 + col;
 #pragma unroll
         for (int b = 0; b < NB; ++b) {
-            const float xs = sCS[b * GEMM_BN + wn * 32 + col];
+            const float xs = sCS[b * BN + wn * 32 + col];
             const gq_v8h bf0 = *reinterpret_cast<const gq_v8h*>(sB + gq_off(bR, 4 * b + half));
             const gq_v8h bf1 = *reinterpret_cast<const gq_v8h*>(sB + gq_off(bR, 4 * b + 2 + half));
 #pragma unroll
@@ -202,7 +231,7 @@ __device__ __forceinline__ void gemm_q6k_f16_body(GemmArgs p) {
                 }
             }
         }
-        __syncthreads();
+        if (NBUF == 1) __syncthreads();
     }
     // ---- store: lane holds token n0 + wn*32 + col, rows 8*blk + 4*half + r of each row tile
     const uint32_t tok = n0 + wn * 32 + col;
@@ -223,7 +252,7 @@ __device__ __forceinline__ void gemm_q6k_f16_body(GemmArgs p) {
                 }
     }
 }
-template <bool DBG = false>
-static __global__ __launch_bounds__(256, 2) void gemm_q6k_f16_kernel(GemmArgs p) {
-    gemm_q6k_f16_body<DBG>(p);
+template <bool DBG = false, int WIDE = 1>
+static __global__ __launch_bounds__(256 * WIDE, 2) void gemm_q6k_f16_kernel(GemmArgs p) {
+    gemm_q6k_f16_body<DBG, WIDE>(p);
 }

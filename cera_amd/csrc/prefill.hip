@@ -87,7 +87,11 @@ cera_hip_status cera_launch_gemm(cera_hip_ctx* ctx, const cera_hip_dtensor* w, c
         }
         a.bf8 = static_cast<const uint8_t*>(b8_ws);
     }
-    const uint32_t BM = fp8 ? G8_BM : GEMM_BM, BN = fp8 ? G8_BN : GEMM_BN;
+    // Q6_K: 128-token tiles (eight wavefronts) from 256 tokens on, where they round the token count up by
+    // at most a tenth more than 64-token tiles do
+    const bool q6_wide = w->dtype == CERA_HIP_Q6_K && !dbg_dots && n >= 256 &&
+                         (n + 127) / 128 * 128 * 10 <= (n + 63) / 64 * 64 * 11;
+    const uint32_t BM = fp8 ? G8_BM : GEMM_BM, BN = fp8 ? G8_BN : (q6_wide ? 2 * GEMM_BN : GEMM_BN);
     if (q5) {
         // hi | lo f16 halves of x and its f32 block sums, in one scratch allocation
         const uint64_t nk = static_cast<uint64_t>(n) * a.k;
@@ -122,9 +126,10 @@ cera_hip_status cera_launch_gemm(cera_hip_ctx* ctx, const cera_hip_dtensor* w, c
     uint32_t split = 1;
     const uint32_t wgs = grid.x * grid.y, nsb = a.k / GEMM_KSUPER;
     const bool dense = (ld_m == 1 && ld_n == a.m) || (ld_n == 1 && ld_m == n);
-    if (!dbg_dots && wgs < 2 * ctx->n_cu && nsb >= 8 && dense && (static_cast<uint64_t>(a.m) * n) % 4 == 0) {
-        // smallest divisor of the super-block count that gives at least two workgroups per CU
-        const uint32_t want = std::min<uint32_t>(8, (2 * ctx->n_cu + wgs - 1) / wgs);
+    const uint32_t per_cu = q6_wide ? 1 : 2;   // workgroups a CU holds at once
+    if (!dbg_dots && wgs < per_cu * ctx->n_cu && nsb >= 8 && dense && (static_cast<uint64_t>(a.m) * n) % 4 == 0) {
+        // smallest divisor of the super-block count that fills every CU
+        const uint32_t want = std::min<uint32_t>(8, (per_cu * ctx->n_cu + wgs - 1) / wgs);
         // (a slice keeps at least two super-blocks: below that the tile's prologue outweighs its K loop)
         for (uint32_t d = 2; d <= 8 && split < want; ++d)
             if (nsb % d == 0 && nsb / d >= 2) split = d;
@@ -156,7 +161,10 @@ cera_hip_status cera_launch_gemm(cera_hip_ctx* ctx, const cera_hip_dtensor* w, c
     }
     switch (w->dtype) {
         case CERA_HIP_Q4_K: hipLaunchKernelGGL((gemm_q4k_fp8_kernel<false, false>), grid, dim3(256), 0, ctx->stream, a); break;
-        case CERA_HIP_Q6_K: hipLaunchKernelGGL(gemm_q6k_f16_kernel<false>, grid, dim3(256), 0, ctx->stream, a); break;
+        case CERA_HIP_Q6_K:
+            if (q6_wide) hipLaunchKernelGGL((gemm_q6k_f16_kernel<false, 2>), grid, dim3(512), 0, ctx->stream, a);
+            else hipLaunchKernelGGL(gemm_q6k_f16_kernel<false>, grid, dim3(256), 0, ctx->stream, a);
+            break;
         case CERA_HIP_Q5_K: hipLaunchKernelGGL(gemm_q5k_f16_kernel, grid, dim3(256), 0, ctx->stream, a); break;
         case CERA_HIP_Q4_0: hipLaunchKernelGGL((gemm_kernel<GemmQ4_0>), grid, dim3(256), 0, ctx->stream, a); break;
         case CERA_HIP_Q4_1: hipLaunchKernelGGL((gemm_kernel<GemmQ4_1>), grid, dim3(256), 0, ctx->stream, a); break;
