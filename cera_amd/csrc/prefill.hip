@@ -87,9 +87,10 @@ cera_hip_status cera_launch_gemm(cera_hip_ctx* ctx, const cera_hip_dtensor* w, c
         }
         a.bf8 = static_cast<const uint8_t*>(b8_ws);
     }
-    // Q6_K: 128-token tiles (eight wavefronts) from 256 tokens on, where they round the token count up by
-    // at most a tenth more than 64-token tiles do
-    const bool q6_wide = w->dtype == CERA_HIP_Q6_K && !dbg_dots && n >= 256 &&
+    // Q6_K: 128-token tiles (eight wavefronts) once there is more than one 64-token tile, where they round the
+    // token count up by at most a tenth more than 64-token tiles do (down projection of the 8B shapes: 71 -> 62 us
+    // at 128 tokens, 243 -> 207 at 512, 828 -> 727 at 2048)
+    const bool q6_wide = w->dtype == CERA_HIP_Q6_K && !dbg_dots && n > 64 &&
                          (n + 127) / 128 * 128 * 10 <= (n + 63) / 64 * 64 * 11;
     const uint32_t BM = fp8 ? G8_BM : GEMM_BM, BN = fp8 ? G8_BN : (q6_wide ? 2 * GEMM_BN : GEMM_BN);
     if (q5) {
