@@ -115,17 +115,45 @@ static __global__ void embed_token_kernel(uint32_t dtype, const uint8_t* __restr
 // The f64 sum is a tree instead of the CPU's serial chain: f64 rounding
 // differences (~1e-16 relative) vanish when inv is narrowed to f32 except in
 // astronomically rare double-rounding cases.
-template <bool QUANT>
-__device__ __forceinline__ void rmsnorm_body(const float* __restrict__ x, const float* __restrict__ w,
+// Split-K partial sums that the consumer of the rows adds up itself (PENDING): x_out[e] = (resid[e] +
+// resid_scale *) sum_z part[z * stride + e], e over [rows][n]
+struct RowsPending {
+    const float* part;
+    uint32_t n_split;
+    uint64_t stride;
+    const float* resid;
+    float resid_scale;
+    float* x_out;
+};
+template <bool QUANT, bool PENDING = false>
+__device__ __forceinline__ void rmsnorm_body(const float* x, const float* __restrict__ w,
                                                       uint32_t n, float eps, float* __restrict__ y,
                                                       float* __restrict__ scales, int8_t* __restrict__ quants,
-                                                      float* __restrict__ bsum) {
+                                                      float* __restrict__ bsum, RowsPending pd = RowsPending{}) {
     __shared__ double part[4];
     const float* xr = x + static_cast<uint64_t>(blockIdx.x) * n;
     float* yr = y + static_cast<uint64_t>(blockIdx.x) * n;
     double s = 0.0;
     for (uint32_t i = threadIdx.x * 4; i < n; i += 1024) {
-        float4 v = *reinterpret_cast<const float4*>(xr + i);
+        float4 v;
+        if (PENDING) {
+            // the rows are not summed yet: x = (resid +) sum_z part[z], in gemm_reduce_kernel's order, stored to
+            // x on the way (the second pass below re-reads what this thread wrote)
+            const uint64_t e = static_cast<uint64_t>(blockIdx.x) * n + i;
+            v = *reinterpret_cast<const float4*>(pd.part + e);
+            for (uint32_t z = 1; z < pd.n_split; ++z) {
+                const float4 a = *reinterpret_cast<const float4*>(pd.part + z * pd.stride + e);
+                v.x += a.x; v.y += a.y; v.z += a.z; v.w += a.w;
+            }
+            if (pd.resid) {
+                const float4 r = *reinterpret_cast<const float4*>(pd.resid + e);
+                if (pd.resid_scale != 1.0f) { v.x *= pd.resid_scale; v.y *= pd.resid_scale; v.z *= pd.resid_scale; v.w *= pd.resid_scale; }
+                v.x = r.x + v.x; v.y = r.y + v.y; v.z = r.z + v.z; v.w = r.w + v.w;
+            }
+            *reinterpret_cast<float4*>(pd.x_out + e) = v;
+        } else {
+            v = *reinterpret_cast<const float4*>(xr + i);
+        }
         s += static_cast<double>(v.x) * v.x;
         s += static_cast<double>(v.y) * v.y;
         s += static_cast<double>(v.z) * v.z;
@@ -166,6 +194,14 @@ static __global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __rest
                                                       float* __restrict__ scales, int8_t* __restrict__ quants,
                                                       float* __restrict__ bsum) {
     rmsnorm_body<QUANT>(x, w, n, eps, y, scales, quants, bsum);
+}
+// The same over rows whose split-K partial sums are still pending (pd.x_out == x): one launch instead of the
+// reduction and the norm.
+static __global__ __launch_bounds__(256) void rmsnorm_pending_kernel(const float* x, const float* __restrict__ w, uint32_t n,
+                                                                     float eps, float* __restrict__ y,
+                                                                     float* __restrict__ scales, int8_t* __restrict__ quants,
+                                                                     float* __restrict__ bsum, RowsPending pd) {
+    rmsnorm_body<true, true>(x, w, n, eps, y, scales, quants, bsum, pd);
 }
 
 // Single-pass variant for the decode step (one row, n <= 16384): 1024 threads

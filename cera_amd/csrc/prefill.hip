@@ -37,7 +37,12 @@ cera_hip_status cera_launch_gemm(cera_hip_ctx* ctx, const cera_hip_dtensor* w, c
                                  const float* resid, float resid_scale, const cera_hip_dtensor* w2 = nullptr,
                                  float* out2 = nullptr, uint64_t ld_n2 = 0, bool* paired = nullptr, void* bh_ws = nullptr,
                                  bool* staged = nullptr, int32_t* dbg_dots = nullptr, const float* x_f32 = nullptr,
-                                 bool* staged_f32 = nullptr, void* b8_ws = nullptr, bool* staged8 = nullptr) {
+                                 bool* staged_f32 = nullptr, void* b8_ws = nullptr, bool* staged8 = nullptr,
+                                 RowsPending* pending = nullptr) {
+    // pending (nullable): a caller whose next launch can add split-K partial sums itself (the row norm of
+    // a prefill); when K is split, the reduction launch is left out and *pending says what to add
+    // (n_split = 0: nothing, out is complete)
+    if (pending) *pending = RowsPending{};
     // Q5_K: x_f32 [n][k] are the activations (bs / bq / bsum are not read); *staged_f32 (nullable)
     // says whether the context's split copy still holds exactly these activations
     const bool q5 = gemm_f32_supports(w->dtype, w->k);
@@ -171,7 +176,9 @@ cera_hip_status cera_launch_gemm(cera_hip_ctx* ctx, const cera_hip_dtensor* w, c
         case CERA_HIP_Q4_1: hipLaunchKernelGGL((gemm_kernel<GemmQ4_1>), grid, dim3(256), 0, ctx->stream, a); break;
         default: hipLaunchKernelGGL((gemm_kernel<GemmQ8_0>), grid, dim3(256), 0, ctx->stream, a); break;
     }
-    if (split > 1)   // one launch reduces both matrices of a pair
+    if (split > 1 && pending && !a.w2 && ld_m == 1 && ld_n == a.m)
+        *pending = RowsPending{a.out, split, a.part_stride, resid, resid_scale, out};
+    else if (split > 1)   // one launch reduces both matrices of a pair
         hipLaunchKernelGGL(gemm_reduce_kernel, dim3(static_cast<uint32_t>(((mn + mn2) / 4 + 255) / 256)), dim3(256), 0,
                            ctx->stream, a.out, split, a.part_stride, (mn + mn2) / 4, out, resid, resid_scale, mn / 4, out2);
     HIP_TRY(ctx, hipGetLastError());
@@ -472,18 +479,26 @@ static cera_hip_status prefill_chunk(cera_hip_model* m, const uint32_t* tokens, 
     bool staged8 = false;
     // the f32 activations whose hi / lo split (Q5_K GEMMs) the context's workspace holds now
     const float* split_of = nullptr;
+    // split-K partial sums of pf_hidden that the next row norm adds up (n_split = 0: none)
+    RowsPending pend{};
     auto norm_rows = [&](const float* x, const float* w, float* y) -> cera_hip_status {
         staged = false;
         staged8 = false;
         split_of = nullptr;
-        hipLaunchKernelGGL((rmsnorm_kernel<true>), dim3(n), dim3(256), 0, s, x, w, hs, c.rms_eps, y, m->pf_xs, m->pf_xq,
-                           m->pf_bsum);
+        if (pend.n_split && pend.x_out == x)
+            hipLaunchKernelGGL(rmsnorm_pending_kernel, dim3(n), dim3(256), 0, s, x, w, hs, c.rms_eps, y, m->pf_xs, m->pf_xq,
+                               m->pf_bsum, pend);
+        else
+            hipLaunchKernelGGL((rmsnorm_kernel<true>), dim3(n), dim3(256), 0, s, x, w, hs, c.rms_eps, y, m->pf_xs, m->pf_xq,
+                               m->pf_bsum);
+        pend = RowsPending{};
         HIP_TRY(ctx, hipGetLastError());
         return CERA_HIP_OK;
     };
     // out[n][w->m] (token-major rows) = B . W^T, optionally added onto resid
     // xf: the f32 activations the quantized ones in pf_xs / pf_xq were made from (what a Q5_K matrix reads)
-    auto gemm = [&](const cera_hip_dtensor* w, float* out, const float* resid, const float* xf) -> cera_hip_status {
+    auto gemm = [&](const cera_hip_dtensor* w, float* out, const float* resid, const float* xf,
+                    RowsPending* pending = nullptr) -> cera_hip_status {
         // a short batch streams the weights once per 8 tokens through the multi-token GEMV (an
         // int8-MFMA tile would be mostly empty); its residual add is unscaled
         if ((n <= PREFILL_SMALL_BATCH || !gemm_batched(w->dtype, w->k)) && (!resid || c.residual_scale == 1.0f)) {
@@ -494,7 +509,7 @@ static cera_hip_status prefill_chunk(cera_hip_model* m, const uint32_t* tokens, 
         }
         bool split_held = split_of == xf;
         CERA_TRY(cera_launch_gemm(ctx, w, m->pf_xs, m->pf_xq, m->pf_bsum, n, out, 1, w->m, resid, c.residual_scale, nullptr,
-                                  nullptr, 0, nullptr, m->pf_xh, &staged, nullptr, xf, &split_held, m->pf_x8, &staged8));
+                                  nullptr, 0, nullptr, m->pf_xh, &staged, nullptr, xf, &split_held, m->pf_x8, &staged8, pending));
         if (w->dtype == CERA_HIP_Q5_K) split_of = xf;
         return CERA_HIP_OK;
     };
@@ -550,7 +565,8 @@ static cera_hip_status prefill_chunk(cera_hip_model* m, const uint32_t* tokens, 
         staged = false;   // the attention merge rewrote the quants
         staged8 = false;
         split_of = nullptr;
-        CERA_TRY(gemm(L.o, m->pf_hidden, m->pf_hidden, m->pf_attn));
+        // (the row norm that follows adds the O projection's split-K partial sums itself)
+        CERA_TRY(gemm(L.o, m->pf_hidden, m->pf_hidden, m->pf_attn, &pend));
 
         CERA_TRY(norm_rows(m->pf_hidden, L.ffn_norm, m->pf_normed));
         // gate, up, SwiGLU and the quantization for the down projection in one launch where the
@@ -564,8 +580,10 @@ static cera_hip_status prefill_chunk(cera_hip_model* m, const uint32_t* tokens, 
         staged = false;   // the down projection's activations are new either way
         if (fused) staged8 = false;
         if (fused && cera_gemm_supports(L.down->dtype, L.down->k)) {
+            // (all layers but the last: the next layer's first row norm adds the partial sums)
             CERA_TRY(cera_launch_gemm(ctx, L.down, hs, hq, hb, n, m->pf_hidden, 1, L.down->m, m->pf_hidden, c.residual_scale,
-                                      nullptr, nullptr, 0, nullptr, m->pf_xh, &staged, nullptr, nullptr, nullptr, m->pf_x8, &staged8));
+                                      nullptr, nullptr, 0, nullptr, m->pf_xh, &staged, nullptr, nullptr, nullptr, m->pf_x8, &staged8,
+                                      i + 1 < c.n_layers ? &pend : nullptr));
             staged = false;   // pf_xh / pf_x8 now mirror hq, not pf_xq
             staged8 = false;
             continue;
@@ -583,7 +601,7 @@ static cera_hip_status prefill_chunk(cera_hip_model* m, const uint32_t* tokens, 
             split_of = nullptr;
         }
         staged8 = false;   // pf_xq holds the SwiGLU output now
-        CERA_TRY(gemm(L.down, m->pf_hidden, m->pf_hidden, m->pf_gate));
+        CERA_TRY(gemm(L.down, m->pf_hidden, m->pf_hidden, m->pf_gate, i + 1 < c.n_layers ? &pend : nullptr));
     }
     m->seq_len = start_pos + n;
     if (all_logits) {
