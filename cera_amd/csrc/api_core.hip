@@ -516,6 +516,9 @@ cera_hip_status cera_launch_gemv_nb(cera_hip_ctx* ctx, const cera_hip_dtensor* w
                                     const float* resid, bool* launched) {
     *launched = false;
     if (!is_int8_type(w->dtype) || n_tok == 0) return CERA_HIP_OK;
+    // a decode copy and rows of one pass per lane: the streaming row kernel (same bits)
+    CERA_TRY(cera_launch_row_gemv_nb(ctx, w, xs, xq, xs_stride, xq_stride, n_tok, y, y_stride, resid, launched));
+    if (*launched) return CERA_HIP_OK;
     const uint32_t n_units = static_cast<uint32_t>(w->k / cera_gemv_unit_elems(w->dtype));
     GemvPlan p;
     if (!gemv_plan(static_cast<uint32_t>(w->m), n_units, ctx->n_cu, false, 2, &p) || p.U != 1) return CERA_HIP_OK;
@@ -970,6 +973,8 @@ cera_hip_status cera_hip_gemv_nb(cera_hip_ctx* ctx, const cera_hip_tensor* t, co
         CERA_TRY(cera_hip_upload(ctx, dx, x, n * k * 4));
         // rows are multiples of 32 long, so quantizing the n rows as one vector is row by row
         CERA_TRY(cera_launch_quantize(ctx, static_cast<float*>(dx), n * k, static_cast<float*>(ds), static_cast<int8_t*>(dq)));
+        // as in a model: a matrix tall enough for the streaming multi-token kernel gets its decode copy
+        if (m >= 8192) CERA_TRY(cera_tensor_prepare_stream(ctx, w));
         bool launched = false;
         CERA_TRY(cera_launch_gemv_nb(ctx, w, static_cast<float*>(ds), static_cast<int8_t*>(dq), static_cast<uint32_t>(k / 32),
                                      static_cast<uint32_t>(k), n, static_cast<float*>(dy), static_cast<uint32_t>(m), nullptr,

@@ -348,6 +348,57 @@ cera_hip_status cera_launch_row_gemv_long_add(cera_hip_ctx* ctx, const cera_hip_
     return CERA_HIP_OK;
 }
 
+// y[t][row] (row stride 1, token stride y_stride) = W . x_t (+ resid, same layout) for a few tokens at
+// once from the decode copy: the weights are streamed once per 8 tokens by the one-wavefront-per-row
+// kernel (row_gemv_nb_kernel).  *launched = false when the matrix has no decode copy or its rows take
+// more than one pass per lane: the caller then takes the K-split multi-token kernel on the native bytes.
+cera_hip_status cera_launch_row_gemv_nb(cera_hip_ctx* ctx, const cera_hip_dtensor* w, const float* xs, const int8_t* xq,
+                                        uint32_t xs_stride, uint32_t xq_stride, uint32_t n_tok, float* y, uint32_t y_stride,
+                                        const float* resid, bool* launched) {
+    *launched = false;
+    if (!w->dev_stream || short_tiles(w->dtype, w->k) != 1 || n_tok == 0 || w->m > (1u << 24)) return CERA_HIP_OK;
+    // Measured on the 8B shapes at 8 tokens against the K-split kernel: gate / up 14336 x 4096 23.1 -> 19.1 us, the
+    // 128256 x 4096 head 157 -> 127 us; the 4096- and 1024-row matrices are too few workgroups of 32 rows to gain
+    // (O 13.2 -> 11.8 us, V 6.4 -> 12.2 us).  Both are bound by the vector ALU's work per (row, token) pair.
+    // (no residual form: the matrices that gain are projections out of the hidden size, not into it)
+    if (w->m < 8192 || resid) return CERA_HIP_OK;
+    constexpr int NW = 8, ROWS = 4;
+    RowGemvNbArgs a{};
+    a.w = w->dev_stream;
+    a.m = static_cast<uint32_t>(w->m);
+    a.k = static_cast<uint32_t>(w->k);
+    a.row_bytes = static_cast<uint32_t>(w->stream_row_bytes);
+    a.xq_stride = xq_stride;
+    a.xs_stride = xs_stride;
+    a.y_stride = y_stride;
+    const dim3 grid((a.m + NW * ROWS - 1) / (NW * ROWS)), block(64 * NW);
+    for (uint32_t t0 = 0; t0 < n_tok; t0 += 8) {
+        const uint32_t nt = std::min(8u, n_tok - t0);
+        a.n_tok = nt;
+        a.xq = xq + static_cast<uint64_t>(t0) * xq_stride;
+        a.xs = xs + static_cast<uint64_t>(t0) * xs_stride;
+        a.y = y + static_cast<uint64_t>(t0) * y_stride;
+        a.resid = nullptr;
+#define NB_LAUNCH_N(TT, NBV) hipLaunchKernelGGL((row_gemv_nb_kernel<TT, NW, ROWS, FEPI_STORE, true, NBV>), grid, block, 0, ctx->stream, a)
+#define NB_LAUNCH(TT)                       \
+    do {                                    \
+        if (nt <= 2) NB_LAUNCH_N(TT, 2);    \
+        else if (nt <= 4) NB_LAUNCH_N(TT, 4); \
+        else NB_LAUNCH_N(TT, 8);            \
+    } while (0)
+        if (w->dtype == CERA_HIP_Q4_K) NB_LAUNCH(Q4K);
+        else if (w->dtype == CERA_HIP_Q6_K) NB_LAUNCH(Q6K);
+        else if (w->dtype == CERA_HIP_Q4_0) NB_LAUNCH(Q4_0);
+        else if (w->dtype == CERA_HIP_Q4_1) NB_LAUNCH(Q4_1);
+        else NB_LAUNCH(Q8_0);
+#undef NB_LAUNCH
+#undef NB_LAUNCH_N
+        HIP_TRY(ctx, hipGetLastError());
+    }
+    *launched = true;
+    return CERA_HIP_OK;
+}
+
 // ---- kernel-level entry points (host buffers) --------------------------------------------------
 extern "C" cera_hip_status cera_hip_ffn_gate_up_fused(cera_hip_ctx* ctx, const cera_hip_tensor* gate, const cera_hip_tensor* up,
                                                       const float* x, const float* norm_w, float eps, int8_t* quants,

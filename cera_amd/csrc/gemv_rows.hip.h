@@ -317,6 +317,95 @@ static __global__ __launch_bounds__(64 * NW) void row_gemv_long_kernel(RowGemvAr
     row_gemv_long_body<T, NW, TILES, EPI, STREAM>(p, s_xq, s_xs);
 }
 
+// ---- a few tokens per weight pass ---------------------------------------------------------------
+// The row kernel above for 2..NB activation vectors at once (short batches: a few new tokens,
+// speculative-decoding verification): a wavefront streams its rows once and dots each with every
+// token's activations.  Eight tokens' prepared activations (T::Act, 22-24 registers each) do not
+// fit a lane's registers at an occupancy that keeps the vector ALU busy, so the workgroup prepares
+// them once -- wavefront w the tokens w, w + NW, ... -- and parks them in LDS as dword planes
+// [token][dword][lane]; a lane reads its own unit's copy back for every (row, token) pair,
+// conflict-free.  Same units per lane, same T::load_act, T::dot and wave_sum as the single-vector
+// kernels, so column b of the result has the bits of a single-vector launch on token b.  One pass
+// per lane (k <= 64 units).
+struct RowGemvNbArgs {
+    const uint8_t* w;       // [m] rows (STREAM: of the decode copy)
+    uint32_t m, k, row_bytes;
+    const int8_t* xq;       // [n_tok][xq_stride]
+    const float* xs;        // [n_tok][xs_stride]
+    uint32_t xq_stride, xs_stride;
+    uint32_t n_tok;         // live tokens, 1 <= n_tok <= NB (surplus columns repeat the last token and are not stored)
+    float* y;               // y[b * y_stride + row]
+    const float* resid;     // ADD: same layout as y
+    uint32_t y_stride;
+};
+
+template <class T, int NW, int ROWS, int EPI, bool STREAM, int NB>
+__device__ __forceinline__ void row_gemv_nb_body(const RowGemvNbArgs& p, uint32_t* s_act) {
+    static_assert(ROWS * NB <= 64, "lane i of a wavefront finishes (row, token) pair i");
+    constexpr int NA = sizeof(typename T::Act) / 4;
+    static_assert(sizeof(typename T::Act) % 4 == 0, "the prepared activations are parked as dwords");
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t n_units = p.k / T::ELEMS_PER_UNIT;
+    const bool live = lane < n_units;
+    const uint32_t unit[1] = {live ? lane : 0};   // dead lanes re-read unit 0 with zeroed activations
+    constexpr int DEPTH = ROWS < 2 ? ROWS : 2;
+    const uint32_t r0 = (blockIdx.x * NW + wave) * ROWS;
+    RowGemvArgs g{};
+    g.w = p.w; g.m = p.m; g.k = p.k; g.row_bytes = p.row_bytes;
+    RowTile<T, 1, STREAM, 1> t[DEPTH];
+#pragma unroll
+    for (int i = 0; i < DEPTH; ++i) t[i].load(g, unit, min(r0 + i, p.m - 1));   // rows past the end re-read the last row
+    __builtin_amdgcn_sched_barrier(0);
+    for (uint32_t b = wave; b < NB; b += NW) {   // wavefront-uniform
+        const uint32_t tok = min(b, p.n_tok - 1);
+        typename T::Act a;
+        T::load_act(a, p.xq + static_cast<uint64_t>(tok) * p.xq_stride, p.xs + static_cast<uint64_t>(tok) * p.xs_stride, unit[0], live);
+        uint32_t raw[NA];
+        __builtin_memcpy(raw, &a, sizeof(a));
+#pragma unroll
+        for (int d = 0; d < NA; ++d) s_act[(b * NA + d) * 64 + lane] = raw[d];
+    }
+    lds_barrier();
+    float mine = 0.0f;   // lane i: the total of row i / NB, token i % NB
+#pragma unroll
+    for (int i = 0; i < ROWS; ++i) {
+        float part[NB];
+#pragma unroll
+        for (int b = 0; b < NB; ++b) {
+            uint32_t raw[NA];
+#pragma unroll
+            for (int d = 0; d < NA; ++d) raw[d] = s_act[(b * NA + d) * 64 + lane];
+            typename T::Act a;
+            __builtin_memcpy(&a, raw, sizeof(a));
+            part[b] = T::dot(t[i % DEPTH].w[0][0], a, unit[0], nullptr);
+            // two tokens' activations in registers at a time: left alone, the scheduler requests all NB
+            // tokens' LDS reads first (200+ registers, or spills under a cap)
+            if (NB >= 4 && (b & 1)) __builtin_amdgcn_sched_barrier(0);
+        }
+        if (i + DEPTH < ROWS) {   // the buffer is free as soon as its dots are formed
+            __builtin_amdgcn_sched_barrier(0);
+            t[i % DEPTH].load_one(g, 0, unit, min(r0 + i + DEPTH, p.m - 1));
+            __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int b = 0; b < NB; ++b) {
+            const float tot = wave_sum(part[b]);
+            if (lane == static_cast<uint32_t>(i * NB + b)) mine = tot;
+        }
+    }
+    const uint32_t row = r0 + lane / NB, b = lane % NB;
+    if (lane < ROWS * NB && row < p.m && b < p.n_tok) {
+        const uint64_t at = static_cast<uint64_t>(b) * p.y_stride + row;
+        p.y[at] = EPI == FEPI_ADD ? p.resid[at] + mine : mine;
+    }
+}
+
+template <class T, int NW, int ROWS, int EPI, bool STREAM, int NB>
+static __global__ __launch_bounds__(64 * NW, 4) void row_gemv_nb_kernel(RowGemvNbArgs p) {
+    __shared__ uint32_t s_act[NB * (sizeof(typename T::Act) / 4) * 64];
+    row_gemv_nb_body<T, NW, ROWS, EPI, STREAM, NB>(p, s_act);
+}
+
 // ---- decode copies ------------------------------------------------------------------------------
 // One thread per unit of a row: the unit's bytes from the native block layout to their places in
 // the decode copy (T::to_stream).  grid = m workgroups of 256 threads.

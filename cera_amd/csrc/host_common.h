@@ -104,6 +104,9 @@ cera_hip_status cera_launch_row_gemv_long_add(cera_hip_ctx* ctx, const cera_hip_
 cera_hip_status cera_launch_gemv_nb(cera_hip_ctx* ctx, const cera_hip_dtensor* w, const float* xs, const int8_t* xq,
                                     uint32_t xs_stride, uint32_t xq_stride, uint32_t n_tok, float* y, uint32_t y_stride,
                                     const float* resid, bool* launched);
+cera_hip_status cera_launch_row_gemv_nb(cera_hip_ctx* ctx, const cera_hip_dtensor* w, const float* xs, const int8_t* xq,
+                                    uint32_t xs_stride, uint32_t xq_stride, uint32_t n_tok, float* y, uint32_t y_stride,
+                                    const float* resid, bool* launched);
 cera_hip_status cera_launch_gemv_pair(cera_hip_ctx* ctx, const cera_hip_dtensor* wa, const cera_hip_dtensor* wb,
                                       const float* xs, const int8_t* xq, float* ya, float* yb, bool* launched);
 // Decode projections with the neighbouring small kernels folded in (gemv_fused.hip); *launched =

@@ -180,7 +180,9 @@ CERA_HIP_API cera_hip_status cera_hip_gemv(cera_hip_ctx*, const cera_hip_tensor*
  * the weights streamed once per 8 vectors: what the prefill path runs instead of the int8 GEMM
  * while a batch is at most 16 tokens (a few new tokens of a chat turn, the verification pass of
  * speculative decoding, cera/src/model/mod.rs:221-249).  Row t of y is bit-identical to
- * cera_hip_gemv on x[t].  CERA_HIP_ERR_UNSUPPORTED_DTYPE for Q5_K and for k beyond one unit per
+ * cera_hip_gemv on x[t].  A matrix of 8192 rows or more is given its decode copy first and read
+ * through the one-wavefront-per-row form, as a model's gate / up / head matrices are (same bits).
+ * CERA_HIP_ERR_UNSUPPORTED_DTYPE for Q5_K and for k beyond one unit per
  * lane (k > 16384; Q4_K and Q6_K 32768). */
 CERA_HIP_API cera_hip_status cera_hip_gemv_nb(cera_hip_ctx*, const cera_hip_tensor* w, const float* x, uint32_t n,
                                               float* y);

@@ -543,7 +543,8 @@ def test_gemv_pair_refuses_what_it_has_no_instance_for(hip):
 def test_gemv_multi_token_is_bitwise_per_token_gemv(hip, orc, dtype, n):
     """Short batches go through the multi-token GEMV: every row of the result equals the
     single-vector kernel on that token bit for bit, for every K-split width."""
-    for m, k in [(37, 256), (130, 4096), (9, 14336), (260, 1024)]:
+    # 8200 rows: tall enough for the one-wavefront-per-row multi-token kernel over the decode copy
+    for m, k in [(37, 256), (130, 4096), (9, 14336), (260, 1024), (8200, 512)]:
         _say(f"gemv_nb {util.NAMES[dtype]} n={n} m={m} k={k}")
         w, _ = util.make_weights(dtype, m, k, seed=dtype * 31 + n)
         x = util.rng(900 + n).standard_normal((n, k)).astype(np.float32)
