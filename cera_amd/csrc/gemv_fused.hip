@@ -357,12 +357,13 @@ cera_hip_status cera_launch_row_gemv_nb(cera_hip_ctx* ctx, const cera_hip_dtenso
                                         const float* resid, bool* launched) {
     *launched = false;
     if (!w->dev_stream || short_tiles(w->dtype, w->k) != 1 || n_tok == 0 || w->m > (1u << 24)) return CERA_HIP_OK;
-    // Measured on the 8B shapes at 8 tokens against the K-split kernel: gate / up 14336 x 4096 23.1 -> 19.1 us, the
-    // 128256 x 4096 head 157 -> 127 us; the 4096- and 1024-row matrices are too few workgroups of 32 rows to gain
-    // (O 13.2 -> 11.8 us, V 6.4 -> 12.2 us).  Both are bound by the vector ALU's work per (row, token) pair.
+    // Measured on the 8B shapes at 8 tokens against the K-split kernel: gate / up 14336 x 4096 23.1 -> 17.3 us, the
+    // 128256 x 4096 head 157 -> 115 us; the 4096- and 1024-row matrices are too few workgroups of 32 rows to gain
+    // (O 13.2 -> 11.8 us, V 6.4 -> 12.2 us).  Both are bound by the vector ALU's work per (row, token) pair
+    // (this kernel: 1073 vector instructions per wavefront for 16 pairs, 16 of each pair's ~55 the v_dot4).
     // (no residual form: the matrices that gain are projections out of the hidden size, not into it)
     if (w->m < 8192 || resid) return CERA_HIP_OK;
-    constexpr int NW = 8, ROWS = 4;
+    constexpr int NW = 8, ROWS = 4;   // two rows per wavefront measured the same
     RowGemvNbArgs a{};
     a.w = w->dev_stream;
     a.m = static_cast<uint32_t>(w->m);

@@ -322,9 +322,9 @@ static __global__ __launch_bounds__(64 * NW) void row_gemv_long_kernel(RowGemvAr
 // speculative-decoding verification): a wavefront streams its rows once and dots each with every
 // token's activations.  Eight tokens' prepared activations (T::Act, 22-24 registers each) do not
 // fit a lane's registers at an occupancy that keeps the vector ALU busy, so the workgroup prepares
-// them once -- wavefront w the tokens w, w + NW, ... -- and parks them in LDS as dword planes
-// [token][dword][lane]; a lane reads its own unit's copy back for every (row, token) pair,
-// conflict-free.  Same units per lane, same T::load_act, T::dot and wave_sum as the single-vector
+// them once -- wavefront w the tokens w, w + NW, ... -- and parks them in LDS as 16-byte planes
+// [token][quad][lane]; a lane reads its own unit's copy back for every (row, token) pair with
+// ds_read_b128, conflict-free (as dword planes the kernel was bound by the LDS instruction rate).  Same units per lane, same T::load_act, T::dot and wave_sum as the single-vector
 // kernels, so column b of the result has the bits of a single-vector launch on token b.  One pass
 // per lane (k <= 64 units).
 struct RowGemvNbArgs {
@@ -340,9 +340,9 @@ struct RowGemvNbArgs {
 };
 
 template <class T, int NW, int ROWS, int EPI, bool STREAM, int NB>
-__device__ __forceinline__ void row_gemv_nb_body(const RowGemvNbArgs& p, uint32_t* s_act) {
+__device__ __forceinline__ void row_gemv_nb_body(const RowGemvNbArgs& p, uint4* s_act) {
     static_assert(ROWS * NB <= 64, "lane i of a wavefront finishes (row, token) pair i");
-    constexpr int NA = sizeof(typename T::Act) / 4;
+    constexpr int NA = sizeof(typename T::Act) / 4, NQ = (NA + 3) / 4;   // dwords, 16-byte quads (the last one padded)
     static_assert(sizeof(typename T::Act) % 4 == 0, "the prepared activations are parked as dwords");
     const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const uint32_t n_units = p.k / T::ELEMS_PER_UNIT;
@@ -360,10 +360,10 @@ __device__ __forceinline__ void row_gemv_nb_body(const RowGemvNbArgs& p, uint32_
         const uint32_t tok = min(b, p.n_tok - 1);
         typename T::Act a;
         T::load_act(a, p.xq + static_cast<uint64_t>(tok) * p.xq_stride, p.xs + static_cast<uint64_t>(tok) * p.xs_stride, unit[0], live);
-        uint32_t raw[NA];
+        uint32_t raw[4 * NQ] = {};
         __builtin_memcpy(raw, &a, sizeof(a));
 #pragma unroll
-        for (int d = 0; d < NA; ++d) s_act[(b * NA + d) * 64 + lane] = raw[d];
+        for (int q = 0; q < NQ; ++q) s_act[(b * NQ + q) * 64 + lane] = make_uint4(raw[4 * q], raw[4 * q + 1], raw[4 * q + 2], raw[4 * q + 3]);
     }
     lds_barrier();
     float mine = 0.0f;   // lane i: the total of row i / NB, token i % NB
@@ -372,9 +372,12 @@ __device__ __forceinline__ void row_gemv_nb_body(const RowGemvNbArgs& p, uint32_
         float part[NB];
 #pragma unroll
         for (int b = 0; b < NB; ++b) {
-            uint32_t raw[NA];
+            uint32_t raw[4 * NQ];
 #pragma unroll
-            for (int d = 0; d < NA; ++d) raw[d] = s_act[(b * NA + d) * 64 + lane];
+            for (int q = 0; q < NQ; ++q) {
+                const uint4 v = s_act[(b * NQ + q) * 64 + lane];
+                raw[4 * q] = v.x; raw[4 * q + 1] = v.y; raw[4 * q + 2] = v.z; raw[4 * q + 3] = v.w;
+            }
             typename T::Act a;
             __builtin_memcpy(&a, raw, sizeof(a));
             part[b] = T::dot(t[i % DEPTH].w[0][0], a, unit[0], nullptr);
@@ -402,7 +405,7 @@ __device__ __forceinline__ void row_gemv_nb_body(const RowGemvNbArgs& p, uint32_
 
 template <class T, int NW, int ROWS, int EPI, bool STREAM, int NB>
 static __global__ __launch_bounds__(64 * NW, 4) void row_gemv_nb_kernel(RowGemvNbArgs p) {
-    __shared__ uint32_t s_act[NB * (sizeof(typename T::Act) / 4) * 64];
+    __shared__ __attribute__((aligned(16))) uint4 s_act[NB * ((sizeof(typename T::Act) / 4 + 3) / 4) * 64];
     row_gemv_nb_body<T, NW, ROWS, EPI, STREAM, NB>(p, s_act);
 }
 
