@@ -176,7 +176,9 @@ cera_hip_status cera_launch_gemm(cera_hip_ctx* ctx, const cera_hip_dtensor* w, c
         case CERA_HIP_Q4_1: hipLaunchKernelGGL((gemm_kernel<GemmQ4_1>), grid, dim3(256), 0, ctx->stream, a); break;
         default: hipLaunchKernelGGL((gemm_kernel<GemmQ8_0>), grid, dim3(256), 0, ctx->stream, a); break;
     }
-    if (split > 1 && pending && !a.w2 && ld_m == 1 && ld_n == a.m)
+    // (from 128 rows on: the norm runs one workgroup per row, and a few dozen workgroups adding up partial sums take
+    // longer than the reduction launch they save -- 12.8 against 4.8 + 5.7 us at 16 rows, 11.3 against 6.3 + 7.4 at 512)
+    if (split > 1 && pending && n >= 128 && !a.w2 && ld_m == 1 && ld_n == a.m)
         *pending = RowsPending{a.out, split, a.part_stride, resid, resid_scale, out};
     else if (split > 1)   // one launch reduces both matrices of a pair
         hipLaunchKernelGGL(gemm_reduce_kernel, dim3(static_cast<uint32_t>(((mn + mn2) / 4 + 255) / 256)), dim3(256), 0,
