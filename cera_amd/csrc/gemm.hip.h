@@ -83,6 +83,9 @@ struct GemmArgs {
     int32_t* dbg_dots;
     // fp8 kernel (gemm_fp8.hip.h) only: the activations' fragment-ordered split copy
     const uint8_t* bf8;
+    // SwiGLU form of the fp8 kernel, nullable: the same quants also as f16 [n][m] in the order
+    // gemm_act_f16_kernel writes them (what a Q6_K down projection reads: saves that launch)
+    uint16_t* hh;
 };
 
 // ---- per-type staging of one 128-element K tile of one row -------------------

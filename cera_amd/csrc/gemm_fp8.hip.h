@@ -456,22 +456,31 @@ __device__ __forceinline__ void gemm_q4k_fp8_body(GemmArgs p) {
             const float id = (d != 0.0f && fabsf(r) != __builtin_inff() && r == r) ? r : 0.0f;
             const float scale = h2f(f2h(d));
             uint32_t packed[4];
+            uint2 halves[4];   // the same four quants as f16, in gemm_act_f16_kernel's order 0, 2, 1, 3
             int sum = 0;
 #pragma unroll
             for (int blk = 0; blk < 4; ++blk) {
                 packed[blk] = 0;
+                uint32_t hb[4];
 #pragma unroll
                 for (int q = 0; q < 4; ++q) {
                     const int v = q8_round(hv[4 * blk + q], id);
                     sum += v;
                     packed[blk] |= (static_cast<uint32_t>(v) & 0xFF) << (8 * q);
+                    hb[q] = f2h(static_cast<float>(v));   // |v| <= 127: exact
                 }
+                halves[blk] = make_uint2(hb[0] | (hb[2] << 16), hb[1] | (hb[3] << 16));
             }
             sum += __shfl_xor(sum, 32, 64);
             if (tok < p.n && row0 < mrows) {   // m % 32 == 0: the block is whole or absent
 #pragma unroll
                 for (int blk = 0; blk < 4; ++blk)
                     *reinterpret_cast<uint32_t*>(p.hq + static_cast<uint64_t>(tok) * mrows + row0 + 8 * blk + 4 * half) = packed[blk];
+                if (p.hh) {
+#pragma unroll
+                    for (int blk = 0; blk < 4; ++blk)
+                        *reinterpret_cast<uint2*>(p.hh + static_cast<uint64_t>(tok) * mrows + row0 + 8 * blk + 4 * half) = halves[blk];
+                }
                 if (half == 0) {
                     const uint64_t b = static_cast<uint64_t>(tok) * (mrows / 32) + row0 / 32;
                     p.hs[b] = scale;

@@ -57,7 +57,7 @@ cera_hip_status cera_launch_gemm(cera_hip_ctx* ctx, const cera_hip_dtensor* w, c
     a.m = static_cast<uint32_t>(w->m); a.n = n; a.k = static_cast<uint32_t>(w->k);
     a.row_bytes = static_cast<uint32_t>(w->row_bytes);
     a.ld_m = ld_m; a.ld_n = ld_n; a.resid = resid; a.resid_scale = resid_scale;
-    a.hq = nullptr; a.hs = nullptr; a.hbsum = nullptr; a.dbg_dots = dbg_dots;
+    a.hq = nullptr; a.hs = nullptr; a.hbsum = nullptr; a.hh = nullptr; a.dbg_dots = dbg_dots;
     // Q6_K runs its block dots on the f16 matrix cores and reads the quants as f16: converted here
     // unless the caller says its workspace (bh_ws) still holds these activations (*staged)
     a.bh = nullptr;
@@ -193,7 +193,9 @@ cera_hip_status cera_launch_gemm(cera_hip_ctx* ctx, const cera_hip_dtensor* w, c
 // need a K split to fill the chip; the caller then takes the GEMM pair and the SwiGLU kernel.
 cera_hip_status cera_launch_gemm_swiglu(cera_hip_ctx* ctx, const cera_hip_dtensor* gate, const cera_hip_dtensor* up,
                                         const float* bs, const int8_t* bq, const float* bsum, uint32_t n, int8_t* hq,
-                                        float* hs, float* hbsum, bool* fused, void* b8_ws = nullptr, bool* staged8 = nullptr) {
+                                        float* hs, float* hbsum, bool* fused, void* b8_ws = nullptr, bool* staged8 = nullptr,
+                                        void* hh_ws = nullptr) {
+    // hh_ws (nullable, Q4_K pairs only): also receives the quants as f16 [n][m] in gemm_act_f16_kernel's order
     *fused = false;
     if (!cera_gemm_supports(gate->dtype, gate->k) || gate->dtype == CERA_HIP_Q6_K || up->dtype != gate->dtype ||
         up->k != gate->k || up->m != gate->m || up->row_bytes != gate->row_bytes || gate->m % 32 || n == 0)
@@ -205,6 +207,7 @@ cera_hip_status cera_launch_gemm_swiglu(cera_hip_ctx* ctx, const cera_hip_dtenso
     a.k_chunk = a.k;
     a.hq = hq; a.hs = hs; a.hbsum = hbsum;
     const bool fp8 = gate->dtype == CERA_HIP_Q4_K;
+    a.hh = fp8 ? static_cast<uint16_t*>(hh_ws) : nullptr;
     const uint32_t BM = fp8 ? G8_BM : GEMM_BM, BN = fp8 ? G8_BN : GEMM_BN;
     const dim3 grid((n + BN - 1) / BN, (a.m + BM / 2 - 1) / (BM / 2));
     if (grid.x * grid.y < 2 * ctx->n_cu) return CERA_HIP_OK;
@@ -356,8 +359,10 @@ extern "C" cera_hip_status cera_hip_gemm_pair(cera_hip_ctx* ctx, const cera_hip_
     return st;
 }
 
-extern "C" cera_hip_status cera_hip_gemm_swiglu(cera_hip_ctx* ctx, const cera_hip_tensor* tg, const cera_hip_tensor* tu,
-                                                const float* x, uint64_t n, int8_t* quants, float* scales, int* fused_out) {
+// halves (nullable, host [n][m] uint16): the quants once more as the f16 words a Q6_K down projection reads
+static cera_hip_status gemm_swiglu_host(cera_hip_ctx* ctx, const cera_hip_tensor* tg, const cera_hip_tensor* tu,
+                                        const float* x, uint64_t n, int8_t* quants, float* scales, uint16_t* halves,
+                                        int* fused_out) {
     if (!ctx || !tg || !tu || !x || !quants || !scales) return CERA_HIP_ERR_ARGUMENT;
     std::lock_guard<std::recursive_mutex> op_lk(ctx->op_mu);
     if (n == 0 || n > 0x7FFFFFFFull) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "gemm_swiglu: bad n");
@@ -384,9 +389,13 @@ extern "C" cera_hip_status cera_hip_gemm_swiglu(cera_hip_ctx* ctx, const cera_hi
         CERA_TRY(quantize_rows(ctx, static_cast<float*>(dx), n, k, static_cast<float*>(ds), static_cast<int8_t*>(dq),
                                static_cast<float*>(db)));
         bool fused = false;
+        void* hh = nullptr;
+        if (halves) CERA_TRY(cera_scratch(ctx, 10, n * mm * 2, &hh));
+        // (a Q4_K pair's epilogue writes the f16 words itself; every other route converts the quants afterwards)
+        const bool hh_in_epilogue = halves && wg->dtype == CERA_HIP_Q4_K;
         CERA_TRY(cera_launch_gemm_swiglu(ctx, wg, wu, static_cast<float*>(ds), static_cast<int8_t*>(dq), static_cast<float*>(db),
                                          static_cast<uint32_t>(n), static_cast<int8_t*>(hq), static_cast<float*>(hs),
-                                         static_cast<float*>(hb), &fused));
+                                         static_cast<float*>(hb), &fused, nullptr, nullptr, hh_in_epilogue ? hh : nullptr));
         if (!fused) {   // the forward pass's other route: the two GEMMs, then the SwiGLU + quantize kernel
             CERA_TRY(cera_launch_gemm(ctx, wg, static_cast<float*>(ds), static_cast<int8_t*>(dq), static_cast<float*>(db),
                                       static_cast<uint32_t>(n), static_cast<float*>(dg), 1, mm, nullptr, 1.0f));
@@ -399,6 +408,16 @@ extern "C" cera_hip_status cera_hip_gemm_swiglu(cera_hip_ctx* ctx, const cera_hi
             HIP_TRY(ctx, hipGetLastError());
         }
         if (fused_out) *fused_out = fused ? 1 : 0;
+        if (halves) {
+            if (!(fused && hh_in_epilogue)) {
+                if ((n * mm) % 16) return cera_fail(ctx, CERA_HIP_ERR_SHAPE, "gemm_swiglu: n * m must be a multiple of 16 for the f16 form");
+                const uint64_t words = n * mm / 16;
+                hipLaunchKernelGGL(gemm_act_f16_kernel, dim3(static_cast<uint32_t>((words + 255) / 256)), dim3(256), 0, ctx->stream,
+                                   static_cast<const uint4*>(hq), static_cast<uint4*>(hh), words);
+                HIP_TRY(ctx, hipGetLastError());
+            }
+            CERA_TRY(cera_hip_download(ctx, halves, hh, n * mm * 2));
+        }
         CERA_TRY(cera_hip_download(ctx, quants, hq, n * mm));
         return cera_hip_download(ctx, scales, hs, n * (mm / 32) * 4);
     };
@@ -406,6 +425,18 @@ extern "C" cera_hip_status cera_hip_gemm_swiglu(cera_hip_ctx* ctx, const cera_hi
     cera_hip_tensor_free(ctx, wg);
     cera_hip_tensor_free(ctx, wu);
     return st;
+}
+
+extern "C" cera_hip_status cera_hip_gemm_swiglu(cera_hip_ctx* ctx, const cera_hip_tensor* tg, const cera_hip_tensor* tu,
+                                                const float* x, uint64_t n, int8_t* quants, float* scales, int* fused_out) {
+    return gemm_swiglu_host(ctx, tg, tu, x, n, quants, scales, nullptr, fused_out);
+}
+
+extern "C" cera_hip_status cera_hip_gemm_swiglu_f16(cera_hip_ctx* ctx, const cera_hip_tensor* tg, const cera_hip_tensor* tu,
+                                                    const float* x, uint64_t n, int8_t* quants, float* scales,
+                                                    uint16_t* halves, int* fused_out) {
+    if (!halves) return CERA_HIP_ERR_ARGUMENT;
+    return gemm_swiglu_host(ctx, tg, tu, x, n, quants, scales, halves, fused_out);
 }
 
 // ---------------------------------------------------------------------------
@@ -577,9 +608,12 @@ static cera_hip_status prefill_chunk(cera_hip_model* m, const uint32_t* tokens, 
         bool fused = false;
         int8_t* const hq = reinterpret_cast<int8_t*>(m->pf_gate);
         float *const hs = m->pf_up, *const hb = m->pf_up + static_cast<uint64_t>(n) * (c.ffn / 32);
+        // a Q6_K down projection reads its activations as f16: the SwiGLU epilogue of the fp8 kernel writes them too
+        const bool hh = L.gate->dtype == CERA_HIP_Q4_K && L.down->dtype == CERA_HIP_Q6_K;
         if (n > PREFILL_SMALL_BATCH && L.down->dtype != CERA_HIP_Q5_K)   // a Q5_K down projection reads the f32 SwiGLU output
-            CERA_TRY(cera_launch_gemm_swiglu(ctx, L.gate, L.up, m->pf_xs, m->pf_xq, m->pf_bsum, n, hq, hs, hb, &fused, m->pf_x8, &staged8));
-        staged = false;   // the down projection's activations are new either way
+            CERA_TRY(cera_launch_gemm_swiglu(ctx, L.gate, L.up, m->pf_xs, m->pf_xq, m->pf_bsum, n, hq, hs, hb, &fused, m->pf_x8, &staged8,
+                                             hh ? m->pf_xh : nullptr));
+        staged = fused && hh;   // pf_xh: the down projection's activations, or stale
         if (fused) staged8 = false;
         if (fused && cera_gemm_supports(L.down->dtype, L.down->k)) {
             // (all layers but the last: the next layer's first row norm adds the partial sums)

@@ -27,7 +27,7 @@ SYMBOLS = [
     "cera_hip_quantize_q8_0_dev", "cera_hip_gemv_q8_dev", "cera_hip_gemv_seq_dev", "cera_hip_decode_ops_dev", "cera_hip_attn_decode_dev",
     "cera_hip_gemm_dev",
     "cera_hip_model_create", "cera_hip_model_destroy", "cera_hip_forward", "cera_hip_forward_greedy",
-    "cera_hip_forward_prefill", "cera_hip_forward_prefill_logits_all", "cera_hip_truncate_kv", "cera_hip_gemv_pair", "cera_hip_gemm_pair", "cera_hip_gemm_swiglu", "cera_hip_gemv_nb", "cera_hip_configure_kv", "cera_hip_kv_type", "cera_hip_attn_f16kv",
+    "cera_hip_forward_prefill", "cera_hip_forward_prefill_logits_all", "cera_hip_truncate_kv", "cera_hip_gemv_pair", "cera_hip_gemm_pair", "cera_hip_gemm_swiglu", "cera_hip_gemm_swiglu_f16", "cera_hip_gemv_nb", "cera_hip_configure_kv", "cera_hip_kv_type", "cera_hip_attn_f16kv",
     "cera_hip_attn_decode_f16_dev", "cera_hip_shift_kv", "cera_hip_write_kv", "cera_hip_set_seq_len", "cera_hip_seq_len", "cera_hip_memory_bytes",
     "cera_hip_read_kv", "cera_hip_read_hidden",
     "cera_hip_gemv_reference_order", "cera_hip_attn_decode_reference_order", "cera_hip_rmsnorm_reference_order",
@@ -137,6 +137,7 @@ def load_library() -> C.CDLL:
         "cera_hip_gemv_pair": (i32, [vp, vp, vp, vp, vp, vp]),
         "cera_hip_gemm_pair": (i32, [vp, vp, vp, vp, u64, vp, vp]),
         "cera_hip_gemm_swiglu": (i32, [vp, vp, vp, vp, u64, vp, vp, vp]),
+        "cera_hip_gemm_swiglu_f16": (i32, [vp, vp, vp, vp, u64, vp, vp, vp, vp]),
         "cera_hip_gemv_nb": (i32, [vp, vp, vp, u32, vp]),
         "cera_hip_configure_kv": (i32, [vp, u32]),
         "cera_hip_kv_type": (u32, [vp]),
@@ -420,6 +421,15 @@ class Context:
         fused = C.c_int(-1)
         self.check(self.lib.cera_hip_gemm_swiglu(self.h, C.byref(tg), C.byref(tu), _p(x), n, _p(q), _p(sc), C.byref(fused)))
         return q, sc, bool(fused.value)
+
+    def gemm_swiglu_f16(self, type_id, w_gate, w_up, m, x, n, k):
+        """gemm_swiglu plus the quants as the f16 words a Q6_K down projection reads: (quants, scales, halves [n][m] uint16, fused?)."""
+        tg, tu = make_tensor(type_id, m, k, w_gate), make_tensor(type_id, m, k, w_up)
+        x = np.ascontiguousarray(x, np.float32).reshape(n, k)
+        q, sc, hv = np.empty((n, m), np.int8), np.empty((n, m // 32), np.float32), np.empty((n, m), np.uint16)
+        fused = C.c_int(-1)
+        self.check(self.lib.cera_hip_gemm_swiglu_f16(self.h, C.byref(tg), C.byref(tu), _p(x), n, _p(q), _p(sc), _p(hv), C.byref(fused)))
+        return q, sc, hv, bool(fused.value)
 
     def attn_f16kv(self, q, k, v, n_heads, n_kv_heads, head_dim, start_pos, n_queries, scale, n_splits=0) -> np.ndarray:
         """Attention over an f16 KV cache: k, v (f32) are narrowed to half before the upload."""

@@ -291,7 +291,7 @@ class GemmArgs(C.Structure):       # cera_k_gemm_args
                 ("ld_m", C.c_uint64), ("ld_n", C.c_uint64), ("resid", C.c_void_p), ("resid_scale", C.c_float),
                 ("k_chunk", C.c_uint32), ("part_stride", C.c_uint64), ("w2", C.c_void_p), ("out2", C.c_void_p),
                 ("m2", C.c_uint32), ("tiles1", C.c_uint32), ("ld_n2", C.c_uint64), ("hq", C.c_void_p), ("hs", C.c_void_p),
-                ("hbsum", C.c_void_p), ("dbg_dots", C.c_void_p), ("bf8", C.c_void_p)]
+                ("hbsum", C.c_void_p), ("dbg_dots", C.c_void_p), ("bf8", C.c_void_p), ("hh", C.c_void_p)]
 
 
 class GemmActFp8Args(C.Structure):

@@ -238,6 +238,17 @@ CERA_HIP_API cera_hip_status cera_hip_gemm_pair(cera_hip_ctx*, const cera_hip_te
 CERA_HIP_API cera_hip_status cera_hip_gemm_swiglu(cera_hip_ctx*, const cera_hip_tensor* gate, const cera_hip_tensor* up,
                                                   const float* x, uint64_t n, int8_t* quants, float* scales, int* fused);
 
+/* The same, and halves[n][m] (uint16) receive the quants once more in the form the batched Q6_K GEMM
+ * reads its activations: IEEE half words of the integer values, the four of every group of four in
+ * the order 0, 2, 1, 3 (n * m a multiple of 16).  The forward pass takes them straight from the
+ * epilogue of a Q4_K gate | up launch when the down projection is Q6_K (the Q4_K_M mix) instead of
+ * converting the quants in a launch of its own; every other route converts afterwards, and both
+ * give the same words.  No counterpart in the reference, whose CPU kernels read the int8 quants
+ * directly (cera/src/model/transformer.rs:865-946). */
+CERA_HIP_API cera_hip_status cera_hip_gemm_swiglu_f16(cera_hip_ctx*, const cera_hip_tensor* gate, const cera_hip_tensor* up,
+                                                      const float* x, uint64_t n, int8_t* quants, float* scales,
+                                                      uint16_t* halves, int* fused);
+
 /* transformer::decode_attention (cera/src/model/transformer.rs:1249-1305) with
  * cpu::attn_scores / softmax_inplace / attn_values (cera/src/backend/cpu.rs:
  * 3222-3363, 2617-2633).  q f32[n_heads*head_dim]; k, v f32 time-major

@@ -342,7 +342,9 @@ typedef struct {
  *                             grid = ceil(n / 64) * 2 * (k / 256) workgroups of 256
  *   cera_k_gemm_q4_k_swiglu   w = gate, w2 = up (both m x k, m % 32 == 0): nothing goes to out; hq [n][m], hs and
  *                             hbsum [n][m/32] receive Q8_0(silu(gate.x) * (up.x)); a workgroup takes 64 gate and the
- *                             same 64 up rows: grid = (ceil(n / 64), ceil(m / 64)), k_chunk = k
+ *                             same 64 up rows: grid = (ceil(n / 64), ceil(m / 64)), k_chunk = k; hh (nullable) also
+ *                             receives the quants as f16 [n][m] in cera_k_gemm_act_f16's order, for a q6_k GEMM that
+ *                             follows (NULL in every other kernel of this family)
  *   cera_k_gemm_q6_k          f16 matrix cores; reads bh, the quants as f16 made by
  *                             cera_k_gemm_act_f16 (n * k * 2 bytes; n_words = n * k / 16,
  *                             grid = ceil(n_words / 256) of 256)
@@ -377,6 +379,7 @@ typedef struct {
     float* hbsum;
     int32_t* dbg_dots;
     const uint8_t* bf8;
+    uint16_t* hh;
 } cera_k_gemm_args;
 typedef struct { const int8_t* quants; const float* scales; const float* bsum; uint8_t* out; uint32_t n, k; } cera_k_gemm_act_fp8_args;
 typedef struct { const void* quants; void* out; uint64_t n_words; } cera_k_gemm_act_f16_args;

@@ -313,6 +313,17 @@ pub fn cera_hip_ctx_create(
         scales: *mut f32,
         fused: *mut c_int,
     ) -> cera_hip_status;
+    pub fn cera_hip_gemm_swiglu_f16(
+        ctx: *mut cera_hip_ctx,
+        gate: *const cera_hip_tensor,
+        up: *const cera_hip_tensor,
+        x: *const f32,
+        n: u64,
+        quants: *mut i8,
+        scales: *mut f32,
+        halves: *mut u16,
+        fused: *mut c_int,
+    ) -> cera_hip_status;
     pub fn cera_hip_attn_decode(
         ctx: *mut cera_hip_ctx,
         q: *const f32,

@@ -125,6 +125,24 @@ def test_gemm_swiglu_epilogue_matches_separate_kernels(hip, orc, dtype, m, k, n,
     assert np.array_equal(sc.reshape(-1).view(np.uint32), ref_s.view(np.uint32))
 
 
+@pytest.mark.parametrize("dtype,m,k,n,want_fused", [(Q4_K, 2048, 512, 1040, True), (Q4_K, 1056, 256, 2000, True),
+                                                      (Q4_K, 512, 256, 80, False), (Q4_0, 2048, 512, 1040, True)])
+def test_gemm_swiglu_f16_words_for_a_q6k_down_projection(hip, dtype, m, k, n, want_fused):
+    """The f16 form of the SwiGLU quants that a Q6_K down projection reads: half words of the integer
+    quants, every four in the order 0, 2, 1, 3 -- whether the Q4_K epilogue writes them or the
+    conversion kernel makes them from the quants afterwards (small batches, other types)."""
+    _say(f"gemm_swiglu_f16 {util.NAMES[dtype]} m={m} k={k} n={n}")
+    wg, _ = util.make_weights(dtype, m, k, seed=43)
+    wu, _ = util.make_weights(dtype, m, k, seed=44)
+    x = util.rng(m + 5 * n).standard_normal((n, k)).astype(np.float32)
+    q, sc, hv, fused = hip.gemm_swiglu_f16(dtype, wg, wu, m, x, n, k)
+    assert fused == want_fused
+    q0, sc0, _ = hip.gemm_swiglu(dtype, wg, wu, m, x, n, k)
+    assert np.array_equal(q, q0) and np.array_equal(sc.view(np.uint32), sc0.view(np.uint32))
+    want = q.astype(np.float16).reshape(-1, 4)[:, [0, 2, 1, 3]].reshape(n, m)
+    assert np.array_equal(hv, want.view(np.uint16))
+
+
 def test_gemm_pair_refuses_mixed_types(hip):
     with pytest.raises(hip_api.HipError) as e:
         hip.gemm_pair(Q4_K, np.zeros(144 * 4, np.uint8), 4, Q6_K, np.zeros(210 * 4, np.uint8), 4,

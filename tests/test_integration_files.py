@@ -14,7 +14,7 @@ SYS = (ROOT / "integration" / "cera-hip-sys" / "src" / "lib.rs").read_text()
 MODEL = (ROOT / "integration" / "cera" / "src" / "model" / "hip_llama.rs").read_text()
 PATCH = (ROOT / "integration" / "cera-hip-backend.patch").read_text()
 
-SCALARS = {"int": "c_int", "uint32_t": "u32", "uint64_t": "u64", "int32_t": "i32", "int8_t": "i8", "uint8_t": "u8",
+SCALARS = {"int": "c_int", "uint32_t": "u32", "uint64_t": "u64", "int32_t": "i32", "int8_t": "i8", "uint8_t": "u8", "uint16_t": "u16",
            "float": "f32", "char": "c_char", "cera_hip_status": "cera_hip_status", "void": "c_void"}
 
 
