@@ -40,6 +40,7 @@
 // FMAs + staging) that sum is what the fp8 dot lowers.
 #pragma once
 #include "gemm.hip.h"
+#include "gemm_q6k_f16.hip.h"
 
 typedef int v8i __attribute__((ext_vector_type(8)));
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
@@ -61,9 +62,11 @@ typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 //   [j 0..2][lane][8 bf16]                      xs*sum(a) of blocks 4*half .. 4*half+3 as three bf16 pieces
 //       b0, b1, b2 in slot order (b0, b1, b0, b2, b1, b0) per block, slots 8j .. 8j+7 of the lane's 24
 // Tokens at or beyond n are zero.
+// halves (nullable): the same quants also as f16 [n][k] in gemm_act_f16_kernel's order, for a Q6_K matrix
+// multiplied by the same activations (a layer's V next to its Q4_K Q and K): one launch for both copies.
 __device__ __forceinline__ void gemm_act_fp8_body(const int8_t* __restrict__ xq, const float* __restrict__ xs,
                                                                   const float* __restrict__ bsum, uint8_t* __restrict__ rec,
-                                                                  uint32_t n, uint32_t k) {
+                                                                  uint32_t n, uint32_t k, uint4* __restrict__ halves = nullptr) {
     const uint32_t nsb = k / 256, tile = blockIdx.x / nsb, sb = blockIdx.x % nsb, tid = threadIdx.x;
     uint8_t* const r = rec + static_cast<uint64_t>(blockIdx.x) * G8_REC;
     // quants: thread t handles (blk = t / 32, token = t % 32): 32 bytes in, 2 x 2 x 16 bytes out
@@ -74,6 +77,11 @@ __device__ __forceinline__ void gemm_act_fp8_body(const int8_t* __restrict__ xq,
             const uint4* src = reinterpret_cast<const uint4*>(xq + static_cast<uint64_t>(tok) * k + sb * 256 + blk * 32);
             in[0] = src[0];
             in[1] = src[1];
+            if (halves) {
+                uint4* const dst = halves + (static_cast<uint64_t>(tok) * k + sb * 256 + blk * 32) / 8;
+                gemm_act_f16_words(in[0], dst[0], dst[1]);
+                gemm_act_f16_words(in[1], dst[2], dst[3]);
+            }
         }
 #pragma unroll
         for (int half = 0; half < 2; ++half) {
@@ -130,8 +138,8 @@ __device__ __forceinline__ void gemm_act_fp8_body(const int8_t* __restrict__ xq,
 }
 static __global__ __launch_bounds__(256) void gemm_act_fp8_kernel(const int8_t* __restrict__ xq, const float* __restrict__ xs,
                                                                   const float* __restrict__ bsum, uint8_t* __restrict__ rec,
-                                                                  uint32_t n, uint32_t k) {
-    gemm_act_fp8_body(xq, xs, bsum, rec, n, k);
+                                                                  uint32_t n, uint32_t k, uint4* __restrict__ halves) {
+    gemm_act_fp8_body(xq, xs, bsum, rec, n, k, halves);
 }
 
 // global -> LDS copy of 1 KB (64 lanes x 16 B) without passing through registers: lane i's 16 bytes

@@ -31,12 +31,8 @@ typedef uint32_t gq_u4 __attribute__((ext_vector_type(4)));
 
 #define GQ_LD 272   // bytes per staged row: 128 f16 + 16 pad
 
-// int8 quants [n_words * 16] -> f16 in the 0,2,1,3 order, 16 per thread
-__device__ __forceinline__ void gemm_act_f16_body(const uint4* __restrict__ q, uint4* __restrict__ out,
-                                                                  uint64_t n_words) {
-    const uint64_t i = static_cast<uint64_t>(blockIdx.x) * 256 + threadIdx.x;
-    if (i >= n_words) return;
-    const uint4 v = q[i];
+// 16 int8 quants -> 16 f16 words in the 0,2,1,3 order
+__device__ __forceinline__ void gemm_act_f16_words(const uint4 v, uint4& out0, uint4& out1) {
     const uint32_t x[4] = {v.x, v.y, v.z, v.w};
     uint32_t o[8];
     const _Float16 mh = static_cast<_Float16>(-1152.0f);
@@ -48,8 +44,15 @@ __device__ __forceinline__ void gemm_act_f16_body(const uint4* __restrict__ q, u
         o[2 * j] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(gq_h2, (y & 0x00FF00FFu) | 0x64006400u) + off);
         o[2 * j + 1] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(gq_h2, ((y >> 8) & 0x00FF00FFu) | 0x64006400u) + off);
     }
-    out[2 * i] = make_uint4(o[0], o[1], o[2], o[3]);
-    out[2 * i + 1] = make_uint4(o[4], o[5], o[6], o[7]);
+    out0 = make_uint4(o[0], o[1], o[2], o[3]);
+    out1 = make_uint4(o[4], o[5], o[6], o[7]);
+}
+// int8 quants [n_words * 16] -> f16 in the 0,2,1,3 order, 16 per thread
+__device__ __forceinline__ void gemm_act_f16_body(const uint4* __restrict__ q, uint4* __restrict__ out,
+                                                                  uint64_t n_words) {
+    const uint64_t i = static_cast<uint64_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (i >= n_words) return;
+    gemm_act_f16_words(q[i], out[2 * i], out[2 * i + 1]);
 }
 static __global__ __launch_bounds__(256) void gemm_act_f16_kernel(const uint4* __restrict__ q, uint4* __restrict__ out,
                                                                   uint64_t n_words) {

@@ -261,7 +261,7 @@ CERA_K_ATTN_PF_G(f16, kv_half, 128)
 
 // ---- batched GEMMs -------------------------------------------------------------------------------
 extern "C" __global__ __launch_bounds__(256) void cera_k_gemm_act_fp8(cera_k_gemm_act_fp8_args a) {
-    gemm_act_fp8_body(a.quants, a.scales, a.bsum, a.out, a.n, a.k);
+    gemm_act_fp8_body(a.quants, a.scales, a.bsum, a.out, a.n, a.k, static_cast<uint4*>(a.halves));
 }
 extern "C" __global__ __launch_bounds__(256) void cera_k_gemm_act_f16(cera_k_gemm_act_f16_args a) {
     gemm_act_f16_body(reinterpret_cast<const uint4*>(a.quants), reinterpret_cast<uint4*>(a.out), a.n_words);

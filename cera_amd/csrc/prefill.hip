@@ -87,7 +87,7 @@ cera_hip_status cera_launch_gemm(cera_hip_ctx* ctx, const cera_hip_dtensor* w, c
         }
         if (!staged8 || !*staged8) {
             hipLaunchKernelGGL(gemm_act_fp8_kernel, dim3(tiles * nsb), dim3(256), 0, ctx->stream, bq, bs, bsum,
-                               static_cast<uint8_t*>(b8_ws), n, a.k);
+                               static_cast<uint8_t*>(b8_ws), n, a.k, static_cast<uint4*>(nullptr));
             if (staged8) *staged8 = true;
         }
         a.bf8 = static_cast<const uint8_t*>(b8_ws);
@@ -218,7 +218,7 @@ cera_hip_status cera_launch_gemm_swiglu(cera_hip_ctx* ctx, const cera_hip_dtenso
         }
         if (!staged8 || !*staged8) {
             hipLaunchKernelGGL(gemm_act_fp8_kernel, dim3((n + G8_BN - 1) / G8_BN * 2 * (a.k / 256)), dim3(256), 0, ctx->stream, bq, bs,
-                               bsum, static_cast<uint8_t*>(b8_ws), n, a.k);
+                               bsum, static_cast<uint8_t*>(b8_ws), n, a.k, static_cast<uint4*>(nullptr));
             if (staged8) *staged8 = true;
         }
         a.bf8 = static_cast<const uint8_t*>(b8_ws);
@@ -567,6 +567,15 @@ static cera_hip_status prefill_chunk(cera_hip_model* m, const uint32_t* tokens, 
     for (uint32_t i = 0; i < c.n_layers; ++i) {
         LayerDev& L = m->layers[i];
         CERA_TRY(norm_rows(m->pf_hidden, L.attn_norm, m->pf_normed));
+        // Q4_K Q and K next to a Q6_K V (the Q4_K_M mix): both re-laid copies of the activations in one launch
+        if (n > PREFILL_SMALL_BATCH && L.q->dtype == CERA_HIP_Q4_K && L.k->dtype == CERA_HIP_Q4_K && L.v->dtype == CERA_HIP_Q6_K &&
+            gemm_batched(CERA_HIP_Q4_K, hs) && gemm_batched(CERA_HIP_Q6_K, hs)) {
+            hipLaunchKernelGGL(gemm_act_fp8_kernel, dim3((n + G8_BN - 1) / G8_BN * 2 * (hs / 256)), dim3(256), 0, s, m->pf_xq, m->pf_xs,
+                               m->pf_bsum, static_cast<uint8_t*>(m->pf_x8), n, hs, static_cast<uint4*>(m->pf_xh));
+            HIP_TRY(ctx, hipGetLastError());
+            staged = true;
+            staged8 = true;
+        }
         CERA_TRY(gemm2(L.q, m->pf_q, L.k, m->pf_k, m->pf_normed));
         CERA_TRY(gemm(L.v, m->pf_v, nullptr, m->pf_normed));
         if (L.q_bias) {

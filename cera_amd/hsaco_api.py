@@ -296,7 +296,7 @@ class GemmArgs(C.Structure):       # cera_k_gemm_args
 
 class GemmActFp8Args(C.Structure):
     _fields_ = [("quants", C.c_void_p), ("scales", C.c_void_p), ("bsum", C.c_void_p), ("out", C.c_void_p), ("n", C.c_uint32),
-                ("k", C.c_uint32)]
+                ("k", C.c_uint32), ("halves", C.c_void_p)]
 
 
 class GemmActF16Args(C.Structure):

@@ -339,7 +339,8 @@ typedef struct {
  * reference's per-block float scales.  k % 256 == 0 for q4_k / q6_k, k % 128 == 0 otherwise.
  *   cera_k_gemm_q4_k          fp8 matrix cores; reads bf8, the split copy cera_k_gemm_act_fp8 makes
  *                             of (bq, bs, bsum): CERA_K_GEMM_FP8_ACT_BYTES(n, k) bytes,
- *                             grid = ceil(n / 64) * 2 * (k / 256) workgroups of 256
+ *                             grid = ceil(n / 64) * 2 * (k / 256) workgroups of 256; its halves (nullable) also
+ *                             receives what cera_k_gemm_act_f16 would write for the same quants ([n][k] f16)
  *   cera_k_gemm_q4_k_swiglu   w = gate, w2 = up (both m x k, m % 32 == 0): nothing goes to out; hq [n][m], hs and
  *                             hbsum [n][m/32] receive Q8_0(silu(gate.x) * (up.x)); a workgroup takes 64 gate and the
  *                             same 64 up rows: grid = (ceil(n / 64), ceil(m / 64)), k_chunk = k; hh (nullable) also
@@ -381,7 +382,7 @@ typedef struct {
     const uint8_t* bf8;
     uint16_t* hh;
 } cera_k_gemm_args;
-typedef struct { const int8_t* quants; const float* scales; const float* bsum; uint8_t* out; uint32_t n, k; } cera_k_gemm_act_fp8_args;
+typedef struct { const int8_t* quants; const float* scales; const float* bsum; uint8_t* out; uint32_t n, k; void* halves; } cera_k_gemm_act_fp8_args;
 typedef struct { const void* quants; void* out; uint64_t n_words; } cera_k_gemm_act_f16_args;
 /* out[e] = (resid[e] + resid_scale *) sum_z part[z * part_stride + e] over n4 float4s; for a pair
  * float4s from n4_first on go to out2 (no pair: n4_first = n4, out2 = NULL).
