@@ -299,6 +299,33 @@ def test_prefill_equals_decode_on_gpu(hip):
     a.close(); b.close()
 
 
+def test_prefill_where_the_norm_adds_split_k_partial_sums(hip, orc):
+    """Projections whose K is split (2048-wide rows, few row tiles) in a pass of 128 tokens or more: the O
+    and down projections leave their partial sums to the row norm that follows (and the last layer's down
+    projection to the reduction kernel).  Logits and both layers' K/V rows track the oracle's batched
+    prefill, and a decode step continues from the cache."""
+    cfg = dict(synth.TINY, hidden=2048, ffn=2048, n_heads=16, n_kv_heads=4, head_dim=128, max_seq_len=192)
+    weights = synth.make_llama(cfg, seed=81, sigma=0.03, norm_jitter=0.1)
+    gm = hip_api.Model(hip, cfg, weights)
+    om = orc.Llama(cfg, weights)
+    toks = [int(t) for t in util.rng(12).integers(0, cfg["vocab"], 130)]
+    _say("model: 130-token prefill, hidden 2048 (split-K O and down projections)")
+    lg = gm.forward_prefill(toks, 0)
+    lo = om.forward_prefill_batched(toks, 0)
+    _say(f"  cos={_cos(lg, lo):.8f} max|err|={np.abs(lg - lo).max():.3e} rms={util.rms(lo):.3e}")
+    assert _cos(lg, lo) > 0.999
+    for layer in range(cfg["n_layers"]):
+        kg, vg = gm.read_kv(layer)
+        ko, vo = om.kv(layer)
+        tol = 2e-3 if layer == 0 else 5e-2
+        assert np.abs(kg - ko).max() <= tol * util.rms(ko), layer
+        assert np.abs(vg - vo).max() <= tol * util.rms(vo), layer
+    lg2 = gm.forward(7, 130)
+    lo2 = om.forward(7, 130)
+    assert _cos(lg2, lo2) > 0.999
+    gm.close(); om.close()
+
+
 @pytest.mark.parametrize("nh,nkv,start,n", [(32, 8, 0, 512), (8, 2, 0, 40), (8, 8, 300, 100), (16, 2, 1000, 33),
                                              (4, 1, 0, 16), (32, 8, 4000, 96), (32, 8, 2048, 2048)])
 def test_attn_prefill_batch_vs_oracle(hip, orc, nh, nkv, start, n):
