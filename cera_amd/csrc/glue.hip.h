@@ -268,23 +268,39 @@ static __global__ __launch_bounds__(1024) void rmsnorm_row_kernel(const float* _
 // threads: blocks [0, n_heads) rotate q; the next n_kv_heads rotate k and
 // store it; the last n_kv_heads copy v.
 // KV cache layout: [kv_head][max_seq][head_dim] f32.
+// Split-K partial sums of q, k or v that this kernel adds up itself instead of a reduction launch in front
+// of it: value e = sum_z part[z * stride + e] in that order (n_split = 0: the rows are complete as they are).
+struct RopePending {
+    const float* part;
+    uint32_t n_split;
+    uint64_t stride;
+};
+__device__ __forceinline__ float rope_pending_ld(const float* rows, const RopePending& pd, uint64_t e) {
+    if (pd.n_split == 0) return rows[e];
+    float s = pd.part[e];
+    for (uint32_t z = 1; z < pd.n_split; ++z) s += pd.part[z * pd.stride + e];
+    return s;
+}
 template <typename KV>
 __device__ __forceinline__ void rope_kv_body(float* __restrict__ q, float* __restrict__ k, const float* v,
                                const float* __restrict__ cs_table, const uint32_t* __restrict__ pos_ptr,
                                uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, uint32_t rope_type,
-                               KV* __restrict__ k_cache, KV* __restrict__ v_cache, uint32_t max_seq) {
+                               KV* __restrict__ k_cache, KV* __restrict__ v_cache, uint32_t max_seq,
+                               RopePending pq = RopePending{}, RopePending pk = RopePending{}, RopePending pv = RopePending{}) {
     // grid.y = tokens of a prefill batch: token t sits at position *pos_ptr + t and its
     // q/k/v rows follow each other ([n][n_heads*head_dim], [n][n_kv_heads*head_dim])
     const uint32_t pos = *pos_ptr + blockIdx.y;
-    q += static_cast<uint64_t>(blockIdx.y) * n_heads * head_dim;
-    k += static_cast<uint64_t>(blockIdx.y) * n_kv_heads * head_dim;
-    if (v) v += static_cast<uint64_t>(blockIdx.y) * n_kv_heads * head_dim;
+    const uint64_t q_row = static_cast<uint64_t>(blockIdx.y) * n_heads * head_dim, kv_row = static_cast<uint64_t>(blockIdx.y) * n_kv_heads * head_dim;
     const uint32_t half = head_dim / 2, i = threadIdx.x, b = blockIdx.x;
     if (b < n_heads + n_kv_heads) {
-        float* head = b < n_heads ? q + b * head_dim : k + (b - n_heads) * head_dim;
+        const bool is_q = b < n_heads;
+        float* const rows = is_q ? q : k;
+        const uint64_t at = is_q ? q_row + b * head_dim : kv_row + (b - n_heads) * head_dim;
+        float* head = rows + at;
         float2 cs = reinterpret_cast<const float2*>(cs_table)[static_cast<uint64_t>(pos) * half + i];
         uint32_t i0 = rope_type == 1 ? 2 * i : i, i1 = rope_type == 1 ? 2 * i + 1 : i + half;
-        float x0 = head[i0], x1 = head[i1];
+        const RopePending& pd = is_q ? pq : pk;
+        float x0 = rope_pending_ld(rows, pd, at + i0), x1 = rope_pending_ld(rows, pd, at + i1);
         float r0 = __fsub_rn(__fmul_rn(x0, cs.x), __fmul_rn(x1, cs.y));
         float r1 = __fadd_rn(__fmul_rn(x0, cs.y), __fmul_rn(x1, cs.x));
         head[i0] = r0;
@@ -297,8 +313,8 @@ __device__ __forceinline__ void rope_kv_body(float* __restrict__ q, float* __res
     } else if (v_cache) {
         uint32_t h = b - n_heads - n_kv_heads;
         KV* dst = v_cache + (static_cast<uint64_t>(h) * max_seq + pos) * head_dim;
-        dst[2 * i] = static_cast<KV>(v[h * head_dim + 2 * i]);
-        dst[2 * i + 1] = static_cast<KV>(v[h * head_dim + 2 * i + 1]);
+        dst[2 * i] = static_cast<KV>(rope_pending_ld(v, pv, kv_row + h * head_dim + 2 * i));
+        dst[2 * i + 1] = static_cast<KV>(rope_pending_ld(v, pv, kv_row + h * head_dim + 2 * i + 1));
     }
 }
 template <typename KV>
@@ -307,6 +323,15 @@ static __global__ void rope_kv_kernel(float* __restrict__ q, float* __restrict__
                                uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, uint32_t rope_type,
                                KV* __restrict__ k_cache, KV* __restrict__ v_cache, uint32_t max_seq) {
     rope_kv_body<KV>(q, k, v, cs_table, pos_ptr, n_heads, n_kv_heads, head_dim, rope_type, k_cache, v_cache, max_seq);
+}
+// The same over q / k / v rows whose split-K partial sums are still pending.
+template <typename KV>
+static __global__ void rope_kv_pending_kernel(float* __restrict__ q, float* __restrict__ k, const float* v,
+                               const float* __restrict__ cs_table, const uint32_t* __restrict__ pos_ptr,
+                               uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, uint32_t rope_type,
+                               KV* __restrict__ k_cache, KV* __restrict__ v_cache, uint32_t max_seq,
+                               RopePending pq, RopePending pk, RopePending pv) {
+    rope_kv_body<KV>(q, k, v, cs_table, pos_ptr, n_heads, n_kv_heads, head_dim, rope_type, k_cache, v_cache, max_seq, pq, pk, pv);
 }
 
 // n_keep context shift (cera/src/kv_cache.rs:1091-1310): rows [src_row, src_row + n_rows) of every

@@ -38,10 +38,12 @@ cera_hip_status cera_launch_gemm(cera_hip_ctx* ctx, const cera_hip_dtensor* w, c
                                  float* out2 = nullptr, uint64_t ld_n2 = 0, bool* paired = nullptr, void* bh_ws = nullptr,
                                  bool* staged = nullptr, int32_t* dbg_dots = nullptr, const float* x_f32 = nullptr,
                                  bool* staged_f32 = nullptr, void* b8_ws = nullptr, bool* staged8 = nullptr,
-                                 RowsPending* pending = nullptr) {
-    // pending (nullable): a caller whose next launch can add split-K partial sums itself (the row norm of
-    // a prefill); when K is split, the reduction launch is left out and *pending says what to add
-    // (n_split = 0: nothing, out is complete)
+                                 RowsPending* pending = nullptr, int part_slot = 9) {
+    // pending (nullable): a caller whose next launch can add split-K partial sums itself (the row norm or the
+    // RoPE kernel of a prefill); when K is split, the reduction launch is left out and *pending says what to
+    // add (n_split = 0: nothing, out is complete).  A pair's partial sums lie side by side: the second
+    // matrix's start m * n floats into every slice.  part_slot: the scratch slot the partial sums go to (a
+    // caller that keeps two sets pending gives the second one a slot of its own).
     if (pending) *pending = RowsPending{};
     // Q5_K: x_f32 [n][k] are the activations (bs / bq / bsum are not read); *staged_f32 (nullable)
     // says whether the context's split copy still holds exactly these activations
@@ -146,7 +148,7 @@ cera_hip_status cera_launch_gemm(cera_hip_ctx* ctx, const cera_hip_dtensor* w, c
     const uint64_t mn = static_cast<uint64_t>(a.m) * n, mn2 = static_cast<uint64_t>(a.m2) * n;
     if (split > 1) {
         void* part;
-        CERA_TRY(cera_scratch(ctx, 9, split * (mn + mn2) * sizeof(float), &part));
+        CERA_TRY(cera_scratch(ctx, part_slot, split * (mn + mn2) * sizeof(float), &part));
         a.out = static_cast<float*>(part);
         if (a.w2) a.out2 = a.out + mn;
         a.part_stride = mn + mn2;
@@ -176,9 +178,7 @@ cera_hip_status cera_launch_gemm(cera_hip_ctx* ctx, const cera_hip_dtensor* w, c
         case CERA_HIP_Q4_1: hipLaunchKernelGGL((gemm_kernel<GemmQ4_1>), grid, dim3(256), 0, ctx->stream, a); break;
         default: hipLaunchKernelGGL((gemm_kernel<GemmQ8_0>), grid, dim3(256), 0, ctx->stream, a); break;
     }
-    // (from 128 rows on: the norm runs one workgroup per row, and a few dozen workgroups adding up partial sums take
-    // longer than the reduction launch they save -- 12.8 against 4.8 + 5.7 us at 16 rows, 11.3 against 6.3 + 7.4 at 512)
-    if (split > 1 && pending && n >= 128 && !a.w2 && ld_m == 1 && ld_n == a.m)
+    if (split > 1 && pending && ld_m == 1 && ld_n == a.m && (!a.w2 || ld_n2 == a.m2))
         *pending = RowsPending{a.out, split, a.part_stride, resid, resid_scale, out};
     else if (split > 1)   // one launch reduces both matrices of a pair
         hipLaunchKernelGGL(gemm_reduce_kernel, dim3(static_cast<uint32_t>(((mn + mn2) / 4 + 255) / 256)), dim3(256), 0,
@@ -512,8 +512,11 @@ static cera_hip_status prefill_chunk(cera_hip_model* m, const uint32_t* tokens, 
     bool staged8 = false;
     // the f32 activations whose hi / lo split (Q5_K GEMMs) the context's workspace holds now
     const float* split_of = nullptr;
-    // split-K partial sums of pf_hidden that the next row norm adds up (n_split = 0: none)
+    // split-K partial sums of pf_hidden that the next row norm adds up (n_split = 0: none).  From 128 rows on:
+    // the norm runs one workgroup per row, and a few dozen workgroups adding up partial sums take longer than
+    // the reduction launch they save (12.8 against 4.8 + 5.7 us at 16 rows, 11.3 against 6.3 + 7.4 at 512).
     RowsPending pend{};
+    const bool norm_adds = n >= 128;
     auto norm_rows = [&](const float* x, const float* w, float* y) -> cera_hip_status {
         staged = false;
         staged8 = false;
@@ -531,7 +534,7 @@ static cera_hip_status prefill_chunk(cera_hip_model* m, const uint32_t* tokens, 
     // out[n][w->m] (token-major rows) = B . W^T, optionally added onto resid
     // xf: the f32 activations the quantized ones in pf_xs / pf_xq were made from (what a Q5_K matrix reads)
     auto gemm = [&](const cera_hip_dtensor* w, float* out, const float* resid, const float* xf,
-                    RowsPending* pending = nullptr) -> cera_hip_status {
+                    RowsPending* pending = nullptr, int part_slot = 9) -> cera_hip_status {
         // a short batch streams the weights once per 8 tokens through the multi-token GEMV (an
         // int8-MFMA tile would be mostly empty); its residual add is unscaled
         if ((n <= PREFILL_SMALL_BATCH || !gemm_batched(w->dtype, w->k)) && (!resid || c.residual_scale == 1.0f)) {
@@ -542,7 +545,8 @@ static cera_hip_status prefill_chunk(cera_hip_model* m, const uint32_t* tokens, 
         }
         bool split_held = split_of == xf;
         CERA_TRY(cera_launch_gemm(ctx, w, m->pf_xs, m->pf_xq, m->pf_bsum, n, out, 1, w->m, resid, c.residual_scale, nullptr,
-                                  nullptr, 0, nullptr, m->pf_xh, &staged, nullptr, xf, &split_held, m->pf_x8, &staged8, pending));
+                                  nullptr, 0, nullptr, m->pf_xh, &staged, nullptr, xf, &split_held, m->pf_x8, &staged8, pending,
+                                  part_slot));
         if (w->dtype == CERA_HIP_Q5_K) split_of = xf;
         return CERA_HIP_OK;
     };
@@ -550,14 +554,26 @@ static cera_hip_status prefill_chunk(cera_hip_model* m, const uint32_t* tokens, 
     // two projections of the same activations: one launch when both have an int8 GEMM of the same
     // type (the tail of one matrix's workgroups then overlaps the other's, and a short K-split
     // matrix like K shares Q's launch), else one after the other
-    auto gemm2 = [&](const cera_hip_dtensor* wa, float* outa, const cera_hip_dtensor* wb, float* outb, const float* xf) -> cera_hip_status {
+    // pending (nullable): filled when the two went out as one launch whose split-K partial sums the caller adds up
+    auto gemm2 = [&](const cera_hip_dtensor* wa, float* outa, const cera_hip_dtensor* wb, float* outb, const float* xf,
+                     RowsPending* pending = nullptr) -> cera_hip_status {
         if (n > PREFILL_SMALL_BATCH && gemm_batched(wa->dtype, wa->k) && gemm_batched(wb->dtype, wb->k)) {
             bool paired = false;
             bool split_held = split_of == xf;
             CERA_TRY(cera_launch_gemm(ctx, wa, m->pf_xs, m->pf_xq, m->pf_bsum, n, outa, 1, wa->m, nullptr, 1.0f, wb, outb,
-                                      wb->m, &paired, m->pf_xh, &staged, nullptr, xf, &split_held, m->pf_x8, &staged8));
+                                      wb->m, &paired, m->pf_xh, &staged, nullptr, xf, &split_held, m->pf_x8, &staged8, pending));
             if (wa->dtype == CERA_HIP_Q5_K) split_of = xf;
             if (paired) return CERA_HIP_OK;
+            if (pending && pending->n_split) {
+                // the first matrix went out alone and left its partial sums pending: the second one's launch reuses
+                // their scratch, so they are added up now
+                const uint64_t n4 = static_cast<uint64_t>(wa->m) * n / 4;
+                hipLaunchKernelGGL(gemm_reduce_kernel, dim3(static_cast<uint32_t>((n4 + 255) / 256)), dim3(256), 0, s, pending->part,
+                                   pending->n_split, pending->stride, n4, outa, static_cast<const float*>(nullptr), 1.0f, n4,
+                                   static_cast<float*>(nullptr));
+                HIP_TRY(ctx, hipGetLastError());
+                *pending = RowsPending{};
+            }
             return gemm(wb, outb, nullptr, xf);
         }
         CERA_TRY(gemm(wa, outa, nullptr, xf));
@@ -576,8 +592,12 @@ static cera_hip_status prefill_chunk(cera_hip_model* m, const uint32_t* tokens, 
             staged = true;
             staged8 = true;
         }
-        CERA_TRY(gemm2(L.q, m->pf_q, L.k, m->pf_k, m->pf_normed));
-        CERA_TRY(gemm(L.v, m->pf_v, nullptr, m->pf_normed));
+        // With nothing between the projections and RoPE (no biases, no QK norm) the RoPE / append kernel adds up
+        // the split-K partial sums of Q | K and of V itself: two reduction launches less.
+        RowsPending pqk{}, pvv{};
+        const bool rope_adds = !L.q_bias && !L.q_norm;
+        CERA_TRY(gemm2(L.q, m->pf_q, L.k, m->pf_k, m->pf_normed, rope_adds ? &pqk : nullptr));
+        CERA_TRY(gemm(L.v, m->pf_v, nullptr, m->pf_normed, rope_adds ? &pvv : nullptr, 14));
         if (L.q_bias) {
             // bias rows: one launch per token keeps the kernel trivial; models with biases are rare here
             for (uint32_t t = 0; t < n; ++t) {
@@ -592,7 +612,19 @@ static cera_hip_status prefill_chunk(cera_hip_model* m, const uint32_t* tokens, 
             hipLaunchKernelGGL((rmsnorm_kernel<false>), dim3(n * c.n_kv_heads), dim3(256), 0, s, m->pf_k, L.k_norm, c.head_dim,
                                c.rms_eps, m->pf_k, nullptr, nullptr, nullptr);
         }
-        if (m->kv_f16)
+        if (pqk.n_split || pvv.n_split) {
+            const RopePending rq{pqk.part, pqk.n_split, pqk.stride};
+            const RopePending rk{pqk.n_split ? pqk.part + static_cast<uint64_t>(n) * q_dim : nullptr, pqk.n_split, pqk.stride};
+            const RopePending rv{pvv.part, pvv.n_split, pvv.stride};
+            if (m->kv_f16)
+                hipLaunchKernelGGL(rope_kv_pending_kernel<kv_half>, dim3(c.n_heads + 2 * c.n_kv_heads, n), dim3(c.head_dim / 2), 0, s,
+                                   m->pf_q, m->pf_k, m->pf_v, m->rope_table, m->scalars + 1, c.n_heads, c.n_kv_heads, c.head_dim,
+                                   c.rope_type, static_cast<kv_half*>(L.kc), static_cast<kv_half*>(L.vc), c.max_seq_len, rq, rk, rv);
+            else
+                hipLaunchKernelGGL(rope_kv_pending_kernel<float>, dim3(c.n_heads + 2 * c.n_kv_heads, n), dim3(c.head_dim / 2), 0, s,
+                                   m->pf_q, m->pf_k, m->pf_v, m->rope_table, m->scalars + 1, c.n_heads, c.n_kv_heads, c.head_dim,
+                                   c.rope_type, static_cast<float*>(L.kc), static_cast<float*>(L.vc), c.max_seq_len, rq, rk, rv);
+        } else if (m->kv_f16)
             hipLaunchKernelGGL(rope_kv_kernel<kv_half>, dim3(c.n_heads + 2 * c.n_kv_heads, n), dim3(c.head_dim / 2), 0, s,
                                m->pf_q, m->pf_k, m->pf_v, m->rope_table, m->scalars + 1, c.n_heads, c.n_kv_heads, c.head_dim,
                                c.rope_type, static_cast<kv_half*>(L.kc), static_cast<kv_half*>(L.vc), c.max_seq_len);
@@ -608,7 +640,7 @@ static cera_hip_status prefill_chunk(cera_hip_model* m, const uint32_t* tokens, 
         staged8 = false;
         split_of = nullptr;
         // (the row norm that follows adds the O projection's split-K partial sums itself)
-        CERA_TRY(gemm(L.o, m->pf_hidden, m->pf_hidden, m->pf_attn, &pend));
+        CERA_TRY(gemm(L.o, m->pf_hidden, m->pf_hidden, m->pf_attn, norm_adds ? &pend : nullptr));
 
         CERA_TRY(norm_rows(m->pf_hidden, L.ffn_norm, m->pf_normed));
         // gate, up, SwiGLU and the quantization for the down projection in one launch where the
@@ -628,7 +660,7 @@ static cera_hip_status prefill_chunk(cera_hip_model* m, const uint32_t* tokens, 
             // (all layers but the last: the next layer's first row norm adds the partial sums)
             CERA_TRY(cera_launch_gemm(ctx, L.down, hs, hq, hb, n, m->pf_hidden, 1, L.down->m, m->pf_hidden, c.residual_scale,
                                       nullptr, nullptr, 0, nullptr, m->pf_xh, &staged, nullptr, nullptr, nullptr, m->pf_x8, &staged8,
-                                      i + 1 < c.n_layers ? &pend : nullptr));
+                                      norm_adds && i + 1 < c.n_layers ? &pend : nullptr));
             staged = false;   // pf_xh / pf_x8 now mirror hq, not pf_xq
             staged8 = false;
             continue;
@@ -646,7 +678,7 @@ static cera_hip_status prefill_chunk(cera_hip_model* m, const uint32_t* tokens, 
             split_of = nullptr;
         }
         staged8 = false;   // pf_xq holds the SwiGLU output now
-        CERA_TRY(gemm(L.down, m->pf_hidden, m->pf_hidden, m->pf_gate, i + 1 < c.n_layers ? &pend : nullptr));
+        CERA_TRY(gemm(L.down, m->pf_hidden, m->pf_hidden, m->pf_gate, norm_adds && i + 1 < c.n_layers ? &pend : nullptr));
     }
     m->seq_len = start_pos + n;
     if (all_logits) {
