@@ -40,11 +40,11 @@ GATE_UP_KERNEL = "row_gemv_kernel<Q4K,16,4,true,2,true,1,4096>"
 # of the whole default run (profiles/gemv_decode_set_llama3_8b_kernel_trace.txt): a recorded figure, kept
 # beside the live back-to-back one because events around a single launch inside a step would time the
 # launch gap, not the kernel.
-GATE_UP_IN_STEP_US = 14.25
+GATE_UP_IN_STEP_US = 14.24
 # Average duration rocprofv3 reports for the same kernel over `bench.py --roofline-probe` (back-to-back launches only,
 # profiles/gemv_gate_up_back_to_back_kernel_trace.txt).  Consecutive launches overlap by a ramp and a tail, so a
 # launch's own start-to-end duration is longer than the time per launch the events measure (wall time / launches).
-GATE_UP_TRACE_BACK_TO_BACK_US = 14.10
+GATE_UP_TRACE_BACK_TO_BACK_US = 14.15
 
 # (name, ggml type name, m, k, copies per step)
 LAYER_SET = [
