@@ -299,15 +299,19 @@ def test_prefill_equals_decode_on_gpu(hip):
     a.close(); b.close()
 
 
-def test_prefill_where_the_norm_adds_split_k_partial_sums(hip, orc):
+@pytest.mark.parametrize("rope_type,kv_f16", [(1, False), (0, False), (1, True)])
+def test_prefill_where_the_norm_adds_split_k_partial_sums(hip, orc, rope_type, kv_f16):
     """Projections whose K is split (2048-wide rows, few row tiles) in a pass of 128 tokens or more: the O
     and down projections leave their partial sums to the row norm that follows (and the last layer's down
-    projection to the reduction kernel).  Logits and both layers' K/V rows track the oracle's batched
-    prefill, and a decode step continues from the cache."""
-    cfg = dict(synth.TINY, hidden=2048, ffn=2048, n_heads=16, n_kv_heads=4, head_dim=128, max_seq_len=192)
+    projection to the reduction kernel), Q | K and V theirs to the RoPE / append kernel (both pair orders,
+    f32 and f16 cache).  Logits and both layers' K/V rows track the oracle's batched prefill, and a decode
+    step continues from the cache."""
+    cfg = dict(synth.TINY, hidden=2048, ffn=2048, n_heads=16, n_kv_heads=4, head_dim=128, max_seq_len=192, rope_type=rope_type)
     weights = synth.make_llama(cfg, seed=81, sigma=0.03, norm_jitter=0.1)
     gm = hip_api.Model(hip, cfg, weights)
     om = orc.Llama(cfg, weights)
+    if kv_f16:
+        gm.configure_kv(True); om.set_kv_f16(True)
     toks = [int(t) for t in util.rng(12).integers(0, cfg["vocab"], 130)]
     _say("model: 130-token prefill, hidden 2048 (split-K O and down projections)")
     lg = gm.forward_prefill(toks, 0)
